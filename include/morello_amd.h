@@ -1,0 +1,209 @@
+/*
+ * morello_amd: MI355X (gfx950) execution backend for Morello Specs -- C ABI.
+ *
+ * This header is the drop-in boundary.  Morello lowers a scheduled Spec to a C function
+ *
+ *     void kernel(const T0 *restrict p0, ..., Tk *restrict pk);
+ *
+ * with one pointer per Spec parameter in Spec parameter order
+ * (morello/src/codegen/cpu.rs:131-219), compiles it (codegen/mod.rs:207-266) and runs it
+ * through a generated `main` (codegen/cpu.rs:284-409).  The entry points below stand where
+ * that emitted kernel and the build/run step stand: they take a plain-C description of the
+ * Spec (type, shape, dtypes, per-parameter layout: morello/src/spec.rs:33-162,
+ * common.rs:15-24, layout.rs:67-81) plus the parameter pointers in the same order, and run
+ * hand-written HIP kernels instead of emitted C.
+ *
+ * Differences from the emitted kernel, all deliberate:
+ *   - every call returns an int status instead of aborting (cpu.rs:1157, :1338);
+ *   - shapes and layouts are run-time arguments, not constants baked into the body;
+ *   - pointers are device (HBM) pointers for mrl_run / mrl_run_async, host pointers for
+ *     mrl_run_host (which stages through device memory and is the literal stand-in for
+ *     calling kernel(...) from the emitted main).
+ * The caller owns every parameter buffer (cpu.rs:399-403); parameters must not alias
+ * (the emitted signature is all-restrict); an accumulating Spec accumulates across calls
+ * exactly as the reference's benchmark loop does (cpu.rs:541-550).
+ *
+ * No type from any framework appears here: plain pointers, sizes and small structs only.
+ */
+#ifndef MORELLO_AMD_H
+#define MORELLO_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------ types */
+
+/* morello/src/common.rs:15-24, same order. */
+typedef enum {
+  MRL_U8 = 0,
+  MRL_I8 = 1,
+  MRL_U16 = 2,
+  MRL_I16 = 3,
+  MRL_U32 = 4,
+  MRL_I32 = 5,
+  MRL_F32 = 6,
+  MRL_BF16 = 7
+} mrl_dtype;
+
+/* morello/src/layout.rs:74-81 */
+typedef enum { MRL_DYNAMIC = 0, MRL_PACKED = 1, MRL_ODDEVEN = 2 } mrl_physdim_kind;
+
+#define MRL_MAX_PHYS 10
+#define MRL_MAX_RANK 5
+#define MRL_MAX_SPEC_RANK 7
+#define MRL_MAX_PARAMS 4
+
+typedef struct {
+  uint8_t logical_dim;
+  uint8_t kind; /* mrl_physdim_kind */
+  uint32_t size; /* Packed / OddEven size; ignored for Dynamic */
+} mrl_physdim;
+
+/* Physical dims listed slowest to fastest (layout.rs:67-70).  ndims == 0 with
+ * `row_major_default` semantics is requested by passing a NULL layout pointer where one is
+ * accepted; inside mrl_spec every parameter carries an explicit layout. */
+typedef struct {
+  uint32_t ndims;
+  mrl_physdim dims[MRL_MAX_PHYS];
+} mrl_layout;
+
+/* The Specs this backend executes (subset of PrimitiveSpecType, spec.rs:57-162, plus the
+ * three-component Compose of examples/matmul_chain.rs). */
+typedef enum {
+  MRL_SPEC_MATMUL = 0,     /* spec_shape [b,m,k,n]; params A[b,m,k] B[b,k,n] C[b,m,n]   */
+  MRL_SPEC_CONV = 1,       /* spec_shape [b,f,c,oh,ow,fh,fw]; params image, filters, out */
+  MRL_SPEC_SOFTMAX = 2,    /* spec_shape = tensor shape; params in, out; uses scan_dim   */
+  MRL_SPEC_COMPOSE_MSM = 3 /* Matmul->Softmax->Matmul; spec_shape [b,m,k,n2,n];
+                              params V[b,n2,n] Q[b,m,k] KT[b,k,n2] out[b,m,n]
+                              (Compose parameter order, spec.rs:3329-3365)               */
+} mrl_spec_kind;
+
+typedef struct {
+  int32_t kind;     /* mrl_spec_kind */
+  int32_t accum;    /* Matmul/Conv: 1 = accumulate into the output (InOut), 0 = overwrite */
+  uint32_t scan_dim; /* Softmax only */
+  uint32_t rank;    /* entries used in spec_shape */
+  uint32_t spec_shape[MRL_MAX_SPEC_RANK];
+  uint32_t n_params;
+  int32_t dtypes[MRL_MAX_PARAMS]; /* mrl_dtype per parameter, Spec parameter order */
+  mrl_layout layouts[MRL_MAX_PARAMS];
+} mrl_spec;
+
+/* Status codes (the emitted C aborts or asserts where these are returned). */
+typedef enum {
+  MRL_OK = 0,
+  MRL_ERR_UNSUPPORTED = 1, /* Spec kind / dtype combination not implemented            */
+  MRL_ERR_BAD_LAYOUT = 2,  /* layout does not apply to the parameter's shape            */
+  MRL_ERR_BAD_SPEC = 3,    /* malformed descriptor: rank, zero dim, n_params, scan_dim  */
+  MRL_ERR_HIP = 4,         /* a HIP runtime call failed; see mrl_last_error()           */
+  MRL_ERR_NO_DEVICE = 5,   /* no gfx950 device visible                                  */
+  MRL_ERR_NULL = 6,        /* NULL pointer argument                                     */
+  MRL_ERR_TOO_LARGE = 7    /* a tensor exceeds the index range the kernels assume      */
+} mrl_status;
+
+/* ------------------------------------------------------------- life cycle */
+
+/* Selects `device` and checks that it is a gfx950 part.  Idempotent. */
+int mrl_init(int device);
+const char *mrl_status_string(int status);
+/* Text of the last HIP error seen by this thread ("" if none). */
+const char *mrl_last_error(void);
+/* "major.minor.patch" of this library. */
+const char *mrl_version(void);
+
+/* --------------------------------------------------- Spec surface (host) */
+
+/* common.rs:30-36 */
+size_t mrl_dtype_size(int dtype);
+/* common.rs:52-65: "u8", "i8", ..., "f32", "bf16" */
+const char *mrl_dtype_name(int dtype);
+
+/* Layout constructors: layout.rs:1234-1247, :1249-1253, :1255-1271, :1273-1279. */
+int mrl_layout_row_major(const uint32_t *shape, uint32_t rank, mrl_layout *out);
+int mrl_layout_col_major(const uint32_t *shape, uint32_t rank, mrl_layout *out);
+int mrl_layout_batched_col_major(const uint32_t *shape, uint32_t rank, mrl_layout *out);
+int mrl_layout_nhwc(const uint32_t *shape, uint32_t rank, mrl_layout *out);
+/* layout.rs:769-810 (expand_physical_shape). */
+int mrl_layout_physical_shape(const mrl_layout *layout, const uint32_t *shape, uint32_t rank,
+                              uint32_t *phys_shape);
+/* layout.rs:221-272 (buffer_indexing_expr) evaluated at `point`; -1 on a bad layout. */
+int64_t mrl_layout_buffer_index(const mrl_layout *layout, const uint32_t *shape, uint32_t rank,
+                                const uint32_t *point);
+
+/* spec.rs:467-583 (parameter_shape): logical shape of parameter `idx`. */
+int mrl_spec_parameter_shape(const mrl_spec *spec, uint32_t idx, uint32_t *shape,
+                             uint32_t *rank);
+/* spec.rs:1204-1245: 0 = In, 1 = Out, 2 = InOut; negative on error. */
+int mrl_spec_parameter_direction(const mrl_spec *spec, uint32_t idx);
+/* tensorspec.rs:153-160 (bytes_used) of parameter `idx`; 0 on error. */
+size_t mrl_spec_parameter_bytes(const mrl_spec *spec, uint32_t idx);
+/* spec.rs:273-305 convention extended to every dtype: Matmul/Conv 2*MACs, Softmax 5/elem,
+ * Compose = sum of its components. */
+uint64_t mrl_spec_ops(const mrl_spec *spec);
+/* MRL_OK if mrl_run would accept the Spec (validates shapes, dtypes, layouts). */
+int mrl_spec_check(const mrl_spec *spec);
+/* Bytes of device scratch mrl_run allocates internally for this Spec (relayout staging,
+ * transposed operands); 0 when the kernels read the parameters in place. */
+size_t mrl_spec_workspace_bytes(const mrl_spec *spec);
+
+/* -------------------------------------------------------------- execution */
+
+/* Stands where the emitted `kernel(p0, ..., pk)` stands (codegen/cpu.rs:131-219,
+ * call site :497-514).  `params` holds n_params DEVICE pointers in Spec parameter order,
+ * each to bytes_used(parameter) bytes laid out by that parameter's layout.  Synchronous:
+ * returns after the work has finished. */
+int mrl_run(const mrl_spec *spec, void *const *params);
+
+/* As mrl_run but only enqueues on `stream` (a hipStream_t, NULL = default stream). */
+int mrl_run_async(const mrl_spec *spec, void *const *params, void *stream);
+
+/* Literal stand-in for calling the emitted kernel from the emitted main
+ * (codegen/cpu.rs:284-409): `params` are HOST pointers; inputs (and the output, when it
+ * is read) are copied to the device, the Spec is run, written parameters are copied back. */
+int mrl_run_host(const mrl_spec *spec, void *const *params);
+
+/* Per-kind conveniences that build the descriptor themselves.  NULL layouts mean
+ * row-major, except Conv where NULL means NHWC image/output and KRSC filters
+ * (layout![0,2,3,1] on [n,c,h,w] and [f,c,fh,fw]; layout.rs:1273-1279). */
+int mrl_matmul(uint32_t b, uint32_t m, uint32_t k, uint32_t n, int dt_a, int dt_b, int dt_c,
+               int accum, const void *a, const void *bmat, void *c, void *stream);
+int mrl_conv(uint32_t b, uint32_t f, uint32_t c, uint32_t oh, uint32_t ow, uint32_t fh,
+             uint32_t fw, int dt_img, int dt_filt, int dt_out, int accum, const void *image,
+             const void *filters, void *out, void *stream);
+int mrl_softmax(const uint32_t *shape, uint32_t rank, uint32_t scan_dim, const void *in,
+                void *out, void *stream);
+/* KT is the B operand of the first Matmul, logical [b,k,n2]; kt_col_major != 0 says it is
+ * stored with layout![0,2,1] (i.e. K stored row-major as [b,n2,k]). */
+int mrl_compose_msm(uint32_t b, uint32_t m, uint32_t k, uint32_t n2, uint32_t n, int dt_v,
+                    int dt_q, int dt_kt, int kt_col_major, const void *v, const void *q,
+                    const void *kt, void *out, void *stream);
+
+/* ------------------------------------------------ benchmark protocol (L5) */
+
+/* Mirrors CodeGen::bench / the emitted benchmarking main (codegen/cpu.rs:516-568,
+ * codegen/mod.rs:133-169,330-340): one warm-up launch, then `iters` back-to-back launches
+ * between two HIP events on `stream`'s queue, repeated `repeats` times.  Writes the best
+ * and the mean per-launch time in nanoseconds.  Accumulating Specs keep accumulating. */
+int mrl_bench(const mrl_spec *spec, void *const *params, uint32_t iters, uint32_t repeats,
+              double *best_ns_per_iter, double *mean_ns_per_iter);
+
+/* ------------------------------------------- device memory (plumbing only) */
+
+int mrl_device_malloc(void **ptr, size_t bytes);
+int mrl_device_free(void *ptr);
+int mrl_memcpy_h2d(void *dst, const void *src, size_t bytes);
+int mrl_memcpy_d2h(void *dst, const void *src, size_t bytes);
+int mrl_memset(void *dst, int value, size_t bytes);
+int mrl_device_synchronize(void);
+/* Name, CU count, clock (kHz) and memory size of the selected device. */
+int mrl_device_info(char *name, size_t name_len, int *compute_units, int *clock_khz,
+                    size_t *total_mem_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

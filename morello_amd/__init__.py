@@ -1,0 +1,348 @@
+"""morello_amd: MI355X execution backend for Morello Specs -- Python view of the C ABI.
+
+The classes mirror the names of Morello's Spec surface so that a test written against the
+reference reads the same here: `Dtype` (morello/src/common.rs:15-65), `PhysDim`/`Layout`
+and the constructors `row_major`, `col_major`, `batched_col_major`, `nhwc`, `layout`
+(morello/src/layout.rs:67-81, 1234-1302), and the Spec constructors `Matmul`, `Conv`,
+`Softmax`, `ComposeMSM` (morello/src/spec.rs:57-162, 467-583).  All arithmetic happens in
+libmorello_amd.so; this module only packs descriptors and moves bytes.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import enum
+from dataclasses import dataclass
+from typing import Optional, Sequence, Tuple
+
+import numpy as np
+
+from . import _binding as B
+
+
+class MorelloError(RuntimeError):
+    def __init__(self, status: int, where: str):
+        lib = B.load()
+        msg = lib.mrl_status_string(status).decode()
+        detail = lib.mrl_last_error().decode()
+        super().__init__(f"{where}: {msg}" + (f" ({detail})" if detail and status == 4 else ""))
+        self.status = status
+
+
+def _check(status: int, where: str):
+    if status != 0:
+        raise MorelloError(status, where)
+
+
+class Dtype(enum.IntEnum):
+    """morello/src/common.rs:15-24."""
+    Uint8 = 0
+    Sint8 = 1
+    Uint16 = 2
+    Sint16 = 3
+    Uint32 = 4
+    Sint32 = 5
+    Float32 = 6
+    Bfloat16 = 7
+
+    @property
+    def size(self) -> int:
+        return int(B.load().mrl_dtype_size(int(self)))
+
+    def __str__(self) -> str:
+        return B.load().mrl_dtype_name(int(self)).decode()
+
+    @property
+    def numpy(self):
+        """Storage dtype; bf16 travels as its 16-bit pattern."""
+        return {0: np.uint8, 1: np.int8, 2: np.uint16, 3: np.int16, 4: np.uint32, 5: np.int32,
+                6: np.float32, 7: np.uint16}[int(self)]
+
+
+u8, i8, u16, i16, u32, i32, f32, bf16 = (Dtype(i) for i in range(8))
+
+
+@dataclass(frozen=True)
+class PhysDim:
+    """morello/src/layout.rs:74-81.  kind: 0 Dynamic, 1 Packed(size), 2 OddEven(size)."""
+    kind: int = 0
+    size: int = 0
+
+
+Dynamic = PhysDim(0, 0)
+
+
+def Packed(n: int) -> PhysDim:
+    return PhysDim(1, n)
+
+
+def OddEven(n: int) -> PhysDim:
+    return PhysDim(2, n)
+
+
+class Layout:
+    """Physical dims, slowest to fastest, as (logical_dim, PhysDim) pairs."""
+
+    def __init__(self, dims: Sequence[Tuple[int, PhysDim]]):
+        self.dims = [(int(d), pd) for d, pd in dims]
+        if len(self.dims) > B.MAX_PHYS:
+            raise ValueError("too many physical dims")
+
+    def to_c(self) -> B.LayoutC:
+        out = B.LayoutC()
+        out.ndims = len(self.dims)
+        for i, (d, pd) in enumerate(self.dims):
+            out.dims[i].logical_dim = d
+            out.dims[i].kind = pd.kind
+            out.dims[i].size = pd.size
+        return out
+
+    @staticmethod
+    def from_c(c: B.LayoutC) -> "Layout":
+        return Layout([(c.dims[i].logical_dim, PhysDim(c.dims[i].kind, c.dims[i].size if c.dims[i].kind else 0))
+                       for i in range(c.ndims)])
+
+    def physical_shape(self, shape: Sequence[int]):
+        """expand_physical_shape (layout.rs:769-810); raises on shapes it does not apply to."""
+        arr = (C.c_uint32 * len(shape))(*shape)
+        out = (C.c_uint32 * B.MAX_PHYS)()
+        lc = self.to_c()
+        _check(B.load().mrl_layout_physical_shape(C.byref(lc), arr, len(shape), out), "physical_shape")
+        return [int(out[i]) for i in range(len(self.dims))]
+
+    def applies_to_shape(self, shape: Sequence[int]) -> bool:
+        try:
+            self.physical_shape(shape)
+            return True
+        except MorelloError:
+            return False
+
+    def buffer_index(self, shape: Sequence[int], point: Sequence[int]) -> int:
+        """buffer_indexing_expr (layout.rs:221-272) evaluated at a logical point."""
+        arr = (C.c_uint32 * len(shape))(*shape)
+        pt = (C.c_uint32 * len(point))(*point)
+        lc = self.to_c()
+        idx = int(B.load().mrl_layout_buffer_index(C.byref(lc), arr, len(shape), pt))
+        if idx < 0:
+            raise MorelloError(2, "buffer_index")
+        return idx
+
+    def __eq__(self, other):
+        return isinstance(other, Layout) and self.dims == other.dims
+
+    def __repr__(self):
+        def one(d, pd):
+            return f"{d}" if pd.kind == 0 else f"{d} {'p' if pd.kind == 1 else 'oe'}({pd.size})"
+        return "layout![" + ", ".join(one(d, pd) for d, pd in self.dims) + "]"
+
+
+def layout(*dims) -> Layout:
+    """The `layout!` macro (layout.rs:1283-1302): ints are Dynamic dims, `(d, Packed(n))` or
+    `(d, OddEven(n))` tuples are packed dims."""
+    out = []
+    for d in dims:
+        out.append((d, Dynamic) if isinstance(d, int) else (d[0], d[1]))
+    return Layout(out)
+
+
+def _ctor(name: str, shape: Sequence[int]) -> Layout:
+    arr = (C.c_uint32 * len(shape))(*shape)
+    out = B.LayoutC()
+    _check(getattr(B.load(), name)(arr, len(shape), C.byref(out)), name)
+    return Layout.from_c(out)
+
+
+def row_major(shape):
+    return _ctor("mrl_layout_row_major", shape)
+
+
+def col_major(shape):
+    return _ctor("mrl_layout_col_major", shape)
+
+
+def batched_col_major(shape):
+    return _ctor("mrl_layout_batched_col_major", shape)
+
+
+def nhwc(shape):
+    return _ctor("mrl_layout_nhwc", shape)
+
+
+class SpecKind(enum.IntEnum):
+    Matmul = 0
+    Conv = 1
+    Softmax = 2
+    ComposeMSM = 3
+
+
+class OperandDirection(enum.IntEnum):
+    """morello/src/spec.rs:1091-1095."""
+    In = 0
+    Out = 1
+    InOut = 2
+
+
+class Spec:
+    """A logical Spec plus one (dtype, layout) per parameter (spec.rs:33-56, tensorspec.rs:19-32).
+
+    `layouts=None` means row-major for every parameter, except Conv where it means NHWC
+    image/output and KRSC filters.
+    """
+
+    def __init__(self, kind: SpecKind, spec_shape, dtypes, layouts=None, accum=False, scan_dim=0):
+        self.kind = SpecKind(kind)
+        self.spec_shape = [int(x) for x in spec_shape]
+        self.dtypes = [Dtype(d) for d in dtypes]
+        self.accum = bool(accum)
+        self.scan_dim = int(scan_dim)
+        self._c = B.SpecC()
+        self._c.kind = int(self.kind)
+        self._c.accum = int(self.accum)
+        self._c.scan_dim = self.scan_dim
+        if len(self.spec_shape) > B.MAX_SPEC_RANK or len(self.dtypes) > B.MAX_PARAMS:
+            raise ValueError("spec_shape or dtypes too long")
+        self._c.rank = len(self.spec_shape)
+        for i, v in enumerate(self.spec_shape):
+            self._c.spec_shape[i] = v
+        self._c.n_params = len(self.dtypes)
+        for i, d in enumerate(self.dtypes):
+            self._c.dtypes[i] = int(d)
+        if layouts is None:
+            layouts = [None] * len(self.dtypes)
+        self.layouts = []
+        for i, l in enumerate(layouts):
+            if l is None:
+                shp = self.parameter_shape(i)
+                l = nhwc(shp) if self.kind == SpecKind.Conv else row_major(shp)
+            self.layouts.append(l)
+            self._c.layouts[i] = l.to_c()
+
+    # -- reference-named accessors ---------------------------------------------------
+    def parameter_shape(self, idx: int):
+        out = (C.c_uint32 * B.MAX_RANK)()
+        rank = C.c_uint32()
+        _check(B.load().mrl_spec_parameter_shape(C.byref(self._c), idx, out, C.byref(rank)),
+               "parameter_shape")
+        return [int(out[i]) for i in range(rank.value)]
+
+    def parameter_shapes(self):
+        return [self.parameter_shape(i) for i in range(len(self.dtypes))]
+
+    def operand_directions(self):
+        lib = B.load()
+        return [OperandDirection(lib.mrl_spec_parameter_direction(C.byref(self._c), i))
+                for i in range(len(self.dtypes))]
+
+    def bytes_used(self, idx: int) -> int:
+        return int(B.load().mrl_spec_parameter_bytes(C.byref(self._c), idx))
+
+    def flops(self) -> int:
+        return int(B.load().mrl_spec_ops(C.byref(self._c)))
+
+    def check(self) -> int:
+        return int(B.load().mrl_spec_check(C.byref(self._c)))
+
+    def workspace_bytes(self) -> int:
+        return int(B.load().mrl_spec_workspace_bytes(C.byref(self._c)))
+
+    # -- execution -------------------------------------------------------------------
+    def run_device(self, ptrs: Sequence[int]):
+        """`ptrs`: device pointers in Spec parameter order.  Synchronous."""
+        arr = (C.c_void_p * len(ptrs))(*ptrs)
+        _check(B.load().mrl_run(C.byref(self._c), arr), "mrl_run")
+
+    def run_host(self, *arrays: np.ndarray):
+        """`arrays`: numpy buffers in Spec parameter order, each already laid out by its
+        parameter's layout; the output array is written in place."""
+        if len(arrays) != len(self.dtypes):
+            raise ValueError("one array per parameter")
+        for i, a in enumerate(arrays):
+            if not a.flags["C_CONTIGUOUS"] or a.nbytes != self.bytes_used(i):
+                raise ValueError(f"parameter {i}: need a contiguous buffer of {self.bytes_used(i)} bytes")
+        arr = (C.c_void_p * len(arrays))(*[a.ctypes.data for a in arrays])
+        _check(B.load().mrl_run_host(C.byref(self._c), arr), "mrl_run_host")
+
+    def bench(self, ptrs: Sequence[int], iters: int, repeats: int = 10):
+        """CodeGen::bench protocol (codegen/mod.rs:133-169): (best, mean) ns per launch."""
+        arr = (C.c_void_p * len(ptrs))(*ptrs)
+        best, mean = C.c_double(), C.c_double()
+        _check(B.load().mrl_bench(C.byref(self._c), arr, iters, repeats, C.byref(best), C.byref(mean)),
+               "mrl_bench")
+        return best.value, mean.value
+
+
+def Matmul(spec_shape, dtypes, layouts=None, accum=False) -> Spec:
+    """Matmul{accum} with spec_shape [b, m, k, n] (spec.rs:480-485)."""
+    return Spec(SpecKind.Matmul, spec_shape, dtypes, layouts, accum)
+
+
+def MatmulAccum(spec_shape, dtypes, layouts=None) -> Spec:
+    return Matmul(spec_shape, dtypes, layouts, accum=True)
+
+
+def Conv(spec_shape, dtypes, layouts=None, accum=False) -> Spec:
+    """Conv{accum} with spec_shape [b, f, c, oh, ow, fh, fw] (spec.rs:486-498)."""
+    return Spec(SpecKind.Conv, spec_shape, dtypes, layouts, accum)
+
+
+def Softmax(shape, scan_dim, layouts=None) -> Spec:
+    """Softmax{scan_dim} on an f32 tensor (spec.rs:86-90, 523-526)."""
+    return Spec(SpecKind.Softmax, shape, [f32, f32], layouts, scan_dim=scan_dim)
+
+
+def ComposeMSM(b, m, k, n2, n, dtypes=(bf16, bf16, bf16, f32), layouts=None) -> Spec:
+    """Compose [Matmul, Softmax{2}, Matmul] with external parameters [V, Q, KT, out]
+    (spec.rs:3329-3365; examples/matmul_chain.rs:26-57)."""
+    return Spec(SpecKind.ComposeMSM, [b, m, k, n2, n], dtypes, layouts)
+
+
+class DeviceBuffer:
+    """A device allocation owned by Python; plumbing for tests and the benchmark."""
+
+    def __init__(self, nbytes: int):
+        self.nbytes = int(nbytes)
+        p = C.c_void_p()
+        _check(B.load().mrl_device_malloc(C.byref(p), self.nbytes), "mrl_device_malloc")
+        self.ptr = p.value
+
+    @staticmethod
+    def from_numpy(a: np.ndarray) -> "DeviceBuffer":
+        a = np.ascontiguousarray(a)
+        buf = DeviceBuffer(a.nbytes)
+        _check(B.load().mrl_memcpy_h2d(buf.ptr, a.ctypes.data, a.nbytes), "mrl_memcpy_h2d")
+        return buf
+
+    def to_numpy(self, dtype, shape) -> np.ndarray:
+        out = np.empty(shape, dtype=dtype)
+        assert out.nbytes <= self.nbytes
+        _check(B.load().mrl_memcpy_d2h(out.ctypes.data, self.ptr, out.nbytes), "mrl_memcpy_d2h")
+        return out
+
+    def zero(self):
+        _check(B.load().mrl_memset(self.ptr, 0, self.nbytes), "mrl_memset")
+
+    def free(self):
+        if self.ptr:
+            B.load().mrl_device_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def init(device: int = 0):
+    _check(B.load().mrl_init(device), "mrl_init")
+
+
+def synchronize():
+    _check(B.load().mrl_device_synchronize(), "mrl_device_synchronize")
+
+
+def device_info():
+    name = C.create_string_buffer(256)
+    cus, khz, mem = C.c_int(), C.c_int(), C.c_size_t()
+    _check(B.load().mrl_device_info(name, 256, C.byref(cus), C.byref(khz), C.byref(mem)), "mrl_device_info")
+    return {"name": name.value.decode(), "compute_units": cus.value, "clock_khz": khz.value,
+            "total_mem_bytes": mem.value}

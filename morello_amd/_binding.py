@@ -1,0 +1,98 @@
+"""ctypes binding of libmorello_amd.so (the C ABI in include/morello_amd.h).
+
+Loading fails loudly: there is no CPU implementation behind this package, so a missing
+library is an ImportError-grade problem, not something to paper over.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libmorello_amd.so")
+
+MAX_PHYS, MAX_RANK, MAX_SPEC_RANK, MAX_PARAMS = 10, 5, 7, 4
+
+
+class PhysDimC(C.Structure):
+    _fields_ = [("logical_dim", C.c_uint8), ("kind", C.c_uint8), ("size", C.c_uint32)]
+
+
+class LayoutC(C.Structure):
+    _fields_ = [("ndims", C.c_uint32), ("dims", PhysDimC * MAX_PHYS)]
+
+
+class SpecC(C.Structure):
+    _fields_ = [
+        ("kind", C.c_int32),
+        ("accum", C.c_int32),
+        ("scan_dim", C.c_uint32),
+        ("rank", C.c_uint32),
+        ("spec_shape", C.c_uint32 * MAX_SPEC_RANK),
+        ("n_params", C.c_uint32),
+        ("dtypes", C.c_int32 * MAX_PARAMS),
+        ("layouts", LayoutC * MAX_PARAMS),
+    ]
+
+
+_U32P = C.POINTER(C.c_uint32)
+_VPP = C.POINTER(C.c_void_p)
+
+# name -> (restype, argtypes); every symbol include/morello_amd.h declares.
+SIGNATURES = {
+    "mrl_init": (C.c_int, [C.c_int]),
+    "mrl_status_string": (C.c_char_p, [C.c_int]),
+    "mrl_last_error": (C.c_char_p, []),
+    "mrl_version": (C.c_char_p, []),
+    "mrl_dtype_size": (C.c_size_t, [C.c_int]),
+    "mrl_dtype_name": (C.c_char_p, [C.c_int]),
+    "mrl_layout_row_major": (C.c_int, [_U32P, C.c_uint32, C.POINTER(LayoutC)]),
+    "mrl_layout_col_major": (C.c_int, [_U32P, C.c_uint32, C.POINTER(LayoutC)]),
+    "mrl_layout_batched_col_major": (C.c_int, [_U32P, C.c_uint32, C.POINTER(LayoutC)]),
+    "mrl_layout_nhwc": (C.c_int, [_U32P, C.c_uint32, C.POINTER(LayoutC)]),
+    "mrl_layout_physical_shape": (C.c_int, [C.POINTER(LayoutC), _U32P, C.c_uint32, _U32P]),
+    "mrl_layout_buffer_index": (C.c_int64, [C.POINTER(LayoutC), _U32P, C.c_uint32, _U32P]),
+    "mrl_spec_parameter_shape": (C.c_int, [C.POINTER(SpecC), C.c_uint32, _U32P, _U32P]),
+    "mrl_spec_parameter_direction": (C.c_int, [C.POINTER(SpecC), C.c_uint32]),
+    "mrl_spec_parameter_bytes": (C.c_size_t, [C.POINTER(SpecC), C.c_uint32]),
+    "mrl_spec_ops": (C.c_uint64, [C.POINTER(SpecC)]),
+    "mrl_spec_check": (C.c_int, [C.POINTER(SpecC)]),
+    "mrl_spec_workspace_bytes": (C.c_size_t, [C.POINTER(SpecC)]),
+    "mrl_run": (C.c_int, [C.POINTER(SpecC), _VPP]),
+    "mrl_run_async": (C.c_int, [C.POINTER(SpecC), _VPP, C.c_void_p]),
+    "mrl_run_host": (C.c_int, [C.POINTER(SpecC), _VPP]),
+    "mrl_matmul": (C.c_int, [C.c_uint32] * 4 + [C.c_int] * 4 + [C.c_void_p] * 4),
+    "mrl_conv": (C.c_int, [C.c_uint32] * 7 + [C.c_int] * 4 + [C.c_void_p] * 4),
+    "mrl_softmax": (C.c_int, [_U32P, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "mrl_compose_msm": (C.c_int, [C.c_uint32] * 5 + [C.c_int] * 4 + [C.c_void_p] * 5),
+    "mrl_bench": (C.c_int, [C.POINTER(SpecC), _VPP, C.c_uint32, C.c_uint32,
+                            C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+    "mrl_device_malloc": (C.c_int, [_VPP, C.c_size_t]),
+    "mrl_device_free": (C.c_int, [C.c_void_p]),
+    "mrl_memcpy_h2d": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    "mrl_memcpy_d2h": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    "mrl_memset": (C.c_int, [C.c_void_p, C.c_int, C.c_size_t]),
+    "mrl_device_synchronize": (C.c_int, []),
+    "mrl_device_info": (C.c_int, [C.c_char_p, C.c_size_t, C.POINTER(C.c_int), C.POINTER(C.c_int),
+                                  C.POINTER(C.c_size_t)]),
+}
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Loads the library (building nothing: run `python -m morello_amd.build` first)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m morello_amd.build` "
+            "(there is no CPU fallback)")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the ABI lost a symbol
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib

@@ -1,0 +1,710 @@
+// Host side of the C ABI declared in include/morello_amd.h: Spec validation, layout
+// handling and dispatch onto the kernels.  No compute happens on the CPU here; a Spec the
+// fast kernels do not cover runs on the generic GPU kernels, and a missing device is an
+// error, never a fallback.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "kernels.h"
+
+namespace {
+
+thread_local std::string g_last_error;
+int g_device = -1;
+
+int hip_fail(hipError_t e, const char *what) {
+  g_last_error = std::string(what) + ": " + hipGetErrorString(e);
+  return MRL_ERR_HIP;
+}
+#define HIP_TRY(expr)                                  \
+  do {                                                 \
+    hipError_t e_ = (expr);                            \
+    if (e_ != hipSuccess) return hip_fail(e_, #expr);  \
+  } while (0)
+
+bool valid_dtype(int d) { return d >= MRL_U8 && d <= MRL_BF16; }
+
+uint64_t volume(const uint32_t *s, uint32_t r) {
+  uint64_t v = 1;
+  for (uint32_t i = 0; i < r; i++) v *= s[i];
+  return v;
+}
+
+uint32_t expected_params(int kind) {
+  switch (kind) {
+    case MRL_SPEC_MATMUL: case MRL_SPEC_CONV: return 3;
+    case MRL_SPEC_SOFTMAX: return 2;
+    case MRL_SPEC_COMPOSE_MSM: return 4;
+    default: return 0;
+  }
+}
+
+uint32_t expected_rank(const mrl_spec &s) {
+  switch (s.kind) {
+    case MRL_SPEC_MATMUL: return 4;
+    case MRL_SPEC_CONV: return 7;
+    case MRL_SPEC_SOFTMAX: return s.rank;
+    case MRL_SPEC_COMPOSE_MSM: return 5;
+    default: return 0;
+  }
+}
+
+// morello/src/spec.rs:467-583
+int parameter_shape(const mrl_spec &s, uint32_t idx, uint32_t *shape, uint32_t *rank) {
+  const uint32_t *ss = s.spec_shape;
+  switch (s.kind) {
+    case MRL_SPEC_MATMUL:
+      *rank = 3;
+      if (idx == 0) shape[0] = ss[0], shape[1] = ss[1], shape[2] = ss[2];
+      else if (idx == 1) shape[0] = ss[0], shape[1] = ss[2], shape[2] = ss[3];
+      else if (idx == 2) shape[0] = ss[0], shape[1] = ss[1], shape[2] = ss[3];
+      else return MRL_ERR_BAD_SPEC;
+      return MRL_OK;
+    case MRL_SPEC_CONV: {
+      const uint32_t b = ss[0], f = ss[1], c = ss[2], oh = ss[3], ow = ss[4], fh = ss[5], fw = ss[6];
+      *rank = 4;
+      if (idx == 0) shape[0] = b, shape[1] = c, shape[2] = oh + fh - 1, shape[3] = ow + fw - 1;
+      else if (idx == 1) shape[0] = f, shape[1] = c, shape[2] = fh, shape[3] = fw;
+      else if (idx == 2) shape[0] = b, shape[1] = f, shape[2] = oh, shape[3] = ow;
+      else return MRL_ERR_BAD_SPEC;
+      return MRL_OK;
+    }
+    case MRL_SPEC_SOFTMAX:
+      if (idx > 1) return MRL_ERR_BAD_SPEC;
+      *rank = s.rank;
+      for (uint32_t d = 0; d < s.rank; d++) shape[d] = ss[d];
+      return MRL_OK;
+    case MRL_SPEC_COMPOSE_MSM: {
+      // spec_shape [b, m, k, n2, n]; parameters V, Q, KT, out (spec.rs:3329-3365).
+      const uint32_t b = ss[0], m = ss[1], k = ss[2], n2 = ss[3], n = ss[4];
+      *rank = 3;
+      if (idx == 0) shape[0] = b, shape[1] = n2, shape[2] = n;
+      else if (idx == 1) shape[0] = b, shape[1] = m, shape[2] = k;
+      else if (idx == 2) shape[0] = b, shape[1] = k, shape[2] = n2;
+      else if (idx == 3) shape[0] = b, shape[1] = m, shape[2] = n;
+      else return MRL_ERR_BAD_SPEC;
+      return MRL_OK;
+    }
+    default:
+      return MRL_ERR_BAD_SPEC;
+  }
+}
+
+// morello/src/spec.rs:1204-1245.  0 In, 1 Out, 2 InOut.
+int parameter_direction(const mrl_spec &s, uint32_t idx) {
+  const uint32_t n = expected_params(s.kind);
+  if (n == 0 || idx >= n) return -1;
+  if (idx + 1 < n) return 0;
+  if ((s.kind == MRL_SPEC_MATMUL || s.kind == MRL_SPEC_CONV) && s.accum) return 2;
+  return 1;
+}
+
+int check_spec(const mrl_spec *sp) {
+  if (!sp) return MRL_ERR_NULL;
+  const mrl_spec &s = *sp;
+  const uint32_t np = expected_params(s.kind);
+  if (np == 0) return MRL_ERR_UNSUPPORTED;
+  if (s.n_params != np) return MRL_ERR_BAD_SPEC;
+  if (s.rank == 0 || s.rank > MRL_MAX_SPEC_RANK || s.rank != expected_rank(s)) return MRL_ERR_BAD_SPEC;
+  if (s.kind == MRL_SPEC_SOFTMAX && (s.rank > MRL_MAX_RANK || s.scan_dim >= s.rank)) return MRL_ERR_BAD_SPEC;
+  for (uint32_t d = 0; d < s.rank; d++)
+    if (s.spec_shape[d] == 0) return MRL_ERR_BAD_SPEC;
+  for (uint32_t i = 0; i < np; i++) {
+    if (!valid_dtype(s.dtypes[i])) return MRL_ERR_BAD_SPEC;
+    uint32_t shape[MRL_MAX_RANK], rank;
+    if (parameter_shape(s, i, shape, &rank) != MRL_OK) return MRL_ERR_BAD_SPEC;
+    // DimSize volume is a u32 in the reference (tensorspec.rs:180-182); buffer indices are i32.
+    if (volume(shape, rank) > 0x7fffffffull) return MRL_ERR_TOO_LARGE;
+    uint32_t phys[MRL_MAX_PHYS];
+    if (!mrl::physical_shape(s.layouts[i], shape, rank, phys)) return MRL_ERR_BAD_LAYOUT;
+  }
+  switch (s.kind) {
+    case MRL_SPEC_MATMUL:
+    case MRL_SPEC_CONV:
+      // bf16 outputs would need bf16 arithmetic in the accumulate; not implemented.
+      if (s.dtypes[2] == MRL_BF16) return MRL_ERR_UNSUPPORTED;
+      break;
+    case MRL_SPEC_SOFTMAX:
+      if (s.dtypes[0] != MRL_F32 || s.dtypes[1] != MRL_F32) return MRL_ERR_UNSUPPORTED;
+      break;
+    case MRL_SPEC_COMPOSE_MSM:
+      if (s.dtypes[3] != MRL_F32) return MRL_ERR_UNSUPPORTED;
+      break;
+  }
+  return MRL_OK;
+}
+
+// A parameter prepared for the kernels: either used in place through strides, or staged
+// into a dense row-major scratch buffer by the relayout kernel.
+struct Prepared {
+  mrl::Strided t;
+  void *scratch = nullptr;      // non-null when staged
+  void *user = nullptr;
+  mrl::LayoutEval user_layout;  // valid when staged
+  mrl::LayoutEval dense_layout;
+  uint64_t count = 0;
+  uint32_t elem = 0;
+};
+
+struct Workspace {
+  hipStream_t stream;
+  std::vector<void *> allocs;
+  explicit Workspace(hipStream_t s) : stream(s) {}
+  hipError_t alloc(void **p, size_t bytes) {
+    hipError_t e = hipMallocAsync(p, bytes ? bytes : 4, stream);
+    if (e == hipSuccess) allocs.push_back(*p);
+    return e;
+  }
+  ~Workspace() {
+    for (void *p : allocs) (void)hipFreeAsync(p, stream);
+  }
+};
+
+int prepare(const mrl_spec &s, uint32_t idx, void *ptr, bool needs_read, Workspace &ws, Prepared *out) {
+  uint32_t shape[MRL_MAX_RANK], rank;
+  parameter_shape(s, idx, shape, &rank);
+  out->t.dtype = s.dtypes[idx];
+  out->t.rank = rank;
+  out->user = ptr;
+  out->elem = uint32_t(mrl_dtype_size(s.dtypes[idx]));
+  out->count = volume(shape, rank);
+  for (uint32_t d = 0; d < MRL_MAX_RANK; d++) out->t.shape[d] = d < rank ? shape[d] : 1;
+  if (mrl::layout_strides(s.layouts[idx], shape, rank, out->t.stride)) {
+    out->t.ptr = ptr;
+    return MRL_OK;
+  }
+  mrl_layout dense;
+  mrl_layout_row_major(shape, rank, &dense);
+  if (!mrl::make_layout_eval(s.layouts[idx], shape, rank, &out->user_layout) ||
+      !mrl::make_layout_eval(dense, shape, rank, &out->dense_layout))
+    return MRL_ERR_BAD_LAYOUT;
+  HIP_TRY(ws.alloc(&out->scratch, out->count * out->elem));
+  out->t.ptr = out->scratch;
+  mrl::layout_strides(dense, shape, rank, out->t.stride);
+  if (needs_read)
+    HIP_TRY(mrl::launch_relayout(ptr, out->scratch, out->user_layout, out->dense_layout, out->elem,
+                                 out->count, ws.stream));
+  return MRL_OK;
+}
+
+int finish_output(Prepared &p, Workspace &ws) {
+  if (!p.scratch) return MRL_OK;
+  HIP_TRY(mrl::launch_relayout(p.scratch, p.user, p.dense_layout, p.user_layout, p.elem, p.count,
+                               ws.stream));
+  return MRL_OK;
+}
+
+bool dense_row_major(const mrl::Strided &t) {
+  int64_t run = 1;
+  for (int d = int(t.rank) - 1; d >= 0; d--) {
+    if (t.shape[d] == 1) continue;
+    if (t.stride[d] != run) return false;
+    run *= t.shape[d];
+  }
+  return true;
+}
+
+// Leading dimension / batch stride of a [b, r, c] tensor whose last dim is contiguous.
+bool as_rows(const mrl::Strided &t, int64_t *ld, int64_t *batch_stride) {
+  if (t.rank != 3) return false;
+  if (t.shape[2] != 1 && t.stride[2] != 1) return false;
+  *ld = t.shape[1] == 1 ? int64_t(t.shape[2]) : t.stride[1];
+  *batch_stride = t.shape[0] == 1 ? 0 : t.stride[0];
+  return *ld >= int64_t(t.shape[2]);
+}
+
+int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws) {
+  Prepared a, b, c;
+  int rc;
+  if ((rc = prepare(s, 0, params[0], true, ws, &a)) != MRL_OK) return rc;
+  if ((rc = prepare(s, 1, params[1], true, ws, &b)) != MRL_OK) return rc;
+  if ((rc = prepare(s, 2, params[2], s.accum != 0, ws, &c)) != MRL_OK) return rc;
+  mrl::GemmArgs g;
+  g.a = a.t.ptr, g.b = b.t.ptr, g.c = c.t.ptr;
+  g.batch = s.spec_shape[0], g.m = s.spec_shape[1], g.k = s.spec_shape[2], g.n = s.spec_shape[3];
+  g.accum = s.accum;
+  const bool rows = as_rows(a.t, &g.lda, &g.sa) && as_rows(b.t, &g.ldb, &g.sb) &&
+                    as_rows(c.t, &g.ldc, &g.sc);
+  const int da = s.dtypes[0], db = s.dtypes[1], dc = s.dtypes[2];
+  bool done = false;
+  if (rows && (da == MRL_U8 || da == MRL_I8) && db == MRL_I8 && dc == MRL_I32 &&
+      mrl::gemm_i8_applicable(g, false)) {
+    HIP_TRY(mrl::launch_gemm_i8(g, da == MRL_U8, ws.stream));
+    done = true;
+  } else if (rows && da == MRL_BF16 && db == MRL_BF16 && dc == MRL_F32 &&
+             mrl::gemm_bf16_applicable(g)) {
+    HIP_TRY(mrl::launch_gemm_bf16(g, ws.stream));
+    done = true;
+  }
+  if (!done) HIP_TRY(mrl::launch_matmul_generic(a.t, b.t, c.t, s.accum, ws.stream));
+  return finish_output(c, ws);
+}
+
+int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
+  Prepared img, filt, out;
+  int rc;
+  if ((rc = prepare(s, 0, params[0], true, ws, &img)) != MRL_OK) return rc;
+  if ((rc = prepare(s, 1, params[1], true, ws, &filt)) != MRL_OK) return rc;
+  if ((rc = prepare(s, 2, params[2], s.accum != 0, ws, &out)) != MRL_OK) return rc;
+  // NHWC / KRSC: logical [n,c,h,w] with channel fastest, then w, then h.
+  auto channels_last = [](const mrl::Strided &t) {
+    const int64_t c = t.shape[1], h = t.shape[2], w = t.shape[3];
+    (void)h;
+    return (c == 1 || t.stride[1] == 1) && (w == 1 || t.stride[3] == c) &&
+           (t.shape[2] == 1 || t.stride[2] == c * w) &&
+           (t.shape[0] == 1 || t.stride[0] == c * w * int64_t(t.shape[2]));
+  };
+  mrl::ConvArgs cv;
+  cv.image = img.t.ptr, cv.filters = filt.t.ptr, cv.out = out.t.ptr;
+  cv.b = s.spec_shape[0], cv.f = s.spec_shape[1], cv.c = s.spec_shape[2], cv.oh = s.spec_shape[3];
+  cv.ow = s.spec_shape[4], cv.fh = s.spec_shape[5], cv.fw = s.spec_shape[6];
+  cv.accum = s.accum;
+  const int di = s.dtypes[0], df = s.dtypes[1], dout = s.dtypes[2];
+  if ((di == MRL_U8 || di == MRL_I8) && df == MRL_I8 && dout == MRL_I32 && channels_last(img.t) &&
+      channels_last(filt.t) && channels_last(out.t) && mrl::conv_i8_applicable(cv)) {
+    HIP_TRY(mrl::launch_conv_i8(cv, di == MRL_U8, ws.stream));
+  } else {
+    HIP_TRY(mrl::launch_conv_generic(img.t, filt.t, out.t, s.accum, ws.stream));
+  }
+  return finish_output(out, ws);
+}
+
+int run_softmax(const mrl_spec &s, void *const *params, Workspace &ws) {
+  Prepared in, out;
+  int rc;
+  if ((rc = prepare(s, 0, params[0], true, ws, &in)) != MRL_OK) return rc;
+  if ((rc = prepare(s, 1, params[1], false, ws, &out)) != MRL_OK) return rc;
+  // Trailing size-one dims do not change which dim is innermost.
+  uint32_t last = s.rank - 1;
+  while (last > s.scan_dim && s.spec_shape[last] == 1) last--;
+  if (s.scan_dim == last && dense_row_major(in.t) && dense_row_major(out.t) &&
+      (reinterpret_cast<uintptr_t>(in.t.ptr) & 15) == 0 &&
+      (reinterpret_cast<uintptr_t>(out.t.ptr) & 15) == 0) {
+    const uint32_t cols = s.spec_shape[s.scan_dim];
+    HIP_TRY(mrl::launch_softmax_rows((const float *)in.t.ptr, (float *)out.t.ptr, in.count / cols,
+                                     cols, ws.stream));
+  } else {
+    HIP_TRY(mrl::launch_softmax_generic(in.t, out.t, s.scan_dim, ws.stream));
+  }
+  return finish_output(out, ws);
+}
+
+int run_compose_msm(const mrl_spec &s, void *const *params, Workspace &ws) {
+  Prepared v, q, kt, out;
+  int rc;
+  if ((rc = prepare(s, 0, params[0], true, ws, &v)) != MRL_OK) return rc;
+  if ((rc = prepare(s, 1, params[1], true, ws, &q)) != MRL_OK) return rc;
+  if ((rc = prepare(s, 2, params[2], true, ws, &kt)) != MRL_OK) return rc;
+  if ((rc = prepare(s, 3, params[3], false, ws, &out)) != MRL_OK) return rc;
+  const uint32_t b = s.spec_shape[0], m = s.spec_shape[1], k = s.spec_shape[2], n2 = s.spec_shape[3],
+                 n = s.spec_shape[4];
+  // Fused path: bf16 Q, V row-major and KT stored k-fastest (layout![0,2,1]).
+  const bool kt_k_fastest = (k == 1 || kt.t.stride[1] == 1) && (n2 == 1 || kt.t.stride[2] == int64_t(k)) &&
+                            (b == 1 || kt.t.stride[0] == int64_t(k) * n2);
+  mrl::AttnArgs at;
+  at.q = q.t.ptr, at.kt = kt.t.ptr, at.v = v.t.ptr, at.out = (float *)out.t.ptr;
+  at.b = b, at.m = m, at.k = k, at.n2 = n2, at.n = n;
+  if (s.dtypes[0] == MRL_BF16 && s.dtypes[1] == MRL_BF16 && s.dtypes[2] == MRL_BF16 &&
+      dense_row_major(q.t) && dense_row_major(v.t) && dense_row_major(out.t) && kt_k_fastest &&
+      mrl::attn_applicable(at)) {
+    HIP_TRY(mrl::launch_attn(at, ws.stream));
+    return finish_output(out, ws);
+  }
+  // Staged path, as the reference schedules it (examples/matmul_chain.rs:60-81): S and P
+  // live in device memory as f32 (verification.rs:239-285).
+  void *sbuf = nullptr;
+  HIP_TRY(ws.alloc(&sbuf, size_t(b) * m * n2 * sizeof(float)));
+  mrl::Strided st;
+  st.ptr = sbuf, st.dtype = MRL_F32, st.rank = 3;
+  st.shape[0] = b, st.shape[1] = m, st.shape[2] = n2, st.shape[3] = st.shape[4] = 1;
+  st.stride[0] = int64_t(m) * n2, st.stride[1] = n2, st.stride[2] = 1, st.stride[3] = st.stride[4] = 0;
+  HIP_TRY(mrl::launch_matmul_generic(q.t, kt.t, st, 0, ws.stream));
+  if ((reinterpret_cast<uintptr_t>(sbuf) & 15) == 0)
+    HIP_TRY(mrl::launch_softmax_rows((const float *)sbuf, (float *)sbuf, uint64_t(b) * m, n2, ws.stream));
+  else
+    HIP_TRY(mrl::launch_softmax_generic(st, st, 2, ws.stream));
+  HIP_TRY(mrl::launch_matmul_generic(st, v.t, out.t, 0, ws.stream));
+  return finish_output(out, ws);
+}
+
+int run_async_impl(const mrl_spec *spec, void *const *params, hipStream_t stream) {
+  if (g_device < 0) {
+    int rc = mrl_init(0);
+    if (rc != MRL_OK) return rc;
+  }
+  int rc = check_spec(spec);
+  if (rc != MRL_OK) return rc;
+  if (!params) return MRL_ERR_NULL;
+  for (uint32_t i = 0; i < spec->n_params; i++)
+    if (!params[i]) return MRL_ERR_NULL;
+  Workspace ws(stream);
+  switch (spec->kind) {
+    case MRL_SPEC_MATMUL: return run_matmul(*spec, params, ws);
+    case MRL_SPEC_CONV: return run_conv(*spec, params, ws);
+    case MRL_SPEC_SOFTMAX: return run_softmax(*spec, params, ws);
+    case MRL_SPEC_COMPOSE_MSM: return run_compose_msm(*spec, params, ws);
+    default: return MRL_ERR_UNSUPPORTED;
+  }
+}
+
+void set_conv_default_layouts(mrl_spec *s) {
+  for (uint32_t i = 0; i < 3; i++) {
+    uint32_t shape[MRL_MAX_RANK], rank;
+    parameter_shape(*s, i, shape, &rank);
+    mrl_layout_nhwc(shape, rank, &s->layouts[i]);
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int mrl_init(int device) {
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count <= 0) {
+    g_last_error = e != hipSuccess ? hipGetErrorString(e) : "no HIP device";
+    return MRL_ERR_NO_DEVICE;
+  }
+  if (device < 0 || device >= count) return MRL_ERR_NO_DEVICE;
+  hipDeviceProp_t prop;
+  HIP_TRY(hipGetDeviceProperties(&prop, device));
+  if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+    g_last_error = std::string("device is ") + prop.gcnArchName + ", kernels are built for gfx950";
+    return MRL_ERR_NO_DEVICE;
+  }
+  HIP_TRY(hipSetDevice(device));
+  g_device = device;
+  return MRL_OK;
+}
+
+const char *mrl_status_string(int status) {
+  switch (status) {
+    case MRL_OK: return "ok";
+    case MRL_ERR_UNSUPPORTED: return "unsupported Spec";
+    case MRL_ERR_BAD_LAYOUT: return "layout does not apply to the parameter shape";
+    case MRL_ERR_BAD_SPEC: return "malformed Spec descriptor";
+    case MRL_ERR_HIP: return "HIP runtime error";
+    case MRL_ERR_NO_DEVICE: return "no gfx950 device";
+    case MRL_ERR_NULL: return "null pointer";
+    case MRL_ERR_TOO_LARGE: return "tensor too large";
+    default: return "unknown status";
+  }
+}
+
+const char *mrl_last_error(void) { return g_last_error.c_str(); }
+const char *mrl_version(void) { return "0.1.0"; }
+
+size_t mrl_dtype_size(int dtype) {
+  switch (dtype) {
+    case MRL_U8: case MRL_I8: return 1;
+    case MRL_U16: case MRL_I16: case MRL_BF16: return 2;
+    case MRL_U32: case MRL_I32: case MRL_F32: return 4;
+    default: return 0;
+  }
+}
+
+const char *mrl_dtype_name(int dtype) {
+  static const char *names[] = {"u8", "i8", "u16", "i16", "u32", "i32", "f32", "bf16"};
+  return valid_dtype(dtype) ? names[dtype] : "?";
+}
+
+int mrl_layout_row_major(const uint32_t *shape, uint32_t rank, mrl_layout *out) {
+  if (!shape || !out) return MRL_ERR_NULL;
+  if (rank > MRL_MAX_RANK) return MRL_ERR_BAD_SPEC;
+  out->ndims = 0;
+  for (uint32_t d = 0; d < rank; d++) {
+    if (shape[d] == 1) continue;  // layout.rs:1234-1247 drops size-one dims
+    out->dims[out->ndims++] = mrl_physdim{uint8_t(d), MRL_DYNAMIC, 0};
+  }
+  return MRL_OK;
+}
+
+int mrl_layout_col_major(const uint32_t *shape, uint32_t rank, mrl_layout *out) {
+  int rc = mrl_layout_row_major(shape, rank, out);
+  if (rc != MRL_OK) return rc;
+  for (uint32_t i = 0; i < out->ndims / 2; i++) {
+    mrl_physdim t = out->dims[i];
+    out->dims[i] = out->dims[out->ndims - 1 - i];
+    out->dims[out->ndims - 1 - i] = t;
+  }
+  return MRL_OK;
+}
+
+int mrl_layout_batched_col_major(const uint32_t *shape, uint32_t rank, mrl_layout *out) {
+  if (!shape || !out) return MRL_ERR_NULL;
+  if (rank == 0) {
+    out->ndims = 0;
+    return MRL_OK;
+  }
+  mrl_layout inner;
+  int rc = mrl_layout_col_major(shape + 1, rank - 1, &inner);
+  if (rc != MRL_OK) return rc;
+  out->ndims = 0;
+  if (shape[0] != 1) out->dims[out->ndims++] = mrl_physdim{0, MRL_DYNAMIC, 0};
+  for (uint32_t i = 0; i < inner.ndims; i++) {
+    mrl_physdim d = inner.dims[i];
+    d.logical_dim = uint8_t(d.logical_dim + 1);
+    out->dims[out->ndims++] = d;
+  }
+  return MRL_OK;
+}
+
+int mrl_layout_nhwc(const uint32_t *shape, uint32_t rank, mrl_layout *out) {
+  if (!shape || !out) return MRL_ERR_NULL;
+  if (rank != 4) return MRL_ERR_BAD_SPEC;
+  static const uint8_t order[4] = {0, 2, 3, 1};
+  out->ndims = 0;
+  for (int i = 0; i < 4; i++)
+    if (shape[order[i]] != 1) out->dims[out->ndims++] = mrl_physdim{order[i], MRL_DYNAMIC, 0};
+  return MRL_OK;
+}
+
+int mrl_layout_physical_shape(const mrl_layout *layout, const uint32_t *shape, uint32_t rank,
+                              uint32_t *phys_shape) {
+  if (!layout || !shape || !phys_shape) return MRL_ERR_NULL;
+  return mrl::physical_shape(*layout, shape, rank, phys_shape) ? MRL_OK : MRL_ERR_BAD_LAYOUT;
+}
+
+int64_t mrl_layout_buffer_index(const mrl_layout *layout, const uint32_t *shape, uint32_t rank,
+                                const uint32_t *point) {
+  if (!layout || !shape || !point) return -1;
+  mrl::LayoutEval ev;
+  if (!mrl::make_layout_eval(*layout, shape, rank, &ev)) return -1;
+  return mrl::layout_offset(ev, point);
+}
+
+int mrl_spec_parameter_shape(const mrl_spec *spec, uint32_t idx, uint32_t *shape, uint32_t *rank) {
+  if (!spec || !shape || !rank) return MRL_ERR_NULL;
+  if (expected_params(spec->kind) == 0 || spec->rank != expected_rank(*spec)) return MRL_ERR_BAD_SPEC;
+  return parameter_shape(*spec, idx, shape, rank);
+}
+
+int mrl_spec_parameter_direction(const mrl_spec *spec, uint32_t idx) {
+  return spec ? parameter_direction(*spec, idx) : -1;
+}
+
+size_t mrl_spec_parameter_bytes(const mrl_spec *spec, uint32_t idx) {
+  uint32_t shape[MRL_MAX_RANK], rank;
+  if (mrl_spec_parameter_shape(spec, idx, shape, &rank) != MRL_OK) return 0;
+  return size_t(volume(shape, rank)) * mrl_dtype_size(spec->dtypes[idx]);
+}
+
+uint64_t mrl_spec_ops(const mrl_spec *spec) {
+  if (!spec) return 0;
+  const uint32_t *s = spec->spec_shape;
+  switch (spec->kind) {
+    case MRL_SPEC_MATMUL: return 2ull * s[0] * s[1] * s[2] * s[3];
+    case MRL_SPEC_CONV: return 2ull * s[0] * s[1] * s[2] * s[3] * s[4] * s[5] * s[6];
+    case MRL_SPEC_SOFTMAX: return 5ull * volume(s, spec->rank);
+    case MRL_SPEC_COMPOSE_MSM:
+      return 2ull * s[0] * s[1] * s[2] * s[3] + 5ull * s[0] * s[1] * s[3] + 2ull * s[0] * s[1] * s[3] * s[4];
+    default: return 0;
+  }
+}
+
+int mrl_spec_check(const mrl_spec *spec) { return check_spec(spec); }
+
+size_t mrl_spec_workspace_bytes(const mrl_spec *spec) {
+  if (check_spec(spec) != MRL_OK) return 0;
+  size_t total = 0;
+  for (uint32_t i = 0; i < spec->n_params; i++) {
+    uint32_t shape[MRL_MAX_RANK], rank;
+    int64_t strides[MRL_MAX_RANK];
+    parameter_shape(*spec, i, shape, &rank);
+    if (!mrl::layout_strides(spec->layouts[i], shape, rank, strides))
+      total += size_t(volume(shape, rank)) * mrl_dtype_size(spec->dtypes[i]);
+  }
+  return total;
+}
+
+int mrl_run_async(const mrl_spec *spec, void *const *params, void *stream) {
+  return run_async_impl(spec, params, (hipStream_t)stream);
+}
+
+int mrl_run(const mrl_spec *spec, void *const *params) {
+  int rc = run_async_impl(spec, params, nullptr);
+  if (rc != MRL_OK) return rc;
+  HIP_TRY(hipStreamSynchronize(nullptr));
+  return MRL_OK;
+}
+
+int mrl_run_host(const mrl_spec *spec, void *const *params) {
+  int rc = check_spec(spec);
+  if (rc != MRL_OK) return rc;
+  if (!params) return MRL_ERR_NULL;
+  if (g_device < 0 && (rc = mrl_init(0)) != MRL_OK) return rc;
+  void *dev[MRL_MAX_PARAMS] = {nullptr, nullptr, nullptr, nullptr};
+  auto cleanup = [&]() {
+    for (void *p : dev)
+      if (p) (void)hipFree(p);
+  };
+  for (uint32_t i = 0; i < spec->n_params; i++) {
+    if (!params[i]) {
+      cleanup();
+      return MRL_ERR_NULL;
+    }
+    const size_t bytes = mrl_spec_parameter_bytes(spec, i);
+    hipError_t e = hipMalloc(&dev[i], bytes ? bytes : 4);
+    if (e == hipSuccess && parameter_direction(*spec, i) != 1)
+      e = hipMemcpy(dev[i], params[i], bytes, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+      cleanup();
+      return hip_fail(e, "staging parameter to device");
+    }
+  }
+  rc = mrl_run(spec, dev);
+  if (rc == MRL_OK) {
+    for (uint32_t i = 0; i < spec->n_params; i++) {
+      if (parameter_direction(*spec, i) == 0) continue;
+      hipError_t e = hipMemcpy(params[i], dev[i], mrl_spec_parameter_bytes(spec, i), hipMemcpyDeviceToHost);
+      if (e != hipSuccess) {
+        cleanup();
+        return hip_fail(e, "copying output to host");
+      }
+    }
+  }
+  cleanup();
+  return rc;
+}
+
+int mrl_matmul(uint32_t b, uint32_t m, uint32_t k, uint32_t n, int dt_a, int dt_b, int dt_c, int accum,
+               const void *a, const void *bmat, void *c, void *stream) {
+  mrl_spec s;
+  std::memset(&s, 0, sizeof s);
+  s.kind = MRL_SPEC_MATMUL, s.accum = accum, s.rank = 4, s.n_params = 3;
+  s.spec_shape[0] = b, s.spec_shape[1] = m, s.spec_shape[2] = k, s.spec_shape[3] = n;
+  s.dtypes[0] = dt_a, s.dtypes[1] = dt_b, s.dtypes[2] = dt_c;
+  for (uint32_t i = 0; i < 3; i++) {
+    uint32_t shape[MRL_MAX_RANK], rank;
+    parameter_shape(s, i, shape, &rank);
+    mrl_layout_row_major(shape, rank, &s.layouts[i]);
+  }
+  void *params[3] = {const_cast<void *>(a), const_cast<void *>(bmat), c};
+  return mrl_run_async(&s, params, stream);
+}
+
+int mrl_conv(uint32_t b, uint32_t f, uint32_t c, uint32_t oh, uint32_t ow, uint32_t fh, uint32_t fw,
+             int dt_img, int dt_filt, int dt_out, int accum, const void *image, const void *filters,
+             void *out, void *stream) {
+  mrl_spec s;
+  std::memset(&s, 0, sizeof s);
+  s.kind = MRL_SPEC_CONV, s.accum = accum, s.rank = 7, s.n_params = 3;
+  const uint32_t ss[7] = {b, f, c, oh, ow, fh, fw};
+  for (int i = 0; i < 7; i++) {
+    if (ss[i] == 0) return MRL_ERR_BAD_SPEC;
+    s.spec_shape[i] = ss[i];
+  }
+  s.dtypes[0] = dt_img, s.dtypes[1] = dt_filt, s.dtypes[2] = dt_out;
+  set_conv_default_layouts(&s);
+  void *params[3] = {const_cast<void *>(image), const_cast<void *>(filters), out};
+  return mrl_run_async(&s, params, stream);
+}
+
+int mrl_softmax(const uint32_t *shape, uint32_t rank, uint32_t scan_dim, const void *in, void *out,
+                void *stream) {
+  if (!shape) return MRL_ERR_NULL;
+  if (rank == 0 || rank > MRL_MAX_RANK) return MRL_ERR_BAD_SPEC;
+  mrl_spec s;
+  std::memset(&s, 0, sizeof s);
+  s.kind = MRL_SPEC_SOFTMAX, s.scan_dim = scan_dim, s.rank = rank, s.n_params = 2;
+  for (uint32_t d = 0; d < rank; d++) s.spec_shape[d] = shape[d];
+  s.dtypes[0] = s.dtypes[1] = MRL_F32;
+  mrl_layout_row_major(shape, rank, &s.layouts[0]);
+  s.layouts[1] = s.layouts[0];
+  void *params[2] = {const_cast<void *>(in), out};
+  return mrl_run_async(&s, params, stream);
+}
+
+int mrl_compose_msm(uint32_t b, uint32_t m, uint32_t k, uint32_t n2, uint32_t n, int dt_v, int dt_q,
+                    int dt_kt, int kt_col_major, const void *v, const void *q, const void *kt,
+                    void *out, void *stream) {
+  mrl_spec s;
+  std::memset(&s, 0, sizeof s);
+  s.kind = MRL_SPEC_COMPOSE_MSM, s.rank = 5, s.n_params = 4;
+  s.spec_shape[0] = b, s.spec_shape[1] = m, s.spec_shape[2] = k, s.spec_shape[3] = n2, s.spec_shape[4] = n;
+  s.dtypes[0] = dt_v, s.dtypes[1] = dt_q, s.dtypes[2] = dt_kt, s.dtypes[3] = MRL_F32;
+  for (uint32_t i = 0; i < 4; i++) {
+    uint32_t shape[MRL_MAX_RANK], rank;
+    if (parameter_shape(s, i, shape, &rank) != MRL_OK) return MRL_ERR_BAD_SPEC;
+    if (i == 2 && kt_col_major) mrl_layout_batched_col_major(shape, rank, &s.layouts[i]);
+    else mrl_layout_row_major(shape, rank, &s.layouts[i]);
+  }
+  void *params[4] = {const_cast<void *>(v), const_cast<void *>(q), const_cast<void *>(kt), out};
+  return mrl_run_async(&s, params, stream);
+}
+
+int mrl_bench(const mrl_spec *spec, void *const *params, uint32_t iters, uint32_t repeats,
+              double *best_ns_per_iter, double *mean_ns_per_iter) {
+  if (!best_ns_per_iter || !mean_ns_per_iter) return MRL_ERR_NULL;
+  if (iters == 0 || repeats == 0) return MRL_ERR_BAD_SPEC;
+  int rc = mrl_run(spec, params);  // warm-up, as the emitted benchmark main does
+  if (rc != MRL_OK) return rc;
+  hipEvent_t t0, t1;
+  HIP_TRY(hipEventCreate(&t0));
+  HIP_TRY(hipEventCreate(&t1));
+  double best = 1e300, total = 0.0;
+  for (uint32_t r = 0; r < repeats && rc == MRL_OK; r++) {
+    (void)hipEventRecord(t0, nullptr);
+    for (uint32_t i = 0; i < iters && rc == MRL_OK; i++) rc = run_async_impl(spec, params, nullptr);
+    (void)hipEventRecord(t1, nullptr);
+    hipError_t e = hipEventSynchronize(t1);
+    if (e != hipSuccess) rc = hip_fail(e, "hipEventSynchronize");
+    float ms = 0.0f;
+    (void)hipEventElapsedTime(&ms, t0, t1);
+    const double ns = double(ms) * 1e6 / iters;
+    if (ns < best) best = ns;
+    total += ns;
+  }
+  (void)hipEventDestroy(t0);
+  (void)hipEventDestroy(t1);
+  *best_ns_per_iter = best;
+  *mean_ns_per_iter = total / repeats;
+  return rc;
+}
+
+int mrl_device_malloc(void **ptr, size_t bytes) {
+  if (!ptr) return MRL_ERR_NULL;
+  int rc;
+  if (g_device < 0 && (rc = mrl_init(0)) != MRL_OK) return rc;
+  HIP_TRY(hipMalloc(ptr, bytes ? bytes : 4));
+  return MRL_OK;
+}
+int mrl_device_free(void *ptr) {
+  HIP_TRY(hipFree(ptr));
+  return MRL_OK;
+}
+int mrl_memcpy_h2d(void *dst, const void *src, size_t bytes) {
+  HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+  return MRL_OK;
+}
+int mrl_memcpy_d2h(void *dst, const void *src, size_t bytes) {
+  HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+  return MRL_OK;
+}
+int mrl_memset(void *dst, int value, size_t bytes) {
+  HIP_TRY(hipMemset(dst, value, bytes));
+  return MRL_OK;
+}
+int mrl_device_synchronize(void) {
+  HIP_TRY(hipDeviceSynchronize());
+  return MRL_OK;
+}
+int mrl_device_info(char *name, size_t name_len, int *compute_units, int *clock_khz,
+                    size_t *total_mem_bytes) {
+  int rc;
+  if (g_device < 0 && (rc = mrl_init(0)) != MRL_OK) return rc;
+  hipDeviceProp_t prop;
+  HIP_TRY(hipGetDeviceProperties(&prop, g_device));
+  if (name && name_len) std::snprintf(name, name_len, "%s (%s)", prop.name, prop.gcnArchName);
+  if (compute_units) *compute_units = prop.multiProcessorCount;
+  if (clock_khz) *clock_khz = prop.clockRate;
+  if (total_mem_bytes) *total_mem_bytes = prop.totalGlobalMem;
+  return MRL_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,290 @@
+// Matmul on the gfx950 matrix cores: u8|i8 x i8 -> i32 (v_mfma_i32_32x32x32_i8) and
+// bf16 x bf16 -> f32 (v_mfma_f32_32x32x16_bf16), one tile pipeline for both.
+//
+// What it computes is Morello's MatmulAccum on row-major operands
+// (morello/src/spec.rs:480-485): C[i,j] (=0 unless accum) += sum_k A[i,k]*B[k,j].  The
+// integer form matches the emitted C bit for bit (widening Assign, morello/src/target/
+// cpu.rs:2860-2872, then MultAdd, morello/src/codegen/cpu.rs:2114-2124): integer addition
+// is associative, so any tiling of the sum gives the same bits.  The bf16 form widens
+// exactly (a 16-bit shift, codegen/partials/x86/cvtbf16_fp32.c) and accumulates in f32 in
+// a different order than the emitted loop nest, hence a tolerance rather than equality.
+//
+// Memory-level mapping of a Morello schedule onto this kernel:
+//   tile_out(256x256)        -> one workgroup per 256x256 tile of C
+//   split(128 bytes of K)    -> the k loop
+//   move_param(A/B, L1)      -> global -> LDS staging, double buffered
+//   move_param(A/B, VRF)     -> LDS -> MFMA operand registers: ds_read_b128 for A (rows
+//                               run along K) and the transposing ds_read_b64_tr_b8/_b16
+//                               for B (rows run along N), so no relayout pass is needed
+//   to_accum + Zero          -> accumulator registers start at zero; C is read only when
+//                               the Spec accumulates
+//
+// The int8 MFMA multiplies signed bytes.  A u8 operand is fed as a' = a xor 0x80
+// (= a - 128 as i8) and the exact correction 128 * sum_k B[k,j] is added per column in the
+// epilogue; the column sums are accumulated from the B operand registers with v_dot4.
+#include "kernels.h"
+
+namespace mrl {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef short v4s __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+
+constexpr int BM = 256, BN = 256;
+constexpr int BKB = 128;                  // bytes of K per k step, both dtypes
+constexpr int A_STAGE = BM * BKB;         // A tile: [BM][128 B], 16-byte chunks XOR-swizzled
+constexpr int B_STAGE = 36864;            // B tile: padded rows, see Traits
+constexpr int STAGE = A_STAGE + B_STAGE;  // 69632 bytes; two stages = 136 KiB of LDS
+constexpr int GROUP_M = 4;                // tile-rows per L2 group
+
+typedef __attribute__((address_space(3))) v2i lds_v2i;
+typedef __attribute__((address_space(3))) v4s lds_v4s;
+
+struct I8 {
+  typedef v16i Acc;
+  typedef int32_t Out;
+  static constexpr int ES = 1;             // element bytes
+  static constexpr int BK = BKB / ES;      // elements of K per k step
+  static constexpr int B_ROW = BN * ES + 32;  // 8 k-rows x 32 B cover all 64 banks
+  static constexpr int K_PER_READ = 8;     // k rows covered by one transposing read
+  __device__ static v2i read_tr(const uint8_t *p) {
+    return __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i *)p);
+  }
+  __device__ static Acc mfma(v4i a, v4i b, Acc c) {
+    return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+  }
+};
+struct BF16 {
+  typedef v16f Acc;
+  typedef float Out;
+  static constexpr int ES = 2;
+  static constexpr int BK = BKB / ES;
+  static constexpr int B_ROW = BN * ES + 64;  // 4 k-rows x 64 B cover all 64 banks
+  static constexpr int K_PER_READ = 4;
+  __device__ static v2i read_tr(const uint8_t *p) {
+    const v4s r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s *)p);
+    return __builtin_bit_cast(v2i, r);
+  }
+  __device__ static Acc mfma(v4i a, v4i b, Acc c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a),
+                                                   __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+  }
+};
+static_assert(I8::BK * I8::B_ROW == B_STAGE && BF16::BK * BF16::B_ROW == B_STAGE, "B stage size");
+
+template <class T, bool A_UNSIGNED, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void k_gemm(GemmArgs g, int tiles_m,
+                                                                 int tiles_n) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  constexpr int NT = 64 * WAVES_M * WAVES_N;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
+  constexpr int ES = T::ES, BK = T::BK, B_ROW = T::B_ROW;
+  constexpr int A_CH = BM * BKB / 16 / NT;       // 16-byte chunks per thread, A tile
+  constexpr int B_ROW_CH = BN * ES / 16;          // chunks per B row
+  constexpr int B_CH = BK * B_ROW_CH / NT;        // chunks per thread, B tile
+  constexpr int SLABS = BKB / 32;                 // MFMA k steps per tile (32 bytes each)
+  constexpr int K_SLAB = 32 / ES;                 // elements of K per MFMA
+  typedef typename T::Acc Acc;
+  typedef typename T::Out Out;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+  // Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous run of
+  // tiles, ordered so that a run covers a compact block of C (shared A rows and B columns
+  // stay in that XCD's L2).
+  int pid = blockIdx.x;
+  const int ntiles = tiles_m * tiles_n;
+  if (ntiles % 8 == 0) pid = (pid % 8) * (ntiles / 8) + pid / 8;
+  const int group = pid / (GROUP_M * tiles_n);
+  const int first_m = group * GROUP_M;
+  const int gsz = min(tiles_m - first_m, GROUP_M);
+  const int in_group = pid % (GROUP_M * tiles_n);
+  const int tile_m = first_m + in_group % gsz, tile_n = in_group / gsz;
+  const int64_t m0 = int64_t(tile_m) * BM, n0 = int64_t(tile_n) * BN;
+
+  const uint8_t *A = (const uint8_t *)g.a + (int64_t(blockIdx.y) * g.sa + m0 * g.lda) * ES;
+  const uint8_t *B = (const uint8_t *)g.b + (int64_t(blockIdx.y) * g.sb + n0) * ES;
+  Out *C = (Out *)g.c + int64_t(blockIdx.y) * g.sc + m0 * g.ldc + n0;
+  const int64_t lda_b = g.lda * ES, ldb_b = g.ldb * ES;
+
+  // Per-thread staging assignments (global source, LDS destination) for one k step.
+  const uint8_t *a_src[A_CH];
+  int a_dst[A_CH];
+#pragma unroll
+  for (int i = 0; i < A_CH; i++) {
+    const int id = tid + i * NT, row = id >> 3, ch = id & 7;
+    a_src[i] = A + int64_t(row) * lda_b + ch * 16;
+    a_dst[i] = row * BKB + ((ch ^ ((row >> 1) & 7)) << 4);
+  }
+  const uint8_t *b_src[B_CH];
+  int b_dst[B_CH];
+#pragma unroll
+  for (int i = 0; i < B_CH; i++) {
+    const int id = tid + i * NT, row = id / B_ROW_CH, ch = id % B_ROW_CH;
+    b_src[i] = B + int64_t(row) * ldb_b + ch * 16;
+    b_dst[i] = A_STAGE + row * B_ROW + ch * 16;
+  }
+  // Operand fragment offsets within a stage for MFMA k step 0.
+  int a_frag[TM];
+#pragma unroll
+  for (int tm = 0; tm < TM; tm++) a_frag[tm] = (wm * WM + tm * 32 + (lane & 31)) * BKB;
+  const int a_swz = ((lane & 31) >> 1) & 7;  // (row >> 1) & 7; WM and 32 are multiples of 16
+  const int a_half = lane >> 5;
+  // Transposing read: a 16-lane group fetches a K_PER_READ x 16 element block; lane p of the
+  // group supplies the address of 8 bytes of one k row, and receives the column it indexes.
+  int b_frag[TN];
+#pragma unroll
+  for (int tn = 0; tn < TN; tn++) {
+    constexpr int LANES_PER_ROW = 16 / (8 / ES);  // lanes that share one k row: 2 (i8), 4 (bf16)
+    const int p = lane & 15;
+    const int k = (K_SLAB / 2) * (lane >> 5) + p / LANES_PER_ROW;
+    const int col = wn * WN + tn * 32 + 16 * ((lane >> 4) & 1) + (8 / ES) * (p % LANES_PER_ROW);
+    b_frag[tn] = A_STAGE + k * B_ROW + col * ES;
+  }
+
+  Acc acc[TM][TN];
+#pragma unroll
+  for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[tm][tn][r] = 0;
+  int colsum[TN];
+#pragma unroll
+  for (int tn = 0; tn < TN; tn++) colsum[tn] = 0;
+
+  v4i a_reg[A_CH], b_reg[B_CH];
+  const int kt_count = int(g.k / BK);
+
+  auto load_global = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < A_CH; i++) a_reg[i] = *(const v4i *)(a_src[i] + int64_t(kt) * BKB);
+#pragma unroll
+    for (int i = 0; i < B_CH; i++) b_reg[i] = *(const v4i *)(b_src[i] + int64_t(kt) * BK * ldb_b);
+  };
+  auto store_lds = [&](int stage) {
+    uint8_t *base = lds + stage * STAGE;
+#pragma unroll
+    for (int i = 0; i < A_CH; i++) {
+      v4i v = a_reg[i];
+      if (A_UNSIGNED) v ^= v4i{int(0x80808080), int(0x80808080), int(0x80808080), int(0x80808080)};
+      *(v4i *)(base + a_dst[i]) = v;
+    }
+#pragma unroll
+    for (int i = 0; i < B_CH; i++) *(v4i *)(base + b_dst[i]) = b_reg[i];
+  };
+
+  load_global(0);
+  store_lds(0);
+  __syncthreads();
+
+  for (int kt = 0; kt < kt_count; kt++) {
+    const int cur = kt & 1;
+    const uint8_t *base = lds + cur * STAGE;
+    if (kt + 1 < kt_count) load_global(kt + 1);
+#pragma unroll
+    for (int s = 0; s < SLABS; s++) {
+      v4i af[TM], bf[TN];
+#pragma unroll
+      for (int tm = 0; tm < TM; tm++)
+        af[tm] = *(const v4i *)(base + a_frag[tm] + (((2 * s + a_half) ^ a_swz) << 4));
+#pragma unroll
+      for (int tn = 0; tn < TN; tn++) {
+        const v2i lo = T::read_tr(base + b_frag[tn] + (s * K_SLAB) * B_ROW);
+        const v2i hi = T::read_tr(base + b_frag[tn] + (s * K_SLAB + T::K_PER_READ) * B_ROW);
+        bf[tn] = v4i{lo[0], lo[1], hi[0], hi[1]};
+      }
+      if (A_UNSIGNED && (s % WAVES_M) == wm) {
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+          for (int w = 0; w < 4; w++)
+            colsum[tn] = __builtin_amdgcn_sdot4(bf[tn][w], 0x01010101, colsum[tn], false);
+      }
+#pragma unroll
+      for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++) acc[tm][tn] = T::mfma(af[tm], bf[tn], acc[tm][tn]);
+    }
+    if (kt + 1 < kt_count) store_lds(cur ^ 1);
+    __syncthreads();
+  }
+
+  // Epilogue.  Column sums: each (wave-row, k-half) pair holds a partial for its columns.
+  int corr[TN];
+#pragma unroll
+  for (int tn = 0; tn < TN; tn++) corr[tn] = 0;
+  if (A_UNSIGNED) {
+    int *part = (int *)lds;  // [WAVES_M * 2][BN]
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++)
+      part[(wm * 2 + (lane >> 5)) * BN + wn * WN + tn * 32 + (lane & 31)] = colsum[tn];
+    __syncthreads();
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++) {
+      int s = 0;
+#pragma unroll
+      for (int w = 0; w < WAVES_M * 2; w++) s += part[w * BN + wn * WN + tn * 32 + (lane & 31)];
+      corr[tn] = s * 128;
+    }
+  }
+#pragma unroll
+  for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int row = wm * WM + tm * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+        const int col = wn * WN + tn * 32 + (lane & 31);
+        Out *dst = C + int64_t(row) * g.ldc + col;
+        Out v = acc[tm][tn][r];
+        if (A_UNSIGNED) v += Out(corr[tn]);
+        if (g.accum) v += *dst;
+        *dst = v;
+      }
+}
+
+template <class T, bool A_UNSIGNED>
+hipError_t launch(const GemmArgs &g, hipStream_t stream) {
+  auto kern = k_gemm<T, A_UNSIGNED, 2, 4>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void *)kern,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 2 * STAGE);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  const int tiles_m = int(g.m / BM), tiles_n = int(g.n / BN);
+  hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n, g.batch), dim3(512), 2 * STAGE, stream, g,
+                     tiles_m, tiles_n);
+  return hipGetLastError();
+}
+
+bool applicable(const GemmArgs &g, int es) {
+  auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  const int64_t per16 = 16 / es;
+  return g.m && g.n && g.k && g.m % BM == 0 && g.n % BN == 0 && g.k % (BKB / es) == 0 &&
+         g.lda % per16 == 0 && g.ldb % per16 == 0 && g.sa % per16 == 0 && g.sb % per16 == 0 &&
+         al16(g.a) && al16(g.b) && (reinterpret_cast<uintptr_t>(g.c) & 3) == 0 &&
+         g.batch <= 65535 && uint64_t(g.m / BM) * (g.n / BN) < (1u << 30);
+}
+
+}  // namespace
+
+bool gemm_i8_applicable(const GemmArgs &g, bool b_k_contiguous) {
+  return !b_k_contiguous && applicable(g, 1);
+}
+hipError_t launch_gemm_i8(const GemmArgs &g, bool a_unsigned, hipStream_t stream) {
+  return a_unsigned ? launch<I8, true>(g, stream) : launch<I8, false>(g, stream);
+}
+bool gemm_bf16_applicable(const GemmArgs &g) { return applicable(g, 2); }
+hipError_t launch_gemm_bf16(const GemmArgs &g, hipStream_t stream) {
+  return launch<BF16, false>(g, stream);
+}
+
+}  // namespace mrl

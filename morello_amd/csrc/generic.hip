@@ -1,0 +1,312 @@
+// Correctness-first kernels: any dtype combination, any strides, any size.  The MFMA
+// kernels cover the shapes that matter for throughput; everything else lands here so that
+// every Spec the descriptor can express still runs on the GPU.
+//
+// Arithmetic follows the reference's oracle (morello/src/verification.rs:115-134,
+// 547-569, 603-643): both inputs are converted to the output dtype, then multiplied and
+// accumulated in that dtype.  Integer outputs are computed modulo 2^32 and truncated on
+// store, which equals wrapping arithmetic in the narrower type.
+#include "kernels.h"
+
+namespace mrl {
+namespace {
+
+__device__ inline float bf16_bits_to_f32(uint16_t v) { return __uint_as_float(uint32_t(v) << 16); }
+
+__device__ inline uint32_t narrow_int(int dtype, uint32_t v) {
+  switch (dtype) {
+    case MRL_U8: return v & 0xffu;
+    case MRL_I8: return uint32_t(int32_t(int8_t(uint8_t(v))));
+    case MRL_U16: return v & 0xffffu;
+    case MRL_I16: return uint32_t(int32_t(int16_t(uint16_t(v))));
+    default: return v;
+  }
+}
+
+__device__ inline float load_f32(const void *p, int dtype, int64_t off) {
+  switch (dtype) {
+    case MRL_U8: return float(((const uint8_t *)p)[off]);
+    case MRL_I8: return float(((const int8_t *)p)[off]);
+    case MRL_U16: return float(((const uint16_t *)p)[off]);
+    case MRL_I16: return float(((const int16_t *)p)[off]);
+    case MRL_U32: return float(((const uint32_t *)p)[off]);
+    case MRL_I32: return float(((const int32_t *)p)[off]);
+    case MRL_F32: return ((const float *)p)[off];
+    default: return bf16_bits_to_f32(((const uint16_t *)p)[off]);
+  }
+}
+
+// Rust `as` semantics: integers wrap, floats saturate and NaN becomes 0.
+__device__ inline uint32_t load_u32(const void *p, int dtype, int64_t off, int out_dtype) {
+  uint32_t v;
+  switch (dtype) {
+    case MRL_U8: v = ((const uint8_t *)p)[off]; break;
+    case MRL_I8: v = uint32_t(int32_t(((const int8_t *)p)[off])); break;
+    case MRL_U16: v = ((const uint16_t *)p)[off]; break;
+    case MRL_I16: v = uint32_t(int32_t(((const int16_t *)p)[off])); break;
+    case MRL_U32: v = ((const uint32_t *)p)[off]; break;
+    case MRL_I32: v = uint32_t(((const int32_t *)p)[off]); break;
+    default: {
+      const float f = load_f32(p, dtype, off);
+      const bool sgn = out_dtype == MRL_I8 || out_dtype == MRL_I16 || out_dtype == MRL_I32;
+      if (f != f) v = 0;
+      else if (sgn) v = f <= -2147483648.0f ? 0x80000000u : f >= 2147483648.0f ? 0x7fffffffu : uint32_t(int32_t(f));
+      else v = f <= 0.0f ? 0u : f >= 4294967296.0f ? 0xffffffffu : uint32_t(f);
+    }
+  }
+  return narrow_int(out_dtype, v);
+}
+
+__device__ inline void store_u32(void *p, int dtype, int64_t off, uint32_t v) {
+  switch (dtype) {
+    case MRL_U8: case MRL_I8: ((uint8_t *)p)[off] = uint8_t(v); break;
+    case MRL_U16: case MRL_I16: ((uint16_t *)p)[off] = uint16_t(v); break;
+    default: ((uint32_t *)p)[off] = v; break;
+  }
+}
+
+// ------------------------------------------------------------------ relayout
+__global__ void k_relayout(const uint8_t *src, uint8_t *dst, LayoutEval sl, LayoutEval dl,
+                           uint32_t es, uint64_t count) {
+  const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  uint32_t pt[MRL_MAX_RANK];
+  uint64_t rem = i;
+  for (int d = int(sl.rank) - 1; d >= 0; d--) {
+    pt[d] = uint32_t(rem % sl.shape[d]);
+    rem /= sl.shape[d];
+  }
+  const int64_t so = layout_offset(sl, pt), d_o = layout_offset(dl, pt);
+  if (es == 1) dst[d_o] = src[so];
+  else if (es == 2) ((uint16_t *)dst)[d_o] = ((const uint16_t *)src)[so];
+  else ((uint32_t *)dst)[d_o] = ((const uint32_t *)src)[so];
+}
+
+// -------------------------------------------------------------------- matmul
+struct MM {
+  const void *a, *b;
+  void *c;
+  int dta, dtb, dtc;
+  uint32_t B, M, K, N;
+  int64_t sa[3], sb[3], sc[3];
+  int accum;
+};
+
+template <bool FLOAT_OUT>
+__global__ __launch_bounds__(256) void k_matmul_generic(MM p) {
+  __shared__ uint32_t ta[16][17], tb[16][17];
+  const uint32_t tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+  const uint32_t j = blockIdx.x * 16 + tx, i = blockIdx.y * 16 + ty, bi = blockIdx.z;
+  const bool live = i < p.M && j < p.N;
+  const int64_t coff = int64_t(bi) * p.sc[0] + int64_t(i) * p.sc[1] + int64_t(j) * p.sc[2];
+  float facc = 0.0f;
+  uint32_t iacc = 0;
+  if (p.accum && live) {
+    if (FLOAT_OUT) facc = ((const float *)p.c)[coff];
+    else iacc = load_u32(p.c, p.dtc, coff, MRL_U32);
+  }
+  for (uint32_t k0 = 0; k0 < p.K; k0 += 16) {
+    {  // A tile: row i, col k0+tx ; B tile: row k0+ty, col j
+      const uint32_t ka = k0 + tx, kb = k0 + ty;
+      uint32_t av = 0, bv = 0;
+      if (i < p.M && ka < p.K) {
+        const int64_t o = int64_t(bi) * p.sa[0] + int64_t(i) * p.sa[1] + int64_t(ka) * p.sa[2];
+        av = FLOAT_OUT ? __float_as_uint(load_f32(p.a, p.dta, o)) : load_u32(p.a, p.dta, o, p.dtc);
+      }
+      if (kb < p.K && j < p.N) {
+        const int64_t o = int64_t(bi) * p.sb[0] + int64_t(kb) * p.sb[1] + int64_t(j) * p.sb[2];
+        bv = FLOAT_OUT ? __float_as_uint(load_f32(p.b, p.dtb, o)) : load_u32(p.b, p.dtb, o, p.dtc);
+      }
+      ta[ty][tx] = av;
+      tb[ty][tx] = bv;
+    }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t kk = 0; kk < 16; kk++) {
+      if (FLOAT_OUT) facc += __uint_as_float(ta[ty][kk]) * __uint_as_float(tb[kk][tx]);
+      else iacc += ta[ty][kk] * tb[kk][tx];
+    }
+    __syncthreads();
+  }
+  if (live) {
+    if (FLOAT_OUT) ((float *)p.c)[coff] = facc;
+    else store_u32(p.c, p.dtc, coff, iacc);
+  }
+}
+
+// ---------------------------------------------------------------------- conv
+struct CV {
+  const void *img, *filt;
+  void *out;
+  int dti, dtf, dto;
+  uint32_t B, F, C, OH, OW, FH, FW;
+  int64_t si[4], sf[4], so[4];
+  int accum;
+};
+
+template <bool FLOAT_OUT>
+__global__ __launch_bounds__(256) void k_conv_generic(CV p) {
+  const uint64_t total = uint64_t(p.B) * p.F * p.OH * p.OW;
+  const uint64_t idx = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  // Decode with f fastest so that NHWC outputs are written contiguously.
+  uint64_t r = idx;
+  const uint32_t f = uint32_t(r % p.F); r /= p.F;
+  const uint32_t x = uint32_t(r % p.OW); r /= p.OW;
+  const uint32_t y = uint32_t(r % p.OH); r /= p.OH;
+  const uint32_t b = uint32_t(r);
+  const int64_t ooff = b * p.so[0] + f * p.so[1] + y * p.so[2] + x * p.so[3];
+  float facc = 0.0f;
+  uint32_t iacc = 0;
+  if (p.accum) {
+    if (FLOAT_OUT) facc = ((const float *)p.out)[ooff];
+    else iacc = load_u32(p.out, p.dto, ooff, MRL_U32);
+  }
+  for (uint32_t c = 0; c < p.C; c++)
+    for (uint32_t rr = 0; rr < p.FH; rr++)
+      for (uint32_t s = 0; s < p.FW; s++) {
+        const int64_t io = b * p.si[0] + c * p.si[1] + int64_t(y + rr) * p.si[2] + int64_t(x + s) * p.si[3];
+        const int64_t fo = f * p.sf[0] + c * p.sf[1] + rr * p.sf[2] + s * p.sf[3];
+        if (FLOAT_OUT) facc += load_f32(p.img, p.dti, io) * load_f32(p.filt, p.dtf, fo);
+        else iacc += load_u32(p.img, p.dti, io, p.dto) * load_u32(p.filt, p.dtf, fo, p.dto);
+      }
+  if (FLOAT_OUT) ((float *)p.out)[ooff] = facc;
+  else store_u32(p.out, p.dto, ooff, iacc);
+}
+
+// ------------------------------------------------------------------- softmax
+// One wavefront per line along an arbitrary-stride scan dim: max, then exp and sum, then
+// divide (morello/src/verification.rs:166-184).
+struct SM {
+  const float *in;
+  float *out;
+  uint32_t rank, scan_dim;
+  uint32_t shape[MRL_MAX_RANK];
+  int64_t si[MRL_MAX_RANK], so[MRL_MAX_RANK];
+  uint64_t lines;
+};
+
+__device__ inline float wave_max(float v) {
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+  return v;
+}
+__device__ inline float wave_sum(float v) {
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+
+__global__ __launch_bounds__(256) void k_softmax_generic(SM p) {
+  const uint64_t line = uint64_t(blockIdx.x) * 4 + threadIdx.x / 64;
+  const uint32_t lane = threadIdx.x % 64;
+  if (line >= p.lines) return;
+  uint64_t r = line;
+  int64_t ibase = 0, obase = 0;
+  for (int d = int(p.rank) - 1; d >= 0; d--) {
+    if (uint32_t(d) == p.scan_dim) continue;
+    const uint32_t c = uint32_t(r % p.shape[d]);
+    r /= p.shape[d];
+    ibase += c * p.si[d];
+    obase += c * p.so[d];
+  }
+  const uint32_t n = p.shape[p.scan_dim];
+  const int64_t is = p.si[p.scan_dim], os = p.so[p.scan_dim];
+  float mx = -3.40282347e+38f;
+  bool nan = false;
+  for (uint32_t i = lane; i < n; i += 64) {
+    const float v = p.in[ibase + i * is];
+    nan |= v != v;
+    mx = fmaxf(mx, v);
+  }
+  mx = wave_max(mx);
+  if (__any(nan)) mx = __uint_as_float(0x7fc00000u);
+  float sum = 0.0f;
+  for (uint32_t i = lane; i < n; i += 64) {
+    const float e = expf(p.in[ibase + i * is] - mx);
+    p.out[obase + i * os] = e;
+    sum += e;
+  }
+  sum = wave_sum(sum);
+  for (uint32_t i = lane; i < n; i += 64) p.out[obase + i * os] /= sum;
+}
+
+__global__ void k_fill_zero(uint32_t *p, uint64_t words, uint8_t *tail, uint32_t tail_bytes) {
+  const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  const uint64_t step = uint64_t(gridDim.x) * blockDim.x;
+  for (uint64_t w = i; w < words; w += step) p[w] = 0;
+  if (i < tail_bytes) tail[i] = 0;
+}
+
+bool float_out(int dt) { return dt == MRL_F32; }
+
+}  // namespace
+
+hipError_t launch_relayout(const void *src, void *dst, const LayoutEval &sl, const LayoutEval &dl,
+                           uint32_t es, uint64_t count, hipStream_t stream) {
+  if (count == 0) return hipSuccess;
+  const uint32_t blocks = uint32_t((count + 255) / 256);
+  hipLaunchKernelGGL(k_relayout, dim3(blocks), dim3(256), 0, stream, (const uint8_t *)src,
+                     (uint8_t *)dst, sl, dl, es, count);
+  return hipGetLastError();
+}
+
+hipError_t launch_matmul_generic(const Strided &a, const Strided &b, const Strided &c, int accum,
+                                 hipStream_t stream) {
+  MM p;
+  p.a = a.ptr, p.b = b.ptr, p.c = c.ptr;
+  p.dta = a.dtype, p.dtb = b.dtype, p.dtc = c.dtype;
+  p.B = a.shape[0], p.M = a.shape[1], p.K = a.shape[2], p.N = b.shape[2];
+  for (int d = 0; d < 3; d++) p.sa[d] = a.stride[d], p.sb[d] = b.stride[d], p.sc[d] = c.stride[d];
+  p.accum = accum;
+  dim3 grid((p.N + 15) / 16, (p.M + 15) / 16, p.B);
+  if (float_out(c.dtype)) hipLaunchKernelGGL(k_matmul_generic<true>, grid, dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL(k_matmul_generic<false>, grid, dim3(256), 0, stream, p);
+  return hipGetLastError();
+}
+
+hipError_t launch_conv_generic(const Strided &img, const Strided &filt, const Strided &out,
+                               int accum, hipStream_t stream) {
+  CV p;
+  p.img = img.ptr, p.filt = filt.ptr, p.out = out.ptr;
+  p.dti = img.dtype, p.dtf = filt.dtype, p.dto = out.dtype;
+  p.B = out.shape[0], p.F = out.shape[1], p.OH = out.shape[2], p.OW = out.shape[3];
+  p.C = filt.shape[1], p.FH = filt.shape[2], p.FW = filt.shape[3];
+  for (int d = 0; d < 4; d++) p.si[d] = img.stride[d], p.sf[d] = filt.stride[d], p.so[d] = out.stride[d];
+  p.accum = accum;
+  const uint64_t total = uint64_t(p.B) * p.F * p.OH * p.OW;
+  const uint32_t blocks = uint32_t((total + 255) / 256);
+  if (float_out(out.dtype)) hipLaunchKernelGGL(k_conv_generic<true>, dim3(blocks), dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL(k_conv_generic<false>, dim3(blocks), dim3(256), 0, stream, p);
+  return hipGetLastError();
+}
+
+hipError_t launch_softmax_generic(const Strided &in, const Strided &out, uint32_t scan_dim,
+                                  hipStream_t stream) {
+  SM p;
+  p.in = (const float *)in.ptr, p.out = (float *)out.ptr;
+  p.rank = in.rank, p.scan_dim = scan_dim;
+  uint64_t lines = 1;
+  for (uint32_t d = 0; d < MRL_MAX_RANK; d++) {
+    p.shape[d] = d < in.rank ? in.shape[d] : 1;
+    p.si[d] = d < in.rank ? in.stride[d] : 0;
+    p.so[d] = d < in.rank ? out.stride[d] : 0;
+    if (d < in.rank && d != scan_dim) lines *= in.shape[d];
+  }
+  p.lines = lines;
+  const uint32_t blocks = uint32_t((lines + 3) / 4);
+  hipLaunchKernelGGL(k_softmax_generic, dim3(blocks), dim3(256), 0, stream, p);
+  return hipGetLastError();
+}
+
+hipError_t launch_fill_zero(void *ptr, uint64_t bytes, hipStream_t stream) {
+  if (bytes == 0) return hipSuccess;
+  const uint64_t words = bytes / 4;
+  const uint32_t tail = uint32_t(bytes % 4);
+  uint64_t blocks = (words + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  if (blocks == 0) blocks = 1;
+  hipLaunchKernelGGL(k_fill_zero, dim3(uint32_t(blocks)), dim3(256), 0, stream, (uint32_t *)ptr,
+                     words, (uint8_t *)ptr + words * 4, tail);
+  return hipGetLastError();
+}
+
+}  // namespace mrl

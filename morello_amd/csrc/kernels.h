@@ -1,0 +1,75 @@
+// Internal interface between the host dispatcher and the kernel translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "layout_math.h"
+
+namespace mrl {
+
+// A tensor whose layout is a pure permutation of its logical dims.
+struct Strided {
+  void *ptr;
+  int dtype;
+  uint32_t rank;
+  uint32_t shape[MRL_MAX_RANK];
+  int64_t stride[MRL_MAX_RANK];  // in elements
+};
+
+// ---- generic.hip: correctness-first kernels for any dtype / stride combination ----------
+hipError_t launch_relayout(const void *src, void *dst, const LayoutEval &src_l,
+                           const LayoutEval &dst_l, uint32_t elem_size, uint64_t count,
+                           hipStream_t stream);
+hipError_t launch_matmul_generic(const Strided &a, const Strided &b, const Strided &c, int accum,
+                                 hipStream_t stream);
+hipError_t launch_conv_generic(const Strided &img, const Strided &filt, const Strided &out,
+                               int accum, hipStream_t stream);
+hipError_t launch_softmax_generic(const Strided &in, const Strided &out, uint32_t scan_dim,
+                                  hipStream_t stream);
+hipError_t launch_fill_zero(void *ptr, uint64_t bytes, hipStream_t stream);
+
+// ---- gemm_i8.hip: u8|i8 x i8 -> i32 on the int8 MFMA -----------------------------------
+// Row-major operands with leading dimensions in elements; batch strides in elements.
+struct GemmArgs {
+  const void *a;
+  const void *b;
+  void *c;
+  uint32_t batch, m, n, k;
+  int64_t lda, ldb, ldc;
+  int64_t sa, sb, sc;  // batch strides
+  int accum;
+};
+bool gemm_i8_applicable(const GemmArgs &g, bool b_k_contiguous);
+hipError_t launch_gemm_i8(const GemmArgs &g, bool a_unsigned, hipStream_t stream);
+
+// ---- gemm_bf16.hip: bf16 x bf16 -> f32 on the bf16 MFMA --------------------------------
+bool gemm_bf16_applicable(const GemmArgs &g);
+hipError_t launch_gemm_bf16(const GemmArgs &g, hipStream_t stream);
+
+// ---- conv_i8.hip: NHWC u8|i8 image x KRSC i8 filters -> NHWC i32, implicit GEMM --------
+struct ConvArgs {
+  const void *image;
+  const void *filters;
+  void *out;
+  uint32_t b, f, c, oh, ow, fh, fw;
+  int accum;
+};
+bool conv_i8_applicable(const ConvArgs &c);
+hipError_t launch_conv_i8(const ConvArgs &c, bool img_unsigned, hipStream_t stream);
+
+// ---- softmax.hip: f32 softmax over a contiguous innermost scan dim ---------------------
+hipError_t launch_softmax_rows(const float *in, float *out, uint64_t rows, uint32_t cols,
+                               hipStream_t stream);
+
+// ---- attention.hip: fused Matmul -> Softmax -> Matmul on bf16 inputs -------------------
+struct AttnArgs {
+  const void *q;   // [b, m, k]   bf16 row-major
+  const void *kt;  // logical [b, k, n2] stored as [b, n2, k] (K row-major)
+  const void *v;   // [b, n2, n]  bf16 row-major
+  float *out;      // [b, m, n]   f32 row-major
+  uint32_t b, m, k, n2, n;
+};
+bool attn_applicable(const AttnArgs &a);
+hipError_t launch_attn(const AttnArgs &a, hipStream_t stream);
+
+}  // namespace mrl
