@@ -191,6 +191,13 @@ int mrl_compose_msm(uint32_t b, uint32_t m, uint32_t k, uint32_t n2, uint32_t n,
 int mrl_bench(const mrl_spec *spec, void *const *params, uint32_t iters, uint32_t repeats,
               double *best_ns_per_iter, double *mean_ns_per_iter);
 
+/* Enqueues `steps` launches of the Spec back to back on the default stream, bracketed by
+ * two HIP events recorded on that same stream, waits, and writes the elapsed device time
+ * for all of them in milliseconds.  The timed region of the benchmark's inner loop
+ * (codegen/cpu.rs:541-550) measured on the device's clock. */
+int mrl_run_timed(const mrl_spec *spec, void *const *params, uint32_t steps,
+                  double *device_ms_total);
+
 /* ------------------------------------------- device memory (plumbing only) */
 
 int mrl_device_malloc(void **ptr, size_t bytes);

@@ -261,6 +261,13 @@ class Spec:
         arr = (C.c_void_p * len(arrays))(*[a.ctypes.data for a in arrays])
         _check(B.load().mrl_run_host(C.byref(self._c), arr), "mrl_run_host")
 
+    def run_timed(self, ptrs: Sequence[int], steps: int) -> float:
+        """`steps` back-to-back launches between two HIP events; total device milliseconds."""
+        arr = (C.c_void_p * len(ptrs))(*ptrs)
+        ms = C.c_double()
+        _check(B.load().mrl_run_timed(C.byref(self._c), arr, steps, C.byref(ms)), "mrl_run_timed")
+        return ms.value
+
     def bench(self, ptrs: Sequence[int], iters: int, repeats: int = 10):
         """CodeGen::bench protocol (codegen/mod.rs:133-169): (best, mean) ns per launch."""
         arr = (C.c_void_p * len(ptrs))(*ptrs)

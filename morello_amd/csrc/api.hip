@@ -667,6 +667,29 @@ int mrl_bench(const mrl_spec *spec, void *const *params, uint32_t iters, uint32_
   return rc;
 }
 
+int mrl_run_timed(const mrl_spec *spec, void *const *params, uint32_t steps,
+                  double *device_ms_total) {
+  if (!device_ms_total) return MRL_ERR_NULL;
+  if (steps == 0) return MRL_ERR_BAD_SPEC;
+  int rc = check_spec(spec);
+  if (rc != MRL_OK) return rc;
+  hipEvent_t t0, t1;
+  HIP_TRY(hipEventCreate(&t0));
+  HIP_TRY(hipEventCreate(&t1));
+  (void)hipEventRecord(t0, nullptr);
+  for (uint32_t i = 0; i < steps && rc == MRL_OK; i++) rc = run_async_impl(spec, params, nullptr);
+  (void)hipEventRecord(t1, nullptr);
+  hipError_t e = hipEventSynchronize(t1);
+  float ms = 0.0f;
+  if (e == hipSuccess) e = hipEventElapsedTime(&ms, t0, t1);
+  (void)hipEventDestroy(t0);
+  (void)hipEventDestroy(t1);
+  if (rc != MRL_OK) return rc;
+  if (e != hipSuccess) return hip_fail(e, "event timing");
+  *device_ms_total = double(ms);
+  return MRL_OK;
+}
+
 int mrl_device_malloc(void **ptr, size_t bytes) {
   if (!ptr) return MRL_ERR_NULL;
   int rc;

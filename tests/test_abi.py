@@ -1,0 +1,93 @@
+"""The C-ABI library loads and exports every symbol the header declares, and the host-side
+Spec surface answers as the reference's does.  No compute, no GPU."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+import morello_amd as M
+from morello_amd import _binding as B
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "morello_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mrl_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    lib = B.load()
+    names = declared_functions()
+    assert len(names) >= 30
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in the header but not exported"
+        assert n in B.SIGNATURES, f"{n} has no ctypes signature"
+    assert set(B.SIGNATURES) <= set(names)
+
+
+def test_struct_sizes_match_the_header():
+    # mrl_physdim {u8,u8,u32} = 8 bytes; mrl_layout = 4 + 10*8; mrl_spec as declared.
+    assert C.sizeof(B.PhysDimC) == 8
+    assert C.sizeof(B.LayoutC) == 84
+    assert C.sizeof(B.SpecC) == 4 * 4 + 7 * 4 + 4 + 4 * 4 + 4 * 84
+
+
+def test_parameter_shapes_and_directions():
+    # spec.rs:480-498, :523-526 and the Conv expectation of spec.rs:3788-3826
+    mm = M.Matmul([32, 2, 3, 3], [M.u8, M.i8, M.u16], accum=True)  # spec.rs:3663-3698
+    assert mm.parameter_shapes() == [[32, 2, 3], [32, 3, 3], [32, 2, 3]]
+    assert mm.operand_directions() == [M.OperandDirection.In, M.OperandDirection.In, M.OperandDirection.InOut]
+    assert M.Matmul([1, 2, 3, 4], [M.f32] * 3).operand_directions()[2] == M.OperandDirection.Out
+    cv = M.Conv([1, 2, 3, 4, 5, 2, 2], [M.u8, M.i8, M.i32])
+    assert cv.parameter_shapes() == [[1, 3, 5, 6], [2, 3, 2, 2], [1, 2, 4, 5]]
+    sm = M.Softmax([4, 8, 16], 2)
+    assert sm.parameter_shapes() == [[4, 8, 16]] * 2
+    assert sm.operand_directions() == [M.OperandDirection.In, M.OperandDirection.Out]
+    # Compose parameters: head's rhs, then the innermost Matmul's lhs and rhs, then the
+    # output (spec.rs:3329-3365, test_compose_parameters spec.rs:3733-3785).
+    cm = M.ComposeMSM(16, 2048, 128, 2048, 128)
+    assert cm.parameter_shapes() == [[16, 2048, 128], [16, 2048, 128], [16, 128, 2048], [16, 2048, 128]]
+    assert [int(d) for d in cm.operand_directions()] == [0, 0, 0, 1]
+    assert cm.bytes_used(0) == 16 * 2048 * 128 * 2 and cm.bytes_used(3) == 16 * 2048 * 128 * 4
+
+
+def test_flops_convention():
+    # spec.rs:273-305: Matmul 2*b*m*k*n, Softmax 5*volume
+    assert M.Matmul([1, 4096, 4096, 4096], [M.u8, M.i8, M.i32]).flops() == 137438953472
+    assert M.Matmul([1, 8192, 8192, 8192], [M.bf16, M.bf16, M.f32]).flops() == 1099511627776
+    assert M.Conv([32, 64, 64, 54, 54, 3, 3], [M.u8, M.i8, M.i32]).flops() == 6879707136
+    assert M.Softmax([16, 2048, 2048], 2).flops() == 335544320
+    assert M.ComposeMSM(16, 2048, 128, 2048, 128).flops() == 34359738368 + 335544320
+
+
+def test_spec_check_status_codes():
+    assert M.Matmul([1, 64, 64, 64], [M.f32] * 3).check() == 0
+    assert M.Matmul([1, 64, 0, 64], [M.f32] * 3).check() == 3          # zero dim
+    assert M.Spec(M.SpecKind.Matmul, [1, 2, 3], [M.f32] * 3, layouts=[M.Layout([])] * 3).check() == 3  # rank
+    assert M.Matmul([1, 4, 4, 4], [M.f32, M.f32, M.bf16]).check() == 1  # bf16 output
+    assert M.Softmax([4, 4], 2).check() == 3                              # scan_dim out of range
+    bad = M.layout((0, M.Packed(4)), 1)                                   # layout.rs:1520-1527
+    assert M.Matmul([1, 8, 64, 64], [M.f32] * 3,
+                    layouts=[M.Layout([(1, M.Packed(4)), (2, M.Dynamic)]), None, None]).check() == 2
+    assert bad.applies_to_shape([1, 64]) and not bad.applies_to_shape([8, 64])
+    assert M.Spec(M.SpecKind.Softmax, [4, 4], [M.u8, M.u8], scan_dim=1).check() == 1
+    assert M.Matmul([1, 65536, 65536, 2], [M.u8, M.i8, M.i32]).check() == 7  # > i32 index range
+
+
+def test_workspace_only_for_non_strided_layouts():
+    assert M.Matmul([1, 64, 64, 64], [M.f32] * 3).workspace_bytes() == 0
+    assert M.Conv([1, 8, 8, 4, 4, 3, 3], [M.u8, M.i8, M.i32]).workspace_bytes() == 0
+    packed = M.layout(0, 2, 1, (2, M.Packed(16)))  # examples/matmul_x86.rs:34-53 style relayout
+    s = M.Matmul([1, 64, 64, 64], [M.f32] * 3, layouts=[None, packed, None])
+    assert s.workspace_bytes() == 64 * 64 * 4
+
+
+def test_null_and_status_strings():
+    lib = B.load()
+    assert lib.mrl_run(None, None) in (5, 6)  # no device here, or NULL spec
+    assert lib.mrl_status_string(0) == b"ok"
+    assert lib.mrl_status_string(2).startswith(b"layout")
+    assert lib.mrl_version().count(b".") == 2

@@ -1,0 +1,196 @@
+"""Matmul Spec on the MI355X against the CPU oracle, through the C ABI.
+
+Integer Specs must match bit for bit; bf16-in/f32-accumulate within 1e-2 relative (measured
+far tighter); f32 within 1e-5 relative, and exactly on the reference's integer-valued check
+inputs (verification.rs:893-952).
+"""
+import numpy as np
+import pytest
+
+import morello_amd as M
+import orc
+from gpu_util import rel_err, run_spec
+from morello_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+GEN = {M.u8: synth.uniform_u8, M.i8: synth.uniform_i8}
+
+
+def int_inputs(seed, dts, b, m, k, n, accum):
+    A = GEN[dts[0]](seed, 0, (b, m, k))
+    Bm = GEN[dts[1]](seed, 1, (b, k, n))
+    C0 = (synth.uniform_u8(seed, 2, (b, m, n)).astype(np.int32) * 1000 - 99) if accum else np.zeros((b, m, n), np.int32)
+    return A, Bm, C0
+
+
+@pytest.mark.parametrize("dts", [(M.u8, M.i8, M.i32), (M.i8, M.i8, M.i32)])
+@pytest.mark.parametrize("shape,accum", [
+    ((1, 64, 64, 64), False),       # below the MFMA tile: generic kernel
+    ((1, 256, 128, 256), False),    # exactly one MFMA tile, one k step
+    ((1, 256, 256, 256), True),
+    ((1, 512, 384, 768), False),    # several tiles, odd tile counts
+    ((3, 256, 256, 512), True),     # batched
+    ((1, 1024, 1024, 1024), True),
+    ((1, 100, 37, 51), True),       # ragged: generic kernel
+    ((1, 1, 1, 1), False),
+])
+def test_int8_matmul_bit_exact(gpu, dts, shape, accum):
+    b, m, k, n = shape
+    A, Bm, C0 = int_inputs(11, dts, b, m, k, n, accum)
+    got = run_spec(M.Matmul(shape, dts, accum=accum), [A, Bm, C0])
+    want = orc.matmul(list(shape), [int(d) for d in dts], A, Bm, C0.copy(), accum)
+    assert np.array_equal(got, want)
+
+
+def test_int8_matmul_extremes(gpu):
+    """All-255 times all-(-128): every partial sum sits on the no-overflow bound, and the
+    u8 -> signed correction term is at its largest."""
+    m, k, n = 256, 4096, 256
+    A = np.full((1, m, k), 255, np.uint8)
+    Bm = np.full((1, k, n), -128, np.int8)
+    got = run_spec(M.Matmul([1, m, k, n], (M.u8, M.i8, M.i32)), [A, Bm, np.zeros((1, m, n), np.int32)])
+    assert (got == -133693440).all()
+    Bm = np.full((1, k, n), 127, np.int8)
+    got = run_spec(M.Matmul([1, m, k, n], (M.u8, M.i8, M.i32)), [A, Bm, np.zeros((1, m, n), np.int32)])
+    assert (got == 255 * 127 * k).all()
+
+
+def test_int8_matmul_reference_check_pattern(gpu):
+    """The reference's own check inputs: counting ints in every parameter, output included."""
+    b, m, k, n = 1, 256, 256, 256
+    A = synth.check_pattern("u8", (b, m, k))
+    Bm = synth.check_pattern("i8", (b, k, n))
+    C0 = synth.check_pattern("i32", (b, m, n))
+    want = np.matmul(A.astype(np.int64), Bm.astype(np.int64))
+    got = run_spec(M.Matmul([b, m, k, n], (M.u8, M.i8, M.i32)), [A, Bm, C0])
+    assert np.array_equal(got, want)
+    got = run_spec(M.MatmulAccum([b, m, k, n], (M.u8, M.i8, M.i32)), [A, Bm, C0])
+    assert np.array_equal(got.astype(np.int64), (want + C0 + 2**31) % 2**32 - 2**31)
+
+
+def test_int8_matmul_full_size_properties(gpu):
+    """BASELINE config 2 (4096^3) through size-independent checks: a band of rows against
+    the oracle, every row/column against checksums computed in int64, and accumulation
+    across two calls (the reference's bench loop accumulates the same way)."""
+    m = k = n = 4096
+    A = synth.uniform_u8(21, 0, (1, m, k))
+    Bm = synth.uniform_i8(21, 1, (1, k, n))
+    spec = M.MatmulAccum([1, m, k, n], (M.u8, M.i8, M.i32))
+    dA, dB = M.DeviceBuffer.from_numpy(A), M.DeviceBuffer.from_numpy(Bm)
+    dC = M.DeviceBuffer(m * n * 4)
+    dC.zero()
+    spec.run_device([dA.ptr, dB.ptr, dC.ptr])
+    got = dC.to_numpy(np.int32, (m, n))
+    for lo in (0, 2017, 4064):
+        want = np.zeros((1, m, n), np.int32)
+        orc.matmul([1, m, k, n], [0, 1, 5], A, Bm, want, True, rows=(lo, lo + 32))
+        assert np.array_equal(got[lo:lo + 32], want[0, lo:lo + 32])
+    a64, b64 = A[0].astype(np.int64), Bm[0].astype(np.int64)
+    assert np.array_equal(got.astype(np.int64).sum(axis=1), a64 @ b64.sum(axis=1))   # row checksums
+    assert np.array_equal(got.astype(np.int64).sum(axis=0), a64.sum(axis=0) @ b64)   # column checksums
+    spec.run_device([dA.ptr, dB.ptr, dC.ptr])
+    assert np.array_equal(dC.to_numpy(np.int32, (m, n)), got * 2)
+
+
+@pytest.mark.parametrize("da,db,dc", [(M.u8, M.u8, M.u32), (M.u8, M.i8, M.i16), (M.i16, M.u16, M.i32),
+                                      (M.u32, M.u32, M.u32), (M.i8, M.u8, M.u8), (M.u8, M.i8, M.f32)])
+def test_other_dtype_combinations_generic(gpu, da, db, dc):
+    b, m, k, n = 2, 33, 70, 45
+    raw = lambda t, d: synth.raw_u64(31, t, int(np.prod(d))).astype(np.uint64)
+    A = raw(0, (b, m, k)).astype(da.numpy).reshape(b, m, k)
+    Bm = raw(1, (b, k, n)).astype(db.numpy).reshape(b, k, n)
+    C0 = np.zeros((b, m, n), dc.numpy)
+    got = run_spec(M.Matmul([b, m, k, n], (da, db, dc)), [A, Bm, C0])
+    want = orc.matmul([b, m, k, n], [int(da), int(db), int(dc)], A, Bm, C0.copy())
+    if dc == M.f32:
+        assert rel_err(got, want) < 1e-6
+    else:
+        assert np.array_equal(got, want)
+
+
+def test_f32_matmul_plumbing_config(gpu):
+    """BASELINE config 1: f32 64^3, uniform[-1,1), accumulate into a zeroed C."""
+    shape = [1, 64, 64, 64]
+    A, Bm = synth.uniform_f32(41, 0, (1, 64, 64)), synth.uniform_f32(41, 1, (1, 64, 64))
+    got = run_spec(M.MatmulAccum(shape, [M.f32] * 3), [A, Bm, np.zeros((1, 64, 64), np.float32)])
+    want = orc.matmul(shape, [6, 6, 6], A, Bm, np.zeros((1, 64, 64), np.float32), True)
+    assert rel_err(got, want) < 1e-5
+    # the reference's check inputs are integer valued: exact
+    A = synth.check_pattern("f32", (1, 64, 64))
+    C0 = synth.check_pattern("f32", (1, 64, 64))
+    got = run_spec(M.MatmulAccum(shape, [M.f32] * 3), [A, A.copy(), C0])
+    want = np.matmul(A.astype(np.int64), A.astype(np.int64)) + C0.astype(np.int64)
+    assert np.array_equal(got, want.astype(np.float32))
+
+
+@pytest.mark.parametrize("shape,accum", [((1, 256, 64, 256), False), ((1, 512, 512, 512), True),
+                                         ((2, 256, 192, 256), False), ((1, 60, 100, 36), False)])
+def test_bf16_matmul(gpu, shape, accum):
+    b, m, k, n = shape
+    A, Bm = synth.normal_bf16(51, 0, (b, m, k)), synth.normal_bf16(51, 1, (b, k, n))
+    C0 = synth.normal_f32(51, 2, (b, m, n)) if accum else np.zeros((b, m, n), np.float32)
+    got = run_spec(M.Matmul(shape, (M.bf16, M.bf16, M.f32), accum=accum), [A, Bm, C0])
+    want = orc.matmul(list(shape), [7, 7, 6], A, Bm, C0.copy(), accum)
+    assert rel_err(got, want) < 1e-2  # stated tolerance
+    assert rel_err(got, want) < 1e-5  # what f32 accumulation actually delivers at these K
+
+
+def test_bf16_matmul_pattern_exact(gpu):
+    """0..3 inputs (verification.rs:933-935): every partial sum is an exact integer."""
+    b, m, k, n = 1, 256, 256, 256
+    A = synth.check_pattern("bf16", (b, m, k))
+    Bm = synth.check_pattern("bf16", (b, k, n))
+    got = run_spec(M.Matmul([b, m, k, n], (M.bf16, M.bf16, M.f32)), [A, Bm, np.zeros((b, m, n), np.float32)])
+    want = np.matmul(synth.bf16_bits_to_f32(A).astype(np.int64), synth.bf16_bits_to_f32(Bm).astype(np.int64))
+    assert np.array_equal(got, want.astype(np.float32))
+
+
+def test_bf16_matmul_full_size_sample(gpu):
+    """BASELINE config 3 (8192^3): sampled rows against the oracle, plus linearity."""
+    m = k = n = 8192
+    A, Bm = synth.normal_bf16(61, 0, (1, m, k)), synth.normal_bf16(61, 1, (1, k, n))
+    dA, dB = M.DeviceBuffer.from_numpy(A), M.DeviceBuffer.from_numpy(Bm)
+    dC = M.DeviceBuffer(m * n * 4)
+    spec = M.Matmul([1, m, k, n], (M.bf16, M.bf16, M.f32))
+    spec.run_device([dA.ptr, dB.ptr, dC.ptr])
+    got = dC.to_numpy(np.float32, (m, n))
+    for lo in (0, 5000, 8184):
+        want = np.zeros((1, m, n), np.float32)
+        orc.matmul([1, m, k, n], [7, 7, 6], A, Bm, want, False, rows=(lo, lo + 8))
+        assert rel_err(got[lo:lo + 8], want[0, lo:lo + 8]) < 1e-2
+        assert rel_err(got[lo:lo + 8], want[0, lo:lo + 8]) < 1e-4
+    spec_acc = M.MatmulAccum([1, m, k, n], (M.bf16, M.bf16, M.f32))
+    spec_acc.run_device([dA.ptr, dB.ptr, dC.ptr])
+    assert rel_err(dC.to_numpy(np.float32, (m, n)), got * 2) < 1e-6
+
+
+def test_matmul_layouts(gpu):
+    """Column-major and packed parameter layouts (layout.rs:1249, examples/matmul_x86.rs
+    relayouts) give the same logical result as row-major."""
+    b, m, k, n = 1, 64, 48, 32
+    A, Bm = synth.uniform_u8(71, 0, (b, m, k)), synth.uniform_i8(71, 1, (b, k, n))
+    want = orc.matmul([b, m, k, n], [0, 1, 5], A, Bm, np.zeros((b, m, n), np.int32))
+    # B column-major: buffer holds B transposed
+    spec = M.Matmul([b, m, k, n], (M.u8, M.i8, M.i32), layouts=[None, M.col_major([b, k, n]), None])
+    got = run_spec(spec, [A, np.ascontiguousarray(Bm.transpose(0, 2, 1)), np.zeros((b, m, n), np.int32)])
+    assert np.array_equal(got, want)
+    # B packed [0,2,1,2 p(16)] and C column-major
+    packed = M.layout(0, 2, 1, (2, M.Packed(16)))
+    Bp = np.zeros(b * k * n, np.int8)
+    for kk in range(k):
+        for nn in range(n):
+            Bp[packed.buffer_index([b, k, n], [0, kk, nn])] = Bm[0, kk, nn]
+    spec = M.Matmul([b, m, k, n], (M.u8, M.i8, M.i32), layouts=[None, packed, M.col_major([b, m, n])])
+    got = run_spec(spec, [A, Bp, np.zeros((b, n, m), np.int32)])
+    assert np.array_equal(got.transpose(0, 2, 1), want)
+
+
+def test_run_host_entry_point(gpu):
+    """mrl_run_host: the stand-in for calling the emitted kernel with host pointers."""
+    b, m, k, n = 1, 256, 128, 256
+    A, Bm = synth.uniform_u8(81, 0, (b, m, k)), synth.uniform_i8(81, 1, (b, k, n))
+    C1 = np.full((b, m, n), 5, np.int32)
+    M.MatmulAccum([b, m, k, n], (M.u8, M.i8, M.i32)).run_host(A, Bm, C1)
+    want = orc.matmul([b, m, k, n], [0, 1, 5], A, Bm, np.full((b, m, n), 5, np.int32), True)
+    assert np.array_equal(C1, want)

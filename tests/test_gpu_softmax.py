@@ -1,0 +1,97 @@
+"""Softmax Spec and the Matmul->Softmax->Matmul Compose on the MI355X vs the CPU oracle."""
+import numpy as np
+import pytest
+
+import morello_amd as M
+import orc
+from gpu_util import rel_err, run_spec
+from morello_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("shape,dim", [((8, 2048), 1), ((5, 33), 1), ((3, 7, 1000), 2), ((2, 64, 4096), 2),
+                                       ((2, 3, 5000), 2), ((4, 9, 16), 1), ((6, 4), 0), ((16, 1), 1),
+                                       ((2, 128, 1), 1)])
+def test_softmax_within_1e5(gpu, shape, dim):
+    x = synth.normal_f32(201, 0, shape, std=3.0)
+    got = run_spec(M.Softmax(list(shape), dim), [x, np.zeros(shape, np.float32)])
+    want = orc.softmax(list(shape), dim, x)
+    # stated tolerance: 1e-5 relative, element-wise with a floor for denormal-small outputs
+    assert (np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-12).all()
+    assert np.abs(got.sum(axis=dim) - 1).max() < 1e-5
+
+
+def test_softmax_edge_values(gpu):
+    x = np.zeros((4, 256), np.float32)
+    x[0] = 2.5                                  # constant row -> exactly 1/n
+    x[1, 7] = 1e4                               # one dominant element
+    x[2] = -1e30                                # huge negatives, still finite
+    x[3] = synth.normal_f32(202, 0, (256,)) + np.float32(80.0)  # exp(x) alone would overflow
+    got = run_spec(M.Softmax([4, 256], 1), [x, np.zeros_like(x)])
+    want = orc.softmax([4, 256], 1, x)
+    assert np.array_equal(got[0], np.full(256, np.float32(1) / np.float32(256)))
+    assert got[1, 7] == 1.0 and got[1].sum() == 1.0
+    assert np.isfinite(got).all() and (np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-12).all()
+
+
+def test_softmax_full_size(gpu):
+    """The Softmax stage of BASELINE config 5 alone: 16x2048 rows of 2048."""
+    shape = (16, 2048, 2048)
+    x = synth.normal_f32(203, 0, shape, std=2.0)
+    got = run_spec(M.Softmax(list(shape), 2), [x, np.zeros((1,), np.float32).repeat(x.size).reshape(shape)])
+    want = orc.softmax(list(shape), 2, x)
+    assert (np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-12).all()
+
+
+def msm_inputs(seed, b, m, k, n2, n):
+    q = synth.normal_bf16(seed, 0, (b, m, k), 0.5)
+    kmat = synth.normal_bf16(seed, 1, (b, n2, k), 0.5)   # K row-major == KT with layout![0,2,1]
+    v = synth.normal_bf16(seed, 2, (b, n2, n), 0.5)
+    return q, kmat, v
+
+
+KT_LAYOUT = M.layout(0, 2, 1)
+KT_ORC = orc.make_layout([0, 2, 1])
+
+
+@pytest.mark.parametrize("dims", [(1, 64, 128, 64, 128), (2, 256, 128, 512, 128), (1, 128, 64, 256, 64),
+                                  (3, 50, 24, 70, 10), (1, 2048, 128, 2048, 128)])
+def test_compose_msm(gpu, dims):
+    b, m, k, n2, n = dims
+    q, kmat, v = msm_inputs(301, *dims)
+    spec = M.ComposeMSM(b, m, k, n2, n, layouts=[None, None, KT_LAYOUT, None])
+    got = run_spec(spec, [v, q, kmat, np.zeros((b, m, n), np.float32)])
+    want = orc.compose_msm(b, m, k, n2, n, [7, 7, 7, 6], v, q, kmat, np.zeros((b, m, n), np.float32),
+                           layouts=[None, None, KT_ORC, None])
+    assert rel_err(got, want) < 1e-2  # stated tolerance for the composed pipeline
+
+
+def test_compose_msm_row_major_kt_and_f32_inputs(gpu):
+    """KT materialised row-major and f32 inputs run on the staged (unfused) path."""
+    b, m, k, n2, n = 2, 40, 32, 48, 24
+    q, kmat, v = msm_inputs(302, b, m, k, n2, n)
+    kt = np.ascontiguousarray(kmat.transpose(0, 2, 1))
+    got = run_spec(M.ComposeMSM(b, m, k, n2, n), [v, q, kt, np.zeros((b, m, n), np.float32)])
+    want = orc.compose_msm(b, m, k, n2, n, [7, 7, 7, 6], v, q, kt, np.zeros((b, m, n), np.float32))
+    assert rel_err(got, want) < 1e-5
+    qf, ktf, vf = (synth.bf16_bits_to_f32(t) for t in (q, kt, v))
+    got = run_spec(M.ComposeMSM(b, m, k, n2, n, dtypes=(M.f32, M.f32, M.f32, M.f32)),
+                   [vf, qf, ktf, np.zeros((b, m, n), np.float32)])
+    assert rel_err(got, want) < 1e-5
+
+
+def test_compose_msm_full_size(gpu):
+    """BASELINE config 5: 16 heads of 2048x128; four heads against the oracle, all heads
+    through the row-stochastic property: with V = ones, out must be all ones."""
+    b, m, k, n2, n = 16, 2048, 128, 2048, 128
+    q, kmat, v = msm_inputs(303, b, m, k, n2, n)
+    spec = M.ComposeMSM(b, m, k, n2, n, layouts=[None, None, KT_LAYOUT, None])
+    got = run_spec(spec, [v, q, kmat, np.zeros((b, m, n), np.float32)])
+    for h in (0, 5, 10, 15):
+        want = orc.compose_msm(1, m, k, n2, n, [7, 7, 7, 6], v[h:h + 1], q[h:h + 1], kmat[h:h + 1],
+                               np.zeros((1, m, n), np.float32), layouts=[None, None, KT_ORC, None])
+        assert rel_err(got[h:h + 1], want) < 1e-2
+    ones = synth.f32_to_bf16_bits(np.ones((b, n2, n), np.float32))
+    got = run_spec(spec, [ones, q, kmat, np.zeros((b, m, n), np.float32)])
+    assert np.abs(got - 1).max() < 1e-2
