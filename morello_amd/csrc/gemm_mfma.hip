@@ -112,23 +112,27 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void k_gemm(GemmArgs g, int
   Out *C = (Out *)g.c + int64_t(blockIdx.y) * g.sc + m0 * g.ldc + n0;
   const int64_t lda_b = g.lda * ES, ldb_b = g.ldb * ES;
 
-  // Per-thread staging assignments (global source, LDS destination) for one k step.
-  const uint8_t *a_src[A_CH];
-  int a_dst[A_CH];
-#pragma unroll
-  for (int i = 0; i < A_CH; i++) {
-    const int id = tid + i * NT, row = id >> 3, ch = id & 7;
-    a_src[i] = A + int64_t(row) * lda_b + ch * 16;
-    a_dst[i] = row * BKB + ((ch ^ ((row >> 1) & 7)) << 4);
+  // Per-thread staging assignments for one k step.  Thread `tid` moves 16-byte chunk
+  // tid + i*NT of each tile; successive i differ by a whole number of rows (a multiple of
+  // 16), so one base pointer / LDS offset per operand plus compile-time strides suffices.
+  constexpr int A_ROWS_PER_I = NT / 8, B_ROWS_PER_I = NT / B_ROW_CH;
+  static_assert(A_ROWS_PER_I % 16 == 0, "swizzle term must not depend on i");
+  const uint8_t *a_src;
+  int a_dst;
+  {
+    const int row = tid >> 3, ch = tid & 7;
+    a_src = A + int64_t(row) * lda_b + ch * 16;
+    a_dst = row * BKB + ((ch ^ ((row >> 1) & 7)) << 4);
   }
-  const uint8_t *b_src[B_CH];
-  int b_dst[B_CH];
-#pragma unroll
-  for (int i = 0; i < B_CH; i++) {
-    const int id = tid + i * NT, row = id / B_ROW_CH, ch = id % B_ROW_CH;
-    b_src[i] = B + int64_t(row) * ldb_b + ch * 16;
-    b_dst[i] = A_STAGE + row * B_ROW + ch * 16;
+  const uint8_t *b_src;
+  int b_dst;
+  {
+    const int row = tid / B_ROW_CH, ch = tid % B_ROW_CH;
+    b_src = B + int64_t(row) * ldb_b + ch * 16;
+    b_dst = A_STAGE + row * B_ROW + ch * 16;
   }
+  const int64_t a_step_i = int64_t(A_ROWS_PER_I) * lda_b, b_step_i = int64_t(B_ROWS_PER_I) * ldb_b;
+  const int64_t b_step_kt = int64_t(BK) * ldb_b;
   // Operand fragment offsets within a stage for MFMA k step 0.
   int a_frag[TM];
 #pragma unroll
@@ -161,11 +165,14 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void k_gemm(GemmArgs g, int
   v4i a_reg[A_CH], b_reg[B_CH];
   const int kt_count = int(g.k / BK);
 
-  auto load_global = [&](int kt) {
+  // Loads the next tile in sequence and advances the source pointers.
+  auto load_global = [&]() {
 #pragma unroll
-    for (int i = 0; i < A_CH; i++) a_reg[i] = *(const v4i *)(a_src[i] + int64_t(kt) * BKB);
+    for (int i = 0; i < A_CH; i++) a_reg[i] = *(const v4i *)(a_src + i * a_step_i);
 #pragma unroll
-    for (int i = 0; i < B_CH; i++) b_reg[i] = *(const v4i *)(b_src[i] + int64_t(kt) * BK * ldb_b);
+    for (int i = 0; i < B_CH; i++) b_reg[i] = *(const v4i *)(b_src + i * b_step_i);
+    a_src += BKB;
+    b_src += b_step_kt;
   };
   auto store_lds = [&](int stage) {
     uint8_t *base = lds + stage * STAGE;
@@ -173,80 +180,115 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void k_gemm(GemmArgs g, int
     for (int i = 0; i < A_CH; i++) {
       v4i v = a_reg[i];
       if (A_UNSIGNED) v ^= v4i{int(0x80808080), int(0x80808080), int(0x80808080), int(0x80808080)};
-      *(v4i *)(base + a_dst[i]) = v;
+      *(v4i *)(base + a_dst + i * A_ROWS_PER_I * BKB) = v;
     }
 #pragma unroll
-    for (int i = 0; i < B_CH; i++) *(v4i *)(base + b_dst[i]) = b_reg[i];
+    for (int i = 0; i < B_CH; i++) *(v4i *)(base + b_dst + i * B_ROWS_PER_I * B_ROW) = b_reg[i];
+  };
+  // MFMA operands for one 32-byte k step, double buffered in registers.
+  v4i af[2][TM], bf[2][TN];
+  auto read_frags = [&](int stage, int s, int buf) {
+    const uint8_t *base = lds + stage * STAGE;
+#pragma unroll
+    for (int tm = 0; tm < TM; tm++)
+      af[buf][tm] = *(const v4i *)(base + a_frag[tm] + (((2 * s + a_half) ^ a_swz) << 4));
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++) {
+      const v2i lo = T::read_tr(base + b_frag[tn] + (s * K_SLAB) * B_ROW);
+      const v2i hi = T::read_tr(base + b_frag[tn] + (s * K_SLAB + T::K_PER_READ) * B_ROW);
+      bf[buf][tn] = v4i{lo[0], lo[1], hi[0], hi[1]};
+    }
+  };
+  auto mfma_slab = [&](int buf) {
+    if (A_UNSIGNED) {
+#pragma unroll
+      for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+        for (int w = 0; w < 4; w++)
+          colsum[tn] = __builtin_amdgcn_sdot4(bf[buf][tn][w], 0x01010101, colsum[tn], false);
+    }
+#pragma unroll
+    for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+      for (int tn = 0; tn < TN; tn++) acc[tm][tn] = T::mfma(af[buf][tm], bf[buf][tn], acc[tm][tn]);
   };
 
-  load_global(0);
+  // Software pipeline.  While tile kt is multiplied out of LDS stage kt&1, tile kt+1 sits
+  // in registers (its global loads were issued one tile earlier) and is written to the
+  // other stage during the second-to-last k step; the barrier comes before the last k
+  // step's MFMAs, so the first operands of tile kt+1 are fetched under them and the matrix
+  // core does not drain at the barrier.  The body is branch-free: past the end of K the
+  // pointers stop advancing, so the last tile is re-read (L2 hits) and re-staged into the
+  // stage nobody reads any more.  sched_group_barrier pins the interleaving of LDS, VMEM
+  // and MFMA issue that the text below spells out.
+  load_global();
   store_lds(0);
+  if (kt_count < 2) a_src -= BKB, b_src -= b_step_kt;
+  load_global();
   __syncthreads();
+  read_frags(0, 0, 0);
 
   for (int kt = 0; kt < kt_count; kt++) {
     const int cur = kt & 1;
-    const uint8_t *base = lds + cur * STAGE;
-    if (kt + 1 < kt_count) load_global(kt + 1);
+    // Tile kt+2 is loaded next (or the last tile again when there is none).
+    if (kt + 2 >= kt_count) a_src -= BKB, b_src -= b_step_kt;
 #pragma unroll
     for (int s = 0; s < SLABS; s++) {
-      v4i af[TM], bf[TN];
-#pragma unroll
-      for (int tm = 0; tm < TM; tm++)
-        af[tm] = *(const v4i *)(base + a_frag[tm] + (((2 * s + a_half) ^ a_swz) << 4));
-#pragma unroll
-      for (int tn = 0; tn < TN; tn++) {
-        const v2i lo = T::read_tr(base + b_frag[tn] + (s * K_SLAB) * B_ROW);
-        const v2i hi = T::read_tr(base + b_frag[tn] + (s * K_SLAB + T::K_PER_READ) * B_ROW);
-        bf[tn] = v4i{lo[0], lo[1], hi[0], hi[1]};
+      if (s + 1 < SLABS) read_frags(cur, s + 1, (s + 1) & 1);
+      if (s == SLABS - 2) {
+        store_lds(cur ^ 1);
+        load_global();
       }
-      if (A_UNSIGNED && (s % WAVES_M) == wm) {
-#pragma unroll
-        for (int tn = 0; tn < TN; tn++)
-#pragma unroll
-          for (int w = 0; w < 4; w++)
-            colsum[tn] = __builtin_amdgcn_sdot4(bf[tn][w], 0x01010101, colsum[tn], false);
+      if (s == SLABS - 1) {
+        __syncthreads();
+        read_frags(cur ^ 1, 0, 0);
       }
+      mfma_slab(s & 1);
+      // One MFMA, then a share of this step's memory instructions, TM*TN times.
 #pragma unroll
-      for (int tm = 0; tm < TM; tm++)
-#pragma unroll
-        for (int tn = 0; tn < TN; tn++) acc[tm][tn] = T::mfma(af[tm], bf[tn], acc[tm][tn]);
+      for (int i = 0; i < TM * TN; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+        if (i < TM + 2 * TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+        if (s == SLABS - 2) {
+          if (i < A_CH + B_CH) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // DS write
+          if (i < A_CH + B_CH) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // VMEM read
+        }
+      }
     }
-    if (kt + 1 < kt_count) store_lds(cur ^ 1);
-    __syncthreads();
   }
 
-  // Epilogue.  Column sums: each (wave-row, k-half) pair holds a partial for its columns.
+  // Epilogue.  Column sums: the two lane halves hold the two k halves of each MFMA step.
   int corr[TN];
 #pragma unroll
   for (int tn = 0; tn < TN; tn++) corr[tn] = 0;
   if (A_UNSIGNED) {
-    int *part = (int *)lds;  // [WAVES_M * 2][BN]
 #pragma unroll
-    for (int tn = 0; tn < TN; tn++)
-      part[(wm * 2 + (lane >> 5)) * BN + wn * WN + tn * 32 + (lane & 31)] = colsum[tn];
-    __syncthreads();
-#pragma unroll
-    for (int tn = 0; tn < TN; tn++) {
-      int s = 0;
-#pragma unroll
-      for (int w = 0; w < WAVES_M * 2; w++) s += part[w * BN + wn * WN + tn * 32 + (lane & 31)];
-      corr[tn] = s * 128;
-    }
+    for (int tn = 0; tn < TN; tn++) corr[tn] = 128 * (colsum[tn] + __shfl_xor(colsum[tn], 32));
   }
+  // Lane (l%32, l/32) of accumulator register r owns C[8*(r/4) + 4*(l/32) + r%4][l%32] of
+  // each 32x32 block.  An accumulating Spec reads its whole block row of C first, so the
+  // loads are in flight together instead of one round trip per element.
+  Out *c_lane = C + int64_t(wm * WM + (lane >> 5) * 4) * g.ldc + wn * WN + (lane & 31);
 #pragma unroll
-  for (int tm = 0; tm < TM; tm++)
+  for (int tm = 0; tm < TM; tm++) {
+    Out prev[TN][16];
+    if (g.accum) {
+#pragma unroll
+      for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+          prev[tn][r] = c_lane[int64_t(tm * 32 + (r >> 2) * 8 + (r & 3)) * g.ldc + tn * 32];
+    }
 #pragma unroll
     for (int tn = 0; tn < TN; tn++)
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        const int row = wm * WM + tm * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-        const int col = wn * WN + tn * 32 + (lane & 31);
-        Out *dst = C + int64_t(row) * g.ldc + col;
         Out v = acc[tm][tn][r];
         if (A_UNSIGNED) v += Out(corr[tn]);
-        if (g.accum) v += *dst;
-        *dst = v;
+        if (g.accum) v += prev[tn][r];
+        c_lane[int64_t(tm * 32 + (r >> 2) * 8 + (r & 3)) * g.ldc + tn * 32] = v;
       }
+  }
 }
 
 template <class T, bool A_UNSIGNED>
