@@ -91,7 +91,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void k_gemm(GemmArgs g, int
   typedef typename T::Acc Acc;
   typedef typename T::Out Out;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lives in an SGPR
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
   // Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous run of
@@ -199,8 +200,10 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void k_gemm(GemmArgs g, int
       bf[buf][tn] = v4i{lo[0], lo[1], hi[0], hi[1]};
     }
   };
-  auto mfma_slab = [&](int buf) {
-    if (A_UNSIGNED) {
+  auto mfma_slab = [&](int s, int buf) {
+    // Column sums of B for the u8 correction: each of the WAVES_M waves that share these
+    // columns takes every WAVES_M-th k step (a scalar branch: `wm` is wave-uniform).
+    if (A_UNSIGNED && (s % WAVES_M) == wm) {
 #pragma unroll
       for (int tn = 0; tn < TN; tn++)
 #pragma unroll
@@ -243,7 +246,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void k_gemm(GemmArgs g, int
         __syncthreads();
         read_frags(cur ^ 1, 0, 0);
       }
-      mfma_slab(s & 1);
+      mfma_slab(s, s & 1);
       // One MFMA, then a share of this step's memory instructions, TM*TN times.
 #pragma unroll
       for (int i = 0; i < TM * TN; i++) {
@@ -257,13 +260,24 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void k_gemm(GemmArgs g, int
     }
   }
 
-  // Epilogue.  Column sums: the two lane halves hold the two k halves of each MFMA step.
+  // Epilogue.  Column sums: combine the partials of the WAVES_M waves and two lane halves.
   int corr[TN];
 #pragma unroll
   for (int tn = 0; tn < TN; tn++) corr[tn] = 0;
   if (A_UNSIGNED) {
+    int *part = (int *)lds;  // [WAVES_M * 2][BN]; the k loop ended on a barrier
+    __syncthreads();         // ... and every wave is past its last LDS read of the tiles
 #pragma unroll
-    for (int tn = 0; tn < TN; tn++) corr[tn] = 128 * (colsum[tn] + __shfl_xor(colsum[tn], 32));
+    for (int tn = 0; tn < TN; tn++)
+      part[(wm * 2 + (lane >> 5)) * BN + wn * WN + tn * 32 + (lane & 31)] = colsum[tn];
+    __syncthreads();
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++) {
+      int sum = 0;
+#pragma unroll
+      for (int w = 0; w < WAVES_M * 2; w++) sum += part[w * BN + wn * WN + tn * 32 + (lane & 31)];
+      corr[tn] = sum * 128;
+    }
   }
   // Lane (l%32, l/32) of accumulator register r owns C[8*(r/4) + 4*(l/32) + r%4][l%32] of
   // each 32x32 block.  An accumulating Spec reads its whole block row of C first, so the
