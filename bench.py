@@ -59,6 +59,13 @@ def workload(name):
                 synth.normal_bf16(5, 1, (b, n2, k), 0.5), np.zeros((b, m, n), np.float32)]
         return ("Compose Matmul->Softmax->Matmul, 16 heads, Q/K/V bf16 2048x128, out f32", spec, arrs,
                 "bf16", "TFLOPS", "mfma", PEAK["bf16"])
+    if name == "move":
+        # Plain copy of 256 MiB: the known-size kernel the HBM byte counters are scaled by.
+        n = 64 * 1024 * 1024
+        spec = M.Move([n], (M.f32, M.f32))
+        arrs = [synth.uniform_f32(6, 0, (n,)), np.zeros((n,), np.float32)]
+        return ("Move f32[67108864] -> f32, same layout (plain copy, 256 MiB read + 256 MiB write)",
+                spec, arrs, "f32", "GB/s", "hbm", PEAK["hbm_gbs"])
     raise SystemExit(f"unknown spec {name}")
 
 
@@ -121,7 +128,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--spec", default="c2", choices=["c2", "c3", "c4", "c5"])
+    ap.add_argument("--spec", default="c2", choices=["c2", "c3", "c4", "c5", "move"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -145,6 +152,8 @@ def main():
     ms_per_step = wall_ms / args.steps
     kernel_ms = device_ms / args.steps
     value = ops / (ms_per_step * 1e-3) / 1e12
+    if args.spec == "move":
+        value = alg_bytes / (ms_per_step * 1e-3) / 1e9
 
     if bound == "mfma":
         achieved = ops / (kernel_ms * 1e-3) / 1e12
@@ -164,7 +173,7 @@ def main():
         "config": {"workload": desc, "spec": args.spec, "device": M.device_info()["name"]},
         "roofline": roofline,
     }
-    if not args.no_cpu:
+    if not args.no_cpu and args.spec != "move":
         out["cpu_baseline"] = cpu_baseline(args.spec, arrs)
     print(json.dumps(out))
 

@@ -77,9 +77,12 @@ typedef enum {
   MRL_SPEC_MATMUL = 0,     /* spec_shape [b,m,k,n]; params A[b,m,k] B[b,k,n] C[b,m,n]   */
   MRL_SPEC_CONV = 1,       /* spec_shape [b,f,c,oh,ow,fh,fw]; params image, filters, out */
   MRL_SPEC_SOFTMAX = 2,    /* spec_shape = tensor shape; params in, out; uses scan_dim   */
-  MRL_SPEC_COMPOSE_MSM = 3 /* Matmul->Softmax->Matmul; spec_shape [b,m,k,n2,n];
+  MRL_SPEC_COMPOSE_MSM = 3,/* Matmul->Softmax->Matmul; spec_shape [b,m,k,n2,n];
                               params V[b,n2,n] Q[b,m,k] KT[b,k,n2] out[b,m,n]
                               (Compose parameter order, spec.rs:3329-3365)               */
+  MRL_SPEC_MOVE = 4        /* Move (spec.rs:57-162; oracle verification.rs assign_cast):
+                              spec_shape = tensor shape; params in, out; the two may
+                              differ in layout and dtype (Rust `as` conversion)          */
 } mrl_spec_kind;
 
 typedef struct {
@@ -176,6 +179,9 @@ int mrl_conv(uint32_t b, uint32_t f, uint32_t c, uint32_t oh, uint32_t ow, uint3
              const void *filters, void *out, void *stream);
 int mrl_softmax(const uint32_t *shape, uint32_t rank, uint32_t scan_dim, const void *in,
                 void *out, void *stream);
+/* Move: copies `in` to `out` (dense row-major both sides, same dtype). */
+int mrl_move(const uint32_t *shape, uint32_t rank, int dtype, const void *in, void *out,
+             void *stream);
 /* KT is the B operand of the first Matmul, logical [b,k,n2]; kt_col_major != 0 says it is
  * stored with layout![0,2,1] (i.e. K stored row-major as [b,n2,k]). */
 int mrl_compose_msm(uint32_t b, uint32_t m, uint32_t k, uint32_t n2, uint32_t n, int dt_v,

@@ -172,6 +172,7 @@ class SpecKind(enum.IntEnum):
     Conv = 1
     Softmax = 2
     ComposeMSM = 3
+    Move = 4
 
 
 class OperandDirection(enum.IntEnum):
@@ -300,6 +301,12 @@ def ComposeMSM(b, m, k, n2, n, dtypes=(bf16, bf16, bf16, f32), layouts=None) -> 
     """Compose [Matmul, Softmax{2}, Matmul] with external parameters [V, Q, KT, out]
     (spec.rs:3329-3365; examples/matmul_chain.rs:26-57)."""
     return Spec(SpecKind.ComposeMSM, [b, m, k, n2, n], dtypes, layouts)
+
+
+def Move(shape, dtypes, layouts=None) -> Spec:
+    """Move Spec: copy `in` to `out`, which may differ in layout and dtype (Rust `as`
+    conversion; oracle: assign_cast in morello/src/verification.rs)."""
+    return Spec(SpecKind.Move, shape, dtypes, layouts)
 
 
 class DeviceBuffer:

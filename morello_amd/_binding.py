@@ -64,6 +64,7 @@ SIGNATURES = {
     "mrl_matmul": (C.c_int, [C.c_uint32] * 4 + [C.c_int] * 4 + [C.c_void_p] * 4),
     "mrl_conv": (C.c_int, [C.c_uint32] * 7 + [C.c_int] * 4 + [C.c_void_p] * 4),
     "mrl_softmax": (C.c_int, [_U32P, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "mrl_move": (C.c_int, [_U32P, C.c_uint32, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
     "mrl_compose_msm": (C.c_int, [C.c_uint32] * 5 + [C.c_int] * 4 + [C.c_void_p] * 5),
     "mrl_bench": (C.c_int, [C.POINTER(SpecC), _VPP, C.c_uint32, C.c_uint32,
                             C.POINTER(C.c_double), C.POINTER(C.c_double)]),

@@ -37,7 +37,7 @@ uint64_t volume(const uint32_t *s, uint32_t r) {
 uint32_t expected_params(int kind) {
   switch (kind) {
     case MRL_SPEC_MATMUL: case MRL_SPEC_CONV: return 3;
-    case MRL_SPEC_SOFTMAX: return 2;
+    case MRL_SPEC_SOFTMAX: case MRL_SPEC_MOVE: return 2;
     case MRL_SPEC_COMPOSE_MSM: return 4;
     default: return 0;
   }
@@ -47,7 +47,7 @@ uint32_t expected_rank(const mrl_spec &s) {
   switch (s.kind) {
     case MRL_SPEC_MATMUL: return 4;
     case MRL_SPEC_CONV: return 7;
-    case MRL_SPEC_SOFTMAX: return s.rank;
+    case MRL_SPEC_SOFTMAX: case MRL_SPEC_MOVE: return s.rank;
     case MRL_SPEC_COMPOSE_MSM: return 5;
     default: return 0;
   }
@@ -74,6 +74,7 @@ int parameter_shape(const mrl_spec &s, uint32_t idx, uint32_t *shape, uint32_t *
       return MRL_OK;
     }
     case MRL_SPEC_SOFTMAX:
+    case MRL_SPEC_MOVE:
       if (idx > 1) return MRL_ERR_BAD_SPEC;
       *rank = s.rank;
       for (uint32_t d = 0; d < s.rank; d++) shape[d] = ss[d];
@@ -111,6 +112,7 @@ int check_spec(const mrl_spec *sp) {
   if (s.n_params != np) return MRL_ERR_BAD_SPEC;
   if (s.rank == 0 || s.rank > MRL_MAX_SPEC_RANK || s.rank != expected_rank(s)) return MRL_ERR_BAD_SPEC;
   if (s.kind == MRL_SPEC_SOFTMAX && (s.rank > MRL_MAX_RANK || s.scan_dim >= s.rank)) return MRL_ERR_BAD_SPEC;
+  if (s.kind == MRL_SPEC_MOVE && s.rank > MRL_MAX_RANK) return MRL_ERR_BAD_SPEC;
   for (uint32_t d = 0; d < s.rank; d++)
     if (s.spec_shape[d] == 0) return MRL_ERR_BAD_SPEC;
   for (uint32_t i = 0; i < np; i++) {
@@ -331,6 +333,27 @@ int run_compose_msm(const mrl_spec &s, void *const *params, Workspace &ws) {
   return finish_output(out, ws);
 }
 
+int run_move(const mrl_spec &s, void *const *params, Workspace &ws) {
+  uint32_t shape[MRL_MAX_RANK], rank;
+  parameter_shape(s, 0, shape, &rank);
+  const uint64_t count = volume(shape, rank);
+  const mrl_layout &li = s.layouts[0], &lo = s.layouts[1];
+  bool same_layout = li.ndims == lo.ndims;
+  for (uint32_t i = 0; same_layout && i < li.ndims; i++)
+    same_layout = li.dims[i].logical_dim == lo.dims[i].logical_dim && li.dims[i].kind == lo.dims[i].kind &&
+                  (li.dims[i].kind == MRL_DYNAMIC || li.dims[i].size == lo.dims[i].size);
+  auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  if (same_layout && s.dtypes[0] == s.dtypes[1] && al16(params[0]) && al16(params[1])) {
+    HIP_TRY(mrl::launch_copy(params[0], params[1], count * mrl_dtype_size(s.dtypes[0]), ws.stream));
+    return MRL_OK;
+  }
+  mrl::LayoutEval sl, dl;
+  if (!mrl::make_layout_eval(li, shape, rank, &sl) || !mrl::make_layout_eval(lo, shape, rank, &dl))
+    return MRL_ERR_BAD_LAYOUT;
+  HIP_TRY(mrl::launch_move_generic(params[0], params[1], sl, dl, s.dtypes[0], s.dtypes[1], count, ws.stream));
+  return MRL_OK;
+}
+
 int run_async_impl(const mrl_spec *spec, void *const *params, hipStream_t stream) {
   if (g_device < 0) {
     int rc = mrl_init(0);
@@ -347,6 +370,7 @@ int run_async_impl(const mrl_spec *spec, void *const *params, hipStream_t stream
     case MRL_SPEC_CONV: return run_conv(*spec, params, ws);
     case MRL_SPEC_SOFTMAX: return run_softmax(*spec, params, ws);
     case MRL_SPEC_COMPOSE_MSM: return run_compose_msm(*spec, params, ws);
+    case MRL_SPEC_MOVE: return run_move(*spec, params, ws);
     default: return MRL_ERR_UNSUPPORTED;
   }
 }
@@ -501,6 +525,7 @@ uint64_t mrl_spec_ops(const mrl_spec *spec) {
     case MRL_SPEC_MATMUL: return 2ull * s[0] * s[1] * s[2] * s[3];
     case MRL_SPEC_CONV: return 2ull * s[0] * s[1] * s[2] * s[3] * s[4] * s[5] * s[6];
     case MRL_SPEC_SOFTMAX: return 5ull * volume(s, spec->rank);
+    case MRL_SPEC_MOVE: return 0;
     case MRL_SPEC_COMPOSE_MSM:
       return 2ull * s[0] * s[1] * s[2] * s[3] + 5ull * s[0] * s[1] * s[3] + 2ull * s[0] * s[1] * s[3] * s[4];
     default: return 0;
@@ -510,7 +535,7 @@ uint64_t mrl_spec_ops(const mrl_spec *spec) {
 int mrl_spec_check(const mrl_spec *spec) { return check_spec(spec); }
 
 size_t mrl_spec_workspace_bytes(const mrl_spec *spec) {
-  if (check_spec(spec) != MRL_OK) return 0;
+  if (check_spec(spec) != MRL_OK || spec->kind == MRL_SPEC_MOVE) return 0;
   size_t total = 0;
   for (uint32_t i = 0; i < spec->n_params; i++) {
     uint32_t shape[MRL_MAX_RANK], rank;
@@ -614,6 +639,20 @@ int mrl_softmax(const uint32_t *shape, uint32_t rank, uint32_t scan_dim, const v
   s.kind = MRL_SPEC_SOFTMAX, s.scan_dim = scan_dim, s.rank = rank, s.n_params = 2;
   for (uint32_t d = 0; d < rank; d++) s.spec_shape[d] = shape[d];
   s.dtypes[0] = s.dtypes[1] = MRL_F32;
+  mrl_layout_row_major(shape, rank, &s.layouts[0]);
+  s.layouts[1] = s.layouts[0];
+  void *params[2] = {const_cast<void *>(in), out};
+  return mrl_run_async(&s, params, stream);
+}
+
+int mrl_move(const uint32_t *shape, uint32_t rank, int dtype, const void *in, void *out, void *stream) {
+  if (!shape) return MRL_ERR_NULL;
+  if (rank == 0 || rank > MRL_MAX_RANK) return MRL_ERR_BAD_SPEC;
+  mrl_spec s;
+  std::memset(&s, 0, sizeof s);
+  s.kind = MRL_SPEC_MOVE, s.rank = rank, s.n_params = 2;
+  for (uint32_t d = 0; d < rank; d++) s.spec_shape[d] = shape[d];
+  s.dtypes[0] = s.dtypes[1] = dtype;
   mrl_layout_row_major(shape, rank, &s.layouts[0]);
   s.layouts[1] = s.layouts[0];
   void *params[2] = {const_cast<void *>(in), out};

@@ -82,6 +82,59 @@ __global__ void k_relayout(const uint8_t *src, uint8_t *dst, LayoutEval sl, Layo
   else ((uint32_t *)dst)[d_o] = ((const uint32_t *)src)[so];
 }
 
+// ---------------------------------------------------------------------- move
+__device__ inline uint16_t f32_to_bf16_bits(float f) {
+  uint32_t bits = __float_as_uint(f);
+  if ((bits & 0x7fffffffu) > 0x7f800000u) return uint16_t((bits >> 16) | 0x40u);
+  bits += 0x7fffu + ((bits >> 16) & 1u);  // round to nearest even
+  return uint16_t(bits >> 16);
+}
+
+// Rust `as` for narrow integer targets saturates floats at the target's own bounds.
+__device__ inline uint32_t float_to_int(float f, int dt) {
+  if (f != f) return 0;
+  float lo, hi;
+  switch (dt) {
+    case MRL_U8: lo = 0.f, hi = 255.f; break;
+    case MRL_I8: lo = -128.f, hi = 127.f; break;
+    case MRL_U16: lo = 0.f, hi = 65535.f; break;
+    case MRL_I16: lo = -32768.f, hi = 32767.f; break;
+    case MRL_U32: return f <= 0.f ? 0u : f >= 4294967296.f ? 0xffffffffu : uint32_t(f);
+    default: return f <= -2147483648.f ? 0x80000000u : f >= 2147483648.f ? 0x7fffffffu : uint32_t(int32_t(f));
+  }
+  f = fminf(fmaxf(f, lo), hi);
+  return uint32_t(int32_t(f));
+}
+
+__global__ void k_move_generic(const void *src, void *dst, LayoutEval sl, LayoutEval dl, int sdt,
+                               int ddt, uint64_t count) {
+  const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  uint32_t pt[MRL_MAX_RANK];
+  uint64_t rem = i;
+  for (int d = int(sl.rank) - 1; d >= 0; d--) {
+    pt[d] = uint32_t(rem % sl.shape[d]);
+    rem /= sl.shape[d];
+  }
+  const int64_t so = layout_offset(sl, pt), d_o = layout_offset(dl, pt);
+  const bool src_float = sdt == MRL_F32 || sdt == MRL_BF16;
+  if (ddt == MRL_F32) ((float *)dst)[d_o] = load_f32(src, sdt, so);
+  else if (ddt == MRL_BF16) ((uint16_t *)dst)[d_o] = f32_to_bf16_bits(load_f32(src, sdt, so));
+  else if (src_float) store_u32(dst, ddt, d_o, float_to_int(load_f32(src, sdt, so), ddt));
+  else store_u32(dst, ddt, d_o, load_u32(src, sdt, so, MRL_U32));  // int -> int wraps
+}
+
+__global__ __launch_bounds__(256) void k_copy16(const uint4 *__restrict__ src, uint4 *__restrict__ dst,
+                                                uint64_t vecs) {
+  const uint64_t step = uint64_t(gridDim.x) * blockDim.x;
+  for (uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < vecs; i += step) dst[i] = src[i];
+}
+
+__global__ void k_copy1(const uint8_t *src, uint8_t *dst, uint64_t bytes) {
+  const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < bytes) dst[i] = src[i];
+}
+
 // -------------------------------------------------------------------- matmul
 struct MM {
   const void *a, *b;
@@ -246,6 +299,28 @@ hipError_t launch_relayout(const void *src, void *dst, const LayoutEval &sl, con
   const uint32_t blocks = uint32_t((count + 255) / 256);
   hipLaunchKernelGGL(k_relayout, dim3(blocks), dim3(256), 0, stream, (const uint8_t *)src,
                      (uint8_t *)dst, sl, dl, es, count);
+  return hipGetLastError();
+}
+
+hipError_t launch_move_generic(const void *src, void *dst, const LayoutEval &sl, const LayoutEval &dl,
+                               int sdt, int ddt, uint64_t count, hipStream_t stream) {
+  if (count == 0) return hipSuccess;
+  const uint32_t blocks = uint32_t((count + 255) / 256);
+  hipLaunchKernelGGL(k_move_generic, dim3(blocks), dim3(256), 0, stream, src, dst, sl, dl, sdt, ddt, count);
+  return hipGetLastError();
+}
+
+hipError_t launch_copy(const void *src, void *dst, uint64_t bytes, hipStream_t stream) {
+  const uint64_t vecs = bytes / 16, tail = bytes % 16;
+  if (vecs) {
+    uint64_t blocks = (vecs + 255) / 256;
+    if (blocks > 16384) blocks = 16384;  // grid-stride: 64 blocks per CU on a 256-CU part
+    hipLaunchKernelGGL(k_copy16, dim3(uint32_t(blocks)), dim3(256), 0, stream, (const uint4 *)src,
+                       (uint4 *)dst, vecs);
+  }
+  if (tail)
+    hipLaunchKernelGGL(k_copy1, dim3(1), dim3(16), 0, stream, (const uint8_t *)src + vecs * 16,
+                       (uint8_t *)dst + vecs * 16, tail);
   return hipGetLastError();
 }
 

@@ -27,6 +27,12 @@ hipError_t launch_conv_generic(const Strided &img, const Strided &filt, const St
 hipError_t launch_softmax_generic(const Strided &in, const Strided &out, uint32_t scan_dim,
                                   hipStream_t stream);
 hipError_t launch_fill_zero(void *ptr, uint64_t bytes, hipStream_t stream);
+// Move Spec: element-wise copy with dtype conversion between two arbitrary layouts.
+hipError_t launch_move_generic(const void *src, void *dst, const LayoutEval &src_l,
+                               const LayoutEval &dst_l, int src_dtype, int dst_dtype,
+                               uint64_t count, hipStream_t stream);
+// Move Spec fast path: same bytes on both sides (16-byte aligned buffers).
+hipError_t launch_copy(const void *src, void *dst, uint64_t bytes, hipStream_t stream);
 
 // ---- gemm_i8.hip: u8|i8 x i8 -> i32 on the int8 MFMA -----------------------------------
 // Row-major operands with leading dimensions in elements; batch strides in elements.

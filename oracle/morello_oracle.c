@@ -491,6 +491,42 @@ int orc_compose_msm(uint32_t b, uint32_t m, uint32_t k, uint32_t n2, uint32_t n,
   return rc;
 }
 
+/* -------------------------------------------------------------------- move */
+
+static uint32_t float_as_int(float f, int dt) {
+  if (f != f) return 0;
+  switch (dt) {
+    case ORC_U8: return f <= 0.f ? 0u : f >= 255.f ? 255u : (uint32_t)f;
+    case ORC_I8: return (uint32_t)(int32_t)(f <= -128.f ? -128 : f >= 127.f ? 127 : (int32_t)f);
+    case ORC_U16: return f <= 0.f ? 0u : f >= 65535.f ? 65535u : (uint32_t)f;
+    case ORC_I16: return (uint32_t)(int32_t)(f <= -32768.f ? -32768 : f >= 32767.f ? 32767 : (int32_t)f);
+    case ORC_U32: return f <= 0.f ? 0u : f >= 4294967296.f ? 0xffffffffu : (uint32_t)f;
+    default: return f <= -2147483648.f ? 0x80000000u : f >= 2147483648.f ? 0x7fffffffu : (uint32_t)(int32_t)f;
+  }
+}
+
+int orc_move(const uint32_t *shape, uint32_t rank, const int dtypes[2], const orc_layout *layouts[2],
+             const void *in, void *out) {
+  int bad_i, bad_o;
+  int64_t *ti = offset_table(layouts ? layouts[0] : NULL, shape, rank, &bad_i);
+  int64_t *to = offset_table(layouts ? layouts[1] : NULL, shape, rank, &bad_o);
+  if (bad_i || bad_o) {
+    free(ti), free(to);
+    return ORC_BAD_LAYOUT;
+  }
+  const size_t n = volume(shape, rank);
+  const int sdt = dtypes[0], ddt = dtypes[1];
+  for (size_t i = 0; i < n; i++) {
+    const int64_t so = ti ? ti[i] : (int64_t)i, d_o = to ? to[i] : (int64_t)i;
+    if (ddt == ORC_F32) ((float *)out)[d_o] = load_as_f32(in, sdt, so);
+    else if (ddt == ORC_BF16) ((uint16_t *)out)[d_o] = orc_f32_to_bf16(load_as_f32(in, sdt, so));
+    else if (is_float(sdt)) store_from_u32(out, ddt, d_o, float_as_int(load_as_f32(in, sdt, so), ddt));
+    else store_from_u32(out, ddt, d_o, load_as_u32(in, sdt, so, 0));
+  }
+  free(ti), free(to);
+  return ORC_OK;
+}
+
 /* ------------------------------------------------------------ input pattern */
 
 int orc_fill_check_pattern(int dtype, void *dst, size_t count) {

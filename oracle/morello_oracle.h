@@ -129,6 +129,14 @@ int orc_compose_msm(uint32_t b, uint32_t m, uint32_t k, uint32_t n2, uint32_t n,
                     const int dtypes[4], const orc_layout *layouts[4], const void *v,
                     const void *q, const void *kt, float *out);
 
+/* Move Spec (verification.rs:521-532, 547-569: assign_cast = element-wise Rust `as`):
+ * ints wrap to the destination width, floats saturate at the destination's bounds with
+ * NaN -> 0, f32 -> bf16 rounds to nearest even, everything -> f32 as C converts.
+ * Pinned by: numpy `astype` for int->int and int->float, known answers for saturation,
+ * identity and layout round trips. */
+int orc_move(const uint32_t *shape, uint32_t rank, const int dtypes[2], const orc_layout *layouts[2],
+             const void *in, void *out);
+
 /* verification.rs:893-952: ints count up from the dtype minimum and wrap at the maximum;
  * f32 and bf16 cycle 0,1,2,3.  Fills `count` elements in logical row-major order. */
 int orc_fill_check_pattern(int dtype, void *dst, size_t count);

@@ -127,6 +127,14 @@ def compose_msm(b, m, k, n2, n, dtypes, v, q, kt, out, layouts=None):
     return out
 
 
+def move(shape, dtypes, x, out, layouts=None):
+    arr, keep = _layouts(layouts, 2)
+    rc = lib().orc_move(_u32(shape), len(shape), (C.c_int * 2)(*dtypes), arr,
+                        x.ctypes.data_as(C.c_void_p), out.ctypes.data_as(C.c_void_p))
+    assert rc == 0, f"oracle move rc={rc}"
+    return out
+
+
 def check_pattern(dtype, count):
     out = np.empty(count, dtype=NP[dtype])
     assert lib().orc_fill_check_pattern(dtype, out.ctypes.data_as(C.c_void_p), count) == 0

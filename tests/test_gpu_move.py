@@ -1,0 +1,55 @@
+"""Move Spec on the MI355X against the CPU oracle (bit exact), through the C ABI."""
+import numpy as np
+import pytest
+
+import morello_amd as M
+import orc
+from gpu_util import run_spec
+from morello_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def test_move_plain_copy(gpu):
+    for shape, dt in [((1024, 1024), M.f32), ((3, 5, 7), M.u8), ((1,), M.i32), ((4097,), M.i16)]:
+        x = synth.raw_u64(401, 0, int(np.prod(shape))).astype(dt.numpy).reshape(shape)
+        got = run_spec(M.Move(list(shape), (dt, dt)), [x, np.zeros(shape, dt.numpy)])
+        assert np.array_equal(got, x)
+
+
+@pytest.mark.parametrize("sdt,ddt", [(M.i32, M.u8), (M.u8, M.i32), (M.u8, M.f32), (M.f32, M.i8), (M.f32, M.u16),
+                                     (M.f32, M.bf16), (M.bf16, M.f32), (M.i8, M.bf16), (M.bf16, M.i32)])
+def test_move_casts(gpu, sdt, ddt):
+    shape = [5, 129]
+    if sdt == M.f32:
+        x = (synth.normal_f32(402, 0, shape) * 200).astype(np.float32)
+        x[0, :4] = [np.nan, 1e20, -1e20, 0.5]
+    elif sdt == M.bf16:
+        x = synth.f32_to_bf16_bits(synth.normal_f32(402, 0, shape) * 200)
+    else:
+        x = synth.raw_u64(402, 0, 5 * 129).astype(sdt.numpy).reshape(shape)
+    got = run_spec(M.Move(shape, (sdt, ddt)), [x, np.zeros(shape, ddt.numpy)])
+    want = orc.move(shape, [int(sdt), int(ddt)], x, np.zeros(shape, ddt.numpy))
+    assert np.array_equal(got, want)
+
+
+def test_move_relayout(gpu):
+    """The relayouts of examples/matmul_x86.rs:34-53 (layout![0,2,1,2 p(16)]) and NHWC."""
+    shape = [2, 32, 48]
+    x = synth.uniform_i8(403, 0, shape)
+    packed = M.layout(0, 2, 1, (2, M.Packed(16)))
+    got = run_spec(M.Move(shape, (M.i8, M.i8), layouts=[None, packed]), [x, np.zeros(x.size, np.int8)])
+    want = orc.move(shape, [1, 1], x, np.zeros(x.size, np.int8),
+                    layouts=[None, orc.make_layout([0, 2, 1, (2, 1, 16)])])
+    assert np.array_equal(got, want)
+    back = run_spec(M.Move(shape, (M.i8, M.i8), layouts=[packed, None]), [got, np.zeros(shape, np.int8)])
+    assert np.array_equal(back, x)
+    img = synth.uniform_u8(404, 0, (2, 3, 5, 7))
+    got = run_spec(M.Move([2, 3, 5, 7], (M.u8, M.u8), layouts=[None, M.nhwc([2, 3, 5, 7])]),
+                   [img, np.zeros((2, 5, 7, 3), np.uint8)])
+    assert np.array_equal(got, img.transpose(0, 2, 3, 1))
+    oe = M.layout(0, 1, (1, M.OddEven(8)))
+    y = synth.uniform_u8(405, 0, (3, 16))
+    got = run_spec(M.Move([3, 16], (M.u8, M.u8), layouts=[None, oe]), [y, np.zeros(48, np.uint8)])
+    want = orc.move([3, 16], [0, 0], y, np.zeros(48, np.uint8), layouts=[None, orc.make_layout([0, 1, (1, 2, 8)])])
+    assert np.array_equal(got, want)

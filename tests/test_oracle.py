@@ -317,3 +317,42 @@ def test_compose_msm_vs_float64():
     out2 = np.zeros((b, m, n), np.float32)
     orc.compose_msm(b, m, k, n2, n, [orc.BF16, orc.BF16, orc.BF16, orc.F32], v, q, kt, out2)
     assert np.array_equal(out, out2)
+
+
+# ---- move ------------------------------------------------------------------------------
+
+def test_move_casts_vs_numpy_and_known_answers():
+    shape = [3, 37]
+    n = 3 * 37
+    # int -> int wraps, int -> float converts: numpy astype does the same
+    for sdt, ddt in [(orc.I32, orc.U8), (orc.U8, orc.I8), (orc.I16, orc.U32), (orc.U32, orc.I16),
+                     (orc.I8, orc.F32), (orc.U32, orc.F32), (orc.I16, orc.I16)]:
+        x = rand_ints(sdt, 21, 0, shape)
+        got = orc.move(shape, [sdt, ddt], x, np.zeros(shape, orc.NP[ddt]))
+        assert np.array_equal(got, x.astype(orc.NP[ddt])), (sdt, ddt)
+    # float -> int saturates at the destination's bounds, NaN -> 0 (Rust `as`)
+    x = np.array([300.7, -5.2, 127.9, -128.5, np.nan, 1e20, -1e20, 0.99], np.float32).reshape(1, 8)
+    assert list(orc.move([1, 8], [orc.F32, orc.U8], x, np.zeros((1, 8), np.uint8))[0]) == [255, 0, 127, 0, 0, 255, 0, 0]
+    assert list(orc.move([1, 8], [orc.F32, orc.I8], x, np.zeros((1, 8), np.int8))[0]) == [127, -5, 127, -128, 0, 127, -128, 0]
+    assert list(orc.move([1, 8], [orc.F32, orc.I32], x, np.zeros((1, 8), np.int32))[0]) == \
+        [300, -5, 127, -128, 0, 2**31 - 1, -2**31, 0]
+    # f32 -> bf16 rounds to nearest even; bf16 -> f32 is exact
+    f = synth.normal_f32(22, 0, (n,)).reshape(shape)
+    b = orc.move(shape, [orc.F32, orc.BF16], f, np.zeros(shape, np.uint16))
+    assert np.array_equal(b, synth.f32_to_bf16_bits(f))
+    assert np.array_equal(orc.move(shape, [orc.BF16, orc.F32], b, np.zeros(shape, np.float32)),
+                          synth.bf16_bits_to_f32(b))
+
+
+def test_move_relayout_round_trip():
+    shape = [4, 6, 8]
+    x = synth.uniform_u8(23, 0, shape)
+    packed = orc.make_layout([0, 2, 1, (2, 1, 4)])      # layout![0,2,1,2 p(4)]
+    mid = orc.move(shape, [orc.U8, orc.U8], x, np.zeros(x.size, np.uint8), layouts=[None, packed])
+    for pt in [(0, 0, 0), (1, 2, 3), (3, 5, 7)]:
+        assert mid[orc.buffer_index(packed, shape, list(pt))] == x[pt]
+    back = orc.move(shape, [orc.U8, orc.U8], mid, np.zeros(shape, np.uint8), layouts=[packed, None])
+    assert np.array_equal(back, x)
+    col = orc.make_layout([2, 1, 0])
+    t = orc.move(shape, [orc.U8, orc.U8], x, np.zeros(x.size, np.uint8), layouts=[None, col])
+    assert np.array_equal(t.reshape(8, 6, 4), x.transpose(2, 1, 0))
