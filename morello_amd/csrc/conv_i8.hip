@@ -9,7 +9,8 @@
 //
 // Memory-level mapping: the whole filter bank (F x FH x FW x C bytes, 36 KiB for the
 // 64x3x3x64 case) is moved once per wavefront into VGPRs (move_param(1, VRF) hoisted out of
-// every loop); image pixels go straight from global memory into MFMA operand registers
+// every loop, staged through LDS so the bank crosses L2 once per workgroup); image pixels
+// go straight from global memory into MFMA operand registers, one tile ahead of the MFMAs
 // (channels are the fastest NHWC dim, so one pixel's 64 channels are 64 contiguous bytes
 // = four lanes x 16 B); the accumulators start at zero (to_accum) and each output pixel is
 // written once, 16 B per lane.  The kernel is bound by the 4-byte-per-element output
@@ -25,42 +26,22 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 
 constexpr int FT = 4;  // filter tiles of 16 -> F = 64
+#ifndef CONV_WAVES
+#define CONV_WAVES 4
+#endif
 
-template <int SLABS, bool IMG_UNSIGNED>
-__global__ __launch_bounds__(256) void k_conv_i8(ConvArgs p, uint32_t pixels, uint32_t tiles) {
+template <int SLABS, bool IMG_UNSIGNED, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void k_conv_i8(ConvArgs p, uint32_t pixels, uint32_t tiles) {
+  // The filter bank, staged once per workgroup: rows of krow bytes, 16-byte chunks.
+  extern __shared__ __attribute__((aligned(16))) uint8_t filt_lds[];
   const int lane = threadIdx.x & 63;
-  const uint32_t wave = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const uint32_t nwaves = gridDim.x * 4;
+  constexpr int NT = 64 * WAVES;
+  const uint32_t wave = blockIdx.x * WAVES + (threadIdx.x >> 6);
+  const uint32_t nwaves = gridDim.x * WAVES;
   const int li = lane & 15, lg = lane >> 4;
   const int H = p.oh + p.fh - 1, W = p.ow + p.fw - 1;
   const int sub = p.c / 64;  // 64-channel slabs per filter position
-
-  // Filter bank -> registers.  Slab s covers filter position (s / sub) and channels
-  // 64*(s % sub) .. +63; lane (li, lg) holds filter row ft*16+li, bytes 16*lg .. +15.
-  v4i filt[FT][SLABS];
-  const uint8_t *fbase = (const uint8_t *)p.filters;
   const int krow = p.fh * p.fw * p.c;  // bytes per filter
-#pragma unroll
-  for (int ft = 0; ft < FT; ft++)
-#pragma unroll
-    for (int s = 0; s < SLABS; s++)
-      filt[ft][s] = *(const v4i *)(fbase + (ft * 16 + li) * krow + s * 64 + lg * 16);
-
-  int corr[FT][4];
-  if (IMG_UNSIGNED) {
-#pragma unroll
-    for (int ft = 0; ft < FT; ft++) {
-      int sum = 0;
-#pragma unroll
-      for (int s = 0; s < SLABS; s++)
-#pragma unroll
-        for (int w = 0; w < 4; w++) sum = __builtin_amdgcn_sdot4(filt[ft][s][w], 0x01010101, sum, false);
-      sum += __shfl_xor(sum, 16);
-      sum += __shfl_xor(sum, 32);  // every lane with the same li now has filter ft*16+li
-#pragma unroll
-      for (int r = 0; r < 4; r++) corr[ft][r] = 128 * __shfl(sum, lg * 4 + r);
-    }
-  }
 
   // Byte offset of each slab's source relative to the pixel's own (y, x) position.
   int slab_off[SLABS];
@@ -69,39 +50,107 @@ __global__ __launch_bounds__(256) void k_conv_i8(ConvArgs p, uint32_t pixels, ui
     const int pos = s / sub, r = pos / p.fw, q = pos % p.fw;
     slab_off[s] = (r * W + q) * p.c + (s % sub) * 64 + lg * 16;
   }
-
-  for (uint32_t t = wave; t < tiles; t += nwaves) {
-    uint32_t pix = t * 16 + li;
-    const bool live = pix < pixels;
-    if (!live) pix = pixels - 1;  // clamp: loads stay in bounds, the store is masked
+  // Pixel operand of one tile: lane (li, lg) holds pixel t*16+li, channels 16*lg .. +15 of
+  // every slab.  Out-of-range pixels of the last tile are clamped for the loads and masked
+  // for the store.
+  auto load_tile = [&](uint32_t t, v4i *img) {
+    uint32_t pix = min(t * 16 + li, pixels - 1);
     const uint32_t x = pix % p.ow, y = (pix / p.ow) % p.oh, b = pix / (p.ow * p.oh);
     const uint8_t *src = (const uint8_t *)p.image + (int64_t(b) * H * W + int64_t(y) * W + x) * p.c;
-    v4i img[SLABS];
 #pragma unroll
-    for (int s = 0; s < SLABS; s++) {
-      img[s] = *(const v4i *)(src + slab_off[s]);
-      if (IMG_UNSIGNED) img[s] ^= v4i{int(0x80808080), int(0x80808080), int(0x80808080), int(0x80808080)};
+    for (int s = 0; s < SLABS; s++) img[s] = *(const v4i *)(src + slab_off[s]);
+  };
+
+  // First tile's pixels are requested before anything else: their latency overlaps the
+  // filter staging below.
+  v4i img[SLABS];
+  uint32_t t = wave;
+  if (t < tiles) load_tile(t, img);
+
+  // Filter bank: global -> LDS (coalesced, once per workgroup) -> registers (per wave).
+  // Slab s covers filter position (s / sub) and channels 64*(s % sub) .. +63; lane (li, lg)
+  // holds filter row ft*16+li, bytes 16*lg .. +15 of the slab.
+  {
+    // 64 filters x (SLABS * 64) bytes = SLABS * 256 chunks of 16 bytes: all loads are
+    // issued before the first store so they share one round trip.
+    constexpr int PER_THREAD = (SLABS * 256 + NT - 1) / NT;
+    const uint8_t *fbase = (const uint8_t *)p.filters;
+    v4i stage[PER_THREAD];
+#pragma unroll
+    for (int i = 0; i < PER_THREAD; i++) {
+      const int c = i * NT + threadIdx.x;
+      if (c < SLABS * 256) stage[i] = *(const v4i *)(fbase + c * 16);
     }
+#pragma unroll
+    for (int i = 0; i < PER_THREAD; i++) {
+      const int c = i * NT + threadIdx.x;
+      if (c < SLABS * 256) *(v4i *)(filt_lds + c * 16) = stage[i];
+    }
+  }
+  __syncthreads();
+  v4i filt[FT][SLABS];
+#pragma unroll
+  for (int ft = 0; ft < FT; ft++)
+#pragma unroll
+    for (int s = 0; s < SLABS; s++)
+      filt[ft][s] = *(const v4i *)(filt_lds + (ft * 16 + li) * krow + s * 64 + lg * 16);
+
+  // u8 correction 128 * sum_k filt[f][k], one value per filter, parked in LDS behind a
+  // barrier (every wave computes the same 64 numbers; wave 0 publishes them).
+  int *corr_lds = (int *)filt_lds;
+  if (IMG_UNSIGNED) {
+    int sums[FT];
+#pragma unroll
+    for (int ft = 0; ft < FT; ft++) {
+      int sum = 0;
+#pragma unroll
+      for (int s = 0; s < SLABS; s++)
+#pragma unroll
+        for (int w = 0; w < 4; w++) sum = __builtin_amdgcn_sdot4(filt[ft][s][w], 0x01010101, sum, false);
+      sum += __shfl_xor(sum, 16);
+      sums[ft] = sum + __shfl_xor(sum, 32);  // every lane with the same li has filter ft*16+li
+    }
+    __syncthreads();  // all waves hold their filters in registers: the staging area is free
+    if (threadIdx.x < 16)
+#pragma unroll
+      for (int ft = 0; ft < FT; ft++) corr_lds[ft * 16 + li] = 128 * sums[ft];
+    __syncthreads();
+  }
+
+  // The pixel registers are refilled slab by slab with the next tile as soon as the MFMAs
+  // of the current tile have consumed them, so the next tile's loads are in flight under
+  // the rest of this tile's MFMAs and its stores.
+  while (t < tiles) {
+    const uint32_t tn = t + nwaves;
+    const uint32_t pix_n = min(min(tn, tiles - 1) * 16 + li, pixels - 1);  // clamped: always loadable
+    const uint32_t xn = pix_n % p.ow, yn = (pix_n / p.ow) % p.oh, bn = pix_n / (p.ow * p.oh);
+    const uint8_t *src_n = (const uint8_t *)p.image + (int64_t(bn) * H * W + int64_t(yn) * W + xn) * p.c;
     v4i acc[FT];
 #pragma unroll
     for (int ft = 0; ft < FT; ft++) acc[ft] = v4i{0, 0, 0, 0};
 #pragma unroll
-    for (int s = 0; s < SLABS; s++)
+    for (int s = 0; s < SLABS; s++) {
+      v4i px = img[s];
+      if (IMG_UNSIGNED) px ^= v4i{int(0x80808080), int(0x80808080), int(0x80808080), int(0x80808080)};
 #pragma unroll
       for (int ft = 0; ft < FT; ft++)
-        acc[ft] = __builtin_amdgcn_mfma_i32_16x16x64_i8(filt[ft][s], img[s], acc[ft], 0, 0, 0);
+        acc[ft] = __builtin_amdgcn_mfma_i32_16x16x64_i8(filt[ft][s], px, acc[ft], 0, 0, 0);
+      img[s] = *(const v4i *)(src_n + slab_off[s]);
+    }
     // D[row = filter 4*lg + r][col = pixel li]: lane owns 4 consecutive filters of its pixel.
-    if (live) {
+    const uint32_t pix = t * 16 + li;
+    if (pix < pixels) {
       int32_t *dst = (int32_t *)p.out + int64_t(pix) * p.f + lg * 4;
 #pragma unroll
       for (int ft = 0; ft < FT; ft++) {
         v4i v = acc[ft];
-        if (IMG_UNSIGNED) v += v4i{corr[ft][0], corr[ft][1], corr[ft][2], corr[ft][3]};
+        if (IMG_UNSIGNED) v += *(const v4i *)(corr_lds + ft * 16 + lg * 4);
         v4i *d = (v4i *)(dst + ft * 16);
         if (p.accum) v += *d;
-        *d = v;
+        __builtin_nontemporal_store(v, d);  // written once, never re-read by this kernel
       }
     }
+    t = tn;
   }
 }
 
@@ -109,13 +158,16 @@ template <int SLABS>
 hipError_t launch_slabs(const ConvArgs &c, bool img_unsigned, hipStream_t stream) {
   const uint64_t pixels = uint64_t(c.b) * c.oh * c.ow;
   const uint32_t tiles = uint32_t((pixels + 15) / 16);
-  // Two workgroups of four waves per CU on a 256-CU part; never more waves than tiles.
-  uint32_t blocks = 512;
-  if (blocks * 4 > tiles) blocks = (tiles + 3) / 4;
+  // 2048 waves = two per SIMD of a 256-CU part at ~250 VGPRs each, as workgroups of
+  // CONV_WAVES waves (4 measured fastest); never more waves than tiles.
+  constexpr int WAVES = CONV_WAVES;
+  uint32_t blocks = 2048 / WAVES;
+  if (blocks * WAVES > tiles) blocks = (tiles + WAVES - 1) / WAVES;
+  const size_t lds = size_t(FT) * 16 * c.fh * c.fw * c.c;  // the whole filter bank
   if (img_unsigned)
-    hipLaunchKernelGGL((k_conv_i8<SLABS, true>), dim3(blocks), dim3(256), 0, stream, c, uint32_t(pixels), tiles);
+    hipLaunchKernelGGL((k_conv_i8<SLABS, true, WAVES>), dim3(blocks), dim3(64 * WAVES), lds, stream, c, uint32_t(pixels), tiles);
   else
-    hipLaunchKernelGGL((k_conv_i8<SLABS, false>), dim3(blocks), dim3(256), 0, stream, c, uint32_t(pixels), tiles);
+    hipLaunchKernelGGL((k_conv_i8<SLABS, false, WAVES>), dim3(blocks), dim3(64 * WAVES), lds, stream, c, uint32_t(pixels), tiles);
   return hipGetLastError();
 }
 
