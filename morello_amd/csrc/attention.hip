@@ -6,17 +6,23 @@
 // with no scale and no mask, one independent problem per batch entry.
 //
 // The reference materialises S and P in memory between three loop nests
-// (matmul_chain.rs:60-81).  Here a workgroup owns 128 query rows of one batch entry and
-// streams blocks of 64 keys: S^T = K.Q^T is formed on the bf16 MFMA, folded into a running
-// (max, denominator) per query with the online update of morello/src/spec.rs:96-123
+// (matmul_chain.rs:60-81).  Here a 512-thread workgroup owns 128 query rows of one batch
+// entry: four waves take 32 queries each over the first half of the keys, four more take
+// the same queries over the second half (the parallel split of
+// morello/src/scheduling/parallel_softmax.rs:31-223, with k = n2/2).  Each wave streams
+// blocks of 64 keys: S^T = K.Q^T is formed on the bf16 MFMA, folded into a running
+// (max, denominator) per query with the online update of morello/src/spec.rs:96-106
 // (new = max(old, x); d = d*exp(old-new) + exp(x-new)), and P^T (rounded to bf16, the one
 // deviation from the f32 closed form; at most 2^-9 relative per element) feeds the second
-// MFMA as O^T += V^T.P^T.  S and P never reach HBM: traffic is Q, K, V once and the
-// output once.
+// MFMA as O^T += V^T.P^T.  At the end the two halves' (max, denominator, O) triples are
+// merged with SoftmaxDenominatorAndMaxFromParts' formula (morello/src/spec.rs:107-132).
+// S and P never reach HBM: traffic is Q, K, V once and the output once.
 //
 // Both products are formed transposed so that a lane owns one query column: the running
 // max, the denominator and the rescale factor are per-lane scalars, and a row reduction is
-// 32 in-register values plus one cross-lane exchange.
+// 32 in-register values plus one cross-lane exchange.  K and V blocks go from global memory
+// straight into LDS (no staging registers), double buffered, one barrier per block; the
+// bank-conflict swizzles are applied on the source side of those loads.
 #include "kernels.h"
 
 namespace mrl {
@@ -28,52 +34,66 @@ typedef short v4s __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) v4s lds_v4s;
+typedef __attribute__((address_space(3))) void lds_void;
+typedef __attribute__((address_space(1))) const void global_cvoid;
 
 constexpr int D = 128;        // head dim of both products (k and n of the Compose)
-constexpr int BQ = 128;       // queries per workgroup (4 waves x 32)
+constexpr int BQ = 128;       // queries per workgroup (4 query groups x 32)
 constexpr int BKV = 64;       // keys per block
-constexpr int K_ROW = D * 2;          // 256 B, 16-byte chunks XOR-swizzled by (row & 15)
-constexpr int V_ROW = D * 2 + 64;     // 320 B: 4 rows x 64 B cover all 64 banks
-constexpr int K_BYTES = BKV * K_ROW, V_BYTES = BKV * V_ROW;
+constexpr int ROW = D * 2;    // bytes per K or V row
+constexpr int TILE = BKV * ROW;           // 16 KiB: one K or V block
+constexpr int STAGE = 2 * TILE;           // K block then V block
+constexpr int HALF = 2 * STAGE;           // two stages per key half
+constexpr float LOG2E = 1.44269504088896340736f;
+constexpr float RESCALE_SLACK = 5.0f;  // e^5 = 148
 
 __device__ inline v2i read_tr16(const uint8_t *p) {
   const v4s r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s *)p);
   return __builtin_bit_cast(v2i, r);
 }
 
-__global__ __launch_bounds__(256) void k_attn(AttnArgs p) {
-  __shared__ __attribute__((aligned(16))) uint8_t lds[K_BYTES + V_BYTES];
-  uint8_t *lk = lds, *lv = lds + K_BYTES;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+__global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int qg = wave & 3, half = wave >> 2;  // query group, key half
   const int lq = lane & 31, lg = lane >> 5;
   const int64_t head = blockIdx.y;
-  const int q0 = blockIdx.x * BQ + wave * 32;
+  const int q0 = blockIdx.x * BQ + qg * 32;
+  const int keys_per_half = int(p.n2 / 2);
+  const int nblocks = keys_per_half / BKV;
 
-  const uint8_t *Q = (const uint8_t *)p.q + (head * p.m + q0 + lq) * int64_t(D) * 2;
-  const uint8_t *K = (const uint8_t *)p.kt + head * int64_t(p.n2) * D * 2;
-  const uint8_t *V = (const uint8_t *)p.v + head * int64_t(p.n2) * D * 2;
+  const uint8_t *Q = (const uint8_t *)p.q + (head * p.m + q0 + lq) * int64_t(ROW);
+  const uint8_t *K = (const uint8_t *)p.kt + (head * p.n2 + int64_t(half) * keys_per_half) * ROW;
+  const uint8_t *V = (const uint8_t *)p.v + (head * p.n2 + int64_t(half) * keys_per_half) * ROW;
+  uint8_t *my_lds = lds + half * HALF;
 
   // Q^T operand: lane (query lq, half lg) holds d = 16*step + 8*lg .. +7.
   v4i qf[D / 16];
 #pragma unroll
   for (int s = 0; s < D / 16; s++) qf[s] = *(const v4i *)(Q + s * 32 + lg * 16);
 
-  // Staging: 1024 16-byte chunks each for K and V per block, 4 per thread.
-  int src_off[4], k_dst[4], v_dst[4];
+  // Block staging.  One direct-to-LDS instruction fills 1 KiB = 4 rows; lane l lands in
+  // 16-byte slot l.  K rows are XOR-swizzled by chunk with (row & 15), V rows by 64-byte
+  // unit with (row & 3); each lane fetches the global chunk that belongs in its slot.
+  // The 4 waves of a key half share its 16 + 16 instructions per block.
+  const int ld_row = lane >> 4, ld_pc = lane & 15;
+  uint32_t k_src[4], v_src[4];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
-    const int id = tid + i * 256, row = id >> 4, ch = id & 15;
-    src_off[i] = row * (D * 2) + ch * 16;
-    k_dst[i] = row * K_ROW + ((ch ^ (row & 15)) << 4);
-    v_dst[i] = row * V_ROW + ch * 16;
+    const int q = qg * 4 + i, row = q * 4 + ld_row;
+    k_src[i] = row * ROW + ((ld_pc ^ (row & 15)) << 4);
+    v_src[i] = row * ROW + ((((ld_pc >> 2) ^ (row & 3)) << 6) | ((ld_pc & 3) << 4));
   }
-  v4i kreg[4], vreg[4];
-  auto load_block = [&](int kb) {
-    const int64_t base = int64_t(kb) * BKV * D * 2;
+  auto load_block = [&](int kb, int stage) {
+    const int64_t base = int64_t(kb) * TILE;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      kreg[i] = *(const v4i *)(K + base + src_off[i]);
-      vreg[i] = *(const v4i *)(V + base + src_off[i]);
+      const int q = qg * 4 + i;
+      __builtin_amdgcn_global_load_lds((global_cvoid *)(K + base + k_src[i]),
+                                       (lds_void *)(my_lds + stage * STAGE + q * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((global_cvoid *)(V + base + v_src[i]),
+                                       (lds_void *)(my_lds + stage * STAGE + TILE + q * 1024), 16, 0, 0);
     }
   };
 
@@ -82,101 +102,164 @@ __global__ __launch_bounds__(256) void k_attn(AttnArgs p) {
   for (int t = 0; t < D / 32; t++)
 #pragma unroll
     for (int r = 0; r < 16; r++) o[t][r] = 0.0f;
-  float m_run = -3.40282347e+38f, l_run = 0.0f;  // l_run: this lane's share of the denominator
+  float m_run = -3.0e38f, l_run = 0.0f;  // l_run: this lane's share of the denominator
 
-  const int nblocks = int(p.n2 / BKV);
-  load_block(0);
+  // Fragment addressing that does not depend on the block.
+  const int v_rl = (lane & 15) >> 2;                                   // row within a 4-row read
+  const int v_within = 32 * ((lane >> 4) & 1) + 8 * (lane & 3);        // bytes within a 64-B unit
+
+  load_block(0, 0);
   for (int kb = 0; kb < nblocks; kb++) {
-    __syncthreads();  // everyone is done reading the previous block
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      *(v4i *)(lk + k_dst[i]) = kreg[i];
-      *(v4i *)(lv + v_dst[i]) = vreg[i];
-    }
+    const int stage = kb & 1;
+    // Block kb has landed (the loads are tracked by vmcnt only) and, after the barrier,
+    // every wave is done reading the other stage, which the next block may now overwrite.
+    __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
-    if (kb + 1 < nblocks) load_block(kb + 1);
+    if (kb + 1 < nblocks) load_block(kb + 1, stage ^ 1);
+    const uint8_t *lk = my_lds + stage * STAGE, *lv = lk + TILE;
 
     // S^T tiles: s[kt][r] is key kt*32 + 8*(r/4) + 4*lg + r%4, query lq.
+    // All K operands of the block are requested up front (LDS latency paid once, not per
+    // MFMA), and the two key tiles' accumulation chains alternate so that no MFMA waits
+    // for the result of the one just before it.
     v16f s[BKV / 32];
+    v4i kf[BKV / 32][D / 16];
 #pragma unroll
-    for (int kt = 0; kt < BKV / 32; kt++) {
+    for (int st = 0; st < D / 16; st++)
+#pragma unroll
+      for (int kt = 0; kt < BKV / 32; kt++) {
+        const int row = kt * 32 + lq;
+        kf[kt][st] = *(const v4i *)(lk + row * ROW + (((2 * st + lg) ^ (row & 15)) << 4));
+      }
+#pragma unroll
+    for (int kt = 0; kt < BKV / 32; kt++)
 #pragma unroll
       for (int r = 0; r < 16; r++) s[kt][r] = 0.0f;
-      const int row = kt * 32 + lq;
 #pragma unroll
-      for (int st = 0; st < D / 16; st++) {
-        const v4i kf = *(const v4i *)(lk + row * K_ROW + (((2 * st + lg) ^ (row & 15)) << 4));
-        s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, kf),
+    for (int st = 0; st < D / 16; st++)
+#pragma unroll
+      for (int kt = 0; kt < BKV / 32; kt++)
+        s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, kf[kt][st]),
                                                         __builtin_bit_cast(v8bf, qf[st]), s[kt], 0, 0, 0);
-      }
-    }
-    // Online softmax update for this lane's query.
+    // Keep that order in the instruction stream: all LDS reads, then the MFMAs.
+    __builtin_amdgcn_sched_group_barrier(0x100, BKV / 32 * (D / 16), 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, BKV / 32 * (D / 16), 0);
+    // Online softmax update for this lane's query, in base 2: exp(x - m) = 2^(x*log2e - m*log2e).
     float mx = s[0][0];
 #pragma unroll
     for (int kt = 0; kt < BKV / 32; kt++)
 #pragma unroll
       for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[kt][r]);
     mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float m_new = fmaxf(m_run, mx);
-    const float alpha = __expf(m_run - m_new);
-    m_run = m_new;
+    // The reference point m_run only moves when some query's max outgrows it by more than
+    // RESCALE_SLACK: until then exp(x - m_run) <= e^RESCALE_SLACK stays comfortably inside
+    // bf16/f32 range, the final division by the denominator (accumulated against the same
+    // reference) cancels the offset exactly, and the 64 accumulator multiplies of a rescale
+    // are skipped for almost every block.
+    if (__any(mx > m_run + RESCALE_SLACK)) {
+      const float m_new = fmaxf(m_run, mx);
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * LOG2E);
+      m_run = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int t = 0; t < D / 32; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[t][r] *= alpha;
+    }
+    const float neg_m2 = -m_run * LOG2E;
     float psum = 0.0f;
     v8bf pb[BKV / 16];
 #pragma unroll
     for (int kt = 0; kt < BKV / 32; kt++)
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        const float e = __expf(s[kt][r] - m_new);
+        const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][r], LOG2E, neg_m2));
         psum += e;
         pb[kt * 2 + r / 8][r % 8] = (__bf16)e;
       }
-    l_run = l_run * alpha + psum;
-    if (__any(alpha != 1.0f)) {
-#pragma unroll
-      for (int t = 0; t < D / 32; t++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) o[t][r] *= alpha;
-    }
+    l_run += psum;
     // O^T += V^T . P^T.  Key step u covers keys 16u + {4*lg + c, 8 + 4*lg + c}, c = 0..3,
     // which is the order P^T's registers already have.
-#pragma unroll
-    for (int u = 0; u < BKV / 16; u++) {
-      const int key0 = 16 * u + 4 * lg + ((lane & 15) >> 2);
+    // V operands one key step ahead of the MFMAs that use them.
+    v4i vf[2][D / 32];
+    auto read_v = [&](int u, int buf) {
+      const int key = 16 * u + 4 * lg + v_rl;  // key & 3 == v_rl
 #pragma unroll
       for (int t = 0; t < D / 32; t++) {
-        const int col = t * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-        const v2i lo = read_tr16(lv + key0 * V_ROW + col * 2);
-        const v2i hi = read_tr16(lv + (key0 + 8) * V_ROW + col * 2);
-        const v4i vf = v4i{lo[0], lo[1], hi[0], hi[1]};
-        o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, vf), pb[u], o[t], 0, 0, 0);
+        const int off = ((t ^ v_rl) << 6) + v_within;
+        const v2i lo = read_tr16(lv + key * ROW + off);
+        const v2i hi = read_tr16(lv + (key + 8) * ROW + off);
+        vf[buf][t] = v4i{lo[0], lo[1], hi[0], hi[1]};
       }
+    };
+    read_v(0, 0);
+#pragma unroll
+    for (int u = 0; u < BKV / 16; u++) {
+      if (u + 1 < BKV / 16) read_v(u + 1, (u + 1) & 1);
+#pragma unroll
+      for (int t = 0; t < D / 32; t++)
+        o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, vf[u & 1][t]), pb[u], o[t], 0, 0, 0);
+    }
+    // Order: reads of step 0; then per step the reads of the next step ahead of its MFMAs.
+    __builtin_amdgcn_sched_group_barrier(0x100, 2 * (D / 32), 1);
+#pragma unroll
+    for (int u = 0; u < BKV / 16; u++) {
+      if (u + 1 < BKV / 16) __builtin_amdgcn_sched_group_barrier(0x100, 2 * (D / 32), 1);
+      __builtin_amdgcn_sched_group_barrier(0x008, D / 32, 1);
     }
   }
 
-  const float denom = l_run + __shfl_xor(l_run, 32);
-  const float inv = 1.0f / denom;
-  float *out = p.out + (head * p.m + q0 + lq) * int64_t(D);
+  // Merge the two key halves: (m, d, O) of half 1 goes through LDS to the wave of half 0
+  // that owns the same queries.  Layout [value][lane] keeps lanes on distinct banks.
+  float l_tot = l_run + __shfl_xor(l_run, 32);
+  __syncthreads();  // all K/V reads are done: the staging area is free
+  float *mbuf = (float *)lds + qg * (66 * 64);
+  if (half == 1) {
 #pragma unroll
-  for (int t = 0; t < D / 32; t++)
+    for (int t = 0; t < D / 32; t++)
 #pragma unroll
-    for (int a = 0; a < 4; a++) {
-      float4 v;
-      v.x = o[t][4 * a + 0] * inv, v.y = o[t][4 * a + 1] * inv;
-      v.z = o[t][4 * a + 2] * inv, v.w = o[t][4 * a + 3] * inv;
-      *(float4 *)(out + t * 32 + 8 * a + 4 * lg) = v;
-    }
+      for (int r = 0; r < 16; r++) mbuf[(t * 16 + r) * 64 + lane] = o[t][r];
+    mbuf[64 * 64 + lane] = m_run;
+    mbuf[65 * 64 + lane] = l_tot;
+  }
+  __syncthreads();
+  if (half == 0) {
+    const float m1 = mbuf[64 * 64 + lane], l1 = mbuf[65 * 64 + lane];
+    const float m = fmaxf(m_run, m1);
+    const float a0 = __builtin_amdgcn_exp2f((m_run - m) * LOG2E), a1 = __builtin_amdgcn_exp2f((m1 - m) * LOG2E);
+    const float inv = 1.0f / (l_tot * a0 + l1 * a1);
+    const float w0 = a0 * inv, w1 = a1 * inv;
+    float *out = p.out + (head * p.m + q0 + lq) * int64_t(D);
+#pragma unroll
+    for (int t = 0; t < D / 32; t++)
+#pragma unroll
+      for (int a = 0; a < 4; a++) {
+        float4 v;
+        v.x = o[t][4 * a + 0] * w0 + mbuf[(t * 16 + 4 * a + 0) * 64 + lane] * w1;
+        v.y = o[t][4 * a + 1] * w0 + mbuf[(t * 16 + 4 * a + 1) * 64 + lane] * w1;
+        v.z = o[t][4 * a + 2] * w0 + mbuf[(t * 16 + 4 * a + 2) * 64 + lane] * w1;
+        v.w = o[t][4 * a + 3] * w0 + mbuf[(t * 16 + 4 * a + 3) * 64 + lane] * w1;
+        *(float4 *)(out + t * 32 + 8 * a + 4 * lg) = v;
+      }
+  }
 }
 
 }  // namespace
 
 bool attn_applicable(const AttnArgs &a) {
   auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-  return a.k == D && a.n == D && a.m % BQ == 0 && a.n2 % BKV == 0 && a.m && a.n2 && a.b &&
+  return a.k == D && a.n == D && a.m % BQ == 0 && a.n2 % (2 * BKV) == 0 && a.m && a.n2 && a.b &&
          a.b <= 65535 && al16(a.q) && al16(a.kt) && al16(a.v) && al16(a.out);
 }
 
 hipError_t launch_attn(const AttnArgs &a, hipStream_t stream) {
-  hipLaunchKernelGGL(k_attn, dim3(a.m / BQ, a.b), dim3(256), 0, stream, a);
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void *)k_attn, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * HALF);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(k_attn, dim3(a.m / BQ, a.b), dim3(512), 2 * HALF, stream, a);
   return hipGetLastError();
 }
 

@@ -300,7 +300,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void k_gemm(GemmArgs g, int
         Out v = acc[tm][tn][r];
         if (A_UNSIGNED) v += Out(corr[tn]);
         if (g.accum) v += prev[tn][r];
-        c_lane[int64_t(tm * 32 + (r >> 2) * 8 + (r & 3)) * g.ldc + tn * 32] = v;
+        __builtin_nontemporal_store(v, &c_lane[int64_t(tm * 32 + (r >> 2) * 8 + (r & 3)) * g.ldc + tn * 32]);
       }
   }
 }
