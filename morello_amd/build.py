@@ -50,8 +50,15 @@ def build(verbose: bool = True) -> str:
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError("link failed:\n" + res.stderr)
+    # The process-level harness (stand-in for an emitted program) links against the library.
+    harness = os.path.join(HERE, "mrl_harness")
+    cmd = ["g++", "-O2", "-std=c++17", "-Wall", os.path.join(CSRC, "harness_main.cpp"), "-o", harness,
+           "-L" + HERE, "-lmorello_amd", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("harness build failed:\n" + res.stderr)
     if verbose:
-        print(f"built {OUT}")
+        print(f"built {OUT} and {harness}")
     return OUT
 
 
