@@ -34,12 +34,20 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
-constexpr int BM = 256, BN = 256;
-constexpr int BKB = 128;                  // bytes of K per k step, both dtypes
-constexpr int A_STAGE = BM * BKB;         // A tile: [BM][128 B], 16-byte chunks XOR-swizzled
-constexpr int B_STAGE = 36864;            // B tile: padded rows, see Traits
-constexpr int STAGE = A_STAGE + B_STAGE;  // 69632 bytes; two stages = 136 KiB of LDS
 constexpr int GROUP_M = 4;                // tile-rows per L2 group
+
+// Workgroup tile: BM x BN outputs, BKB bytes of K per k step, WAVES_M x WAVES_N waves.
+template <int BM_, int BN_, int BKB_, int WAVES_M_, int WAVES_N_>
+struct Tile {
+  static constexpr int BM = BM_, BN = BN_, BKB = BKB_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+  static constexpr int NT = 64 * WAVES_M * WAVES_N;
+  static constexpr int A_STAGE = BM * BKB;  // A tile: [BM][BKB B], 16-byte chunks XOR-swizzled
+  // B tile: [BK][BN] elements in global orientation, rows padded so that the rows one
+  // transposing read touches fall on different banks (see Traits::PAD).
+  template <class T> static constexpr int b_row() { return BN * T::ES + T::PAD; }
+  template <class T> static constexpr int stage() { return A_STAGE + (BKB / T::ES) * b_row<T>(); }
+};
+typedef Tile<256, 256, 128, 2, 4> TileBig;   // one workgroup per CU, 136 KiB of LDS
 
 typedef __attribute__((address_space(3))) v2i lds_v2i;
 typedef __attribute__((address_space(3))) v4s lds_v4s;
@@ -48,8 +56,7 @@ struct I8 {
   typedef v16i Acc;
   typedef int32_t Out;
   static constexpr int ES = 1;             // element bytes
-  static constexpr int BK = BKB / ES;      // elements of K per k step
-  static constexpr int B_ROW = BN * ES + 32;  // 8 k-rows x 32 B cover all 64 banks
+  static constexpr int PAD = 32;           // 8 k-rows x 32 B cover all 64 banks
   static constexpr int K_PER_READ = 8;     // k rows covered by one transposing read
   __device__ static v2i read_tr(const uint8_t *p) {
     return __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i *)p);
@@ -62,8 +69,7 @@ struct BF16 {
   typedef v16f Acc;
   typedef float Out;
   static constexpr int ES = 2;
-  static constexpr int BK = BKB / ES;
-  static constexpr int B_ROW = BN * ES + 64;  // 4 k-rows x 64 B cover all 64 banks
+  static constexpr int PAD = 64;           // 4 k-rows x 64 B cover all 64 banks
   static constexpr int K_PER_READ = 4;
   __device__ static v2i read_tr(const uint8_t *p) {
     const v4s r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s *)p);
@@ -74,15 +80,17 @@ struct BF16 {
                                                    __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
   }
 };
-static_assert(I8::BK * I8::B_ROW == B_STAGE && BF16::BK * BF16::B_ROW == B_STAGE, "B stage size");
 
-template <class T, bool A_UNSIGNED, int WAVES_M, int WAVES_N>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void k_gemm(GemmArgs g, int tiles_m,
-                                                                 int tiles_n) {
+template <class T, bool A_UNSIGNED, class TL>
+__global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int tiles_n) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-  constexpr int NT = 64 * WAVES_M * WAVES_N;
+  constexpr int BM = TL::BM, BN = TL::BN, BKB = TL::BKB, WAVES_M = TL::WAVES_M, WAVES_N = TL::WAVES_N;
+  constexpr int NT = TL::NT, A_STAGE = TL::A_STAGE;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
-  constexpr int ES = T::ES, BK = T::BK, B_ROW = T::B_ROW;
+  constexpr int ES = T::ES, BK = BKB / ES, B_ROW = TL::template b_row<T>();
+  constexpr int STAGE = TL::template stage<T>();
+  constexpr int A_ROW_CH = BKB / 16;              // 16-byte chunks per A tile row
+  constexpr int A_ROWS_PER_LINE = 256 / BKB;      // A tile rows per 256-byte bank line
   constexpr int A_CH = BM * BKB / 16 / NT;       // 16-byte chunks per thread, A tile
   constexpr int B_ROW_CH = BN * ES / 16;          // chunks per B row
   constexpr int B_CH = BK * B_ROW_CH / NT;        // chunks per thread, B tile
@@ -116,14 +124,16 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void k_gemm(GemmArgs g, int
   // Per-thread staging assignments for one k step.  Thread `tid` moves 16-byte chunk
   // tid + i*NT of each tile; successive i differ by a whole number of rows (a multiple of
   // 16), so one base pointer / LDS offset per operand plus compile-time strides suffices.
-  constexpr int A_ROWS_PER_I = NT / 8, B_ROWS_PER_I = NT / B_ROW_CH;
+  constexpr int A_ROWS_PER_I = NT / A_ROW_CH, B_ROWS_PER_I = NT / B_ROW_CH;
   static_assert(A_ROWS_PER_I % 16 == 0, "swizzle term must not depend on i");
   const uint8_t *a_src;
   int a_dst;
   {
-    const int row = tid >> 3, ch = tid & 7;
+    // 16 lanes of an operand read hit 16 consecutive rows at one chunk index; XOR-ing the
+    // chunk with (row / rows-per-bank-line) spreads them over all 64 banks.
+    const int row = tid / A_ROW_CH, ch = tid % A_ROW_CH;
     a_src = A + int64_t(row) * lda_b + ch * 16;
-    a_dst = row * BKB + ((ch ^ ((row >> 1) & 7)) << 4);
+    a_dst = row * BKB + ((ch ^ ((row / A_ROWS_PER_LINE) & (A_ROW_CH - 1))) << 4);
   }
   const uint8_t *b_src;
   int b_dst;
@@ -138,7 +148,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void k_gemm(GemmArgs g, int
   int a_frag[TM];
 #pragma unroll
   for (int tm = 0; tm < TM; tm++) a_frag[tm] = (wm * WM + tm * 32 + (lane & 31)) * BKB;
-  const int a_swz = ((lane & 31) >> 1) & 7;  // (row >> 1) & 7; WM and 32 are multiples of 16
+  const int a_swz = ((lane & 31) / A_ROWS_PER_LINE) & (A_ROW_CH - 1);  // WM, 32 are multiples of 16
   const int a_half = lane >> 5;
   // Transposing read: a 16-lane group fetches a K_PER_READ x 16 element block; lane p of the
   // group supplies the address of 8 bytes of one k row, and receives the column it indexes.
@@ -305,9 +315,11 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void k_gemm(GemmArgs g, int
   }
 }
 
-template <class T, bool A_UNSIGNED>
+template <class T, bool A_UNSIGNED, class TL>
 hipError_t launch(const GemmArgs &g, hipStream_t stream) {
-  auto kern = k_gemm<T, A_UNSIGNED, 2, 4>;
+  auto kern = k_gemm<T, A_UNSIGNED, TL>;
+  constexpr int BM = TL::BM, BN = TL::BN;
+  constexpr int STAGE = TL::template stage<T>();
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void *)kern,
@@ -316,12 +328,13 @@ hipError_t launch(const GemmArgs &g, hipStream_t stream) {
     attr_set = true;
   }
   const int tiles_m = int(g.m / BM), tiles_n = int(g.n / BN);
-  hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n, g.batch), dim3(512), 2 * STAGE, stream, g,
+  hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n, g.batch), dim3(TL::NT), 2 * STAGE, stream, g,
                      tiles_m, tiles_n);
   return hipGetLastError();
 }
 
 bool applicable(const GemmArgs &g, int es) {
+  constexpr int BM = TileBig::BM, BN = TileBig::BN, BKB = TileBig::BKB;
   auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
   const int64_t per16 = 16 / es;
   return g.m && g.n && g.k && g.m % BM == 0 && g.n % BN == 0 && g.k % (BKB / es) == 0 &&
@@ -336,11 +349,11 @@ bool gemm_i8_applicable(const GemmArgs &g, bool b_k_contiguous) {
   return !b_k_contiguous && applicable(g, 1);
 }
 hipError_t launch_gemm_i8(const GemmArgs &g, bool a_unsigned, hipStream_t stream) {
-  return a_unsigned ? launch<I8, true>(g, stream) : launch<I8, false>(g, stream);
+  return a_unsigned ? launch<I8, true, TileBig>(g, stream) : launch<I8, false, TileBig>(g, stream);
 }
 bool gemm_bf16_applicable(const GemmArgs &g) { return applicable(g, 2); }
 hipError_t launch_gemm_bf16(const GemmArgs &g, hipStream_t stream) {
-  return launch<BF16, false>(g, stream);
+  return launch<BF16, false, TileBig>(g, stream);
 }
 
 }  // namespace mrl
