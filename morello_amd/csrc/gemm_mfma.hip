@@ -81,6 +81,62 @@ struct BF16 {
   }
 };
 
+// Writes one wave's TM x TN blocks of 32 x 32 accumulators to C (adding the u8 correction
+// and, for an accumulating Spec, the previous contents).  `colsum` holds this wave's partial
+// column sums of B; the partials of the PARTS waves that share the columns (and of the two
+// lane halves) are combined through LDS, which every wave must be done reading.
+template <class T, bool A_UNSIGNED, int BN, int PARTS, int TM, int TN>
+__device__ inline void epilogue(const GemmArgs &g, typename T::Out *C, uint8_t *lds,
+                                typename T::Acc (&acc)[TM][TN], int (&colsum)[TN], int lane,
+                                int part_idx, int row0, int col0) {
+  typedef typename T::Out Out;
+  constexpr int WAVES_M = PARTS;
+  const int wm = part_idx;
+  // Epilogue.  Column sums: combine the partials of the WAVES_M waves and two lane halves.
+  int corr[TN];
+#pragma unroll
+  for (int tn = 0; tn < TN; tn++) corr[tn] = 0;
+  if (A_UNSIGNED) {
+    int *part = (int *)lds;  // [WAVES_M * 2][BN]; the k loop ended on a barrier
+    __syncthreads();         // ... and every wave is past its last LDS read of the tiles
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++)
+      part[(wm * 2 + (lane >> 5)) * BN + col0 + tn * 32 + (lane & 31)] = colsum[tn];
+    __syncthreads();
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++) {
+      int sum = 0;
+#pragma unroll
+      for (int w = 0; w < WAVES_M * 2; w++) sum += part[w * BN + col0 + tn * 32 + (lane & 31)];
+      corr[tn] = sum * 128;
+    }
+  }
+  // Lane (l%32, l/32) of accumulator register r owns C[8*(r/4) + 4*(l/32) + r%4][l%32] of
+  // each 32x32 block.  An accumulating Spec reads its whole block row of C first, so the
+  // loads are in flight together instead of one round trip per element.
+  Out *c_lane = C + int64_t(row0 + (lane >> 5) * 4) * g.ldc + col0 + (lane & 31);
+#pragma unroll
+  for (int tm = 0; tm < TM; tm++) {
+    Out prev[TN][16];
+    if (g.accum) {
+#pragma unroll
+      for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+          prev[tn][r] = c_lane[int64_t(tm * 32 + (r >> 2) * 8 + (r & 3)) * g.ldc + tn * 32];
+    }
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        Out v = acc[tm][tn][r];
+        if (A_UNSIGNED) v += Out(corr[tn]);
+        if (g.accum) v += prev[tn][r];
+        __builtin_nontemporal_store(v, &c_lane[int64_t(tm * 32 + (r >> 2) * 8 + (r & 3)) * g.ldc + tn * 32]);
+      }
+  }
+}
+
 template <class T, bool A_UNSIGNED, class TL>
 __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int tiles_n) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -270,49 +326,7 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
     }
   }
 
-  // Epilogue.  Column sums: combine the partials of the WAVES_M waves and two lane halves.
-  int corr[TN];
-#pragma unroll
-  for (int tn = 0; tn < TN; tn++) corr[tn] = 0;
-  if (A_UNSIGNED) {
-    int *part = (int *)lds;  // [WAVES_M * 2][BN]; the k loop ended on a barrier
-    __syncthreads();         // ... and every wave is past its last LDS read of the tiles
-#pragma unroll
-    for (int tn = 0; tn < TN; tn++)
-      part[(wm * 2 + (lane >> 5)) * BN + wn * WN + tn * 32 + (lane & 31)] = colsum[tn];
-    __syncthreads();
-#pragma unroll
-    for (int tn = 0; tn < TN; tn++) {
-      int sum = 0;
-#pragma unroll
-      for (int w = 0; w < WAVES_M * 2; w++) sum += part[w * BN + wn * WN + tn * 32 + (lane & 31)];
-      corr[tn] = sum * 128;
-    }
-  }
-  // Lane (l%32, l/32) of accumulator register r owns C[8*(r/4) + 4*(l/32) + r%4][l%32] of
-  // each 32x32 block.  An accumulating Spec reads its whole block row of C first, so the
-  // loads are in flight together instead of one round trip per element.
-  Out *c_lane = C + int64_t(wm * WM + (lane >> 5) * 4) * g.ldc + wn * WN + (lane & 31);
-#pragma unroll
-  for (int tm = 0; tm < TM; tm++) {
-    Out prev[TN][16];
-    if (g.accum) {
-#pragma unroll
-      for (int tn = 0; tn < TN; tn++)
-#pragma unroll
-        for (int r = 0; r < 16; r++)
-          prev[tn][r] = c_lane[int64_t(tm * 32 + (r >> 2) * 8 + (r & 3)) * g.ldc + tn * 32];
-    }
-#pragma unroll
-    for (int tn = 0; tn < TN; tn++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        Out v = acc[tm][tn][r];
-        if (A_UNSIGNED) v += Out(corr[tn]);
-        if (g.accum) v += prev[tn][r];
-        __builtin_nontemporal_store(v, &c_lane[int64_t(tm * 32 + (r >> 2) * 8 + (r & 3)) * g.ldc + tn * 32]);
-      }
-  }
+  epilogue<T, A_UNSIGNED, BN, WAVES_M, TM, TN>(g, C, lds, acc, colsum, lane, wm, wm * WM, wn * WN);
 }
 
 template <class T, bool A_UNSIGNED, class TL>
