@@ -85,10 +85,10 @@ struct BF16 {
 // and, for an accumulating Spec, the previous contents).  `colsum` holds this wave's partial
 // column sums of B; the partials of the PARTS waves that share the columns (and of the two
 // lane halves) are combined through LDS, which every wave must be done reading.
-template <class T, bool A_UNSIGNED, int BN, int PARTS, int TM, int TN>
+template <class T, bool A_UNSIGNED, bool EDGE, int BN, int PARTS, int TM, int TN>
 __device__ inline void epilogue(const GemmArgs &g, typename T::Out *C, uint8_t *lds,
                                 typename T::Acc (&acc)[TM][TN], int (&colsum)[TN], int lane,
-                                int part_idx, int row0, int col0) {
+                                int part_idx, int row0, int col0, int rows_left, int cols_left) {
   typedef typename T::Out Out;
   constexpr int WAVES_M = PARTS;
   const int wm = part_idx;
@@ -114,7 +114,13 @@ __device__ inline void epilogue(const GemmArgs &g, typename T::Out *C, uint8_t *
   // Lane (l%32, l/32) of accumulator register r owns C[8*(r/4) + 4*(l/32) + r%4][l%32] of
   // each 32x32 block.  An accumulating Spec reads its whole block row of C first, so the
   // loads are in flight together instead of one round trip per element.
-  Out *c_lane = C + int64_t(row0 + (lane >> 5) * 4) * g.ldc + col0 + (lane & 31);
+  // With EDGE the tile may hang over the bottom / right border of C: rows_left and
+  // cols_left bound what this workgroup owns.
+  const int lane_row = row0 + (lane >> 5) * 4, lane_col = col0 + (lane & 31);
+  Out *c_lane = C + int64_t(lane_row) * g.ldc + lane_col;
+  auto inside = [&](int tm, int tn, int r) {
+    return !EDGE || (lane_row + tm * 32 + (r >> 2) * 8 + (r & 3) < rows_left && lane_col + tn * 32 < cols_left);
+  };
 #pragma unroll
   for (int tm = 0; tm < TM; tm++) {
     Out prev[TN][16];
@@ -122,8 +128,10 @@ __device__ inline void epilogue(const GemmArgs &g, typename T::Out *C, uint8_t *
 #pragma unroll
       for (int tn = 0; tn < TN; tn++)
 #pragma unroll
-        for (int r = 0; r < 16; r++)
-          prev[tn][r] = c_lane[int64_t(tm * 32 + (r >> 2) * 8 + (r & 3)) * g.ldc + tn * 32];
+        for (int r = 0; r < 16; r++) {
+          prev[tn][r] = 0;
+          if (inside(tm, tn, r)) prev[tn][r] = c_lane[int64_t(tm * 32 + (r >> 2) * 8 + (r & 3)) * g.ldc + tn * 32];
+        }
     }
 #pragma unroll
     for (int tn = 0; tn < TN; tn++)
@@ -132,12 +140,17 @@ __device__ inline void epilogue(const GemmArgs &g, typename T::Out *C, uint8_t *
         Out v = acc[tm][tn][r];
         if (A_UNSIGNED) v += Out(corr[tn]);
         if (g.accum) v += prev[tn][r];
-        __builtin_nontemporal_store(v, &c_lane[int64_t(tm * 32 + (r >> 2) * 8 + (r & 3)) * g.ldc + tn * 32]);
+        if (inside(tm, tn, r))
+          __builtin_nontemporal_store(v, &c_lane[int64_t(tm * 32 + (r >> 2) * 8 + (r & 3)) * g.ldc + tn * 32]);
       }
   }
 }
 
-template <class T, bool A_UNSIGNED, class TL>
+// EDGE = false: M, N multiples of the tile and K a multiple of the k step.  EDGE = true: any
+// M, any N and K whose rows are whole 16-byte chunks; chunks outside the matrices are fed as
+// zeros (a zero row of B makes the product and the column-sum correction vanish whatever A
+// holds there) and stores outside C are masked.
+template <class T, bool A_UNSIGNED, class TL, bool EDGE>
 __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int tiles_n) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   constexpr int BM = TL::BM, BN = TL::BN, BKB = TL::BKB, WAVES_M = TL::WAVES_M, WAVES_N = TL::WAVES_N;
@@ -230,16 +243,38 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
   for (int tn = 0; tn < TN; tn++) colsum[tn] = 0;
 
   v4i a_reg[A_CH], b_reg[B_CH];
-  const int kt_count = int(g.k / BK);
+  const int kt_count = int((g.k + BK - 1) / BK);
+  // EDGE bookkeeping: what is left of the matrices from this thread's first chunk on.
+  const int k_bytes = int(g.k) * ES;
+  const int a_rows_left = int(g.m - m0) - tid / A_ROW_CH;            // rows of A below the thread's
+  const int a_kb0 = (tid % A_ROW_CH) * 16;                            // its k byte within a tile
+  const int b_cols_left = int(g.n - n0) * ES - (tid % B_ROW_CH) * 16; // bytes of the B row right of it
+  const int b_k0 = tid / B_ROW_CH;                                    // its k row within a tile
+  int ld_kb = 0;  // k byte offset of the tile the next load_global() fetches
 
   // Loads the next tile in sequence and advances the source pointers.
   auto load_global = [&]() {
 #pragma unroll
-    for (int i = 0; i < A_CH; i++) a_reg[i] = *(const v4i *)(a_src + i * a_step_i);
+    for (int i = 0; i < A_CH; i++) {
+      if (EDGE) {
+        a_reg[i] = v4i{0, 0, 0, 0};
+        if (i * A_ROWS_PER_I < a_rows_left && ld_kb + a_kb0 < k_bytes) a_reg[i] = *(const v4i *)(a_src + i * a_step_i);
+      } else {
+        a_reg[i] = *(const v4i *)(a_src + i * a_step_i);
+      }
+    }
 #pragma unroll
-    for (int i = 0; i < B_CH; i++) b_reg[i] = *(const v4i *)(b_src + i * b_step_i);
+    for (int i = 0; i < B_CH; i++) {
+      if (EDGE) {
+        b_reg[i] = v4i{0, 0, 0, 0};
+        if (b_cols_left > 0 && ld_kb / ES + b_k0 + i * B_ROWS_PER_I < int(g.k)) b_reg[i] = *(const v4i *)(b_src + i * b_step_i);
+      } else {
+        b_reg[i] = *(const v4i *)(b_src + i * b_step_i);
+      }
+    }
     a_src += BKB;
     b_src += b_step_kt;
+    ld_kb += BKB;
   };
   auto store_lds = [&](int stage) {
     uint8_t *base = lds + stage * STAGE;
@@ -292,7 +327,7 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
   // and MFMA issue that the text below spells out.
   load_global();
   store_lds(0);
-  if (kt_count < 2) a_src -= BKB, b_src -= b_step_kt;
+  if (kt_count < 2) a_src -= BKB, b_src -= b_step_kt, ld_kb -= BKB;
   load_global();
   __syncthreads();
   read_frags(0, 0, 0);
@@ -300,7 +335,7 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
   for (int kt = 0; kt < kt_count; kt++) {
     const int cur = kt & 1;
     // Tile kt+2 is loaded next (or the last tile again when there is none).
-    if (kt + 2 >= kt_count) a_src -= BKB, b_src -= b_step_kt;
+    if (kt + 2 >= kt_count) a_src -= BKB, b_src -= b_step_kt, ld_kb -= BKB;
 #pragma unroll
     for (int s = 0; s < SLABS; s++) {
       if (s + 1 < SLABS) read_frags(cur, s + 1, (s + 1) & 1);
@@ -326,12 +361,13 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
     }
   }
 
-  epilogue<T, A_UNSIGNED, BN, WAVES_M, TM, TN>(g, C, lds, acc, colsum, lane, wm, wm * WM, wn * WN);
+  epilogue<T, A_UNSIGNED, EDGE, BN, WAVES_M, TM, TN>(g, C, lds, acc, colsum, lane, wm, wm * WM, wn * WN,
+                                                     int(g.m - m0), int(g.n - n0));
 }
 
-template <class T, bool A_UNSIGNED, class TL>
+template <class T, bool A_UNSIGNED, class TL, bool EDGE>
 hipError_t launch(const GemmArgs &g, hipStream_t stream) {
-  auto kern = k_gemm<T, A_UNSIGNED, TL>;
+  auto kern = k_gemm<T, A_UNSIGNED, TL, EDGE>;
   constexpr int BM = TL::BM, BN = TL::BN;
   constexpr int STAGE = TL::template stage<T>();
   static bool attr_set = false;
@@ -341,20 +377,26 @@ hipError_t launch(const GemmArgs &g, hipStream_t stream) {
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  const int tiles_m = int(g.m / BM), tiles_n = int(g.n / BN);
+  const int tiles_m = int((g.m + BM - 1) / BM), tiles_n = int((g.n + BN - 1) / BN);
   hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n, g.batch), dim3(TL::NT), 2 * STAGE, stream, g,
                      tiles_m, tiles_n);
   return hipGetLastError();
 }
 
+// Whole tiles only (the fast instantiation) or any shape whose rows are whole 16-byte chunks.
+bool whole_tiles(const GemmArgs &g, int es) {
+  return g.m % TileBig::BM == 0 && g.n % TileBig::BN == 0 && g.k % (TileBig::BKB / es) == 0;
+}
+
 bool applicable(const GemmArgs &g, int es) {
-  constexpr int BM = TileBig::BM, BN = TileBig::BN, BKB = TileBig::BKB;
   auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
   const int64_t per16 = 16 / es;
-  return g.m && g.n && g.k && g.m % BM == 0 && g.n % BN == 0 && g.k % (BKB / es) == 0 &&
+  constexpr int BM = TileBig::BM, BN = TileBig::BN;
+  // Below a tile's worth of work in either direction the generic kernel is the better fit.
+  return g.m >= 64 && g.n >= 64 && g.k >= 64 && g.n % per16 == 0 && g.k % per16 == 0 &&
          g.lda % per16 == 0 && g.ldb % per16 == 0 && g.sa % per16 == 0 && g.sb % per16 == 0 &&
          al16(g.a) && al16(g.b) && (reinterpret_cast<uintptr_t>(g.c) & 3) == 0 &&
-         g.batch <= 65535 && uint64_t(g.m / BM) * (g.n / BN) < (1u << 30);
+         g.batch <= 65535 && uint64_t((g.m + BM - 1) / BM) * ((g.n + BN - 1) / BN) < (1u << 30);
 }
 
 }  // namespace
@@ -363,11 +405,14 @@ bool gemm_i8_applicable(const GemmArgs &g, bool b_k_contiguous) {
   return !b_k_contiguous && applicable(g, 1);
 }
 hipError_t launch_gemm_i8(const GemmArgs &g, bool a_unsigned, hipStream_t stream) {
-  return a_unsigned ? launch<I8, true, TileBig>(g, stream) : launch<I8, false, TileBig>(g, stream);
+  if (whole_tiles(g, 1))
+    return a_unsigned ? launch<I8, true, TileBig, false>(g, stream) : launch<I8, false, TileBig, false>(g, stream);
+  return a_unsigned ? launch<I8, true, TileBig, true>(g, stream) : launch<I8, false, TileBig, true>(g, stream);
 }
 bool gemm_bf16_applicable(const GemmArgs &g) { return applicable(g, 2); }
 hipError_t launch_gemm_bf16(const GemmArgs &g, hipStream_t stream) {
-  return launch<BF16, false, TileBig>(g, stream);
+  return whole_tiles(g, 2) ? launch<BF16, false, TileBig, false>(g, stream)
+                           : launch<BF16, false, TileBig, true>(g, stream);
 }
 
 }  // namespace mrl

@@ -32,7 +32,11 @@ def int_inputs(seed, dts, b, m, k, n, accum):
     ((1, 512, 384, 768), False),    # several tiles, odd tile counts
     ((3, 256, 256, 512), True),     # batched
     ((1, 1024, 1024, 1024), True),
-    ((1, 100, 37, 51), True),       # ragged: generic kernel
+    ((1, 100, 37, 51), True),       # ragged, rows not whole 16-byte chunks: generic kernel
+    ((1, 300, 208, 272), True),     # ragged, whole chunks: MFMA kernel with masked borders
+    ((2, 257, 144, 1040), False),
+    ((1, 1000, 1008, 1024), True),
+    ((1, 64, 4096, 64), False),     # one sliver of a tile, long K
     ((1, 1, 1, 1), False),
 ])
 def test_int8_matmul_bit_exact(gpu, dts, shape, accum):
@@ -125,7 +129,8 @@ def test_f32_matmul_plumbing_config(gpu):
 
 
 @pytest.mark.parametrize("shape,accum", [((1, 256, 64, 256), False), ((1, 512, 512, 512), True),
-                                         ((2, 256, 192, 256), False), ((1, 60, 100, 36), False)])
+                                         ((2, 256, 192, 256), False), ((1, 60, 100, 36), False),
+                                         ((1, 300, 200, 264), True), ((2, 129, 72, 520), False)])
 def test_bf16_matmul(gpu, shape, accum):
     b, m, k, n = shape
     A, Bm = synth.normal_bf16(51, 0, (b, m, k)), synth.normal_bf16(51, 1, (b, k, n))
