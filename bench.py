@@ -59,6 +59,12 @@ def workload(name):
                 synth.normal_bf16(5, 1, (b, n2, k), 0.5), np.zeros((b, m, n), np.float32)]
         return ("Compose Matmul->Softmax->Matmul, 16 heads, Q/K/V bf16 2048x128, out f32", spec, arrs,
                 "bf16", "TFLOPS", "mfma", PEAK["bf16"])
+    if name == "softmax":
+        # The Softmax stage of the composed pipeline on its own: 16 x 2048 rows of 2048 f32.
+        shape = [16, 2048, 2048]
+        spec = M.Softmax(shape, 2)
+        arrs = [synth.normal_f32(7, 0, tuple(shape), 2.0), np.zeros(tuple(shape), np.float32)]
+        return ("Softmax{scan_dim 2} f32[16x2048x2048]", spec, arrs, "f32", "GFLOPS", "hbm", PEAK["hbm_gbs"])
     if name == "move":
         # Plain copy of 256 MiB: the known-size kernel the HBM byte counters are scaled by.
         n = 64 * 1024 * 1024
@@ -128,7 +134,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--spec", default="c2", choices=["c2", "c3", "c4", "c5", "move"])
+    ap.add_argument("--spec", default="c2", choices=["c2", "c3", "c4", "c5", "softmax", "move"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -154,6 +160,8 @@ def main():
     value = ops / (ms_per_step * 1e-3) / 1e12
     if args.spec == "move":
         value = alg_bytes / (ms_per_step * 1e-3) / 1e9
+    if args.spec == "softmax":
+        value = ops / (ms_per_step * 1e-3) / 1e9
 
     if bound == "mfma":
         achieved = ops / (kernel_ms * 1e-3) / 1e12
@@ -173,7 +181,7 @@ def main():
         "config": {"workload": desc, "spec": args.spec, "device": M.device_info()["name"]},
         "roofline": roofline,
     }
-    if not args.no_cpu and args.spec != "move":
+    if not args.no_cpu and args.spec not in ("move", "softmax"):
         out["cpu_baseline"] = cpu_baseline(args.spec, arrs)
     print(json.dumps(out))
 

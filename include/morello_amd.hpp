@@ -1,0 +1,229 @@
+// C++ view of the MI355X backend with Morello's own vocabulary.
+//
+// Morello's host side is Rust; this header is its C++ mirror over the C ABI in
+// morello_amd.h, so that code written against the reference's Spec surface reads the same:
+//
+//   reference (Rust)                                   here (C++)
+//   ------------------------------------------------   ---------------------------------
+//   Dtype::{Uint8, .., Bfloat16}      common.rs:15-24   morello::Dtype
+//   PhysDim::{Dynamic, Packed, OddEven} layout.rs:74-81 morello::PhysDim
+//   Layout, row_major, col_major, nhwc layout.rs:67-70,  morello::Layout, row_major(), ...
+//     batched_col_major, layout!       1234-1302
+//   TensorSpec{shape,dtype,aux}     tensorspec.rs:19-32 morello::TensorSpec
+//   PrimitiveSpecType::{Matmul,Conv,Softmax,Move}       morello::SpecType
+//   LogicalSpec / Spec, lspec!/spec!   spec.rs:33-162   morello::Spec, Spec::matmul(...), ...
+//   parameter_shape / parameters     spec.rs:467-583    Spec::parameter_shape / parameters
+//   OperandDirection              spec.rs:1091-1095     morello::OperandDirection
+//   BuiltArtifact::run / bench  codegen/mod.rs:269-341  Spec::run / Spec::run_host / Spec::bench
+//   RunError / BuildError        codegen/mod.rs:66-91   morello::Error (carries the status code)
+//
+// Header-only; link with -lmorello_amd.
+#pragma once
+#include <initializer_list>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "morello_amd.h"
+
+namespace morello {
+
+class Error : public std::runtime_error {
+ public:
+  Error(int status, const std::string &where)
+      : std::runtime_error(where + ": " + mrl_status_string(status) +
+                           (status == MRL_ERR_HIP ? std::string(" (") + mrl_last_error() + ")" : "")),
+        status_(status) {}
+  int status() const { return status_; }
+
+ private:
+  int status_;
+};
+
+inline void check(int status, const char *where) {
+  if (status != MRL_OK) throw Error(status, where);
+}
+
+enum class Dtype : int { Uint8 = 0, Sint8, Uint16, Sint16, Uint32, Sint32, Float32, Bfloat16 };
+inline size_t size_of(Dtype d) { return mrl_dtype_size(int(d)); }
+inline const char *to_string(Dtype d) { return mrl_dtype_name(int(d)); }
+
+enum class OperandDirection : int { In = 0, Out = 1, InOut = 2 };
+
+struct PhysDim {
+  enum Kind : uint8_t { Dynamic = 0, Packed = 1, OddEven = 2 } kind = Dynamic;
+  uint32_t size = 0;
+  static PhysDim dynamic() { return {}; }
+  static PhysDim packed(uint32_t n) { return {Packed, n}; }
+  static PhysDim odd_even(uint32_t n) { return {OddEven, n}; }
+};
+
+using Shape = std::vector<uint32_t>;
+
+class Layout {
+ public:
+  Layout() { c_.ndims = 0; }
+  // `layout![...]`: physical dims slowest to fastest.
+  Layout(std::initializer_list<std::pair<uint8_t, PhysDim>> dims) {
+    if (dims.size() > MRL_MAX_PHYS) throw Error(MRL_ERR_BAD_LAYOUT, "Layout");
+    c_.ndims = 0;
+    for (const auto &d : dims) c_.dims[c_.ndims++] = mrl_physdim{d.first, uint8_t(d.second.kind), d.second.size};
+  }
+  explicit Layout(const mrl_layout &c) : c_(c) {}
+  const mrl_layout &c() const { return c_; }
+  size_t len() const { return c_.ndims; }
+
+  // expand_physical_shape (layout.rs:769-810)
+  Shape physical_shape(const Shape &shape) const {
+    Shape out(c_.ndims);
+    check(mrl_layout_physical_shape(&c_, shape.data(), uint32_t(shape.size()), out.data()), "physical_shape");
+    return out;
+  }
+  bool applies_to_shape(const Shape &shape) const {
+    Shape out(MRL_MAX_PHYS);
+    return mrl_layout_physical_shape(&c_, shape.data(), uint32_t(shape.size()), out.data()) == MRL_OK;
+  }
+  // buffer_indexing_expr (layout.rs:221-272) at a concrete point.
+  int64_t buffer_index(const Shape &shape, const Shape &point) const {
+    const int64_t i = mrl_layout_buffer_index(&c_, shape.data(), uint32_t(shape.size()), point.data());
+    if (i < 0) throw Error(MRL_ERR_BAD_LAYOUT, "buffer_index");
+    return i;
+  }
+
+ private:
+  mrl_layout c_;
+};
+
+inline Layout row_major(const Shape &s) {
+  mrl_layout l;
+  check(mrl_layout_row_major(s.data(), uint32_t(s.size()), &l), "row_major");
+  return Layout(l);
+}
+inline Layout col_major(const Shape &s) {
+  mrl_layout l;
+  check(mrl_layout_col_major(s.data(), uint32_t(s.size()), &l), "col_major");
+  return Layout(l);
+}
+inline Layout batched_col_major(const Shape &s) {
+  mrl_layout l;
+  check(mrl_layout_batched_col_major(s.data(), uint32_t(s.size()), &l), "batched_col_major");
+  return Layout(l);
+}
+inline Layout nhwc(const Shape &s) {
+  mrl_layout l;
+  check(mrl_layout_nhwc(s.data(), uint32_t(s.size()), &l), "nhwc");
+  return Layout(l);
+}
+
+// One parameter's type: tensorspec.rs:19-32 without the memory level (every parameter of a
+// top-level Spec lives in GL, which is HBM here).
+struct TensorSpec {
+  Shape shape;
+  Dtype dtype;
+  Layout layout;
+  size_t volume() const {
+    size_t v = 1;
+    for (uint32_t d : shape) v *= d;
+    return v;
+  }
+  size_t bytes_used() const { return volume() * size_of(dtype); }
+};
+
+enum class SpecType : int { Matmul = 0, Conv = 1, Softmax = 2, ComposeMatmulSoftmaxMatmul = 3, Move = 4 };
+
+class Spec {
+ public:
+  // Matmul{accum} over [b, m, k, n] (spec.rs:480-485).  Layouts default to row-major.
+  static Spec matmul(const Shape &bmkn, Dtype a, Dtype b, Dtype c, bool accum = false) {
+    return make(SpecType::Matmul, bmkn, {a, b, c}, accum, 0, false);
+  }
+  // Conv{accum} over [b, f, c, oh, ow, fh, fw] (spec.rs:486-498).  Layouts default to NHWC /
+  // KRSC (layout![0,2,3,1]).
+  static Spec conv(const Shape &s, Dtype image, Dtype filters, Dtype out, bool accum = false) {
+    return make(SpecType::Conv, s, {image, filters, out}, accum, 0, true);
+  }
+  static Spec softmax(const Shape &shape, uint32_t scan_dim) {
+    return make(SpecType::Softmax, shape, {Dtype::Float32, Dtype::Float32}, false, scan_dim, false);
+  }
+  static Spec move(const Shape &shape, Dtype from, Dtype to) {
+    return make(SpecType::Move, shape, {from, to}, false, 0, false);
+  }
+  // Compose [Matmul, Softmax{2}, Matmul] over [b, m, k, n2, n]; parameters V, Q, KT, out
+  // (spec.rs:3329-3365).
+  static Spec compose_msm(const Shape &bmkn2n, Dtype v, Dtype q, Dtype kt) {
+    return make(SpecType::ComposeMatmulSoftmaxMatmul, bmkn2n, {v, q, kt, Dtype::Float32}, false, 0, false);
+  }
+
+  Spec &with_layout(uint32_t param, const Layout &l) {
+    if (param >= c_.n_params) throw Error(MRL_ERR_BAD_SPEC, "with_layout");
+    c_.layouts[param] = l.c();
+    return *this;
+  }
+
+  size_t parameter_count() const { return c_.n_params; }
+  Shape parameter_shape(uint32_t idx) const {
+    uint32_t shape[MRL_MAX_RANK], rank = 0;
+    check(mrl_spec_parameter_shape(&c_, idx, shape, &rank), "parameter_shape");
+    return Shape(shape, shape + rank);
+  }
+  std::vector<TensorSpec> parameters() const {
+    std::vector<TensorSpec> out;
+    for (uint32_t i = 0; i < c_.n_params; i++)
+      out.push_back(TensorSpec{parameter_shape(i), Dtype(c_.dtypes[i]), Layout(c_.layouts[i])});
+    return out;
+  }
+  OperandDirection parameter_direction(uint32_t idx) const {
+    const int d = mrl_spec_parameter_direction(&c_, idx);
+    if (d < 0) throw Error(MRL_ERR_BAD_SPEC, "parameter_direction");
+    return OperandDirection(d);
+  }
+  uint64_t flops() const { return mrl_spec_ops(&c_); }
+  bool is_supported() const { return mrl_spec_check(&c_) == MRL_OK; }
+  const mrl_spec &c() const { return c_; }
+
+  // Where `kernel(p0, .., pk)` is called: device pointers in parameter order.
+  void run(const std::vector<void *> &device_params) const {
+    if (device_params.size() != c_.n_params) throw Error(MRL_ERR_BAD_SPEC, "run");
+    check(mrl_run(&c_, device_params.data()), "run");
+  }
+  void run_async(const std::vector<void *> &device_params, void *stream) const {
+    if (device_params.size() != c_.n_params) throw Error(MRL_ERR_BAD_SPEC, "run_async");
+    check(mrl_run_async(&c_, device_params.data(), stream), "run_async");
+  }
+  // BuiltArtifact::run_with_input_data without the files: host buffers laid out by each
+  // parameter's layout; written parameters are copied back.
+  void run_host(const std::vector<void *> &host_params) const {
+    if (host_params.size() != c_.n_params) throw Error(MRL_ERR_BAD_SPEC, "run_host");
+    check(mrl_run_host(&c_, host_params.data()), "run_host");
+  }
+  // CodeGen::bench: best inner-loop runtime in nanoseconds over `repeats` trials.
+  double bench(const std::vector<void *> &device_params, uint32_t iters, uint32_t repeats = 10) const {
+    double best = 0, mean = 0;
+    check(mrl_bench(&c_, device_params.data(), iters, repeats, &best, &mean), "bench");
+    return best;
+  }
+
+ private:
+  static Spec make(SpecType t, const Shape &shape, std::initializer_list<Dtype> dts, bool accum,
+                   uint32_t scan_dim, bool channels_last) {
+    Spec s;
+    s.c_ = mrl_spec{};
+    if (shape.size() > MRL_MAX_SPEC_RANK || dts.size() > MRL_MAX_PARAMS) throw Error(MRL_ERR_BAD_SPEC, "Spec");
+    s.c_.kind = int(t), s.c_.accum = accum, s.c_.scan_dim = scan_dim, s.c_.rank = uint32_t(shape.size());
+    for (size_t i = 0; i < shape.size(); i++) s.c_.spec_shape[i] = shape[i];
+    s.c_.n_params = uint32_t(dts.size());
+    uint32_t i = 0;
+    for (Dtype d : dts) s.c_.dtypes[i++] = int(d);
+    for (i = 0; i < s.c_.n_params; i++) {
+      const Shape ps = s.parameter_shape(i);
+      s.c_.layouts[i] = (channels_last ? nhwc(ps) : row_major(ps)).c();
+    }
+    return s;
+  }
+  mrl_spec c_;
+};
+
+inline void init(int device = 0) { check(mrl_init(device), "init"); }
+
+}  // namespace morello

@@ -1,0 +1,50 @@
+// Host-only exercise of include/morello_amd.hpp (no device needed): the same expectations
+// the Python tests assert, through the C++ view.  Built and run by tests/test_cpp_api.py.
+#include <cstdio>
+
+#include "morello_amd.hpp"
+
+#define EXPECT(c)                                            \
+  do {                                                       \
+    if (!(c)) {                                              \
+      std::printf("FAILED: %s (line %d)\n", #c, __LINE__);   \
+      return 1;                                              \
+    }                                                        \
+  } while (0)
+
+int main() {
+  using namespace morello;
+  EXPECT(size_of(Dtype::Bfloat16) == 2 && std::string(to_string(Dtype::Sint8)) == "i8");
+  // layout.rs:2391-2433 and book/src/data_layouts.md:59-99
+  EXPECT(row_major({16, 4}).buffer_index({16, 4}, {3, 2}) == 14);
+  Layout oe{{0, PhysDim::odd_even(8)}};
+  EXPECT(oe.buffer_index({8}, {3}) == 5);
+  Layout packed{{1, PhysDim::dynamic()}, {0, PhysDim::dynamic()}, {1, PhysDim::packed(4)}};
+  EXPECT(packed.buffer_index({6, 8}, {2, 5}) == 24 * (5 / 4) + 4 * 2 + 5 % 4);
+  EXPECT((packed.physical_shape({6, 8}) == Shape{2, 6, 4}));
+  Layout bad{{0, PhysDim::packed(4)}, {1, PhysDim::dynamic()}};
+  EXPECT(bad.applies_to_shape({1, 64}) && !bad.applies_to_shape({8, 64}));  // layout.rs:1470-1527
+  EXPECT(batched_col_major({2, 2, 2, 2}).len() == 4);
+  // spec.rs:480-498, 3329-3365
+  Spec mm = Spec::matmul({32, 2, 3, 3}, Dtype::Uint8, Dtype::Sint8, Dtype::Uint16, true);
+  EXPECT((mm.parameter_shape(1) == Shape{32, 3, 3}));
+  EXPECT(mm.parameter_direction(2) == OperandDirection::InOut);
+  Spec cv = Spec::conv({1, 2, 3, 4, 5, 2, 2}, Dtype::Uint8, Dtype::Sint8, Dtype::Sint32);
+  EXPECT((cv.parameter_shape(0) == Shape{1, 3, 5, 6}) && (cv.parameter_shape(2) == Shape{1, 2, 4, 5}));
+  EXPECT(cv.parameters()[1].bytes_used() == 2 * 3 * 2 * 2);
+  Spec msm = Spec::compose_msm({16, 2048, 128, 2048, 128}, Dtype::Bfloat16, Dtype::Bfloat16, Dtype::Bfloat16)
+                 .with_layout(2, Layout{{0, PhysDim::dynamic()}, {2, PhysDim::dynamic()}, {1, PhysDim::dynamic()}});
+  EXPECT(msm.is_supported() && msm.flops() == 34359738368ull + 335544320ull);
+  EXPECT((msm.parameter_shape(2) == Shape{16, 128, 2048}));
+  EXPECT(Spec::matmul({1, 4096, 4096, 4096}, Dtype::Uint8, Dtype::Sint8, Dtype::Sint32).flops() == 137438953472ull);
+  EXPECT(!Spec::matmul({1, 4, 4, 4}, Dtype::Float32, Dtype::Float32, Dtype::Bfloat16).is_supported());
+  // error behaviour: exceptions carry the status code
+  try {
+    Spec::softmax({4, 4}, 1).parameter_shape(5);
+    EXPECT(false);
+  } catch (const Error &e) {
+    EXPECT(e.status() == MRL_ERR_BAD_SPEC);
+  }
+  std::printf("cpp api ok\n");
+  return 0;
+}

@@ -1,0 +1,18 @@
+"""include/morello_amd.hpp (the C++ mirror of the reference's Spec surface) compiles and its
+host-side answers match the reference's expectations.  No GPU needed."""
+import os
+import subprocess
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_cpp_header_host_surface(tmp_path):
+    exe = tmp_path / "cpp_api_check"
+    lib_dir = os.path.join(ROOT, "morello_amd")
+    cmd = ["g++", "-std=c++17", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"),
+           os.path.join(ROOT, "tests", "cpp_api_check.cpp"), "-o", str(exe), "-L", lib_dir, "-lmorello_amd",
+           f"-Wl,-rpath,{lib_dir}", "-Wl,-rpath,/opt/rocm/lib"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
+    run = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert run.returncode == 0 and "cpp api ok" in run.stdout, run.stdout + run.stderr
