@@ -58,8 +58,14 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int qg = wave & 3, half = wave >> 2;  // query group, key half
   const int lq = lane & 31, lg = lane >> 5;
-  const int64_t head = blockIdx.y;
-  const int q0 = blockIdx.x * BQ + qg * 32;
+  // Workgroups go to the 8 XCDs round-robin.  All query blocks of a batch entry share its K
+  // and V, so a batch entry's blocks are kept on one XCD (one L2) whenever the counts allow:
+  // XCD x takes the x-th run of consecutive (entry, block) pairs.
+  const uint32_t nqb = p.m / BQ, total = nqb * p.b;
+  uint32_t lin = blockIdx.x;
+  if (total % 8 == 0) lin = (lin % 8) * (total / 8) + lin / 8;
+  const int64_t head = lin / nqb;
+  const int q0 = int(lin % nqb) * BQ + qg * 32;
   const int keys_per_half = int(p.n2 / 2);
   const int nblocks = keys_per_half / BKV;
 
@@ -249,7 +255,7 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
 bool attn_applicable(const AttnArgs &a) {
   auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
   return a.k == D && a.n == D && a.m % BQ == 0 && a.n2 % (2 * BKV) == 0 && a.m && a.n2 && a.b &&
-         a.b <= 65535 && al16(a.q) && al16(a.kt) && al16(a.v) && al16(a.out);
+         uint64_t(a.m / BQ) * a.b < (1u << 31) && al16(a.q) && al16(a.kt) && al16(a.v) && al16(a.out);
 }
 
 hipError_t launch_attn(const AttnArgs &a, hipStream_t stream) {
@@ -259,7 +265,7 @@ hipError_t launch_attn(const AttnArgs &a, hipStream_t stream) {
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  hipLaunchKernelGGL(k_attn, dim3(a.m / BQ, a.b), dim3(512), 2 * HALF, stream, a);
+  hipLaunchKernelGGL(k_attn, dim3((a.m / BQ) * a.b), dim3(512), 2 * HALF, stream, a);
   return hipGetLastError();
 }
 
