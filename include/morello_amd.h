@@ -188,6 +188,31 @@ int mrl_compose_msm(uint32_t b, uint32_t m, uint32_t k, uint32_t n2, uint32_t n,
                     int dt_q, int dt_kt, int kt_col_major, const void *v, const void *q,
                     const void *kt, void *out, void *stream);
 
+/* ------------------------------------------------ schedule-driven execution */
+
+/* A Morello manual schedule for a Matmul Spec, reduced to the two steps that have a knob in
+ * the GPU kernel: `tile_out([1, tile_m, tile_n])` (one workgroup per output tile) followed
+ * by `split(split_k)` (elements of K per step of the k loop)
+ * (morello/src/scheduling_sugar.rs:37-132; worked schedules in
+ * morello/examples/simple_matmul_x86.rs:60-100, matmul_x86.rs:27-70).  The memory-level
+ * moves of a CPU schedule (move_param to L1 / RF / VRF) are fixed by the kernel: HBM -> LDS
+ * -> VGPR. */
+typedef struct {
+  uint32_t tile_m, tile_n; /* tile_out */
+  uint32_t split_k;        /* split, in elements of K */
+} mrl_matmul_schedule;
+
+/* Lists the schedules the matrix-core Matmul kernel is built for, for this Spec's dtypes
+ * (u8|i8 x i8 -> i32, bf16 x bf16 -> f32).  Writes up to `cap` entries, returns how many
+ * exist (0 if the Spec has no matrix-core kernel). */
+uint32_t mrl_matmul_schedules(const mrl_spec *spec, mrl_matmul_schedule *out, uint32_t cap);
+
+/* mrl_run_async under a caller-chosen schedule.  MRL_ERR_UNSUPPORTED if the schedule is not
+ * in mrl_matmul_schedules() or the operands do not meet the kernel's alignment rules; the
+ * result is identical to mrl_run's whatever the schedule (integer Specs bit for bit). */
+int mrl_run_matmul_scheduled(const mrl_spec *spec, void *const *params,
+                             const mrl_matmul_schedule *schedule, void *stream);
+
 /* ------------------------------------------------ benchmark protocol (L5) */
 
 /* Mirrors CodeGen::bench / the emitted benchmarking main (codegen/cpu.rs:516-568,

@@ -269,6 +269,19 @@ class Spec:
         _check(B.load().mrl_run_timed(C.byref(self._c), arr, steps, C.byref(ms)), "mrl_run_timed")
         return ms.value
 
+    # -- scheduling sugar (scheduling_sugar.rs:37-132), the subset with a knob in the kernels
+    def available_schedules(self):
+        """[(tile_m, tile_n, split_k)] the matrix-core Matmul kernel is built for."""
+        buf = (B.MatmulScheduleC * 16)()
+        n = B.load().mrl_matmul_schedules(C.byref(self._c), buf, 16)
+        return [(buf[i].tile_m, buf[i].tile_n, buf[i].split_k) for i in range(min(n, 16))]
+
+    def tile_out(self, tile_shape: Sequence[int]) -> "ScheduledMatmul":
+        """`spec.tile_out([1, m, n])`: one workgroup per m x n tile of the output."""
+        if self.kind != SpecKind.Matmul or len(tile_shape) != 3 or tile_shape[0] != 1:
+            raise MorelloError(1, "tile_out")
+        return ScheduledMatmul(self, int(tile_shape[1]), int(tile_shape[2]), None)
+
     def bench(self, ptrs: Sequence[int], iters: int, repeats: int = 10):
         """CodeGen::bench protocol (codegen/mod.rs:133-169): (best, mean) ns per launch."""
         arr = (C.c_void_p * len(ptrs))(*ptrs)
@@ -276,6 +289,25 @@ class Spec:
         _check(B.load().mrl_bench(C.byref(self._c), arr, iters, repeats, C.byref(best), C.byref(mean)),
                "mrl_bench")
         return best.value, mean.value
+
+
+class ScheduledMatmul:
+    """A Matmul Spec under a manual schedule: `spec.tile_out([1, m, n]).split(k)`."""
+
+    def __init__(self, spec: Spec, tile_m: int, tile_n: int, split_k: Optional[int]):
+        self.spec, self.tile_m, self.tile_n, self.split_k = spec, tile_m, tile_n, split_k
+
+    def split(self, k: int) -> "ScheduledMatmul":
+        return ScheduledMatmul(self.spec, self.tile_m, self.tile_n, int(k))
+
+    def run_device(self, ptrs: Sequence[int]):
+        if self.split_k is None:
+            raise MorelloError(1, "schedule needs .split(k)")
+        sched = B.MatmulScheduleC(self.tile_m, self.tile_n, self.split_k)
+        arr = (C.c_void_p * len(ptrs))(*ptrs)
+        _check(B.load().mrl_run_matmul_scheduled(C.byref(self.spec._c), arr, C.byref(sched), None),
+               "mrl_run_matmul_scheduled")
+        synchronize()
 
 
 def Matmul(spec_shape, dtypes, layouts=None, accum=False) -> Spec:

@@ -22,6 +22,10 @@ class LayoutC(C.Structure):
     _fields_ = [("ndims", C.c_uint32), ("dims", PhysDimC * MAX_PHYS)]
 
 
+class MatmulScheduleC(C.Structure):
+    _fields_ = [("tile_m", C.c_uint32), ("tile_n", C.c_uint32), ("split_k", C.c_uint32)]
+
+
 class SpecC(C.Structure):
     _fields_ = [
         ("kind", C.c_int32),
@@ -66,6 +70,8 @@ SIGNATURES = {
     "mrl_softmax": (C.c_int, [_U32P, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p]),
     "mrl_move": (C.c_int, [_U32P, C.c_uint32, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
     "mrl_compose_msm": (C.c_int, [C.c_uint32] * 5 + [C.c_int] * 4 + [C.c_void_p] * 5),
+    "mrl_matmul_schedules": (C.c_uint32, [C.POINTER(SpecC), C.POINTER(MatmulScheduleC), C.c_uint32]),
+    "mrl_run_matmul_scheduled": (C.c_int, [C.POINTER(SpecC), _VPP, C.POINTER(MatmulScheduleC), C.c_void_p]),
     "mrl_bench": (C.c_int, [C.POINTER(SpecC), _VPP, C.c_uint32, C.c_uint32,
                             C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "mrl_run_timed": (C.c_int, [C.POINTER(SpecC), _VPP, C.c_uint32, C.POINTER(C.c_double)]),

@@ -219,7 +219,8 @@ bool as_rows(const mrl::Strided &t, int64_t *ld, int64_t *batch_stride) {
   return *ld >= int64_t(t.shape[2]);
 }
 
-int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws) {
+int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
+               const mrl_matmul_schedule *sched = nullptr) {
   Prepared a, b, c;
   int rc;
   if ((rc = prepare(s, 0, params[0], true, ws, &a)) != MRL_OK) return rc;
@@ -233,6 +234,18 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws) {
                     as_rows(c.t, &g.ldc, &g.sc);
   const int da = s.dtypes[0], db = s.dtypes[1], dc = s.dtypes[2];
   bool done = false;
+  if (sched) {
+    const int kind = (da == MRL_I8 && db == MRL_I8 && dc == MRL_I32)     ? 0
+                     : (da == MRL_U8 && db == MRL_I8 && dc == MRL_I32)   ? 1
+                     : (da == MRL_BF16 && db == MRL_BF16 && dc == MRL_F32) ? 2
+                                                                           : -1;
+    const bool ok = kind >= 0 && rows && (kind == 2 ? mrl::gemm_bf16_applicable(g) : mrl::gemm_i8_applicable(g, false));
+    if (!ok) return MRL_ERR_UNSUPPORTED;
+    hipError_t e = mrl::launch_gemm_scheduled(g, kind, sched->tile_m, sched->tile_n, sched->split_k, ws.stream);
+    if (e == hipErrorInvalidValue) return MRL_ERR_UNSUPPORTED;
+    HIP_TRY(e);
+    return finish_output(c, ws);
+  }
   if (rows && (da == MRL_U8 || da == MRL_I8) && db == MRL_I8 && dc == MRL_I32 &&
       mrl::gemm_i8_applicable(g, false)) {
     HIP_TRY(mrl::launch_gemm_i8(g, da == MRL_U8, ws.stream));
@@ -675,6 +688,32 @@ int mrl_compose_msm(uint32_t b, uint32_t m, uint32_t k, uint32_t n2, uint32_t n,
   }
   void *params[4] = {const_cast<void *>(v), const_cast<void *>(q), const_cast<void *>(kt), out};
   return mrl_run_async(&s, params, stream);
+}
+
+uint32_t mrl_matmul_schedules(const mrl_spec *spec, mrl_matmul_schedule *out, uint32_t cap) {
+  if (!spec || spec->kind != MRL_SPEC_MATMUL || check_spec(spec) != MRL_OK) return 0;
+  const int da = spec->dtypes[0], db = spec->dtypes[1], dc = spec->dtypes[2];
+  int es = 0;
+  if ((da == MRL_U8 || da == MRL_I8) && db == MRL_I8 && dc == MRL_I32) es = 1;
+  if (da == MRL_BF16 && db == MRL_BF16 && dc == MRL_F32) es = 2;
+  if (!es) return 0;
+  const uint32_t n = mrl::gemm_schedule_count();
+  for (uint32_t i = 0; i < n && out && i < cap; i++)
+    mrl::gemm_schedule_at(i, es, &out[i].tile_m, &out[i].tile_n, &out[i].split_k);
+  return n;
+}
+
+int mrl_run_matmul_scheduled(const mrl_spec *spec, void *const *params,
+                             const mrl_matmul_schedule *schedule, void *stream) {
+  if (!schedule || !params) return MRL_ERR_NULL;
+  int rc;
+  if (g_device < 0 && (rc = mrl_init(0)) != MRL_OK) return rc;
+  if ((rc = check_spec(spec)) != MRL_OK) return rc;
+  if (spec->kind != MRL_SPEC_MATMUL) return MRL_ERR_UNSUPPORTED;
+  for (uint32_t i = 0; i < spec->n_params; i++)
+    if (!params[i]) return MRL_ERR_NULL;
+  Workspace ws((hipStream_t)stream);
+  return run_matmul(*spec, params, ws, schedule);
 }
 
 int mrl_bench(const mrl_spec *spec, void *const *params, uint32_t iters, uint32_t repeats,

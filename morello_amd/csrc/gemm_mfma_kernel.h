@@ -1,0 +1,390 @@
+// Matmul on the gfx950 matrix cores: u8|i8 x i8 -> i32 (v_mfma_i32_32x32x32_i8) and
+// bf16 x bf16 -> f32 (v_mfma_f32_32x32x16_bf16), one tile pipeline for both.
+//
+// What it computes is Morello's MatmulAccum on row-major operands
+// (morello/src/spec.rs:480-485): C[i,j] (=0 unless accum) += sum_k A[i,k]*B[k,j].  The
+// integer form matches the emitted C bit for bit (widening Assign, morello/src/target/
+// cpu.rs:2860-2872, then MultAdd, morello/src/codegen/cpu.rs:2114-2124): integer addition
+// is associative, so any tiling of the sum gives the same bits.  The bf16 form widens
+// exactly (a 16-bit shift, codegen/partials/x86/cvtbf16_fp32.c) and accumulates in f32 in
+// a different order than the emitted loop nest, hence a tolerance rather than equality.
+//
+// Memory-level mapping of a Morello schedule onto this kernel:
+//   tile_out(256x256)        -> one workgroup per 256x256 tile of C
+//   split(128 bytes of K)    -> the k loop
+//   move_param(A/B, L1)      -> global -> LDS staging, double buffered
+//   move_param(A/B, VRF)     -> LDS -> MFMA operand registers: ds_read_b128 for A (rows
+//                               run along K) and the transposing ds_read_b64_tr_b8/_b16
+//                               for B (rows run along N), so no relayout pass is needed
+//   to_accum + Zero          -> accumulator registers start at zero; C is read only when
+//                               the Spec accumulates
+//
+// The int8 MFMA multiplies signed bytes.  A u8 operand is fed as a' = a xor 0x80
+// (= a - 128 as i8) and the exact correction 128 * sum_k B[k,j] is added per column in the
+// epilogue; the column sums are accumulated from the B operand registers with v_dot4.
+#pragma once
+#include "kernels.h"
+
+
+namespace mrl {
+namespace gemm {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef short v4s __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+
+constexpr int GROUP_M = 4;                // tile-rows per L2 group
+
+// Workgroup tile: BM x BN outputs, BKB bytes of K per k step, WAVES_M x WAVES_N waves.
+template <int BM_, int BN_, int BKB_, int WAVES_M_, int WAVES_N_>
+struct Tile {
+  static constexpr int BM = BM_, BN = BN_, BKB = BKB_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+  static constexpr int NT = 64 * WAVES_M * WAVES_N;
+  static constexpr int A_STAGE = BM * BKB;  // A tile: [BM][BKB B], 16-byte chunks XOR-swizzled
+  // B tile: [BK][BN] elements in global orientation, rows padded so that the rows one
+  // transposing read touches fall on different banks (see Traits::PAD).
+  template <class T> static constexpr int b_row() { return BN * T::ES + T::PAD; }
+  template <class T> static constexpr int stage() { return A_STAGE + (BKB / T::ES) * b_row<T>(); }
+};
+typedef Tile<256, 256, 128, 2, 4> TileBig;   // one workgroup per CU, 136 KiB of LDS
+
+typedef __attribute__((address_space(3))) v2i lds_v2i;
+typedef __attribute__((address_space(3))) v4s lds_v4s;
+
+struct I8 {
+  typedef v16i Acc;
+  typedef int32_t Out;
+  static constexpr int ES = 1;             // element bytes
+  static constexpr int PAD = 32;           // 8 k-rows x 32 B cover all 64 banks
+  static constexpr int K_PER_READ = 8;     // k rows covered by one transposing read
+  __device__ static v2i read_tr(const uint8_t *p) {
+    return __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i *)p);
+  }
+  __device__ static Acc mfma(v4i a, v4i b, Acc c) {
+    return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+  }
+};
+struct BF16 {
+  typedef v16f Acc;
+  typedef float Out;
+  static constexpr int ES = 2;
+  static constexpr int PAD = 64;           // 4 k-rows x 64 B cover all 64 banks
+  static constexpr int K_PER_READ = 4;
+  __device__ static v2i read_tr(const uint8_t *p) {
+    const v4s r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s *)p);
+    return __builtin_bit_cast(v2i, r);
+  }
+  __device__ static Acc mfma(v4i a, v4i b, Acc c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a),
+                                                   __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+  }
+};
+
+// Writes one wave's TM x TN blocks of 32 x 32 accumulators to C (adding the u8 correction
+// and, for an accumulating Spec, the previous contents).  `colsum` holds this wave's partial
+// column sums of B; the partials of the PARTS waves that share the columns (and of the two
+// lane halves) are combined through LDS, which every wave must be done reading.
+template <class T, bool A_UNSIGNED, bool EDGE, int BN, int PARTS, int TM, int TN>
+__device__ inline void epilogue(const GemmArgs &g, typename T::Out *C, uint8_t *lds,
+                                typename T::Acc (&acc)[TM][TN], int (&colsum)[TN], int lane,
+                                int part_idx, int row0, int col0, int rows_left, int cols_left) {
+  typedef typename T::Out Out;
+  constexpr int WAVES_M = PARTS;
+  const int wm = part_idx;
+  // Epilogue.  Column sums: combine the partials of the WAVES_M waves and two lane halves.
+  int corr[TN];
+#pragma unroll
+  for (int tn = 0; tn < TN; tn++) corr[tn] = 0;
+  if (A_UNSIGNED) {
+    int *part = (int *)lds;  // [WAVES_M * 2][BN]; the k loop ended on a barrier
+    __syncthreads();         // ... and every wave is past its last LDS read of the tiles
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++)
+      part[(wm * 2 + (lane >> 5)) * BN + col0 + tn * 32 + (lane & 31)] = colsum[tn];
+    __syncthreads();
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++) {
+      int sum = 0;
+#pragma unroll
+      for (int w = 0; w < WAVES_M * 2; w++) sum += part[w * BN + col0 + tn * 32 + (lane & 31)];
+      corr[tn] = sum * 128;
+    }
+  }
+  // Lane (l%32, l/32) of accumulator register r owns C[8*(r/4) + 4*(l/32) + r%4][l%32] of
+  // each 32x32 block.  An accumulating Spec reads its whole block row of C first, so the
+  // loads are in flight together instead of one round trip per element.
+  // With EDGE the tile may hang over the bottom / right border of C: rows_left and
+  // cols_left bound what this workgroup owns.
+  const int lane_row = row0 + (lane >> 5) * 4, lane_col = col0 + (lane & 31);
+  Out *c_lane = C + int64_t(lane_row) * g.ldc + lane_col;
+  auto inside = [&](int tm, int tn, int r) {
+    return !EDGE || (lane_row + tm * 32 + (r >> 2) * 8 + (r & 3) < rows_left && lane_col + tn * 32 < cols_left);
+  };
+#pragma unroll
+  for (int tm = 0; tm < TM; tm++) {
+    Out prev[TN][16];
+    if (g.accum) {
+#pragma unroll
+      for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          prev[tn][r] = 0;
+          if (inside(tm, tn, r)) prev[tn][r] = c_lane[int64_t(tm * 32 + (r >> 2) * 8 + (r & 3)) * g.ldc + tn * 32];
+        }
+    }
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        Out v = acc[tm][tn][r];
+        if (A_UNSIGNED) v += Out(corr[tn]);
+        if (g.accum) v += prev[tn][r];
+        if (inside(tm, tn, r))
+          __builtin_nontemporal_store(v, &c_lane[int64_t(tm * 32 + (r >> 2) * 8 + (r & 3)) * g.ldc + tn * 32]);
+      }
+  }
+}
+
+// EDGE = false: M, N multiples of the tile and K a multiple of the k step.  EDGE = true: any
+// M, any N and K whose rows are whole 16-byte chunks; chunks outside the matrices are fed as
+// zeros (a zero row of B makes the product and the column-sum correction vanish whatever A
+// holds there) and stores outside C are masked.
+template <class T, bool A_UNSIGNED, class TL, bool EDGE>
+__global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int tiles_n) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  constexpr int BM = TL::BM, BN = TL::BN, BKB = TL::BKB, WAVES_M = TL::WAVES_M, WAVES_N = TL::WAVES_N;
+  constexpr int NT = TL::NT, A_STAGE = TL::A_STAGE;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
+  constexpr int ES = T::ES, BK = BKB / ES, B_ROW = TL::template b_row<T>();
+  constexpr int STAGE = TL::template stage<T>();
+  constexpr int A_ROW_CH = BKB / 16;              // 16-byte chunks per A tile row
+  constexpr int A_ROWS_PER_LINE = 256 / BKB;      // A tile rows per 256-byte bank line
+  constexpr int A_CH = BM * BKB / 16 / NT;       // 16-byte chunks per thread, A tile
+  constexpr int B_ROW_CH = BN * ES / 16;          // chunks per B row
+  constexpr int B_CH = BK * B_ROW_CH / NT;        // chunks per thread, B tile
+  constexpr int SLABS = BKB / 32;                 // MFMA k steps per tile (32 bytes each)
+  constexpr int K_SLAB = 32 / ES;                 // elements of K per MFMA
+  typedef typename T::Acc Acc;
+  typedef typename T::Out Out;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lives in an SGPR
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+  // Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous run of
+  // tiles, ordered so that a run covers a compact block of C (shared A rows and B columns
+  // stay in that XCD's L2).
+  int pid = blockIdx.x;
+  const int ntiles = tiles_m * tiles_n;
+  if (ntiles % 8 == 0) pid = (pid % 8) * (ntiles / 8) + pid / 8;
+  const int group = pid / (GROUP_M * tiles_n);
+  const int first_m = group * GROUP_M;
+  const int gsz = min(tiles_m - first_m, GROUP_M);
+  const int in_group = pid % (GROUP_M * tiles_n);
+  const int tile_m = first_m + in_group % gsz, tile_n = in_group / gsz;
+  const int64_t m0 = int64_t(tile_m) * BM, n0 = int64_t(tile_n) * BN;
+
+  const uint8_t *A = (const uint8_t *)g.a + (int64_t(blockIdx.y) * g.sa + m0 * g.lda) * ES;
+  const uint8_t *B = (const uint8_t *)g.b + (int64_t(blockIdx.y) * g.sb + n0) * ES;
+  Out *C = (Out *)g.c + int64_t(blockIdx.y) * g.sc + m0 * g.ldc + n0;
+  const int64_t lda_b = g.lda * ES, ldb_b = g.ldb * ES;
+
+  // Per-thread staging assignments for one k step.  Thread `tid` moves 16-byte chunk
+  // tid + i*NT of each tile; successive i differ by a whole number of rows (a multiple of
+  // 16), so one base pointer / LDS offset per operand plus compile-time strides suffices.
+  constexpr int A_ROWS_PER_I = NT / A_ROW_CH, B_ROWS_PER_I = NT / B_ROW_CH;
+  static_assert(A_ROWS_PER_I % 16 == 0, "swizzle term must not depend on i");
+  const uint8_t *a_src;
+  int a_dst;
+  {
+    // 16 lanes of an operand read hit 16 consecutive rows at one chunk index; XOR-ing the
+    // chunk with (row / rows-per-bank-line) spreads them over all 64 banks.
+    const int row = tid / A_ROW_CH, ch = tid % A_ROW_CH;
+    a_src = A + int64_t(row) * lda_b + ch * 16;
+    a_dst = row * BKB + ((ch ^ ((row / A_ROWS_PER_LINE) & (A_ROW_CH - 1))) << 4);
+  }
+  const uint8_t *b_src;
+  int b_dst;
+  {
+    const int row = tid / B_ROW_CH, ch = tid % B_ROW_CH;
+    b_src = B + int64_t(row) * ldb_b + ch * 16;
+    b_dst = A_STAGE + row * B_ROW + ch * 16;
+  }
+  const int64_t a_step_i = int64_t(A_ROWS_PER_I) * lda_b, b_step_i = int64_t(B_ROWS_PER_I) * ldb_b;
+  const int64_t b_step_kt = int64_t(BK) * ldb_b;
+  // Operand fragment offsets within a stage for MFMA k step 0.
+  int a_frag[TM];
+#pragma unroll
+  for (int tm = 0; tm < TM; tm++) a_frag[tm] = (wm * WM + tm * 32 + (lane & 31)) * BKB;
+  const int a_swz = ((lane & 31) / A_ROWS_PER_LINE) & (A_ROW_CH - 1);  // WM, 32 are multiples of 16
+  const int a_half = lane >> 5;
+  // Transposing read: a 16-lane group fetches a K_PER_READ x 16 element block; lane p of the
+  // group supplies the address of 8 bytes of one k row, and receives the column it indexes.
+  int b_frag[TN];
+#pragma unroll
+  for (int tn = 0; tn < TN; tn++) {
+    constexpr int LANES_PER_ROW = 16 / (8 / ES);  // lanes that share one k row: 2 (i8), 4 (bf16)
+    const int p = lane & 15;
+    const int k = (K_SLAB / 2) * (lane >> 5) + p / LANES_PER_ROW;
+    const int col = wn * WN + tn * 32 + 16 * ((lane >> 4) & 1) + (8 / ES) * (p % LANES_PER_ROW);
+    b_frag[tn] = A_STAGE + k * B_ROW + col * ES;
+  }
+
+  Acc acc[TM][TN];
+#pragma unroll
+  for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[tm][tn][r] = 0;
+  int colsum[TN];
+#pragma unroll
+  for (int tn = 0; tn < TN; tn++) colsum[tn] = 0;
+
+  v4i a_reg[A_CH], b_reg[B_CH];
+  const int kt_count = int((g.k + BK - 1) / BK);
+  // EDGE bookkeeping: what is left of the matrices from this thread's first chunk on.
+  const int k_bytes = int(g.k) * ES;
+  const int a_rows_left = int(g.m - m0) - tid / A_ROW_CH;            // rows of A below the thread's
+  const int a_kb0 = (tid % A_ROW_CH) * 16;                            // its k byte within a tile
+  const int b_cols_left = int(g.n - n0) * ES - (tid % B_ROW_CH) * 16; // bytes of the B row right of it
+  const int b_k0 = tid / B_ROW_CH;                                    // its k row within a tile
+  int ld_kb = 0;  // k byte offset of the tile the next load_global() fetches
+
+  // Loads the next tile in sequence and advances the source pointers.
+  auto load_global = [&]() {
+#pragma unroll
+    for (int i = 0; i < A_CH; i++) {
+      if (EDGE) {
+        a_reg[i] = v4i{0, 0, 0, 0};
+        if (i * A_ROWS_PER_I < a_rows_left && ld_kb + a_kb0 < k_bytes) a_reg[i] = *(const v4i *)(a_src + i * a_step_i);
+      } else {
+        a_reg[i] = *(const v4i *)(a_src + i * a_step_i);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < B_CH; i++) {
+      if (EDGE) {
+        b_reg[i] = v4i{0, 0, 0, 0};
+        if (b_cols_left > 0 && ld_kb / ES + b_k0 + i * B_ROWS_PER_I < int(g.k)) b_reg[i] = *(const v4i *)(b_src + i * b_step_i);
+      } else {
+        b_reg[i] = *(const v4i *)(b_src + i * b_step_i);
+      }
+    }
+    a_src += BKB;
+    b_src += b_step_kt;
+    ld_kb += BKB;
+  };
+  auto store_lds = [&](int stage) {
+    uint8_t *base = lds + stage * STAGE;
+#pragma unroll
+    for (int i = 0; i < A_CH; i++) {
+      v4i v = a_reg[i];
+      if (A_UNSIGNED) v ^= v4i{int(0x80808080), int(0x80808080), int(0x80808080), int(0x80808080)};
+      *(v4i *)(base + a_dst + i * A_ROWS_PER_I * BKB) = v;
+    }
+#pragma unroll
+    for (int i = 0; i < B_CH; i++) *(v4i *)(base + b_dst + i * B_ROWS_PER_I * B_ROW) = b_reg[i];
+  };
+  // MFMA operands for one 32-byte k step, double buffered in registers.
+  v4i af[2][TM], bf[2][TN];
+  auto read_frags = [&](int stage, int s, int buf) {
+    const uint8_t *base = lds + stage * STAGE;
+#pragma unroll
+    for (int tm = 0; tm < TM; tm++)
+      af[buf][tm] = *(const v4i *)(base + a_frag[tm] + (((2 * s + a_half) ^ a_swz) << 4));
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++) {
+      const v2i lo = T::read_tr(base + b_frag[tn] + (s * K_SLAB) * B_ROW);
+      const v2i hi = T::read_tr(base + b_frag[tn] + (s * K_SLAB + T::K_PER_READ) * B_ROW);
+      bf[buf][tn] = v4i{lo[0], lo[1], hi[0], hi[1]};
+    }
+  };
+  auto mfma_slab = [&](int s, int buf) {
+    // Column sums of B for the u8 correction: each of the WAVES_M waves that share these
+    // columns takes every WAVES_M-th k step (a scalar branch: `wm` is wave-uniform).
+    if (A_UNSIGNED && (s % WAVES_M) == wm) {
+#pragma unroll
+      for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+        for (int w = 0; w < 4; w++)
+          colsum[tn] = __builtin_amdgcn_sdot4(bf[buf][tn][w], 0x01010101, colsum[tn], false);
+    }
+#pragma unroll
+    for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+      for (int tn = 0; tn < TN; tn++) acc[tm][tn] = T::mfma(af[buf][tm], bf[buf][tn], acc[tm][tn]);
+  };
+
+  // Software pipeline.  While tile kt is multiplied out of LDS stage kt&1, tile kt+1 sits
+  // in registers (its global loads were issued one tile earlier) and is written to the
+  // other stage during the second-to-last k step; the barrier comes before the last k
+  // step's MFMAs, so the first operands of tile kt+1 are fetched under them and the matrix
+  // core does not drain at the barrier.  The body is branch-free: past the end of K the
+  // pointers stop advancing, so the last tile is re-read (L2 hits) and re-staged into the
+  // stage nobody reads any more.  sched_group_barrier pins the interleaving of LDS, VMEM
+  // and MFMA issue that the text below spells out.
+  load_global();
+  store_lds(0);
+  if (kt_count < 2) a_src -= BKB, b_src -= b_step_kt, ld_kb -= BKB;
+  load_global();
+  __syncthreads();
+  read_frags(0, 0, 0);
+
+  for (int kt = 0; kt < kt_count; kt++) {
+    const int cur = kt & 1;
+    // Tile kt+2 is loaded next (or the last tile again when there is none).
+    if (kt + 2 >= kt_count) a_src -= BKB, b_src -= b_step_kt, ld_kb -= BKB;
+#pragma unroll
+    for (int s = 0; s < SLABS; s++) {
+      if (s + 1 < SLABS) read_frags(cur, s + 1, (s + 1) & 1);
+      if (s == SLABS - 2) {
+        store_lds(cur ^ 1);
+        load_global();
+      }
+      if (s == SLABS - 1) {
+        __syncthreads();
+        read_frags(cur ^ 1, 0, 0);
+      }
+      mfma_slab(s, s & 1);
+      // One MFMA, then a share of this step's memory instructions, TM*TN times.
+#pragma unroll
+      for (int i = 0; i < TM * TN; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+        if (i < TM + 2 * TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+        if (s == SLABS - 2) {
+          if (i < A_CH + B_CH) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // DS write
+          if (i < A_CH + B_CH) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // VMEM read
+        }
+      }
+    }
+  }
+
+  epilogue<T, A_UNSIGNED, EDGE, BN, WAVES_M, TM, TN>(g, C, lds, acc, colsum, lane, wm, wm * WM, wn * WN,
+                                                     int(g.m - m0), int(g.n - n0));
+}
+
+template <class T, bool A_UNSIGNED, class TL, bool EDGE>
+hipError_t launch(const GemmArgs &g, hipStream_t stream) {
+  auto kern = k_gemm<T, A_UNSIGNED, TL, EDGE>;
+  constexpr int BM = TL::BM, BN = TL::BN;
+  constexpr int STAGE = TL::template stage<T>();
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void *)kern,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 2 * STAGE);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  const int tiles_m = int((g.m + BM - 1) / BM), tiles_n = int((g.n + BN - 1) / BN);
+  hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n, g.batch), dim3(TL::NT), 2 * STAGE, stream, g,
+                     tiles_m, tiles_n);
+  return hipGetLastError();
+}
+
+
+}  // namespace gemm
+}  // namespace mrl

@@ -52,6 +52,12 @@ hipError_t launch_gemm_i8(const GemmArgs &g, bool a_unsigned, hipStream_t stream
 bool gemm_bf16_applicable(const GemmArgs &g);
 hipError_t launch_gemm_bf16(const GemmArgs &g, hipStream_t stream);
 
+// ---- gemm_sched.hip: the same kernel under a caller-chosen tile_out / split schedule -----
+uint32_t gemm_schedule_count();
+void gemm_schedule_at(uint32_t i, int elem_size, uint32_t *tile_m, uint32_t *tile_n, uint32_t *split_k);
+hipError_t launch_gemm_scheduled(const GemmArgs &g, int kind, uint32_t tile_m, uint32_t tile_n,
+                                 uint32_t split_k, hipStream_t stream);
+
 // ---- conv_i8.hip: NHWC u8|i8 image x KRSC i8 filters -> NHWC i32, implicit GEMM --------
 struct ConvArgs {
   const void *image;

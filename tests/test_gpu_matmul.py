@@ -199,3 +199,41 @@ def test_run_host_entry_point(gpu):
     M.MatmulAccum([b, m, k, n], (M.u8, M.i8, M.i32)).run_host(A, Bm, C1)
     want = orc.matmul([b, m, k, n], [0, 1, 5], A, Bm, np.full((b, m, n), 5, np.int32), True)
     assert np.array_equal(C1, want)
+
+
+def test_manual_schedules_give_identical_results(gpu):
+    """Every tile_out/split schedule the kernel is built for computes the same Spec: bit for
+    bit for the integer Spec, and to f32 rounding for bf16 (the k loop order changes)."""
+    b, m, k, n = 2, 512, 384, 768
+    A, Bm = synth.uniform_u8(91, 0, (b, m, k)), synth.uniform_i8(91, 1, (b, k, n))
+    C0 = synth.uniform_u8(91, 2, (b, m, n)).astype(np.int32)
+    spec = M.MatmulAccum([b, m, k, n], (M.u8, M.i8, M.i32))
+    want = orc.matmul([b, m, k, n], [0, 1, 5], A, Bm, C0.copy(), True)
+    scheds = spec.available_schedules()
+    assert (256, 256, 128) in scheds and len(scheds) >= 4
+    for tm, tn, sk in scheds:
+        bufs = [M.DeviceBuffer.from_numpy(x) for x in (A, Bm, C0)]
+        spec.tile_out([1, tm, tn]).split(sk).run_device([x.ptr for x in bufs])
+        assert np.array_equal(bufs[2].to_numpy(np.int32, (b, m, n)), want), (tm, tn, sk)
+    # ragged problem under a small-tile schedule
+    b, m, k, n = 1, 200, 144, 336
+    A, Bm = synth.uniform_i8(92, 0, (b, m, k)), synth.uniform_i8(92, 1, (b, k, n))
+    spec = M.Matmul([b, m, k, n], (M.i8, M.i8, M.i32))
+    want = orc.matmul([b, m, k, n], [1, 1, 5], A, Bm, np.zeros((b, m, n), np.int32))
+    bufs = [M.DeviceBuffer.from_numpy(x) for x in (A, Bm, np.zeros((b, m, n), np.int32))]
+    spec.tile_out([1, 128, 128]).split(64).run_device([x.ptr for x in bufs])
+    assert np.array_equal(bufs[2].to_numpy(np.int32, (b, m, n)), want)
+    # bf16: split counted in elements (32 bf16 = 64 bytes)
+    b, m, k, n = 1, 256, 256, 512
+    A, Bm = synth.normal_bf16(93, 0, (b, m, k)), synth.normal_bf16(93, 1, (b, k, n))
+    spec = M.Matmul([b, m, k, n], (M.bf16, M.bf16, M.f32))
+    want = orc.matmul([b, m, k, n], [7, 7, 6], A, Bm, np.zeros((b, m, n), np.float32))
+    for tm, tn, sk in spec.available_schedules():
+        bufs = [M.DeviceBuffer.from_numpy(x) for x in (A, Bm, np.zeros((b, m, n), np.float32))]
+        spec.tile_out([1, tm, tn]).split(sk).run_device([x.ptr for x in bufs])
+        assert rel_err(bufs[2].to_numpy(np.float32, (b, m, n)), want) < 1e-5, (tm, tn, sk)
+    # a schedule that is not built, and a Spec without a matrix-core kernel
+    with pytest.raises(M.MorelloError) as e:
+        spec.tile_out([1, 64, 64]).split(32).run_device([x.ptr for x in bufs])
+    assert e.value.status == 1
+    assert M.Matmul([1, 64, 64, 64], [M.f32] * 3).available_schedules() == []
