@@ -80,15 +80,49 @@ typedef enum {
   MRL_SPEC_COMPOSE_MSM = 3,/* Matmul->Softmax->Matmul; spec_shape [b,m,k,n2,n];
                               params V[b,n2,n] Q[b,m,k] KT[b,k,n2] out[b,m,n]
                               (Compose parameter order, spec.rs:3329-3365)               */
-  MRL_SPEC_MOVE = 4        /* Move (spec.rs:57-162; oracle verification.rs assign_cast):
+  MRL_SPEC_MOVE = 4,       /* Move (spec.rs:57-162; oracle verification.rs assign_cast):
                               spec_shape = tensor shape; params in, out; the two may
                               differ in layout and dtype (Rust `as` conversion)          */
+  /* The primitives Softmax decomposes into (spec.rs:86-162).  spec_shape = the full tensor
+   * shape (rank <= 5); "reduced" parameters have size one on scan_dim (spec.rs:524-583).
+   * f32 only.  `accum` as in spec.rs:1214-1241: accumulating forms read their outputs. */
+  MRL_SPEC_FILL = 5,       /* params out; scan_dim holds the mrl_fill_value; any dtype     */
+  MRL_SPEC_MAX = 6,        /* params in, out(reduced): out = max(out?, in) over scan_dim  */
+  MRL_SPEC_SOFTMAX_DENOMINATOR = 7,
+                           /* params in, max(reduced), denom(reduced):
+                              denom (+)= sum exp(in - max)                                */
+  MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX = 8,
+                           /* params in, max(reduced), denom(reduced): online update of
+                              (max, denom) (spec.rs:96-101; cpu.rs:1360-1389)             */
+  MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX_FROM_PARTS = 9,
+                           /* params tile_max, tile_denom (full shape: one entry per tile
+                              along scan_dim), out_max, out_denom (reduced): merges the
+                              per-tile pairs (spec.rs:102-132; cpu.rs:1390-1413)          */
+  MRL_SPEC_SOFTMAX_DENOMINATOR_AND_UNSCALED = 10,
+                           /* params in, denom(reduced), unscaled: unscaled = exp(in-max),
+                              denom = its sum; never accumulates (spec.rs:133-141)        */
+  MRL_SPEC_SOFTMAX_DENOMINATOR_AND_UNSCALED_FROM_MAX = 11,
+                           /* params in, max(reduced), denom(reduced), unscaled
+                              (cpu.rs:1425-1433)                                          */
+  MRL_SPEC_SOFTMAX_COMPLETE = 12,
+                           /* params in, max(reduced), denom(reduced), out:
+                              out = exp(in - max) / denom (cpu.rs:1350-1359)              */
+  MRL_SPEC_DIVIDE_VEC = 13,/* params numer (InOut), denom, same shape: numer /= denom     */
+  MRL_SPEC_DIVIDE_VEC_SCALAR = 14,
+                           /* params numer (InOut), denom(reduced): numer /= denom        */
+  MRL_SPEC_BROADCAST = 15, /* params in(size one on scan_dim), out: copies along scan_dim;
+                              any dtype, both the same (spec.rs:70-75)                    */
+  MRL_SPEC_ONE_PREFIX = 16 /* params in[shape], out[1, shape...]: a copy under a leading
+                              unit dim (spec.rs:59, 469-479); rank <= 4; same dtype       */
 } mrl_spec_kind;
+
+/* spec.rs:165-170 */
+typedef enum { MRL_FILL_ZERO = 0, MRL_FILL_NEG_INF = 1, MRL_FILL_MIN = 2 } mrl_fill_value;
 
 typedef struct {
   int32_t kind;     /* mrl_spec_kind */
-  int32_t accum;    /* Matmul/Conv: 1 = accumulate into the output (InOut), 0 = overwrite */
-  uint32_t scan_dim; /* Softmax only */
+  int32_t accum;    /* 1 = accumulate into the output(s) (InOut), 0 = overwrite */
+  uint32_t scan_dim; /* Softmax family, Max, DivideVecScalar, Broadcast: the dim; Fill: the value */
   uint32_t rank;    /* entries used in spec_shape */
   uint32_t spec_shape[MRL_MAX_SPEC_RANK];
   uint32_t n_params;

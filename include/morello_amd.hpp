@@ -130,7 +130,16 @@ struct TensorSpec {
   size_t bytes_used() const { return volume() * size_of(dtype); }
 };
 
-enum class SpecType : int { Matmul = 0, Conv = 1, Softmax = 2, ComposeMatmulSoftmaxMatmul = 3, Move = 4 };
+enum class SpecType : int {
+  Matmul = 0, Conv = 1, Softmax = 2, ComposeMatmulSoftmaxMatmul = 3, Move = 4,
+  // The primitives Softmax decomposes into (spec.rs:57-162).
+  Fill = 5, Max = 6, SoftmaxDenominator = 7, SoftmaxDenominatorAndMax = 8,
+  SoftmaxDenominatorAndMaxFromParts = 9, SoftmaxDenominatorAndUnscaled = 10,
+  SoftmaxDenominatorAndUnscaledFromMax = 11, SoftmaxComplete = 12, DivideVec = 13,
+  DivideVecScalar = 14, Broadcast = 15, OnePrefix = 16
+};
+// spec.rs:165-170
+enum class FillValue : uint32_t { Zero = 0, NegInf = 1, Min = 2 };
 
 class Spec {
  public:
@@ -153,6 +162,29 @@ class Spec {
   // (spec.rs:3329-3365).
   static Spec compose_msm(const Shape &bmkn2n, Dtype v, Dtype q, Dtype kt) {
     return make(SpecType::ComposeMatmulSoftmaxMatmul, bmkn2n, {v, q, kt, Dtype::Float32}, false, 0, false);
+  }
+
+  // The remaining primitives, f32 (spec.rs:57-162; parameter lists spec.rs:499-583).
+  // `n_params` f32 parameters of kind `t` over `shape`, reducing over `dim`.
+  static Spec softmax_part(SpecType t, const Shape &shape, uint32_t dim, bool accum = false) {
+    static const uint8_t count[] = {1, 2, 3, 3, 4, 3, 4, 4, 2, 2, 2, 2};
+    const int k = int(t);
+    if (k < int(SpecType::Max) || k > int(SpecType::DivideVecScalar)) throw Error(MRL_ERR_BAD_SPEC, "softmax_part");
+    const Dtype f = Dtype::Float32;
+    switch (count[k - int(SpecType::Fill)]) {
+      case 2: return make(t, shape, {f, f}, accum, dim, false);
+      case 3: return make(t, shape, {f, f, f}, accum, dim, false);
+      default: return make(t, shape, {f, f, f, f}, accum, dim, false);
+    }
+  }
+  static Spec fill(const Shape &shape, Dtype dt, FillValue v) {
+    return make(SpecType::Fill, shape, {dt}, false, uint32_t(v), false);
+  }
+  static Spec broadcast(const Shape &shape, uint32_t dim, Dtype dt) {
+    return make(SpecType::Broadcast, shape, {dt, dt}, false, dim, false);
+  }
+  static Spec one_prefix(const Shape &shape, Dtype dt) {
+    return make(SpecType::OnePrefix, shape, {dt, dt}, false, 0, false);
   }
 
   Spec &with_layout(uint32_t param, const Layout &l) {

@@ -173,6 +173,25 @@ class SpecKind(enum.IntEnum):
     Softmax = 2
     ComposeMSM = 3
     Move = 4
+    Fill = 5
+    Max = 6
+    SoftmaxDenominator = 7
+    SoftmaxDenominatorAndMax = 8
+    SoftmaxDenominatorAndMaxFromParts = 9
+    SoftmaxDenominatorAndUnscaled = 10
+    SoftmaxDenominatorAndUnscaledFromMax = 11
+    SoftmaxComplete = 12
+    DivideVec = 13
+    DivideVecScalar = 14
+    Broadcast = 15
+    OnePrefix = 16
+
+
+class FillValue(enum.IntEnum):
+    """morello/src/spec.rs:165-170."""
+    Zero = 0
+    NegInf = 1
+    Min = 2
 
 
 class OperandDirection(enum.IntEnum):
@@ -339,6 +358,67 @@ def Move(shape, dtypes, layouts=None) -> Spec:
     """Move Spec: copy `in` to `out`, which may differ in layout and dtype (Rust `as`
     conversion; oracle: assign_cast in morello/src/verification.rs)."""
     return Spec(SpecKind.Move, shape, dtypes, layouts)
+
+
+def Fill(shape, dtype, value: FillValue, layout=None) -> Spec:
+    """Fill{value} (spec.rs:143-147): one Out parameter set to zero, -inf or the dtype's minimum."""
+    return Spec(SpecKind.Fill, shape, [dtype], [layout], scan_dim=int(FillValue(value)))
+
+
+def Max(shape, dim, layouts=None, accum=False) -> Spec:
+    """Max{dim, accum} (spec.rs:142): params [in, out (size one on dim)], f32."""
+    return Spec(SpecKind.Max, shape, [f32] * 2, layouts, accum, dim)
+
+
+def SoftmaxDenominator(shape, scan_dim, layouts=None, accum=False) -> Spec:
+    """params [in, max, denom]: denom (+)= sum exp(in - max) (spec.rs:91-95)."""
+    return Spec(SpecKind.SoftmaxDenominator, shape, [f32] * 3, layouts, accum, scan_dim)
+
+
+def SoftmaxDenominatorAndMax(shape, scan_dim, layouts=None, accum=False) -> Spec:
+    """params [in, max, denom]: the online (max, denominator) pair (spec.rs:96-101)."""
+    return Spec(SpecKind.SoftmaxDenominatorAndMax, shape, [f32] * 3, layouts, accum, scan_dim)
+
+
+def SoftmaxDenominatorAndMaxFromParts(shape, scan_dim, layouts=None, accum=False) -> Spec:
+    """params [tile_max, tile_denom, out_max, out_denom]: merges per-tile (max, denominator)
+    pairs listed along scan_dim (spec.rs:102-132)."""
+    return Spec(SpecKind.SoftmaxDenominatorAndMaxFromParts, shape, [f32] * 4, layouts, accum, scan_dim)
+
+
+def SoftmaxDenominatorAndUnscaled(shape, scan_dim, layouts=None) -> Spec:
+    """params [in, denom, unscaled] (spec.rs:133-136)."""
+    return Spec(SpecKind.SoftmaxDenominatorAndUnscaled, shape, [f32] * 3, layouts, False, scan_dim)
+
+
+def SoftmaxDenominatorAndUnscaledFromMax(shape, scan_dim, layouts=None, accum=False) -> Spec:
+    """params [in, max, denom, unscaled] (spec.rs:137-141)."""
+    return Spec(SpecKind.SoftmaxDenominatorAndUnscaledFromMax, shape, [f32] * 4, layouts, accum, scan_dim)
+
+
+def SoftmaxComplete(shape, scan_dim, layouts=None) -> Spec:
+    """params [in, max, denom, out]: out = exp(in - max) / denom (spec.rs:86-90)."""
+    return Spec(SpecKind.SoftmaxComplete, shape, [f32] * 4, layouts, False, scan_dim)
+
+
+def DivideVec(shape, layouts=None) -> Spec:
+    """params [numer (InOut), denom], same shape (spec.rs:76)."""
+    return Spec(SpecKind.DivideVec, shape, [f32] * 2, layouts)
+
+
+def DivideVecScalar(shape, scan_dim, layouts=None) -> Spec:
+    """params [numer (InOut), denom (size one on scan_dim)] (spec.rs:77-85)."""
+    return Spec(SpecKind.DivideVecScalar, shape, [f32] * 2, layouts, False, scan_dim)
+
+
+def Broadcast(shape, dim, dtype=f32, layouts=None) -> Spec:
+    """Broadcast{dim} (spec.rs:70-75): params [in (size one on dim), out]."""
+    return Spec(SpecKind.Broadcast, shape, [dtype] * 2, layouts, False, dim)
+
+
+def OnePrefix(shape, dtype=f32, layouts=None) -> Spec:
+    """OnePrefix (spec.rs:59, 469-479): params [in[shape], out[1, *shape]]."""
+    return Spec(SpecKind.OnePrefix, shape, [dtype] * 2, layouts)
 
 
 class DeviceBuffer:

@@ -39,6 +39,30 @@ uint32_t expected_params(int kind) {
     case MRL_SPEC_MATMUL: case MRL_SPEC_CONV: return 3;
     case MRL_SPEC_SOFTMAX: case MRL_SPEC_MOVE: return 2;
     case MRL_SPEC_COMPOSE_MSM: return 4;
+    case MRL_SPEC_FILL: return 1;
+    case MRL_SPEC_MAX: case MRL_SPEC_DIVIDE_VEC: case MRL_SPEC_DIVIDE_VEC_SCALAR:
+    case MRL_SPEC_BROADCAST: case MRL_SPEC_ONE_PREFIX: return 2;
+    case MRL_SPEC_SOFTMAX_DENOMINATOR: case MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX:
+    case MRL_SPEC_SOFTMAX_DENOMINATOR_AND_UNSCALED: return 3;
+    case MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX_FROM_PARTS:
+    case MRL_SPEC_SOFTMAX_DENOMINATOR_AND_UNSCALED_FROM_MAX: case MRL_SPEC_SOFTMAX_COMPLETE: return 4;
+    default: return 0;
+  }
+}
+
+// Kinds whose spec_shape is one tensor's shape and which reduce or broadcast over scan_dim.
+bool is_parts_kind(int kind) { return kind >= MRL_SPEC_MAX && kind <= MRL_SPEC_DIVIDE_VEC_SCALAR; }
+
+// Bit i set: parameter i has size one on scan_dim (spec.rs:499-583).
+uint32_t reduced_mask(int kind) {
+  switch (kind) {
+    case MRL_SPEC_MAX: return 0b0010;
+    case MRL_SPEC_SOFTMAX_DENOMINATOR: case MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX: return 0b0110;
+    case MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX_FROM_PARTS: return 0b1100;
+    case MRL_SPEC_SOFTMAX_DENOMINATOR_AND_UNSCALED: return 0b0010;
+    case MRL_SPEC_SOFTMAX_DENOMINATOR_AND_UNSCALED_FROM_MAX: case MRL_SPEC_SOFTMAX_COMPLETE: return 0b0110;
+    case MRL_SPEC_DIVIDE_VEC_SCALAR: return 0b0010;
+    case MRL_SPEC_BROADCAST: return 0b0001;
     default: return 0;
   }
 }
@@ -49,7 +73,7 @@ uint32_t expected_rank(const mrl_spec &s) {
     case MRL_SPEC_CONV: return 7;
     case MRL_SPEC_SOFTMAX: case MRL_SPEC_MOVE: return s.rank;
     case MRL_SPEC_COMPOSE_MSM: return 5;
-    default: return 0;
+    default: return s.kind >= MRL_SPEC_FILL && s.kind <= MRL_SPEC_ONE_PREFIX ? s.rank : 0;
   }
 }
 
@@ -75,7 +99,7 @@ int parameter_shape(const mrl_spec &s, uint32_t idx, uint32_t *shape, uint32_t *
     }
     case MRL_SPEC_SOFTMAX:
     case MRL_SPEC_MOVE:
-      if (idx > 1) return MRL_ERR_BAD_SPEC;
+      if (idx > 1 || s.rank > MRL_MAX_RANK) return MRL_ERR_BAD_SPEC;
       *rank = s.rank;
       for (uint32_t d = 0; d < s.rank; d++) shape[d] = ss[d];
       return MRL_OK;
@@ -90,8 +114,20 @@ int parameter_shape(const mrl_spec &s, uint32_t idx, uint32_t *shape, uint32_t *
       else return MRL_ERR_BAD_SPEC;
       return MRL_OK;
     }
+    case MRL_SPEC_ONE_PREFIX:
+      if (idx > 1 || s.rank + idx > MRL_MAX_RANK) return MRL_ERR_BAD_SPEC;
+      *rank = s.rank + idx;
+      if (idx == 1) shape[0] = 1;
+      for (uint32_t d = 0; d < s.rank; d++) shape[d + idx] = ss[d];
+      return MRL_OK;
     default:
-      return MRL_ERR_BAD_SPEC;
+      if (s.kind < MRL_SPEC_FILL || s.kind > MRL_SPEC_BROADCAST || idx >= expected_params(s.kind) ||
+          s.rank > MRL_MAX_RANK || (s.kind != MRL_SPEC_FILL && s.scan_dim >= s.rank))
+        return MRL_ERR_BAD_SPEC;
+      *rank = s.rank;
+      for (uint32_t d = 0; d < s.rank; d++) shape[d] = ss[d];
+      if (s.kind != MRL_SPEC_FILL && ((reduced_mask(s.kind) >> idx) & 1)) shape[s.scan_dim] = 1;
+      return MRL_OK;
   }
 }
 
@@ -99,9 +135,17 @@ int parameter_shape(const mrl_spec &s, uint32_t idx, uint32_t *shape, uint32_t *
 int parameter_direction(const mrl_spec &s, uint32_t idx) {
   const uint32_t n = expected_params(s.kind);
   if (n == 0 || idx >= n) return -1;
-  if (idx + 1 < n) return 0;
-  if ((s.kind == MRL_SPEC_MATMUL || s.kind == MRL_SPEC_CONV) && s.accum) return 2;
-  return 1;
+  const int acc = s.accum ? 2 : 1;
+  switch (s.kind) {
+    case MRL_SPEC_DIVIDE_VEC: case MRL_SPEC_DIVIDE_VEC_SCALAR: return idx == 0 ? 2 : 0;
+    case MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX: return idx == 0 ? 0 : acc;
+    case MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX_FROM_PARTS: return idx < 2 ? 0 : acc;
+    case MRL_SPEC_SOFTMAX_DENOMINATOR_AND_UNSCALED: return idx == 0 ? 0 : 1;
+    case MRL_SPEC_SOFTMAX_DENOMINATOR_AND_UNSCALED_FROM_MAX: return idx < 2 ? 0 : (idx == 2 ? acc : 1);
+    case MRL_SPEC_MATMUL: case MRL_SPEC_CONV: case MRL_SPEC_MAX: case MRL_SPEC_SOFTMAX_DENOMINATOR:
+      return idx + 1 < n ? 0 : acc;
+    default: return idx + 1 < n ? 0 : 1;
+  }
 }
 
 int check_spec(const mrl_spec *sp) {
@@ -113,6 +157,12 @@ int check_spec(const mrl_spec *sp) {
   if (s.rank == 0 || s.rank > MRL_MAX_SPEC_RANK || s.rank != expected_rank(s)) return MRL_ERR_BAD_SPEC;
   if (s.kind == MRL_SPEC_SOFTMAX && (s.rank > MRL_MAX_RANK || s.scan_dim >= s.rank)) return MRL_ERR_BAD_SPEC;
   if (s.kind == MRL_SPEC_MOVE && s.rank > MRL_MAX_RANK) return MRL_ERR_BAD_SPEC;
+  if (s.kind >= MRL_SPEC_FILL && s.rank > MRL_MAX_RANK) return MRL_ERR_BAD_SPEC;
+  if (s.kind == MRL_SPEC_ONE_PREFIX && s.rank + 1 > MRL_MAX_RANK) return MRL_ERR_BAD_SPEC;
+  if ((is_parts_kind(s.kind) && s.kind != MRL_SPEC_DIVIDE_VEC) || s.kind == MRL_SPEC_BROADCAST) {
+    if (s.scan_dim >= s.rank) return MRL_ERR_BAD_SPEC;
+  }
+  if (s.kind == MRL_SPEC_FILL && s.scan_dim > MRL_FILL_MIN) return MRL_ERR_BAD_SPEC;
   for (uint32_t d = 0; d < s.rank; d++)
     if (s.spec_shape[d] == 0) return MRL_ERR_BAD_SPEC;
   for (uint32_t i = 0; i < np; i++) {
@@ -135,6 +185,23 @@ int check_spec(const mrl_spec *sp) {
       break;
     case MRL_SPEC_COMPOSE_MSM:
       if (s.dtypes[3] != MRL_F32) return MRL_ERR_UNSUPPORTED;
+      break;
+    case MRL_SPEC_FILL:
+      // NegInf exists only for floats (verification.rs fill_neg_inf).
+      if (s.scan_dim == MRL_FILL_NEG_INF && s.dtypes[0] != MRL_F32 && s.dtypes[0] != MRL_BF16)
+        return MRL_ERR_BAD_SPEC;
+      break;
+    case MRL_SPEC_BROADCAST:
+    case MRL_SPEC_ONE_PREFIX:
+      if (s.dtypes[0] != s.dtypes[1]) return MRL_ERR_UNSUPPORTED;
+      break;
+    default:
+      if (is_parts_kind(s.kind)) {
+        for (uint32_t i = 0; i < np; i++)
+          if (s.dtypes[i] != MRL_F32) return MRL_ERR_UNSUPPORTED;
+        // The accumulating form of this one is unimplemented in the reference too (spec.rs:688).
+        if (s.kind == MRL_SPEC_SOFTMAX_DENOMINATOR_AND_UNSCALED && s.accum) return MRL_ERR_UNSUPPORTED;
+      }
       break;
   }
   return MRL_OK;
@@ -367,6 +434,83 @@ int run_move(const mrl_spec &s, void *const *params, Workspace &ws) {
   return MRL_OK;
 }
 
+// Max, the SoftmaxDenominator* family, SoftmaxComplete, DivideVec, DivideVecScalar: one
+// wavefront per line along scan_dim over strided f32 tensors.
+int run_parts(const mrl_spec &s, void *const *params, Workspace &ws) {
+  Prepared pr[4];
+  mrl::PartsArgs pa;
+  pa.kind = s.kind, pa.accum = s.accum, pa.rank = s.rank, pa.n_params = s.n_params;
+  // DivideVec has no dim of its own: walk the innermost one.
+  pa.scan_dim = s.kind == MRL_SPEC_DIVIDE_VEC ? s.rank - 1 : s.scan_dim;
+  pa.lines = 1;
+  for (uint32_t d = 0; d < MRL_MAX_RANK; d++) {
+    pa.shape[d] = d < s.rank ? s.spec_shape[d] : 1;
+    if (d < s.rank && d != pa.scan_dim) pa.lines *= pa.shape[d];
+  }
+  for (uint32_t i = 0; i < 4; i++) {
+    pa.ptr[i] = nullptr;
+    for (uint32_t d = 0; d < MRL_MAX_RANK; d++) pa.stride[i][d] = 0;
+  }
+  for (uint32_t i = 0; i < s.n_params; i++) {
+    const int dir = parameter_direction(s, i);
+    int rc = prepare(s, i, params[i], dir != 1, ws, &pr[i]);
+    if (rc != MRL_OK) return rc;
+    pa.ptr[i] = (float *)pr[i].t.ptr;
+    for (uint32_t d = 0; d < s.rank; d++) pa.stride[i][d] = pr[i].t.shape[d] == 1 ? 0 : pr[i].t.stride[d];
+  }
+  HIP_TRY(mrl::launch_parts(pa, ws.stream));
+  for (uint32_t i = 0; i < s.n_params; i++) {
+    if (parameter_direction(s, i) == 0) continue;
+    int rc = finish_output(pr[i], ws);
+    if (rc != MRL_OK) return rc;
+  }
+  return MRL_OK;
+}
+
+int run_fill(const mrl_spec &s, void *const *params, Workspace &ws) {
+  // Every element of the buffer is written, so the layout (a bijection onto the buffer)
+  // does not matter.
+  HIP_TRY(mrl::launch_fill(params[0], s.dtypes[0], int(s.scan_dim), volume(s.spec_shape, s.rank), ws.stream));
+  return MRL_OK;
+}
+
+int run_broadcast(const mrl_spec &s, void *const *params, Workspace &ws) {
+  uint32_t ishape[MRL_MAX_RANK], oshape[MRL_MAX_RANK], rank;
+  parameter_shape(s, 0, ishape, &rank);
+  parameter_shape(s, 1, oshape, &rank);
+  mrl::LayoutEval il, ol;
+  if (!mrl::make_layout_eval(s.layouts[0], ishape, rank, &il) ||
+      !mrl::make_layout_eval(s.layouts[1], oshape, rank, &ol))
+    return MRL_ERR_BAD_LAYOUT;
+  HIP_TRY(mrl::launch_broadcast(params[0], params[1], il, ol, s.scan_dim, uint32_t(mrl_dtype_size(s.dtypes[0])),
+                                volume(oshape, rank), ws.stream));
+  return MRL_OK;
+}
+
+int run_one_prefix(const mrl_spec &s, void *const *params, Workspace &ws) {
+  // The output's leading unit dim takes no part in addressing: restate its layout over the
+  // input's shape (drop physical dims of logical dim 0, renumber the rest) and copy.
+  uint32_t shape[MRL_MAX_RANK], oshape[MRL_MAX_RANK], rank, orank;
+  parameter_shape(s, 0, shape, &rank);
+  parameter_shape(s, 1, oshape, &orank);
+  uint32_t phys[MRL_MAX_PHYS];
+  if (!mrl::physical_shape(s.layouts[1], oshape, orank, phys)) return MRL_ERR_BAD_LAYOUT;
+  mrl_layout lo;
+  lo.ndims = 0;
+  for (uint32_t i = 0; i < s.layouts[1].ndims; i++) {
+    mrl_physdim pd = s.layouts[1].dims[i];
+    if (pd.logical_dim == 0) continue;
+    pd.logical_dim--;
+    lo.dims[lo.ndims++] = pd;
+  }
+  mrl::LayoutEval sl, dl;
+  if (!mrl::make_layout_eval(s.layouts[0], shape, rank, &sl) || !mrl::make_layout_eval(lo, shape, rank, &dl))
+    return MRL_ERR_BAD_LAYOUT;
+  HIP_TRY(mrl::launch_move_generic(params[0], params[1], sl, dl, s.dtypes[0], s.dtypes[1],
+                                   volume(shape, rank), ws.stream));
+  return MRL_OK;
+}
+
 int run_async_impl(const mrl_spec *spec, void *const *params, hipStream_t stream) {
   if (g_device < 0) {
     int rc = mrl_init(0);
@@ -384,7 +528,10 @@ int run_async_impl(const mrl_spec *spec, void *const *params, hipStream_t stream
     case MRL_SPEC_SOFTMAX: return run_softmax(*spec, params, ws);
     case MRL_SPEC_COMPOSE_MSM: return run_compose_msm(*spec, params, ws);
     case MRL_SPEC_MOVE: return run_move(*spec, params, ws);
-    default: return MRL_ERR_UNSUPPORTED;
+    case MRL_SPEC_FILL: return run_fill(*spec, params, ws);
+    case MRL_SPEC_BROADCAST: return run_broadcast(*spec, params, ws);
+    case MRL_SPEC_ONE_PREFIX: return run_one_prefix(*spec, params, ws);
+    default: return is_parts_kind(spec->kind) ? run_parts(*spec, params, ws) : MRL_ERR_UNSUPPORTED;
   }
 }
 
@@ -548,7 +695,11 @@ uint64_t mrl_spec_ops(const mrl_spec *spec) {
 int mrl_spec_check(const mrl_spec *spec) { return check_spec(spec); }
 
 size_t mrl_spec_workspace_bytes(const mrl_spec *spec) {
-  if (check_spec(spec) != MRL_OK || spec->kind == MRL_SPEC_MOVE) return 0;
+  if (check_spec(spec) != MRL_OK) return 0;
+  // These run on the parameters' own layouts and stage nothing.
+  if (spec->kind == MRL_SPEC_MOVE || spec->kind == MRL_SPEC_FILL || spec->kind == MRL_SPEC_BROADCAST ||
+      spec->kind == MRL_SPEC_ONE_PREFIX)
+    return 0;
   size_t total = 0;
   for (uint32_t i = 0; i < spec->n_params; i++) {
     uint32_t shape[MRL_MAX_RANK], rank;

@@ -3,8 +3,8 @@
 // Morello's generated `main` (morello/src/codegen/cpu.rs:284-409) takes one file per Spec
 // parameter, output included, each holding raw little-endian values in logical row-major
 // order (morello/src/verification.rs:957-1001, loader cpu.rs:221-270), calls the kernel,
-// and prints the last parameter: a line with its shape `AxBxC`, then every element in
-// logical row-major order, space separated, one newline at the end of every loop level but
+// and prints the output parameter (every written parameter, for Specs with several): a
+// line with its shape `AxBxC`, then every element in logical row-major order, space separated, one newline at the end of every loop level but
 // the outermost (cpu.rs:570-618), integers in decimal and floats as %.10f
 // (codegen/c_utils.rs:334-344).  With no files the buffers are zero-filled (cpu.rs:320).
 // Exit status 1 = wrong argument count, 2 = an input could not be loaded (cpu.rs:344-364).
@@ -17,7 +17,11 @@
 //   mrl_harness <spec> --bench <iters>              benchmark mode
 //
 //   <spec> = kind:shape:dtypes[:flag]...
-//     kind   matmul | conv | softmax | msm | move
+//     kind   matmul | conv | softmax | msm | move | fill | max | softmaxdenominator |
+//            softmaxdenominatorandmax | softmaxdenominatorandmaxfromparts |
+//            softmaxdenominatorandunscaled | softmaxdenominatorandunscaledfrommax |
+//            softmaxcomplete | dividevec | dividevecscalar | broadcast | oneprefix
+//            (these take the tensor shape; scan=d names the dim, for fill the value 0/1/2)
 //     shape  the Spec shape, `x` separated (matmul b x m x k x n; conv b x f x c x oh x ow x fh x fw;
 //            softmax/move the tensor shape; msm b x m x k x n2 x n)
 //     dtypes one per parameter, comma separated: u8 i8 u16 i16 u32 i32 f32 bf16
@@ -67,7 +71,23 @@ bool parse_spec(const std::string &text, mrl_spec *spec, std::string *err) {
   else if (kind == "softmax") spec->kind = MRL_SPEC_SOFTMAX, spec->n_params = 2;
   else if (kind == "msm") spec->kind = MRL_SPEC_COMPOSE_MSM, spec->n_params = 4;
   else if (kind == "move") spec->kind = MRL_SPEC_MOVE, spec->n_params = 2;
-  else return *err = "unknown kind " + kind, false;
+  else {
+    // The primitives Softmax decomposes into, by their reference names in lower case.
+    static const struct { const char *name; int kind; uint32_t n; } parts[] = {
+        {"fill", MRL_SPEC_FILL, 1}, {"max", MRL_SPEC_MAX, 2},
+        {"softmaxdenominator", MRL_SPEC_SOFTMAX_DENOMINATOR, 3},
+        {"softmaxdenominatorandmax", MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX, 3},
+        {"softmaxdenominatorandmaxfromparts", MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX_FROM_PARTS, 4},
+        {"softmaxdenominatorandunscaled", MRL_SPEC_SOFTMAX_DENOMINATOR_AND_UNSCALED, 3},
+        {"softmaxdenominatorandunscaledfrommax", MRL_SPEC_SOFTMAX_DENOMINATOR_AND_UNSCALED_FROM_MAX, 4},
+        {"softmaxcomplete", MRL_SPEC_SOFTMAX_COMPLETE, 4}, {"dividevec", MRL_SPEC_DIVIDE_VEC, 2},
+        {"dividevecscalar", MRL_SPEC_DIVIDE_VEC_SCALAR, 2}, {"broadcast", MRL_SPEC_BROADCAST, 2},
+        {"oneprefix", MRL_SPEC_ONE_PREFIX, 2}};
+    bool found = false;
+    for (const auto &p : parts)
+      if (kind == p.name) spec->kind = p.kind, spec->n_params = p.n, found = true;
+    if (!found) return *err = "unknown kind " + kind, false;
+  }
   const auto dims = split(parts[1], 'x');
   if (dims.empty() || dims.size() > MRL_MAX_SPEC_RANK) return *err = "bad shape", false;
   spec->rank = uint32_t(dims.size());
@@ -238,13 +258,17 @@ int main(int argc, char *argv[]) {
   } else {
     rc = mrl_run(&spec, dev.data());
     if (rc != MRL_OK) DIE(3, "Run failed: %s (%s)", mrl_status_string(rc), mrl_last_error());
-    const uint32_t last = spec.n_params - 1;
-    if (relayout(spec, last, dev[last], staged[last], false) != MRL_OK ||
-        mrl_memcpy_d2h(host[last].data(), staged[last], bytes[last]) != MRL_OK)
-      DIE(3, "Reading the output failed: %s", mrl_last_error());
-    uint32_t shape[MRL_MAX_RANK], rank;
-    mrl_spec_parameter_shape(&spec, last, shape, &rank);
-    print_tensor(spec.dtypes[last], host[last].data(), shape, rank);
+    // Every parameter the Spec writes, in parameter order (one for Matmul, Conv, Softmax, Move
+    // and the Compose: the last, as the reference's emitted main prints).
+    for (uint32_t o = 0; o < spec.n_params; o++) {
+      if (mrl_spec_parameter_direction(&spec, o) == 0) continue;
+      if (relayout(spec, o, dev[o], staged[o], false) != MRL_OK ||
+          mrl_memcpy_d2h(host[o].data(), staged[o], bytes[o]) != MRL_OK)
+        DIE(3, "Reading the output failed: %s", mrl_last_error());
+      uint32_t shape[MRL_MAX_RANK], rank;
+      mrl_spec_parameter_shape(&spec, o, shape, &rank);
+      print_tensor(spec.dtypes[o], host[o].data(), shape, rank);
+    }
   }
   for (uint32_t i = 0; i < spec.n_params; i++) {
     mrl_device_free(dev[i]);

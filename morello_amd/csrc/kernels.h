@@ -73,6 +73,21 @@ hipError_t launch_conv_i8(const ConvArgs &c, bool img_unsigned, hipStream_t stre
 hipError_t launch_softmax_rows(const float *in, float *out, uint64_t rows, uint32_t cols,
                                hipStream_t stream);
 
+// ---- parts.hip: the primitive Specs of the Softmax decomposition, Broadcast, Fill ----------
+struct PartsArgs {
+  int kind;  // mrl_spec_kind
+  int accum;
+  uint32_t rank, scan_dim, n_params;
+  uint32_t shape[MRL_MAX_RANK];           // the Spec shape (full tensor)
+  float *ptr[4];
+  int64_t stride[4][MRL_MAX_RANK];        // element strides per parameter (0 on reduced dims)
+  uint64_t lines;                         // product of the dims other than scan_dim
+};
+hipError_t launch_parts(const PartsArgs &p, hipStream_t stream);
+hipError_t launch_broadcast(const void *in, void *out, const LayoutEval &il, const LayoutEval &ol,
+                            uint32_t dim, uint32_t elem_size, uint64_t count, hipStream_t stream);
+hipError_t launch_fill(void *out, int dtype, int fill_value, uint64_t count, hipStream_t stream);
+
 // ---- attention.hip: fused Matmul -> Softmax -> Matmul on bf16 inputs -------------------
 struct AttnArgs {
   const void *q;   // [b, m, k]   bf16 row-major

@@ -9,6 +9,7 @@
  */
 #include "morello_oracle.h"
 
+#include <float.h>
 #include <math.h>
 #include <stdlib.h>
 #include <string.h>
@@ -560,4 +561,149 @@ int orc_fill_check_pattern(int dtype, void *dst, size_t count) {
     default:
       return ORC_BAD_ARG;
   }
+}
+
+/* ------------------------------------------- primitives of the Softmax decomposition */
+
+/* One line along the scan dim, visited element by element as the scalar kernels the
+ * emitter prints are visited by the loops around them (codegen/cpu.rs:1350-1433,
+ * 1968-2113).  `x`, `y`: full-shape parameters of the line with element stride `st`;
+ * `r0`, `r1`: the line's entries of the reduced parameters. */
+static void part_line(int kind, int accum, size_t n, size_t st, float *p0, float *p1, float *p2,
+                      float *p3) {
+  switch (kind) {
+    case ORC_PART_MAX: /* [in, out] */
+      if (!accum) *p1 = -INFINITY;
+      for (size_t i = 0; i < n; i++) *p1 = fmaxf(*p1, p0[i * st]);
+      break;
+    case ORC_PART_DENOMINATOR: /* [in, max, denom]: cpu.rs:1414-1424 */
+      if (!accum) *p2 = 0.0f;
+      for (size_t i = 0; i < n; i++) *p2 += expf(p0[i * st] - *p1);
+      break;
+    case ORC_PART_DENOMINATOR_AND_MAX: /* [in, max, denom]: cpu.rs:1360-1389 */
+      if (!accum) *p1 = -INFINITY, *p2 = 0.0f;
+      for (size_t i = 0; i < n; i++) {
+        const float old_max = *p1;
+        const float new_max = fmaxf(old_max, p0[i * st]);
+        *p2 = *p2 * expf(old_max - new_max) + expf(p0[i * st] - new_max);
+        *p1 = new_max;
+      }
+      break;
+    case ORC_PART_DENOMINATOR_AND_MAX_FROM_PARTS: /* [tile_max, tile_denom, max, denom]: cpu.rs:1390-1413 */
+      if (!accum) *p2 = -INFINITY, *p3 = 0.0f;
+      for (size_t i = 0; i < n; i++) {
+        const float old_max = *p2;
+        const float new_max = fmaxf(old_max, p0[i * st]);
+        *p3 = *p3 * expf(old_max - new_max) + p1[i * st] * expf(p0[i * st] - new_max);
+        *p2 = new_max;
+      }
+      break;
+    case ORC_PART_DENOMINATOR_AND_UNSCALED: { /* [in, denom, unscaled]: spec.rs:133-136 */
+      float m = -INFINITY;
+      for (size_t i = 0; i < n; i++) m = fmaxf(m, p0[i * st]);
+      *p1 = 0.0f;
+      for (size_t i = 0; i < n; i++) {
+        const float e = expf(p0[i * st] - m);
+        *p1 += e;
+        p2[i * st] = e;
+      }
+      break;
+    }
+    case ORC_PART_DENOMINATOR_AND_UNSCALED_FROM_MAX: /* [in, max, denom, unscaled]: cpu.rs:1425-1433 */
+      if (!accum) *p2 = 0.0f;
+      for (size_t i = 0; i < n; i++) {
+        const float e = expf(p0[i * st] - *p1);
+        *p2 += e;
+        p3[i * st] = e;
+      }
+      break;
+    case ORC_PART_COMPLETE: /* [in, max, denom, out]: cpu.rs:1350-1359 */
+      for (size_t i = 0; i < n; i++) p3[i * st] = expf(p0[i * st] - *p1) / *p2;
+      break;
+    case ORC_PART_DIVIDE_VEC: /* [numer, denom]: verification.rs:191-197 */
+      for (size_t i = 0; i < n; i++) p0[i * st] /= p1[i * st];
+      break;
+    case ORC_PART_DIVIDE_VEC_SCALAR: /* [numer, denom]: verification.rs:198-204 */
+      for (size_t i = 0; i < n; i++) p0[i * st] /= *p1;
+      break;
+  }
+}
+
+int orc_softmax_part(int kind, int accum, const uint32_t *shape, uint32_t rank, uint32_t scan_dim,
+                     float *const params[4]) {
+  /* Which parameters have size one on the scan dim (spec.rs:499-583). */
+  static const unsigned reduced[] = {
+      [ORC_PART_MAX] = 2u,
+      [ORC_PART_DENOMINATOR] = 6u,
+      [ORC_PART_DENOMINATOR_AND_MAX] = 6u,
+      [ORC_PART_DENOMINATOR_AND_MAX_FROM_PARTS] = 12u,
+      [ORC_PART_DENOMINATOR_AND_UNSCALED] = 2u,
+      [ORC_PART_DENOMINATOR_AND_UNSCALED_FROM_MAX] = 6u,
+      [ORC_PART_COMPLETE] = 6u,
+      [ORC_PART_DIVIDE_VEC] = 0u,
+      [ORC_PART_DIVIDE_VEC_SCALAR] = 2u,
+  };
+  static const unsigned nparams[] = {
+      [ORC_PART_MAX] = 2, [ORC_PART_DENOMINATOR] = 3, [ORC_PART_DENOMINATOR_AND_MAX] = 3,
+      [ORC_PART_DENOMINATOR_AND_MAX_FROM_PARTS] = 4, [ORC_PART_DENOMINATOR_AND_UNSCALED] = 3,
+      [ORC_PART_DENOMINATOR_AND_UNSCALED_FROM_MAX] = 4, [ORC_PART_COMPLETE] = 4,
+      [ORC_PART_DIVIDE_VEC] = 2, [ORC_PART_DIVIDE_VEC_SCALAR] = 2,
+  };
+  if (kind < ORC_PART_MAX || kind > ORC_PART_DIVIDE_VEC_SCALAR || rank == 0 || rank > ORC_MAX_RANK)
+    return ORC_BAD_ARG;
+  if (kind == ORC_PART_DIVIDE_VEC) scan_dim = rank - 1;
+  if (scan_dim >= rank) return ORC_BAD_ARG;
+  if (kind == ORC_PART_DENOMINATOR_AND_UNSCALED && accum) return ORC_UNSUPPORTED;
+  size_t outer = 1, inner = 1;
+  for (uint32_t d = 0; d < scan_dim; d++) outer *= shape[d];
+  for (uint32_t d = scan_dim + 1; d < rank; d++) inner *= shape[d];
+  const size_t n = shape[scan_dim];
+  for (size_t o = 0; o < outer; o++)
+    for (size_t in = 0; in < inner; in++) {
+      float *p[4] = {0, 0, 0, 0};
+      for (unsigned t = 0; t < nparams[kind]; t++)
+        p[t] = (reduced[kind] >> t) & 1 ? params[t] + o * inner + in : params[t] + o * n * inner + in;
+      part_line(kind, accum, n, inner, p[0], p[1], p[2], p[3]);
+    }
+  return ORC_OK;
+}
+
+int orc_broadcast(const uint32_t *shape, uint32_t rank, uint32_t dim, size_t elem_size,
+                  const void *in, void *out) {
+  if (rank == 0 || rank > ORC_MAX_RANK || dim >= rank) return ORC_BAD_ARG;
+  size_t outer = 1, inner = 1;
+  for (uint32_t d = 0; d < dim; d++) outer *= shape[d];
+  for (uint32_t d = dim + 1; d < rank; d++) inner *= shape[d];
+  for (size_t o = 0; o < outer; o++)
+    for (size_t i = 0; i < shape[dim]; i++)
+      memcpy((char *)out + ((o * shape[dim] + i) * inner) * elem_size,
+             (const char *)in + o * inner * elem_size, inner * elem_size);
+  return ORC_OK;
+}
+
+int orc_fill(int dtype, int value, void *dst, size_t count) {
+  /* verification.rs:214-222 with DynArray::zero / fill_neg_inf / fill_min (:521-545). */
+  uint32_t pattern = 0;
+  if (value == 1) {
+    if (!is_float(dtype)) return ORC_BAD_ARG;
+    const float ninf = -INFINITY;
+    memcpy(&pattern, &ninf, 4);
+    if (dtype == ORC_BF16) pattern >>= 16;
+  } else if (value == 2) {
+    const float fmin_ = -FLT_MAX;
+    switch (dtype) {
+      case ORC_I8: pattern = (uint8_t)INT8_MIN; break;
+      case ORC_I16: pattern = (uint16_t)INT16_MIN; break;
+      case ORC_I32: pattern = (uint32_t)INT32_MIN; break;
+      case ORC_F32: memcpy(&pattern, &fmin_, 4); break;
+      case ORC_BF16: pattern = 0xff7fu; break; /* half::bf16::MIN */
+      default: pattern = 0; break;
+    }
+  } else if (value != 0) {
+    return ORC_BAD_ARG;
+  }
+  const size_t es = orc_dtype_size(dtype);
+  if (es == 0) return ORC_BAD_ARG;
+  for (size_t i = 0; i < count; i++) memcpy((char *)dst + i * es, &pattern, es); /* little endian */
+  return ORC_OK;
 }

@@ -137,6 +137,37 @@ int orc_compose_msm(uint32_t b, uint32_t m, uint32_t k, uint32_t n2, uint32_t n,
 int orc_move(const uint32_t *shape, uint32_t rank, const int dtypes[2], const orc_layout *layouts[2],
              const void *in, void *out);
 
+/* The primitives Softmax decomposes into (spec.rs:86-162), numbered as in the GPU library's
+ * ABI.  f32, dense row-major; `params` in Spec parameter order; a "reduced" parameter is
+ * dense over the shape with scan_dim set to one.  Each line is updated element by element
+ * exactly as the emitter's scalar kernels would be (codegen/cpu.rs:1350-1433).
+ * Pinned by: numpy max / logsumexp identities in float64, scipy.special.softmax for
+ * Complete, splitting a row into tiles and merging for FromParts, and accum == running the
+ * non-accumulating form on the concatenated input.  The reference's interpreter leaves
+ * these as todo!() (verification.rs:185-205) except DivideVec/DivideVecScalar, so parity
+ * with a reference *execution* is unpinned; the arithmetic is pinned. */
+enum {
+  ORC_PART_MAX = 6,
+  ORC_PART_DENOMINATOR = 7,
+  ORC_PART_DENOMINATOR_AND_MAX = 8,
+  ORC_PART_DENOMINATOR_AND_MAX_FROM_PARTS = 9,
+  ORC_PART_DENOMINATOR_AND_UNSCALED = 10,
+  ORC_PART_DENOMINATOR_AND_UNSCALED_FROM_MAX = 11,
+  ORC_PART_COMPLETE = 12,
+  ORC_PART_DIVIDE_VEC = 13,
+  ORC_PART_DIVIDE_VEC_SCALAR = 14
+};
+int orc_softmax_part(int kind, int accum, const uint32_t *shape, uint32_t rank, uint32_t scan_dim,
+                     float *const params[4]);
+
+/* Broadcast{dim} (spec.rs:70-75, 499-507): out[.., i, ..] = in[.., 0, ..]; dense row-major. */
+int orc_broadcast(const uint32_t *shape, uint32_t rank, uint32_t dim, size_t elem_size,
+                  const void *in, void *out);
+
+/* Fill{value} (spec.rs:143-170; verification.rs:214-222): value 0 Zero, 1 NegInf (floats
+ * only), 2 Min (the dtype's minimum; f32::MIN / bf16::MIN for floats). */
+int orc_fill(int dtype, int value, void *dst, size_t count);
+
 /* verification.rs:893-952: ints count up from the dtype minimum and wrap at the maximum;
  * f32 and bf16 cycle 0,1,2,3.  Fills `count` elements in logical row-major order. */
 int orc_fill_check_pattern(int dtype, void *dst, size_t count);

@@ -145,3 +145,35 @@ def ref_lib(name):
     """A library built from the reference's own C (oracle/_ref), or None when absent."""
     path = os.path.join(REF_DIR, name)
     return C.CDLL(path) if os.path.exists(path) else None
+
+
+# Kind codes shared by the oracle and the GPU library's ABI.
+PART_MAX, PART_DENOM, PART_DENOM_MAX, PART_FROM_PARTS, PART_UNSCALED, PART_UNSCALED_FROM_MAX, \
+    PART_COMPLETE, PART_DIVIDE_VEC, PART_DIVIDE_VEC_SCALAR = range(6, 15)
+
+
+def softmax_part(kind, shape, scan_dim, params, accum=False):
+    """Runs one primitive of the Softmax decomposition in place on `params` (f32 arrays,
+    dense row-major, Spec parameter order)."""
+    ptrs = (C.c_void_p * 4)()
+    for i, p in enumerate(params):
+        assert p.dtype == np.float32 and p.flags["C_CONTIGUOUS"]
+        ptrs[i] = p.ctypes.data
+    rc = lib().orc_softmax_part(kind, int(accum), _u32(shape), len(shape), scan_dim, ptrs)
+    assert rc == 0, f"oracle softmax_part rc={rc}"
+    return params
+
+
+def broadcast(shape, dim, x):
+    out = np.empty(shape, dtype=x.dtype)
+    rc = lib().orc_broadcast(_u32(shape), len(shape), dim, C.c_size_t(x.itemsize),
+                             x.ctypes.data_as(C.c_void_p), out.ctypes.data_as(C.c_void_p))
+    assert rc == 0
+    return out
+
+
+def fill(dtype, value, count):
+    out = np.full(count, 0x55, dtype=NP[dtype])
+    rc = lib().orc_fill(dtype, value, out.ctypes.data_as(C.c_void_p), C.c_size_t(count))
+    assert rc == 0, f"oracle fill rc={rc}"
+    return out

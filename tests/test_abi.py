@@ -54,6 +54,53 @@ def test_parameter_shapes_and_directions():
     assert cm.bytes_used(0) == 16 * 2048 * 128 * 2 and cm.bytes_used(3) == 16 * 2048 * 128 * 4
 
 
+def test_primitive_spec_parameter_shapes_and_directions():
+    # spec.rs:499-583 (shapes) and spec.rs:1204-1245 (directions); 0 In, 1 Out, 2 InOut.
+    def dirs(spec):
+        return [int(d) for d in spec.operand_directions()]
+
+    full, red = [4, 6, 8], [4, 1, 8]
+    mx = M.Max(full, 1)
+    assert mx.parameter_shapes() == [full, red] and dirs(mx) == [0, 1]
+    assert dirs(M.Max(full, 1, accum=True)) == [0, 2]
+    sd = M.SoftmaxDenominator(full, 1)
+    assert sd.parameter_shapes() == [full, red, red] and dirs(sd) == [0, 0, 1]
+    assert dirs(M.SoftmaxDenominator(full, 1, accum=True)) == [0, 0, 2]
+    sdm = M.SoftmaxDenominatorAndMax(full, 1)
+    assert sdm.parameter_shapes() == [full, red, red] and dirs(sdm) == [0, 1, 1]
+    assert dirs(M.SoftmaxDenominatorAndMax(full, 1, accum=True)) == [0, 2, 2]
+    fp = M.SoftmaxDenominatorAndMaxFromParts(full, 1)
+    assert fp.parameter_shapes() == [full, full, red, red] and dirs(fp) == [0, 0, 1, 1]
+    assert dirs(M.SoftmaxDenominatorAndMaxFromParts(full, 1, accum=True)) == [0, 0, 2, 2]
+    un = M.SoftmaxDenominatorAndUnscaled(full, 1)
+    assert un.parameter_shapes() == [full, red, full] and dirs(un) == [0, 1, 1]
+    ufm = M.SoftmaxDenominatorAndUnscaledFromMax(full, 1)
+    assert ufm.parameter_shapes() == [full, red, red, full] and dirs(ufm) == [0, 0, 1, 1]
+    assert dirs(M.SoftmaxDenominatorAndUnscaledFromMax(full, 1, accum=True)) == [0, 0, 2, 1]
+    sc = M.SoftmaxComplete(full, 1)
+    assert sc.parameter_shapes() == [full, red, red, full] and dirs(sc) == [0, 0, 0, 1]
+    dv = M.DivideVec(full)
+    assert dv.parameter_shapes() == [full, full] and dirs(dv) == [2, 0]
+    dvs = M.DivideVecScalar(full, 1)
+    assert dvs.parameter_shapes() == [full, red] and dirs(dvs) == [2, 0]
+    bc = M.Broadcast(full, 1)
+    assert bc.parameter_shapes() == [red, full] and dirs(bc) == [0, 1]
+    op = M.OnePrefix([6, 8])
+    assert op.parameter_shapes() == [[6, 8], [1, 6, 8]] and dirs(op) == [0, 1]
+    fl = M.Fill(full, M.i32, M.FillValue.Min)
+    assert fl.parameter_shapes() == [full] and dirs(fl) == [1]
+    for s in (mx, sd, sdm, fp, un, ufm, sc, dv, dvs, bc, op, fl):
+        assert s.check() == 0, s.kind
+    # f32 only; scan_dim in range; no -inf among the integers; OnePrefix output rank <= 5.
+    assert M.Spec(M.SpecKind.Max, full, [M.u8, M.u8], scan_dim=1).check() == 1
+    with pytest.raises(M.MorelloError):
+        M.Max(full, 3)  # no parameter shape exists for a dim outside the tensor
+    assert M.Fill(full, M.i32, M.FillValue.NegInf).check() == 3
+    with pytest.raises(M.MorelloError):
+        M.OnePrefix([2, 2, 2, 2, 2])
+    assert M.Spec(M.SpecKind.SoftmaxDenominatorAndUnscaled, full, [M.f32] * 3, accum=True, scan_dim=1).check() == 1
+
+
 def test_flops_convention():
     # spec.rs:273-305: Matmul 2*b*m*k*n, Softmax 5*volume
     assert M.Matmul([1, 4096, 4096, 4096], [M.u8, M.i8, M.i32]).flops() == 137438953472

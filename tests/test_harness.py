@@ -122,6 +122,17 @@ def test_check_mode_other_specs(gpu, tmp_path):
     want = orc.compose_msm(b, m, k, n2, n, [7, 7, 7, 6], v, q, kt, np.zeros((b, m, n), np.float32))
     got = parse_output(r.stdout, np.float32)
     assert np.abs(got - want).max() / np.abs(want).max() < 1e-2
+    # A primitive with two written parameters prints both, in parameter order.
+    x = synth.normal_f32(504, 0, (4, 50))
+    r = run("softmaxdenominatorandmax:4x50:f32,f32,f32:scan=1",
+            *files_for([x, np.zeros((4, 1), np.float32), np.zeros((4, 1), np.float32)]))
+    assert r.returncode == 0, r.stderr
+    first, second = r.stdout.split("4x1\n")[1:]
+    mx = np.array(first.split(), np.float32).reshape(4, 1)
+    dn = np.array(second.split(), np.float32).reshape(4, 1)
+    wmx, wdn = np.zeros((4, 1), np.float32), np.zeros((4, 1), np.float32)
+    orc.softmax_part(orc.PART_DENOM_MAX, (4, 50), 1, [x, wmx, wdn])
+    assert np.abs(mx - wmx).max() < 1e-6 and np.abs(dn - wdn).max() / wdn.max() < 1e-5
 
 
 @pytest.mark.gpu
