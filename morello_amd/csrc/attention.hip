@@ -125,31 +125,56 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
     const uint8_t *lk = my_lds + stage * STAGE, *lv = lk + TILE;
 
     // S^T tiles: s[kt][r] is key kt*32 + 8*(r/4) + 4*lg + r%4, query lq.
-    // All K operands of the block are requested up front (LDS latency paid once, not per
-    // MFMA), and the two key tiles' accumulation chains alternate so that no MFMA waits
-    // for the result of the one just before it.
+    // K operands come in batches of two d-steps (four MFMAs), two batches ahead of their
+    // MFMAs, so the first MFMA starts after one batch's LDS latency instead of the whole
+    // block's; the two key tiles' accumulation chains alternate.
     v16f s[BKV / 32];
-    v4i kf[BKV / 32][D / 16];
+    v4i kf[3][BKV / 32][2];
+    auto read_k = [&](int q, int buf) {
 #pragma unroll
-    for (int st = 0; st < D / 16; st++)
+      for (int c = 0; c < 2; c++)
 #pragma unroll
-      for (int kt = 0; kt < BKV / 32; kt++) {
-        const int row = kt * 32 + lq;
-        kf[kt][st] = *(const v4i *)(lk + row * ROW + (((2 * st + lg) ^ (row & 15)) << 4));
-      }
+        for (int kt = 0; kt < BKV / 32; kt++) {
+          const int row = kt * 32 + lq, st = 2 * q + c;
+          kf[buf][kt][c] = *(const v4i *)(lk + row * ROW + (((2 * st + lg) ^ (row & 15)) << 4));
+        }
+    };
 #pragma unroll
     for (int kt = 0; kt < BKV / 32; kt++)
 #pragma unroll
       for (int r = 0; r < 16; r++) s[kt][r] = 0.0f;
+    read_k(0, 0);
+    read_k(1, 1);
 #pragma unroll
-    for (int st = 0; st < D / 16; st++)
+    for (int q = 0; q < D / 32; q++) {
+      if (q + 2 < D / 32) read_k(q + 2, (q + 2) % 3);
 #pragma unroll
-      for (int kt = 0; kt < BKV / 32; kt++)
-        s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, kf[kt][st]),
-                                                        __builtin_bit_cast(v8bf, qf[st]), s[kt], 0, 0, 0);
-    // Keep that order in the instruction stream: all LDS reads, then the MFMAs.
-    __builtin_amdgcn_sched_group_barrier(0x100, BKV / 32 * (D / 16), 0);
-    __builtin_amdgcn_sched_group_barrier(0x008, BKV / 32 * (D / 16), 0);
+      for (int c = 0; c < 2; c++)
+#pragma unroll
+        for (int kt = 0; kt < BKV / 32; kt++)
+          s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, kf[q % 3][kt][c]),
+                                                          __builtin_bit_cast(v8bf, qf[2 * q + c]), s[kt], 0, 0, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x100, 4 * (BKV / 32), 0);
+#pragma unroll
+    for (int q = 0; q < D / 32; q++) {
+      if (q + 2 < D / 32) __builtin_amdgcn_sched_group_barrier(0x100, 2 * (BKV / 32), 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 2 * (BKV / 32), 0);
+    }
+    // All V operands of the block are requested now: they land while the softmax runs.
+    v4i vf[BKV / 16][D / 32];
+#pragma unroll
+    for (int u = 0; u < BKV / 16; u++) {
+      const int key = 16 * u + 4 * lg + v_rl;  // key & 3 == v_rl
+#pragma unroll
+      for (int t = 0; t < D / 32; t++) {
+        const int off = ((t ^ v_rl) << 6) + v_within;
+        const v2i lo = read_tr16(lv + key * ROW + off);
+        const v2i hi = read_tr16(lv + (key + 8) * ROW + off);
+        vf[u][t] = v4i{lo[0], lo[1], hi[0], hi[1]};
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
     // Online softmax update for this lane's query, in base 2: exp(x - m) = 2^(x*log2e - m*log2e).
     float mx = s[0][0];
 #pragma unroll
@@ -186,33 +211,11 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
     l_run += psum;
     // O^T += V^T . P^T.  Key step u covers keys 16u + {4*lg + c, 8 + 4*lg + c}, c = 0..3,
     // which is the order P^T's registers already have.
-    // V operands one key step ahead of the MFMAs that use them.
-    v4i vf[2][D / 32];
-    auto read_v = [&](int u, int buf) {
-      const int key = 16 * u + 4 * lg + v_rl;  // key & 3 == v_rl
 #pragma unroll
-      for (int t = 0; t < D / 32; t++) {
-        const int off = ((t ^ v_rl) << 6) + v_within;
-        const v2i lo = read_tr16(lv + key * ROW + off);
-        const v2i hi = read_tr16(lv + (key + 8) * ROW + off);
-        vf[buf][t] = v4i{lo[0], lo[1], hi[0], hi[1]};
-      }
-    };
-    read_v(0, 0);
-#pragma unroll
-    for (int u = 0; u < BKV / 16; u++) {
-      if (u + 1 < BKV / 16) read_v(u + 1, (u + 1) & 1);
+    for (int u = 0; u < BKV / 16; u++)
 #pragma unroll
       for (int t = 0; t < D / 32; t++)
-        o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, vf[u & 1][t]), pb[u], o[t], 0, 0, 0);
-    }
-    // Order: reads of step 0; then per step the reads of the next step ahead of its MFMAs.
-    __builtin_amdgcn_sched_group_barrier(0x100, 2 * (D / 32), 1);
-#pragma unroll
-    for (int u = 0; u < BKV / 16; u++) {
-      if (u + 1 < BKV / 16) __builtin_amdgcn_sched_group_barrier(0x100, 2 * (D / 32), 1);
-      __builtin_amdgcn_sched_group_barrier(0x008, D / 32, 1);
-    }
+        o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, vf[u][t]), pb[u], o[t], 0, 0, 0);
   }
 
   // Merge the two key halves: (m, d, O) of half 1 goes through LDS to the wave of half 0
