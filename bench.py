@@ -185,6 +185,15 @@ def main():
     roofline = {"bound": bound, "achieved": achieved, "peak": peak, "unit": roof_unit,
                 "frac": achieved / peak, "traffic": MEASURED_TRAFFIC_BYTES.get(args.spec),
                 "kernel_ms": kernel_ms, "algorithmic_ops": ops, "algorithmic_bytes": alg_bytes}
+    if bound == "mfma":
+        # What the matrix cores of this board sustain with no memory traffic at all, on
+        # operands distributed like the workload's: the published peak assumes the full
+        # clock, which random operands do not hold at the power limit.
+        kind = "int8" if dtype == "u8" else "bf16"
+        sustained = M.measure_mfma_rate(kind, True) / 1e12
+        roofline["sustained_mfma_peak"] = sustained
+        roofline["sustained_mfma_peak_zero_operands"] = M.measure_mfma_rate(kind, False) / 1e12
+        roofline["frac_of_sustained"] = achieved / sustained
 
     out = {
         "metric": "int8 TOPS / bf16 TFLOPS per Spec on 1 MI355X; % of MFMA or HBM roofline",

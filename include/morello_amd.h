@@ -263,6 +263,15 @@ int mrl_bench(const mrl_spec *spec, void *const *params, uint32_t iters, uint32_
 int mrl_run_timed(const mrl_spec *spec, void *const *params, uint32_t steps,
                   double *device_ms_total);
 
+/* No counterpart in the reference.  Measures what the matrix cores of this board sustain
+ * with every SIMD issuing back-to-back MFMAs on register operands and no memory traffic:
+ * kind 0 = int8 (u8/i8 -> i32), 1 = bf16 (-> f32); random_operands 0 = all-zero operands (the
+ * datapath barely toggles: close to the datasheet rate), 1 = operands distributed like a
+ * benchmark's (the clock settles at the power limit: the ceiling a Matmul kernel can
+ * approach on such data).  `iters` x 32 MFMAs per wavefront (20000 runs about 20 ms).
+ * Writes operations per second (2 per multiply-add). */
+int mrl_measure_mfma_rate(int kind, int random_operands, uint32_t iters, double *ops_per_second);
+
 /* ------------------------------------------- device memory (plumbing only) */
 
 int mrl_device_malloc(void **ptr, size_t bytes);

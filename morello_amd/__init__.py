@@ -462,6 +462,16 @@ def init(device: int = 0):
     _check(B.load().mrl_init(device), "mrl_init")
 
 
+def measure_mfma_rate(kind: str, random_operands: bool, iters: int = 20000) -> float:
+    """Operations per second the matrix cores sustain on register operands: `kind` "int8" or
+    "bf16"; all-zero operands (near the datasheet rate) or benchmark-like random ones (the
+    rate at the board's power limit)."""
+    out = C.c_double()
+    _check(B.load().mrl_measure_mfma_rate({"int8": 0, "bf16": 1}[kind], int(random_operands), iters,
+                                          C.byref(out)), "mrl_measure_mfma_rate")
+    return out.value
+
+
 def synchronize():
     _check(B.load().mrl_device_synchronize(), "mrl_device_synchronize")
 

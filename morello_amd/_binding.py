@@ -75,6 +75,7 @@ SIGNATURES = {
     "mrl_bench": (C.c_int, [C.POINTER(SpecC), _VPP, C.c_uint32, C.c_uint32,
                             C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "mrl_run_timed": (C.c_int, [C.POINTER(SpecC), _VPP, C.c_uint32, C.POINTER(C.c_double)]),
+    "mrl_measure_mfma_rate": (C.c_int, [C.c_int, C.c_int, C.c_uint32, C.POINTER(C.c_double)]),
     "mrl_device_malloc": (C.c_int, [_VPP, C.c_size_t]),
     "mrl_device_free": (C.c_int, [C.c_void_p]),
     "mrl_memcpy_h2d": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),

@@ -919,6 +919,15 @@ int mrl_run_timed(const mrl_spec *spec, void *const *params, uint32_t steps,
   return MRL_OK;
 }
 
+int mrl_measure_mfma_rate(int kind, int random_operands, uint32_t iters, double *ops_per_second) {
+  if (!ops_per_second) return MRL_ERR_NULL;
+  if ((kind != 0 && kind != 1) || iters == 0) return MRL_ERR_BAD_SPEC;
+  int rc;
+  if (g_device < 0 && (rc = mrl_init(0)) != MRL_OK) return rc;
+  HIP_TRY(mrl::measure_mfma_rate(kind, random_operands != 0, iters, nullptr, ops_per_second));
+  return MRL_OK;
+}
+
 int mrl_device_malloc(void **ptr, size_t bytes) {
   if (!ptr) return MRL_ERR_NULL;
   int rc;

@@ -88,6 +88,10 @@ hipError_t launch_broadcast(const void *in, void *out, const LayoutEval &il, con
                             uint32_t dim, uint32_t elem_size, uint64_t count, hipStream_t stream);
 hipError_t launch_fill(void *out, int dtype, int fill_value, uint64_t count, hipStream_t stream);
 
+// ---- mfma_rate.hip: sustained matrix-core rate of this board (measurement, not a Spec) ----
+hipError_t measure_mfma_rate(int kind, bool random_operands, uint32_t iters, hipStream_t stream,
+                             double *ops_per_second);
+
 // ---- attention.hip: fused Matmul -> Softmax -> Matmul on bf16 inputs -------------------
 struct AttnArgs {
   const void *q;   // [b, m, k]   bf16 row-major
