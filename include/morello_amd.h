@@ -263,6 +263,49 @@ int mrl_bench(const mrl_spec *spec, void *const *params, uint32_t iters, uint32_
 int mrl_run_timed(const mrl_spec *spec, void *const *params, uint32_t steps,
                   double *device_ms_total);
 
+/* ------------------------------------------------ general Compose Specs */
+
+/* LogicalSpec::Compose (spec.rs:39-45, 1519-1590): a pipeline of primitive Specs listed
+ * last-executed first, each consuming the output of the one listed after it as its first
+ * input.  A component is a PrimitiveBasics (spec.rs:47-55): type, spec_shape, dtypes. */
+#define MRL_MAX_COMPONENTS 8
+#define MRL_MAX_COMPOSE_PARAMS 12
+
+typedef struct {
+  int32_t kind;      /* mrl_spec_kind with exactly one written parameter; not a Compose   */
+  int32_t accum;     /* must be 0: a component overwrites its output                      */
+  uint32_t scan_dim;
+  uint32_t rank;
+  uint32_t spec_shape[MRL_MAX_SPEC_RANK];
+  uint32_t n_params;
+  int32_t dtypes[MRL_MAX_PARAMS];
+} mrl_component;
+
+typedef struct {
+  uint32_t n_components;
+  mrl_component components[MRL_MAX_COMPONENTS];
+  /* External parameters in the order of compose_parameter_visit (spec.rs:3329-3365): the
+   * first-listed component's inputs after its first, the middle components' likewise, all
+   * inputs of the last-listed component, then the first-listed component's output. */
+  uint32_t n_params;                          /* set by mrl_compose_init */
+  mrl_layout layouts[MRL_MAX_COMPOSE_PARAMS]; /* row-major after mrl_compose_init */
+} mrl_compose;
+
+/* Validates the chain (every component's first input has the shape and dtype of the next
+ * component's output), counts the external parameters and gives each a row-major layout;
+ * the caller may then replace layouts. */
+int mrl_compose_init(mrl_compose *c);
+/* Which (component, component parameter) external parameter `idx` is. */
+int mrl_compose_parameter(const mrl_compose *c, uint32_t idx, uint32_t *component, uint32_t *param);
+int mrl_compose_parameter_shape(const mrl_compose *c, uint32_t idx, uint32_t *shape, uint32_t *rank);
+int mrl_compose_parameter_dtype(const mrl_compose *c, uint32_t idx);
+/* Runs the pipeline on device pointers in external parameter order.  The attention-shaped
+ * [Matmul, Softmax{2}, Matmul] runs on the fused kernel when its conditions hold; any other
+ * chain runs component by component with row-major intermediates of each component's
+ * output dtype in a stream-ordered scratch allocation (the reference's interpreter also
+ * materialises them: verification.rs:239-285, 286-335). */
+int mrl_run_compose(const mrl_compose *c, void *const *params, void *stream);
+
 /* No counterpart in the reference.  Measures what the matrix cores of this board sustain
  * with every SIMD issuing back-to-back MFMAs on register operands and no memory traffic:
  * kind 0 = int8 (u8/i8 -> i32), 1 = bf16 (-> f32); random_operands 0 = all-zero operands (the

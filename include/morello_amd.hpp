@@ -256,6 +256,49 @@ class Spec {
   mrl_spec c_;
 };
 
+// LogicalSpec::Compose (spec.rs:39-45, 1519-1590): components listed last-executed first; the
+// external parameters follow compose_parameter_visit (spec.rs:3329-3365).
+class Compose {
+ public:
+  explicit Compose(const std::vector<Spec> &components) {
+    c_ = mrl_compose{};
+    if (components.size() > MRL_MAX_COMPONENTS) throw Error(MRL_ERR_BAD_SPEC, "Compose");
+    c_.n_components = uint32_t(components.size());
+    for (size_t i = 0; i < components.size(); i++) {
+      const mrl_spec &s = components[i].c();
+      mrl_component &d = c_.components[i];
+      d.kind = s.kind, d.accum = s.accum, d.scan_dim = s.scan_dim, d.rank = s.rank, d.n_params = s.n_params;
+      for (uint32_t k = 0; k < s.rank; k++) d.spec_shape[k] = s.spec_shape[k];
+      for (uint32_t k = 0; k < s.n_params; k++) d.dtypes[k] = s.dtypes[k];
+    }
+    check(mrl_compose_init(&c_), "Compose");
+  }
+  Compose &with_layout(uint32_t param, const Layout &l) {
+    if (param >= c_.n_params) throw Error(MRL_ERR_BAD_SPEC, "with_layout");
+    c_.layouts[param] = l.c();
+    return *this;
+  }
+  size_t parameter_count() const { return c_.n_params; }
+  std::vector<TensorSpec> parameters() const {
+    std::vector<TensorSpec> out;
+    for (uint32_t i = 0; i < c_.n_params; i++) {
+      uint32_t shape[MRL_MAX_RANK], rank = 0;
+      check(mrl_compose_parameter_shape(&c_, i, shape, &rank), "parameters");
+      out.push_back(TensorSpec{Shape(shape, shape + rank), Dtype(mrl_compose_parameter_dtype(&c_, i)),
+                               Layout(c_.layouts[i])});
+    }
+    return out;
+  }
+  void run(const std::vector<void *> &device_params, void *stream = nullptr) const {
+    if (device_params.size() != c_.n_params) throw Error(MRL_ERR_BAD_SPEC, "run");
+    check(mrl_run_compose(&c_, device_params.data(), stream), "run");
+  }
+  const mrl_compose &c() const { return c_; }
+
+ private:
+  mrl_compose c_;
+};
+
 inline void init(int device = 0) { check(mrl_init(device), "init"); }
 
 }  // namespace morello

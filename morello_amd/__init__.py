@@ -421,6 +421,62 @@ def OnePrefix(shape, dtype=f32, layouts=None) -> Spec:
     return Spec(SpecKind.OnePrefix, shape, [dtype] * 2, layouts)
 
 
+class Compose:
+    """LogicalSpec::Compose (spec.rs:39-45, 1519-1590): `components` are Specs listed
+    last-executed first, each consuming the output of the one listed after it as its first
+    input.  External parameters follow compose_parameter_visit (spec.rs:3329-3365).
+    `layouts`: one per external parameter, None = row-major."""
+
+    def __init__(self, components: Sequence[Spec], layouts=None):
+        self.components = list(components)
+        self._c = B.ComposeC()
+        if len(self.components) > B.MAX_COMPONENTS:
+            raise ValueError("too many components")
+        self._c.n_components = len(self.components)
+        for i, comp in enumerate(self.components):
+            cc = self._c.components[i]
+            cc.kind, cc.accum, cc.scan_dim = int(comp.kind), int(comp.accum), comp.scan_dim
+            cc.rank, cc.n_params = len(comp.spec_shape), len(comp.dtypes)
+            for d, v in enumerate(comp.spec_shape):
+                cc.spec_shape[d] = v
+            for p, dt in enumerate(comp.dtypes):
+                cc.dtypes[p] = int(dt)
+        _check(B.load().mrl_compose_init(C.byref(self._c)), "mrl_compose_init")
+        self.n_params = int(self._c.n_params)
+        if layouts is not None:
+            if len(layouts) != self.n_params:
+                raise ValueError("one layout per external parameter")
+            for i, l in enumerate(layouts):
+                if l is not None:
+                    self._c.layouts[i] = l.to_c()
+
+    def parameter(self, idx: int):
+        """(component index, component parameter index) of external parameter `idx`."""
+        comp, par = C.c_uint32(), C.c_uint32()
+        _check(B.load().mrl_compose_parameter(C.byref(self._c), idx, C.byref(comp), C.byref(par)),
+               "mrl_compose_parameter")
+        return comp.value, par.value
+
+    def parameter_shape(self, idx: int):
+        out = (C.c_uint32 * B.MAX_RANK)()
+        rank = C.c_uint32()
+        _check(B.load().mrl_compose_parameter_shape(C.byref(self._c), idx, out, C.byref(rank)),
+               "mrl_compose_parameter_shape")
+        return [int(out[i]) for i in range(rank.value)]
+
+    def parameter_shapes(self):
+        return [self.parameter_shape(i) for i in range(self.n_params)]
+
+    def parameter_dtypes(self):
+        lib = B.load()
+        return [Dtype(lib.mrl_compose_parameter_dtype(C.byref(self._c), i)) for i in range(self.n_params)]
+
+    def run_device(self, ptrs: Sequence[int]):
+        arr = (C.c_void_p * len(ptrs))(*ptrs)
+        _check(B.load().mrl_run_compose(C.byref(self._c), arr, None), "mrl_run_compose")
+        synchronize()
+
+
 class DeviceBuffer:
     """A device allocation owned by Python; plumbing for tests and the benchmark."""
 

@@ -39,6 +39,31 @@ class SpecC(C.Structure):
     ]
 
 
+MAX_COMPONENTS = 8
+MAX_COMPOSE_PARAMS = 12
+
+
+class ComponentC(C.Structure):
+    _fields_ = [
+        ("kind", C.c_int32),
+        ("accum", C.c_int32),
+        ("scan_dim", C.c_uint32),
+        ("rank", C.c_uint32),
+        ("spec_shape", C.c_uint32 * MAX_SPEC_RANK),
+        ("n_params", C.c_uint32),
+        ("dtypes", C.c_int32 * MAX_PARAMS),
+    ]
+
+
+class ComposeC(C.Structure):
+    _fields_ = [
+        ("n_components", C.c_uint32),
+        ("components", ComponentC * MAX_COMPONENTS),
+        ("n_params", C.c_uint32),
+        ("layouts", LayoutC * MAX_COMPOSE_PARAMS),
+    ]
+
+
 _U32P = C.POINTER(C.c_uint32)
 _VPP = C.POINTER(C.c_void_p)
 
@@ -75,6 +100,11 @@ SIGNATURES = {
     "mrl_bench": (C.c_int, [C.POINTER(SpecC), _VPP, C.c_uint32, C.c_uint32,
                             C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "mrl_run_timed": (C.c_int, [C.POINTER(SpecC), _VPP, C.c_uint32, C.POINTER(C.c_double)]),
+    "mrl_compose_init": (C.c_int, [C.POINTER(ComposeC)]),
+    "mrl_compose_parameter": (C.c_int, [C.POINTER(ComposeC), C.c_uint32, _U32P, _U32P]),
+    "mrl_compose_parameter_shape": (C.c_int, [C.POINTER(ComposeC), C.c_uint32, _U32P, _U32P]),
+    "mrl_compose_parameter_dtype": (C.c_int, [C.POINTER(ComposeC), C.c_uint32]),
+    "mrl_run_compose": (C.c_int, [C.POINTER(ComposeC), _VPP, C.c_void_p]),
     "mrl_measure_mfma_rate": (C.c_int, [C.c_int, C.c_int, C.c_uint32, C.POINTER(C.c_double)]),
     "mrl_device_malloc": (C.c_int, [_VPP, C.c_size_t]),
     "mrl_device_free": (C.c_int, [C.c_void_p]),

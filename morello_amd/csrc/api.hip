@@ -511,6 +511,137 @@ int run_one_prefix(const mrl_spec &s, void *const *params, Workspace &ws) {
   return MRL_OK;
 }
 
+int dispatch(const mrl_spec &spec, void *const *params, Workspace &ws) {
+  switch (spec.kind) {
+    case MRL_SPEC_MATMUL: return run_matmul(spec, params, ws);
+    case MRL_SPEC_CONV: return run_conv(spec, params, ws);
+    case MRL_SPEC_SOFTMAX: return run_softmax(spec, params, ws);
+    case MRL_SPEC_COMPOSE_MSM: return run_compose_msm(spec, params, ws);
+    case MRL_SPEC_MOVE: return run_move(spec, params, ws);
+    case MRL_SPEC_FILL: return run_fill(spec, params, ws);
+    case MRL_SPEC_BROADCAST: return run_broadcast(spec, params, ws);
+    case MRL_SPEC_ONE_PREFIX: return run_one_prefix(spec, params, ws);
+    default: return is_parts_kind(spec.kind) ? run_parts(spec, params, ws) : MRL_ERR_UNSUPPORTED;
+  }
+}
+
+// ---- general Compose (spec.rs:1519-1590, 3329-3365) ----
+
+// A component as a stand-alone Spec with row-major layouts.
+int component_spec(const mrl_component &c, mrl_spec *s) {
+  std::memset(s, 0, sizeof *s);
+  s->kind = c.kind, s->accum = c.accum, s->scan_dim = c.scan_dim, s->rank = c.rank, s->n_params = c.n_params;
+  if (c.rank > MRL_MAX_SPEC_RANK || c.n_params > MRL_MAX_PARAMS) return MRL_ERR_BAD_SPEC;
+  for (uint32_t d = 0; d < c.rank; d++) s->spec_shape[d] = c.spec_shape[d];
+  for (uint32_t i = 0; i < c.n_params; i++) s->dtypes[i] = c.dtypes[i];
+  if (c.kind == MRL_SPEC_COMPOSE_MSM || expected_params(c.kind) != c.n_params) return MRL_ERR_BAD_SPEC;
+  for (uint32_t i = 0; i < c.n_params; i++) {
+    uint32_t shape[MRL_MAX_RANK], rank;
+    if (parameter_shape(*s, i, shape, &rank) != MRL_OK) return MRL_ERR_BAD_SPEC;
+    mrl_layout_row_major(shape, rank, &s->layouts[i]);
+  }
+  return MRL_OK;
+}
+
+// spec.rs:1270-1278: the index of the only written parameter, or -1.
+int unique_output_index(const mrl_spec &s) {
+  int found = -1;
+  for (uint32_t i = 0; i < s.n_params; i++)
+    if (parameter_direction(s, i) != 0) {
+      if (found >= 0) return -1;
+      found = int(i);
+    }
+  return found;
+}
+
+struct ComposeParam {
+  uint32_t component, param;
+};
+
+// compose_parameter_visit, spec.rs:3329-3365.
+int compose_parameters(const mrl_compose &c, std::vector<ComposeParam> *out, std::vector<mrl_spec> *specs) {
+  if (c.n_components < 2 || c.n_components > MRL_MAX_COMPONENTS) return MRL_ERR_BAD_SPEC;
+  specs->resize(c.n_components);
+  std::vector<int> out_idx(c.n_components);
+  for (uint32_t i = 0; i < c.n_components; i++) {
+    int rc = component_spec(c.components[i], &(*specs)[i]);
+    if (rc != MRL_OK) return rc;
+    if (c.components[i].accum) return MRL_ERR_BAD_SPEC;
+    if ((rc = check_spec(&(*specs)[i])) != MRL_OK) return rc;
+    if ((out_idx[i] = unique_output_index((*specs)[i])) < 0) return MRL_ERR_BAD_SPEC;
+    if (out_idx[i] == 0) return MRL_ERR_BAD_SPEC;  // the first parameter must be an input to chain on
+  }
+  const uint32_t last = c.n_components - 1;
+  for (uint32_t i = 0; i < c.n_components; i++) {
+    const uint32_t first = i == last ? 0 : 1;
+    for (uint32_t p = first; p < (*specs)[i].n_params; p++)
+      if (int(p) != out_idx[i]) out->push_back({i, p});
+  }
+  out->push_back({0, uint32_t(out_idx[0])});
+  if (out->size() > MRL_MAX_COMPOSE_PARAMS) return MRL_ERR_BAD_SPEC;
+  // Each component's first input is the next-listed component's output.
+  for (uint32_t i = 0; i < last; i++) {
+    uint32_t in_shape[MRL_MAX_RANK], in_rank, o_shape[MRL_MAX_RANK], o_rank;
+    parameter_shape((*specs)[i], 0, in_shape, &in_rank);
+    parameter_shape((*specs)[i + 1], uint32_t(out_idx[i + 1]), o_shape, &o_rank);
+    if (in_rank != o_rank) return MRL_ERR_BAD_SPEC;
+    for (uint32_t d = 0; d < in_rank; d++)
+      if (in_shape[d] != o_shape[d]) return MRL_ERR_BAD_SPEC;
+    if ((*specs)[i].dtypes[0] != (*specs)[i + 1].dtypes[out_idx[i + 1]]) return MRL_ERR_BAD_SPEC;
+  }
+  return MRL_OK;
+}
+
+int run_compose_general(const mrl_compose &c, void *const *params, Workspace &ws) {
+  std::vector<ComposeParam> ext;
+  std::vector<mrl_spec> specs;
+  int rc = compose_parameters(c, &ext, &specs);
+  if (rc != MRL_OK) return rc;
+  if (ext.size() != c.n_params) return MRL_ERR_BAD_SPEC;
+  for (size_t i = 0; i < ext.size(); i++) {
+    if (!params[i]) return MRL_ERR_NULL;
+    mrl_spec &s = specs[ext[i].component];
+    uint32_t shape[MRL_MAX_RANK], rank, phys[MRL_MAX_PHYS];
+    parameter_shape(s, ext[i].param, shape, &rank);
+    if (!mrl::physical_shape(c.layouts[i], shape, rank, phys)) return MRL_ERR_BAD_LAYOUT;
+    s.layouts[ext[i].param] = c.layouts[i];
+  }
+  const uint32_t n = c.n_components;
+  // The attention shape: [Matmul[b,m,n2,n], Softmax{2}[b,m,n2], Matmul[b,m,k,n2]] -> the fused path.
+  if (n == 3 && specs[0].kind == MRL_SPEC_MATMUL && specs[1].kind == MRL_SPEC_SOFTMAX && specs[1].rank == 3 &&
+      specs[1].scan_dim == 2 && specs[2].kind == MRL_SPEC_MATMUL && specs[0].dtypes[2] == MRL_F32 &&
+      specs[0].dtypes[0] == MRL_F32) {
+    mrl_spec msm;
+    std::memset(&msm, 0, sizeof msm);
+    msm.kind = MRL_SPEC_COMPOSE_MSM, msm.rank = 5, msm.n_params = 4;
+    msm.spec_shape[0] = specs[2].spec_shape[0], msm.spec_shape[1] = specs[2].spec_shape[1];
+    msm.spec_shape[2] = specs[2].spec_shape[2], msm.spec_shape[3] = specs[2].spec_shape[3];
+    msm.spec_shape[4] = specs[0].spec_shape[3];
+    msm.dtypes[0] = specs[0].dtypes[1], msm.dtypes[1] = specs[2].dtypes[0], msm.dtypes[2] = specs[2].dtypes[1];
+    msm.dtypes[3] = MRL_F32;
+    for (uint32_t i = 0; i < 4; i++) msm.layouts[i] = c.layouts[i];
+    if (check_spec(&msm) == MRL_OK) return run_compose_msm(msm, params, ws);
+  }
+  // Component by component, last-listed first.
+  void *carried = nullptr;  // the previous component's output
+  for (int i = int(n) - 1; i >= 0; i--) {
+    const mrl_spec &s = specs[i];
+    const int out_idx = unique_output_index(s);
+    void *cp[MRL_MAX_PARAMS] = {nullptr, nullptr, nullptr, nullptr};
+    for (size_t e = 0; e < ext.size(); e++)
+      if (ext[e].component == uint32_t(i)) cp[ext[e].param] = params[e];
+    if (i < int(n) - 1) cp[0] = carried;
+    if (i > 0) {
+      uint32_t shape[MRL_MAX_RANK], rank;
+      parameter_shape(s, uint32_t(out_idx), shape, &rank);
+      HIP_TRY(ws.alloc(&cp[out_idx], size_t(volume(shape, rank)) * mrl_dtype_size(s.dtypes[out_idx])));
+      carried = cp[out_idx];
+    }
+    if ((rc = dispatch(s, cp, ws)) != MRL_OK) return rc;
+  }
+  return MRL_OK;
+}
+
 int run_async_impl(const mrl_spec *spec, void *const *params, hipStream_t stream) {
   if (g_device < 0) {
     int rc = mrl_init(0);
@@ -522,17 +653,7 @@ int run_async_impl(const mrl_spec *spec, void *const *params, hipStream_t stream
   for (uint32_t i = 0; i < spec->n_params; i++)
     if (!params[i]) return MRL_ERR_NULL;
   Workspace ws(stream);
-  switch (spec->kind) {
-    case MRL_SPEC_MATMUL: return run_matmul(*spec, params, ws);
-    case MRL_SPEC_CONV: return run_conv(*spec, params, ws);
-    case MRL_SPEC_SOFTMAX: return run_softmax(*spec, params, ws);
-    case MRL_SPEC_COMPOSE_MSM: return run_compose_msm(*spec, params, ws);
-    case MRL_SPEC_MOVE: return run_move(*spec, params, ws);
-    case MRL_SPEC_FILL: return run_fill(*spec, params, ws);
-    case MRL_SPEC_BROADCAST: return run_broadcast(*spec, params, ws);
-    case MRL_SPEC_ONE_PREFIX: return run_one_prefix(*spec, params, ws);
-    default: return is_parts_kind(spec->kind) ? run_parts(*spec, params, ws) : MRL_ERR_UNSUPPORTED;
-  }
+  return dispatch(*spec, params, ws);
 }
 
 void set_conv_default_layouts(mrl_spec *s) {
@@ -917,6 +1038,54 @@ int mrl_run_timed(const mrl_spec *spec, void *const *params, uint32_t steps,
   if (e != hipSuccess) return hip_fail(e, "event timing");
   *device_ms_total = double(ms);
   return MRL_OK;
+}
+
+int mrl_compose_init(mrl_compose *c) {
+  if (!c) return MRL_ERR_NULL;
+  std::vector<ComposeParam> ext;
+  std::vector<mrl_spec> specs;
+  int rc = compose_parameters(*c, &ext, &specs);
+  if (rc != MRL_OK) return rc;
+  c->n_params = uint32_t(ext.size());
+  for (size_t i = 0; i < ext.size(); i++) c->layouts[i] = specs[ext[i].component].layouts[ext[i].param];
+  return MRL_OK;
+}
+
+int mrl_compose_parameter(const mrl_compose *c, uint32_t idx, uint32_t *component, uint32_t *param) {
+  if (!c || !component || !param) return MRL_ERR_NULL;
+  std::vector<ComposeParam> ext;
+  std::vector<mrl_spec> specs;
+  int rc = compose_parameters(*c, &ext, &specs);
+  if (rc != MRL_OK) return rc;
+  if (idx >= ext.size()) return MRL_ERR_BAD_SPEC;
+  *component = ext[idx].component, *param = ext[idx].param;
+  return MRL_OK;
+}
+
+int mrl_compose_parameter_shape(const mrl_compose *c, uint32_t idx, uint32_t *shape, uint32_t *rank) {
+  if (!c || !shape || !rank) return MRL_ERR_NULL;
+  std::vector<ComposeParam> ext;
+  std::vector<mrl_spec> specs;
+  int rc = compose_parameters(*c, &ext, &specs);
+  if (rc != MRL_OK) return rc;
+  if (idx >= ext.size()) return MRL_ERR_BAD_SPEC;
+  return parameter_shape(specs[ext[idx].component], ext[idx].param, shape, rank);
+}
+
+int mrl_compose_parameter_dtype(const mrl_compose *c, uint32_t idx) {
+  if (!c) return -1;
+  std::vector<ComposeParam> ext;
+  std::vector<mrl_spec> specs;
+  if (compose_parameters(*c, &ext, &specs) != MRL_OK || idx >= ext.size()) return -1;
+  return specs[ext[idx].component].dtypes[ext[idx].param];
+}
+
+int mrl_run_compose(const mrl_compose *c, void *const *params, void *stream) {
+  if (!c || !params) return MRL_ERR_NULL;
+  int rc;
+  if (g_device < 0 && (rc = mrl_init(0)) != MRL_OK) return rc;
+  Workspace ws(static_cast<hipStream_t>(stream));
+  return run_compose_general(*c, params, ws);
 }
 
 int mrl_measure_mfma_rate(int kind, int random_operands, uint32_t iters, double *ops_per_second) {

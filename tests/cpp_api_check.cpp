@@ -38,6 +38,25 @@ int main() {
   EXPECT((msm.parameter_shape(2) == Shape{16, 128, 2048}));
   EXPECT(Spec::matmul({1, 4096, 4096, 4096}, Dtype::Uint8, Dtype::Sint8, Dtype::Sint32).flops() == 137438953472ull);
   EXPECT(!Spec::matmul({1, 4, 4, 4}, Dtype::Float32, Dtype::Float32, Dtype::Bfloat16).is_supported());
+  // The primitives of the Softmax decomposition and a general Compose (spec.rs:3733-3785).
+  Spec sdm = Spec::softmax_part(SpecType::SoftmaxDenominatorAndMax, {4, 6, 8}, 1, true);
+  EXPECT(sdm.parameter_count() == 3 && (sdm.parameter_shape(2) == Shape{4, 1, 8}));
+  EXPECT(sdm.parameter_direction(1) == OperandDirection::InOut);
+  EXPECT(Spec::fill({3, 3}, Dtype::Sint32, FillValue::Min).parameter_direction(0) == OperandDirection::Out);
+  EXPECT((Spec::one_prefix({6, 8}, Dtype::Float32).parameter_shape(1) == Shape{1, 6, 8}));
+  Compose chain({Spec::matmul({16, 128, 128, 128}, Dtype::Uint8, Dtype::Uint16, Dtype::Uint32),
+                 Spec::matmul({16, 128, 128, 128}, Dtype::Uint32, Dtype::Uint16, Dtype::Uint8),
+                 Spec::matmul({16, 128, 128, 128}, Dtype::Uint8, Dtype::Uint8, Dtype::Uint32)});
+  EXPECT(chain.parameter_count() == 5);
+  EXPECT(chain.parameters()[0].dtype == Dtype::Uint16 && chain.parameters()[2].dtype == Dtype::Uint8 &&
+         chain.parameters()[4].dtype == Dtype::Uint32);
+  try {
+    Compose bad_chain({Spec::matmul({1, 4, 8, 4}, Dtype::Float32, Dtype::Float32, Dtype::Float32),
+                       Spec::matmul({1, 4, 4, 4}, Dtype::Float32, Dtype::Float32, Dtype::Float32)});
+    EXPECT(false);
+  } catch (const Error &e) {
+    EXPECT(e.status() == MRL_ERR_BAD_SPEC);
+  }
   // error behaviour: exceptions carry the status code
   try {
     Spec::softmax({4, 4}, 1).parameter_shape(5);
