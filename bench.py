@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the Spec execution path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--spec c2|c3|c4|c5] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--spec c1|c2|c2o|c3|c4|c5|softmax|move] [--no-cpu]
 
 A step is one launch of the workload Spec through the C ABI on tensors already resident in
 HBM.  The default workload is the one the headline metric is quoted on: the quantized
@@ -46,11 +46,27 @@ KT_LAYOUT = M.layout(0, 2, 1)
 def workload(name):
     """-> (description, spec, input arrays in Spec order, compute dtype, unit, bound, peak,
     algorithmic ops per launch, algorithmic bytes per launch)."""
+    if name == "c1":
+        # The reference's own CPU-runnable case (examples/simple_matmul_x86.rs): launch-latency
+        # bound on a GPU, reported as a time; the roofline fraction is not meaningful here.
+        m = k = n = 64
+        spec = M.MatmulAccum([1, m, k, n], (M.f32, M.f32, M.f32))
+        arrs = [synth.uniform_f32(1, 0, (m, k)), synth.uniform_f32(1, 1, (k, n)), np.zeros((m, n), np.float32)]
+        return ("MatmulAccum f32[64x64] x f32[64x64] -> f32, row-major (launch-latency bound)", spec, arrs,
+                "f32", "GFLOPS", "hbm", PEAK["hbm_gbs"])
     if name == "c2":
         m = k = n = 4096
         spec = M.MatmulAccum([1, m, k, n], (M.u8, M.i8, M.i32))
         arrs = [synth.uniform_u8(2, 0, (m, k)), synth.uniform_i8(2, 1, (k, n)), np.zeros((m, n), np.int32)]
         return ("MatmulAccum u8[4096x4096] x i8[4096x4096] -> i32[4096x4096], row-major", spec, arrs,
+                "u8", "TOPS", "mfma", PEAK["int8"])
+    if name == "c2o":
+        # The same Matmul without accumulation (overwrites C): what the vendor library's
+        # int8 GEMM computes, for a like-for-like comparison with --vendor-ref.
+        m = k = n = 4096
+        spec = M.Matmul([1, m, k, n], (M.u8, M.i8, M.i32))
+        arrs = [synth.uniform_u8(2, 0, (m, k)), synth.uniform_i8(2, 1, (k, n)), np.zeros((m, n), np.int32)]
+        return ("Matmul (no accumulate) u8[4096x4096] x i8[4096x4096] -> i32[4096x4096], row-major", spec, arrs,
                 "u8", "TOPS", "mfma", PEAK["int8"])
     if name == "c3":
         m = k = n = 8192
@@ -142,14 +158,68 @@ def cpu_baseline(name, arrs):
             "sample": "hand-restated Morello-lowered C (oracle/lowered), OpenMP over output tiles; " + sample}
 
 
+def vendor_reference(name, steps):
+    """What the vendor's library reaches on this box for the nearest operation it offers,
+    through PyTorch (hipBLASLt GEMMs, the built-in attention).  A yardstick printed beside
+    the measurement, not part of it: it runs after the timed region, only with --vendor-ref,
+    and its operations differ as `note` says."""
+    try:
+        import torch
+    except ImportError:
+        return None
+    dev = "cuda"
+
+    def timed(fn):
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps
+
+    if name in ("c2", "c2o"):
+        a = torch.randint(-128, 128, (4096, 4096), device=dev, dtype=torch.int8)
+        b = torch.randint(-128, 128, (4096, 4096), device=dev, dtype=torch.int8)
+        ms = timed(lambda: torch._int_mm(a, b))
+        return {"op": "torch._int_mm i8[4096x4096] x i8[4096x4096] -> i32", "ms": ms,
+                "value": 2 * 4096 ** 3 / ms / 1e9, "unit": "TOPS",
+                "note": "signed x signed, overwrites its output (no accumulate, no u8 operand)"}
+    if name == "c3":
+        a = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
+        b = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
+        ms = timed(lambda: torch.matmul(a, b))
+        return {"op": "torch.matmul bf16[8192x8192] x bf16[8192x8192] -> bf16", "ms": ms,
+                "value": 2 * 8192 ** 3 / ms / 1e9, "unit": "TFLOPS",
+                "note": "bf16 output, overwrites (the Spec writes f32 and accumulates: 4x the output bytes)"}
+    if name == "c5":
+        q, k, v = (torch.randn(1, 16, 2048, 128, device=dev, dtype=torch.bfloat16) * 0.5 for _ in range(3))
+        ms = timed(lambda: torch.nn.functional.scaled_dot_product_attention(q, k, v, scale=1.0))
+        return {"op": "torch scaled_dot_product_attention 16 x 2048 x 128 bf16, scale 1, no mask", "ms": ms,
+                "value": 2 * 2 * 16 * 2048 * 2048 * 128 / ms / 1e9, "unit": "TFLOPS",
+                "note": "bf16 output (the Compose writes f32)"}
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--spec", default="c2", choices=["c2", "c3", "c4", "c5", "softmax", "move"])
+    ap.add_argument("--spec", default="c2", choices=["c1", "c2", "c2o", "c3", "c4", "c5", "softmax", "move"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--vendor-ref", action="store_true",
+                    help="also time the vendor library's nearest operation through PyTorch (c2, c3, c5)")
+    ap.add_argument("--vendor-child", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()
+    if args.vendor_child:
+        # PyTorch brings its own HIP runtime, which cannot share a process with the library's:
+        # the yardstick runs in a child process that touches nothing else.
+        print(json.dumps(vendor_reference(args.spec, args.steps)))
+        return
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this backend has no multi-GPU path "
                          "(Matmul/Conv/Compose tiles shard without communication); run with --gpus 1")
@@ -173,7 +243,7 @@ def main():
     value = ops / (ms_per_step * 1e-3) / 1e12
     if args.spec == "move":
         value = alg_bytes / (ms_per_step * 1e-3) / 1e9
-    if args.spec == "softmax":
+    if args.spec in ("softmax", "c1"):
         value = ops / (ms_per_step * 1e-3) / 1e9
 
     if bound == "mfma":
@@ -203,8 +273,14 @@ def main():
         "config": {"workload": desc, "spec": args.spec, "device": M.device_info()["name"]},
         "roofline": roofline,
     }
-    if not args.no_cpu and args.spec not in ("move", "softmax"):
+    if not args.no_cpu and args.spec not in ("move", "softmax", "c1", "c2o"):
         out["cpu_baseline"] = cpu_baseline(args.spec, arrs)
+    if args.vendor_ref:
+        import subprocess
+        child = subprocess.run([sys.executable, os.path.abspath(__file__), "--vendor-child", "--spec", args.spec,
+                                "--steps", str(args.steps)], capture_output=True, text=True, timeout=600)
+        lines = [l for l in child.stdout.splitlines() if l.startswith("{") or l == "null"]
+        out["vendor_reference"] = json.loads(lines[-1]) if child.returncode == 0 and lines else None
     print(json.dumps(out))
 
 
