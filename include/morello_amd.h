@@ -289,6 +289,12 @@ typedef struct {
    * inputs of the last-listed component, then the first-listed component's output. */
   uint32_t n_params;                          /* set by mrl_compose_init */
   mrl_layout layouts[MRL_MAX_COMPOSE_PARAMS]; /* row-major after mrl_compose_init */
+  /* The schedule knob of scheduling/bufferize.rs:24-116: bit i set = the tensor feeding
+   * component i (the output of component i+1) is materialised in device memory, row-major,
+   * as `bufferize(i, GL, row_major)` would.  Zero (what mrl_compose_init leaves) lets the
+   * library fuse across every boundary it has a kernel for; any set bit runs the pipeline
+   * component by component. */
+  uint32_t bufferize_mask;
 } mrl_compose;
 
 /* Validates the chain (every component's first input has the shape and dtype of the next

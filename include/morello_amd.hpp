@@ -278,6 +278,12 @@ class Compose {
     c_.layouts[param] = l.c();
     return *this;
   }
+  // scheduling/bufferize.rs:24-116 with memory GL and a row-major layout.
+  Compose &bufferize(uint32_t index) {
+    if (index + 1 >= c_.n_components) throw Error(MRL_ERR_BAD_SPEC, "bufferize");
+    c_.bufferize_mask |= 1u << index;
+    return *this;
+  }
   size_t parameter_count() const { return c_.n_params; }
   std::vector<TensorSpec> parameters() const {
     std::vector<TensorSpec> out;

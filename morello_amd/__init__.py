@@ -450,6 +450,18 @@ class Compose:
                 if l is not None:
                     self._c.layouts[i] = l.to_c()
 
+    def bufferize(self, index: int) -> "Compose":
+        """`spec.bufferize(index, GL, row_major)` (scheduling/bufferize.rs:24-116): the tensor
+        feeding component `index` is materialised in device memory instead of staying inside a
+        fused kernel.  Returns a new Compose; the knob accumulates."""
+        if not 0 <= index < len(self.components) - 1:
+            raise MorelloError(3, "bufferize")
+        import copy
+        other = copy.copy(self)
+        other._c = B.ComposeC.from_buffer_copy(self._c)
+        other._c.bufferize_mask |= 1 << index
+        return other
+
     def parameter(self, idx: int):
         """(component index, component parameter index) of external parameter `idx`."""
         comp, par = C.c_uint32(), C.c_uint32()

@@ -61,6 +61,7 @@ class ComposeC(C.Structure):
         ("components", ComponentC * MAX_COMPONENTS),
         ("n_params", C.c_uint32),
         ("layouts", LayoutC * MAX_COMPOSE_PARAMS),
+        ("bufferize_mask", C.c_uint32),
     ]
 
 

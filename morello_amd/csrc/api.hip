@@ -608,7 +608,8 @@ int run_compose_general(const mrl_compose &c, void *const *params, Workspace &ws
   }
   const uint32_t n = c.n_components;
   // The attention shape: [Matmul[b,m,n2,n], Softmax{2}[b,m,n2], Matmul[b,m,k,n2]] -> the fused path.
-  if (n == 3 && specs[0].kind == MRL_SPEC_MATMUL && specs[1].kind == MRL_SPEC_SOFTMAX && specs[1].rank == 3 &&
+  if (c.bufferize_mask >> (n - 1)) return MRL_ERR_BAD_SPEC;  // only boundaries 0 .. n-2 exist
+  if (c.bufferize_mask == 0 && n == 3 && specs[0].kind == MRL_SPEC_MATMUL && specs[1].kind == MRL_SPEC_SOFTMAX && specs[1].rank == 3 &&
       specs[1].scan_dim == 2 && specs[2].kind == MRL_SPEC_MATMUL && specs[0].dtypes[2] == MRL_F32 &&
       specs[0].dtypes[0] == MRL_F32) {
     mrl_spec msm;
@@ -1047,6 +1048,7 @@ int mrl_compose_init(mrl_compose *c) {
   int rc = compose_parameters(*c, &ext, &specs);
   if (rc != MRL_OK) return rc;
   c->n_params = uint32_t(ext.size());
+  c->bufferize_mask = 0;
   for (size_t i = 0; i < ext.size(); i++) c->layouts[i] = specs[ext[i].component].layouts[ext[i].param];
   return MRL_OK;
 }

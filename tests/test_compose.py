@@ -95,6 +95,15 @@ def test_general_compose_equals_the_attention_spec(gpu):
     kt = np.ascontiguousarray(kmat.transpose(0, 2, 1))
     want = orc.compose_msm(b, m, k, n2, n, [7, 7, 7, 6], v, q, kt, np.zeros((b, m, n), np.float32))
     assert np.abs(got - want).max() / np.abs(want).max() < 1e-2
+    # bufferize (scheduling/bufferize.rs): with the softmax input or output materialised the
+    # pipeline runs component by component with f32 intermediates, as the reference's
+    # interpreter does, and lands within 1e-5 of the oracle instead of the fused kernel's 1e-3.
+    fused_err = np.abs(got - want).max() / np.abs(want).max()
+    for idx in (0, 1):
+        staged = _run(c.bufferize(idx), [v, q, kmat, np.zeros((b, m, n), np.float32)])
+        assert np.abs(staged - want).max() / np.abs(want).max() < 1e-5 < fused_err
+    with pytest.raises(M.MorelloError):
+        c.bufferize(2)
     # A shape the fused kernel does not take (head dim 64) runs component by component.
     b, m, k, n2, n = 2, 48, 64, 80, 24
     q = synth.normal_f32(903, 0, (b, m, k), 0.5)
