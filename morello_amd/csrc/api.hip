@@ -305,8 +305,12 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
     const int kind = (da == MRL_I8 && db == MRL_I8 && dc == MRL_I32)     ? 0
                      : (da == MRL_U8 && db == MRL_I8 && dc == MRL_I32)   ? 1
                      : (da == MRL_BF16 && db == MRL_BF16 && dc == MRL_F32) ? 2
+                     : (da == MRL_F32 && db == MRL_F32 && dc == MRL_F32)   ? 3
                                                                            : -1;
-    const bool ok = kind >= 0 && rows && (kind == 2 ? mrl::gemm_bf16_applicable(g) : mrl::gemm_i8_applicable(g, false));
+    const bool ok = kind >= 0 && rows &&
+                    (kind == 3   ? mrl::gemm_f32_applicable(g)
+                     : kind == 2 ? mrl::gemm_bf16_applicable(g)
+                                 : mrl::gemm_i8_applicable(g, false));
     if (!ok) return MRL_ERR_UNSUPPORTED;
     hipError_t e = mrl::launch_gemm_scheduled(g, kind, sched->tile_m, sched->tile_n, sched->split_k, ws.stream);
     if (e == hipErrorInvalidValue) return MRL_ERR_UNSUPPORTED;
@@ -320,6 +324,9 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
   } else if (rows && da == MRL_BF16 && db == MRL_BF16 && dc == MRL_F32 &&
              mrl::gemm_bf16_applicable(g)) {
     HIP_TRY(mrl::launch_gemm_bf16(g, ws.stream));
+    done = true;
+  } else if (rows && da == MRL_F32 && db == MRL_F32 && dc == MRL_F32 && mrl::gemm_f32_applicable(g)) {
+    HIP_TRY(mrl::launch_gemm_f32(g, ws.stream));
     done = true;
   }
   if (!done) HIP_TRY(mrl::launch_matmul_generic(a.t, b.t, c.t, s.accum, ws.stream));
@@ -969,6 +976,7 @@ uint32_t mrl_matmul_schedules(const mrl_spec *spec, mrl_matmul_schedule *out, ui
   int es = 0;
   if ((da == MRL_U8 || da == MRL_I8) && db == MRL_I8 && dc == MRL_I32) es = 1;
   if (da == MRL_BF16 && db == MRL_BF16 && dc == MRL_F32) es = 2;
+  if (da == MRL_F32 && db == MRL_F32 && dc == MRL_F32) es = 4;
   if (!es) return 0;
   const uint32_t n = mrl::gemm_schedule_count();
   for (uint32_t i = 0; i < n && out && i < cap; i++)

@@ -32,6 +32,11 @@ hipError_t launch_gemm_i8(const GemmArgs &g, bool a_unsigned, hipStream_t stream
     return a_unsigned ? launch<I8, true, TileBig, false>(g, stream) : launch<I8, false, TileBig, false>(g, stream);
   return a_unsigned ? launch<I8, true, TileBig, true>(g, stream) : launch<I8, false, TileBig, true>(g, stream);
 }
+bool gemm_f32_applicable(const GemmArgs &g) { return applicable(g, 4); }
+hipError_t launch_gemm_f32(const GemmArgs &g, hipStream_t stream) {
+  return whole_tiles(g, 4) ? launch<F32, false, TileBig, false>(g, stream)
+                           : launch<F32, false, TileBig, true>(g, stream);
+}
 bool gemm_bf16_applicable(const GemmArgs &g) { return applicable(g, 2); }
 hipError_t launch_gemm_bf16(const GemmArgs &g, hipStream_t stream) {
   return whole_tiles(g, 2) ? launch<BF16, false, TileBig, false>(g, stream)

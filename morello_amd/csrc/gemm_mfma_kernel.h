@@ -1,5 +1,6 @@
-// Matmul on the gfx950 matrix cores: u8|i8 x i8 -> i32 (v_mfma_i32_32x32x32_i8) and
-// bf16 x bf16 -> f32 (v_mfma_f32_32x32x16_bf16), one tile pipeline for both.
+// Matmul on the gfx950 matrix cores: u8|i8 x i8 -> i32 (v_mfma_i32_32x32x32_i8),
+// bf16 x bf16 -> f32 (v_mfma_f32_32x32x16_bf16) and f32 x f32 -> f32
+// (v_mfma_f32_32x32x2_f32), one tile pipeline for all three.
 //
 // What it computes is Morello's MatmulAccum on row-major operands
 // (morello/src/spec.rs:480-485): C[i,j] (=0 unless accum) += sum_k A[i,k]*B[k,j].  The
@@ -60,6 +61,7 @@ struct I8 {
   static constexpr int ES = 1;             // element bytes
   static constexpr int PAD = 32;           // 8 k-rows x 32 B cover all 64 banks
   static constexpr int K_PER_READ = 8;     // k rows covered by one transposing read
+  static constexpr bool TRANSPOSED_READ = true;
   __device__ static v2i read_tr(const uint8_t *p) {
     return __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i *)p);
   }
@@ -73,6 +75,7 @@ struct BF16 {
   static constexpr int ES = 2;
   static constexpr int PAD = 64;           // 4 k-rows x 64 B cover all 64 banks
   static constexpr int K_PER_READ = 4;
+  static constexpr bool TRANSPOSED_READ = true;
   __device__ static v2i read_tr(const uint8_t *p) {
     const v4s r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s *)p);
     return __builtin_bit_cast(v2i, r);
@@ -80,6 +83,30 @@ struct BF16 {
   __device__ static Acc mfma(v4i a, v4i b, Acc c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a),
                                                    __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+  }
+};
+
+// f32 operands, f32 accumulation.  One 32-byte k step is 8 values of k = four MFMAs of k = 2:
+// lane half h of MFMA j takes k = 4h + j from both operands (any pairing of k values is a
+// valid order of the sum as long as A and B agree), which makes A's share 16 contiguous
+// bytes like the other types.  B needs no transposition: a lane reads its column's value from
+// each of its four k rows (32 lanes x 4 bytes = 128 contiguous bytes per row).
+struct F32 {
+  typedef v16f Acc;
+  typedef float Out;
+  static constexpr int ES = 4;
+  static constexpr int PAD = 32;           // rows k and k+4 land on opposite bank halves
+  static constexpr int K_PER_READ = 1;
+  static constexpr bool TRANSPOSED_READ = false;
+  __device__ static v2i read_tr(const uint8_t *) { return v2i{0, 0}; }
+  __device__ static Acc mfma(v4i a, v4i b, Acc c) {
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    const v4f fa = __builtin_bit_cast(v4f, a), fb = __builtin_bit_cast(v4f, b);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[0], fb[0], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[1], fb[1], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[2], fb[2], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[3], fb[3], c, 0, 0, 0);
+    return c;
   }
 };
 
@@ -145,6 +172,23 @@ __device__ inline void epilogue(const GemmArgs &g, typename T::Out *C, uint8_t *
         if (inside(tm, tn, r))
           __builtin_nontemporal_store(v, &c_lane[int64_t(tm * 32 + (r >> 2) * 8 + (r & 3)) * g.ldc + tn * 32]);
       }
+  }
+}
+
+// Pins the instruction order of one k step: slot I of N issues MFMA_PER MFMAs, then its even
+// share of the step's DS_READS operand reads, then (in the step that stages the next tile)
+// one LDS write and one global load while any of the MEM_OPS are left.
+template <int I, int N, int MFMA_PER, int DS_READS, int MEM_OPS>
+__device__ inline void sched_slots(bool staging) {
+  if constexpr (I < N) {
+    __builtin_amdgcn_sched_group_barrier(0x008, MFMA_PER, 0);  // MFMA
+    constexpr int FIRST = DS_READS * I / N, END = DS_READS * (I + 1) / N;
+    if constexpr (END > FIRST) __builtin_amdgcn_sched_group_barrier(0x100, END - FIRST, 0);  // DS read
+    if (staging && I < MEM_OPS) {
+      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // DS write
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // VMEM read
+    }
+    sched_slots<I + 1, N, MFMA_PER, DS_READS, MEM_OPS>(staging);
   }
 }
 
@@ -226,11 +270,15 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
   int b_frag[TN];
 #pragma unroll
   for (int tn = 0; tn < TN; tn++) {
-    constexpr int LANES_PER_ROW = 16 / (8 / ES);  // lanes that share one k row: 2 (i8), 4 (bf16)
-    const int p = lane & 15;
-    const int k = (K_SLAB / 2) * (lane >> 5) + p / LANES_PER_ROW;
-    const int col = wn * WN + tn * 32 + 16 * ((lane >> 4) & 1) + (8 / ES) * (p % LANES_PER_ROW);
-    b_frag[tn] = A_STAGE + k * B_ROW + col * ES;
+    if constexpr (T::TRANSPOSED_READ) {
+      constexpr int LANES_PER_ROW = 16 / (8 / ES);  // lanes that share one k row: 2 (i8), 4 (bf16)
+      const int p = lane & 15;
+      const int k = (K_SLAB / 2) * (lane >> 5) + p / LANES_PER_ROW;
+      const int col = wn * WN + tn * 32 + 16 * ((lane >> 4) & 1) + (8 / ES) * (p % LANES_PER_ROW);
+      b_frag[tn] = A_STAGE + k * B_ROW + col * ES;
+    } else {
+      b_frag[tn] = A_STAGE + (K_SLAB / 2) * (lane >> 5) * B_ROW + (wn * WN + tn * 32 + (lane & 31)) * ES;
+    }
   }
 
   Acc acc[TM][TN];
@@ -298,9 +346,15 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
       af[buf][tm] = *(const v4i *)(base + a_frag[tm] + (((2 * s + a_half) ^ a_swz) << 4));
 #pragma unroll
     for (int tn = 0; tn < TN; tn++) {
-      const v2i lo = T::read_tr(base + b_frag[tn] + (s * K_SLAB) * B_ROW);
-      const v2i hi = T::read_tr(base + b_frag[tn] + (s * K_SLAB + T::K_PER_READ) * B_ROW);
-      bf[buf][tn] = v4i{lo[0], lo[1], hi[0], hi[1]};
+      if constexpr (T::TRANSPOSED_READ) {
+        const v2i lo = T::read_tr(base + b_frag[tn] + (s * K_SLAB) * B_ROW);
+        const v2i hi = T::read_tr(base + b_frag[tn] + (s * K_SLAB + T::K_PER_READ) * B_ROW);
+        bf[buf][tn] = v4i{lo[0], lo[1], hi[0], hi[1]};
+      } else {
+        const uint8_t *col = base + b_frag[tn] + (s * K_SLAB) * B_ROW;
+        bf[buf][tn] = v4i{*(const int *)col, *(const int *)(col + B_ROW), *(const int *)(col + 2 * B_ROW),
+                          *(const int *)(col + 3 * B_ROW)};
+      }
     }
   };
   auto mfma_slab = [&](int s, int buf) {
@@ -350,16 +404,9 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
         read_frags(cur ^ 1, 0, 0);
       }
       mfma_slab(s, s & 1);
-      // One MFMA, then a share of this step's memory instructions, TM*TN times.
-#pragma unroll
-      for (int i = 0; i < TM * TN; i++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-        if (i < TM + 2 * TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
-        if (s == SLABS - 2) {
-          if (i < A_CH + B_CH) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // DS write
-          if (i < A_CH + B_CH) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // VMEM read
-        }
-      }
+      // One output block's MFMAs, then a share of this step's memory instructions, TM*TN times.
+      sched_slots<0, TM * TN, T::TRANSPOSED_READ ? 1 : 4, TM + (T::TRANSPOSED_READ ? 2 : 4) * TN, A_CH + B_CH>(
+          s == SLABS - 2);
     }
   }
 

@@ -19,7 +19,7 @@ typedef Tile<128, 128, 64, 2, 2> T128x128k64;
 struct Entry {
   uint32_t tile_m, tile_n, k_bytes;
 };
-// k_bytes is the k step in bytes of an operand row: 128 = 128 i8 or 64 bf16 elements.
+// k_bytes is the k step in bytes of an operand row: 128 = 128 i8, 64 bf16 or 32 f32 elements.
 const Entry kSchedules[] = {{256, 256, 128}, {256, 256, 64}, {256, 128, 64}, {128, 256, 64}, {128, 128, 64}};
 
 template <class TL>
@@ -27,7 +27,8 @@ hipError_t launch_kind(const GemmArgs &g, int kind, hipStream_t stream) {
   switch (kind) {
     case 0: return launch<I8, false, TL, true>(g, stream);
     case 1: return launch<I8, true, TL, true>(g, stream);
-    default: return launch<BF16, false, TL, true>(g, stream);
+    case 2: return launch<BF16, false, TL, true>(g, stream);
+    default: return launch<F32, false, TL, true>(g, stream);
   }
 }
 
@@ -39,13 +40,14 @@ void gemm_schedule_at(uint32_t i, int elem_size, uint32_t *tile_m, uint32_t *til
   *tile_m = kSchedules[i].tile_m, *tile_n = kSchedules[i].tile_n, *split_k = kSchedules[i].k_bytes / elem_size;
 }
 
-// kind: 0 = i8 x i8, 1 = u8 x i8, 2 = bf16 x bf16.  Returns hipErrorInvalidValue for a
+// kind: 0 = i8 x i8, 1 = u8 x i8, 2 = bf16 x bf16, 3 = f32 x f32.  Returns hipErrorInvalidValue for a
 // schedule that is not built.
 hipError_t launch_gemm_scheduled(const GemmArgs &g, int kind, uint32_t tile_m, uint32_t tile_n,
                                  uint32_t split_k, hipStream_t stream) {
-  const uint32_t k_bytes = split_k * (kind == 2 ? 2 : 1);
+  const uint32_t k_bytes = split_k * (kind == 2 ? 2 : kind == 3 ? 4 : 1);
   if (tile_m == 256 && tile_n == 256 && k_bytes == 128)
-    return kind == 2 ? launch_gemm_bf16(g, stream) : launch_gemm_i8(g, kind == 1, stream);
+    return kind == 3 ? launch_gemm_f32(g, stream)
+                     : kind == 2 ? launch_gemm_bf16(g, stream) : launch_gemm_i8(g, kind == 1, stream);
   if (tile_m == 256 && tile_n == 256 && k_bytes == 64) return launch_kind<T256x256k64>(g, kind, stream);
   if (tile_m == 256 && tile_n == 128 && k_bytes == 64) return launch_kind<T256x128k64>(g, kind, stream);
   if (tile_m == 128 && tile_n == 256 && k_bytes == 64) return launch_kind<T128x256k64>(g, kind, stream);

@@ -49,6 +49,8 @@ bool gemm_i8_applicable(const GemmArgs &g, bool b_k_contiguous);
 hipError_t launch_gemm_i8(const GemmArgs &g, bool a_unsigned, hipStream_t stream);
 
 // ---- gemm_bf16.hip: bf16 x bf16 -> f32 on the bf16 MFMA --------------------------------
+bool gemm_f32_applicable(const GemmArgs &g);
+hipError_t launch_gemm_f32(const GemmArgs &g, hipStream_t stream);
 bool gemm_bf16_applicable(const GemmArgs &g);
 hipError_t launch_gemm_bf16(const GemmArgs &g, hipStream_t stream);
 

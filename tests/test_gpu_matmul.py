@@ -141,6 +141,25 @@ def test_bf16_matmul(gpu, shape, accum):
     assert rel_err(got, want) < 1e-5  # what f32 accumulation actually delivers at these K
 
 
+@pytest.mark.parametrize("shape,accum", [((1, 256, 32, 256), False), ((1, 512, 512, 512), True),
+                                         ((2, 256, 96, 256), False), ((1, 300, 100, 264), True),
+                                         ((2, 129, 68, 516), False), ((1, 64, 64, 64), True)])
+def test_f32_matmul_on_the_matrix_cores(gpu, shape, accum):
+    """f32 x f32 -> f32 from 64 x 64 x 64 up runs on v_mfma_f32_32x32x2_f32: whole tiles,
+    ragged borders (rows of whole 16-byte chunks), batches, accumulation."""
+    b, m, k, n = shape
+    A, Bm = synth.uniform_f32(61, 0, (b, m, k)), synth.uniform_f32(61, 1, (b, k, n))
+    C0 = synth.normal_f32(61, 2, (b, m, n)) if accum else np.zeros((b, m, n), np.float32)
+    got = run_spec(M.Matmul(shape, [M.f32] * 3, accum=accum), [A, Bm, C0])
+    want = np.matmul(A.astype(np.float64), Bm.astype(np.float64)) + (C0 if accum else 0)
+    assert rel_err(got, want) < 1e-5
+    assert rel_err(got, orc.matmul(list(shape), [6, 6, 6], A, Bm, C0.copy(), accum)) < 1e-5
+    # Integer-valued inputs (the reference's 0..3 pattern): every partial sum is exact.
+    A, Bm = synth.check_pattern("f32", (b, m, k)), synth.check_pattern("f32", (b, k, n))
+    got = run_spec(M.Matmul(shape, [M.f32] * 3), [A, Bm, np.zeros((b, m, n), np.float32)])
+    assert np.array_equal(got, np.matmul(A.astype(np.int64), Bm.astype(np.int64)).astype(np.float32))
+
+
 def test_bf16_matmul_pattern_exact(gpu):
     """0..3 inputs (verification.rs:933-935): every partial sum is an exact integer."""
     b, m, k, n = 1, 256, 256, 256
@@ -232,8 +251,18 @@ def test_manual_schedules_give_identical_results(gpu):
         bufs = [M.DeviceBuffer.from_numpy(x) for x in (A, Bm, np.zeros((b, m, n), np.float32))]
         spec.tile_out([1, tm, tn]).split(sk).run_device([x.ptr for x in bufs])
         assert rel_err(bufs[2].to_numpy(np.float32, (b, m, n)), want) < 1e-5, (tm, tn, sk)
+    # f32: split counted in elements (16 f32 = 64 bytes)
+    b, m, k, n = 1, 320, 136, 264
+    A, Bm = synth.uniform_f32(94, 0, (b, m, k)), synth.uniform_f32(94, 1, (b, k, n))
+    fspec = M.Matmul([b, m, k, n], [M.f32] * 3)
+    want = np.matmul(A.astype(np.float64), Bm.astype(np.float64))
+    assert (256, 256, 32) in fspec.available_schedules() and (128, 128, 16) in fspec.available_schedules()
+    for tm, tn, sk in fspec.available_schedules():
+        fb = [M.DeviceBuffer.from_numpy(x) for x in (A, Bm, np.zeros((b, m, n), np.float32))]
+        fspec.tile_out([1, tm, tn]).split(sk).run_device([x.ptr for x in fb])
+        assert rel_err(fb[2].to_numpy(np.float32, (b, m, n)), want) < 1e-5, (tm, tn, sk)
     # a schedule that is not built, and a Spec without a matrix-core kernel
     with pytest.raises(M.MorelloError) as e:
         spec.tile_out([1, 64, 64]).split(32).run_device([x.ptr for x in bufs])
     assert e.value.status == 1
-    assert M.Matmul([1, 64, 64, 64], [M.f32] * 3).available_schedules() == []
+    assert M.Matmul([1, 64, 64, 64], [M.u32] * 3).available_schedules() == []
