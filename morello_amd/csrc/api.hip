@@ -383,41 +383,60 @@ int run_softmax(const mrl_spec &s, void *const *params, Workspace &ws) {
 }
 
 int run_compose_msm(const mrl_spec &s, void *const *params, Workspace &ws) {
-  Prepared v, q, kt, out;
-  int rc;
-  if ((rc = prepare(s, 0, params[0], true, ws, &v)) != MRL_OK) return rc;
-  if ((rc = prepare(s, 1, params[1], true, ws, &q)) != MRL_OK) return rc;
-  if ((rc = prepare(s, 2, params[2], true, ws, &kt)) != MRL_OK) return rc;
-  if ((rc = prepare(s, 3, params[3], false, ws, &out)) != MRL_OK) return rc;
   const uint32_t b = s.spec_shape[0], m = s.spec_shape[1], k = s.spec_shape[2], n2 = s.spec_shape[3],
                  n = s.spec_shape[4];
-  // Fused path: bf16 Q, V row-major and KT stored k-fastest (layout![0,2,1]).
-  const bool kt_k_fastest = (k == 1 || kt.t.stride[1] == 1) && (n2 == 1 || kt.t.stride[2] == int64_t(k)) &&
-                            (b == 1 || kt.t.stride[0] == int64_t(k) * n2);
-  mrl::AttnArgs at;
-  at.q = q.t.ptr, at.kt = kt.t.ptr, at.v = v.t.ptr, at.out = (float *)out.t.ptr;
-  at.b = b, at.m = m, at.k = k, at.n2 = n2, at.n = n;
-  if (s.dtypes[0] == MRL_BF16 && s.dtypes[1] == MRL_BF16 && s.dtypes[2] == MRL_BF16 &&
-      dense_row_major(q.t) && dense_row_major(v.t) && dense_row_major(out.t) && kt_k_fastest &&
-      mrl::attn_applicable(at)) {
-    HIP_TRY(mrl::launch_attn(at, ws.stream));
-    return finish_output(out, ws);
+  // Fused path: bf16 Q, V row-major and KT stored k-fastest (layout![0,2,1]), all usable in place.
+  mrl::Strided t[4];
+  bool in_place = true;
+  for (uint32_t i = 0; i < 4; i++) {
+    uint32_t shape[MRL_MAX_RANK], rank;
+    parameter_shape(s, i, shape, &rank);
+    t[i].ptr = params[i], t[i].dtype = s.dtypes[i], t[i].rank = rank;
+    for (uint32_t d = 0; d < MRL_MAX_RANK; d++) t[i].shape[d] = d < rank ? shape[d] : 1;
+    in_place = in_place && mrl::layout_strides(s.layouts[i], shape, rank, t[i].stride);
+  }
+  if (in_place && s.dtypes[0] == MRL_BF16 && s.dtypes[1] == MRL_BF16 && s.dtypes[2] == MRL_BF16) {
+    const mrl::Strided &v = t[0], &q = t[1], &kt = t[2], &out = t[3];
+    const bool kt_k_fastest = (k == 1 || kt.stride[1] == 1) && (n2 == 1 || kt.stride[2] == int64_t(k)) &&
+                              (b == 1 || kt.stride[0] == int64_t(k) * n2);
+    mrl::AttnArgs at;
+    at.q = q.ptr, at.kt = kt.ptr, at.v = v.ptr, at.out = (float *)out.ptr;
+    at.b = b, at.m = m, at.k = k, at.n2 = n2, at.n = n;
+    if (dense_row_major(q) && dense_row_major(v) && dense_row_major(out) && kt_k_fastest && mrl::attn_applicable(at)) {
+      HIP_TRY(mrl::launch_attn(at, ws.stream));
+      return MRL_OK;
+    }
   }
   // Staged path, as the reference schedules it (examples/matmul_chain.rs:60-81): S and P
-  // live in device memory as f32 (verification.rs:239-285).
+  // live in device memory as f32 (verification.rs:239-285); each stage is the Spec it is.
   void *sbuf = nullptr;
   HIP_TRY(ws.alloc(&sbuf, size_t(b) * m * n2 * sizeof(float)));
-  mrl::Strided st;
-  st.ptr = sbuf, st.dtype = MRL_F32, st.rank = 3;
-  st.shape[0] = b, st.shape[1] = m, st.shape[2] = n2, st.shape[3] = st.shape[4] = 1;
-  st.stride[0] = int64_t(m) * n2, st.stride[1] = n2, st.stride[2] = 1, st.stride[3] = st.stride[4] = 0;
-  HIP_TRY(mrl::launch_matmul_generic(q.t, kt.t, st, 0, ws.stream));
-  if ((reinterpret_cast<uintptr_t>(sbuf) & 15) == 0)
+  mrl_spec st;
+  std::memset(&st, 0, sizeof st);
+  st.kind = MRL_SPEC_MATMUL, st.rank = 4, st.n_params = 3;
+  st.spec_shape[0] = b, st.spec_shape[1] = m, st.spec_shape[2] = k, st.spec_shape[3] = n2;
+  st.dtypes[0] = s.dtypes[1], st.dtypes[1] = s.dtypes[2], st.dtypes[2] = MRL_F32;
+  st.layouts[0] = s.layouts[1], st.layouts[1] = s.layouts[2];
+  const uint32_t s_shape[3] = {b, m, n2};
+  mrl_layout_row_major(s_shape, 3, &st.layouts[2]);
+  void *p1[3] = {params[1], params[2], sbuf};
+  int rc = run_matmul(st, p1, ws);
+  if (rc != MRL_OK) return rc;
+  if ((reinterpret_cast<uintptr_t>(sbuf) & 15) == 0) {
     HIP_TRY(mrl::launch_softmax_rows((const float *)sbuf, (float *)sbuf, uint64_t(b) * m, n2, ws.stream));
-  else
-    HIP_TRY(mrl::launch_softmax_generic(st, st, 2, ws.stream));
-  HIP_TRY(mrl::launch_matmul_generic(st, v.t, out.t, 0, ws.stream));
-  return finish_output(out, ws);
+  } else {
+    mrl::Strided sv;
+    sv.ptr = sbuf, sv.dtype = MRL_F32, sv.rank = 3;
+    sv.shape[0] = b, sv.shape[1] = m, sv.shape[2] = n2, sv.shape[3] = sv.shape[4] = 1;
+    sv.stride[0] = int64_t(m) * n2, sv.stride[1] = n2, sv.stride[2] = 1, sv.stride[3] = sv.stride[4] = 0;
+    HIP_TRY(mrl::launch_softmax_generic(sv, sv, 2, ws.stream));
+  }
+  st.spec_shape[2] = n2, st.spec_shape[3] = n;
+  st.dtypes[0] = MRL_F32, st.dtypes[1] = s.dtypes[0], st.dtypes[2] = s.dtypes[3];
+  st.layouts[0] = st.layouts[2];  // S: row-major [b, m, n2]
+  st.layouts[1] = s.layouts[0], st.layouts[2] = s.layouts[3];
+  void *p2[3] = {sbuf, params[0], params[3]};
+  return run_matmul(st, p2, ws);
 }
 
 int run_move(const mrl_spec &s, void *const *params, Workspace &ws) {
