@@ -121,7 +121,18 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
     // every wave is done reading the other stage, which the next block may now overwrite.
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
-    if (kb + 1 < nblocks) load_block(kb + 1, stage ^ 1);
+    // The next block's global->LDS loads are issued one K and one V instruction at a time
+    // between the MFMA batches below (such an instruction holds its wave for tens of cycles;
+    // in a burst behind the barrier all eight waves queue up on the one memory pipe while
+    // the matrix cores idle).  Past the last block the same block is fetched again into the
+    // stage nobody reads.
+    const int64_t next_base = int64_t(min(kb + 1, nblocks - 1)) * TILE;
+    uint8_t *next_lds = my_lds + (stage ^ 1) * STAGE;
+    auto load_pair = [&](int i) {
+      const int q = qg * 4 + i;
+      __builtin_amdgcn_global_load_lds((global_cvoid *)(K + next_base + k_src[i]), (lds_void *)(next_lds + q * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((global_cvoid *)(V + next_base + v_src[i]), (lds_void *)(next_lds + TILE + q * 1024), 16, 0, 0);
+    };
     const uint8_t *lk = my_lds + stage * STAGE, *lv = lk + TILE;
 
     // S^T tiles: s[kt][r] is key kt*32 + 8*(r/4) + 4*lg + r%4, query lq.
@@ -148,6 +159,7 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
 #pragma unroll
     for (int q = 0; q < D / 32; q++) {
       if (q + 2 < D / 32) read_k(q + 2, (q + 2) % 3);
+      load_pair(q);
 #pragma unroll
       for (int c = 0; c < 2; c++)
 #pragma unroll
@@ -159,7 +171,10 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
 #pragma unroll
     for (int q = 0; q < D / 32; q++) {
       if (q + 2 < D / 32) __builtin_amdgcn_sched_group_barrier(0x100, 2 * (BKV / 32), 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 2 * (BKV / 32), 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, BKV / 32, 0);
+      __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, BKV / 32, 0);
+      __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
     }
     // All V operands of the block are requested now: they land while the softmax runs.
     v4i vf[BKV / 16][D / 32];
