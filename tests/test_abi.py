@@ -138,3 +138,17 @@ def test_null_and_status_strings():
     assert lib.mrl_status_string(0) == b"ok"
     assert lib.mrl_status_string(2).startswith(b"layout")
     assert lib.mrl_version().count(b".") == 2
+
+
+@pytest.mark.gpu
+def test_sustained_matrix_core_rate_is_sane(gpu):
+    """All-zero operands run near the datasheet rate; benchmark-like operands lower, never
+    higher, and both within physical bounds."""
+    for kind, nominal in (("int8", 5033e12), ("bf16", 2516e12)):
+        zero = M.measure_mfma_rate(kind, False, 4000)
+        rand = M.measure_mfma_rate(kind, True, 4000)
+        assert 0.2 * nominal < rand <= zero * 1.02 < 1.1 * nominal, (kind, zero, rand)
+    lib = B.load()
+    out = C.c_double()
+    assert lib.mrl_measure_mfma_rate(2, 0, 10, C.byref(out)) == 3   # unknown kind
+    assert lib.mrl_measure_mfma_rate(0, 0, 10, None) == 6           # NULL result pointer

@@ -25,7 +25,7 @@ def nhwc_inputs(seed, b, f, c, oh, ow, fh, fw, dt_img=M.u8):
     ((2, 64, 64, 9, 11, 3, 3), True),
     ((1, 8, 8, 1, 1, 3, 3), False),      # examples/simple_conv_x86.rs shape
     ((2, 5, 7, 4, 3, 2, 3), True),       # ragged channels: generic kernel
-    ((3, 64, 64, 54, 54, 3, 3), False),  # BASELINE config 4 at batch 3
+    ((3, 64, 64, 54, 54, 3, 3), False),  # benchmark configuration 4 at batch 3
     ((1, 64, 64, 5, 5, 1, 1), False),    # 1x1 filter
 ])
 def test_conv_nhwc_bit_exact(gpu, dt_img, shape, accum):
@@ -50,7 +50,7 @@ def test_conv_nchw_layout_generic(gpu):
 
 
 def test_conv_full_size_properties(gpu):
-    """BASELINE config 4 (32x56x56x64 -> 64, 3x3): a few images against the oracle, every
+    """benchmark configuration 4 (32x56x56x64 -> 64, 3x3): a few images against the oracle, every
     image through a checksum (sum over filters and pixels, computed in int64 from box sums),
     and the extreme-value bound 576*255*128."""
     shape = (32, 64, 64, 54, 54, 3, 3)

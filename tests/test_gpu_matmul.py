@@ -74,7 +74,7 @@ def test_int8_matmul_reference_check_pattern(gpu):
 
 
 def test_int8_matmul_full_size_properties(gpu):
-    """BASELINE config 2 (4096^3) through size-independent checks: a band of rows against
+    """benchmark configuration 2 (4096^3) through size-independent checks: a band of rows against
     the oracle, every row/column against checksums computed in int64, and accumulation
     across two calls (the reference's bench loop accumulates the same way)."""
     m = k = n = 4096
@@ -114,7 +114,7 @@ def test_other_dtype_combinations_generic(gpu, da, db, dc):
 
 
 def test_f32_matmul_plumbing_config(gpu):
-    """BASELINE config 1: f32 64^3, uniform[-1,1), accumulate into a zeroed C."""
+    """benchmark configuration 1: f32 64^3, uniform[-1,1), accumulate into a zeroed C."""
     shape = [1, 64, 64, 64]
     A, Bm = synth.uniform_f32(41, 0, (1, 64, 64)), synth.uniform_f32(41, 1, (1, 64, 64))
     got = run_spec(M.MatmulAccum(shape, [M.f32] * 3), [A, Bm, np.zeros((1, 64, 64), np.float32)])
@@ -171,7 +171,7 @@ def test_bf16_matmul_pattern_exact(gpu):
 
 
 def test_bf16_matmul_full_size_sample(gpu):
-    """BASELINE config 3 (8192^3): sampled rows against the oracle, plus linearity."""
+    """benchmark configuration 3 (8192^3): sampled rows against the oracle, plus linearity."""
     m = k = n = 8192
     A, Bm = synth.normal_bf16(61, 0, (1, m, k)), synth.normal_bf16(61, 1, (1, k, n))
     dA, dB = M.DeviceBuffer.from_numpy(A), M.DeviceBuffer.from_numpy(Bm)

@@ -36,7 +36,7 @@ def test_softmax_edge_values(gpu):
 
 
 def test_softmax_full_size(gpu):
-    """The Softmax stage of BASELINE config 5 alone: 16x2048 rows of 2048."""
+    """The Softmax stage of benchmark configuration 5 alone: 16x2048 rows of 2048."""
     shape = (16, 2048, 2048)
     x = synth.normal_f32(203, 0, shape, std=2.0)
     got = run_spec(M.Softmax(list(shape), 2), [x, np.zeros((1,), np.float32).repeat(x.size).reshape(shape)])
@@ -82,7 +82,7 @@ def test_compose_msm_row_major_kt_and_f32_inputs(gpu):
 
 
 def test_compose_msm_full_size(gpu):
-    """BASELINE config 5: 16 heads of 2048x128; four heads against the oracle, all heads
+    """benchmark configuration 5: 16 heads of 2048x128; four heads against the oracle, all heads
     through the row-stochastic property: with V = ones, out must be all ones."""
     b, m, k, n2, n = 16, 2048, 128, 2048, 128
     q, kmat, v = msm_inputs(303, b, m, k, n2, n)
