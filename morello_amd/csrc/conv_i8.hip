@@ -43,6 +43,18 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(ConvArgs p, uint32_t pix
   const int sub = p.c / 64;  // 64-channel slabs per filter position
   const int krow = p.fh * p.fw * p.c;  // bytes per filter
 
+  // Filter bank: global -> LDS (coalesced, once per workgroup) -> registers (per wave).
+  // 64 filters x (SLABS * 64) bytes = SLABS * 256 chunks of 16 bytes.  These loads need
+  // nothing but the pointer and the thread index, so they go out first and are in flight
+  // during the address arithmetic of the first pixel tile.
+  constexpr int PER_THREAD = (SLABS * 256 + NT - 1) / NT;
+  v4i stage[PER_THREAD];
+#pragma unroll
+  for (int i = 0; i < PER_THREAD; i++) {
+    const int c = i * NT + threadIdx.x;
+    if (c < SLABS * 256) stage[i] = *(const v4i *)((const uint8_t *)p.filters + c * 16);
+  }
+
   // Byte offset of each slab's source relative to the pixel's own (y, x) position.
   int slab_off[SLABS];
 #pragma unroll
@@ -67,25 +79,11 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(ConvArgs p, uint32_t pix
   uint32_t t = wave;
   if (t < tiles) load_tile(t, img);
 
-  // Filter bank: global -> LDS (coalesced, once per workgroup) -> registers (per wave).
-  // Slab s covers filter position (s / sub) and channels 64*(s % sub) .. +63; lane (li, lg)
-  // holds filter row ft*16+li, bytes 16*lg .. +15 of the slab.
-  {
-    // 64 filters x (SLABS * 64) bytes = SLABS * 256 chunks of 16 bytes: all loads are
-    // issued before the first store so they share one round trip.
-    constexpr int PER_THREAD = (SLABS * 256 + NT - 1) / NT;
-    const uint8_t *fbase = (const uint8_t *)p.filters;
-    v4i stage[PER_THREAD];
+  // Filter bank, second half of its staging: registers -> LDS.
 #pragma unroll
-    for (int i = 0; i < PER_THREAD; i++) {
-      const int c = i * NT + threadIdx.x;
-      if (c < SLABS * 256) stage[i] = *(const v4i *)(fbase + c * 16);
-    }
-#pragma unroll
-    for (int i = 0; i < PER_THREAD; i++) {
-      const int c = i * NT + threadIdx.x;
-      if (c < SLABS * 256) *(v4i *)(filt_lds + c * 16) = stage[i];
-    }
+  for (int i = 0; i < PER_THREAD; i++) {
+    const int c = i * NT + threadIdx.x;
+    if (c < SLABS * 256) *(v4i *)(filt_lds + c * 16) = stage[i];
   }
   __syncthreads();
   v4i filt[FT][SLABS];
@@ -95,26 +93,20 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(ConvArgs p, uint32_t pix
     for (int s = 0; s < SLABS; s++)
       filt[ft][s] = *(const v4i *)(filt_lds + (ft * 16 + li) * krow + s * 64 + lg * 16);
 
-  // u8 correction 128 * sum_k filt[f][k], one value per filter, parked in LDS behind a
-  // barrier (every wave computes the same 64 numbers; wave 0 publishes them).
-  int *corr_lds = (int *)filt_lds;
+  // u8 correction 128 * sum_k filt[f][k]: the same MFMAs against an all-ones pixel leave, in
+  // every column, the filter sums in exactly the accumulator layout the stores use.  They are
+  // parked in LDS past the filter bank (every wave writes the same 64 numbers and reads back
+  // its own writes, so no barrier is needed).
+  int *corr_lds = (int *)(filt_lds + FT * 16 * krow);
   if (IMG_UNSIGNED) {
-    int sums[FT];
+    const v4i ones = v4i{0x01010101, 0x01010101, 0x01010101, 0x01010101};
 #pragma unroll
     for (int ft = 0; ft < FT; ft++) {
-      int sum = 0;
+      v4i sum = v4i{0, 0, 0, 0};
 #pragma unroll
-      for (int s = 0; s < SLABS; s++)
-#pragma unroll
-        for (int w = 0; w < 4; w++) sum = __builtin_amdgcn_sdot4(filt[ft][s][w], 0x01010101, sum, false);
-      sum += __shfl_xor(sum, 16);
-      sums[ft] = sum + __shfl_xor(sum, 32);  // every lane with the same li has filter ft*16+li
+      for (int s = 0; s < SLABS; s++) sum = __builtin_amdgcn_mfma_i32_16x16x64_i8(filt[ft][s], ones, sum, 0, 0, 0);
+      if (li == 0) *(v4i *)(corr_lds + ft * 16 + lg * 4) = sum * 128;
     }
-    __syncthreads();  // all waves hold their filters in registers: the staging area is free
-    if (threadIdx.x < 16)
-#pragma unroll
-      for (int ft = 0; ft < FT; ft++) corr_lds[ft * 16 + li] = 128 * sums[ft];
-    __syncthreads();
   }
 
   // The pixel registers are refilled slab by slab with the next tile as soon as the MFMAs
@@ -163,7 +155,7 @@ hipError_t launch_slabs(const ConvArgs &c, bool img_unsigned, hipStream_t stream
   constexpr int WAVES = CONV_WAVES;
   uint32_t blocks = 2048 / WAVES;
   if (blocks * WAVES > tiles) blocks = (tiles + WAVES - 1) / WAVES;
-  const size_t lds = size_t(FT) * 16 * c.fh * c.fw * c.c;  // the whole filter bank
+  const size_t lds = size_t(FT) * 16 * c.fh * c.fw * c.c + FT * 16 * sizeof(int);  // the filter bank + corrections
   if (img_unsigned)
     hipLaunchKernelGGL((k_conv_i8<SLABS, true, WAVES>), dim3(blocks), dim3(64 * WAVES), lds, stream, c, uint32_t(pixels), tiles);
   else
