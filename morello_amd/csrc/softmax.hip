@@ -24,6 +24,7 @@ __device__ inline float wave_sum(float v) {
   return v;
 }
 
+typedef float f4 __attribute__((ext_vector_type(4)));
 constexpr float F32_MIN = -3.40282347e+38f;  // f32::MIN, the oracle's max identity
 
 // NV float4 vectors per lane; cols is a multiple of 4 and <= NV * 256.
@@ -44,7 +45,9 @@ __global__ __launch_bounds__(256) void k_softmax_regs(const float *__restrict__ 
   for (int i = 0; i < NV; i++) {
     const uint32_t idx = i * 64 + lane;
     if (idx < nvec) {
-      v[i] = src[idx];
+      // Streamed once: keep it out of the caches' way.
+      const f4 t = __builtin_nontemporal_load((const f4 *)src + idx);
+      v[i] = float4{t[0], t[1], t[2], t[3]};
       nan |= (v[i].x != v[i].x) | (v[i].y != v[i].y) | (v[i].z != v[i].z) | (v[i].w != v[i].w);
       mx = fmaxf(fmaxf(mx, fmaxf(v[i].x, v[i].y)), fmaxf(v[i].z, v[i].w));
     }
@@ -69,7 +72,7 @@ __global__ __launch_bounds__(256) void k_softmax_regs(const float *__restrict__ 
     const uint32_t idx = i * 64 + lane;
     if (idx < nvec) {
       v[i].x /= sum, v[i].y /= sum, v[i].z /= sum, v[i].w /= sum;
-      dst[idx] = v[i];
+      __builtin_nontemporal_store(f4{v[i].x, v[i].y, v[i].z, v[i].w}, (f4 *)dst + idx);
     }
   }
 }
