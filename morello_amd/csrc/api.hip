@@ -293,13 +293,32 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
   if ((rc = prepare(s, 0, params[0], true, ws, &a)) != MRL_OK) return rc;
   if ((rc = prepare(s, 1, params[1], true, ws, &b)) != MRL_OK) return rc;
   if ((rc = prepare(s, 2, params[2], s.accum != 0, ws, &c)) != MRL_OK) return rc;
+  int da = s.dtypes[0], db = s.dtypes[1];
+  const int dc = s.dtypes[2];
+  // f32 output with one bf16 and one f32 input: the reference converts both inputs to the
+  // output dtype before multiplying (verification.rs:115-134); widening the bf16 operand
+  // (exact) makes it an f32 Matmul, which the matrix cores take.
+  if (dc == MRL_F32 && ((da == MRL_BF16 && db == MRL_F32) || (da == MRL_F32 && db == MRL_BF16))) {
+    Prepared &narrow = da == MRL_BF16 ? a : b;
+    void *wide = nullptr;
+    HIP_TRY(ws.alloc(&wide, narrow.count * sizeof(float)));
+    HIP_TRY(mrl::launch_widen_bf16(narrow.t.ptr, wide, narrow.count, ws.stream));
+    narrow.t.ptr = wide, narrow.t.dtype = MRL_F32;
+    da = db = MRL_F32;
+  }
   mrl::GemmArgs g;
   g.a = a.t.ptr, g.b = b.t.ptr, g.c = c.t.ptr;
   g.batch = s.spec_shape[0], g.m = s.spec_shape[1], g.k = s.spec_shape[2], g.n = s.spec_shape[3];
   g.accum = s.accum;
-  const bool rows = as_rows(a.t, &g.lda, &g.sa) && as_rows(b.t, &g.ldb, &g.sb) &&
-                    as_rows(c.t, &g.ldc, &g.sc);
-  const int da = s.dtypes[0], db = s.dtypes[1], dc = s.dtypes[2];
+  // B either with n fastest (row-major) or with k fastest (col-major, layout![0,2,1]).
+  bool b_ok = as_rows(b.t, &g.ldb, &g.sb);
+  if (!b_ok) {
+    mrl::Strided bt = b.t;  // view [b, k, n] as [b, n, k]
+    std::swap(bt.shape[1], bt.shape[2]);
+    std::swap(bt.stride[1], bt.stride[2]);
+    b_ok = g.b_kmajor = as_rows(bt, &g.ldb, &g.sb);
+  }
+  const bool rows = as_rows(a.t, &g.lda, &g.sa) && b_ok && as_rows(c.t, &g.ldc, &g.sc);
   bool done = false;
   if (sched) {
     const int kind = (da == MRL_I8 && db == MRL_I8 && dc == MRL_I32)     ? 0
@@ -307,7 +326,7 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
                      : (da == MRL_BF16 && db == MRL_BF16 && dc == MRL_F32) ? 2
                      : (da == MRL_F32 && db == MRL_F32 && dc == MRL_F32)   ? 3
                                                                            : -1;
-    const bool ok = kind >= 0 && rows &&
+    const bool ok = kind >= 0 && rows && !g.b_kmajor &&
                     (kind == 3   ? mrl::gemm_f32_applicable(g)
                      : kind == 2 ? mrl::gemm_bf16_applicable(g)
                                  : mrl::gemm_i8_applicable(g, false));

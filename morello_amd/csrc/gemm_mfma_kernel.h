@@ -196,7 +196,10 @@ __device__ inline void sched_slots(bool staging) {
 // M, any N and K whose rows are whole 16-byte chunks; chunks outside the matrices are fed as
 // zeros (a zero row of B makes the product and the column-sum correction vanish whatever A
 // holds there) and stores outside C are masked.
-template <class T, bool A_UNSIGNED, class TL, bool EDGE>
+// B_KMAJOR: B is stored with k fastest (each of its n rows runs along K, `ldb` elements apart:
+// Morello's col_major / batched_col_major layouts, or layout![0,2,1]).  Its tile is then staged
+// and read exactly like A's, and no transposing read is involved.
+template <class T, bool A_UNSIGNED, class TL, bool EDGE, bool B_KMAJOR = false>
 __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int tiles_n) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   constexpr int BM = TL::BM, BN = TL::BN, BKB = TL::BKB, WAVES_M = TL::WAVES_M, WAVES_N = TL::WAVES_N;
@@ -207,8 +210,9 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
   constexpr int A_ROW_CH = BKB / 16;              // 16-byte chunks per A tile row
   constexpr int A_ROWS_PER_LINE = 256 / BKB;      // A tile rows per 256-byte bank line
   constexpr int A_CH = BM * BKB / 16 / NT;       // 16-byte chunks per thread, A tile
-  constexpr int B_ROW_CH = BN * ES / 16;          // chunks per B row
-  constexpr int B_CH = BK * B_ROW_CH / NT;        // chunks per thread, B tile
+  constexpr int B_ROW_CH = B_KMAJOR ? BKB / 16 : BN * ES / 16;               // chunks per B tile row
+  constexpr int B_CH = (B_KMAJOR ? BN : BK) * B_ROW_CH / NT;                  // chunks per thread, B tile
+  constexpr int B_LDS_ROW = B_KMAJOR ? BKB : B_ROW;                          // bytes per B tile row in LDS
   constexpr int SLABS = BKB / 32;                 // MFMA k steps per tile (32 bytes each)
   constexpr int K_SLAB = 32 / ES;                 // elements of K per MFMA
   typedef typename T::Acc Acc;
@@ -232,7 +236,7 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
   const int64_t m0 = int64_t(tile_m) * BM, n0 = int64_t(tile_n) * BN;
 
   const uint8_t *A = (const uint8_t *)g.a + (int64_t(blockIdx.y) * g.sa + m0 * g.lda) * ES;
-  const uint8_t *B = (const uint8_t *)g.b + (int64_t(blockIdx.y) * g.sb + n0) * ES;
+  const uint8_t *B = (const uint8_t *)g.b + (int64_t(blockIdx.y) * g.sb + (B_KMAJOR ? n0 * g.ldb : n0)) * ES;
   Out *C = (Out *)g.c + int64_t(blockIdx.y) * g.sc + m0 * g.ldc + n0;
   const int64_t lda_b = g.lda * ES, ldb_b = g.ldb * ES;
 
@@ -255,10 +259,11 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
   {
     const int row = tid / B_ROW_CH, ch = tid % B_ROW_CH;
     b_src = B + int64_t(row) * ldb_b + ch * 16;
-    b_dst = A_STAGE + row * B_ROW + ch * 16;
+    if constexpr (B_KMAJOR) b_dst = A_STAGE + row * BKB + ((ch ^ ((row / A_ROWS_PER_LINE) & (A_ROW_CH - 1))) << 4);
+    else b_dst = A_STAGE + row * B_ROW + ch * 16;
   }
   const int64_t a_step_i = int64_t(A_ROWS_PER_I) * lda_b, b_step_i = int64_t(B_ROWS_PER_I) * ldb_b;
-  const int64_t b_step_kt = int64_t(BK) * ldb_b;
+  const int64_t b_step_kt = B_KMAJOR ? int64_t(BKB) : int64_t(BK) * ldb_b;
   // Operand fragment offsets within a stage for MFMA k step 0.
   int a_frag[TM];
 #pragma unroll
@@ -270,7 +275,9 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
   int b_frag[TN];
 #pragma unroll
   for (int tn = 0; tn < TN; tn++) {
-    if constexpr (T::TRANSPOSED_READ) {
+    if constexpr (B_KMAJOR) {
+      b_frag[tn] = A_STAGE + (wn * WN + tn * 32 + (lane & 31)) * BKB;
+    } else if constexpr (T::TRANSPOSED_READ) {
       constexpr int LANES_PER_ROW = 16 / (8 / ES);  // lanes that share one k row: 2 (i8), 4 (bf16)
       const int p = lane & 15;
       const int k = (K_SLAB / 2) * (lane >> 5) + p / LANES_PER_ROW;
@@ -300,6 +307,8 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
   const int a_kb0 = (tid % A_ROW_CH) * 16;                            // its k byte within a tile
   const int b_cols_left = int(g.n - n0) * ES - (tid % B_ROW_CH) * 16; // bytes of the B row right of it
   const int b_k0 = tid / B_ROW_CH;                                    // its k row within a tile
+  const int b_rows_left = int(g.n - n0) - tid / B_ROW_CH;             // B_KMAJOR: n rows below the thread's
+  const int b_kb0 = (tid % B_ROW_CH) * 16;                            // B_KMAJOR: its k byte within a tile
   int ld_kb = 0;  // k byte offset of the tile the next load_global() fetches
 
   // Loads the next tile in sequence and advances the source pointers.
@@ -317,7 +326,9 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
     for (int i = 0; i < B_CH; i++) {
       if (EDGE) {
         b_reg[i] = v4i{0, 0, 0, 0};
-        if (b_cols_left > 0 && ld_kb / ES + b_k0 + i * B_ROWS_PER_I < int(g.k)) b_reg[i] = *(const v4i *)(b_src + i * b_step_i);
+        const bool in_b = B_KMAJOR ? (i * B_ROWS_PER_I < b_rows_left && ld_kb + b_kb0 < k_bytes)
+                                   : (b_cols_left > 0 && ld_kb / ES + b_k0 + i * B_ROWS_PER_I < int(g.k));
+        if (in_b) b_reg[i] = *(const v4i *)(b_src + i * b_step_i);
       } else {
         b_reg[i] = *(const v4i *)(b_src + i * b_step_i);
       }
@@ -335,7 +346,7 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
       *(v4i *)(base + a_dst + i * A_ROWS_PER_I * BKB) = v;
     }
 #pragma unroll
-    for (int i = 0; i < B_CH; i++) *(v4i *)(base + b_dst + i * B_ROWS_PER_I * B_ROW) = b_reg[i];
+    for (int i = 0; i < B_CH; i++) *(v4i *)(base + b_dst + i * B_ROWS_PER_I * B_LDS_ROW) = b_reg[i];
   };
   // MFMA operands for one 32-byte k step, double buffered in registers.
   v4i af[2][TM], bf[2][TN];
@@ -346,7 +357,9 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
       af[buf][tm] = *(const v4i *)(base + a_frag[tm] + (((2 * s + a_half) ^ a_swz) << 4));
 #pragma unroll
     for (int tn = 0; tn < TN; tn++) {
-      if constexpr (T::TRANSPOSED_READ) {
+      if constexpr (B_KMAJOR) {
+        bf[buf][tn] = *(const v4i *)(base + b_frag[tn] + (((2 * s + a_half) ^ a_swz) << 4));
+      } else if constexpr (T::TRANSPOSED_READ) {
         const v2i lo = T::read_tr(base + b_frag[tn] + (s * K_SLAB) * B_ROW);
         const v2i hi = T::read_tr(base + b_frag[tn] + (s * K_SLAB + T::K_PER_READ) * B_ROW);
         bf[buf][tn] = v4i{lo[0], lo[1], hi[0], hi[1]};
@@ -405,7 +418,8 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
       }
       mfma_slab(s, s & 1);
       // One output block's MFMAs, then a share of this step's memory instructions, TM*TN times.
-      sched_slots<0, TM * TN, T::TRANSPOSED_READ ? 1 : 4, TM + (T::TRANSPOSED_READ ? 2 : 4) * TN, A_CH + B_CH>(
+      sched_slots<0, TM * TN, T::TRANSPOSED_READ ? 1 : 4,
+                  TM + (B_KMAJOR ? 1 : T::TRANSPOSED_READ ? 2 : 4) * TN, A_CH + B_CH>(
           s == SLABS - 2);
     }
   }
@@ -414,9 +428,9 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
                                                      int(g.m - m0), int(g.n - n0));
 }
 
-template <class T, bool A_UNSIGNED, class TL, bool EDGE>
+template <class T, bool A_UNSIGNED, class TL, bool EDGE, bool B_KMAJOR = false>
 hipError_t launch(const GemmArgs &g, hipStream_t stream) {
-  auto kern = k_gemm<T, A_UNSIGNED, TL, EDGE>;
+  auto kern = k_gemm<T, A_UNSIGNED, TL, EDGE, B_KMAJOR>;
   constexpr int BM = TL::BM, BN = TL::BN;
   constexpr int STAGE = TL::template stage<T>();
   static bool attr_set = false;

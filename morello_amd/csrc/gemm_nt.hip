@@ -1,0 +1,29 @@
+// Matmul whose B operand is stored with k fastest (Morello's col_major / batched_col_major
+// layouts, layout![0,2,1]): the matrix-core kernel of gemm_mfma_kernel.h with B staged and read
+// like A.  Kept in its own translation unit so the instantiations compile in parallel.
+#include "gemm_mfma_kernel.h"
+
+namespace mrl {
+namespace {
+using namespace gemm;
+
+template <class T, bool A_UNSIGNED>
+hipError_t launch_for(const GemmArgs &g, hipStream_t stream) {
+  const bool whole = g.m % TileBig::BM == 0 && g.n % TileBig::BN == 0 && g.k % (TileBig::BKB / T::ES) == 0;
+  return whole ? launch<T, A_UNSIGNED, TileBig, false, true>(g, stream)
+               : launch<T, A_UNSIGNED, TileBig, true, true>(g, stream);
+}
+
+}  // namespace
+
+hipError_t launch_gemm_nt(const GemmArgs &g, int kind, hipStream_t stream) {
+  switch (kind) {
+    case 0: return launch_for<I8, false>(g, stream);
+    case 1: return launch_for<I8, true>(g, stream);
+    case 2: return launch_for<BF16, false>(g, stream);
+    case 3: return launch_for<F32, false>(g, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace mrl

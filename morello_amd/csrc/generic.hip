@@ -142,6 +142,14 @@ __global__ __launch_bounds__(256) void k_copy16(const v4u *__restrict__ src, v4u
   }
 }
 
+// bf16 -> f32 of a whole buffer, position by position (exact: a 16-bit shift).
+__global__ __launch_bounds__(256) void k_widen_bf16(const uint16_t *__restrict__ src, uint32_t *__restrict__ dst,
+                                                    uint64_t count) {
+  const uint64_t step = uint64_t(gridDim.x) * blockDim.x;
+  for (uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += step)
+    dst[i] = uint32_t(src[i]) << 16;
+}
+
 __global__ void k_copy1(const uint8_t *src, uint8_t *dst, uint64_t bytes) {
   const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i < bytes) dst[i] = src[i];
@@ -333,6 +341,15 @@ hipError_t launch_copy(const void *src, void *dst, uint64_t bytes, hipStream_t s
   if (tail)
     hipLaunchKernelGGL(k_copy1, dim3(1), dim3(16), 0, stream, (const uint8_t *)src + vecs * 16,
                        (uint8_t *)dst + vecs * 16, tail);
+  return hipGetLastError();
+}
+
+hipError_t launch_widen_bf16(const void *src, void *dst, uint64_t count, hipStream_t stream) {
+  if (count == 0) return hipSuccess;
+  uint64_t blocks = (count + 255) / 256;
+  if (blocks > 16384) blocks = 16384;
+  hipLaunchKernelGGL(k_widen_bf16, dim3(uint32_t(blocks)), dim3(256), 0, stream, (const uint16_t *)src,
+                     (uint32_t *)dst, count);
   return hipGetLastError();
 }
 

@@ -32,6 +32,7 @@ hipError_t launch_move_generic(const void *src, void *dst, const LayoutEval &src
                                const LayoutEval &dst_l, int src_dtype, int dst_dtype,
                                uint64_t count, hipStream_t stream);
 // Move Spec fast path: same bytes on both sides (16-byte aligned buffers).
+hipError_t launch_widen_bf16(const void *src, void *dst, uint64_t count, hipStream_t stream);
 hipError_t launch_copy(const void *src, void *dst, uint64_t bytes, hipStream_t stream);
 
 // ---- gemm_i8.hip: u8|i8 x i8 -> i32 on the int8 MFMA -----------------------------------
@@ -44,7 +45,12 @@ struct GemmArgs {
   int64_t lda, ldb, ldc;
   int64_t sa, sb, sc;  // batch strides
   int accum;
+  // false: B rows run along N (`ldb` = elements between k rows); true: B rows run along K
+  // (`ldb` = elements between n rows), as col_major / layout![0,2,1] store it.
+  bool b_kmajor = false;
 };
+// kind: 0 = i8 x i8, 1 = u8 x i8, 2 = bf16 x bf16, 3 = f32 x f32; B stored k-fastest (gemm_nt.hip).
+hipError_t launch_gemm_nt(const GemmArgs &g, int kind, hipStream_t stream);
 bool gemm_i8_applicable(const GemmArgs &g, bool b_k_contiguous);
 hipError_t launch_gemm_i8(const GemmArgs &g, bool a_unsigned, hipStream_t stream);
 

@@ -160,6 +160,40 @@ def test_f32_matmul_on_the_matrix_cores(gpu, shape, accum):
     assert np.array_equal(got, np.matmul(A.astype(np.int64), Bm.astype(np.int64)).astype(np.float32))
 
 
+@pytest.mark.parametrize("dts,codes", [((M.u8, M.i8, M.i32), [0, 1, 5]), ((M.i8, M.i8, M.i32), [1, 1, 5]),
+                                        ((M.bf16, M.bf16, M.f32), [7, 7, 6]), ((M.f32, M.f32, M.f32), [6, 6, 6])])
+@pytest.mark.parametrize("shape,accum", [((1, 256, 256, 256), False), ((2, 300, 136, 200), True),
+                                         ((1, 64, 64, 70), False), ((3, 512, 128, 256), True)])
+def test_matmul_with_k_fastest_b(gpu, dts, codes, shape, accum):
+    """B stored with k fastest (batched_col_major, layout.rs:1255-1271) runs on the matrix cores
+    with its tile staged like A's: whole tiles, ragged borders (any N), batches, accumulation."""
+    b, m, k, n = shape
+    gen = {M.u8: synth.uniform_u8, M.i8: synth.uniform_i8, M.bf16: synth.normal_bf16, M.f32: synth.uniform_f32}
+    A, Bm = gen[dts[0]](71, 0, (b, m, k)), gen[dts[1]](71, 1, (b, k, n))
+    out_np = np.int32 if dts[2] == M.i32 else np.float32
+    C0 = (synth.uniform_u8(71, 2, (b, m, n)).astype(out_np) if accum else np.zeros((b, m, n), out_np))
+    layouts = [None, M.batched_col_major([b, k, n]), None]
+    Bt = np.ascontiguousarray(Bm.transpose(0, 2, 1))  # the buffer a k-fastest layout describes
+    got = run_spec(M.Matmul(shape, dts, layouts=layouts, accum=accum), [A, Bt, C0])
+    want = orc.matmul(list(shape), codes, A, Bm, C0.copy(), accum)
+    if dts[2] == M.i32:
+        assert np.array_equal(got, want)
+    else:
+        assert rel_err(got, want) < 1e-5
+
+
+@pytest.mark.parametrize("dts,codes", [((M.f32, M.bf16, M.f32), [6, 7, 6]), ((M.bf16, M.f32, M.f32), [7, 6, 6])])
+def test_mixed_bf16_f32_matmul(gpu, dts, codes):
+    """One bf16 and one f32 input with an f32 output: both are taken to f32 before the product,
+    as the reference's interpreter does (verification.rs:115-134)."""
+    b, m, k, n = 2, 192, 136, 264
+    gen = {M.bf16: synth.normal_bf16, M.f32: synth.uniform_f32}
+    A, Bm = gen[dts[0]](81, 0, (b, m, k)), gen[dts[1]](81, 1, (b, k, n))
+    C0 = synth.normal_f32(81, 2, (b, m, n))
+    got = run_spec(M.MatmulAccum([b, m, k, n], dts), [A, Bm, C0])
+    assert rel_err(got, orc.matmul([b, m, k, n], codes, A, Bm, C0.copy(), True)) < 1e-5
+
+
 def test_bf16_matmul_pattern_exact(gpu):
     """0..3 inputs (verification.rs:933-935): every partial sum is an exact integer."""
     b, m, k, n = 1, 256, 256, 256

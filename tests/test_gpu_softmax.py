@@ -67,6 +67,20 @@ def test_compose_msm(gpu, dims):
     assert rel_err(got, want) < 1e-2  # stated tolerance for the composed pipeline
 
 
+@pytest.mark.parametrize("dims", [(2, 200, 64, 328, 64), (1, 136, 128, 1000, 128), (2, 256, 96, 192, 72)])
+def test_compose_msm_staged_on_the_matrix_cores(gpu, dims):
+    """Shapes the fused kernel does not take (ragged sequence lengths, head dims other than
+    128): Q.KT runs as a bf16 Matmul with a k-fastest B, softmax over f32 rows, and P.V as an
+    f32 Matmul after widening V.  f32 intermediates: within 1e-5 of the oracle."""
+    b, m, k, n2, n = dims
+    q, kmat, v = msm_inputs(303, *dims)
+    spec = M.ComposeMSM(b, m, k, n2, n, layouts=[None, None, KT_LAYOUT, None])
+    got = run_spec(spec, [v, q, kmat, np.zeros((b, m, n), np.float32)])
+    want = orc.compose_msm(b, m, k, n2, n, [7, 7, 7, 6], v, q, kmat, np.zeros((b, m, n), np.float32),
+                           layouts=[None, None, KT_ORC, None])
+    assert rel_err(got, want) < 1e-5
+
+
 def test_compose_msm_row_major_kt_and_f32_inputs(gpu):
     """KT materialised row-major and f32 inputs run on the staged (unfused) path."""
     b, m, k, n2, n = 2, 40, 32, 48, 24
