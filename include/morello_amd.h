@@ -329,6 +329,11 @@ int mrl_memcpy_h2d(void *dst, const void *src, size_t bytes);
 int mrl_memcpy_d2h(void *dst, const void *src, size_t bytes);
 int mrl_memset(void *dst, int value, size_t bytes);
 int mrl_device_synchronize(void);
+/* HIP streams (default priority) for callers that have no HIP binding of their own: the
+ * handle is what mrl_run_async, mrl_run_compose and the per-kind conveniences take. */
+int mrl_stream_create(void **stream);
+int mrl_stream_synchronize(void *stream);
+int mrl_stream_destroy(void *stream);
 /* Name, CU count, clock (kHz) and memory size of the selected device. */
 int mrl_device_info(char *name, size_t name_len, int *compute_units, int *clock_khz,
                     size_t *total_mem_bytes);

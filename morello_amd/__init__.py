@@ -270,6 +270,11 @@ class Spec:
         arr = (C.c_void_p * len(ptrs))(*ptrs)
         _check(B.load().mrl_run(C.byref(self._c), arr), "mrl_run")
 
+    def run_async(self, ptrs: Sequence[int], stream: "Stream"):
+        """Enqueues the Spec on `stream` and returns; `stream.synchronize()` waits for it."""
+        arr = (C.c_void_p * len(ptrs))(*ptrs)
+        _check(B.load().mrl_run_async(C.byref(self._c), arr, stream.handle), "mrl_run_async")
+
     def run_host(self, *arrays: np.ndarray):
         """`arrays`: numpy buffers in Spec parameter order, each already laid out by its
         parameter's layout; the output array is written in place."""
@@ -487,6 +492,23 @@ class Compose:
         arr = (C.c_void_p * len(ptrs))(*ptrs)
         _check(B.load().mrl_run_compose(C.byref(self._c), arr, None), "mrl_run_compose")
         synchronize()
+
+
+class Stream:
+    """A HIP stream owned by Python; plumbing for asynchronous launches."""
+
+    def __init__(self):
+        h = C.c_void_p()
+        _check(B.load().mrl_stream_create(C.byref(h)), "mrl_stream_create")
+        self.handle = h
+
+    def synchronize(self):
+        _check(B.load().mrl_stream_synchronize(self.handle), "mrl_stream_synchronize")
+
+    def destroy(self):
+        if self.handle:
+            B.load().mrl_stream_destroy(self.handle)
+            self.handle = None
 
 
 class DeviceBuffer:

@@ -113,6 +113,9 @@ SIGNATURES = {
     "mrl_memcpy_d2h": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "mrl_memset": (C.c_int, [C.c_void_p, C.c_int, C.c_size_t]),
     "mrl_device_synchronize": (C.c_int, []),
+    "mrl_stream_create": (C.c_int, [_VPP]),
+    "mrl_stream_synchronize": (C.c_int, [C.c_void_p]),
+    "mrl_stream_destroy": (C.c_int, [C.c_void_p]),
     "mrl_device_info": (C.c_int, [C.c_char_p, C.c_size_t, C.POINTER(C.c_int), C.POINTER(C.c_int),
                                   C.POINTER(C.c_size_t)]),
 }

@@ -1168,6 +1168,27 @@ int mrl_memset(void *dst, int value, size_t bytes) {
   HIP_TRY(hipMemset(dst, value, bytes));
   return MRL_OK;
 }
+int mrl_stream_create(void **stream) {
+  if (!stream) return MRL_ERR_NULL;
+  int rc;
+  if (g_device < 0 && (rc = mrl_init(0)) != MRL_OK) return rc;
+  hipStream_t st = nullptr;
+  HIP_TRY(hipStreamCreate(&st));
+  *stream = st;
+  return MRL_OK;
+}
+
+int mrl_stream_synchronize(void *stream) {
+  HIP_TRY(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  return MRL_OK;
+}
+
+int mrl_stream_destroy(void *stream) {
+  if (!stream) return MRL_ERR_NULL;
+  HIP_TRY(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+  return MRL_OK;
+}
+
 int mrl_device_synchronize(void) {
   HIP_TRY(hipDeviceSynchronize());
   return MRL_OK;

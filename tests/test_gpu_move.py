@@ -53,3 +53,29 @@ def test_move_relayout(gpu):
     got = run_spec(M.Move([3, 16], (M.u8, M.u8), layouts=[None, oe]), [y, np.zeros(48, np.uint8)])
     want = orc.move([3, 16], [0, 0], y, np.zeros(48, np.uint8), layouts=[None, orc.make_layout([0, 1, (1, 2, 8)])])
     assert np.array_equal(got, want)
+
+
+def test_async_launches_on_two_streams(gpu):
+    """Independent Specs enqueued on two streams (mrl_run_async), including one that stages a
+    packed layout through the stream-ordered scratch allocation, then a dependent Spec on the
+    first stream: results equal the synchronous ones."""
+    s1, s2 = M.Stream(), M.Stream()
+    b, m, k, n = 1, 256, 128, 256
+    A, Bm = synth.uniform_u8(801, 0, (b, m, k)), synth.uniform_i8(801, 1, (b, k, n))
+    x = synth.normal_f32(801, 2, (64, 96))
+    da, db, dc = (M.DeviceBuffer.from_numpy(t) for t in (A, Bm, np.zeros((b, m, n), np.int32)))
+    dx, dy = M.DeviceBuffer.from_numpy(x), M.DeviceBuffer.from_numpy(np.zeros((64, 96), np.float32))
+    mm = M.MatmulAccum([b, m, k, n], (M.u8, M.i8, M.i32))
+    sm = M.Softmax([64, 96], 1, layouts=[None, M.layout(0, 1, (1, M.Packed(8)))])
+    for _ in range(3):
+        mm.run_async([da.ptr, db.ptr, dc.ptr], s1)   # accumulates three times, in stream order
+        sm.run_async([dx.ptr, dy.ptr], s2)
+    s1.synchronize()
+    s2.synchronize()
+    want = orc.matmul([b, m, k, n], [0, 1, 5], A, Bm, np.zeros((b, m, n), np.int32))
+    assert np.array_equal(dc.to_numpy(np.int32, (b, m, n)), 3 * want)
+    # [0, 1, (1, Packed 8)] over [64, 96] keeps the row-major element order.
+    got = dy.to_numpy(np.float32, (64, 96))
+    assert np.abs(got - orc.softmax([64, 96], 1, x)).max() < 1e-6
+    s1.destroy()
+    s2.destroy()
