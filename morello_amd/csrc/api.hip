@@ -329,7 +329,7 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
     const bool ok = kind >= 0 && rows && !g.b_kmajor &&
                     (kind == 3   ? mrl::gemm_f32_applicable(g)
                      : kind == 2 ? mrl::gemm_bf16_applicable(g)
-                                 : mrl::gemm_i8_applicable(g, false));
+                                 : mrl::gemm_i8_applicable(g));
     if (!ok) return MRL_ERR_UNSUPPORTED;
     hipError_t e = mrl::launch_gemm_scheduled(g, kind, sched->tile_m, sched->tile_n, sched->split_k, ws.stream);
     if (e == hipErrorInvalidValue) return MRL_ERR_UNSUPPORTED;
@@ -337,7 +337,7 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
     return finish_output(c, ws);
   }
   if (rows && (da == MRL_U8 || da == MRL_I8) && db == MRL_I8 && dc == MRL_I32 &&
-      mrl::gemm_i8_applicable(g, false)) {
+      mrl::gemm_i8_applicable(g)) {
     HIP_TRY(mrl::launch_gemm_i8(g, da == MRL_U8, ws.stream));
     done = true;
   } else if (rows && da == MRL_BF16 && db == MRL_BF16 && dc == MRL_F32 &&

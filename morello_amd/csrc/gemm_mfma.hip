@@ -24,7 +24,7 @@ bool applicable(const GemmArgs &g, int es) {
 
 }  // namespace
 
-bool gemm_i8_applicable(const GemmArgs &g, bool) { return applicable(g, 1); }
+bool gemm_i8_applicable(const GemmArgs &g) { return applicable(g, 1); }
 hipError_t launch_gemm_i8(const GemmArgs &g, bool a_unsigned, hipStream_t stream) {
   if (g.b_kmajor) return launch_gemm_nt(g, a_unsigned ? 1 : 0, stream);
   if (whole_tiles(g, 1))

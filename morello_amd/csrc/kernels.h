@@ -31,12 +31,13 @@ hipError_t launch_fill_zero(void *ptr, uint64_t bytes, hipStream_t stream);
 hipError_t launch_move_generic(const void *src, void *dst, const LayoutEval &src_l,
                                const LayoutEval &dst_l, int src_dtype, int dst_dtype,
                                uint64_t count, hipStream_t stream);
-// Move Spec fast path: same bytes on both sides (16-byte aligned buffers).
+// bf16 -> f32 of a whole buffer, position by position.
 hipError_t launch_widen_bf16(const void *src, void *dst, uint64_t count, hipStream_t stream);
+// Move Spec fast path: same bytes on both sides (16-byte aligned buffers).
 hipError_t launch_copy(const void *src, void *dst, uint64_t bytes, hipStream_t stream);
 
-// ---- gemm_i8.hip: u8|i8 x i8 -> i32 on the int8 MFMA -----------------------------------
-// Row-major operands with leading dimensions in elements; batch strides in elements.
+// ---- gemm_mfma.hip / gemm_nt.hip: Matmul on the matrix cores (kernel: gemm_mfma_kernel.h) ----
+// A and C row-major, B row-major or k-fastest; leading dimensions and batch strides in elements.
 struct GemmArgs {
   const void *a;
   const void *b;
@@ -51,10 +52,9 @@ struct GemmArgs {
 };
 // kind: 0 = i8 x i8, 1 = u8 x i8, 2 = bf16 x bf16, 3 = f32 x f32; B stored k-fastest (gemm_nt.hip).
 hipError_t launch_gemm_nt(const GemmArgs &g, int kind, hipStream_t stream);
-bool gemm_i8_applicable(const GemmArgs &g, bool b_k_contiguous);
+// u8|i8 x i8 -> i32, bf16 x bf16 -> f32, f32 x f32 -> f32.
+bool gemm_i8_applicable(const GemmArgs &g);
 hipError_t launch_gemm_i8(const GemmArgs &g, bool a_unsigned, hipStream_t stream);
-
-// ---- gemm_bf16.hip: bf16 x bf16 -> f32 on the bf16 MFMA --------------------------------
 bool gemm_f32_applicable(const GemmArgs &g);
 hipError_t launch_gemm_f32(const GemmArgs &g, hipStream_t stream);
 bool gemm_bf16_applicable(const GemmArgs &g);

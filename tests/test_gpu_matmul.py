@@ -300,3 +300,30 @@ def test_manual_schedules_give_identical_results(gpu):
         spec.tile_out([1, 64, 64]).split(32).run_device([x.ptr for x in bufs])
     assert e.value.status == 1
     assert M.Matmul([1, 64, 64, 64], [M.u32] * 3).available_schedules() == []
+
+
+def test_matmul_output_beyond_4_gib(gpu):
+    """Near the largest output the Spec surface admits (volume < 2^31 elements,
+    tensorspec.rs:180-182): C is 8.5 GB, so byte offsets pass 2^32 and 2^33 is near.  Bands of rows at the
+    start, across the 4 GiB and 6 GiB marks and at the end, bit-exact against the oracle;
+    the rows between must have been written too (a sentinel would survive otherwise)."""
+    import ctypes as C
+    from morello_amd import _binding as B
+    m, k, n = 1 << 20, 64, 2040
+    A = synth.uniform_u8(99, 0, (1, m, k))
+    Bm = synth.uniform_i8(99, 1, (1, k, n))
+    spec = M.Matmul([1, m, k, n], (M.u8, M.i8, M.i32))
+    assert spec.check() == 0 and spec.bytes_used(2) == m * n * 4 > (1 << 32)
+    da, db = M.DeviceBuffer.from_numpy(A), M.DeviceBuffer.from_numpy(Bm)
+    dc = M.DeviceBuffer(m * n * 4)
+    assert B.load().mrl_memset(dc.ptr, 0x5a, m * n * 4) == 0
+    spec.run_device([da.ptr, db.ptr, dc.ptr])
+    row_bytes = n * 4
+    for r0 in (0, (1 << 32) // row_bytes - 2, (3 << 31) // row_bytes - 2, m // 3, m - 4):
+        got = np.empty((4, n), np.int32)
+        assert B.load().mrl_memcpy_d2h(got.ctypes.data_as(C.c_void_p), C.c_void_p(dc.ptr + r0 * row_bytes),
+                                       4 * row_bytes) == 0
+        want = A[0, r0:r0 + 4].astype(np.int32) @ Bm[0].astype(np.int32)
+        assert np.array_equal(got, want), r0
+    for buf in (da, db, dc):
+        buf.free()

@@ -109,3 +109,38 @@ def test_compose_msm_full_size(gpu):
     ones = synth.f32_to_bf16_bits(np.ones((b, n2, n), np.float32))
     got = run_spec(spec, [ones, q, kmat, np.zeros((b, m, n), np.float32)])
     assert np.abs(got - 1).max() < 1e-2
+
+
+def test_softmax_tensor_beyond_4_gib(gpu):
+    """2^19 rows of 4092 f32 = 8.6 GB in, 8.6 GB out: the largest tensor the Spec surface admits, byte
+    offsets up to 2^33.  Rows at the start, near the 4 GiB and 6 GiB marks and at the end, each within 1e-5
+    of the oracle; the input is one 64 MiB pattern repeated, uploaded piecewise."""
+    import ctypes as C
+    from morello_amd import _binding as B
+    rows, cols = 1 << 19, 4092
+    spec = M.Softmax([rows, cols], 1)
+    assert spec.check() == 0 and spec.bytes_used(0) > (1 << 32)
+    lib = B.load()
+    din, dout = M.DeviceBuffer(rows * cols * 4), M.DeviceBuffer(rows * cols * 4)
+    piece_rows = 4096
+    piece = synth.normal_f32(77, 0, (piece_rows, cols), 3.0)
+    for r0 in range(0, rows, piece_rows):
+        assert lib.mrl_memcpy_h2d(C.c_void_p(din.ptr + r0 * cols * 4), piece.ctypes.data_as(C.c_void_p),
+                                  piece.nbytes) == 0
+    spec.run_device([din.ptr, dout.ptr])
+    want = orc.softmax([8, cols], 1, piece[:8].copy())
+    row_bytes = cols * 4
+    for r0 in (0, ((1 << 32) // row_bytes // piece_rows) * piece_rows, ((3 << 31) // row_bytes // piece_rows) * piece_rows,
+               rows - piece_rows):
+        got = np.empty((8, cols), np.float32)
+        assert lib.mrl_memcpy_d2h(got.ctypes.data_as(C.c_void_p), C.c_void_p(dout.ptr + r0 * row_bytes),
+                                  8 * row_bytes) == 0
+        np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-9)
+    # The row that straddles the 4 GiB mark, whatever its place in the pattern.
+    r = (1 << 32) // row_bytes
+    got = np.empty((1, cols), np.float32)
+    assert lib.mrl_memcpy_d2h(got.ctypes.data_as(C.c_void_p), C.c_void_p(dout.ptr + r * row_bytes), row_bytes) == 0
+    np.testing.assert_allclose(got, orc.softmax([1, cols], 1, piece[r % piece_rows:r % piece_rows + 1].copy()),
+                               rtol=1e-5, atol=1e-9)
+    din.free()
+    dout.free()
