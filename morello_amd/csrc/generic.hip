@@ -169,7 +169,12 @@ template <bool FLOAT_OUT>
 __global__ __launch_bounds__(256) void k_matmul_generic(MM p) {
   __shared__ uint32_t ta[16][17], tb[16][17];
   const uint32_t tx = threadIdx.x % 16, ty = threadIdx.x / 16;
-  const uint32_t j = blockIdx.x * 16 + tx, i = blockIdx.y * 16 + ty, bi = blockIdx.z;
+  // One 16 x 16 output tile per workgroup, tiles numbered n-fastest, then m, then batch, in
+  // grid.x alone (grid.y and grid.z stop at 65535, which 2^20 rows would pass).
+  const uint32_t tiles_n = (p.N + 15) / 16, tiles_m = (p.M + 15) / 16;
+  const uint32_t tile_j = blockIdx.x % tiles_n, tile_i = (blockIdx.x / tiles_n) % tiles_m;
+  const uint32_t bi = blockIdx.x / tiles_n / tiles_m;
+  const uint32_t j = tile_j * 16 + tx, i = tile_i * 16 + ty;
   const bool live = i < p.M && j < p.N;
   const int64_t coff = int64_t(bi) * p.sc[0] + int64_t(i) * p.sc[1] + int64_t(j) * p.sc[2];
   float facc = 0.0f;
@@ -361,7 +366,9 @@ hipError_t launch_matmul_generic(const Strided &a, const Strided &b, const Strid
   p.B = a.shape[0], p.M = a.shape[1], p.K = a.shape[2], p.N = b.shape[2];
   for (int d = 0; d < 3; d++) p.sa[d] = a.stride[d], p.sb[d] = b.stride[d], p.sc[d] = c.stride[d];
   p.accum = accum;
-  dim3 grid((p.N + 15) / 16, (p.M + 15) / 16, p.B);
+  const uint64_t tiles = uint64_t((p.N + 15) / 16) * ((p.M + 15) / 16) * p.B;
+  if (tiles > 0x7fffffffull) return hipErrorInvalidValue;
+  dim3 grid{uint32_t(tiles)};
   if (float_out(c.dtype)) hipLaunchKernelGGL(k_matmul_generic<true>, grid, dim3(256), 0, stream, p);
   else hipLaunchKernelGGL(k_matmul_generic<false>, grid, dim3(256), 0, stream, p);
   return hipGetLastError();

@@ -327,3 +327,14 @@ def test_matmul_output_beyond_4_gib(gpu):
         assert np.array_equal(got, want), r0
     for buf in (da, db, dc):
         buf.free()
+
+
+def test_generic_matmul_with_a_million_rows(gpu):
+    """A dtype triple without a matrix-core kernel at 2^20 + 5 rows: the generic kernel's tile
+    numbering must not depend on the 65535 limit of the second grid dimension."""
+    m, k, n = (1 << 20) + 5, 3, 20
+    A = synth.check_pattern("u16", (1, m, k))
+    Bm = synth.check_pattern("u16", (1, k, n))
+    got = run_spec(M.Matmul([1, m, k, n], (M.u16, M.u16, M.u32)), [A, Bm, np.zeros((1, m, n), np.uint32)])
+    want = (A[0].astype(np.uint64) @ Bm[0].astype(np.uint64)).astype(np.uint32)
+    assert np.array_equal(got[0], want)
