@@ -472,6 +472,16 @@ int run_move(const mrl_spec &s, void *const *params, Workspace &ws) {
     HIP_TRY(mrl::launch_copy(params[0], params[1], count * mrl_dtype_size(s.dtypes[0]), ws.stream));
     return MRL_OK;
   }
+  // Both layouts permutations of the logical dims: strided kernels, coalesced on both sides.
+  mrl::Strided st, dt;
+  st.ptr = params[0], st.dtype = s.dtypes[0], st.rank = rank;
+  dt.ptr = params[1], dt.dtype = s.dtypes[1], dt.rank = rank;
+  for (uint32_t d = 0; d < MRL_MAX_RANK; d++) st.shape[d] = dt.shape[d] = d < rank ? shape[d] : 1;
+  if (mrl::layout_strides(li, shape, rank, st.stride) && mrl::layout_strides(lo, shape, rank, dt.stride)) {
+    const hipError_t e = mrl::launch_move_strided(st, dt, ws.stream);
+    if (e == hipSuccess) return MRL_OK;
+    if (e != hipErrorInvalidValue) HIP_TRY(e);
+  }
   mrl::LayoutEval sl, dl;
   if (!mrl::make_layout_eval(li, shape, rank, &sl) || !mrl::make_layout_eval(lo, shape, rank, &dl))
     return MRL_ERR_BAD_LAYOUT;

@@ -6,6 +6,8 @@
 // 547-569, 603-643): both inputs are converted to the output dtype, then multiplied and
 // accumulated in that dtype.  Integer outputs are computed modulo 2^32 and truncated on
 // store, which equals wrapping arithmetic in the narrower type.
+#include <utility>
+
 #include "kernels.h"
 
 namespace mrl {
@@ -60,7 +62,7 @@ __device__ inline uint32_t load_u32(const void *p, int dtype, int64_t off, int o
 __device__ inline void store_u32(void *p, int dtype, int64_t off, uint32_t v) {
   switch (dtype) {
     case MRL_U8: case MRL_I8: ((uint8_t *)p)[off] = uint8_t(v); break;
-    case MRL_U16: case MRL_I16: ((uint16_t *)p)[off] = uint16_t(v); break;
+    case MRL_U16: case MRL_I16: case MRL_BF16: ((uint16_t *)p)[off] = uint16_t(v); break;
     default: ((uint32_t *)p)[off] = v; break;
   }
 }
@@ -106,6 +108,15 @@ __device__ inline uint32_t float_to_int(float f, int dt) {
   return uint32_t(int32_t(f));
 }
 
+// One element: read as `sdt`, converted with Rust `as` semantics, returned as the bits of `ddt`.
+__device__ inline uint32_t move_bits(const void *src, int sdt, int64_t so, int ddt) {
+  const bool src_float = sdt == MRL_F32 || sdt == MRL_BF16;
+  if (ddt == MRL_F32) return __float_as_uint(load_f32(src, sdt, so));
+  if (ddt == MRL_BF16) return f32_to_bf16_bits(load_f32(src, sdt, so));
+  if (src_float) return float_to_int(load_f32(src, sdt, so), ddt);
+  return load_u32(src, sdt, so, MRL_U32);  // int -> int wraps
+}
+
 __global__ void k_move_generic(const void *src, void *dst, LayoutEval sl, LayoutEval dl, int sdt,
                                int ddt, uint64_t count) {
   const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -117,11 +128,69 @@ __global__ void k_move_generic(const void *src, void *dst, LayoutEval sl, Layout
     rem /= sl.shape[d];
   }
   const int64_t so = layout_offset(sl, pt), d_o = layout_offset(dl, pt);
-  const bool src_float = sdt == MRL_F32 || sdt == MRL_BF16;
-  if (ddt == MRL_F32) ((float *)dst)[d_o] = load_f32(src, sdt, so);
-  else if (ddt == MRL_BF16) ((uint16_t *)dst)[d_o] = f32_to_bf16_bits(load_f32(src, sdt, so));
-  else if (src_float) store_u32(dst, ddt, d_o, float_to_int(load_f32(src, sdt, so), ddt));
-  else store_u32(dst, ddt, d_o, load_u32(src, sdt, so, MRL_U32));  // int -> int wraps
+  store_u32(dst, ddt, d_o, move_bits(src, sdt, so, ddt));
+}
+
+// Move between two layouts that are permutations of the logical dims (element strides on both
+// sides).  `order` lists the dims slowest to fastest for the index decode.
+struct MoveStrided {
+  const void *src;
+  void *dst;
+  int sdt, ddt;
+  uint32_t rank;
+  uint32_t shape[MRL_MAX_RANK];
+  int64_t ss[MRL_MAX_RANK], ds[MRL_MAX_RANK];
+  uint32_t order[MRL_MAX_RANK];
+  uint32_t dim_s, dim_d;      // the dim each side stores contiguously
+  uint32_t tiles_s, tiles_d;  // 64-element tiles along them
+  uint64_t count;
+};
+
+// Both sides contiguous along the same dim: consecutive threads take consecutive elements of
+// that dim, so reads and writes are both coalesced.
+__global__ __launch_bounds__(256) void k_move_rows(MoveStrided p) {
+  const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= p.count) return;
+  uint64_t rem = i;
+  int64_t so = 0, d_o = 0;
+  for (int o = int(p.rank) - 1; o >= 0; o--) {
+    const uint32_t d = p.order[o], c = uint32_t(rem % p.shape[d]);
+    rem /= p.shape[d];
+    so += int64_t(c) * p.ss[d], d_o += int64_t(c) * p.ds[d];
+  }
+  store_u32(p.dst, p.ddt, d_o, move_bits(p.src, p.sdt, so, p.ddt));
+}
+
+// The two sides are contiguous along different dims: a 64 x 64 tile of (dim_d, dim_s) goes
+// through LDS, read with dim_s fastest and written with dim_d fastest, so both sides see
+// whole contiguous runs (move_relayout of morello/src/scheduling/moves.rs as a transpose).
+__global__ __launch_bounds__(256) void k_move_tiled(MoveStrided p) {
+  __shared__ uint32_t tile[64][65];
+  uint64_t blk = blockIdx.x;
+  const uint32_t ts = uint32_t(blk % p.tiles_s);
+  blk /= p.tiles_s;
+  const uint32_t td = uint32_t(blk % p.tiles_d);
+  blk /= p.tiles_d;
+  // The remaining dims, slowest to fastest in `order` (dim_s and dim_d are skipped).
+  int64_t so = 0, d_o = 0;
+  for (int o = int(p.rank) - 1; o >= 0; o--) {
+    const uint32_t d = p.order[o];
+    if (d == p.dim_s || d == p.dim_d) continue;
+    const uint32_t c = uint32_t(blk % p.shape[d]);
+    blk /= p.shape[d];
+    so += int64_t(c) * p.ss[d], d_o += int64_t(c) * p.ds[d];
+  }
+  const uint32_t lane = threadIdx.x & 63, quad = threadIdx.x >> 6;
+  const uint32_t s0 = ts * 64, d0 = td * 64, ns = p.shape[p.dim_s], nd = p.shape[p.dim_d];
+#pragma unroll 4
+  for (uint32_t r = quad; r < 64; r += 4)
+    if (d0 + r < nd && s0 + lane < ns)
+      tile[r][lane] = move_bits(p.src, p.sdt, so + int64_t(d0 + r) * p.ss[p.dim_d] + int64_t(s0 + lane) * p.ss[p.dim_s], p.ddt);
+  __syncthreads();
+#pragma unroll 4
+  for (uint32_t r = quad; r < 64; r += 4)
+    if (s0 + r < ns && d0 + lane < nd)
+      store_u32(p.dst, p.ddt, d_o + int64_t(s0 + r) * p.ds[p.dim_s] + int64_t(d0 + lane) * p.ds[p.dim_d], tile[lane][r]);
 }
 
 // Four 16-byte vectors per thread in flight, streamed past the caches: 6.5 TB/s on a 256 MiB
@@ -346,6 +415,43 @@ hipError_t launch_copy(const void *src, void *dst, uint64_t bytes, hipStream_t s
   if (tail)
     hipLaunchKernelGGL(k_copy1, dim3(1), dim3(16), 0, stream, (const uint8_t *)src + vecs * 16,
                        (uint8_t *)dst + vecs * 16, tail);
+  return hipGetLastError();
+}
+
+// Move between two strided layouts of the same logical shape.  Returns hipErrorInvalidValue
+// when the shape does not fit the kernels' index ranges (the caller then takes the generic path).
+hipError_t launch_move_strided(const Strided &src, const Strided &dst, hipStream_t stream) {
+  MoveStrided p;
+  p.src = src.ptr, p.dst = dst.ptr, p.sdt = src.dtype, p.ddt = dst.dtype, p.rank = src.rank;
+  p.count = 1;
+  int dim_s = -1, dim_d = -1;
+  for (uint32_t d = 0; d < MRL_MAX_RANK; d++) {
+    p.shape[d] = d < src.rank ? src.shape[d] : 1;
+    p.ss[d] = d < src.rank ? src.stride[d] : 0;
+    p.ds[d] = d < src.rank ? dst.stride[d] : 0;
+    p.count *= p.shape[d];
+    if (d < src.rank && p.shape[d] > 1 && p.ss[d] == 1) dim_s = int(d);
+    if (d < src.rank && p.shape[d] > 1 && p.ds[d] == 1) dim_d = int(d);
+  }
+  if (p.count == 0) return hipSuccess;
+  // Decode order: by decreasing destination stride, the destination's contiguous dim last.
+  for (uint32_t d = 0; d < MRL_MAX_RANK; d++) p.order[d] = d;
+  for (uint32_t i = 0; i < p.rank; i++)
+    for (uint32_t j = i + 1; j < p.rank; j++)
+      if (p.ds[p.order[j]] > p.ds[p.order[i]]) std::swap(p.order[i], p.order[j]);
+  if (dim_s < 0 || dim_d < 0 || dim_s == dim_d) {
+    const uint64_t blocks = (p.count + 255) / 256;
+    if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(k_move_rows, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+    return hipGetLastError();
+  }
+  p.dim_s = uint32_t(dim_s), p.dim_d = uint32_t(dim_d);
+  p.tiles_s = (p.shape[dim_s] + 63) / 64, p.tiles_d = (p.shape[dim_d] + 63) / 64;
+  uint64_t blocks = uint64_t(p.tiles_s) * p.tiles_d;
+  for (uint32_t d = 0; d < p.rank; d++)
+    if (int(d) != dim_s && int(d) != dim_d) blocks *= p.shape[d];
+  if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(k_move_tiled, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
   return hipGetLastError();
 }
 

@@ -31,6 +31,9 @@ hipError_t launch_fill_zero(void *ptr, uint64_t bytes, hipStream_t stream);
 hipError_t launch_move_generic(const void *src, void *dst, const LayoutEval &src_l,
                                const LayoutEval &dst_l, int src_dtype, int dst_dtype,
                                uint64_t count, hipStream_t stream);
+// Move between two layouts that are permutations of the logical dims (strides in elements):
+// coalesced on both sides, through an LDS transpose when their contiguous dims differ.
+hipError_t launch_move_strided(const Strided &src, const Strided &dst, hipStream_t stream);
 // bf16 -> f32 of a whole buffer, position by position.
 hipError_t launch_widen_bf16(const void *src, void *dst, uint64_t count, hipStream_t stream);
 // Move Spec fast path: same bytes on both sides (16-byte aligned buffers).
