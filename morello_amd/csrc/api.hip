@@ -303,7 +303,7 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
     void *wide = nullptr;
     HIP_TRY(ws.alloc(&wide, narrow.count * sizeof(float)));
     HIP_TRY(mrl::launch_widen_bf16(narrow.t.ptr, wide, narrow.count, ws.stream));
-    narrow.t.ptr = wide, narrow.t.dtype = MRL_F32;
+    narrow.t.ptr = wide, narrow.t.dtype = MRL_F32, narrow.elem = sizeof(float);
     da = db = MRL_F32;
   }
   mrl::GemmArgs g;
@@ -318,7 +318,40 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
     std::swap(bt.stride[1], bt.stride[2]);
     b_ok = g.b_kmajor = as_rows(bt, &g.ldb, &g.sb);
   }
-  const bool rows = as_rows(a.t, &g.lda, &g.sa) && b_ok && as_rows(c.t, &g.ldc, &g.sc);
+  bool rows = as_rows(a.t, &g.lda, &g.sa) && b_ok && as_rows(c.t, &g.ldc, &g.sc);
+  // Operands the matrix-core kernels cannot walk in place (A or C stored column-major, say)
+  // are brought to row-major with the strided Move first when that opens the fast path: two
+  // extra passes over one operand against a generic kernel that is tens of times slower.
+  mrl::Strided c_user = c.t;
+  bool c_densified = false;
+  const bool mfma_types = (((da == MRL_U8 || da == MRL_I8) && db == MRL_I8 && dc == MRL_I32) ||
+                           (da == MRL_BF16 && db == MRL_BF16 && dc == MRL_F32) ||
+                           (da == MRL_F32 && db == MRL_F32 && dc == MRL_F32));
+  if (!rows && !sched && mfma_types && g.m >= 64 && g.n >= 64 && g.k >= 64) {
+    auto densify = [&](Prepared &p, bool read) -> int {
+      int64_t ld, bs;
+      if (as_rows(p.t, &ld, &bs)) return MRL_OK;
+      mrl::Strided dense = p.t;
+      HIP_TRY(ws.alloc(&dense.ptr, p.count * p.elem));
+      dense.stride[2] = 1, dense.stride[1] = p.t.shape[2], dense.stride[0] = int64_t(p.t.shape[1]) * p.t.shape[2];
+      if (read) HIP_TRY(mrl::launch_move_strided(p.t, dense, ws.stream));
+      p.t = dense;
+      return MRL_OK;
+    };
+    if ((rc = densify(a, true)) != MRL_OK) return rc;
+    if (!b_ok && (rc = densify(b, true)) != MRL_OK) return rc;
+    int64_t ld, bs;
+    c_densified = !as_rows(c.t, &ld, &bs);
+    if ((rc = densify(c, s.accum != 0)) != MRL_OK) return rc;
+    g.a = a.t.ptr, g.b = b.t.ptr, g.c = c.t.ptr;
+    if (!b_ok) b_ok = as_rows(b.t, &g.ldb, &g.sb);
+    rows = as_rows(a.t, &g.lda, &g.sa) && b_ok && as_rows(c.t, &g.ldc, &g.sc);
+  }
+  auto finish = [&]() -> int {
+    if (c_densified) HIP_TRY(mrl::launch_move_strided(c.t, c_user, ws.stream));
+    if (c_densified) c.t = c_user;
+    return finish_output(c, ws);
+  };
   bool done = false;
   if (sched) {
     const int kind = (da == MRL_I8 && db == MRL_I8 && dc == MRL_I32)     ? 0
@@ -349,7 +382,7 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
     done = true;
   }
   if (!done) HIP_TRY(mrl::launch_matmul_generic(a.t, b.t, c.t, s.accum, ws.stream));
-  return finish_output(c, ws);
+  return finish();
 }
 
 int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {

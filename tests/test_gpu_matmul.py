@@ -194,6 +194,29 @@ def test_mixed_bf16_f32_matmul(gpu, dts, codes):
     assert rel_err(got, orc.matmul([b, m, k, n], codes, A, Bm, C0.copy(), True)) < 1e-5
 
 
+@pytest.mark.parametrize("dts,codes", [((M.u8, M.i8, M.i32), [0, 1, 5]), ((M.bf16, M.bf16, M.f32), [7, 7, 6]),
+                                        ((M.f32, M.bf16, M.f32), [6, 7, 6])])
+@pytest.mark.parametrize("accum", [False, True])
+def test_matmul_with_column_major_a_and_c(gpu, dts, codes, accum):
+    """A and C stored column-major (m fastest): brought to row-major with the strided Move,
+    multiplied on the matrix cores, and C moved back."""
+    b, m, k, n = 2, 192, 128, 136
+    gen = {M.u8: synth.uniform_u8, M.i8: synth.uniform_i8, M.bf16: synth.normal_bf16, M.f32: synth.uniform_f32}
+    A, Bm = gen[dts[0]](72, 0, (b, m, k)), gen[dts[1]](72, 1, (b, k, n))
+    out_np = np.int32 if dts[2] == M.i32 else np.float32
+    C0 = synth.uniform_u8(72, 2, (b, m, n)).astype(out_np) if accum else np.zeros((b, m, n), out_np)
+    layouts = [M.batched_col_major([b, m, k]), None, M.batched_col_major([b, m, n])]
+    At = np.ascontiguousarray(A.transpose(0, 2, 1))
+    C0t = np.ascontiguousarray(C0.transpose(0, 2, 1))
+    got_t = run_spec(M.Matmul([b, m, k, n], dts, layouts=layouts, accum=accum), [At, Bm, C0t])
+    want = orc.matmul([b, m, k, n], codes, A, Bm, C0.copy(), accum)
+    got = got_t.transpose(0, 2, 1)
+    if dts[2] == M.i32:
+        assert np.array_equal(got, want)
+    else:
+        assert rel_err(got, want) < 1e-5
+
+
 def test_bf16_matmul_pattern_exact(gpu):
     """0..3 inputs (verification.rs:933-935): every partial sum is an exact integer."""
     b, m, k, n = 1, 256, 256, 256
