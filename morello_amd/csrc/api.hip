@@ -405,11 +405,38 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
   cv.ow = s.spec_shape[4], cv.fh = s.spec_shape[5], cv.fw = s.spec_shape[6];
   cv.accum = s.accum;
   const int di = s.dtypes[0], df = s.dtypes[1], dout = s.dtypes[2];
-  if ((di == MRL_U8 || di == MRL_I8) && df == MRL_I8 && dout == MRL_I32 && channels_last(img.t) &&
-      channels_last(filt.t) && channels_last(out.t) && mrl::conv_i8_applicable(cv)) {
+  const bool fast_types = (di == MRL_U8 || di == MRL_I8) && df == MRL_I8 && dout == MRL_I32;
+  // Tensors in another permutation layout (NCHW, say) are moved to channels-last when the
+  // shape suits the matrix-core kernel: three small extra passes against a generic kernel
+  // that is hundreds of times slower.
+  const mrl::Strided out_user = out.t;
+  bool out_moved = false;
+  if (fast_types && cv.f == 64 && cv.c % 64 == 0 && (cv.fh * cv.fw * (cv.c / 64) == 1 || cv.fh * cv.fw * (cv.c / 64) == 9)) {
+    auto to_channels_last = [&](Prepared &p, bool read) -> int {
+      if (channels_last(p.t)) return MRL_OK;
+      mrl::Strided dense = p.t;
+      HIP_TRY(ws.alloc(&dense.ptr, p.count * p.elem));
+      const int64_t c = p.t.shape[1], h = p.t.shape[2], w = p.t.shape[3];
+      dense.stride[1] = 1, dense.stride[3] = c, dense.stride[2] = c * w, dense.stride[0] = c * w * h;
+      if (read) HIP_TRY(mrl::launch_move_strided(p.t, dense, ws.stream));
+      p.t = dense;
+      return MRL_OK;
+    };
+    if ((rc = to_channels_last(img, true)) != MRL_OK) return rc;
+    if ((rc = to_channels_last(filt, true)) != MRL_OK) return rc;
+    out_moved = !channels_last(out.t);
+    if ((rc = to_channels_last(out, s.accum != 0)) != MRL_OK) return rc;
+    cv.image = img.t.ptr, cv.filters = filt.t.ptr, cv.out = out.t.ptr;
+  }
+  if (fast_types && channels_last(img.t) && channels_last(filt.t) && channels_last(out.t) &&
+      mrl::conv_i8_applicable(cv)) {
     HIP_TRY(mrl::launch_conv_i8(cv, di == MRL_U8, ws.stream));
   } else {
     HIP_TRY(mrl::launch_conv_generic(img.t, filt.t, out.t, s.accum, ws.stream));
+  }
+  if (out_moved) {
+    HIP_TRY(mrl::launch_move_strided(out.t, out_user, ws.stream));
+    out.t = out_user;
   }
   return finish_output(out, ws);
 }

@@ -49,6 +49,27 @@ def test_conv_nchw_layout_generic(gpu):
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("accum", [False, True])
+def test_conv_nchw_layout_on_the_matrix_cores(gpu, accum):
+    """NCHW image and output, FCRS filters (all row-major) at a shape the matrix-core kernel
+    takes: the tensors are moved to channels-last and back around it.  Mixed: only the output
+    in NCHW."""
+    shape = (3, 64, 64, 9, 11, 3, 3)
+    b, f, c, oh, ow, fh, fw = shape
+    img = synth.uniform_u8(112, 0, (b, c, oh + 2, ow + 2))
+    filt = synth.uniform_i8(112, 1, (f, c, fh, fw))
+    out0 = synth.uniform_u8(112, 2, (b, f, oh, ow)).astype(np.int32) if accum else np.zeros((b, f, oh, ow), np.int32)
+    want = orc.conv(list(shape), [0, 1, 5], img, filt, out0.copy(), accum)
+    rm = [M.row_major(s) for s in M.Conv(shape, (M.u8, M.i8, M.i32)).parameter_shapes()]
+    got = run_spec(M.Conv(shape, (M.u8, M.i8, M.i32), layouts=rm, accum=accum), [img, filt, out0.copy()])
+    assert np.array_equal(got, want)
+    nhwc_img = np.ascontiguousarray(img.transpose(0, 2, 3, 1))
+    krsc = np.ascontiguousarray(filt.transpose(0, 2, 3, 1))
+    got = run_spec(M.Conv(shape, (M.u8, M.i8, M.i32), layouts=[None, None, rm[2]], accum=accum),
+                   [nhwc_img, krsc, out0.copy()])
+    assert np.array_equal(got, want)
+
+
 def test_conv_full_size_properties(gpu):
     """benchmark configuration 4 (32x56x56x64 -> 64, 3x3): a few images against the oracle, every
     image through a checksum (sum over filters and pixels, computed in int64 from box sums),
