@@ -376,6 +376,59 @@ __global__ __launch_bounds__(256) void k_softmax_generic(SM p) {
   for (uint32_t i = lane; i < n; i += 64) p.out[obase + i * os] /= sum;
 }
 
+// The scan dim is strided but another dim (`fast`) is contiguous on both sides: a workgroup
+// takes 64 consecutive positions of `fast` (one per lane, so every access is a 256-byte run)
+// and its four waves split the scan dim; each lane keeps the online (max, denominator) pair of
+// morello/src/spec.rs:96-106 over its share, the four shares are merged through LDS with the
+// parts formula (spec.rs:107-132), and a second sweep writes exp(x - max) / denominator.
+struct SMC {
+  SM s;
+  uint32_t fast, fast_tiles;
+};
+__global__ __launch_bounds__(256) void k_softmax_cols(SMC q) {
+  const SM &p = q.s;
+  __shared__ float sm_max[4][64], sm_den[4][64];
+  const uint32_t lane = threadIdx.x % 64, w = threadIdx.x / 64;
+  uint64_t r = blockIdx.x;
+  const uint32_t f = uint32_t(r % q.fast_tiles) * 64 + lane;
+  r /= q.fast_tiles;
+  int64_t ibase = 0, obase = 0;
+  for (int d = int(p.rank) - 1; d >= 0; d--) {
+    if (uint32_t(d) == p.scan_dim || uint32_t(d) == q.fast) continue;
+    const uint32_t c = uint32_t(r % p.shape[d]);
+    r /= p.shape[d];
+    ibase += c * p.si[d];
+    obase += c * p.so[d];
+  }
+  const bool live = f < p.shape[q.fast];
+  ibase += f, obase += f;  // unit stride on both sides
+  const uint32_t n = p.shape[p.scan_dim];
+  const int64_t is = p.si[p.scan_dim], os = p.so[p.scan_dim];
+  float mx = -3.40282347e+38f, den = 0.0f;
+  bool nan = false;
+  if (live)
+    for (uint32_t i = w; i < n; i += 4) {
+      const float x = p.in[ibase + i * is];
+      nan |= x != x;
+      const float nm = fmaxf(mx, x);
+      den = den * expf(mx - nm) + expf(x - nm);
+      mx = nm;
+    }
+  if (nan) mx = __uint_as_float(0x7fc00000u);
+  sm_max[w][lane] = mx, sm_den[w][lane] = den;
+  __syncthreads();
+  float m = sm_max[0][lane], d = sm_den[0][lane];
+#pragma unroll
+  for (int o = 1; o < 4; o++) {
+    const float om = sm_max[o][lane], od = sm_den[o][lane];
+    const float nm = (om != om || m != m) ? __uint_as_float(0x7fc00000u) : fmaxf(m, om);
+    d = d * expf(m - nm) + od * expf(om - nm);
+    m = nm;
+  }
+  if (live)
+    for (uint32_t i = w; i < n; i += 4) p.out[obase + i * os] = expf(p.in[ibase + i * is] - m) / d;
+}
+
 __global__ void k_fill_zero(uint32_t *p, uint64_t words, uint8_t *tail, uint32_t tail_bytes) {
   const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
   const uint64_t step = uint64_t(gridDim.x) * blockDim.x;
@@ -509,6 +562,16 @@ hipError_t launch_softmax_generic(const Strided &in, const Strided &out, uint32_
     if (d < in.rank && d != scan_dim) lines *= in.shape[d];
   }
   p.lines = lines;
+  // A dim other than the scan dim that both sides store contiguously: the column kernel.
+  for (uint32_t d = 0; d < in.rank; d++)
+    if (d != scan_dim && in.shape[d] >= 16 && in.stride[d] == 1 && out.stride[d] == 1) {
+      SMC q;
+      q.s = p, q.fast = d, q.fast_tiles = (in.shape[d] + 63) / 64;
+      const uint64_t blocks = lines / in.shape[d] * q.fast_tiles;
+      if (blocks > 0x7fffffffull) break;
+      hipLaunchKernelGGL(k_softmax_cols, dim3(uint32_t(blocks)), dim3(256), 0, stream, q);
+      return hipGetLastError();
+    }
   const uint32_t blocks = uint32_t((lines + 3) / 4);
   hipLaunchKernelGGL(k_softmax_generic, dim3(blocks), dim3(256), 0, stream, p);
   return hipGetLastError();
