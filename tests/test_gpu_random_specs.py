@@ -1,0 +1,137 @@
+"""Differential test over seeded random Specs: random shapes (through and around the
+matrix-core kernels' thresholds), dtype triples, accumulation and per-parameter layouts
+(random permutations of the logical dims, optionally with a Packed or OddEven dim), run through
+the C ABI and compared with the CPU oracle on the very same parameter buffers.  Integers must
+match bit for bit, floating point to 1e-5 (norm-wise)."""
+import numpy as np
+import pytest
+
+import morello_amd as M
+import orc
+from gpu_util import rel_err, run_spec
+from morello_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+SIZES = list(range(1, 20)) + [24, 31, 32, 33, 48, 63, 64, 65, 72, 96, 100, 128, 136, 200, 264]
+NP = {M.u8: np.uint8, M.i8: np.int8, M.u16: np.uint16, M.i16: np.int16, M.u32: np.uint32, M.i32: np.int32,
+      M.f32: np.float32, M.bf16: np.uint16}
+
+
+def random_layout(rng, shape):
+    """-> (M.Layout, orc layout) over `shape`: a random order of the dims, and sometimes one dim
+    split off as a trailing Packed(n) / OddEven(n) dim (n divides the dim, layout.rs:769-810)."""
+    rank = len(shape)
+    order = list(rng.permutation(rank))
+    m_dims, o_dims = [int(d) for d in order], [int(d) for d in order]
+    if rng.random() < 0.35:
+        d = int(rng.integers(rank))
+        divisors = [n for n in (2, 4, 8, 16) if shape[d] % n == 0 and shape[d] > n]
+        if divisors:
+            n = int(rng.choice(divisors))
+            if rng.random() < 0.7:
+                m_dims.append((d, M.Packed(n)))
+                o_dims.append((d, 1, n))
+            else:
+                m_dims.append((d, M.OddEven(n)))
+                o_dims.append((d, 2, n))
+    return M.layout(*m_dims), orc.make_layout(o_dims)
+
+
+def random_values(rng, dtype, shape, seed):
+    if dtype == M.f32:
+        return synth.normal_f32(seed, 0, shape)
+    if dtype == M.bf16:
+        return synth.normal_bf16(seed, 1, shape)
+    return synth.raw_u64(seed, 2, int(np.prod(shape))).astype(NP[dtype]).reshape(shape)
+
+
+def compare(got, want, dtype, what):
+    if dtype in (M.f32, M.bf16):
+        assert rel_err(got, want) < 1e-5, what
+    else:
+        assert np.array_equal(got, want), what
+
+
+MATMUL_DTYPES = [(M.u8, M.i8, M.i32), (M.i8, M.i8, M.i32), (M.bf16, M.bf16, M.f32), (M.f32, M.f32, M.f32),
+                 (M.f32, M.bf16, M.f32), (M.u16, M.u16, M.u32), (M.u8, M.u8, M.u8), (M.i8, M.u8, M.f32),
+                 (M.i16, M.i8, M.i32)]
+
+
+@pytest.mark.parametrize("seed", range(120))
+def test_random_matmul(gpu, seed):
+    rng = np.random.default_rng(7000 + seed)
+    b = int(rng.choice([1, 1, 2, 3]))
+    # Half of the cases at sizes the matrix-core kernels take (every dim >= 64).
+    sizes = [64, 65, 72, 96, 100, 128, 136, 200, 264, 300] if rng.random() < 0.5 else SIZES
+    m, k, n = (int(rng.choice(sizes)) for _ in range(3))
+    dts = MATMUL_DTYPES[int(rng.integers(len(MATMUL_DTYPES)))]
+    accum = bool(rng.integers(2))
+    shape = [b, m, k, n]
+    pshapes = [[b, m, k], [b, k, n], [b, m, n]]
+    lay = [random_layout(rng, s) for s in pshapes]
+    bufs = [random_values(rng, dt, s, 7000 + seed * 3 + i) for i, (dt, s) in enumerate(zip(dts, pshapes))]
+    if not accum:
+        bufs[2] = np.zeros(pshapes[2], NP[dts[2]])
+    spec = M.Matmul(shape, dts, layouts=[l[0] for l in lay], accum=accum)
+    got = run_spec(spec, bufs)
+    want = orc.matmul(shape, [int(d) for d in dts], bufs[0], bufs[1], bufs[2].copy(), accum,
+                      layouts=[l[1] for l in lay])
+    compare(got, want, dts[2], (shape, dts, accum, [repr(l[0]) for l in lay]))
+
+
+MOVE_DTYPES = [M.u8, M.i8, M.u16, M.i16, M.u32, M.i32, M.f32, M.bf16]
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_move(gpu, seed):
+    rng = np.random.default_rng(8000 + seed)
+    rank = int(rng.integers(1, 5))
+    shape = [int(rng.choice(SIZES)) for _ in range(rank)]
+    sdt, ddt = (MOVE_DTYPES[int(rng.integers(8))] for _ in range(2))
+    (ls, lso), (ld, ldo) = random_layout(rng, shape), random_layout(rng, shape)
+    x = random_values(rng, sdt, shape, 8000 + seed)
+    if sdt == M.f32:
+        x = (x * 300).astype(np.float32)
+    got = run_spec(M.Move(shape, (sdt, ddt), layouts=[ls, ld]), [x, np.zeros(shape, NP[ddt])])
+    want = orc.move(shape, [int(sdt), int(ddt)], x, np.zeros(shape, NP[ddt]), layouts=[lso, ldo])
+    assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (shape, sdt, ddt, repr(ls), repr(ld))
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_softmax(gpu, seed):
+    rng = np.random.default_rng(9000 + seed)
+    rank = int(rng.integers(1, 5))
+    shape = [int(rng.choice(SIZES)) for _ in range(rank)]
+    dim = int(rng.integers(rank))
+    (li, lio), (lo, loo) = random_layout(rng, shape), random_layout(rng, shape)
+    x = (synth.normal_f32(9000 + seed, 0, shape) * 4).astype(np.float32)
+    got = run_spec(M.Softmax(shape, dim, layouts=[li, lo]), [x, np.zeros(shape, np.float32)])
+    want = orc.softmax(shape, dim, x, np.zeros(shape, np.float32), layouts=[lio, loo])
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-8, err_msg=str((shape, dim, repr(li), repr(lo))))
+
+
+CONV_DTYPES = [(M.u8, M.i8, M.i32), (M.i8, M.i8, M.i32), (M.f32, M.f32, M.f32), (M.u8, M.u8, M.u16)]
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_conv(gpu, seed):
+    rng = np.random.default_rng(9500 + seed)
+    big = rng.random() < 0.4  # shapes the matrix-core kernel takes
+    b = int(rng.integers(1, 3))
+    f = 64 if big else int(rng.integers(1, 9))
+    c = 64 if big else int(rng.integers(1, 9))
+    oh, ow = int(rng.integers(1, 7)), int(rng.integers(1, 7))
+    fh, fw = ((3, 3) if rng.random() < 0.6 else (1, 1)) if big else (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+    dts = CONV_DTYPES[int(rng.integers(2 if big else 4))]
+    accum = bool(rng.integers(2))
+    shape = [b, f, c, oh, ow, fh, fw]
+    pshapes = [[b, c, oh + fh - 1, ow + fw - 1], [f, c, fh, fw], [b, f, oh, ow]]
+    lay = [random_layout(rng, s) for s in pshapes]
+    bufs = [random_values(rng, dt, s, 9500 + seed * 3 + i) for i, (dt, s) in enumerate(zip(dts, pshapes))]
+    if not accum:
+        bufs[2] = np.zeros(pshapes[2], NP[dts[2]])
+    got = run_spec(M.Conv(shape, dts, layouts=[l[0] for l in lay], accum=accum), bufs)
+    want = orc.conv(shape, [int(d) for d in dts], bufs[0], bufs[1], bufs[2].copy(), accum,
+                    layouts=[l[1] for l in lay])
+    compare(got, want, dts[2], (shape, dts, accum, [repr(l[0]) for l in lay]))
