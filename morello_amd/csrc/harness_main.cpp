@@ -27,6 +27,7 @@
 //     dtypes one per parameter, comma separated: u8 i8 u16 i16 u32 i32 f32 bf16
 //     flags  accum | scan=<dim> | layouts=<l0,l1,..> with each l one of rm cm bcm nhwc
 //            (row-major, col-major, batched col-major, NHWC; default rm, conv default nhwc)
+//            or a layout! spelled with dots: 0.2.1.2p16 = layout![0, 2, 1, 2 p(16)], 1o8 = OddEven
 //
 // Unlike the reference's loader, which refuses non-row-major top-level tensors
 // (cpu.rs:226-231), files are always logical row-major and parameters with another layout
@@ -59,6 +60,32 @@ std::vector<std::string> split(const std::string &s, char sep) {
     start = pos + 1;
   }
   return out;
+}
+
+// The `layout!` macro as text: physical dims slowest to fastest separated by dots, each a
+// logical dim index, optionally followed by p<n> (Packed) or o<n> (OddEven): "0.2.1.2p16" is
+// layout![0, 2, 1, 2 p(16)] (examples/matmul_x86.rs:34-53).
+bool parse_layout(const std::string &text, mrl_layout *out) {
+  const auto dims = split(text, '.');
+  if (dims.empty() || dims.size() > MRL_MAX_PHYS) return false;
+  out->ndims = 0;
+  for (const std::string &d : dims) {
+    char *end = nullptr;
+    const unsigned long dim = std::strtoul(d.c_str(), &end, 10);
+    if (end == d.c_str() || dim >= MRL_MAX_RANK) return false;
+    mrl_physdim pd = {uint8_t(dim), MRL_DYNAMIC, 0};
+    if (*end == 'p' || *end == 'o') {
+      pd.kind = *end == 'p' ? MRL_PACKED : MRL_ODDEVEN;
+      char *end2 = nullptr;
+      const unsigned long n = std::strtoul(end + 1, &end2, 10);
+      if (end2 == end + 1 || *end2 || n == 0 || n > 0xffffffffull) return false;
+      pd.size = uint32_t(n);
+    } else if (*end) {
+      return false;
+    }
+    out->dims[out->ndims++] = pd;
+  }
+  return true;
 }
 
 bool parse_spec(const std::string &text, mrl_spec *spec, std::string *err) {
@@ -119,7 +146,12 @@ bool parse_spec(const std::string &text, mrl_spec *spec, std::string *err) {
     else if (layouts[i] == "cm") rc = mrl_layout_col_major(shape, rank, &spec->layouts[i]);
     else if (layouts[i] == "bcm") rc = mrl_layout_batched_col_major(shape, rank, &spec->layouts[i]);
     else if (layouts[i] == "nhwc") rc = mrl_layout_nhwc(shape, rank, &spec->layouts[i]);
+    else if (parse_layout(layouts[i], &spec->layouts[i])) rc = MRL_OK;
     else return *err = "unknown layout " + layouts[i], false;
+    if (rc == MRL_OK) {
+      uint32_t phys[MRL_MAX_PHYS];
+      rc = mrl_layout_physical_shape(&spec->layouts[i], shape, rank, phys);
+    }
     if (rc != MRL_OK) return *err = "layout " + layouts[i] + " does not fit parameter", false;
   }
   return true;

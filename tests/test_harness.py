@@ -122,6 +122,14 @@ def test_check_mode_other_specs(gpu, tmp_path):
     want = orc.compose_msm(b, m, k, n2, n, [7, 7, 7, 6], v, q, kt, np.zeros((b, m, n), np.float32))
     got = parse_output(r.stdout, np.float32)
     assert np.abs(got - want).max() / np.abs(want).max() < 1e-2
+    # A packed B layout spelled out (layout![0, 2, 1, 2 p(16)], examples/matmul_x86.rs:34-53):
+    # the file stays logical row-major, the harness brings it to the layout on the device.
+    A, Bm = synth.uniform_u8(505, 0, (1, 8, 32)), synth.uniform_i8(505, 1, (1, 32, 48))
+    r = run("matmul:1x8x32x48:u8,i8,i32:layouts=rm,0.2.1.2p16,rm", *files_for([A, Bm, np.zeros((1, 8, 48), np.int32)]))
+    assert r.returncode == 0, r.stderr
+    assert np.array_equal(parse_output(r.stdout, np.int32),
+                          orc.matmul([1, 8, 32, 48], [0, 1, 5], A, Bm, np.zeros((1, 8, 48), np.int32)))
+    assert run("matmul:1x8x32x48:u8,i8,i32:layouts=rm,0.2.1.2p7,rm").returncode == 1   # 7 does not divide 48
     # A primitive with two written parameters prints both, in parameter order.
     x = synth.normal_f32(504, 0, (4, 50))
     r = run("softmaxdenominatorandmax:4x50:f32,f32,f32:scan=1",
