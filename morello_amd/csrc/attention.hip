@@ -52,6 +52,11 @@ __device__ inline v2i read_tr16(const uint8_t *p) {
   return __builtin_bit_cast(v2i, r);
 }
 
+// RAGGED: m need not be a multiple of 128 nor n2 of 128.  Query rows past m are computed on
+// a clamped (valid) row and not stored; the key blocks are dealt ceil/floor to the two halves,
+// loads past the end of K / V are clamped to the entry's last 16 bytes (finite data, weighted
+// by exp(-inf) = 0), and the scores of keys past n2 are set to -inf before the softmax.
+template <bool RAGGED>
 __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -61,17 +66,23 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
   // Workgroups go to the 8 XCDs round-robin.  All query blocks of a batch entry share its K
   // and V, so a batch entry's blocks are kept on one XCD (one L2) whenever the counts allow:
   // XCD x takes the x-th run of consecutive (entry, block) pairs.
-  const uint32_t nqb = p.m / BQ, total = nqb * p.b;
+  const uint32_t nqb = (p.m + BQ - 1) / BQ, total = nqb * p.b;
   uint32_t lin = blockIdx.x;
   if (total % 8 == 0) lin = (lin % 8) * (total / 8) + lin / 8;
   const int64_t head = lin / nqb;
   const int q0 = int(lin % nqb) * BQ + qg * 32;
-  const int keys_per_half = int(p.n2 / 2);
-  const int nblocks = keys_per_half / BKV;
+  // Key blocks of this half: [first_block, first_block + nblocks); both halves run `steps`
+  // iterations so that they meet at the same barriers.
+  const int all_blocks = int((p.n2 + BKV - 1) / BKV);
+  const int steps = (all_blocks + 1) / 2;
+  const int first_block = half ? steps : 0;
+  const int nblocks = half ? all_blocks - steps : steps;
+  const uint32_t head_bytes = p.n2 * ROW;  // K or V of one batch entry
 
-  const uint8_t *Q = (const uint8_t *)p.q + (head * p.m + q0 + lq) * int64_t(ROW);
-  const uint8_t *K = (const uint8_t *)p.kt + (head * p.n2 + int64_t(half) * keys_per_half) * ROW;
-  const uint8_t *V = (const uint8_t *)p.v + (head * p.n2 + int64_t(half) * keys_per_half) * ROW;
+  const int q_row = RAGGED ? min(q0 + lq, int(p.m) - 1) : q0 + lq;
+  const uint8_t *Q = (const uint8_t *)p.q + (head * p.m + q_row) * int64_t(ROW);
+  const uint8_t *K = (const uint8_t *)p.kt + head * p.n2 * ROW;
+  const uint8_t *V = (const uint8_t *)p.v + head * p.n2 * ROW;
   uint8_t *my_lds = lds + half * HALF;
 
   // Q^T operand: lane (query lq, half lg) holds d = 16*step + 8*lg .. +7.
@@ -91,14 +102,22 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
     k_src[i] = row * ROW + ((ld_pc ^ (row & 15)) << 4);
     v_src[i] = row * ROW + ((((ld_pc >> 2) ^ (row & 3)) << 6) | ((ld_pc & 3) << 4));
   }
+  // Byte offset within the batch entry's K (V) of this lane's chunk i of block kb.
+  auto k_off = [&](int kb, int i) {
+    const uint32_t off = uint32_t(first_block + kb) * TILE + k_src[i];
+    return RAGGED ? min(off, head_bytes - 16) : off;
+  };
+  auto v_off = [&](int kb, int i) {
+    const uint32_t off = uint32_t(first_block + kb) * TILE + v_src[i];
+    return RAGGED ? min(off, head_bytes - 16) : off;
+  };
   auto load_block = [&](int kb, int stage) {
-    const int64_t base = int64_t(kb) * TILE;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int q = qg * 4 + i;
-      __builtin_amdgcn_global_load_lds((global_cvoid *)(K + base + k_src[i]),
+      __builtin_amdgcn_global_load_lds((global_cvoid *)(K + k_off(kb, i)),
                                        (lds_void *)(my_lds + stage * STAGE + q * 1024), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((global_cvoid *)(V + base + v_src[i]),
+      __builtin_amdgcn_global_load_lds((global_cvoid *)(V + v_off(kb, i)),
                                        (lds_void *)(my_lds + stage * STAGE + TILE + q * 1024), 16, 0, 0);
     }
   };
@@ -114,24 +133,25 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
   const int v_rl = (lane & 15) >> 2;                                   // row within a 4-row read
   const int v_within = 32 * ((lane >> 4) & 1) + 8 * (lane & 3);        // bytes within a 64-B unit
 
-  load_block(0, 0);
-  for (int kb = 0; kb < nblocks; kb++) {
+  if (nblocks > 0) load_block(0, 0);
+  for (int kb = 0; kb < steps; kb++) {
     const int stage = kb & 1;
     // Block kb has landed (the loads are tracked by vmcnt only) and, after the barrier,
     // every wave is done reading the other stage, which the next block may now overwrite.
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
+    if (kb >= nblocks) continue;  // the shorter half idles through its partner's last block
     // The next block's global->LDS loads are issued one K and one V instruction at a time
     // between the MFMA batches below (such an instruction holds its wave for tens of cycles;
     // in a burst behind the barrier all eight waves queue up on the one memory pipe while
     // the matrix cores idle).  Past the last block the same block is fetched again into the
     // stage nobody reads.
-    const int64_t next_base = int64_t(min(kb + 1, nblocks - 1)) * TILE;
+    const int next_kb = min(kb + 1, nblocks - 1);
     uint8_t *next_lds = my_lds + (stage ^ 1) * STAGE;
     auto load_pair = [&](int i) {
       const int q = qg * 4 + i;
-      __builtin_amdgcn_global_load_lds((global_cvoid *)(K + next_base + k_src[i]), (lds_void *)(next_lds + q * 1024), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((global_cvoid *)(V + next_base + v_src[i]), (lds_void *)(next_lds + TILE + q * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((global_cvoid *)(K + k_off(next_kb, i)), (lds_void *)(next_lds + q * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((global_cvoid *)(V + v_off(next_kb, i)), (lds_void *)(next_lds + TILE + q * 1024), 16, 0, 0);
     };
     const uint8_t *lk = my_lds + stage * STAGE, *lv = lk + TILE;
 
@@ -190,6 +210,17 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
       }
     }
     __builtin_amdgcn_sched_barrier(0);
+    if (RAGGED) {
+      // Keys past n2 (only ever in the very last block): their scores leave the softmax.
+      const int valid = int(p.n2) - (first_block + kb) * BKV;
+      if (valid < BKV) {
+#pragma unroll
+        for (int kt = 0; kt < BKV / 32; kt++)
+#pragma unroll
+          for (int r = 0; r < 16; r++)
+            if (kt * 32 + 8 * (r / 4) + 4 * lg + r % 4 >= valid) s[kt][r] = -__builtin_inff();
+      }
+    }
     // Online softmax update for this lane's query, in base 2: exp(x - m) = 2^(x*log2e - m*log2e).
     float mx = s[0][0];
 #pragma unroll
@@ -254,6 +285,7 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
     const float inv = 1.0f / (l_tot * a0 + l1 * a1);
     const float w0 = a0 * inv, w1 = a1 * inv;
     float *out = p.out + (head * p.m + q0 + lq) * int64_t(D);
+    if (!RAGGED || q0 + lq < int(p.m))
 #pragma unroll
     for (int t = 0; t < D / 32; t++)
 #pragma unroll
@@ -272,18 +304,22 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
 
 bool attn_applicable(const AttnArgs &a) {
   auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-  return a.k == D && a.n == D && a.m % BQ == 0 && a.n2 % (2 * BKV) == 0 && a.m && a.n2 && a.b &&
-         uint64_t(a.m / BQ) * a.b < (1u << 31) && al16(a.q) && al16(a.kt) && al16(a.v) && al16(a.out);
+  return a.k == D && a.n == D && a.m && a.n2 && a.b && uint64_t(a.n2) * ROW < (1ull << 31) &&
+         uint64_t((a.m + BQ - 1) / BQ) * a.b < (1u << 31) && al16(a.q) && al16(a.kt) && al16(a.v) && al16(a.out);
 }
 
 hipError_t launch_attn(const AttnArgs &a, hipStream_t stream) {
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void *)k_attn, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * HALF);
+    hipError_t e = hipFuncSetAttribute((const void *)k_attn<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * HALF);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void *)k_attn<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * HALF);
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  hipLaunchKernelGGL(k_attn, dim3((a.m / BQ) * a.b), dim3(512), 2 * HALF, stream, a);
+  const dim3 grid(((a.m + BQ - 1) / BQ) * a.b);
+  if (a.m % BQ == 0 && a.n2 % (2 * BKV) == 0) hipLaunchKernelGGL(k_attn<false>, grid, dim3(512), 2 * HALF, stream, a);
+  else hipLaunchKernelGGL(k_attn<true>, grid, dim3(512), 2 * HALF, stream, a);
   return hipGetLastError();
 }
 
