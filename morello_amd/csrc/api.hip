@@ -324,10 +324,14 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
   // extra passes over one operand against a generic kernel that is tens of times slower.
   mrl::Strided c_user = c.t;
   bool c_densified = false;
-  const bool mfma_types = (((da == MRL_U8 || da == MRL_I8) && db == MRL_I8 && dc == MRL_I32) ||
-                           (da == MRL_BF16 && db == MRL_BF16 && dc == MRL_F32) ||
-                           (da == MRL_F32 && db == MRL_F32 && dc == MRL_F32));
-  if (!rows && !sched && mfma_types && g.m >= 64 && g.n >= 64 && g.k >= 64) {
+  // -1: no matrix-core kernel for these dtypes.
+  const int kind = (da == MRL_I8 && db == MRL_I8 && dc == MRL_I32)       ? 0
+                   : (da == MRL_U8 && db == MRL_I8 && dc == MRL_I32)     ? 1
+                   : (da == MRL_BF16 && db == MRL_BF16 && dc == MRL_F32) ? 2
+                   : (da == MRL_F32 && db == MRL_F32 && dc == MRL_F32)   ? 3
+                                                                         : -1;
+  const bool worth_two_more_passes = double(g.m) * g.n * g.k * g.batch >= 256.0 * 256 * 256;
+  if (!rows && !sched && kind >= 0 && g.m >= 64 && g.n >= 64 && g.k >= 64 && worth_two_more_passes) {
     auto densify = [&](Prepared &p, bool read) -> int {
       int64_t ld, bs;
       if (as_rows(p.t, &ld, &bs)) return MRL_OK;
@@ -352,36 +356,18 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
     if (c_densified) c.t = c_user;
     return finish_output(c, ws);
   };
-  bool done = false;
   if (sched) {
-    const int kind = (da == MRL_I8 && db == MRL_I8 && dc == MRL_I32)     ? 0
-                     : (da == MRL_U8 && db == MRL_I8 && dc == MRL_I32)   ? 1
-                     : (da == MRL_BF16 && db == MRL_BF16 && dc == MRL_F32) ? 2
-                     : (da == MRL_F32 && db == MRL_F32 && dc == MRL_F32)   ? 3
-                                                                           : -1;
-    const bool ok = kind >= 0 && rows && !g.b_kmajor &&
-                    (kind == 3   ? mrl::gemm_f32_applicable(g)
-                     : kind == 2 ? mrl::gemm_bf16_applicable(g)
-                                 : mrl::gemm_i8_applicable(g));
-    if (!ok) return MRL_ERR_UNSUPPORTED;
+    // A manual schedule is honoured wherever the kernel can run, whatever the size model says.
+    if (kind < 0 || !rows || g.b_kmajor || !mrl::gemm_possible(g, kind)) return MRL_ERR_UNSUPPORTED;
     hipError_t e = mrl::launch_gemm_scheduled(g, kind, sched->tile_m, sched->tile_n, sched->split_k, ws.stream);
     if (e == hipErrorInvalidValue) return MRL_ERR_UNSUPPORTED;
     HIP_TRY(e);
     return finish_output(c, ws);
   }
-  if (rows && (da == MRL_U8 || da == MRL_I8) && db == MRL_I8 && dc == MRL_I32 &&
-      mrl::gemm_i8_applicable(g)) {
-    HIP_TRY(mrl::launch_gemm_i8(g, da == MRL_U8, ws.stream));
-    done = true;
-  } else if (rows && da == MRL_BF16 && db == MRL_BF16 && dc == MRL_F32 &&
-             mrl::gemm_bf16_applicable(g)) {
-    HIP_TRY(mrl::launch_gemm_bf16(g, ws.stream));
-    done = true;
-  } else if (rows && da == MRL_F32 && db == MRL_F32 && dc == MRL_F32 && mrl::gemm_f32_applicable(g)) {
-    HIP_TRY(mrl::launch_gemm_f32(g, ws.stream));
-    done = true;
-  }
-  if (!done) HIP_TRY(mrl::launch_matmul_generic(a.t, b.t, c.t, s.accum, ws.stream));
+  if (kind >= 0 && rows && mrl::gemm_possible(g, kind) && mrl::gemm_pays(g, kind))
+    HIP_TRY(mrl::launch_gemm(g, kind, ws.stream));
+  else
+    HIP_TRY(mrl::launch_matmul_generic(a.t, b.t, c.t, s.accum, ws.stream));
   return finish();
 }
 

@@ -1,5 +1,7 @@
-// Dispatch of the Matmul Spec onto the matrix-core kernel of gemm_mfma_kernel.h with the
-// default tile (256 x 256 outputs, 128 bytes of K per step).
+// Dispatch of the Matmul Spec onto the matrix-core kernel of gemm_mfma_kernel.h.  Without a
+// manual schedule the workgroup tile is chosen from the problem size (the reference prices
+// schedules with a cost model before it emits one, morello/src/cost.rs; here the table is
+// three entries long and comes from measurement).
 #include "gemm_mfma_kernel.h"
 
 namespace mrl {
@@ -15,33 +17,62 @@ bool applicable(const GemmArgs &g, int es) {
   auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
   const int64_t per16 = 16 / es;
   constexpr int BM = TileBig::BM, BN = TileBig::BN;
-  // Below a tile's worth of work in either direction the generic kernel is the better fit.
-  return g.m >= 64 && g.n >= 64 && g.k >= 64 && (g.b_kmajor || g.n % per16 == 0) && g.k % per16 == 0 &&
+  return g.m >= 1 && g.n >= 1 && g.k >= 1 && (g.b_kmajor || g.n % per16 == 0) && g.k % per16 == 0 &&
          g.lda % per16 == 0 && g.ldb % per16 == 0 && g.sa % per16 == 0 && g.sb % per16 == 0 &&
          al16(g.a) && al16(g.b) && (reinterpret_cast<uintptr_t>(g.c) & 3) == 0 &&
          g.batch <= 65535 && uint64_t((g.m + BM - 1) / BM) * ((g.n + BN - 1) / BN) < (1u << 30);
 }
 
+// Side of the square workgroup tile for a problem size, from launch timings on an MI355X of
+// every built tile over cubes from 64^3 to 4096^3.  The 256 x 256 tile is the fastest per CU
+// but fills the chip in rounds of 256 tiles, one per CU; smaller tiles run several to a CU.
+//   int8, bf16: 256 once a round is at least half full (3072^3, 144 tiles: int8 47 us against
+//     55 us for 128 and 74 us for 64); below that 64 up to 384 of its tiles (1024^3: 8.0 us
+//     against 10.8 and 17.7), then 128 (2048^3: 19.6 us against 25.1 and 29.9).
+//   f32: its MFMA has a sixteenth of the int8 rate, so operand traffic never limits a small
+//     tile: 64 (1024^3: 30 us against 77 and 239; 3072^3: 463 against 592 and 714) until the
+//     256 tile fills its rounds (4096^3: 952 us against 1062).
+uint32_t tile_side(const GemmArgs &g, int es) {
+  const uint64_t big = uint64_t((g.m + 255) / 256) * ((g.n + 255) / 256) * g.batch;
+  const double round_fill = double(big) / double((big + 255) / 256 * 256);
+  if (round_fill >= (es == 4 ? 0.85 : 0.5)) return 256;
+  if (es == 4) return 64;
+  const uint64_t small = uint64_t((g.m + 63) / 64) * ((g.n + 63) / 64) * g.batch;
+  return small <= 384 ? 64 : 128;
+}
+
+constexpr int elem_size_of(int kind) { return kind == 3 ? 4 : kind == 2 ? 2 : 1; }
+
 }  // namespace
 
-bool gemm_i8_applicable(const GemmArgs &g) { return applicable(g, 1); }
-hipError_t launch_gemm_i8(const GemmArgs &g, bool a_unsigned, hipStream_t stream) {
-  if (g.b_kmajor) return launch_gemm_nt(g, a_unsigned ? 1 : 0, stream);
-  if (whole_tiles(g, 1))
-    return a_unsigned ? launch<I8, true, TileBig, false>(g, stream) : launch<I8, false, TileBig, false>(g, stream);
-  return a_unsigned ? launch<I8, true, TileBig, true>(g, stream) : launch<I8, false, TileBig, true>(g, stream);
+// Ragged shapes also need leading dimensions the EDGE kernels' 32-bit offsets can span.
+bool gemm_possible(const GemmArgs &g, int kind) {
+  const int es = elem_size_of(kind);
+  return applicable(g, es) && (edge_addressable(g, es) || whole_tiles(g, es));
 }
-bool gemm_f32_applicable(const GemmArgs &g) { return applicable(g, 4); }
-hipError_t launch_gemm_f32(const GemmArgs &g, hipStream_t stream) {
-  if (g.b_kmajor) return launch_gemm_nt(g, 3, stream);
-  return whole_tiles(g, 4) ? launch<F32, false, TileBig, false>(g, stream)
-                           : launch<F32, false, TileBig, true>(g, stream);
+// The 64 x 64 tile beats the generic kernel on anything but the tiniest problems, skinny ones
+// included (int8 32 x 4096 x 4096: 23 us against 237 us; f32 16 x 64 x 16: 4.1 us against 3.6 us).
+bool gemm_pays(const GemmArgs &g, int) { return double(g.m) * g.n * g.k * g.batch >= 100e3; }
+
+hipError_t launch_gemm_big(const GemmArgs &g, int kind, hipStream_t stream) {
+  if (g.b_kmajor) return launch_gemm_nt(g, kind, 256, stream);
+  const bool whole = whole_tiles(g, elem_size_of(kind));
+  switch (kind) {
+    case 0: return whole ? launch<I8, false, TileBig, false>(g, stream) : launch<I8, false, TileBig, true>(g, stream);
+    case 1: return whole ? launch<I8, true, TileBig, false>(g, stream) : launch<I8, true, TileBig, true>(g, stream);
+    case 2: return whole ? launch<BF16, false, TileBig, false>(g, stream) : launch<BF16, false, TileBig, true>(g, stream);
+    case 3: return whole ? launch<F32, false, TileBig, false>(g, stream) : launch<F32, false, TileBig, true>(g, stream);
+  }
+  return hipErrorInvalidValue;
 }
-bool gemm_bf16_applicable(const GemmArgs &g) { return applicable(g, 2); }
-hipError_t launch_gemm_bf16(const GemmArgs &g, hipStream_t stream) {
-  if (g.b_kmajor) return launch_gemm_nt(g, 2, stream);
-  return whole_tiles(g, 2) ? launch<BF16, false, TileBig, false>(g, stream)
-                           : launch<BF16, false, TileBig, true>(g, stream);
+
+hipError_t launch_gemm(const GemmArgs &g, int kind, hipStream_t stream) {
+  const int es = elem_size_of(kind);
+  // Only the 256 tile has a build without the EDGE kernels' limit on leading dimensions.
+  const uint32_t side = edge_addressable(g, es) ? tile_side(g, es) : 256;
+  if (side == 256) return launch_gemm_big(g, kind, stream);
+  if (g.b_kmajor) return launch_gemm_nt(g, kind, side, stream);
+  return launch_gemm_scheduled(g, kind, side, side, 64 / es, stream);
 }
 
 }  // namespace mrl

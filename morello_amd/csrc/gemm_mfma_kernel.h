@@ -37,7 +37,20 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
 constexpr int GROUP_M = 4;                // tile-rows per L2 group
+
+// Ragged tiles (EDGE) address memory through buffer resources: `records` bytes from `base` on
+// are in range, a load beyond them returns zeros and a store beyond them is dropped, both
+// without a branch.  Offsets are unsigned 32-bit, which is why the EDGE kernels want every
+// leading dimension below EDGE_MAX_ROW_BYTES: 256 rows of a tile then stay below 4 GiB.
+constexpr int64_t EDGE_MAX_ROW_BYTES = int64_t(1) << 24;
+constexpr uint32_t OUT_OF_RANGE = 0xffffffffu;  // an offset no resource holds
+__device__ inline __amdgpu_buffer_rsrc_t buffer_of(const void *base, int64_t records) {
+  const int64_t clamped = records < 0 ? 0 : records > int64_t(0xffffffffu) ? int64_t(0xffffffffu) : records;
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, int(uint32_t(clamped)), 0x00020000);
+}
 
 // Workgroup tile: BM x BN outputs, BKB bytes of K per k step, WAVES_M x WAVES_N waves.
 template <int BM_, int BN_, int BKB_, int WAVES_M_, int WAVES_N_>
@@ -144,11 +157,17 @@ __device__ inline void epilogue(const GemmArgs &g, typename T::Out *C, uint8_t *
   // each 32x32 block.  An accumulating Spec reads its whole block row of C first, so the
   // loads are in flight together instead of one round trip per element.
   // With EDGE the tile may hang over the bottom / right border of C: rows_left and
-  // cols_left bound what this workgroup owns.
+  // cols_left bound what this workgroup owns.  The rows are cut off by the range check of
+  // the buffer resource (an offset in a row past the last lies beyond its records); a lane
+  // whose column is past the last gets the out-of-range offset.
   const int lane_row = row0 + (lane >> 5) * 4, lane_col = col0 + (lane & 31);
   Out *c_lane = C + int64_t(lane_row) * g.ldc + lane_col;
-  auto inside = [&](int tm, int tn, int r) {
-    return !EDGE || (lane_row + tm * 32 + (r >> 2) * 8 + (r & 3) < rows_left && lane_col + tn * 32 < cols_left);
+  const uint32_t ldc_b = uint32_t(g.ldc) * sizeof(Out);
+  const auto c_buf = buffer_of(C, EDGE ? int64_t(rows_left - 1) * ldc_b + int64_t(cols_left) * sizeof(Out) : 0);
+  const uint32_t lane_off = uint32_t(lane_row) * ldc_b + uint32_t(lane_col) * sizeof(Out);
+  auto offset_of = [&](int tm, int tn, int r) -> uint32_t {
+    const uint32_t off = lane_off + uint32_t(tm * 32 + (r >> 2) * 8 + (r & 3)) * ldc_b + tn * 32 * sizeof(Out);
+    return lane_col + tn * 32 < cols_left ? off : OUT_OF_RANGE;
   };
 #pragma unroll
   for (int tm = 0; tm < TM; tm++) {
@@ -158,8 +177,10 @@ __device__ inline void epilogue(const GemmArgs &g, typename T::Out *C, uint8_t *
       for (int tn = 0; tn < TN; tn++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          prev[tn][r] = 0;
-          if (inside(tm, tn, r)) prev[tn][r] = c_lane[int64_t(tm * 32 + (r >> 2) * 8 + (r & 3)) * g.ldc + tn * 32];
+          if constexpr (EDGE)
+            prev[tn][r] = __builtin_bit_cast(Out, __builtin_amdgcn_raw_buffer_load_b32(c_buf, offset_of(tm, tn, r), 0, 0));
+          else
+            prev[tn][r] = c_lane[int64_t(tm * 32 + (r >> 2) * 8 + (r & 3)) * g.ldc + tn * 32];
         }
     }
 #pragma unroll
@@ -169,7 +190,9 @@ __device__ inline void epilogue(const GemmArgs &g, typename T::Out *C, uint8_t *
         Out v = acc[tm][tn][r];
         if (A_UNSIGNED) v += Out(corr[tn]);
         if (g.accum) v += prev[tn][r];
-        if (inside(tm, tn, r))
+        if constexpr (EDGE)
+          __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), c_buf, offset_of(tm, tn, r), 0, 2);
+        else
           __builtin_nontemporal_store(v, &c_lane[int64_t(tm * 32 + (r >> 2) * 8 + (r & 3)) * g.ldc + tn * 32]);
       }
   }
@@ -193,9 +216,11 @@ __device__ inline void sched_slots(bool staging) {
 }
 
 // EDGE = false: M, N multiples of the tile and K a multiple of the k step.  EDGE = true: any
-// M, any N and K whose rows are whole 16-byte chunks; chunks outside the matrices are fed as
-// zeros (a zero row of B makes the product and the column-sum correction vanish whatever A
-// holds there) and stores outside C are masked.
+// M, any N and K whose rows are whole 16-byte chunks (leading dimensions below
+// EDGE_MAX_ROW_BYTES); chunks past the last row or past K are fed as zeros and stores outside
+// C are dropped, both by the range check of buffer loads and stores, so the k loop and the
+// epilogue stay free of branches.  Chunks to the right of B's last column hold whatever
+// follows in memory: they only reach columns of C that are not stored.
 // B_KMAJOR: B is stored with k fastest (each of its n rows runs along K, `ldb` elements apart:
 // Morello's col_major / batched_col_major layouts, or layout![0,2,1]).  Its tile is then staged
 // and read exactly like A's, and no transposing read is involved.
@@ -301,41 +326,61 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
 
   v4i a_reg[A_CH], b_reg[B_CH];
   const int kt_count = int((g.k + BK - 1) / BK);
-  // EDGE bookkeeping: what is left of the matrices from this thread's first chunk on.
+  // EDGE bookkeeping.  The tiles are addressed relative to `a_tile` / `b_tile` (wave-uniform,
+  // advanced by one k step per load) with per-thread 32-bit offsets; what lies past the last
+  // row of the tile is out of the resource's range.  The end of K inside a row is not (the
+  // next row follows), so a thread whose chunk starts at or past K asks for the
+  // out-of-range offset instead.
   const int k_bytes = int(g.k) * ES;
-  const int a_rows_left = int(g.m - m0) - tid / A_ROW_CH;            // rows of A below the thread's
-  const int a_kb0 = (tid % A_ROW_CH) * 16;                            // its k byte within a tile
-  const int b_cols_left = int(g.n - n0) * ES - (tid % B_ROW_CH) * 16; // bytes of the B row right of it
-  const int b_k0 = tid / B_ROW_CH;                                    // its k row within a tile
-  const int b_rows_left = int(g.n - n0) - tid / B_ROW_CH;             // B_KMAJOR: n rows below the thread's
-  const int b_kb0 = (tid % B_ROW_CH) * 16;                            // B_KMAJOR: its k byte within a tile
+  const uint8_t *a_tile = A, *b_tile = B;
+  const int a_rows = min(BM, int(g.m - m0)), b_rows = min(BN, int(g.n - n0));  // rows the tile owns
+  const uint32_t a_off = uint32_t(tid / A_ROW_CH) * uint32_t(lda_b) + (tid % A_ROW_CH) * 16;
+  const uint32_t b_off = uint32_t(tid / B_ROW_CH) * uint32_t(ldb_b) + (tid % B_ROW_CH) * 16;
+  const int a_kb0 = (tid % A_ROW_CH) * 16;  // the thread's k byte within a tile
+  const int b_kb0 = (tid % B_ROW_CH) * 16;  // B_KMAJOR: likewise
   int ld_kb = 0;  // k byte offset of the tile the next load_global() fetches
 
   // Loads the next tile in sequence and advances the source pointers.
   auto load_global = [&]() {
+    if constexpr (EDGE) {
+      const auto a_buf = buffer_of(a_tile, int64_t(a_rows - 1) * lda_b + (k_bytes - ld_kb));
+      const bool a_in = ld_kb + a_kb0 < k_bytes;
 #pragma unroll
-    for (int i = 0; i < A_CH; i++) {
-      if (EDGE) {
-        a_reg[i] = v4i{0, 0, 0, 0};
-        if (i * A_ROWS_PER_I < a_rows_left && ld_kb + a_kb0 < k_bytes) a_reg[i] = *(const v4i *)(a_src + i * a_step_i);
-      } else {
-        a_reg[i] = *(const v4i *)(a_src + i * a_step_i);
-      }
-    }
+      for (int i = 0; i < A_CH; i++)
+        a_reg[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(
+                                               a_buf, a_in ? a_off + i * uint32_t(a_step_i) : OUT_OF_RANGE, 0, 0));
+      if constexpr (B_KMAJOR) {
+        const auto b_buf = buffer_of(b_tile, int64_t(b_rows - 1) * ldb_b + (k_bytes - ld_kb));
+        const bool b_in = ld_kb + b_kb0 < k_bytes;
 #pragma unroll
-    for (int i = 0; i < B_CH; i++) {
-      if (EDGE) {
-        b_reg[i] = v4i{0, 0, 0, 0};
-        const bool in_b = B_KMAJOR ? (i * B_ROWS_PER_I < b_rows_left && ld_kb + b_kb0 < k_bytes)
-                                   : (b_cols_left > 0 && ld_kb / ES + b_k0 + i * B_ROWS_PER_I < int(g.k));
-        if (in_b) b_reg[i] = *(const v4i *)(b_src + i * b_step_i);
+        for (int i = 0; i < B_CH; i++)
+          b_reg[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(
+                                                 b_buf, b_in ? b_off + i * uint32_t(b_step_i) : OUT_OF_RANGE, 0, 0));
       } else {
-        b_reg[i] = *(const v4i *)(b_src + i * b_step_i);
+        // k rows left from this tile's first on, the last of them as wide as what is left of N.
+        const auto b_buf = buffer_of(b_tile, (int64_t(g.k) - ld_kb / ES - 1) * ldb_b + (int64_t(g.n) - n0) * ES);
+#pragma unroll
+        for (int i = 0; i < B_CH; i++)
+          b_reg[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(
+                                                 b_buf, b_off + i * uint32_t(b_step_i), 0, 0));
       }
+      a_tile += BKB;
+      b_tile += b_step_kt;
+    } else {
+#pragma unroll
+      for (int i = 0; i < A_CH; i++) a_reg[i] = *(const v4i *)(a_src + i * a_step_i);
+#pragma unroll
+      for (int i = 0; i < B_CH; i++) b_reg[i] = *(const v4i *)(b_src + i * b_step_i);
+      a_src += BKB;
+      b_src += b_step_kt;
     }
-    a_src += BKB;
-    b_src += b_step_kt;
     ld_kb += BKB;
+  };
+  // Steps one tile back, so that the next load_global() fetches the same tile again.
+  auto rewind = [&]() {
+    if constexpr (EDGE) a_tile -= BKB, b_tile -= b_step_kt;
+    else a_src -= BKB, b_src -= b_step_kt;
+    ld_kb -= BKB;
   };
   auto store_lds = [&](int stage) {
     uint8_t *base = lds + stage * STAGE;
@@ -396,7 +441,7 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
   // and MFMA issue that the text below spells out.
   load_global();
   store_lds(0);
-  if (kt_count < 2) a_src -= BKB, b_src -= b_step_kt, ld_kb -= BKB;
+  if (kt_count < 2) rewind();
   load_global();
   __syncthreads();
   read_frags(0, 0, 0);
@@ -404,7 +449,7 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
   for (int kt = 0; kt < kt_count; kt++) {
     const int cur = kt & 1;
     // Tile kt+2 is loaded next (or the last tile again when there is none).
-    if (kt + 2 >= kt_count) a_src -= BKB, b_src -= b_step_kt, ld_kb -= BKB;
+    if (kt + 2 >= kt_count) rewind();
 #pragma unroll
     for (int s = 0; s < SLABS; s++) {
       if (s + 1 < SLABS) read_frags(cur, s + 1, (s + 1) & 1);
@@ -428,11 +473,18 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
                                                      int(g.m - m0), int(g.n - n0));
 }
 
+// Whether the 32-bit offsets of the EDGE kernels reach every row of a tile.
+inline bool edge_addressable(const GemmArgs &g, int elem_size) {
+  return g.lda * elem_size < EDGE_MAX_ROW_BYTES && g.ldb * elem_size < EDGE_MAX_ROW_BYTES &&
+         g.ldc * 4 < EDGE_MAX_ROW_BYTES;
+}
+
 template <class T, bool A_UNSIGNED, class TL, bool EDGE, bool B_KMAJOR = false>
 hipError_t launch(const GemmArgs &g, hipStream_t stream) {
   auto kern = k_gemm<T, A_UNSIGNED, TL, EDGE, B_KMAJOR>;
   constexpr int BM = TL::BM, BN = TL::BN;
   constexpr int STAGE = TL::template stage<T>();
+  if (EDGE && !edge_addressable(g, T::ES)) return hipErrorInvalidValue;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void *)kern,

@@ -15,12 +15,13 @@ typedef Tile<256, 256, 64, 2, 4> T256x256k64;
 typedef Tile<256, 128, 64, 2, 2> T256x128k64;
 typedef Tile<128, 256, 64, 2, 2> T128x256k64;
 typedef Tile<128, 128, 64, 2, 2> T128x128k64;
+typedef Tile<64, 64, 64, 2, 2> T64x64k64;
 
 struct Entry {
   uint32_t tile_m, tile_n, k_bytes;
 };
 // k_bytes is the k step in bytes of an operand row: 128 = 128 i8, 64 bf16 or 32 f32 elements.
-const Entry kSchedules[] = {{256, 256, 128}, {256, 256, 64}, {256, 128, 64}, {128, 256, 64}, {128, 128, 64}};
+const Entry kSchedules[] = {{256, 256, 128}, {256, 256, 64}, {256, 128, 64}, {128, 256, 64}, {128, 128, 64}, {64, 64, 64}};
 
 template <class TL>
 hipError_t launch_kind(const GemmArgs &g, int kind, hipStream_t stream) {
@@ -46,12 +47,12 @@ hipError_t launch_gemm_scheduled(const GemmArgs &g, int kind, uint32_t tile_m, u
                                  uint32_t split_k, hipStream_t stream) {
   const uint32_t k_bytes = split_k * (kind == 2 ? 2 : kind == 3 ? 4 : 1);
   if (tile_m == 256 && tile_n == 256 && k_bytes == 128)
-    return kind == 3 ? launch_gemm_f32(g, stream)
-                     : kind == 2 ? launch_gemm_bf16(g, stream) : launch_gemm_i8(g, kind == 1, stream);
+    return launch_gemm_big(g, kind, stream);
   if (tile_m == 256 && tile_n == 256 && k_bytes == 64) return launch_kind<T256x256k64>(g, kind, stream);
   if (tile_m == 256 && tile_n == 128 && k_bytes == 64) return launch_kind<T256x128k64>(g, kind, stream);
   if (tile_m == 128 && tile_n == 256 && k_bytes == 64) return launch_kind<T128x256k64>(g, kind, stream);
   if (tile_m == 128 && tile_n == 128 && k_bytes == 64) return launch_kind<T128x128k64>(g, kind, stream);
+  if (tile_m == 64 && tile_n == 64 && k_bytes == 64) return launch_kind<T64x64k64>(g, kind, stream);
   return hipErrorInvalidValue;
 }
 

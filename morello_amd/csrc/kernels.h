@@ -54,14 +54,17 @@ struct GemmArgs {
   bool b_kmajor = false;
 };
 // kind: 0 = i8 x i8, 1 = u8 x i8, 2 = bf16 x bf16, 3 = f32 x f32; B stored k-fastest (gemm_nt.hip).
-hipError_t launch_gemm_nt(const GemmArgs &g, int kind, hipStream_t stream);
-// u8|i8 x i8 -> i32, bf16 x bf16 -> f32, f32 x f32 -> f32.
-bool gemm_i8_applicable(const GemmArgs &g);
-hipError_t launch_gemm_i8(const GemmArgs &g, bool a_unsigned, hipStream_t stream);
-bool gemm_f32_applicable(const GemmArgs &g);
-hipError_t launch_gemm_f32(const GemmArgs &g, hipStream_t stream);
-bool gemm_bf16_applicable(const GemmArgs &g);
-hipError_t launch_gemm_bf16(const GemmArgs &g, hipStream_t stream);
+// tile: 64, 128 or 256 (square workgroup tiles).
+hipError_t launch_gemm_nt(const GemmArgs &g, int kind, uint32_t tile, hipStream_t stream);
+// kind: 0 = i8 x i8 -> i32, 1 = u8 x i8 -> i32, 2 = bf16 x bf16 -> f32, 3 = f32 x f32 -> f32.
+// Shapes, leading dimensions and alignment the kernel can walk.
+bool gemm_possible(const GemmArgs &g, int kind);
+// Whether the matrix-core kernel is the faster choice for this size (else the generic kernel).
+bool gemm_pays(const GemmArgs &g, int kind);
+// Tile chosen by size: 256 x 256 with enough tiles to occupy the chip, else 128 x 128 or 64 x 64.
+hipError_t launch_gemm(const GemmArgs &g, int kind, hipStream_t stream);
+// Always the 256 x 256 tile, 128 bytes of K per step.
+hipError_t launch_gemm_big(const GemmArgs &g, int kind, hipStream_t stream);
 
 // ---- gemm_sched.hip: the same kernel under a caller-chosen tile_out / split schedule -----
 uint32_t gemm_schedule_count();

@@ -26,7 +26,7 @@ def int_inputs(seed, dts, b, m, k, n, accum):
 
 @pytest.mark.parametrize("dts", [(M.u8, M.i8, M.i32), (M.i8, M.i8, M.i32)])
 @pytest.mark.parametrize("shape,accum", [
-    ((1, 64, 64, 64), False),       # below the MFMA tile: generic kernel
+    ((1, 64, 64, 64), False),       # one 64 x 64 tile
     ((1, 256, 128, 256), False),    # exactly one MFMA tile, one k step
     ((1, 256, 256, 256), True),
     ((1, 512, 384, 768), False),    # several tiles, odd tile counts
@@ -182,6 +182,36 @@ def test_matmul_with_k_fastest_b(gpu, dts, codes, shape, accum):
         assert rel_err(got, want) < 1e-5
 
 
+@pytest.mark.parametrize("b_k_fastest", [False, True])
+@pytest.mark.parametrize("dts,codes", [((M.u8, M.i8, M.i32), [0, 1, 5]), ((M.i8, M.i8, M.i32), [1, 1, 5]),
+                                        ((M.bf16, M.bf16, M.f32), [7, 7, 6]), ((M.f32, M.f32, M.f32), [6, 6, 6])])
+@pytest.mark.parametrize("shape,accum", [
+    ((1, 1, 256, 512), False),      # a single row: the 64 x 64 tile with 63 rows out of range
+    ((1, 16, 64, 16), True),        # less than one small tile in every direction
+    ((3, 40, 48, 80), True),
+    ((1, 768, 64, 704), False),     # 132 tiles of 64 x 64
+    ((2, 1500, 32, 1296), True),    # int8 / bf16: 128 x 128 tiles (1008 small ones would be too many)
+    ((1, 2900, 48, 2832), False),   # 144 tiles of 256 x 256, ragged on both borders and in K
+    ((1, 3840, 32, 3600), True),    # 225 tiles: the 256 x 256 tile for f32 too
+])
+def test_matmul_every_tile_choice(gpu, dts, codes, shape, accum, b_k_fastest):
+    """The library picks the workgroup tile (64, 128 or 256 square) from the problem size; each
+    choice, with B stored n-fastest and k-fastest, against the oracle."""
+    b, m, k, n = shape
+    gen = {M.u8: synth.uniform_u8, M.i8: synth.uniform_i8, M.bf16: synth.normal_bf16, M.f32: synth.uniform_f32}
+    A, Bm = gen[dts[0]](73, 0, (b, m, k)), gen[dts[1]](73, 1, (b, k, n))
+    out_np = np.int32 if dts[2] == M.i32 else np.float32
+    C0 = (synth.uniform_u8(73, 2, (b, m, n)).astype(out_np) if accum else np.zeros((b, m, n), out_np))
+    layouts = [None, M.batched_col_major([b, k, n]), None] if b_k_fastest else None
+    Bbuf = np.ascontiguousarray(Bm.transpose(0, 2, 1)) if b_k_fastest else Bm
+    got = run_spec(M.Matmul(shape, dts, layouts=layouts, accum=accum), [A, Bbuf, C0])
+    want = orc.matmul(list(shape), codes, A, Bm, C0.copy(), accum)
+    if dts[2] == M.i32:
+        assert np.array_equal(got, want)
+    else:
+        assert rel_err(got, want) < 1e-5
+
+
 @pytest.mark.parametrize("dts,codes", [((M.f32, M.bf16, M.f32), [6, 7, 6]), ((M.bf16, M.f32, M.f32), [7, 6, 6])])
 def test_mixed_bf16_f32_matmul(gpu, dts, codes):
     """One bf16 and one f32 input with an f32 output: both are taken to f32 before the product,
@@ -320,7 +350,7 @@ def test_manual_schedules_give_identical_results(gpu):
         assert rel_err(fb[2].to_numpy(np.float32, (b, m, n)), want) < 1e-5, (tm, tn, sk)
     # a schedule that is not built, and a Spec without a matrix-core kernel
     with pytest.raises(M.MorelloError) as e:
-        spec.tile_out([1, 64, 64]).split(32).run_device([x.ptr for x in bufs])
+        spec.tile_out([1, 32, 32]).split(32).run_device([x.ptr for x in bufs])
     assert e.value.status == 1
     assert M.Matmul([1, 64, 64, 64], [M.u32] * 3).available_schedules() == []
 
