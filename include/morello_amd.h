@@ -195,7 +195,11 @@ size_t mrl_spec_workspace_bytes(const mrl_spec *spec);
  * returns after the work has finished. */
 int mrl_run(const mrl_spec *spec, void *const *params);
 
-/* As mrl_run but only enqueues on `stream` (a hipStream_t, NULL = default stream). */
+/* As mrl_run but only enqueues on `stream` (a hipStream_t, NULL = default stream).  Scratch
+ * memory of up to 64 MiB per call (relayout staging, padded operands) comes from an arena the
+ * library keeps per stream it has seen; calls from several host threads onto one stream take
+ * turns for it.  mrl_stream_destroy releases the arena of its stream; the arena of a stream
+ * the caller created itself stays until the process ends. */
 int mrl_run_async(const mrl_spec *spec, void *const *params, void *stream);
 
 /* Literal stand-in for calling the emitted kernel from the emitted main
@@ -237,7 +241,7 @@ typedef struct {
 } mrl_matmul_schedule;
 
 /* Lists the schedules the matrix-core Matmul kernel is built for, for this Spec's dtypes
- * (u8|i8 x i8 -> i32, bf16 x bf16 -> f32).  Writes up to `cap` entries, returns how many
+ * (u8|i8 x i8 -> i32, bf16 x bf16 -> f32, f32 x f32 -> f32).  Writes up to `cap` entries, returns how many
  * exist (0 if the Spec has no matrix-core kernel). */
 uint32_t mrl_matmul_schedules(const mrl_spec *spec, mrl_matmul_schedule *out, uint32_t cap);
 
@@ -330,7 +334,8 @@ int mrl_memcpy_d2h(void *dst, const void *src, size_t bytes);
 int mrl_memset(void *dst, int value, size_t bytes);
 int mrl_device_synchronize(void);
 /* HIP streams (default priority) for callers that have no HIP binding of their own: the
- * handle is what mrl_run_async, mrl_run_compose and the per-kind conveniences take. */
+ * handle is what mrl_run_async, mrl_run_compose and the per-kind conveniences take.
+ * mrl_stream_destroy waits for the stream's work, then frees the stream and its scratch arena. */
 int mrl_stream_create(void **stream);
 int mrl_stream_synchronize(void *stream);
 int mrl_stream_destroy(void *stream);

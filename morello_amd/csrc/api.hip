@@ -6,6 +6,9 @@
 
 #include <cstdio>
 #include <cstring>
+#include <map>
+#include <memory>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -219,17 +222,75 @@ struct Prepared {
   uint32_t elem = 0;
 };
 
+// Scratch memory of one call.  Small requests are carved out of an arena that stays allocated
+// per stream (work on a stream runs in order, so the next call may overwrite what this one
+// staged): hipMallocAsync / hipFreeAsync cost several microseconds of host time apiece, more
+// than the kernels of a small Spec.  A call holds its stream's arena until it returns, so host
+// threads that share a stream take turns.  Requests that do not fit come from the stream-ordered
+// allocator.
+constexpr size_t ARENA_BYTES = size_t(64) << 20;
+struct Arena {
+  std::mutex in_use;
+  void *base = nullptr;
+};
+std::mutex g_arenas_mutex;
+std::map<hipStream_t, std::unique_ptr<Arena>> g_arenas;
+
+Arena *arena_of(hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(g_arenas_mutex);
+  std::unique_ptr<Arena> &slot = g_arenas[stream];
+  if (!slot) slot.reset(new Arena);
+  return slot.get();
+}
+
+// Frees the arena of a stream whose work has completed.
+void drop_arena(hipStream_t stream) {
+  std::unique_ptr<Arena> arena;
+  {
+    std::lock_guard<std::mutex> lock(g_arenas_mutex);
+    auto it = g_arenas.find(stream);
+    if (it == g_arenas.end()) return;
+    arena = std::move(it->second);
+    g_arenas.erase(it);
+  }
+  std::lock_guard<std::mutex> lock(arena->in_use);
+  if (arena->base) (void)hipFree(arena->base);
+}
+
 struct Workspace {
   hipStream_t stream;
   std::vector<void *> allocs;
+  Arena *arena = nullptr;  // locked while non-null
+  size_t arena_used = 0;
   explicit Workspace(hipStream_t s) : stream(s) {}
+  Workspace(const Workspace &) = delete;
+  Workspace &operator=(const Workspace &) = delete;
   hipError_t alloc(void **p, size_t bytes) {
+    const size_t rounded = (bytes + 255) & ~size_t(255);
+    if (rounded <= ARENA_BYTES - arena_used) {
+      if (!arena) {
+        arena = arena_of(stream);
+        arena->in_use.lock();
+        if (!arena->base) {
+          hipError_t e = hipMalloc(&arena->base, ARENA_BYTES);
+          if (e != hipSuccess) {
+            arena->in_use.unlock();
+            arena = nullptr;
+            return e;
+          }
+        }
+      }
+      *p = static_cast<uint8_t *>(arena->base) + arena_used;
+      arena_used += rounded ? rounded : 256;
+      return hipSuccess;
+    }
     hipError_t e = hipMallocAsync(p, bytes ? bytes : 4, stream);
     if (e == hipSuccess) allocs.push_back(*p);
     return e;
   }
   ~Workspace() {
     for (void *p : allocs) (void)hipFreeAsync(p, stream);
+    if (arena) arena->in_use.unlock();
   }
 };
 
@@ -319,9 +380,6 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
     b_ok = g.b_kmajor = as_rows(bt, &g.ldb, &g.sb);
   }
   bool rows = as_rows(a.t, &g.lda, &g.sa) && b_ok && as_rows(c.t, &g.ldc, &g.sc);
-  // Operands the matrix-core kernels cannot walk in place (A or C stored column-major, say)
-  // are brought to row-major with the strided Move first when that opens the fast path: two
-  // extra passes over one operand against a generic kernel that is tens of times slower.
   mrl::Strided c_user = c.t;
   bool c_densified = false;
   // -1: no matrix-core kernel for these dtypes.
@@ -330,25 +388,51 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
                    : (da == MRL_BF16 && db == MRL_BF16 && dc == MRL_F32) ? 2
                    : (da == MRL_F32 && db == MRL_F32 && dc == MRL_F32)   ? 3
                                                                          : -1;
+  // Operands the matrix-core kernels cannot walk in place are copied with the strided Move
+  // first when that opens the fast path: A or C stored column-major becomes row-major, and rows
+  // that are not whole 16-byte chunks (K or N not a multiple of 16 bytes) are padded with zeros
+  // to the next chunk.  Two extra passes over an operand against a generic kernel that is tens
+  // of times slower.
   const bool worth_two_more_passes = double(g.m) * g.n * g.k * g.batch >= 256.0 * 256 * 256;
-  if (!rows && !sched && kind >= 0 && g.m >= 64 && g.n >= 64 && g.k >= 64 && worth_two_more_passes) {
-    auto densify = [&](Prepared &p, bool read) -> int {
+  if (!sched && kind >= 0 && worth_two_more_passes) {
+    const int64_t per16 = 16 / int64_t(a.elem);
+    auto walkable = [&](const mrl::Strided &t) {
       int64_t ld, bs;
-      if (as_rows(p.t, &ld, &bs)) return MRL_OK;
+      return as_rows(t, &ld, &bs) && ld % per16 == 0 && bs % per16 == 0;
+    };
+    auto densify = [&](Prepared &p, bool read, bool pad) -> int {
       mrl::Strided dense = p.t;
-      HIP_TRY(ws.alloc(&dense.ptr, p.count * p.elem));
-      dense.stride[2] = 1, dense.stride[1] = p.t.shape[2], dense.stride[0] = int64_t(p.t.shape[1]) * p.t.shape[2];
-      if (read) HIP_TRY(mrl::launch_move_strided(p.t, dense, ws.stream));
+      const int64_t cols = p.t.shape[2], ld = pad ? (cols + per16 - 1) / per16 * per16 : cols;
+      dense.stride[2] = 1, dense.stride[1] = ld, dense.stride[0] = int64_t(p.t.shape[1]) * ld;
+      const size_t bytes = size_t(p.t.shape[0]) * dense.stride[0] * p.elem;
+      HIP_TRY(ws.alloc(&dense.ptr, bytes));
+      int64_t old_ld, old_bs;
+      if (read && as_rows(p.t, &old_ld, &old_bs)) {  // rows stay rows: one pass, padding included
+        HIP_TRY(mrl::launch_pad_rows(p.t, dense.ptr, uint32_t(ld), p.elem, ws.stream));
+      } else if (read) {
+        if (ld != cols) HIP_TRY(mrl::launch_fill_zero(dense.ptr, bytes, ws.stream));
+        HIP_TRY(mrl::launch_move_strided(p.t, dense, ws.stream));
+      }
       p.t = dense;
       return MRL_OK;
     };
-    if ((rc = densify(a, true)) != MRL_OK) return rc;
-    if (!b_ok && (rc = densify(b, true)) != MRL_OK) return rc;
+    if (!walkable(a.t) && (rc = densify(a, true, true)) != MRL_OK) return rc;
+    bool b_walkable = walkable(b.t);
+    if (!b_walkable) {
+      mrl::Strided bt = b.t;  // [b, n, k] view: B with k fastest needs whole chunks along K
+      std::swap(bt.shape[1], bt.shape[2]);
+      std::swap(bt.stride[1], bt.stride[2]);
+      b_walkable = walkable(bt);
+    }
+    if (!b_walkable) {
+      if ((rc = densify(b, true, true)) != MRL_OK) return rc;
+      g.b_kmajor = false;
+    }
     int64_t ld, bs;
     c_densified = !as_rows(c.t, &ld, &bs);
-    if ((rc = densify(c, s.accum != 0)) != MRL_OK) return rc;
+    if (c_densified && (rc = densify(c, s.accum != 0, false)) != MRL_OK) return rc;
     g.a = a.t.ptr, g.b = b.t.ptr, g.c = c.t.ptr;
-    if (!b_ok) b_ok = as_rows(b.t, &g.ldb, &g.sb);
+    b_ok = g.b_kmajor || as_rows(b.t, &g.ldb, &g.sb);
     rows = as_rows(a.t, &g.lda, &g.sa) && b_ok && as_rows(c.t, &g.ldc, &g.sc);
   }
   auto finish = [&]() -> int {
@@ -1241,6 +1325,8 @@ int mrl_stream_synchronize(void *stream) {
 
 int mrl_stream_destroy(void *stream) {
   if (!stream) return MRL_ERR_NULL;
+  HIP_TRY(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  drop_arena(static_cast<hipStream_t>(stream));
   HIP_TRY(hipStreamDestroy(static_cast<hipStream_t>(stream)));
   return MRL_OK;
 }

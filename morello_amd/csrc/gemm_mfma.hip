@@ -17,7 +17,9 @@ bool applicable(const GemmArgs &g, int es) {
   auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
   const int64_t per16 = 16 / es;
   constexpr int BM = TileBig::BM, BN = TileBig::BN;
-  return g.m >= 1 && g.n >= 1 && g.k >= 1 && (g.b_kmajor || g.n % per16 == 0) && g.k % per16 == 0 &&
+  // K and N themselves may be anything: a row's bytes from its end to its leading dimension are
+  // read along with it, and are zeros wherever the caller padded the row.
+  return g.m >= 1 && g.n >= 1 && g.k >= 1 &&
          g.lda % per16 == 0 && g.ldb % per16 == 0 && g.sa % per16 == 0 && g.sb % per16 == 0 &&
          al16(g.a) && al16(g.b) && (reinterpret_cast<uintptr_t>(g.c) & 3) == 0 &&
          g.batch <= 65535 && uint64_t((g.m + BM - 1) / BM) * ((g.n + BN - 1) / BN) < (1u << 30);

@@ -216,11 +216,13 @@ __device__ inline void sched_slots(bool staging) {
 }
 
 // EDGE = false: M, N multiples of the tile and K a multiple of the k step.  EDGE = true: any
-// M, any N and K whose rows are whole 16-byte chunks (leading dimensions below
+// M, N and K, with leading dimensions that are whole 16-byte chunks (and below
 // EDGE_MAX_ROW_BYTES); chunks past the last row or past K are fed as zeros and stores outside
 // C are dropped, both by the range check of buffer loads and stores, so the k loop and the
-// epilogue stay free of branches.  Chunks to the right of B's last column hold whatever
-// follows in memory: they only reach columns of C that are not stored.
+// epilogue stay free of branches.  A chunk that straddles the end of K brings along the bytes
+// between the row's end and its leading dimension: the caller keeps those zero (they are its
+// own padding whenever K is not a whole number of chunks).  Chunks to the right of B's last
+// column hold whatever follows in memory: they only reach columns of C that are not stored.
 // B_KMAJOR: B is stored with k fastest (each of its n rows runs along K, `ldb` elements apart:
 // Morello's col_major / batched_col_major layouts, or layout![0,2,1]).  Its tile is then staged
 // and read exactly like A's, and no transposing read is involved.
@@ -343,22 +345,22 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
   // Loads the next tile in sequence and advances the source pointers.
   auto load_global = [&]() {
     if constexpr (EDGE) {
-      const auto a_buf = buffer_of(a_tile, int64_t(a_rows - 1) * lda_b + (k_bytes - ld_kb));
+      const auto a_buf = buffer_of(a_tile, int64_t(a_rows) * lda_b - ld_kb);
       const bool a_in = ld_kb + a_kb0 < k_bytes;
 #pragma unroll
       for (int i = 0; i < A_CH; i++)
         a_reg[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(
                                                a_buf, a_in ? a_off + i * uint32_t(a_step_i) : OUT_OF_RANGE, 0, 0));
       if constexpr (B_KMAJOR) {
-        const auto b_buf = buffer_of(b_tile, int64_t(b_rows - 1) * ldb_b + (k_bytes - ld_kb));
+        const auto b_buf = buffer_of(b_tile, int64_t(b_rows) * ldb_b - ld_kb);
         const bool b_in = ld_kb + b_kb0 < k_bytes;
 #pragma unroll
         for (int i = 0; i < B_CH; i++)
           b_reg[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(
                                                  b_buf, b_in ? b_off + i * uint32_t(b_step_i) : OUT_OF_RANGE, 0, 0));
       } else {
-        // k rows left from this tile's first on, the last of them as wide as what is left of N.
-        const auto b_buf = buffer_of(b_tile, (int64_t(g.k) - ld_kb / ES - 1) * ldb_b + (int64_t(g.n) - n0) * ES);
+        // k rows left from this tile's first on, each up to its leading dimension.
+        const auto b_buf = buffer_of(b_tile, (int64_t(g.k) - ld_kb / ES) * ldb_b - n0 * ES);
 #pragma unroll
         for (int i = 0; i < B_CH; i++)
           b_reg[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(

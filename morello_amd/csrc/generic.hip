@@ -6,6 +6,7 @@
 // 547-569, 603-643): both inputs are converted to the output dtype, then multiplied and
 // accumulated in that dtype.  Integer outputs are computed modulo 2^32 and truncated on
 // store, which equals wrapping arithmetic in the narrower type.
+#include <algorithm>
 #include <utility>
 
 #include "kernels.h"
@@ -217,6 +218,29 @@ __global__ __launch_bounds__(256) void k_widen_bf16(const uint16_t *__restrict__
   const uint64_t step = uint64_t(gridDim.x) * blockDim.x;
   for (uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += step)
     dst[i] = uint32_t(src[i]) << 16;
+}
+
+// Copies [batch][rows][cols] with contiguous rows into rows of `dst_ld` elements (a whole number
+// of dwords), writing zeros from the end of each row to its leading dimension.  One thread per
+// destination dword, assembled from element-sized loads (the source rows need not be aligned
+// beyond their element size).
+template <class E>
+__global__ __launch_bounds__(256) void k_pad_rows(const E *__restrict__ src, uint32_t *__restrict__ dst,
+                                                  uint32_t rows, uint32_t cols, int64_t src_batch,
+                                                  int64_t src_ld, uint32_t dst_ld, uint64_t dwords) {
+  constexpr uint32_t PER = 4 / sizeof(E);
+  const uint32_t row_dwords = dst_ld / PER;
+  const uint64_t step = uint64_t(gridDim.x) * blockDim.x;
+  for (uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < dwords; i += step) {
+    const uint64_t line = i / row_dwords;
+    const uint32_t col0 = uint32_t(i % row_dwords) * PER;
+    const E *from = src + int64_t(line / rows) * src_batch + int64_t(line % rows) * src_ld;
+    uint32_t word = 0;
+#pragma unroll
+    for (uint32_t e = 0; e < PER; e++)
+      if (col0 + e < cols) word |= uint32_t(from[col0 + e]) << (8 * sizeof(E) * e);
+    dst[i] = word;
+  }
 }
 
 __global__ void k_copy1(const uint8_t *src, uint8_t *dst, uint64_t bytes) {
@@ -505,6 +529,30 @@ hipError_t launch_move_strided(const Strided &src, const Strided &dst, hipStream
     if (int(d) != dim_s && int(d) != dim_d) blocks *= p.shape[d];
   if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
   hipLaunchKernelGGL(k_move_tiled, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+  return hipGetLastError();
+}
+
+hipError_t launch_pad_rows(const Strided &src, void *dst, uint32_t dst_ld, uint32_t elem_size,
+                           hipStream_t stream) {
+  if (src.rank != 3 || (src.shape[2] != 1 && src.stride[2] != 1) || dst_ld * elem_size % 4 != 0 ||
+      dst_ld < src.shape[2])
+    return hipErrorInvalidValue;
+  const uint32_t batch = src.shape[0], rows = src.shape[1], cols = src.shape[2];
+  const uint64_t dwords = uint64_t(batch) * rows * (dst_ld * elem_size / 4);
+  if (dwords == 0) return hipSuccess;
+  const uint32_t blocks = uint32_t(std::min<uint64_t>((dwords + 255) / 256, 65536));
+  const int64_t sb = batch == 1 ? 0 : src.stride[0], sl = rows == 1 ? 0 : src.stride[1];
+  if (elem_size == 1)
+    hipLaunchKernelGGL(k_pad_rows<uint8_t>, dim3(blocks), dim3(256), 0, stream, (const uint8_t *)src.ptr,
+                       (uint32_t *)dst, rows, cols, sb, sl, dst_ld, dwords);
+  else if (elem_size == 2)
+    hipLaunchKernelGGL(k_pad_rows<uint16_t>, dim3(blocks), dim3(256), 0, stream, (const uint16_t *)src.ptr,
+                       (uint32_t *)dst, rows, cols, sb, sl, dst_ld, dwords);
+  else if (elem_size == 4)
+    hipLaunchKernelGGL(k_pad_rows<uint32_t>, dim3(blocks), dim3(256), 0, stream, (const uint32_t *)src.ptr,
+                       (uint32_t *)dst, rows, cols, sb, sl, dst_ld, dwords);
+  else
+    return hipErrorInvalidValue;
   return hipGetLastError();
 }
 

@@ -34,6 +34,10 @@ hipError_t launch_move_generic(const void *src, void *dst, const LayoutEval &src
 // Move between two layouts that are permutations of the logical dims (strides in elements):
 // coalesced on both sides, through an LDS transpose when their contiguous dims differ.
 hipError_t launch_move_strided(const Strided &src, const Strided &dst, hipStream_t stream);
+// Copy of a [batch][rows][cols] tensor with contiguous rows into dense rows of `dst_ld` elements
+// (a whole number of dwords), zeros from each row's end to `dst_ld`.
+hipError_t launch_pad_rows(const Strided &src, void *dst, uint32_t dst_ld, uint32_t elem_size,
+                           hipStream_t stream);
 // bf16 -> f32 of a whole buffer, position by position.
 hipError_t launch_widen_bf16(const void *src, void *dst, uint64_t count, hipStream_t stream);
 // Move Spec fast path: same bytes on both sides (16-byte aligned buffers).

@@ -193,6 +193,9 @@ def test_matmul_with_k_fastest_b(gpu, dts, codes, shape, accum):
     ((2, 1500, 32, 1296), True),    # int8 / bf16: 128 x 128 tiles (1008 small ones would be too many)
     ((1, 2900, 48, 2832), False),   # 144 tiles of 256 x 256, ragged on both borders and in K
     ((1, 3840, 32, 3600), True),    # 225 tiles: the 256 x 256 tile for f32 too
+    ((2, 333, 77, 515), True),      # rows that are not whole 16-byte chunks: zero-padded copies
+    ((1, 1000, 1001, 999), False),
+    ((1, 1, 4099, 4101), True),
 ])
 def test_matmul_every_tile_choice(gpu, dts, codes, shape, accum, b_k_fastest):
     """The library picks the workgroup tile (64, 128 or 256 square) from the problem size; each
