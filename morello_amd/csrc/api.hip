@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
+#include <algorithm>
 #include <cstring>
 #include <map>
 #include <memory>
@@ -476,12 +477,28 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
   cv.accum = s.accum;
   const int di = s.dtypes[0], df = s.dtypes[1], dout = s.dtypes[2];
   const bool fast_types = (di == MRL_U8 || di == MRL_I8) && df == MRL_I8 && dout == MRL_I32;
-  // Tensors in another permutation layout (NCHW, say) are moved to channels-last when the
-  // shape suits the matrix-core kernel: three small extra passes against a generic kernel
+  const bool fused_shape = fast_types && cv.f == 64 && cv.c % 64 == 0 &&
+                           (cv.fh * cv.fw * (cv.c / 64) == 1 || cv.fh * cv.fw * (cv.c / 64) == 9);
+  // Matmul kind of the same dtypes (-1: none): any other shape runs as unfold + Matmul.
+  const int kind = (di == MRL_I8 && df == MRL_I8 && dout == MRL_I32)       ? 0
+                   : (di == MRL_U8 && df == MRL_I8 && dout == MRL_I32)     ? 1
+                   : (di == MRL_BF16 && df == MRL_BF16 && dout == MRL_F32) ? 2
+                   : (di == MRL_F32 && df == MRL_F32 && dout == MRL_F32)   ? 3
+                                                                           : -1;
+  const uint64_t pixels = uint64_t(cv.oh) * cv.ow, window = uint64_t(cv.fh) * cv.fw * cv.c;
+  const int64_t per16 = 16 / int64_t(img.elem);
+  const uint64_t row_elems = (window + per16 - 1) / per16 * per16;  // a window, padded to whole chunks
+  // Windows of this many images are unfolded at a time.
+  constexpr uint64_t UNFOLD_BYTES = uint64_t(1) << 30;
+  const uint64_t image_rows_bytes = pixels * row_elems * img.elem;
+  const bool as_matmul = !fused_shape && kind >= 0 && image_rows_bytes <= UNFOLD_BYTES && window < (1u << 24) &&
+                         double(cv.b) * pixels * cv.f * window >= 1e6;
+  // Tensors in another permutation layout (NCHW, say) are moved to channels-last when a
+  // matrix-core path takes the shape: three small extra passes against a generic kernel
   // that is hundreds of times slower.
   const mrl::Strided out_user = out.t;
   bool out_moved = false;
-  if (fast_types && cv.f == 64 && cv.c % 64 == 0 && (cv.fh * cv.fw * (cv.c / 64) == 1 || cv.fh * cv.fw * (cv.c / 64) == 9)) {
+  if (fused_shape || as_matmul) {
     auto to_channels_last = [&](Prepared &p, bool read) -> int {
       if (channels_last(p.t)) return MRL_OK;
       mrl::Strided dense = p.t;
@@ -501,6 +518,44 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
   if (fast_types && channels_last(img.t) && channels_last(filt.t) && channels_last(out.t) &&
       mrl::conv_i8_applicable(cv)) {
     HIP_TRY(mrl::launch_conv_i8(cv, di == MRL_U8, ws.stream));
+  } else if (as_matmul && (reinterpret_cast<uintptr_t>(img.t.ptr) & 15) == 0 &&
+             (reinterpret_cast<uintptr_t>(filt.t.ptr) & 15) == 0 && (reinterpret_cast<uintptr_t>(out.t.ptr) & 3) == 0) {
+    // Filters in KRSC order are the B operand stored k-fastest; their rows padded like U's.
+    const void *weights = filt.t.ptr;
+    if (row_elems != window) {
+      void *padded = nullptr;
+      HIP_TRY(ws.alloc(&padded, size_t(cv.f) * row_elems * filt.elem));
+      mrl::Strided flat;
+      flat.ptr = filt.t.ptr, flat.dtype = filt.t.dtype, flat.rank = 3;
+      flat.shape[0] = 1, flat.shape[1] = cv.f, flat.shape[2] = uint32_t(window);
+      flat.stride[0] = 0, flat.stride[1] = int64_t(window), flat.stride[2] = 1;
+      HIP_TRY(mrl::launch_pad_rows(flat, padded, uint32_t(row_elems), filt.elem, ws.stream));
+      weights = padded;
+    }
+    // A 1x1 filter over whole chunks of channels: the image is U already.
+    const bool in_place = cv.fh == 1 && cv.fw == 1 && row_elems == window;
+    const uint32_t per_pass = uint32_t(std::min<uint64_t>(cv.b, std::max<uint64_t>(1, UNFOLD_BYTES / image_rows_bytes)));
+    void *rows_buf = nullptr;
+    if (!in_place) HIP_TRY(ws.alloc(&rows_buf, size_t(per_pass) * image_rows_bytes));
+    const uint64_t image_bytes = uint64_t(cv.oh + cv.fh - 1) * (cv.ow + cv.fw - 1) * cv.c * img.elem;
+    for (uint32_t b0 = 0; b0 < cv.b; b0 += per_pass) {
+      const uint32_t nb = std::min(per_pass, cv.b - b0);
+      const uint8_t *images = static_cast<const uint8_t *>(img.t.ptr) + b0 * image_bytes;
+      if (!in_place)
+        HIP_TRY(mrl::launch_unfold(images, rows_buf, nb, cv.c, cv.oh, cv.ow, cv.fh, cv.fw, uint32_t(row_elems),
+                                   img.elem, ws.stream));
+      mrl::GemmArgs g;
+      g.a = in_place ? static_cast<const void *>(images) : rows_buf;
+      g.b = weights;
+      g.c = static_cast<uint8_t *>(out.t.ptr) + uint64_t(b0) * pixels * cv.f * out.elem;
+      g.batch = 1, g.m = uint32_t(nb * pixels), g.n = cv.f, g.k = uint32_t(window);
+      g.lda = g.ldb = int64_t(row_elems), g.ldc = cv.f;
+      g.sa = g.sb = g.sc = 0;
+      g.accum = s.accum;
+      g.b_kmajor = true;
+      if (!mrl::gemm_possible(g, kind)) return MRL_ERR_UNSUPPORTED;  // ruled out by the checks above
+      HIP_TRY(mrl::launch_gemm(g, kind, ws.stream));
+    }
   } else {
     HIP_TRY(mrl::launch_conv_generic(img.t, filt.t, out.t, s.accum, ws.stream));
   }

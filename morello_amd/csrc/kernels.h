@@ -87,6 +87,13 @@ struct ConvArgs {
 bool conv_i8_applicable(const ConvArgs &c);
 hipError_t launch_conv_i8(const ConvArgs &c, bool img_unsigned, hipStream_t stream);
 
+// ---- unfold.hip: the windows of a channels-last image as rows, for Conv as a Matmul ---------
+// image: [batch][oh+fh-1][ow+fw-1][c]; rows: [batch*oh*ow][row_elems], each row the fh*fw*c
+// elements of one window in (r, s, c) order followed by zeros.
+hipError_t launch_unfold(const void *image, void *rows, uint32_t batch, uint32_t c, uint32_t oh,
+                         uint32_t ow, uint32_t fh, uint32_t fw, uint32_t row_elems,
+                         uint32_t elem_size, hipStream_t stream);
+
 // ---- softmax.hip: f32 softmax over a contiguous innermost scan dim ---------------------
 hipError_t launch_softmax_rows(const float *in, float *out, uint64_t rows, uint32_t cols,
                                hipStream_t stream);

@@ -70,6 +70,71 @@ def test_conv_nchw_layout_on_the_matrix_cores(gpu, accum):
     assert np.array_equal(got, want)
 
 
+CONV_GEN = {M.u8: synth.uniform_u8, M.i8: synth.uniform_i8, M.bf16: synth.normal_bf16, M.f32: synth.uniform_f32}
+
+
+@pytest.mark.parametrize("dts,codes", [((M.u8, M.i8, M.i32), [0, 1, 5]), ((M.i8, M.i8, M.i32), [1, 1, 5]),
+                                        ((M.bf16, M.bf16, M.f32), [7, 7, 6]), ((M.f32, M.f32, M.f32), [6, 6, 6])])
+@pytest.mark.parametrize("shape,accum", [
+    ((2, 48, 24, 20, 17, 3, 3), True),     # window of 216 elements: rows padded to whole chunks
+    ((1, 32, 3, 40, 40, 7, 7), False),     # three channels: the window is gathered element by element
+    ((3, 128, 128, 9, 9, 1, 1), True),     # 1x1 filter: the image is the left operand as it lies
+    ((2, 64, 32, 12, 12, 5, 5), False),    # 64 filters but not the fused kernel's channel count
+    ((1, 7, 20, 30, 30, 2, 4), True),      # few filters, uneven window
+    ((5, 96, 64, 14, 14, 3, 3), False),    # 64 channels but not the fused kernel's filter count
+])
+def test_conv_as_matmul(gpu, dts, codes, shape, accum):
+    """Shapes outside the fused kernel's (64 filters, channels in 64s, 1x1 or 3x3) are unfolded into
+    rows of windows and run as a Matmul on the matrix cores, for every dtype triple those take."""
+    b, f, c, oh, ow, fh, fw = shape
+    img = CONV_GEN[dts[0]](131, 0, (b, oh + fh - 1, ow + fw - 1, c))
+    filt = CONV_GEN[dts[1]](131, 1, (f, fh, fw, c))
+    out_np = np.int32 if dts[2] == M.i32 else np.float32
+    out0 = synth.uniform_u8(131, 2, (b, oh, ow, f)).astype(out_np) if accum else np.zeros((b, oh, ow, f), out_np)
+    got = run_spec(M.Conv(shape, dts, accum=accum), [img, filt, out0.copy()])
+    want = orc.conv(list(shape), codes, img, filt, out0.copy(), accum, layouts=[NHWC] * 3)
+    if dts[2] == M.i32:
+        assert np.array_equal(got, want)
+    else:
+        err = float(np.abs(got.astype(np.float64) - want).max() / np.abs(want).max())
+        assert err < 1e-5
+
+
+def test_conv_as_matmul_from_nchw(gpu):
+    """Row-major (NCHW / FCRS) tensors at a shape the unfolded path takes: moved to channels-last
+    and back around it."""
+    shape = (2, 40, 12, 18, 21, 3, 2)
+    b, f, c, oh, ow, fh, fw = shape
+    img = synth.uniform_u8(132, 0, (b, c, oh + fh - 1, ow + fw - 1))
+    filt = synth.uniform_i8(132, 1, (f, c, fh, fw))
+    out0 = synth.uniform_u8(132, 2, (b, f, oh, ow)).astype(np.int32)
+    rm = [M.row_major(s) for s in M.Conv(shape, (M.u8, M.i8, M.i32)).parameter_shapes()]
+    got = run_spec(M.Conv(shape, (M.u8, M.i8, M.i32), layouts=rm, accum=True), [img, filt, out0.copy()])
+    assert np.array_equal(got, orc.conv(list(shape), [0, 1, 5], img, filt, out0.copy(), True))
+
+
+def test_conv_as_matmul_in_several_passes(gpu):
+    """More windows than one pass unfolds (1 GiB of rows): the batch is cut into passes.  Checked
+    on the first and last image and through the per-image checksum."""
+    # 62 500 windows of 1024 bytes per image: 16 images per pass, so passes of 16, 16 and 4
+    b, f, c, oh, ow, fh, fw = shape = (36, 8, 64, 250, 250, 4, 4)
+    img = synth.uniform_u8(133, 0, (b, oh + fh - 1, ow + fw - 1, c))
+    filt = synth.uniform_i8(133, 1, (f, fh, fw, c))
+    got = run_spec(M.Conv(shape, (M.u8, M.i8, M.i32)), [img, filt, np.zeros((b, oh, ow, f), np.int32)])
+    for bi in (0, 16, 35):
+        sub = (1,) + shape[1:]
+        want = orc.conv(list(sub), [0, 1, 5], img[bi:bi + 1], filt, np.zeros((1, oh, ow, f), np.int32), layouts=[NHWC] * 3)
+        assert np.array_equal(got[bi:bi + 1], want)
+    fsum = filt.astype(np.int64).sum(axis=0)  # [r,s,c]
+    for bi in range(b):
+        im = img[bi].astype(np.int64)
+        total = 0
+        for r in range(fh):
+            for s in range(fw):
+                total += int((im[r:r + oh, s:s + ow, :].sum(axis=(0, 1)) * fsum[r, s]).sum())
+        assert int(got[bi].astype(np.int64).sum()) == total
+
+
 def test_conv_full_size_properties(gpu):
     """benchmark configuration 4 (32x56x56x64 -> 64, 3x3): a few images against the oracle, every
     image through a checksum (sum over filters and pixels, computed in int64 from box sums),
