@@ -605,10 +605,41 @@ int run_compose_msm(const mrl_spec &s, void *const *params, Workspace &ws) {
                               (b == 1 || kt.stride[0] == int64_t(k) * n2);
     mrl::AttnArgs at;
     at.q = q.ptr, at.kt = kt.ptr, at.v = v.ptr, at.out = (float *)out.ptr;
-    at.b = b, at.m = m, at.k = k, at.n2 = n2, at.n = n;
-    if (dense_row_major(q) && dense_row_major(v) && dense_row_major(out) && kt_k_fastest && mrl::attn_applicable(at)) {
+    at.b = b, at.m = m, at.k = k, at.n2 = n2, at.n = n, at.n_out = n;
+    const bool fusable_layouts = dense_row_major(q) && dense_row_major(v) && dense_row_major(out) && kt_k_fastest;
+    if (fusable_layouts && mrl::attn_applicable(at)) {
       HIP_TRY(mrl::launch_attn(at, ws.stream));
       return MRL_OK;
+    }
+    // Other head dims up to 128 (and different ones for the two products): Q, K and V rows are
+    // padded with zeros to the next head dim the kernel is built for.  Zero columns of Q and K add
+    // nothing to the scores, zero columns of V give result columns that are not stored.
+    const uint32_t widest = std::max(k, n), dp = widest <= 32 ? 32 : widest <= 64 ? 64 : 128;
+    if (fusable_layouts && widest <= 128 && (reinterpret_cast<uintptr_t>(out.ptr) & 3) == 0) {
+      auto padded = [&](const mrl::Strided &src, uint32_t rows, uint32_t cols, const void **dst) -> int {
+        if (cols == dp && (reinterpret_cast<uintptr_t>(src.ptr) & 15) == 0) {
+          *dst = src.ptr;
+          return MRL_OK;
+        }
+        void *buf = nullptr;
+        HIP_TRY(ws.alloc(&buf, size_t(b) * rows * dp * 2));
+        mrl::Strided flat;
+        flat.ptr = src.ptr, flat.dtype = MRL_BF16, flat.rank = 3;
+        flat.shape[0] = 1, flat.shape[1] = b * rows, flat.shape[2] = cols;
+        flat.stride[0] = 0, flat.stride[1] = cols, flat.stride[2] = 1;
+        HIP_TRY(mrl::launch_pad_rows(flat, buf, dp, 2, ws.stream));
+        *dst = buf;
+        return MRL_OK;
+      };
+      int rc;
+      if ((rc = padded(q, m, k, &at.q)) != MRL_OK) return rc;
+      if ((rc = padded(kt, n2, k, &at.kt)) != MRL_OK) return rc;
+      if ((rc = padded(v, n2, n, &at.v)) != MRL_OK) return rc;
+      at.k = at.n = dp;
+      if (mrl::attn_applicable(at)) {
+        HIP_TRY(mrl::launch_attn(at, ws.stream));
+        return MRL_OK;
+      }
     }
   }
   // Staged path, as the reference schedules it (examples/matmul_chain.rs:60-81): S and P

@@ -37,13 +37,25 @@ typedef __attribute__((address_space(3))) v4s lds_v4s;
 typedef __attribute__((address_space(3))) void lds_void;
 typedef __attribute__((address_space(1))) const void global_cvoid;
 
-constexpr int D = 128;        // head dim of both products (k and n of the Compose)
 constexpr int BQ = 128;       // queries per workgroup (4 query groups x 32)
 constexpr int BKV = 64;       // keys per block
-constexpr int ROW = D * 2;    // bytes per K or V row
-constexpr int TILE = BKV * ROW;           // 16 KiB: one K or V block
-constexpr int STAGE = 2 * TILE;           // K block then V block
-constexpr int HALF = 2 * STAGE;           // two stages per key half
+// Sizes that follow from the head dim D (k and n of the Compose; 32, 64 or 128).
+template <int D>
+struct Dims {
+  static constexpr int ROW = D * 2;             // bytes per K or V row
+  static constexpr int TILE = BKV * ROW;        // one K or V block (16 KiB at D = 128)
+  static constexpr int STAGE = 2 * TILE;        // K block then V block
+  static constexpr int HALF = 2 * STAGE;        // two stages per key half
+  static constexpr int CHUNKS = ROW / 16;       // 16-byte chunks per row
+  static constexpr int UNITS = ROW / 64;        // 64-byte units per row
+  static constexpr int ROWS_PER_LINE = ROW >= 256 ? 1 : 256 / ROW;  // rows per 256-byte bank line
+  static constexpr int ROWS_PER_LOAD = 1024 / ROW;  // rows one direct-to-LDS instruction fills
+  static constexpr int LDS_BYTES = 2 * HALF > 4 * (D / 2 + 2) * 64 * 4 ? 2 * HALF : 4 * (D / 2 + 2) * 64 * 4;
+  // Rows that one operand read touches at the same chunk index lie 256 bytes apart or closer;
+  // XOR-ing the chunk (K) or the 64-byte unit (V) with the row's bank-line index spreads them.
+  __device__ static constexpr int k_swizzle(int row) { return (row / ROWS_PER_LINE) & (CHUNKS - 1); }
+  __device__ static constexpr int v_swizzle(int row) { return (row / ROWS_PER_LINE) & (UNITS - 1); }
+};
 constexpr float LOG2E = 1.44269504088896340736f;
 constexpr float RESCALE_SLACK = 5.0f;  // e^5 = 148
 
@@ -56,8 +68,10 @@ __device__ inline v2i read_tr16(const uint8_t *p) {
 // a clamped (valid) row and not stored; the key blocks are dealt ceil/floor to the two halves,
 // loads past the end of K / V are clamped to the entry's last 16 bytes (finite data, weighted
 // by exp(-inf) = 0), and the scores of keys past n2 are set to -inf before the softmax.
-template <bool RAGGED>
+template <int D, bool RAGGED>
 __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
+  typedef Dims<D> DD;
+  constexpr int ROW = DD::ROW, TILE = DD::TILE, STAGE = DD::STAGE, HALF = DD::HALF;
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -90,17 +104,19 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
 #pragma unroll
   for (int s = 0; s < D / 16; s++) qf[s] = *(const v4i *)(Q + s * 32 + lg * 16);
 
-  // Block staging.  One direct-to-LDS instruction fills 1 KiB = 4 rows; lane l lands in
-  // 16-byte slot l.  K rows are XOR-swizzled by chunk with (row & 15), V rows by 64-byte
-  // unit with (row & 3); each lane fetches the global chunk that belongs in its slot.
-  // The 4 waves of a key half share its 16 + 16 instructions per block.
-  const int ld_row = lane >> 4, ld_pc = lane & 15;
-  uint32_t k_src[4], v_src[4];
+  // Block staging.  One direct-to-LDS instruction fills 1 KiB (4 rows at D = 128); lane l lands
+  // in 16-byte slot l.  K rows are XOR-swizzled by chunk, V rows by 64-byte unit; each lane
+  // fetches the global chunk that belongs in its slot.  The 4 waves of a key half share its
+  // instructions: PER_WAVE for K and as many for V per block and wave.
+  constexpr int PER_WAVE = TILE / 1024 / 4;
+  static_assert(PER_WAVE == D / 32, "one staging pair per batch of S MFMAs");
+  const int ld_row = lane / DD::CHUNKS, ld_pc = lane % DD::CHUNKS;
+  uint32_t k_src[PER_WAVE], v_src[PER_WAVE];
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const int q = qg * 4 + i, row = q * 4 + ld_row;
-    k_src[i] = row * ROW + ((ld_pc ^ (row & 15)) << 4);
-    v_src[i] = row * ROW + ((((ld_pc >> 2) ^ (row & 3)) << 6) | ((ld_pc & 3) << 4));
+  for (int i = 0; i < PER_WAVE; i++) {
+    const int q = qg * PER_WAVE + i, row = q * DD::ROWS_PER_LOAD + ld_row;
+    k_src[i] = row * ROW + ((ld_pc ^ DD::k_swizzle(row)) << 4);
+    v_src[i] = row * ROW + ((((ld_pc >> 2) ^ DD::v_swizzle(row)) << 6) | ((ld_pc & 3) << 4));
   }
   // Byte offset within the batch entry's K (V) of this lane's chunk i of block kb.
   auto k_off = [&](int kb, int i) {
@@ -113,8 +129,8 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
   };
   auto load_block = [&](int kb, int stage) {
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int q = qg * 4 + i;
+    for (int i = 0; i < PER_WAVE; i++) {
+      const int q = qg * PER_WAVE + i;
       __builtin_amdgcn_global_load_lds((global_cvoid *)(K + k_off(kb, i)),
                                        (lds_void *)(my_lds + stage * STAGE + q * 1024), 16, 0, 0);
       __builtin_amdgcn_global_load_lds((global_cvoid *)(V + v_off(kb, i)),
@@ -149,7 +165,7 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
     const int next_kb = min(kb + 1, nblocks - 1);
     uint8_t *next_lds = my_lds + (stage ^ 1) * STAGE;
     auto load_pair = [&](int i) {
-      const int q = qg * 4 + i;
+      const int q = qg * PER_WAVE + i;
       __builtin_amdgcn_global_load_lds((global_cvoid *)(K + k_off(next_kb, i)), (lds_void *)(next_lds + q * 1024), 16, 0, 0);
       __builtin_amdgcn_global_load_lds((global_cvoid *)(V + v_off(next_kb, i)), (lds_void *)(next_lds + TILE + q * 1024), 16, 0, 0);
     };
@@ -167,7 +183,7 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
 #pragma unroll
         for (int kt = 0; kt < BKV / 32; kt++) {
           const int row = kt * 32 + lq, st = 2 * q + c;
-          kf[buf][kt][c] = *(const v4i *)(lk + row * ROW + (((2 * st + lg) ^ (row & 15)) << 4));
+          kf[buf][kt][c] = *(const v4i *)(lk + row * ROW + (((2 * st + lg) ^ DD::k_swizzle(row)) << 4));
         }
     };
 #pragma unroll
@@ -175,7 +191,7 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; r++) s[kt][r] = 0.0f;
     read_k(0, 0);
-    read_k(1, 1);
+    if (D / 32 > 1) read_k(1, 1);
 #pragma unroll
     for (int q = 0; q < D / 32; q++) {
       if (q + 2 < D / 32) read_k(q + 2, (q + 2) % 3);
@@ -187,7 +203,7 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
           s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, kf[q % 3][kt][c]),
                                                           __builtin_bit_cast(v8bf, qf[2 * q + c]), s[kt], 0, 0, 0);
     }
-    __builtin_amdgcn_sched_group_barrier(0x100, 4 * (BKV / 32), 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, (D / 32 > 1 ? 4 : 2) * (BKV / 32), 0);
 #pragma unroll
     for (int q = 0; q < D / 32; q++) {
       if (q + 2 < D / 32) __builtin_amdgcn_sched_group_barrier(0x100, 2 * (BKV / 32), 0);
@@ -200,10 +216,10 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
     v4i vf[BKV / 16][D / 32];
 #pragma unroll
     for (int u = 0; u < BKV / 16; u++) {
-      const int key = 16 * u + 4 * lg + v_rl;  // key & 3 == v_rl
+      const int key = 16 * u + 4 * lg + v_rl;  // key & 3 == v_rl; key + 8 swizzles alike
 #pragma unroll
       for (int t = 0; t < D / 32; t++) {
-        const int off = ((t ^ v_rl) << 6) + v_within;
+        const int off = ((t ^ DD::v_swizzle(key)) << 6) + v_within;
         const v2i lo = read_tr16(lv + key * ROW + off);
         const v2i hi = read_tr16(lv + (key + 8) * ROW + off);
         vf[u][t] = v4i{lo[0], lo[1], hi[0], hi[1]};
@@ -268,23 +284,24 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
   // that owns the same queries.  Layout [value][lane] keeps lanes on distinct banks.
   float l_tot = l_run + __shfl_xor(l_run, 32);
   __syncthreads();  // all K/V reads are done: the staging area is free
-  float *mbuf = (float *)lds + qg * (66 * 64);
+  float *mbuf = (float *)lds + qg * ((D / 2 + 2) * 64);
   if (half == 1) {
 #pragma unroll
     for (int t = 0; t < D / 32; t++)
 #pragma unroll
       for (int r = 0; r < 16; r++) mbuf[(t * 16 + r) * 64 + lane] = o[t][r];
-    mbuf[64 * 64 + lane] = m_run;
-    mbuf[65 * 64 + lane] = l_tot;
+    mbuf[(D / 2) * 64 + lane] = m_run;
+    mbuf[(D / 2 + 1) * 64 + lane] = l_tot;
   }
   __syncthreads();
   if (half == 0) {
-    const float m1 = mbuf[64 * 64 + lane], l1 = mbuf[65 * 64 + lane];
+    const float m1 = mbuf[(D / 2) * 64 + lane], l1 = mbuf[(D / 2 + 1) * 64 + lane];
     const float m = fmaxf(m_run, m1);
     const float a0 = __builtin_amdgcn_exp2f((m_run - m) * LOG2E), a1 = __builtin_amdgcn_exp2f((m1 - m) * LOG2E);
     const float inv = 1.0f / (l_tot * a0 + l1 * a1);
     const float w0 = a0 * inv, w1 = a1 * inv;
-    float *out = p.out + (head * p.m + q0 + lq) * int64_t(D);
+    float *out = p.out + (head * p.m + q0 + lq) * int64_t(p.n_out);
+    const bool whole_rows = p.n_out == D;  // else: padded head dim, columns past n_out are dropped
     if (!RAGGED || q0 + lq < int(p.m))
 #pragma unroll
     for (int t = 0; t < D / 32; t++)
@@ -295,7 +312,15 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
         v.y = o[t][4 * a + 1] * w0 + mbuf[(t * 16 + 4 * a + 1) * 64 + lane] * w1;
         v.z = o[t][4 * a + 2] * w0 + mbuf[(t * 16 + 4 * a + 2) * 64 + lane] * w1;
         v.w = o[t][4 * a + 3] * w0 + mbuf[(t * 16 + 4 * a + 3) * 64 + lane] * w1;
-        *(float4 *)(out + t * 32 + 8 * a + 4 * lg) = v;
+        const int col = t * 32 + 8 * a + 4 * lg;
+        if (whole_rows) {
+          *(float4 *)(out + col) = v;
+        } else {
+          if (col + 0 < int(p.n_out)) out[col + 0] = v.x;
+          if (col + 1 < int(p.n_out)) out[col + 1] = v.y;
+          if (col + 2 < int(p.n_out)) out[col + 2] = v.z;
+          if (col + 3 < int(p.n_out)) out[col + 3] = v.w;
+        }
       }
   }
 }
@@ -304,23 +329,37 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
 
 bool attn_applicable(const AttnArgs &a) {
   auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-  return a.k == D && a.n == D && a.m && a.n2 && a.b && uint64_t(a.n2) * ROW < (1ull << 31) &&
-         uint64_t((a.m + BQ - 1) / BQ) * a.b < (1u << 31) && al16(a.q) && al16(a.kt) && al16(a.v) && al16(a.out);
+  return a.k == a.n && (a.k == 32 || a.k == 64 || a.k == 128) && a.n_out >= 1 && a.n_out <= a.n && a.m && a.n2 && a.b &&
+         uint64_t(a.n2) * a.k * 2 < (1ull << 31) && uint64_t((a.m + BQ - 1) / BQ) * a.b < (1u << 31) &&
+         al16(a.q) && al16(a.kt) && al16(a.v) && al16(a.out);
 }
 
-hipError_t launch_attn(const AttnArgs &a, hipStream_t stream) {
+namespace {
+template <int D>
+hipError_t launch_for(const AttnArgs &a, hipStream_t stream) {
+  constexpr int LDS = Dims<D>::LDS_BYTES;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void *)k_attn<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * HALF);
+    hipError_t e = hipFuncSetAttribute((const void *)k_attn<D, false>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
     if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void *)k_attn<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * HALF);
+      e = hipFuncSetAttribute((const void *)k_attn<D, true>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
     if (e != hipSuccess) return e;
     attr_set = true;
   }
   const dim3 grid(((a.m + BQ - 1) / BQ) * a.b);
-  if (a.m % BQ == 0 && a.n2 % (2 * BKV) == 0) hipLaunchKernelGGL(k_attn<false>, grid, dim3(512), 2 * HALF, stream, a);
-  else hipLaunchKernelGGL(k_attn<true>, grid, dim3(512), 2 * HALF, stream, a);
+  if (a.m % BQ == 0 && a.n2 % (2 * BKV) == 0) hipLaunchKernelGGL((k_attn<D, false>), grid, dim3(512), LDS, stream, a);
+  else hipLaunchKernelGGL((k_attn<D, true>), grid, dim3(512), LDS, stream, a);
   return hipGetLastError();
+}
+}  // namespace
+
+hipError_t launch_attn(const AttnArgs &a, hipStream_t stream) {
+  if (!attn_applicable(a)) return hipErrorInvalidValue;
+  switch (a.k) {
+    case 32: return launch_for<32>(a, stream);
+    case 64: return launch_for<64>(a, stream);
+    default: return launch_for<128>(a, stream);
+  }
 }
 
 }  // namespace mrl

@@ -122,8 +122,11 @@ struct AttnArgs {
   const void *q;   // [b, m, k]   bf16 row-major
   const void *kt;  // logical [b, k, n2] stored as [b, n2, k] (K row-major)
   const void *v;   // [b, n2, n]  bf16 row-major
-  float *out;      // [b, m, n]   f32 row-major
+  float *out;      // [b, m, n_out] f32 row-major
   uint32_t b, m, k, n2, n;
+  // Columns of the result that exist in `out` (its rows are n_out floats): n, or fewer when V
+  // was padded with zero columns up to a head dim the kernel is built for.
+  uint32_t n_out;
 };
 bool attn_applicable(const AttnArgs &a);
 hipError_t launch_attn(const AttnArgs &a, hipStream_t stream);

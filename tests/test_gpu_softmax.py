@@ -56,7 +56,8 @@ KT_ORC = orc.make_layout([0, 2, 1])
 
 
 @pytest.mark.parametrize("dims", [(1, 64, 128, 64, 128), (2, 256, 128, 512, 128), (1, 128, 64, 256, 64),
-                                  (3, 50, 24, 70, 10), (1, 2048, 128, 2048, 128)])
+                                  (3, 50, 24, 70, 10), (1, 2048, 128, 2048, 128), (2, 256, 64, 512, 64),
+                                  (4, 128, 32, 256, 32), (2, 1024, 64, 1024, 64)])
 def test_compose_msm(gpu, dims):
     b, m, k, n2, n = dims
     q, kmat, v = msm_inputs(301, *dims)
@@ -67,10 +68,9 @@ def test_compose_msm(gpu, dims):
     assert rel_err(got, want) < 1e-2  # stated tolerance for the composed pipeline
 
 
-@pytest.mark.parametrize("dims", [(2, 200, 64, 328, 64), (1, 136, 96, 1000, 96), (2, 256, 96, 192, 72)])
+@pytest.mark.parametrize("dims", [(2, 200, 160, 328, 160), (1, 136, 136, 1000, 96), (2, 256, 192, 192, 72)])
 def test_compose_msm_staged_on_the_matrix_cores(gpu, dims):
-    """Shapes the fused kernel does not take (ragged sequence lengths, head dims other than
-    128): Q.KT runs as a bf16 Matmul with a k-fastest B, softmax over f32 rows, and P.V as an
+    """Head dims beyond 128, which the fused kernel does not take: Q.KT runs as a bf16 Matmul with a k-fastest B, softmax over f32 rows, and P.V as an
     f32 Matmul after widening V.  f32 intermediates: within 1e-5 of the oracle."""
     b, m, k, n2, n = dims
     q, kmat, v = msm_inputs(303, *dims)
@@ -83,7 +83,10 @@ def test_compose_msm_staged_on_the_matrix_cores(gpu, dims):
 
 @pytest.mark.parametrize("dims", [(1, 136, 128, 1000, 128), (2, 1, 128, 1, 128), (1, 130, 128, 64, 128),
                                   (3, 200, 128, 70, 128), (1, 128, 128, 2049, 128), (2, 300, 128, 129, 128),
-                                  (1, 257, 128, 65, 128), (2, 384, 128, 192, 128)])
+                                  (1, 257, 128, 65, 128), (2, 384, 128, 192, 128),
+                                  (1, 136, 64, 1000, 64), (2, 1, 64, 1, 64), (2, 200, 64, 328, 64),
+                                  (1, 257, 64, 65, 64), (3, 200, 32, 70, 32), (2, 300, 32, 129, 32),
+                                  (1, 1, 32, 2049, 32)])
 def test_compose_msm_fused_ragged(gpu, dims):
     """Sequence lengths that are not multiples of the fused kernel's blocks (128 queries,
     2 x 64 keys): clamped rows, masked keys, uneven split of the key blocks over the two
@@ -105,6 +108,22 @@ def test_compose_msm_fused_ragged(gpu, dims):
                       [v, q, kmat, np.zeros((b, m, n), np.float32)])
     assert rel_err(staged, want) < 1e-5
     assert rel_err(got, staged) < 1e-2
+
+
+@pytest.mark.parametrize("dims", [(2, 200, 48, 328, 48), (1, 136, 96, 1000, 96), (2, 256, 96, 192, 72),
+                                  (1, 128, 64, 256, 128), (3, 50, 24, 70, 10), (1, 77, 100, 130, 30),
+                                  (2, 128, 128, 256, 2), (1, 64, 8, 64, 128)])
+def test_compose_msm_fused_with_padded_head_dims(gpu, dims):
+    """Head dims up to 128 other than 32 / 64 / 128, and different ones for the two products: Q, K
+    and V are zero-padded to the next size the fused kernel is built for and only the n real
+    columns of the result are stored (the buffer is exactly b x m x n)."""
+    b, m, k, n2, n = dims
+    q, kmat, v = msm_inputs(305, *dims)
+    spec = M.ComposeMSM(b, m, k, n2, n, layouts=[None, None, KT_LAYOUT, None])
+    got = run_spec(spec, [v, q, kmat, np.full((b, m, n), 7.5, np.float32)])
+    want = orc.compose_msm(b, m, k, n2, n, [7, 7, 7, 6], v, q, kmat, np.zeros((b, m, n), np.float32),
+                           layouts=[None, None, KT_ORC, None])
+    assert rel_err(got, want) < 1e-2
 
 
 def test_compose_msm_row_major_kt_and_f32_inputs(gpu):
