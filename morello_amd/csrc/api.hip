@@ -14,6 +14,7 @@
 #include <vector>
 
 #include "kernels.h"
+#include "layout_factor.h"
 
 namespace {
 
@@ -219,6 +220,7 @@ struct Prepared {
   void *user = nullptr;
   mrl::LayoutEval user_layout;  // valid when staged
   mrl::LayoutEval dense_layout;
+  mrl_layout user_desc, dense_desc;  // the same two as descriptors
   uint64_t count = 0;
   uint32_t elem = 0;
 };
@@ -295,6 +297,23 @@ struct Workspace {
   }
 };
 
+// Same dtype, between the caller's layout of parameter `p` and its dense staging copy (to_dense:
+// caller's -> dense): as a strided permutation of the two layouts' common view when they have
+// one (Packed and OddEven dims are digits of their logical index), else by index arithmetic
+// per element.
+int relayout(const void *src, void *dst, bool to_dense, const Prepared &p, Workspace &ws) {
+  const mrl_layout &from = to_dense ? p.user_desc : p.dense_desc, &to = to_dense ? p.dense_desc : p.user_desc;
+  std::vector<mrl::MoveDim> view;
+  if (mrl::common_view(from, to, p.t.shape, p.t.rank, &view)) {
+    const hipError_t e = mrl::launch_move_view(src, p.t.dtype, dst, p.t.dtype, view.data(), uint32_t(view.size()), ws.stream);
+    if (e == hipSuccess) return MRL_OK;
+    if (e != hipErrorInvalidValue) HIP_TRY(e);
+  }
+  HIP_TRY(mrl::launch_relayout(src, dst, to_dense ? p.user_layout : p.dense_layout,
+                               to_dense ? p.dense_layout : p.user_layout, p.elem, p.count, ws.stream));
+  return MRL_OK;
+}
+
 int prepare(const mrl_spec &s, uint32_t idx, void *ptr, bool needs_read, Workspace &ws, Prepared *out) {
   uint32_t shape[MRL_MAX_RANK], rank;
   parameter_shape(s, idx, shape, &rank);
@@ -316,17 +335,14 @@ int prepare(const mrl_spec &s, uint32_t idx, void *ptr, bool needs_read, Workspa
   HIP_TRY(ws.alloc(&out->scratch, out->count * out->elem));
   out->t.ptr = out->scratch;
   mrl::layout_strides(dense, shape, rank, out->t.stride);
-  if (needs_read)
-    HIP_TRY(mrl::launch_relayout(ptr, out->scratch, out->user_layout, out->dense_layout, out->elem,
-                                 out->count, ws.stream));
+  out->user_desc = s.layouts[idx], out->dense_desc = dense;
+  if (needs_read) return relayout(ptr, out->scratch, true, *out, ws);
   return MRL_OK;
 }
 
 int finish_output(Prepared &p, Workspace &ws) {
   if (!p.scratch) return MRL_OK;
-  HIP_TRY(mrl::launch_relayout(p.scratch, p.user, p.dense_layout, p.user_layout, p.elem, p.count,
-                               ws.stream));
-  return MRL_OK;
+  return relayout(p.scratch, p.user, false, p, ws);
 }
 
 bool dense_row_major(const mrl::Strided &t) {
@@ -688,13 +704,12 @@ int run_move(const mrl_spec &s, void *const *params, Workspace &ws) {
     HIP_TRY(mrl::launch_copy(params[0], params[1], count * mrl_dtype_size(s.dtypes[0]), ws.stream));
     return MRL_OK;
   }
-  // Both layouts permutations of the logical dims: strided kernels, coalesced on both sides.
-  mrl::Strided st, dt;
-  st.ptr = params[0], st.dtype = s.dtypes[0], st.rank = rank;
-  dt.ptr = params[1], dt.dtype = s.dtypes[1], dt.rank = rank;
-  for (uint32_t d = 0; d < MRL_MAX_RANK; d++) st.shape[d] = dt.shape[d] = d < rank ? shape[d] : 1;
-  if (mrl::layout_strides(li, shape, rank, st.stride) && mrl::layout_strides(lo, shape, rank, dt.stride)) {
-    const hipError_t e = mrl::launch_move_strided(st, dt, ws.stream);
+  // Layouts with a common strided view (permutations of the logical dims; Packed and OddEven
+  // dims whose sizes refine each other): strided kernels, coalesced on both sides.
+  std::vector<mrl::MoveDim> view;
+  if (mrl::common_view(li, lo, shape, rank, &view)) {
+    const hipError_t e = mrl::launch_move_view(params[0], s.dtypes[0], params[1], s.dtypes[1], view.data(),
+                                               uint32_t(view.size()), ws.stream);
     if (e == hipSuccess) return MRL_OK;
     if (e != hipErrorInvalidValue) HIP_TRY(e);
   }

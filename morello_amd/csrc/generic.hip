@@ -7,9 +7,11 @@
 // accumulated in that dtype.  Integer outputs are computed modulo 2^32 and truncated on
 // store, which equals wrapping arithmetic in the narrower type.
 #include <algorithm>
+#include <type_traits>
 #include <utility>
 
 #include "kernels.h"
+#include "layout_factor.h"
 
 namespace mrl {
 namespace {
@@ -139,9 +141,9 @@ struct MoveStrided {
   void *dst;
   int sdt, ddt;
   uint32_t rank;
-  uint32_t shape[MRL_MAX_RANK];
-  int64_t ss[MRL_MAX_RANK], ds[MRL_MAX_RANK];
-  uint32_t order[MRL_MAX_RANK];
+  uint32_t shape[MOVE_MAX_RANK];
+  int64_t ss[MOVE_MAX_RANK], ds[MOVE_MAX_RANK];
+  uint32_t order[MOVE_MAX_RANK];
   uint32_t dim_s, dim_d;      // the dim each side stores contiguously
   uint32_t tiles_s, tiles_d;  // 64-element tiles along them
   uint64_t count;
@@ -160,6 +162,21 @@ __global__ __launch_bounds__(256) void k_move_rows(MoveStrided p) {
     so += int64_t(c) * p.ss[d], d_o += int64_t(c) * p.ds[d];
   }
   store_u32(p.dst, p.ddt, d_o, move_bits(p.src, p.sdt, so, p.ddt));
+}
+
+// The same when nothing is converted and every run along the shared contiguous dim is whole
+// 16-byte vectors on both sides: shapes and strides count vectors.
+__global__ __launch_bounds__(256) void k_move_rows16(MoveStrided p) {
+  const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= p.count) return;
+  uint64_t rem = i;
+  int64_t so = 0, d_o = 0;
+  for (int o = int(p.rank) - 1; o >= 0; o--) {
+    const uint32_t d = p.order[o], c = uint32_t(rem % p.shape[d]);
+    rem /= p.shape[d];
+    so += int64_t(c) * p.ss[d], d_o += int64_t(c) * p.ds[d];
+  }
+  static_cast<uint4 *>(p.dst)[d_o] = static_cast<const uint4 *>(p.src)[so];
 }
 
 // The two sides are contiguous along different dims: a 64 x 64 tile of (dim_d, dim_s) goes
@@ -192,6 +209,83 @@ __global__ __launch_bounds__(256) void k_move_tiled(MoveStrided p) {
   for (uint32_t r = quad; r < 64; r += 4)
     if (s0 + r < ns && d0 + lane < nd)
       store_u32(p.dst, p.ddt, d_o + int64_t(s0 + r) * p.ds[p.dim_s] + int64_t(d0 + lane) * p.ds[p.dim_d], tile[lane][r]);
+}
+
+// Any other pair of contiguous dims (a Packed(8) digit on one side, say, too short for the
+// 64 x 64 transpose): a tile of up to 4096 elements, `ext[d]` along each digit, chosen on the host
+// so that it holds runs of 64 contiguous elements on both sides.  Read in source order into LDS,
+// written in destination order.  Element t of the tile in source order has digit
+// (t / tstride_s[d]) % ext[d] along d, likewise tstride_d in destination order; the divisions are
+// multiplications by precomputed reciprocals (exact for operands below 2^16).
+struct MoveTile {
+  MoveStrided m;
+  uint32_t ext[MOVE_MAX_RANK], chunks[MOVE_MAX_RANK];
+  uint32_t tstride_s[MOVE_MAX_RANK], tstride_d[MOVE_MAX_RANK];
+  uint32_t inv_s[MOVE_MAX_RANK], inv_d[MOVE_MAX_RANK], inv_ext[MOVE_MAX_RANK];  // ceil(2^32 / x)
+  uint32_t tile;  // elements per tile
+};
+constexpr uint32_t MOVE_TILE_MAX = 4096;
+
+__device__ inline uint32_t div_small(uint32_t n, uint32_t d, uint32_t inv) {
+  return d == 1 ? n : __umulhi(n, inv);
+}
+
+// E: the element type when nothing is converted (typed loads and stores), void when the dtypes
+// differ (conversion per element).  Offsets fit 32 bits: a tensor has fewer than 2^31 elements.
+template <class E>
+__global__ __launch_bounds__(256) void k_move_gather(MoveTile p) {
+  constexpr bool CONVERT = std::is_void<E>::value;
+  typedef typename std::conditional<CONVERT, uint32_t, E>::type Cell;
+  __shared__ Cell lds[MOVE_TILE_MAX + MOVE_TILE_MAX / 64];
+  uint64_t blk = blockIdx.x;
+  int64_t base_s = 0, base_d = 0;
+  uint32_t room[MOVE_MAX_RANK];  // how much of each digit is left from this tile's origin on
+#pragma unroll
+  for (uint32_t d = 0; d < MOVE_MAX_RANK; d++) {
+    room[d] = 1;
+    if (d < p.m.rank) {
+      const uint32_t origin = uint32_t(blk % p.chunks[d]) * p.ext[d];
+      blk /= p.chunks[d];
+      room[d] = p.m.shape[d] - origin;
+      base_s += int64_t(origin) * p.m.ss[d], base_d += int64_t(origin) * p.m.ds[d];
+    }
+  }
+#pragma unroll 4
+  for (uint32_t t = threadIdx.x; t < p.tile; t += 256) {
+    uint32_t so = 0;
+    bool inside = true;
+#pragma unroll
+    for (uint32_t d = 0; d < MOVE_MAX_RANK; d++)
+      if (d < p.m.rank && p.ext[d] > 1) {
+        const uint32_t q = div_small(t, p.tstride_s[d], p.inv_s[d]);
+        const uint32_t c = q - div_small(q, p.ext[d], p.inv_ext[d]) * p.ext[d];
+        inside = inside && c < room[d];
+        so += c * uint32_t(p.m.ss[d]);
+      }
+    if (inside) {
+      if constexpr (CONVERT) lds[t + t / 64] = move_bits(p.m.src, p.m.sdt, base_s + so, p.m.ddt);
+      else lds[t + t / 64] = static_cast<const E *>(p.m.src)[base_s + so];
+    }
+  }
+  __syncthreads();
+#pragma unroll 4
+  for (uint32_t t = threadIdx.x; t < p.tile; t += 256) {
+    uint32_t d_o = 0, at = 0;
+    bool inside = true;
+#pragma unroll
+    for (uint32_t d = 0; d < MOVE_MAX_RANK; d++)
+      if (d < p.m.rank && p.ext[d] > 1) {
+        const uint32_t q = div_small(t, p.tstride_d[d], p.inv_d[d]);
+        const uint32_t c = q - div_small(q, p.ext[d], p.inv_ext[d]) * p.ext[d];
+        inside = inside && c < room[d];
+        d_o += c * uint32_t(p.m.ds[d]);
+        at += c * p.tstride_s[d];
+      }
+    if (inside) {
+      if constexpr (CONVERT) store_u32(p.m.dst, p.m.ddt, base_d + d_o, lds[at + at / 64]);
+      else static_cast<E *>(p.m.dst)[base_d + d_o] = lds[at + at / 64];
+    }
+  }
 }
 
 // Four 16-byte vectors per thread in flight, streamed past the caches: 6.5 TB/s on a 256 MiB
@@ -495,41 +589,148 @@ hipError_t launch_copy(const void *src, void *dst, uint64_t bytes, hipStream_t s
   return hipGetLastError();
 }
 
-// Move between two strided layouts of the same logical shape.  Returns hipErrorInvalidValue
-// when the shape does not fit the kernels' index ranges (the caller then takes the generic path).
-hipError_t launch_move_strided(const Strided &src, const Strided &dst, hipStream_t stream) {
+// Move over a common strided view of the two sides (layout_factor.h).  Returns
+// hipErrorInvalidValue when the view does not fit the kernels' index ranges (the caller then
+// takes the generic path).
+hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_dtype,
+                            const MoveDim *dims, uint32_t rank, hipStream_t stream) {
+  if (rank > MOVE_MAX_RANK) return hipErrorInvalidValue;
+  // Elements narrower than 4 bytes that travel together (a digit contiguous on both sides, no
+  // conversion) are moved as 2- or 4-byte units: a Packed(4) digit of bytes becomes one u32.
+  MoveDim wide[MOVE_MAX_RANK];
+  if (src_dtype == dst_dtype && mrl_dtype_size(src_dtype) < 4) {
+    const uint32_t elem = uint32_t(mrl_dtype_size(src_dtype));
+    for (uint32_t unit = 4; unit > elem; unit /= 2) {
+      const uint32_t per = unit / elem;
+      int shared = -1;
+      bool fits = (reinterpret_cast<uintptr_t>(src) % unit) == 0 && (reinterpret_cast<uintptr_t>(dst) % unit) == 0;
+      for (uint32_t d = 0; d < rank; d++)
+        if (dims[d].size > 1 && dims[d].ss == 1 && dims[d].ds == 1) shared = int(d);
+      for (uint32_t d = 0; fits && d < rank; d++)
+        fits = int(d) == shared ? dims[d].size % per == 0 : (dims[d].ss % per == 0 && dims[d].ds % per == 0);
+      if (shared < 0 || !fits) continue;
+      uint32_t n = 0;
+      for (uint32_t d = 0; d < rank; d++) {
+        MoveDim m = dims[d];
+        if (int(d) == shared) m.size /= per;
+        else m.ss /= per, m.ds /= per;
+        if (m.size > 1) wide[n++] = m;
+      }
+      if (n == 0) wide[n++] = {1, 1, 1};
+      dims = wide, rank = n;
+      src_dtype = dst_dtype = unit == 4 ? MRL_U32 : MRL_U16;
+      break;
+    }
+  }
   MoveStrided p;
-  p.src = src.ptr, p.dst = dst.ptr, p.sdt = src.dtype, p.ddt = dst.dtype, p.rank = src.rank;
+  p.src = src, p.dst = dst, p.sdt = src_dtype, p.ddt = dst_dtype, p.rank = rank;
   p.count = 1;
   int dim_s = -1, dim_d = -1;
-  for (uint32_t d = 0; d < MRL_MAX_RANK; d++) {
-    p.shape[d] = d < src.rank ? src.shape[d] : 1;
-    p.ss[d] = d < src.rank ? src.stride[d] : 0;
-    p.ds[d] = d < src.rank ? dst.stride[d] : 0;
+  for (uint32_t d = 0; d < MOVE_MAX_RANK; d++) {
+    p.shape[d] = d < rank ? dims[d].size : 1;
+    p.ss[d] = d < rank ? dims[d].ss : 0;
+    p.ds[d] = d < rank ? dims[d].ds : 0;
     p.count *= p.shape[d];
-    if (d < src.rank && p.shape[d] > 1 && p.ss[d] == 1) dim_s = int(d);
-    if (d < src.rank && p.shape[d] > 1 && p.ds[d] == 1) dim_d = int(d);
+    if (d < rank && p.shape[d] > 1 && p.ss[d] == 1) dim_s = int(d);
+    if (d < rank && p.shape[d] > 1 && p.ds[d] == 1) dim_d = int(d);
   }
   if (p.count == 0) return hipSuccess;
   // Decode order: by decreasing destination stride, the destination's contiguous dim last.
-  for (uint32_t d = 0; d < MRL_MAX_RANK; d++) p.order[d] = d;
+  for (uint32_t d = 0; d < MOVE_MAX_RANK; d++) p.order[d] = d;
   for (uint32_t i = 0; i < p.rank; i++)
     for (uint32_t j = i + 1; j < p.rank; j++)
       if (p.ds[p.order[j]] > p.ds[p.order[i]]) std::swap(p.order[i], p.order[j]);
-  if (dim_s < 0 || dim_d < 0 || dim_s == dim_d) {
+  // A shared contiguous dim serves both sides when its runs are at least 64 bytes long.
+  const bool shared_runs = dim_s >= 0 && dim_s == dim_d &&
+                           (rank == 1 || uint64_t(p.shape[dim_s]) * mrl_dtype_size(src_dtype) >= 64);
+  if (dim_s < 0 || dim_d < 0 || shared_runs) {
+    // Whole 16-byte vectors along the shared dim, everywhere: move vectors, not elements.
+    const int64_t per = 16 / int64_t(mrl_dtype_size(src_dtype));
+    bool vectors = dim_s >= 0 && dim_s == dim_d && src_dtype == dst_dtype && p.shape[dim_s] % per == 0 &&
+                   (reinterpret_cast<uintptr_t>(src) & 15) == 0 && (reinterpret_cast<uintptr_t>(dst) & 15) == 0;
+    for (uint32_t d = 0; vectors && d < rank; d++)
+      vectors = int(d) == dim_s || (p.ss[d] % per == 0 && p.ds[d] % per == 0);
+    if (vectors && rank == 1)
+      return launch_copy(src, dst, p.count * mrl_dtype_size(src_dtype), stream);
+    if (vectors) {
+      for (uint32_t d = 0; d < rank; d++) {
+        if (int(d) == dim_s) p.shape[d] /= uint32_t(per);
+        else p.ss[d] /= per, p.ds[d] /= per;
+      }
+      p.count /= uint64_t(per);
+    }
     const uint64_t blocks = (p.count + 255) / 256;
     if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(k_move_rows, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+    if (vectors) hipLaunchKernelGGL(k_move_rows16, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL(k_move_rows, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
     return hipGetLastError();
   }
-  p.dim_s = uint32_t(dim_s), p.dim_d = uint32_t(dim_d);
-  p.tiles_s = (p.shape[dim_s] + 63) / 64, p.tiles_d = (p.shape[dim_d] + 63) / 64;
-  uint64_t blocks = uint64_t(p.tiles_s) * p.tiles_d;
-  for (uint32_t d = 0; d < p.rank; d++)
-    if (int(d) != dim_s && int(d) != dim_d) blocks *= p.shape[d];
-  if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(k_move_tiled, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+  // Two long contiguous dims: the 64 x 64 transpose.
+  if (dim_s != dim_d && p.shape[dim_s] >= 32 && p.shape[dim_d] >= 32) {
+    p.dim_s = uint32_t(dim_s), p.dim_d = uint32_t(dim_d);
+    p.tiles_s = (p.shape[dim_s] + 63) / 64, p.tiles_d = (p.shape[dim_d] + 63) / 64;
+    uint64_t blocks = uint64_t(p.tiles_s) * p.tiles_d;
+    for (uint32_t d = 0; d < p.rank; d++)
+      if (int(d) != dim_s && int(d) != dim_d) blocks *= p.shape[d];
+    if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(k_move_tiled, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+    return hipGetLastError();
+  }
+  // Otherwise a tile grown digit by digit: along the destination's fastest digits until they
+  // make a run of 64, along the source's fastest until they do, then along the destination's
+  // again while the tile stays within MOVE_TILE_MAX.
+  MoveTile t;
+  t.m = p;
+  uint32_t by_ss[MOVE_MAX_RANK], by_ds[MOVE_MAX_RANK];  // digits, fastest first
+  for (uint32_t d = 0; d < MOVE_MAX_RANK; d++) by_ss[d] = by_ds[d] = d, t.ext[d] = 1;
+  std::sort(by_ss, by_ss + rank, [&](uint32_t x, uint32_t y) { return p.ss[x] < p.ss[y]; });
+  std::sort(by_ds, by_ds + rank, [&](uint32_t x, uint32_t y) { return p.ds[x] < p.ds[y]; });
+  uint32_t tile = 1;
+  auto grow = [&](const uint32_t *order, uint32_t run_target, uint32_t tile_cap) {
+    uint32_t run = 1;
+    for (uint32_t i = 0; i < rank && run < run_target; i++) {
+      const uint32_t d = order[i];
+      run *= t.ext[d];
+      if (t.ext[d] == p.shape[d] || run >= run_target) continue;
+      const uint32_t want = std::min<uint32_t>({p.shape[d] / t.ext[d], (run_target + run - 1) / run,
+                                                std::max<uint32_t>(1, tile_cap / tile)});
+      if (want <= 1) break;
+      tile = tile / t.ext[d] * (t.ext[d] * want), run *= want, t.ext[d] *= want;
+      if (t.ext[d] != p.shape[d]) break;  // a partly covered digit ends the contiguous run
+    }
+  };
+  grow(by_ds, 64, MOVE_TILE_MAX / 64);
+  grow(by_ss, 64, MOVE_TILE_MAX);
+  grow(by_ds, MOVE_TILE_MAX, MOVE_TILE_MAX);
+  t.tile = tile;
+  uint64_t blocks = 1;
+  uint32_t stride_s = 1, stride_d = 1;
+  auto inverse = [](uint32_t x) { return x <= 1 ? 0u : uint32_t(((uint64_t(1) << 32) + x - 1) / x); };
+  for (uint32_t i = 0; i < rank; i++) {
+    t.tstride_s[by_ss[i]] = stride_s, stride_s *= t.ext[by_ss[i]];
+    t.tstride_d[by_ds[i]] = stride_d, stride_d *= t.ext[by_ds[i]];
+  }
+  for (uint32_t d = 0; d < MOVE_MAX_RANK; d++) {
+    if (d >= rank) t.tstride_s[d] = t.tstride_d[d] = 1;
+    t.chunks[d] = d < rank ? (p.shape[d] + t.ext[d] - 1) / t.ext[d] : 1;
+    t.inv_s[d] = inverse(t.tstride_s[d]), t.inv_d[d] = inverse(t.tstride_d[d]), t.inv_ext[d] = inverse(t.ext[d]);
+    blocks *= t.chunks[d];
+  }
+  if (blocks > 0x7fffffffull || tile > MOVE_TILE_MAX) return hipErrorInvalidValue;
+  const dim3 grid{uint32_t(blocks)};
+  const size_t elem = mrl_dtype_size(src_dtype);
+  if (src_dtype != dst_dtype) hipLaunchKernelGGL(k_move_gather<void>, grid, dim3(256), 0, stream, t);
+  else if (elem == 4) hipLaunchKernelGGL(k_move_gather<uint32_t>, grid, dim3(256), 0, stream, t);
+  else if (elem == 2) hipLaunchKernelGGL(k_move_gather<uint16_t>, grid, dim3(256), 0, stream, t);
+  else hipLaunchKernelGGL(k_move_gather<uint8_t>, grid, dim3(256), 0, stream, t);
   return hipGetLastError();
+}
+
+// Move between two strided layouts of the same logical shape.
+hipError_t launch_move_strided(const Strided &src, const Strided &dst, hipStream_t stream) {
+  MoveDim dims[MRL_MAX_RANK];
+  for (uint32_t d = 0; d < src.rank; d++) dims[d] = {src.shape[d], src.stride[d], dst.stride[d]};
+  return launch_move_view(src.ptr, src.dtype, dst.ptr, dst.dtype, dims, src.rank, stream);
 }
 
 hipError_t launch_pad_rows(const Strided &src, void *dst, uint32_t dst_ld, uint32_t elem_size,

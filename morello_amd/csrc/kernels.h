@@ -34,6 +34,10 @@ hipError_t launch_move_generic(const void *src, void *dst, const LayoutEval &src
 // Move between two layouts that are permutations of the logical dims (strides in elements):
 // coalesced on both sides, through an LDS transpose when their contiguous dims differ.
 hipError_t launch_move_strided(const Strided &src, const Strided &dst, hipStream_t stream);
+// The same over a common strided view of two layouts (layout_factor.h): `rank` digits.
+struct MoveDim;
+hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_dtype,
+                            const MoveDim *dims, uint32_t rank, hipStream_t stream);
 // Copy of a [batch][rows][cols] tensor with contiguous rows into dense rows of `dst_ld` elements
 // (a whole number of dwords), zeros from each row's end to `dst_ld`.
 hipError_t launch_pad_rows(const Strided &src, void *dst, uint32_t dst_ld, uint32_t elem_size,
