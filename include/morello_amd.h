@@ -183,8 +183,11 @@ size_t mrl_spec_parameter_bytes(const mrl_spec *spec, uint32_t idx);
 uint64_t mrl_spec_ops(const mrl_spec *spec);
 /* MRL_OK if mrl_run would accept the Spec (validates shapes, dtypes, layouts). */
 int mrl_spec_check(const mrl_spec *spec);
-/* Bytes of device scratch mrl_run allocates internally for this Spec (relayout staging,
- * transposed operands); 0 when the kernels read the parameters in place. */
+/* Bytes of device scratch mrl_run takes for staging this Spec's parameters out of layouts the
+ * kernels do not walk in place (Packed / OddEven dims in another order than row-major); 0 when
+ * every parameter is read in place.  A lower bound on the call's scratch: operand copies made
+ * for speed (zero-padded rows, column-major operands made row-major, unfolded Conv windows, up
+ * to 1 GiB) and the intermediates of a Compose come from the same allocator on top of it. */
 size_t mrl_spec_workspace_bytes(const mrl_spec *spec);
 
 /* -------------------------------------------------------------- execution */

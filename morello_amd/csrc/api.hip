@@ -329,6 +329,14 @@ int prepare(const mrl_spec &s, uint32_t idx, void *ptr, bool needs_read, Workspa
   }
   mrl_layout dense;
   mrl_layout_row_major(shape, rank, &dense);
+  // A layout with Packed dims can still be row-major order (layout![0, 1, 1p16], say).
+  std::vector<mrl::MoveDim> view;
+  if (mrl::common_view(s.layouts[idx], dense, shape, rank, &view) &&
+      (view.empty() || (view.size() == 1 && view[0].ss == 1 && view[0].ds == 1))) {
+    out->t.ptr = ptr;
+    mrl::layout_strides(dense, shape, rank, out->t.stride);
+    return MRL_OK;
+  }
   if (!mrl::make_layout_eval(s.layouts[idx], shape, rank, &out->user_layout) ||
       !mrl::make_layout_eval(dense, shape, rank, &out->dense_layout))
     return MRL_ERR_BAD_LAYOUT;
@@ -1113,8 +1121,14 @@ size_t mrl_spec_workspace_bytes(const mrl_spec *spec) {
     uint32_t shape[MRL_MAX_RANK], rank;
     int64_t strides[MRL_MAX_RANK];
     parameter_shape(*spec, i, shape, &rank);
-    if (!mrl::layout_strides(spec->layouts[i], shape, rank, strides))
-      total += size_t(volume(shape, rank)) * mrl_dtype_size(spec->dtypes[i]);
+    if (mrl::layout_strides(spec->layouts[i], shape, rank, strides)) continue;
+    mrl_layout dense;
+    mrl_layout_row_major(shape, rank, &dense);
+    std::vector<mrl::MoveDim> view;
+    if (mrl::common_view(spec->layouts[i], dense, shape, rank, &view) &&
+        (view.empty() || (view.size() == 1 && view[0].ss == 1 && view[0].ds == 1)))
+      continue;  // Packed dims in row-major order
+    total += size_t(volume(shape, rank)) * mrl_dtype_size(spec->dtypes[i]);
   }
   return total;
 }

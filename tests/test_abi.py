@@ -130,6 +130,9 @@ def test_workspace_only_for_non_strided_layouts():
     packed = M.layout(0, 2, 1, (2, M.Packed(16)))  # examples/matmul_x86.rs:34-53 style relayout
     s = M.Matmul([1, 64, 64, 64], [M.f32] * 3, layouts=[None, packed, None])
     assert s.workspace_bytes() == 64 * 64 * 4
+    # Packed dims that leave the row-major order as it is are read in place.
+    same_order = M.layout(0, 1, 2, (2, M.Packed(16)))
+    assert M.Matmul([1, 64, 64, 64], [M.f32] * 3, layouts=[None, same_order, None]).workspace_bytes() == 0
 
 
 def test_null_and_status_strings():

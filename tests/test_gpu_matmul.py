@@ -298,6 +298,21 @@ def test_matmul_layouts(gpu):
     spec = M.Matmul([b, m, k, n], (M.u8, M.i8, M.i32), layouts=[None, packed, M.col_major([b, m, n])])
     got = run_spec(spec, [A, Bp, np.zeros((b, n, m), np.int32)])
     assert np.array_equal(got.transpose(0, 2, 1), want)
+    # Packed dims that spell row-major order (read in place), on A and on the output
+    same_a, same_c = M.layout(0, 1, 2, (2, M.Packed(16))), M.layout(0, 1, 2, (2, M.Packed(8)))
+    spec = M.Matmul([b, m, k, n], (M.u8, M.i8, M.i32), layouts=[same_a, None, same_c])
+    assert np.array_equal(run_spec(spec, [A, Bm, np.zeros((b, m, n), np.int32)]), want)
+    # OddEven on K of A, Packed on N of B: staged through the layouts' common strided view
+    oe, pk = M.layout(0, 1, 2, (2, M.OddEven(8))), M.layout(0, 1, 2, (1, M.Packed(4)))
+    Ao, Bk = np.zeros(b * m * k, np.uint8), np.zeros(b * k * n, np.int8)
+    for i in range(m):
+        for kk in range(k):
+            Ao[oe.buffer_index([b, m, k], [0, i, kk])] = A[0, i, kk]
+    for kk in range(k):
+        for nn in range(n):
+            Bk[pk.buffer_index([b, k, n], [0, kk, nn])] = Bm[0, kk, nn]
+    spec = M.Matmul([b, m, k, n], (M.u8, M.i8, M.i32), layouts=[oe, pk, None])
+    assert np.array_equal(run_spec(spec, [Ao, Bk, np.zeros((b, m, n), np.int32)]), want)
 
 
 def test_run_host_entry_point(gpu):
