@@ -613,57 +613,68 @@ int run_softmax(const mrl_spec &s, void *const *params, Workspace &ws) {
 int run_compose_msm(const mrl_spec &s, void *const *params, Workspace &ws) {
   const uint32_t b = s.spec_shape[0], m = s.spec_shape[1], k = s.spec_shape[2], n2 = s.spec_shape[3],
                  n = s.spec_shape[4];
-  // Fused path: bf16 Q, V row-major and KT stored k-fastest (layout![0,2,1]), all usable in place.
-  mrl::Strided t[4];
-  bool in_place = true;
-  for (uint32_t i = 0; i < 4; i++) {
-    uint32_t shape[MRL_MAX_RANK], rank;
-    parameter_shape(s, i, shape, &rank);
-    t[i].ptr = params[i], t[i].dtype = s.dtypes[i], t[i].rank = rank;
-    for (uint32_t d = 0; d < MRL_MAX_RANK; d++) t[i].shape[d] = d < rank ? shape[d] : 1;
-    in_place = in_place && mrl::layout_strides(s.layouts[i], shape, rank, t[i].stride);
-  }
-  if (in_place && s.dtypes[0] == MRL_BF16 && s.dtypes[1] == MRL_BF16 && s.dtypes[2] == MRL_BF16) {
-    const mrl::Strided &v = t[0], &q = t[1], &kt = t[2], &out = t[3];
-    const bool kt_k_fastest = (k == 1 || kt.stride[1] == 1) && (n2 == 1 || kt.stride[2] == int64_t(k)) &&
-                              (b == 1 || kt.stride[0] == int64_t(k) * n2);
-    mrl::AttnArgs at;
-    at.q = q.ptr, at.kt = kt.ptr, at.v = v.ptr, at.out = (float *)out.ptr;
-    at.b = b, at.m = m, at.k = k, at.n2 = n2, at.n = n, at.n_out = n;
-    const bool fusable_layouts = dense_row_major(q) && dense_row_major(v) && dense_row_major(out) && kt_k_fastest;
-    if (fusable_layouts && mrl::attn_applicable(at)) {
-      HIP_TRY(mrl::launch_attn(at, ws.stream));
-      return MRL_OK;
-    }
-    // Other head dims up to 128 (and different ones for the two products): Q, K and V rows are
-    // padded with zeros to the next head dim the kernel is built for.  Zero columns of Q and K add
-    // nothing to the scores, zero columns of V give result columns that are not stored.
-    const uint32_t widest = std::max(k, n), dp = widest <= 32 ? 32 : widest <= 64 ? 64 : 128;
-    if (fusable_layouts && widest <= 128 && (reinterpret_cast<uintptr_t>(out.ptr) & 3) == 0) {
-      auto padded = [&](const mrl::Strided &src, uint32_t rows, uint32_t cols, const void **dst) -> int {
-        if (cols == dp && (reinterpret_cast<uintptr_t>(src.ptr) & 15) == 0) {
-          *dst = src.ptr;
-          return MRL_OK;
-        }
+  // Fused path: bf16 Q, K, V and an f32 result, head dims up to 128.  The kernel wants Q and V
+  // row-major, KT with k fastest (layout![0,2,1]: K row-major) and rows of a head dim it is built
+  // for (32, 64, 128).  Parameters that lie so are used in place; others are copied once: to that
+  // order through the layouts' common strided view, and / or to rows padded with zeros (zero
+  // columns of Q and K add nothing to the scores, zero columns of V give result columns that are
+  // not stored).  A result in another layout is formed in scratch memory and moved out.
+  const uint32_t widest = std::max(k, n), dp = widest <= 32 ? 32 : widest <= 64 ? 64 : 128;
+  if (s.dtypes[0] == MRL_BF16 && s.dtypes[1] == MRL_BF16 && s.dtypes[2] == MRL_BF16 && s.dtypes[3] == MRL_F32 &&
+      widest <= 128 && (reinterpret_cast<uintptr_t>(params[3]) & 15) == 0) {
+    // Parameter i as `rows` rows of `cols` bf16 per batch entry; wanted: the order of `want`.
+    auto operand = [&](uint32_t i, const uint32_t *shape, const mrl_layout &want, uint32_t rows, uint32_t cols,
+                       const void **result) -> int {
+      const void *dense = params[i];
+      std::vector<mrl::MoveDim> view;
+      if (!mrl::common_view(s.layouts[i], want, shape, 3, &view)) return MRL_ERR_UNSUPPORTED;
+      const bool in_order = view.empty() || (view.size() == 1 && view[0].ss == 1 && view[0].ds == 1);
+      if (!in_order) {
+        void *buf = nullptr;
+        HIP_TRY(ws.alloc(&buf, size_t(b) * rows * cols * 2));
+        HIP_TRY(mrl::launch_move_view(params[i], MRL_BF16, buf, MRL_BF16, view.data(), uint32_t(view.size()), ws.stream));
+        dense = buf;
+      }
+      if (cols != dp || (reinterpret_cast<uintptr_t>(dense) & 15) != 0) {
         void *buf = nullptr;
         HIP_TRY(ws.alloc(&buf, size_t(b) * rows * dp * 2));
         mrl::Strided flat;
-        flat.ptr = src.ptr, flat.dtype = MRL_BF16, flat.rank = 3;
+        flat.ptr = const_cast<void *>(dense), flat.dtype = MRL_BF16, flat.rank = 3;
         flat.shape[0] = 1, flat.shape[1] = b * rows, flat.shape[2] = cols;
         flat.stride[0] = 0, flat.stride[1] = cols, flat.stride[2] = 1;
         HIP_TRY(mrl::launch_pad_rows(flat, buf, dp, 2, ws.stream));
-        *dst = buf;
-        return MRL_OK;
-      };
-      int rc;
-      if ((rc = padded(q, m, k, &at.q)) != MRL_OK) return rc;
-      if ((rc = padded(kt, n2, k, &at.kt)) != MRL_OK) return rc;
-      if ((rc = padded(v, n2, n, &at.v)) != MRL_OK) return rc;
-      at.k = at.n = dp;
+        dense = buf;
+      }
+      *result = dense;
+      return MRL_OK;
+    };
+    const uint32_t v_shape[3] = {b, n2, n}, q_shape[3] = {b, m, k}, kt_shape[3] = {b, k, n2}, o_shape[3] = {b, m, n};
+    mrl_layout rows_v, rows_q, rows_o, k_fastest;
+    mrl_layout_row_major(v_shape, 3, &rows_v);
+    mrl_layout_row_major(q_shape, 3, &rows_q);
+    mrl_layout_row_major(o_shape, 3, &rows_o);
+    k_fastest.ndims = 3;
+    k_fastest.dims[0] = {0, MRL_DYNAMIC, 0}, k_fastest.dims[1] = {2, MRL_DYNAMIC, 0}, k_fastest.dims[2] = {1, MRL_DYNAMIC, 0};
+    mrl::AttnArgs at;
+    at.b = b, at.m = m, at.k = at.n = dp, at.n2 = n2, at.n_out = n;
+    std::vector<mrl::MoveDim> out_view;
+    int rc = MRL_OK;
+    if (mrl::common_view(rows_o, s.layouts[3], o_shape, 3, &out_view) &&
+        (rc = operand(0, v_shape, rows_v, n2, n, &at.v)) == MRL_OK &&
+        (rc = operand(1, q_shape, rows_q, m, k, &at.q)) == MRL_OK &&
+        (rc = operand(2, kt_shape, k_fastest, n2, k, &at.kt)) == MRL_OK) {
+      const bool out_in_order = out_view.empty() || (out_view.size() == 1 && out_view[0].ss == 1 && out_view[0].ds == 1);
+      void *result = params[3];
+      if (!out_in_order) HIP_TRY(ws.alloc(&result, size_t(b) * m * n * sizeof(float)));
+      at.out = static_cast<float *>(result);
       if (mrl::attn_applicable(at)) {
         HIP_TRY(mrl::launch_attn(at, ws.stream));
+        if (!out_in_order)
+          HIP_TRY(mrl::launch_move_view(result, MRL_F32, params[3], MRL_F32, out_view.data(), uint32_t(out_view.size()), ws.stream));
         return MRL_OK;
       }
+    } else if (rc != MRL_OK && rc != MRL_ERR_UNSUPPORTED) {
+      return rc;
     }
   }
   // Staged path, as the reference schedules it (examples/matmul_chain.rs:60-81): S and P

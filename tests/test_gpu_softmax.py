@@ -126,18 +126,35 @@ def test_compose_msm_fused_with_padded_head_dims(gpu, dims):
     assert rel_err(got, want) < 1e-2
 
 
-def test_compose_msm_row_major_kt_and_f32_inputs(gpu):
-    """KT materialised row-major and f32 inputs run on the staged (unfused) path."""
+def test_compose_msm_f32_inputs_stay_staged(gpu):
+    """f32 inputs run on the staged (unfused) path, exact to 1e-5: nothing is rounded to bf16."""
     b, m, k, n2, n = 2, 40, 32, 48, 24
     q, kmat, v = msm_inputs(302, b, m, k, n2, n)
     kt = np.ascontiguousarray(kmat.transpose(0, 2, 1))
-    got = run_spec(M.ComposeMSM(b, m, k, n2, n), [v, q, kt, np.zeros((b, m, n), np.float32)])
     want = orc.compose_msm(b, m, k, n2, n, [7, 7, 7, 6], v, q, kt, np.zeros((b, m, n), np.float32))
-    assert rel_err(got, want) < 1e-5
     qf, ktf, vf = (synth.bf16_bits_to_f32(t) for t in (q, kt, v))
     got = run_spec(M.ComposeMSM(b, m, k, n2, n, dtypes=(M.f32, M.f32, M.f32, M.f32)),
                    [vf, qf, ktf, np.zeros((b, m, n), np.float32)])
     assert rel_err(got, want) < 1e-5
+
+
+@pytest.mark.parametrize("dims", [(2, 40, 32, 48, 24), (2, 256, 128, 384, 128), (1, 200, 64, 130, 64)])
+def test_compose_msm_fused_from_other_layouts(gpu, dims):
+    """The reference's default layouts (everything row-major, KT as [b, k, n2] with n2 fastest,
+    examples/matmul_chain.rs:26-57), a batched column-major Q, a V with a Packed dim and a batched column-major
+    result: each is brought to the order the fused kernel reads (one copy) and the result moved
+    out, within the composed pipeline's tolerance."""
+    b, m, k, n2, n = dims
+    q, kmat, v = msm_inputs(306, *dims)
+    kt = np.ascontiguousarray(kmat.transpose(0, 2, 1))                       # [b, k, n2] row-major
+    want = orc.compose_msm(b, m, k, n2, n, [7, 7, 7, 6], v, q, kt, np.zeros((b, m, n), np.float32))
+    got = run_spec(M.ComposeMSM(b, m, k, n2, n), [v, q, kt, np.zeros((b, m, n), np.float32)])
+    assert rel_err(got, want) < 1e-2
+    layouts = [M.layout(0, 1, 2, (1, M.Packed(2))), M.batched_col_major([b, m, k]), None, M.batched_col_major([b, m, n])]
+    vp = np.ascontiguousarray(v.reshape(b, n2 // 2, 2, n).transpose(0, 1, 3, 2))      # [b, n2/2, n, 2]
+    qc = np.ascontiguousarray(q.transpose(0, 2, 1))
+    got = run_spec(M.ComposeMSM(b, m, k, n2, n, layouts=layouts), [vp, qc, kt, np.zeros((b, n, m), np.float32)])
+    assert rel_err(got.transpose(0, 2, 1), want) < 1e-2
 
 
 def test_compose_msm_full_size(gpu):
