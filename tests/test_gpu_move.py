@@ -79,3 +79,38 @@ def test_async_launches_on_two_streams(gpu):
     assert np.abs(got - orc.softmax([64, 96], 1, x)).max() < 1e-6
     s1.destroy()
     s2.destroy()
+
+
+def test_host_threads_share_a_stream_and_its_scratch(gpu):
+    """Four host threads enqueue Matmuls that need scratch memory (K and N are not whole 16-byte
+    chunks, so A and B are copied into padded rows) onto one stream, each thread several times
+    with its own operands.  The stream's scratch arena is handed from call to call, so every
+    result must still be its own thread's."""
+    import threading
+    stream = M.Stream()
+    shapes = [(1, 300, 270, 290), (2, 257, 333, 201), (1, 400, 250, 310), (1, 260, 267, 500)]
+    jobs = []
+    for t, (b, m, k, n) in enumerate(shapes):
+        A, Bm = synth.uniform_u8(820 + t, 0, (b, m, k)), synth.uniform_i8(820 + t, 1, (b, k, n))
+        bufs = [M.DeviceBuffer.from_numpy(x) for x in (A, Bm, np.zeros((b, m, n), np.int32))]
+        want = orc.matmul([b, m, k, n], [0, 1, 5], A, Bm, np.zeros((b, m, n), np.int32))
+        jobs.append((M.MatmulAccum([b, m, k, n], (M.u8, M.i8, M.i32)), bufs, want, (b, m, n)))
+    rounds, errors = 5, []
+
+    def work(spec, bufs):
+        try:
+            for _ in range(rounds):
+                spec.run_async([x.ptr for x in bufs], stream)
+        except Exception as e:  # surfaced below: a thread's exception is otherwise lost
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(spec, bufs)) for spec, bufs, _, _ in jobs]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    stream.synchronize()
+    assert not errors, errors
+    for spec, bufs, want, shape in jobs:
+        assert np.array_equal(bufs[2].to_numpy(np.int32, shape), rounds * want)
+    stream.destroy()
