@@ -69,6 +69,7 @@ hipError_t launch_gemm_big(const GemmArgs &g, int kind, hipStream_t stream) {
 }
 
 hipError_t launch_gemm(const GemmArgs &g, int kind, hipStream_t stream) {
+  if (gemv_applicable(g, kind)) return launch_gemv(g, kind, stream);
   const int es = elem_size_of(kind);
   // Only the 256 tile has a build without the EDGE kernels' limit on leading dimensions.
   const uint32_t side = edge_addressable(g, es) ? tile_side(g, es) : 256;

@@ -74,6 +74,10 @@ hipError_t launch_gemm(const GemmArgs &g, int kind, hipStream_t stream);
 // Always the 256 x 256 tile, 128 bytes of K per step.
 hipError_t launch_gemm_big(const GemmArgs &g, int kind, hipStream_t stream);
 
+// ---- gemv.hip: at most four rows of A against a k-fastest B, as dot products (a stream over B) ----
+bool gemv_applicable(const GemmArgs &g, int kind);
+hipError_t launch_gemv(const GemmArgs &g, int kind, hipStream_t stream);
+
 // ---- gemm_sched.hip: the same kernel under a caller-chosen tile_out / split schedule -----
 uint32_t gemm_schedule_count();
 void gemm_schedule_at(uint32_t i, int elem_size, uint32_t *tile_m, uint32_t *tile_n, uint32_t *split_k);

@@ -215,6 +215,35 @@ def test_matmul_every_tile_choice(gpu, dts, codes, shape, accum, b_k_fastest):
         assert rel_err(got, want) < 1e-5
 
 
+@pytest.mark.parametrize("dts,codes", [((M.u8, M.i8, M.i32), [0, 1, 5]), ((M.i8, M.i8, M.i32), [1, 1, 5]),
+                                        ((M.bf16, M.bf16, M.f32), [7, 7, 6]), ((M.f32, M.f32, M.f32), [6, 6, 6])])
+@pytest.mark.parametrize("shape,accum", [
+    ((1, 1, 2048, 16384), False),   # examples/matvec_gemma_x86_bf16f32.rs:24-37
+    ((1, 1, 1024, 70), True),       # columns that do not fill the last wavefront
+    ((3, 2, 4096, 129), True),      # batched, two rows
+    ((2, 3, 1040, 256), False),     # three rows on the four-row build, K not a multiple of a wave's stride
+    ((1, 4, 8192, 64), True),
+    ((2, 7, 2064, 100), True),      # seven rows on the eight-row build
+    ((1, 8, 1024, 1000), False),
+])
+def test_matrix_vector_shapes(gpu, dts, codes, shape, accum):
+    """At most eight rows of A against a B stored k-fastest run as dot products that stream B once
+    (no matrix cores); same results as any other Matmul."""
+    b, m, k, n = shape
+    gen = {M.u8: synth.uniform_u8, M.i8: synth.uniform_i8, M.bf16: synth.normal_bf16, M.f32: synth.uniform_f32}
+    A, Bm = gen[dts[0]](75, 0, (b, m, k)), gen[dts[1]](75, 1, (b, k, n))
+    out_np = np.int32 if dts[2] == M.i32 else np.float32
+    C0 = (synth.uniform_u8(75, 2, (b, m, n)).astype(out_np) if accum else np.zeros((b, m, n), out_np))
+    Bt = np.ascontiguousarray(Bm.transpose(0, 2, 1))
+    spec = M.Matmul(shape, dts, layouts=[None, M.layout(0, 2, 1), None], accum=accum)
+    got = run_spec(spec, [A, Bt, C0])
+    want = orc.matmul(list(shape), codes, A, Bm, C0.copy(), accum)
+    if dts[2] == M.i32:
+        assert np.array_equal(got, want)
+    else:
+        assert rel_err(got, want) < 1e-5
+
+
 @pytest.mark.parametrize("dts,codes", [((M.f32, M.bf16, M.f32), [6, 7, 6]), ((M.bf16, M.f32, M.f32), [7, 6, 6])])
 def test_mixed_bf16_f32_matmul(gpu, dts, codes):
     """One bf16 and one f32 input with an f32 output: both are taken to f32 before the product,
