@@ -439,6 +439,44 @@ __global__ __launch_bounds__(256) void k_conv_generic(CV p) {
   else store_u32(p.out, p.dto, ooff, iacc);
 }
 
+// The same with one wavefront per output element, its lanes striding over the C * FH * FW
+// products: for a handful of outputs with a long reduction (examples/simple_conv_x86.rs: 8 outputs
+// of 72 products each) the one-thread-per-output kernel is a chain of dependent loads.
+template <bool FLOAT_OUT>
+__global__ __launch_bounds__(256) void k_conv_generic_wave(CV p) {
+  const uint64_t total = uint64_t(p.B) * p.F * p.OH * p.OW;
+  const uint64_t idx = uint64_t(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (idx >= total) return;
+  const uint32_t lane = threadIdx.x & 63;
+  uint64_t r = idx;
+  const uint32_t f = uint32_t(r % p.F); r /= p.F;
+  const uint32_t x = uint32_t(r % p.OW); r /= p.OW;
+  const uint32_t y = uint32_t(r % p.OH); r /= p.OH;
+  const uint32_t b = uint32_t(r);
+  const int64_t ooff = b * p.so[0] + f * p.so[1] + y * p.so[2] + x * p.so[3];
+  float facc = 0.0f;
+  uint32_t iacc = 0;
+  const uint32_t window = p.FH * p.FW, terms = p.C * window;
+  for (uint32_t t = lane; t < terms; t += 64) {
+    const uint32_t c = t / window, rr = (t % window) / p.FW, s = t % p.FW;
+    const int64_t io = b * p.si[0] + c * p.si[1] + int64_t(y + rr) * p.si[2] + int64_t(x + s) * p.si[3];
+    const int64_t fo = f * p.sf[0] + c * p.sf[1] + rr * p.sf[2] + s * p.sf[3];
+    if (FLOAT_OUT) facc += load_f32(p.img, p.dti, io) * load_f32(p.filt, p.dtf, fo);
+    else iacc += load_u32(p.img, p.dti, io, p.dto) * load_u32(p.filt, p.dtf, fo, p.dto);
+  }
+  for (int o = 32; o > 0; o >>= 1) {
+    facc += __shfl_xor(facc, o);
+    iacc += uint32_t(__shfl_xor(int(iacc), o));
+  }
+  if (lane != 0) return;
+  if (p.accum) {
+    if (FLOAT_OUT) facc += ((const float *)p.out)[ooff];
+    else iacc += load_u32(p.out, p.dto, ooff, MRL_U32);
+  }
+  if (FLOAT_OUT) ((float *)p.out)[ooff] = facc;
+  else store_u32(p.out, p.dto, ooff, iacc);
+}
+
 // ------------------------------------------------------------------- softmax
 // One wavefront per line along an arbitrary-stride scan dim: max, then exp and sum, then
 // divide (morello/src/verification.rs:166-184).
@@ -792,6 +830,12 @@ hipError_t launch_conv_generic(const Strided &img, const Strided &filt, const St
   for (int d = 0; d < 4; d++) p.si[d] = img.stride[d], p.sf[d] = filt.stride[d], p.so[d] = out.stride[d];
   p.accum = accum;
   const uint64_t total = uint64_t(p.B) * p.F * p.OH * p.OW;
+  if (total <= 16384 && uint64_t(p.C) * p.FH * p.FW >= 32) {  // few outputs, long reductions
+    const uint32_t wave_blocks = uint32_t((total + 3) / 4);
+    if (float_out(out.dtype)) hipLaunchKernelGGL(k_conv_generic_wave<true>, dim3(wave_blocks), dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL(k_conv_generic_wave<false>, dim3(wave_blocks), dim3(256), 0, stream, p);
+    return hipGetLastError();
+  }
   const uint32_t blocks = uint32_t((total + 255) / 256);
   if (float_out(out.dtype)) hipLaunchKernelGGL(k_conv_generic<true>, dim3(blocks), dim3(256), 0, stream, p);
   else hipLaunchKernelGGL(k_conv_generic<false>, dim3(blocks), dim3(256), 0, stream, p);
