@@ -28,12 +28,13 @@ bool applicable(const GemmArgs &g, int es) {
 // Side of the square workgroup tile for a problem size, from launch timings on an MI355X of
 // every built tile over cubes from 64^3 to 4096^3.  The 256 x 256 tile is the fastest per CU
 // but fills the chip in rounds of 256 tiles, one per CU; smaller tiles run several to a CU.
+// All three step through K 128 bytes at a time (a 64-byte step costs the small tiles 10-30 %).
 //   int8, bf16: 256 once a round is at least half full (3072^3, 144 tiles: int8 47 us against
-//     55 us for 128 and 74 us for 64); below that 64 up to 384 of its tiles (1024^3: 8.0 us
-//     against 10.8 and 17.7), then 128 (2048^3: 19.6 us against 25.1 and 29.9).
+//     49 us for 128 and 62 us for 64); below that 64 up to 384 of its tiles (1024^3: 6.5 us
+//     against 10.0 and 17.7), then 128 (2048^3: 17.3 us against 20.6 and 29.9).
 //   f32: its MFMA has a sixteenth of the int8 rate, so operand traffic never limits a small
-//     tile: 64 (1024^3: 30 us against 77 and 239; 3072^3: 463 against 592 and 714) until the
-//     256 tile fills its rounds (4096^3: 952 us against 1062).
+//     tile: 64 (1024^3: 27 us against 70 and 239; 3072^3: 460 against 559 and 711) until the
+//     256 tile fills its rounds (4096^3: 948 us against 1066).
 uint32_t tile_side(const GemmArgs &g, int es) {
   const uint64_t big = uint64_t((g.m + 255) / 256) * ((g.n + 255) / 256) * g.batch;
   const double round_fill = double(big) / double((big + 255) / 256 * 256);
@@ -75,7 +76,7 @@ hipError_t launch_gemm(const GemmArgs &g, int kind, hipStream_t stream) {
   const uint32_t side = edge_addressable(g, es) ? tile_side(g, es) : 256;
   if (side == 256) return launch_gemm_big(g, kind, stream);
   if (g.b_kmajor) return launch_gemm_nt(g, kind, side, stream);
-  return launch_gemm_scheduled(g, kind, side, side, 64 / es, stream);
+  return launch_gemm_scheduled(g, kind, side, side, 128 / es, stream);
 }
 
 }  // namespace mrl

@@ -7,8 +7,8 @@ namespace mrl {
 namespace {
 using namespace gemm;
 
-typedef Tile<128, 128, 64, 2, 2> T128;
-typedef Tile<64, 64, 64, 2, 2> T64;
+typedef Tile<128, 128, 128, 2, 2> T128;
+typedef Tile<64, 64, 128, 2, 2> T64;
 
 template <class T, bool A_UNSIGNED>
 hipError_t launch_for(const GemmArgs &g, uint32_t tile, hipStream_t stream) {

@@ -16,12 +16,14 @@ typedef Tile<256, 128, 64, 2, 2> T256x128k64;
 typedef Tile<128, 256, 64, 2, 2> T128x256k64;
 typedef Tile<128, 128, 64, 2, 2> T128x128k64;
 typedef Tile<64, 64, 64, 2, 2> T64x64k64;
+typedef Tile<64, 64, 128, 2, 2> T64x64k128;
+typedef Tile<128, 128, 128, 2, 2> T128x128k128;
 
 struct Entry {
   uint32_t tile_m, tile_n, k_bytes;
 };
 // k_bytes is the k step in bytes of an operand row: 128 = 128 i8, 64 bf16 or 32 f32 elements.
-const Entry kSchedules[] = {{256, 256, 128}, {256, 256, 64}, {256, 128, 64}, {128, 256, 64}, {128, 128, 64}, {64, 64, 64}};
+const Entry kSchedules[] = {{256, 256, 128}, {256, 256, 64}, {256, 128, 64}, {128, 256, 64}, {128, 128, 64}, {64, 64, 64}, {128, 128, 128}, {64, 64, 128}};
 
 template <class TL>
 hipError_t launch_kind(const GemmArgs &g, int kind, hipStream_t stream) {
@@ -53,6 +55,8 @@ hipError_t launch_gemm_scheduled(const GemmArgs &g, int kind, uint32_t tile_m, u
   if (tile_m == 128 && tile_n == 256 && k_bytes == 64) return launch_kind<T128x256k64>(g, kind, stream);
   if (tile_m == 128 && tile_n == 128 && k_bytes == 64) return launch_kind<T128x128k64>(g, kind, stream);
   if (tile_m == 64 && tile_n == 64 && k_bytes == 64) return launch_kind<T64x64k64>(g, kind, stream);
+  if (tile_m == 128 && tile_n == 128 && k_bytes == 128) return launch_kind<T128x128k128>(g, kind, stream);
+  if (tile_m == 64 && tile_n == 64 && k_bytes == 128) return launch_kind<T64x64k128>(g, kind, stream);
   return hipErrorInvalidValue;
 }
 
