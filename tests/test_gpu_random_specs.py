@@ -135,3 +135,69 @@ def test_random_conv(gpu, seed):
     want = orc.conv(shape, [int(d) for d in dts], bufs[0], bufs[1], bufs[2].copy(), accum,
                     layouts=[l[1] for l in lay])
     compare(got, want, dts[2], (shape, dts, accum, [repr(l[0]) for l in lay]))
+
+
+MFMA_DTYPES = [(M.u8, M.i8, M.i32), (M.i8, M.i8, M.i32), (M.bf16, M.bf16, M.f32), (M.f32, M.f32, M.f32),
+               (M.bf16, M.f32, M.f32)]
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_matmul_mid_sizes(gpu, seed):
+    """Sizes where the library's own choices change: which tile (64 / 128 / 256), padded copies
+    for rows that are not whole 16-byte chunks, the matrix-vector kernel (few rows, k-fastest B),
+    column-major operands made row-major; dims drawn so that the product stays below 2e8."""
+    rng = np.random.default_rng(7500 + seed)
+    b = int(rng.choice([1, 1, 1, 2]))
+    pool = [1, 2, 3, 5, 8, 9, 16, 40, 64, 100, 128, 129, 255, 256, 257, 300, 384, 500, 512, 513, 640, 777, 1000, 1024, 1100]
+    while True:
+        m, k, n = (int(rng.choice(pool)) for _ in range(3))
+        if b * m * k * n <= 2e8:
+            break
+    dts = MFMA_DTYPES[int(rng.integers(len(MFMA_DTYPES)))]
+    accum = bool(rng.integers(2))
+    shape = [b, m, k, n]
+    pshapes = [[b, m, k], [b, k, n], [b, m, n]]
+    # Row-major mostly; B k-fastest in a third of the cases; now and then any layout.
+    lay = []
+    for i, s in enumerate(pshapes):
+        roll = rng.random()
+        if i == 1 and roll < 0.35:
+            lay.append((M.layout(0, 2, 1), orc.make_layout([0, 2, 1])))
+        elif roll < 0.8:
+            lay.append((M.row_major(s), orc.make_layout([0, 1, 2])))
+        else:
+            lay.append(random_layout(rng, s))
+    bufs = [random_values(rng, dt, s, 7500 + seed * 3 + i) for i, (dt, s) in enumerate(zip(dts, pshapes))]
+    if not accum:
+        bufs[2] = np.zeros(pshapes[2], NP[dts[2]])
+    spec = M.Matmul(shape, dts, layouts=[l[0] for l in lay], accum=accum)
+    got = run_spec(spec, bufs)
+    want = orc.matmul(shape, [int(d) for d in dts], bufs[0], bufs[1], bufs[2].copy(), accum,
+                      layouts=[l[1] for l in lay])
+    compare(got, want, dts[2], (shape, dts, accum, [repr(l[0]) for l in lay]))
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_conv_mid_sizes(gpu, seed):
+    """Conv shapes the unfolded (Conv as Matmul) path takes, next to the fused kernel's and the
+    generic kernel's: channel counts that are and are not whole dwords / 16-byte chunks, filters
+    from 1x1 to 5x5, every Matmul dtype triple, random layouts now and then."""
+    rng = np.random.default_rng(9700 + seed)
+    b = int(rng.integers(1, 4))
+    f = int(rng.choice([1, 8, 24, 64, 65, 100]))
+    c = int(rng.choice([1, 3, 4, 16, 24, 64, 128]))
+    oh, ow = int(rng.integers(1, 21)), int(rng.integers(1, 21))
+    fh, fw = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+    dts = [(M.u8, M.i8, M.i32), (M.i8, M.i8, M.i32), (M.bf16, M.bf16, M.f32), (M.f32, M.f32, M.f32)][int(rng.integers(4))]
+    accum = bool(rng.integers(2))
+    shape = [b, f, c, oh, ow, fh, fw]
+    pshapes = [[b, c, oh + fh - 1, ow + fw - 1], [f, c, fh, fw], [b, f, oh, ow]]
+    nhwc = (lambda s: (M.nhwc(s), orc.make_layout([0, 2, 3, 1])))
+    lay = [nhwc(s) if rng.random() < 0.75 else random_layout(rng, s) for s in pshapes]
+    bufs = [random_values(rng, dt, s, 9700 + seed * 3 + i) for i, (dt, s) in enumerate(zip(dts, pshapes))]
+    if not accum:
+        bufs[2] = np.zeros(pshapes[2], NP[dts[2]])
+    got = run_spec(M.Conv(shape, dts, layouts=[l[0] for l in lay], accum=accum), bufs)
+    want = orc.conv(shape, [int(d) for d in dts], bufs[0], bufs[1], bufs[2].copy(), accum,
+                    layouts=[l[1] for l in lay])
+    compare(got, want, dts[2], (shape, dts, accum, [repr(l[0]) for l in lay]))
