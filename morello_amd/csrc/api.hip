@@ -501,8 +501,9 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
   cv.accum = s.accum;
   const int di = s.dtypes[0], df = s.dtypes[1], dout = s.dtypes[2];
   const bool fast_types = (di == MRL_U8 || di == MRL_I8) && df == MRL_I8 && dout == MRL_I32;
-  const bool fused_shape = fast_types && cv.f == 64 && cv.c % 64 == 0 &&
-                           (cv.fh * cv.fw * (cv.c / 64) == 1 || cv.fh * cv.fw * (cv.c / 64) == 9);
+  const uint32_t slabs = cv.c % 64 == 0 ? cv.fh * cv.fw * (cv.c / 64) : 0;
+  const bool fused_shape = fast_types && cv.f % 64 == 0 && cv.f <= 64 * 65535 &&
+                           (slabs == 1 || slabs == 2 || slabs == 3 || slabs == 4 || slabs == 6 || slabs == 9);
   // Matmul kind of the same dtypes (-1: none): any other shape runs as unfold + Matmul.
   const int kind = (di == MRL_I8 && df == MRL_I8 && dout == MRL_I32)       ? 0
                    : (di == MRL_U8 && df == MRL_I8 && dout == MRL_I32)     ? 1

@@ -18,6 +18,8 @@
 //
 // u8 images: a' = a xor 0x80 and the per-filter correction 128 * sum_{r,s,c} filt[f,r,s,c]
 // is added at the end (exact in i32).
+#include <algorithm>
+
 #include "kernels.h"
 
 namespace mrl {
@@ -42,6 +44,9 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(ConvArgs p, uint32_t pix
   const int H = p.oh + p.fh - 1, W = p.ow + p.fw - 1;
   const int sub = p.c / 64;  // 64-channel slabs per filter position
   const int krow = p.fh * p.fw * p.c;  // bytes per filter
+  // blockIdx.y: which group of 64 filters (= 64 output channels) this workgroup computes.
+  const uint8_t *filters = (const uint8_t *)p.filters + int64_t(blockIdx.y) * (FT * 16) * krow;
+  int32_t *out = (int32_t *)p.out + blockIdx.y * (FT * 16);
 
   // Filter bank: global -> LDS (coalesced, once per workgroup) -> registers (per wave).
   // 64 filters x (SLABS * 64) bytes = SLABS * 256 chunks of 16 bytes.  These loads need
@@ -52,7 +57,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(ConvArgs p, uint32_t pix
 #pragma unroll
   for (int i = 0; i < PER_THREAD; i++) {
     const int c = i * NT + threadIdx.x;
-    if (c < SLABS * 256) stage[i] = *(const v4i *)((const uint8_t *)p.filters + c * 16);
+    if (c < SLABS * 256) stage[i] = *(const v4i *)(filters + c * 16);
   }
 
   // Byte offset of each slab's source relative to the pixel's own (y, x) position.
@@ -132,7 +137,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(ConvArgs p, uint32_t pix
     // D[row = filter 4*lg + r][col = pixel li]: lane owns 4 consecutive filters of its pixel.
     const uint32_t pix = t * 16 + li;
     if (pix < pixels) {
-      int32_t *dst = (int32_t *)p.out + int64_t(pix) * p.f + lg * 4;
+      int32_t *dst = out + int64_t(pix) * p.f + lg * 4;
 #pragma unroll
       for (int ft = 0; ft < FT; ft++) {
         v4i v = acc[ft];
@@ -153,13 +158,14 @@ hipError_t launch_slabs(const ConvArgs &c, bool img_unsigned, hipStream_t stream
   // 2048 waves = two per SIMD of a 256-CU part at ~250 VGPRs each, as workgroups of
   // CONV_WAVES waves (4 measured fastest); never more waves than tiles.
   constexpr int WAVES = CONV_WAVES;
-  uint32_t blocks = 2048 / WAVES;
+  const uint32_t groups = c.f / (FT * 16);
+  uint32_t blocks = std::max<uint32_t>(1, 2048 / WAVES / groups);
   if (blocks * WAVES > tiles) blocks = (tiles + WAVES - 1) / WAVES;
   const size_t lds = size_t(FT) * 16 * c.fh * c.fw * c.c + FT * 16 * sizeof(int);  // the filter bank + corrections
   if (img_unsigned)
-    hipLaunchKernelGGL((k_conv_i8<SLABS, true, WAVES>), dim3(blocks), dim3(64 * WAVES), lds, stream, c, uint32_t(pixels), tiles);
+    hipLaunchKernelGGL((k_conv_i8<SLABS, true, WAVES>), dim3(blocks, groups), dim3(64 * WAVES), lds, stream, c, uint32_t(pixels), tiles);
   else
-    hipLaunchKernelGGL((k_conv_i8<SLABS, false, WAVES>), dim3(blocks), dim3(64 * WAVES), lds, stream, c, uint32_t(pixels), tiles);
+    hipLaunchKernelGGL((k_conv_i8<SLABS, false, WAVES>), dim3(blocks, groups), dim3(64 * WAVES), lds, stream, c, uint32_t(pixels), tiles);
   return hipGetLastError();
 }
 
@@ -169,9 +175,9 @@ int slabs_of(const ConvArgs &c) { return int(c.fh * c.fw * (c.c / 64)); }
 
 bool conv_i8_applicable(const ConvArgs &c) {
   auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-  if (c.f != 64 || c.c == 0 || c.c % 64 != 0) return false;
-  const int s = slabs_of(c);
-  if (s != 1 && s != 9) return false;
+  if (c.f == 0 || c.f % 64 != 0 || c.f > 64 * 65535 || c.c == 0 || c.c % 64 != 0) return false;
+  const int s = slabs_of(c);  // 16 VGPRs of filter operands per slab and lane
+  if (s != 1 && s != 2 && s != 3 && s != 4 && s != 6 && s != 9) return false;
   const uint64_t pixels = uint64_t(c.b) * c.oh * c.ow;
   const uint64_t in_bytes = uint64_t(c.b) * (c.oh + c.fh - 1) * (c.ow + c.fw - 1) * c.c;
   return pixels > 0 && pixels < (1ull << 31) && in_bytes < (1ull << 31) && al16(c.image) &&
@@ -181,6 +187,10 @@ bool conv_i8_applicable(const ConvArgs &c) {
 hipError_t launch_conv_i8(const ConvArgs &c, bool img_unsigned, hipStream_t stream) {
   switch (slabs_of(c)) {
     case 1: return launch_slabs<1>(c, img_unsigned, stream);
+    case 2: return launch_slabs<2>(c, img_unsigned, stream);
+    case 3: return launch_slabs<3>(c, img_unsigned, stream);
+    case 4: return launch_slabs<4>(c, img_unsigned, stream);
+    case 6: return launch_slabs<6>(c, img_unsigned, stream);
     case 9: return launch_slabs<9>(c, img_unsigned, stream);
     default: return hipErrorInvalidValue;
   }

@@ -27,6 +27,11 @@ def nhwc_inputs(seed, b, f, c, oh, ow, fh, fw, dt_img=M.u8):
     ((2, 5, 7, 4, 3, 2, 3), True),       # ragged channels: generic kernel
     ((3, 64, 64, 54, 54, 3, 3), False),  # benchmark configuration 4 at batch 3
     ((1, 64, 64, 5, 5, 1, 1), False),    # 1x1 filter
+    ((2, 128, 64, 9, 11, 3, 3), True),   # two groups of 64 filters on the fused kernel
+    ((1, 192, 128, 7, 7, 1, 1), False),  # three groups, two 64-channel slabs
+    ((2, 64, 256, 5, 6, 1, 1), True),    # four slabs
+    ((1, 128, 64, 6, 6, 3, 1), False),   # three slabs (3x1 filter)
+    ((1, 64, 128, 6, 5, 1, 3), True),    # six slabs (1x3 filter over 128 channels)
 ])
 def test_conv_nhwc_bit_exact(gpu, dt_img, shape, accum):
     b, f, c, oh, ow, fh, fw = shape
