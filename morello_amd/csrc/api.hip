@@ -516,7 +516,7 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
   // Windows of this many images are unfolded at a time.
   constexpr uint64_t UNFOLD_BYTES = uint64_t(1) << 30;
   const uint64_t image_rows_bytes = pixels * row_elems * img.elem;
-  const bool as_matmul = !fused_shape && kind >= 0 && image_rows_bytes <= UNFOLD_BYTES && window < (1u << 24) &&
+  const bool as_matmul = !fused_shape && kind >= 0 && image_rows_bytes <= UNFOLD_BYTES && row_elems * img.elem < (1u << 24) &&
                          double(cv.b) * pixels * cv.f * window >= 1e6;
   // Tensors in another permutation layout (NCHW, say) are moved to channels-last when a
   // matrix-core path takes the shape: three small extra passes against a generic kernel
