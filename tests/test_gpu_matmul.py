@@ -225,18 +225,23 @@ def test_matmul_every_tile_choice(gpu, dts, codes, shape, accum, b_k_fastest):
     ((1, 4, 8192, 64), True),
     ((2, 7, 2064, 100), True),      # seven rows on the eight-row build
     ((1, 8, 1024, 1000), False),
+    ((1, 1, 300, 4096), False),     # row-major B: one slice of K that is not whole steps of 64
+    ((2, 3, 1000, 8192), True),
+    ((1, 4, 2048, 4112), True),
 ])
-def test_matrix_vector_shapes(gpu, dts, codes, shape, accum):
-    """At most eight rows of A against a B stored k-fastest run as dot products that stream B once
-    (no matrix cores); same results as any other Matmul."""
+@pytest.mark.parametrize("b_k_fastest", [True, False])
+def test_matrix_vector_shapes(gpu, dts, codes, shape, accum, b_k_fastest):
+    """Up to eight rows of A against a k-fastest B run as dot products that stream B once instead
+    of on the matrix cores; the same shapes with a row-major B stay on the 64 x 64 MFMA tile.
+    Same results as any other Matmul."""
     b, m, k, n = shape
     gen = {M.u8: synth.uniform_u8, M.i8: synth.uniform_i8, M.bf16: synth.normal_bf16, M.f32: synth.uniform_f32}
     A, Bm = gen[dts[0]](75, 0, (b, m, k)), gen[dts[1]](75, 1, (b, k, n))
     out_np = np.int32 if dts[2] == M.i32 else np.float32
     C0 = (synth.uniform_u8(75, 2, (b, m, n)).astype(out_np) if accum else np.zeros((b, m, n), out_np))
-    Bt = np.ascontiguousarray(Bm.transpose(0, 2, 1))
-    spec = M.Matmul(shape, dts, layouts=[None, M.layout(0, 2, 1), None], accum=accum)
-    got = run_spec(spec, [A, Bt, C0])
+    Bbuf = np.ascontiguousarray(Bm.transpose(0, 2, 1)) if b_k_fastest else Bm
+    spec = M.Matmul(shape, dts, layouts=[None, M.layout(0, 2, 1) if b_k_fastest else None, None], accum=accum)
+    got = run_spec(spec, [A, Bbuf, C0])
     want = orc.matmul(list(shape), codes, A, Bm, C0.copy(), accum)
     if dts[2] == M.i32:
         assert np.array_equal(got, want)
