@@ -120,6 +120,56 @@ __device__ inline uint32_t move_bits(const void *src, int sdt, int64_t so, int d
   return load_u32(src, sdt, so, MRL_U32);  // int -> int wraps
 }
 
+// The same conversions on an element already in a register (`raw`: its bits, zero-extended).
+__device__ inline float raw_to_f32(uint32_t raw, int dtype) {
+  switch (dtype) {
+    case MRL_U8: return float(raw & 0xffu);
+    case MRL_I8: return float(int8_t(uint8_t(raw)));
+    case MRL_U16: return float(raw & 0xffffu);
+    case MRL_I16: return float(int16_t(uint16_t(raw)));
+    case MRL_U32: return float(raw);
+    case MRL_I32: return float(int32_t(raw));
+    case MRL_F32: return __uint_as_float(raw);
+    default: return bf16_bits_to_f32(uint16_t(raw));
+  }
+}
+__device__ inline uint32_t convert_raw(uint32_t raw, int sdt, int ddt) {
+  const bool src_float = sdt == MRL_F32 || sdt == MRL_BF16;
+  if (ddt == MRL_F32) return __float_as_uint(raw_to_f32(raw, sdt));
+  if (ddt == MRL_BF16) return f32_to_bf16_bits(raw_to_f32(raw, sdt));
+  if (src_float) return float_to_int(raw_to_f32(raw, sdt), ddt);
+  return narrow_int(sdt, raw);  // int -> int: extend by the source's sign, the store truncates
+}
+
+// Move of a contiguous run with a dtype conversion: four elements per thread, one vector load
+// and one vector store (SE, DE: element sizes in bytes).
+template <int SE, int DE>
+__global__ __launch_bounds__(256) void k_convert4(const void *__restrict__ src, void *__restrict__ dst, int sdt,
+                                                  int ddt, uint64_t count) {
+  struct alignas(SE * 4) SrcQuad { uint8_t b[SE * 4]; };
+  struct alignas(DE * 4) DstQuad { uint8_t b[DE * 4]; };
+  const uint64_t quads = count / 4, step = uint64_t(gridDim.x) * 256;
+  for (uint64_t i = uint64_t(blockIdx.x) * 256 + threadIdx.x; i < quads; i += step) {
+    const SrcQuad in = static_cast<const SrcQuad *>(src)[i];
+    DstQuad out;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      uint32_t raw = 0;
+#pragma unroll
+      for (int k = 0; k < SE; k++) raw |= uint32_t(in.b[e * SE + k]) << (8 * k);
+      const uint32_t v = convert_raw(raw, sdt, ddt);
+#pragma unroll
+      for (int k = 0; k < DE; k++) out.b[e * DE + k] = uint8_t(v >> (8 * k));
+    }
+    static_cast<DstQuad *>(dst)[i] = out;
+  }
+  // The up to three elements past the last quad.
+  if (blockIdx.x == 0 && threadIdx.x < count % 4) {
+    const int64_t at = int64_t(quads * 4 + threadIdx.x);
+    store_u32(dst, ddt, at, move_bits(src, sdt, at, ddt));
+  }
+}
+
 __global__ void k_move_generic(const void *src, void *dst, LayoutEval sl, LayoutEval dl, int sdt,
                                int ddt, uint64_t count) {
   const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -690,6 +740,20 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
       vectors = int(d) == dim_s || (p.ss[d] % per == 0 && p.ds[d] % per == 0);
     if (vectors && rank == 1)
       return launch_copy(src, dst, p.count * mrl_dtype_size(src_dtype), stream);
+    // One contiguous run with a conversion: four elements per thread.
+    const size_t se = mrl_dtype_size(src_dtype), de = mrl_dtype_size(dst_dtype);
+    if (rank == 1 && dim_s == 0 && dim_d == 0 && src_dtype != dst_dtype && p.count >= 1024 &&
+        (reinterpret_cast<uintptr_t>(src) % (4 * se)) == 0 && (reinterpret_cast<uintptr_t>(dst) % (4 * de)) == 0) {
+      const uint32_t blocks = uint32_t(std::min<uint64_t>((p.count / 4 + 255) / 256, 1u << 20));
+      const dim3 grid{blocks}, block{256};
+#define MRL_CONVERT(SE, DE) \
+  if (se == SE && de == DE) hipLaunchKernelGGL((k_convert4<SE, DE>), grid, block, 0, stream, src, dst, src_dtype, dst_dtype, p.count)
+      MRL_CONVERT(1, 1); MRL_CONVERT(1, 2); MRL_CONVERT(1, 4);
+      MRL_CONVERT(2, 1); MRL_CONVERT(2, 2); MRL_CONVERT(2, 4);
+      MRL_CONVERT(4, 1); MRL_CONVERT(4, 2); MRL_CONVERT(4, 4);
+#undef MRL_CONVERT
+      return hipGetLastError();
+    }
     if (vectors) {
       for (uint32_t d = 0; d < rank; d++) {
         if (int(d) == dim_s) p.shape[d] /= uint32_t(per);

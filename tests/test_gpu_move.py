@@ -19,15 +19,15 @@ def test_move_plain_copy(gpu):
 
 @pytest.mark.parametrize("sdt,ddt", [(M.i32, M.u8), (M.u8, M.i32), (M.u8, M.f32), (M.f32, M.i8), (M.f32, M.u16),
                                      (M.f32, M.bf16), (M.bf16, M.f32), (M.i8, M.bf16), (M.bf16, M.i32)])
-def test_move_casts(gpu, sdt, ddt):
-    shape = [5, 129]
+@pytest.mark.parametrize("shape", [[5, 129], [3, 4099]])   # the second: four elements per thread plus a tail
+def test_move_casts(gpu, sdt, ddt, shape):
     if sdt == M.f32:
         x = (synth.normal_f32(402, 0, shape) * 200).astype(np.float32)
         x[0, :4] = [np.nan, 1e20, -1e20, 0.5]
     elif sdt == M.bf16:
         x = synth.f32_to_bf16_bits(synth.normal_f32(402, 0, shape) * 200)
     else:
-        x = synth.raw_u64(402, 0, 5 * 129).astype(sdt.numpy).reshape(shape)
+        x = synth.raw_u64(402, 0, shape[0] * shape[1]).astype(sdt.numpy).reshape(shape)
     got = run_spec(M.Move(shape, (sdt, ddt)), [x, np.zeros(shape, ddt.numpy)])
     want = orc.move(shape, [int(sdt), int(ddt)], x, np.zeros(shape, ddt.numpy))
     assert np.array_equal(got, want)
