@@ -113,6 +113,10 @@ __device__ inline uint32_t float_to_int(float f, int dt) {
 
 // One element: read as `sdt`, converted with Rust `as` semantics, returned as the bits of `ddt`.
 __device__ inline uint32_t move_bits(const void *src, int sdt, int64_t so, int ddt) {
+  if (sdt == ddt) {  // bits as they are (a NaN keeps its payload)
+    const size_t size = sdt == MRL_U8 || sdt == MRL_I8 ? 1 : sdt == MRL_U16 || sdt == MRL_I16 || sdt == MRL_BF16 ? 2 : 4;
+    return size == 1 ? ((const uint8_t *)src)[so] : size == 2 ? ((const uint16_t *)src)[so] : ((const uint32_t *)src)[so];
+  }
   const bool src_float = sdt == MRL_F32 || sdt == MRL_BF16;
   if (ddt == MRL_F32) return __float_as_uint(load_f32(src, sdt, so));
   if (ddt == MRL_BF16) return f32_to_bf16_bits(load_f32(src, sdt, so));
@@ -134,6 +138,7 @@ __device__ inline float raw_to_f32(uint32_t raw, int dtype) {
   }
 }
 __device__ inline uint32_t convert_raw(uint32_t raw, int sdt, int ddt) {
+  if (sdt == ddt) return raw;
   const bool src_float = sdt == MRL_F32 || sdt == MRL_BF16;
   if (ddt == MRL_F32) return __float_as_uint(raw_to_f32(raw, sdt));
   if (ddt == MRL_BF16) return f32_to_bf16_bits(raw_to_f32(raw, sdt));
@@ -259,6 +264,43 @@ __global__ __launch_bounds__(256) void k_move_tiled(MoveStrided p) {
   for (uint32_t r = quad; r < 64; r += 4)
     if (s0 + r < ns && d0 + lane < nd)
       store_u32(p.dst, p.ddt, d_o + int64_t(s0 + r) * p.ds[p.dim_s] + int64_t(d0 + lane) * p.ds[p.dim_d], tile[lane][r]);
+}
+
+// The same transpose for 16-bit elements that are not converted: 128 x 128 tiles, two elements
+// (one dword) per lane on both sides.  Needs even extents along both contiguous dims and even
+// strides elsewhere, so that every dword is whole and aligned.
+__global__ __launch_bounds__(256) void k_move_tiled16(MoveStrided p) {
+  __shared__ uint16_t tile[128][130];
+  uint64_t blk = blockIdx.x;
+  const uint32_t ts = uint32_t(blk % p.tiles_s);
+  blk /= p.tiles_s;
+  const uint32_t td = uint32_t(blk % p.tiles_d);
+  blk /= p.tiles_d;
+  int64_t so = 0, d_o = 0;
+  for (int o = int(p.rank) - 1; o >= 0; o--) {
+    const uint32_t d = p.order[o];
+    if (d == p.dim_s || d == p.dim_d) continue;
+    const uint32_t c = uint32_t(blk % p.shape[d]);
+    blk /= p.shape[d];
+    so += int64_t(c) * p.ss[d], d_o += int64_t(c) * p.ds[d];
+  }
+  const uint32_t lane = threadIdx.x & 63, quad = threadIdx.x >> 6;
+  const uint32_t s0 = ts * 128, d0 = td * 128, ns = p.shape[p.dim_s], nd = p.shape[p.dim_d];
+  const uint16_t *src = static_cast<const uint16_t *>(p.src);
+  uint16_t *dst = static_cast<uint16_t *>(p.dst);
+#pragma unroll 4
+  for (uint32_t r = quad; r < 128; r += 4)
+    if (d0 + r < nd && s0 + 2 * lane < ns) {
+      const uint32_t pair = *(const uint32_t *)(src + so + int64_t(d0 + r) * p.ss[p.dim_d] + (s0 + 2 * lane));
+      tile[r][2 * lane] = uint16_t(pair), tile[r][2 * lane + 1] = uint16_t(pair >> 16);
+    }
+  __syncthreads();
+#pragma unroll 4
+  for (uint32_t r = quad; r < 128; r += 4)
+    if (s0 + r < ns && d0 + 2 * lane < nd) {
+      const uint32_t pair = uint32_t(tile[2 * lane][r]) | (uint32_t(tile[2 * lane + 1][r]) << 16);
+      *(uint32_t *)(dst + d_o + int64_t(s0 + r) * p.ds[p.dim_s] + (d0 + 2 * lane)) = pair;
+    }
 }
 
 // Any other pair of contiguous dims (a Packed(8) digit on one side, say, too short for the
@@ -770,12 +812,20 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
   // Two long contiguous dims: the 64 x 64 transpose.
   if (dim_s != dim_d && p.shape[dim_s] >= 32 && p.shape[dim_d] >= 32) {
     p.dim_s = uint32_t(dim_s), p.dim_d = uint32_t(dim_d);
-    p.tiles_s = (p.shape[dim_s] + 63) / 64, p.tiles_d = (p.shape[dim_d] + 63) / 64;
+    // 16-bit elements, nothing converted, every dword whole and aligned: two elements per lane.
+    bool pairs = src_dtype == dst_dtype && mrl_dtype_size(src_dtype) == 2 && p.shape[dim_s] % 2 == 0 &&
+                 p.shape[dim_d] % 2 == 0 && (reinterpret_cast<uintptr_t>(src) & 3) == 0 &&
+                 (reinterpret_cast<uintptr_t>(dst) & 3) == 0;
+    for (uint32_t d = 0; pairs && d < p.rank; d++)
+      pairs = (int(d) == dim_s || p.ss[d] % 2 == 0) && (int(d) == dim_d || p.ds[d] % 2 == 0);
+    const uint32_t side = pairs ? 128 : 64;
+    p.tiles_s = (p.shape[dim_s] + side - 1) / side, p.tiles_d = (p.shape[dim_d] + side - 1) / side;
     uint64_t blocks = uint64_t(p.tiles_s) * p.tiles_d;
     for (uint32_t d = 0; d < p.rank; d++)
       if (int(d) != dim_s && int(d) != dim_d) blocks *= p.shape[d];
     if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(k_move_tiled, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+    if (pairs) hipLaunchKernelGGL(k_move_tiled16, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL(k_move_tiled, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
     return hipGetLastError();
   }
   // Otherwise a tile grown digit by digit: along the destination's fastest digits until they

@@ -114,3 +114,16 @@ def test_host_threads_share_a_stream_and_its_scratch(gpu):
     for spec, bufs, want, shape in jobs:
         assert np.array_equal(bufs[2].to_numpy(np.int32, shape), rounds * want)
     stream.destroy()
+
+
+@pytest.mark.parametrize("dt", [M.bf16, M.i16, M.u16])
+@pytest.mark.parametrize("shape", [(2, 200, 136), (1, 130, 258), (3, 64, 64), (1, 1000, 2), (2, 33, 64), (1, 2048, 128)])
+def test_transpose_of_16_bit_elements(gpu, dt, shape):
+    """Row-major <-> batched column-major of 16-bit elements: two elements per lane on both sides
+    where the extents are even, one where they are not."""
+    x = synth.raw_u64(830, 0, int(np.prod(shape))).astype(np.uint16).reshape(shape)
+    cm = M.batched_col_major(list(shape))
+    got = run_spec(M.Move(list(shape), (dt, dt), layouts=[None, cm]), [x, np.zeros((shape[0], shape[2], shape[1]), np.uint16)])
+    assert np.array_equal(got, x.transpose(0, 2, 1))
+    back = run_spec(M.Move(list(shape), (dt, dt), layouts=[cm, None]), [got, np.zeros(shape, np.uint16)])
+    assert np.array_equal(back, x)
