@@ -516,8 +516,9 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
   // Windows of this many images are unfolded at a time.
   constexpr uint64_t UNFOLD_BYTES = uint64_t(1) << 30;
   const uint64_t image_rows_bytes = pixels * row_elems * img.elem;
-  const bool as_matmul = !fused_shape && kind >= 0 && image_rows_bytes <= UNFOLD_BYTES && row_elems * img.elem < (1u << 24) &&
+  const bool as_matmul = !fused_shape && kind >= 0 && row_elems * img.elem < (1u << 24) &&
                          double(cv.b) * pixels * cv.f * window >= 1e6;
+  const bool can_unfold = image_rows_bytes <= UNFOLD_BYTES;
   // Tensors in another permutation layout (NCHW, say) are moved to channels-last when a
   // matrix-core path takes the shape: three small extra passes against a generic kernel
   // that is hundreds of times slower.
@@ -540,10 +541,31 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
     if ((rc = to_channels_last(out, s.accum != 0)) != MRL_OK) return rc;
     cv.image = img.t.ptr, cv.filters = filt.t.ptr, cv.out = out.t.ptr;
   }
+  // The Conv as an implicit Matmul: left operand = the image's windows, B = the KRSC filters.
+  mrl::GemmArgs conv_args;
+  auto implicit_args = [&](mrl::GemmArgs *g) {
+    const uint64_t c_bytes = uint64_t(cv.c) * img.elem, h = cv.oh + cv.fh - 1, w = cv.ow + cv.fw - 1;
+    if (c_bytes % 16 != 0 || uint64_t(cv.b) * pixels >= (1ull << 31)) return false;
+    g->a = img.t.ptr, g->b = filt.t.ptr, g->c = out.t.ptr;
+    g->batch = 1, g->m = uint32_t(cv.b * pixels), g->n = cv.f, g->k = uint32_t(window);
+    g->lda = 0, g->ldb = int64_t(window), g->ldc = cv.f;
+    g->sa = g->sb = g->sc = 0;
+    g->accum = s.accum;
+    g->b_kmajor = true;
+    g->conv.h = uint32_t(h), g->conv.w = uint32_t(w), g->conv.oh = cv.oh, g->conv.ow = cv.ow, g->conv.fw = cv.fw;
+    g->conv.c_bytes = uint32_t(c_bytes);
+    g->conv.image_bytes = uint64_t(cv.b) * h * w * c_bytes;
+    return true;
+  };
   if (fast_types && channels_last(img.t) && channels_last(filt.t) && channels_last(out.t) &&
       mrl::conv_i8_applicable(cv)) {
     HIP_TRY(mrl::launch_conv_i8(cv, di == MRL_U8, ws.stream));
-  } else if (as_matmul && (reinterpret_cast<uintptr_t>(img.t.ptr) & 15) == 0 &&
+  } else if (as_matmul && !(cv.fh == 1 && cv.fw == 1) && implicit_args(&conv_args) &&
+             mrl::conv_gemm_applicable(conv_args, kind)) {
+    // Channel vectors of whole 16-byte chunks: the windows are read where they lie.  (A 1x1 filter
+    // needs no window arithmetic: its image is the left operand of a plain Matmul, below.)
+    HIP_TRY(mrl::launch_conv_gemm(conv_args, kind, ws.stream));
+  } else if (as_matmul && can_unfold && (reinterpret_cast<uintptr_t>(img.t.ptr) & 15) == 0 &&
              (reinterpret_cast<uintptr_t>(filt.t.ptr) & 15) == 0 && (reinterpret_cast<uintptr_t>(out.t.ptr) & 3) == 0) {
     // Filters in KRSC order are the B operand stored k-fastest; their rows padded like U's.
     const void *weights = filt.t.ptr;

@@ -57,6 +57,8 @@ bool gemm_possible(const GemmArgs &g, int kind) {
 // included (int8 32 x 4096 x 4096: 23 us against 237 us; f32 16 x 64 x 16: 4.1 us against 3.6 us).
 bool gemm_pays(const GemmArgs &g, int) { return double(g.m) * g.n * g.k * g.batch >= 100e3; }
 
+uint32_t gemm_tile_side(const GemmArgs &g, int kind) { return tile_side(g, elem_size_of(kind)); }
+
 hipError_t launch_gemm_big(const GemmArgs &g, int kind, hipStream_t stream) {
   if (g.b_kmajor) return launch_gemm_nt(g, kind, 256, stream);
   const bool whole = whole_tiles(g, elem_size_of(kind));

@@ -226,8 +226,12 @@ __device__ inline void sched_slots(bool staging) {
 // B_KMAJOR: B is stored with k fastest (each of its n rows runs along K, `ldb` elements apart:
 // Morello's col_major / batched_col_major layouts, or layout![0,2,1]).  Its tile is then staged
 // and read exactly like A's, and no transposing read is involved.
-template <class T, bool A_UNSIGNED, class TL, bool EDGE, bool B_KMAJOR = false>
+// CONV (with EDGE and B_KMAJOR): the left operand is not a matrix in memory but the windows of
+// a channels-last image, g.conv; row p's 16-byte chunk at k byte kb lies at
+// corner(p) + ((r * w + s) * c_bytes + kb % c_bytes) with (r, s) = divmod(kb / c_bytes, fw).
+template <class T, bool A_UNSIGNED, class TL, bool EDGE, bool B_KMAJOR = false, bool CONV = false>
 __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int tiles_n) {
+  static_assert(!CONV || (EDGE && B_KMAJOR), "the implicit Conv operand is addressed through the buffer path");
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   constexpr int BM = TL::BM, BN = TL::BN, BKB = TL::BKB, WAVES_M = TL::WAVES_M, WAVES_N = TL::WAVES_N;
   constexpr int NT = TL::NT, A_STAGE = TL::A_STAGE;
@@ -337,6 +341,17 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
   const uint8_t *a_tile = A, *b_tile = B;
   const int a_rows = min(BM, int(g.m - m0)), b_rows = min(BN, int(g.n - n0));  // rows the tile owns
   const uint32_t a_off = uint32_t(tid / A_ROW_CH) * uint32_t(lda_b) + (tid % A_ROW_CH) * 16;
+  // CONV: byte offset of the window corner of each of the thread's rows (out of range past M).
+  uint32_t a_corner[A_CH];
+  if constexpr (CONV) {
+#pragma unroll
+    for (int i = 0; i < A_CH; i++) {
+      const int64_t p = m0 + tid / A_ROW_CH + i * A_ROWS_PER_I;
+      const uint32_t q = uint32_t(min(p, int64_t(g.m) - 1));
+      const uint32_t x = q % g.conv.ow, y = (q / g.conv.ow) % g.conv.oh, img = q / (g.conv.ow * g.conv.oh);
+      a_corner[i] = p < int64_t(g.m) ? ((img * g.conv.h + y) * g.conv.w + x) * g.conv.c_bytes : OUT_OF_RANGE;
+    }
+  }
   const uint32_t b_off = uint32_t(tid / B_ROW_CH) * uint32_t(ldb_b) + (tid % B_ROW_CH) * 16;
   const int a_kb0 = (tid % A_ROW_CH) * 16;  // the thread's k byte within a tile
   const int b_kb0 = (tid % B_ROW_CH) * 16;  // B_KMAJOR: likewise
@@ -345,12 +360,22 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
   // Loads the next tile in sequence and advances the source pointers.
   auto load_global = [&]() {
     if constexpr (EDGE) {
-      const auto a_buf = buffer_of(a_tile, int64_t(a_rows) * lda_b - ld_kb);
       const bool a_in = ld_kb + a_kb0 < k_bytes;
+      if constexpr (CONV) {
+        const auto a_buf = buffer_of(g.a, int64_t(g.conv.image_bytes));
+        const uint32_t kb = uint32_t(ld_kb + a_kb0), pos = kb / g.conv.c_bytes, r = pos / g.conv.fw;
+        const uint32_t in_window = ((r * g.conv.w + (pos - r * g.conv.fw)) * g.conv.c_bytes) + (kb - pos * g.conv.c_bytes);
 #pragma unroll
-      for (int i = 0; i < A_CH; i++)
-        a_reg[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(
-                                               a_buf, a_in ? a_off + i * uint32_t(a_step_i) : OUT_OF_RANGE, 0, 0));
+        for (int i = 0; i < A_CH; i++)
+          a_reg[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(
+                                                 a_buf, a_in && a_corner[i] != OUT_OF_RANGE ? a_corner[i] + in_window : OUT_OF_RANGE, 0, 0));
+      } else {
+        const auto a_buf = buffer_of(a_tile, int64_t(a_rows) * lda_b - ld_kb);
+#pragma unroll
+        for (int i = 0; i < A_CH; i++)
+          a_reg[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(
+                                                 a_buf, a_in ? a_off + i * uint32_t(a_step_i) : OUT_OF_RANGE, 0, 0));
+      }
       if constexpr (B_KMAJOR) {
         const auto b_buf = buffer_of(b_tile, int64_t(b_rows) * ldb_b - ld_kb);
         const bool b_in = ld_kb + b_kb0 < k_bytes;
@@ -481,9 +506,9 @@ inline bool edge_addressable(const GemmArgs &g, int elem_size) {
          g.ldc * 4 < EDGE_MAX_ROW_BYTES;
 }
 
-template <class T, bool A_UNSIGNED, class TL, bool EDGE, bool B_KMAJOR = false>
+template <class T, bool A_UNSIGNED, class TL, bool EDGE, bool B_KMAJOR = false, bool CONV = false>
 hipError_t launch(const GemmArgs &g, hipStream_t stream) {
-  auto kern = k_gemm<T, A_UNSIGNED, TL, EDGE, B_KMAJOR>;
+  auto kern = k_gemm<T, A_UNSIGNED, TL, EDGE, B_KMAJOR, CONV>;
   constexpr int BM = TL::BM, BN = TL::BN;
   constexpr int STAGE = TL::template stage<T>();
   if (EDGE && !edge_addressable(g, T::ES)) return hipErrorInvalidValue;

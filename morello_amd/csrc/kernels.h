@@ -60,10 +60,21 @@ struct GemmArgs {
   // false: B rows run along N (`ldb` = elements between k rows); true: B rows run along K
   // (`ldb` = elements between n rows), as col_major / layout![0,2,1] store it.
   bool b_kmajor = false;
+  // Conv as an implicit Matmul (the CONV build of the kernel): `a` is a channels-last image
+  // [batch][h][w][c], row p of the left operand is the window of output pixel p (fh runs of
+  // fw * c contiguous elements), never materialised.  m = batch * oh * ow, k = fh * fw * c.
+  struct {
+    uint32_t h, w, oh, ow, fw;
+    uint32_t c_bytes;       // bytes of one pixel's channels (a whole number of 16-byte chunks)
+    uint64_t image_bytes;   // all of `a`
+  } conv = {};
 };
 // kind: 0 = i8 x i8, 1 = u8 x i8, 2 = bf16 x bf16, 3 = f32 x f32; B stored k-fastest (gemm_nt.hip).
 // tile: 64, 128 or 256 (square workgroup tiles).
 hipError_t launch_gemm_nt(const GemmArgs &g, int kind, uint32_t tile, hipStream_t stream);
+// Conv as an implicit Matmul (g.conv filled in, B = the KRSC filters, k-fastest); tile chosen by size.
+bool conv_gemm_applicable(const GemmArgs &g, int kind);
+hipError_t launch_conv_gemm(const GemmArgs &g, int kind, hipStream_t stream);
 // kind: 0 = i8 x i8 -> i32, 1 = u8 x i8 -> i32, 2 = bf16 x bf16 -> f32, 3 = f32 x f32 -> f32.
 // Shapes, leading dimensions and alignment the kernel can walk.
 bool gemm_possible(const GemmArgs &g, int kind);
@@ -71,6 +82,8 @@ bool gemm_possible(const GemmArgs &g, int kind);
 bool gemm_pays(const GemmArgs &g, int kind);
 // Tile chosen by size: 256 x 256 with enough tiles to occupy the chip, else 128 x 128 or 64 x 64.
 hipError_t launch_gemm(const GemmArgs &g, int kind, hipStream_t stream);
+// Side of the square tile launch_gemm would take for this size: 64, 128 or 256.
+uint32_t gemm_tile_side(const GemmArgs &g, int kind);
 // Always the 256 x 256 tile, 128 bytes of K per step.
 hipError_t launch_gemm_big(const GemmArgs &g, int kind, hipStream_t stream);
 

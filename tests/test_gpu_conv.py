@@ -87,10 +87,14 @@ CONV_GEN = {M.u8: synth.uniform_u8, M.i8: synth.uniform_i8, M.bf16: synth.normal
     ((2, 64, 32, 12, 12, 5, 5), False),    # 64 filters but not the fused kernel's channel count
     ((1, 7, 20, 30, 30, 2, 4), True),      # few filters, uneven window
     ((5, 96, 64, 14, 14, 3, 3), False),    # 64 channels but not the fused kernel's filter count
+    ((2, 130, 128, 17, 19, 3, 3), True),   # implicit for every dtype: 18 slabs of 64 channels, ragged everywhere
+    ((1, 64, 16, 70, 70, 5, 5), False),    # 16 channels: implicit for int8 too, windows of 400 elements
+    ((3, 256, 32, 9, 9, 2, 2), True),
 ])
 def test_conv_as_matmul(gpu, dts, codes, shape, accum):
-    """Shapes outside the fused kernel's (64 filters, channels in 64s, 1x1 or 3x3) are unfolded into
-    rows of windows and run as a Matmul on the matrix cores, for every dtype triple those take."""
+    """Shapes outside the fused kernel's run as a Matmul on the matrix cores, for every dtype triple
+    those take: implicitly (the kernel reads the windows where they lie) when a pixel's channels
+    are whole 16-byte chunks, through windows unfolded into rows otherwise."""
     b, f, c, oh, ow, fh, fw = shape
     img = CONV_GEN[dts[0]](131, 0, (b, oh + fh - 1, ow + fw - 1, c))
     filt = CONV_GEN[dts[1]](131, 1, (f, fh, fw, c))
