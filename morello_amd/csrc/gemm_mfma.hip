@@ -2,6 +2,8 @@
 // manual schedule the workgroup tile is chosen from the problem size (the reference prices
 // schedules with a cost model before it emits one, morello/src/cost.rs; here the table is
 // three entries long and comes from measurement).
+#include <algorithm>
+
 #include "gemm_mfma_kernel.h"
 
 namespace mrl {
@@ -35,11 +37,14 @@ bool applicable(const GemmArgs &g, int es) {
 //   f32: its MFMA has a sixteenth of the int8 rate, so operand traffic never limits a small
 //     tile: 64 (1024^3: 27 us against 70 and 239; 3072^3: 460 against 559 and 711) until the
 //     256 tile fills its rounds (4096^3: 948 us against 1066).
+// A tile wider than the matrix is mostly padding: at most 64 (128) rows or columns cap the side
+// at 64 (128) whatever the counts say.
 uint32_t tile_side(const GemmArgs &g, int es) {
+  const uint32_t narrow = std::min(g.m, g.n), cap = narrow <= 64 ? 64 : narrow <= 128 ? 128 : 256;
   const uint64_t big = uint64_t((g.m + 255) / 256) * ((g.n + 255) / 256) * g.batch;
   const double round_fill = double(big) / double((big + 255) / 256 * 256);
-  if (round_fill >= (es == 4 ? 0.85 : 0.5)) return 256;
-  if (es == 4) return 64;
+  if (cap == 256 && round_fill >= (es == 4 ? 0.85 : 0.5)) return 256;
+  if (es == 4 || cap == 64) return 64;
   const uint64_t small = uint64_t((g.m + 63) / 64) * ((g.n + 63) / 64) * g.batch;
   return small <= 384 ? 64 : 128;
 }
