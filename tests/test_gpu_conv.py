@@ -123,18 +123,40 @@ def test_conv_as_matmul_from_nchw(gpu):
 
 
 def test_conv_as_matmul_in_several_passes(gpu):
-    """More windows than one pass unfolds (1 GiB of rows): the batch is cut into passes.  Checked
-    on the first and last image and through the per-image checksum."""
-    # 62 500 windows of 1024 bytes per image: 16 images per pass, so passes of 16, 16 and 4
-    b, f, c, oh, ow, fh, fw = shape = (36, 8, 64, 250, 250, 4, 4)
+    """Three channels (windows are unfolded into rows) and more windows than one pass unfolds
+    (1 GiB of rows): the batch is cut into passes.  Checked on the first, a middle and the last
+    image and through the per-image checksum."""
+    # 62 500 windows of 147 bytes padded to 160 per image: 107 images per pass, so passes of 107 and 3
+    b, f, c, oh, ow, fh, fw = shape = (110, 8, 3, 250, 250, 7, 7)
     img = synth.uniform_u8(133, 0, (b, oh + fh - 1, ow + fw - 1, c))
     filt = synth.uniform_i8(133, 1, (f, fh, fw, c))
     got = run_spec(M.Conv(shape, (M.u8, M.i8, M.i32)), [img, filt, np.zeros((b, oh, ow, f), np.int32)])
-    for bi in (0, 16, 35):
+    for bi in (0, 106, 107, 109):
         sub = (1,) + shape[1:]
         want = orc.conv(list(sub), [0, 1, 5], img[bi:bi + 1], filt, np.zeros((1, oh, ow, f), np.int32), layouts=[NHWC] * 3)
         assert np.array_equal(got[bi:bi + 1], want)
     fsum = filt.astype(np.int64).sum(axis=0)  # [r,s,c]
+    for bi in range(b):
+        im = img[bi].astype(np.int64)
+        total = 0
+        for r in range(fh):
+            for s in range(fw):
+                total += int((im[r:r + oh, s:s + ow, :].sum(axis=(0, 1)) * fsum[r, s]).sum())
+        assert int(got[bi].astype(np.int64).sum()) == total
+
+
+def test_implicit_conv_at_a_large_image_count(gpu):
+    """The implicit Matmul form at 2.3 million windows (row offsets of the left operand up to
+    150 MB into the image): first and last image against the oracle, all through the checksum."""
+    b, f, c, oh, ow, fh, fw = shape = (36, 8, 64, 250, 250, 4, 4)
+    img = synth.uniform_u8(134, 0, (b, oh + fh - 1, ow + fw - 1, c))
+    filt = synth.uniform_i8(134, 1, (f, fh, fw, c))
+    got = run_spec(M.Conv(shape, (M.u8, M.i8, M.i32)), [img, filt, np.zeros((b, oh, ow, f), np.int32)])
+    for bi in (0, 35):
+        sub = (1,) + shape[1:]
+        want = orc.conv(list(sub), [0, 1, 5], img[bi:bi + 1], filt, np.zeros((1, oh, ow, f), np.int32), layouts=[NHWC] * 3)
+        assert np.array_equal(got[bi:bi + 1], want)
+    fsum = filt.astype(np.int64).sum(axis=0)
     for bi in range(b):
         im = img[bi].astype(np.int64)
         total = 0
