@@ -680,12 +680,26 @@ int run_compose_msm(const mrl_spec &s, void *const *params, Workspace &ws) {
     k_fastest.dims[0] = {0, MRL_DYNAMIC, 0}, k_fastest.dims[1] = {2, MRL_DYNAMIC, 0}, k_fastest.dims[2] = {1, MRL_DYNAMIC, 0};
     mrl::AttnArgs at;
     at.b = b, at.m = m, at.k = at.n = dp, at.n2 = n2, at.n_out = n;
+    // KT row-major as the reference lays it out by default ([b, k, n2], n2 fastest) is read in
+    // place by the kernel's own build for it; any other order is brought to k-fastest.
+    auto kt_operand = [&]() -> int {
+      mrl_layout rows_kt;
+      mrl_layout_row_major(kt_shape, 3, &rows_kt);
+      std::vector<mrl::MoveDim> view;
+      if (k == dp && n2 % 8 == 0 && (reinterpret_cast<uintptr_t>(params[2]) & 15) == 0 &&
+          mrl::common_view(s.layouts[2], rows_kt, kt_shape, 3, &view) &&
+          (view.empty() || (view.size() == 1 && view[0].ss == 1 && view[0].ds == 1))) {
+        at.kt = params[2], at.kt_rows = true;
+        return MRL_OK;
+      }
+      return operand(2, kt_shape, k_fastest, n2, k, &at.kt);
+    };
     std::vector<mrl::MoveDim> out_view;
     int rc = MRL_OK;
     if (mrl::common_view(rows_o, s.layouts[3], o_shape, 3, &out_view) &&
         (rc = operand(0, v_shape, rows_v, n2, n, &at.v)) == MRL_OK &&
         (rc = operand(1, q_shape, rows_q, m, k, &at.q)) == MRL_OK &&
-        (rc = operand(2, kt_shape, k_fastest, n2, k, &at.kt)) == MRL_OK) {
+        (rc = kt_operand()) == MRL_OK) {
       const bool out_in_order = out_view.empty() || (out_view.size() == 1 && out_view[0].ss == 1 && out_view[0].ds == 1);
       void *result = params[3];
       if (!out_in_order) HIP_TRY(ws.alloc(&result, size_t(b) * m * n * sizeof(float)));

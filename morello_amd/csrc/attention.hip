@@ -68,7 +68,12 @@ __device__ inline v2i read_tr16(const uint8_t *p) {
 // a clamped (valid) row and not stored; the key blocks are dealt ceil/floor to the two halves,
 // loads past the end of K / V are clamped to the entry's last 16 bytes (finite data, weighted
 // by exp(-inf) = 0), and the scores of keys past n2 are set to -inf before the softmax.
-template <int D, bool RAGGED>
+// KT_ROWS: KT is given row-major, [b][k][n2] with n2 fastest (the reference's default layout for
+// the Compose's third parameter) instead of k-fastest.  A block of 64 keys is then D rows of 128
+// bytes in LDS (one row per d), and the K operand comes out of it through the same transposing
+// read that serves V; the MFMA's k index runs over d in the order that read delivers (4 + 4
+// values per lane half), so Q's operand is loaded in that order too.  n2 must be a multiple of 8.
+template <int D, bool RAGGED, bool KT_ROWS>
 __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
   typedef Dims<D> DD;
   constexpr int ROW = DD::ROW, TILE = DD::TILE, STAGE = DD::STAGE, HALF = DD::HALF;
@@ -102,7 +107,14 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
   // Q^T operand: lane (query lq, half lg) holds d = 16*step + 8*lg .. +7.
   v4i qf[D / 16];
 #pragma unroll
-  for (int s = 0; s < D / 16; s++) qf[s] = *(const v4i *)(Q + s * 32 + lg * 16);
+  for (int s = 0; s < D / 16; s++) {
+    if constexpr (KT_ROWS) {
+      const v2i lo = *(const v2i *)(Q + s * 32 + lg * 8), hi = *(const v2i *)(Q + s * 32 + 16 + lg * 8);
+      qf[s] = v4i{lo[0], lo[1], hi[0], hi[1]};  // d = 16s + 4lg + 0..3, then 16s + 8 + 4lg + 0..3
+    } else {
+      qf[s] = *(const v4i *)(Q + s * 32 + lg * 16);
+    }
+  }
 
   // Block staging.  One direct-to-LDS instruction fills 1 KiB (4 rows at D = 128); lane l lands
   // in 16-byte slot l.  K rows are XOR-swizzled by chunk, V rows by 64-byte unit; each lane
@@ -115,12 +127,18 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
 #pragma unroll
   for (int i = 0; i < PER_WAVE; i++) {
     const int q = qg * PER_WAVE + i, row = q * DD::ROWS_PER_LOAD + ld_row;
-    k_src[i] = row * ROW + ((ld_pc ^ DD::k_swizzle(row)) << 4);
+    if constexpr (KT_ROWS) {
+      // 8 rows (d) of 128 bytes per instruction; 64-byte units swizzled like a V tile of D = 64.
+      const int krow = q * 8 + (lane >> 3), kpc = lane & 7;
+      k_src[i] = krow * (p.n2 * 2) + ((((kpc >> 2) ^ Dims<64>::v_swizzle(krow)) << 6) | ((kpc & 3) << 4));
+    } else {
+      k_src[i] = row * ROW + ((ld_pc ^ DD::k_swizzle(row)) << 4);
+    }
     v_src[i] = row * ROW + ((((ld_pc >> 2) ^ DD::v_swizzle(row)) << 6) | ((ld_pc & 3) << 4));
   }
   // Byte offset within the batch entry's K (V) of this lane's chunk i of block kb.
   auto k_off = [&](int kb, int i) {
-    const uint32_t off = uint32_t(first_block + kb) * TILE + k_src[i];
+    const uint32_t off = uint32_t(first_block + kb) * (KT_ROWS ? BKV * 2 : TILE) + k_src[i];
     return RAGGED ? min(off, head_bytes - 16) : off;
   };
   auto v_off = [&](int kb, int i) {
@@ -183,7 +201,14 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
 #pragma unroll
         for (int kt = 0; kt < BKV / 32; kt++) {
           const int row = kt * 32 + lq, st = 2 * q + c;
-          kf[buf][kt][c] = *(const v4i *)(lk + row * ROW + (((2 * st + lg) ^ DD::k_swizzle(row)) << 4));
+          if constexpr (KT_ROWS) {
+            const int drow = 16 * st + 4 * lg + v_rl;  // drow + 8 swizzles alike
+            const int off = ((kt ^ Dims<64>::v_swizzle(drow)) << 6) + v_within;
+            const v2i lo = read_tr16(lk + drow * (BKV * 2) + off), hi = read_tr16(lk + (drow + 8) * (BKV * 2) + off);
+            kf[buf][kt][c] = v4i{lo[0], lo[1], hi[0], hi[1]};
+          } else {
+            kf[buf][kt][c] = *(const v4i *)(lk + row * ROW + (((2 * st + lg) ^ DD::k_swizzle(row)) << 4));
+          }
         }
     };
 #pragma unroll
@@ -203,10 +228,10 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
           s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, kf[q % 3][kt][c]),
                                                           __builtin_bit_cast(v8bf, qf[2 * q + c]), s[kt], 0, 0, 0);
     }
-    __builtin_amdgcn_sched_group_barrier(0x100, (D / 32 > 1 ? 4 : 2) * (BKV / 32), 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, (KT_ROWS ? 2 : 1) * (D / 32 > 1 ? 4 : 2) * (BKV / 32), 0);
 #pragma unroll
     for (int q = 0; q < D / 32; q++) {
-      if (q + 2 < D / 32) __builtin_amdgcn_sched_group_barrier(0x100, 2 * (BKV / 32), 0);
+      if (q + 2 < D / 32) __builtin_amdgcn_sched_group_barrier(0x100, (KT_ROWS ? 4 : 2) * (BKV / 32), 0);
       __builtin_amdgcn_sched_group_barrier(0x008, BKV / 32, 0);
       __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x008, BKV / 32, 0);
@@ -330,26 +355,31 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
 bool attn_applicable(const AttnArgs &a) {
   auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
   return a.k == a.n && (a.k == 32 || a.k == 64 || a.k == 128) && a.n_out >= 1 && a.n_out <= a.n && a.m && a.n2 && a.b &&
+         (!a.kt_rows || a.n2 % 8 == 0) &&
          uint64_t(a.n2) * a.k * 2 < (1ull << 31) && uint64_t((a.m + BQ - 1) / BQ) * a.b < (1u << 31) &&
          al16(a.q) && al16(a.kt) && al16(a.v) && al16(a.out);
 }
 
 namespace {
-template <int D>
-hipError_t launch_for(const AttnArgs &a, hipStream_t stream) {
+template <int D, bool RAGGED, bool KT_ROWS>
+hipError_t launch_one(const AttnArgs &a, hipStream_t stream) {
   constexpr int LDS = Dims<D>::LDS_BYTES;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void *)k_attn<D, false>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void *)k_attn<D, true>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+    hipError_t e = hipFuncSetAttribute((const void *)k_attn<D, RAGGED, KT_ROWS>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
     if (e != hipSuccess) return e;
     attr_set = true;
   }
   const dim3 grid(((a.m + BQ - 1) / BQ) * a.b);
-  if (a.m % BQ == 0 && a.n2 % (2 * BKV) == 0) hipLaunchKernelGGL((k_attn<D, false>), grid, dim3(512), LDS, stream, a);
-  else hipLaunchKernelGGL((k_attn<D, true>), grid, dim3(512), LDS, stream, a);
+  hipLaunchKernelGGL((k_attn<D, RAGGED, KT_ROWS>), grid, dim3(512), LDS, stream, a);
   return hipGetLastError();
+}
+
+template <int D>
+hipError_t launch_for(const AttnArgs &a, hipStream_t stream) {
+  const bool whole = a.m % BQ == 0 && a.n2 % (2 * BKV) == 0;
+  if (a.kt_rows) return whole ? launch_one<D, false, true>(a, stream) : launch_one<D, true, true>(a, stream);
+  return whole ? launch_one<D, false, false>(a, stream) : launch_one<D, true, false>(a, stream);
 }
 }  // namespace
 

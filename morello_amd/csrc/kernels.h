@@ -141,13 +141,14 @@ hipError_t measure_mfma_rate(int kind, bool random_operands, uint32_t iters, hip
 // ---- attention.hip: fused Matmul -> Softmax -> Matmul on bf16 inputs -------------------
 struct AttnArgs {
   const void *q;   // [b, m, k]   bf16 row-major
-  const void *kt;  // logical [b, k, n2] stored as [b, n2, k] (K row-major)
+  const void *kt;  // logical [b, k, n2]: stored as [b, n2, k] (K row-major), or as it reads when kt_rows
   const void *v;   // [b, n2, n]  bf16 row-major
   float *out;      // [b, m, n_out] f32 row-major
   uint32_t b, m, k, n2, n;
   // Columns of the result that exist in `out` (its rows are n_out floats): n, or fewer when V
   // was padded with zero columns up to a head dim the kernel is built for.
   uint32_t n_out;
+  bool kt_rows = false;  // KT stored row-major, n2 fastest (n2 a multiple of 8)
 };
 bool attn_applicable(const AttnArgs &a);
 hipError_t launch_attn(const AttnArgs &a, hipStream_t stream);

@@ -138,12 +138,16 @@ def test_compose_msm_f32_inputs_stay_staged(gpu):
     assert rel_err(got, want) < 1e-5
 
 
-@pytest.mark.parametrize("dims", [(2, 40, 32, 48, 24), (2, 256, 128, 384, 128), (1, 200, 64, 130, 64)])
+@pytest.mark.parametrize("dims", [(2, 40, 32, 48, 24), (2, 256, 128, 384, 128), (1, 200, 64, 130, 64),
+                                  (1, 128, 64, 256, 64), (2, 136, 128, 1000, 128), (1, 77, 32, 72, 32),
+                                  (3, 128, 32, 128, 32), (1, 300, 64, 2056, 64), (1, 64, 128, 8, 128)])
 def test_compose_msm_fused_from_other_layouts(gpu, dims):
     """The reference's default layouts (everything row-major, KT as [b, k, n2] with n2 fastest,
     examples/matmul_chain.rs:26-57), a batched column-major Q, a V with a Packed dim and a batched column-major
-    result: each is brought to the order the fused kernel reads (one copy) and the result moved
-    out, within the composed pipeline's tolerance."""
+    result.  A row-major KT whose n2 is a multiple of 8 is read in place by the kernel's build for
+    it (whole and ragged sequence lengths, head dims 32 / 64 / 128); everything else is brought
+    to the order the fused kernel reads (one copy) and the result moved out.  Within the composed
+    pipeline's tolerance."""
     b, m, k, n2, n = dims
     q, kmat, v = msm_inputs(306, *dims)
     kt = np.ascontiguousarray(kmat.transpose(0, 2, 1))                       # [b, k, n2] row-major
