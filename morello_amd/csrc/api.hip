@@ -332,7 +332,7 @@ int prepare(const mrl_spec &s, uint32_t idx, void *ptr, bool needs_read, Workspa
   // A layout with Packed dims can still be row-major order (layout![0, 1, 1p16], say).
   std::vector<mrl::MoveDim> view;
   if (mrl::common_view(s.layouts[idx], dense, shape, rank, &view) &&
-      (view.empty() || (view.size() == 1 && view[0].ss == 1 && view[0].ds == 1))) {
+      mrl::same_order(view)) {
     out->t.ptr = ptr;
     mrl::layout_strides(dense, shape, rank, out->t.stride);
     return MRL_OK;
@@ -651,7 +651,7 @@ int run_compose_msm(const mrl_spec &s, void *const *params, Workspace &ws) {
       const void *dense = params[i];
       std::vector<mrl::MoveDim> view;
       if (!mrl::common_view(s.layouts[i], want, shape, 3, &view)) return MRL_ERR_UNSUPPORTED;
-      const bool in_order = view.empty() || (view.size() == 1 && view[0].ss == 1 && view[0].ds == 1);
+      const bool in_order = mrl::same_order(view);
       if (!in_order) {
         void *buf = nullptr;
         HIP_TRY(ws.alloc(&buf, size_t(b) * rows * cols * 2));
@@ -687,8 +687,7 @@ int run_compose_msm(const mrl_spec &s, void *const *params, Workspace &ws) {
       mrl_layout_row_major(kt_shape, 3, &rows_kt);
       std::vector<mrl::MoveDim> view;
       if (k == dp && n2 % 8 == 0 && (reinterpret_cast<uintptr_t>(params[2]) & 15) == 0 &&
-          mrl::common_view(s.layouts[2], rows_kt, kt_shape, 3, &view) &&
-          (view.empty() || (view.size() == 1 && view[0].ss == 1 && view[0].ds == 1))) {
+          mrl::common_view(s.layouts[2], rows_kt, kt_shape, 3, &view) && mrl::same_order(view)) {
         at.kt = params[2], at.kt_rows = true;
         return MRL_OK;
       }
@@ -700,7 +699,7 @@ int run_compose_msm(const mrl_spec &s, void *const *params, Workspace &ws) {
         (rc = operand(0, v_shape, rows_v, n2, n, &at.v)) == MRL_OK &&
         (rc = operand(1, q_shape, rows_q, m, k, &at.q)) == MRL_OK &&
         (rc = kt_operand()) == MRL_OK) {
-      const bool out_in_order = out_view.empty() || (out_view.size() == 1 && out_view[0].ss == 1 && out_view[0].ds == 1);
+      const bool out_in_order = mrl::same_order(out_view);
       void *result = params[3];
       if (!out_in_order) HIP_TRY(ws.alloc(&result, size_t(b) * m * n * sizeof(float)));
       at.out = static_cast<float *>(result);
@@ -1173,8 +1172,7 @@ size_t mrl_spec_workspace_bytes(const mrl_spec *spec) {
     mrl_layout dense;
     mrl_layout_row_major(shape, rank, &dense);
     std::vector<mrl::MoveDim> view;
-    if (mrl::common_view(spec->layouts[i], dense, shape, rank, &view) &&
-        (view.empty() || (view.size() == 1 && view[0].ss == 1 && view[0].ds == 1)))
+    if (mrl::common_view(spec->layouts[i], dense, shape, rank, &view) && mrl::same_order(view))
       continue;  // Packed dims in row-major order
     total += size_t(volume(shape, rank)) * mrl_dtype_size(spec->dtypes[i]);
   }

@@ -103,4 +103,9 @@ inline bool common_view(const mrl_layout &src, const mrl_layout &dst, const uint
   return view->size() <= MOVE_MAX_RANK;
 }
 
+// Whether a common view says that both sides store the elements in the same order.
+inline bool same_order(const std::vector<MoveDim> &view) {
+  return view.empty() || (view.size() == 1 && view[0].ss == 1 && view[0].ds == 1);
+}
+
 }  // namespace mrl
