@@ -209,10 +209,10 @@ struct MoveStrided {
 __global__ __launch_bounds__(256) void k_move_rows(MoveStrided p) {
   const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i >= p.count) return;
-  uint64_t rem = i;
+  uint32_t rem = uint32_t(i);  // a tensor has fewer than 2^31 elements
   int64_t so = 0, d_o = 0;
   for (int o = int(p.rank) - 1; o >= 0; o--) {
-    const uint32_t d = p.order[o], c = uint32_t(rem % p.shape[d]);
+    const uint32_t d = p.order[o], c = rem % p.shape[d];
     rem /= p.shape[d];
     so += int64_t(c) * p.ss[d], d_o += int64_t(c) * p.ds[d];
   }
@@ -224,10 +224,10 @@ __global__ __launch_bounds__(256) void k_move_rows(MoveStrided p) {
 __global__ __launch_bounds__(256) void k_move_rows16(MoveStrided p) {
   const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i >= p.count) return;
-  uint64_t rem = i;
+  uint32_t rem = uint32_t(i);
   int64_t so = 0, d_o = 0;
   for (int o = int(p.rank) - 1; o >= 0; o--) {
-    const uint32_t d = p.order[o], c = uint32_t(rem % p.shape[d]);
+    const uint32_t d = p.order[o], c = rem % p.shape[d];
     rem /= p.shape[d];
     so += int64_t(c) * p.ss[d], d_o += int64_t(c) * p.ds[d];
   }
@@ -765,6 +765,7 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
     if (d < rank && p.shape[d] > 1 && p.ds[d] == 1) dim_d = int(d);
   }
   if (p.count == 0) return hipSuccess;
+  if (p.count > 0xffffffffull) return hipErrorInvalidValue;  // the kernels index elements with 32 bits
   // Decode order: by decreasing destination stride, the destination's contiguous dim last.
   for (uint32_t d = 0; d < MOVE_MAX_RANK; d++) p.order[d] = d;
   for (uint32_t i = 0; i < p.rank; i++)
