@@ -315,6 +315,10 @@ struct MoveTile {
   uint32_t tstride_s[MOVE_MAX_RANK], tstride_d[MOVE_MAX_RANK];
   uint32_t inv_s[MOVE_MAX_RANK], inv_d[MOVE_MAX_RANK], inv_ext[MOVE_MAX_RANK];  // ceil(2^32 / x)
   uint32_t tile;  // elements per tile
+  // Runs of V > 1 elements per thread: the LDS distance between neighbours along the
+  // destination's fastest digit, and whether whole runs may be loaded / stored as one vector.
+  uint32_t lds_step;
+  bool vec_s, vec_d;
 };
 constexpr uint32_t MOVE_TILE_MAX = 4096;
 
@@ -324,10 +328,15 @@ __device__ inline uint32_t div_small(uint32_t n, uint32_t d, uint32_t inv) {
 
 // E: the element type when nothing is converted (typed loads and stores), void when the dtypes
 // differ (conversion per element).  Offsets fit 32 bits: a tensor has fewer than 2^31 elements.
-template <class E>
+// V: elements per thread and step, a run along the fastest digit of the side being walked (the
+// host picks V > 1 only when those digits, their tile extents and their sizes are multiples of
+// V): one digit extraction serves V elements.
+template <class E, int V>
 __global__ __launch_bounds__(256) void k_move_gather(MoveTile p) {
   constexpr bool CONVERT = std::is_void<E>::value;
   typedef typename std::conditional<CONVERT, uint32_t, E>::type Cell;
+  static_assert(V == 1 || (!CONVERT && sizeof(Cell) == 4), "runs are for 4-byte elements");
+  typedef Cell Run __attribute__((ext_vector_type(V == 1 ? 2 : V)));  // used only when V > 1
   __shared__ Cell lds[MOVE_TILE_MAX + MOVE_TILE_MAX / 64];
   uint64_t blk = blockIdx.x;
   int64_t base_s = 0, base_d = 0;
@@ -343,7 +352,7 @@ __global__ __launch_bounds__(256) void k_move_gather(MoveTile p) {
     }
   }
 #pragma unroll 4
-  for (uint32_t t = threadIdx.x; t < p.tile; t += 256) {
+  for (uint32_t t = threadIdx.x * V; t < p.tile; t += 256 * V) {
     uint32_t so = 0;
     bool inside = true;
 #pragma unroll
@@ -355,13 +364,25 @@ __global__ __launch_bounds__(256) void k_move_gather(MoveTile p) {
         so += c * uint32_t(p.m.ss[d]);
       }
     if (inside) {
-      if constexpr (CONVERT) lds[t + t / 64] = move_bits(p.m.src, p.m.sdt, base_s + so, p.m.ddt);
-      else lds[t + t / 64] = static_cast<const E *>(p.m.src)[base_s + so];
+      if constexpr (CONVERT) {
+        lds[t + t / 64] = move_bits(p.m.src, p.m.sdt, base_s + so, p.m.ddt);
+      } else if constexpr (V == 1) {
+        lds[t + t / 64] = static_cast<const E *>(p.m.src)[base_s + so];
+      } else {
+        const E *from = static_cast<const E *>(p.m.src) + base_s + so;
+        Run run;
+        if (p.vec_s) run = *reinterpret_cast<const Run *>(from);
+        else
+#pragma unroll
+          for (int e = 0; e < V; e++) run[e] = from[e];
+#pragma unroll
+        for (int e = 0; e < V; e++) lds[t + t / 64 + e] = run[e];
+      }
     }
   }
   __syncthreads();
 #pragma unroll 4
-  for (uint32_t t = threadIdx.x; t < p.tile; t += 256) {
+  for (uint32_t t = threadIdx.x * V; t < p.tile; t += 256 * V) {
     uint32_t d_o = 0, at = 0;
     bool inside = true;
 #pragma unroll
@@ -374,8 +395,23 @@ __global__ __launch_bounds__(256) void k_move_gather(MoveTile p) {
         at += c * p.tstride_s[d];
       }
     if (inside) {
-      if constexpr (CONVERT) store_u32(p.m.dst, p.m.ddt, base_d + d_o, lds[at + at / 64]);
-      else static_cast<E *>(p.m.dst)[base_d + d_o] = lds[at + at / 64];
+      if constexpr (CONVERT) {
+        store_u32(p.m.dst, p.m.ddt, base_d + d_o, lds[at + at / 64]);
+      } else if constexpr (V == 1) {
+        static_cast<E *>(p.m.dst)[base_d + d_o] = lds[at + at / 64];
+      } else {
+        Run run;
+#pragma unroll
+        for (int e = 0; e < V; e++) {
+          const uint32_t from = at + e * p.lds_step;  // the next element along the destination's fastest digit
+          run[e] = lds[from + from / 64];
+        }
+        E *to = static_cast<E *>(p.m.dst) + base_d + d_o;
+        if (p.vec_d) *reinterpret_cast<Run *>(to) = run;
+        else
+#pragma unroll
+          for (int e = 0; e < V; e++) to[e] = run[e];
+      }
     }
   }
 }
@@ -872,10 +908,25 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
   if (blocks > 0x7fffffffull || tile > MOVE_TILE_MAX) return hipErrorInvalidValue;
   const dim3 grid{uint32_t(blocks)};
   const size_t elem = mrl_dtype_size(src_dtype);
-  if (src_dtype != dst_dtype) hipLaunchKernelGGL(k_move_gather<void>, grid, dim3(256), 0, stream, t);
-  else if (elem == 4) hipLaunchKernelGGL(k_move_gather<uint32_t>, grid, dim3(256), 0, stream, t);
-  else if (elem == 2) hipLaunchKernelGGL(k_move_gather<uint16_t>, grid, dim3(256), 0, stream, t);
-  else hipLaunchKernelGGL(k_move_gather<uint8_t>, grid, dim3(256), 0, stream, t);
+  // Runs of 4 or 2 elements per thread where both sides' fastest digits allow.
+  const uint32_t fs = by_ss[0], fd = by_ds[0];
+  uint32_t run = 1;
+  if (src_dtype == dst_dtype && elem == 4 && p.ss[fs] == 1 && p.ds[fd] == 1)
+    for (uint32_t v : {4u, 2u})
+      if (run == 1 && t.ext[fs] % v == 0 && p.shape[fs] % v == 0 && t.ext[fd] % v == 0 && p.shape[fd] % v == 0) run = v;
+  t.lds_step = t.tstride_s[fd];
+  t.vec_s = (reinterpret_cast<uintptr_t>(src) % (4 * run)) == 0;
+  t.vec_d = (reinterpret_cast<uintptr_t>(dst) % (4 * run)) == 0;
+  for (uint32_t d = 0; d < rank; d++) {
+    if (d != fs && p.ss[d] % run != 0) t.vec_s = false;
+    if (d != fd && p.ds[d] % run != 0) t.vec_d = false;
+  }
+  if (src_dtype != dst_dtype) hipLaunchKernelGGL((k_move_gather<void, 1>), grid, dim3(256), 0, stream, t);
+  else if (elem == 4 && run == 4) hipLaunchKernelGGL((k_move_gather<uint32_t, 4>), grid, dim3(256), 0, stream, t);
+  else if (elem == 4 && run == 2) hipLaunchKernelGGL((k_move_gather<uint32_t, 2>), grid, dim3(256), 0, stream, t);
+  else if (elem == 4) hipLaunchKernelGGL((k_move_gather<uint32_t, 1>), grid, dim3(256), 0, stream, t);
+  else if (elem == 2) hipLaunchKernelGGL((k_move_gather<uint16_t, 1>), grid, dim3(256), 0, stream, t);
+  else hipLaunchKernelGGL((k_move_gather<uint8_t, 1>), grid, dim3(256), 0, stream, t);
   return hipGetLastError();
 }
 
