@@ -728,7 +728,16 @@ int run_compose_msm(const mrl_spec &s, void *const *params, Workspace &ws) {
   void *p1[3] = {params[1], params[2], sbuf};
   int rc = run_matmul(st, p1, ws);
   if (rc != MRL_OK) return rc;
-  if ((reinterpret_cast<uintptr_t>(sbuf) & 15) == 0) {
+  // bf16 inputs: P is rounded to bf16 on its way out of the Softmax, as in the fused kernel (the
+  // one deviation from the f32 closed form, within the Compose's 1e-2), so that the second
+  // product runs at the bf16 rate of the matrix cores instead of the f32 rate.
+  const bool p_bf16 = s.dtypes[0] == MRL_BF16 && s.dtypes[1] == MRL_BF16 && s.dtypes[2] == MRL_BF16 &&
+                      s.dtypes[3] == MRL_F32;
+  void *pbuf = sbuf;
+  if (p_bf16) {
+    HIP_TRY(ws.alloc(&pbuf, size_t(b) * m * n2 * 2));
+    HIP_TRY(mrl::launch_softmax_rows_bf16((const float *)sbuf, pbuf, uint64_t(b) * m, n2, ws.stream));
+  } else if ((reinterpret_cast<uintptr_t>(sbuf) & 15) == 0) {
     HIP_TRY(mrl::launch_softmax_rows((const float *)sbuf, (float *)sbuf, uint64_t(b) * m, n2, ws.stream));
   } else {
     mrl::Strided sv;
@@ -738,10 +747,10 @@ int run_compose_msm(const mrl_spec &s, void *const *params, Workspace &ws) {
     HIP_TRY(mrl::launch_softmax_generic(sv, sv, 2, ws.stream));
   }
   st.spec_shape[2] = n2, st.spec_shape[3] = n;
-  st.dtypes[0] = MRL_F32, st.dtypes[1] = s.dtypes[0], st.dtypes[2] = s.dtypes[3];
-  st.layouts[0] = st.layouts[2];  // S: row-major [b, m, n2]
+  st.dtypes[0] = p_bf16 ? MRL_BF16 : MRL_F32, st.dtypes[1] = s.dtypes[0], st.dtypes[2] = s.dtypes[3];
+  st.layouts[0] = st.layouts[2];  // P: row-major [b, m, n2]
   st.layouts[1] = s.layouts[0], st.layouts[2] = s.layouts[3];
-  void *p2[3] = {sbuf, params[0], params[3]};
+  void *p2[3] = {pbuf, params[0], params[3]};
   return run_matmul(st, p2, ws);
 }
 

@@ -118,6 +118,9 @@ hipError_t launch_unfold(const void *image, void *rows, uint32_t batch, uint32_t
 // ---- softmax.hip: f32 softmax over a contiguous innermost scan dim ---------------------
 hipError_t launch_softmax_rows(const float *in, float *out, uint64_t rows, uint32_t cols,
                                hipStream_t stream);
+// The same with the result rounded to bf16 (rows of `cols` 16-bit values).
+hipError_t launch_softmax_rows_bf16(const float *in, void *out, uint64_t rows, uint32_t cols,
+                                    hipStream_t stream);
 
 // ---- parts.hip: the primitive Specs of the Softmax decomposition, Broadcast, Fill ----------
 struct PartsArgs {

@@ -27,11 +27,20 @@ __device__ inline float wave_sum(float v) {
 typedef float f4 __attribute__((ext_vector_type(4)));
 constexpr float F32_MIN = -3.40282347e+38f;  // f32::MIN, the oracle's max identity
 
-// NV float4 vectors per lane; cols is a multiple of 4 and <= NV * 256.
-template <int NV>
+// f32 -> bf16, round to nearest even (softmax values are finite and in [0, 1]).
+__device__ inline uint32_t bf16_bits(float f) {
+  const uint32_t bits = __float_as_uint(f);
+  return (bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16;
+}
+
+// NV float4 vectors per lane; cols is a multiple of 4 and <= NV * 256.  OUT_BF16: the result is
+// written as bf16 (the left operand of the product that follows a Softmax in a Compose whose
+// inputs are bf16).
+template <int NV, bool OUT_BF16>
 __global__ __launch_bounds__(256) void k_softmax_regs(const float *__restrict__ in,
-                                                      float *__restrict__ out, uint64_t rows,
+                                                      void *__restrict__ out_any, uint64_t rows,
                                                       uint32_t cols) {
+  float *out = static_cast<float *>(out_any);
   const uint64_t row = uint64_t(blockIdx.x) * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
   const uint32_t lane = threadIdx.x & 63;
@@ -72,16 +81,25 @@ __global__ __launch_bounds__(256) void k_softmax_regs(const float *__restrict__ 
     const uint32_t idx = i * 64 + lane;
     if (idx < nvec) {
       v[i].x /= sum, v[i].y /= sum, v[i].z /= sum, v[i].w /= sum;
-      __builtin_nontemporal_store(f4{v[i].x, v[i].y, v[i].z, v[i].w}, (f4 *)dst + idx);
+      if constexpr (OUT_BF16) {
+        typedef unsigned u2 __attribute__((ext_vector_type(2)));
+        u2 *dst16 = reinterpret_cast<u2 *>(static_cast<uint16_t *>(out_any) + row * cols);
+        __builtin_nontemporal_store(u2{bf16_bits(v[i].x) | (bf16_bits(v[i].y) << 16), bf16_bits(v[i].z) | (bf16_bits(v[i].w) << 16)},
+                                    dst16 + idx);
+      } else {
+        __builtin_nontemporal_store(f4{v[i].x, v[i].y, v[i].z, v[i].w}, (f4 *)dst + idx);
+      }
     }
   }
 }
 
 // Any cols: each lane runs the online (max, denom) update over its elements, the lanes'
 // pairs are merged, then the row is read again to write exp(x - max) / denom.
+template <bool OUT_BF16>
 __global__ __launch_bounds__(256) void k_softmax_stream(const float *__restrict__ in,
-                                                        float *__restrict__ out, uint64_t rows,
+                                                        void *__restrict__ out_any, uint64_t rows,
                                                         uint32_t cols) {
+  float *out = static_cast<float *>(out_any);
   const uint64_t row = uint64_t(blockIdx.x) * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
   const uint32_t lane = threadIdx.x & 63;
@@ -104,28 +122,44 @@ __global__ __launch_bounds__(256) void k_softmax_stream(const float *__restrict_
     mx = nm;
   }
   if (__any(nan)) mx = __uint_as_float(0x7fc00000u);
-  for (uint32_t i = lane; i < cols; i += 64) dst[i] = expf(src[i] - mx) / den;
+  for (uint32_t i = lane; i < cols; i += 64) {
+    const float y = expf(src[i] - mx) / den;
+    if constexpr (OUT_BF16) (static_cast<uint16_t *>(out_any) + row * cols)[i] = uint16_t(bf16_bits(y));
+    else dst[i] = y;
+  }
 }
 
 }  // namespace
 
-hipError_t launch_softmax_rows(const float *in, float *out, uint64_t rows, uint32_t cols,
-                               hipStream_t stream) {
+namespace {
+template <bool OUT_BF16>
+hipError_t launch_rows(const float *in, void *out, uint64_t rows, uint32_t cols, hipStream_t stream) {
   if (rows == 0 || cols == 0) return hipSuccess;
   const uint64_t blocks64 = (rows + 3) / 4;
   if (blocks64 > 0x7fffffffull) return hipErrorInvalidValue;
   const dim3 grid{uint32_t(blocks64)}, block{256};
   if (cols % 4 == 0 && cols <= 16 * 256) {
     const uint32_t nv = (cols / 4 + 63) / 64;
-    if (nv <= 1) hipLaunchKernelGGL(k_softmax_regs<1>, grid, block, 0, stream, in, out, rows, cols);
-    else if (nv <= 2) hipLaunchKernelGGL(k_softmax_regs<2>, grid, block, 0, stream, in, out, rows, cols);
-    else if (nv <= 4) hipLaunchKernelGGL(k_softmax_regs<4>, grid, block, 0, stream, in, out, rows, cols);
-    else if (nv <= 8) hipLaunchKernelGGL(k_softmax_regs<8>, grid, block, 0, stream, in, out, rows, cols);
-    else hipLaunchKernelGGL(k_softmax_regs<16>, grid, block, 0, stream, in, out, rows, cols);
+    if (nv <= 1) hipLaunchKernelGGL((k_softmax_regs<1, OUT_BF16>), grid, block, 0, stream, in, out, rows, cols);
+    else if (nv <= 2) hipLaunchKernelGGL((k_softmax_regs<2, OUT_BF16>), grid, block, 0, stream, in, out, rows, cols);
+    else if (nv <= 4) hipLaunchKernelGGL((k_softmax_regs<4, OUT_BF16>), grid, block, 0, stream, in, out, rows, cols);
+    else if (nv <= 8) hipLaunchKernelGGL((k_softmax_regs<8, OUT_BF16>), grid, block, 0, stream, in, out, rows, cols);
+    else hipLaunchKernelGGL((k_softmax_regs<16, OUT_BF16>), grid, block, 0, stream, in, out, rows, cols);
   } else {
-    hipLaunchKernelGGL(k_softmax_stream, grid, block, 0, stream, in, out, rows, cols);
+    hipLaunchKernelGGL(k_softmax_stream<OUT_BF16>, grid, block, 0, stream, in, out, rows, cols);
   }
   return hipGetLastError();
+}
+}  // namespace
+
+hipError_t launch_softmax_rows(const float *in, float *out, uint64_t rows, uint32_t cols,
+                               hipStream_t stream) {
+  return launch_rows<false>(in, out, rows, cols, stream);
+}
+
+hipError_t launch_softmax_rows_bf16(const float *in, void *out, uint64_t rows, uint32_t cols,
+                                    hipStream_t stream) {
+  return launch_rows<true>(in, out, rows, cols, stream);
 }
 
 }  // namespace mrl
