@@ -703,6 +703,12 @@ int run_compose_msm(const mrl_spec &s, void *const *params, Workspace &ws) {
       void *result = params[3];
       if (!out_in_order) HIP_TRY(ws.alloc(&result, size_t(b) * m * n * sizeof(float)));
       at.out = static_cast<float *>(result);
+      at.key_splits = mrl::attn_key_splits(at);
+      if (at.key_splits > 1) {
+        void *partials = nullptr;
+        HIP_TRY(ws.alloc(&partials, mrl::attn_partial_bytes(at, at.key_splits)));
+        at.partials = static_cast<float *>(partials);
+      }
       if (mrl::attn_applicable(at)) {
         HIP_TRY(mrl::launch_attn(at, ws.stream));
         if (!out_in_order)

@@ -23,6 +23,8 @@
 // 32 in-register values plus one cross-lane exchange.  K and V blocks go from global memory
 // straight into LDS (no staging registers), double buffered, one barrier per block; the
 // bank-conflict swizzles are applied on the source side of those loads.
+#include <algorithm>
+
 #include "kernels.h"
 
 namespace mrl {
@@ -93,9 +95,19 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
   // Key blocks of this half: [first_block, first_block + nblocks); both halves run `steps`
   // iterations so that they meet at the same barriers.
   const int all_blocks = int((p.n2 + BKV - 1) / BKV);
-  const int steps = (all_blocks + 1) / 2;
-  const int first_block = half ? steps : 0;
-  const int nblocks = half ? all_blocks - steps : steps;
+  // With key_splits > 1 (few queries, many keys: too few workgroups otherwise) blockIdx.y picks
+  // a contiguous share of the key blocks; the result is then a partial (max, denominator, O)
+  // triple per split, merged by k_attn_merge.
+  int split_first = 0, split_end = all_blocks;
+  if (p.key_splits > 1) {
+    const int per = (all_blocks + int(p.key_splits) - 1) / int(p.key_splits);
+    split_first = min(all_blocks, int(blockIdx.y) * per);
+    split_end = min(all_blocks, split_first + per);
+  }
+  const int my_blocks = split_end - split_first;
+  const int steps = (my_blocks + 1) / 2;
+  const int first_block = split_first + (half ? steps : 0);
+  const int nblocks = half ? my_blocks - steps : steps;
   const uint32_t head_bytes = p.n2 * ROW;  // K or V of one batch entry
 
   const int q_row = RAGGED ? min(q0 + lq, int(p.m) - 1) : q0 + lq;
@@ -323,6 +335,26 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
     const float m1 = mbuf[(D / 2) * 64 + lane], l1 = mbuf[(D / 2 + 1) * 64 + lane];
     const float m = fmaxf(m_run, m1);
     const float a0 = __builtin_amdgcn_exp2f((m_run - m) * LOG2E), a1 = __builtin_amdgcn_exp2f((m1 - m) * LOG2E);
+    if (p.key_splits > 1) {
+      // Partial triple of this split, relative to m: rows of D + 4 floats (O, then m, then the
+      // denominator), [query][split].
+      if (q0 + lq < int(p.m)) {
+        float *part = p.partials + ((head * p.m + q0 + lq) * int64_t(p.key_splits) + blockIdx.y) * (D + 4);
+#pragma unroll
+        for (int t = 0; t < D / 32; t++)
+#pragma unroll
+          for (int a = 0; a < 4; a++) {
+            float4 v;
+            v.x = o[t][4 * a + 0] * a0 + mbuf[(t * 16 + 4 * a + 0) * 64 + lane] * a1;
+            v.y = o[t][4 * a + 1] * a0 + mbuf[(t * 16 + 4 * a + 1) * 64 + lane] * a1;
+            v.z = o[t][4 * a + 2] * a0 + mbuf[(t * 16 + 4 * a + 2) * 64 + lane] * a1;
+            v.w = o[t][4 * a + 3] * a0 + mbuf[(t * 16 + 4 * a + 3) * 64 + lane] * a1;
+            *(float4 *)(part + t * 32 + 8 * a + 4 * lg) = v;
+          }
+        if (lg == 0) part[D] = m, part[D + 1] = l_tot * a0 + l1 * a1;
+      }
+      return;
+    }
     const float inv = 1.0f / (l_tot * a0 + l1 * a1);
     const float w0 = a0 * inv, w1 = a1 * inv;
     float *out = p.out + (head * p.m + q0 + lq) * int64_t(p.n_out);
@@ -350,12 +382,54 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
   }
 }
 
+// out[row][0 .. n_out) = sum_s O_s * 2^((m_s - M) log2 e) / sum_s l_s * 2^((m_s - M) log2 e), M = max_s m_s:
+// the parts formula of morello/src/spec.rs:107-132 over the splits' triples.  One thread per
+// output element; a split that saw no key has l = 0 and the smallest m, so it drops out.
+__global__ __launch_bounds__(256) void k_attn_merge(const float *__restrict__ partials, float *__restrict__ out,
+                                                    uint64_t rows, uint32_t splits, uint32_t d, uint32_t n_out) {
+  const uint64_t i = uint64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= rows * n_out) return;
+  const uint64_t row = i / n_out;
+  const uint32_t col = uint32_t(i % n_out);
+  const float *part = partials + row * splits * (d + 4);
+  float m = part[d];
+  for (uint32_t s = 1; s < splits; s++) m = fmaxf(m, part[s * (d + 4) + d]);
+  float num = 0.0f, den = 0.0f;
+  for (uint32_t s = 0; s < splits; s++) {
+    const float w = __builtin_amdgcn_exp2f((part[s * (d + 4) + d] - m) * LOG2E);
+    num += part[s * (d + 4) + col] * w;
+    den += part[s * (d + 4) + d + 1] * w;
+  }
+  out[row * n_out + col] = num / den;
+}
+
 }  // namespace
+
+// Key splits for a launch: 1 unless the (entry, query block) pairs fill at most half of the
+// compute units and there are keys enough to share out (four blocks of 64 per workgroup at
+// least).  The workgroups then number at most one per compute unit: measured on 256 units, 256
+// workgroups stream K and V at 4.9-5.6 TB/s where 320 or 512 reach 3.6-4.8.
+uint32_t attn_key_splits(const AttnArgs &a) {
+  static const uint64_t units = [] {
+    int device = 0, count = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count <= 0)
+      return uint64_t(256);
+    return uint64_t(count);
+  }();
+  const uint64_t groups = uint64_t((a.m + BQ - 1) / BQ) * a.b, blocks = (a.n2 + BKV - 1) / BKV;
+  if (groups == 0) return 1;
+  const uint64_t splits = std::min<uint64_t>({units / groups, blocks / 4, 256});
+  return splits < 2 ? 1 : uint32_t(splits);
+}
+size_t attn_partial_bytes(const AttnArgs &a, uint32_t splits) {
+  return splits > 1 ? size_t(a.b) * a.m * splits * (a.k + 4) * sizeof(float) : 0;
+}
 
 bool attn_applicable(const AttnArgs &a) {
   auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
   return a.k == a.n && (a.k == 32 || a.k == 64 || a.k == 128) && a.n_out >= 1 && a.n_out <= a.n && a.m && a.n2 && a.b &&
-         (!a.kt_rows || a.n2 % 8 == 0) &&
+         (!a.kt_rows || a.n2 % 8 == 0) && (a.key_splits <= 1 || (a.partials && a.key_splits <= 65535)) &&
          uint64_t(a.n2) * a.k * 2 < (1ull << 31) && uint64_t((a.m + BQ - 1) / BQ) * a.b < (1u << 31) &&
          al16(a.q) && al16(a.kt) && al16(a.v) && al16(a.out);
 }
@@ -370,8 +444,13 @@ hipError_t launch_one(const AttnArgs &a, hipStream_t stream) {
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  const dim3 grid(((a.m + BQ - 1) / BQ) * a.b);
+  const dim3 grid(((a.m + BQ - 1) / BQ) * a.b, std::max(1u, a.key_splits));
   hipLaunchKernelGGL((k_attn<D, RAGGED, KT_ROWS>), grid, dim3(512), LDS, stream, a);
+  if (a.key_splits > 1) {
+    const uint64_t rows = uint64_t(a.b) * a.m, total = rows * a.n_out;
+    hipLaunchKernelGGL(k_attn_merge, dim3(uint32_t((total + 255) / 256)), dim3(256), 0, stream, a.partials, a.out, rows,
+                       a.key_splits, uint32_t(D), a.n_out);
+  }
   return hipGetLastError();
 }
 

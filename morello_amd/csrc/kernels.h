@@ -152,7 +152,13 @@ struct AttnArgs {
   // was padded with zero columns up to a head dim the kernel is built for.
   uint32_t n_out;
   bool kt_rows = false;  // KT stored row-major, n2 fastest (n2 a multiple of 8)
+  // More than 1: the keys are shared out over that many workgroups per query block and the
+  // partial results merged afterwards; `partials` holds attn_partial_bytes() of scratch.
+  uint32_t key_splits = 1;
+  float *partials = nullptr;
 };
+uint32_t attn_key_splits(const AttnArgs &a);
+size_t attn_partial_bytes(const AttnArgs &a, uint32_t splits);
 bool attn_applicable(const AttnArgs &a);
 hipError_t launch_attn(const AttnArgs &a, hipStream_t stream);
 

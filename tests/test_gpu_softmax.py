@@ -134,6 +134,27 @@ def test_compose_msm_fused_with_padded_head_dims(gpu, dims):
     assert rel_err(got, want) < 1e-2
 
 
+@pytest.mark.parametrize("dims", [(16, 1, 128, 2048, 128), (2, 1, 128, 32768, 128), (4, 16, 64, 8200, 64),
+                                  (3, 130, 32, 1100, 32), (2, 5, 96, 3000, 72), (1, 1, 128, 257, 128),
+                                  (5, 3, 64, 640, 64)])
+def test_compose_msm_few_queries_many_keys(gpu, dims):
+    """Few (entry, query block) pairs and many keys: the keys are shared out over several
+    workgroups per query block and the partial (max, denominator, O) triples merged afterwards.
+    Covers splits that end up without a key block, ragged key counts, padded head dims, and both
+    KT orders."""
+    b, m, k, n2, n = dims
+    q, kmat, v = msm_inputs(307, *dims)
+    want = orc.compose_msm(b, m, k, n2, n, [7, 7, 7, 6], v, q, kmat, np.zeros((b, m, n), np.float32),
+                           layouts=[None, None, KT_ORC, None])
+    spec = M.ComposeMSM(b, m, k, n2, n, layouts=[None, None, KT_LAYOUT, None])
+    got = run_spec(spec, [v, q, kmat, np.full((b, m, n), 7.5, np.float32)])
+    assert rel_err(got, want) < 1e-2
+    if n2 % 8 == 0:
+        kt = np.ascontiguousarray(kmat.transpose(0, 2, 1))
+        got = run_spec(M.ComposeMSM(b, m, k, n2, n), [v, q, kt, np.full((b, m, n), 7.5, np.float32)])
+        assert rel_err(got, want) < 1e-2
+
+
 def test_compose_msm_f32_inputs_stay_staged(gpu):
     """f32 inputs run on the staged (unfused) path, exact to 1e-5: nothing is rounded to bf16."""
     b, m, k, n2, n = 2, 40, 32, 48, 24
