@@ -346,6 +346,62 @@ int mrl_stream_destroy(void *stream);
 int mrl_device_info(char *name, size_t name_len, int *compute_units, int *clock_khz,
                     size_t *total_mem_bytes);
 
+/* ---- The backend as a search target -------------------------------------------------------
+ * What morello's `Target` / `Memory` / `Kernel` traits ask of a backend
+ * (morello/src/target/mod.rs:37-117), as data a Rust `impl Target for Gfx950Target` would
+ * forward.  All of it is host code: none of these calls needs a GPU. */
+
+/* Target::target_id (target/mod.rs:74): "Gfx950". */
+const char *mrl_target_id(void);
+/* Target::line_size (target/mod.rs:50): bytes of one L2 cache line. */
+uint32_t mrl_target_line_size(void);
+/* Target::processors (target/mod.rs:53): compute units (the reference's u8 cannot hold 256). */
+uint32_t mrl_target_processors(void);
+
+/* One level of Target::memories (target/mod.rs:55), fastest first, with the `Memory` trait's
+ * answers (target/mod.rs:80-95), Target::max_mem's limit for it (target/mod.rs:52; per
+ * processor for registers and LDS) and Target::cache_hit_cost (target/mod.rs:51). */
+typedef struct {
+  char name[8];               /* "ACC", "VGPR", "LDS", "HBM" */
+  uint8_t is_addressed;       /* Memory::is_addressed */
+  uint8_t can_parallel_tile;  /* Memory::can_parallel_tile */
+  uint8_t counts_registers;   /* Memory::counts_registers: the limit counts registers, not bytes */
+  uint8_t has_layout;         /* Memory::has_layout */
+  uint32_t vector_bytes[4];   /* Memory::vector_bytes, 0-terminated */
+  uint64_t limit;             /* Target::max_mem: registers per lane, or bytes */
+  uint32_t cache_hit_cost;    /* Target::cache_hit_cost */
+} mrl_target_memory;
+/* Writes up to `cap` levels; returns how many there are (4, the reference's MEMORY_COUNT). */
+uint32_t mrl_target_memories(mrl_target_memory *out, uint32_t cap);
+
+/* Kernel::name of every kernel family of the backend (target/mod.rs:111); returns the count. */
+uint32_t mrl_target_kernels(const char **names, uint32_t cap);
+
+/* One kernel launch a Spec would make. */
+typedef struct {
+  char kernel[160];    /* the kernel and the template arguments it was built with,
+                          "k_attn [D = 128, RAGGED = false, KT_ROWS = false]" */
+  uint32_t grid[3], block[3];
+  uint32_t lds_bytes;  /* dynamic LDS per workgroup: Kernel::memory_allocated's LDS figure */
+  int32_t unit;        /* what bounds it besides traffic: 0 HBM stream, 1 int8 MFMA, 2 bf16 MFMA,
+                          3 f32 MFMA, 4 vector ALU */
+  double ops, bytes;   /* arithmetic (2 per multiply-add) and HBM traffic the kernel is charged */
+  double cost_ns;      /* predicted duration, launch gap included */
+} mrl_plan_step;
+typedef struct {
+  uint32_t n_steps;        /* launches the Spec makes (may exceed the `cap` that was passed) */
+  uint64_t scratch_bytes;  /* device scratch the call takes: Kernel::memory_allocated's HBM figure */
+  double cost_ns;          /* sum over the steps: Kernel::main_cost (target/mod.rs:109), in ns */
+} mrl_plan;
+/* Which kernels mrl_run would launch for `spec` with 256-byte-aligned parameters, and the cost
+ * model's prediction for them (Kernel::applies_to_logical_spec + main_cost + memory_allocated,
+ * target/mod.rs:103-109; Cost, cost.rs:13-17).  The plan is produced by the same dispatch code
+ * that runs a Spec, with launches recorded instead of made, so it cannot disagree with a run.
+ * MRL_ERR_UNSUPPORTED / MRL_ERR_BAD_SPEC as mrl_run. */
+int mrl_spec_plan(const mrl_spec *spec, mrl_plan *plan, mrl_plan_step *steps, uint32_t cap);
+/* The same for a general Compose. */
+int mrl_compose_plan(const mrl_compose *c, mrl_plan *plan, mrl_plan_step *steps, uint32_t cap);
+
 #ifdef __cplusplus
 }
 #endif

@@ -141,6 +141,14 @@ enum class SpecType : int {
 // spec.rs:165-170
 enum class FillValue : uint32_t { Zero = 0, NegInf = 1, Min = 2 };
 
+// What a run of a Spec would launch and what the cost model expects of it: the backend's answer
+// to Kernel::applies_to_logical_spec / main_cost / memory_allocated (target/mod.rs:103-109).
+struct Plan {
+  std::vector<mrl_plan_step> steps;
+  double cost_ns = 0;
+  uint64_t scratch_bytes = 0;
+};
+
 class Spec {
  public:
   // Matmul{accum} over [b, m, k, n] (spec.rs:480-485).  Layouts default to row-major.
@@ -212,6 +220,16 @@ class Spec {
   }
   uint64_t flops() const { return mrl_spec_ops(&c_); }
   bool is_supported() const { return mrl_spec_check(&c_) == MRL_OK; }
+  // Host-only: needs no GPU.
+  Plan plan() const {
+    mrl_plan head{};
+    Plan out;
+    out.steps.resize(64);
+    check(mrl_spec_plan(&c_, &head, out.steps.data(), 64), "plan");
+    out.steps.resize(head.n_steps < 64 ? head.n_steps : 64);
+    out.cost_ns = head.cost_ns, out.scratch_bytes = head.scratch_bytes;
+    return out;
+  }
   const mrl_spec &c() const { return c_; }
 
   // Where `kernel(p0, .., pk)` is called: device pointers in parameter order.

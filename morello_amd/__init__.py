@@ -264,6 +264,10 @@ class Spec:
     def workspace_bytes(self) -> int:
         return int(B.load().mrl_spec_workspace_bytes(C.byref(self._c)))
 
+    def plan(self) -> "Plan":
+        """The kernels a run would launch and the cost model's prediction (no GPU needed)."""
+        return _plan_of(B.load().mrl_spec_plan, self._c, "mrl_spec_plan")
+
     # -- execution -------------------------------------------------------------------
     def run_device(self, ptrs: Sequence[int]):
         """`ptrs`: device pointers in Spec parameter order.  Synchronous."""
@@ -488,10 +492,88 @@ class Compose:
         lib = B.load()
         return [Dtype(lib.mrl_compose_parameter_dtype(C.byref(self._c), i)) for i in range(self.n_params)]
 
+    def plan(self) -> "Plan":
+        return _plan_of(B.load().mrl_compose_plan, self._c, "mrl_compose_plan")
+
     def run_device(self, ptrs: Sequence[int]):
         arr = (C.c_void_p * len(ptrs))(*ptrs)
         _check(B.load().mrl_run_compose(C.byref(self._c), arr, None), "mrl_run_compose")
         synchronize()
+
+
+class PlanStep:
+    """One planned launch: `kernel` (with its template arguments in brackets), `family` (the name before them),
+    grid, block, LDS bytes, the bounding unit, declared ops / bytes and the predicted ns."""
+    UNITS = ("hbm", "mfma_i8", "mfma_bf16", "mfma_f32", "valu")
+
+    def __init__(self, c: B.PlanStepC):
+        self.kernel = c.kernel.decode()
+        self.family = self.kernel.split(" [")[0]
+        self.grid, self.block = tuple(c.grid), tuple(c.block)
+        self.lds_bytes, self.unit = int(c.lds_bytes), self.UNITS[c.unit]
+        self.ops, self.bytes, self.cost_ns = c.ops, c.bytes, c.cost_ns
+
+    def __repr__(self):
+        return f"{self.kernel} grid={self.grid} block={self.block} {self.unit} {self.cost_ns:.0f} ns"
+
+
+class Plan:
+    """Kernel::applies_to_logical_spec / main_cost / memory_allocated (target/mod.rs:103-109) of
+    the backend for one Spec: `steps`, `cost_ns` (their sum) and `scratch_bytes`."""
+
+    def __init__(self, steps, cost_ns: float, scratch_bytes: int):
+        self.steps, self.cost_ns, self.scratch_bytes = steps, cost_ns, scratch_bytes
+
+    @property
+    def kernels(self):
+        return [s.family for s in self.steps]
+
+    def __repr__(self):
+        return f"Plan({self.cost_ns:.0f} ns, scratch {self.scratch_bytes} B, {self.steps})"
+
+
+def _plan_of(fn, c_spec, where: str) -> Plan:
+    head, cap = B.PlanC(), 64
+    steps = (B.PlanStepC * cap)()
+    _check(fn(C.byref(c_spec), C.byref(head), steps, cap), where)
+    return Plan([PlanStep(steps[i]) for i in range(min(cap, head.n_steps))], head.cost_ns, int(head.scratch_bytes))
+
+
+class TargetMemory:
+    def __init__(self, c: B.TargetMemoryC):
+        self.name = c.name.decode()
+        self.is_addressed, self.can_parallel_tile = bool(c.is_addressed), bool(c.can_parallel_tile)
+        self.counts_registers, self.has_layout = bool(c.counts_registers), bool(c.has_layout)
+        self.vector_bytes = [v for v in c.vector_bytes if v]
+        self.limit, self.cache_hit_cost = int(c.limit), int(c.cache_hit_cost)
+
+
+class Target:
+    """The backend as morello's `Target` trait sees it (target/mod.rs:37-78)."""
+
+    @staticmethod
+    def target_id() -> str:
+        return B.load().mrl_target_id().decode()
+
+    @staticmethod
+    def line_size() -> int:
+        return int(B.load().mrl_target_line_size())
+
+    @staticmethod
+    def processors() -> int:
+        return int(B.load().mrl_target_processors())
+
+    @staticmethod
+    def memories():
+        buf = (B.TargetMemoryC * 4)()
+        n = B.load().mrl_target_memories(buf, 4)
+        return [TargetMemory(buf[i]) for i in range(n)]
+
+    @staticmethod
+    def kernels():
+        buf = (C.c_char_p * 64)()
+        n = B.load().mrl_target_kernels(buf, 64)
+        return [buf[i].decode() for i in range(n)]
 
 
 class Stream:

@@ -68,6 +68,22 @@ class ComposeC(C.Structure):
 _U32P = C.POINTER(C.c_uint32)
 _VPP = C.POINTER(C.c_void_p)
 
+class TargetMemoryC(C.Structure):
+    _fields_ = [("name", C.c_char * 8), ("is_addressed", C.c_uint8), ("can_parallel_tile", C.c_uint8),
+                ("counts_registers", C.c_uint8), ("has_layout", C.c_uint8), ("vector_bytes", C.c_uint32 * 4),
+                ("limit", C.c_uint64), ("cache_hit_cost", C.c_uint32)]
+
+
+class PlanStepC(C.Structure):
+    _fields_ = [("kernel", C.c_char * 160), ("grid", C.c_uint32 * 3), ("block", C.c_uint32 * 3),
+                ("lds_bytes", C.c_uint32), ("unit", C.c_int32), ("ops", C.c_double), ("bytes", C.c_double),
+                ("cost_ns", C.c_double)]
+
+
+class PlanC(C.Structure):
+    _fields_ = [("n_steps", C.c_uint32), ("scratch_bytes", C.c_uint64), ("cost_ns", C.c_double)]
+
+
 # name -> (restype, argtypes); every symbol include/morello_amd.h declares.
 SIGNATURES = {
     "mrl_init": (C.c_int, [C.c_int]),
@@ -116,6 +132,13 @@ SIGNATURES = {
     "mrl_stream_create": (C.c_int, [_VPP]),
     "mrl_stream_synchronize": (C.c_int, [C.c_void_p]),
     "mrl_stream_destroy": (C.c_int, [C.c_void_p]),
+    "mrl_target_id": (C.c_char_p, []),
+    "mrl_target_line_size": (C.c_uint32, []),
+    "mrl_target_processors": (C.c_uint32, []),
+    "mrl_target_memories": (C.c_uint32, [C.POINTER(TargetMemoryC), C.c_uint32]),
+    "mrl_target_kernels": (C.c_uint32, [C.POINTER(C.c_char_p), C.c_uint32]),
+    "mrl_spec_plan": (C.c_int, [C.POINTER(SpecC), C.POINTER(PlanC), C.POINTER(PlanStepC), C.c_uint32]),
+    "mrl_compose_plan": (C.c_int, [C.POINTER(ComposeC), C.POINTER(PlanC), C.POINTER(PlanStepC), C.c_uint32]),
     "mrl_device_info": (C.c_int, [C.c_char_p, C.c_size_t, C.POINTER(C.c_int), C.POINTER(C.c_int),
                                   C.POINTER(C.c_size_t)]),
 }

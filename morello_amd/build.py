@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libmorello_amd.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
-SOURCES = ["api.hip", "generic.hip", "gemm_mfma.hip", "gemm_sched.hip", "gemm_nt.hip", "gemv.hip", "conv_gemm.hip", "conv_i8.hip", "unfold.hip", "softmax.hip", "parts.hip", "mfma_rate.hip", "attention.hip"]
+SOURCES = ["api.hip", "generic.hip", "gemm_mfma.hip", "gemm_sched.hip", "gemm_nt.hip", "gemv.hip", "conv_gemm.hip", "conv_i8.hip", "unfold.hip", "softmax.hip", "parts.hip", "mfma_rate.hip", "attention.hip", "plan.hip"]
 
 # -packed-fp32-ops off: the compiler must not form v_pk_{add,mul,fma}_f32.
 FLAGS = [

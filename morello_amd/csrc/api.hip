@@ -270,6 +270,13 @@ struct Workspace {
   Workspace &operator=(const Workspace &) = delete;
   hipError_t alloc(void **p, size_t bytes) {
     const size_t rounded = (bytes + 255) & ~size_t(255);
+    if (mrl::plan::recording()) {
+      // Planning: a stand-in address, aligned as the allocator's are, never dereferenced.
+      mrl::plan::Recorder *r = mrl::plan::g_recorder;
+      *p = reinterpret_cast<void *>((uintptr_t(1) << 44) + r->scratch_bytes);
+      r->scratch_bytes += rounded ? rounded : 256;
+      return hipSuccess;
+    }
     if (rounded <= ARENA_BYTES - arena_used) {
       if (!arena) {
         arena = arena_of(stream);
@@ -625,8 +632,10 @@ int run_softmax(const mrl_spec &s, void *const *params, Workspace &ws) {
       (reinterpret_cast<uintptr_t>(in.t.ptr) & 15) == 0 &&
       (reinterpret_cast<uintptr_t>(out.t.ptr) & 15) == 0) {
     const uint32_t cols = s.spec_shape[s.scan_dim];
+    void *scratch = nullptr;
+    if (const size_t bytes = mrl::softmax_scratch_bytes(in.count / cols, cols)) HIP_TRY(ws.alloc(&scratch, bytes));
     HIP_TRY(mrl::launch_softmax_rows((const float *)in.t.ptr, (float *)out.t.ptr, in.count / cols,
-                                     cols, ws.stream));
+                                     cols, scratch, ws.stream));
   } else {
     HIP_TRY(mrl::launch_softmax_generic(in.t, out.t, s.scan_dim, ws.stream));
   }
@@ -739,12 +748,13 @@ int run_compose_msm(const mrl_spec &s, void *const *params, Workspace &ws) {
   // product runs at the bf16 rate of the matrix cores instead of the f32 rate.
   const bool p_bf16 = s.dtypes[0] == MRL_BF16 && s.dtypes[1] == MRL_BF16 && s.dtypes[2] == MRL_BF16 &&
                       s.dtypes[3] == MRL_F32;
-  void *pbuf = sbuf;
+  void *pbuf = sbuf, *stats = nullptr;
+  if (const size_t bytes = mrl::softmax_scratch_bytes(uint64_t(b) * m, n2)) HIP_TRY(ws.alloc(&stats, bytes));
   if (p_bf16) {
     HIP_TRY(ws.alloc(&pbuf, size_t(b) * m * n2 * 2));
-    HIP_TRY(mrl::launch_softmax_rows_bf16((const float *)sbuf, pbuf, uint64_t(b) * m, n2, ws.stream));
+    HIP_TRY(mrl::launch_softmax_rows_bf16((const float *)sbuf, pbuf, uint64_t(b) * m, n2, stats, ws.stream));
   } else if ((reinterpret_cast<uintptr_t>(sbuf) & 15) == 0) {
-    HIP_TRY(mrl::launch_softmax_rows((const float *)sbuf, (float *)sbuf, uint64_t(b) * m, n2, ws.stream));
+    HIP_TRY(mrl::launch_softmax_rows((const float *)sbuf, (float *)sbuf, uint64_t(b) * m, n2, stats, ws.stream));
   } else {
     mrl::Strided sv;
     sv.ptr = sbuf, sv.dtype = MRL_F32, sv.rank = 3;
@@ -1013,6 +1023,41 @@ int run_async_impl(const mrl_spec *spec, void *const *params, hipStream_t stream
   return dispatch(*spec, params, ws);
 }
 
+// Runs `body` (a dispatch) with a Recorder installed on this thread and stand-in parameter
+// addresses, then writes the recorded launches out.
+template <class Body>
+int plan_with(uint32_t n_params, mrl_plan *plan, mrl_plan_step *steps, uint32_t cap, Body body) {
+  if (!plan || (cap && !steps)) return MRL_ERR_NULL;
+  void *params[64];
+  if (n_params > 64) return MRL_ERR_BAD_SPEC;
+  for (uint32_t i = 0; i < n_params; i++) params[i] = reinterpret_cast<void *>((uintptr_t(1) << 40) + (uintptr_t(i) << 36));
+  mrl::plan::Recorder recorder;
+  int rc;
+  {
+    mrl::plan::g_recorder = &recorder;
+    Workspace ws(nullptr);
+    rc = body(params, ws);
+    mrl::plan::g_recorder = nullptr;
+  }
+  if (rc != MRL_OK) return rc;
+  int units = 256;
+  if (g_device >= 0) (void)hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, g_device);
+  plan->n_steps = uint32_t(recorder.steps.size());
+  plan->scratch_bytes = recorder.scratch_bytes;
+  plan->cost_ns = 0;
+  for (uint32_t i = 0; i < plan->n_steps; i++) {
+    const mrl::plan::Step &from = recorder.steps[i];
+    const double ns = mrl::plan::step_ns(from, uint32_t(units));
+    plan->cost_ns += ns;
+    if (i >= cap) continue;
+    mrl_plan_step &to = steps[i];
+    std::snprintf(to.kernel, sizeof to.kernel, "%s", from.kernel.c_str());
+    for (int d = 0; d < 3; d++) to.grid[d] = from.grid[d], to.block[d] = from.block[d];
+    to.lds_bytes = from.lds_bytes, to.unit = from.unit, to.ops = from.ops, to.bytes = from.bytes, to.cost_ns = ns;
+  }
+  return MRL_OK;
+}
+
 void set_conv_default_layouts(mrl_spec *s) {
   for (uint32_t i = 0; i < 3; i++) {
     uint32_t shape[MRL_MAX_RANK], rank;
@@ -1192,6 +1237,60 @@ size_t mrl_spec_workspace_bytes(const mrl_spec *spec) {
     total += size_t(volume(shape, rank)) * mrl_dtype_size(spec->dtypes[i]);
   }
   return total;
+}
+
+const char *mrl_target_id(void) { return "Gfx950"; }
+uint32_t mrl_target_line_size(void) { return 128; }
+uint32_t mrl_target_processors(void) {
+  int units = 256;
+  if (g_device >= 0) (void)hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, g_device);
+  return uint32_t(units);
+}
+
+uint32_t mrl_target_memories(mrl_target_memory *out, uint32_t cap) {
+  // Fastest first, as CpuMemory's order (target/cpu.rs:2536-2560).  ACC: the MFMA accumulators
+  // (a wavefront's share of the unified 512-register file the kernels give them); VGPR: the
+  // rest of the register file, whose 4 / 8 / 16-byte forms are what loads and stores move per
+  // lane; LDS: 160 KiB per compute unit, addressed by the kernels (unlike the reference's L1);
+  // HBM: 288 GB, the only level a grid can tile in parallel.  Hit costs follow the reference's
+  // scale of 1 for registers (target/cpu.rs cache_hit_cost) by latency ratio.
+  static const mrl_target_memory levels[4] = {
+      {"ACC", 1, 0, 1, 0, {0, 0, 0, 0}, 256, 0},
+      {"VGPR", 1, 0, 1, 1, {4, 8, 16, 0}, 256, 0},
+      {"LDS", 1, 0, 0, 1, {0, 0, 0, 0}, 160 * 1024, 8},
+      {"HBM", 1, 1, 0, 1, {0, 0, 0, 0}, 288ull << 30, 100},
+  };
+  for (uint32_t i = 0; i < 4 && i < cap && out; i++) out[i] = levels[i];
+  return 4;
+}
+
+uint32_t mrl_target_kernels(const char **names, uint32_t cap) {
+  static const char *const families[] = {
+      "k_gemm", "k_gemv", "k_matmul_generic", "k_conv_i8", "k_conv_generic", "k_conv_generic_wave", "k_unfold",
+      "k_unfold_gather", "k_attn", "k_attn_merge", "k_softmax_regs", "k_softmax_stream", "k_softmax_cols",
+      "k_softmax_generic", "k_parts", "k_broadcast", "k_fill", "k_fill_zero", "k_move_rows", "k_move_rows16",
+      "k_move_tiled", "k_move_tiled16", "k_move_gather", "k_move_generic", "k_relayout", "k_convert4", "k_copy1",
+      "k_copy16", "k_pad_rows", "k_widen_bf16"};
+  const uint32_t n = sizeof families / sizeof families[0];
+  for (uint32_t i = 0; i < n && i < cap && names; i++) names[i] = families[i];
+  return n;
+}
+
+int mrl_spec_plan(const mrl_spec *spec, mrl_plan *plan, mrl_plan_step *steps, uint32_t cap) {
+  int rc = check_spec(spec);
+  if (rc != MRL_OK) return rc;
+  return plan_with(spec->n_params, plan, steps, cap,
+                   [&](void *const *params, Workspace &ws) { return dispatch(*spec, params, ws); });
+}
+
+int mrl_compose_plan(const mrl_compose *c, mrl_plan *plan, mrl_plan_step *steps, uint32_t cap) {
+  if (!c) return MRL_ERR_NULL;
+  std::vector<ComposeParam> ext;
+  std::vector<mrl_spec> specs;
+  int rc = compose_parameters(*c, &ext, &specs);
+  if (rc != MRL_OK) return rc;
+  return plan_with(uint32_t(ext.size()), plan, steps, cap,
+                   [&](void *const *params, Workspace &ws) { return run_compose_general(*c, params, ws); });
 }
 
 int mrl_run_async(const mrl_spec *spec, void *const *params, void *stream) {

@@ -439,19 +439,25 @@ template <int D, bool RAGGED, bool KT_ROWS>
 hipError_t launch_one(const AttnArgs &a, hipStream_t stream) {
   constexpr int LDS = Dims<D>::LDS_BYTES;
   static bool attr_set = false;
-  if (!attr_set) {
+  if (!attr_set && !plan::recording()) {
     hipError_t e = hipFuncSetAttribute((const void *)k_attn<D, RAGGED, KT_ROWS>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
     if (e != hipSuccess) return e;
     attr_set = true;
   }
   const dim3 grid(((a.m + BQ - 1) / BQ) * a.b, std::max(1u, a.key_splits));
-  hipLaunchKernelGGL((k_attn<D, RAGGED, KT_ROWS>), grid, dim3(512), LDS, stream, a);
+  plan::work(plan::UNIT_MFMA_BF16, 4.0 * a.b * a.m * a.n2 * D,
+             double(a.b) * (2.0 * a.m * D + 4.0 * a.n2 * D + 4.0 * a.m * a.n_out) + attn_partial_bytes(a, a.key_splits),
+             // the softmax between the two products shares the issue slots: 1.45 x the MFMA time
+             1.45 * 4.0 * BQ * D * (double((a.n2 + BKV - 1) / BKV) * BKV / std::max(1u, a.key_splits)),
+             3000.0);
+  MRL_LAUNCH((k_attn<D, RAGGED, KT_ROWS>), grid, dim3(512), LDS, stream, a);
   if (a.key_splits > 1) {
     const uint64_t rows = uint64_t(a.b) * a.m, total = rows * a.n_out;
-    hipLaunchKernelGGL(k_attn_merge, dim3(uint32_t((total + 255) / 256)), dim3(256), 0, stream, a.partials, a.out, rows,
+    plan::work(plan::UNIT_STREAM, 0, double(attn_partial_bytes(a, a.key_splits)) + 4.0 * total);
+    MRL_LAUNCH(k_attn_merge, dim3(uint32_t((total + 255) / 256)), dim3(256), 0, stream, a.partials, a.out, rows,
                        a.key_splits, uint32_t(D), a.n_out);
   }
-  return hipGetLastError();
+  return mrl::plan::last_error();
 }
 
 template <int D>

@@ -162,11 +162,14 @@ hipError_t launch_slabs(const ConvArgs &c, bool img_unsigned, hipStream_t stream
   uint32_t blocks = std::max<uint32_t>(1, 2048 / WAVES / groups);
   if (blocks * WAVES > tiles) blocks = (tiles + WAVES - 1) / WAVES;
   const size_t lds = size_t(FT) * 16 * c.fh * c.fw * c.c + FT * 16 * sizeof(int);  // the filter bank + corrections
+  plan::work(plan::UNIT_MFMA_I8, 2.0 * pixels * c.f * c.fh * c.fw * c.c,
+             double(c.b) * (c.oh + c.fh - 1) * (c.ow + c.fw - 1) * c.c + double(c.f) * c.fh * c.fw * c.c +
+                 4.0 * pixels * c.f * (c.accum ? 2 : 1));
   if (img_unsigned)
-    hipLaunchKernelGGL((k_conv_i8<SLABS, true, WAVES>), dim3(blocks, groups), dim3(64 * WAVES), lds, stream, c, uint32_t(pixels), tiles);
+    MRL_LAUNCH((k_conv_i8<SLABS, true, WAVES>), dim3(blocks, groups), dim3(64 * WAVES), lds, stream, c, uint32_t(pixels), tiles);
   else
-    hipLaunchKernelGGL((k_conv_i8<SLABS, false, WAVES>), dim3(blocks, groups), dim3(64 * WAVES), lds, stream, c, uint32_t(pixels), tiles);
-  return hipGetLastError();
+    MRL_LAUNCH((k_conv_i8<SLABS, false, WAVES>), dim3(blocks, groups), dim3(64 * WAVES), lds, stream, c, uint32_t(pixels), tiles);
+  return mrl::plan::last_error();
 }
 
 int slabs_of(const ConvArgs &c) { return int(c.fh * c.fw * (c.c / 64)); }

@@ -508,21 +508,30 @@ inline bool edge_addressable(const GemmArgs &g, int elem_size) {
 
 template <class T, bool A_UNSIGNED, class TL, bool EDGE, bool B_KMAJOR = false, bool CONV = false>
 hipError_t launch(const GemmArgs &g, hipStream_t stream) {
-  auto kern = k_gemm<T, A_UNSIGNED, TL, EDGE, B_KMAJOR, CONV>;
+  constexpr auto kern = k_gemm<T, A_UNSIGNED, TL, EDGE, B_KMAJOR, CONV>;
   constexpr int BM = TL::BM, BN = TL::BN;
   constexpr int STAGE = TL::template stage<T>();
   if (EDGE && !edge_addressable(g, T::ES)) return hipErrorInvalidValue;
   static bool attr_set = false;
-  if (!attr_set) {
+  if (!attr_set && !plan::recording()) {
     hipError_t e = hipFuncSetAttribute((const void *)kern,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, 2 * STAGE);
     if (e != hipSuccess) return e;
     attr_set = true;
   }
   const int tiles_m = int((g.m + BM - 1) / BM), tiles_n = int((g.n + BN - 1) / BN);
-  hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n, g.batch), dim3(TL::NT), 2 * STAGE, stream, g,
-                     tiles_m, tiles_n);
-  return hipGetLastError();
+  {
+    const double k_steps = double((g.k * T::ES + TL::BKB - 1) / TL::BKB) * (TL::BKB / T::ES);  // k, padded to steps
+    const double mn = double(g.m) * g.n * g.batch;
+    plan::work(T::ES == 1 ? plan::UNIT_MFMA_I8 : T::ES == 2 ? plan::UNIT_MFMA_BF16 : plan::UNIT_MFMA_F32,
+               2.0 * mn * g.k, (double(g.m) * g.k + double(g.k) * g.n) * g.batch * T::ES + mn * 4 * (g.accum ? 2 : 1),
+               2.0 * BM * BN * k_steps,
+               // prologue and epilogue, then one barrier-to-barrier trip per 128 bytes of K
+               500.0 + 450.0 * double((g.k * T::ES + TL::BKB - 1) / TL::BKB));
+  }
+  MRL_LAUNCH((k_gemm<T, A_UNSIGNED, TL, EDGE, B_KMAJOR, CONV>), dim3(tiles_m * tiles_n, g.batch), dim3(TL::NT),
+             2 * STAGE, stream, g, tiles_m, tiles_n);
+  return mrl::plan::last_error();
 }
 
 

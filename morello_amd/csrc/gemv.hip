@@ -124,8 +124,11 @@ __global__ __launch_bounds__(64 * WAVES) void k_gemv(GemmArgs g) {
 template <int KIND, int ROWS, int COLS>
 hipError_t launch_as(const GemmArgs &g, hipStream_t stream) {
   const dim3 grid(uint32_t((uint64_t(g.n) + COLS * WAVES - 1) / (COLS * WAVES)), g.batch), block(64 * WAVES);
-  hipLaunchKernelGGL((k_gemv<KIND, ROWS, COLS>), grid, block, 0, stream, g);
-  return hipGetLastError();
+  constexpr int ES = KIND == 3 ? 4 : KIND == 2 ? 2 : 1;
+  plan::work(plan::UNIT_STREAM, 2.0 * g.m * g.n * g.k * g.batch,
+             double(g.batch) * ((double(g.m) + g.n) * g.k * ES + 4.0 * g.m * g.n));
+  MRL_LAUNCH((k_gemv<KIND, ROWS, COLS>), grid, block, 0, stream, g);
+  return mrl::plan::last_error();
 }
 
 template <int KIND>

@@ -662,16 +662,17 @@ __global__ __launch_bounds__(256) void k_softmax_generic(SM p) {
 
 // The scan dim is strided but another dim (`fast`) is contiguous on both sides: a workgroup
 // takes 64 consecutive positions of `fast` (one per lane, so every access is a 256-byte run)
-// and its four waves split the scan dim; each lane keeps the online (max, denominator) pair of
-// morello/src/spec.rs:96-106 over its share, the four shares are merged through LDS with the
+// and its WAVES waves (16 for long scan dims) split the scan dim; each lane keeps the online (max, denominator) pair of
+// morello/src/spec.rs:96-106 over its share, the shares are merged through LDS with the
 // parts formula (spec.rs:107-132), and a second sweep writes exp(x - max) / denominator.
 struct SMC {
   SM s;
   uint32_t fast, fast_tiles;
 };
-__global__ __launch_bounds__(256) void k_softmax_cols(SMC q) {
+template <int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void k_softmax_cols(SMC q) {
   const SM &p = q.s;
-  __shared__ float sm_max[4][64], sm_den[4][64];
+  __shared__ float sm_max[WAVES][64], sm_den[WAVES][64];
   const uint32_t lane = threadIdx.x % 64, w = threadIdx.x / 64;
   uint64_t r = blockIdx.x;
   const uint32_t f = uint32_t(r % q.fast_tiles) * 64 + lane;
@@ -690,12 +691,23 @@ __global__ __launch_bounds__(256) void k_softmax_cols(SMC q) {
   const int64_t is = p.si[p.scan_dim], os = p.so[p.scan_dim];
   float mx = -3.40282347e+38f, den = 0.0f;
   bool nan = false;
+  // Eight loads in flight per lane, then one rescale of the running denominator for the eight.
+  constexpr int UNROLL = 8;
   if (live)
-    for (uint32_t i = w; i < n; i += 4) {
-      const float x = p.in[ibase + i * is];
-      nan |= x != x;
-      const float nm = fmaxf(mx, x);
-      den = den * expf(mx - nm) + expf(x - nm);
+    for (uint32_t i0 = w; i0 < n; i0 += WAVES * UNROLL) {
+      float x[UNROLL];
+      float nm = mx;
+#pragma unroll
+      for (int j = 0; j < UNROLL; j++) {
+        const uint32_t i = i0 + j * WAVES;
+        x[j] = i < n ? p.in[ibase + i * is] : -3.40282347e+38f;
+        nan |= x[j] != x[j];
+        nm = fmaxf(nm, x[j]);
+      }
+      float add = 0.0f;
+#pragma unroll
+      for (int j = 0; j < UNROLL; j++) add += i0 + j * WAVES < n ? expf(x[j] - nm) : 0.0f;
+      den = den * expf(mx - nm) + add;
       mx = nm;
     }
   if (nan) mx = __uint_as_float(0x7fc00000u);
@@ -703,14 +715,26 @@ __global__ __launch_bounds__(256) void k_softmax_cols(SMC q) {
   __syncthreads();
   float m = sm_max[0][lane], d = sm_den[0][lane];
 #pragma unroll
-  for (int o = 1; o < 4; o++) {
+  for (int o = 1; o < WAVES; o++) {
     const float om = sm_max[o][lane], od = sm_den[o][lane];
     const float nm = (om != om || m != m) ? __uint_as_float(0x7fc00000u) : fmaxf(m, om);
     d = d * expf(m - nm) + od * expf(om - nm);
     m = nm;
   }
   if (live)
-    for (uint32_t i = w; i < n; i += 4) p.out[obase + i * os] = expf(p.in[ibase + i * is] - m) / d;
+    for (uint32_t i0 = w; i0 < n; i0 += WAVES * UNROLL) {
+      float x[UNROLL];
+#pragma unroll
+      for (int j = 0; j < UNROLL; j++) {
+        const uint32_t i = i0 + j * WAVES;
+        x[j] = i < n ? p.in[ibase + i * is] : 0.0f;
+      }
+#pragma unroll
+      for (int j = 0; j < UNROLL; j++) {
+        const uint32_t i = i0 + j * WAVES;
+        if (i < n) p.out[obase + i * os] = expf(x[j] - m) / d;
+      }
+    }
 }
 
 __global__ void k_fill_zero(uint32_t *p, uint64_t words, uint8_t *tail, uint32_t tail_bytes) {
@@ -728,17 +752,19 @@ hipError_t launch_relayout(const void *src, void *dst, const LayoutEval &sl, con
                            uint32_t es, uint64_t count, hipStream_t stream) {
   if (count == 0) return hipSuccess;
   const uint32_t blocks = uint32_t((count + 255) / 256);
-  hipLaunchKernelGGL(k_relayout, dim3(blocks), dim3(256), 0, stream, (const uint8_t *)src,
+  plan::work(plan::UNIT_VALU, 40.0 * count, 2.0 * count * es);  // index arithmetic per element
+  MRL_LAUNCH(k_relayout, dim3(blocks), dim3(256), 0, stream, (const uint8_t *)src,
                      (uint8_t *)dst, sl, dl, es, count);
-  return hipGetLastError();
+  return mrl::plan::last_error();
 }
 
 hipError_t launch_move_generic(const void *src, void *dst, const LayoutEval &sl, const LayoutEval &dl,
                                int sdt, int ddt, uint64_t count, hipStream_t stream) {
   if (count == 0) return hipSuccess;
   const uint32_t blocks = uint32_t((count + 255) / 256);
-  hipLaunchKernelGGL(k_move_generic, dim3(blocks), dim3(256), 0, stream, src, dst, sl, dl, sdt, ddt, count);
-  return hipGetLastError();
+  plan::work(plan::UNIT_VALU, 40.0 * count, double(count) * (mrl_dtype_size(sdt) + mrl_dtype_size(ddt)));
+  MRL_LAUNCH(k_move_generic, dim3(blocks), dim3(256), 0, stream, src, dst, sl, dl, sdt, ddt, count);
+  return mrl::plan::last_error();
 }
 
 hipError_t launch_copy(const void *src, void *dst, uint64_t bytes, hipStream_t stream) {
@@ -746,13 +772,14 @@ hipError_t launch_copy(const void *src, void *dst, uint64_t bytes, hipStream_t s
   if (vecs) {
     uint64_t blocks = (vecs + 256 * COPY_UNROLL - 1) / (256 * COPY_UNROLL);
     if (blocks > 8192) blocks = 8192;  // grid-stride: 32 blocks per CU on a 256-CU part
-    hipLaunchKernelGGL(k_copy16, dim3(uint32_t(blocks)), dim3(256), 0, stream, (const v4u *)src,
+    plan::work(plan::UNIT_STREAM, 0, 2.0 * bytes);
+    MRL_LAUNCH(k_copy16, dim3(uint32_t(blocks)), dim3(256), 0, stream, (const v4u *)src,
                        (v4u *)dst, vecs);
   }
   if (tail)
-    hipLaunchKernelGGL(k_copy1, dim3(1), dim3(16), 0, stream, (const uint8_t *)src + vecs * 16,
+    MRL_LAUNCH(k_copy1, dim3(1), dim3(16), 0, stream, (const uint8_t *)src + vecs * 16,
                        (uint8_t *)dst + vecs * 16, tail);
-  return hipGetLastError();
+  return mrl::plan::last_error();
 }
 
 // Move over a common strided view of the two sides (layout_factor.h).  Returns
@@ -761,6 +788,11 @@ hipError_t launch_copy(const void *src, void *dst, uint64_t bytes, hipStream_t s
 hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_dtype,
                             const MoveDim *dims, uint32_t rank, hipStream_t stream) {
   if (rank > MOVE_MAX_RANK) return hipErrorInvalidValue;
+  {
+    double count = 1;
+    for (uint32_t d = 0; d < rank; d++) count *= dims[d].size;
+    plan::work(plan::UNIT_STREAM, 0, count * (mrl_dtype_size(src_dtype) + mrl_dtype_size(dst_dtype)));
+  }
   // Elements narrower than 4 bytes that travel together (a digit contiguous on both sides, no
   // conversion) are moved as 2- or 4-byte units: a Packed(4) digit of bytes becomes one u32.
   MoveDim wide[MOVE_MAX_RANK];
@@ -826,12 +858,12 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
       const uint32_t blocks = uint32_t(std::min<uint64_t>((p.count / 4 + 255) / 256, 1u << 20));
       const dim3 grid{blocks}, block{256};
 #define MRL_CONVERT(SE, DE) \
-  if (se == SE && de == DE) hipLaunchKernelGGL((k_convert4<SE, DE>), grid, block, 0, stream, src, dst, src_dtype, dst_dtype, p.count)
+  if (se == SE && de == DE) MRL_LAUNCH((k_convert4<SE, DE>), grid, block, 0, stream, src, dst, src_dtype, dst_dtype, p.count)
       MRL_CONVERT(1, 1); MRL_CONVERT(1, 2); MRL_CONVERT(1, 4);
       MRL_CONVERT(2, 1); MRL_CONVERT(2, 2); MRL_CONVERT(2, 4);
       MRL_CONVERT(4, 1); MRL_CONVERT(4, 2); MRL_CONVERT(4, 4);
 #undef MRL_CONVERT
-      return hipGetLastError();
+      return mrl::plan::last_error();
     }
     if (vectors) {
       for (uint32_t d = 0; d < rank; d++) {
@@ -842,9 +874,9 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
     }
     const uint64_t blocks = (p.count + 255) / 256;
     if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
-    if (vectors) hipLaunchKernelGGL(k_move_rows16, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
-    else hipLaunchKernelGGL(k_move_rows, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
-    return hipGetLastError();
+    if (vectors) MRL_LAUNCH(k_move_rows16, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+    else MRL_LAUNCH(k_move_rows, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+    return mrl::plan::last_error();
   }
   // Two long contiguous dims: the 64 x 64 transpose.
   if (dim_s != dim_d && p.shape[dim_s] >= 32 && p.shape[dim_d] >= 32) {
@@ -861,9 +893,9 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
     for (uint32_t d = 0; d < p.rank; d++)
       if (int(d) != dim_s && int(d) != dim_d) blocks *= p.shape[d];
     if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
-    if (pairs) hipLaunchKernelGGL(k_move_tiled16, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
-    else hipLaunchKernelGGL(k_move_tiled, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
-    return hipGetLastError();
+    if (pairs) MRL_LAUNCH(k_move_tiled16, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+    else MRL_LAUNCH(k_move_tiled, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+    return mrl::plan::last_error();
   }
   // Otherwise a tile grown digit by digit: along the destination's fastest digits until they
   // make a run of 64, along the source's fastest until they do, then along the destination's
@@ -921,13 +953,13 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
     if (d != fs && p.ss[d] % run != 0) t.vec_s = false;
     if (d != fd && p.ds[d] % run != 0) t.vec_d = false;
   }
-  if (src_dtype != dst_dtype) hipLaunchKernelGGL((k_move_gather<void, 1>), grid, dim3(256), 0, stream, t);
-  else if (elem == 4 && run == 4) hipLaunchKernelGGL((k_move_gather<uint32_t, 4>), grid, dim3(256), 0, stream, t);
-  else if (elem == 4 && run == 2) hipLaunchKernelGGL((k_move_gather<uint32_t, 2>), grid, dim3(256), 0, stream, t);
-  else if (elem == 4) hipLaunchKernelGGL((k_move_gather<uint32_t, 1>), grid, dim3(256), 0, stream, t);
-  else if (elem == 2) hipLaunchKernelGGL((k_move_gather<uint16_t, 1>), grid, dim3(256), 0, stream, t);
-  else hipLaunchKernelGGL((k_move_gather<uint8_t, 1>), grid, dim3(256), 0, stream, t);
-  return hipGetLastError();
+  if (src_dtype != dst_dtype) MRL_LAUNCH((k_move_gather<void, 1>), grid, dim3(256), 0, stream, t);
+  else if (elem == 4 && run == 4) MRL_LAUNCH((k_move_gather<uint32_t, 4>), grid, dim3(256), 0, stream, t);
+  else if (elem == 4 && run == 2) MRL_LAUNCH((k_move_gather<uint32_t, 2>), grid, dim3(256), 0, stream, t);
+  else if (elem == 4) MRL_LAUNCH((k_move_gather<uint32_t, 1>), grid, dim3(256), 0, stream, t);
+  else if (elem == 2) MRL_LAUNCH((k_move_gather<uint16_t, 1>), grid, dim3(256), 0, stream, t);
+  else MRL_LAUNCH((k_move_gather<uint8_t, 1>), grid, dim3(256), 0, stream, t);
+  return mrl::plan::last_error();
 }
 
 // Move between two strided layouts of the same logical shape.
@@ -947,27 +979,29 @@ hipError_t launch_pad_rows(const Strided &src, void *dst, uint32_t dst_ld, uint3
   if (dwords == 0) return hipSuccess;
   const uint32_t blocks = uint32_t(std::min<uint64_t>((dwords + 255) / 256, 65536));
   const int64_t sb = batch == 1 ? 0 : src.stride[0], sl = rows == 1 ? 0 : src.stride[1];
+  plan::work(plan::UNIT_STREAM, 0, double(batch) * rows * cols * elem_size + 4.0 * dwords);
   if (elem_size == 1)
-    hipLaunchKernelGGL(k_pad_rows<uint8_t>, dim3(blocks), dim3(256), 0, stream, (const uint8_t *)src.ptr,
+    MRL_LAUNCH(k_pad_rows<uint8_t>, dim3(blocks), dim3(256), 0, stream, (const uint8_t *)src.ptr,
                        (uint32_t *)dst, rows, cols, sb, sl, dst_ld, dwords);
   else if (elem_size == 2)
-    hipLaunchKernelGGL(k_pad_rows<uint16_t>, dim3(blocks), dim3(256), 0, stream, (const uint16_t *)src.ptr,
+    MRL_LAUNCH(k_pad_rows<uint16_t>, dim3(blocks), dim3(256), 0, stream, (const uint16_t *)src.ptr,
                        (uint32_t *)dst, rows, cols, sb, sl, dst_ld, dwords);
   else if (elem_size == 4)
-    hipLaunchKernelGGL(k_pad_rows<uint32_t>, dim3(blocks), dim3(256), 0, stream, (const uint32_t *)src.ptr,
+    MRL_LAUNCH(k_pad_rows<uint32_t>, dim3(blocks), dim3(256), 0, stream, (const uint32_t *)src.ptr,
                        (uint32_t *)dst, rows, cols, sb, sl, dst_ld, dwords);
   else
     return hipErrorInvalidValue;
-  return hipGetLastError();
+  return mrl::plan::last_error();
 }
 
 hipError_t launch_widen_bf16(const void *src, void *dst, uint64_t count, hipStream_t stream) {
   if (count == 0) return hipSuccess;
   uint64_t blocks = (count + 255) / 256;
   if (blocks > 16384) blocks = 16384;
-  hipLaunchKernelGGL(k_widen_bf16, dim3(uint32_t(blocks)), dim3(256), 0, stream, (const uint16_t *)src,
+  plan::work(plan::UNIT_STREAM, 0, 6.0 * count);
+  MRL_LAUNCH(k_widen_bf16, dim3(uint32_t(blocks)), dim3(256), 0, stream, (const uint16_t *)src,
                      (uint32_t *)dst, count);
-  return hipGetLastError();
+  return mrl::plan::last_error();
 }
 
 hipError_t launch_matmul_generic(const Strided &a, const Strided &b, const Strided &c, int accum,
@@ -981,9 +1015,15 @@ hipError_t launch_matmul_generic(const Strided &a, const Strided &b, const Strid
   const uint64_t tiles = uint64_t((p.N + 15) / 16) * ((p.M + 15) / 16) * p.B;
   if (tiles > 0x7fffffffull) return hipErrorInvalidValue;
   dim3 grid{uint32_t(tiles)};
-  if (float_out(c.dtype)) hipLaunchKernelGGL(k_matmul_generic<true>, grid, dim3(256), 0, stream, p);
-  else hipLaunchKernelGGL(k_matmul_generic<false>, grid, dim3(256), 0, stream, p);
-  return hipGetLastError();
+  {
+    const double mn = double(p.B) * p.M * p.N;
+    plan::work(plan::UNIT_VALU, 2.0 * mn * p.K,
+               double(p.B) * (double(p.M) * p.K * mrl_dtype_size(a.dtype) + double(p.K) * p.N * mrl_dtype_size(b.dtype)) +
+                   mn * mrl_dtype_size(c.dtype));
+  }
+  if (float_out(c.dtype)) MRL_LAUNCH(k_matmul_generic<true>, grid, dim3(256), 0, stream, p);
+  else MRL_LAUNCH(k_matmul_generic<false>, grid, dim3(256), 0, stream, p);
+  return mrl::plan::last_error();
 }
 
 hipError_t launch_conv_generic(const Strided &img, const Strided &filt, const Strided &out,
@@ -996,16 +1036,19 @@ hipError_t launch_conv_generic(const Strided &img, const Strided &filt, const St
   for (int d = 0; d < 4; d++) p.si[d] = img.stride[d], p.sf[d] = filt.stride[d], p.so[d] = out.stride[d];
   p.accum = accum;
   const uint64_t total = uint64_t(p.B) * p.F * p.OH * p.OW;
+  plan::work(plan::UNIT_VALU, 2.0 * total * p.C * p.FH * p.FW,
+             double(p.B) * p.C * (p.OH + p.FH - 1) * (p.OW + p.FW - 1) * mrl_dtype_size(img.dtype) +
+                 double(total) * mrl_dtype_size(out.dtype));
   if (total <= 16384 && uint64_t(p.C) * p.FH * p.FW >= 32) {  // few outputs, long reductions
     const uint32_t wave_blocks = uint32_t((total + 3) / 4);
-    if (float_out(out.dtype)) hipLaunchKernelGGL(k_conv_generic_wave<true>, dim3(wave_blocks), dim3(256), 0, stream, p);
-    else hipLaunchKernelGGL(k_conv_generic_wave<false>, dim3(wave_blocks), dim3(256), 0, stream, p);
-    return hipGetLastError();
+    if (float_out(out.dtype)) MRL_LAUNCH(k_conv_generic_wave<true>, dim3(wave_blocks), dim3(256), 0, stream, p);
+    else MRL_LAUNCH(k_conv_generic_wave<false>, dim3(wave_blocks), dim3(256), 0, stream, p);
+    return mrl::plan::last_error();
   }
   const uint32_t blocks = uint32_t((total + 255) / 256);
-  if (float_out(out.dtype)) hipLaunchKernelGGL(k_conv_generic<true>, dim3(blocks), dim3(256), 0, stream, p);
-  else hipLaunchKernelGGL(k_conv_generic<false>, dim3(blocks), dim3(256), 0, stream, p);
-  return hipGetLastError();
+  if (float_out(out.dtype)) MRL_LAUNCH(k_conv_generic<true>, dim3(blocks), dim3(256), 0, stream, p);
+  else MRL_LAUNCH(k_conv_generic<false>, dim3(blocks), dim3(256), 0, stream, p);
+  return mrl::plan::last_error();
 }
 
 hipError_t launch_softmax_generic(const Strided &in, const Strided &out, uint32_t scan_dim,
@@ -1021,6 +1064,7 @@ hipError_t launch_softmax_generic(const Strided &in, const Strided &out, uint32_
     if (d < in.rank && d != scan_dim) lines *= in.shape[d];
   }
   p.lines = lines;
+  plan::work(plan::UNIT_VALU, 20.0 * lines * in.shape[scan_dim], 8.0 * lines * in.shape[scan_dim]);
   // A dim other than the scan dim that both sides store contiguously: the column kernel.
   for (uint32_t d = 0; d < in.rank; d++)
     if (d != scan_dim && in.shape[d] >= 16 && in.stride[d] == 1 && out.stride[d] == 1) {
@@ -1028,12 +1072,13 @@ hipError_t launch_softmax_generic(const Strided &in, const Strided &out, uint32_
       q.s = p, q.fast = d, q.fast_tiles = (in.shape[d] + 63) / 64;
       const uint64_t blocks = lines / in.shape[d] * q.fast_tiles;
       if (blocks > 0x7fffffffull) break;
-      hipLaunchKernelGGL(k_softmax_cols, dim3(uint32_t(blocks)), dim3(256), 0, stream, q);
-      return hipGetLastError();
+      if (in.shape[scan_dim] >= 512) MRL_LAUNCH(k_softmax_cols<16>, dim3(uint32_t(blocks)), dim3(1024), 0, stream, q);
+      else MRL_LAUNCH(k_softmax_cols<4>, dim3(uint32_t(blocks)), dim3(256), 0, stream, q);
+      return mrl::plan::last_error();
     }
   const uint32_t blocks = uint32_t((lines + 3) / 4);
-  hipLaunchKernelGGL(k_softmax_generic, dim3(blocks), dim3(256), 0, stream, p);
-  return hipGetLastError();
+  MRL_LAUNCH(k_softmax_generic, dim3(blocks), dim3(256), 0, stream, p);
+  return mrl::plan::last_error();
 }
 
 hipError_t launch_fill_zero(void *ptr, uint64_t bytes, hipStream_t stream) {
@@ -1043,9 +1088,10 @@ hipError_t launch_fill_zero(void *ptr, uint64_t bytes, hipStream_t stream) {
   uint64_t blocks = (words + 255) / 256;
   if (blocks > 65536) blocks = 65536;
   if (blocks == 0) blocks = 1;
-  hipLaunchKernelGGL(k_fill_zero, dim3(uint32_t(blocks)), dim3(256), 0, stream, (uint32_t *)ptr,
+  plan::work(plan::UNIT_STREAM, 0, double(bytes));
+  MRL_LAUNCH(k_fill_zero, dim3(uint32_t(blocks)), dim3(256), 0, stream, (uint32_t *)ptr,
                      words, (uint8_t *)ptr + words * 4, tail);
-  return hipGetLastError();
+  return mrl::plan::last_error();
 }
 
 }  // namespace mrl

@@ -4,6 +4,7 @@
 #include <stdint.h>
 
 #include "layout_math.h"
+#include "plan.h"
 
 namespace mrl {
 
@@ -116,10 +117,15 @@ hipError_t launch_unfold(const void *image, void *rows, uint32_t batch, uint32_t
                          uint32_t elem_size, hipStream_t stream);
 
 // ---- softmax.hip: f32 softmax over a contiguous innermost scan dim ---------------------
-hipError_t launch_softmax_rows(const float *in, float *out, uint64_t rows, uint32_t cols,
+// Rows longer than 4096 run a workgroup per SOFTMAX_CHUNK elements and want
+// softmax_scratch_bytes() of device scratch for the chunks' (max, denominator) pairs; with a
+// null `scratch` they fall back to one wavefront per row.  `out` may be `in`.
+constexpr uint32_t SOFTMAX_CHUNK = 4096;
+size_t softmax_scratch_bytes(uint64_t rows, uint32_t cols);
+hipError_t launch_softmax_rows(const float *in, float *out, uint64_t rows, uint32_t cols, void *scratch,
                                hipStream_t stream);
 // The same with the result rounded to bf16 (rows of `cols` 16-bit values).
-hipError_t launch_softmax_rows_bf16(const float *in, void *out, uint64_t rows, uint32_t cols,
+hipError_t launch_softmax_rows_bf16(const float *in, void *out, uint64_t rows, uint32_t cols, void *scratch,
                                     hipStream_t stream);
 
 // ---- parts.hip: the primitive Specs of the Softmax decomposition, Broadcast, Fill ----------

@@ -177,16 +177,18 @@ hipError_t launch_parts(const PartsArgs &p, hipStream_t stream) {
   if (p.lines == 0) return hipSuccess;
   const uint64_t blocks = (p.lines + 3) / 4;
   if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(k_parts, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
-  return hipGetLastError();
+  plan::work(plan::UNIT_STREAM, 0, 8.0 * p.lines * p.shape[p.scan_dim]);  // the full-size tensors, read and written
+  MRL_LAUNCH(k_parts, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+  return mrl::plan::last_error();
 }
 
 hipError_t launch_broadcast(const void *in, void *out, const LayoutEval &il, const LayoutEval &ol,
                             uint32_t dim, uint32_t elem_size, uint64_t count, hipStream_t stream) {
   if (count == 0) return hipSuccess;
-  hipLaunchKernelGGL(k_broadcast, dim3(uint32_t((count + 255) / 256)), dim3(256), 0, stream,
+  plan::work(plan::UNIT_VALU, 30.0 * count, 2.0 * count * elem_size);
+  MRL_LAUNCH(k_broadcast, dim3(uint32_t((count + 255) / 256)), dim3(256), 0, stream,
                      (const uint8_t *)in, (uint8_t *)out, il, ol, dim, elem_size, count);
-  return hipGetLastError();
+  return mrl::plan::last_error();
 }
 
 // FillValue (spec.rs:165-170): 0 Zero, 1 NegInf (floats), 2 Min (the dtype's minimum;
@@ -206,9 +208,10 @@ hipError_t launch_fill(void *out, int dtype, int fill_value, uint64_t count, hip
     }
   }
   const uint32_t es = dtype == MRL_U8 || dtype == MRL_I8 ? 1 : (dtype == MRL_U16 || dtype == MRL_I16 || dtype == MRL_BF16 ? 2 : 4);
-  hipLaunchKernelGGL(k_fill, dim3(uint32_t((count + 255) / 256)), dim3(256), 0, stream, (uint8_t *)out,
+  plan::work(plan::UNIT_STREAM, 0, double(count) * es);
+  MRL_LAUNCH(k_fill, dim3(uint32_t((count + 255) / 256)), dim3(256), 0, stream, (uint8_t *)out,
                      pattern, es, count);
-  return hipGetLastError();
+  return mrl::plan::last_error();
 }
 
 }  // namespace mrl

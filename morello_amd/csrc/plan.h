@@ -1,0 +1,70 @@
+// Planning a Spec without running it.
+//
+// Morello's search asks a target two things about a Spec: which kernel applies
+// (Kernel::applies_to_logical_spec, morello/src/target/mod.rs:97-117) and what it costs
+// (Kernel::main_cost, Kernel::memory_allocated; morello/src/cost.rs:33-76).  This backend picks
+// its kernels inside the dispatch code, from shapes, dtypes, layouts and alignment.  So that the
+// answers can never drift from what a run does, planning *is* that dispatch code: a thread that
+// has a Recorder installed goes through the same decisions with stand-in addresses, and every
+// launch site notes the kernel it would have launched instead of launching it.  No HIP call is
+// made in that mode, so planning works on a machine without a GPU.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <string>
+#include <vector>
+
+namespace mrl {
+namespace plan {
+
+// What bounds a kernel besides its traffic.
+enum Unit : int { UNIT_STREAM = 0, UNIT_MFMA_I8 = 1, UNIT_MFMA_BF16 = 2, UNIT_MFMA_F32 = 3, UNIT_VALU = 4 };
+
+struct Step {
+  std::string kernel;       // "k_gemm [T = I8, A_UNSIGNED = true, TL = Tile<256, 256, 128, 2, 4>, EDGE = false, ...]"
+  uint32_t grid[3], block[3];
+  uint32_t lds_bytes;       // dynamic LDS of the launch
+  int unit;                 // Unit
+  double ops, bytes;        // arithmetic and HBM traffic the launcher declared (0 when it did not)
+  double tile_ops;          // MFMA kernels: arithmetic of one workgroup, padding included
+  double serial_ns;         // a workgroup's dependent chain (loop trips x their latency): no launch is shorter
+};
+
+struct Recorder {
+  std::vector<Step> steps;
+  size_t scratch_bytes = 0;  // device scratch the call would take
+  // Declared for the next launch.
+  int unit = UNIT_STREAM;
+  double ops = 0, bytes = 0, tile_ops = 0, serial_ns = 0;
+};
+
+extern thread_local Recorder *g_recorder;
+
+inline bool recording() { return g_recorder != nullptr; }
+
+// The launch site's declaration of the next kernel's work; a no-op outside planning.
+inline void work(int unit, double ops, double bytes, double tile_ops = 0, double serial_ns = 0) {
+  if (!g_recorder) return;
+  g_recorder->unit = unit, g_recorder->ops = ops, g_recorder->bytes = bytes;
+  g_recorder->tile_ops = tile_ops, g_recorder->serial_ns = serial_ns;
+}
+
+// `kernel_text`: the kernel expression as written at the launch site; `launcher`: the
+// __PRETTY_FUNCTION__ of the function around it, whose "[T = ..., EDGE = ...]" part spells out the
+// template arguments the kernel was instantiated with.
+void note(const char *kernel_text, const char *launcher, dim3 grid, dim3 block, size_t lds_bytes);
+
+// Predicted duration of one planned launch, in nanoseconds.
+double step_ns(const Step &s, uint32_t compute_units);
+
+inline hipError_t last_error() { return g_recorder ? hipSuccess : hipGetLastError(); }
+
+}  // namespace plan
+}  // namespace mrl
+
+#define MRL_LAUNCH(kernel, grid, block, lds, stream, ...)                                              \
+  do {                                                                                                 \
+    if (mrl::plan::recording()) mrl::plan::note(#kernel, __PRETTY_FUNCTION__, grid, block, lds);            \
+    else hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);                             \
+  } while (0)

@@ -1,0 +1,87 @@
+// Recorder of planned launches and the cost model over them (host code only).
+#include "plan.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+
+namespace mrl {
+namespace plan {
+
+thread_local Recorder *g_recorder = nullptr;
+
+// "(k_attn<D, RAGGED, KT_ROWS>)" within "hipError_t mrl::(anonymous namespace)::launch_one(...)
+// [D = 128, RAGGED = false, KT_ROWS = false]" -> "k_attn [D = 128, RAGGED = false, KT_ROWS = false]".
+static std::string kernel_name(const char *kernel_text, const char *launcher) {
+  std::string family(kernel_text);
+  family.erase(0, family.find_first_not_of("( "));
+  family = family.substr(0, family.find_first_of("<) "));
+  std::string args(launcher);
+  const size_t at = args.rfind(" [");
+  if (at == std::string::npos || !std::strchr(kernel_text, '<')) return family;  // not a template kernel
+  args = args.substr(at);
+  for (const char *drop : {"mrl::", "gemm::", "(anonymous namespace)::", "plan::"}) {
+    const size_t n = std::strlen(drop);
+    for (size_t i = args.find(drop); i != std::string::npos; i = args.find(drop, i)) args.erase(i, n);
+  }
+  return family + args;
+}
+
+void note(const char *kernel_text, const char *launcher, dim3 grid, dim3 block, size_t lds_bytes) {
+  Recorder *r = g_recorder;
+  if (!r) return;
+  Step step;
+  step.kernel = kernel_name(kernel_text, launcher);
+  step.grid[0] = grid.x, step.grid[1] = grid.y, step.grid[2] = grid.z;
+  step.block[0] = block.x, step.block[1] = block.y, step.block[2] = block.z;
+  step.lds_bytes = uint32_t(lds_bytes);
+  step.unit = r->unit, step.ops = r->ops, step.bytes = r->bytes, step.tile_ops = r->tile_ops;
+  step.serial_ns = r->serial_ns;
+  r->steps.push_back(step);
+  r->unit = UNIT_STREAM, r->ops = r->bytes = r->tile_ops = r->serial_ns = 0;
+}
+
+// Nanoseconds of one planned launch on an MI355X, launches queued back to back on one stream.
+// Constants are fits to launches measured through the timed-run entry point (benchmark
+// configurations and the size sweeps the tests cover): the model is
+//     launch gap + max(traffic / streaming rate, arithmetic / sustained rate),
+// the arithmetic of a matrix-core kernel being its workgroups' padded tiles taken in rounds over
+// the compute units.
+double step_ns(const Step &s, uint32_t compute_units) {
+  constexpr double LAUNCH_NS = 2200.0;        // gap between dependent launches on a stream
+  constexpr double STREAM_BYTES_PER_NS = 5500.0;  // 5.5 TB/s: what copy / softmax / GEMV kernels sustain
+  // Sustained whole-chip rates under the board's power limit, ops per ns.
+  double rate = 0;
+  switch (s.unit) {
+    case UNIT_MFMA_I8: rate = 1440e3; break;
+    case UNIT_MFMA_BF16: rate = 1150e3; break;
+    case UNIT_MFMA_F32: rate = 95e3; break;
+    case UNIT_VALU: rate = 3e3; break;   // the generic kernels: dtype switches and index arithmetic per term
+    default: break;
+  }
+  const double workgroups = double(s.grid[0]) * s.grid[1] * s.grid[2];
+  double bytes = s.bytes;
+  if (bytes == 0 && s.ops == 0) bytes = workgroups * s.block[0] * s.block[1] * s.block[2] * 16.0;  // undeclared: a guess
+  double compute = 0;
+  if (rate > 0) {
+    if (s.tile_ops > 0) {
+      // Workgroups per compute unit at a time: bounded by LDS (160 KiB) and by threads (2048).
+      const double threads = double(s.block[0]) * s.block[1] * s.block[2];
+      double resident = std::floor(2048.0 / std::max(64.0, threads));
+      if (s.lds_bytes) resident = std::min(resident, std::floor(160.0 * 1024 / s.lds_bytes));
+      resident = std::max(1.0, std::min(resident, 8.0));
+      const double slots = compute_units * resident;
+      const double rounds = std::ceil(workgroups / slots);
+      // A round's workgroups share their compute unit's matrix pipes.
+      const double in_round = std::min(workgroups, slots) / compute_units;   // per CU, first round
+      const double per_round = s.tile_ops * std::max(1.0, std::min(resident, std::ceil(in_round))) / (rate / compute_units);
+      compute = rounds * per_round;
+    } else {
+      compute = s.ops / rate;
+    }
+  }
+  return LAUNCH_NS + std::max({bytes / STREAM_BYTES_PER_NS, compute, s.serial_ns});
+}
+
+}  // namespace plan
+}  // namespace mrl

@@ -129,37 +129,248 @@ __global__ __launch_bounds__(256) void k_softmax_stream(const float *__restrict_
   }
 }
 
+// ---- rows longer than the register kernel takes: a workgroup per 4096-element chunk ----
+// One wavefront per row leaves a few long rows (64 x 100000) on a handful of compute units, and
+// its scalar loop waits out every load.  Here a workgroup owns SOFTMAX_CHUNK consecutive elements
+// of one row, 16 per thread in registers: k_softmax_chunk_stats writes the chunk's (max,
+// denominator) pair, k_softmax_chunk_write merges the pairs of its row with the parts formula
+// (morello/src/spec.rs:107-132), reads its chunk again (from the cache, for tensors that fit
+// it) and writes exp(x - max) / denominator.  V: floats per load (4 when cols is a multiple
+// of 4, so that every chunk and row starts on 16 bytes; else 1).
+constexpr uint32_t CHUNK = SOFTMAX_CHUNK, PER_THREAD = CHUNK / 256;
+
+template <int V>
+__device__ inline void load_chunk(const float *__restrict__ row, uint32_t first, uint32_t cols, float (&x)[PER_THREAD],
+                                  uint32_t &valid) {
+  valid = 0;
+#pragma unroll
+  for (uint32_t i = 0; i < PER_THREAD / V; i++) {
+    const uint32_t idx = first + (i * 256 + threadIdx.x) * V;
+    if (idx < cols) {
+      valid |= ((1u << V) - 1) << (i * V);
+      if constexpr (V == 4) {
+        const f4 t = *(const f4 *)(row + idx);
+        x[4 * i] = t[0], x[4 * i + 1] = t[1], x[4 * i + 2] = t[2], x[4 * i + 3] = t[3];
+      } else {
+        x[i] = row[idx];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < V; j++) x[i * V + j] = F32_MIN;
+    }
+  }
+}
+
+// (max, denominator) pairs of the four waves -> the workgroup's, in every thread.
+__device__ inline void merge_waves(float &mx, float &den, bool &nan, float (*lds)[4]) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float om = __shfl_xor(mx, o), od = __shfl_xor(den, o);
+    const float nm = fmaxf(mx, om);
+    den = den * expf(mx - nm) + od * expf(om - nm);
+    mx = nm;
+  }
+  nan = __any(nan);
+  const uint32_t w = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) lds[0][w] = mx, lds[1][w] = den, lds[2][w] = nan ? 1.0f : 0.0f;
+  __syncthreads();
+  mx = lds[0][0], den = lds[1][0], nan = lds[2][0] != 0.0f;
+#pragma unroll
+  for (int o = 1; o < 4; o++) {
+    const float om = lds[0][o], od = lds[1][o];
+    const float nm = fmaxf(mx, om);
+    den = den * expf(mx - nm) + od * expf(om - nm);
+    mx = nm;
+    nan |= lds[2][o] != 0.0f;
+  }
+}
+
+template <int V>
+__global__ __launch_bounds__(256) void k_softmax_chunk_stats(const float *__restrict__ in, float2 *__restrict__ stats,
+                                                             uint32_t cols, uint32_t chunks) {
+  __shared__ float lds[3][4];
+  const uint32_t chunk = blockIdx.x % chunks;
+  const uint64_t row = blockIdx.x / chunks;
+  float x[PER_THREAD];
+  uint32_t valid;
+  load_chunk<V>(in + row * cols, chunk * CHUNK, cols, x, valid);
+  float mx = F32_MIN;
+  bool nan = false;
+#pragma unroll
+  for (uint32_t i = 0; i < PER_THREAD; i++) {
+    nan |= x[i] != x[i];
+    mx = fmaxf(mx, x[i]);  // slots past the row hold f32::MIN
+  }
+  float den = 0.0f;
+#pragma unroll
+  for (uint32_t i = 0; i < PER_THREAD; i++) den += (valid >> i & 1) ? expf(x[i] - mx) : 0.0f;
+  merge_waves(mx, den, nan, lds);
+  if (threadIdx.x == 0) stats[blockIdx.x] = float2{nan ? __uint_as_float(0x7fc00000u) : mx, den};
+}
+
+template <int V, bool OUT_BF16>
+__global__ __launch_bounds__(256) void k_softmax_chunk_write(const float *__restrict__ in, void *__restrict__ out_any,
+                                                             const float2 *__restrict__ stats, uint32_t cols,
+                                                             uint32_t chunks) {
+  __shared__ float lds[3][4];
+  const uint32_t chunk = blockIdx.x % chunks;
+  const uint64_t row = blockIdx.x / chunks;
+  // The chunk first: it may be overwritten below (the Spec's output can be its input's buffer).
+  float x[PER_THREAD];
+  uint32_t valid;
+  load_chunk<V>(in + row * cols, chunk * CHUNK, cols, x, valid);
+  float mx = F32_MIN, den = 0.0f;
+  bool nan = false;
+  for (uint32_t c = threadIdx.x; c < chunks; c += 256) {
+    const float2 s = stats[row * chunks + c];
+    nan |= s.x != s.x;
+    const float nm = fmaxf(mx, s.x);
+    den = den * expf(mx - nm) + s.y * expf(s.x - nm);
+    mx = nm;
+  }
+  merge_waves(mx, den, nan, lds);
+  if (nan) mx = __uint_as_float(0x7fc00000u);
+#pragma unroll
+  for (uint32_t i = 0; i < PER_THREAD / V; i++) {
+    const uint32_t idx = chunk * CHUNK + (i * 256 + threadIdx.x) * V;
+    if (idx >= cols) continue;
+    float y[V];
+#pragma unroll
+    for (int j = 0; j < V; j++) y[j] = expf(x[i * V + j] - mx) / den;
+    if constexpr (V == 4 && OUT_BF16) {
+      typedef unsigned u2 __attribute__((ext_vector_type(2)));
+      __builtin_nontemporal_store(u2{bf16_bits(y[0]) | (bf16_bits(y[1]) << 16), bf16_bits(y[2]) | (bf16_bits(y[3]) << 16)},
+                                  reinterpret_cast<u2 *>(static_cast<uint16_t *>(out_any) + row * cols + idx));
+    } else if constexpr (V == 4) {
+      __builtin_nontemporal_store(f4{y[0], y[1], y[2], y[3]}, (f4 *)(static_cast<float *>(out_any) + row * cols + idx));
+    } else if constexpr (OUT_BF16) {
+      (static_cast<uint16_t *>(out_any) + row * cols)[idx] = uint16_t(bf16_bits(y[0]));
+    } else {
+      (static_cast<float *>(out_any) + row * cols)[idx] = y[0];
+    }
+  }
+}
+
+// Rows of 4096 < cols <= NV * 1024 (cols a multiple of 4) when there are rows enough to fill
+// the chip with a workgroup each: the row stays in the workgroup's registers between the passes,
+// as in k_softmax_regs, so it is read once.
+template <int NV, bool OUT_BF16>
+__global__ __launch_bounds__(256) void k_softmax_block(const float *__restrict__ in, void *__restrict__ out_any,
+                                                       uint32_t cols) {
+  __shared__ float lds[2][4];
+  const uint64_t row = blockIdx.x;
+  const uint32_t nvec = cols / 4, w = threadIdx.x >> 6;
+  const f4 *src = (const f4 *)(in + row * cols);
+  f4 v[NV];
+  float mx = F32_MIN;
+  bool nan = false;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const uint32_t idx = i * 256 + threadIdx.x;
+    if (idx < nvec) {
+      v[i] = __builtin_nontemporal_load(src + idx);
+      nan |= (v[i][0] != v[i][0]) | (v[i][1] != v[i][1]) | (v[i][2] != v[i][2]) | (v[i][3] != v[i][3]);
+      mx = fmaxf(fmaxf(mx, fmaxf(v[i][0], v[i][1])), fmaxf(v[i][2], v[i][3]));
+    }
+  }
+  mx = wave_max(mx);
+  if ((threadIdx.x & 63) == 0) lds[0][w] = __any(nan) ? __uint_as_float(0x7fc00000u) : mx;
+  __syncthreads();
+  {
+    const float a = lds[0][0], b = lds[0][1], c = lds[0][2], d = lds[0][3];
+    mx = (a != a || b != b || c != c || d != d) ? __uint_as_float(0x7fc00000u) : fmaxf(fmaxf(a, b), fmaxf(c, d));
+  }
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const uint32_t idx = i * 256 + threadIdx.x;
+    if (idx < nvec) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) v[i][j] = expf(v[i][j] - mx);
+      sum += (v[i][0] + v[i][1]) + (v[i][2] + v[i][3]);
+    }
+  }
+  sum = wave_sum(sum);
+  if ((threadIdx.x & 63) == 0) lds[1][w] = sum;
+  __syncthreads();
+  sum = (lds[1][0] + lds[1][1]) + (lds[1][2] + lds[1][3]);
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const uint32_t idx = i * 256 + threadIdx.x;
+    if (idx < nvec) {
+      const f4 y = v[i] / sum;
+      if constexpr (OUT_BF16) {
+        typedef unsigned u2 __attribute__((ext_vector_type(2)));
+        __builtin_nontemporal_store(u2{bf16_bits(y[0]) | (bf16_bits(y[1]) << 16), bf16_bits(y[2]) | (bf16_bits(y[3]) << 16)},
+                                    reinterpret_cast<u2 *>(static_cast<uint16_t *>(out_any) + row * cols) + idx);
+      } else {
+        __builtin_nontemporal_store(y, (f4 *)(static_cast<float *>(out_any) + row * cols) + idx);
+      }
+    }
+  }
+}
+
+template <int V, bool OUT_BF16>
+hipError_t launch_chunks(const float *in, void *out, uint64_t rows, uint32_t cols, float2 *stats, hipStream_t stream) {
+  const uint32_t chunks = (cols + CHUNK - 1) / CHUNK;
+  const dim3 grid{uint32_t(rows * chunks)}, block{256};
+  plan::work(plan::UNIT_STREAM, 0, 4.0 * rows * cols);
+  MRL_LAUNCH(k_softmax_chunk_stats<V>, grid, block, 0, stream, in, stats, cols, chunks);
+  plan::work(plan::UNIT_STREAM, 0, double(rows) * cols * (4 + (OUT_BF16 ? 2 : 4)));
+  MRL_LAUNCH((k_softmax_chunk_write<V, OUT_BF16>), grid, block, 0, stream, in, out, stats, cols, chunks);
+  return mrl::plan::last_error();
+}
+
 }  // namespace
 
 namespace {
 template <bool OUT_BF16>
-hipError_t launch_rows(const float *in, void *out, uint64_t rows, uint32_t cols, hipStream_t stream) {
+hipError_t launch_rows(const float *in, void *out, uint64_t rows, uint32_t cols, void *scratch, hipStream_t stream) {
   if (rows == 0 || cols == 0) return hipSuccess;
+  if (cols > 16 * 256 && cols <= 16 * 1024 && cols % 4 == 0 && rows >= 256 && rows <= 0x7fffffffull) {
+    plan::work(plan::UNIT_STREAM, 0, double(rows) * cols * (4 + (OUT_BF16 ? 2 : 4)));
+    if (cols <= 8 * 1024) MRL_LAUNCH((k_softmax_block<8, OUT_BF16>), dim3(uint32_t(rows)), dim3(256), 0, stream, in, out, cols);
+    else MRL_LAUNCH((k_softmax_block<16, OUT_BF16>), dim3(uint32_t(rows)), dim3(256), 0, stream, in, out, cols);
+    return mrl::plan::last_error();
+  }
+  if (scratch && softmax_scratch_bytes(rows, cols)) {
+    if (cols % 4 == 0) return launch_chunks<4, OUT_BF16>(in, out, rows, cols, static_cast<float2 *>(scratch), stream);
+    return launch_chunks<1, OUT_BF16>(in, out, rows, cols, static_cast<float2 *>(scratch), stream);
+  }
   const uint64_t blocks64 = (rows + 3) / 4;
   if (blocks64 > 0x7fffffffull) return hipErrorInvalidValue;
   const dim3 grid{uint32_t(blocks64)}, block{256};
+  plan::work(plan::UNIT_STREAM, 0, double(rows) * cols * (4 + (OUT_BF16 ? 2 : 4)));
   if (cols % 4 == 0 && cols <= 16 * 256) {
     const uint32_t nv = (cols / 4 + 63) / 64;
-    if (nv <= 1) hipLaunchKernelGGL((k_softmax_regs<1, OUT_BF16>), grid, block, 0, stream, in, out, rows, cols);
-    else if (nv <= 2) hipLaunchKernelGGL((k_softmax_regs<2, OUT_BF16>), grid, block, 0, stream, in, out, rows, cols);
-    else if (nv <= 4) hipLaunchKernelGGL((k_softmax_regs<4, OUT_BF16>), grid, block, 0, stream, in, out, rows, cols);
-    else if (nv <= 8) hipLaunchKernelGGL((k_softmax_regs<8, OUT_BF16>), grid, block, 0, stream, in, out, rows, cols);
-    else hipLaunchKernelGGL((k_softmax_regs<16, OUT_BF16>), grid, block, 0, stream, in, out, rows, cols);
+    if (nv <= 1) MRL_LAUNCH((k_softmax_regs<1, OUT_BF16>), grid, block, 0, stream, in, out, rows, cols);
+    else if (nv <= 2) MRL_LAUNCH((k_softmax_regs<2, OUT_BF16>), grid, block, 0, stream, in, out, rows, cols);
+    else if (nv <= 4) MRL_LAUNCH((k_softmax_regs<4, OUT_BF16>), grid, block, 0, stream, in, out, rows, cols);
+    else if (nv <= 8) MRL_LAUNCH((k_softmax_regs<8, OUT_BF16>), grid, block, 0, stream, in, out, rows, cols);
+    else MRL_LAUNCH((k_softmax_regs<16, OUT_BF16>), grid, block, 0, stream, in, out, rows, cols);
   } else {
-    hipLaunchKernelGGL(k_softmax_stream<OUT_BF16>, grid, block, 0, stream, in, out, rows, cols);
+    MRL_LAUNCH(k_softmax_stream<OUT_BF16>, grid, block, 0, stream, in, out, rows, cols);
   }
-  return hipGetLastError();
+  return mrl::plan::last_error();
 }
 }  // namespace
 
-hipError_t launch_softmax_rows(const float *in, float *out, uint64_t rows, uint32_t cols,
-                               hipStream_t stream) {
-  return launch_rows<false>(in, out, rows, cols, stream);
+// Scratch the chunked kernels want for this shape (0: the shape runs without).
+size_t softmax_scratch_bytes(uint64_t rows, uint32_t cols) {
+  if (cols <= 16 * 256) return 0;
+  const uint64_t chunks = (cols + SOFTMAX_CHUNK - 1) / SOFTMAX_CHUNK;
+  if (rows * chunks > 0x7fffffffull) return 0;
+  return size_t(rows * chunks * sizeof(float2));
 }
 
-hipError_t launch_softmax_rows_bf16(const float *in, void *out, uint64_t rows, uint32_t cols,
+hipError_t launch_softmax_rows(const float *in, float *out, uint64_t rows, uint32_t cols, void *scratch,
+                               hipStream_t stream) {
+  return launch_rows<false>(in, out, rows, cols, scratch, stream);
+}
+
+hipError_t launch_softmax_rows_bf16(const float *in, void *out, uint64_t rows, uint32_t cols, void *scratch,
                                     hipStream_t stream) {
-  return launch_rows<true>(in, out, rows, cols, stream);
+  return launch_rows<true>(in, out, rows, cols, scratch, stream);
 }
 
 }  // namespace mrl

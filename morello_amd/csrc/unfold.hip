@@ -94,11 +94,12 @@ hipError_t launch_unfold(const void *image, void *rows, uint32_t batch, uint32_t
   p.units = uint64_t(batch) * oh * ow * p.row_units;
   if (p.units == 0) return hipSuccess;
   const uint32_t blocks = uint32_t(std::min<uint64_t>((p.units + 255) / 256, 1u << 20));
-  if (gather && elem_size == 1) hipLaunchKernelGGL(k_unfold_gather<uint8_t>, dim3(blocks), dim3(256), 0, stream, p);
-  else if (gather) hipLaunchKernelGGL(k_unfold_gather<uint16_t>, dim3(blocks), dim3(256), 0, stream, p);
-  else if (unit == 16) hipLaunchKernelGGL(k_unfold<uint4>, dim3(blocks), dim3(256), 0, stream, p, elem_size);
-  else hipLaunchKernelGGL(k_unfold<uint32_t>, dim3(blocks), dim3(256), 0, stream, p, elem_size);
-  return hipGetLastError();
+  plan::work(plan::UNIT_STREAM, 0, 2.0 * p.units * (gather ? 4 : unit));
+  if (gather && elem_size == 1) MRL_LAUNCH(k_unfold_gather<uint8_t>, dim3(blocks), dim3(256), 0, stream, p);
+  else if (gather) MRL_LAUNCH(k_unfold_gather<uint16_t>, dim3(blocks), dim3(256), 0, stream, p);
+  else if (unit == 16) MRL_LAUNCH(k_unfold<uint4>, dim3(blocks), dim3(256), 0, stream, p, elem_size);
+  else MRL_LAUNCH(k_unfold<uint32_t>, dim3(blocks), dim3(256), 0, stream, p, elem_size);
+  return mrl::plan::last_error();
 }
 
 }  // namespace mrl

@@ -1,6 +1,7 @@
 // Host-only exercise of include/morello_amd.hpp (no device needed): the same expectations
 // the Python tests assert, through the C++ view.  Built and run by tests/test_cpp_api.py.
 #include <cstdio>
+#include <string>
 
 #include "morello_amd.hpp"
 
@@ -63,6 +64,13 @@ int main() {
     EXPECT(false);
   } catch (const Error &e) {
     EXPECT(e.status() == MRL_ERR_BAD_SPEC);
+  }
+  // The plan of a Spec (host only): benchmark configuration 2 is one launch of the int8 256-tile.
+  {
+    const Plan p = Spec::matmul({1, 4096, 4096, 4096}, Dtype::Uint8, Dtype::Sint8, Dtype::Sint32).plan();
+    EXPECT(p.steps.size() == 1 && p.scratch_bytes == 0 && p.cost_ns > 20e3 && p.cost_ns < 500e3);
+    EXPECT(std::string(p.steps[0].kernel).find("k_gemm [T = I8, A_UNSIGNED = true, TL = Tile<256, 256, 128") == 0);
+    EXPECT(std::string(mrl_target_id()) == "Gfx950" && mrl_target_memories(nullptr, 0) == 4);
   }
   std::printf("cpp api ok\n");
   return 0;

@@ -35,6 +35,56 @@ def test_softmax_edge_values(gpu):
     assert np.isfinite(got).all() and (np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-12).all()
 
 
+@pytest.mark.parametrize("shape,dim", [((64, 100000), 1), ((3, 4097), 1), ((5, 20000), 1), ((2, 8192), 1),
+                                       ((1, 1 << 20), 1), ((300, 4100), 1), ((2, 3, 12290), 2), ((256, 8192), 1),
+                                       ((300, 16384), 1), ((260, 4100), 1), ((257, 12292), 1)])
+def test_softmax_long_rows(gpu, shape, dim):
+    """Rows beyond the register kernel's 4096 columns: a workgroup per 4096-element chunk, the
+    chunks' (max, denominator) pairs merged per row.  Column counts that are and are not
+    multiples of 4 (vector and scalar loads), whole and ragged last chunks, one row.  With 256
+    rows or more of up to 16384 columns a workgroup keeps its whole row in registers instead."""
+    x = synth.normal_f32(204, 0, shape, std=3.0)
+    got = run_spec(M.Softmax(list(shape), dim), [x, np.zeros(shape, np.float32)])
+    want = orc.softmax(list(shape), dim, x)
+    # The oracle sums a row's exponentials one after another in f32, as the reference's
+    # interpreter does (verification.rs:166-184); over 1e5 terms that sum is itself 1.3e-4 away
+    # from the exact value.  So: 1e-5 against the value computed in f64, and against the oracle
+    # 1e-5 plus the oracle's own distance from it.
+    x64 = x.astype(np.float64)
+    e = np.exp(x64 - x64.max(axis=dim, keepdims=True))
+    exact = e / e.sum(axis=dim, keepdims=True)
+    assert (np.abs(got - exact) <= 1e-5 * exact + 1e-12).all()
+    oracle_off = (np.abs(want - exact) / np.maximum(exact, 1e-30)).max()
+    assert (np.abs(got - want) <= (1e-5 + oracle_off) * np.abs(want) + 1e-12).all()
+    assert np.abs(got.sum(axis=dim, dtype=np.float64) - 1).max() < 1e-5
+
+
+def test_softmax_long_rows_edge_values(gpu):
+    """The chunked path's edges: the maximum in one chunk and everything else far below it, a
+    chunk of f32::MIN, a NaN (the whole row becomes NaN, other rows do not)."""
+    x = synth.normal_f32(205, 0, (4, 9000))
+    x[0, 8999] = 1e4
+    x[1, :4096] = np.finfo(np.float32).min
+    x[2, 5000] = np.nan
+    got = run_spec(M.Softmax([4, 9000], 1), [x, np.zeros_like(x)])
+    want = orc.softmax([3, 9000], 1, np.ascontiguousarray(x[[0, 1, 3]]))
+    assert got[0, 8999] == 1.0 and got[0].sum() == 1.0
+    assert (got[1, :4096] == 0).all()
+    assert np.isnan(got[2]).all()
+    assert (np.abs(got[[0, 1, 3]] - want) <= 1e-5 * np.abs(want) + 1e-12).all()
+
+
+@pytest.mark.parametrize("shape,dim", [((2048, 4096), 0), ((600, 70), 0), ((3, 1000, 130), 1), ((513, 64), 0),
+                                       ((7, 16), 0), ((2, 5000, 17), 1)])
+def test_softmax_over_an_outer_dim(gpu, shape, dim):
+    """The scan dim is not the contiguous one: 64 columns per workgroup, the scan dim split over
+    its 4 or 16 waves (short and long scan dims, ragged column tiles and scan lengths)."""
+    x = synth.normal_f32(206, 0, shape, std=3.0)
+    got = run_spec(M.Softmax(list(shape), dim), [x, np.zeros(shape, np.float32)])
+    want = orc.softmax(list(shape), dim, x)
+    assert (np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-12).all()
+
+
 def test_softmax_full_size(gpu):
     """The Softmax stage of benchmark configuration 5 alone: 16x2048 rows of 2048."""
     shape = (16, 2048, 2048)

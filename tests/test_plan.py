@@ -1,0 +1,186 @@
+"""The backend as a search target (morello/src/target/mod.rs:37-117): the target description, the
+plan of a Spec (which kernels a run launches: Kernel::applies_to_logical_spec) and the cost model
+over it (Kernel::main_cost / memory_allocated).  Planning is the run's own dispatch code with the
+launches recorded instead of made, so everything except the last two tests runs without a GPU."""
+import numpy as np
+import pytest
+
+import morello_amd as M
+from morello_amd import synth
+
+KT = M.layout(0, 2, 1)
+
+
+def c1(): return M.MatmulAccum([1, 64, 64, 64], (M.f32, M.f32, M.f32))
+def c2(): return M.MatmulAccum([1, 4096, 4096, 4096], (M.u8, M.i8, M.i32))
+def c3(): return M.MatmulAccum([1, 8192, 8192, 8192], (M.bf16, M.bf16, M.f32))
+def c4(): return M.Conv([32, 64, 64, 54, 54, 3, 3], (M.u8, M.i8, M.i32))
+def c5(): return M.ComposeMSM(16, 2048, 128, 2048, 128, layouts=[None, None, KT, None])
+
+
+def test_target_description():
+    """The answers an `impl Target` forwards: four memories fastest first (MEMORY_COUNT,
+    target/mod.rs:30-33), registers counted and not parallel-tiled, HBM the level a grid tiles
+    (Memory trait, target/mod.rs:80-95)."""
+    assert M.Target.target_id() == "Gfx950"
+    assert M.Target.line_size() == 128
+    assert M.Target.processors() == 256
+    mems = M.Target.memories()
+    assert [m.name for m in mems] == ["ACC", "VGPR", "LDS", "HBM"]
+    assert [m.counts_registers for m in mems] == [True, True, False, False]
+    assert [m.can_parallel_tile for m in mems] == [False, False, False, True]
+    assert mems[1].vector_bytes == [4, 8, 16] and mems[0].has_layout is False
+    assert mems[2].limit == 160 * 1024 and mems[3].limit == 288 << 30
+    assert [m.cache_hit_cost for m in mems] == sorted(m.cache_hit_cost for m in mems)
+    kernels = M.Target.kernels()
+    assert len(kernels) == len(set(kernels)) and {"k_gemm", "k_conv_i8", "k_attn", "k_softmax_regs"} <= set(kernels)
+
+
+def test_benchmark_configurations_pick_their_kernels():
+    p = c1().plan()
+    assert p.kernels == ["k_gemm"] and "T = F32" in p.steps[0].kernel and "Tile<64, 64, 128" in p.steps[0].kernel
+    p = c2().plan()
+    assert p.kernels == ["k_gemm"] and p.scratch_bytes == 0
+    assert "T = I8, A_UNSIGNED = true, TL = Tile<256, 256, 128, 2, 4>, EDGE = false" in p.steps[0].kernel
+    assert p.steps[0].grid == (256, 1, 1) and p.steps[0].block == (512, 1, 1) and p.steps[0].unit == "mfma_i8"
+    assert p.steps[0].ops == 2 * 4096 ** 3 and p.steps[0].bytes == 2 * 4096 ** 2 + 2 * 4 * 4096 ** 2  # accumulating: C read too
+    p = c3().plan()
+    assert p.kernels == ["k_gemm"] and "T = BF16" in p.steps[0].kernel and p.steps[0].grid == (1024, 1, 1)
+    p = c4().plan()
+    assert p.kernels == ["k_conv_i8"] and "SLABS = 9" in p.steps[0].kernel and p.steps[0].ops == 6879707136
+    p = c5().plan()
+    assert p.kernels == ["k_attn"] and "D = 128, RAGGED = false, KT_ROWS = false" in p.steps[0].kernel
+    assert p.steps[0].grid == (256, 1, 1) and p.steps[0].lds_bytes > 64 * 1024
+    p = M.Softmax([16, 2048, 2048], 2).plan()
+    assert p.kernels == ["k_softmax_regs"] and p.steps[0].bytes == 2 * 4 * 16 * 2048 * 2048
+
+
+def test_plans_follow_shape_dtype_and_layout():
+    # The reference's default layouts: KT row-major, read in place by its own build of the kernel.
+    assert "KT_ROWS = true" in M.ComposeMSM(16, 2048, 128, 2048, 128).plan().steps[0].kernel
+    # Few queries, many keys: the keys are shared out, at most one workgroup per compute unit.
+    p = M.ComposeMSM(16, 1, 128, 32768, 128, layouts=[None, None, KT, None]).plan()
+    assert p.kernels == ["k_attn", "k_attn_merge"]
+    gx, gy, _ = p.steps[0].grid
+    assert gx == 16 and gy > 1 and gx * gy <= 256 and p.scratch_bytes >= 16 * gy * (128 + 4) * 4
+    # Head dim 256: staged, P in bf16.
+    p = M.ComposeMSM(16, 2048, 256, 2048, 256, layouts=[None, None, KT, None]).plan()
+    assert p.kernels == ["k_gemm", "k_softmax_regs", "k_gemm"] and "OUT_BF16 = true" in p.steps[1].kernel
+    assert "B_KMAJOR = true" in p.steps[0].kernel
+    # Ragged sizes: zero-padded copies of A and B, then the edge build of a small tile.
+    p = M.Matmul([1, 1000, 1000, 1000], (M.u8, M.i8, M.i32)).plan()
+    assert p.kernels == ["k_pad_rows", "k_pad_rows", "k_gemm"] and "EDGE = true" in p.steps[2].kernel
+    # Matrix-vector with a k-fastest B: dot products, not the matrix cores.
+    p = M.Matmul([1, 1, 2048, 16384], (M.bf16, M.bf16, M.f32), layouts=[None, KT, None]).plan()
+    assert p.kernels == ["k_gemv"] and p.steps[0].unit == "hbm"
+    # A dtype triple without an MFMA form, and a problem too small to pay for one.
+    assert M.Matmul([1, 256, 256, 256], (M.i16, M.i16, M.i32)).plan().kernels == ["k_matmul_generic"]
+    assert M.Matmul([1, 8, 8, 8], (M.f32, M.f32, M.f32)).plan().kernels == ["k_matmul_generic"]
+    # Conv shapes beside the benchmark's: implicit Matmul; three channels: unfolded first.
+    assert M.Conv([32, 128, 128, 26, 26, 3, 3], (M.bf16, M.bf16, M.f32)).plan().kernels == ["k_gemm"]
+    assert "CONV = true" in M.Conv([32, 128, 128, 26, 26, 3, 3], (M.bf16, M.bf16, M.f32)).plan().steps[0].kernel
+    assert "k_unfold_gather" in M.Conv([8, 32, 3, 110, 110, 5, 5], (M.u8, M.i8, M.i32)).plan().kernels
+    # Softmax by row length and by which dim is scanned.
+    assert M.Softmax([64, 100000], 1).plan().kernels == ["k_softmax_chunk_stats", "k_softmax_chunk_write"]
+    assert M.Softmax([8192, 8192], 1).plan().kernels == ["k_softmax_block"]
+    assert M.Softmax([2048, 4096], 0).plan().kernels == ["k_softmax_cols"]
+    # Moves: transpose tiled through LDS, Packed destination gathered, plain copy.
+    sq = [4096, 4096]
+    assert M.Move(sq, (M.f32, M.f32), layouts=[M.row_major(sq), M.col_major(sq)]).plan().kernels == ["k_move_tiled"]
+    assert M.Move(sq, (M.f32, M.f32)).plan().kernels == ["k_copy16"]
+    assert M.Move(sq, (M.bf16, M.f32)).plan().kernels == ["k_convert4"]
+
+
+def test_scratch_of_a_plan_covers_the_staging_bytes():
+    packed = M.layout(0, 2, 1, (2, M.Packed(16)))
+    s = M.Matmul([1, 64, 64, 64], [M.f32] * 3, layouts=[None, packed, None])
+    p = s.plan()
+    assert s.workspace_bytes() == 64 * 64 * 4 and p.scratch_bytes >= s.workspace_bytes()
+    assert p.kernels[0].startswith("k_move") and p.kernels[-1] in ("k_gemm", "k_matmul_generic")
+    for spec in (c1(), c2(), c4(), c5()):
+        assert spec.plan().scratch_bytes == 0 == spec.workspace_bytes()
+
+
+def test_every_planned_kernel_is_a_kernel_of_the_target():
+    families = set(M.Target.kernels())
+    specs = [c1(), c2(), c3(), c4(), c5(), M.Softmax([3, 7, 1001], 2), M.Softmax([5, 9, 64], 1),
+             M.Matmul([2, 100, 70, 50], (M.i8, M.i8, M.i32)), M.Matmul([1, 300, 300, 300], (M.bf16, M.f32, M.f32)),
+             M.Conv([2, 8, 8, 30, 30, 3, 3], (M.i16, M.i16, M.i32)), M.Conv([1, 4, 4, 3, 3, 2, 2], (M.f32, M.f32, M.f32)),
+             M.Move([64, 48], (M.u8, M.u8), layouts=[M.row_major([64, 48]), M.layout(0, 1, (1, M.OddEven(16)))]),
+             M.Fill([100, 100], M.f32, M.FillValue.NegInf), M.Max([64, 64], 1), M.Broadcast([4, 8], 1),
+             M.SoftmaxDenominatorAndMax([16, 256], 1), M.DivideVecScalar([16, 256], 1), M.OnePrefix([4, 8])]
+    for spec in specs:
+        plan = spec.plan()
+        assert plan.steps and set(plan.kernels) <= families, (spec, plan)
+        assert plan.cost_ns >= 2000 * len(plan.steps) and abs(plan.cost_ns - sum(s.cost_ns for s in plan.steps)) < 1e-3
+
+
+def test_cost_orders_what_search_has_to_order():
+    """The model is only asked to rank alternatives (cost.rs:13-17 compares `main` first)."""
+    mm = lambda n, dts: M.Matmul([1, n, n, n], dts).plan().cost_ns
+    i8, bf, f32 = (M.u8, M.i8, M.i32), (M.bf16, M.bf16, M.f32), (M.f32, M.f32, M.f32)
+    for dts in (i8, bf, f32):
+        costs = [mm(n, dts) for n in (256, 1024, 2048, 4096, 8192)]
+        assert costs == sorted(costs) and costs[-1] > 6 * costs[-2] > 30 * costs[-3]
+    assert mm(4096, i8) < mm(4096, bf) < mm(4096, f32)
+    # Fused attention beats the same Compose with its intermediates materialised (bufferize).
+    staged = M.Compose([M.Matmul([16, 2048, 2048, 128], [M.f32, M.bf16, M.f32]), M.Softmax([16, 2048, 2048], 2),
+                        M.Matmul([16, 2048, 128, 2048], [M.bf16, M.bf16, M.f32])], layouts=[None, None, KT, None])
+    fused, unfused = staged.plan(), staged.bufferize(0).plan()
+    assert fused.kernels == ["k_attn"] and len(unfused.steps) >= 3
+    assert fused.cost_ns * 4 < unfused.cost_ns and unfused.scratch_bytes >= 16 * 2048 * 2048 * 4
+    # A column-major A costs its transposing copy on top.
+    a_t = M.Matmul([1, 4096, 4096, 4096], bf, layouts=[M.batched_col_major([1, 4096, 4096]), None, None]).plan()
+    assert a_t.kernels[-1] == "k_gemm" and len(a_t.steps) == 2 and a_t.cost_ns > mm(4096, bf)
+
+
+def test_plan_errors_are_the_run_errors():
+    import ctypes as C
+    from morello_amd import _binding as B
+    bad = M.Matmul([1, 65536, 65536, 2], [M.u8, M.i8, M.i32])
+    head = B.PlanC()
+    assert B.load().mrl_spec_plan(C.byref(bad._c), C.byref(head), None, 0) == bad.check() != 0
+    ok = c2()
+    assert B.load().mrl_spec_plan(C.byref(ok._c), None, None, 0) != 0       # null plan
+    assert B.load().mrl_spec_plan(C.byref(ok._c), C.byref(head), None, 0) == 0 and head.n_steps == 1  # count only
+
+
+@pytest.mark.gpu
+def test_planning_leaves_runs_alone(gpu):
+    """A plan between two runs changes nothing: the recorder is per call and per thread."""
+    from gpu_util import run_spec
+    spec = M.Matmul([1, 96, 200, 72], (M.u8, M.i8, M.i32))
+    a, b = synth.uniform_u8(501, 0, (1, 96, 200)), synth.uniform_i8(501, 1, (1, 200, 72))
+    first = run_spec(spec, [a, b, np.zeros((1, 96, 72), np.int32)])
+    assert spec.plan().steps
+    second = run_spec(spec, [a, b, np.zeros((1, 96, 72), np.int32)])
+    want = a.astype(np.int32)[0] @ b.astype(np.int32)[0]
+    assert np.array_equal(first[0], want) and np.array_equal(second[0], want)
+
+
+@pytest.mark.gpu
+def test_cost_model_against_measured_launches(gpu):
+    """Predicted / measured per-launch time stays within [0.4, 2.5] on benchmark-like operands for
+    the kernels the benchmark configurations and their neighbours run (the fit's own spread is
+    0.6-1.5; the bound leaves room for the board's clock state)."""
+    rng = np.random.default_rng(7)
+    specs = [c2(), c4(), c5(), M.Matmul([1, 2048, 2048, 2048], (M.bf16, M.bf16, M.f32)),
+             M.Matmul([1, 1024, 1024, 1024], (M.f32, M.f32, M.f32)), M.Softmax([16, 2048, 2048], 2),
+             M.Softmax([64, 100000], 1), M.ComposeMSM(16, 1, 128, 32768, 128, layouts=[None, None, KT, None]),
+             M.Matmul([1, 1, 2048, 16384], (M.bf16, M.bf16, M.f32), layouts=[None, KT, None]),
+             M.Move([4096, 4096], (M.f32, M.f32), layouts=[M.row_major([4096, 4096]), M.col_major([4096, 4096])])]
+    for spec in specs:
+        bufs = []
+        for i, dt in enumerate(spec.dtypes):
+            n = spec.bytes_used(i)
+            if dt == M.f32: arr = rng.standard_normal(n // 4, dtype=np.float32)
+            elif dt == M.bf16: arr = (rng.standard_normal(n // 2, dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16)
+            else: arr = rng.integers(0, 256, n, dtype=np.uint8)
+            bufs.append(M.DeviceBuffer.from_numpy(arr))
+        ptrs = [b.ptr for b in bufs]
+        spec.run_timed(ptrs, 3)
+        measured_ns = min(spec.run_timed(ptrs, 20) for _ in range(3)) / 20 * 1e6
+        predicted_ns = spec.plan().cost_ns
+        for b in bufs:
+            b.free()
+        assert 0.4 < predicted_ns / measured_ns < 2.5, (spec, predicted_ns, measured_ns)
