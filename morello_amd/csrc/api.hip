@@ -1269,7 +1269,7 @@ uint32_t mrl_target_kernels(const char **names, uint32_t cap) {
       "k_gemm", "k_gemv", "k_matmul_generic", "k_conv_i8", "k_conv_generic", "k_conv_generic_wave", "k_unfold",
       "k_unfold_gather", "k_attn", "k_attn_merge", "k_softmax_regs", "k_softmax_stream", "k_softmax_cols",
       "k_softmax_generic", "k_parts", "k_broadcast", "k_fill", "k_fill_zero", "k_move_rows", "k_move_rows16",
-      "k_move_tiled", "k_move_tiled16", "k_move_gather", "k_move_generic", "k_relayout", "k_convert4", "k_copy1",
+      "k_move_tiled", "k_move_tiled16", "k_move_tiled16v", "k_move_tiled32", "k_move_gather", "k_move_generic", "k_relayout", "k_convert4", "k_copy1",
       "k_copy16", "k_pad_rows", "k_widen_bf16"};
   const uint32_t n = sizeof families / sizeof families[0];
   for (uint32_t i = 0; i < n && i < cap && names; i++) names[i] = families[i];

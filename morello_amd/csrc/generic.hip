@@ -242,7 +242,10 @@ __global__ __launch_bounds__(256) void k_move_tiled(MoveStrided p) {
   uint64_t blk = blockIdx.x;
   const uint32_t ts = uint32_t(blk % p.tiles_s);
   blk /= p.tiles_s;
-  const uint32_t td = uint32_t(blk % p.tiles_d);
+  // Diagonal order: workgroups that run together differ in both tile coordinates.  In row or
+  // column order they would all read (or all write) addresses a whole number of rows apart,
+  // which with power-of-two row lengths is one memory channel for all of them.
+  const uint32_t td = uint32_t((blk + ts) % p.tiles_d);
   blk /= p.tiles_d;
   // The remaining dims, slowest to fastest in `order` (dim_s and dim_d are skipped).
   int64_t so = 0, d_o = 0;
@@ -274,7 +277,7 @@ __global__ __launch_bounds__(256) void k_move_tiled16(MoveStrided p) {
   uint64_t blk = blockIdx.x;
   const uint32_t ts = uint32_t(blk % p.tiles_s);
   blk /= p.tiles_s;
-  const uint32_t td = uint32_t(blk % p.tiles_d);
+  const uint32_t td = uint32_t((blk + ts) % p.tiles_d);  // diagonal order, see k_move_tiled
   blk /= p.tiles_d;
   int64_t so = 0, d_o = 0;
   for (int o = int(p.rank) - 1; o >= 0; o--) {
@@ -301,6 +304,105 @@ __global__ __launch_bounds__(256) void k_move_tiled16(MoveStrided p) {
       const uint32_t pair = uint32_t(tile[2 * lane][r]) | (uint32_t(tile[2 * lane + 1][r]) << 16);
       *(uint32_t *)(dst + d_o + int64_t(s0 + r) * p.ds[p.dim_s] + (d0 + 2 * lane)) = pair;
     }
+}
+
+// 16-bit elements whose source rows are whole 16-byte vectors: the 128 x 128 tile sits in LDS as
+// dwords (pairs along the source's contiguous dim), loaded eight elements per lane; a lane then
+// takes the dwords of two neighbouring tile rows and regroups their halves into the two dwords
+// it stores (pairs along the destination's contiguous dim).  No 16-bit LDS access, no bank
+// conflict beyond the two passes 64 lanes need anyway.
+__global__ __launch_bounds__(256) void k_move_tiled16v(MoveStrided p) {
+  __shared__ uint32_t tile[128][65];
+  uint64_t blk = blockIdx.x;
+  const uint32_t ts = uint32_t(blk % p.tiles_s);
+  blk /= p.tiles_s;
+  const uint32_t td = uint32_t((blk + ts) % p.tiles_d);  // diagonal order, see k_move_tiled
+  blk /= p.tiles_d;
+  int64_t so = 0, d_o = 0;
+  for (int o = int(p.rank) - 1; o >= 0; o--) {
+    const uint32_t d = p.order[o];
+    if (d == p.dim_s || d == p.dim_d) continue;
+    const uint32_t c = uint32_t(blk % p.shape[d]);
+    blk /= p.shape[d];
+    so += int64_t(c) * p.ss[d], d_o += int64_t(c) * p.ds[d];
+  }
+  typedef uint32_t quad_t __attribute__((ext_vector_type(4)));
+  const uint32_t s0 = ts * 128, d0 = td * 128, ns = p.shape[p.dim_s], nd = p.shape[p.dim_d];
+  const uint16_t *src = static_cast<const uint16_t *>(p.src);
+  uint16_t *dst = static_cast<uint16_t *>(p.dst);
+  const uint32_t col = (threadIdx.x & 15) * 8, row = threadIdx.x >> 4;
+  quad_t v[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const uint32_t r = row + 16 * i;
+    v[i] = quad_t{0, 0, 0, 0};
+    if (d0 + r < nd && s0 + col < ns)
+      v[i] = __builtin_nontemporal_load((const quad_t *)(src + so + int64_t(d0 + r) * p.ss[p.dim_d] + (s0 + col)));
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const uint32_t r = row + 16 * i;
+#pragma unroll
+    for (int j = 0; j < 4; j++) tile[r][col / 2 + j] = v[i][j];
+  }
+  __syncthreads();
+  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t d = d0 + 2 * lane;
+  if (d >= nd) return;
+#pragma unroll 4
+  for (uint32_t sp = wave; sp < 64; sp += 4) {
+    const uint32_t a = tile[2 * lane][sp], b = tile[2 * lane + 1][sp];
+    const uint32_t sidx = s0 + 2 * sp;
+    if (sidx < ns) *(uint32_t *)(dst + d_o + int64_t(sidx) * p.ds[p.dim_s] + d) = (a & 0xffffu) | (b << 16);
+    if (sidx + 1 < ns) *(uint32_t *)(dst + d_o + int64_t(sidx + 1) * p.ds[p.dim_s] + d) = (a >> 16) | (b & 0xffff0000u);
+  }
+}
+
+// The same for 32-bit elements that are not converted: 64 x 64 tiles, four elements (16 bytes)
+// per lane on both sides.  Needs extents along both contiguous dims and all other strides in
+// multiples of 4 elements and 16-byte aligned bases, so that every vector is whole and aligned.
+__global__ __launch_bounds__(256) void k_move_tiled32(MoveStrided p) {
+  __shared__ uint32_t tile[64][65];
+  uint64_t blk = blockIdx.x;
+  const uint32_t ts = uint32_t(blk % p.tiles_s);
+  blk /= p.tiles_s;
+  const uint32_t td = uint32_t((blk + ts) % p.tiles_d);  // diagonal order, see k_move_tiled
+  blk /= p.tiles_d;
+  int64_t so = 0, d_o = 0;
+  for (int o = int(p.rank) - 1; o >= 0; o--) {
+    const uint32_t d = p.order[o];
+    if (d == p.dim_s || d == p.dim_d) continue;
+    const uint32_t c = uint32_t(blk % p.shape[d]);
+    blk /= p.shape[d];
+    so += int64_t(c) * p.ss[d], d_o += int64_t(c) * p.ds[d];
+  }
+  const uint32_t col = (threadIdx.x & 15) * 4, row = threadIdx.x >> 4;  // 16 lanes per 64-element row
+  const uint32_t s0 = ts * 64, d0 = td * 64, ns = p.shape[p.dim_s], nd = p.shape[p.dim_d];
+  const uint32_t *src = static_cast<const uint32_t *>(p.src);
+  uint32_t *dst = static_cast<uint32_t *>(p.dst);
+  typedef uint32_t quad_t __attribute__((ext_vector_type(4)));
+  quad_t v[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const uint32_t r = row + 16 * i;
+    v[i] = quad_t{0, 0, 0, 0};
+    if (d0 + r < nd && s0 + col < ns)
+      v[i] = __builtin_nontemporal_load((const quad_t *)(src + so + int64_t(d0 + r) * p.ss[p.dim_d] + (s0 + col)));
+  }
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const uint32_t r = row + 16 * i;
+    tile[r][col] = v[i][0], tile[r][col + 1] = v[i][1], tile[r][col + 2] = v[i][2], tile[r][col + 3] = v[i][3];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const uint32_t r = row + 16 * i;
+    if (s0 + r < ns && d0 + col < nd) {
+      const quad_t out{tile[col][r], tile[col + 1][r], tile[col + 2][r], tile[col + 3][r]};
+      __builtin_nontemporal_store(out, (quad_t *)(dst + d_o + int64_t(s0 + r) * p.ds[p.dim_s] + (d0 + col)));
+    }
+  }
 }
 
 // Any other pair of contiguous dims (a Packed(8) digit on one side, say, too short for the
@@ -887,13 +989,24 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
                  (reinterpret_cast<uintptr_t>(dst) & 3) == 0;
     for (uint32_t d = 0; pairs && d < p.rank; d++)
       pairs = (int(d) == dim_s || p.ss[d] % 2 == 0) && (int(d) == dim_d || p.ds[d] % 2 == 0);
+    // ... and the source side in whole 16-byte vectors.
+    bool octets = pairs && p.shape[dim_s] % 8 == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0;
+    for (uint32_t d = 0; octets && d < p.rank; d++) octets = int(d) == dim_s || p.ss[d] % 8 == 0;
+    // 32-bit elements likewise, four per lane.
+    bool quads = src_dtype == dst_dtype && mrl_dtype_size(src_dtype) == 4 && p.shape[dim_s] % 4 == 0 &&
+                 p.shape[dim_d] % 4 == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0 &&
+                 (reinterpret_cast<uintptr_t>(dst) & 15) == 0;
+    for (uint32_t d = 0; quads && d < p.rank; d++)
+      quads = (int(d) == dim_s || p.ss[d] % 4 == 0) && (int(d) == dim_d || p.ds[d] % 4 == 0);
     const uint32_t side = pairs ? 128 : 64;
     p.tiles_s = (p.shape[dim_s] + side - 1) / side, p.tiles_d = (p.shape[dim_d] + side - 1) / side;
     uint64_t blocks = uint64_t(p.tiles_s) * p.tiles_d;
     for (uint32_t d = 0; d < p.rank; d++)
       if (int(d) != dim_s && int(d) != dim_d) blocks *= p.shape[d];
     if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
-    if (pairs) MRL_LAUNCH(k_move_tiled16, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+    if (octets) MRL_LAUNCH(k_move_tiled16v, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+    else if (pairs) MRL_LAUNCH(k_move_tiled16, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+    else if (quads) MRL_LAUNCH(k_move_tiled32, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
     else MRL_LAUNCH(k_move_tiled, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
     return mrl::plan::last_error();
   }

@@ -117,13 +117,29 @@ def test_host_threads_share_a_stream_and_its_scratch(gpu):
 
 
 @pytest.mark.parametrize("dt", [M.bf16, M.i16, M.u16])
-@pytest.mark.parametrize("shape", [(2, 200, 136), (1, 130, 258), (3, 64, 64), (1, 1000, 2), (2, 33, 64), (1, 2048, 128)])
+@pytest.mark.parametrize("shape", [(2, 200, 136), (1, 130, 258), (3, 64, 64), (1, 1000, 2), (2, 33, 64), (1, 2048, 128),
+                                   (1, 264, 520), (2, 136, 72), (1, 1030, 8)])
 def test_transpose_of_16_bit_elements(gpu, dt, shape):
-    """Row-major <-> batched column-major of 16-bit elements: two elements per lane on both sides
-    where the extents are even, one where they are not."""
+    """Row-major <-> batched column-major of 16-bit elements: eight elements per lane on the
+    source side where its rows are whole 16-byte vectors, two per lane on both sides where the
+    extents are even, one where they are not; whole and ragged 128 x 128 tiles."""
     x = synth.raw_u64(830, 0, int(np.prod(shape))).astype(np.uint16).reshape(shape)
     cm = M.batched_col_major(list(shape))
     got = run_spec(M.Move(list(shape), (dt, dt), layouts=[None, cm]), [x, np.zeros((shape[0], shape[2], shape[1]), np.uint16)])
     assert np.array_equal(got, x.transpose(0, 2, 1))
     back = run_spec(M.Move(list(shape), (dt, dt), layouts=[cm, None]), [got, np.zeros(shape, np.uint16)])
     assert np.array_equal(back, x)
+
+
+@pytest.mark.parametrize("dt,npd", [(M.f32, np.float32), (M.i32, np.int32), (M.u32, np.uint32)])
+@pytest.mark.parametrize("shape", [(2, 200, 136), (1, 132, 260), (3, 64, 64), (1, 1000, 4), (2, 33, 64), (1, 2048, 128),
+                                   (1, 130, 258)])
+def test_transpose_of_32_bit_elements(gpu, dt, npd, shape):
+    """The same for 32-bit elements: four per lane on both sides where both extents are multiples
+    of 4, one per lane otherwise; tiles in diagonal order."""
+    x = synth.raw_u64(831, 0, int(np.prod(shape))).astype(np.uint32).view(npd).reshape(shape)
+    cm = M.batched_col_major(list(shape))
+    got = run_spec(M.Move(list(shape), (dt, dt), layouts=[None, cm]), [x, np.zeros((shape[0], shape[2], shape[1]), npd)])
+    assert np.array_equal(got.view(np.uint32), x.transpose(0, 2, 1).view(np.uint32))
+    back = run_spec(M.Move(list(shape), (dt, dt), layouts=[cm, None]), [got, np.zeros(shape, npd)])
+    assert np.array_equal(back.view(np.uint32), x.view(np.uint32))
