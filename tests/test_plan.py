@@ -86,7 +86,12 @@ def test_plans_follow_shape_dtype_and_layout():
     assert M.Softmax([2048, 4096], 0).plan().kernels == ["k_softmax_cols"]
     # Moves: transpose tiled through LDS, Packed destination gathered, plain copy.
     sq = [4096, 4096]
-    assert M.Move(sq, (M.f32, M.f32), layouts=[M.row_major(sq), M.col_major(sq)]).plan().kernels == ["k_move_tiled"]
+    transposed = [M.row_major(sq), M.col_major(sq)]
+    assert M.Move(sq, (M.f32, M.f32), layouts=transposed).plan().kernels == ["k_move_tiled32"]
+    assert M.Move(sq, (M.bf16, M.bf16), layouts=transposed).plan().kernels == ["k_move_tiled16v"]
+    assert M.Move(sq, (M.u8, M.u8), layouts=transposed).plan().kernels == ["k_move_tiled"]
+    odd = [4098, 4098]
+    assert M.Move(odd, (M.bf16, M.bf16), layouts=[M.row_major(odd), M.col_major(odd)]).plan().kernels == ["k_move_tiled16"]
     assert M.Move(sq, (M.f32, M.f32)).plan().kernels == ["k_copy16"]
     assert M.Move(sq, (M.bf16, M.f32)).plan().kernels == ["k_convert4"]
 
