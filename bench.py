@@ -290,6 +290,10 @@ def main():
         "config": {"workload": desc, "spec": args.spec, "device": M.device_info()["name"]},
         "roofline": roofline,
     }
+    # Which kernels the timed launches were, and what the library's cost model expected of them.
+    plan = spec.plan()
+    out["plan"] = {"kernels": [s.kernel for s in plan.steps], "predicted_ms": plan.cost_ns * 1e-6,
+                   "scratch_bytes": plan.scratch_bytes}
     if not args.no_cpu and args.spec in ("c2", "c3", "c4", "c5"):
         out["cpu_baseline"] = cpu_baseline(args.spec, arrs)
     if args.vendor_ref:
