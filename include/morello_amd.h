@@ -199,10 +199,13 @@ size_t mrl_spec_workspace_bytes(const mrl_spec *spec);
 int mrl_run(const mrl_spec *spec, void *const *params);
 
 /* As mrl_run but only enqueues on `stream` (a hipStream_t, NULL = default stream).  Scratch
- * memory of up to 64 MiB per call (relayout staging, padded operands) comes from an arena the
- * library keeps per stream it has seen; calls from several host threads onto one stream take
- * turns for it.  mrl_stream_destroy releases the arena of its stream; the arena of a stream
- * the caller created itself stays until the process ends. */
+ * memory (relayout staging, padded operands, a Compose's intermediates) comes from an arena
+ * the library keeps per stream it has seen: 64 MiB at first; a call that needs more takes the
+ * excess from the stream-ordered allocator and, before it returns, waits for the stream once and
+ * replaces the arena by one that holds the whole call (up to 16 GiB), so that its next run
+ * allocates nothing.  mrl_spec_plan tells the amount (scratch_bytes).  Calls from several host
+ * threads onto one stream take turns for the arena.  mrl_stream_destroy releases the arena of
+ * its stream; the arena of a stream the caller created itself stays until the process ends. */
 int mrl_run_async(const mrl_spec *spec, void *const *params, void *stream);
 
 /* Literal stand-in for calling the emitted kernel from the emitted main

@@ -225,16 +225,18 @@ struct Prepared {
   uint32_t elem = 0;
 };
 
-// Scratch memory of one call.  Small requests are carved out of an arena that stays allocated
-// per stream (work on a stream runs in order, so the next call may overwrite what this one
-// staged): hipMallocAsync / hipFreeAsync cost several microseconds of host time apiece, more
-// than the kernels of a small Spec.  A call holds its stream's arena until it returns, so host
-// threads that share a stream take turns.  Requests that do not fit come from the stream-ordered
-// allocator.
-constexpr size_t ARENA_BYTES = size_t(64) << 20;
+// Scratch memory of one call.  Requests are carved out of an arena that stays allocated per
+// stream (work on a stream runs in order, so the next call may overwrite what this one staged):
+// hipMallocAsync / hipFreeAsync cost several microseconds of host time apiece for small blocks
+// and hundreds for blocks of 100 MB, more than the kernels of most Specs.  A call holds its
+// stream's arena until it returns, so host threads that share a stream take turns.  The arena
+// starts at 64 MiB; a call that asks for more gets the excess from the stream-ordered allocator
+// and leaves behind an arena large enough for its next run (up to ARENA_MAX_BYTES).
+constexpr size_t ARENA_BYTES = size_t(64) << 20, ARENA_MAX_BYTES = size_t(16) << 30;
 struct Arena {
   std::mutex in_use;
   void *base = nullptr;
+  size_t size = 0;
 };
 std::mutex g_arenas_mutex;
 std::map<hipStream_t, std::unique_ptr<Arena>> g_arenas;
@@ -265,42 +267,51 @@ struct Workspace {
   std::vector<void *> allocs;
   Arena *arena = nullptr;  // locked while non-null
   size_t arena_used = 0;
+  size_t requested = 0;    // everything this call asked for
   explicit Workspace(hipStream_t s) : stream(s) {}
   Workspace(const Workspace &) = delete;
   Workspace &operator=(const Workspace &) = delete;
   hipError_t alloc(void **p, size_t bytes) {
-    const size_t rounded = (bytes + 255) & ~size_t(255);
+    const size_t rounded = std::max<size_t>(256, (bytes + 255) & ~size_t(255));
     if (mrl::plan::recording()) {
       // Planning: a stand-in address, aligned as the allocator's are, never dereferenced.
       mrl::plan::Recorder *r = mrl::plan::g_recorder;
       *p = reinterpret_cast<void *>((uintptr_t(1) << 44) + r->scratch_bytes);
-      r->scratch_bytes += rounded ? rounded : 256;
+      r->scratch_bytes += rounded;
       return hipSuccess;
     }
-    if (rounded <= ARENA_BYTES - arena_used) {
-      if (!arena) {
-        arena = arena_of(stream);
-        arena->in_use.lock();
-        if (!arena->base) {
-          hipError_t e = hipMalloc(&arena->base, ARENA_BYTES);
-          if (e != hipSuccess) {
-            arena->in_use.unlock();
-            arena = nullptr;
-            return e;
-          }
-        }
-      }
+    if (!arena) {
+      arena = arena_of(stream);
+      arena->in_use.lock();
+    }
+    requested += rounded;
+    if (!arena->base && rounded <= ARENA_BYTES && hipMalloc(&arena->base, ARENA_BYTES) == hipSuccess)
+      arena->size = ARENA_BYTES;
+    if (arena->base && rounded <= arena->size - arena_used) {
       *p = static_cast<uint8_t *>(arena->base) + arena_used;
-      arena_used += rounded ? rounded : 256;
+      arena_used += rounded;
       return hipSuccess;
     }
-    hipError_t e = hipMallocAsync(p, bytes ? bytes : 4, stream);
+    hipError_t e = hipMallocAsync(p, rounded, stream);
     if (e == hipSuccess) allocs.push_back(*p);
     return e;
   }
   ~Workspace() {
     for (void *p : allocs) (void)hipFreeAsync(p, stream);
-    if (arena) arena->in_use.unlock();
+    if (!arena) return;
+    if (requested > arena->size && requested <= ARENA_MAX_BYTES) {
+      // Once per size: wait for the work that uses the old arena, free it, allocate one that
+      // holds this call.
+      size_t grown = ARENA_BYTES;
+      while (grown < requested) grown *= 2;
+      if (hipStreamSynchronize(stream) == hipSuccess) {
+        if (arena->base) (void)hipFree(arena->base);
+        arena->base = nullptr, arena->size = 0;
+        if (hipMalloc(&arena->base, grown) == hipSuccess) arena->size = grown;
+        else arena->base = nullptr;
+      }
+    }
+    arena->in_use.unlock();
   }
 };
 
@@ -425,7 +436,13 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
   // that are not whole 16-byte chunks (K or N not a multiple of 16 bytes) are padded with zeros
   // to the next chunk.  Two extra passes over an operand against a generic kernel that is tens
   // of times slower.
-  const bool worth_two_more_passes = double(g.m) * g.n * g.k * g.batch >= 256.0 * 256 * 256;
+  // The generic kernel's threads each walk K on their own: measured ~2.5 us + 40 ns per step of
+  // K + 2 ops per 3e6 per us; a copy pass costs ~3 us at these sizes, the matrix-core kernel
+  // ~3.5 us + 0.45 us per 128 bytes of K.
+  const double macs = double(g.m) * g.n * g.k * g.batch;
+  const double generic_us = 2.5 + 0.04 * g.k + 2.0 * macs / 3e6;
+  const double copies_us = 6.0 + 3.5 + 0.45 * double((uint64_t(g.k) * a.elem + 127) / 128);
+  const bool worth_two_more_passes = macs >= 256.0 * 256 * 256 || generic_us > copies_us;
   if (!sched && kind >= 0 && worth_two_more_passes) {
     const int64_t per16 = 16 / int64_t(a.elem);
     auto walkable = [&](const mrl::Strided &t) {
@@ -1267,10 +1284,11 @@ uint32_t mrl_target_memories(mrl_target_memory *out, uint32_t cap) {
 uint32_t mrl_target_kernels(const char **names, uint32_t cap) {
   static const char *const families[] = {
       "k_gemm", "k_gemv", "k_matmul_generic", "k_conv_i8", "k_conv_generic", "k_conv_generic_wave", "k_unfold",
-      "k_unfold_gather", "k_attn", "k_attn_merge", "k_softmax_regs", "k_softmax_stream", "k_softmax_cols",
+      "k_unfold_gather", "k_attn", "k_attn_merge", "k_softmax_regs", "k_softmax_block", "k_softmax_chunk_stats", "k_softmax_chunk_write", "k_softmax_stream",
+      "k_softmax_cols",
       "k_softmax_generic", "k_parts", "k_broadcast", "k_fill", "k_fill_zero", "k_move_rows", "k_move_rows16",
-      "k_move_tiled", "k_move_tiled16", "k_move_tiled16v", "k_move_tiled32", "k_move_gather", "k_move_generic", "k_relayout", "k_convert4", "k_copy1",
-      "k_copy16", "k_pad_rows", "k_widen_bf16"};
+      "k_move_tiled", "k_move_tiled_as", "k_move_tiled16", "k_move_tiled16v", "k_move_tiled32", "k_move_gather", "k_move_generic", "k_relayout", "k_convert4", "k_copy1",
+      "k_copy16", "k_pad_rows", "k_pad_rows16", "k_widen_bf16"};
   const uint32_t n = sizeof families / sizeof families[0];
   for (uint32_t i = 0; i < n && i < cap && names; i++) names[i] = families[i];
   return n;

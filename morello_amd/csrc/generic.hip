@@ -258,15 +258,67 @@ __global__ __launch_bounds__(256) void k_move_tiled(MoveStrided p) {
   }
   const uint32_t lane = threadIdx.x & 63, quad = threadIdx.x >> 6;
   const uint32_t s0 = ts * 64, d0 = td * 64, ns = p.shape[p.dim_s], nd = p.shape[p.dim_d];
-#pragma unroll 4
-  for (uint32_t r = quad; r < 64; r += 4)
+  // All sixteen loads of a thread are issued before the first is used: a small tensor is a
+  // handful of tiles, and their time is these loads' latency.
+  uint32_t v[16];
+#pragma unroll
+  for (uint32_t i = 0; i < 16; i++) {
+    const uint32_t r = quad + 4 * i;
+    v[i] = 0;
     if (d0 + r < nd && s0 + lane < ns)
-      tile[r][lane] = move_bits(p.src, p.sdt, so + int64_t(d0 + r) * p.ss[p.dim_d] + int64_t(s0 + lane) * p.ss[p.dim_s], p.ddt);
+      v[i] = move_bits(p.src, p.sdt, so + int64_t(d0 + r) * p.ss[p.dim_d] + int64_t(s0 + lane) * p.ss[p.dim_s], p.ddt);
+  }
+#pragma unroll
+  for (uint32_t i = 0; i < 16; i++) tile[quad + 4 * i][lane] = v[i];
   __syncthreads();
-#pragma unroll 4
-  for (uint32_t r = quad; r < 64; r += 4)
+#pragma unroll
+  for (uint32_t i = 0; i < 16; i++) {
+    const uint32_t r = quad + 4 * i;
     if (s0 + r < ns && d0 + lane < nd)
       store_u32(p.dst, p.ddt, d_o + int64_t(s0 + r) * p.ds[p.dim_s] + int64_t(d0 + lane) * p.ds[p.dim_d], tile[lane][r]);
+  }
+}
+
+// The same with nothing converted: typed loads and stores (the dtype switch of the converting
+// form puts a branch between any two loads, so none of them overlap).
+template <class E>
+__global__ __launch_bounds__(256) void k_move_tiled_as(MoveStrided p) {
+  __shared__ uint32_t tile[64][65];
+  const E *src = static_cast<const E *>(p.src);
+  E *dst = static_cast<E *>(p.dst);
+  uint64_t blk = blockIdx.x;
+  const uint32_t ts = uint32_t(blk % p.tiles_s);
+  blk /= p.tiles_s;
+  const uint32_t td = uint32_t((blk + ts) % p.tiles_d);
+  blk /= p.tiles_d;
+  // The remaining dims, slowest to fastest in `order` (dim_s and dim_d are skipped).
+  int64_t so = 0, d_o = 0;
+  for (int o = int(p.rank) - 1; o >= 0; o--) {
+    const uint32_t d = p.order[o];
+    if (d == p.dim_s || d == p.dim_d) continue;
+    const uint32_t c = uint32_t(blk % p.shape[d]);
+    blk /= p.shape[d];
+    so += int64_t(c) * p.ss[d], d_o += int64_t(c) * p.ds[d];
+  }
+  const uint32_t lane = threadIdx.x & 63, quad = threadIdx.x >> 6;
+  const uint32_t s0 = ts * 64, d0 = td * 64, ns = p.shape[p.dim_s], nd = p.shape[p.dim_d];
+  uint32_t v[16];
+#pragma unroll
+  for (uint32_t i = 0; i < 16; i++) {
+    const uint32_t r = quad + 4 * i;
+    v[i] = 0;
+    if (d0 + r < nd && s0 + lane < ns)
+      v[i] = src[so + int64_t(d0 + r) * p.ss[p.dim_d] + int64_t(s0 + lane) * p.ss[p.dim_s]];
+  }
+#pragma unroll
+  for (uint32_t i = 0; i < 16; i++) tile[quad + 4 * i][lane] = v[i];
+  __syncthreads();
+#pragma unroll
+  for (uint32_t i = 0; i < 16; i++) {
+    const uint32_t r = quad + 4 * i;
+    if (s0 + r < ns && d0 + lane < nd)
+      dst[d_o + int64_t(s0 + r) * p.ds[p.dim_s] + int64_t(d0 + lane) * p.ds[p.dim_d]] = E(tile[lane][r]);
+  }
 }
 
 // The same transpose for 16-bit elements that are not converted: 128 x 128 tiles, two elements
@@ -565,6 +617,20 @@ __global__ __launch_bounds__(256) void k_pad_rows(const E *__restrict__ src, uin
       if (col0 + e < cols) word |= uint32_t(from[col0 + e]) << (8 * sizeof(E) * e);
     dst[i] = word;
   }
+}
+
+// The same when rows start on 16 bytes on both sides and `cols` is whole 16-byte vectors: one
+// thread per destination vector (sizes and strides here count vectors).
+__global__ __launch_bounds__(256) void k_pad_rows16(const v4u *__restrict__ src, v4u *__restrict__ dst, uint32_t rows,
+                                                    uint32_t cols, int64_t src_batch, int64_t src_ld, uint32_t dst_ld,
+                                                    uint64_t vectors) {
+  const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= vectors) return;
+  const uint64_t line = i / dst_ld;
+  const uint32_t col = uint32_t(i % dst_ld);
+  v4u v{0, 0, 0, 0};
+  if (col < cols) v = __builtin_nontemporal_load(src + int64_t(line / rows) * src_batch + int64_t(line % rows) * src_ld + col);
+  __builtin_nontemporal_store(v, dst + i);
 }
 
 __global__ void k_copy1(const uint8_t *src, uint8_t *dst, uint64_t bytes) {
@@ -944,7 +1010,10 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
   // A shared contiguous dim serves both sides when its runs are at least 64 bytes long.
   const bool shared_runs = dim_s >= 0 && dim_s == dim_d &&
                            (rank == 1 || uint64_t(p.shape[dim_s]) * mrl_dtype_size(src_dtype) >= 64);
-  if (dim_s < 0 || dim_d < 0 || shared_runs) {
+  // A tensor this small is one round of workgroups either way: an element per thread finishes
+  // in a third of the time the tiled kernels' loops over a handful of tiles take.
+  const bool tiny = p.count <= 32768;
+  if (dim_s < 0 || dim_d < 0 || shared_runs || tiny) {
     // Whole 16-byte vectors along the shared dim, everywhere: move vectors, not elements.
     const int64_t per = 16 / int64_t(mrl_dtype_size(src_dtype));
     bool vectors = dim_s >= 0 && dim_s == dim_d && src_dtype == dst_dtype && p.shape[dim_s] % per == 0 &&
@@ -1007,7 +1076,10 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
     if (octets) MRL_LAUNCH(k_move_tiled16v, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
     else if (pairs) MRL_LAUNCH(k_move_tiled16, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
     else if (quads) MRL_LAUNCH(k_move_tiled32, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
-    else MRL_LAUNCH(k_move_tiled, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+    else if (src_dtype != dst_dtype) MRL_LAUNCH(k_move_tiled, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+    else if (mrl_dtype_size(src_dtype) == 1) MRL_LAUNCH(k_move_tiled_as<uint8_t>, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+    else if (mrl_dtype_size(src_dtype) == 2) MRL_LAUNCH(k_move_tiled_as<uint16_t>, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+    else MRL_LAUNCH(k_move_tiled_as<uint32_t>, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
     return mrl::plan::last_error();
   }
   // Otherwise a tile grown digit by digit: along the destination's fastest digits until they
@@ -1093,6 +1165,15 @@ hipError_t launch_pad_rows(const Strided &src, void *dst, uint32_t dst_ld, uint3
   const uint32_t blocks = uint32_t(std::min<uint64_t>((dwords + 255) / 256, 65536));
   const int64_t sb = batch == 1 ? 0 : src.stride[0], sl = rows == 1 ? 0 : src.stride[1];
   plan::work(plan::UNIT_STREAM, 0, double(batch) * rows * cols * elem_size + 4.0 * dwords);
+  const uint32_t per16 = 16 / elem_size;
+  if (cols % per16 == 0 && dst_ld % per16 == 0 && sb % per16 == 0 && sl % per16 == 0 &&
+      (reinterpret_cast<uintptr_t>(src.ptr) & 15) == 0 && (reinterpret_cast<uintptr_t>(dst) & 15) == 0 &&
+      dwords / 4 <= 0x7fffffffull * 256) {
+    const uint64_t vectors = dwords / 4;
+    MRL_LAUNCH(k_pad_rows16, dim3(uint32_t((vectors + 255) / 256)), dim3(256), 0, stream, (const v4u *)src.ptr, (v4u *)dst,
+               rows, cols / per16, sb / per16, sl / per16, dst_ld / per16, vectors);
+    return mrl::plan::last_error();
+  }
   if (elem_size == 1)
     MRL_LAUNCH(k_pad_rows<uint8_t>, dim3(blocks), dim3(256), 0, stream, (const uint8_t *)src.ptr,
                        (uint32_t *)dst, rows, cols, sb, sl, dst_ld, dwords);

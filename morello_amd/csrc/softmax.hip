@@ -357,7 +357,10 @@ hipError_t launch_rows(const float *in, void *out, uint64_t rows, uint32_t cols,
 
 // Scratch the chunked kernels want for this shape (0: the shape runs without).
 size_t softmax_scratch_bytes(uint64_t rows, uint32_t cols) {
-  if (cols <= 16 * 256) return 0;
+  // Up to 4096 columns the register kernel serves (a multiple of 4), or one wavefront per row
+  // when the rows are many or short; fewer, longer rows that are not whole vectors go in chunks
+  // too (a single one), with scalar loads: a wavefront's loop over such a row is all latency.
+  if (cols <= 16 * 256 && (cols % 4 == 0 || cols <= 256 || rows >= 4096)) return 0;
   const uint64_t chunks = (cols + SOFTMAX_CHUNK - 1) / SOFTMAX_CHUNK;
   if (rows * chunks > 0x7fffffffull) return 0;
   return size_t(rows * chunks * sizeof(float2));

@@ -37,7 +37,8 @@ def test_softmax_edge_values(gpu):
 
 @pytest.mark.parametrize("shape,dim", [((64, 100000), 1), ((3, 4097), 1), ((5, 20000), 1), ((2, 8192), 1),
                                        ((1, 1 << 20), 1), ((300, 4100), 1), ((2, 3, 12290), 2), ((256, 8192), 1),
-                                       ((300, 16384), 1), ((260, 4100), 1), ((257, 12292), 1)])
+                                       ((300, 16384), 1), ((260, 4100), 1), ((257, 12292), 1), ((134, 2350), 1),
+                                       ((7, 3, 1001), 2), ((4000, 258), 1)])
 def test_softmax_long_rows(gpu, shape, dim):
     """Rows beyond the register kernel's 4096 columns: a workgroup per 4096-element chunk, the
     chunks' (max, denominator) pairs merged per row.  Column counts that are and are not

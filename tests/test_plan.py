@@ -89,7 +89,8 @@ def test_plans_follow_shape_dtype_and_layout():
     transposed = [M.row_major(sq), M.col_major(sq)]
     assert M.Move(sq, (M.f32, M.f32), layouts=transposed).plan().kernels == ["k_move_tiled32"]
     assert M.Move(sq, (M.bf16, M.bf16), layouts=transposed).plan().kernels == ["k_move_tiled16v"]
-    assert M.Move(sq, (M.u8, M.u8), layouts=transposed).plan().kernels == ["k_move_tiled"]
+    assert M.Move(sq, (M.u8, M.u8), layouts=transposed).plan().kernels == ["k_move_tiled_as"]
+    assert M.Move(sq, (M.u8, M.f32), layouts=transposed).plan().kernels == ["k_move_tiled"]
     odd = [4098, 4098]
     assert M.Move(odd, (M.bf16, M.bf16), layouts=[M.row_major(odd), M.col_major(odd)]).plan().kernels == ["k_move_tiled16"]
     assert M.Move(sq, (M.f32, M.f32)).plan().kernels == ["k_copy16"]
@@ -118,6 +119,16 @@ def test_every_planned_kernel_is_a_kernel_of_the_target():
         plan = spec.plan()
         assert plan.steps and set(plan.kernels) <= families, (spec, plan)
         assert plan.cost_ns >= 2000 * len(plan.steps) and abs(plan.cost_ns - sum(s.cost_ns for s in plan.steps)) < 1e-3
+
+
+def test_target_kernel_list_is_the_kernels_in_the_sources():
+    import glob, os, re
+    root = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "morello_amd", "csrc")
+    found = set()
+    for path in glob.glob(os.path.join(root, "*.hip")) + glob.glob(os.path.join(root, "*.h")):
+        found |= set(re.findall(r"__global__[^;{]*?void (k_\w+)\(", open(path).read(), flags=re.S))
+    found.discard("k_mfma_rate")  # the rate measurement, not a Spec's kernel
+    assert found == set(M.Target.kernels())
 
 
 def test_cost_orders_what_search_has_to_order():
