@@ -402,6 +402,10 @@ typedef struct {
  * that runs a Spec, with launches recorded instead of made, so it cannot disagree with a run.
  * MRL_ERR_UNSUPPORTED / MRL_ERR_BAD_SPEC as mrl_run. */
 int mrl_spec_plan(const mrl_spec *spec, mrl_plan *plan, mrl_plan_step *steps, uint32_t cap);
+/* The same for a Matmul under a manual schedule (mrl_run_matmul_scheduled): what a search over
+ * tile_out / split (scheduling_sugar.rs:37-132) compares. */
+int mrl_matmul_scheduled_plan(const mrl_spec *spec, const mrl_matmul_schedule *schedule, mrl_plan *plan,
+                              mrl_plan_step *steps, uint32_t cap);
 /* The same for a general Compose. */
 int mrl_compose_plan(const mrl_compose *c, mrl_plan *plan, mrl_plan_step *steps, uint32_t cap);
 

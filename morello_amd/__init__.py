@@ -328,6 +328,29 @@ class ScheduledMatmul:
     def split(self, k: int) -> "ScheduledMatmul":
         return ScheduledMatmul(self.spec, self.tile_m, self.tile_n, int(k))
 
+    def plan(self) -> "Plan":
+        if self.split_k is None:
+            raise MorelloError(1, "schedule needs .split(k)")
+        sched = B.MatmulScheduleC(self.tile_m, self.tile_n, self.split_k)
+        fn = lambda spec, head, steps, cap: B.load().mrl_matmul_scheduled_plan(spec, C.byref(sched), head, steps, cap)
+        return _plan_of(fn, self.spec._c, "mrl_matmul_scheduled_plan")
+
+    def run_timed(self, ptrs: Sequence[int], steps: int) -> float:
+        """Host-clock milliseconds for `steps` launches of this schedule, queue drained."""
+        import time
+        if self.split_k is None:
+            raise MorelloError(1, "schedule needs .split(k)")
+        sched = B.MatmulScheduleC(self.tile_m, self.tile_n, self.split_k)
+        arr = (C.c_void_p * len(ptrs))(*ptrs)
+        lib = B.load()
+        synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            _check(lib.mrl_run_matmul_scheduled(C.byref(self.spec._c), arr, C.byref(sched), None),
+                   "mrl_run_matmul_scheduled")
+        synchronize()
+        return (time.perf_counter() - t0) * 1e3
+
     def run_device(self, ptrs: Sequence[int]):
         if self.split_k is None:
             raise MorelloError(1, "schedule needs .split(k)")

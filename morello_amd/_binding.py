@@ -138,6 +138,8 @@ SIGNATURES = {
     "mrl_target_memories": (C.c_uint32, [C.POINTER(TargetMemoryC), C.c_uint32]),
     "mrl_target_kernels": (C.c_uint32, [C.POINTER(C.c_char_p), C.c_uint32]),
     "mrl_spec_plan": (C.c_int, [C.POINTER(SpecC), C.POINTER(PlanC), C.POINTER(PlanStepC), C.c_uint32]),
+    "mrl_matmul_scheduled_plan": (C.c_int, [C.POINTER(SpecC), C.POINTER(MatmulScheduleC), C.POINTER(PlanC),
+                                            C.POINTER(PlanStepC), C.c_uint32]),
     "mrl_compose_plan": (C.c_int, [C.POINTER(ComposeC), C.POINTER(PlanC), C.POINTER(PlanStepC), C.c_uint32]),
     "mrl_device_info": (C.c_int, [C.c_char_p, C.c_size_t, C.POINTER(C.c_int), C.POINTER(C.c_int),
                                   C.POINTER(C.c_size_t)]),

@@ -1468,6 +1468,16 @@ int mrl_run_matmul_scheduled(const mrl_spec *spec, void *const *params,
   return run_matmul(*spec, params, ws, schedule);
 }
 
+int mrl_matmul_scheduled_plan(const mrl_spec *spec, const mrl_matmul_schedule *schedule, mrl_plan *plan,
+                              mrl_plan_step *steps, uint32_t cap) {
+  if (!schedule) return MRL_ERR_NULL;
+  int rc = check_spec(spec);
+  if (rc != MRL_OK) return rc;
+  if (spec->kind != MRL_SPEC_MATMUL) return MRL_ERR_UNSUPPORTED;
+  return plan_with(spec->n_params, plan, steps, cap,
+                   [&](void *const *params, Workspace &ws) { return run_matmul(*spec, params, ws, schedule); });
+}
+
 int mrl_bench(const mrl_spec *spec, void *const *params, uint32_t iters, uint32_t repeats,
               double *best_ns_per_iter, double *mean_ns_per_iter) {
   if (!best_ns_per_iter || !mean_ns_per_iter) return MRL_ERR_NULL;

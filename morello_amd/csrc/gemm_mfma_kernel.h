@@ -526,8 +526,9 @@ hipError_t launch(const GemmArgs &g, hipStream_t stream) {
     plan::work(T::ES == 1 ? plan::UNIT_MFMA_I8 : T::ES == 2 ? plan::UNIT_MFMA_BF16 : plan::UNIT_MFMA_F32,
                2.0 * mn * g.k, (double(g.m) * g.k + double(g.k) * g.n) * g.batch * T::ES + mn * 4 * (g.accum ? 2 : 1),
                2.0 * BM * BN * k_steps,
-               // prologue and epilogue, then one barrier-to-barrier trip per 128 bytes of K
-               500.0 + 450.0 * double((g.k * T::ES + TL::BKB - 1) / TL::BKB));
+               // prologue and epilogue, then one barrier-to-barrier trip per step of K, longer for a
+               // larger tile (measured 0.4-0.55 us at 64 x 64, 0.6-1.0 at 128 x 128, 1.4-2.0 at 256 x 256)
+               500.0 + (100.0 + 3.0 * (BM + BN)) * double((g.k * T::ES + TL::BKB - 1) / TL::BKB));
   }
   MRL_LAUNCH((k_gemm<T, A_UNSIGNED, TL, EDGE, B_KMAJOR, CONV>), dim3(tiles_m * tiles_n, g.batch), dim3(TL::NT),
              2 * STAGE, stream, g, tiles_m, tiles_n);
