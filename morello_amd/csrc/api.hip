@@ -385,7 +385,8 @@ bool dense_row_major(const mrl::Strided &t) {
 bool as_rows(const mrl::Strided &t, int64_t *ld, int64_t *batch_stride) {
   if (t.rank != 3) return false;
   if (t.shape[2] != 1 && t.stride[2] != 1) return false;
-  *ld = t.shape[1] == 1 ? int64_t(t.shape[2]) : t.stride[1];
+  // A single row has no stride of its own to go by, unless it is a padded one.
+  *ld = (t.shape[1] == 1 && t.stride[1] < int64_t(t.shape[2])) ? int64_t(t.shape[2]) : t.stride[1];
   *batch_stride = t.shape[0] == 1 ? 0 : t.stride[0];
   return *ld >= int64_t(t.shape[2]);
 }
@@ -1284,7 +1285,7 @@ uint32_t mrl_target_memories(mrl_target_memory *out, uint32_t cap) {
 uint32_t mrl_target_kernels(const char **names, uint32_t cap) {
   static const char *const families[] = {
       "k_gemm", "k_gemv", "k_matmul_generic", "k_conv_i8", "k_conv_generic", "k_conv_generic_wave", "k_unfold",
-      "k_unfold_gather", "k_attn", "k_attn_merge", "k_softmax_regs", "k_softmax_block", "k_softmax_chunk_stats", "k_softmax_chunk_write", "k_softmax_stream",
+      "k_unfold_gather", "k_attn", "k_attn_merge", "k_softmax_regs", "k_softmax_short", "k_softmax_block", "k_softmax_chunk_stats", "k_softmax_chunk_write", "k_softmax_stream",
       "k_softmax_cols",
       "k_softmax_generic", "k_parts", "k_broadcast", "k_fill", "k_fill_zero", "k_move_rows", "k_move_rows16",
       "k_move_tiled", "k_move_tiled_as", "k_move_tiled16", "k_move_tiled16v", "k_move_tiled32", "k_move_gather", "k_move_generic", "k_relayout", "k_convert4", "k_copy1",

@@ -392,13 +392,37 @@ __global__ __launch_bounds__(256) void k_attn_merge(const float *__restrict__ pa
   const uint64_t row = i / n_out;
   const uint32_t col = uint32_t(i % n_out);
   const float *part = partials + row * splits * (d + 4);
-  float m = part[d];
-  for (uint32_t s = 1; s < splits; s++) m = fmaxf(m, part[s * (d + 4) + d]);
+  const uint32_t stride = d + 4;
+  // Eight splits' loads in flight at a time: the loop is all latency otherwise (35 splits one
+  // after another took 20 us).
+  constexpr uint32_t U = 8;
+  float m = -3.0e38f;
+  for (uint32_t s0 = 0; s0 < splits; s0 += U) {
+    float ms[U];
+#pragma unroll
+    for (uint32_t u = 0; u < U; u++) {
+      const float v = part[(s0 + u < splits ? s0 + u : 0) * stride + d];  // always a valid address
+      ms[u] = s0 + u < splits ? v : -3.0e38f;
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < U; u++) m = fmaxf(m, ms[u]);
+  }
   float num = 0.0f, den = 0.0f;
-  for (uint32_t s = 0; s < splits; s++) {
-    const float w = __builtin_amdgcn_exp2f((part[s * (d + 4) + d] - m) * LOG2E);
-    num += part[s * (d + 4) + col] * w;
-    den += part[s * (d + 4) + d + 1] * w;
+  for (uint32_t s0 = 0; s0 < splits; s0 += U) {
+    float ms[U], ls[U], os[U];
+#pragma unroll
+    for (uint32_t u = 0; u < U; u++) {
+      const bool in = s0 + u < splits;
+      const float *p = part + (in ? s0 + u : 0) * stride;
+      const float mv = p[d], lv = p[d + 1], ov = p[col];
+      ms[u] = in ? mv : -3.0e38f, ls[u] = in ? lv : 0.0f, os[u] = in ? ov : 0.0f;
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < U; u++) {
+      const float w = __builtin_amdgcn_exp2f((ms[u] - m) * LOG2E);
+      num += os[u] * w;
+      den += ls[u] * w;
+    }
   }
   out[row * n_out + col] = num / den;
 }

@@ -1012,7 +1012,7 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
                            (rank == 1 || uint64_t(p.shape[dim_s]) * mrl_dtype_size(src_dtype) >= 64);
   // A tensor this small is one round of workgroups either way: an element per thread finishes
   // in a third of the time the tiled kernels' loops over a handful of tiles take.
-  const bool tiny = p.count <= 32768;
+  const bool tiny = p.count <= 65536;
   if (dim_s < 0 || dim_d < 0 || shared_runs || tiny) {
     // Whole 16-byte vectors along the shared dim, everywhere: move vectors, not elements.
     const int64_t per = 16 / int64_t(mrl_dtype_size(src_dtype));

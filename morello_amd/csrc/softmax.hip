@@ -129,6 +129,62 @@ __global__ __launch_bounds__(256) void k_softmax_stream(const float *__restrict_
   }
 }
 
+// Rows of up to 256 elements: L lanes per row (a power of two, 64 / L rows per wavefront), up to
+// eight elements per lane in registers, the reductions by shuffles within the L lanes.  A wavefront
+// per row would leave most lanes idle and cost a wavefront's fixed work for a handful of elements
+// (2.7 million rows of 67: 1.28 ms).
+template <int L, bool OUT_BF16>
+__global__ __launch_bounds__(256) void k_softmax_short(const float *__restrict__ in, void *__restrict__ out_any,
+                                                       uint64_t rows, uint32_t cols) {
+  constexpr int PER = 8;
+  const uint64_t thread = uint64_t(blockIdx.x) * 256 + threadIdx.x;
+  const uint64_t row = thread / L;
+  const uint32_t j = uint32_t(thread % L);
+  const bool live = row < rows;
+  const float *src = in + (live ? row : 0) * cols;
+  float x[PER];
+  float mx = F32_MIN;
+  bool nan = false;
+#pragma unroll
+  for (int i = 0; i < PER; i++) {
+    const uint32_t e = j + i * L;
+    x[i] = (live && e < cols) ? src[e] : F32_MIN;
+    nan |= x[i] != x[i];
+    mx = fmaxf(mx, x[i]);
+  }
+#pragma unroll
+  for (int o = L / 2; o > 0; o >>= 1) {
+    mx = fmaxf(mx, __shfl_xor(mx, o));
+    nan |= __shfl_xor(int(nan), o) != 0;
+  }
+  if (nan) mx = __uint_as_float(0x7fc00000u);
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < PER; i++) {
+    x[i] = expf(x[i] - mx);
+    sum += (j + i * L < cols) ? x[i] : 0.0f;
+  }
+#pragma unroll
+  for (int o = L / 2; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+  if (!live) return;
+#pragma unroll
+  for (int i = 0; i < PER; i++) {
+    const uint32_t e = j + i * L;
+    if (e >= cols) continue;
+    const float y = x[i] / sum;
+    if constexpr (OUT_BF16) (static_cast<uint16_t *>(out_any) + row * cols)[e] = uint16_t(bf16_bits(y));
+    else (static_cast<float *>(out_any) + row * cols)[e] = y;
+  }
+}
+
+template <int L, bool OUT_BF16>
+hipError_t launch_short(const float *in, void *out, uint64_t rows, uint32_t cols, hipStream_t stream) {
+  const uint64_t blocks = (rows * L + 255) / 256;
+  if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
+  MRL_LAUNCH((k_softmax_short<L, OUT_BF16>), dim3(uint32_t(blocks)), dim3(256), 0, stream, in, out, rows, cols);
+  return mrl::plan::last_error();
+}
+
 // ---- rows longer than the register kernel takes: a workgroup per 4096-element chunk ----
 // One wavefront per row leaves a few long rows (64 x 100000) on a handful of compute units, and
 // its scalar loop waits out every load.  Here a workgroup owns SOFTMAX_CHUNK consecutive elements
@@ -327,6 +383,15 @@ namespace {
 template <bool OUT_BF16>
 hipError_t launch_rows(const float *in, void *out, uint64_t rows, uint32_t cols, void *scratch, hipStream_t stream) {
   if (rows == 0 || cols == 0) return hipSuccess;
+  if (cols <= 256 && rows * 32 <= 0x7fffffffull * 256) {
+    plan::work(plan::UNIT_STREAM, 0, double(rows) * cols * (4 + (OUT_BF16 ? 2 : 4)));
+    if (cols <= 8) return launch_short<1, OUT_BF16>(in, out, rows, cols, stream);
+    if (cols <= 16) return launch_short<2, OUT_BF16>(in, out, rows, cols, stream);
+    if (cols <= 32) return launch_short<4, OUT_BF16>(in, out, rows, cols, stream);
+    if (cols <= 64) return launch_short<8, OUT_BF16>(in, out, rows, cols, stream);
+    if (cols <= 128) return launch_short<16, OUT_BF16>(in, out, rows, cols, stream);
+    return launch_short<32, OUT_BF16>(in, out, rows, cols, stream);
+  }
   if (cols > 16 * 256 && cols <= 16 * 1024 && cols % 4 == 0 && rows >= 256 && rows <= 0x7fffffffull) {
     plan::work(plan::UNIT_STREAM, 0, double(rows) * cols * (4 + (OUT_BF16 ? 2 : 4)));
     if (cols <= 8 * 1024) MRL_LAUNCH((k_softmax_block<8, OUT_BF16>), dim3(uint32_t(rows)), dim3(256), 0, stream, in, out, cols);

@@ -228,6 +228,8 @@ def test_matmul_every_tile_choice(gpu, dts, codes, shape, accum, b_k_fastest):
     ((1, 1, 300, 4096), False),     # row-major B: one slice of K that is not whole steps of 64
     ((2, 3, 1000, 8192), True),
     ((1, 4, 2048, 4112), True),
+    ((4, 1, 3565, 256), False),     # one row whose K is not whole 16-byte chunks: the padded copy keeps its stride
+    ((2, 1, 1001, 300), True),
 ])
 @pytest.mark.parametrize("b_k_fastest", [True, False])
 def test_matrix_vector_shapes(gpu, dts, codes, shape, accum, b_k_fastest):

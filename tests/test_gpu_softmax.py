@@ -75,6 +75,26 @@ def test_softmax_long_rows_edge_values(gpu):
     assert (np.abs(got[[0, 1, 3]] - want) <= 1e-5 * np.abs(want) + 1e-12).all()
 
 
+@pytest.mark.parametrize("shape,dim", [((100000, 3), 1), ((5000, 67), 1), ((1000, 5, 12), 2), ((4097, 255), 1), ((3, 256), 1),
+                                       ((7, 1), 1), ((300, 584, 5), 2), ((1, 129), 1), ((65, 33), 1), ((4, 9, 16), 2)])
+def test_softmax_short_rows(gpu, shape, dim):
+    """Rows of up to 256 elements: 1 to 32 lanes per row, several rows per wavefront (every lane
+    count, row counts that leave a wavefront partly empty, a NaN confined to its row)."""
+    x = synth.normal_f32(207, 0, shape, std=3.0)
+    got = run_spec(M.Softmax(list(shape), dim), [x, np.zeros(shape, np.float32)])
+    want = orc.softmax(list(shape), dim, x)
+    assert (np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-12).all()
+    flat = x.reshape(-1, shape[-1]).copy()
+    flat[0, 0] = np.nan
+    if flat.shape[0] > 1:
+        flat[1, :] = -np.inf
+    got = run_spec(M.Softmax(list(flat.shape), 1), [flat, np.zeros_like(flat)])
+    assert np.isnan(got[0]).all() and not np.isnan(got[2:]).any()
+    want = orc.softmax(list(flat.shape), 1, flat)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert (np.abs(got[2:] - want[2:]) <= 1e-5 * np.abs(want[2:]) + 1e-12).all()
+
+
 @pytest.mark.parametrize("shape,dim", [((2048, 4096), 0), ((600, 70), 0), ((3, 1000, 130), 1), ((513, 64), 0),
                                        ((7, 16), 0), ((2, 5000, 17), 1)])
 def test_softmax_over_an_outer_dim(gpu, shape, dim):

@@ -70,6 +70,8 @@ def test_plans_follow_shape_dtype_and_layout():
     # Ragged sizes: zero-padded copies of A and B, then the edge build of a small tile.
     p = M.Matmul([1, 1000, 1000, 1000], (M.u8, M.i8, M.i32)).plan()
     assert p.kernels == ["k_pad_rows", "k_pad_rows", "k_gemm"] and "EDGE = true" in p.steps[2].kernel
+    # One row of A with a ragged K: padded, and still on the matrix cores.
+    assert M.Matmul([4, 1, 3565, 256], (M.bf16, M.bf16, M.f32)).plan().kernels == ["k_pad_rows", "k_gemm"]
     # Matrix-vector with a k-fastest B: dot products, not the matrix cores.
     p = M.Matmul([1, 1, 2048, 16384], (M.bf16, M.bf16, M.f32), layouts=[None, KT, None]).plan()
     assert p.kernels == ["k_gemv"] and p.steps[0].unit == "hbm"
@@ -84,6 +86,7 @@ def test_plans_follow_shape_dtype_and_layout():
     assert M.Softmax([64, 100000], 1).plan().kernels == ["k_softmax_chunk_stats", "k_softmax_chunk_write"]
     assert M.Softmax([8192, 8192], 1).plan().kernels == ["k_softmax_block"]
     assert M.Softmax([2048, 4096], 0).plan().kernels == ["k_softmax_cols"]
+    assert M.Softmax([100000, 67], 1).plan().kernels == ["k_softmax_short"]
     # Moves: transpose tiled through LDS, Packed destination gathered, plain copy.
     sq = [4096, 4096]
     transposed = [M.row_major(sq), M.col_major(sq)]
