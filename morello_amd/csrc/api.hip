@@ -498,9 +498,22 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
     HIP_TRY(e);
     return finish_output(c, ws);
   }
-  if (kind >= 0 && rows && mrl::gemm_possible(g, kind) && mrl::gemm_pays(g, kind))
-    HIP_TRY(mrl::launch_gemm(g, kind, ws.stream));
-  else
+  if (kind >= 0 && rows && mrl::gemm_possible(g, kind) && mrl::gemm_pays(g, kind)) {
+    const uint32_t splits = mrl::gemm_k_splits(g, kind);
+    if (splits > 1) {
+      // Slices of K as batch entries writing dense partial results, summed into C in slice order.
+      void *partial = nullptr;
+      HIP_TRY(ws.alloc(&partial, size_t(splits) * g.m * g.n * 4));
+      mrl::GemmArgs slices = g;
+      slices.batch = splits, slices.k = g.k / splits;
+      slices.sa = slices.k, slices.sb = g.b_kmajor ? int64_t(slices.k) : int64_t(slices.k) * g.ldb;
+      slices.c = partial, slices.ldc = g.n, slices.sc = int64_t(g.m) * g.n, slices.accum = 0;
+      HIP_TRY(mrl::launch_gemm(slices, kind, ws.stream));
+      HIP_TRY(mrl::launch_sum_splits(partial, g.c, splits, g.m, g.n, g.ldc, g.accum != 0, kind <= 1, ws.stream));
+    } else {
+      HIP_TRY(mrl::launch_gemm(g, kind, ws.stream));
+    }
+  } else
     HIP_TRY(mrl::launch_matmul_generic(a.t, b.t, c.t, s.accum, ws.stream));
   return finish();
 }
@@ -541,9 +554,12 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
   // Windows of this many images are unfolded at a time.
   constexpr uint64_t UNFOLD_BYTES = uint64_t(1) << 30;
   const uint64_t image_rows_bytes = pixels * row_elems * img.elem;
-  const bool as_matmul = !fused_shape && kind >= 0 && row_elems * img.elem < (1u << 24) &&
-                         double(cv.b) * pixels * cv.f * window >= 1e6;
-  const bool can_unfold = image_rows_bytes <= UNFOLD_BYTES;
+  // One kernel (windows read in place, or a 1x1 filter) pays from 1e5 multiply-adds on, as a
+  // Matmul does; unfolding first (two or three launches) from 1e6.
+  const double macs = double(cv.b) * pixels * cv.f * window;
+  const bool as_matmul = !fused_shape && kind >= 0 && row_elems * img.elem < (1u << 24) && macs >= 1e5;
+  const bool can_unfold = image_rows_bytes <= UNFOLD_BYTES &&
+                          (macs >= 1e6 || (cv.fh == 1 && cv.fw == 1 && row_elems == window));
   // Tensors in another permutation layout (NCHW, say) are moved to channels-last when a
   // matrix-core path takes the shape: three small extra passes against a generic kernel
   // that is hundreds of times slower.
@@ -1284,7 +1300,7 @@ uint32_t mrl_target_memories(mrl_target_memory *out, uint32_t cap) {
 
 uint32_t mrl_target_kernels(const char **names, uint32_t cap) {
   static const char *const families[] = {
-      "k_gemm", "k_gemv", "k_matmul_generic", "k_conv_i8", "k_conv_generic", "k_conv_generic_wave", "k_unfold",
+      "k_gemm", "k_gemv", "k_matmul_generic", "k_sum_splits", "k_conv_i8", "k_conv_generic", "k_conv_generic_wave", "k_unfold",
       "k_unfold_gather", "k_attn", "k_attn_merge", "k_softmax_regs", "k_softmax_short", "k_softmax_block", "k_softmax_chunk_stats", "k_softmax_chunk_write", "k_softmax_stream",
       "k_softmax_cols",
       "k_softmax_generic", "k_parts", "k_broadcast", "k_fill", "k_fill_zero", "k_move_rows", "k_move_rows16",

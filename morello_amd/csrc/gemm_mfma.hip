@@ -64,6 +64,20 @@ bool gemm_pays(const GemmArgs &g, int) { return double(g.m) * g.n * g.k * g.batc
 
 uint32_t gemm_tile_side(const GemmArgs &g, int kind) { return tile_side(g, elem_size_of(kind)); }
 
+// Fewer than three quarters of the compute units would get a 64 x 64 tile and every tile walks at
+// least sixteen k steps: share K out so that up to 512 workgroups run, eight steps each at least
+// (int8 512 x 8192 x 512: 64 tiles of 64 steps, 36 us; as 8 x 64 tiles of 8 steps plus the sum, 10 us).
+uint32_t gemm_k_splits(const GemmArgs &g, int kind) {
+  const uint64_t es = elem_size_of(kind);
+  if (g.batch != 1 || gemv_applicable(g, kind) || (uint64_t(g.k) * es) % 128 != 0) return 1;
+  const uint64_t steps = uint64_t(g.k) * es / 128;
+  const uint64_t tiles = uint64_t((g.m + 63) / 64) * ((g.n + 63) / 64);
+  if (tiles >= 384 || steps < 16) return 1;
+  uint64_t want = std::min<uint64_t>({32, 768 / tiles, steps / 8});
+  while (want > 1 && steps % want != 0) want--;
+  return uint32_t(std::max<uint64_t>(1, want));
+}
+
 hipError_t launch_gemm_big(const GemmArgs &g, int kind, hipStream_t stream) {
   if (g.b_kmajor) return launch_gemm_nt(g, kind, 256, stream);
   const bool whole = whole_tiles(g, elem_size_of(kind));

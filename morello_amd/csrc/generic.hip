@@ -1275,6 +1275,43 @@ hipError_t launch_softmax_generic(const Strided &in, const Strided &out, uint32_
   return mrl::plan::last_error();
 }
 
+namespace {
+// One thread per 32-bit element of C.
+template <class T>
+__global__ __launch_bounds__(256) void k_sum_splits(const T *__restrict__ partial, T *__restrict__ c, uint32_t splits,
+                                                    uint32_t n, uint64_t count, int64_t ldc, int accum) {
+  const uint64_t i = uint64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (i >= count) return;
+  T *to = c + int64_t(i / n) * ldc + int64_t(i % n);
+  T sum = accum ? *to : T(0);
+  constexpr uint32_t U = 8;  // loads in flight together
+  for (uint32_t s0 = 0; s0 < splits; s0 += U) {
+    T v[U];
+#pragma unroll
+    for (uint32_t u = 0; u < U; u++) v[u] = partial[uint64_t(s0 + u < splits ? s0 + u : s0) * count + i];
+#pragma unroll
+    for (uint32_t u = 0; u < U; u++) sum += s0 + u < splits ? v[u] : T(0);
+  }
+  *to = sum;
+}
+}  // namespace
+
+hipError_t launch_sum_splits(const void *partial, void *c, uint32_t splits, uint32_t m, uint32_t n, int64_t ldc,
+                             bool accum, bool integers, hipStream_t stream) {
+  const uint64_t count = uint64_t(m) * n;
+  if (count == 0) return hipSuccess;
+  const uint64_t blocks = (count + 255) / 256;
+  if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
+  plan::work(plan::UNIT_STREAM, 0, 4.0 * count * (splits + 1 + (accum ? 1 : 0)));
+  if (integers)
+    MRL_LAUNCH(k_sum_splits<int>, dim3(uint32_t(blocks)), dim3(256), 0, stream, (const int *)partial, (int *)c, splits, n,
+               count, ldc, int(accum));
+  else
+    MRL_LAUNCH(k_sum_splits<float>, dim3(uint32_t(blocks)), dim3(256), 0, stream, (const float *)partial, (float *)c, splits,
+               n, count, ldc, int(accum));
+  return mrl::plan::last_error();
+}
+
 hipError_t launch_fill_zero(void *ptr, uint64_t bytes, hipStream_t stream) {
   if (bytes == 0) return hipSuccess;
   const uint64_t words = bytes / 4;

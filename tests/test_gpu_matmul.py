@@ -251,6 +251,35 @@ def test_matrix_vector_shapes(gpu, dts, codes, shape, accum, b_k_fastest):
         assert rel_err(got, want) < 1e-5
 
 
+@pytest.mark.parametrize("dts,codes", [((M.u8, M.i8, M.i32), [0, 1, 5]), ((M.i8, M.i8, M.i32), [1, 1, 5]),
+                                       ((M.bf16, M.bf16, M.f32), [7, 7, 6]), ((M.f32, M.f32, M.f32), [6, 6, 6])])
+@pytest.mark.parametrize("shape,accum", [((1, 512, 8192, 512), False), ((1, 256, 16384, 192), True),
+                                         ((1, 100, 4096, 300), True), ((1, 32, 4096, 1000), False),
+                                         ((1, 130, 2048, 70), False)])
+@pytest.mark.parametrize("b_k_fastest", [True, False])
+def test_matmul_with_k_shared_out_over_workgroups(gpu, dts, codes, shape, accum, b_k_fastest):
+    """Few output tiles and a long K: slices of K run as batch entries and their partial results
+    are summed in slice order (exact for integers, the f32 sum in another association for floats).
+    Whole and ragged M and N, accumulation into C, both B orientations, every dtype kind."""
+    b, m, k, n = shape
+    if dts[0] == M.f32:
+        k //= 2  # the same number of 128-byte k steps at twice the element size would take twice as long on the oracle
+    shape = (b, m, k, n)
+    gen = {M.u8: synth.uniform_u8, M.i8: synth.uniform_i8, M.bf16: synth.normal_bf16, M.f32: synth.uniform_f32}
+    A, Bm = gen[dts[0]](76, 0, (b, m, k)), gen[dts[1]](76, 1, (b, k, n))
+    out_np = np.int32 if dts[2] == M.i32 else np.float32
+    C0 = (synth.uniform_u8(76, 2, (b, m, n)).astype(out_np) if accum else np.zeros((b, m, n), out_np))
+    Bbuf = np.ascontiguousarray(Bm.transpose(0, 2, 1)) if b_k_fastest else Bm
+    spec = M.Matmul(list(shape), dts, layouts=[None, M.layout(0, 2, 1) if b_k_fastest else None, None], accum=accum)
+    assert "k_sum_splits" in spec.plan().kernels
+    got = run_spec(spec, [A, Bbuf, C0])
+    want = orc.matmul(list(shape), codes, A, Bm, C0.copy(), accum)
+    if dts[2] == M.i32:
+        assert np.array_equal(got, want)
+    else:
+        assert rel_err(got, want) < (1e-2 if dts[0] == M.bf16 else 1e-5)
+
+
 @pytest.mark.parametrize("dts,codes", [((M.f32, M.bf16, M.f32), [6, 7, 6]), ((M.bf16, M.f32, M.f32), [7, 6, 6])])
 def test_mixed_bf16_f32_matmul(gpu, dts, codes):
     """One bf16 and one f32 input with an f32 output: both are taken to f32 before the product,
