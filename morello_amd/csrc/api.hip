@@ -670,6 +670,44 @@ int run_softmax(const mrl_spec &s, void *const *params, Workspace &ws) {
     if (const size_t bytes = mrl::softmax_scratch_bytes(in.count / cols, cols)) HIP_TRY(ws.alloc(&scratch, bytes));
     HIP_TRY(mrl::launch_softmax_rows((const float *)in.t.ptr, (float *)out.t.ptr, in.count / cols,
                                      cols, scratch, ws.stream));
+  } else if (s.scan_dim < last && dense_row_major(in.t) && dense_row_major(out.t) && in.count < (1ull << 31) &&
+             [&] {
+               // The tensor as [before][scan][after].  The kernel that scans an outer dim takes 64
+               // positions of `after` per workgroup and walks the scan dim in a loop: too few
+               // workgroups (or an `after` too short for it) make that loop the whole run time.
+               uint64_t after = 1;
+               for (uint32_t d = s.scan_dim + 1; d < s.rank; d++) after *= s.spec_shape[d];
+               const uint64_t groups = in.count / s.spec_shape[s.scan_dim] / after * ((after + 63) / 64);
+               // Small tensors: three or four launches, ~14 us, against the one kernel's measured
+               // 2.5 us + 10 ns per scan step (generic) or 5 us + 50 ns (24 ns from 512 steps on).
+               const double scan = s.spec_shape[s.scan_dim];
+               if (in.count <= (1u << 20))
+                 return (after < 16 ? 2.5 + 0.010 * scan : 5.0 + (scan < 512 ? 0.050 : 0.024) * scan) > 15.0;
+               return after < 16 || groups < 256;
+             }()) {
+    // Scan dim made innermost by a transposing Move, the row kernels, and a Move back: three
+    // passes of tuned kernels ([2149, 172] over dim 0: 57 -> 9 us; [1818, 10]: 23 -> 8 us).
+    const uint32_t scan = s.spec_shape[s.scan_dim];
+    uint64_t before = 1, after = 1;
+    for (uint32_t d = 0; d < s.scan_dim; d++) before *= s.spec_shape[d];
+    for (uint32_t d = s.scan_dim + 1; d < s.rank; d++) after *= s.spec_shape[d];
+    void *turned = nullptr, *scratch = nullptr;
+    HIP_TRY(ws.alloc(&turned, in.count * sizeof(float)));
+    mrl::Strided as_given, as_turned;  // both over the index space (before, scan, after)
+    as_given.dtype = as_turned.dtype = MRL_F32, as_given.rank = as_turned.rank = 3;
+    for (uint32_t d = 0; d < MRL_MAX_RANK; d++) as_given.shape[d] = as_turned.shape[d] = 1, as_given.stride[d] = as_turned.stride[d] = 0;
+    as_given.shape[0] = as_turned.shape[0] = uint32_t(before);
+    as_given.shape[1] = as_turned.shape[1] = scan;
+    as_given.shape[2] = as_turned.shape[2] = uint32_t(after);
+    as_given.stride[0] = int64_t(scan) * after, as_given.stride[1] = int64_t(after), as_given.stride[2] = 1;
+    as_turned.stride[0] = int64_t(scan) * after, as_turned.stride[1] = 1, as_turned.stride[2] = scan;
+    as_given.ptr = in.t.ptr, as_turned.ptr = turned;
+    HIP_TRY(mrl::launch_move_strided(as_given, as_turned, ws.stream));
+    const uint64_t rows = before * after;
+    if (const size_t bytes = mrl::softmax_scratch_bytes(rows, scan)) HIP_TRY(ws.alloc(&scratch, bytes));
+    HIP_TRY(mrl::launch_softmax_rows((const float *)turned, (float *)turned, rows, scan, scratch, ws.stream));
+    as_given.ptr = out.t.ptr;
+    HIP_TRY(mrl::launch_move_strided(as_turned, as_given, ws.stream));
   } else {
     HIP_TRY(mrl::launch_softmax_generic(in.t, out.t, s.scan_dim, ws.stream));
   }

@@ -1082,6 +1082,12 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
     else MRL_LAUNCH(k_move_tiled_as<uint32_t>, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
     return mrl::plan::last_error();
   }
+  // Neither pattern above, up to a million elements: an element per thread again (a [45, 1963, 4]
+  // tensor turned to [45, 4, 1963] took 20 us through the tile below, 4 us this way).
+  if (p.count <= (1u << 20)) {
+    MRL_LAUNCH(k_move_rows, dim3(uint32_t((p.count + 255) / 256)), dim3(256), 0, stream, p);
+    return mrl::plan::last_error();
+  }
   // Otherwise a tile grown digit by digit: along the destination's fastest digits until they
   // make a run of 64, along the source's fastest until they do, then along the destination's
   // again while the tile stays within MOVE_TILE_MAX.

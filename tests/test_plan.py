@@ -85,7 +85,9 @@ def test_plans_follow_shape_dtype_and_layout():
     # Softmax by row length and by which dim is scanned.
     assert M.Softmax([64, 100000], 1).plan().kernels == ["k_softmax_chunk_stats", "k_softmax_chunk_write"]
     assert M.Softmax([8192, 8192], 1).plan().kernels == ["k_softmax_block"]
-    assert M.Softmax([2048, 4096], 0).plan().kernels == ["k_softmax_cols"]
+    assert M.Softmax([16, 2048, 2048], 1).plan().kernels == ["k_softmax_cols"]
+    # ... unless that kernel would have too few workgroups: scan dim turned innermost and back.
+    assert M.Softmax([2048, 4096], 0).plan().kernels == ["k_move_tiled32", "k_softmax_regs", "k_move_tiled32"]
     assert M.Softmax([100000, 67], 1).plan().kernels == ["k_softmax_short"]
     # Moves: transpose tiled through LDS, Packed destination gathered, plain copy.
     sq = [4096, 4096]
