@@ -431,7 +431,7 @@ __global__ __launch_bounds__(256) void k_attn_merge(const float *__restrict__ pa
 
 // Key splits for a launch: 1 unless the (entry, query block) pairs fill at most half of the
 // compute units and there are keys enough to share out (four blocks of 64 per workgroup at
-// least).  The workgroups then number at most one per compute unit: measured on 256 units, 256
+// least, and more time saved than the partial results cost).  The workgroups then number at most one per compute unit: measured on 256 units, 256
 // workgroups stream K and V at 4.9-5.6 TB/s where 320 or 512 reach 3.6-4.8.
 uint32_t attn_key_splits(const AttnArgs &a) {
   static const uint64_t units = [] {
@@ -444,7 +444,9 @@ uint32_t attn_key_splits(const AttnArgs &a) {
   const uint64_t groups = uint64_t((a.m + BQ - 1) / BQ) * a.b, blocks = (a.n2 + BKV - 1) / BKV;
   if (groups == 0) return 1;
   const uint64_t splits = std::min<uint64_t>({units / groups, blocks / 4, 256});
-  return splits < 2 ? 1 : uint32_t(splits);
+  // A workgroup spends ~0.5 us per block; the partial results and their merge cost ~4 us.
+  if (splits < 2 || blocks * (splits - 1) <= 8 * splits) return 1;
+  return uint32_t(splits);
 }
 size_t attn_partial_bytes(const AttnArgs &a, uint32_t splits) {
   return splits > 1 ? size_t(a.b) * a.m * splits * (a.k + 4) * sizeof(float) : 0;

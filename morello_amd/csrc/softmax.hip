@@ -93,6 +93,44 @@ __global__ __launch_bounds__(256) void k_softmax_regs(const float *__restrict__ 
   }
 }
 
+// The same for rows that are not whole 16-byte vectors (cols not a multiple of 4, so rows start
+// on any 4 bytes): NE scalars per lane, element i * 64 + lane, cols <= NE * 64.
+template <int NE, bool OUT_BF16>
+__global__ __launch_bounds__(256) void k_softmax_regs1(const float *__restrict__ in, void *__restrict__ out_any,
+                                                       uint64_t rows, uint32_t cols) {
+  const uint64_t row = uint64_t(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const uint32_t lane = threadIdx.x & 63;
+  const float *src = in + row * cols;
+  float v[NE];
+  float mx = F32_MIN;
+  bool nan = false;
+#pragma unroll
+  for (int i = 0; i < NE; i++) {
+    const uint32_t e = i * 64 + lane;
+    v[i] = e < cols ? __builtin_nontemporal_load(src + e) : F32_MIN;
+    nan |= v[i] != v[i];
+    mx = fmaxf(mx, v[i]);
+  }
+  mx = wave_max(mx);
+  if (__any(nan)) mx = __uint_as_float(0x7fc00000u);
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NE; i++) {
+    v[i] = expf(v[i] - mx);
+    sum += uint32_t(i * 64) + lane < cols ? v[i] : 0.0f;
+  }
+  sum = wave_sum(sum);
+#pragma unroll
+  for (int i = 0; i < NE; i++) {
+    const uint32_t e = i * 64 + lane;
+    if (e >= cols) continue;
+    const float y = v[i] / sum;
+    if constexpr (OUT_BF16) (static_cast<uint16_t *>(out_any) + row * cols)[e] = uint16_t(bf16_bits(y));
+    else __builtin_nontemporal_store(y, static_cast<float *>(out_any) + row * cols + e);
+  }
+}
+
 // Any cols: each lane runs the online (max, denom) update over its elements, the lanes'
 // pairs are merged, then the row is read again to write exp(x - max) / denom.
 template <bool OUT_BF16>
@@ -392,10 +430,22 @@ hipError_t launch_rows(const float *in, void *out, uint64_t rows, uint32_t cols,
     if (cols <= 128) return launch_short<16, OUT_BF16>(in, out, rows, cols, stream);
     return launch_short<32, OUT_BF16>(in, out, rows, cols, stream);
   }
-  if (cols > 16 * 256 && cols <= 16 * 1024 && cols % 4 == 0 && rows >= 256 && rows <= 0x7fffffffull) {
+  // A workgroup per row with the row in registers: rows beyond the wavefront kernel's 4096
+  // columns when there are 256 of them or more, and rows of more than 1024 columns when there are
+  // too few of them to occupy the chip a wavefront each.
+  if (cols % 4 == 0 && rows <= 0x7fffffffull &&
+      ((cols > 16 * 256 && cols <= 16 * 1024 && rows >= 256) || (cols > 1024 && cols <= 16 * 256 && rows < 2048))) {
     plan::work(plan::UNIT_STREAM, 0, double(rows) * cols * (4 + (OUT_BF16 ? 2 : 4)));
     if (cols <= 8 * 1024) MRL_LAUNCH((k_softmax_block<8, OUT_BF16>), dim3(uint32_t(rows)), dim3(256), 0, stream, in, out, cols);
     else MRL_LAUNCH((k_softmax_block<16, OUT_BF16>), dim3(uint32_t(rows)), dim3(256), 0, stream, in, out, cols);
+    return mrl::plan::last_error();
+  }
+  if (cols % 4 != 0 && cols <= 64 * 64 && rows >= 512 && (rows + 3) / 4 <= 0x7fffffffull) {
+    const dim3 grid{uint32_t((rows + 3) / 4)}, block{256};
+    plan::work(plan::UNIT_STREAM, 0, double(rows) * cols * (4 + (OUT_BF16 ? 2 : 4)));
+    if (cols <= 16 * 64) MRL_LAUNCH((k_softmax_regs1<16, OUT_BF16>), grid, block, 0, stream, in, out, rows, cols);
+    else if (cols <= 32 * 64) MRL_LAUNCH((k_softmax_regs1<32, OUT_BF16>), grid, block, 0, stream, in, out, rows, cols);
+    else MRL_LAUNCH((k_softmax_regs1<64, OUT_BF16>), grid, block, 0, stream, in, out, rows, cols);
     return mrl::plan::last_error();
   }
   if (scratch && softmax_scratch_bytes(rows, cols)) {
@@ -422,10 +472,9 @@ hipError_t launch_rows(const float *in, void *out, uint64_t rows, uint32_t cols,
 
 // Scratch the chunked kernels want for this shape (0: the shape runs without).
 size_t softmax_scratch_bytes(uint64_t rows, uint32_t cols) {
-  // Up to 4096 columns the register kernel serves (a multiple of 4), or one wavefront per row
-  // when the rows are many or short; fewer, longer rows that are not whole vectors go in chunks
-  // too (a single one), with scalar loads: a wavefront's loop over such a row is all latency.
-  if (cols <= 16 * 256 && (cols % 4 == 0 || cols <= 256 || rows >= 4096)) return 0;
+  // Up to 4096 columns the register kernels serve; fewer than 512 rows that are not whole
+  // vectors go in chunks too (a single one), with scalar loads.
+  if (cols <= 16 * 256 && (cols % 4 == 0 || cols <= 256 || rows >= 512)) return 0;
   const uint64_t chunks = (cols + SOFTMAX_CHUNK - 1) / SOFTMAX_CHUNK;
   if (rows * chunks > 0x7fffffffull) return 0;
   return size_t(rows * chunks * sizeof(float2));
