@@ -485,11 +485,14 @@ __device__ inline uint32_t div_small(uint32_t n, uint32_t d, uint32_t inv) {
 // V: elements per thread and step, a run along the fastest digit of the side being walked (the
 // host picks V > 1 only when those digits, their tile extents and their sizes are multiples of
 // V): one digit extraction serves V elements.
-template <class E, int V>
+// NACT: the digits along which the tile extends come first (the host orders them so) and number
+// at most NACT; the per-element digit loops run over exactly those, unrolled, with no test of
+// which digits matter.
+template <class E, int V, int NACT>
 __global__ __launch_bounds__(256) void k_move_gather(MoveTile p) {
   constexpr bool CONVERT = std::is_void<E>::value;
   typedef typename std::conditional<CONVERT, uint32_t, E>::type Cell;
-  static_assert(V == 1 || (!CONVERT && sizeof(Cell) == 4), "runs are for 4-byte elements");
+  static_assert(V == 1 || !CONVERT, "runs are for elements that are not converted");
   typedef Cell Run __attribute__((ext_vector_type(V == 1 ? 2 : V)));  // used only when V > 1
   __shared__ Cell lds[MOVE_TILE_MAX + MOVE_TILE_MAX / 64];
   uint64_t blk = blockIdx.x;
@@ -510,13 +513,12 @@ __global__ __launch_bounds__(256) void k_move_gather(MoveTile p) {
     uint32_t so = 0;
     bool inside = true;
 #pragma unroll
-    for (uint32_t d = 0; d < MOVE_MAX_RANK; d++)
-      if (d < p.m.rank && p.ext[d] > 1) {
-        const uint32_t q = div_small(t, p.tstride_s[d], p.inv_s[d]);
-        const uint32_t c = q - div_small(q, p.ext[d], p.inv_ext[d]) * p.ext[d];
-        inside = inside && c < room[d];
-        so += c * uint32_t(p.m.ss[d]);
-      }
+    for (uint32_t d = 0; d < uint32_t(NACT); d++) {
+      const uint32_t q = div_small(t, p.tstride_s[d], p.inv_s[d]);
+      const uint32_t c = q - div_small(q, p.ext[d], p.inv_ext[d]) * p.ext[d];
+      inside = inside && c < room[d];
+      so += c * uint32_t(p.m.ss[d]);
+    }
     if (inside) {
       if constexpr (CONVERT) {
         lds[t + t / 64] = move_bits(p.m.src, p.m.sdt, base_s + so, p.m.ddt);
@@ -540,14 +542,13 @@ __global__ __launch_bounds__(256) void k_move_gather(MoveTile p) {
     uint32_t d_o = 0, at = 0;
     bool inside = true;
 #pragma unroll
-    for (uint32_t d = 0; d < MOVE_MAX_RANK; d++)
-      if (d < p.m.rank && p.ext[d] > 1) {
-        const uint32_t q = div_small(t, p.tstride_d[d], p.inv_d[d]);
-        const uint32_t c = q - div_small(q, p.ext[d], p.inv_ext[d]) * p.ext[d];
-        inside = inside && c < room[d];
-        d_o += c * uint32_t(p.m.ds[d]);
-        at += c * p.tstride_s[d];
-      }
+    for (uint32_t d = 0; d < uint32_t(NACT); d++) {
+      const uint32_t q = div_small(t, p.tstride_d[d], p.inv_d[d]);
+      const uint32_t c = q - div_small(q, p.ext[d], p.inv_ext[d]) * p.ext[d];
+      inside = inside && c < room[d];
+      d_o += c * uint32_t(p.m.ds[d]);
+      at += c * p.tstride_s[d];
+    }
     if (inside) {
       if constexpr (CONVERT) {
         store_u32(p.m.dst, p.m.ddt, base_d + d_o, lds[at + at / 64]);
@@ -1114,6 +1115,14 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
   grow(by_ds, 64, MOVE_TILE_MAX / 64);
   grow(by_ss, 64, MOVE_TILE_MAX);
   grow(by_ds, MOVE_TILE_MAX, MOVE_TILE_MAX);
+  // The runs are as long as they get; a tile still far below the cap (a digit covered in part
+  // ends the growth above: 4 of 6 strips of an OddEven(16) dim left a tile of 64 elements, 20000
+  // workgroups for 5 MB) is filled along whatever digits have room, more runs per workgroup.
+  for (uint32_t i = 0; i < rank && tile < MOVE_TILE_MAX; i++) {
+    const uint32_t d = by_ds[i];
+    const uint32_t grown = std::min<uint32_t>(p.shape[d], uint32_t(uint64_t(t.ext[d]) * (MOVE_TILE_MAX / tile)));
+    if (grown > t.ext[d]) tile = tile / t.ext[d] * grown, t.ext[d] = grown;
+  }
   t.tile = tile;
   uint64_t blocks = 1;
   uint32_t stride_s = 1, stride_d = 1;
@@ -1131,25 +1140,54 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
   if (blocks > 0x7fffffffull || tile > MOVE_TILE_MAX) return hipErrorInvalidValue;
   const dim3 grid{uint32_t(blocks)};
   const size_t elem = mrl_dtype_size(src_dtype);
-  // Runs of 4 or 2 elements per thread where both sides' fastest digits allow.
+  // Runs of 4 or 2 elements per thread (any element size) where both sides' fastest digits allow.
   const uint32_t fs = by_ss[0], fd = by_ds[0];
   uint32_t run = 1;
-  if (src_dtype == dst_dtype && elem == 4 && p.ss[fs] == 1 && p.ds[fd] == 1)
+  if (src_dtype == dst_dtype && p.ss[fs] == 1 && p.ds[fd] == 1)
     for (uint32_t v : {4u, 2u})
       if (run == 1 && t.ext[fs] % v == 0 && p.shape[fs] % v == 0 && t.ext[fd] % v == 0 && p.shape[fd] % v == 0) run = v;
   t.lds_step = t.tstride_s[fd];
-  t.vec_s = (reinterpret_cast<uintptr_t>(src) % (4 * run)) == 0;
-  t.vec_d = (reinterpret_cast<uintptr_t>(dst) % (4 * run)) == 0;
+  if (elem == 1 && run == 2) run = 1;  // bytes travel in fours or alone
+  t.vec_s = (reinterpret_cast<uintptr_t>(src) % (elem * run)) == 0;
+  t.vec_d = (reinterpret_cast<uintptr_t>(dst) % (elem * run)) == 0;
   for (uint32_t d = 0; d < rank; d++) {
     if (d != fs && p.ss[d] % run != 0) t.vec_s = false;
     if (d != fd && p.ds[d] % run != 0) t.vec_d = false;
   }
-  if (src_dtype != dst_dtype) MRL_LAUNCH((k_move_gather<void, 1>), grid, dim3(256), 0, stream, t);
-  else if (elem == 4 && run == 4) MRL_LAUNCH((k_move_gather<uint32_t, 4>), grid, dim3(256), 0, stream, t);
-  else if (elem == 4 && run == 2) MRL_LAUNCH((k_move_gather<uint32_t, 2>), grid, dim3(256), 0, stream, t);
-  else if (elem == 4) MRL_LAUNCH((k_move_gather<uint32_t, 1>), grid, dim3(256), 0, stream, t);
-  else if (elem == 2) MRL_LAUNCH((k_move_gather<uint16_t, 1>), grid, dim3(256), 0, stream, t);
-  else MRL_LAUNCH((k_move_gather<uint8_t, 1>), grid, dim3(256), 0, stream, t);
+  // Digits the tile extends along first (any order of the digits serves the kernel, as long as
+  // every per-digit array follows it).
+  uint32_t perm[MOVE_MAX_RANK], n_act = 0, n_rest = 0;
+  for (uint32_t d = 0; d < MOVE_MAX_RANK; d++)
+    if (t.ext[d] > 1) perm[n_act++] = d;
+  for (uint32_t d = 0; d < MOVE_MAX_RANK; d++)
+    if (t.ext[d] <= 1) perm[n_act + n_rest++] = d;
+  {
+    const MoveTile o = t;
+    for (uint32_t i = 0; i < MOVE_MAX_RANK; i++) {
+      const uint32_t d = perm[i];
+      t.m.shape[i] = o.m.shape[d], t.m.ss[i] = o.m.ss[d], t.m.ds[i] = o.m.ds[d];
+      t.ext[i] = o.ext[d], t.chunks[i] = o.chunks[d];
+      t.tstride_s[i] = o.tstride_s[d], t.tstride_d[i] = o.tstride_d[d];
+      t.inv_s[i] = o.inv_s[d], t.inv_d[i] = o.inv_d[d], t.inv_ext[i] = o.inv_ext[d];
+    }
+    t.m.rank = MOVE_MAX_RANK;  // size-one digits fill the tail: shape 1, one chunk
+  }
+#define MRL_GATHER(E, V)                                                                              \
+  do {                                                                                                \
+    if (n_act <= 3) MRL_LAUNCH((k_move_gather<E, V, 3>), grid, dim3(256), 0, stream, t);              \
+    else if (n_act <= 5) MRL_LAUNCH((k_move_gather<E, V, 5>), grid, dim3(256), 0, stream, t);         \
+    else MRL_LAUNCH((k_move_gather<E, V, int(MOVE_MAX_RANK)>), grid, dim3(256), 0, stream, t);        \
+  } while (0)
+  if (src_dtype != dst_dtype) MRL_GATHER(void, 1);
+  else if (elem == 4 && run == 4) MRL_GATHER(uint32_t, 4);
+  else if (elem == 4 && run == 2) MRL_GATHER(uint32_t, 2);
+  else if (elem == 4) MRL_GATHER(uint32_t, 1);
+  else if (elem == 2 && run == 4) MRL_GATHER(uint16_t, 4);
+  else if (elem == 2 && run == 2) MRL_GATHER(uint16_t, 2);
+  else if (elem == 2) MRL_GATHER(uint16_t, 1);
+  else if (run == 4) MRL_GATHER(uint8_t, 4);
+  else MRL_GATHER(uint8_t, 1);
+#undef MRL_GATHER
   return mrl::plan::last_error();
 }
 
