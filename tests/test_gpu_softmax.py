@@ -140,7 +140,11 @@ def test_compose_msm(gpu, dims):
 
 
 @pytest.mark.parametrize("dims", [(2, 200, 160, 328, 160), (1, 136, 136, 1000, 96), (2, 256, 192, 192, 72),
-                                  (1, 512, 256, 1024, 256)])
+                                  (1, 512, 256, 1024, 256),
+                                  # every Softmax kernel that writes P as bf16: rows that are not whole
+                                  # vectors (many, few), a workgroup per row, short rows, rows in chunks
+                                  (1, 600, 160, 1001, 160), (1, 100, 160, 1001, 160), (1, 300, 160, 2048, 160),
+                                  (2, 130, 160, 67, 160), (1, 40, 160, 9000, 160)])
 def test_compose_msm_staged_on_the_matrix_cores(gpu, dims):
     """Head dims beyond 128, which the fused kernel does not take: Q.KT runs as a bf16 Matmul with
     a k-fastest B, Softmax over f32 rows writes P rounded to bf16 (as the fused kernel does), and
@@ -157,7 +161,9 @@ def test_compose_msm_staged_on_the_matrix_cores(gpu, dims):
                                  M.Matmul([b, m, k, n2], [M.bf16, M.bf16, M.f32])],
                                 layouts=[None, None, KT_LAYOUT, None]).bufferize(0),
                       [v, q, kmat, np.zeros((b, m, n), np.float32)])
-    assert rel_err(staged, want) < 1e-5
+    # Sums of 9000 f32 terms: the oracle adds them one after another, the kernels in trees; the two
+    # associations differ by more than 1e-5 of the largest output at that length.
+    assert rel_err(staged, want) < (1e-5 if n2 <= 4096 else 5e-5)
 
 
 @pytest.mark.parametrize("dims", [(1, 136, 128, 1000, 128), (2, 1, 128, 1, 128), (1, 130, 128, 64, 128),
