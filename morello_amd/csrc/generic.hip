@@ -124,6 +124,20 @@ __device__ inline uint32_t move_bits(const void *src, int sdt, int64_t so, int d
   return load_u32(src, sdt, so, MRL_U32);  // int -> int wraps
 }
 
+// An element's bits, zero-extended, by element size alone (no dtype switch around the load).
+template <int SIZE>
+__device__ inline uint32_t load_sized(const void *p, int64_t off) {
+  if constexpr (SIZE == 1) return static_cast<const uint8_t *>(p)[off];
+  else if constexpr (SIZE == 2) return static_cast<const uint16_t *>(p)[off];
+  else return static_cast<const uint32_t *>(p)[off];
+}
+template <int SIZE>
+__device__ inline void store_sized(void *p, int64_t off, uint32_t v) {
+  if constexpr (SIZE == 1) static_cast<uint8_t *>(p)[off] = uint8_t(v);
+  else if constexpr (SIZE == 2) static_cast<uint16_t *>(p)[off] = uint16_t(v);
+  else static_cast<uint32_t *>(p)[off] = v;
+}
+
 // The same conversions on an element already in a register (`raw`: its bits, zero-extended).
 __device__ inline float raw_to_f32(uint32_t raw, int dtype) {
   switch (dtype) {
@@ -237,6 +251,7 @@ __global__ __launch_bounds__(256) void k_move_rows16(MoveStrided p) {
 // The two sides are contiguous along different dims: a 64 x 64 tile of (dim_d, dim_s) goes
 // through LDS, read with dim_s fastest and written with dim_d fastest, so both sides see
 // whole contiguous runs (move_relayout of morello/src/scheduling/moves.rs as a transpose).
+template <int SE, int DE>
 __global__ __launch_bounds__(256) void k_move_tiled(MoveStrided p) {
   __shared__ uint32_t tile[64][65];
   uint64_t blk = blockIdx.x;
@@ -266,16 +281,18 @@ __global__ __launch_bounds__(256) void k_move_tiled(MoveStrided p) {
     const uint32_t r = quad + 4 * i;
     v[i] = 0;
     if (d0 + r < nd && s0 + lane < ns)
-      v[i] = move_bits(p.src, p.sdt, so + int64_t(d0 + r) * p.ss[p.dim_d] + int64_t(s0 + lane) * p.ss[p.dim_s], p.ddt);
+      v[i] = load_sized<SE>(p.src, so + int64_t(d0 + r) * p.ss[p.dim_d] + int64_t(s0 + lane) * p.ss[p.dim_s]);
   }
+  // The conversion is arithmetic on registers, after the loads: a dtype switch around each load
+  // would put a branch between any two of them.
 #pragma unroll
-  for (uint32_t i = 0; i < 16; i++) tile[quad + 4 * i][lane] = v[i];
+  for (uint32_t i = 0; i < 16; i++) tile[quad + 4 * i][lane] = convert_raw(v[i], p.sdt, p.ddt);
   __syncthreads();
 #pragma unroll
   for (uint32_t i = 0; i < 16; i++) {
     const uint32_t r = quad + 4 * i;
     if (s0 + r < ns && d0 + lane < nd)
-      store_u32(p.dst, p.ddt, d_o + int64_t(s0 + r) * p.ds[p.dim_s] + int64_t(d0 + lane) * p.ds[p.dim_d], tile[lane][r]);
+      store_sized<DE>(p.dst, d_o + int64_t(s0 + r) * p.ds[p.dim_s] + int64_t(d0 + lane) * p.ds[p.dim_d], tile[lane][r]);
   }
 }
 
@@ -488,7 +505,8 @@ __device__ inline uint32_t div_small(uint32_t n, uint32_t d, uint32_t inv) {
 // NACT: the digits along which the tile extends come first (the host orders them so) and number
 // at most NACT; the per-element digit loops run over exactly those, unrolled, with no test of
 // which digits matter.
-template <class E, int V, int NACT>
+// E void: elements are converted, SSIZE and DSIZE their sizes in bytes on the two sides.
+template <class E, int V, int NACT, int SSIZE = 0, int DSIZE = 0>
 __global__ __launch_bounds__(256) void k_move_gather(MoveTile p) {
   constexpr bool CONVERT = std::is_void<E>::value;
   typedef typename std::conditional<CONVERT, uint32_t, E>::type Cell;
@@ -521,7 +539,7 @@ __global__ __launch_bounds__(256) void k_move_gather(MoveTile p) {
     }
     if (inside) {
       if constexpr (CONVERT) {
-        lds[t + t / 64] = move_bits(p.m.src, p.m.sdt, base_s + so, p.m.ddt);
+        lds[t + t / 64] = load_sized<SSIZE ? SSIZE : 4>(p.m.src, base_s + so);
       } else if constexpr (V == 1) {
         lds[t + t / 64] = static_cast<const E *>(p.m.src)[base_s + so];
       } else {
@@ -551,7 +569,8 @@ __global__ __launch_bounds__(256) void k_move_gather(MoveTile p) {
     }
     if (inside) {
       if constexpr (CONVERT) {
-        store_u32(p.m.dst, p.m.ddt, base_d + d_o, lds[at + at / 64]);
+        const uint32_t v = convert_raw(lds[at + at / 64], p.m.sdt, p.m.ddt);
+        store_sized<DSIZE ? DSIZE : 4>(p.m.dst, base_d + d_o, v);
       } else if constexpr (V == 1) {
         static_cast<E *>(p.m.dst)[base_d + d_o] = lds[at + at / 64];
       } else {
@@ -1077,7 +1096,15 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
     if (octets) MRL_LAUNCH(k_move_tiled16v, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
     else if (pairs) MRL_LAUNCH(k_move_tiled16, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
     else if (quads) MRL_LAUNCH(k_move_tiled32, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
-    else if (src_dtype != dst_dtype) MRL_LAUNCH(k_move_tiled, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+    else if (src_dtype != dst_dtype) {
+      const int se = int(mrl_dtype_size(src_dtype)), de = int(mrl_dtype_size(dst_dtype));
+#define MRL_TILED(SE, DE) \
+  if (se == SE && de == DE) MRL_LAUNCH((k_move_tiled<SE, DE>), dim3(uint32_t(blocks)), dim3(256), 0, stream, p)
+      MRL_TILED(1, 1); MRL_TILED(1, 2); MRL_TILED(1, 4);
+      MRL_TILED(2, 1); MRL_TILED(2, 2); MRL_TILED(2, 4);
+      MRL_TILED(4, 1); MRL_TILED(4, 2); MRL_TILED(4, 4);
+#undef MRL_TILED
+    }
     else if (mrl_dtype_size(src_dtype) == 1) MRL_LAUNCH(k_move_tiled_as<uint8_t>, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
     else if (mrl_dtype_size(src_dtype) == 2) MRL_LAUNCH(k_move_tiled_as<uint16_t>, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
     else MRL_LAUNCH(k_move_tiled_as<uint32_t>, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
@@ -1178,7 +1205,18 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
     else if (n_act <= 5) MRL_LAUNCH((k_move_gather<E, V, 5>), grid, dim3(256), 0, stream, t);         \
     else MRL_LAUNCH((k_move_gather<E, V, int(MOVE_MAX_RANK)>), grid, dim3(256), 0, stream, t);        \
   } while (0)
-  if (src_dtype != dst_dtype) MRL_GATHER(void, 1);
+  if (src_dtype != dst_dtype) {
+    const int se = int(elem), de = int(mrl_dtype_size(dst_dtype));
+#define MRL_GATHER_CV(SE, DE)                                                                                      \
+  if (se == SE && de == DE) {                                                                                      \
+    if (n_act <= 5) MRL_LAUNCH((k_move_gather<void, 1, 5, SE, DE>), grid, dim3(256), 0, stream, t);                \
+    else MRL_LAUNCH((k_move_gather<void, 1, int(MOVE_MAX_RANK), SE, DE>), grid, dim3(256), 0, stream, t);          \
+  }
+    MRL_GATHER_CV(1, 1) MRL_GATHER_CV(1, 2) MRL_GATHER_CV(1, 4)
+    MRL_GATHER_CV(2, 1) MRL_GATHER_CV(2, 2) MRL_GATHER_CV(2, 4)
+    MRL_GATHER_CV(4, 1) MRL_GATHER_CV(4, 2) MRL_GATHER_CV(4, 4)
+#undef MRL_GATHER_CV
+  }
   else if (elem == 4 && run == 4) MRL_GATHER(uint32_t, 4);
   else if (elem == 4 && run == 2) MRL_GATHER(uint32_t, 2);
   else if (elem == 4) MRL_GATHER(uint32_t, 1);
