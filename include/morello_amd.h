@@ -406,6 +406,10 @@ int mrl_spec_plan(const mrl_spec *spec, mrl_plan *plan, mrl_plan_step *steps, ui
  * tile_out / split (scheduling_sugar.rs:37-132) compares. */
 int mrl_matmul_scheduled_plan(const mrl_spec *spec, const mrl_matmul_schedule *schedule, mrl_plan *plan,
                               mrl_plan_step *steps, uint32_t cap);
+/* The smallest search there is: the manual schedule of lowest predicted cost among those the
+ * kernel is built for (what morello's top-down search does over its actions, search.rs, with
+ * this backend's cost model in place of cost.rs).  MRL_ERR_UNSUPPORTED when none applies. */
+int mrl_matmul_search_schedule(const mrl_spec *spec, mrl_matmul_schedule *best, double *cost_ns);
 /* The same for a general Compose. */
 int mrl_compose_plan(const mrl_compose *c, mrl_plan *plan, mrl_plan_step *steps, uint32_t cap);
 

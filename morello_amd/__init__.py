@@ -304,6 +304,13 @@ class Spec:
         n = B.load().mrl_matmul_schedules(C.byref(self._c), buf, 16)
         return [(buf[i].tile_m, buf[i].tile_n, buf[i].split_k) for i in range(min(n, 16))]
 
+    def search_schedule(self) -> "ScheduledMatmul":
+        """The manual schedule the cost model predicts cheapest (host only)."""
+        sched, cost = B.MatmulScheduleC(), C.c_double()
+        _check(B.load().mrl_matmul_search_schedule(C.byref(self._c), C.byref(sched), C.byref(cost)),
+               "mrl_matmul_search_schedule")
+        return ScheduledMatmul(self, sched.tile_m, sched.tile_n, sched.split_k)
+
     def tile_out(self, tile_shape: Sequence[int]) -> "ScheduledMatmul":
         """`spec.tile_out([1, m, n])`: one workgroup per m x n tile of the output."""
         if self.kind != SpecKind.Matmul or len(tile_shape) != 3 or tile_shape[0] != 1:

@@ -140,6 +140,7 @@ SIGNATURES = {
     "mrl_spec_plan": (C.c_int, [C.POINTER(SpecC), C.POINTER(PlanC), C.POINTER(PlanStepC), C.c_uint32]),
     "mrl_matmul_scheduled_plan": (C.c_int, [C.POINTER(SpecC), C.POINTER(MatmulScheduleC), C.POINTER(PlanC),
                                             C.POINTER(PlanStepC), C.c_uint32]),
+    "mrl_matmul_search_schedule": (C.c_int, [C.POINTER(SpecC), C.POINTER(MatmulScheduleC), C.POINTER(C.c_double)]),
     "mrl_compose_plan": (C.c_int, [C.POINTER(ComposeC), C.POINTER(PlanC), C.POINTER(PlanStepC), C.c_uint32]),
     "mrl_device_info": (C.c_int, [C.c_char_p, C.c_size_t, C.POINTER(C.c_int), C.POINTER(C.c_int),
                                   C.POINTER(C.c_size_t)]),

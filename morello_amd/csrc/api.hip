@@ -1533,6 +1533,23 @@ int mrl_matmul_scheduled_plan(const mrl_spec *spec, const mrl_matmul_schedule *s
                    [&](void *const *params, Workspace &ws) { return run_matmul(*spec, params, ws, schedule); });
 }
 
+int mrl_matmul_search_schedule(const mrl_spec *spec, mrl_matmul_schedule *best, double *cost_ns) {
+  if (!best) return MRL_ERR_NULL;
+  mrl_matmul_schedule all[16];
+  const uint32_t n = mrl_matmul_schedules(spec, all, 16);
+  if (n == 0) return MRL_ERR_UNSUPPORTED;
+  double lowest = 0;
+  bool found = false;
+  for (uint32_t i = 0; i < n && i < 16; i++) {
+    mrl_plan plan;
+    if (mrl_matmul_scheduled_plan(spec, &all[i], &plan, nullptr, 0) != MRL_OK) continue;  // not for this shape
+    if (!found || plan.cost_ns < lowest) lowest = plan.cost_ns, *best = all[i], found = true;
+  }
+  if (!found) return MRL_ERR_UNSUPPORTED;
+  if (cost_ns) *cost_ns = lowest;
+  return MRL_OK;
+}
+
 int mrl_bench(const mrl_spec *spec, void *const *params, uint32_t iters, uint32_t repeats,
               double *best_ns_per_iter, double *mean_ns_per_iter) {
   if (!best_ns_per_iter || !mean_ns_per_iter) return MRL_ERR_NULL;

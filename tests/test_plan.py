@@ -170,6 +170,19 @@ def test_every_manual_schedule_has_its_plan():
     assert min(costs, key=costs.get)[0] < 256
 
 
+def test_schedule_search_returns_the_cheapest_plan():
+    for dts, n in (((M.u8, M.i8, M.i32), 1024), ((M.bf16, M.bf16, M.f32), 4096), ((M.f32, M.f32, M.f32), 512)):
+        spec = M.Matmul([1, n, n, n], dts)
+        found = spec.search_schedule()
+        costs = {s: spec.tile_out([1, s[0], s[1]]).split(s[2]).plan().cost_ns for s in spec.available_schedules()}
+        assert (found.tile_m, found.tile_n, found.split_k) in costs
+        assert found.plan().cost_ns == min(costs.values())
+    assert M.Matmul([1, 4096, 4096, 4096], (M.u8, M.i8, M.i32)).search_schedule().tile_m == 256
+    assert M.Matmul([1, 512, 1024, 512], (M.u8, M.i8, M.i32)).search_schedule().tile_m == 64
+    with pytest.raises(M.MorelloError):
+        M.Matmul([1, 64, 64, 64], (M.i16, M.i16, M.i32)).search_schedule()   # no matrix-core form
+
+
 def test_plan_errors_are_the_run_errors():
     import ctypes as C
     from morello_amd import _binding as B
