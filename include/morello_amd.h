@@ -377,6 +377,19 @@ typedef struct {
 /* Writes up to `cap` levels; returns how many there are (4, the reference's MEMORY_COUNT). */
 uint32_t mrl_target_memories(mrl_target_memory *out, uint32_t cap);
 
+/* Target::default_memory (target/mod.rs:54): index into mrl_target_memories of the level Spec
+ * parameters live in (HBM). */
+uint32_t mrl_target_default_memory(void);
+/* Target::possible_destination_memories (target/mod.rs:56): where a Move out of level `slower`
+ * may land, itself first; returns the count. */
+uint32_t mrl_target_destination_memories(uint32_t slower, uint32_t *out, uint32_t cap);
+/* Target::all_layouts_for_shape / move_destination_layouts (target/mod.rs:58-67), built as the
+ * reference's CPU targets build theirs (target/cpu.rs:317-398): row-major, plus column-major
+ * (rank 2), k-fastest `layout![0,2,1]` (rank 3; read in place by the Matmul and Compose kernels)
+ * or NHWC (rank 4); each of those with one more Packed(n) dim for n = 2 and the register file's
+ * vector widths in elements, and with one more OddEven(n) dim for twice those widths, wherever
+ * the result applies to `shape`.  Writes up to `cap` layouts, returns how many there are. */
+uint32_t mrl_target_layouts_for_shape(const uint32_t *shape, uint32_t rank, int dtype, mrl_layout *out, uint32_t cap);
 /* Kernel::name of every kernel family of the backend (target/mod.rs:111); returns the count. */
 uint32_t mrl_target_kernels(const char **names, uint32_t cap);
 

@@ -600,6 +600,27 @@ class Target:
         return [TargetMemory(buf[i]) for i in range(n)]
 
     @staticmethod
+    def default_memory() -> "TargetMemory":
+        return Target.memories()[B.load().mrl_target_default_memory()]
+
+    @staticmethod
+    def possible_destination_memories(slower: str):
+        names = [m.name for m in Target.memories()]
+        buf = (C.c_uint32 * 4)()
+        n = B.load().mrl_target_destination_memories(names.index(slower), buf, 4)
+        return [names[buf[i]] for i in range(n)]
+
+    @staticmethod
+    def all_layouts_for_shape(shape: Sequence[int], dtype: "Dtype"):
+        arr = (C.c_uint32 * len(shape))(*shape)
+        n = B.load().mrl_target_layouts_for_shape(arr, len(shape), int(dtype), None, 0)
+        buf = (B.LayoutC * n)()
+        B.load().mrl_target_layouts_for_shape(arr, len(shape), int(dtype), buf, n)
+        return [Layout.from_c(buf[i]) for i in range(n)]
+
+    move_destination_layouts = all_layouts_for_shape
+
+    @staticmethod
     def kernels():
         buf = (C.c_char_p * 64)()
         n = B.load().mrl_target_kernels(buf, 64)

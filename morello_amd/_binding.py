@@ -136,6 +136,10 @@ SIGNATURES = {
     "mrl_target_line_size": (C.c_uint32, []),
     "mrl_target_processors": (C.c_uint32, []),
     "mrl_target_memories": (C.c_uint32, [C.POINTER(TargetMemoryC), C.c_uint32]),
+    "mrl_target_default_memory": (C.c_uint32, []),
+    "mrl_target_destination_memories": (C.c_uint32, [C.c_uint32, C.POINTER(C.c_uint32), C.c_uint32]),
+    "mrl_target_layouts_for_shape": (C.c_uint32, [C.POINTER(C.c_uint32), C.c_uint32, C.c_int, C.POINTER(LayoutC),
+                                                  C.c_uint32]),
     "mrl_target_kernels": (C.c_uint32, [C.POINTER(C.c_char_p), C.c_uint32]),
     "mrl_spec_plan": (C.c_int, [C.POINTER(SpecC), C.POINTER(PlanC), C.POINTER(PlanStepC), C.c_uint32]),
     "mrl_matmul_scheduled_plan": (C.c_int, [C.POINTER(SpecC), C.POINTER(MatmulScheduleC), C.POINTER(PlanC),

@@ -1336,6 +1336,83 @@ uint32_t mrl_target_memories(mrl_target_memory *out, uint32_t cap) {
   return 4;
 }
 
+uint32_t mrl_target_default_memory(void) { return 3; }
+
+uint32_t mrl_target_destination_memories(uint32_t slower, uint32_t *out, uint32_t cap) {
+  // HBM feeds LDS (global_load ... lds) and registers directly; LDS feeds registers; the MFMA
+  // accumulators are initialised from and drained to VGPRs.
+  static const uint32_t table[4][3] = {{0, 0, 0}, {1, 0, 0}, {2, 1, 0}, {3, 2, 1}};
+  static const uint32_t counts[4] = {1, 2, 2, 3};
+  if (slower > 3) return 0;
+  for (uint32_t i = 0; i < counts[slower] && i < cap && out; i++) out[i] = table[slower][i];
+  return counts[slower];
+}
+
+uint32_t mrl_target_layouts_for_shape(const uint32_t *shape, uint32_t rank, int dtype, mrl_layout *out, uint32_t cap) {
+  if (!shape || rank == 0 || rank > MRL_MAX_RANK || mrl_dtype_size(dtype) == 0) return 0;
+  const uint32_t es = uint32_t(mrl_dtype_size(dtype));
+  std::vector<mrl_layout> base(1), result;
+  mrl_layout_row_major(shape, rank, &base[0]);
+  bool only_ones = true;
+  for (uint32_t d = 0; d < rank; d++) only_ones = only_ones && shape[d] == 1;
+  auto same = [](const mrl_layout &a, const mrl_layout &b) {
+    if (a.ndims != b.ndims) return false;
+    for (uint32_t i = 0; i < a.ndims; i++)
+      if (a.dims[i].logical_dim != b.dims[i].logical_dim || a.dims[i].kind != b.dims[i].kind ||
+          a.dims[i].size != b.dims[i].size)
+        return false;
+    return true;
+  };
+  if (!only_ones && (rank == 2 || rank == 3 || rank == 4)) {
+    mrl_layout other;
+    const int rc = rank == 2   ? mrl_layout_col_major(shape, rank, &other)
+                   : rank == 3 ? mrl_layout_batched_col_major(shape, rank, &other)
+                               : mrl_layout_nhwc(shape, rank, &other);
+    if (rc == MRL_OK && !same(other, base[0])) base.push_back(other);
+  }
+  result = base;
+  // Vector widths of the register file in elements, and 2 (pack_sizes_all, target/cpu.rs:2894-2906);
+  // twice the widths for OddEven (oddeven_sizes_all, target/cpu.rs:2935-2947).
+  std::vector<uint32_t> pack{2}, oddeven;
+  for (uint32_t bytes : {4u, 8u, 16u}) {
+    if (bytes % es == 0 && bytes / es > 1 && std::find(pack.begin(), pack.end(), bytes / es) == pack.end())
+      pack.push_back(bytes / es);
+    if ((2 * bytes) % es == 0 && 2 * bytes / es > 1 &&
+        std::find(oddeven.begin(), oddeven.end(), 2 * bytes / es) == oddeven.end())
+      oddeven.push_back(2 * bytes / es);
+  }
+  auto extend = [&](const mrl_layout &from, uint32_t dim, uint8_t kind, uint32_t size) {
+    if (from.ndims >= MRL_MAX_PHYS) return;
+    mrl_layout l = from;
+    l.dims[l.ndims].logical_dim = uint8_t(dim), l.dims[l.ndims].kind = kind, l.dims[l.ndims].size = size;
+    l.ndims++;
+    uint32_t phys[MRL_MAX_PHYS];
+    if (!mrl::physical_shape(l, shape, rank, phys)) return;  // does not apply to this shape
+    for (const mrl_layout &have : result)
+      if (same(have, l)) return;
+    result.push_back(l);
+  };
+  for (const mrl_layout &b : base) {
+    std::vector<uint32_t> dims;
+    for (uint32_t i = 0; i < b.ndims; i++)
+      if (std::find(dims.begin(), dims.end(), b.dims[i].logical_dim) == dims.end()) dims.push_back(b.dims[i].logical_dim);
+    const uint32_t innermost = b.dims[b.ndims - 1].logical_dim;
+    for (uint32_t d : dims)
+      for (uint32_t size : pack)
+        if (d != innermost && shape[d] % size == 0) extend(b, d, MRL_PACKED, size);
+  }
+  for (const mrl_layout &b : base) {
+    std::vector<uint32_t> dims;
+    for (uint32_t i = 0; i < b.ndims; i++)
+      if (std::find(dims.begin(), dims.end(), b.dims[i].logical_dim) == dims.end()) dims.push_back(b.dims[i].logical_dim);
+    for (uint32_t d : dims)
+      for (uint32_t size : oddeven)
+        if (shape[d] % size == 0) extend(b, d, MRL_ODDEVEN, size);
+  }
+  for (uint32_t i = 0; i < result.size() && i < cap && out; i++) out[i] = result[i];
+  return uint32_t(result.size());
+}
+
 uint32_t mrl_target_kernels(const char **names, uint32_t cap) {
   static const char *const families[] = {
       "k_gemm", "k_gemv", "k_matmul_generic", "k_sum_splits", "k_conv_i8", "k_conv_generic", "k_conv_generic_wave", "k_unfold",

@@ -36,6 +36,36 @@ def test_target_description():
     assert len(kernels) == len(set(kernels)) and {"k_gemm", "k_conv_i8", "k_attn", "k_softmax_regs"} <= set(kernels)
 
 
+def test_target_memories_and_layouts_for_search():
+    """Target::default_memory, possible_destination_memories, all_layouts_for_shape
+    (target/mod.rs:54-67), the last built as target/cpu.rs:317-398 builds it."""
+    T = M.Target
+    assert T.default_memory().name == "HBM"
+    assert T.possible_destination_memories("HBM") == ["HBM", "LDS", "VGPR"]
+    assert T.possible_destination_memories("LDS") == ["LDS", "VGPR"]
+    assert T.possible_destination_memories("ACC") == ["ACC"]
+    sq = [64, 64]
+    layouts = T.all_layouts_for_shape(sq, M.f32)
+    reprs = [repr(l) for l in layouts]
+    assert layouts[0] == M.row_major(sq) and layouts[1] == M.col_major(sq) and len(set(reprs)) == len(reprs)
+    # f32: Packed 2 and 4 (8 / 4 and 16 / 4 bytes), never of the innermost dim; OddEven 2, 4, 8, any dim.
+    assert "layout![0, 1, 0 p(4)]" in reprs and "layout![1, 0, 1 p(2)]" in reprs
+    assert not any(r.startswith("layout![0, 1, 1 p(") or r.startswith("layout![1, 0, 0 p(") for r in reprs)
+    assert {r for r in reprs if "oe" in r and r.startswith("layout![0, 1,")} == {
+        f"layout![0, 1, {d} oe({n})]" for d in (0, 1) for n in (2, 4, 8)}
+    assert len(layouts) == 2 + 2 * 2 + 2 * 6
+    # bytes pack up to 16; rank 3 adds the k-fastest order, rank 4 channels-last.
+    assert "layout![0, 1, 2, 1 p(16)]" in [repr(l) for l in T.all_layouts_for_shape([4, 64, 32], M.u8)]
+    assert T.all_layouts_for_shape([4, 64, 32], M.bf16)[1] == M.layout(0, 2, 1)
+    assert T.all_layouts_for_shape([2, 16, 8, 8], M.u8)[1] == M.nhwc([2, 16, 8, 8])
+    # Sizes that do not divide the dim are left out; every layout listed applies and can be moved to.
+    for shape, dt in (([6, 10], M.f32), ([4, 64, 32], M.bf16), ([2, 16, 8, 8], M.u8), ([1, 1], M.f32), ([7], M.i32)):
+        for l in T.all_layouts_for_shape(shape, dt):
+            assert l.applies_to_shape(shape), (shape, l)
+            assert M.Move(shape, (dt, dt), layouts=[M.row_major(shape), l]).plan().steps
+    assert [repr(l) for l in T.all_layouts_for_shape([6, 10], M.f32) if "p(4)" in repr(l)] == []
+
+
 def test_benchmark_configurations_pick_their_kernels():
     p = c1().plan()
     assert p.kernels == ["k_gemm"] and "T = F32" in p.steps[0].kernel and "Tile<64, 64, 128" in p.steps[0].kernel
