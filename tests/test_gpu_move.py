@@ -143,3 +143,51 @@ def test_transpose_of_32_bit_elements(gpu, dt, npd, shape):
     assert np.array_equal(got.view(np.uint32), x.transpose(0, 2, 1).view(np.uint32))
     back = run_spec(M.Move(list(shape), (dt, dt), layouts=[cm, None]), [got, np.zeros(shape, npd)])
     assert np.array_equal(back.view(np.uint32), x.view(np.uint32))
+
+
+def _both(*dims):
+    """A layout for the library and the same for the oracle: ints are Dynamic dims, (d, 'p', n) a
+    Packed(n) dim and (d, 'oe', n) an OddEven(n) dim of logical dim d."""
+    m, o = [], []
+    for d in dims:
+        if isinstance(d, tuple):
+            m.append((d[0], M.Packed(d[2]) if d[1] == "p" else M.OddEven(d[2])))
+            o.append((d[0], 1 if d[1] == "p" else 2, d[2]))
+        else:
+            m.append(d)
+            o.append(d)
+    return M.layout(*m), orc.make_layout(o)
+
+
+GATHER_CASES = [
+    (M.u8, M.u8, [40, 32, 96, 224], (3, 2, 1, 0), (1, 0, 3, 2, (3, "p", 8))),          # bytes in runs of four
+    (M.u8, M.u8, [328, 640, 48], (1, 0, 2, (1, "oe", 4)), (1, 0, 2)),
+    (M.i32, M.i32, [96, 208, 64], (2, 1, 0), (1, 2, 0, (0, "oe", 16))),                 # a digit covered in part
+    (M.bf16, M.bf16, [16, 512, 64, 32], (3, 1, 2, 0, (3, "oe", 4)), (1, 0, 2, 3)),
+    (M.u16, M.u16, [1152, 16, 32, 64], (2, 0, 3, 1), (1, 0, 2, 3)),                     # 16-bit runs
+    (M.bf16, M.f32, [16, 280, 4, 504], (0, 2, 1, 3), (1, 2, 3, 0)),                     # converting, 2 -> 4 bytes
+    (M.f32, M.bf16, [160, 35, 1024], (2, 0, 1, (2, "p", 8)), (0, 2, 1)),
+    (M.i32, M.u8, [192, 35, 752], (0, 2, 1, (2, "oe", 8)), (0, 1, 2)),
+    (M.u8, M.i32, [227, 35, 192], (0, 1, 2), (2, 0, 1, (2, "oe", 4))),
+    (M.f32, M.f32, [12, 6, 20, 30, 40], (4, 3, 1, 2, 0), (0, 2, 1, 3, 4)),              # five digits
+]
+
+
+@pytest.mark.parametrize("sdt,ddt,shape,src,dst", GATHER_CASES)
+def test_move_through_the_gather_kernel(gpu, sdt, ddt, shape, src, dst):
+    """Layout pairs with neither a shared contiguous run nor two long contiguous dims, above the
+    million elements up to which an element per thread serves: the tile kernel with runs of
+    elements of every size, with and without conversion, with three to five digits in its tile."""
+    NP = {M.u8: np.uint8, M.u16: np.uint16, M.i32: np.int32, M.f32: np.float32, M.bf16: np.uint16}
+    (ls, lso), (ld, ldo) = _both(*src), _both(*dst)
+    spec = M.Move(shape, (sdt, ddt), layouts=[ls, ld])
+    assert spec.plan().kernels == ["k_move_gather"]
+    if sdt == M.f32:
+        x = (synth.normal_f32(840, 0, shape) * 300).astype(np.float32)
+    elif sdt == M.bf16:
+        x = synth.normal_bf16(840, 1, shape, 100.0)
+    else:
+        x = synth.raw_u64(840, 2, int(np.prod(shape))).astype(NP[sdt]).reshape(shape)
+    got = run_spec(spec, [x, np.zeros(shape, NP[ddt])])
+    want = orc.move(shape, [int(sdt), int(ddt)], x, np.zeros(shape, NP[ddt]), layouts=[lso, ldo])
+    assert np.array_equal(got.view(np.uint8), want.view(np.uint8))

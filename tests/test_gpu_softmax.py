@@ -98,6 +98,18 @@ def test_softmax_short_rows(gpu, shape, dim):
 @pytest.mark.parametrize("shape,dim", [((2048, 4096), 0), ((600, 70), 0), ((3, 1000, 130), 1), ((513, 64), 0),
                                        ((7, 16), 0), ((2, 5000, 17), 1)])
 def test_softmax_over_an_outer_dim(gpu, shape, dim):
+    _softmax_outer(shape, dim)
+
+
+@pytest.mark.parametrize("shape,dim", [((600, 64, 300), 0), ((100, 64, 300), 0), ((3, 520, 20000), 1)])
+def test_softmax_over_an_outer_dim_in_one_kernel(gpu, shape, dim):
+    """Enough columns for 256 workgroups of 64: the kernel that walks the scan dim itself, on 16
+    waves (scan dims from 512) and on 4."""
+    assert M.Softmax(list(shape), dim).plan().kernels == ["k_softmax_cols"]
+    _softmax_outer(shape, dim)
+
+
+def _softmax_outer(shape, dim):
     """The scan dim is not the contiguous one: 64 columns per workgroup, the scan dim split over
     its 4 or 16 waves (short and long scan dims, ragged column tiles and scan lengths)."""
     x = synth.normal_f32(206, 0, shape, std=3.0)
