@@ -125,8 +125,8 @@ hipError_t launch_unfold(const void *image, void *rows, uint32_t batch, uint32_t
 
 // ---- softmax.hip: f32 softmax over a contiguous innermost scan dim ---------------------
 // Rows longer than 4096 run a workgroup per SOFTMAX_CHUNK elements and want
-// softmax_scratch_bytes() of device scratch for the chunks' (max, denominator) pairs; with a
-// null `scratch` they fall back to one wavefront per row.  `out` may be `in`.
+// softmax_scratch_bytes() of device scratch for the chunks' (max, denominator) pairs
+// (hipErrorInvalidValue without it).  `out` may be `in`.
 constexpr uint32_t SOFTMAX_CHUNK = 4096;
 size_t softmax_scratch_bytes(uint64_t rows, uint32_t cols);
 hipError_t launch_softmax_rows(const float *in, float *out, uint64_t rows, uint32_t cols, void *scratch,

@@ -5,8 +5,8 @@
 // (morello/src/scheduling/to_softmax_parts.rs:33-181, examples/softmax2.rs:47-113: three
 // trips through memory).  Here one wavefront owns a row, keeps it in registers between the
 // passes (one HBM read, one HBM write per element) and reduces with cross-lane shuffles;
-// rows too long for the register budget fall back to re-reading, and the per-lane partial
-// (max, denom) pairs are merged with the reference's online formula
+// rows too long for that are taken in chunks by whole workgroups, whose partial (max, denom)
+// pairs are merged with the reference's online formula
 // new = max(a,b); d = d_a*exp(a-new) + d_b*exp(b-new) (morello/src/spec.rs:116-123).
 #include "kernels.h"
 
@@ -128,42 +128,6 @@ __global__ __launch_bounds__(256) void k_softmax_regs1(const float *__restrict__
     const float y = v[i] / sum;
     if constexpr (OUT_BF16) (static_cast<uint16_t *>(out_any) + row * cols)[e] = uint16_t(bf16_bits(y));
     else __builtin_nontemporal_store(y, static_cast<float *>(out_any) + row * cols + e);
-  }
-}
-
-// Any cols: each lane runs the online (max, denom) update over its elements, the lanes'
-// pairs are merged, then the row is read again to write exp(x - max) / denom.
-template <bool OUT_BF16>
-__global__ __launch_bounds__(256) void k_softmax_stream(const float *__restrict__ in,
-                                                        void *__restrict__ out_any, uint64_t rows,
-                                                        uint32_t cols) {
-  float *out = static_cast<float *>(out_any);
-  const uint64_t row = uint64_t(blockIdx.x) * 4 + (threadIdx.x >> 6);
-  if (row >= rows) return;
-  const uint32_t lane = threadIdx.x & 63;
-  const float *src = in + row * cols;
-  float *dst = out + row * cols;
-  float mx = F32_MIN, den = 0.0f;
-  bool nan = false;
-  for (uint32_t i = lane; i < cols; i += 64) {
-    const float x = src[i];
-    nan |= x != x;
-    const float nm = fmaxf(mx, x);
-    den = den * expf(mx - nm) + expf(x - nm);
-    mx = nm;
-  }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    const float om = __shfl_xor(mx, o), od = __shfl_xor(den, o);
-    const float nm = fmaxf(mx, om);
-    den = den * expf(mx - nm) + od * expf(om - nm);
-    mx = nm;
-  }
-  if (__any(nan)) mx = __uint_as_float(0x7fc00000u);
-  for (uint32_t i = lane; i < cols; i += 64) {
-    const float y = expf(src[i] - mx) / den;
-    if constexpr (OUT_BF16) (static_cast<uint16_t *>(out_any) + row * cols)[i] = uint16_t(bf16_bits(y));
-    else dst[i] = y;
   }
 }
 
@@ -464,7 +428,7 @@ hipError_t launch_rows(const float *in, void *out, uint64_t rows, uint32_t cols,
     else if (nv <= 8) MRL_LAUNCH((k_softmax_regs<8, OUT_BF16>), grid, block, 0, stream, in, out, rows, cols);
     else MRL_LAUNCH((k_softmax_regs<16, OUT_BF16>), grid, block, 0, stream, in, out, rows, cols);
   } else {
-    MRL_LAUNCH(k_softmax_stream<OUT_BF16>, grid, block, 0, stream, in, out, rows, cols);
+    return hipErrorInvalidValue;  // rows in chunks, and no scratch was passed for them
   }
   return mrl::plan::last_error();
 }
