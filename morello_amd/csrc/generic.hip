@@ -427,6 +427,77 @@ __global__ __launch_bounds__(256) void k_move_tiled16v(MoveStrided p) {
   }
 }
 
+// Bytes whose source rows are whole 16-byte vectors: a 128 x 128 tile as dwords (four bytes along
+// the source's contiguous dim each), loaded sixteen bytes per lane.  A lane then takes the dwords
+// of four neighbouring tile rows at one column, transposes the 4 x 4 bytes in registers (byte
+// permutes) and stores the four dwords into four destination rows.  The four rows are read in
+// an order rotated by the lane's group, which spreads the 32 lanes of a half-wave over all banks.
+__global__ __launch_bounds__(256) void k_move_tiled8v(MoveStrided p) {
+  __shared__ uint32_t tile[128][33];
+  uint64_t blk = blockIdx.x;
+  const uint32_t ts = uint32_t(blk % p.tiles_s);
+  blk /= p.tiles_s;
+  const uint32_t td = uint32_t((blk + ts) % p.tiles_d);  // diagonal order, see k_move_tiled
+  blk /= p.tiles_d;
+  int64_t so = 0, d_o = 0;
+  for (int o = int(p.rank) - 1; o >= 0; o--) {
+    const uint32_t d = p.order[o];
+    if (d == p.dim_s || d == p.dim_d) continue;
+    const uint32_t c = uint32_t(blk % p.shape[d]);
+    blk /= p.shape[d];
+    so += int64_t(c) * p.ss[d], d_o += int64_t(c) * p.ds[d];
+  }
+  typedef uint32_t quad_t __attribute__((ext_vector_type(4)));
+  const uint32_t s0 = ts * 128, d0 = td * 128, ns = p.shape[p.dim_s], nd = p.shape[p.dim_d];
+  const uint8_t *src = static_cast<const uint8_t *>(p.src);
+  uint8_t *dst = static_cast<uint8_t *>(p.dst);
+  const uint32_t col = (threadIdx.x & 7) * 16, row = threadIdx.x >> 3;  // 8 lanes per 128-byte row
+  quad_t v[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const uint32_t r = row + 32 * i;
+    v[i] = quad_t{0, 0, 0, 0};
+    if (d0 + r < nd && s0 + col < ns)
+      v[i] = __builtin_nontemporal_load((const quad_t *)(src + so + int64_t(d0 + r) * p.ss[p.dim_d] + (s0 + col)));
+  }
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const uint32_t r = row + 32 * i;
+#pragma unroll
+    for (int j = 0; j < 4; j++) tile[r][col / 4 + j] = v[i][j];
+  }
+  __syncthreads();
+  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t group = lane & 31, half = lane >> 5;  // four tile rows 4 * group .. + 3
+  const uint32_t turn = group >> 3;
+  const uint32_t d = d0 + 4 * group;
+#pragma unroll
+  for (uint32_t it = 0; it < 4; it++) {
+    const uint32_t sq = it * 8 + wave * 2 + half;  // which four source bytes (one dword of a tile row)
+    uint32_t x[4];
+#pragma unroll
+    for (uint32_t j = 0; j < 4; j++) x[j] = tile[4 * group + ((j + turn) & 3)][sq];
+    // x[j] is tile row (j + turn) % 4: undo the rotation.
+    uint32_t a[4];
+#pragma unroll
+    for (uint32_t k = 0; k < 4; k++) {
+      const uint32_t from = (k - turn) & 3;
+      a[k] = from == 0 ? x[0] : from == 1 ? x[1] : from == 2 ? x[2] : x[3];
+    }
+    const uint32_t lo01 = __builtin_amdgcn_perm(a[1], a[0], 0x05010400u), hi01 = __builtin_amdgcn_perm(a[1], a[0], 0x07030602u);
+    const uint32_t lo23 = __builtin_amdgcn_perm(a[3], a[2], 0x05010400u), hi23 = __builtin_amdgcn_perm(a[3], a[2], 0x07030602u);
+    const uint32_t out[4] = {__builtin_amdgcn_perm(lo23, lo01, 0x05040100u), __builtin_amdgcn_perm(lo23, lo01, 0x07060302u),
+                             __builtin_amdgcn_perm(hi23, hi01, 0x05040100u), __builtin_amdgcn_perm(hi23, hi01, 0x07060302u)};
+    if (d < nd) {
+#pragma unroll
+      for (uint32_t k = 0; k < 4; k++) {
+        const uint32_t sidx = s0 + 4 * sq + k;
+        if (sidx < ns) *(uint32_t *)(dst + d_o + int64_t(sidx) * p.ds[p.dim_s] + d) = out[k];
+      }
+    }
+  }
+}
+
 // The same for 32-bit elements that are not converted: 64 x 64 tiles, four elements (16 bytes)
 // per lane on both sides.  Needs extents along both contiguous dims and all other strides in
 // multiples of 4 elements and 16-byte aligned bases, so that every vector is whole and aligned.
@@ -1081,19 +1152,26 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
     // ... and the source side in whole 16-byte vectors.
     bool octets = pairs && p.shape[dim_s] % 8 == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0;
     for (uint32_t d = 0; octets && d < p.rank; d++) octets = int(d) == dim_s || p.ss[d] % 8 == 0;
+    // Bytes: sixteen per lane on the source side, four on the destination side.
+    bool bytes16 = src_dtype == dst_dtype && mrl_dtype_size(src_dtype) == 1 && p.shape[dim_s] % 16 == 0 &&
+                   p.shape[dim_d] % 4 == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(dst) & 3) == 0;
+    for (uint32_t d = 0; bytes16 && d < p.rank; d++)
+      bytes16 = (int(d) == dim_s || p.ss[d] % 16 == 0) && (int(d) == dim_d || p.ds[d] % 4 == 0);
     // 32-bit elements likewise, four per lane.
     bool quads = src_dtype == dst_dtype && mrl_dtype_size(src_dtype) == 4 && p.shape[dim_s] % 4 == 0 &&
                  p.shape[dim_d] % 4 == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0 &&
                  (reinterpret_cast<uintptr_t>(dst) & 15) == 0;
     for (uint32_t d = 0; quads && d < p.rank; d++)
       quads = (int(d) == dim_s || p.ss[d] % 4 == 0) && (int(d) == dim_d || p.ds[d] % 4 == 0);
-    const uint32_t side = pairs ? 128 : 64;
+    const uint32_t side = pairs || bytes16 ? 128 : 64;
     p.tiles_s = (p.shape[dim_s] + side - 1) / side, p.tiles_d = (p.shape[dim_d] + side - 1) / side;
     uint64_t blocks = uint64_t(p.tiles_s) * p.tiles_d;
     for (uint32_t d = 0; d < p.rank; d++)
       if (int(d) != dim_s && int(d) != dim_d) blocks *= p.shape[d];
     if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
-    if (octets) MRL_LAUNCH(k_move_tiled16v, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+    if (bytes16) MRL_LAUNCH(k_move_tiled8v, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
+    else if (octets) MRL_LAUNCH(k_move_tiled16v, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
     else if (pairs) MRL_LAUNCH(k_move_tiled16, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
     else if (quads) MRL_LAUNCH(k_move_tiled32, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
     else if (src_dtype != dst_dtype) {

@@ -191,3 +191,21 @@ def test_move_through_the_gather_kernel(gpu, sdt, ddt, shape, src, dst):
     got = run_spec(spec, [x, np.zeros(shape, NP[ddt])])
     want = orc.move(shape, [int(sdt), int(ddt)], x, np.zeros(shape, NP[ddt]), layouts=[lso, ldo])
     assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+
+
+@pytest.mark.parametrize("dt,npd", [(M.u8, np.uint8), (M.i8, np.int8)])
+@pytest.mark.parametrize("shape", [(2, 208, 144), (1, 132, 272), (3, 64, 64), (1, 1000, 16), (2, 36, 64), (1, 2048, 128),
+                                   (1, 130, 258), (1, 400, 4000)])
+def test_transpose_of_8_bit_elements(gpu, dt, npd, shape):
+    """Bytes: sixteen per lane on the source side and a 4 x 4 byte transpose in registers where
+    the source rows are whole 16-byte vectors and the destination rows whole dwords (whole and
+    ragged 128 x 128 tiles, either direction), one byte per lane otherwise."""
+    x = synth.raw_u64(832, 0, int(np.prod(shape))).astype(np.uint8).view(npd).reshape(shape)
+    cm = M.batched_col_major(list(shape))
+    spec = M.Move(list(shape), (dt, dt), layouts=[None, cm])
+    if shape[2] % 16 == 0 and shape[1] % 4 == 0 and shape[1] * shape[2] * shape[0] > 65536:
+        assert spec.plan().kernels == ["k_move_tiled8v"]
+    got = run_spec(spec, [x, np.zeros((shape[0], shape[2], shape[1]), npd)])
+    assert np.array_equal(got, x.transpose(0, 2, 1))
+    back = run_spec(M.Move(list(shape), (dt, dt), layouts=[cm, None]), [got, np.zeros(shape, npd)])
+    assert np.array_equal(back, x)

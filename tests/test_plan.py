@@ -124,7 +124,9 @@ def test_plans_follow_shape_dtype_and_layout():
     transposed = [M.row_major(sq), M.col_major(sq)]
     assert M.Move(sq, (M.f32, M.f32), layouts=transposed).plan().kernels == ["k_move_tiled32"]
     assert M.Move(sq, (M.bf16, M.bf16), layouts=transposed).plan().kernels == ["k_move_tiled16v"]
-    assert M.Move(sq, (M.u8, M.u8), layouts=transposed).plan().kernels == ["k_move_tiled_as"]
+    assert M.Move(sq, (M.u8, M.u8), layouts=transposed).plan().kernels == ["k_move_tiled8v"]
+    odd8 = [4100, 4100]
+    assert M.Move(odd8, (M.u8, M.u8), layouts=[M.row_major(odd8), M.col_major(odd8)]).plan().kernels == ["k_move_tiled_as"]
     assert M.Move(sq, (M.u8, M.f32), layouts=transposed).plan().kernels == ["k_move_tiled"]
     odd = [4098, 4098]
     assert M.Move(odd, (M.bf16, M.bf16), layouts=[M.row_major(odd), M.col_major(odd)]).plan().kernels == ["k_move_tiled16"]
