@@ -75,7 +75,16 @@ uint32_t gemm_k_splits(const GemmArgs &g, int kind) {
   if (tiles >= 384 || steps < 16) return 1;
   uint64_t want = std::min<uint64_t>({32, 768 / tiles, steps / 8});
   while (want > 1 && steps % want != 0) want--;
-  return uint32_t(std::max<uint64_t>(1, want));
+  if (want <= 1) return 1;
+  // What the slices save: a workgroup's chain of k steps (~0.48 us each on the 64 x 64 tile)
+  // shortens by the factor by which they add workgroups the chip has room for (about 384
+  // overlap well); what they cost: the summing launch and its traffic.  bf16 1024^3 (256 tiles
+  // of 16 steps) ran 15 us in two slices against 8.8 us whole.
+  const double spread = std::min<double>(double(want), 384.0 / double(tiles));
+  const double saved_us = double(steps) * (1.0 - 1.0 / spread) * 0.48;
+  const double cost_us = 2.5 + (double(want) + 1.0) * double(g.m) * double(g.n) * 4.0 / 5.5e6;
+  if (spread <= 1.0 || saved_us < 1.2 * cost_us) return 1;
+  return uint32_t(want);
 }
 
 hipError_t launch_gemm_big(const GemmArgs &g, int kind, hipStream_t stream) {
