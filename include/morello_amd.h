@@ -415,6 +415,9 @@ typedef struct {
  * that runs a Spec, with launches recorded instead of made, so it cannot disagree with a run.
  * MRL_ERR_UNSUPPORTED / MRL_ERR_BAD_SPEC as mrl_run. */
 int mrl_spec_plan(const mrl_spec *spec, mrl_plan *plan, mrl_plan_step *steps, uint32_t cap);
+/* Kernels the calling thread has launched through this library so far: after a run of a Spec the
+ * count has grown by that Spec's plan.n_steps (tests hold the two against each other). */
+uint64_t mrl_launch_count(void);
 /* The same for a Matmul under a manual schedule (mrl_run_matmul_scheduled): what a search over
  * tile_out / split (scheduling_sugar.rs:37-132) compares. */
 int mrl_matmul_scheduled_plan(const mrl_spec *spec, const mrl_matmul_schedule *schedule, mrl_plan *plan,

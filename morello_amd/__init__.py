@@ -695,6 +695,11 @@ def measure_mfma_rate(kind: str, random_operands: bool, iters: int = 20000) -> f
     return out.value
 
 
+def launch_count() -> int:
+    """Kernels this thread has launched through the library so far."""
+    return int(B.load().mrl_launch_count())
+
+
 def synchronize():
     _check(B.load().mrl_device_synchronize(), "mrl_device_synchronize")
 

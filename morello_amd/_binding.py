@@ -145,6 +145,7 @@ SIGNATURES = {
     "mrl_matmul_scheduled_plan": (C.c_int, [C.POINTER(SpecC), C.POINTER(MatmulScheduleC), C.POINTER(PlanC),
                                             C.POINTER(PlanStepC), C.c_uint32]),
     "mrl_matmul_search_schedule": (C.c_int, [C.POINTER(SpecC), C.POINTER(MatmulScheduleC), C.POINTER(C.c_double)]),
+    "mrl_launch_count": (C.c_uint64, []),
     "mrl_compose_plan": (C.c_int, [C.POINTER(ComposeC), C.POINTER(PlanC), C.POINTER(PlanStepC), C.c_uint32]),
     "mrl_device_info": (C.c_int, [C.c_char_p, C.c_size_t, C.POINTER(C.c_int), C.POINTER(C.c_int),
                                   C.POINTER(C.c_size_t)]),

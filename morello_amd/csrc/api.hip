@@ -1311,6 +1311,8 @@ size_t mrl_spec_workspace_bytes(const mrl_spec *spec) {
   return total;
 }
 
+uint64_t mrl_launch_count(void) { return mrl::plan::g_launches; }
+
 const char *mrl_target_id(void) { return "Gfx950"; }
 uint32_t mrl_target_line_size(void) { return 128; }
 uint32_t mrl_target_processors(void) {

@@ -40,6 +40,9 @@ struct Recorder {
 };
 
 extern thread_local Recorder *g_recorder;
+// Kernels this thread has launched through MRL_LAUNCH (not recorded ones): lets a test hold a
+// plan against what a run of the same Spec did.
+extern thread_local uint64_t g_launches;
 
 inline bool recording() { return g_recorder != nullptr; }
 
@@ -66,5 +69,8 @@ inline hipError_t last_error() { return g_recorder ? hipSuccess : hipGetLastErro
 #define MRL_LAUNCH(kernel, grid, block, lds, stream, ...)                                              \
   do {                                                                                                 \
     if (mrl::plan::recording()) mrl::plan::note(#kernel, __PRETTY_FUNCTION__, grid, block, lds);            \
-    else hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);                             \
+    else {                                                                                             \
+      mrl::plan::g_launches++;                                                                         \
+      hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);                               \
+    }                                                                                                  \
   } while (0)

@@ -9,6 +9,7 @@ namespace mrl {
 namespace plan {
 
 thread_local Recorder *g_recorder = nullptr;
+thread_local uint64_t g_launches = 0;
 
 // "(k_attn<D, RAGGED, KT_ROWS>)" within "hipError_t mrl::(anonymous namespace)::launch_one(...)
 // [D = 128, RAGGED = false, KT_ROWS = false]" -> "k_attn [D = 128, RAGGED = false, KT_ROWS = false]".

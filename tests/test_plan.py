@@ -293,3 +293,47 @@ def test_cost_model_ranks_manual_schedules(gpu):
                 b.free()
             pick = min(predicted, key=predicted.get)
             assert measured[pick] <= 1.5 * min(measured.values()), (dts[0], m, k, n, pick, measured)
+
+
+@pytest.mark.gpu
+def test_a_run_launches_what_its_plan_lists(gpu):
+    """The plan comes from the dispatch code itself; this holds the two against each other from
+    outside: a run launches as many kernels as its plan has steps, for Specs of every kind and
+    path (matrix cores, padded and transposed operands, slices of K, fused and staged Compose,
+    split keys, every Softmax and Move kernel family, generic kernels)."""
+    sq = [600, 520]
+    specs = [
+        c1(), M.Matmul([1, 1000, 1000, 1000], (M.u8, M.i8, M.i32)), M.Matmul([1, 512, 8192, 512], (M.bf16, M.bf16, M.f32)),
+        M.Matmul([2, 100, 70, 50], (M.i16, M.i16, M.i32)), M.Matmul([1, 1, 2048, 4096], (M.bf16, M.bf16, M.f32), layouts=[None, KT, None]),
+        M.Matmul([1, 300, 256, 200], (M.f32, M.f32, M.f32), layouts=[M.batched_col_major([1, 300, 256]), None, M.batched_col_major([1, 300, 200])]),
+        M.Matmul([1, 64, 64, 64], [M.f32] * 3, layouts=[None, M.layout(0, 2, 1, (2, M.Packed(16))), None]),
+        M.Conv([2, 64, 64, 20, 20, 3, 3], (M.u8, M.i8, M.i32)), M.Conv([2, 32, 16, 20, 20, 3, 3], (M.bf16, M.bf16, M.f32)),
+        M.Conv([2, 16, 3, 30, 30, 5, 5], (M.u8, M.i8, M.i32)), M.Conv([1, 4, 4, 6, 6, 3, 3], (M.u16, M.u16, M.u32)),
+        M.ComposeMSM(2, 256, 128, 512, 128, layouts=[None, None, KT, None]), M.ComposeMSM(2, 256, 128, 512, 128),
+        M.ComposeMSM(2, 100, 96, 300, 72, layouts=[None, None, KT, None]), M.ComposeMSM(4, 1, 128, 8192, 128, layouts=[None, None, KT, None]),
+        M.ComposeMSM(1, 200, 160, 1001, 160, layouts=[None, None, KT, None]),
+        M.Compose([M.Matmul([2, 64, 96, 32], [M.f32, M.bf16, M.f32]), M.Softmax([2, 64, 96], 2),
+                   M.Matmul([2, 64, 32, 96], [M.bf16, M.bf16, M.f32])], layouts=[None, None, KT, None]).bufferize(0),
+        M.Softmax([64, 2048], 1), M.Softmax([1000, 67], 1), M.Softmax([300, 8192], 1), M.Softmax([40, 100000], 1),
+        M.Softmax([600, 1001], 1), M.Softmax([2149, 172], 0), M.Softmax([600, 64, 300], 0), M.Softmax([6, 4], 0),
+        M.Move(sq, (M.f32, M.f32), layouts=[M.row_major(sq), M.col_major(sq)]), M.Move(sq, (M.u8, M.u8), layouts=[M.row_major(sq), M.col_major(sq)]),
+        M.Move(sq, (M.bf16, M.f32)), M.Move([96, 208, 64], (M.i32, M.i32), layouts=[M.layout(2, 1, 0), M.layout(1, 2, 0, (0, M.OddEven(16)))]),
+        M.Move([64, 48], (M.u8, M.u8), layouts=[M.row_major([64, 48]), M.layout(0, 1, (1, M.OddEven(16)))]),
+        M.Fill([100, 100], M.f32, M.FillValue.NegInf), M.Max([64, 64], 1), M.Broadcast([4, 8], 1), M.OnePrefix([4, 8]),
+    ]
+    for spec in specs:
+        n_params = spec.n_params if hasattr(spec, "n_params") and not isinstance(spec, M.Spec) else len(spec.dtypes)
+        if isinstance(spec, M.Spec):
+            sizes = [spec.bytes_used(i) for i in range(len(spec.dtypes))]
+        else:
+            sizes = [int(np.prod(spec.parameter_shape(i))) * spec.parameter_dtypes()[i].size for i in range(n_params)]
+        bufs = [M.DeviceBuffer(max(4, s)) for s in sizes]
+        for b in bufs:
+            b.zero()
+        steps = len(spec.plan().steps)
+        before = M.launch_count()
+        spec.run_device([b.ptr for b in bufs])
+        launched = M.launch_count() - before
+        for b in bufs:
+            b.free()
+        assert launched == steps, (spec.plan(), launched)
