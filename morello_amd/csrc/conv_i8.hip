@@ -103,6 +103,9 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(ConvArgs p, uint32_t pix
   // parked in LDS past the filter bank (every wave writes the same 64 numbers and reads back
   // its own writes, so no barrier is needed).
   int *corr_lds = (int *)(filt_lds + FT * 16 * krow);
+  // Per wave: 16 pixel rows of 64 results, rows 68 dwords apart (16-byte aligned, banks shifted).
+  constexpr int TURN_ROW = 68;
+  int *turn_lds = corr_lds + FT * 16 + (threadIdx.x >> 6) * (16 * TURN_ROW);
   if (IMG_UNSIGNED) {
     const v4i ones = v4i{0x01010101, 0x01010101, 0x01010101, 0x01010101};
 #pragma unroll
@@ -134,19 +137,28 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(ConvArgs p, uint32_t pix
         acc[ft] = __builtin_amdgcn_mfma_i32_16x16x64_i8(filt[ft][s], px, acc[ft], 0, 0, 0);
       img[s] = *(const v4i *)(src_n + slab_off[s]);
     }
-    // D[row = filter 4*lg + r][col = pixel li]: lane owns 4 consecutive filters of its pixel.
-    const uint32_t pix = t * 16 + li;
-    if (pix < pixels) {
-      int32_t *dst = out + int64_t(pix) * p.f + lg * 4;
+    // D[row = filter 4*lg + r][col = pixel li]: lane owns 4 consecutive filters of its pixel in
+    // each filter tile, i.e. 16-byte pieces 64 bytes apart.  The tile's 16 x 64 results go through
+    // this wave's own patch of LDS so that the stores are whole 256-byte pixel rows, four
+    // pixels per instruction (1 KiB contiguous when F = 64), instead of 64-byte segments.
 #pragma unroll
-      for (int ft = 0; ft < FT; ft++) {
-        v4i v = acc[ft];
-        if (IMG_UNSIGNED) v += *(const v4i *)(corr_lds + ft * 16 + lg * 4);
-        v4i *d = (v4i *)(dst + ft * 16);
+    for (int ft = 0; ft < FT; ft++) {
+      v4i v = acc[ft];
+      if (IMG_UNSIGNED) v += *(const v4i *)(corr_lds + ft * 16 + lg * 4);
+      *(v4i *)(turn_lds + li * TURN_ROW + ft * 16 + lg * 4) = v;
+    }
+    __builtin_amdgcn_wave_barrier();  // LDS operations of a wave complete in order
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t row = i * 4 + lg, pix = t * 16 + row;  // lane (li, lg): pixel row, filters 4*li .. +3
+      v4i v = *(const v4i *)(turn_lds + row * TURN_ROW + li * 4);
+      if (pix < pixels) {
+        v4i *d = (v4i *)(out + int64_t(pix) * p.f + li * 4);
         if (p.accum) v += *d;
         __builtin_nontemporal_store(v, d);  // written once, never re-read by this kernel
       }
     }
+    __builtin_amdgcn_wave_barrier();
     t = tn;
   }
 }
@@ -161,7 +173,8 @@ hipError_t launch_slabs(const ConvArgs &c, bool img_unsigned, hipStream_t stream
   const uint32_t groups = c.f / (FT * 16);
   uint32_t blocks = std::max<uint32_t>(1, 2048 / WAVES / groups);
   if (blocks * WAVES > tiles) blocks = (tiles + WAVES - 1) / WAVES;
-  const size_t lds = size_t(FT) * 16 * c.fh * c.fw * c.c + FT * 16 * sizeof(int);  // the filter bank + corrections
+  // the filter bank + corrections + a 16 x 68-dword patch per wave for the output rows
+  const size_t lds = size_t(FT) * 16 * c.fh * c.fw * c.c + FT * 16 * sizeof(int) + size_t(WAVES) * 16 * 68 * sizeof(int);
   plan::work(plan::UNIT_MFMA_I8, 2.0 * pixels * c.f * c.fh * c.fw * c.c,
              double(c.b) * (c.oh + c.fh - 1) * (c.ow + c.fw - 1) * c.c + double(c.f) * c.fh * c.fw * c.c +
                  4.0 * pixels * c.f * (c.accum ? 2 : 1));
