@@ -322,11 +322,10 @@ def test_a_run_launches_what_its_plan_lists(gpu):
         M.Fill([100, 100], M.f32, M.FillValue.NegInf), M.Max([64, 64], 1), M.Broadcast([4, 8], 1), M.OnePrefix([4, 8]),
     ]
     for spec in specs:
-        n_params = spec.n_params if hasattr(spec, "n_params") and not isinstance(spec, M.Spec) else len(spec.dtypes)
         if isinstance(spec, M.Spec):
             sizes = [spec.bytes_used(i) for i in range(len(spec.dtypes))]
-        else:
-            sizes = [int(np.prod(spec.parameter_shape(i))) * spec.parameter_dtypes()[i].size for i in range(n_params)]
+        else:  # a general Compose: dense row-major external parameters
+            sizes = [int(np.prod(shape)) * dt.size for shape, dt in zip(spec.parameter_shapes(), spec.parameter_dtypes())]
         bufs = [M.DeviceBuffer(max(4, s)) for s in sizes]
         for b in bufs:
             b.zero()
