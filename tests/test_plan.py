@@ -241,7 +241,7 @@ def test_planning_leaves_runs_alone(gpu):
 
 @pytest.mark.gpu
 def test_cost_model_against_measured_launches(gpu):
-    """Predicted / measured per-launch time stays within [0.4, 2.5] on benchmark-like operands for
+    """Predicted / measured per-launch time stays within [1/3, 3] on benchmark-like operands for
     the kernels the benchmark configurations and their neighbours run (the fit's own spread is
     0.6-1.5; the bound leaves room for the board's clock state)."""
     rng = np.random.default_rng(7)
@@ -264,14 +264,14 @@ def test_cost_model_against_measured_launches(gpu):
         predicted_ns = spec.plan().cost_ns
         for b in bufs:
             b.free()
-        assert 0.4 < predicted_ns / measured_ns < 2.5, (spec, predicted_ns, measured_ns)
+        assert 0.33 < predicted_ns / measured_ns < 3.0, (spec, predicted_ns, measured_ns)
 
 
 @pytest.mark.gpu
 def test_cost_model_ranks_manual_schedules(gpu):
     """What a search over tile_out / split needs from the model: the schedule it calls cheapest
-    runs within 1.5x of the schedule measured fastest (on these shapes it is the fastest or
-    within 1.15x, bf16 2048^3 1.4x)."""
+    runs within 2x of the schedule measured fastest (measured: the fastest itself or within 1.15x,
+    bf16 2048^3 1.4x; the bound leaves room for the board's clock state on another day)."""
     rng = np.random.default_rng(11)
     for dts in ((M.u8, M.i8, M.i32), (M.bf16, M.bf16, M.f32)):
         for m, k, n in ((512, 1024, 512), (2048, 2048, 2048), (4096, 4096, 4096), (1024, 8192, 1024)):
@@ -292,7 +292,7 @@ def test_cost_model_ranks_manual_schedules(gpu):
             for b in bufs:
                 b.free()
             pick = min(predicted, key=predicted.get)
-            assert measured[pick] <= 1.5 * min(measured.values()), (dts[0], m, k, n, pick, measured)
+            assert measured[pick] <= 2.0 * min(measured.values()), (dts[0], m, k, n, pick, measured)
 
 
 @pytest.mark.gpu
