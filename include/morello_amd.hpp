@@ -220,6 +220,13 @@ class Spec {
   }
   uint64_t flops() const { return mrl_spec_ops(&c_); }
   bool is_supported() const { return mrl_spec_check(&c_) == MRL_OK; }
+  // The manual Matmul schedule the cost model predicts cheapest, as {tile_m, tile_n, split_k}
+  // (scheduling_sugar.rs:37-132: what `tile_out([1, m, n])` and `split(k)` would be called with).
+  mrl_matmul_schedule search_schedule() const {
+    mrl_matmul_schedule best{};
+    check(mrl_matmul_search_schedule(&c_, &best, nullptr), "search_schedule");
+    return best;
+  }
   // Host-only: needs no GPU.
   Plan plan() const {
     mrl_plan head{};
