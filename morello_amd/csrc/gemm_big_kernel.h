@@ -161,20 +161,6 @@ inline bool big_applicable(const GemmArgs &g, int elem_size) {
          g.ldc * 4 < EDGE_MAX_ROW_BYTES;
 }
 
-// Tile rows per L2 group: the run of tiles one XCD gets (an eighth of them) should cover a block
-// of C as close to square as the counts allow, since its perimeter is what the XCD's L2 fetches.
-inline int big_group_m(int tiles_m, int tiles_n) {
-  const int ntiles = tiles_m * tiles_n;
-  if (ntiles % 8 != 0) return 4;
-  const int run = ntiles / 8;
-  int best = 0;
-  for (int gm = 1; gm <= tiles_m && gm <= run; gm *= 2) {
-    if (run % gm != 0 || (gm * tiles_n) % run != 0 || tiles_m % gm != 0) continue;
-    if (gm * gm <= run) best = gm;
-  }
-  return best ? best : 4;
-}
-
 template <class T, bool A_UNSIGNED>
 hipError_t launch_big(const GemmArgs &g, hipStream_t stream) {
   constexpr auto kern = k_gemm_big<T, A_UNSIGNED>;
@@ -190,7 +176,7 @@ hipError_t launch_big(const GemmArgs &g, hipStream_t stream) {
              (double(g.m) * g.k + double(g.k) * g.n) * g.batch * T::ES + mn * 4 * (g.accum ? 2 : 1),
              2.0 * 256 * 256 * double(g.k), 500.0 + 1200.0 * double(g.k * T::ES / 128));
   MRL_LAUNCH((k_gemm_big<T, A_UNSIGNED>), dim3(tiles_m * tiles_n, g.batch), dim3(512), BIG_LDS_BYTES, stream, g,
-             tiles_m, tiles_n, big_group_m(tiles_m, tiles_n));
+             tiles_m, tiles_n, group_rows(tiles_m, tiles_n));
   return mrl::plan::last_error();
 }
 

@@ -4,6 +4,7 @@
 // three entries long and comes from measurement).
 #include <algorithm>
 
+#include "gemm_big_kernel.h"
 #include "gemm_mfma_kernel.h"
 
 namespace mrl {
@@ -90,6 +91,15 @@ uint32_t gemm_k_splits(const GemmArgs &g, int kind) {
 hipError_t launch_gemm_big(const GemmArgs &g, int kind, hipStream_t stream) {
   if (g.b_kmajor) return launch_gemm_nt(g, kind, 256, stream);
   const bool whole = whole_tiles(g, elem_size_of(kind));
+  // Whole tiles and an even number of k steps: the tile with the hand-scheduled k loop
+  // (int8 4096^3 accumulating: 78 us against 87 us for the compiler-scheduled loop).
+  if (whole && kind <= 2 && big_applicable(g, elem_size_of(kind))) {
+    switch (kind) {
+      case 0: return launch_big<I8, false>(g, stream);
+      case 1: return launch_big<I8, true>(g, stream);
+      case 2: return launch_big<BF16, false>(g, stream);
+    }
+  }
   switch (kind) {
     case 0: return whole ? launch<I8, false, TileBig, false>(g, stream) : launch<I8, false, TileBig, true>(g, stream);
     case 1: return whole ? launch<I8, true, TileBig, false>(g, stream) : launch<I8, true, TileBig, true>(g, stream);

@@ -41,7 +41,22 @@ typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
 
-constexpr int GROUP_M = 4;                // tile-rows per L2 group
+// Tile rows per L2 group.  The workgroups of a launch go to the 8 XCDs round-robin and each XCD
+// gets a contiguous run of tiles (an eighth of them); taken group_m tile rows at a time, such a
+// run covers a block of C whose perimeter is what that XCD's L2 has to fetch, so the block
+// should be as close to square as the counts allow (8192^3 with 256-tiles: 8 x 16 tiles per XCD,
+// not 4 x 32, which made every XCD read all of B).
+inline int group_rows(int tiles_m, int tiles_n) {
+  const int ntiles = tiles_m * tiles_n;
+  if (ntiles % 8 != 0) return 4;
+  const int run = ntiles / 8;
+  int best = 0;
+  for (int gm = 1; gm <= tiles_m && gm <= run; gm *= 2) {
+    if (run % gm != 0 || (gm * tiles_n) % run != 0 || tiles_m % gm != 0) continue;
+    if (gm * gm <= run) best = gm;
+  }
+  return best ? best : 4;
+}
 
 // Ragged tiles (EDGE) address memory through buffer resources: `records` bytes from `base` on
 // are in range, a load beyond them returns zeros and a store beyond them is dropped, both
@@ -248,7 +263,7 @@ __device__ inline void sched_slots(bool staging) {
 // a channels-last image, g.conv; row p's 16-byte chunk at k byte kb lies at
 // corner(p) + ((r * w + s) * c_bytes + kb % c_bytes) with (r, s) = divmod(kb / c_bytes, fw).
 template <class T, bool A_UNSIGNED, class TL, bool EDGE, bool B_KMAJOR = false, bool CONV = false>
-__global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int tiles_n) {
+__global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int tiles_n, int group_m) {
   static_assert(!CONV || (EDGE && B_KMAJOR), "the implicit Conv operand is addressed through the buffer path");
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   constexpr int BM = TL::BM, BN = TL::BN, BKB = TL::BKB, WAVES_M = TL::WAVES_M, WAVES_N = TL::WAVES_N;
@@ -277,10 +292,10 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
   int pid = blockIdx.x;
   const int ntiles = tiles_m * tiles_n;
   if (ntiles % 8 == 0) pid = (pid % 8) * (ntiles / 8) + pid / 8;
-  const int group = pid / (GROUP_M * tiles_n);
-  const int first_m = group * GROUP_M;
-  const int gsz = min(tiles_m - first_m, GROUP_M);
-  const int in_group = pid % (GROUP_M * tiles_n);
+  const int group = pid / (group_m * tiles_n);
+  const int first_m = group * group_m;
+  const int gsz = min(tiles_m - first_m, group_m);
+  const int in_group = pid % (group_m * tiles_n);
   const int tile_m = first_m + in_group % gsz, tile_n = in_group / gsz;
   const int64_t m0 = int64_t(tile_m) * BM, n0 = int64_t(tile_n) * BN;
 
@@ -549,7 +564,7 @@ hipError_t launch(const GemmArgs &g, hipStream_t stream) {
                500.0 + (100.0 + 3.0 * (BM + BN)) * double((g.k * T::ES + TL::BKB - 1) / TL::BKB));
   }
   MRL_LAUNCH((k_gemm<T, A_UNSIGNED, TL, EDGE, B_KMAJOR, CONV>), dim3(tiles_m * tiles_n, g.batch), dim3(TL::NT),
-             2 * STAGE, stream, g, tiles_m, tiles_n);
+             2 * STAGE, stream, g, tiles_m, tiles_n, group_rows(tiles_m, tiles_n));
   return mrl::plan::last_error();
 }
 

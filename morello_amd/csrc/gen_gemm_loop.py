@@ -96,8 +96,10 @@ class Emitter:
         self.lds_done = self.lds_issued
 
 
-def gen(kind, wm):
-    """kind: 'u8' (A unsigned bytes), 'i8', 'bf16'.  wm: the wave row (which slabs' column sums it adds)."""
+def gen(kind, wm, opts=None):
+    """kind: 'u8' (A unsigned bytes), 'i8', 'bf16'.  wm: the wave row (which slabs' column sums it adds).
+    opts: experiment switches (lab use); the shipped loops are generated with none."""
+    opts = opts or {}
     unsigned = kind == "u8"
     mfma = "v_mfma_f32_32x32x16_bf16" if kind == "bf16" else "v_mfma_i32_32x32x32_i8"
     tr = "ds_read_b64_tr_b16" if kind == "bf16" else "ds_read_b64_tr_b8"
@@ -191,7 +193,7 @@ def gen(kind, wm):
         for s in range(4):
             buf, nb = s & 1, (s & 1) ^ 1
             others = []
-            chunks = [s] if s < 2 else [2, 3] if s == 2 else []
+            chunks = opts.get("chunks", [[0], [1], [2, 3], []])[s]
             for i in chunks:
                 others.append(lambda i=i: store_a(p, i, cur ^ 1))
                 others.append(lambda i=i: load_a(p, i))
@@ -199,37 +201,59 @@ def gen(kind, wm):
             if s == 2:
                 others.append(lambda: advance("s60", "s61", "s67", "128"))
                 others.append(lambda: advance("s62", "s63", "s68", "%[bstep]"))
-            if unsigned and s % 2 == wm:
+            if unsigned and s % 2 == wm and not opts.get("no_dot4"):
                 for tn in range(2):
                     for w in range(4):
                         others.append(lambda tn=tn, w=w: (e.need(bf(buf, tn, w // 2)),
                                                           E(f"v_dot4c_i32_i8 v{210 + tn}, 0x1010101, {bf(buf, tn, w=w)}")))
-            if s < 3:
-                rd = reads(cur, s + 1, nb)
-            else:
+            def sync():
                 # everything requested before this step has landed (B of tile kt+1, A of tile kt+2);
                 # this wave's LDS writes are done and the operands of this slab are in
                 E("s_waitcnt vmcnt(8) lgkmcnt(0)")
                 e.all_lds_done()
+                if opts.get("trace"):
+                    E("s_memtime s[72:73]")
                 E("s_barrier")
+                if opts.get("trace"):
+                    E("s_memtime s[74:75]")
+                    E("s_waitcnt lgkmcnt(0)")
+                    E("s_sub_u32 s76, s74, s72")
+                    E("s_add_u32 s77, s77, s76")
                 set_b_read_base("s65")
+            before_sync = opts.get("mfma_before_barrier", 0) if s == 3 else 0
+            if s < 3:
+                rd = reads(cur, s + 1, nb)
+            else:
+                if before_sync == 0:
+                    sync()
                 rd = reads(cur ^ 1, 0, nb)
+                rd = [[] for _ in range(before_sync)] + [g for g in rd if g] + [[] for _ in range(8)]
+                rd = rd[:8] if len([g for g in rd[8:] if g]) == 0 else None
             # spread the other work over the gaps behind the MFMAs, in order
             gaps = [[] for _ in range(8)]
-            first = 1 if (unsigned and s % 2 == wm) else 0  # dot4 needs both halves of B: not before MFMA 1
+            first = 1 if (unsigned and s % 2 == wm and not opts.get("no_dot4")) else 0  # dot4 needs both halves of B: not before MFMA 1
             for j, item in enumerate(others):
                 gaps[min(7, first + j * (8 - first) // max(1, len(others)))].append(item)
             n = 0
             for tm in range(4):
                 for tn in range(2):
                     e.need(af(buf, tm), bf(buf, tn, 0), bf(buf, tn, 1))
+                    if opts.get("prio") and n == 0:
+                        E("s_setprio 1")
                     E(f"{mfma} {acc(tm, tn)}, {af(buf, tm)}, {bf(buf, tn)}, {acc(tm, tn)}")
+                    if opts.get("prio") and n == 7:
+                        E("s_setprio 0")
+                    if s == 3 and before_sync and n == before_sync - 1:
+                        sync()
                     for r in rd[n]:
                         r()
                     for item in gaps[n]:
                         item()
                     n += 1
 
+    if opts.get("trace"):
+        E("s_mov_b32 s77, 0")
+        E("s_memtime s[78:79]")
     E("1:")
     step(0)
     step(1)
@@ -239,6 +263,12 @@ def gen(kind, wm):
     # nothing may land in LDS once the epilogue reuses it; the last MFMAs must have written the
     # accumulators before compiler-scheduled code reads them
     E("s_waitcnt vmcnt(0) lgkmcnt(0)")
+    if opts.get("trace"):
+        E("s_memtime s[80:81]")
+        E("s_waitcnt lgkmcnt(0)")
+        E("s_sub_u32 s76, s80, s78")
+        E("v_mov_b32 v208, s77")
+        E("v_mov_b32 v209, s76")
     E("s_barrier")
     E("s_nop 15")
     E("s_nop 15")
