@@ -44,6 +44,8 @@ def _compile(src: str) -> str:
 
 def build(verbose: bool = True) -> str:
     os.makedirs(OBJ_DIR, exist_ok=True)
+    # The assembly of the four-wave Matmul tile is generated (1.5 MB of text): not kept in the tree.
+    subprocess.run([sys.executable, os.path.join(CSRC, "gen_gemm_wide.py")], check=True, capture_output=True)
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
         objs = list(pool.map(_compile, SOURCES))
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", OUT, *objs]

@@ -1417,7 +1417,7 @@ uint32_t mrl_target_layouts_for_shape(const uint32_t *shape, uint32_t rank, int 
 
 uint32_t mrl_target_kernels(const char **names, uint32_t cap) {
   static const char *const families[] = {
-      "k_gemm", "k_gemm_big", "k_gemv", "k_matmul_generic", "k_sum_splits", "k_conv_i8", "k_conv_generic", "k_conv_generic_wave", "k_unfold",
+      "k_gemm", "k_gemm_big", "k_gemm_wide", "k_gemv", "k_matmul_generic", "k_sum_splits", "k_conv_i8", "k_conv_generic", "k_conv_generic_wave", "k_unfold",
       "k_unfold_gather", "k_attn", "k_attn_merge", "k_softmax_regs", "k_softmax_regs1", "k_softmax_short", "k_softmax_block", "k_softmax_chunk_stats", "k_softmax_chunk_write",
       "k_softmax_cols",
       "k_softmax_generic", "k_parts", "k_broadcast", "k_fill", "k_fill_zero", "k_move_rows", "k_move_rows16",

@@ -5,6 +5,7 @@
 #include <algorithm>
 
 #include "gemm_big_kernel.h"
+#include "gemm_wide_kernel.h"
 #include "gemm_mfma_kernel.h"
 
 namespace mrl {
@@ -91,8 +92,16 @@ uint32_t gemm_k_splits(const GemmArgs &g, int kind) {
 hipError_t launch_gemm_big(const GemmArgs &g, int kind, hipStream_t stream) {
   if (g.b_kmajor) return launch_gemm_nt(g, kind, 256, stream);
   const bool whole = whole_tiles(g, elem_size_of(kind));
-  // Whole tiles and an even number of k steps: the tile with the hand-scheduled k loop
-  // (int8 4096^3 accumulating: 78 us against 87 us for the compiler-scheduled loop).
+  // Whole tiles and an even number of k steps: the tiles with hand-scheduled k loops.  With a K
+  // long enough for its first steps to carry C's old values, four waves with 128 x 128 outputs each
+  // (int8 4096^3 accumulating: 69 us; eight waves of 128 x 64: 76 us; the compiler-scheduled loop: 87 us).
+  if (whole && kind <= 2 && wide_applicable(g, elem_size_of(kind))) {
+    switch (kind) {
+      case 0: return launch_wide<I8, false>(g, stream);
+      case 1: return launch_wide<I8, true>(g, stream);
+      case 2: return launch_wide<BF16, false>(g, stream);
+    }
+  }
   if (whole && kind <= 2 && big_applicable(g, elem_size_of(kind))) {
     switch (kind) {
       case 0: return launch_big<I8, false>(g, stream);

@@ -1,0 +1,478 @@
+#!/usr/bin/env python3
+"""Writes gemm_wide_gfx950.inc: the 256 x 256 Matmul tile on four waves, one per SIMD, each with a
+128 x 128 block of C in 256 accumulation registers; k loop and epilogue in gfx950 assembly.
+
+Why this shape.  Measured on the matrix cores of an MI355X: an MFMA of 32 x 32 x 32 bytes keeps a
+SIMD's matrix core busy for 32 cycles, and about four and a half other instructions of the waves
+of that SIMD issue under it for free; every further one delays the next MFMA by about four
+cycles, whichever wave it comes from.  So the k loop wants as few instructions per MFMA as it
+can get: the largest block of C per wave (operands read from LDS once serve four MFMAs each way)
+and one wave per SIMD (no per-wave bookkeeping twice).  Per 32-byte slab of K a wave issues
+16 MFMAs against 12 LDS reads (4 ds_read_b128 of A, 8 transposing ds_read_b64_tr of B).
+
+One k step (tile kt, 128 bytes of K, four slabs):
+  * the operands of slab s + 1 are read from LDS behind the first MFMAs of slab s;
+  * A of tile kt + 1 goes from a register set to its LDS stage (xor 0x80 on the way for a u8
+    operand: a - 128, once per byte) and the set is refilled with tile kt + 3 from global memory:
+    two register sets, two LDS stages;
+  * B of tile kt + 2 is requested straight into the third of three LDS slots
+    (global_load_lds_dwordx4; one M0 per step, the instructions' immediate offsets, added to both
+    addresses, tell the pieces apart);
+  * the column sums of B that the u8 correction needs are added up from the B operand registers
+    (xor 0x80, sum of unsigned bytes: b + 128; the dot-product instructions hold up the MFMAs
+    behind them); the two wave rows share the columns and take every other slab each;
+  * one barrier, before the MFMAs of the last slab, preceded by the step's wait for memory:
+    everything requested before this step began has landed;
+  * an accumulating Spec loads C's old values during the first sixteen steps, one block a step,
+    and adds them to the block's accumulators a step later, between two of the block's MFMAs,
+    so that the epilogue only stores.
+
+Register map (all named in the clobber list of the asm statement):
+  a[0:255]    accumulators, block (tm, tn) at 16 * (4 * tm + tn)
+  v[0:63]     A staging, set p chunk i at 32 * p + 4 * i; after the loop: values on their way to C
+  v[64:95]    A operands, buffer b block tm at 64 + 16 * b + 4 * tm
+  v[96:127]   B operands, buffer b block tn at 96 + 16 * b + 4 * tn
+  v[128:131]  LDS address of the lane's B operand, per tn, in the slot being read
+  v[132:135]  column sums of B (u8 correction), one per tn; after the loop: 128 * column sum
+  v[136:137]  scratch
+  v[140:171]  old values of two blocks of C
+  s[60:61] A tile pointer   s[62:63] B tile pointer   s64 loop counter   s67 index of the next
+  A tile to fetch, s68 of the next B tile   s71 byte offset of tile kt's B slot   s[72:73] C block row pointer
+  s65, s66, s69, s70, s[78:81] scratch
+"""
+import os
+import sys
+
+A_STAGE = 32768
+B_SLOT = 32768
+B_BASE = 2 * A_STAGE
+SLAB_BYTES = 8192   # one 32-byte slab of K in a B slot: its k rows x 256 (i8) / 512 (bf16) bytes
+HI_BYTES = 2048     # second transposing read of a slab
+TM, TN = 4, 4       # MFMA blocks per wave
+MF = TM * TN        # MFMAs per slab
+GAPS = 4 * MF       # MFMAs per k step
+GAP_SLOTS = 6       # instructions placed behind one MFMA before the next is due
+C_STEPS = 16        # k steps that carry the loads of C's old values (16 registers a step)
+
+
+def acc(tm, tn):
+    b = 16 * (TN * tm + tn)
+    return f"a[{b}:{b + 15}]"
+
+
+def areg(p, i, w=None):
+    b = 32 * p + 4 * i
+    return f"v[{b}:{b + 3}]" if w is None else f"v{b + w}"
+
+
+def af(buf, tm):
+    b = 64 + 16 * buf + 4 * tm
+    return f"v[{b}:{b + 3}]"
+
+
+def bf(buf, tn, half=None, w=None):
+    b = 96 + 16 * buf + 4 * tn
+    if w is not None:
+        return f"v{b + w}"
+    if half is None:
+        return f"v[{b}:{b + 3}]"
+    return f"v[{b + 2 * half}:{b + 2 * half + 1}]"
+
+
+class Emitter:
+    """Collects instructions; derives s_waitcnt from the order of LDS and vector memory operations."""
+
+    def __init__(self):
+        self.lines = []
+        self.lds_issued = 0
+        self.lds_done = 0
+        self.producer = {}      # register name -> index of the LDS read that fills it
+        self.vm_issued = 0
+        self.vm_done = 0        # vector memory operations with index < vm_done are known complete
+        self.vm_producer = {}
+
+    def emit(self, text):
+        self.lines.append(text)
+
+    def lds_read(self, dst, text):
+        self.producer[dst] = self.lds_issued
+        self.lds_issued += 1
+        self.emit(text)
+
+    def lds_write(self, text):
+        self.lds_issued += 1
+        self.emit(text)
+
+    def need(self, *regs):
+        idx = max((self.producer.get(r, -1) for r in regs), default=-1)
+        if idx >= self.lds_done:
+            allowed = self.lds_issued - idx - 1
+            self.emit(f"s_waitcnt lgkmcnt({min(allowed, 15)})")
+            self.lds_done = idx + 1 if allowed <= 15 else self.lds_issued - 15
+
+    def all_lds_done(self):
+        self.lds_done = self.lds_issued
+
+    def vm(self, text, dst=None):
+        if dst is not None:
+            self.vm_producer[dst] = self.vm_issued
+        self.vm_issued += 1
+        self.emit(text)
+
+    def vm_wait_index(self, idx):
+        """Every vector memory operation up to and including index idx has completed."""
+        if idx >= self.vm_done:
+            allowed = min(self.vm_issued - idx - 1, 63)   # the counter holds 63 at most
+            self.emit(f"s_waitcnt vmcnt({allowed})")
+            self.vm_done = self.vm_issued - allowed
+
+    def vm_need(self, reg):
+        self.vm_wait_index(self.vm_producer.get(reg, -1))
+
+
+class Item:
+    """A piece of work to place behind some MFMA of a step: fn emits it, cost is its instruction
+    count, earliest / latest the gaps (MFMA indices) it may go to, after an Item it follows."""
+
+    def __init__(self, fn, cost, earliest=0, latest=GAPS - 1, after=None):
+        self.fn, self.cost, self.earliest, self.latest, self.after = fn, cost, earliest, latest, after
+        self.gap = None
+
+
+def gen(kind, wm, accum, opts=None):
+    """kind: 'u8' (A unsigned bytes), 'i8', 'bf16'.  wm: the wave row (which slabs' column sums it adds).
+    accum: the Spec accumulates into C (its old contents are read)."""
+    opts = opts or {}     # experiment switches; the shipped loops are generated with none
+    unsigned = kind == "u8" and not opts.get("no_valu")
+    is_float = kind == "bf16"
+    mfma = "v_mfma_f32_32x32x16_bf16" if is_float else "v_mfma_i32_32x32x32_i8"
+    tr = "ds_read_b64_tr_b16" if is_float else "ds_read_b64_tr_b8"
+    e = Emitter()
+    E = e.emit
+
+    def advance(ptr_lo, ptr_hi, idx, step):
+        """Next tile: one k step on; past the last tile the pointer stays (that tile is fetched
+        again, into places nobody reads)."""
+        E(f"s_add_u32 {idx}, {idx}, 1")
+        E(f"s_cmp_lt_u32 {idx}, %[nk]")
+        E(f"s_cselect_b32 s69, {step}, 0")
+        E(f"s_add_u32 {ptr_lo}, {ptr_lo}, s69")
+        E(f"s_addc_u32 {ptr_hi}, {ptr_hi}, 0")
+
+    def advance_a():
+        advance("s60", "s61", "s67", "128")
+
+    def advance_b():
+        advance("s62", "s63", "s68", "%[bstep]")
+
+    def load_a(p, i):
+        e.vm(f"global_load_dwordx4 {areg(p, i)}, %[a_off{i}], s[60:61]", dst=areg(p, i))
+
+    def store_a(p, i, stage):
+        e.vm_need(areg(p, i))
+        if unsigned:
+            for w in range(4):
+                E(f"v_xor_b32 {areg(p, i, w)}, 0x80808080, {areg(p, i, w)}")
+        e.lds_write(f"ds_write_b128 %[a_wr], {areg(p, i)} offset:{stage * A_STAGE + i * 4096}")
+
+    def set_m0(base_sgpr):
+        E(f"s_add_u32 m0, {base_sgpr}, 4096")   # the immediate offsets run from -4096 to 3072
+        E("s_nop 0")                              # one wait state before M0 is read
+
+    def dma_b(j):
+        e.vm(f"global_load_lds_dwordx4 %[b_off{j}], s[62:63] offset:{j * 1024 - 4096}")
+
+    def a_read(stage, slab, buf, tm):
+        return lambda: e.lds_read(af(buf, tm), f"ds_read_b128 {af(buf, tm)}, %[a_rd{slab}] offset:{stage * A_STAGE + tm * 4096}")
+
+    def b_read(slab, buf, tn, half):
+        reg = bf(buf, tn, half)
+        return lambda: e.lds_read(reg, f"{tr} {reg}, v{128 + tn} offset:{slab * SLAB_BYTES + half * HI_BYTES}")
+
+    def reads(stage, slab, buf):
+        """The operand reads of one slab in the order the MFMAs want them, one list per gap."""
+        out = [[a_read(stage, slab, buf, 0)]]
+        for tn in range(TN):
+            out.append([b_read(slab, buf, tn, 0), b_read(slab, buf, tn, 1)])
+        for tm in range(1, TM):
+            out.append([a_read(stage, slab, buf, tm)])
+        return out
+
+    def set_b_read_base(slot_off_sgpr):
+        for tn in range(TN):
+            E(f"v_add_u32 v{128 + tn}, {slot_off_sgpr}, %[b_rd{tn}]")
+
+    # ---- prologue -------------------------------------------------------------------------
+    E("s_mov_b64 s[60:61], %[abase]")
+    E("s_mov_b64 s[62:63], %[bbase]")
+    E("s_mov_b32 s67, 0")
+    E("s_mov_b32 s68, 0")
+    E("s_mov_b32 s71, 0")
+    # A tiles 0 and 1 into the two register sets, B tiles 0 and 1 into slots 0 and 1
+    for p in range(2):
+        for i in range(8):
+            load_a(p, i)
+        advance_a()
+    for slot in range(2):
+        E(f"s_add_u32 s66, %[dma_base], {slot * B_SLOT}")
+        set_m0("s66")
+        for j in range(8):
+            dma_b(j)
+        advance_b()
+    for tn in range(TN):
+        E(f"v_mov_b32 v{132 + tn}, 0")
+    for i in range(8):
+        store_a(0, i, 0)            # waits for A tile 0 only
+    for i in range(8):
+        load_a(0, i)                # A tile 2
+    advance_a()
+    e.vm_wait_index(e.vm_issued - 9)  # all but A tile 2: B tiles 0 and 1 have landed
+    E("s_waitcnt lgkmcnt(0)")
+    e.all_lds_done()
+    E("s_barrier")
+    E(f"s_mov_b32 s65, {B_BASE}")
+    set_b_read_base("s65")
+    for group in reads(0, 0, 0):
+        for r in group:
+            r()
+
+    # ---- one k step ----------------------------------------------------------------------
+    def step(cur, zero_first=False, extra=()):
+        """cur: LDS stage of tile kt.  zero_first: the accumulators start from zero in this step.
+        extra: Items to place in the gaps besides the step's own."""
+        p = cur ^ 1  # register set holding tile kt + 1 = LDS stage it goes to
+        vm_before_step = e.vm_issued
+        items = []
+
+        def add(fn, cost, earliest, latest=GAPS - 1, after=None):
+            items.append(Item(fn, cost, earliest, latest, after))
+            return items[-1]
+
+        def header():
+            # s69: slot of tile kt + 1 (read after the barrier); s70: slot of tile kt + 2 (fetched now)
+            E(f"s_add_u32 s69, s71, {B_SLOT}")
+            E(f"s_cmp_eq_u32 s69, {3 * B_SLOT}")
+            E("s_cselect_b32 s69, 0, s69")
+            E(f"s_sub_u32 s70, s71, {B_SLOT}")
+            E("s_cmp_eq_u32 s71, 0")
+            E(f"s_cselect_b32 s70, {2 * B_SLOT}, s70")
+            E("s_add_u32 s66, %[dma_base], s70")
+            E(f"s_add_u32 s65, s69, {B_BASE}")
+            E("s_mov_b32 s71, s69")
+        # The step's own work.  LDS writes must be out before the barrier.
+        last_a = None
+        for i, g in enumerate([2, 8, 14, 20, 26, 32, 38, 44]):
+            last_a = add(lambda i=i: (store_a(p, i, cur ^ 1), load_a(p, i)), 6 if unsigned else 2, g, 3 * MF - 1)
+        m0 = add(lambda: set_m0("s66"), 2, 0)
+        last_b = m0
+        for j, g in enumerate([5, 11, 17, 23, 29, 35, 41, 46]):
+            last_b = add(lambda j=j: dma_b(j), 1, g, after=last_b)
+        add(advance_a, 5, 45, after=last_a)
+        add(advance_b, 5, 47, after=last_b)
+        if unsigned:
+            for s in range(4):
+                if s % 2 != wm:
+                    continue
+                for tn in range(TN):
+                    for w in range(4):
+                        # after the MFMA that waited for this operand, before the reads that overwrite it
+                        add(lambda s=s, tn=tn, w=w: (e.need(bf(s & 1, tn, w // 2)),
+                                                      E(f"v_xor_b32 v136, 0x80808080, {bf(s & 1, tn, w=w)}"),
+                                                      E(f"v_sad_u8 v{132 + tn}, v136, 0, v{132 + tn}")),
+                            2, MF * s + tn, min(GAPS - 1, MF * s + MF + tn))
+        for it in extra:
+            items.append(it)
+        # operand reads: fixed places
+        read_at = {}
+        for s in range(3):
+            for n, group in enumerate(reads(cur, s + 1, (s + 1) & 1)):
+                read_at[MF * s + n] = group
+        for n, group in enumerate(reads(cur ^ 1, 0, 0)):
+            read_at[MF * 3 + n] = group
+        # Place the items in the order given, each into the first gap from its earliest on with room.
+        room = [GAP_SLOTS - len(read_at.get(g, [])) for g in range(GAPS)]
+        room[3 * MF - 1] -= 3              # the waits and the barrier
+        placed = [[] for _ in range(GAPS)]
+        for it in items:
+            first = max(it.earliest, it.after.gap if it.after is not None else 0)
+            last_gap = max(first, it.latest)
+            g = first
+            while g <= last_gap and room[g] < it.cost:
+                g += 1
+            if g > last_gap:               # no gap has room: the emptiest one allowed
+                g = max(range(first, last_gap + 1), key=lambda x: (room[x], -x))
+            room[g] -= it.cost
+            it.gap = g
+            placed[g].append(it)
+        if os.environ.get("WIDE_SHOW_GAPS"):
+            sys.stderr.write("gaps " + " ".join(str(GAP_SLOTS - r) for r in room) + "\n")
+
+        def sync():
+            # everything requested before this step has landed (B of tile kt + 1, A of tile kt + 2);
+            # this wave's LDS writes are done and the operands of this slab are in
+            e.vm_wait_index(vm_before_step - 1)
+            E("s_waitcnt lgkmcnt(0)")
+            e.all_lds_done()
+            E("s_barrier")
+            set_b_read_base("s65")
+
+        header()
+        n = 0
+        for s in range(4):
+            buf = s & 1
+            if s == 3:
+                sync()
+            for tm in range(TM):
+                for tn in range(TN):
+                    e.need(af(buf, tm), bf(buf, tn, 0), bf(buf, tn, 1))
+                    src_c = "0" if (zero_first and s == 0) else acc(tm, tn)
+                    E(f"{mfma} {acc(tm, tn)}, {af(buf, tm)}, {bf(buf, tn)}, {src_c}")
+                    for r in read_at.get(n, []):
+                        r()
+                    for it in placed[n]:
+                        it.fn()
+                    n += 1
+
+    # ---- C: register q = 0..255: block q / 16 (tm = block / 4, tn = block % 4), register r = q % 16,
+    # which holds row 8 * (r / 4) + 4 * (lane / 32) + r % 4 of the block (%[c_row r]) and column lane % 32.
+    ptr_tm = [None]
+
+    def c_ptr(tm):
+        """s[72:73] = the wave's corner of C + tm * 32 rows, if it is not that already."""
+        if ptr_tm[0] == tm:
+            return
+        ptr_tm[0] = tm
+        E("s_mov_b64 s[72:73], %[cbase]")
+        if tm:
+            E(f"s_mul_i32 s78, %[ldc32], {tm}")
+            E(f"s_mul_hi_u32 s79, %[ldc32], {tm}")
+            E("s_add_u32 s72, s72, s78")
+            E("s_addc_u32 s73, s73, s79")
+
+    def where(q):
+        block = q // 16
+        return block // TN, block % TN, q % 16
+
+    def old_values(j):
+        """C's old values of block j into bank j % 2 of the temporaries: one step before they are added."""
+        tm, tn = j // TN, j % TN
+        out = []
+        for r in range(16):
+            reg = f"v{140 + 16 * (j & 1) + r}"
+
+            def ld(r=r, reg=reg):
+                c_ptr(tm)
+                e.vm(f"global_load_dword {reg}, %[c_row{r}], s[72:73] offset:{tn * 128}", dst=reg)
+            out.append(Item(ld, 1, 3 * r))
+        return out
+
+    def add_old_values(j):
+        """The old values of block j join its accumulators between two of the block's MFMAs (which
+        come 16 apart): an MFMA's result may be read four MFMAs after it at the earliest, and a
+        register written for the block's next MFMA wants another instruction in between."""
+        out = []
+        for r in range(16):
+            s = r * 3 // 16                      # behind the block's MFMA of slab 0, 1 or 2
+            first, last = MF * s + j + 4, MF * s + j + 14
+            k = r - (16 * s + 2) // 3            # position among the registers of this window
+            reg = f"v{140 + 16 * (j & 1) + r}"
+
+            def rmw(r=r, reg=reg):
+                q = 16 * j + r
+                e.vm_need(reg)
+                E(f"v_accvgpr_read_b32 v137, a{q}")
+                E(f"v_add_f32 v137, v137, {reg}" if is_float else f"v_add_u32 v137, v137, {reg}")
+                E(f"v_accvgpr_write_b32 a{q}, v137")
+            out.append(Item(rmw, 3, min(last, first + 2 * max(0, k)), last))
+        return out
+
+    def loop():
+        E("1:")
+        step(0)
+        step(1)
+        E("s_sub_u32 s64, s64, 2")
+        E("s_cmp_lg_u32 s64, 0")
+        E("s_cbranch_scc1 1b")
+
+    # ---- the k loop ---------------------------------------------------------------------------------
+    unrolled = C_STEPS + 2 if accum else 2
+    for j in range(unrolled):
+        extra = []
+        if accum and j < C_STEPS and not opts.get("no_cops"):
+            extra += old_values(j)
+        if accum and 1 <= j <= C_STEPS and not opts.get("no_cops"):
+            extra += add_old_values(j - 1)
+        step(j & 1, zero_first=(j == 0), extra=extra)
+    E(f"s_sub_u32 s64, %[nk], {unrolled}")
+    E("s_cmp_eq_u32 s64, 0")
+    E("s_cbranch_scc1 2f")
+    loop()
+    E("2:")
+    # nothing may land in LDS once the epilogue reuses it; the last MFMAs must have written the
+    # accumulators before they are read
+    E("s_waitcnt vmcnt(0) lgkmcnt(0)")
+    E("s_barrier")
+
+    # ---- epilogue -----------------------------------------------------------------------------------
+    if unsigned:
+        # Column sums: the partials of the two wave rows and the two lane halves meet in LDS
+        # (each summed K / 4 values of b + 128).
+        for tn in range(TN):
+            E(f"v_subrev_u32 v{132 + tn}, %[k32], v{132 + tn}")
+            e.lds_write(f"ds_write_b32 %[part_wr], v{132 + tn} offset:{tn * 128}")
+        E("s_waitcnt lgkmcnt(0)")
+        e.all_lds_done()
+        E("s_barrier")
+        for tn in range(TN):
+            for w in range(4):
+                reg = f"v{4 * tn + w}"
+                e.lds_read(reg, f"ds_read_b32 {reg}, %[part_rd] offset:{w * 1024 + tn * 128}")
+        for tn in range(TN):
+            regs = [f"v{4 * tn + w}" for w in range(4)]
+            e.need(*regs)
+            E(f"v_add3_u32 v{132 + tn}, {regs[0]}, {regs[1]}, {regs[2]}")
+            E(f"v_add_lshl_u32 v{132 + tn}, v{132 + tn}, {regs[3]}, 7")
+    else:
+        E("s_nop 15")
+        E("s_nop 15")
+    for q in range(0 if not opts.get("no_epilogue") else 256, 256):
+        tm, tn, r = where(q)
+        c_ptr(tm)
+        if not unsigned:
+            E(f"global_store_dword %[c_row{r}], a{q}, s[72:73] offset:{tn * 128}")
+        else:
+            t = f"v{16 + q % 32}"
+            E(f"v_accvgpr_read_b32 {t}, a{q}")
+            E(f"v_add_u32 {t}, {t}, v{132 + tn}")
+            E(f"global_store_dword %[c_row{r}], {t}, s[72:73] offset:{tn * 128}")
+    return e.lines
+
+
+MIN_STEPS = C_STEPS + 4   # k steps a problem needs: the steps that carry C's old values, then the loop
+
+
+def variants():
+    for kind, wms in (("u8", (0, 1)), ("i8", (0,)), ("bf16", (0,))):
+        for wm in wms:
+            for accum in (False, True):
+                name = f"GEMM_WIDE_{kind.upper()}" + (f"_{wm}" if kind == "u8" else "") + ("_ACC" if accum else "")
+                yield name, kind, wm, accum
+
+
+def main():
+    out_path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "gemm_wide_gfx950.inc")
+    if len(sys.argv) > 1:
+        out_path = sys.argv[1]
+    parts = ["// Generated by gen_gemm_wide.py -- do not edit; the generator documents the schedule.\n",
+             f"#define GEMM_WIDE_MIN_STEPS {MIN_STEPS}\n"]
+    for name, kind, wm, accum in variants():
+        lines = gen(kind, wm, accum)
+        body = " \\\n".join('  "' + l + '\\n"' for l in lines)
+        parts.append(f"#define {name} \\\n{body}\n")
+    with open(out_path, "w") as f:
+        f.write("\n".join(parts))
+    print(f"wrote {out_path}")
+
+
+if __name__ == "__main__":
+    main()

@@ -69,7 +69,7 @@ int main() {
   {
     const Plan p = Spec::matmul({1, 4096, 4096, 4096}, Dtype::Uint8, Dtype::Sint8, Dtype::Sint32).plan();
     EXPECT(p.steps.size() == 1 && p.scratch_bytes == 0 && p.cost_ns > 20e3 && p.cost_ns < 500e3);
-    EXPECT(std::string(p.steps[0].kernel).find("k_gemm_big [T = I8, A_UNSIGNED = true") == 0);
+    EXPECT(std::string(p.steps[0].kernel).find("k_gemm_wide [T = I8, A_UNSIGNED = true") == 0);
     EXPECT(std::string(mrl_target_id()) == "Gfx950" && mrl_target_memories(nullptr, 0) == 4);
     const mrl_matmul_schedule best =
         Spec::matmul({1, 4096, 4096, 4096}, Dtype::Uint8, Dtype::Sint8, Dtype::Sint32).search_schedule();
