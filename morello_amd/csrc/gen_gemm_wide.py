@@ -166,9 +166,13 @@ def gen(kind, wm, accum, opts=None):
         advance("s62", "s63", "s68", "%[bstep]")
 
     def load_a(p, i):
+        if opts.get("no_stage"):
+            return
         e.vm(f"global_load_dwordx4 {areg(p, i)}, %[a_off{i}], s[60:61]", dst=areg(p, i))
 
     def store_a(p, i, stage):
+        if opts.get("no_stage"):
+            return
         e.vm_need(areg(p, i))
         if unsigned:
             for w in range(4):
@@ -180,13 +184,19 @@ def gen(kind, wm, accum, opts=None):
         E("s_nop 0")                              # one wait state before M0 is read
 
     def dma_b(j):
+        if opts.get("no_dma"):
+            return
         e.vm(f"global_load_lds_dwordx4 %[b_off{j}], s[62:63] offset:{j * 1024 - 4096}")
 
     def a_read(stage, slab, buf, tm):
+        if opts.get("no_reads"):
+            return lambda: None
         return lambda: e.lds_read(af(buf, tm), f"ds_read_b128 {af(buf, tm)}, %[a_rd{slab}] offset:{stage * A_STAGE + tm * 4096}")
 
     def b_read(slab, buf, tn, half):
         reg = bf(buf, tn, half)
+        if opts.get("no_reads"):
+            return lambda: None
         return lambda: e.lds_read(reg, f"{tr} {reg}, v{128 + tn} offset:{slab * SLAB_BYTES + half * HI_BYTES}")
 
     def reads(stage, slab, buf):
@@ -203,6 +213,10 @@ def gen(kind, wm, accum, opts=None):
             E(f"v_add_u32 v{128 + tn}, {slot_off_sgpr}, %[b_rd{tn}]")
 
     # ---- prologue -------------------------------------------------------------------------
+    if opts.get("trace") or opts.get("stamp"):
+        for r in (88, 89, 90):
+            E(f"s_mov_b32 s{r}, 0")
+        E("s_memtime s[92:93]")
     E("s_mov_b64 s[60:61], %[abase]")
     E("s_mov_b64 s[62:63], %[bbase]")
     E("s_mov_b32 s67, 0")
@@ -260,6 +274,9 @@ def gen(kind, wm, accum, opts=None):
             E(f"s_add_u32 s65, s69, {B_BASE}")
             E("s_mov_b32 s71, s69")
         # The step's own work.  LDS writes must be out before the barrier.
+        # (Issuing these at different gaps in each of the four waves was measured and changes nothing:
+        # a vector memory or LDS write instruction costs its wave about 13 cycles of MFMA issue
+        # whether or not the other waves issue theirs at the same moment.)
         last_a = None
         for i, g in enumerate([2, 8, 14, 20, 26, 32, 38, 44]):
             last_a = add(lambda i=i: (store_a(p, i, cur ^ 1), load_a(p, i)), 6 if unsigned else 2, g, 3 * MF - 1)
@@ -310,10 +327,26 @@ def gen(kind, wm, accum, opts=None):
         def sync():
             # everything requested before this step has landed (B of tile kt + 1, A of tile kt + 2);
             # this wave's LDS writes are done and the operands of this slab are in
+            if opts.get("trace"):
+                E("s_memtime s[80:81]")
+                E("s_waitcnt lgkmcnt(0)")
+                E("s_memtime s[82:83]")
             e.vm_wait_index(vm_before_step - 1)
             E("s_waitcnt lgkmcnt(0)")
             e.all_lds_done()
+            if opts.get("trace"):
+                E("s_memtime s[84:85]")
+                E("s_waitcnt lgkmcnt(0)")
             E("s_barrier")
+            if opts.get("trace"):
+                E("s_memtime s[86:87]")
+                E("s_waitcnt lgkmcnt(0)")
+                E("s_sub_u32 s80, s82, s80")
+                E("s_add_u32 s88, s88, s80")
+                E("s_sub_u32 s80, s84, s82")
+                E("s_add_u32 s89, s89, s80")
+                E("s_sub_u32 s80, s86, s84")
+                E("s_add_u32 s90, s90, s80")
             set_b_read_base("s65")
 
         header()
@@ -412,6 +445,10 @@ def gen(kind, wm, accum, opts=None):
     # accumulators before they are read
     E("s_waitcnt vmcnt(0) lgkmcnt(0)")
     E("s_barrier")
+    if opts.get("trace") or opts.get("stamp"):
+        E("s_memtime s[94:95]")
+        E("s_waitcnt lgkmcnt(0)")
+        E("s_sub_u32 s91, s94, s92")
 
     # ---- epilogue -----------------------------------------------------------------------------------
     if unsigned:
