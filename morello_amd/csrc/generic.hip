@@ -41,7 +41,24 @@ __device__ inline float load_f32(const void *p, int dtype, int64_t off) {
   }
 }
 
-// Rust `as` semantics: integers wrap, floats saturate and NaN becomes 0.
+// Rust `as` for narrow integer targets saturates floats at the target's own bounds.
+__device__ inline uint32_t float_to_int(float f, int dt) {
+  if (f != f) return 0;
+  float lo, hi;
+  switch (dt) {
+    case MRL_U8: lo = 0.f, hi = 255.f; break;
+    case MRL_I8: lo = -128.f, hi = 127.f; break;
+    case MRL_U16: lo = 0.f, hi = 65535.f; break;
+    case MRL_I16: lo = -32768.f, hi = 32767.f; break;
+    case MRL_U32: return f <= 0.f ? 0u : f >= 4294967296.f ? 0xffffffffu : uint32_t(f);
+    default: return f <= -2147483648.f ? 0x80000000u : f >= 2147483648.f ? 0x7fffffffu : uint32_t(int32_t(f));
+  }
+  f = fminf(fmaxf(f, lo), hi);
+  return uint32_t(int32_t(f));
+}
+
+// Rust `as` semantics (verification.rs:547-569, `x.as_()` into the output dtype): integers wrap,
+// floats saturate at the bounds of the dtype they are cast to and NaN becomes 0.
 __device__ inline uint32_t load_u32(const void *p, int dtype, int64_t off, int out_dtype) {
   uint32_t v;
   switch (dtype) {
@@ -51,13 +68,7 @@ __device__ inline uint32_t load_u32(const void *p, int dtype, int64_t off, int o
     case MRL_I16: v = uint32_t(int32_t(((const int16_t *)p)[off])); break;
     case MRL_U32: v = ((const uint32_t *)p)[off]; break;
     case MRL_I32: v = uint32_t(((const int32_t *)p)[off]); break;
-    default: {
-      const float f = load_f32(p, dtype, off);
-      const bool sgn = out_dtype == MRL_I8 || out_dtype == MRL_I16 || out_dtype == MRL_I32;
-      if (f != f) v = 0;
-      else if (sgn) v = f <= -2147483648.0f ? 0x80000000u : f >= 2147483648.0f ? 0x7fffffffu : uint32_t(int32_t(f));
-      else v = f <= 0.0f ? 0u : f >= 4294967296.0f ? 0xffffffffu : uint32_t(f);
-    }
+    default: v = float_to_int(load_f32(p, dtype, off), out_dtype);
   }
   return narrow_int(out_dtype, v);
 }
@@ -93,22 +104,6 @@ __device__ inline uint16_t f32_to_bf16_bits(float f) {
   if ((bits & 0x7fffffffu) > 0x7f800000u) return uint16_t((bits >> 16) | 0x40u);
   bits += 0x7fffu + ((bits >> 16) & 1u);  // round to nearest even
   return uint16_t(bits >> 16);
-}
-
-// Rust `as` for narrow integer targets saturates floats at the target's own bounds.
-__device__ inline uint32_t float_to_int(float f, int dt) {
-  if (f != f) return 0;
-  float lo, hi;
-  switch (dt) {
-    case MRL_U8: lo = 0.f, hi = 255.f; break;
-    case MRL_I8: lo = -128.f, hi = 127.f; break;
-    case MRL_U16: lo = 0.f, hi = 65535.f; break;
-    case MRL_I16: lo = -32768.f, hi = 32767.f; break;
-    case MRL_U32: return f <= 0.f ? 0u : f >= 4294967296.f ? 0xffffffffu : uint32_t(f);
-    default: return f <= -2147483648.f ? 0x80000000u : f >= 2147483648.f ? 0x7fffffffu : uint32_t(int32_t(f));
-  }
-  f = fminf(fmaxf(f, lo), hi);
-  return uint32_t(int32_t(f));
 }
 
 // One element: read as `sdt`, converted with Rust `as` semantics, returned as the bits of `ddt`.

@@ -264,12 +264,35 @@ static uint32_t narrow_to(int dtype, uint32_t v) {
   }
 }
 
+/* Rust `as` from a float to an integer dtype: saturates at that dtype's own bounds, NaN -> 0
+ * (verification.rs:547-569 casts every operand with `x.as_()` into the output dtype). */
+static uint32_t float_as_int(float f, int out_dtype) {
+  float lo, hi;
+  if (f != f) return 0;
+  switch (out_dtype) {
+    case ORC_U8: lo = 0.0f, hi = 255.0f; break;
+    case ORC_I8: lo = -128.0f, hi = 127.0f; break;
+    case ORC_U16: lo = 0.0f, hi = 65535.0f; break;
+    case ORC_I16: lo = -32768.0f, hi = 32767.0f; break;
+    case ORC_U32: return f <= 0.0f ? 0u : f >= 4294967296.0f ? 0xffffffffu : (uint32_t)f;
+    default: return f <= -2147483648.0f ? 0x80000000u : f >= 2147483648.0f ? 0x7fffffffu : (uint32_t)(int32_t)f;
+  }
+  if (f < lo) f = lo;
+  if (f > hi) f = hi;
+  return (uint32_t)(int32_t)f;
+}
+
 static uint32_t *gather_u32(const void *buf, int dtype, const int64_t *tab, size_t n,
                             int out_dtype) {
   uint32_t *dst = (uint32_t *)malloc(sizeof(uint32_t) * (n ? n : 1));
   int sgn = out_is_signed(out_dtype);
-  for (size_t i = 0; i < n; i++)
-    dst[i] = narrow_to(out_dtype, load_as_u32(buf, dtype, tab ? tab[i] : (int64_t)i, sgn));
+  for (size_t i = 0; i < n; i++) {
+    int64_t off = tab ? tab[i] : (int64_t)i;
+    if (is_float(dtype))
+      dst[i] = narrow_to(out_dtype, float_as_int(load_as_f32(buf, dtype, off), out_dtype));
+    else
+      dst[i] = narrow_to(out_dtype, load_as_u32(buf, dtype, off, sgn));
+  }
   return dst;
 }
 
@@ -493,18 +516,6 @@ int orc_compose_msm(uint32_t b, uint32_t m, uint32_t k, uint32_t n2, uint32_t n,
 }
 
 /* -------------------------------------------------------------------- move */
-
-static uint32_t float_as_int(float f, int dt) {
-  if (f != f) return 0;
-  switch (dt) {
-    case ORC_U8: return f <= 0.f ? 0u : f >= 255.f ? 255u : (uint32_t)f;
-    case ORC_I8: return (uint32_t)(int32_t)(f <= -128.f ? -128 : f >= 127.f ? 127 : (int32_t)f);
-    case ORC_U16: return f <= 0.f ? 0u : f >= 65535.f ? 65535u : (uint32_t)f;
-    case ORC_I16: return (uint32_t)(int32_t)(f <= -32768.f ? -32768 : f >= 32767.f ? 32767 : (int32_t)f);
-    case ORC_U32: return f <= 0.f ? 0u : f >= 4294967296.f ? 0xffffffffu : (uint32_t)f;
-    default: return f <= -2147483648.f ? 0x80000000u : f >= 2147483648.f ? 0x7fffffffu : (uint32_t)(int32_t)f;
-  }
-}
 
 int orc_move(const uint32_t *shape, uint32_t rank, const int dtypes[2], const orc_layout *layouts[2],
              const void *in, void *out) {

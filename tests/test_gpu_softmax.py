@@ -4,7 +4,7 @@ import pytest
 
 import morello_amd as M
 import orc
-from gpu_util import rel_err, run_spec
+from gpu_util import elem_err, rel_err, run_spec
 from morello_amd import synth
 
 pytestmark = pytest.mark.gpu
@@ -289,7 +289,14 @@ def test_compose_msm_full_size(gpu):
     for h in (0, 5, 10, 15):
         want = orc.compose_msm(1, m, k, n2, n, [7, 7, 7, 6], v[h:h + 1], q[h:h + 1], kmat[h:h + 1],
                                np.zeros((1, m, n), np.float32), layouts=[None, None, KT_ORC, None])
+        # Stated tolerance 1e-2, norm-wise (measured 1e-3).  Element by element: an output is a sum of
+        # 2048 signed terms p * v whose P factors are rounded to bf16 for the second product (half an
+        # ulp, 2^-9, each), so its error is bounded by 2^-9 * sum p |v|, about 1.3e-2 of the RMS
+        # output for these inputs, whatever the element's own value where the terms cancel.  With |r|
+        # floored at that RMS the worst of 262144 elements measures 1.2e-2; the gate of 2e-2 is what
+        # a kernel wrong on small outputs (a dropped key block, a stale row) cannot pass.
         assert rel_err(got[h:h + 1], want) < 1e-2
+        assert elem_err(got[h:h + 1], want, floor_frac=1.0) < 2e-2
     ones = synth.f32_to_bf16_bits(np.ones((b, n2, n), np.float32))
     got = run_spec(spec, [ones, q, kmat, np.zeros((b, m, n), np.float32)])
     assert np.abs(got - 1).max() < 1e-2

@@ -207,6 +207,57 @@ def test_conv_vs_scipy(accum):
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("in_dtype", ["f32", "bf16"])
+def test_conv_float_vs_scipy(in_dtype):
+    """The float branch of the Conv oracle (bf16 or f32 operands, f32 result) against scipy's
+    correlate2d in float64; bf16 operands widen exactly, so only the f32 sum's rounding is left."""
+    b, f, c, oh, ow, fh, fw = 2, 3, 5, 4, 6, 3, 2
+    img = synth.normal_f32(21, 0, (b, c, oh + fh - 1, ow + fw - 1))
+    filt = synth.normal_f32(21, 1, (f, c, fh, fw))
+    if in_dtype == "bf16":
+        img_b, filt_b = synth.f32_to_bf16_bits(img), synth.f32_to_bf16_bits(filt)
+        img, filt = synth.bf16_bits_to_f32(img_b), synth.bf16_bits_to_f32(filt_b)
+        dts, args = [orc.BF16, orc.BF16, orc.F32], (img_b, filt_b)
+    else:
+        dts, args = [orc.F32, orc.F32, orc.F32], (img, filt)
+    out0 = synth.normal_f32(21, 2, (b, f, oh, ow))
+    want = np.zeros((b, f, oh, ow), np.float64)
+    for bi in range(b):
+        for fi in range(f):
+            for ci in range(c):
+                want[bi, fi] += scipy.signal.correlate2d(img[bi, ci].astype(np.float64),
+                                                         filt[fi, ci].astype(np.float64), mode="valid")
+    for accum in (False, True):
+        got = orc.conv([b, f, c, oh, ow, fh, fw], dts, args[0], args[1], out0.copy(), accum)
+        ref = want + (out0 if accum else 0)
+        assert np.abs(got - ref).max() <= 1e-5 * np.abs(ref).max()
+    # a dropped tap or a flipped filter would be far outside: the asymmetric-filter case in floats
+    one = np.zeros((1, 1, 2, 2), np.float32)
+    one[0, 0, 0, 1] = 1.0
+    ramp = np.arange(9, dtype=np.float32).reshape(1, 1, 3, 3)
+    got = orc.conv([1, 1, 1, 2, 2, 2, 2], [orc.F32, orc.F32, orc.F32], ramp, one, np.zeros((1, 1, 2, 2), np.float32))
+    assert np.array_equal(got.reshape(2, 2), [[1, 2], [4, 5]])
+
+
+def test_float_operands_saturate_at_the_output_dtype():
+    """verification.rs:547-569 casts operands with Rust `as` into the output dtype: floats saturate
+    at the bounds of the dtype they are cast to.  Expected values computed by hand from that rule."""
+    a = np.array([[300.0, -200.0, -5.0, 70000.0, np.nan, 2.9]], np.float32)
+    b = np.eye(6, dtype=np.float32)
+    for dt, np_dt, want in ((orc.I8, np.int8, [127, -128, -5, 127, 0, 2]),
+                            (orc.U8, np.uint8, [255, 0, 0, 255, 0, 2]),
+                            (orc.U16, np.uint16, [300, 0, 0, 65535, 0, 2]),
+                            (orc.I16, np.int16, [300, -200, -5, 32767, 0, 2]),
+                            (orc.I32, np.int32, [300, -200, -5, 70000, 0, 2]),
+                            (orc.U32, np.uint32, [300, 0, 0, 70000, 0, 2])):
+        got = orc.matmul([1, 1, 6, 6], [orc.F32, orc.F32, dt], a, b, np.zeros((1, 6), np_dt))
+        assert got.reshape(-1).tolist() == want, dt
+    # and the product wraps in the output dtype like any integer product: 127 * 127 as i8
+    big = np.array([[300.0]], np.float32)
+    got = orc.matmul([1, 1, 1, 1], [orc.F32, orc.F32, orc.I8], big, big, np.zeros((1, 1), np.int8))
+    assert int(got[0, 0]) == np.int8((127 * 127) & 0xff)
+
+
 def test_conv_degenerate_cases():
     # 1x1 filter == Matmul [1, B*H*W, C, F] (scheduling/spatial_split.rs:73-102)
     b, f, c, h, w = 2, 5, 7, 3, 4
