@@ -208,6 +208,19 @@ int mrl_run(const mrl_spec *spec, void *const *params);
  * its stream; the arena of a stream the caller created itself stays until the process ends. */
 int mrl_run_async(const mrl_spec *spec, void *const *params, void *stream);
 
+/* As mrl_run_async, for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid it).  No counterpart in the reference, whose emitted
+ * programs allocate their buffers up front.  Calls no hipMalloc / hipFree / stream-ordered
+ * allocator: scratch comes out of one fixed array of MRL_NOALLOC_SCRATCH_BYTES per GPU, which the
+ * library's code object brings along (each GPU the library runs on holds it until the process
+ * ends).  mrl_init must have been called for the device (it looks the array up).  A Spec whose
+ * scratch need (mrl_spec_plan: scratch_bytes) exceeds the array is turned down with
+ * MRL_ERR_TOO_LARGE before anything is launched.  All calls on one GPU share the array: two that
+ * overlap in time (different streams, or different host threads on one stream) race; the caller
+ * serialises them. */
+#define MRL_NOALLOC_SCRATCH_BYTES (32u << 20)
+int mrl_run_noalloc(const mrl_spec *spec, void *const *params, void *stream);
+
 /* Literal stand-in for calling the emitted kernel from the emitted main
  * (codegen/cpu.rs:284-409): `params` are HOST pointers; inputs (and the output, when it
  * is read) are copied to the device, the Spec is run, written parameters are copied back. */

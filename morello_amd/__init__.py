@@ -24,7 +24,8 @@ class MorelloError(RuntimeError):
         lib = B.load()
         msg = lib.mrl_status_string(status).decode()
         detail = lib.mrl_last_error().decode()
-        super().__init__(f"{where}: {msg}" + (f" ({detail})" if detail and status == 4 else ""))
+        with_detail = status == 4 or where == "mrl_run_noalloc"   # the calls that set the detail they fail with
+        super().__init__(f"{where}: {msg}" + (f" ({detail})" if detail and with_detail else ""))
         self.status = status
 
 
@@ -278,6 +279,12 @@ class Spec:
         """Enqueues the Spec on `stream` and returns; `stream.synchronize()` waits for it."""
         arr = (C.c_void_p * len(ptrs))(*ptrs)
         _check(B.load().mrl_run_async(C.byref(self._c), arr, stream.handle), "mrl_run_async")
+
+    def run_noalloc(self, ptrs: Sequence[int], stream: "Stream | None" = None):
+        """As run_async without any device allocation: scratch comes from the library's fixed
+        per-GPU array (NOALLOC_SCRATCH_BYTES); MorelloError (tensor too large) if the Spec needs more."""
+        arr = (C.c_void_p * len(ptrs))(*ptrs)
+        _check(B.load().mrl_run_noalloc(C.byref(self._c), arr, stream.handle if stream else None), "mrl_run_noalloc")
 
     def run_host(self, *arrays: np.ndarray):
         """`arrays`: numpy buffers in Spec parameter order, each already laid out by its
@@ -702,6 +709,9 @@ def launch_count() -> int:
 
 def synchronize():
     _check(B.load().mrl_device_synchronize(), "mrl_device_synchronize")
+
+
+NOALLOC_SCRATCH_BYTES = 32 << 20   # MRL_NOALLOC_SCRATCH_BYTES
 
 
 def device_info():

@@ -106,6 +106,7 @@ SIGNATURES = {
     "mrl_spec_workspace_bytes": (C.c_size_t, [C.POINTER(SpecC)]),
     "mrl_run": (C.c_int, [C.POINTER(SpecC), _VPP]),
     "mrl_run_async": (C.c_int, [C.POINTER(SpecC), _VPP, C.c_void_p]),
+    "mrl_run_noalloc": (C.c_int, [C.POINTER(SpecC), _VPP, C.c_void_p]),
     "mrl_run_host": (C.c_int, [C.POINTER(SpecC), _VPP]),
     "mrl_matmul": (C.c_int, [C.c_uint32] * 4 + [C.c_int] * 4 + [C.c_void_p] * 4),
     "mrl_conv": (C.c_int, [C.c_uint32] * 7 + [C.c_int] * 4 + [C.c_void_p] * 4),

@@ -262,13 +262,26 @@ void drop_arena(hipStream_t stream) {
   if (arena->base) (void)hipFree(arena->base);
 }
 
+// Scratch for callers that may not allocate (mrl_run_noalloc): one array per GPU, there from the
+// moment the library's code is loaded onto it until the process ends.  Host code never uses
+// the array's name as an address: mrl_init asks the runtime where the current device holds it
+// (hipGetSymbolAddress) and keeps that pointer per device.
+constexpr size_t NOALLOC_SCRATCH_BYTES = size_t(MRL_NOALLOC_SCRATCH_BYTES);
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+constexpr int MAX_DEVICES = 64;
+void *g_scratch_ptr[MAX_DEVICES] = {};
+
 struct Workspace {
   hipStream_t stream;
   std::vector<void *> allocs;
   Arena *arena = nullptr;  // locked while non-null
   size_t arena_used = 0;
   size_t requested = 0;    // everything this call asked for
+  uint8_t *fixed = nullptr;  // non-null: requests come out of these fixed_size bytes and nowhere else
+  size_t fixed_size = 0;
+  bool fixed_overflow = false;
   explicit Workspace(hipStream_t s) : stream(s) {}
+  Workspace(hipStream_t s, void *region, size_t bytes) : stream(s), fixed(static_cast<uint8_t *>(region)), fixed_size(bytes) {}
   Workspace(const Workspace &) = delete;
   Workspace &operator=(const Workspace &) = delete;
   hipError_t alloc(void **p, size_t bytes) {
@@ -278,6 +291,15 @@ struct Workspace {
       mrl::plan::Recorder *r = mrl::plan::g_recorder;
       *p = reinterpret_cast<void *>((uintptr_t(1) << 44) + r->scratch_bytes);
       r->scratch_bytes += rounded;
+      return hipSuccess;
+    }
+    if (fixed) {
+      if (rounded > fixed_size - arena_used) {
+        fixed_overflow = true;
+        return hipErrorOutOfMemory;
+      }
+      *p = fixed + arena_used;
+      arena_used += rounded;
       return hipSuccess;
     }
     if (!arena) {
@@ -1157,6 +1179,11 @@ int mrl_init(int device) {
     return MRL_ERR_NO_DEVICE;
   }
   HIP_TRY(hipSetDevice(device));
+  if (device < MAX_DEVICES && !g_scratch_ptr[device]) {
+    void *ptr = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));  // this device's copy of the array
+    g_scratch_ptr[device] = ptr;
+  }
   g_device = device;
   return MRL_OK;
 }
@@ -1447,6 +1474,35 @@ int mrl_compose_plan(const mrl_compose *c, mrl_plan *plan, mrl_plan_step *steps,
 
 int mrl_run_async(const mrl_spec *spec, void *const *params, void *stream) {
   return run_async_impl(spec, params, (hipStream_t)stream);
+}
+
+int mrl_run_noalloc(const mrl_spec *spec, void *const *params, void *stream) {
+  if (g_device < 0 || g_device >= MAX_DEVICES || !g_scratch_ptr[g_device]) {
+    g_last_error = "mrl_run_noalloc: call mrl_init first (it looks up the device's scratch array)";
+    return MRL_ERR_NO_DEVICE;
+  }
+  int rc = check_spec(spec);
+  if (rc != MRL_OK) return rc;
+  if (!params) return MRL_ERR_NULL;
+  for (uint32_t i = 0; i < spec->n_params; i++)
+    if (!params[i]) return MRL_ERR_NULL;
+  // What the call would take, from the plan (host arithmetic only), so that a Spec that does not
+  // fit is turned down before anything is launched.
+  mrl_plan plan;
+  if ((rc = mrl_spec_plan(spec, &plan, nullptr, 0)) != MRL_OK) return rc;
+  const std::string too_large = "mrl_run_noalloc: the Spec needs " + std::to_string(plan.scratch_bytes) +
+                                " bytes of scratch, the fixed array holds " + std::to_string(NOALLOC_SCRATCH_BYTES);
+  if (plan.scratch_bytes > NOALLOC_SCRATCH_BYTES) {
+    g_last_error = too_large;
+    return MRL_ERR_TOO_LARGE;
+  }
+  Workspace ws((hipStream_t)stream, g_scratch_ptr[g_device], NOALLOC_SCRATCH_BYTES);
+  rc = dispatch(*spec, params, ws);
+  if (ws.fixed_overflow) {  // parameters aligned otherwise than the plan assumes can take another path
+    g_last_error = too_large + " (exceeded during the run: parameters not 256-byte aligned?)";
+    return MRL_ERR_TOO_LARGE;
+  }
+  return rc;
 }
 
 int mrl_run(const mrl_spec *spec, void *const *params) {
