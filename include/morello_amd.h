@@ -442,6 +442,48 @@ int mrl_matmul_search_schedule(const mrl_spec *spec, mrl_matmul_schedule *best, 
 /* The same for a general Compose. */
 int mrl_compose_plan(const mrl_compose *c, mrl_plan *plan, mrl_plan_step *steps, uint32_t cap);
 
+/* Target::actions (target/mod.rs:69): the lowerings of a Spec this backend can run, each with what
+ * Kernel::main_cost and Kernel::memory_allocated would say of it, for a search to choose among.
+ * A CPU action rewrites one step of a schedule; the lowerings here are whole paths to a kernel, so
+ * an action names the scheduling steps it stands for (scheduling_sugar.rs:37-132):
+ *   SELECT          the dispatch rules' own choice for the Spec as it stands (Action::Select)
+ *   TILE_OUT_SPLIT  Matmul: tile_out([1, tile_m, tile_n]).split(split_k), then the matrix-core kernel
+ *   FUSED           Conv: the fused NHWC/KRSC kernel; Compose Matmul->Softmax->Matmul: the fused kernel
+ *                   with the keys in `parts` shares (parallel_softmax.rs:31-223; 1 = one workgroup
+ *                   per 128 queries, more = partial results merged with the parts formula)
+ *   SPATIAL_SPLIT   Conv as a Matmul over its windows read in place (spatial_split.rs:73-118),
+ *                   tile_out([tile_m, tile_n]) on that Matmul
+ *   UNFOLD          Conv: the windows materialised (a Move), then the Matmul
+ *   BUFFERIZE       Compose: both intermediates materialised (bufferize.rs:24-116), a kernel per stage
+ *   GENERIC         Conv on the any-dtype kernel */
+typedef enum {
+  MRL_ACTION_SELECT = 0,
+  MRL_ACTION_TILE_OUT_SPLIT = 1,
+  MRL_ACTION_FUSED = 2,
+  MRL_ACTION_SPATIAL_SPLIT = 3,
+  MRL_ACTION_UNFOLD = 4,
+  MRL_ACTION_BUFFERIZE = 5,
+  MRL_ACTION_GENERIC = 6
+} mrl_action_kind;
+typedef struct {
+  int32_t kind;             /* mrl_action_kind */
+  uint32_t tile_m, tile_n;  /* TILE_OUT_SPLIT, SPATIAL_SPLIT */
+  uint32_t split_k;         /* TILE_OUT_SPLIT: elements of K per step */
+  uint32_t parts;           /* FUSED on a Compose: shares of the keys */
+  uint32_t n_steps;         /* filled by mrl_target_actions: launches, */
+  uint64_t scratch_bytes;   /*   device scratch (Kernel::memory_allocated) */
+  double cost_ns;           /*   and predicted time (Kernel::main_cost) of the action */
+} mrl_action;
+/* Writes up to `cap` actions that apply to `spec` (those whose plan succeeds), priced; returns how
+ * many there are.  Host code: needs no GPU. */
+uint32_t mrl_target_actions(const mrl_spec *spec, mrl_action *out, uint32_t cap);
+/* The plan of one action (its kernels, step by step). */
+int mrl_action_plan(const mrl_spec *spec, const mrl_action *action, mrl_plan *plan, mrl_plan_step *steps, uint32_t cap);
+/* mrl_run_async under the chosen action.  MRL_ERR_UNSUPPORTED if it does not apply to the Spec or
+ * to these operands (alignment); the result is the Spec's whatever the action: integer Specs bit
+ * for bit, floating-point ones within the Spec's tolerance. */
+int mrl_run_action(const mrl_spec *spec, void *const *params, const mrl_action *action, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

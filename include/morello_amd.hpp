@@ -227,6 +227,16 @@ class Spec {
     check(mrl_matmul_search_schedule(&c_, &best, nullptr), "search_schedule");
     return best;
   }
+  // Target::actions (target/mod.rs:69): the lowerings the backend can run for this Spec, priced.
+  std::vector<mrl_action> actions() const {
+    std::vector<mrl_action> out(mrl_target_actions(&c_, nullptr, 0));
+    if (!out.empty()) out.resize(mrl_target_actions(&c_, out.data(), uint32_t(out.size())));
+    return out;
+  }
+  // Runs the Spec under one of its actions: `params` are device pointers in parameter order.
+  void run(const mrl_action &action, void *const *params, void *stream = nullptr) const {
+    check(mrl_run_action(&c_, params, &action, stream), "run_action");
+  }
   // Host-only: needs no GPU.
   Plan plan() const {
     mrl_plan head{};

@@ -318,6 +318,13 @@ class Spec:
                "mrl_matmul_search_schedule")
         return ScheduledMatmul(self, sched.tile_m, sched.tile_n, sched.split_k)
 
+    def actions(self) -> "list[Action]":
+        """Target::actions for this Spec (target/mod.rs:69): the lowerings the backend can run,
+        each priced by the cost model (host only)."""
+        buf = (B.ActionC * 32)()
+        n = B.load().mrl_target_actions(C.byref(self._c), buf, 32)
+        return [Action(self, buf[i]) for i in range(min(n, 32))]
+
     def tile_out(self, tile_shape: Sequence[int]) -> "ScheduledMatmul":
         """`spec.tile_out([1, m, n])`: one workgroup per m x n tile of the output."""
         if self.kind != SpecKind.Matmul or len(tile_shape) != 3 or tile_shape[0] != 1:
@@ -567,6 +574,45 @@ class Plan:
 
     def __repr__(self):
         return f"Plan({self.cost_ns:.0f} ns, scratch {self.scratch_bytes} B, {self.steps})"
+
+
+class ActionKind(enum.IntEnum):
+    Select = 0
+    TileOutSplit = 1
+    Fused = 2
+    SpatialSplit = 3
+    Unfold = 4
+    Bufferize = 5
+    Generic = 6
+
+
+class Action:
+    """One lowering of a Spec (mrl_action): what it is, what the cost model says of it, and a way
+    to run the Spec under it."""
+
+    def __init__(self, spec: "Spec", c: B.ActionC):
+        self.spec = spec
+        self._c = B.ActionC(c.kind, c.tile_m, c.tile_n, c.split_k, c.parts, c.n_steps, c.scratch_bytes, c.cost_ns)
+        self.kind = ActionKind(c.kind)
+        self.tile_m, self.tile_n, self.split_k, self.parts = c.tile_m, c.tile_n, c.split_k, c.parts
+        self.n_steps, self.scratch_bytes, self.cost_ns = c.n_steps, int(c.scratch_bytes), c.cost_ns
+
+    def __repr__(self):
+        knobs = {ActionKind.TileOutSplit: f" tile {self.tile_m}x{self.tile_n} split {self.split_k}",
+                 ActionKind.SpatialSplit: f" tile {self.tile_m}x{self.tile_n}",
+                 ActionKind.Fused: f" parts {self.parts}" if self.parts else ""}.get(self.kind, "")
+        return f"Action({self.kind.name}{knobs}: {self.cost_ns:.0f} ns, {self.n_steps} launches, scratch {self.scratch_bytes} B)"
+
+    def plan(self) -> "Plan":
+        head, cap = B.PlanC(), 64
+        steps = (B.PlanStepC * cap)()
+        _check(B.load().mrl_action_plan(C.byref(self.spec._c), C.byref(self._c), C.byref(head), steps, cap), "mrl_action_plan")
+        return Plan([PlanStep(steps[i]) for i in range(min(cap, head.n_steps))], head.cost_ns, int(head.scratch_bytes))
+
+    def run_device(self, ptrs: Sequence[int]):
+        arr = (C.c_void_p * len(ptrs))(*ptrs)
+        _check(B.load().mrl_run_action(C.byref(self.spec._c), arr, C.byref(self._c), None), "mrl_run_action")
+        synchronize()
 
 
 def _plan_of(fn, c_spec, where: str) -> Plan:

@@ -26,6 +26,11 @@ class MatmulScheduleC(C.Structure):
     _fields_ = [("tile_m", C.c_uint32), ("tile_n", C.c_uint32), ("split_k", C.c_uint32)]
 
 
+class ActionC(C.Structure):
+    _fields_ = [("kind", C.c_int32), ("tile_m", C.c_uint32), ("tile_n", C.c_uint32), ("split_k", C.c_uint32),
+                ("parts", C.c_uint32), ("n_steps", C.c_uint32), ("scratch_bytes", C.c_uint64), ("cost_ns", C.c_double)]
+
+
 class SpecC(C.Structure):
     _fields_ = [
         ("kind", C.c_int32),
@@ -146,6 +151,9 @@ SIGNATURES = {
     "mrl_matmul_scheduled_plan": (C.c_int, [C.POINTER(SpecC), C.POINTER(MatmulScheduleC), C.POINTER(PlanC),
                                             C.POINTER(PlanStepC), C.c_uint32]),
     "mrl_matmul_search_schedule": (C.c_int, [C.POINTER(SpecC), C.POINTER(MatmulScheduleC), C.POINTER(C.c_double)]),
+    "mrl_target_actions": (C.c_uint32, [C.POINTER(SpecC), C.POINTER(ActionC), C.c_uint32]),
+    "mrl_action_plan": (C.c_int, [C.POINTER(SpecC), C.POINTER(ActionC), C.POINTER(PlanC), C.POINTER(PlanStepC), C.c_uint32]),
+    "mrl_run_action": (C.c_int, [C.POINTER(SpecC), _VPP, C.POINTER(ActionC), C.c_void_p]),
     "mrl_launch_count": (C.c_uint64, []),
     "mrl_compose_plan": (C.c_int, [C.POINTER(ComposeC), C.POINTER(PlanC), C.POINTER(PlanStepC), C.c_uint32]),
     "mrl_device_info": (C.c_int, [C.c_char_p, C.c_size_t, C.POINTER(C.c_int), C.POINTER(C.c_int),

@@ -540,7 +540,18 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
   return finish();
 }
 
+// A lowering picked from outside (mrl_run_action / mrl_action_plan) instead of by the dispatch
+// rules: which of a Conv's or a Compose's paths to take.  Zero everywhere = the rules decide.
+struct Forced {
+  int conv_path = 0;        // 1 fused kernel, 2 implicit Matmul (tile side conv_tile), 3 unfold + Matmul, 4 generic
+  uint32_t conv_tile = 0;
+  int msm_path = 0;         // 1 fused kernel (key_splits workgroups per query block), 2 staged
+  uint32_t key_splits = 0;
+};
+thread_local const Forced *g_forced = nullptr;
+
 int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
+  const int forced = g_forced ? g_forced->conv_path : 0;
   Prepared img, filt, out;
   int rc;
   if ((rc = prepare(s, 0, params[0], true, ws, &img)) != MRL_OK) return rc;
@@ -579,7 +590,8 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
   // One kernel (windows read in place, or a 1x1 filter) pays from 1e5 multiply-adds on, as a
   // Matmul does; unfolding first (two or three launches) from 1e6.
   const double macs = double(cv.b) * pixels * cv.f * window;
-  const bool as_matmul = !fused_shape && kind >= 0 && row_elems * img.elem < (1u << 24) && macs >= 1e5;
+  const bool as_matmul = (!fused_shape || forced == 2 || forced == 3) && forced != 4 && kind >= 0 &&
+                         row_elems * img.elem < (1u << 24) && macs >= 1e5;
   const bool can_unfold = image_rows_bytes <= UNFOLD_BYTES &&
                           (macs >= 1e6 || (cv.fh == 1 && cv.fw == 1 && row_elems == window));
   // Tensors in another permutation layout (NCHW, say) are moved to channels-last when a
@@ -620,16 +632,20 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
     g->conv.image_bytes = uint64_t(cv.b) * h * w * c_bytes;
     return true;
   };
-  if (fast_types && channels_last(img.t) && channels_last(filt.t) && channels_last(out.t) &&
-      mrl::conv_i8_applicable(cv)) {
+  const bool fused_ok = fast_types && channels_last(img.t) && channels_last(filt.t) && channels_last(out.t) &&
+                        mrl::conv_i8_applicable(cv);
+  const bool implicit_ok = as_matmul && !(cv.fh == 1 && cv.fw == 1) && implicit_args(&conv_args) &&
+                           mrl::conv_gemm_applicable(conv_args, kind);
+  const bool unfold_ok = as_matmul && can_unfold && (reinterpret_cast<uintptr_t>(img.t.ptr) & 15) == 0 &&
+                         (reinterpret_cast<uintptr_t>(filt.t.ptr) & 15) == 0 && (reinterpret_cast<uintptr_t>(out.t.ptr) & 3) == 0;
+  if ((forced == 1 && !fused_ok) || (forced == 2 && !implicit_ok) || (forced == 3 && !unfold_ok)) return MRL_ERR_UNSUPPORTED;
+  if (fused_ok && forced <= 1) {
     HIP_TRY(mrl::launch_conv_i8(cv, di == MRL_U8, ws.stream));
-  } else if (as_matmul && !(cv.fh == 1 && cv.fw == 1) && implicit_args(&conv_args) &&
-             mrl::conv_gemm_applicable(conv_args, kind)) {
+  } else if (implicit_ok && (forced == 0 || forced == 2)) {
     // Channel vectors of whole 16-byte chunks: the windows are read where they lie.  (A 1x1 filter
     // needs no window arithmetic: its image is the left operand of a plain Matmul, below.)
-    HIP_TRY(mrl::launch_conv_gemm(conv_args, kind, ws.stream));
-  } else if (as_matmul && can_unfold && (reinterpret_cast<uintptr_t>(img.t.ptr) & 15) == 0 &&
-             (reinterpret_cast<uintptr_t>(filt.t.ptr) & 15) == 0 && (reinterpret_cast<uintptr_t>(out.t.ptr) & 3) == 0) {
+    HIP_TRY(mrl::launch_conv_gemm(conv_args, kind, ws.stream, forced == 2 ? g_forced->conv_tile : 0));
+  } else if (unfold_ok && (forced == 0 || forced == 3)) {
     // Filters in KRSC order are the B operand stored k-fastest; their rows padded like U's.
     const void *weights = filt.t.ptr;
     if (row_elems != window) {
@@ -746,7 +762,8 @@ int run_compose_msm(const mrl_spec &s, void *const *params, Workspace &ws) {
   // columns of Q and K add nothing to the scores, zero columns of V give result columns that are
   // not stored).  A result in another layout is formed in scratch memory and moved out.
   const uint32_t widest = std::max(k, n), dp = widest <= 32 ? 32 : widest <= 64 ? 64 : 128;
-  if (s.dtypes[0] == MRL_BF16 && s.dtypes[1] == MRL_BF16 && s.dtypes[2] == MRL_BF16 && s.dtypes[3] == MRL_F32 &&
+  const int forced = g_forced ? g_forced->msm_path : 0;
+  if (forced != 2 && s.dtypes[0] == MRL_BF16 && s.dtypes[1] == MRL_BF16 && s.dtypes[2] == MRL_BF16 && s.dtypes[3] == MRL_F32 &&
       widest <= 128 && (reinterpret_cast<uintptr_t>(params[3]) & 15) == 0) {
     // Parameter i as `rows` rows of `cols` bf16 per batch entry; wanted: the order of `want`.
     auto operand = [&](uint32_t i, const uint32_t *shape, const mrl_layout &want, uint32_t rows, uint32_t cols,
@@ -806,7 +823,7 @@ int run_compose_msm(const mrl_spec &s, void *const *params, Workspace &ws) {
       void *result = params[3];
       if (!out_in_order) HIP_TRY(ws.alloc(&result, size_t(b) * m * n * sizeof(float)));
       at.out = static_cast<float *>(result);
-      at.key_splits = mrl::attn_key_splits(at);
+      at.key_splits = forced == 1 && g_forced->key_splits ? g_forced->key_splits : mrl::attn_key_splits(at);
       if (at.key_splits > 1) {
         void *partials = nullptr;
         HIP_TRY(ws.alloc(&partials, mrl::attn_partial_bytes(at, at.key_splits)));
@@ -822,6 +839,7 @@ int run_compose_msm(const mrl_spec &s, void *const *params, Workspace &ws) {
       return rc;
     }
   }
+  if (forced == 1) return MRL_ERR_UNSUPPORTED;  // the fused kernel was asked for and does not take this Spec
   // Staged path, as the reference schedules it (examples/matmul_chain.rs:60-81): S and P
   // live in device memory as f32 (verification.rs:239-285); each stage is the Spec it is.
   void *sbuf = nullptr;
@@ -1683,6 +1701,94 @@ int mrl_matmul_search_schedule(const mrl_spec *spec, mrl_matmul_schedule *best, 
   if (!found) return MRL_ERR_UNSUPPORTED;
   if (cost_ns) *cost_ns = lowest;
   return MRL_OK;
+}
+
+// ---- actions: the lowerings a search may choose among (Target::actions, target/mod.rs:69) ----
+
+namespace {
+// Runs `spec` under `action` through `ws` (a recording Workspace when planning).
+int dispatch_action(const mrl_spec &spec, void *const *params, Workspace &ws, const mrl_action &a) {
+  Forced f;
+  switch (a.kind) {
+    case MRL_ACTION_SELECT: return dispatch(spec, params, ws);
+    case MRL_ACTION_TILE_OUT_SPLIT: {
+      if (spec.kind != MRL_SPEC_MATMUL) return MRL_ERR_UNSUPPORTED;
+      const mrl_matmul_schedule sched = {a.tile_m, a.tile_n, a.split_k};
+      return run_matmul(spec, params, ws, &sched);
+    }
+    case MRL_ACTION_SPATIAL_SPLIT: f.conv_path = 2, f.conv_tile = a.tile_m; break;
+    case MRL_ACTION_UNFOLD: f.conv_path = 3; break;
+    case MRL_ACTION_GENERIC: f.conv_path = 4; break;
+    case MRL_ACTION_FUSED: f.conv_path = 1, f.msm_path = 1, f.key_splits = a.parts ? a.parts : 1; break;
+    case MRL_ACTION_BUFFERIZE: f.msm_path = 2; break;
+    default: return MRL_ERR_BAD_SPEC;
+  }
+  const bool conv_action = a.kind == MRL_ACTION_SPATIAL_SPLIT || a.kind == MRL_ACTION_UNFOLD || a.kind == MRL_ACTION_GENERIC;
+  if ((conv_action && spec.kind != MRL_SPEC_CONV) || (a.kind == MRL_ACTION_BUFFERIZE && spec.kind != MRL_SPEC_COMPOSE_MSM) ||
+      (a.kind == MRL_ACTION_FUSED && spec.kind != MRL_SPEC_CONV && spec.kind != MRL_SPEC_COMPOSE_MSM) ||
+      (a.kind == MRL_ACTION_SPATIAL_SPLIT && (a.tile_m != a.tile_n || (a.tile_m != 64 && a.tile_m != 128 && a.tile_m != 256))))
+    return MRL_ERR_UNSUPPORTED;
+  g_forced = &f;
+  const int rc = dispatch(spec, params, ws);
+  g_forced = nullptr;
+  return rc;
+}
+}  // namespace
+
+int mrl_action_plan(const mrl_spec *spec, const mrl_action *action, mrl_plan *plan, mrl_plan_step *steps, uint32_t cap) {
+  if (!action) return MRL_ERR_NULL;
+  int rc = check_spec(spec);
+  if (rc != MRL_OK) return rc;
+  return plan_with(spec->n_params, plan, steps, cap,
+                   [&](void *const *params, Workspace &ws) { return dispatch_action(*spec, params, ws, *action); });
+}
+
+int mrl_run_action(const mrl_spec *spec, void *const *params, const mrl_action *action, void *stream) {
+  if (!action || !params) return MRL_ERR_NULL;
+  int rc;
+  if (g_device < 0 && (rc = mrl_init(0)) != MRL_OK) return rc;
+  if ((rc = check_spec(spec)) != MRL_OK) return rc;
+  for (uint32_t i = 0; i < spec->n_params; i++)
+    if (!params[i]) return MRL_ERR_NULL;
+  Workspace ws((hipStream_t)stream);
+  return dispatch_action(*spec, params, ws, *action);
+}
+
+uint32_t mrl_target_actions(const mrl_spec *spec, mrl_action *out, uint32_t cap) {
+  if (check_spec(spec) != MRL_OK) return 0;
+  std::vector<mrl_action> candidates;
+  auto candidate = [&](int kind, uint32_t tm = 0, uint32_t tn = 0, uint32_t sk = 0, uint32_t parts = 0) {
+    mrl_action a;
+    std::memset(&a, 0, sizeof a);
+    a.kind = kind, a.tile_m = tm, a.tile_n = tn, a.split_k = sk, a.parts = parts;
+    candidates.push_back(a);
+  };
+  candidate(MRL_ACTION_SELECT);
+  if (spec->kind == MRL_SPEC_MATMUL) {
+    mrl_matmul_schedule all[16];
+    const uint32_t n = std::min<uint32_t>(16, mrl_matmul_schedules(spec, all, 16));
+    for (uint32_t i = 0; i < n; i++) candidate(MRL_ACTION_TILE_OUT_SPLIT, all[i].tile_m, all[i].tile_n, all[i].split_k);
+  } else if (spec->kind == MRL_SPEC_CONV) {
+    candidate(MRL_ACTION_FUSED);
+    for (uint32_t side : {64u, 128u, 256u}) candidate(MRL_ACTION_SPATIAL_SPLIT, side, side, 0);
+    candidate(MRL_ACTION_UNFOLD);
+    candidate(MRL_ACTION_GENERIC);
+  } else if (spec->kind == MRL_SPEC_COMPOSE_MSM) {
+    // parallel_softmax.rs:31-223: the keys in `parts` shares, each at least two blocks of 64.
+    const uint32_t blocks = (spec->spec_shape[3] + 63) / 64;
+    for (uint32_t parts = 1; parts <= 64 && (parts == 1 || 2 * parts <= blocks); parts *= 2)
+      candidate(MRL_ACTION_FUSED, 0, 0, 0, parts);
+    candidate(MRL_ACTION_BUFFERIZE);
+  }
+  uint32_t n = 0;
+  for (mrl_action &a : candidates) {
+    mrl_plan plan;
+    if (mrl_action_plan(spec, &a, &plan, nullptr, 0) != MRL_OK) continue;   // not for this Spec
+    a.n_steps = plan.n_steps, a.scratch_bytes = plan.scratch_bytes, a.cost_ns = plan.cost_ns;
+    if (out && n < cap) out[n] = a;
+    n++;
+  }
+  return n;
 }
 
 int mrl_bench(const mrl_spec *spec, void *const *params, uint32_t iters, uint32_t repeats,

@@ -75,7 +75,8 @@ struct GemmArgs {
 hipError_t launch_gemm_nt(const GemmArgs &g, int kind, uint32_t tile, hipStream_t stream);
 // Conv as an implicit Matmul (g.conv filled in, B = the KRSC filters, k-fastest); tile chosen by size.
 bool conv_gemm_applicable(const GemmArgs &g, int kind);
-hipError_t launch_conv_gemm(const GemmArgs &g, int kind, hipStream_t stream);
+// `tile`: side of the workgroup tile (64, 128, 256), or 0 for the choice by problem size.
+hipError_t launch_conv_gemm(const GemmArgs &g, int kind, hipStream_t stream, uint32_t tile = 0);
 // kind: 0 = i8 x i8 -> i32, 1 = u8 x i8 -> i32, 2 = bf16 x bf16 -> f32, 3 = f32 x f32 -> f32.
 // Shapes, leading dimensions and alignment the kernel can walk.
 bool gemm_possible(const GemmArgs &g, int kind);

@@ -1,0 +1,98 @@
+"""Every action Target::actions lists for a Spec (mrl_target_actions; target/mod.rs:69), run through
+mrl_run_action and held against the CPU oracle: integer Specs bit for bit, the bf16 Compose within
+its 1e-2.  Small shapes against the oracle itself; the benchmark configurations against the
+result of the dispatch rules' own choice (which the other GPU tests hold against the oracle)."""
+import numpy as np
+import pytest
+
+import morello_amd as M
+import orc
+from gpu_util import rel_err
+from morello_amd import synth
+
+pytestmark = pytest.mark.gpu
+KT = M.layout(0, 2, 1)
+KT_ORC = orc.make_layout([0, 2, 1])
+
+
+def run_action(action, arrays):
+    bufs = [M.DeviceBuffer.from_numpy(a) for a in arrays]
+    action.run_device([b.ptr for b in bufs])
+    out = bufs[-1].to_numpy(arrays[-1].dtype, arrays[-1].shape)
+    for b in bufs:
+        b.free()
+    return out
+
+
+def test_matmul_actions_against_the_oracle(gpu):
+    for dts, np_out, odt in (((M.u8, M.i8, M.i32), np.int32, [orc.U8, orc.I8, orc.I32]),
+                             ((M.bf16, M.bf16, M.f32), np.float32, [orc.BF16, orc.BF16, orc.F32])):
+        m, k, n = 512, 384, 256
+        spec = M.MatmulAccum([1, m, k, n], dts)
+        if dts[0] == M.u8:
+            a, b = synth.uniform_u8(31, 0, (1, m, k)), synth.uniform_i8(31, 1, (1, k, n))
+            c0 = synth.uniform_u8(31, 2, (1, m, n)).astype(np.int32) - 99
+        else:
+            a, b = synth.normal_bf16(31, 0, (1, m, k)), synth.normal_bf16(31, 1, (1, k, n))
+            c0 = synth.normal_f32(31, 2, (1, m, n))
+        want = orc.matmul([1, m, k, n], odt, a, b, c0.copy(), True)
+        acts = spec.actions()
+        assert len(acts) == 9
+        for act in acts:
+            got = run_action(act, [a, b, c0.copy()])
+            if np_out == np.int32:
+                assert np.array_equal(got, want), act
+            else:
+                assert rel_err(got, want) < 1e-4, act
+
+
+def test_conv_actions_against_the_oracle(gpu):
+    b, f, c, oh, ow, fh, fw = 2, 64, 64, 12, 10, 3, 3
+    spec = M.Conv([b, f, c, oh, ow, fh, fw], (M.u8, M.i8, M.i32))
+    img = synth.uniform_u8(32, 0, (b, oh + fh - 1, ow + fw - 1, c))
+    filt = synth.uniform_i8(32, 1, (f, fh, fw, c))
+    nhwc = orc.make_layout([0, 2, 3, 1])
+    want = orc.conv([b, f, c, oh, ow, fh, fw], [orc.U8, orc.I8, orc.I32], img, filt, np.zeros((b, oh, ow, f), np.int32),
+                    layouts=[nhwc, nhwc, nhwc])
+    acts = spec.actions()
+    assert {a.kind for a in acts} == {M.ActionKind.Select, M.ActionKind.Fused, M.ActionKind.SpatialSplit,
+                                      M.ActionKind.Unfold, M.ActionKind.Generic}
+    for act in acts:
+        got = run_action(act, [img, filt, np.full((b, oh, ow, f), -7, np.int32)])
+        assert np.array_equal(got, want), act
+
+
+def test_compose_actions_against_the_oracle(gpu):
+    b, m, k, n2, n = 2, 256, 64, 1024, 64
+    spec = M.ComposeMSM(b, m, k, n2, n, layouts=[None, None, KT, None])
+    v, q, kmat = (synth.normal_bf16(33, 2, (b, n2, n), 0.5), synth.normal_bf16(33, 0, (b, m, k), 0.5),
+                  synth.normal_bf16(33, 1, (b, n2, k), 0.5))
+    want = orc.compose_msm(b, m, k, n2, n, [7, 7, 7, 6], v, q, kmat, np.zeros((b, m, n), np.float32),
+                           layouts=[None, None, KT_ORC, None])
+    acts = spec.actions()
+    assert [a.parts for a in acts if a.kind == M.ActionKind.Fused] == [1, 2, 4, 8] and acts[-1].kind == M.ActionKind.Bufferize
+    for act in acts:
+        got = run_action(act, [v, q, kmat, np.zeros((b, m, n), np.float32)])
+        assert rel_err(got, want) < 1e-2, act
+
+
+def test_actions_of_the_benchmark_configurations_agree(gpu):
+    """C2, C4, C5 at full size: every action gives what Select gives (bit for bit for the integer
+    Specs; C3's eight tiles take seconds each on the slower ones and are covered by the 512 x 384 x 256 case)."""
+    a, b = synth.uniform_u8(2, 0, (1, 4096, 4096)), synth.uniform_i8(2, 1, (1, 4096, 4096))
+    acts = M.MatmulAccum([1, 4096, 4096, 4096], (M.u8, M.i8, M.i32)).actions()
+    ref = run_action(acts[0], [a, b, np.ones((1, 4096, 4096), np.int32)])
+    for act in acts[1:]:
+        assert np.array_equal(run_action(act, [a, b, np.ones((1, 4096, 4096), np.int32)]), ref), act
+    img, filt = synth.uniform_u8(4, 0, (32, 56, 56, 64)), synth.uniform_i8(4, 1, (64, 3, 3, 64))
+    acts = M.Conv([32, 64, 64, 54, 54, 3, 3], (M.u8, M.i8, M.i32)).actions()
+    ref = run_action(acts[0], [img, filt, np.zeros((32, 54, 54, 64), np.int32)])
+    for act in acts[1:]:
+        if act.kind != M.ActionKind.Generic:     # 2.3 ms a launch, and held against the oracle above
+            assert np.array_equal(run_action(act, [img, filt, np.zeros((32, 54, 54, 64), np.int32)]), ref), act
+    v, q, kmat = (synth.normal_bf16(5, 2, (16, 2048, 128), 0.5), synth.normal_bf16(5, 0, (16, 2048, 128), 0.5),
+                  synth.normal_bf16(5, 1, (16, 2048, 128), 0.5))
+    acts = M.ComposeMSM(16, 2048, 128, 2048, 128, layouts=[None, None, KT, None]).actions()
+    ref = run_action(acts[0], [v, q, kmat, np.zeros((16, 2048, 128), np.float32)])
+    for act in acts[1:]:
+        assert rel_err(run_action(act, [v, q, kmat, np.zeros((16, 2048, 128), np.float32)]), ref) < 1e-2, act

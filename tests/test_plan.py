@@ -322,6 +322,39 @@ def test_cost_model_ranks_manual_schedules(gpu):
                         assert measured[x] <= 1.25 * measured[y], (dts[0], m, k, n, x, y, measured, predicted)
 
 
+def test_actions_of_the_benchmark_configurations():
+    """Target::actions (target/mod.rs:69) for C2-C5, host only: every lowering the backend can run,
+    priced; the dispatch rules' own choice (Select) is among the cheapest the model knows."""
+    K = M.ActionKind
+    acts = c2().actions()
+    tiles = {(a.tile_m, a.tile_n, a.split_k) for a in acts if a.kind == K.TileOutSplit}
+    assert acts[0].kind == K.Select and tiles == set(c2().available_schedules()) and len(tiles) == 8
+    assert all(a.n_steps == 1 and a.scratch_bytes == 0 and a.cost_ns > 20e3 for a in acts)
+    assert acts[0].plan().kernels == ["k_gemm_wide"]
+    acts = c3().actions()
+    assert len(acts) == 9 and acts[0].cost_ns == min(a.cost_ns for a in acts)
+    acts = {(a.kind, a.tile_m): a for a in c4().actions()}
+    assert set(acts) == {(K.Select, 0), (K.Fused, 0), (K.SpatialSplit, 64), (K.SpatialSplit, 128), (K.SpatialSplit, 256),
+                         (K.Unfold, 0), (K.Generic, 0)}
+    assert acts[(K.Fused, 0)].plan().kernels == ["k_conv_i8"] and acts[(K.Select, 0)].cost_ns == acts[(K.Fused, 0)].cost_ns
+    assert acts[(K.SpatialSplit, 128)].plan().kernels == ["k_gemm"] and "CONV = true" in acts[(K.SpatialSplit, 128)].plan().steps[0].kernel
+    assert acts[(K.Unfold, 0)].plan().kernels == ["k_unfold", "k_gemm"] and acts[(K.Unfold, 0)].scratch_bytes > 50e6
+    assert acts[(K.Generic, 0)].plan().kernels == ["k_conv_generic"]
+    assert acts[(K.Fused, 0)].cost_ns < acts[(K.SpatialSplit, 64)].cost_ns < acts[(K.Unfold, 0)].cost_ns < acts[(K.Generic, 0)].cost_ns
+    acts = c5().actions()
+    parts = [a.parts for a in acts if a.kind == K.Fused]
+    assert parts == [1, 2, 4, 8, 16] and acts[-1].kind == K.Bufferize and len(acts[-1].plan().steps) == 3
+    fused = {a.parts: a for a in acts if a.kind == K.Fused}
+    assert fused[1].scratch_bytes == 0 and fused[2].plan().kernels == ["k_attn", "k_attn_merge"]
+    assert fused[2].scratch_bytes == 16 * 2048 * 2 * (128 + 4) * 4
+    assert acts[0].cost_ns == fused[1].cost_ns == min(a.cost_ns for a in acts)
+    # Specs with one lowering list it alone; what no kernel takes lists nothing it cannot run.
+    assert [a.kind for a in M.Softmax([16, 2048, 2048], 2).actions()] == [K.Select]
+    odd = M.Conv([2, 3, 5, 6, 6, 2, 2], (M.i16, M.i16, M.i32)).actions()
+    assert {a.kind for a in odd} == {K.Select, K.Generic}
+    assert [a.kind for a in M.ComposeMSM(2, 64, 256, 128, 256, layouts=[None, None, KT, None]).actions()] == [K.Select, K.Bufferize]
+
+
 @pytest.mark.gpu
 def test_a_run_launches_what_its_plan_lists(gpu):
     """The plan comes from the dispatch code itself; this holds the two against each other from
