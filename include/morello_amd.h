@@ -204,8 +204,11 @@ int mrl_run(const mrl_spec *spec, void *const *params);
  * excess from the stream-ordered allocator and, before it returns, waits for the stream once and
  * replaces the arena by one that holds the whole call (up to 16 GiB), so that its next run
  * allocates nothing.  mrl_spec_plan tells the amount (scratch_bytes).  Calls from several host
- * threads onto one stream take turns for the arena.  mrl_stream_destroy releases the arena of
- * its stream; the arena of a stream the caller created itself stays until the process ends. */
+ * threads onto one stream take turns for the arena.  That one wait and reallocation cannot
+ * happen under stream capture: a capturing caller uses mrl_run_noalloc or runs the Spec once
+ * beforehand.  mrl_stream_destroy releases the arena of its stream; for a stream the caller
+ * created itself, mrl_stream_release does, and without it that arena stays until the process
+ * ends. */
 int mrl_run_async(const mrl_spec *spec, void *const *params, void *stream);
 
 /* As mrl_run_async, for callers that cannot allocate device memory (code under HIP graph capture,
@@ -296,7 +299,9 @@ int mrl_run_timed(const mrl_spec *spec, void *const *params, uint32_t steps,
 
 typedef struct {
   int32_t kind;      /* mrl_spec_kind with exactly one written parameter; not a Compose   */
-  int32_t accum;     /* must be 0: a component overwrites its output                      */
+  int32_t accum;     /* 1 only on components[0], the head: the Compose then accumulates
+                        into its output (spec.rs:3829-3838); elsewhere it must be 0, a
+                        side-effecting tail component is rejected (spec.rs:1760-1764)     */
   uint32_t scan_dim;
   uint32_t rank;
   uint32_t spec_shape[MRL_MAX_SPEC_RANK];
@@ -352,11 +357,19 @@ int mrl_memcpy_h2d(void *dst, const void *src, size_t bytes);
 int mrl_memcpy_d2h(void *dst, const void *src, size_t bytes);
 int mrl_memset(void *dst, int value, size_t bytes);
 int mrl_device_synchronize(void);
+/* Device memory not allocated at the moment, in bytes (hipMemGetInfo): what a caller sizing
+ * its buffers against the arenas the library keeps per stream wants to know. */
+int mrl_device_mem_free(size_t *free_bytes);
 /* HIP streams (default priority) for callers that have no HIP binding of their own: the
  * handle is what mrl_run_async, mrl_run_compose and the per-kind conveniences take.
- * mrl_stream_destroy waits for the stream's work, then frees the stream and its scratch arena. */
+ * mrl_stream_destroy waits for the stream's work, then frees the stream and its scratch arena.
+ * mrl_stream_release waits for the work of a stream the CALLER owns (any hipStream_t that was
+ * passed to mrl_run_async, NULL included) and frees only the arena the library kept for it:
+ * call it before hipStreamDestroy, or to give the memory back; the stream stays usable and its
+ * next call starts a new arena. */
 int mrl_stream_create(void **stream);
 int mrl_stream_synchronize(void *stream);
+int mrl_stream_release(void *stream);
 int mrl_stream_destroy(void *stream);
 /* Name, CU count, clock (kHz) and memory size of the selected device. */
 int mrl_device_info(char *name, size_t name_len, int *compute_units, int *clock_khz,
@@ -422,7 +435,9 @@ typedef struct {
   uint64_t scratch_bytes;  /* device scratch the call takes: Kernel::memory_allocated's HBM figure */
   double cost_ns;          /* sum over the steps: Kernel::main_cost (target/mod.rs:109), in ns */
 } mrl_plan;
-/* Which kernels mrl_run would launch for `spec` with 256-byte-aligned parameters, and the cost
+/* Which kernels mrl_run would launch for `spec` with 256-byte-aligned parameters (what
+ * mrl_device_alloc and hipMalloc return; a parameter aligned below 16 bytes makes a run take the
+ * element-wise paths instead of the 16-byte ones listed here), and the cost
  * model's prediction for them (Kernel::applies_to_logical_spec + main_cost + memory_allocated,
  * target/mod.rs:103-109; Cost, cost.rs:13-17).  The plan is produced by the same dispatch code
  * that runs a Spec, with launches recorded instead of made, so it cannot disagree with a run.

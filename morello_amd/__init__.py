@@ -697,6 +697,20 @@ class Stream:
             self.handle = None
 
 
+def device_free_bytes() -> int:
+    """Device memory that is not allocated at the moment."""
+    n = C.c_size_t()
+    _check(B.load().mrl_device_mem_free(C.byref(n)), "mrl_device_mem_free")
+    return n.value
+
+
+def release_stream(stream=None) -> None:
+    """Waits for a caller-owned HIP stream (an integer or ctypes handle; None = the default
+    stream) and frees the scratch arena the library kept for it."""
+    handle = stream.handle if isinstance(stream, Stream) else C.c_void_p(stream or 0)
+    _check(B.load().mrl_stream_release(handle), "mrl_stream_release")
+
+
 class DeviceBuffer:
     """A device allocation owned by Python; plumbing for tests and the benchmark."""
 

@@ -137,6 +137,8 @@ SIGNATURES = {
     "mrl_device_synchronize": (C.c_int, []),
     "mrl_stream_create": (C.c_int, [_VPP]),
     "mrl_stream_synchronize": (C.c_int, [C.c_void_p]),
+    "mrl_stream_release": (C.c_int, [C.c_void_p]),
+    "mrl_device_mem_free": (C.c_int, [C.POINTER(C.c_size_t)]),
     "mrl_stream_destroy": (C.c_int, [C.c_void_p]),
     "mrl_target_id": (C.c_char_p, []),
     "mrl_target_line_size": (C.c_uint32, []),

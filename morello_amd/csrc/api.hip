@@ -1044,7 +1044,10 @@ int compose_parameters(const mrl_compose &c, std::vector<ComposeParam> *out, std
   for (uint32_t i = 0; i < c.n_components; i++) {
     int rc = component_spec(c.components[i], &(*specs)[i]);
     if (rc != MRL_OK) return rc;
-    if (c.components[i].accum) return MRL_ERR_BAD_SPEC;
+    // Only the head (listed first, run last) may accumulate: a tail component with side effects is
+    // CanonicalizeError::SideEffectingComponent (spec.rs:1760-1764); an accumulating head is
+    // accepted (spec.rs:3829-3838) and makes the Compose's output parameter read-write.
+    if (i > 0 && c.components[i].accum) return MRL_ERR_BAD_SPEC;
     if ((rc = check_spec(&(*specs)[i])) != MRL_OK) return rc;
     if ((out_idx[i] = unique_output_index((*specs)[i])) < 0) return MRL_ERR_BAD_SPEC;
     if (out_idx[i] == 0) return MRL_ERR_BAD_SPEC;  // the first parameter must be an input to chain on
@@ -1089,7 +1092,7 @@ int run_compose_general(const mrl_compose &c, void *const *params, Workspace &ws
   if (c.bufferize_mask >> (n - 1)) return MRL_ERR_BAD_SPEC;  // only boundaries 0 .. n-2 exist
   if (c.bufferize_mask == 0 && n == 3 && specs[0].kind == MRL_SPEC_MATMUL && specs[1].kind == MRL_SPEC_SOFTMAX && specs[1].rank == 3 &&
       specs[1].scan_dim == 2 && specs[2].kind == MRL_SPEC_MATMUL && specs[0].dtypes[2] == MRL_F32 &&
-      specs[0].dtypes[0] == MRL_F32) {
+      specs[0].dtypes[0] == MRL_F32 && !specs[0].accum) {
     mrl_spec msm;
     std::memset(&msm, 0, sizeof msm);
     msm.kind = MRL_SPEC_COMPOSE_MSM, msm.rank = 5, msm.n_params = 4;
@@ -1203,6 +1206,7 @@ int mrl_init(int device) {
     g_scratch_ptr[device] = ptr;
   }
   g_device = device;
+  mrl::g_compute_units = prop.multiProcessorCount > 0 ? uint32_t(prop.multiProcessorCount) : 256u;
   return MRL_OK;
 }
 
@@ -1360,11 +1364,7 @@ uint64_t mrl_launch_count(void) { return mrl::plan::g_launches; }
 
 const char *mrl_target_id(void) { return "Gfx950"; }
 uint32_t mrl_target_line_size(void) { return 128; }
-uint32_t mrl_target_processors(void) {
-  int units = 256;
-  if (g_device >= 0) (void)hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, g_device);
-  return uint32_t(units);
-}
+uint32_t mrl_target_processors(void) { return mrl::g_compute_units; }
 
 uint32_t mrl_target_memories(mrl_target_memory *out, uint32_t cap) {
   // Fastest first, as CpuMemory's order (target/cpu.rs:2536-2560).  ACC: the MFMA accumulators
@@ -1939,11 +1939,24 @@ int mrl_stream_synchronize(void *stream) {
   return MRL_OK;
 }
 
+int mrl_stream_release(void *stream) {
+  HIP_TRY(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  drop_arena(static_cast<hipStream_t>(stream));
+  return MRL_OK;
+}
+
 int mrl_stream_destroy(void *stream) {
   if (!stream) return MRL_ERR_NULL;
   HIP_TRY(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
   drop_arena(static_cast<hipStream_t>(stream));
   HIP_TRY(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+  return MRL_OK;
+}
+
+int mrl_device_mem_free(size_t *free_bytes) {
+  if (!free_bytes) return MRL_ERR_NULL;
+  size_t total = 0;
+  HIP_TRY(hipMemGetInfo(free_bytes, &total));
   return MRL_OK;
 }
 

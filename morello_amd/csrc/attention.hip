@@ -433,14 +433,10 @@ __global__ __launch_bounds__(256) void k_attn_merge(const float *__restrict__ pa
 // compute units and there are keys enough to share out (four blocks of 64 per workgroup at
 // least, and more time saved than the partial results cost).  The workgroups then number at most one per compute unit: measured on 256 units, 256
 // workgroups stream K and V at 4.9-5.6 TB/s where 320 or 512 reach 3.6-4.8.
+uint32_t g_compute_units = 256;
+
 uint32_t attn_key_splits(const AttnArgs &a) {
-  static const uint64_t units = [] {
-    int device = 0, count = 0;
-    if (hipGetDevice(&device) != hipSuccess ||
-        hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count <= 0)
-      return uint64_t(256);
-    return uint64_t(count);
-  }();
+  const uint64_t units = g_compute_units;  // set by mrl_init: planning makes no runtime call
   const uint64_t groups = uint64_t((a.m + BQ - 1) / BQ) * a.b, blocks = (a.n2 + BKV - 1) / BKV;
   if (groups == 0) return 1;
   const uint64_t splits = std::min<uint64_t>({units / groups, blocks / 4, 256});

@@ -155,6 +155,10 @@ hipError_t launch_fill(void *out, int dtype, int fill_value, uint64_t count, hip
 hipError_t measure_mfma_rate(int kind, bool random_operands, uint32_t iters, hipStream_t stream,
                              double *ops_per_second);
 
+// Compute units of the selected device (mrl_init sets it; 256 on an MI355X).  Heuristics read
+// this instead of asking the runtime, so that planning a Spec makes no runtime call.
+extern uint32_t g_compute_units;
+
 // ---- attention.hip: fused Matmul -> Softmax -> Matmul on bf16 inputs -------------------
 struct AttnArgs {
   const void *q;   // [b, m, k]   bf16 row-major

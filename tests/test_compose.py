@@ -47,8 +47,11 @@ def test_chain_validation():
         M.Compose([mm([1, 4, 8, 4]), mm([1, 4, 4, 4])])
     with pytest.raises(M.MorelloError):  # dtypes do not chain: i32 output into an f32 input
         M.Compose([mm([1, 4, 4, 4]), mm([1, 4, 4, 4], (M.u8, M.i8, M.i32))])
-    with pytest.raises(M.MorelloError):  # accumulating component
+    with pytest.raises(M.MorelloError):  # accumulating tail component (spec.rs:1760-1764, 3840-3847)
         M.Compose([mm([1, 4, 4, 4]), mm([1, 4, 4, 4], accum=True)])
+    # An accumulating head is a Compose (spec.rs:3829-3838) with the same parameters.
+    c = M.Compose([mm([1, 4, 4, 4], accum=True), mm([1, 4, 4, 4])])
+    assert [c.parameter(i) for i in range(c.n_params)] == [(0, 1), (1, 0), (1, 1), (0, 2)]
     with pytest.raises(M.MorelloError):  # two written parameters: no unique output to chain on
         M.Compose([mm([1, 4, 4, 4]), M.SoftmaxDenominatorAndMax([1, 4, 4], 2)])
     with pytest.raises(M.MorelloError):  # DivideVec writes its first parameter
@@ -80,6 +83,37 @@ def test_integer_matmul_chain_is_exact(gpu):
     t1 = orc.matmul([b, m, 16, 72], [orc.I32] * 3, t2, w1, np.zeros((b, m, 72), np.int32))
     want = orc.matmul([b, m, 72, 8], [orc.I32] * 3, t1, w0, np.zeros((b, m, 8), np.int32))
     assert np.array_equal(got, want)
+
+
+@pytest.mark.gpu
+def test_accumulating_head(gpu):
+    """components[0] = Matmul{accum: true} (spec.rs:3829-3838): the pipeline's result is added to
+    what the output holds, wrapping for integers, and a second run adds it again."""
+    b, m = 2, 24
+    a = synth.uniform_u8(905, 0, (b, m, 40))
+    w1 = synth.uniform_i8(905, 1, (b, 40, 16))
+    w0 = synth.uniform_i8(905, 2, (b, 16, 72)).astype(np.int32)
+    init = synth.uniform_i8(905, 3, (b, m, 72)).astype(np.int32) * 16777259
+    c = M.Compose([M.Matmul([b, m, 16, 72], [M.i32] * 3, accum=True), M.Matmul([b, m, 40, 16], [M.u8, M.i8, M.i32])])
+    t1 = orc.matmul([b, m, 40, 16], [orc.U8, orc.I8, orc.I32], a, w1, np.zeros((b, m, 16), np.int32))
+    want = orc.matmul([b, m, 16, 72], [orc.I32] * 3, t1, w0, init.copy(), accum=True)
+    got = _run(c, [w0, a, w1, init.copy()])
+    assert np.array_equal(got, want)
+    want2 = orc.matmul([b, m, 16, 72], [orc.I32] * 3, t1, w0, want.copy(), accum=True)
+    assert np.array_equal(_run(c, [w0, a, w1, got.copy()]), want2)
+    # The attention shape with an accumulating head: Matmul -> Softmax -> MatmulAccum.
+    b, m, k, n2, n = 2, 128, 128, 256, 128
+    q = synth.normal_bf16(906, 0, (b, m, k), 0.5)
+    kmat = synth.normal_bf16(906, 1, (b, n2, k), 0.5)
+    v = synth.normal_bf16(906, 2, (b, n2, n), 0.5)
+    init = synth.normal_f32(906, 3, (b, m, n), 1.0)
+    c = M.Compose([M.Matmul([b, m, n2, n], [M.f32, M.bf16, M.f32], accum=True), M.Softmax([b, m, n2], 2),
+                   M.Matmul([b, m, k, n2], [M.bf16, M.bf16, M.f32])], layouts=[None, None, M.layout(0, 2, 1), None])
+    got = _run(c, [v, q, kmat, init.copy()])
+    kt = np.ascontiguousarray(kmat.transpose(0, 2, 1))
+    want = init + orc.compose_msm(b, m, k, n2, n, [7, 7, 7, 6], v, q, kt, np.zeros((b, m, n), np.float32))
+    assert np.abs(got - want).max() / np.abs(want).max() < 1e-2  # the Compose's tolerance: P is rounded to bf16
+    assert np.abs(got - init).max() > 0.01
 
 
 @pytest.mark.gpu

@@ -81,6 +81,30 @@ def test_async_launches_on_two_streams(gpu):
     s2.destroy()
 
 
+def test_releasing_a_streams_arena(gpu):
+    """mrl_stream_release: a Spec that stages operands (ragged K and N) runs on a stream, the
+    stream's scratch arena is given back while the stream lives on, and the next call on the same
+    stream (it starts a new arena) still accumulates onto the first one's result."""
+    stream = M.Stream()
+    b, m, k, n = 1, 300, 270, 290
+    A, Bm = synth.uniform_u8(830, 0, (b, m, k)), synth.uniform_i8(830, 1, (b, k, n))
+    bufs = [M.DeviceBuffer.from_numpy(x) for x in (A, Bm, np.zeros((b, m, n), np.int32))]
+    spec = M.MatmulAccum([b, m, k, n], (M.u8, M.i8, M.i32))
+    want = orc.matmul([b, m, k, n], [0, 1, 5], A, Bm, np.zeros((b, m, n), np.int32))
+    free0 = M.device_free_bytes()
+    spec.run_async([x.ptr for x in bufs], stream)
+    stream.synchronize()
+    held = free0 - M.device_free_bytes()
+    M.release_stream(stream)  # waits for the work, then frees
+    assert np.array_equal(bufs[2].to_numpy(np.int32, (b, m, n)), want)
+    assert held >= 64 << 20 and M.device_free_bytes() >= free0 - (8 << 20)
+    spec.run_async([x.ptr for x in bufs], stream)
+    stream.synchronize()
+    assert np.array_equal(bufs[2].to_numpy(np.int32, (b, m, n)), 2 * want)
+    M.release_stream(None)  # the default stream: nothing kept, nothing to free, still fine
+    stream.destroy()
+
+
 def test_host_threads_share_a_stream_and_its_scratch(gpu):
     """Four host threads enqueue Matmuls that need scratch memory (K and N are not whole 16-byte
     chunks, so A and B are copied into padded rows) onto one stream, each thread several times
