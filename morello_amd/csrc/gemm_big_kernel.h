@@ -174,7 +174,8 @@ hipError_t launch_big(const GemmArgs &g, hipStream_t stream) {
   const double mn = double(g.m) * g.n * g.batch;
   plan::work(T::ES == 1 ? plan::UNIT_MFMA_I8 : plan::UNIT_MFMA_BF16, 2.0 * mn * g.k,
              (double(g.m) * g.k + double(g.k) * g.n) * g.batch * T::ES + mn * 4 * (g.accum ? 2 : 1),
-             2.0 * 256 * 256 * double(g.k), 500.0 + 1200.0 * double(g.k * T::ES / 128));
+             2.0 * 256 * 256 * double(g.k), 500.0 + 1200.0 * double(g.k * T::ES / 128),
+             T::ES == 1 ? 1.25 : 1.08);  // measured: 1800 TOPS int8 at 4096^3
   MRL_LAUNCH((k_gemm_big<T, A_UNSIGNED>), dim3(tiles_m * tiles_n, g.batch), dim3(512), BIG_LDS_BYTES, stream, g,
              tiles_m, tiles_n, group_rows(tiles_m, tiles_n));
   return mrl::plan::last_error();

@@ -29,6 +29,7 @@ struct Step {
   double ops, bytes;        // arithmetic and HBM traffic the launcher declared (0 when it did not)
   double tile_ops;          // MFMA kernels: arithmetic of one workgroup, padding included
   double serial_ns;         // a workgroup's dependent chain (loop trips x their latency): no launch is shorter
+  double rate_scale;        // the kernel's measured rate over the model's sustained rate for its unit
 };
 
 struct Recorder {
@@ -36,7 +37,7 @@ struct Recorder {
   size_t scratch_bytes = 0;  // device scratch the call would take
   // Declared for the next launch.
   int unit = UNIT_STREAM;
-  double ops = 0, bytes = 0, tile_ops = 0, serial_ns = 0;
+  double ops = 0, bytes = 0, tile_ops = 0, serial_ns = 0, rate_scale = 1;
 };
 
 extern thread_local Recorder *g_recorder;
@@ -47,10 +48,11 @@ extern thread_local uint64_t g_launches;
 inline bool recording() { return g_recorder != nullptr; }
 
 // The launch site's declaration of the next kernel's work; a no-op outside planning.
-inline void work(int unit, double ops, double bytes, double tile_ops = 0, double serial_ns = 0) {
+inline void work(int unit, double ops, double bytes, double tile_ops = 0, double serial_ns = 0,
+                 double rate_scale = 1) {
   if (!g_recorder) return;
   g_recorder->unit = unit, g_recorder->ops = ops, g_recorder->bytes = bytes;
-  g_recorder->tile_ops = tile_ops, g_recorder->serial_ns = serial_ns;
+  g_recorder->tile_ops = tile_ops, g_recorder->serial_ns = serial_ns, g_recorder->rate_scale = rate_scale;
 }
 
 // `kernel_text`: the kernel expression as written at the launch site; `launcher`: the

@@ -37,9 +37,9 @@ void note(const char *kernel_text, const char *launcher, dim3 grid, dim3 block, 
   step.block[0] = block.x, step.block[1] = block.y, step.block[2] = block.z;
   step.lds_bytes = uint32_t(lds_bytes);
   step.unit = r->unit, step.ops = r->ops, step.bytes = r->bytes, step.tile_ops = r->tile_ops;
-  step.serial_ns = r->serial_ns;
+  step.serial_ns = r->serial_ns, step.rate_scale = r->rate_scale;
   r->steps.push_back(step);
-  r->unit = UNIT_STREAM, r->ops = r->bytes = r->tile_ops = r->serial_ns = 0;
+  r->unit = UNIT_STREAM, r->ops = r->bytes = r->tile_ops = r->serial_ns = 0, r->rate_scale = 1;
 }
 
 // Nanoseconds of one planned launch on an MI355X, launches queued back to back on one stream.
@@ -62,6 +62,7 @@ double step_ns(const Step &s, uint32_t compute_units) {
     case UNIT_VALU: rate = 3e3; break;   // the generic kernels: dtype switches and index arithmetic per term
     default: break;
   }
+  rate *= s.rate_scale;
   const double workgroups = double(s.grid[0]) * s.grid[1] * s.grid[2];
   double bytes = s.bytes;
   if (bytes == 0 && s.ops == 0) bytes = workgroups * s.block[0] * s.block[1] * s.block[2] * 16.0;  // undeclared: a guess
