@@ -21,8 +21,9 @@
 // Both products are formed transposed so that a lane owns one query column: the running
 // max, the denominator and the rescale factor are per-lane scalars, and a row reduction is
 // 32 in-register values plus one cross-lane exchange.  K and V blocks go from global memory
-// straight into LDS (no staging registers), double buffered, one barrier per block; the
-// bank-conflict swizzles are applied on the source side of those loads.
+// straight into LDS (no staging registers; two K tiles and three V tiles per key half), the
+// bank-conflict swizzles applied on the source side of those loads.  The two key halves run one
+// slot apart (matrix work of one beside vector work of the other), two barriers per block.
 #include <algorithm>
 
 #include "kernels.h"
@@ -46,8 +47,7 @@ template <int D>
 struct Dims {
   static constexpr int ROW = D * 2;             // bytes per K or V row
   static constexpr int TILE = BKV * ROW;        // one K or V block (16 KiB at D = 128)
-  static constexpr int STAGE = 2 * TILE;        // K block then V block
-  static constexpr int HALF = 2 * STAGE;        // two stages per key half
+  static constexpr int HALF = 5 * TILE;         // per key half: two K tiles, three V tiles
   static constexpr int CHUNKS = ROW / 16;       // 16-byte chunks per row
   static constexpr int UNITS = ROW / 64;        // 64-byte units per row
   static constexpr int ROWS_PER_LINE = ROW >= 256 ? 1 : 256 / ROW;  // rows per 256-byte bank line
@@ -59,7 +59,19 @@ struct Dims {
   __device__ static constexpr int v_swizzle(int row) { return (row / ROWS_PER_LINE) & (UNITS - 1); }
 };
 constexpr float LOG2E = 1.44269504088896340736f;
-constexpr float RESCALE_SLACK = 5.0f;  // e^5 = 148
+constexpr float STALE_REFERENCE_SUM = 1.0e12f;  // ~2^40: a lane's sum of 64 exponentials beyond it moves the reference
+
+// One direct-to-LDS load: 64 lanes x 16 bytes from `base + voff` (voff per lane) to the 1 KiB at
+// LDS address `lds_addr` (wave-uniform), lane l to slot l.  Written as assembly so that the
+// compiler does not know of it: it would otherwise make every later LDS read wait for all such
+// loads in flight (it cannot tell the stages apart), which serialises a block's softmax behind
+// the next block's fetch.  The waits that matter are the explicit ones before the barriers.
+__device__ inline void dma16(const uint8_t *base, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base));
+}
+__device__ inline uint32_t lds_address(const void *p) {
+  return uint32_t(reinterpret_cast<uintptr_t>((lds_void *)p));
+}
 
 __device__ inline v2i read_tr16(const uint8_t *p) {
   const v4s r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s *)p);
@@ -78,7 +90,7 @@ __device__ inline v2i read_tr16(const uint8_t *p) {
 template <int D, bool RAGGED, bool KT_ROWS>
 __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
   typedef Dims<D> DD;
-  constexpr int ROW = DD::ROW, TILE = DD::TILE, STAGE = DD::STAGE, HALF = DD::HALF;
+  constexpr int ROW = DD::ROW, TILE = DD::TILE, HALF = DD::HALF;
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -157,17 +169,6 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
     const uint32_t off = uint32_t(first_block + kb) * TILE + v_src[i];
     return RAGGED ? min(off, head_bytes - 16) : off;
   };
-  auto load_block = [&](int kb, int stage) {
-#pragma unroll
-    for (int i = 0; i < PER_WAVE; i++) {
-      const int q = qg * PER_WAVE + i;
-      __builtin_amdgcn_global_load_lds((global_cvoid *)(K + k_off(kb, i)),
-                                       (lds_void *)(my_lds + stage * STAGE + q * 1024), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((global_cvoid *)(V + v_off(kb, i)),
-                                       (lds_void *)(my_lds + stage * STAGE + TILE + q * 1024), 16, 0, 0);
-    }
-  };
-
   v16f o[D / 32];
 #pragma unroll
   for (int t = 0; t < D / 32; t++)
@@ -179,93 +180,169 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
   const int v_rl = (lane & 15) >> 2;                                   // row within a 4-row read
   const int v_within = 32 * ((lane >> 4) & 1) + 8 * (lane & 3);        // bytes within a 64-B unit
 
-  if (nblocks > 0) load_block(0, 0);
-  for (int kb = 0; kb < steps; kb++) {
-    const int stage = kb & 1;
-    // Block kb has landed (the loads are tracked by vmcnt only) and, after the barrier,
-    // every wave is done reading the other stage, which the next block may now overwrite.
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
-    if (kb >= nblocks) continue;  // the shorter half idles through its partner's last block
-    // The next block's global->LDS loads are issued one K and one V instruction at a time
-    // between the MFMA batches below (such an instruction holds its wave for tens of cycles;
-    // in a burst behind the barrier all eight waves queue up on the one memory pipe while
-    // the matrix cores idle).  Past the last block the same block is fetched again into the
-    // stage nobody reads.
-    const int next_kb = min(kb + 1, nblocks - 1);
-    uint8_t *next_lds = my_lds + (stage ^ 1) * STAGE;
-    auto load_pair = [&](int i) {
-      const int q = qg * PER_WAVE + i;
-      __builtin_amdgcn_global_load_lds((global_cvoid *)(K + k_off(next_kb, i)), (lds_void *)(next_lds + q * 1024), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((global_cvoid *)(V + v_off(next_kb, i)), (lds_void *)(next_lds + TILE + q * 1024), 16, 0, 0);
-    };
-    const uint8_t *lk = my_lds + stage * STAGE, *lv = lk + TILE;
+  // LDS of a key half: K tiles 0 and 1, then V tiles 0, 1 and 2.  K block kb goes to K tile
+  // kb & 1, V block kb to V tile kb % 3.  A block index past the half's last block fetches the
+  // last block again, into a tile that nobody reads any more, so that every slot issues the same
+  // number of loads and the counts given to s_waitcnt below hold.
+  auto issue_k = [&](int kb) {
+    const int src = min(kb, nblocks - 1);
+    const uint32_t dst = lds_address(my_lds + (kb & 1) * TILE);
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; i++) dma16(K, k_off(src, i), dst + (qg * PER_WAVE + i) * 1024);
+  };
+  auto issue_v = [&](int kb) {
+    const int src = min(kb, nblocks - 1);
+    const uint32_t dst = lds_address(my_lds + (2 + kb % 3) * TILE);
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; i++) dma16(V, v_off(src, i), dst + (qg * PER_WAVE + i) * 1024);
+  };
 
-    // S^T tiles: s[kt][r] is key kt*32 + 8*(r/4) + 4*lg + r%4, query lq.
-    // K operands come in batches of two d-steps (four MFMAs), two batches ahead of their
-    // MFMAs, so the first MFMA starts after one batch's LDS latency instead of the whole
-    // block's; the two key tiles' accumulation chains alternate.
-    v16f s[BKV / 32];
-    v4i kf[3][BKV / 32][2];
-    auto read_k = [&](int q, int buf) {
+  // The two key halves of a workgroup run the same program ONE SLOT APART.  A wave's work per
+  // block is a slot of matrix-core work (A_j: O += V.P of block j - 1, then S = K.Q of block j)
+  // and a slot of vector-unit work (B_j: the online softmax of block j), a barrier after each.
+  // Half 1 passes one extra barrier first, so whenever the wave of half 0 on a SIMD is in a matrix
+  // slot its partner of half 1 is in a softmax slot and the other way round: measured, one wave
+  // issues a vector instruction every 6-7 cycles at best and an MFMA wave beside it keeps its
+  // full rate, so the exponentials of one half ride under the MFMAs of the other, where two
+  // waves in step would queue for the matrix core and then for the vector unit.
+  //   A_j issues the fetch of V(j + 1) (into the tile of V(j - 2), last read in A_(j-1));
+  //   B_j issues the fetch of K(j + 2) (into the tile of K(j), last read in A_j), one instruction
+  //   at a time between the exponentials, and ends by waiting for everything but the last two
+  //   fetches: K(j + 1) and V(j), which A_(j+1) reads, have then landed.  A fetch has two slots.
+  v16f s[BKV / 32];
+  v8bf pb[BKV / 16];
+  // Lane-dependent, block-independent parts of the operand addresses (the swizzles depend on the
+  // lane only: the row offsets that vary per read are multiples of the swizzle periods).
+  uint32_t v_lane[D / 32], k_lane[KT_ROWS ? BKV / 32 : D / 16];
+  {
+    const int key = 4 * lg + v_rl;
 #pragma unroll
-      for (int c = 0; c < 2; c++)
+    for (int t = 0; t < D / 32; t++) v_lane[t] = key * ROW + ((t ^ DD::v_swizzle(key)) << 6) + v_within;
+    if constexpr (KT_ROWS) {
 #pragma unroll
-        for (int kt = 0; kt < BKV / 32; kt++) {
-          const int row = kt * 32 + lq, st = 2 * q + c;
-          if constexpr (KT_ROWS) {
-            const int drow = 16 * st + 4 * lg + v_rl;  // drow + 8 swizzles alike
-            const int off = ((kt ^ Dims<64>::v_swizzle(drow)) << 6) + v_within;
-            const v2i lo = read_tr16(lk + drow * (BKV * 2) + off), hi = read_tr16(lk + (drow + 8) * (BKV * 2) + off);
-            kf[buf][kt][c] = v4i{lo[0], lo[1], hi[0], hi[1]};
-          } else {
-            kf[buf][kt][c] = *(const v4i *)(lk + row * ROW + (((2 * st + lg) ^ DD::k_swizzle(row)) << 4));
-          }
+      for (int kt = 0; kt < BKV / 32; kt++) k_lane[kt] = key * (BKV * 2) + ((kt ^ Dims<64>::v_swizzle(key)) << 6) + v_within;
+    } else {
+#pragma unroll
+      for (int st = 0; st < D / 16; st++) k_lane[st] = lq * ROW + (((2 * st + lg) ^ DD::k_swizzle(lq)) << 4);
+    }
+  }
+  if (nblocks > 0) {
+    issue_k(0);
+    issue_v(0);
+    issue_k(1);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  __syncthreads();
+  if (half) __syncthreads();
+  // s_waitcnt vmcnt(n), n < 16, the other counters left alone.
+  constexpr int WAIT_BUT_TWO = 0x0F70 | (2 * PER_WAVE);
+  constexpr int NU = BKV / 16, NQ = D / 32;
+  constexpr int VR = 2 * (D / 32), KR = (KT_ROWS ? 4 : 2) * (BKV / 32), PM = D / 32, QM = 2 * (BKV / 32);
+  v4i kf[2][BKV / 32][2];
+  v4i vf[3][D / 32];
+  // K operands of batch q (two d-steps, both key tiles) of the K tile at `lk`.
+  auto read_k = [&](const uint8_t *lk, int q, int buf) {
+#pragma unroll
+    for (int c = 0; c < 2; c++)
+#pragma unroll
+      for (int kt = 0; kt < BKV / 32; kt++) {
+        const int st = 2 * q + c;
+        if constexpr (KT_ROWS) {
+          const uint8_t *a = lk + k_lane[kt] + st * 16 * (BKV * 2);
+          const v2i lo = read_tr16(a), hi = read_tr16(a + 8 * (BKV * 2));
+          kf[buf][kt][c] = v4i{lo[0], lo[1], hi[0], hi[1]};
+        } else {
+          kf[buf][kt][c] = *(const v4i *)(lk + k_lane[st] + kt * 32 * ROW);
         }
-    };
+      }
+  };
+  auto read_v = [&](const uint8_t *lv, int u, int buf) {
+#pragma unroll
+    for (int t = 0; t < D / 32; t++) {
+      const uint8_t *a = lv + v_lane[t] + u * 16 * ROW;
+      const v2i lo = read_tr16(a), hi = read_tr16(a + 8 * ROW);
+      vf[buf][t] = v4i{lo[0], lo[1], hi[0], hi[1]};
+    }
+  };
+  auto pv_step = [&](int u, int buf) {
+#pragma unroll
+    for (int t = 0; t < D / 32; t++)
+      o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, vf[buf][t]), pb[u], o[t], 0, 0, 0);
+  };
+  auto qk_step = [&](int q, int buf) {
+#pragma unroll
+    for (int c = 0; c < 2; c++)
+#pragma unroll
+      for (int kt = 0; kt < BKV / 32; kt++)
+        s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, kf[buf][kt][c]),
+                                                        __builtin_bit_cast(v8bf, qf[2 * q + c]), s[kt], 0, 0, 0);
+  };
+  auto zero_s = [&]() {
 #pragma unroll
     for (int kt = 0; kt < BKV / 32; kt++)
 #pragma unroll
       for (int r = 0; r < 16; r++) s[kt][r] = 0.0f;
-    read_k(0, 0);
-    if (D / 32 > 1) read_k(1, 1);
+  };
+  // Slot A of the first block: S = K.Q only.
+  auto slot_a_first = [&]() {
+    const uint8_t *lk = my_lds;
+    issue_v(1);
+    zero_s();
+    read_k(lk, 0, 0);
 #pragma unroll
-    for (int q = 0; q < D / 32; q++) {
-      if (q + 2 < D / 32) read_k(q + 2, (q + 2) % 3);
-      load_pair(q);
-#pragma unroll
-      for (int c = 0; c < 2; c++)
-#pragma unroll
-        for (int kt = 0; kt < BKV / 32; kt++)
-          s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, kf[q % 3][kt][c]),
-                                                          __builtin_bit_cast(v8bf, qf[2 * q + c]), s[kt], 0, 0, 0);
+    for (int q = 0; q < NQ; q++) {
+      if (q + 1 < NQ) read_k(lk, q + 1, (q + 1) & 1);
+      qk_step(q, q & 1);
     }
-    __builtin_amdgcn_sched_group_barrier(0x100, (KT_ROWS ? 2 : 1) * (D / 32 > 1 ? 4 : 2) * (BKV / 32), 0);
+  };
+  // Slot A of block j, 1 <= j < nblocks: O += V.P of block j - 1, then S = K.Q of block j.
+  auto slot_a = [&](int j, const uint8_t *lv) {
+    const uint8_t *lk = my_lds + (j & 1) * TILE;
+    issue_v(j + 1);
+    zero_s();
+    // V operands three key steps deep, K operands two batches deep; the reads of a step go out
+    // behind the MFMAs of the step two (one) before it.
+    read_v(lv, 0, 0);
+    read_v(lv, 1, 1);
+    read_k(lk, 0, 0);
 #pragma unroll
-    for (int q = 0; q < D / 32; q++) {
-      if (q + 2 < D / 32) __builtin_amdgcn_sched_group_barrier(0x100, (KT_ROWS ? 4 : 2) * (BKV / 32), 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, BKV / 32, 0);
-      __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, BKV / 32, 0);
-      __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+    for (int u = 0; u < NU; u++) {
+      if (u + 2 < NU) read_v(lv, u + 2, (u + 2) % 3);
+      if (u == NU - 1 && NQ > 1) read_k(lk, 1, 1);
+      pv_step(u, u % 3);
     }
-    // All V operands of the block are requested now: they land while the softmax runs.
-    v4i vf[BKV / 16][D / 32];
 #pragma unroll
-    for (int u = 0; u < BKV / 16; u++) {
-      const int key = 16 * u + 4 * lg + v_rl;  // key & 3 == v_rl; key + 8 swizzles alike
-#pragma unroll
-      for (int t = 0; t < D / 32; t++) {
-        const int off = ((t ^ DD::v_swizzle(key)) << 6) + v_within;
-        const v2i lo = read_tr16(lv + key * ROW + off);
-        const v2i hi = read_tr16(lv + (key + 8) * ROW + off);
-        vf[u][t] = v4i{lo[0], lo[1], hi[0], hi[1]};
-      }
+    for (int q = 0; q < NQ; q++) {
+      qk_step(q, q & 1);
+      if (q + 2 < NQ) read_k(lk, q + 2, q & 1);
     }
-    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 2 * VR + KR, 0);
+#pragma unroll
+    for (int u = 0; u < NU; u++) {
+      if (u + 2 < NU) __builtin_amdgcn_sched_group_barrier(0x100, VR, 0);
+      if (u == NU - 1 && NQ > 1) __builtin_amdgcn_sched_group_barrier(0x100, KR, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, PM, 0);
+    }
+#pragma unroll
+    for (int q = 0; q < NQ; q++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, QM, 0);
+      if (q + 2 < NQ) __builtin_amdgcn_sched_group_barrier(0x100, KR, 0);
+    }
+  };
+  // Slot A after the last block: O += V.P of block nblocks - 1.
+  auto slot_a_last = [&](const uint8_t *lv) {
+    read_v(lv, 0, 0);
+#pragma unroll
+    for (int u = 0; u < NU; u++) {
+      if (u + 1 < NU) read_v(lv, u + 1, (u + 1) % 3);
+      pv_step(u, u % 3);
+    }
+  };
+  // Slot B of block j: the online softmax of S into P (bf16), the running max and denominator.
+  auto slot_b = [&](int j) {
     if (RAGGED) {
       // Keys past n2 (only ever in the very last block): their scores leave the softmax.
-      const int valid = int(p.n2) - (first_block + kb) * BKV;
+      const int valid = int(p.n2) - (first_block + j) * BKV;
       if (valid < BKV) {
 #pragma unroll
         for (int kt = 0; kt < BKV / 32; kt++)
@@ -274,19 +351,20 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
             if (kt * 32 + 8 * (r / 4) + 4 * lg + r % 4 >= valid) s[kt][r] = -__builtin_inff();
       }
     }
-    // Online softmax update for this lane's query, in base 2: exp(x - m) = 2^(x*log2e - m*log2e).
-    float mx = s[0][0];
+    // The running reference m_run (exponentials are taken as exp(x - m_run); the final division
+    // by the denominator, accumulated against the same reference, cancels it exactly) is set from
+    // the first block's maxima and then left alone: a block's maximum is only looked for when its
+    // sum of exponentials shows that some score outgrew the reference by more than 2^40, far
+    // inside f32 and bf16 range.  That block's exponentials are then redone against the moved
+    // reference, and the running sums and the 64 accumulators rescaled.  This takes the maximum
+    // (a quarter of the softmax's instructions and a cross-lane exchange) out of almost every block.
+    auto move_reference = [&]() {
+      float mx = s[0][0];
 #pragma unroll
-    for (int kt = 0; kt < BKV / 32; kt++)
+      for (int kt = 0; kt < BKV / 32; kt++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[kt][r]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    // The reference point m_run only moves when some query's max outgrows it by more than
-    // RESCALE_SLACK: until then exp(x - m_run) <= e^RESCALE_SLACK stays comfortably inside
-    // bf16/f32 range, the final division by the denominator (accumulated against the same
-    // reference) cancels the offset exactly, and the 64 accumulator multiplies of a rescale
-    // are skipped for almost every block.
-    if (__any(mx > m_run + RESCALE_SLACK)) {
+        for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[kt][r]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
       const float m_new = fmaxf(m_run, mx);
       const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * LOG2E);
       m_run = m_new;
@@ -295,10 +373,14 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
       for (int t = 0; t < D / 32; t++)
 #pragma unroll
         for (int r = 0; r < 16; r++) o[t][r] *= alpha;
-    }
+    };
+    if (j == 0) move_reference();
+    // In base 2: exp(x - m) = 2^(x*log2e - m*log2e).
     const float neg_m2 = -m_run * LOG2E;
     float psum = 0.0f;
-    v8bf pb[BKV / 16];
+    // The fetch of K(j + 2) goes out one instruction at a time between the exponentials.
+    const int ksrc = min(j + 2, nblocks - 1);
+    const uint32_t kdst = lds_address(my_lds + (j & 1) * TILE);
 #pragma unroll
     for (int kt = 0; kt < BKV / 32; kt++)
 #pragma unroll
@@ -306,16 +388,48 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
         const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][r], LOG2E, neg_m2));
         psum += e;
         pb[kt * 2 + r / 8][r % 8] = (__bf16)e;
+        constexpr int EVERY = 32 / PER_WAVE;
+        if ((kt * 16 + r) % EVERY == EVERY - 1) {
+          const int i = (kt * 16 + r) / EVERY;
+          dma16(K, k_off(ksrc, i), kdst + (qg * PER_WAVE + i) * 1024);
+        }
       }
+    if (j > 0 && __any(!(psum < STALE_REFERENCE_SUM))) {
+      move_reference();
+      const float neg2 = -m_run * LOG2E;
+      psum = 0.0f;
+#pragma unroll
+      for (int kt = 0; kt < BKV / 32; kt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][r], LOG2E, neg2));
+          psum += e;
+          pb[kt * 2 + r / 8][r % 8] = (__bf16)e;
+        }
+    }
     l_run += psum;
-    // O^T += V^T . P^T.  Key step u covers keys 16u + {4*lg + c, 8 + 4*lg + c}, c = 0..3,
-    // which is the order P^T's registers already have.
-#pragma unroll
-    for (int u = 0; u < BKV / 16; u++)
-#pragma unroll
-      for (int t = 0; t < D / 32; t++)
-        o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, vf[u][t]), pb[u], o[t], 0, 0, 0);
+    __builtin_amdgcn_s_waitcnt(WAIT_BUT_TWO);
+  };
+
+  // Every wave passes steps + 1 pairs of barriers; a half with fewer blocks idles through the rest.
+  if (nblocks > 0) slot_a_first();
+  __syncthreads();
+  if (nblocks > 0) slot_b(0);
+  __syncthreads();
+  int vstage = 0;  // V stage of block j - 1
+  for (int j = 1; j < nblocks; j++) {
+    slot_a(j, my_lds + (2 + vstage) * TILE);
+    vstage = vstage == 2 ? 0 : vstage + 1;
+    __syncthreads();
+    slot_b(j);
+    __syncthreads();
   }
+  if (nblocks > 0) slot_a_last(my_lds + (2 + vstage) * TILE);
+  for (int j = max(nblocks, 1); j <= steps; j++) {
+    __syncthreads();
+    __syncthreads();
+  }
+  if (!half) __syncthreads();
 
   // Merge the two key halves: (m, d, O) of half 1 goes through LDS to the wave of half 0
   // that owns the same queries.  Layout [value][lane] keeps lanes on distinct banks.

@@ -178,6 +178,30 @@ def test_compose_msm_staged_on_the_matrix_cores(gpu, dims):
     assert rel_err(staged, want) < (1e-5 if n2 <= 4096 else 5e-5)
 
 
+@pytest.mark.parametrize("trend", ["rising", "falling", "spike"])
+@pytest.mark.parametrize("dims", [(2, 256, 128, 1024, 128), (1, 130, 64, 700, 64)])
+def test_compose_msm_scores_that_outgrow_the_reference(gpu, dims, trend):
+    """The fused kernel takes its exponentials against a reference it sets from the first block of
+    keys and moves only when a block's sum shows a score more than 2^40 above it.  Keys whose
+    magnitude rises along the sequence (scores from ~1 to ~100: the reference must move, more than
+    once), falls (everything after the first blocks underflows towards zero), or spikes in one
+    late block, against the oracle and against the staged pipeline."""
+    b, m, k, n2, n = dims
+    q, kmat, v = msm_inputs(311, *dims)
+    pos = np.arange(n2, dtype=np.float32) / n2
+    scale = {"rising": 0.05 + 12.0 * pos ** 2, "falling": 12.0 * (1 - pos) ** 2 + 0.05,
+             "spike": np.where((pos > 0.7) & (pos < 0.75), 15.0, 0.2)}[trend]
+    kf = synth.bf16_bits_to_f32(kmat) * scale[None, :, None]
+    kmat = synth.f32_to_bf16_bits(kf.astype(np.float32))
+    spec = M.ComposeMSM(b, m, k, n2, n, layouts=[None, None, KT_LAYOUT, None])
+    got = run_spec(spec, [v, q, kmat, np.zeros((b, m, n), np.float32)])
+    want = orc.compose_msm(b, m, k, n2, n, [7, 7, 7, 6], v, q, kmat, np.zeros((b, m, n), np.float32),
+                           layouts=[None, None, KT_ORC, None])
+    assert np.isfinite(got).all()
+    assert rel_err(got, want) < 1e-2
+    assert elem_err(got, want, floor_frac=1.0) < 2e-2
+
+
 @pytest.mark.parametrize("dims", [(1, 136, 128, 1000, 128), (2, 1, 128, 1, 128), (1, 130, 128, 64, 128),
                                   (3, 200, 128, 70, 128), (1, 128, 128, 2049, 128), (2, 300, 128, 129, 128),
                                   (1, 257, 128, 65, 128), (2, 384, 128, 192, 128),
