@@ -205,10 +205,11 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
   // issues a vector instruction every 6-7 cycles at best and an MFMA wave beside it keeps its
   // full rate, so the exponentials of one half ride under the MFMAs of the other, where two
   // waves in step would queue for the matrix core and then for the vector unit.
-  //   A_j issues the fetch of V(j + 1) (into the tile of V(j - 2), last read in A_(j-1));
-  //   B_j issues the fetch of K(j + 2) (into the tile of K(j), last read in A_j), one instruction
-  //   at a time between the exponentials, and ends by waiting for everything but the last two
-  //   fetches: K(j + 1) and V(j), which A_(j+1) reads, have then landed.  A fetch has two slots.
+  //   B_j issues the fetches of V(j + 1) (into the tile of V(j - 2), last read in A_(j-1)) and of
+  //   K(j + 2) (into the tile of K(j), last read in A_j), one instruction at a time between the
+  //   exponentials (the softmax slot is the shorter one; in the matrix slot they cost more), and
+  //   ends by waiting for everything but its own fetches: K(j + 1) and V(j), which A_(j+1) reads,
+  //   have then landed.
   v16f s[BKV / 32];
   v8bf pb[BKV / 16];
   // Lane-dependent, block-independent parts of the operand addresses (the swizzles depend on the
@@ -286,7 +287,6 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
   // Slot A of the first block: S = K.Q only.
   auto slot_a_first = [&]() {
     const uint8_t *lk = my_lds;
-    issue_v(1);
     zero_s();
     read_k(lk, 0, 0);
 #pragma unroll
@@ -298,7 +298,6 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
   // Slot A of block j, 1 <= j < nblocks: O += V.P of block j - 1, then S = K.Q of block j.
   auto slot_a = [&](int j, const uint8_t *lv) {
     const uint8_t *lk = my_lds + (j & 1) * TILE;
-    issue_v(j + 1);
     zero_s();
     // V operands three key steps deep, K operands two batches deep; the reads of a step go out
     // behind the MFMAs of the step two (one) before it.
@@ -378,9 +377,9 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
     // In base 2: exp(x - m) = 2^(x*log2e - m*log2e).
     const float neg_m2 = -m_run * LOG2E;
     float psum = 0.0f;
-    // The fetch of K(j + 2) goes out one instruction at a time between the exponentials.
-    const int ksrc = min(j + 2, nblocks - 1);
-    const uint32_t kdst = lds_address(my_lds + (j & 1) * TILE);
+    // The fetches of V(j + 1) and K(j + 2) go out one instruction at a time between the exponentials.
+    const int ksrc = min(j + 2, nblocks - 1), vsrc = min(j + 1, nblocks - 1);
+    const uint32_t kdst = lds_address(my_lds + (j & 1) * TILE), vdst = lds_address(my_lds + (2 + (j + 1) % 3) * TILE);
 #pragma unroll
     for (int kt = 0; kt < BKV / 32; kt++)
 #pragma unroll
@@ -388,10 +387,11 @@ __global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
         const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][r], LOG2E, neg_m2));
         psum += e;
         pb[kt * 2 + r / 8][r % 8] = (__bf16)e;
-        constexpr int EVERY = 32 / PER_WAVE;
+        constexpr int EVERY = 16 / PER_WAVE;
         if ((kt * 16 + r) % EVERY == EVERY - 1) {
           const int i = (kt * 16 + r) / EVERY;
-          dma16(K, k_off(ksrc, i), kdst + (qg * PER_WAVE + i) * 1024);
+          if (i < PER_WAVE) dma16(V, v_off(vsrc, i), vdst + (qg * PER_WAVE + i) * 1024);
+          else dma16(K, k_off(ksrc, i - PER_WAVE), kdst + (qg * PER_WAVE + i - PER_WAVE) * 1024);
         }
       }
     if (j > 0 && __any(!(psum < STALE_REFERENCE_SUM))) {
