@@ -254,12 +254,22 @@ int mrl_compose_msm(uint32_t b, uint32_t m, uint32_t k, uint32_t n2, uint32_t n,
  * the GPU kernel: `tile_out([1, tile_m, tile_n])` (one workgroup per output tile) followed
  * by `split(split_k)` (elements of K per step of the k loop)
  * (morello/src/scheduling_sugar.rs:37-132; worked schedules in
- * morello/examples/simple_matmul_x86.rs:60-100, matmul_x86.rs:27-70).  The memory-level
- * moves of a CPU schedule (move_param to L1 / RF / VRF) are fixed by the kernel: HBM -> LDS
- * -> VGPR. */
+ * morello/examples/simple_matmul_x86.rs:60-100, matmul_x86.rs:27-70), and `staging`: the
+ * counterpart of the schedule's move_param steps (which operand is staged in which memory
+ * level, how many buffers deep).  Every tile exists with both operands moved HBM -> VGPR -> LDS
+ * -> VGPR through two LDS stages; the 256 x 256 tile with a 128-byte k step also with B moved
+ * HBM -> LDS directly (three slots, no staging registers) and A through registers, on eight
+ * waves of 128 x 64 outputs or on four waves of 128 x 128, one per SIMD. */
+typedef enum {
+  MRL_STAGING_DEFAULT = 0,        /* what the dispatch rules pick for the tile and shape           */
+  MRL_STAGING_REGISTERS = 1,      /* A, B: HBM -> VGPR -> LDS (2 stages); eight waves (k_gemm)      */
+  MRL_STAGING_DIRECT_B = 2,       /* B: HBM -> LDS (3 slots); eight waves of 128 x 64 (k_gemm_big)  */
+  MRL_STAGING_DIRECT_B_WIDE = 3   /* B: HBM -> LDS (3 slots); four waves of 128 x 128 (k_gemm_wide) */
+} mrl_staging;
 typedef struct {
   uint32_t tile_m, tile_n; /* tile_out */
   uint32_t split_k;        /* split, in elements of K */
+  uint32_t staging;        /* mrl_staging: the move_param steps */
 } mrl_matmul_schedule;
 
 /* Lists the schedules the matrix-core Matmul kernel is built for, for this Spec's dtypes
@@ -485,6 +495,7 @@ typedef struct {
   uint32_t tile_m, tile_n;  /* TILE_OUT_SPLIT, SPATIAL_SPLIT */
   uint32_t split_k;         /* TILE_OUT_SPLIT: elements of K per step */
   uint32_t parts;           /* FUSED on a Compose: shares of the keys */
+  uint32_t staging;         /* TILE_OUT_SPLIT: mrl_staging */
   uint32_t n_steps;         /* filled by mrl_target_actions: launches, */
   uint64_t scratch_bytes;   /*   device scratch (Kernel::memory_allocated) */
   double cost_ns;           /*   and predicted time (Kernel::main_cost) of the action */

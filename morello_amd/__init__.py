@@ -305,18 +305,21 @@ class Spec:
         return ms.value
 
     # -- scheduling sugar (scheduling_sugar.rs:37-132), the subset with a knob in the kernels
-    def available_schedules(self):
-        """[(tile_m, tile_n, split_k)] the matrix-core Matmul kernel is built for."""
+    def available_schedules(self, with_staging: bool = False):
+        """[(tile_m, tile_n, split_k)] the matrix-core Matmul kernel is built for; with_staging:
+        [(tile_m, tile_n, split_k, Staging)], the explicitly staged variants included."""
         buf = (B.MatmulScheduleC * 16)()
-        n = B.load().mrl_matmul_schedules(C.byref(self._c), buf, 16)
-        return [(buf[i].tile_m, buf[i].tile_n, buf[i].split_k) for i in range(min(n, 16))]
+        n = min(B.load().mrl_matmul_schedules(C.byref(self._c), buf, 16), 16)
+        if with_staging:
+            return [(buf[i].tile_m, buf[i].tile_n, buf[i].split_k, Staging(buf[i].staging)) for i in range(n)]
+        return [(buf[i].tile_m, buf[i].tile_n, buf[i].split_k) for i in range(n) if buf[i].staging == 0]
 
     def search_schedule(self) -> "ScheduledMatmul":
         """The manual schedule the cost model predicts cheapest (host only)."""
         sched, cost = B.MatmulScheduleC(), C.c_double()
         _check(B.load().mrl_matmul_search_schedule(C.byref(self._c), C.byref(sched), C.byref(cost)),
                "mrl_matmul_search_schedule")
-        return ScheduledMatmul(self, sched.tile_m, sched.tile_n, sched.split_k)
+        return ScheduledMatmul(self, sched.tile_m, sched.tile_n, sched.split_k, Staging(sched.staging))
 
     def actions(self) -> "list[Action]":
         """Target::actions for this Spec (target/mod.rs:69): the lowerings the backend can run,
@@ -340,19 +343,32 @@ class Spec:
         return best.value, mean.value
 
 
-class ScheduledMatmul:
-    """A Matmul Spec under a manual schedule: `spec.tile_out([1, m, n]).split(k)`."""
+class Staging(enum.IntEnum):
+    """How the k loop brings operand tiles to the matrix cores: the GPU counterpart of a CPU
+    schedule's move_param steps (mrl_staging)."""
+    Default = 0
+    Registers = 1      # A, B: HBM -> VGPR -> LDS, two LDS stages, eight waves
+    DirectB = 2        # B: HBM -> LDS directly, three slots; eight waves of 128 x 64
+    DirectBWide = 3    # the same on four waves of 128 x 128, one per SIMD
 
-    def __init__(self, spec: Spec, tile_m: int, tile_n: int, split_k: Optional[int]):
-        self.spec, self.tile_m, self.tile_n, self.split_k = spec, tile_m, tile_n, split_k
+
+class ScheduledMatmul:
+    """A Matmul Spec under a manual schedule: `spec.tile_out([1, m, n]).split(k)`, optionally
+    `.staged(Staging.X)` for the move_param steps."""
+
+    def __init__(self, spec: Spec, tile_m: int, tile_n: int, split_k: Optional[int], staging: "Staging" = Staging.Default):
+        self.spec, self.tile_m, self.tile_n, self.split_k, self.staging = spec, tile_m, tile_n, split_k, Staging(staging)
 
     def split(self, k: int) -> "ScheduledMatmul":
-        return ScheduledMatmul(self.spec, self.tile_m, self.tile_n, int(k))
+        return ScheduledMatmul(self.spec, self.tile_m, self.tile_n, int(k), self.staging)
+
+    def staged(self, staging: "Staging") -> "ScheduledMatmul":
+        return ScheduledMatmul(self.spec, self.tile_m, self.tile_n, self.split_k, staging)
 
     def plan(self) -> "Plan":
         if self.split_k is None:
             raise MorelloError(1, "schedule needs .split(k)")
-        sched = B.MatmulScheduleC(self.tile_m, self.tile_n, self.split_k)
+        sched = B.MatmulScheduleC(self.tile_m, self.tile_n, self.split_k, int(self.staging))
         fn = lambda spec, head, steps, cap: B.load().mrl_matmul_scheduled_plan(spec, C.byref(sched), head, steps, cap)
         return _plan_of(fn, self.spec._c, "mrl_matmul_scheduled_plan")
 
@@ -361,7 +377,7 @@ class ScheduledMatmul:
         import time
         if self.split_k is None:
             raise MorelloError(1, "schedule needs .split(k)")
-        sched = B.MatmulScheduleC(self.tile_m, self.tile_n, self.split_k)
+        sched = B.MatmulScheduleC(self.tile_m, self.tile_n, self.split_k, int(self.staging))
         arr = (C.c_void_p * len(ptrs))(*ptrs)
         lib = B.load()
         synchronize()
@@ -375,7 +391,7 @@ class ScheduledMatmul:
     def run_device(self, ptrs: Sequence[int]):
         if self.split_k is None:
             raise MorelloError(1, "schedule needs .split(k)")
-        sched = B.MatmulScheduleC(self.tile_m, self.tile_n, self.split_k)
+        sched = B.MatmulScheduleC(self.tile_m, self.tile_n, self.split_k, int(self.staging))
         arr = (C.c_void_p * len(ptrs))(*ptrs)
         _check(B.load().mrl_run_matmul_scheduled(C.byref(self.spec._c), arr, C.byref(sched), None),
                "mrl_run_matmul_scheduled")
@@ -592,13 +608,14 @@ class Action:
 
     def __init__(self, spec: "Spec", c: B.ActionC):
         self.spec = spec
-        self._c = B.ActionC(c.kind, c.tile_m, c.tile_n, c.split_k, c.parts, c.n_steps, c.scratch_bytes, c.cost_ns)
+        self._c = B.ActionC(c.kind, c.tile_m, c.tile_n, c.split_k, c.parts, c.staging, c.n_steps, c.scratch_bytes, c.cost_ns)
         self.kind = ActionKind(c.kind)
         self.tile_m, self.tile_n, self.split_k, self.parts = c.tile_m, c.tile_n, c.split_k, c.parts
+        self.staging = Staging(c.staging)
         self.n_steps, self.scratch_bytes, self.cost_ns = c.n_steps, int(c.scratch_bytes), c.cost_ns
 
     def __repr__(self):
-        knobs = {ActionKind.TileOutSplit: f" tile {self.tile_m}x{self.tile_n} split {self.split_k}",
+        knobs = {ActionKind.TileOutSplit: f" tile {self.tile_m}x{self.tile_n} split {self.split_k}" + (f" {self.staging.name}" if self.staging else ""),
                  ActionKind.SpatialSplit: f" tile {self.tile_m}x{self.tile_n}",
                  ActionKind.Fused: f" parts {self.parts}" if self.parts else ""}.get(self.kind, "")
         return f"Action({self.kind.name}{knobs}: {self.cost_ns:.0f} ns, {self.n_steps} launches, scratch {self.scratch_bytes} B)"

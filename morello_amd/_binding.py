@@ -23,12 +23,12 @@ class LayoutC(C.Structure):
 
 
 class MatmulScheduleC(C.Structure):
-    _fields_ = [("tile_m", C.c_uint32), ("tile_n", C.c_uint32), ("split_k", C.c_uint32)]
+    _fields_ = [("tile_m", C.c_uint32), ("tile_n", C.c_uint32), ("split_k", C.c_uint32), ("staging", C.c_uint32)]
 
 
 class ActionC(C.Structure):
     _fields_ = [("kind", C.c_int32), ("tile_m", C.c_uint32), ("tile_n", C.c_uint32), ("split_k", C.c_uint32),
-                ("parts", C.c_uint32), ("n_steps", C.c_uint32), ("scratch_bytes", C.c_uint64), ("cost_ns", C.c_double)]
+                ("parts", C.c_uint32), ("staging", C.c_uint32), ("n_steps", C.c_uint32), ("scratch_bytes", C.c_uint64), ("cost_ns", C.c_double)]
 
 
 class SpecC(C.Structure):

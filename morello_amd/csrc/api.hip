@@ -515,7 +515,7 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
   if (sched) {
     // A manual schedule is honoured wherever the kernel can run, whatever the size model says.
     if (kind < 0 || !rows || g.b_kmajor || !mrl::gemm_possible(g, kind)) return MRL_ERR_UNSUPPORTED;
-    hipError_t e = mrl::launch_gemm_scheduled(g, kind, sched->tile_m, sched->tile_n, sched->split_k, ws.stream);
+    hipError_t e = mrl::launch_gemm_scheduled(g, kind, sched->tile_m, sched->tile_n, sched->split_k, ws.stream, sched->staging);
     if (e == hipErrorInvalidValue) return MRL_ERR_UNSUPPORTED;
     HIP_TRY(e);
     return finish_output(c, ws);
@@ -1659,7 +1659,7 @@ uint32_t mrl_matmul_schedules(const mrl_spec *spec, mrl_matmul_schedule *out, ui
   if (!es) return 0;
   const uint32_t n = mrl::gemm_schedule_count();
   for (uint32_t i = 0; i < n && out && i < cap; i++)
-    mrl::gemm_schedule_at(i, es, &out[i].tile_m, &out[i].tile_n, &out[i].split_k);
+    mrl::gemm_schedule_at(i, es, &out[i].tile_m, &out[i].tile_n, &out[i].split_k, &out[i].staging);
   return n;
 }
 
@@ -1713,7 +1713,7 @@ int dispatch_action(const mrl_spec &spec, void *const *params, Workspace &ws, co
     case MRL_ACTION_SELECT: return dispatch(spec, params, ws);
     case MRL_ACTION_TILE_OUT_SPLIT: {
       if (spec.kind != MRL_SPEC_MATMUL) return MRL_ERR_UNSUPPORTED;
-      const mrl_matmul_schedule sched = {a.tile_m, a.tile_n, a.split_k};
+      const mrl_matmul_schedule sched = {a.tile_m, a.tile_n, a.split_k, a.staging};
       return run_matmul(spec, params, ws, &sched);
     }
     case MRL_ACTION_SPATIAL_SPLIT: f.conv_path = 2, f.conv_tile = a.tile_m; break;
@@ -1767,7 +1767,10 @@ uint32_t mrl_target_actions(const mrl_spec *spec, mrl_action *out, uint32_t cap)
   if (spec->kind == MRL_SPEC_MATMUL) {
     mrl_matmul_schedule all[16];
     const uint32_t n = std::min<uint32_t>(16, mrl_matmul_schedules(spec, all, 16));
-    for (uint32_t i = 0; i < n; i++) candidate(MRL_ACTION_TILE_OUT_SPLIT, all[i].tile_m, all[i].tile_n, all[i].split_k);
+    for (uint32_t i = 0; i < n; i++) {
+      candidate(MRL_ACTION_TILE_OUT_SPLIT, all[i].tile_m, all[i].tile_n, all[i].split_k);
+      candidates.back().staging = all[i].staging;
+    }
   } else if (spec->kind == MRL_SPEC_CONV) {
     candidate(MRL_ACTION_FUSED);
     for (uint32_t side : {64u, 128u, 256u}) candidate(MRL_ACTION_SPATIAL_SPLIT, side, side, 0);

@@ -89,26 +89,28 @@ uint32_t gemm_k_splits(const GemmArgs &g, int kind) {
   return uint32_t(want);
 }
 
-hipError_t launch_gemm_big(const GemmArgs &g, int kind, hipStream_t stream) {
+hipError_t launch_gemm_big(const GemmArgs &g, int kind, hipStream_t stream, uint32_t staging) {
   if (g.b_kmajor) return launch_gemm_nt(g, kind, 256, stream);
   const bool whole = whole_tiles(g, elem_size_of(kind));
   // Whole tiles and an even number of k steps: the tiles with hand-scheduled k loops.  With a K
   // long enough for its first steps to carry C's old values, four waves with 128 x 128 outputs each
   // (int8 4096^3 accumulating: 69 us; eight waves of 128 x 64: 76 us; the compiler-scheduled loop: 87 us).
-  if (whole && kind <= 2 && wide_applicable(g, elem_size_of(kind))) {
+  if ((staging == 0 || staging == 3) && whole && kind <= 2 && wide_applicable(g, elem_size_of(kind))) {
     switch (kind) {
       case 0: return launch_wide<I8, false>(g, stream);
       case 1: return launch_wide<I8, true>(g, stream);
       case 2: return launch_wide<BF16, false>(g, stream);
     }
   }
-  if (whole && kind <= 2 && big_applicable(g, elem_size_of(kind))) {
+  if (staging == 3) return hipErrorInvalidValue;
+  if ((staging == 0 || staging == 2) && whole && kind <= 2 && big_applicable(g, elem_size_of(kind))) {
     switch (kind) {
       case 0: return launch_big<I8, false>(g, stream);
       case 1: return launch_big<I8, true>(g, stream);
       case 2: return launch_big<BF16, false>(g, stream);
     }
   }
+  if (staging == 2) return hipErrorInvalidValue;
   switch (kind) {
     case 0: return whole ? launch<I8, false, TileBig, false>(g, stream) : launch<I8, false, TileBig, true>(g, stream);
     case 1: return whole ? launch<I8, true, TileBig, false>(g, stream) : launch<I8, true, TileBig, true>(g, stream);

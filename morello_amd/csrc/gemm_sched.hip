@@ -3,8 +3,9 @@
 // (morello/src/scheduling_sugar.rs:37-132; the worked examples are
 // morello/examples/simple_matmul_x86.rs:60-100 and matmul_x86.rs:27-70) picks the workgroup
 // tile and the k step of the matrix-core kernel instead of the library's default.  Only the
-// shapes listed in kSchedules are built; move_param / select steps of a CPU schedule have no
-// knob here (the LDS / register staging is fixed by the kernel).
+// shapes listed in kSchedules are built.  The move_param steps of a CPU schedule (which operand is
+// staged in which memory, how many buffers deep) have one counterpart: `staging` chooses among the
+// three 256 x 256 kernels, which differ in exactly that (mrl_staging in the public header).
 #include "gemm_mfma_kernel.h"
 
 namespace mrl {
@@ -20,10 +21,11 @@ typedef Tile<64, 64, 128, 2, 2> T64x64k128;
 typedef Tile<128, 128, 128, 2, 2> T128x128k128;
 
 struct Entry {
-  uint32_t tile_m, tile_n, k_bytes;
+  uint32_t tile_m, tile_n, k_bytes, staging;
 };
 // k_bytes is the k step in bytes of an operand row: 128 = 128 i8, 64 bf16 or 32 f32 elements.
-const Entry kSchedules[] = {{256, 256, 128}, {256, 256, 64}, {256, 128, 64}, {128, 256, 64}, {128, 128, 64}, {64, 64, 64}, {128, 128, 128}, {64, 64, 128}};
+const Entry kSchedules[] = {{256, 256, 128, 0}, {256, 256, 64, 0}, {256, 128, 64, 0}, {128, 256, 64, 0}, {128, 128, 64, 0}, {64, 64, 64, 0},
+                            {128, 128, 128, 0}, {64, 64, 128, 0}, {256, 256, 128, 1}, {256, 256, 128, 2}, {256, 256, 128, 3}};
 
 template <class TL>
 hipError_t launch_kind(const GemmArgs &g, int kind, hipStream_t stream) {
@@ -39,17 +41,20 @@ hipError_t launch_kind(const GemmArgs &g, int kind, hipStream_t stream) {
 
 uint32_t gemm_schedule_count() { return sizeof(kSchedules) / sizeof(kSchedules[0]); }
 
-void gemm_schedule_at(uint32_t i, int elem_size, uint32_t *tile_m, uint32_t *tile_n, uint32_t *split_k) {
+void gemm_schedule_at(uint32_t i, int elem_size, uint32_t *tile_m, uint32_t *tile_n, uint32_t *split_k, uint32_t *staging) {
   *tile_m = kSchedules[i].tile_m, *tile_n = kSchedules[i].tile_n, *split_k = kSchedules[i].k_bytes / elem_size;
+  *staging = kSchedules[i].staging;
 }
 
 // kind: 0 = i8 x i8, 1 = u8 x i8, 2 = bf16 x bf16, 3 = f32 x f32.  Returns hipErrorInvalidValue for a
 // schedule that is not built.
 hipError_t launch_gemm_scheduled(const GemmArgs &g, int kind, uint32_t tile_m, uint32_t tile_n,
-                                 uint32_t split_k, hipStream_t stream) {
+                                 uint32_t split_k, hipStream_t stream, uint32_t staging) {
   const uint32_t k_bytes = split_k * (kind == 2 ? 2 : kind == 3 ? 4 : 1);
+  if (staging > 3) return hipErrorInvalidValue;
   if (tile_m == 256 && tile_n == 256 && k_bytes == 128)
-    return launch_gemm_big(g, kind, stream);
+    return launch_gemm_big(g, kind, stream, staging);
+  if (staging > 1) return hipErrorInvalidValue;  // the other tiles exist with register staging only
   if (tile_m == 256 && tile_n == 256 && k_bytes == 64) return launch_kind<T256x256k64>(g, kind, stream);
   if (tile_m == 256 && tile_n == 128 && k_bytes == 64) return launch_kind<T256x128k64>(g, kind, stream);
   if (tile_m == 128 && tile_n == 256 && k_bytes == 64) return launch_kind<T128x256k64>(g, kind, stream);

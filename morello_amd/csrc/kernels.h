@@ -94,7 +94,9 @@ uint32_t gemm_k_splits(const GemmArgs &g, int kind);
 hipError_t launch_sum_splits(const void *partial, void *c, uint32_t splits, uint32_t m, uint32_t n, int64_t ldc,
                              bool accum, bool integers, hipStream_t stream);
 // Always the 256 x 256 tile, 128 bytes of K per step.
-hipError_t launch_gemm_big(const GemmArgs &g, int kind, hipStream_t stream);
+// staging: 0 = whichever of the 256 x 256 kernels applies (four waves, eight waves, compiler-scheduled),
+// 1 / 2 / 3 = mrl_staging's REGISTERS / DIRECT_B / DIRECT_B_WIDE only (hipErrorInvalidValue where that one does not apply).
+hipError_t launch_gemm_big(const GemmArgs &g, int kind, hipStream_t stream, uint32_t staging = 0);
 
 // ---- gemv.hip: at most four rows of A against a k-fastest B, as dot products (a stream over B) ----
 bool gemv_applicable(const GemmArgs &g, int kind);
@@ -102,9 +104,9 @@ hipError_t launch_gemv(const GemmArgs &g, int kind, hipStream_t stream);
 
 // ---- gemm_sched.hip: the same kernel under a caller-chosen tile_out / split schedule -----
 uint32_t gemm_schedule_count();
-void gemm_schedule_at(uint32_t i, int elem_size, uint32_t *tile_m, uint32_t *tile_n, uint32_t *split_k);
+void gemm_schedule_at(uint32_t i, int elem_size, uint32_t *tile_m, uint32_t *tile_n, uint32_t *split_k, uint32_t *staging);
 hipError_t launch_gemm_scheduled(const GemmArgs &g, int kind, uint32_t tile_m, uint32_t tile_n,
-                                 uint32_t split_k, hipStream_t stream);
+                                 uint32_t split_k, hipStream_t stream, uint32_t staging = 0);
 
 // ---- conv_i8.hip: NHWC u8|i8 image x KRSC i8 filters -> NHWC i32, implicit GEMM --------
 struct ConvArgs {

@@ -27,7 +27,7 @@ def run_action(action, arrays):
 def test_matmul_actions_against_the_oracle(gpu):
     for dts, np_out, odt in (((M.u8, M.i8, M.i32), np.int32, [orc.U8, orc.I8, orc.I32]),
                              ((M.bf16, M.bf16, M.f32), np.float32, [orc.BF16, orc.BF16, orc.F32])):
-        m, k, n = 512, 384, 256
+        m, k, n = 512, 2560, 256  # K long enough (20 steps of 128 bytes) for every staging of the 256 x 256 tile
         spec = M.MatmulAccum([1, m, k, n], dts)
         if dts[0] == M.u8:
             a, b = synth.uniform_u8(31, 0, (1, m, k)), synth.uniform_i8(31, 1, (1, k, n))
@@ -37,7 +37,7 @@ def test_matmul_actions_against_the_oracle(gpu):
             c0 = synth.normal_f32(31, 2, (1, m, n))
         want = orc.matmul([1, m, k, n], odt, a, b, c0.copy(), True)
         acts = spec.actions()
-        assert len(acts) == 9
+        assert len(acts) == 12 and {a.staging for a in acts} == set(M.Staging)
         for act in acts:
             got = run_action(act, [a, b, c0.copy()])
             if np_out == np.int32:

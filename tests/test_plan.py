@@ -331,8 +331,17 @@ def test_actions_of_the_benchmark_configurations():
     assert acts[0].kind == K.Select and tiles == set(c2().available_schedules()) and len(tiles) == 8
     assert all(a.n_steps == 1 and a.scratch_bytes == 0 and a.cost_ns > 20e3 for a in acts)
     assert acts[0].plan().kernels == ["k_gemm_wide"]
+    # The move_param steps: the 256 x 256 tile under each staging is an action of its own kernel.
+    staged = {a.staging: a for a in acts if a.kind == K.TileOutSplit and a.staging}
+    assert {st: a.plan().kernels for st, a in staged.items()} == {
+        M.Staging.Registers: ["k_gemm"], M.Staging.DirectB: ["k_gemm_big"], M.Staging.DirectBWide: ["k_gemm_wide"]}
+    assert staged[M.Staging.DirectBWide].cost_ns == acts[0].cost_ns < staged[M.Staging.DirectB].cost_ns < staged[M.Staging.Registers].cost_ns
+    assert len(c2().available_schedules(with_staging=True)) == 11
+    # A staging the shape does not admit is no action: K = 1024 is too short for the four-wave kernel.
+    short = M.MatmulAccum([1, 512, 1024, 512], (M.u8, M.i8, M.i32)).actions()
+    assert {a.staging for a in short if a.kind == K.TileOutSplit} == {M.Staging.Default, M.Staging.Registers, M.Staging.DirectB}
     acts = c3().actions()
-    assert len(acts) == 9 and acts[0].cost_ns == min(a.cost_ns for a in acts)
+    assert len(acts) == 12 and acts[0].cost_ns == min(a.cost_ns for a in acts)
     acts = {(a.kind, a.tile_m): a for a in c4().actions()}
     assert set(acts) == {(K.Select, 0), (K.Fused, 0), (K.SpatialSplit, 64), (K.SpatialSplit, 128), (K.SpatialSplit, 256),
                          (K.Unfold, 0), (K.Generic, 0)}
