@@ -33,7 +33,17 @@ constexpr int FT = 4;  // filter tiles of 16 -> F = 64
 #endif
 
 template <int SLABS, bool IMG_UNSIGNED, int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void k_conv_i8(ConvArgs p, uint32_t pixels, uint32_t tiles) {
+__global__ __launch_bounds__(64 * WAVES) void k_conv_i8(const void *image, const void *filters_all, void *out_all, uint32_t c, uint32_t f,
+                                                         uint32_t oh, uint32_t ow, uint32_t fh, uint32_t fw, int accum, uint32_t pixels,
+                                                         uint32_t tiles) {
+  // Scalar arguments, fifteen dwords: few enough to arrive preloaded in SGPRs with the wave
+  // instead of through a load the first instructions would wait for.
+  struct {
+    const void *image, *filters;
+    void *out;
+    uint32_t c, f, oh, ow, fh, fw;
+    int accum;
+  } const p = {image, filters_all, out_all, c, f, oh, ow, fh, fw, accum};
   // The filter bank, staged once per workgroup: rows of krow bytes, 16-byte chunks.
   extern __shared__ __attribute__((aligned(16))) uint8_t filt_lds[];
   const int lane = threadIdx.x & 63;
@@ -100,21 +110,27 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(ConvArgs p, uint32_t pix
 
   // u8 correction 128 * sum_k filt[f][k]: the same MFMAs against an all-ones pixel leave, in
   // every column, the filter sums in exactly the accumulator layout the stores use.  They are
-  // parked in LDS past the filter bank (every wave writes the same 64 numbers and reads back
-  // its own writes, so no barrier is needed).
+  // parked in LDS past the filter bank.  With as many waves as filter tiles each wave forms one
+  // tile's sums (a quarter of the MFMAs, which sit on every wave's path to its first store) and a
+  // barrier hands them round; otherwise every wave writes the same 64 numbers and reads back its
+  // own writes.
   int *corr_lds = (int *)(filt_lds + FT * 16 * krow);
   // Per wave: 16 pixel rows of 64 results, rows 68 dwords apart (16-byte aligned, banks shifted).
   constexpr int TURN_ROW = 68;
   int *turn_lds = corr_lds + FT * 16 + (threadIdx.x >> 6) * (16 * TURN_ROW);
   if (IMG_UNSIGNED) {
     const v4i ones = v4i{0x01010101, 0x01010101, 0x01010101, 0x01010101};
+    constexpr bool SHARED = WAVES == FT;
+    const int my_ft = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 #pragma unroll
     for (int ft = 0; ft < FT; ft++) {
+      if (SHARED && ft != my_ft) continue;
       v4i sum = v4i{0, 0, 0, 0};
 #pragma unroll
       for (int s = 0; s < SLABS; s++) sum = __builtin_amdgcn_mfma_i32_16x16x64_i8(filt[ft][s], ones, sum, 0, 0, 0);
       if (li == 0) *(v4i *)(corr_lds + ft * 16 + lg * 4) = sum * 128;
     }
+    if (SHARED) __syncthreads();
   }
 
   // The pixel registers are refilled slab by slab with the next tile as soon as the MFMAs
@@ -179,9 +195,11 @@ hipError_t launch_slabs(const ConvArgs &c, bool img_unsigned, hipStream_t stream
              double(c.b) * (c.oh + c.fh - 1) * (c.ow + c.fw - 1) * c.c + double(c.f) * c.fh * c.fw * c.c +
                  4.0 * pixels * c.f * (c.accum ? 2 : 1));
   if (img_unsigned)
-    MRL_LAUNCH((k_conv_i8<SLABS, true, WAVES>), dim3(blocks, groups), dim3(64 * WAVES), lds, stream, c, uint32_t(pixels), tiles);
+    MRL_LAUNCH((k_conv_i8<SLABS, true, WAVES>), dim3(blocks, groups), dim3(64 * WAVES), lds, stream, c.image, c.filters, c.out, c.c, c.f, c.oh, c.ow,
+               c.fh, c.fw, c.accum, uint32_t(pixels), tiles);
   else
-    MRL_LAUNCH((k_conv_i8<SLABS, false, WAVES>), dim3(blocks, groups), dim3(64 * WAVES), lds, stream, c, uint32_t(pixels), tiles);
+    MRL_LAUNCH((k_conv_i8<SLABS, false, WAVES>), dim3(blocks, groups), dim3(64 * WAVES), lds, stream, c.image, c.filters, c.out, c.c, c.f, c.oh, c.ow,
+               c.fh, c.fw, c.accum, uint32_t(pixels), tiles);
   return mrl::plan::last_error();
 }
 
