@@ -30,6 +30,7 @@ FLAGS = [
 # start of kernels that only run for a few microseconds.
 EXTRA_FLAGS = {
     "conv_i8.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
+    "attention.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
 }
 
 

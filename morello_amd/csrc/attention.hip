@@ -88,7 +88,16 @@ __device__ inline v2i read_tr16(const uint8_t *p) {
 // read that serves V; the MFMA's k index runs over d in the order that read delivers (4 + 4
 // values per lane half), so Q's operand is loaded in that order too.  n2 must be a multiple of 8.
 template <int D, bool RAGGED, bool KT_ROWS>
-__global__ __launch_bounds__(512) void k_attn(AttnArgs p) {
+__global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, const void *v, float *out, uint32_t b, uint32_t m,
+                                              uint32_t n2, uint32_t n_out, uint32_t key_splits, float *partials) {
+  // Scalar arguments (the file is built with kernel-argument preloading): the first fourteen
+  // dwords arrive in SGPRs with the wave instead of through a load the prologue would wait for.
+  struct {
+    const void *q, *kt, *v;
+    float *out;
+    uint32_t b, m, n2, n_out, key_splits;
+    float *partials;
+  } const p = {q, kt, v, out, b, m, n2, n_out, key_splits, partials};
   typedef Dims<D> DD;
   constexpr int ROW = DD::ROW, TILE = DD::TILE, HALF = DD::HALF;
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
@@ -586,7 +595,8 @@ hipError_t launch_one(const AttnArgs &a, hipStream_t stream) {
              // the softmax between the two products shares the issue slots: 1.45 x the MFMA time
              1.45 * 4.0 * BQ * D * (double((a.n2 + BKV - 1) / BKV) * BKV / std::max(1u, a.key_splits)),
              3000.0);
-  MRL_LAUNCH((k_attn<D, RAGGED, KT_ROWS>), grid, dim3(512), LDS, stream, a);
+  MRL_LAUNCH((k_attn<D, RAGGED, KT_ROWS>), grid, dim3(512), LDS, stream, a.q, a.kt, a.v, a.out, a.b, a.m, a.n2, a.n_out,
+             a.key_splits, a.partials);
   if (a.key_splits > 1) {
     const uint64_t rows = uint64_t(a.b) * a.m, total = rows * a.n_out;
     plan::work(plan::UNIT_STREAM, 0, double(attn_partial_bytes(a, a.key_splits)) + 4.0 * total);
