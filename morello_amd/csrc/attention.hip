@@ -236,16 +236,26 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
       for (int st = 0; st < D / 16; st++) k_lane[st] = lq * ROW + (((2 * st + lg) ^ DD::k_swizzle(lq)) << 4);
     }
   }
+  // s_waitcnt vmcnt(n), n < 16, the other counters left alone.
+  constexpr int WAIT_BUT_TWO = 0x0F70 | (2 * PER_WAVE);
+  // Start-up.  Everything a workgroup asks for at once goes through its compute unit's vector
+  // cache at 64 bytes a clock, so only what the first matrix slot needs is asked for first: Q and
+  // half 0's K(0).  Behind the barrier that says they are in go V(0) and K(1), and all of half 1's
+  // fetches, which have half 0's first slot to land in.  (The wait is for everything in flight, Q's
+  // operand registers included: from there on the only loads in flight are the block fetches,
+  // which the compiler does not know of, so it adds no waits of its own for them in the loop.)
+  if (nblocks > 0 && !half) issue_k(0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  __syncthreads();
   if (nblocks > 0) {
-    issue_k(0);
+    if (half) issue_k(0);
     issue_v(0);
     issue_k(1);
   }
-  __builtin_amdgcn_s_waitcnt(0x0F70);
-  __syncthreads();
-  if (half) __syncthreads();
-  // s_waitcnt vmcnt(n), n < 16, the other counters left alone.
-  constexpr int WAIT_BUT_TWO = 0x0F70 | (2 * PER_WAVE);
+  if (half) {
+    __builtin_amdgcn_s_waitcnt(WAIT_BUT_TWO);  // K(0)
+    __syncthreads();
+  }
   constexpr int NU = BKV / 16, NQ = D / 32;
   constexpr int VR = 2 * (D / 32), KR = (KT_ROWS ? 4 : 2) * (BKV / 32), PM = D / 32, QM = 2 * (BKV / 32);
   v4i kf[2][BKV / 32][2];
