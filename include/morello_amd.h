@@ -474,8 +474,9 @@ int mrl_compose_plan(const mrl_compose *c, mrl_plan *plan, mrl_plan_step *steps,
  *   SELECT          the dispatch rules' own choice for the Spec as it stands (Action::Select)
  *   TILE_OUT_SPLIT  Matmul: tile_out([1, tile_m, tile_n]).split(split_k), then the matrix-core kernel
  *   FUSED           Conv: the fused NHWC/KRSC kernel; Compose Matmul->Softmax->Matmul: the fused kernel
- *                   with the keys in `parts` shares (parallel_softmax.rs:31-223; 1 = one workgroup
- *                   per 128 queries, more = partial results merged with the parts formula)
+ *                   with tile_out over the rows (`tile_m` = 128 or 64 queries per workgroup, 0 = the
+ *                   dispatch rules' choice) and the keys in `parts` shares (parallel_softmax.rs:31-223;
+ *                   1 = one workgroup per query block, more = partial results merged with the parts formula)
  *   SPATIAL_SPLIT   Conv as a Matmul over its windows read in place (spatial_split.rs:73-118),
  *                   tile_out([tile_m, tile_n]) on that Matmul
  *   UNFOLD          Conv: the windows materialised (a Move), then the Matmul
@@ -492,7 +493,7 @@ typedef enum {
 } mrl_action_kind;
 typedef struct {
   int32_t kind;             /* mrl_action_kind */
-  uint32_t tile_m, tile_n;  /* TILE_OUT_SPLIT, SPATIAL_SPLIT */
+  uint32_t tile_m, tile_n;  /* TILE_OUT_SPLIT, SPATIAL_SPLIT; FUSED on a Compose: tile_m = queries per workgroup */
   uint32_t split_k;         /* TILE_OUT_SPLIT: elements of K per step */
   uint32_t parts;           /* FUSED on a Compose: shares of the keys */
   uint32_t staging;         /* TILE_OUT_SPLIT: mrl_staging */

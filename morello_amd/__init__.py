@@ -617,7 +617,8 @@ class Action:
     def __repr__(self):
         knobs = {ActionKind.TileOutSplit: f" tile {self.tile_m}x{self.tile_n} split {self.split_k}" + (f" {self.staging.name}" if self.staging else ""),
                  ActionKind.SpatialSplit: f" tile {self.tile_m}x{self.tile_n}",
-                 ActionKind.Fused: f" parts {self.parts}" if self.parts else ""}.get(self.kind, "")
+                 ActionKind.Fused: (f" rows {self.tile_m}" if self.tile_m else "") + (f" parts {self.parts}" if self.parts else ""),
+                 }.get(self.kind, "")
         return f"Action({self.kind.name}{knobs}: {self.cost_ns:.0f} ns, {self.n_steps} launches, scratch {self.scratch_bytes} B)"
 
     def plan(self) -> "Plan":

@@ -547,6 +547,7 @@ struct Forced {
   uint32_t conv_tile = 0;
   int msm_path = 0;         // 1 fused kernel (key_splits workgroups per query block), 2 staged
   uint32_t key_splits = 0;
+  uint32_t query_block = 0; // fused kernel: queries per workgroup (64 or 128), 0 = the rule below
 };
 thread_local const Forced *g_forced = nullptr;
 
@@ -823,6 +824,11 @@ int run_compose_msm(const mrl_spec &s, void *const *params, Workspace &ws) {
       void *result = params[3];
       if (!out_in_order) HIP_TRY(ws.alloc(&result, size_t(b) * m * n * sizeof(float)));
       at.out = static_cast<float *>(result);
+      // Queries per workgroup (tile_out over the Compose's rows): 64 where 128 would leave half of
+      // the compute units or more without a workgroup, or pad a query dimension of 64 or less.
+      const uint64_t groups128 = uint64_t(b) * ((m + 127) / 128);
+      at.query_block = forced == 1 && g_forced->query_block ? g_forced->query_block
+                       : (m <= 64 || 2 * groups128 <= mrl::g_compute_units) && m > 32 ? 64 : 128;
       at.key_splits = forced == 1 && g_forced->key_splits ? g_forced->key_splits : mrl::attn_key_splits(at);
       if (at.key_splits > 1) {
         void *partials = nullptr;
@@ -1719,7 +1725,9 @@ int dispatch_action(const mrl_spec &spec, void *const *params, Workspace &ws, co
     case MRL_ACTION_SPATIAL_SPLIT: f.conv_path = 2, f.conv_tile = a.tile_m; break;
     case MRL_ACTION_UNFOLD: f.conv_path = 3; break;
     case MRL_ACTION_GENERIC: f.conv_path = 4; break;
-    case MRL_ACTION_FUSED: f.conv_path = 1, f.msm_path = 1, f.key_splits = a.parts ? a.parts : 1; break;
+    case MRL_ACTION_FUSED:
+      f.conv_path = 1, f.msm_path = 1, f.key_splits = a.parts ? a.parts : 1, f.query_block = a.tile_m;
+      break;
     case MRL_ACTION_BUFFERIZE: f.msm_path = 2; break;
     default: return MRL_ERR_BAD_SPEC;
   }
@@ -1780,7 +1788,7 @@ uint32_t mrl_target_actions(const mrl_spec *spec, mrl_action *out, uint32_t cap)
     // parallel_softmax.rs:31-223: the keys in `parts` shares, each at least two blocks of 64.
     const uint32_t blocks = (spec->spec_shape[3] + 63) / 64;
     for (uint32_t parts = 1; parts <= 64 && (parts == 1 || 2 * parts <= blocks); parts *= 2)
-      candidate(MRL_ACTION_FUSED, 0, 0, 0, parts);
+      for (uint32_t rows : {128u, 64u}) candidate(MRL_ACTION_FUSED, rows, 0, 0, parts);
     candidate(MRL_ACTION_BUFFERIZE);
   }
   uint32_t n = 0;

@@ -40,7 +40,7 @@ typedef __attribute__((address_space(3))) v4s lds_v4s;
 typedef __attribute__((address_space(3))) void lds_void;
 typedef __attribute__((address_space(1))) const void global_cvoid;
 
-constexpr int BQ = 128;       // queries per workgroup (4 query groups x 32)
+constexpr int BQ = 128;       // queries per workgroup by default (4 query groups x 32); 64 (2 groups) on request
 constexpr int BKV = 64;       // keys per block
 // Sizes that follow from the head dim D (k and n of the Compose; 32, 64 or 128).
 template <int D>
@@ -87,7 +87,11 @@ __device__ inline v2i read_tr16(const uint8_t *p) {
 // bytes in LDS (one row per d), and the K operand comes out of it through the same transposing
 // read that serves V; the MFMA's k index runs over d in the order that read delivers (4 + 4
 // values per lane half), so Q's operand is loaded in that order too.  n2 must be a multiple of 8.
-template <int D, bool RAGGED, bool KT_ROWS>
+// QG: query groups of 32 per workgroup (4 or 2): the Compose's tile_out over its rows.  A workgroup
+// is 2 * QG waves; with 2 groups the four waves share a compute unit's LDS and matrix cores between
+// them alone, which pays when 128-query blocks would leave half of the compute units without work
+// or pad a short query dimension.
+template <int D, bool RAGGED, bool KT_ROWS, int QG>
 __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, const void *v, float *out, uint32_t b, uint32_t m,
                                               uint32_t n2, uint32_t n_out, uint32_t key_splits, float *partials) {
   // Scalar arguments (the file is built with kernel-argument preloading): the first fourteen
@@ -103,7 +107,8 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int qg = wave & 3, half = wave >> 2;  // query group, key half
+  const int qg = wave % QG, half = wave / QG;  // query group, key half
+  constexpr int BQ = 32 * QG;
   const int lq = lane & 31, lg = lane >> 5;
   // Workgroups go to the 8 XCDs round-robin.  All query blocks of a batch entry share its K
   // and V, so a batch entry's blocks are kept on one XCD (one L2) whenever the counts allow:
@@ -153,8 +158,8 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
   // in 16-byte slot l.  K rows are XOR-swizzled by chunk, V rows by 64-byte unit; each lane
   // fetches the global chunk that belongs in its slot.  The 4 waves of a key half share its
   // instructions: PER_WAVE for K and as many for V per block and wave.
-  constexpr int PER_WAVE = TILE / 1024 / 4;
-  static_assert(PER_WAVE == D / 32, "one staging pair per batch of S MFMAs");
+  constexpr int PER_WAVE = TILE / 1024 / QG;
+  static_assert(PER_WAVE >= 1 && 16 % PER_WAVE == 0, "the fetches are dealt evenly over the softmax's exponentials");
   const int ld_row = lane / DD::CHUNKS, ld_pc = lane % DD::CHUNKS;
   uint32_t k_src[PER_WAVE], v_src[PER_WAVE];
 #pragma unroll
@@ -236,8 +241,8 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
       for (int st = 0; st < D / 16; st++) k_lane[st] = lq * ROW + (((2 * st + lg) ^ DD::k_swizzle(lq)) << 4);
     }
   }
-  // s_waitcnt vmcnt(n), n < 16, the other counters left alone.
-  constexpr int WAIT_BUT_TWO = 0x0F70 | (2 * PER_WAVE);
+  // s_waitcnt vmcnt(n) (six bits: the low four and two at the top), the other counters left alone.
+  constexpr int WAIT_BUT_TWO = 0x0F70 | ((2 * PER_WAVE) & 15) | (((2 * PER_WAVE) >> 4) << 14);
   // Start-up.  Everything a workgroup asks for at once goes through its compute unit's vector
   // cache at 64 bytes a clock, so only what the first matrix slot needs is asked for first: Q and
   // half 0's K(0).  Behind the barrier that says they are in go V(0) and K(1), and all of half 1's
@@ -570,7 +575,7 @@ uint32_t g_compute_units = 256;
 
 uint32_t attn_key_splits(const AttnArgs &a) {
   const uint64_t units = g_compute_units;  // set by mrl_init: planning makes no runtime call
-  const uint64_t groups = uint64_t((a.m + BQ - 1) / BQ) * a.b, blocks = (a.n2 + BKV - 1) / BKV;
+  const uint64_t bq = a.query_block, groups = uint64_t((a.m + bq - 1) / bq) * a.b, blocks = (a.n2 + BKV - 1) / BKV;
   if (groups == 0) return 1;
   const uint64_t splits = std::min<uint64_t>({units / groups, blocks / 4, 256});
   // A workgroup spends ~0.5 us per block; the partial results and their merge cost ~4 us.
@@ -585,17 +590,18 @@ bool attn_applicable(const AttnArgs &a) {
   auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
   return a.k == a.n && (a.k == 32 || a.k == 64 || a.k == 128) && a.n_out >= 1 && a.n_out <= a.n && a.m && a.n2 && a.b &&
          (!a.kt_rows || a.n2 % 8 == 0) && (a.key_splits <= 1 || (a.partials && a.key_splits <= 65535)) &&
-         uint64_t(a.n2) * a.k * 2 < (1ull << 31) && uint64_t((a.m + BQ - 1) / BQ) * a.b < (1u << 31) &&
+         uint64_t(a.n2) * a.k * 2 < (1ull << 31) && (a.query_block == 64 || a.query_block == 128) &&
+         uint64_t((a.m + a.query_block - 1) / a.query_block) * a.b < (1u << 31) &&
          al16(a.q) && al16(a.kt) && al16(a.v) && al16(a.out);
 }
 
 namespace {
-template <int D, bool RAGGED, bool KT_ROWS>
+template <int D, bool RAGGED, bool KT_ROWS, int QG>
 hipError_t launch_one(const AttnArgs &a, hipStream_t stream) {
-  constexpr int LDS = Dims<D>::LDS_BYTES;
+  constexpr int LDS = Dims<D>::LDS_BYTES, BQ = 32 * QG;
   static bool attr_set = false;
   if (!attr_set && !plan::recording()) {
-    hipError_t e = hipFuncSetAttribute((const void *)k_attn<D, RAGGED, KT_ROWS>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+    hipError_t e = hipFuncSetAttribute((const void *)k_attn<D, RAGGED, KT_ROWS, QG>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
     if (e != hipSuccess) return e;
     attr_set = true;
   }
@@ -605,7 +611,7 @@ hipError_t launch_one(const AttnArgs &a, hipStream_t stream) {
              // the softmax between the two products shares the issue slots: 1.45 x the MFMA time
              1.45 * 4.0 * BQ * D * (double((a.n2 + BKV - 1) / BKV) * BKV / std::max(1u, a.key_splits)),
              3000.0);
-  MRL_LAUNCH((k_attn<D, RAGGED, KT_ROWS>), grid, dim3(512), LDS, stream, a.q, a.kt, a.v, a.out, a.b, a.m, a.n2, a.n_out,
+  MRL_LAUNCH((k_attn<D, RAGGED, KT_ROWS, QG>), grid, dim3(128 * QG), LDS, stream, a.q, a.kt, a.v, a.out, a.b, a.m, a.n2, a.n_out,
              a.key_splits, a.partials);
   if (a.key_splits > 1) {
     const uint64_t rows = uint64_t(a.b) * a.m, total = rows * a.n_out;
@@ -616,20 +622,27 @@ hipError_t launch_one(const AttnArgs &a, hipStream_t stream) {
   return mrl::plan::last_error();
 }
 
-template <int D>
+template <int D, int QG>
 hipError_t launch_for(const AttnArgs &a, hipStream_t stream) {
-  const bool whole = a.m % BQ == 0 && a.n2 % (2 * BKV) == 0;
-  if (a.kt_rows) return whole ? launch_one<D, false, true>(a, stream) : launch_one<D, true, true>(a, stream);
-  return whole ? launch_one<D, false, false>(a, stream) : launch_one<D, true, false>(a, stream);
+  const bool whole = a.m % (32 * QG) == 0 && a.n2 % (2 * BKV) == 0;
+  if (a.kt_rows) return whole ? launch_one<D, false, true, QG>(a, stream) : launch_one<D, true, true, QG>(a, stream);
+  return whole ? launch_one<D, false, false, QG>(a, stream) : launch_one<D, true, false, QG>(a, stream);
 }
 }  // namespace
 
 hipError_t launch_attn(const AttnArgs &a, hipStream_t stream) {
   if (!attn_applicable(a)) return hipErrorInvalidValue;
+  if (a.query_block == 64) {
+    switch (a.k) {
+      case 32: return launch_for<32, 2>(a, stream);
+      case 64: return launch_for<64, 2>(a, stream);
+      default: return launch_for<128, 2>(a, stream);
+    }
+  }
   switch (a.k) {
-    case 32: return launch_for<32>(a, stream);
-    case 64: return launch_for<64>(a, stream);
-    default: return launch_for<128>(a, stream);
+    case 32: return launch_for<32, 4>(a, stream);
+    case 64: return launch_for<64, 4>(a, stream);
+    default: return launch_for<128, 4>(a, stream);
   }
 }
 

@@ -172,6 +172,8 @@ struct AttnArgs {
   // was padded with zero columns up to a head dim the kernel is built for.
   uint32_t n_out;
   bool kt_rows = false;  // KT stored row-major, n2 fastest (n2 a multiple of 8)
+  // Queries per workgroup: 128 (eight waves) or 64 (four).
+  uint32_t query_block = 128;
   // More than 1: the keys are shared out over that many workgroups per query block and the
   // partial results merged afterwards; `partials` holds attn_partial_bytes() of scratch.
   uint32_t key_splits = 1;

@@ -70,10 +70,30 @@ def test_compose_actions_against_the_oracle(gpu):
     want = orc.compose_msm(b, m, k, n2, n, [7, 7, 7, 6], v, q, kmat, np.zeros((b, m, n), np.float32),
                            layouts=[None, None, KT_ORC, None])
     acts = spec.actions()
-    assert [a.parts for a in acts if a.kind == M.ActionKind.Fused] == [1, 2, 4, 8] and acts[-1].kind == M.ActionKind.Bufferize
+    assert [(a.parts, a.tile_m) for a in acts if a.kind == M.ActionKind.Fused] == [(p, r) for p in (1, 2, 4, 8) for r in (128, 64)]
+    assert acts[-1].kind == M.ActionKind.Bufferize
     for act in acts:
         got = run_action(act, [v, q, kmat, np.zeros((b, m, n), np.float32)])
         assert rel_err(got, want) < 1e-2, act
+
+
+@pytest.mark.parametrize("dims", [(1, 136, 128, 1000, 128), (3, 200, 128, 70, 128), (2, 1, 128, 1, 128), (1, 257, 64, 65, 64),
+                                  (2, 300, 32, 129, 32), (2, 70, 96, 333, 40)])
+def test_compose_query_blocks_on_ragged_shapes(gpu, dims):
+    """Both query-block sizes of the fused kernel (tile_out over the Compose's rows: 128 or 64
+    queries per workgroup) and every key share count, on sequence lengths that are multiples of
+    neither, head dims the kernel has and one it pads: against the oracle."""
+    b, m, k, n2, n = dims
+    spec = M.ComposeMSM(b, m, k, n2, n, layouts=[None, None, KT, None])
+    v, q, kmat = (synth.normal_bf16(34, 2, (b, n2, n), 0.5), synth.normal_bf16(34, 0, (b, m, k), 0.5),
+                  synth.normal_bf16(34, 1, (b, n2, k), 0.5))
+    want = orc.compose_msm(b, m, k, n2, n, [7, 7, 7, 6], v, q, kmat, np.zeros((b, m, n), np.float32),
+                           layouts=[None, None, KT_ORC, None])
+    fused = [a for a in spec.actions() if a.kind == M.ActionKind.Fused]
+    assert {a.tile_m for a in fused} == {64, 128}
+    for act in fused:
+        sentinel = np.full((b, m, n), 7.5, np.float32)
+        assert rel_err(run_action(act, [v, q, kmat, sentinel]), want) < 1e-2, act
 
 
 def test_actions_of_the_benchmark_configurations_agree(gpu):

@@ -351,9 +351,14 @@ def test_actions_of_the_benchmark_configurations():
     assert acts[(K.Generic, 0)].plan().kernels == ["k_conv_generic"]
     assert acts[(K.Fused, 0)].cost_ns < acts[(K.SpatialSplit, 64)].cost_ns < acts[(K.Unfold, 0)].cost_ns < acts[(K.Generic, 0)].cost_ns
     acts = c5().actions()
-    parts = [a.parts for a in acts if a.kind == K.Fused]
-    assert parts == [1, 2, 4, 8, 16] and acts[-1].kind == K.Bufferize and len(acts[-1].plan().steps) == 3
-    fused = {a.parts: a for a in acts if a.kind == K.Fused}
+    # Fused: the keys in `parts` shares (parallel_softmax.rs) x 128 or 64 queries per workgroup (tile_out over the rows).
+    assert [(a.parts, a.tile_m) for a in acts if a.kind == K.Fused] == [(p, r) for p in (1, 2, 4, 8, 16) for r in (128, 64)]
+    assert acts[-1].kind == K.Bufferize and len(acts[-1].plan().steps) == 3
+    fused = {a.parts: a for a in acts if a.kind == K.Fused and a.tile_m == 128}
+    narrow = {a.parts: a for a in acts if a.kind == K.Fused and a.tile_m == 64}
+    assert "QG = 4" in fused[1].plan().steps[0].kernel and fused[1].plan().steps[0].block == (512, 1, 1)
+    assert "QG = 2" in narrow[1].plan().steps[0].kernel and narrow[1].plan().steps[0].block == (256, 1, 1)
+    assert narrow[1].plan().steps[0].grid[0] == 2 * fused[1].plan().steps[0].grid[0]
     assert fused[1].scratch_bytes == 0 and fused[2].plan().kernels == ["k_attn", "k_attn_merge"]
     assert fused[2].scratch_bytes == 16 * 2048 * 2 * (128 + 4) * 4
     assert acts[0].cost_ns == fused[1].cost_ns == min(a.cost_ns for a in acts)
