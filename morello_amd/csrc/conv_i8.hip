@@ -110,7 +110,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(const void *image, const
 
   // u8 correction 128 * sum_k filt[f][k]: the same MFMAs against an all-ones pixel leave, in
   // every column, the filter sums in exactly the accumulator layout the stores use.  They are
-  // parked in LDS past the filter bank.  With as many waves as filter tiles each wave forms one
+  // parked in LDS past the filter bank.  With a multiple of the filter tiles in waves each wave forms one
   // tile's sums (a quarter of the MFMAs, which sit on every wave's path to its first store) and a
   // barrier hands them round; otherwise every wave writes the same 64 numbers and reads back its
   // own writes.
@@ -120,8 +120,8 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(const void *image, const
   int *turn_lds = corr_lds + FT * 16 + (threadIdx.x >> 6) * (16 * TURN_ROW);
   if (IMG_UNSIGNED) {
     const v4i ones = v4i{0x01010101, 0x01010101, 0x01010101, 0x01010101};
-    constexpr bool SHARED = WAVES == FT;
-    const int my_ft = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    constexpr bool SHARED = WAVES % FT == 0;  // several waves per filter tile write the same numbers
+    const int my_ft = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) % FT;
 #pragma unroll
     for (int ft = 0; ft < FT; ft++) {
       if (SHARED && ft != my_ft) continue;
