@@ -40,7 +40,6 @@ typedef __attribute__((address_space(3))) v4s lds_v4s;
 typedef __attribute__((address_space(3))) void lds_void;
 typedef __attribute__((address_space(1))) const void global_cvoid;
 
-constexpr int BQ = 128;       // queries per workgroup by default (4 query groups x 32); 64 (2 groups) on request
 constexpr int BKV = 64;       // keys per block
 // Sizes that follow from the head dim D (k and n of the Compose; 32, 64 or 128).
 template <int D>

@@ -228,6 +228,21 @@ static float load_as_f32(const void *buf, int dtype, int64_t off) {
   }
 }
 
+/* Float outputs: f32 as it is; bf16 read by widening and written by one rounding to nearest even. */
+static float load_out_f32(const void *buf, int dtype, int64_t off) {
+  return dtype == ORC_BF16 ? orc_bf16_to_f32(((const uint16_t *)buf)[off]) : ((const float *)buf)[off];
+}
+static void store_out_f32(void *buf, int dtype, int64_t off, float v) {
+  if (dtype == ORC_BF16) ((uint16_t *)buf)[off] = orc_f32_to_bf16(v);
+  else ((float *)buf)[off] = v;
+}
+/* Inputs are cast to the output dtype first (verification.rs:629-631): for a bf16 output that
+ * rounds f32 inputs to bf16. */
+static void round_inputs_to(float *v, size_t n, int dt_out) {
+  if (dt_out != ORC_BF16) return;
+  for (size_t i = 0; i < n; i++) v[i] = orc_bf16_to_f32(orc_f32_to_bf16(v[i]));
+}
+
 static void store_from_u32(void *buf, int dtype, int64_t off, uint32_t v) {
   switch (dtype) {
     case ORC_U8:
@@ -310,7 +325,6 @@ int orc_matmul_rows(const uint32_t spec_shape[4], const int dtypes[3],
   const uint32_t B = spec_shape[0], M = spec_shape[1], K = spec_shape[2], N = spec_shape[3];
   const uint32_t sa[3] = {B, M, K}, sb[3] = {B, K, N}, sc[3] = {B, M, N};
   const int dt_out = dtypes[2];
-  if (dt_out == ORC_BF16) return ORC_UNSUPPORTED;
   if (row_end > M || row_begin > row_end) return ORC_BAD_ARG;
   int bad_a, bad_b, bad_c;
   int64_t *ta = offset_table(layouts ? layouts[0] : NULL, sa, 3, &bad_a);
@@ -322,14 +336,18 @@ int orc_matmul_rows(const uint32_t spec_shape[4], const int dtypes[3],
   }
   const size_t na = (size_t)B * M * K, nb = (size_t)B * K * N;
   if (is_float(dt_out)) {
+    /* A bf16 output: inputs cast to bf16, products summed in f32, one rounding at the end.  The
+     * reference rounds after every operation (bf16 arithmetic) and has no comparison for it
+     * (verification.rs:597 `todo!`): this is the documented, more accurate reading. */
     float *fa = gather_f32(a, dtypes[0], ta, na);
     float *fb = gather_f32(b, dtypes[1], tb, nb);
+    round_inputs_to(fa, na, dt_out), round_inputs_to(fb, nb, dt_out);
     float *row = (float *)malloc(sizeof(float) * N);
     for (uint32_t bi = 0; bi < B; bi++) {
       for (uint32_t i = row_begin; i < row_end; i++) {
         for (uint32_t j = 0; j < N; j++) {
           size_t ci = ((size_t)bi * M + i) * N + j;
-          row[j] = accum ? ((const float *)c)[tc ? tc[ci] : (int64_t)ci] : 0.0f;
+          row[j] = accum ? load_out_f32(c, dt_out, tc ? tc[ci] : (int64_t)ci) : 0.0f;
         }
         const float *ar = fa + ((size_t)bi * M + i) * K;
         for (uint32_t k = 0; k < K; k++) {
@@ -339,7 +357,7 @@ int orc_matmul_rows(const uint32_t spec_shape[4], const int dtypes[3],
         }
         for (uint32_t j = 0; j < N; j++) {
           size_t ci = ((size_t)bi * M + i) * N + j;
-          ((float *)c)[tc ? tc[ci] : (int64_t)ci] = row[j];
+          store_out_f32(c, dt_out, tc ? tc[ci] : (int64_t)ci, row[j]);
         }
       }
     }
@@ -386,7 +404,6 @@ int orc_conv(const uint32_t spec_shape[7], const int dtypes[3], const orc_layout
   const uint32_t H = OH + FH - 1, W = OW + FW - 1;
   const uint32_t si[4] = {B, C, H, W}, sf[4] = {F, C, FH, FW}, so[4] = {B, F, OH, OW};
   const int dt_out = dtypes[2];
-  if (dt_out == ORC_BF16) return ORC_UNSUPPORTED;
   int bad_i, bad_f, bad_o;
   int64_t *ti = offset_table(layouts ? layouts[0] : NULL, si, 4, &bad_i);
   int64_t *tf = offset_table(layouts ? layouts[1] : NULL, sf, 4, &bad_f);
@@ -399,19 +416,20 @@ int orc_conv(const uint32_t spec_shape[7], const int dtypes[3], const orc_layout
   if (is_float(dt_out)) {
     float *im = gather_f32(image, dtypes[0], ti, ni);
     float *fl = gather_f32(filters, dtypes[1], tf, nf);
+    round_inputs_to(im, ni, dt_out), round_inputs_to(fl, nf, dt_out);
     for (uint32_t b = 0; b < B; b++)
       for (uint32_t f = 0; f < F; f++)
         for (uint32_t y = 0; y < OH; y++)
           for (uint32_t x = 0; x < OW; x++) {
             size_t oi = (((size_t)b * F + f) * OH + y) * OW + x;
             int64_t off = to ? to[oi] : (int64_t)oi;
-            float acc = accum ? ((const float *)out)[off] : 0.0f;
+            float acc = accum ? load_out_f32(out, dt_out, off) : 0.0f;
             for (uint32_t c = 0; c < C; c++)
               for (uint32_t r = 0; r < FH; r++)
                 for (uint32_t s = 0; s < FW; s++)
                   acc += im[(((size_t)b * C + c) * H + y + r) * W + x + s] *
                          fl[(((size_t)f * C + c) * FH + r) * FW + s];
-            ((float *)out)[off] = acc;
+            store_out_f32(out, dt_out, off, acc);
           }
     free(im), free(fl);
   } else {

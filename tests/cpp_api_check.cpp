@@ -38,7 +38,7 @@ int main() {
   EXPECT(msm.is_supported() && msm.flops() == 34359738368ull + 335544320ull);
   EXPECT((msm.parameter_shape(2) == Shape{16, 128, 2048}));
   EXPECT(Spec::matmul({1, 4096, 4096, 4096}, Dtype::Uint8, Dtype::Sint8, Dtype::Sint32).flops() == 137438953472ull);
-  EXPECT(!Spec::matmul({1, 4, 4, 4}, Dtype::Float32, Dtype::Float32, Dtype::Bfloat16).is_supported());
+  EXPECT(Spec::matmul({1, 4, 4, 4}, Dtype::Float32, Dtype::Float32, Dtype::Bfloat16).is_supported());  // bf16 output: a legal triple
   // The primitives of the Softmax decomposition and a general Compose (spec.rs:3733-3785).
   Spec sdm = Spec::softmax_part(SpecType::SoftmaxDenominatorAndMax, {4, 6, 8}, 1, true);
   EXPECT(sdm.parameter_count() == 3 && (sdm.parameter_shape(2) == Shape{4, 1, 8}));

@@ -114,7 +114,7 @@ def test_spec_check_status_codes():
     assert M.Matmul([1, 64, 64, 64], [M.f32] * 3).check() == 0
     assert M.Matmul([1, 64, 0, 64], [M.f32] * 3).check() == 3          # zero dim
     assert M.Spec(M.SpecKind.Matmul, [1, 2, 3], [M.f32] * 3, layouts=[M.Layout([])] * 3).check() == 3  # rank
-    assert M.Matmul([1, 4, 4, 4], [M.f32, M.f32, M.bf16]).check() == 1  # bf16 output
+    assert M.Matmul([1, 4, 4, 4], [M.f32, M.f32, M.bf16]).check() == 0  # bf16 output: a legal triple (spec.rs:3663-3698)
     assert M.Softmax([4, 4], 2).check() == 3                              # scan_dim out of range
     bad = M.layout((0, M.Packed(4)), 1)                                   # layout.rs:1520-1527
     assert M.Matmul([1, 8, 64, 64], [M.f32] * 3,

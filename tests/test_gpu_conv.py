@@ -191,3 +191,19 @@ def test_conv_full_size_properties(gpu):
     filt[:] = -128
     got = run_spec(M.Conv((1,) + shape[1:], (M.u8, M.i8, M.i32)), [img[:1], filt, np.zeros((1, oh, ow, f), np.int32)])
     assert (got == -18800640).all()
+
+
+@pytest.mark.parametrize("accum", [False, True])
+def test_conv_with_bf16_output(gpu, accum):
+    """Conv bf16 x bf16 -> bf16 (NHWC / KRSC buffers): f32 sums, one rounding (see
+    test_matmul_with_bf16_output)."""
+    b, f, c, oh, ow, fh, fw = 2, 24, 40, 9, 11, 3, 2
+    img = synth.normal_bf16(78, 0, (b, oh + fh - 1, ow + fw - 1, c), 0.5)
+    filt = synth.normal_bf16(78, 1, (f, fh, fw, c), 0.5)
+    out0 = synth.normal_bf16(78, 2, (b, oh, ow, f), 2.0) if accum else np.zeros((b, oh, ow, f), np.uint16)
+    want = synth.bf16_bits_to_f32(orc.conv([b, f, c, oh, ow, fh, fw], [7, 7, 7], img, filt, out0.copy(), accum=accum,
+                                           layouts=[NHWC, NHWC, NHWC]))
+    got = synth.bf16_bits_to_f32(run_spec(M.Conv([b, f, c, oh, ow, fh, fw], (M.bf16, M.bf16, M.bf16), accum=accum),
+                                          [img, filt, out0.copy()]))
+    assert (got == want).mean() > 0.97
+    assert np.all(np.abs(got - want) <= 2.0 ** -7 * np.maximum(np.abs(want), 2.0 ** -10 * np.abs(want).max()))

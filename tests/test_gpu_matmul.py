@@ -494,3 +494,30 @@ def test_float_operands_saturate_at_the_output_dtype(gpu):
         orc_dt = {M.i8: orc.I8, M.u8: orc.U8, M.u16: orc.U16, M.i16: orc.I16}[dt]
         ref = orc.matmul([1, 1, 6, 6], [orc.F32, orc.F32, orc_dt], a, b, np.zeros((1, 6), np_dt))
         assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("dts,codes", [((M.bf16, M.bf16, M.bf16), [7, 7, 7]), ((M.f32, M.f32, M.bf16), [6, 6, 7]),
+                                       ((M.bf16, M.f32, M.bf16), [7, 6, 7]), ((M.u8, M.i8, M.bf16), [0, 1, 7])])
+@pytest.mark.parametrize("accum", [False, True])
+def test_matmul_with_bf16_output(gpu, dts, codes, accum):
+    """bf16 outputs (spec.rs:3663-3698): inputs cast to bf16, f32 sums on the matrix cores, one
+    rounding to bf16 (old output included for the accumulating form).  The oracle sums in k order,
+    the kernel in its own, so sums may round to neighbouring bf16 values: nearly all elements are
+    bit-identical and none is further than one rounding step (2^-8 relative) apart.  The reference
+    itself has no comparison for bf16 (verification.rs:597)."""
+    b, m, k, n = 2, 200, 384, 136
+    def operand(dt, tid, shape):
+        return {M.bf16: lambda: synth.normal_bf16(77, tid, shape, 0.5), M.f32: lambda: synth.normal_f32(77, tid, shape, 0.5),
+                M.u8: lambda: synth.uniform_u8(77, tid, shape), M.i8: lambda: synth.uniform_i8(77, tid, shape)}[dt]()
+    a, bm = operand(dts[0], 0, (b, m, k)), operand(dts[1], 1, (b, k, n))
+    c0 = synth.normal_bf16(77, 2, (b, m, n), 3.0) if accum else np.zeros((b, m, n), np.uint16)
+    want = synth.bf16_bits_to_f32(orc.matmul([b, m, k, n], codes, a, bm, c0.copy(), accum))
+    got = synth.bf16_bits_to_f32(run_spec(M.Matmul([b, m, k, n], dts, accum=accum), [a, bm, c0.copy()]))
+    assert np.isfinite(got).all()
+    assert (got == want).mean() > 0.97
+    assert np.all(np.abs(got - want) <= 2.0 ** -7 * np.maximum(np.abs(want), 2.0 ** -10 * np.abs(want).max()))
+    # A column-major output and a packed input keep working through the same road.
+    if dts == (M.bf16, M.bf16, M.bf16) and not accum:
+        spec = M.Matmul([b, m, k, n], dts, layouts=[None, None, M.batched_col_major([b, m, n])])
+        got_t = synth.bf16_bits_to_f32(run_spec(spec, [a, bm, np.zeros((b, n, m), np.uint16)]))
+        assert np.array_equal(got_t.transpose(0, 2, 1), got)

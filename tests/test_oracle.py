@@ -258,6 +258,40 @@ def test_float_operands_saturate_at_the_output_dtype():
     assert int(got[0, 0]) == np.int8((127 * 127) & 0xff)
 
 
+def test_bf16_outputs_round_once():
+    """A bf16 output (spec.rs:3663-3698): both inputs cast to bf16 first (verification.rs:629-631),
+    products summed in f32, the sum rounded to bf16 once, to nearest even.  Expected values worked out
+    by hand: small integers are exact in bf16, so products and short sums are, and the first sums that
+    are not (257, 259: ties between neighbours 2 apart) show the rounding."""
+    bf = synth.f32_to_bf16_bits
+    val = synth.bf16_bits_to_f32
+    a = bf(np.array([[[1, 2, 3], [4, 5, 6]]], np.float32))                 # [1, 2, 3]
+    b = bf(np.array([[[1, 0, 16], [0, 1, 32], [1, 1, 64]]], np.float32))   # [1, 3, 3]
+    got = orc.matmul([1, 2, 3, 3], [orc.BF16] * 3, a, b, np.zeros((1, 2, 3), np.uint16))
+    # row 0: [1+3, 2+3, 16+64+192] = [4, 5, 272]; row 1: [4+6, 5+6, 64+160+384] = [10, 11, 608]
+    assert val(got).tolist() == [[[4, 5, 272], [10, 11, 608]]]
+    ones = bf(np.ones((1, 1, 257), np.float32))
+    col = bf(np.ones((1, 257, 1), np.float32))
+    assert val(orc.matmul([1, 1, 257, 1], [orc.BF16] * 3, ones, col, np.zeros((1, 1, 1), np.uint16)))[0, 0, 0] == 256.0  # 257: tie, to even
+    ones, col = bf(np.ones((1, 1, 259), np.float32)), bf(np.ones((1, 259, 1), np.float32))
+    assert val(orc.matmul([1, 1, 259, 1], [orc.BF16] * 3, ones, col, np.zeros((1, 1, 1), np.uint16)))[0, 0, 0] == 260.0  # 259: tie, to even
+    # accumulating: the old output joins the f32 sum before the rounding: 256 + 1 -> 257 -> 256, 256 + 3 -> 259 -> 260
+    c = bf(np.array([[[256.0, 256.0]]], np.float32))
+    got = orc.matmul([1, 1, 1, 2], [orc.BF16] * 3, bf(np.ones((1, 1, 1), np.float32)), bf(np.array([[[1.0, 3.0]]], np.float32)), c, accum=True)
+    assert val(got).tolist() == [[[256.0, 260.0]]]
+    # f32 inputs are cast to bf16 first: 1 + 2^-8 is a tie and becomes 1, 1 + 3 * 2^-8 becomes 1 + 2^-6
+    af = np.array([[[1 + 2.0 ** -8, 1 + 3 * 2.0 ** -8]]], np.float32)
+    eye = np.eye(2, dtype=np.float32)[None]
+    got = orc.matmul([1, 1, 2, 2], [orc.F32, orc.F32, orc.BF16], af, eye, np.zeros((1, 1, 2), np.uint16))
+    assert val(got).tolist() == [[[1.0, 1 + 2.0 ** -6]]]
+    # Conv takes the same road: a 1x1 filter over small integers is the exact integer result
+    img = bf(np.arange(2 * 3 * 2 * 2, dtype=np.float32).reshape(2, 3, 2, 2) % 5)
+    filt = bf(np.array([[[[1]], [[2]], [[3]]], [[[0]], [[1]], [[0]]]], np.float32))
+    got = orc.conv([2, 2, 3, 2, 2, 1, 1], [orc.BF16] * 3, img, filt, np.zeros((2, 2, 2, 2), np.uint16))
+    want = np.einsum("bchw,fc->bfhw", val(img), val(filt)[:, :, 0, 0])
+    assert np.array_equal(val(got), want)
+
+
 def test_conv_degenerate_cases():
     # 1x1 filter == Matmul [1, B*H*W, C, F] (scheduling/spatial_split.rs:73-102)
     b, f, c, h, w = 2, 5, 7, 3, 4
