@@ -75,7 +75,10 @@ typedef struct {
  * three-component Compose of examples/matmul_chain.rs). */
 typedef enum {
   MRL_SPEC_MATMUL = 0,     /* spec_shape [b,m,k,n]; params A[b,m,k] B[b,k,n] C[b,m,n]   */
-  MRL_SPEC_CONV = 1,       /* spec_shape [b,f,c,oh,ow,fh,fw]; params image, filters, out */
+  MRL_SPEC_CONV = 1,       /* spec_shape [b,f,c,oh,ow,fh,fw]; params image, filters, out.
+                              Both: any dtype triple; inputs are cast to the output dtype
+                              (verification.rs:547-569, 629-631), integer outputs wrap, f32
+                              outputs sum in f32, bf16 outputs sum in f32 and round once    */
   MRL_SPEC_SOFTMAX = 2,    /* spec_shape = tensor shape; params in, out; uses scan_dim   */
   MRL_SPEC_COMPOSE_MSM = 3,/* Matmul->Softmax->Matmul; spec_shape [b,m,k,n2,n];
                               params V[b,n2,n] Q[b,m,k] KT[b,k,n2] out[b,m,n]
