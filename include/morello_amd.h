@@ -190,7 +190,8 @@ int mrl_spec_check(const mrl_spec *spec);
  * kernels do not walk in place (Packed / OddEven dims in another order than row-major); 0 when
  * every parameter is read in place.  A lower bound on the call's scratch: operand copies made
  * for speed (zero-padded rows, column-major operands made row-major, unfolded Conv windows, up
- * to 1 GiB) and the intermediates of a Compose come from the same allocator on top of it. */
+ * to 1 GiB), the f32 image of a bf16 Matmul/Conv output with the bf16 copies of its inputs, and
+ * the intermediates of a Compose come from the same allocator on top of it. */
 size_t mrl_spec_workspace_bytes(const mrl_spec *spec);
 
 /* -------------------------------------------------------------- execution */
