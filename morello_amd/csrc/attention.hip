@@ -176,14 +176,18 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
     }
     v_src[i] = row * ROW + ((((ld_pc >> 2) ^ DD::v_swizzle(row)) << 6) | ((ld_pc & 3) << 4));
   }
-  // Byte offset within the batch entry's K (V) of this lane's chunk i of block kb.
-  auto k_off = [&](int kb, int i) {
-    const uint32_t off = uint32_t(first_block + kb) * (KT_ROWS ? BKV * 2 : TILE) + k_src[i];
-    return RAGGED ? min(off, head_bytes - 16) : off;
+  // Fetch of this lane's chunk i of K (V) block kb into the KiB at LDS address `dst`.  The block's
+  // offset is wave-uniform and goes into the scalar base; only the ragged form, which clamps
+  // each lane's address to the entry's last bytes, forms the offset per lane.
+  auto fetch_k = [&](int kb, int i, uint32_t dst) {
+    const uint32_t block = uint32_t(first_block + kb) * (KT_ROWS ? BKV * 2 : TILE);
+    if constexpr (RAGGED) dma16(K, min(block + k_src[i], head_bytes - 16), dst);
+    else dma16(K + block, k_src[i], dst);
   };
-  auto v_off = [&](int kb, int i) {
-    const uint32_t off = uint32_t(first_block + kb) * TILE + v_src[i];
-    return RAGGED ? min(off, head_bytes - 16) : off;
+  auto fetch_v = [&](int kb, int i, uint32_t dst) {
+    const uint32_t block = uint32_t(first_block + kb) * TILE;
+    if constexpr (RAGGED) dma16(V, min(block + v_src[i], head_bytes - 16), dst);
+    else dma16(V + block, v_src[i], dst);
   };
   v16f o[D / 32];
 #pragma unroll
@@ -204,13 +208,13 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
     const int src = min(kb, nblocks - 1);
     const uint32_t dst = lds_address(my_lds + (kb & 1) * TILE);
 #pragma unroll
-    for (int i = 0; i < PER_WAVE; i++) dma16(K, k_off(src, i), dst + (qg * PER_WAVE + i) * 1024);
+    for (int i = 0; i < PER_WAVE; i++) fetch_k(src, i, dst + (qg * PER_WAVE + i) * 1024);
   };
   auto issue_v = [&](int kb) {
     const int src = min(kb, nblocks - 1);
     const uint32_t dst = lds_address(my_lds + (2 + kb % 3) * TILE);
 #pragma unroll
-    for (int i = 0; i < PER_WAVE; i++) dma16(V, v_off(src, i), dst + (qg * PER_WAVE + i) * 1024);
+    for (int i = 0; i < PER_WAVE; i++) fetch_v(src, i, dst + (qg * PER_WAVE + i) * 1024);
   };
 
   // The two key halves of a workgroup run the same program ONE SLOT APART.  A wave's work per
@@ -418,8 +422,8 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
         constexpr int EVERY = 16 / PER_WAVE;
         if ((kt * 16 + r) % EVERY == EVERY - 1) {
           const int i = (kt * 16 + r) / EVERY;
-          if (i < PER_WAVE) dma16(V, v_off(vsrc, i), vdst + (qg * PER_WAVE + i) * 1024);
-          else dma16(K, k_off(ksrc, i - PER_WAVE), kdst + (qg * PER_WAVE + i - PER_WAVE) * 1024);
+          if (i < PER_WAVE) fetch_v(vsrc, i, vdst + (qg * PER_WAVE + i) * 1024);
+          else fetch_k(ksrc, i - PER_WAVE, kdst + (qg * PER_WAVE + i - PER_WAVE) * 1024);
         }
       }
     if (j > 0 && __any(!(psum < STALE_REFERENCE_SUM))) {
