@@ -201,3 +201,47 @@ def test_random_conv_mid_sizes(gpu, seed):
     want = orc.conv(shape, [int(d) for d in dts], bufs[0], bufs[1], bufs[2].copy(), accum,
                     layouts=[l[1] for l in lay])
     compare(got, want, dts[2], (shape, dts, accum, [repr(l[0]) for l in lay]))
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_compose_msm(gpu, seed):
+    """Matmul -> Softmax -> Matmul over random shapes: sequence lengths around the fused kernel's
+    blocks (128 or 64 queries, 2 x 64 keys), head dims it is built for and ones it pads, the two
+    head dims equal or not, KT k-fastest (layout![0,2,1]) or in the reference's default order,
+    scores of random spread.  The dispatch rules' own choice and every fused action (both query
+    blocks, every key share count) against the oracle: norm-wise 1e-2, and element-wise against
+    a floor of the result's rms (bf16 rounding of P bounds the error per output, not per digit)."""
+    from gpu_util import elem_err
+    rng = np.random.default_rng(9900 + seed)
+    b = int(rng.integers(1, 5))
+    m = int(rng.choice([1, 2, 17, 31, 32, 33, 63, 64, 65, 100, 127, 128, 129, 200, 256, 300]))
+    n2 = int(rng.choice([1, 7, 8, 63, 64, 65, 127, 128, 129, 200, 256, 264, 500, 777, 1024, 1500]))
+    k = int(rng.choice([8, 16, 24, 32, 40, 64, 96, 128]))
+    n = k if rng.random() < 0.6 else int(rng.choice([2, 8, 32, 48, 64, 100, 128]))
+    kt_fastest = rng.random() < 0.6
+    spread = float(rng.choice([0.2, 0.5, 1.0, 1.5]))
+    q = synth.normal_bf16(9900 + seed, 0, (b, m, k), spread)
+    v = synth.normal_bf16(9900 + seed, 2, (b, n2, n), 0.5)
+    if kt_fastest:
+        kmat = synth.normal_bf16(9900 + seed, 1, (b, n2, k), spread)   # K row-major == KT as layout![0,2,1]
+        lay, olay = [None, None, M.layout(0, 2, 1), None], [None, None, orc.make_layout([0, 2, 1]), None]
+    else:
+        kmat = synth.normal_bf16(9900 + seed, 1, (b, k, n2), spread)   # KT row-major, n2 fastest
+        lay, olay = None, None
+    spec = M.ComposeMSM(b, m, k, n2, n, layouts=lay)
+    want = orc.compose_msm(b, m, k, n2, n, [7, 7, 7, 6], v, q, kmat, np.zeros((b, m, n), np.float32), layouts=olay)
+    what = (b, m, k, n2, n, kt_fastest, spread)
+
+    def run(target):
+        bufs = [M.DeviceBuffer.from_numpy(a) for a in (v, q, kmat, np.full((b, m, n), 7.5, np.float32))]
+        target.run_device([x.ptr for x in bufs])
+        out = bufs[-1].to_numpy(np.float32, (b, m, n))
+        for x in bufs:
+            x.free()
+        return out
+
+    for target in [spec] + [a for a in spec.actions() if a.kind == M.ActionKind.Fused]:
+        got = run(target)
+        assert np.isfinite(got).all(), (what, target)
+        assert rel_err(got, want) < 1e-2, (what, target)
+        assert elem_err(got, want, floor_frac=1.0) < 2e-2, (what, target)
