@@ -303,6 +303,8 @@ def measure(name, steps, warmup, min_gpu_s):
                 "frac": achieved / peak, "traffic": MEASURED_TRAFFIC_BYTES.get(name),
                 "kernel_ms": kernel_ms, "kernel_ms_min": kernel_ms_min, "kernel_ms_sustained": kernel_ms,
                 "algorithmic_ops": ops, "algorithmic_bytes": alg_bytes}
+    if name == "c1":
+        roofline["note"] = "launch-latency bound (a 64^3 problem): kernel_ms is the figure, frac is not a roofline claim"
     if bound == "mfma":
         # What the matrix cores of this board sustain with no memory traffic at all, on
         # operands distributed like the workload's: the published peak assumes the full
