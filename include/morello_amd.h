@@ -147,7 +147,8 @@ typedef enum {
 
 /* ------------------------------------------------------------- life cycle */
 
-/* Selects `device` and checks that it is a gfx950 part.  Idempotent. */
+/* Selects `device` and checks that it is a gfx950 part.  Idempotent.  (No counterpart in the
+ * reference, whose target is the host CPU.) */
 int mrl_init(int device);
 const char *mrl_status_string(int status);
 /* Text of the last HIP error seen by this thread ("" if none). */
@@ -243,7 +244,8 @@ int mrl_conv(uint32_t b, uint32_t f, uint32_t c, uint32_t oh, uint32_t ow, uint3
              const void *filters, void *out, void *stream);
 int mrl_softmax(const uint32_t *shape, uint32_t rank, uint32_t scan_dim, const void *in,
                 void *out, void *stream);
-/* Move: copies `in` to `out` (dense row-major both sides, same dtype). */
+/* Move (spec.rs:63, scheduling/moves.rs:16-22): copies `in` to `out` (dense row-major both
+ * sides, same dtype). */
 int mrl_move(const uint32_t *shape, uint32_t rank, int dtype, const void *in, void *out,
              void *stream);
 /* KT is the B operand of the first Matmul, logical [b,k,n2]; kt_col_major != 0 says it is
@@ -365,6 +367,10 @@ int mrl_measure_mfma_rate(int kind, int random_operands, uint32_t iters, double 
 
 /* ------------------------------------------- device memory (plumbing only) */
 
+/* What the emitted main does around the kernel call on the host: 128-byte aligned buffers per
+ * parameter (codegen/c_utils.rs:77-93, codegen/cpu.rs:38), filled from the parameter files
+ * (cpu.rs:221-270) or with zeros (cpu.rs:320), freed after the call (cpu.rs:399-403).  Device
+ * allocations are aligned to 256 bytes or more. */
 int mrl_device_malloc(void **ptr, size_t bytes);
 int mrl_device_free(void *ptr);
 int mrl_memcpy_h2d(void *dst, const void *src, size_t bytes);
