@@ -359,3 +359,59 @@ def test_softmax_tensor_beyond_4_gib(gpu):
                                rtol=1e-5, atol=1e-9)
     din.free()
     dout.free()
+
+
+@pytest.mark.parametrize("shape,dim", [((6, 256), 1), ((6, 2048), 1), ((6, 4100), 1), ((6, 9000), 1), ((6, 40000), 1),
+                                       ((6, 33), 1), ((6, 5), 1), ((300, 6, 12), 2), ((6, 700, 8), 1), ((3, 2, 1100), 2)])
+def test_softmax_infinities_follow_the_reference(gpu, shape, dim):
+    """Rows with infinities and NaNs on every Softmax kernel (rows in registers, short rows, a
+    workgroup per row, rows in chunks, a scan dim that is not the innermost), as the reference's
+    interpreter treats them (verification.rs:166-184 with the NaN-propagating max that starts
+    from f32::MIN, :842-861): -inf among finite scores gives exact zeros; a row that is all
+    -inf, or holds +inf or a NaN, is NaN throughout; the other rows are untouched by it."""
+    x = synth.normal_f32(206, 0, shape)
+    lines = np.moveaxis(x, dim, -1).reshape(-1, shape[dim])   # a copy: one row per softmax
+    n = lines.shape[1]
+    lines[0, ::2] = -np.inf          # finite scores between -inf
+    lines[1, :] = -np.inf            # nothing but -inf
+    lines[2, n // 2] = np.inf        # one +inf
+    lines[3, n - 1] = np.nan         # a NaN in the last place
+    lines[4, 0] = -np.inf            # a single -inf
+    moved = np.moveaxis(x, dim, -1)
+    x = np.ascontiguousarray(np.moveaxis(lines.reshape(moved.shape), -1, dim))
+    got = run_spec(M.Softmax(list(shape), dim), [x, np.zeros_like(x)])
+    want = orc.softmax(list(shape), dim, x)
+    g = np.moveaxis(got, dim, -1).reshape(-1, n)
+    w = np.moveaxis(want, dim, -1).reshape(-1, n)
+    assert np.isnan(w[1]).all() and np.isnan(w[2]).all() and np.isnan(w[3]).all()   # the oracle itself
+    assert np.array_equal(np.isnan(g), np.isnan(w))
+    assert (g[0, ::2] == 0).all() and g[4, 0] == 0
+    ok = ~np.isnan(w)
+    assert (np.abs(g[ok] - w[ok]) <= 1e-5 * np.abs(w[ok]) + 1e-12).all()
+
+
+@pytest.mark.parametrize("dims,where", [((2, 200, 64, 300, 64), 150), ((1, 130, 128, 700, 128), 5), ((1, 64, 32, 1100, 32), 1099)])
+def test_compose_msm_with_an_infinite_key(gpu, dims, where):
+    """One +inf in K: a query whose product with it is +inf has a NaN row (inf - inf in the
+    softmax, verification.rs:166-184), one whose product is -inf gives that key weight zero and
+    is otherwise unchanged.  On the fused kernel the infinity arrives in the first key block or
+    in a later one, where the running reference has to move to it; every fused action agrees."""
+    b, m, k, n2, n = dims
+    q, kmat, v = msm_inputs(312, *dims)
+    kf = synth.bf16_bits_to_f32(kmat)
+    kf[0, where, 3] = np.inf
+    kmat = synth.f32_to_bf16_bits(kf)
+    spec = M.ComposeMSM(b, m, k, n2, n, layouts=[None, None, KT_LAYOUT, None])
+    want = orc.compose_msm(b, m, k, n2, n, [7, 7, 7, 6], v, q, kmat, np.zeros((b, m, n), np.float32),
+                           layouts=[None, None, KT_ORC, None])
+    nan_rows = np.isnan(want).all(axis=2)
+    assert nan_rows[0].any() and not nan_rows[0].all() and np.array_equal(np.isnan(want).any(axis=2), nan_rows)
+    for target in [spec] + [a for a in spec.actions() if a.kind == M.ActionKind.Fused]:
+        bufs = [M.DeviceBuffer.from_numpy(a) for a in (v, q, kmat, np.zeros((b, m, n), np.float32))]
+        target.run_device([x.ptr for x in bufs])
+        got = bufs[-1].to_numpy(np.float32, (b, m, n))
+        for x in bufs:
+            x.free()
+        assert np.array_equal(np.isnan(got), np.isnan(want)), target
+        ok = ~np.isnan(want)
+        assert np.abs(got[ok] - want[ok]).max() / np.abs(want[ok]).max() < 1e-2, target
