@@ -607,11 +607,10 @@ namespace {
 template <int D, bool RAGGED, bool KT_ROWS, int QG>
 hipError_t launch_one(const AttnArgs &a, hipStream_t stream) {
   constexpr int LDS = Dims<D>::LDS_BYTES, BQ = 32 * QG;
-  static bool attr_set = false;
-  if (!attr_set && !plan::recording()) {
-    hipError_t e = hipFuncSetAttribute((const void *)k_attn<D, RAGGED, KT_ROWS, QG>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+  static std::atomic<uint64_t> lds_limit_set{0};
+  if (!plan::recording()) {
+    hipError_t e = raise_lds_limit(lds_limit_set, (const void *)k_attn<D, RAGGED, KT_ROWS, QG>, LDS);
     if (e != hipSuccess) return e;
-    attr_set = true;
   }
   const dim3 grid(((a.m + BQ - 1) / BQ) * a.b, std::max(1u, a.key_splits));
   plan::work(plan::UNIT_MFMA_BF16, 4.0 * a.b * a.m * a.n2 * D,

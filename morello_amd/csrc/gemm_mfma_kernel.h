@@ -545,12 +545,10 @@ hipError_t launch(const GemmArgs &g, hipStream_t stream) {
   constexpr int BM = TL::BM, BN = TL::BN;
   constexpr int STAGE = TL::template stage<T>();
   if (EDGE && !edge_addressable(g, T::ES)) return hipErrorInvalidValue;
-  static bool attr_set = false;
-  if (!attr_set && !plan::recording()) {
-    hipError_t e = hipFuncSetAttribute((const void *)kern,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 2 * STAGE);
+  static std::atomic<uint64_t> lds_limit_set{0};
+  if (!plan::recording()) {
+    hipError_t e = raise_lds_limit(lds_limit_set, (const void *)kern, 2 * STAGE);
     if (e != hipSuccess) return e;
-    attr_set = true;
   }
   const int tiles_m = int((g.m + BM - 1) / BM), tiles_n = int((g.n + BN - 1) / BN);
   {

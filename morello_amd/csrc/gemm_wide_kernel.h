@@ -184,11 +184,10 @@ inline bool wide_applicable(const GemmArgs &g, int elem_size) {
 template <class T, bool A_UNSIGNED>
 hipError_t launch_wide(const GemmArgs &g, hipStream_t stream) {
   constexpr auto kern = k_gemm_wide<T, A_UNSIGNED>;
-  static bool attr_set = false;
-  if (!attr_set && !plan::recording()) {
-    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, WIDE_LDS_BYTES);
+  static std::atomic<uint64_t> lds_limit_set{0};
+  if (!plan::recording()) {
+    hipError_t e = raise_lds_limit(lds_limit_set, (const void *)kern, WIDE_LDS_BYTES);
     if (e != hipSuccess) return e;
-    attr_set = true;
   }
   const int tiles_m = int(g.m / 256), tiles_n = int(g.n / 256);
   const double mn = double(g.m) * g.n * g.batch;

@@ -3,10 +3,27 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "layout_math.h"
 #include "plan.h"
 
 namespace mrl {
+
+// Raises a kernel's limit of dynamic LDS to `bytes`, once per device: the attribute belongs to
+// the device the calling thread has selected, and launches may come from several threads.
+// `done` is the kernel's own flag word, one bit per device.
+inline hipError_t raise_lds_limit(std::atomic<uint64_t> &done, const void *kernel, int bytes) {
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = 1ull << (device & 63);
+  if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+  return e;
+}
+
 
 // A tensor whose layout is a pure permutation of its logical dims.
 struct Strided {
