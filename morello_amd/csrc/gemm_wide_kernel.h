@@ -1,19 +1,23 @@
 // The 256 x 256 Matmul tile on four waves, one per SIMD, each holding a 128 x 128 block of C in
 // 256 accumulation registers: u8|i8 x i8 -> i32 and bf16 x bf16 -> f32 on whole tiles with a long
 // K.  k loop and epilogue are written in assembly (gemm_wide_gfx950.inc, generated and
-// documented by gen_gemm_wide.py, which also says why this shape: the fewest instructions per
-// MFMA).
+// documented by gen_gemm_wide.py, which also says why this shape -- the fewest instructions per
+// MFMA cycle -- and why MFMAs of 16 x 16 x 64 bytes: the least energy per multiply-add on a
+// power-limited board).
 //
-// Same arithmetic and LDS operand layouts as k_gemm (gemm_mfma_kernel.h; semantics:
-// morello/src/spec.rs:480-485, morello/src/codegen/cpu.rs:2114-2124).  For an accumulating
-// Spec the old value of an element joins its sum during the first k steps instead of after the
-// last; integers are exact either way, floats differ from k_gemm's order by one rounding.
+// Same arithmetic as k_gemm (gemm_mfma_kernel.h; semantics: morello/src/spec.rs:480-485,
+// morello/src/codegen/cpu.rs:2114-2124).  For an accumulating Spec the old value of an element
+// joins its sum during the first k steps instead of after the last; integers are exact either
+// way, floats differ from k_gemm's order by one rounding.
 //   move_param(A, L1)  -> global_load_dwordx4 -> (xor 0x80 for u8) -> ds_write_b128, two stages
 //   move_param(B, L1)  -> global_load_lds_dwordx4 into a ring of three 32 KiB slots
-// The B tile is stored [k][n] without row padding; the pieces of a row (32 bytes for i8, 64 for
-// bf16) are XOR-ed with the low bits of the row number so that the rows one transposing read
-// touches fall on different banks.  A direct-to-LDS instruction writes 1 KiB of consecutive LDS
-// bytes, 16 per lane, so the swizzle is applied on the source side.
+// The A tile is stored as k_gemm stores it (rows of 128 bytes, 16-byte chunks XOR-ed with
+// (row / 2) & 7).  The B tile is stored [k][n] without row padding.  One half of a transposing
+// read (32 lanes) touches 8 (i8) / 4 (bf16) k rows of two lane groups, 16 k (8 k) apart, at the
+// same 16 (32) bytes of the row: the pieces of a row (32 bytes for i8, 64 for bf16) are XOR-ed
+// with the low bits of the row number and the halves of a piece with the row bit that tells the
+// two lane groups apart, so that these rows fall on different banks.  A direct-to-LDS instruction
+// writes 1 KiB of consecutive LDS bytes, 16 per lane, so the swizzle is applied on the source side.
 #pragma once
 #include "gemm_mfma_kernel.h"
 #include "gemm_wide_gfx950.inc"
@@ -22,8 +26,18 @@ namespace mrl {
 namespace gemm {
 
 template <class T> struct WideTraits;
-template <> struct WideTraits<I8> { static constexpr int PIECE = 32, RMASK = 7; };
-template <> struct WideTraits<BF16> { static constexpr int PIECE = 64, RMASK = 3; };
+// PIECE, RMASK: see above; GROUP_SHIFT: log2 of the k rows one lane group of an MFMA operand holds.
+template <> struct WideTraits<I8> { static constexpr int PIECE = 32, RMASK = 7, GROUP_SHIFT = 4; };
+template <> struct WideTraits<BF16> { static constexpr int PIECE = 64, RMASK = 3, GROUP_SHIFT = 3; };
+
+// Byte position within a k row of the B tile in LDS <-> within the row in memory (an involution).
+template <class T>
+__device__ inline int wide_b_swizzle(int byte, int k) {
+  constexpr int PIECE = WideTraits<T>::PIECE, HALF = PIECE / 2;
+  const int piece = (byte / PIECE) ^ (k & WideTraits<T>::RMASK);
+  const int half = ((byte % PIECE) / HALF) ^ ((k >> WideTraits<T>::GROUP_SHIFT) & 1);
+  return piece * PIECE + half * HALF + byte % HALF;
+}
 
 constexpr int WIDE_B_BASE = 2 * 32768;       // LDS: [A stage 0][A stage 1][B slot 0][B slot 1][B slot 2]
 constexpr int WIDE_LDS_BYTES = 5 * 32768;
@@ -38,9 +52,8 @@ constexpr int WIDE_MIN_STEPS = GEMM_WIDE_MIN_STEPS;
       MRL_WIDE_10(p, 3), MRL_WIDE_10(p, 4), MRL_WIDE_10(p, 5), MRL_WIDE_10(p, 6), MRL_WIDE_10(p, 7),        \
       MRL_WIDE_10(p, 8), MRL_WIDE_10(p, 9)
 #define MRL_WIDE_CLOBBERS                                                                                   \
-  MRL_WIDE_FIRST_100("v"), MRL_WIDE_10("v", 10), MRL_WIDE_10("v", 11), MRL_WIDE_10("v", 12),                \
-      MRL_WIDE_10("v", 13), MRL_WIDE_10("v", 14), MRL_WIDE_10("v", 15), MRL_WIDE_10("v", 16), "v170",       \
-      "v171", MRL_WIDE_FIRST_100("a"), MRL_WIDE_100("a", 1), MRL_WIDE_10("a", 20), MRL_WIDE_10("a", 21),    \
+  MRL_WIDE_FIRST_100("v"), MRL_WIDE_100("v", 1), MRL_WIDE_10("v", 20), "v210", "v211",                      \
+      MRL_WIDE_FIRST_100("a"), MRL_WIDE_100("a", 1), MRL_WIDE_10("a", 20), MRL_WIDE_10("a", 21),            \
       MRL_WIDE_10("a", 22), MRL_WIDE_10("a", 23), MRL_WIDE_10("a", 24), "a250", "a251", "a252", "a253",     \
       "a254", "a255", "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71",   \
       "s72", "s73", "s78", "s79", "scc", "memory"
@@ -52,28 +65,23 @@ constexpr int WIDE_MIN_STEPS = GEMM_WIDE_MIN_STEPS;
                  [a_off4] "v"(a_off[4]), [a_off5] "v"(a_off[5]), [a_off6] "v"(a_off[6]), [a_off7] "v"(a_off[7]),   \
                  [b_off0] "v"(b_off[0]), [b_off1] "v"(b_off[1]), [b_off2] "v"(b_off[2]), [b_off3] "v"(b_off[3]),   \
                  [b_off4] "v"(b_off[4]), [b_off5] "v"(b_off[5]), [b_off6] "v"(b_off[6]), [b_off7] "v"(b_off[7]),   \
-                 [a_wr] "v"(a_wr), [a_rd0] "v"(a_rd[0]), [a_rd1] "v"(a_rd[1]), [a_rd2] "v"(a_rd[2]),               \
-                 [a_rd3] "v"(a_rd[3]), [b_rd0] "v"(b_rd[0]), [b_rd1] "v"(b_rd[1]), [b_rd2] "v"(b_rd[2]),           \
-                 [b_rd3] "v"(b_rd[3]), [c_row0] "v"(c_row[0]), [c_row1] "v"(c_row[1]), [c_row2] "v"(c_row[2]),     \
-                 [c_row3] "v"(c_row[3]), [c_row4] "v"(c_row[4]), [c_row5] "v"(c_row[5]), [c_row6] "v"(c_row[6]),   \
-                 [c_row7] "v"(c_row[7]), [c_row8] "v"(c_row[8]), [c_row9] "v"(c_row[9]),                           \
-                 [c_row10] "v"(c_row[10]), [c_row11] "v"(c_row[11]), [c_row12] "v"(c_row[12]),                     \
-                 [c_row13] "v"(c_row[13]), [c_row14] "v"(c_row[14]), [c_row15] "v"(c_row[15]),                     \
-                 [part_wr] "v"(part_wr), [part_rd] "v"(part_rd), [abase] "s"(A), [bbase] "s"(B),                   \
-                 [bstep] "s"(b_step), [nk] "s"(nk), [dma_base] "s"(dma_base), [cbase] "s"(c_base),                 \
-                 [ldc32] "s"(ldc32), [k32] "s"(k32)                                                                \
+                 [a_wr] "v"(a_wr), [a_rd0] "v"(a_rd[0]), [a_rd1] "v"(a_rd[1]), [b_rd0] "v"(b_rd[0]),               \
+                 [b_rd1] "v"(b_rd[1]), [b_rd2] "v"(b_rd[2]), [b_rd3] "v"(b_rd[3]), [b_rd4] "v"(b_rd[4]),           \
+                 [b_rd5] "v"(b_rd[5]), [b_rd6] "v"(b_rd[6]), [b_rd7] "v"(b_rd[7]), [c_row0] "v"(c_row[0]),         \
+                 [c_row1] "v"(c_row[1]), [c_row2] "v"(c_row[2]), [c_row3] "v"(c_row[3]), [part_wr] "v"(part_wr),   \
+                 [part_rd] "v"(part_rd), [abase] "s"(A), [bbase] "s"(B), [bstep] "s"(b_step), [nk] "s"(nk),        \
+                 [dma_base] "s"(dma_base), [cbase] "s"(c_base), [ldc16] "s"(ldc16), [k16] "s"(k16)                 \
                : MRL_WIDE_CLOBBERS)
 
 // M, N multiples of 256; K an even number of k steps, GEMM_WIDE_MIN_STEPS at least; see wide_applicable().
 template <class T, bool A_UNSIGNED>
 __global__ __launch_bounds__(256) void k_gemm_wide(GemmArgs g, int tiles_m, int tiles_n, int group_m) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-  constexpr int BM = 256, BN = 256, BKB = 128, WM = 128, WN = 128, TN = 4;
+  constexpr int BM = 256, BN = 256, BKB = 128, WM = 128, WN = 128, TN = 8;
   constexpr int ES = T::ES, BK = BKB / ES;
   constexpr int B_ROWB = BN * ES;              // bytes per k row of the B tile
-  constexpr int PIECE = WideTraits<T>::PIECE, RMASK = WideTraits<T>::RMASK;
   constexpr int ROWS_PER_DMA = 1024 / B_ROWB;  // k rows one direct-to-LDS instruction fills: 4 (i8), 2 (bf16)
-  constexpr int K_SLAB = 32 / ES;
+  constexpr int GROUP_K = 16 / ES;             // k rows a lane group of an MFMA operand holds: 16 (i8), 8 (bf16)
   typedef typename T::Out Out;
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -115,44 +123,44 @@ __global__ __launch_bounds__(256) void k_gemm_wide(GemmArgs g, int tiles_m, int 
 #pragma unroll
   for (int j = 0; j < 8; j++) {
     const int r = (wave * 8 + j) * ROWS_PER_DMA + (lane * 16) / B_ROWB;
-    const int inrow = (lane * 16) % B_ROWB;
-    const int piece = (inrow / PIECE) ^ (r & RMASK);
-    b_off[j] = uint32_t(r) * ldb_b + piece * PIECE + inrow % PIECE + 4096 - j * 1024;
+    b_off[j] = uint32_t(r) * ldb_b + wide_b_swizzle<T>((lane * 16) % B_ROWB, r) + 4096 - j * 1024;
   }
   const uint32_t dma_base = lds0 + WIDE_B_BASE + wave * 8192;
-  // Operand reads.  A: lane (l % 32, l / 32) of MFMA block tm reads 16 bytes of row
-  // wm * 128 + tm * 32 + l % 32 at chunk 2 * s + l / 32 of slab s.
-  uint32_t a_rd[4];
+  // Operand reads.  A: lane (l % 16, l / 16) of block row tm reads 16 bytes of row
+  // wm * 128 + tm * 16 + l % 16 at chunk 4 * s + l / 16 of the 64-byte slab s.
+  uint32_t a_rd[2];
   {
-    const int sw = ((lane & 31) / 2) & 7, half = lane >> 5;
+    const int sw = ((lane & 15) / 2) & 7, group = lane >> 4;
 #pragma unroll
-    for (int s = 0; s < 4; s++) a_rd[s] = lds0 + (wm * WM + (lane & 31)) * BKB + (((2 * s + half) ^ sw) << 4);
+    for (int s = 0; s < 2; s++) a_rd[s] = lds0 + (wm * WM + (lane & 15)) * BKB + (((4 * s + group) ^ sw) << 4);
   }
-  // B: a 16-lane group of a transposing read fetches K_PER_READ k rows x 16 columns; lane p of
-  // the group addresses 8 bytes of one k row and receives the column it indexes.
-  uint32_t b_rd[4];
+  // B: a 16-lane group of a transposing read fetches 8 (i8) / 4 (bf16) k rows x 16 columns; lane p
+  // of the group addresses 8 bytes of one k row and receives the column it indexes.  Group g reads
+  // the k rows GROUP_K * g on of the slab (a second read takes the other half of them) for the
+  // 16 columns of block column tn.
+  uint32_t b_rd[TN];
   {
     constexpr int LANES_PER_ROW = 16 / (8 / ES);
     const int p = lane & 15;
-    const int k = (K_SLAB / 2) * (lane >> 5) + p / LANES_PER_ROW;
+    const int k = GROUP_K * (lane >> 4) + p / LANES_PER_ROW;
 #pragma unroll
     for (int tn = 0; tn < TN; tn++) {
-      const int byte = (wn * WN + tn * 32 + 16 * ((lane >> 4) & 1) + (8 / ES) * (p % LANES_PER_ROW)) * ES;
-      b_rd[tn] = lds0 + k * B_ROWB + (((byte / PIECE) ^ (k & RMASK)) * PIECE) + byte % PIECE;
+      const int byte = (wn * WN + tn * 16 + (8 / ES) * (p % LANES_PER_ROW)) * ES;
+      b_rd[tn] = lds0 + k * B_ROWB + wide_b_swizzle<T>(byte, k);
     }
   }
-  // C: register r of a 32 x 32 block holds row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32.
-  uint32_t c_row[16];
+  // C: register i of a 16 x 16 block holds row 4 * (l / 16) + i, column l % 16.
+  uint32_t c_row[4];
 #pragma unroll
-  for (int r = 0; r < 16; r++) c_row[r] = uint32_t((lane >> 5) * 4 + (r >> 2) * 8 + (r & 3)) * ldc_b + (lane & 31) * 4;
+  for (int i = 0; i < 4; i++) c_row[i] = uint32_t((lane >> 4) * 4 + i) * ldc_b + (lane & 15) * 4;
   const uint8_t *c_base = (const uint8_t *)(C + int64_t(wm * WM) * g.ldc + wn * WN);
-  const uint32_t ldc32 = 32 * ldc_b;
-  // Column-sum partials [wave row x lane half][256 columns], in LDS from its start once the loop is over.
-  const uint32_t part_wr = lds0 + ((wm * 2 + (lane >> 5)) * BN + wn * WN + (lane & 31)) * 4;
-  const uint32_t part_rd = lds0 + (wn * WN + (lane & 31)) * 4;
+  const uint32_t ldc16 = 16 * ldc_b;
+  // Column-sum partials [wave row x lane group][256 columns], in LDS from its start once the loop is over.
+  const uint32_t part_wr = lds0 + ((wm * 4 + (lane >> 4)) * BN + wn * WN + (lane & 15)) * 4;
+  const uint32_t part_rd = lds0 + (wn * WN + (lane & 15)) * 4;
 
   const uint32_t b_step = uint32_t(BK) * ldb_b;
-  const uint32_t nk = g.k / BK, k32 = 32 * g.k;
+  const uint32_t nk = g.k / BK, k16 = 16 * g.k;
 
   if constexpr (std::is_same<T, BF16>::value) {
     if (g.accum) MRL_WIDE_RUN(GEMM_WIDE_BF16_ACC);
@@ -161,7 +169,7 @@ __global__ __launch_bounds__(256) void k_gemm_wide(GemmArgs g, int tiles_m, int 
     if (g.accum) MRL_WIDE_RUN(GEMM_WIDE_I8_ACC);
     else MRL_WIDE_RUN(GEMM_WIDE_I8);
   } else {
-    // The two wave rows share B's columns and each adds up the column sums of every other slab.
+    // The two wave rows share B's columns and each adds up the column sums of one slab of every step.
     if (g.accum) {
       if (wm == 0) MRL_WIDE_RUN(GEMM_WIDE_U8_0_ACC);
       else MRL_WIDE_RUN(GEMM_WIDE_U8_1_ACC);

@@ -2,16 +2,28 @@
 """Writes gemm_wide_gfx950.inc: the 256 x 256 Matmul tile on four waves, one per SIMD, each with a
 128 x 128 block of C in 256 accumulation registers; k loop and epilogue in gfx950 assembly.
 
-Why this shape.  Measured on the matrix cores of an MI355X: an MFMA of 32 x 32 x 32 bytes keeps a
-SIMD's matrix core busy for 32 cycles, and about four and a half other instructions of the waves
-of that SIMD issue under it for free; every further one delays the next MFMA by about four
-cycles, whichever wave it comes from.  So the k loop wants as few instructions per MFMA as it
-can get: the largest block of C per wave (operands read from LDS once serve four MFMAs each way)
-and one wave per SIMD (no per-wave bookkeeping twice).  Per 32-byte slab of K a wave issues
-16 MFMAs against 12 LDS reads (4 ds_read_b128 of A, 8 transposing ds_read_b64_tr of B).
+Why this shape.  Measured on the matrix cores of an MI355X: about two other instructions of a
+SIMD's waves issue for free under 16 cycles of MFMA work, every further one delays the next MFMA by
+about four cycles, whichever wave it comes from.  So the k loop wants as few instructions per MFMA
+cycle as it can get: the largest block of C per wave (an operand read from LDS once serves eight
+MFMAs) and one wave per SIMD (no per-wave bookkeeping twice).
 
-One k step (tile kt, 128 bytes of K, four slabs):
-  * the operands of slab s + 1 are read from LDS behind the first MFMAs of slab s;
+Why MFMAs of 16 x 16 x 64 bytes (v_mfma_i32_16x16x64_i8, v_mfma_f32_16x16x32_bf16) and not of
+32 x 32 x 32: the board is power-limited, and on operands distributed like a benchmark's the
+16 x 16 form sustains 4000 TOPS int8 / 2070 TFLOPS bf16 where the 32 x 32 form sustains 3360 /
+1840 (back-to-back MFMAs on register operands, all SIMDs): it updates an accumulator once per 64
+multiply-adds instead of once per 32.  The same k loop with either form: 65.1 against 70.6 us at
+4096^3 int8, 798 against 842 us at 8192^3 bf16, same box.
+
+One k step (tile kt, 128 bytes of K) is two slabs of 64 bytes; a slab is 8 x 8 MFMAs, block row
+tm outermost.  Per slab a wave reads 8 A operands (ds_read_b128: lane (l % 16, l / 16) takes row
+l % 16 of the block row and the l / 16-th 16 bytes of the slab) and 8 B operands (two transposing
+ds_read_b64_tr each: the 16-lane group l / 16 takes the same 16 k of the slab for the block's 16
+columns).  The k index of an MFMA is a contraction index: which 16 bytes of K a lane group holds is
+free as long as both operands agree, and here both hold bytes 16 g .. 16 g + 15 of the slab.
+  * A operands have ONE register set: block row tm's operand is used by eight MFMAs in a row and
+    is dead after them, so the next slab's goes into the same registers right behind its last use,
+    56 MFMAs before its first.  B operands are used all through a slab and have two sets.
   * A of tile kt + 1 goes from a register set to its LDS stage (xor 0x80 on the way for a u8
     operand: a - 128, once per byte) and the set is refilled with tile kt + 3 from global memory:
     two register sets, two LDS stages;
@@ -20,25 +32,27 @@ One k step (tile kt, 128 bytes of K, four slabs):
     addresses, tell the pieces apart);
   * the column sums of B that the u8 correction needs are added up from the B operand registers
     (xor 0x80, sum of unsigned bytes: b + 128; the dot-product instructions hold up the MFMAs
-    behind them); the two wave rows share the columns and take every other slab each;
-  * one barrier, before the MFMAs of the last slab, preceded by the step's wait for memory:
-    everything requested before this step began has landed;
-  * an accumulating Spec loads C's old values during the first sixteen steps, one block a step,
-    and adds them to the block's accumulators a step later, between two of the block's MFMAs,
-    so that the epilogue only stores.
+    behind them); the two wave rows share the columns and take one slab of a step each;
+  * one barrier, three quarters through the step, preceded by the step's wait for memory:
+    everything requested before this step began has landed; the next tile's first operands are
+    read behind it;
+  * an accumulating Spec loads C's old values during the first sixteen steps, four blocks a step,
+    and adds them to the blocks' accumulators a step later, between two of a block's MFMAs, so
+    that the epilogue only stores.
 
 Register map (all named in the clobber list of the asm statement):
-  a[0:255]    accumulators, block (tm, tn) at 16 * (4 * tm + tn)
+  a[0:255]    accumulators, block (tm, tn) at 4 * (8 * tm + tn); register i of lane l holds row
+              4 * (l / 16) + i, column l % 16 of the block
   v[0:63]     A staging, set p chunk i at 32 * p + 4 * i; after the loop: values on their way to C
-  v[64:95]    A operands, buffer b block tm at 64 + 16 * b + 4 * tm
-  v[96:127]   B operands, buffer b block tn at 96 + 16 * b + 4 * tn
-  v[128:131]  LDS address of the lane's B operand, per tn, in the slot being read
-  v[132:135]  column sums of B (u8 correction), one per tn; after the loop: 128 * column sum
-  v[136:137]  scratch
-  v[140:171]  old values of two blocks of C
+  v[64:95]    A operands, block row tm at 64 + 4 * tm; after the loop: the column sums' partials
+  v[96:159]   B operands, set b block column tn at 96 + 32 * b + 4 * tn; after the loop: partials
+  v[160:167]  LDS address of the lane's B operand, per tn, in the slot being read
+  v[168:175]  column sums of B (u8 correction), one per tn; after the loop: 128 * column sum
+  v[176:177]  scratch
+  v[180:211]  old values of two times four blocks of C
   s[60:61] A tile pointer   s[62:63] B tile pointer   s64 loop counter   s67 index of the next
   A tile to fetch, s68 of the next B tile   s71 byte offset of tile kt's B slot   s[72:73] C block row pointer
-  s65, s66, s69, s70, s[78:81] scratch
+  s65, s66, s69, s70, s[78:79] scratch
 """
 import os
 import sys
@@ -46,18 +60,21 @@ import sys
 A_STAGE = 32768
 B_SLOT = 32768
 B_BASE = 2 * A_STAGE
-SLAB_BYTES = 8192   # one 32-byte slab of K in a B slot: its k rows x 256 (i8) / 512 (bf16) bytes
-HI_BYTES = 2048     # second transposing read of a slab
-TM, TN = 4, 4       # MFMA blocks per wave
+SLAB_BYTES = 16384  # one 64-byte slab of K in a B slot: its k rows x 256 (i8) / 512 (bf16) bytes
+HI_BYTES = 2048     # second transposing read of an operand: 8 (i8) / 4 (bf16) k rows on
+TM, TN = 8, 8       # MFMA blocks per wave
 MF = TM * TN        # MFMAs per slab
-GAPS = 4 * MF       # MFMAs per k step
-GAP_SLOTS = 6       # instructions placed behind one MFMA before the next is due
+SLABS = 2
+GAPS = SLABS * MF   # MFMAs per k step
+BARRIER_AT = 96     # the step's barrier comes before this MFMA
+GAP_SLOTS = 3       # instructions placed behind one MFMA before the next is due
 C_STEPS = 16        # k steps that carry the loads of C's old values (16 registers a step)
+C_BLOCKS = 4        # blocks of C a step loads
 
 
 def acc(tm, tn):
-    b = 16 * (TN * tm + tn)
-    return f"a[{b}:{b + 15}]"
+    b = 4 * (TN * tm + tn)
+    return f"a[{b}:{b + 3}]"
 
 
 def areg(p, i, w=None):
@@ -65,18 +82,24 @@ def areg(p, i, w=None):
     return f"v[{b}:{b + 3}]" if w is None else f"v{b + w}"
 
 
-def af(buf, tm):
-    b = 64 + 16 * buf + 4 * tm
+def af(tm):
+    b = 64 + 4 * tm
     return f"v[{b}:{b + 3}]"
 
 
 def bf(buf, tn, half=None, w=None):
-    b = 96 + 16 * buf + 4 * tn
+    b = 96 + 32 * buf + 4 * tn
     if w is not None:
         return f"v{b + w}"
     if half is None:
         return f"v[{b}:{b + 3}]"
     return f"v[{b + 2 * half}:{b + 2 * half + 1}]"
+
+
+B_ADDR = 160    # v[160:167]
+COL_SUM = 168   # v[168:175]
+TMP0, TMP1 = 176, 177
+OLD_C = 180     # v[180:211]
 
 
 class Emitter:
@@ -140,41 +163,50 @@ class Item:
 
 
 def gen(kind, wm, accum, opts=None):
-    """kind: 'u8' (A unsigned bytes), 'i8', 'bf16'.  wm: the wave row (which slabs' column sums it adds).
+    """kind: 'u8' (A unsigned bytes), 'i8', 'bf16'.  wm: the wave row (which slab's column sums it adds).
     accum: the Spec accumulates into C (its old contents are read)."""
     opts = opts or {}     # experiment switches; the shipped loops are generated with none
     unsigned = kind == "u8" and not opts.get("no_valu")
     is_float = kind == "bf16"
-    mfma = "v_mfma_f32_32x32x16_bf16" if is_float else "v_mfma_i32_32x32x32_i8"
+    mfma = "v_mfma_f32_16x16x32_bf16" if is_float else "v_mfma_i32_16x16x64_i8"
     tr = "ds_read_b64_tr_b16" if is_float else "ds_read_b64_tr_b8"
     e = Emitter()
     E = e.emit
 
-    def advance(ptr_lo, ptr_hi, idx, step):
+    def advance(ptr_lo, ptr_hi, idx, step, tmp):
         """Next tile: one k step on; past the last tile the pointer stays (that tile is fetched
-        again, into places nobody reads)."""
+        again, into places nobody reads).  In one piece: the carry and the comparison's result
+        live in SCC."""
         E(f"s_add_u32 {idx}, {idx}, 1")
         E(f"s_cmp_lt_u32 {idx}, %[nk]")
-        E(f"s_cselect_b32 s69, {step}, 0")
-        E(f"s_add_u32 {ptr_lo}, {ptr_lo}, s69")
+        E(f"s_cselect_b32 {tmp}, {step}, 0")
+        E(f"s_add_u32 {ptr_lo}, {ptr_lo}, {tmp}")
         E(f"s_addc_u32 {ptr_hi}, {ptr_hi}, 0")
 
     def advance_a():
-        advance("s60", "s61", "s67", "128")
+        advance("s60", "s61", "s67", "128", "s69")
 
     def advance_b():
-        advance("s62", "s63", "s68", "%[bstep]")
+        advance("s62", "s63", "s68", "%[bstep]", "s69")
 
     def load_a(p, i):
         if opts.get("no_stage"):
             return
         e.vm(f"global_load_dwordx4 {areg(p, i)}, %[a_off{i}], s[60:61]", dst=areg(p, i))
 
-    def store_a(p, i, stage):
+    def flip_a(p, i, words):
+        """u8 -> i8 (a - 128) of two of the chunk's four registers."""
         if opts.get("no_stage"):
             return
         e.vm_need(areg(p, i))
-        if unsigned:
+        for w in words:
+            E(f"v_xor_b32 {areg(p, i, w)}, 0x80808080, {areg(p, i, w)}")
+
+    def store_a(p, i, stage, flip=True):
+        if opts.get("no_stage"):
+            return
+        e.vm_need(areg(p, i))
+        if unsigned and flip:
             for w in range(4):
                 E(f"v_xor_b32 {areg(p, i, w)}, 0x80808080, {areg(p, i, w)}")
         e.lds_write(f"ds_write_b128 %[a_wr], {areg(p, i)} offset:{stage * A_STAGE + i * 4096}")
@@ -188,35 +220,22 @@ def gen(kind, wm, accum, opts=None):
             return
         e.vm(f"global_load_lds_dwordx4 %[b_off{j}], s[62:63] offset:{j * 1024 - 4096}")
 
-    def a_read(stage, slab, buf, tm):
+    def a_read(stage, slab, tm):
         if opts.get("no_reads"):
             return lambda: None
-        return lambda: e.lds_read(af(buf, tm), f"ds_read_b128 {af(buf, tm)}, %[a_rd{slab}] offset:{stage * A_STAGE + tm * 4096}")
+        return lambda: e.lds_read(af(tm), f"ds_read_b128 {af(tm)}, %[a_rd{slab}] offset:{stage * A_STAGE + tm * 2048}")
 
     def b_read(slab, buf, tn, half):
         reg = bf(buf, tn, half)
         if opts.get("no_reads"):
             return lambda: None
-        return lambda: e.lds_read(reg, f"{tr} {reg}, v{128 + tn} offset:{slab * SLAB_BYTES + half * HI_BYTES}")
-
-    def reads(stage, slab, buf):
-        """The operand reads of one slab in the order the MFMAs want them, one list per gap."""
-        out = [[a_read(stage, slab, buf, 0)]]
-        for tn in range(TN):
-            out.append([b_read(slab, buf, tn, 0), b_read(slab, buf, tn, 1)])
-        for tm in range(1, TM):
-            out.append([a_read(stage, slab, buf, tm)])
-        return out
+        return lambda: e.lds_read(reg, f"{tr} {reg}, v{B_ADDR + tn} offset:{slab * SLAB_BYTES + half * HI_BYTES}")
 
     def set_b_read_base(slot_off_sgpr):
         for tn in range(TN):
-            E(f"v_add_u32 v{128 + tn}, {slot_off_sgpr}, %[b_rd{tn}]")
+            E(f"v_add_u32 v{B_ADDR + tn}, {slot_off_sgpr}, %[b_rd{tn}]")
 
     # ---- prologue -------------------------------------------------------------------------
-    if opts.get("trace") or opts.get("stamp"):
-        for r in (88, 89, 90):
-            E(f"s_mov_b32 s{r}, 0")
-        E("s_memtime s[92:93]")
     E("s_mov_b64 s[60:61], %[abase]")
     E("s_mov_b64 s[62:63], %[bbase]")
     E("s_mov_b32 s67, 0")
@@ -234,7 +253,7 @@ def gen(kind, wm, accum, opts=None):
             dma_b(j)
         advance_b()
     for tn in range(TN):
-        E(f"v_mov_b32 v{132 + tn}, 0")
+        E(f"v_mov_b32 v{COL_SUM + tn}, 0")
     for i in range(8):
         store_a(0, i, 0)            # waits for A tile 0 only
     for i in range(8):
@@ -246,9 +265,13 @@ def gen(kind, wm, accum, opts=None):
     E("s_barrier")
     E(f"s_mov_b32 s65, {B_BASE}")
     set_b_read_base("s65")
-    for group in reads(0, 0, 0):
-        for r in group:
-            r()
+    # What a step expects to find: slab 0's B operands in set 0 and its A operands but the last,
+    # which every step reads behind its first MFMA.
+    for tn in range(TN):
+        b_read(0, 0, tn, 0)()
+        b_read(0, 0, tn, 1)()
+    for tm in range(TM - 1):
+        a_read(0, 0, tm)()
 
     # ---- one k step ----------------------------------------------------------------------
     def step(cur, zero_first=False, extra=()):
@@ -273,42 +296,55 @@ def gen(kind, wm, accum, opts=None):
             E("s_add_u32 s66, %[dma_base], s70")
             E(f"s_add_u32 s65, s69, {B_BASE}")
             E("s_mov_b32 s71, s69")
+
+        # Operand reads: fixed places.  A's block row tm for the next slab right behind the last of
+        # the eight MFMAs that use the current one (the last block row's lands in the next slab /
+        # step); B's set for the next slab spread over the current one; what comes from the next
+        # tile, behind the barrier.
+        read_at = {}
+
+        def at(g, r):
+            read_at.setdefault(g, []).append(r)
+
+        at(0, a_read(cur, 0, TM - 1))                       # this step's own: slab 0, last block row
+        for tm in range(TM):
+            at(8 * tm + 8, a_read(cur, 1, tm))              # slab 1 (tm = 7: behind slab 1's first MFMA)
+        for tn in range(TN):                                 # slab 1's B operands into set 1
+            at(2 + 6 * tn, b_read(1, 1, tn, 0))
+            at(3 + 6 * tn, b_read(1, 1, tn, 1))
+        for tn in range(TN):                                 # the next tile's slab 0 into set 0
+            at(BARRIER_AT + 3 * tn, b_read(0, 0, tn, 0))
+            at(BARRIER_AT + 1 + 3 * tn, b_read(0, 0, tn, 1))
+        for tm in range(TM - 1):                             # and its A operands as theirs go dead
+            at(max(MF + 8 * tm + 8, BARRIER_AT + 2 + 3 * tm), a_read(cur ^ 1, 0, tm))
+
         # The step's own work.  LDS writes must be out before the barrier.
-        # (Issuing these at different gaps in each of the four waves was measured and changes nothing:
-        # a vector memory or LDS write instruction costs its wave about 13 cycles of MFMA issue
-        # whether or not the other waves issue theirs at the same moment.)
         last_a = None
-        for i, g in enumerate([2, 8, 14, 20, 26, 32, 38, 44]):
-            last_a = add(lambda i=i: (store_a(p, i, cur ^ 1), load_a(p, i)), 6 if unsigned else 2, g, 3 * MF - 1)
+        for i, g in enumerate([1, 12, 23, 34, 45, 56, 67, 78]):
+            if unsigned:   # in pieces that fit a gap
+                last_a = add(lambda i=i: flip_a(p, i, (0, 1)), 2, g, BARRIER_AT - 4, after=last_a)
+                last_a = add(lambda i=i: flip_a(p, i, (2, 3)), 2, g, BARRIER_AT - 3, after=last_a)
+            last_a = add(lambda i=i: (store_a(p, i, cur ^ 1, flip=False), load_a(p, i)), 2, g, BARRIER_AT - 2, after=last_a)
         m0 = add(lambda: set_m0("s66"), 2, 0)
         last_b = m0
-        for j, g in enumerate([5, 11, 17, 23, 29, 35, 41, 46]):
+        for j, g in enumerate([6, 17, 28, 39, 50, 61, 72, 83]):
             last_b = add(lambda j=j: dma_b(j), 1, g, after=last_b)
-        add(advance_a, 5, 45, after=last_a)
-        add(advance_b, 5, 47, after=last_b)
+        add(advance_a, 5, 84, after=last_a)
+        add(advance_b, 5, 88, after=last_b)
         if unsigned:
-            for s in range(4):
-                if s % 2 != wm:
-                    continue
-                for tn in range(TN):
-                    for w in range(4):
-                        # after the MFMA that waited for this operand, before the reads that overwrite it
-                        add(lambda s=s, tn=tn, w=w: (e.need(bf(s & 1, tn, w // 2)),
-                                                      E(f"v_xor_b32 v136, 0x80808080, {bf(s & 1, tn, w=w)}"),
-                                                      E(f"v_sad_u8 v{132 + tn}, v136, 0, v{132 + tn}")),
-                            2, MF * s + tn, min(GAPS - 1, MF * s + MF + tn))
+            s = wm                       # this wave row sums slab wm of every step
+            for tn in range(TN):
+                for w in range(4):
+                    # after the first MFMA that waited for this operand, before the reads that overwrite it
+                    add(lambda s=s, tn=tn, w=w: (e.need(bf(s, tn, w // 2)),
+                                                  E(f"v_xor_b32 v{TMP0}, 0x80808080, {bf(s, tn, w=w)}"),
+                                                  E(f"v_sad_u8 v{COL_SUM + tn}, v{TMP0}, 0, v{COL_SUM + tn}")),
+                        2, MF * s + tn + 1, MF * s + MF - 1 if s == 0 else GAPS - 1)
         for it in extra:
             items.append(it)
-        # operand reads: fixed places
-        read_at = {}
-        for s in range(3):
-            for n, group in enumerate(reads(cur, s + 1, (s + 1) & 1)):
-                read_at[MF * s + n] = group
-        for n, group in enumerate(reads(cur ^ 1, 0, 0)):
-            read_at[MF * 3 + n] = group
         # Place the items in the order given, each into the first gap from its earliest on with room.
         room = [GAP_SLOTS - len(read_at.get(g, [])) for g in range(GAPS)]
-        room[3 * MF - 1] -= 3              # the waits and the barrier
+        room[BARRIER_AT - 1] -= 3              # the waits and the barrier
         placed = [[] for _ in range(GAPS)]
         for it in items:
             first = max(it.earliest, it.after.gap if it.after is not None else 0)
@@ -326,97 +362,85 @@ def gen(kind, wm, accum, opts=None):
 
         def sync():
             # everything requested before this step has landed (B of tile kt + 1, A of tile kt + 2);
-            # this wave's LDS writes are done and the operands of this slab are in
-            if opts.get("trace"):
-                E("s_memtime s[80:81]")
-                E("s_waitcnt lgkmcnt(0)")
-                E("s_memtime s[82:83]")
+            # this wave's LDS writes are done and the operands of the rest of the step are in
             e.vm_wait_index(vm_before_step - 1)
             E("s_waitcnt lgkmcnt(0)")
             e.all_lds_done()
-            if opts.get("trace"):
-                E("s_memtime s[84:85]")
-                E("s_waitcnt lgkmcnt(0)")
             E("s_barrier")
-            if opts.get("trace"):
-                E("s_memtime s[86:87]")
-                E("s_waitcnt lgkmcnt(0)")
-                E("s_sub_u32 s80, s82, s80")
-                E("s_add_u32 s88, s88, s80")
-                E("s_sub_u32 s80, s84, s82")
-                E("s_add_u32 s89, s89, s80")
-                E("s_sub_u32 s80, s86, s84")
-                E("s_add_u32 s90, s90, s80")
             set_b_read_base("s65")
 
         header()
         n = 0
-        for s in range(4):
-            buf = s & 1
-            if s == 3:
-                sync()
+        for s in range(SLABS):
             for tm in range(TM):
                 for tn in range(TN):
-                    e.need(af(buf, tm), bf(buf, tn, 0), bf(buf, tn, 1))
+                    if n == BARRIER_AT:
+                        sync()
+                    e.need(af(tm), bf(s, tn, 0), bf(s, tn, 1))
                     src_c = "0" if (zero_first and s == 0) else acc(tm, tn)
-                    E(f"{mfma} {acc(tm, tn)}, {af(buf, tm)}, {bf(buf, tn)}, {src_c}")
+                    E(f"{mfma} {acc(tm, tn)}, {af(tm)}, {bf(s, tn)}, {src_c}")
                     for r in read_at.get(n, []):
                         r()
                     for it in placed[n]:
                         it.fn()
                     n += 1
 
-    # ---- C: register q = 0..255: block q / 16 (tm = block / 4, tn = block % 4), register r = q % 16,
-    # which holds row 8 * (r / 4) + 4 * (lane / 32) + r % 4 of the block (%[c_row r]) and column lane % 32.
+    # ---- C: register q = 0..255: block q / 4 (tm = block / 8, tn = block % 8), register i = q % 4,
+    # which holds row 4 * (lane / 16) + i of the block (%[c_row i]) and column lane % 16.
     ptr_tm = [None]
 
     def c_ptr(tm):
-        """s[72:73] = the wave's corner of C + tm * 32 rows, if it is not that already."""
+        """s[72:73] = the wave's corner of C + tm * 16 rows, if it is not that already."""
         if ptr_tm[0] == tm:
             return
         ptr_tm[0] = tm
         E("s_mov_b64 s[72:73], %[cbase]")
         if tm:
-            E(f"s_mul_i32 s78, %[ldc32], {tm}")
-            E(f"s_mul_hi_u32 s79, %[ldc32], {tm}")
+            E(f"s_mul_i32 s78, %[ldc16], {tm}")
+            E(f"s_mul_hi_u32 s79, %[ldc16], {tm}")
             E("s_add_u32 s72, s72, s78")
             E("s_addc_u32 s73, s73, s79")
 
     def where(q):
-        block = q // 16
-        return block // TN, block % TN, q % 16
+        block = q // 4
+        return block // TN, block % TN, q % 4
+
+    def old_reg(j, r):
+        return f"v{OLD_C + 16 * (j & 1) + r}"
 
     def old_values(j):
-        """C's old values of block j into bank j % 2 of the temporaries: one step before they are added."""
-        tm, tn = j // TN, j % TN
+        """C's old values of blocks 4 j .. 4 j + 3 into bank j % 2 of the temporaries: one step before
+        they are added."""
         out = []
         for r in range(16):
-            reg = f"v{140 + 16 * (j & 1) + r}"
+            tm, tn, i = where(16 * j + r)
+            reg = old_reg(j, r)
 
-            def ld(r=r, reg=reg):
+            def ld(tm=tm, tn=tn, i=i, reg=reg):
                 c_ptr(tm)
-                e.vm(f"global_load_dword {reg}, %[c_row{r}], s[72:73] offset:{tn * 128}", dst=reg)
-            out.append(Item(ld, 1, 3 * r))
+                e.vm(f"global_load_dword {reg}, %[c_row{i}], s[72:73] offset:{tn * 64}", dst=reg)
+            out.append(Item(ld, 1, 6 * r))
         return out
 
     def add_old_values(j):
-        """The old values of block j join its accumulators between two of the block's MFMAs (which
-        come 16 apart): an MFMA's result may be read four MFMAs after it at the earliest, and a
-        register written for the block's next MFMA wants another instruction in between."""
+        """The old values of blocks 4 j .. 4 j + 3 join their accumulators between a block's MFMA of
+        slab 0 and its MFMA of slab 1 (64 apart): an MFMA's result is read four MFMAs after it at
+        the earliest, and a register written for the block's next MFMA has other instructions
+        between the write and that MFMA."""
         out = []
         for r in range(16):
-            s = r * 3 // 16                      # behind the block's MFMA of slab 0, 1 or 2
-            first, last = MF * s + j + 4, MF * s + j + 14
-            k = r - (16 * s + 2) // 3            # position among the registers of this window
-            reg = f"v{140 + 16 * (j & 1) + r}"
+            q = 16 * j + r
+            tm, tn, _ = where(q)
+            n0 = TN * tm + tn                    # the block's MFMA in slab 0
+            first, last = n0 + 4, n0 + MF - 4
+            reg = old_reg(j, r)
 
-            def rmw(r=r, reg=reg):
-                q = 16 * j + r
+            def rmw(q=q, reg=reg):
                 e.vm_need(reg)
-                E(f"v_accvgpr_read_b32 v137, a{q}")
-                E(f"v_add_f32 v137, v137, {reg}" if is_float else f"v_add_u32 v137, v137, {reg}")
-                E(f"v_accvgpr_write_b32 a{q}, v137")
-            out.append(Item(rmw, 3, min(last, first + 2 * max(0, k)), last))
+                E(f"v_accvgpr_read_b32 v{TMP1}, a{q}")
+                E(f"v_add_f32 v{TMP1}, v{TMP1}, {reg}" if is_float else f"v_add_u32 v{TMP1}, v{TMP1}, {reg}")
+                E(f"v_accvgpr_write_b32 a{q}, v{TMP1}")
+            out.append(Item(rmw, 3, min(last, first + 3 * (r % 4) + 12 * ((r // 4) % 2)), last))
         return out
 
     def loop():
@@ -445,43 +469,41 @@ def gen(kind, wm, accum, opts=None):
     # accumulators before they are read
     E("s_waitcnt vmcnt(0) lgkmcnt(0)")
     E("s_barrier")
-    if opts.get("trace") or opts.get("stamp"):
-        E("s_memtime s[94:95]")
-        E("s_waitcnt lgkmcnt(0)")
-        E("s_sub_u32 s91, s94, s92")
 
     # ---- epilogue -----------------------------------------------------------------------------------
     if unsigned:
-        # Column sums: the partials of the two wave rows and the two lane halves meet in LDS
-        # (each summed K / 4 values of b + 128).
+        # Column sums: the partials of the two wave rows and the four lane groups meet in LDS
+        # (each summed K / 8 values of b + 128).
         for tn in range(TN):
-            E(f"v_subrev_u32 v{132 + tn}, %[k32], v{132 + tn}")
-            e.lds_write(f"ds_write_b32 %[part_wr], v{132 + tn} offset:{tn * 128}")
+            E(f"v_subrev_u32 v{COL_SUM + tn}, %[k16], v{COL_SUM + tn}")
+            e.lds_write(f"ds_write_b32 %[part_wr], v{COL_SUM + tn} offset:{tn * 64}")
         E("s_waitcnt lgkmcnt(0)")
         e.all_lds_done()
         E("s_barrier")
         for tn in range(TN):
-            for w in range(4):
-                reg = f"v{4 * tn + w}"
-                e.lds_read(reg, f"ds_read_b32 {reg}, %[part_rd] offset:{w * 1024 + tn * 128}")
+            for w in range(8):
+                reg = f"v{64 + 8 * tn + w}"
+                e.lds_read(reg, f"ds_read_b32 {reg}, %[part_rd] offset:{w * 1024 + tn * 64}")
         for tn in range(TN):
-            regs = [f"v{4 * tn + w}" for w in range(4)]
+            regs = [f"v{64 + 8 * tn + w}" for w in range(8)]
             e.need(*regs)
-            E(f"v_add3_u32 v{132 + tn}, {regs[0]}, {regs[1]}, {regs[2]}")
-            E(f"v_add_lshl_u32 v{132 + tn}, v{132 + tn}, {regs[3]}, 7")
+            E(f"v_add3_u32 v{COL_SUM + tn}, {regs[0]}, {regs[1]}, {regs[2]}")
+            E(f"v_add3_u32 v{COL_SUM + tn}, v{COL_SUM + tn}, {regs[3]}, {regs[4]}")
+            E(f"v_add3_u32 v{COL_SUM + tn}, v{COL_SUM + tn}, {regs[5]}, {regs[6]}")
+            E(f"v_add_lshl_u32 v{COL_SUM + tn}, v{COL_SUM + tn}, {regs[7]}, 7")
     else:
         E("s_nop 15")
         E("s_nop 15")
     for q in range(0 if not opts.get("no_epilogue") else 256, 256):
-        tm, tn, r = where(q)
+        tm, tn, i = where(q)
         c_ptr(tm)
         if not unsigned:
-            E(f"global_store_dword %[c_row{r}], a{q}, s[72:73] offset:{tn * 128}")
+            E(f"global_store_dword %[c_row{i}], a{q}, s[72:73] offset:{tn * 64}")
         else:
             t = f"v{16 + q % 32}"
             E(f"v_accvgpr_read_b32 {t}, a{q}")
-            E(f"v_add_u32 {t}, {t}, v{132 + tn}")
-            E(f"global_store_dword %[c_row{r}], {t}, s[72:73] offset:{tn * 128}")
+            E(f"v_add_u32 {t}, {t}, v{COL_SUM + tn}")
+            E(f"global_store_dword %[c_row{i}], {t}, s[72:73] offset:{tn * 64}")
     return e.lines
 
 
