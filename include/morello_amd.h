@@ -361,7 +361,7 @@ int mrl_run_compose(const mrl_compose *c, void *const *params, void *stream);
  * kind 0 = int8 (u8/i8 -> i32), 1 = bf16 (-> f32); random_operands 0 = all-zero operands (the
  * datapath barely toggles: close to the datasheet rate), 1 = operands distributed like a
  * benchmark's (the clock settles at the power limit: the ceiling a Matmul kernel can
- * approach on such data).  `iters` x 32 MFMAs per wavefront (20000 runs about 20 ms).
+ * approach on such data).  `iters` x 64 MFMAs of 16 x 16 x 64 bytes per wavefront (20000 runs about 20 ms).
  * Writes operations per second (2 per multiply-add). */
 int mrl_measure_mfma_rate(int kind, int random_operands, uint32_t iters, double *ops_per_second);
 
