@@ -18,12 +18,19 @@
 // merged with SoftmaxDenominatorAndMaxFromParts' formula (morello/src/spec.rs:107-132).
 // S and P never reach HBM: traffic is Q, K, V once and the output once.
 //
-// Both products are formed transposed so that a lane owns one query column: the running
-// max, the denominator and the rescale factor are per-lane scalars, and a row reduction is
-// 32 in-register values plus one cross-lane exchange.  K and V blocks go from global memory
-// straight into LDS (no staging registers; two K tiles and three V tiles per key half), the
-// bank-conflict swizzles applied on the source side of those loads.  The two key halves run one
-// slot apart (matrix work of one beside vector work of the other), two barriers per block.
+// Both products are formed transposed, in 16 x 16 blocks (v_mfma_f32_16x16x32_bf16: on a
+// power-limited board this form sustains 12 % more than the 32 x 32 one, an accumulator being
+// updated once per 32 multiply-adds instead of once per 16), so that a lane owns query columns
+// (two of a wave's 32: l % 16 and 16 + l % 16): the running max, the denominator and the rescale
+// factor are per-lane scalars, and a row reduction is 16 in-register values plus two cross-lane
+// exchanges.  The k index of an MFMA is a contraction index, so which keys a lane group holds in
+// the second product is free as long as both operands agree: lane group g takes keys
+// 4 g .. 4 g + 3 of each of two 16-key blocks, exactly the P values its own accumulators of the
+// first product hold, and V^T's operand is read from LDS with the same choice of rows.  K and V
+// blocks go from global memory straight into LDS (no staging registers; two K tiles and three V
+// tiles per key half), the bank-conflict swizzles applied on the source side of those loads.  The
+// two key halves run one slot apart (matrix work of one beside vector work of the other), two
+// barriers per block.
 #include <algorithm>
 
 #include "kernels.h"
@@ -34,7 +41,7 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
 typedef short v4s __attribute__((ext_vector_type(4)));
-typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef __attribute__((address_space(3))) v4s lds_v4s;
 typedef __attribute__((address_space(3))) void lds_void;
@@ -48,20 +55,25 @@ struct Dims {
   static constexpr int TILE = BKV * ROW;        // one K or V block (16 KiB at D = 128)
   static constexpr int HALF = 5 * TILE;         // per key half: two K tiles, three V tiles
   static constexpr int CHUNKS = ROW / 16;       // 16-byte chunks per row
-  static constexpr int UNITS = ROW / 64;        // 64-byte units per row
+  static constexpr int SLOTS = ROW / 32;        // 32-byte slots per row (16 values: a block's share of a V row)
   static constexpr int ROWS_PER_LINE = ROW >= 256 ? 1 : 256 / ROW;  // rows per 256-byte bank line
   static constexpr int ROWS_PER_LOAD = 1024 / ROW;  // rows one direct-to-LDS instruction fills
-  static constexpr int LDS_BYTES = 2 * HALF > 4 * (D / 2 + 2) * 64 * 4 ? 2 * HALF : 4 * (D / 2 + 2) * 64 * 4;
-  // Rows that one operand read touches at the same chunk index lie 256 bytes apart or closer;
-  // XOR-ing the chunk (K) or the 64-byte unit (V) with the row's bank-line index spreads them.
+  static constexpr int MERGE_ROWS = D / 2 + 4;  // a lane's O, two maxima and two denominators
+  static constexpr int LDS_BYTES = 2 * HALF > 4 * MERGE_ROWS * 64 * 4 ? 2 * HALF : 4 * MERGE_ROWS * 64 * 4;
+  // 16 lanes of a K operand read touch 16 consecutive rows at one chunk index, 32 lanes of a V
+  // operand read 8 rows (4 g .. 4 g + 3 of two lane groups) at one slot index; rows lie 256 bytes
+  // apart or closer.  XOR-ing the chunk (K) or the slot (V) with the row's bank-line index spreads them.
   __device__ static constexpr int k_swizzle(int row) { return (row / ROWS_PER_LINE) & (CHUNKS - 1); }
-  __device__ static constexpr int v_swizzle(int row) { return (row / ROWS_PER_LINE) & (UNITS - 1); }
+  __device__ static constexpr int v_swizzle(int row) { return (row / ROWS_PER_LINE) & (SLOTS - 1); }
 };
+// KT given row-major: a block is D rows (one per d) of 64 keys, 128 bytes; 32 lanes of a K operand
+// read touch rows 8 g .. 8 g + 3 of two lane groups (two rows to a bank line) at one 32-byte slot.
+__device__ constexpr int kt_swizzle(int d) { return ((d >> 1) & 1) | (((d >> 3) & 1) << 1); }
 // Wave priorities of the two kinds of slot: the matrix slot is the longer one and its MFMAs
 // should not queue behind the partner wave's vector instructions (worth ~0.5 % at 16 x 2048 x 128).
 constexpr int PRIO_A = 2, PRIO_B = 0;
 constexpr float LOG2E = 1.44269504088896340736f;
-constexpr float STALE_REFERENCE_SUM = 1.0e12f;  // ~2^40: a lane's sum of 64 exponentials beyond it moves the reference
+constexpr float STALE_REFERENCE_SUM = 1.0e12f;  // ~2^40: a lane's sum of 32 exponentials beyond it moves the reference
 
 // One direct-to-LDS load: 64 lanes x 16 bytes from `base + voff` (voff per lane) to the 1 KiB at
 // LDS address `lds_addr` (wave-uniform), lane l to slot l.  Written as assembly so that the
@@ -87,8 +99,7 @@ __device__ inline v2i read_tr16(const uint8_t *p) {
 // KT_ROWS: KT is given row-major, [b][k][n2] with n2 fastest (the reference's default layout for
 // the Compose's third parameter) instead of k-fastest.  A block of 64 keys is then D rows of 128
 // bytes in LDS (one row per d), and the K operand comes out of it through the same transposing
-// read that serves V; the MFMA's k index runs over d in the order that read delivers (4 + 4
-// values per lane half), so Q's operand is loaded in that order too.  n2 must be a multiple of 8.
+// read that serves V.  n2 must be a multiple of 8.
 // QG: query groups of 32 per workgroup (4 or 2): the Compose's tile_out over its rows.  A workgroup
 // is 2 * QG waves; with 2 groups the four waves share a compute unit's LDS and matrix cores between
 // them alone, which pays when 128-query blocks would leave half of the compute units without work
@@ -106,12 +117,15 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
   } const p = {q, kt, v, out, b, m, n2, n_out, key_splits, partials};
   typedef Dims<D> DD;
   constexpr int ROW = DD::ROW, TILE = DD::TILE, HALF = DD::HALF;
+  constexpr int NC = D / 32;   // 32-wide chunks of d: k steps of S = K.Q
+  constexpr int NDB = D / 16;  // 16-row blocks of O^T
+  constexpr int NKB = BKV / 16, NKC = BKV / 32;  // 16-key blocks of S^T, 32-key k steps of O += V.P
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int qg = wave % QG, half = wave / QG;  // query group, key half
   constexpr int BQ = 32 * QG;
-  const int lq = lane & 31, lg = lane >> 5;
+  const int lr = lane & 15, lgp = lane >> 4;   // position within a block's 16 rows / columns, lane group
   // Workgroups go to the 8 XCDs round-robin.  All query blocks of a batch entry share its K
   // and V, so a batch entry's blocks are kept on one XCD (one L2) whenever the counts allow:
   // XCD x takes the x-th run of consecutive (entry, block) pairs.
@@ -138,26 +152,23 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
   const int nblocks = half ? my_blocks - steps : steps;
   const uint32_t head_bytes = p.n2 * ROW;  // K or V of one batch entry
 
-  const int q_row = RAGGED ? min(q0 + lq, int(p.m) - 1) : q0 + lq;
-  const uint8_t *Q = (const uint8_t *)p.q + (head * p.m + q_row) * int64_t(ROW);
   const uint8_t *K = (const uint8_t *)p.kt + head * p.n2 * ROW;
   const uint8_t *V = (const uint8_t *)p.v + head * p.n2 * ROW;
   uint8_t *my_lds = lds + half * HALF;
 
-  // Q^T operand: lane (query lq, half lg) holds d = 16*step + 8*lg .. +7.
-  v4i qf[D / 16];
+  // Q^T operands: block column qb (queries 16 qb + l % 16 of the wave's 32), chunk c of d:
+  // lane (l % 16, l / 16) holds d = 32 c + 8 (l / 16) .. + 7.
+  v4i qf[2][NC];
 #pragma unroll
-  for (int s = 0; s < D / 16; s++) {
-    if constexpr (KT_ROWS) {
-      const v2i lo = *(const v2i *)(Q + s * 32 + lg * 8), hi = *(const v2i *)(Q + s * 32 + 16 + lg * 8);
-      qf[s] = v4i{lo[0], lo[1], hi[0], hi[1]};  // d = 16s + 4lg + 0..3, then 16s + 8 + 4lg + 0..3
-    } else {
-      qf[s] = *(const v4i *)(Q + s * 32 + lg * 16);
-    }
+  for (int qb = 0; qb < 2; qb++) {
+    const int q_row = RAGGED ? min(q0 + 16 * qb + lr, int(p.m) - 1) : q0 + 16 * qb + lr;
+    const uint8_t *Q = (const uint8_t *)p.q + (head * p.m + q_row) * int64_t(ROW);
+#pragma unroll
+    for (int c = 0; c < NC; c++) qf[qb][c] = *(const v4i *)(Q + c * 64 + lgp * 16);
   }
 
   // Block staging.  One direct-to-LDS instruction fills 1 KiB (4 rows at D = 128); lane l lands
-  // in 16-byte slot l.  K rows are XOR-swizzled by chunk, V rows by 64-byte unit; each lane
+  // in 16-byte slot l.  K rows are XOR-swizzled by chunk, V rows by 32-byte slot; each lane
   // fetches the global chunk that belongs in its slot.  The 4 waves of a key half share its
   // instructions: PER_WAVE for K and as many for V per block and wave.
   constexpr int PER_WAVE = TILE / 1024 / QG;
@@ -168,13 +179,13 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
   for (int i = 0; i < PER_WAVE; i++) {
     const int q = qg * PER_WAVE + i, row = q * DD::ROWS_PER_LOAD + ld_row;
     if constexpr (KT_ROWS) {
-      // 8 rows (d) of 128 bytes per instruction; 64-byte units swizzled like a V tile of D = 64.
+      // 8 rows (d) of 128 bytes per instruction
       const int krow = q * 8 + (lane >> 3), kpc = lane & 7;
-      k_src[i] = krow * (p.n2 * 2) + ((((kpc >> 2) ^ Dims<64>::v_swizzle(krow)) << 6) | ((kpc & 3) << 4));
+      k_src[i] = krow * (p.n2 * 2) + ((((kpc >> 1) ^ kt_swizzle(krow)) << 5) | ((kpc & 1) << 4));
     } else {
       k_src[i] = row * ROW + ((ld_pc ^ DD::k_swizzle(row)) << 4);
     }
-    v_src[i] = row * ROW + ((((ld_pc >> 2) ^ DD::v_swizzle(row)) << 6) | ((ld_pc & 3) << 4));
+    v_src[i] = row * ROW + ((((ld_pc >> 1) ^ DD::v_swizzle(row)) << 5) | ((ld_pc & 1) << 4));
   }
   // Fetch of this lane's chunk i of K (V) block kb into the KiB at LDS address `dst`.  The block's
   // offset is wave-uniform and goes into the scalar base; only the ragged form, which clamps
@@ -189,16 +200,15 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
     if constexpr (RAGGED) dma16(V, min(block + v_src[i], head_bytes - 16), dst);
     else dma16(V + block, v_src[i], dst);
   };
-  v16f o[D / 32];
+  // O^T: block row db (d = 16 db + 4 (l / 16) + i in register i), block column qb.
+  v4f o[NDB][2];
 #pragma unroll
-  for (int t = 0; t < D / 32; t++)
+  for (int db = 0; db < NDB; db++)
 #pragma unroll
-    for (int r = 0; r < 16; r++) o[t][r] = 0.0f;
-  float m_run = -3.0e38f, l_run = 0.0f;  // l_run: this lane's share of the denominator
-
-  // Fragment addressing that does not depend on the block.
-  const int v_rl = (lane & 15) >> 2;                                   // row within a 4-row read
-  const int v_within = 32 * ((lane >> 4) & 1) + 8 * (lane & 3);        // bytes within a 64-B unit
+    for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) o[db][qb][r] = 0.0f;
+  float m_run[2] = {-3.0e38f, -3.0e38f}, l_run[2] = {0.0f, 0.0f};  // l_run: this lane's share of the denominators
 
   // LDS of a key half: K tiles 0 and 1, then V tiles 0, 1 and 2.  K block kb goes to K tile
   // kb & 1, V block kb to V tile kb % 3.  A block index past the half's last block fetches the
@@ -230,21 +240,26 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
   //   exponentials (the softmax slot is the shorter one; in the matrix slot they cost more), and
   //   ends by waiting for everything but its own fetches: K(j + 1) and V(j), which A_(j+1) reads,
   //   have then landed.
-  v16f s[BKV / 32];
-  v8bf pb[BKV / 16];
+  // S^T: block row kb (key 16 kb + 4 (l / 16) + i in register i), block column qb.
+  v4f s[NKB][2];
+  // P^T operands of the second product: k step kc covers key blocks 2 kc and 2 kc + 1; lane group g
+  // holds keys 4 g .. 4 g + 3 of each, its own eight values of S^T.
+  v8bf pb[NKC][2];
   // Lane-dependent, block-independent parts of the operand addresses (the swizzles depend on the
   // lane only: the row offsets that vary per read are multiples of the swizzle periods).
-  uint32_t v_lane[D / 32], k_lane[KT_ROWS ? BKV / 32 : D / 16];
+  uint32_t v_lane[NDB], k_lane[KT_ROWS ? NKB : NC];
   {
-    const int key = 4 * lg + v_rl;
+    const int piece = (lr & 3) * 8;     // a lane's 8 bytes of a transposing read's 32
+    const int vrow = 4 * lgp + (lr >> 2);
 #pragma unroll
-    for (int t = 0; t < D / 32; t++) v_lane[t] = key * ROW + ((t ^ DD::v_swizzle(key)) << 6) + v_within;
+    for (int db = 0; db < NDB; db++) v_lane[db] = vrow * ROW + ((db ^ DD::v_swizzle(vrow)) << 5) + piece;
     if constexpr (KT_ROWS) {
+      const int drow = 8 * lgp + (lr >> 2);
 #pragma unroll
-      for (int kt = 0; kt < BKV / 32; kt++) k_lane[kt] = key * (BKV * 2) + ((kt ^ Dims<64>::v_swizzle(key)) << 6) + v_within;
+      for (int kb = 0; kb < NKB; kb++) k_lane[kb] = drow * (BKV * 2) + ((kb ^ kt_swizzle(drow)) << 5) + piece;
     } else {
 #pragma unroll
-      for (int st = 0; st < D / 16; st++) k_lane[st] = lq * ROW + (((2 * st + lg) ^ DD::k_swizzle(lq)) << 4);
+      for (int c = 0; c < NC; c++) k_lane[c] = lr * ROW + (((4 * c + lgp) ^ DD::k_swizzle(lr)) << 4);
     }
   }
   // s_waitcnt vmcnt(n) (six bits: the low four and two at the top), the other counters left alone.
@@ -267,108 +282,97 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
     __builtin_amdgcn_s_waitcnt(WAIT_BUT_TWO);  // K(0)
     __syncthreads();
   }
-  constexpr int NU = BKV / 16, NQ = D / 32;
-  constexpr int VR = 2 * (D / 32), KR = (KT_ROWS ? 4 : 2) * (BKV / 32), PM = D / 32, QM = 2 * (BKV / 32);
-  v4i kf[2][BKV / 32][2];
-  v4i vf[3][D / 32];
-  // K operands of batch q (two d-steps, both key tiles) of the K tile at `lk`.
-  auto read_k = [&](const uint8_t *lk, int q, int buf) {
-#pragma unroll
-    for (int c = 0; c < 2; c++)
-#pragma unroll
-      for (int kt = 0; kt < BKV / 32; kt++) {
-        const int st = 2 * q + c;
-        if constexpr (KT_ROWS) {
-          const uint8_t *a = lk + k_lane[kt] + st * 16 * (BKV * 2);
-          const v2i lo = read_tr16(a), hi = read_tr16(a + 8 * (BKV * 2));
-          kf[buf][kt][c] = v4i{lo[0], lo[1], hi[0], hi[1]};
-        } else {
-          kf[buf][kt][c] = *(const v4i *)(lk + k_lane[st] + kt * 32 * ROW);
-        }
-      }
-  };
-  auto read_v = [&](const uint8_t *lv, int u, int buf) {
-#pragma unroll
-    for (int t = 0; t < D / 32; t++) {
-      const uint8_t *a = lv + v_lane[t] + u * 16 * ROW;
-      const v2i lo = read_tr16(a), hi = read_tr16(a + 8 * ROW);
-      vf[buf][t] = v4i{lo[0], lo[1], hi[0], hi[1]};
+  // K operand of key block kb, chunk c of d: lane (key 16 kb + l % 16, group g) holds d = 32 c + 8 g .. + 7.
+  auto read_k = [&](const uint8_t *lk, int kb, int c) {
+    if constexpr (KT_ROWS) {
+      const uint8_t *a = lk + k_lane[kb] + c * 32 * (BKV * 2);
+      const v2i lo = read_tr16(a), hi = read_tr16(a + 4 * (BKV * 2));
+      return v4i{lo[0], lo[1], hi[0], hi[1]};
+    } else {
+      return *(const v4i *)(lk + k_lane[c] + kb * 16 * ROW);
     }
   };
-  auto pv_step = [&](int u, int buf) {
-#pragma unroll
-    for (int t = 0; t < D / 32; t++)
-      o[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, vf[buf][t]), pb[u], o[t], 0, 0, 0);
+  // V^T operand of block row db, k step kc: lane (d 16 db + l % 16, group g) holds keys 4 g .. + 3 of
+  // key block 2 kc, then of key block 2 kc + 1.
+  auto read_v = [&](const uint8_t *lv, int db, int kc) {
+    const uint8_t *a = lv + v_lane[db] + kc * 32 * ROW;
+    const v2i lo = read_tr16(a), hi = read_tr16(a + 16 * ROW);
+    return v4i{lo[0], lo[1], hi[0], hi[1]};
   };
-  auto qk_step = [&](int q, int buf) {
+  auto mfma = [](v4i a, auto bop, v4f c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, bop), c, 0, 0, 0);
+  };
+  // A matrix slot is a sequence of steps of two MFMAs on one operand read from LDS (a V operand
+  // against the two block columns of P, or a K operand against those of Q); the operand of step
+  // t + AHEAD is read behind the MFMAs of step t.  Two steps ahead measured best (16 x 2048 x 128:
+  // 33.8 us; 1: 34.1, 3: 33.9, 4: 34.5, 8: 35.6, 12: 36.1, none: 45.4): the reads ahead of a
+  // slot's first MFMA are time the matrix core of that SIMD stands still.
+  constexpr int PV_STEPS = NKC * NDB, QK_STEPS = NC * NKB, AHEAD = 2, RING = AHEAD + 1;
+  constexpr int K_READS = KT_ROWS ? 2 : 1;   // LDS instructions per K operand (V: always 2)
+  v4i ring[RING];
+  // steps [first, last) of the sequence PV(0 .. PV_STEPS) then QK(0 .. QK_STEPS)
+  auto run_steps = [&](auto first_c, auto last_c, const uint8_t *lv, const uint8_t *lk) {
+    constexpr int FIRST = decltype(first_c)::value, LAST = decltype(last_c)::value;
+    auto fetch = [&](int t) {
+      if (t < PV_STEPS) ring[t % RING] = read_v(lv, t % NDB, t / NDB);
+      else ring[t % RING] = read_k(lk, (t - PV_STEPS) % NKB, (t - PV_STEPS) / NKB);
+    };
+    auto reads_of = [](int t) { return t < PV_STEPS ? 2 : K_READS; };
 #pragma unroll
-    for (int c = 0; c < 2; c++)
+    for (int t = FIRST; t < LAST && t < FIRST + AHEAD; t++) fetch(t);
 #pragma unroll
-      for (int kt = 0; kt < BKV / 32; kt++)
-        s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, kf[buf][kt][c]),
-                                                        __builtin_bit_cast(v8bf, qf[2 * q + c]), s[kt], 0, 0, 0);
+    for (int t = FIRST; t < LAST; t++) {
+      if (t + AHEAD < LAST) fetch(t + AHEAD);
+      const v4i a = ring[t % RING];
+      if (t < PV_STEPS) {
+        const int db = t % NDB, kc = t / NDB;
+        o[db][0] = mfma(a, pb[kc][0], o[db][0]);
+        o[db][1] = mfma(a, pb[kc][1], o[db][1]);
+      } else {
+        const int kb = (t - PV_STEPS) % NKB, c = (t - PV_STEPS) / NKB;
+        s[kb][0] = mfma(a, qf[0][c], s[kb][0]);
+        s[kb][1] = mfma(a, qf[1][c], s[kb][1]);
+      }
+    }
+    // The order wanted of the scheduler: the first AHEAD operands' reads, then per step the reads
+    // of the operand AHEAD steps on and the step's two MFMAs.
+    auto reads_group = [&](int t) {   // the builtin wants literal sizes
+      if (reads_of(t) == 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      else __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    };
+#pragma unroll
+    for (int t = FIRST; t < LAST && t < FIRST + AHEAD; t++) reads_group(t);
+#pragma unroll
+    for (int t = FIRST; t < LAST; t++) {
+      if (t + AHEAD < LAST) reads_group(t + AHEAD);
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+    }
   };
   auto zero_s = [&]() {
 #pragma unroll
-    for (int kt = 0; kt < BKV / 32; kt++)
+    for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) s[kt][r] = 0.0f;
+      for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) s[kb][qb][r] = 0.0f;
   };
+  using std::integral_constant;
   // Slot A of the first block: S = K.Q only.
   auto slot_a_first = [&]() {
-    const uint8_t *lk = my_lds;
     zero_s();
-    read_k(lk, 0, 0);
-#pragma unroll
-    for (int q = 0; q < NQ; q++) {
-      if (q + 1 < NQ) read_k(lk, q + 1, (q + 1) & 1);
-      qk_step(q, q & 1);
-    }
+    run_steps(integral_constant<int, PV_STEPS>{}, integral_constant<int, PV_STEPS + QK_STEPS>{}, my_lds, my_lds);
   };
   // Slot A of block j, 1 <= j < nblocks: O += V.P of block j - 1, then S = K.Q of block j.
   auto slot_a = [&](int j, const uint8_t *lv) {
     __builtin_amdgcn_s_setprio(PRIO_A);
-    const uint8_t *lk = my_lds + (j & 1) * TILE;
     zero_s();
-    // V operands three key steps deep, K operands two batches deep; the reads of a step go out
-    // behind the MFMAs of the step two (one) before it.
-    read_v(lv, 0, 0);
-    read_v(lv, 1, 1);
-    read_k(lk, 0, 0);
-#pragma unroll
-    for (int u = 0; u < NU; u++) {
-      if (u + 2 < NU) read_v(lv, u + 2, (u + 2) % 3);
-      if (u == NU - 1 && NQ > 1) read_k(lk, 1, 1);
-      pv_step(u, u % 3);
-    }
-#pragma unroll
-    for (int q = 0; q < NQ; q++) {
-      qk_step(q, q & 1);
-      if (q + 2 < NQ) read_k(lk, q + 2, q & 1);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x100, 2 * VR + KR, 0);
-#pragma unroll
-    for (int u = 0; u < NU; u++) {
-      if (u + 2 < NU) __builtin_amdgcn_sched_group_barrier(0x100, VR, 0);
-      if (u == NU - 1 && NQ > 1) __builtin_amdgcn_sched_group_barrier(0x100, KR, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, PM, 0);
-    }
-#pragma unroll
-    for (int q = 0; q < NQ; q++) {
-      __builtin_amdgcn_sched_group_barrier(0x008, QM, 0);
-      if (q + 2 < NQ) __builtin_amdgcn_sched_group_barrier(0x100, KR, 0);
-    }
+    run_steps(integral_constant<int, 0>{}, integral_constant<int, PV_STEPS + QK_STEPS>{}, lv, my_lds + (j & 1) * TILE);
   };
   // Slot A after the last block: O += V.P of block nblocks - 1.
   auto slot_a_last = [&](const uint8_t *lv) {
-    read_v(lv, 0, 0);
-#pragma unroll
-    for (int u = 0; u < NU; u++) {
-      if (u + 1 < NU) read_v(lv, u + 1, (u + 1) % 3);
-      pv_step(u, u % 3);
-    }
+    run_steps(integral_constant<int, 0>{}, integral_constant<int, PV_STEPS>{}, lv, my_lds);
   };
-  // Slot B of block j: the online softmax of S into P (bf16), the running max and denominator.
+  // Slot B of block j: the online softmax of S into P (bf16), the running maxima and denominators.
   auto slot_b = [&](int j) {
     __builtin_amdgcn_s_setprio(PRIO_B);
     if (RAGGED) {
@@ -376,10 +380,12 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
       const int valid = int(p.n2) - (first_block + j) * BKV;
       if (valid < BKV) {
 #pragma unroll
-        for (int kt = 0; kt < BKV / 32; kt++)
+        for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
-          for (int r = 0; r < 16; r++)
-            if (kt * 32 + 8 * (r / 4) + 4 * lg + r % 4 >= valid) s[kt][r] = -__builtin_inff();
+          for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+              if (kb * 16 + 4 * lgp + r >= valid) s[kb][qb][r] = -__builtin_inff();
       }
     }
     // The running reference m_run (exponentials are taken as exp(x - m_run); the final division
@@ -387,59 +393,69 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
     // the first block's maxima and then left alone: a block's maximum is only looked for when its
     // sum of exponentials shows that some score outgrew the reference by more than 2^40, far
     // inside f32 and bf16 range.  That block's exponentials are then redone against the moved
-    // reference, and the running sums and the 64 accumulators rescaled.  This takes the maximum
-    // (a quarter of the softmax's instructions and a cross-lane exchange) out of almost every block.
+    // reference, and the running sums and the accumulators rescaled.  This takes the maximum
+    // (a quarter of the softmax's instructions and two cross-lane exchanges) out of almost every block.
     auto move_reference = [&]() {
-      float mx = s[0][0];
 #pragma unroll
-      for (int kt = 0; kt < BKV / 32; kt++)
+      for (int qb = 0; qb < 2; qb++) {
+        float mx = s[0][qb][0];
 #pragma unroll
-        for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[kt][r]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32));
-      const float m_new = fmaxf(m_run, mx);
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * LOG2E);
-      m_run = m_new;
-      l_run *= alpha;
+        for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
-      for (int t = 0; t < D / 32; t++)
+          for (int r = 0; r < 4; r++) mx = fmaxf(mx, s[kb][qb][r]);
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run[qb], mx);
+        const float alpha = __builtin_amdgcn_exp2f((m_run[qb] - m_new) * LOG2E);
+        m_run[qb] = m_new;
+        l_run[qb] *= alpha;
 #pragma unroll
-        for (int r = 0; r < 16; r++) o[t][r] *= alpha;
+        for (int db = 0; db < NDB; db++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) o[db][qb][r] *= alpha;
+      }
     };
     if (j == 0) move_reference();
     // In base 2: exp(x - m) = 2^(x*log2e - m*log2e).
-    const float neg_m2 = -m_run * LOG2E;
-    float psum = 0.0f;
+    const float neg_m2[2] = {-m_run[0] * LOG2E, -m_run[1] * LOG2E};
+    float psum[2] = {0.0f, 0.0f};
     // The fetches of V(j + 1) and K(j + 2) go out one instruction at a time between the exponentials.
     const int ksrc = min(j + 2, nblocks - 1), vsrc = min(j + 1, nblocks - 1);
     const uint32_t kdst = lds_address(my_lds + (j & 1) * TILE), vdst = lds_address(my_lds + (2 + (j + 1) % 3) * TILE);
 #pragma unroll
-    for (int kt = 0; kt < BKV / 32; kt++)
+    for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][r], LOG2E, neg_m2));
-        psum += e;
-        pb[kt * 2 + r / 8][r % 8] = (__bf16)e;
-        constexpr int EVERY = 16 / PER_WAVE;
-        if ((kt * 16 + r) % EVERY == EVERY - 1) {
-          const int i = (kt * 16 + r) / EVERY;
-          if (i < PER_WAVE) fetch_v(vsrc, i, vdst + (qg * PER_WAVE + i) * 1024);
-          else fetch_k(ksrc, i - PER_WAVE, kdst + (qg * PER_WAVE + i - PER_WAVE) * 1024);
+      for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][qb][r], LOG2E, neg_m2[qb]));
+          psum[qb] += e;
+          pb[kb / 2][qb][(kb % 2) * 4 + r] = (__bf16)e;
+          constexpr int EVERY = 16 / PER_WAVE;
+          const int n = (kb * 2 + qb) * 4 + r;   // 0 .. 31
+          if (n % EVERY == EVERY - 1) {
+            const int i = n / EVERY;
+            if (i < PER_WAVE) fetch_v(vsrc, i, vdst + (qg * PER_WAVE + i) * 1024);
+            else fetch_k(ksrc, i - PER_WAVE, kdst + (qg * PER_WAVE + i - PER_WAVE) * 1024);
+          }
         }
-      }
-    if (j > 0 && __any(!(psum < STALE_REFERENCE_SUM))) {
+    if (j > 0 && __any(!(psum[0] < STALE_REFERENCE_SUM) || !(psum[1] < STALE_REFERENCE_SUM))) {
       move_reference();
-      const float neg2 = -m_run * LOG2E;
-      psum = 0.0f;
 #pragma unroll
-      for (int kt = 0; kt < BKV / 32; kt++)
+      for (int qb = 0; qb < 2; qb++) {
+        const float neg2 = -m_run[qb] * LOG2E;
+        psum[qb] = 0.0f;
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][r], LOG2E, neg2));
-          psum += e;
-          pb[kt * 2 + r / 8][r % 8] = (__bf16)e;
-        }
+        for (int kb = 0; kb < NKB; kb++)
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][qb][r], LOG2E, neg2));
+            psum[qb] += e;
+            pb[kb / 2][qb][(kb % 2) * 4 + r] = (__bf16)e;
+          }
+      }
     }
-    l_run += psum;
+    l_run[0] += psum[0], l_run[1] += psum[1];
     __builtin_amdgcn_s_waitcnt(WAIT_BUT_TWO);
   };
 
@@ -465,66 +481,77 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
 
   // Merge the two key halves: (m, d, O) of half 1 goes through LDS to the wave of half 0
   // that owns the same queries.  Layout [value][lane] keeps lanes on distinct banks.
-  float l_tot = l_run + __shfl_xor(l_run, 32);
+  float l_tot[2];
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++) {
+    const float t = l_run[qb] + __shfl_xor(l_run[qb], 16);
+    l_tot[qb] = t + __shfl_xor(t, 32);
+  }
   __syncthreads();  // all K/V reads are done: the staging area is free
-  float *mbuf = (float *)lds + qg * ((D / 2 + 2) * 64);
+  constexpr int MR = DD::MERGE_ROWS;
+  float *mbuf = (float *)lds + qg * (MR * 64);
   if (half == 1) {
 #pragma unroll
-    for (int t = 0; t < D / 32; t++)
+    for (int db = 0; db < NDB; db++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) mbuf[(t * 16 + r) * 64 + lane] = o[t][r];
-    mbuf[(D / 2) * 64 + lane] = m_run;
-    mbuf[(D / 2 + 1) * 64 + lane] = l_tot;
+      for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) mbuf[((db * 2 + qb) * 4 + r) * 64 + lane] = o[db][qb][r];
+#pragma unroll
+    for (int qb = 0; qb < 2; qb++) {
+      mbuf[(D / 2 + qb) * 64 + lane] = m_run[qb];
+      mbuf[(D / 2 + 2 + qb) * 64 + lane] = l_tot[qb];
+    }
   }
   __syncthreads();
   if (half == 0) {
-    const float m1 = mbuf[(D / 2) * 64 + lane], l1 = mbuf[(D / 2 + 1) * 64 + lane];
-    const float m = fmaxf(m_run, m1);
-    const float a0 = __builtin_amdgcn_exp2f((m_run - m) * LOG2E), a1 = __builtin_amdgcn_exp2f((m1 - m) * LOG2E);
-    if (p.key_splits > 1) {
-      // Partial triple of this split, relative to m: rows of D + 4 floats (O, then m, then the
-      // denominator), [query][split].
-      if (q0 + lq < int(p.m)) {
-        float *part = p.partials + ((head * p.m + q0 + lq) * int64_t(p.key_splits) + blockIdx.y) * (D + 4);
 #pragma unroll
-        for (int t = 0; t < D / 32; t++)
+    for (int qb = 0; qb < 2; qb++) {
+      const float m1 = mbuf[(D / 2 + qb) * 64 + lane], l1 = mbuf[(D / 2 + 2 + qb) * 64 + lane];
+      const float mm = fmaxf(m_run[qb], m1);
+      const float a0 = __builtin_amdgcn_exp2f((m_run[qb] - mm) * LOG2E), a1 = __builtin_amdgcn_exp2f((m1 - mm) * LOG2E);
+      const int row = q0 + 16 * qb + lr;
+      if (p.key_splits > 1) {
+        // Partial triple of this split, relative to mm: rows of D + 4 floats (O, then the maximum,
+        // then the denominator), [query][split].
+        if (row < int(p.m)) {
+          float *part = p.partials + ((head * p.m + row) * int64_t(p.key_splits) + blockIdx.y) * (D + 4);
 #pragma unroll
-          for (int a = 0; a < 4; a++) {
+          for (int db = 0; db < NDB; db++) {
             float4 v;
-            v.x = o[t][4 * a + 0] * a0 + mbuf[(t * 16 + 4 * a + 0) * 64 + lane] * a1;
-            v.y = o[t][4 * a + 1] * a0 + mbuf[(t * 16 + 4 * a + 1) * 64 + lane] * a1;
-            v.z = o[t][4 * a + 2] * a0 + mbuf[(t * 16 + 4 * a + 2) * 64 + lane] * a1;
-            v.w = o[t][4 * a + 3] * a0 + mbuf[(t * 16 + 4 * a + 3) * 64 + lane] * a1;
-            *(float4 *)(part + t * 32 + 8 * a + 4 * lg) = v;
+            v.x = o[db][qb][0] * a0 + mbuf[((db * 2 + qb) * 4 + 0) * 64 + lane] * a1;
+            v.y = o[db][qb][1] * a0 + mbuf[((db * 2 + qb) * 4 + 1) * 64 + lane] * a1;
+            v.z = o[db][qb][2] * a0 + mbuf[((db * 2 + qb) * 4 + 2) * 64 + lane] * a1;
+            v.w = o[db][qb][3] * a0 + mbuf[((db * 2 + qb) * 4 + 3) * 64 + lane] * a1;
+            *(float4 *)(part + db * 16 + 4 * lgp) = v;
           }
-        if (lg == 0) part[D] = m, part[D + 1] = l_tot * a0 + l1 * a1;
-      }
-      return;
-    }
-    const float inv = 1.0f / (l_tot * a0 + l1 * a1);
-    const float w0 = a0 * inv, w1 = a1 * inv;
-    float *out = p.out + (head * p.m + q0 + lq) * int64_t(p.n_out);
-    const bool whole_rows = p.n_out == D;  // else: padded head dim, columns past n_out are dropped
-    if (!RAGGED || q0 + lq < int(p.m))
-#pragma unroll
-    for (int t = 0; t < D / 32; t++)
-#pragma unroll
-      for (int a = 0; a < 4; a++) {
-        float4 v;
-        v.x = o[t][4 * a + 0] * w0 + mbuf[(t * 16 + 4 * a + 0) * 64 + lane] * w1;
-        v.y = o[t][4 * a + 1] * w0 + mbuf[(t * 16 + 4 * a + 1) * 64 + lane] * w1;
-        v.z = o[t][4 * a + 2] * w0 + mbuf[(t * 16 + 4 * a + 2) * 64 + lane] * w1;
-        v.w = o[t][4 * a + 3] * w0 + mbuf[(t * 16 + 4 * a + 3) * 64 + lane] * w1;
-        const int col = t * 32 + 8 * a + 4 * lg;
-        if (whole_rows) {
-          *(float4 *)(out + col) = v;
-        } else {
-          if (col + 0 < int(p.n_out)) out[col + 0] = v.x;
-          if (col + 1 < int(p.n_out)) out[col + 1] = v.y;
-          if (col + 2 < int(p.n_out)) out[col + 2] = v.z;
-          if (col + 3 < int(p.n_out)) out[col + 3] = v.w;
+          if (lgp == 0) part[D] = mm, part[D + 1] = l_tot[qb] * a0 + l1 * a1;
         }
+        continue;
       }
+      const float inv = 1.0f / (l_tot[qb] * a0 + l1 * a1);
+      const float w0 = a0 * inv, w1 = a1 * inv;
+      float *orow = p.out + (head * p.m + row) * int64_t(p.n_out);
+      const bool whole_rows = p.n_out == D;  // else: padded head dim, columns past n_out are dropped
+      if (!RAGGED || row < int(p.m))
+#pragma unroll
+        for (int db = 0; db < NDB; db++) {
+          float4 v;
+          v.x = o[db][qb][0] * w0 + mbuf[((db * 2 + qb) * 4 + 0) * 64 + lane] * w1;
+          v.y = o[db][qb][1] * w0 + mbuf[((db * 2 + qb) * 4 + 1) * 64 + lane] * w1;
+          v.z = o[db][qb][2] * w0 + mbuf[((db * 2 + qb) * 4 + 2) * 64 + lane] * w1;
+          v.w = o[db][qb][3] * w0 + mbuf[((db * 2 + qb) * 4 + 3) * 64 + lane] * w1;
+          const int col = db * 16 + 4 * lgp;
+          if (whole_rows) {
+            *(float4 *)(orow + col) = v;
+          } else {
+            if (col + 0 < int(p.n_out)) orow[col + 0] = v.x;
+            if (col + 1 < int(p.n_out)) orow[col + 1] = v.y;
+            if (col + 2 < int(p.n_out)) orow[col + 2] = v.z;
+            if (col + 3 < int(p.n_out)) orow[col + 3] = v.w;
+          }
+        }
+    }
   }
 }
 
