@@ -73,7 +73,7 @@ __device__ constexpr int kt_swizzle(int d) { return ((d >> 1) & 1) | (((d >> 3) 
 // should not queue behind the partner wave's vector instructions (worth ~0.5 % at 16 x 2048 x 128).
 constexpr int PRIO_A = 2, PRIO_B = 0;
 constexpr float LOG2E = 1.44269504088896340736f;
-constexpr float STALE_REFERENCE_SUM = 1.0e12f;  // ~2^40: a lane's sum of 32 exponentials beyond it moves the reference
+constexpr float STALE_REFERENCE = 1.0e12f;  // ~2^40: an exponential beyond it moves the reference
 
 // One direct-to-LDS load: 64 lanes x 16 bytes from `base + voff` (voff per lane) to the 1 KiB at
 // LDS address `lds_addr` (wave-uniform), lane l to slot l.  Written as assembly so that the
@@ -208,7 +208,16 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
     for (int qb = 0; qb < 2; qb++)
 #pragma unroll
       for (int r = 0; r < 4; r++) o[db][qb][r] = 0.0f;
-  float m_run[2] = {-3.0e38f, -3.0e38f}, l_run[2] = {0.0f, 0.0f};  // l_run: this lane's share of the denominators
+  float m_run[2] = {-3.0e38f, -3.0e38f};
+  // The denominators come out of the second product too: one more block row of V^T, all ones,
+  // sums P over the keys (every register of every lane then holds its query's denominator: the
+  // sum of the very values, rounded to bf16, that O is made of).
+  v4f den[2];
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+    for (int r = 0; r < 4; r++) den[qb][r] = 0.0f;
+  const v4i ones = {0x3f803f80, 0x3f803f80, 0x3f803f80, 0x3f803f80};
 
   // LDS of a key half: K tiles 0 and 1, then V tiles 0, 1 and 2.  K block kb goes to K tile
   // kb & 1, V block kb to V tile kb % 3.  A block index past the half's last block fetches the
@@ -307,17 +316,21 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
   // t + AHEAD is read behind the MFMAs of step t.  Two steps ahead measured best (16 x 2048 x 128:
   // 33.8 us; 1: 34.1, 3: 33.9, 4: 34.5, 8: 35.6, 12: 36.1, none: 45.4): the reads ahead of a
   // slot's first MFMA are time the matrix core of that SIMD stands still.
-  constexpr int PV_STEPS = NKC * NDB, QK_STEPS = NC * NKB, AHEAD = 2, RING = AHEAD + 1;
+  constexpr int PV_ROWS = NDB + 1;   // block rows of the second product: O^T's and the denominators'
+  constexpr int PV_STEPS = NKC * PV_ROWS, QK_STEPS = NC * NKB, AHEAD = 2, RING = AHEAD + 1;
   constexpr int K_READS = KT_ROWS ? 2 : 1;   // LDS instructions per K operand (V: always 2)
   v4i ring[RING];
   // steps [first, last) of the sequence PV(0 .. PV_STEPS) then QK(0 .. QK_STEPS)
   auto run_steps = [&](auto first_c, auto last_c, const uint8_t *lv, const uint8_t *lk) {
     constexpr int FIRST = decltype(first_c)::value, LAST = decltype(last_c)::value;
     auto fetch = [&](int t) {
-      if (t < PV_STEPS) ring[t % RING] = read_v(lv, t % NDB, t / NDB);
-      else ring[t % RING] = read_k(lk, (t - PV_STEPS) % NKB, (t - PV_STEPS) / NKB);
+      if (t < PV_STEPS) {
+        if (t % PV_ROWS < NDB) ring[t % RING] = read_v(lv, t % PV_ROWS, t / PV_ROWS);
+      } else {
+        ring[t % RING] = read_k(lk, (t - PV_STEPS) % NKB, (t - PV_STEPS) / NKB);
+      }
     };
-    auto reads_of = [](int t) { return t < PV_STEPS ? 2 : K_READS; };
+    auto reads_of = [](int t) { return t < PV_STEPS ? (t % PV_ROWS < NDB ? 2 : 0) : K_READS; };
 #pragma unroll
     for (int t = FIRST; t < LAST && t < FIRST + AHEAD; t++) fetch(t);
 #pragma unroll
@@ -325,9 +338,14 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
       if (t + AHEAD < LAST) fetch(t + AHEAD);
       const v4i a = ring[t % RING];
       if (t < PV_STEPS) {
-        const int db = t % NDB, kc = t / NDB;
-        o[db][0] = mfma(a, pb[kc][0], o[db][0]);
-        o[db][1] = mfma(a, pb[kc][1], o[db][1]);
+        const int db = t % PV_ROWS, kc = t / PV_ROWS;
+        if (db < NDB) {
+          o[db][0] = mfma(a, pb[kc][0], o[db][0]);
+          o[db][1] = mfma(a, pb[kc][1], o[db][1]);
+        } else {
+          den[0] = mfma(ones, pb[kc][0], den[0]);
+          den[1] = mfma(ones, pb[kc][1], den[1]);
+        }
       } else {
         const int kb = (t - PV_STEPS) % NKB, c = (t - PV_STEPS) / NKB;
         s[kb][0] = mfma(a, qf[0][c], s[kb][0]);
@@ -338,7 +356,7 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
     // of the operand AHEAD steps on and the step's two MFMAs.
     auto reads_group = [&](int t) {   // the builtin wants literal sizes
       if (reads_of(t) == 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-      else __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      else if (reads_of(t) == 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     };
 #pragma unroll
     for (int t = FIRST; t < LAST && t < FIRST + AHEAD; t++) reads_group(t);
@@ -391,9 +409,9 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
     // The running reference m_run (exponentials are taken as exp(x - m_run); the final division
     // by the denominator, accumulated against the same reference, cancels it exactly) is set from
     // the first block's maxima and then left alone: a block's maximum is only looked for when its
-    // sum of exponentials shows that some score outgrew the reference by more than 2^40, far
+    // largest exponential shows that some score outgrew the reference by more than 2^40, far
     // inside f32 and bf16 range.  That block's exponentials are then redone against the moved
-    // reference, and the running sums and the accumulators rescaled.  This takes the maximum
+    // reference, and the accumulators (the denominators' among them) rescaled.  This takes the maximum
     // (a quarter of the softmax's instructions and two cross-lane exchanges) out of almost every block.
     auto move_reference = [&]() {
 #pragma unroll
@@ -408,7 +426,8 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
         const float m_new = fmaxf(m_run[qb], mx);
         const float alpha = __builtin_amdgcn_exp2f((m_run[qb] - m_new) * LOG2E);
         m_run[qb] = m_new;
-        l_run[qb] *= alpha;
+#pragma unroll
+        for (int r = 0; r < 4; r++) den[qb][r] *= alpha;
 #pragma unroll
         for (int db = 0; db < NDB; db++)
 #pragma unroll
@@ -418,7 +437,7 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
     if (j == 0) move_reference();
     // In base 2: exp(x - m) = 2^(x*log2e - m*log2e).
     const float neg_m2[2] = {-m_run[0] * LOG2E, -m_run[1] * LOG2E};
-    float psum[2] = {0.0f, 0.0f};
+    float pmax[2] = {0.0f, 0.0f};   // the block's largest exponential per query: what tells a stale reference
     // The fetches of V(j + 1) and K(j + 2) go out one instruction at a time between the exponentials.
     const int ksrc = min(j + 2, nblocks - 1), vsrc = min(j + 1, nblocks - 1);
     const uint32_t kdst = lds_address(my_lds + (j & 1) * TILE), vdst = lds_address(my_lds + (2 + (j + 1) % 3) * TILE);
@@ -429,7 +448,7 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
 #pragma unroll
         for (int r = 0; r < 4; r++) {
           const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][qb][r], LOG2E, neg_m2[qb]));
-          psum[qb] += e;
+          pmax[qb] = fmaxf(pmax[qb], e);
           pb[kb / 2][qb][(kb % 2) * 4 + r] = (__bf16)e;
           constexpr int EVERY = 16 / PER_WAVE;
           const int n = (kb * 2 + qb) * 4 + r;   // 0 .. 31
@@ -439,23 +458,18 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
             else fetch_k(ksrc, i - PER_WAVE, kdst + (qg * PER_WAVE + i - PER_WAVE) * 1024);
           }
         }
-    if (j > 0 && __any(!(psum[0] < STALE_REFERENCE_SUM) || !(psum[1] < STALE_REFERENCE_SUM))) {
+    if (j > 0 && __any(!(pmax[0] < STALE_REFERENCE) || !(pmax[1] < STALE_REFERENCE))) {
       move_reference();
 #pragma unroll
       for (int qb = 0; qb < 2; qb++) {
         const float neg2 = -m_run[qb] * LOG2E;
-        psum[qb] = 0.0f;
 #pragma unroll
         for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
-          for (int r = 0; r < 4; r++) {
-            const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][qb][r], LOG2E, neg2));
-            psum[qb] += e;
-            pb[kb / 2][qb][(kb % 2) * 4 + r] = (__bf16)e;
-          }
+          for (int r = 0; r < 4; r++)
+            pb[kb / 2][qb][(kb % 2) * 4 + r] = (__bf16)__builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][qb][r], LOG2E, neg2));
       }
     }
-    l_run[0] += psum[0], l_run[1] += psum[1];
     __builtin_amdgcn_s_waitcnt(WAIT_BUT_TWO);
   };
 
@@ -481,12 +495,7 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
 
   // Merge the two key halves: (m, d, O) of half 1 goes through LDS to the wave of half 0
   // that owns the same queries.  Layout [value][lane] keeps lanes on distinct banks.
-  float l_tot[2];
-#pragma unroll
-  for (int qb = 0; qb < 2; qb++) {
-    const float t = l_run[qb] + __shfl_xor(l_run[qb], 16);
-    l_tot[qb] = t + __shfl_xor(t, 32);
-  }
+  const float l_tot[2] = {den[0][0], den[1][0]};
   __syncthreads();  // all K/V reads are done: the staging area is free
   constexpr int MR = DD::MERGE_ROWS;
   float *mbuf = (float *)lds + qg * (MR * 64);
