@@ -158,13 +158,18 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
 
   // Q^T operands: block column qb (queries 16 qb + l % 16 of the wave's 32), chunk c of d:
   // lane (l % 16, l / 16) holds d = 32 c + 8 (l / 16) .. + 7.
+  // Only the waves of half 0 load them; their partners of half 1, which own the same queries,
+  // get them through LDS at the first barrier (below): the start-up of a workgroup is bound by
+  // what it asks of its compute unit's load path, and Q twice was two fifths of that.
   v4i qf[2][NC];
+  if (!half) {
 #pragma unroll
-  for (int qb = 0; qb < 2; qb++) {
-    const int q_row = RAGGED ? min(q0 + 16 * qb + lr, int(p.m) - 1) : q0 + 16 * qb + lr;
-    const uint8_t *Q = (const uint8_t *)p.q + (head * p.m + q_row) * int64_t(ROW);
+    for (int qb = 0; qb < 2; qb++) {
+      const int q_row = RAGGED ? min(q0 + 16 * qb + lr, int(p.m) - 1) : q0 + 16 * qb + lr;
+      const uint8_t *Q = (const uint8_t *)p.q + (head * p.m + q_row) * int64_t(ROW);
 #pragma unroll
-    for (int c = 0; c < NC; c++) qf[qb][c] = *(const v4i *)(Q + c * 64 + lgp * 16);
+      for (int c = 0; c < NC; c++) qf[qb][c] = *(const v4i *)(Q + c * 64 + lgp * 16);
+    }
   }
 
   // Block staging.  One direct-to-LDS instruction fills 1 KiB (4 rows at D = 128); lane l lands
@@ -281,7 +286,25 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
   // which the compiler does not know of, so it adds no waits of its own for them in the loop.)
   if (nblocks > 0 && !half) issue_k(0);
   __builtin_amdgcn_s_waitcnt(0x0F70);
-  __syncthreads();
+  {
+    // Q's operands from half 0 to half 1, through V tiles 1 and 2 of half 1 (QG * D * 64 bytes: two
+    // tiles at most), which no fetch touches before that half's first softmax slot.
+    static_assert(QG * D * 64 <= 2 * TILE, "the exchange fits the two tiles");
+    v4i *qx = (v4i *)(lds + HALF + 3 * TILE) + qg * (2 * NC * 64) + lane;
+    if (!half) {
+#pragma unroll
+      for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+        for (int c = 0; c < NC; c++) qx[(qb * NC + c) * 64] = qf[qb][c];
+    }
+    __syncthreads();
+    if (half) {
+#pragma unroll
+      for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+        for (int c = 0; c < NC; c++) qf[qb][c] = qx[(qb * NC + c) * 64];
+    }
+  }
   if (nblocks > 0) {
     if (half) issue_k(0);
     issue_v(0);
