@@ -520,26 +520,22 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
   // that owns the same queries.  Layout [value][lane] keeps lanes on distinct banks.
   const float l_tot[2] = {den[0][0], den[1][0]};
   __syncthreads();  // all K/V reads are done: the staging area is free
-  constexpr int MR = DD::MERGE_ROWS;
-  float *mbuf = (float *)lds + qg * (MR * 64);
+  // [quad of values][lane], 16 bytes per lane: lanes on distinct banks, one instruction per quad.
+  constexpr int MQ = DD::MERGE_ROWS / 4;   // a lane's quads: O^T's blocks, then (m, m, l, l)
+  v4f *mbuf = (v4f *)lds + qg * (MQ * 64) + lane;
   if (half == 1) {
 #pragma unroll
     for (int db = 0; db < NDB; db++)
 #pragma unroll
-      for (int qb = 0; qb < 2; qb++)
-#pragma unroll
-        for (int r = 0; r < 4; r++) mbuf[((db * 2 + qb) * 4 + r) * 64 + lane] = o[db][qb][r];
-#pragma unroll
-    for (int qb = 0; qb < 2; qb++) {
-      mbuf[(D / 2 + qb) * 64 + lane] = m_run[qb];
-      mbuf[(D / 2 + 2 + qb) * 64 + lane] = l_tot[qb];
-    }
+      for (int qb = 0; qb < 2; qb++) mbuf[(db * 2 + qb) * 64] = o[db][qb];
+    mbuf[(NDB * 2) * 64] = v4f{m_run[0], m_run[1], l_tot[0], l_tot[1]};
   }
   __syncthreads();
   if (half == 0) {
+    const v4f ml = mbuf[(NDB * 2) * 64];
 #pragma unroll
     for (int qb = 0; qb < 2; qb++) {
-      const float m1 = mbuf[(D / 2 + qb) * 64 + lane], l1 = mbuf[(D / 2 + 2 + qb) * 64 + lane];
+      const float m1 = ml[qb], l1 = ml[2 + qb];
       const float mm = fmaxf(m_run[qb], m1);
       const float a0 = __builtin_amdgcn_exp2f((m_run[qb] - mm) * LOG2E), a1 = __builtin_amdgcn_exp2f((m1 - mm) * LOG2E);
       const int row = q0 + 16 * qb + lr;
@@ -550,12 +546,8 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
           float *part = p.partials + ((head * p.m + row) * int64_t(p.key_splits) + blockIdx.y) * (D + 4);
 #pragma unroll
           for (int db = 0; db < NDB; db++) {
-            float4 v;
-            v.x = o[db][qb][0] * a0 + mbuf[((db * 2 + qb) * 4 + 0) * 64 + lane] * a1;
-            v.y = o[db][qb][1] * a0 + mbuf[((db * 2 + qb) * 4 + 1) * 64 + lane] * a1;
-            v.z = o[db][qb][2] * a0 + mbuf[((db * 2 + qb) * 4 + 2) * 64 + lane] * a1;
-            v.w = o[db][qb][3] * a0 + mbuf[((db * 2 + qb) * 4 + 3) * 64 + lane] * a1;
-            *(float4 *)(part + db * 16 + 4 * lgp) = v;
+            const v4f v = o[db][qb] * a0 + mbuf[(db * 2 + qb) * 64] * a1;
+            *(float4 *)(part + db * 16 + 4 * lgp) = float4{v[0], v[1], v[2], v[3]};
           }
           if (lgp == 0) part[D] = mm, part[D + 1] = l_tot[qb] * a0 + l1 * a1;
         }
@@ -568,19 +560,15 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
       if (!RAGGED || row < int(p.m))
 #pragma unroll
         for (int db = 0; db < NDB; db++) {
-          float4 v;
-          v.x = o[db][qb][0] * w0 + mbuf[((db * 2 + qb) * 4 + 0) * 64 + lane] * w1;
-          v.y = o[db][qb][1] * w0 + mbuf[((db * 2 + qb) * 4 + 1) * 64 + lane] * w1;
-          v.z = o[db][qb][2] * w0 + mbuf[((db * 2 + qb) * 4 + 2) * 64 + lane] * w1;
-          v.w = o[db][qb][3] * w0 + mbuf[((db * 2 + qb) * 4 + 3) * 64 + lane] * w1;
+          const v4f v = o[db][qb] * w0 + mbuf[(db * 2 + qb) * 64] * w1;
           const int col = db * 16 + 4 * lgp;
           if (whole_rows) {
-            *(float4 *)(orow + col) = v;
+            *(float4 *)(orow + col) = float4{v[0], v[1], v[2], v[3]};
           } else {
-            if (col + 0 < int(p.n_out)) orow[col + 0] = v.x;
-            if (col + 1 < int(p.n_out)) orow[col + 1] = v.y;
-            if (col + 2 < int(p.n_out)) orow[col + 2] = v.z;
-            if (col + 3 < int(p.n_out)) orow[col + 3] = v.w;
+            if (col + 0 < int(p.n_out)) orow[col + 0] = v[0];
+            if (col + 1 < int(p.n_out)) orow[col + 1] = v[1];
+            if (col + 2 < int(p.n_out)) orow[col + 2] = v[2];
+            if (col + 3 < int(p.n_out)) orow[col + 3] = v[3];
           }
         }
     }
