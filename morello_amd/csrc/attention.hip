@@ -662,8 +662,11 @@ hipError_t launch_one(const AttnArgs &a, hipStream_t stream) {
   const dim3 grid(((a.m + BQ - 1) / BQ) * a.b, std::max(1u, a.key_splits));
   plan::work(plan::UNIT_MFMA_BF16, 4.0 * a.b * a.m * a.n2 * D,
              double(a.b) * (2.0 * a.m * D + 4.0 * a.n2 * D + 4.0 * a.m * a.n_out) + attn_partial_bytes(a, a.key_splits),
-             // the softmax between the two products shares the issue slots: 1.17 x the MFMA time at the
-             // sustained rate (measured at 16 x 2048 x 128); four waves hide less than eight: 1.2 x that
+             // the softmax between the two products shares the issue slots and the launch has fixed
+             // costs the model does not price: 1.17 x the MFMA time at the model's sustained rate puts
+             // 16 x 2048 x 128 at 37 us (measured 33-35 with the launch gap) and head dim 64, half the
+             // heads or twice the keys at 0.87-0.9 of their measured times; four waves hide less than
+             // eight: 1.2 x that
              (QG == 2 ? 1.2 : 1.0) * 1.17 * 4.0 * BQ * D * (double((a.n2 + BKV - 1) / BKV) * BKV / std::max(1u, a.key_splits)),
              3000.0);
   MRL_LAUNCH((k_attn<D, RAGGED, KT_ROWS, QG>), grid, dim3(128 * QG), LDS, stream, a.q, a.kt, a.v, a.out, a.b, a.m, a.n2, a.n_out,
