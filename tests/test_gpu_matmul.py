@@ -521,3 +521,44 @@ def test_matmul_with_bf16_output(gpu, dts, codes, accum):
         spec = M.Matmul([b, m, k, n], dts, layouts=[None, None, M.batched_col_major([b, m, n])])
         got_t = synth.bf16_bits_to_f32(run_spec(spec, [a, bm, np.zeros((b, n, m), np.uint16)]))
         assert np.array_equal(got_t.transpose(0, 2, 1), got)
+
+
+@pytest.mark.parametrize("dts,codes", [((M.u8, M.i8, M.i32), [0, 1, 5]), ((M.i8, M.i8, M.i32), [1, 1, 5]),
+                                       ((M.bf16, M.bf16, M.f32), [7, 7, 6])])
+@pytest.mark.parametrize("shape", [(1, 256, 20, 256), (2, 512, 22, 256), (1, 256, 36, 768), (1, 768, 52, 512)])
+@pytest.mark.parametrize("accum", [False, True])
+def test_the_four_wave_kernel_on_its_shapes(gpu, dts, codes, shape, accum):
+    """k_gemm_wide (256 x 256 tiles on four waves, MFMAs of 16 x 16) named through its schedule:
+    one and several tiles each way, batch entries, every length of the unrolled prologue
+    (accumulating Specs read C's old values during the first sixteen k steps) and of the rolled
+    loop behind it, all three operand types; K in steps of 128 bytes.  Integers bit for bit."""
+    b, m, steps, n = shape
+    es = 2 if dts[0] == M.bf16 else 1
+    k = steps * 128 // es
+    if dts[0] == M.bf16:
+        A, Bm = synth.normal_bf16(95, 0, (b, m, k)), synth.normal_bf16(95, 1, (b, k, n))
+        C0 = synth.normal_f32(95, 2, (b, m, n)) if accum else np.zeros((b, m, n), np.float32)
+    else:
+        A = synth.uniform_u8(95, 0, (b, m, k)) if dts[0] == M.u8 else synth.uniform_i8(95, 0, (b, m, k))
+        Bm = synth.uniform_i8(95, 1, (b, k, n))
+        C0 = (synth.uniform_u8(95, 2, (b, m, n)).astype(np.int32) * 1000003 - 77) if accum else np.zeros((b, m, n), np.int32)
+    spec = M.Matmul([b, m, k, n], dts, accum=accum)
+    sched = spec.tile_out([1, 256, 256]).split(128 // es).staged(M.Staging.DirectBWide)
+    assert sched.plan().kernels == ["k_gemm_wide"]
+    bufs = [M.DeviceBuffer.from_numpy(x) for x in (A, Bm, C0)]
+    sched.run_device([x.ptr for x in bufs])
+    got = bufs[2].to_numpy(C0.dtype, (b, m, n))
+    for x in bufs:
+        x.free()
+    want = orc.matmul([b, m, k, n], codes, A, Bm, C0.copy(), accum)
+    if dts[2] == M.i32:
+        assert np.array_equal(got, want)
+    else:
+        assert rel_err(got, want) < 1e-5
+
+
+def test_the_four_wave_kernel_turns_down_other_shapes(gpu):
+    spec = M.Matmul([1, 256, 2432, 256], (M.u8, M.i8, M.i32))     # 19 steps: an odd number, and too few
+    with pytest.raises(M.MorelloError) as e:
+        spec.tile_out([1, 256, 256]).split(128).staged(M.Staging.DirectBWide).plan()
+    assert e.value.status == 1
