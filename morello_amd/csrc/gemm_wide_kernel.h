@@ -73,7 +73,8 @@ constexpr int WIDE_MIN_STEPS = GEMM_WIDE_MIN_STEPS;
                  [dma_base] "s"(dma_base), [cbase] "s"(c_base), [ldc16] "s"(ldc16), [k16] "s"(k16)                 \
                : MRL_WIDE_CLOBBERS)
 
-// M, N multiples of 256; K an even number of k steps, GEMM_WIDE_MIN_STEPS at least; see wide_applicable().
+// M, N multiples of 256; K an even number of k steps: GEMM_WIDE_MIN_STEPS at least for an accumulating
+// Spec (whose first sixteen steps carry the loads of C's old values), four otherwise; see wide_applicable().
 template <class T, bool A_UNSIGNED>
 __global__ __launch_bounds__(256) void k_gemm_wide(GemmArgs g, int tiles_m, int tiles_n, int group_m) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -180,11 +181,18 @@ __global__ __launch_bounds__(256) void k_gemm_wide(GemmArgs g, int tiles_m, int 
   }
 }
 
-// Whole tiles, an even number of k steps (enough for the steps that carry C's old values), offsets
-// the loop's 32-bit arithmetic can hold.
+// Whole tiles, an even number of k steps, offsets the loop's 32-bit arithmetic can hold.  An
+// accumulating Spec needs the steps that carry C's old values; another one may be as short as four
+// steps, and is taken that short when its tiles run in one round (measured against the eight-wave
+// tile, non-accumulating: int8 4096 x 512 x 4096 19.5 against 21.3 us, 3072 x 2048 x 3072 27.3 / 31.0,
+// bf16 4096 x 1024 x 4096 34.6 / 38.4; but 8192 x 768 x 8192, four rounds of tiles bound by the
+// write of C, 99.0 / 94.3: this kernel's stores are 64-byte row segments).
 inline bool wide_applicable(const GemmArgs &g, int elem_size) {
   const int64_t bk = 128 / elem_size;
-  return !g.b_kmajor && g.m % 256 == 0 && g.n % 256 == 0 && g.k % (2 * bk) == 0 && g.k >= WIDE_MIN_STEPS * bk &&
+  const bool long_k = g.k >= WIDE_MIN_STEPS * bk;
+  const bool one_round = uint64_t(g.m / 256) * (g.n / 256) * g.batch <= g_compute_units;
+  return !g.b_kmajor && g.m % 256 == 0 && g.n % 256 == 0 && g.k % (2 * bk) == 0 &&
+         (long_k || (!g.accum && g.k >= 4 * bk && one_round)) &&
          g.lda * elem_size * 256 < (int64_t(1) << 32) && g.ldb * elem_size * (bk + 1) < (int64_t(1) << 31) &&
          g.ldc * 4 * 32 < (int64_t(1) << 31);
 }

@@ -562,3 +562,37 @@ def test_the_four_wave_kernel_turns_down_other_shapes(gpu):
     with pytest.raises(M.MorelloError) as e:
         spec.tile_out([1, 256, 256]).split(128).staged(M.Staging.DirectBWide).plan()
     assert e.value.status == 1
+
+
+@pytest.mark.parametrize("dts,codes", [((M.u8, M.i8, M.i32), [0, 1, 5]), ((M.bf16, M.bf16, M.f32), [7, 7, 6])])
+@pytest.mark.parametrize("steps", [4, 6, 14])
+def test_the_four_wave_kernel_on_a_short_k(gpu, dts, codes, steps):
+    """A Spec that does not accumulate needs none of the sixteen k steps that carry C's old values:
+    the kernel takes it from four steps of 128 bytes on (the dispatch rules' own choice where the
+    tiles run in one round); an accumulating Spec that short is turned down."""
+    b, m, n = 1, 512, 768
+    es = 2 if dts[0] == M.bf16 else 1
+    k = steps * 128 // es
+    if dts[0] == M.bf16:
+        A, Bm = synth.normal_bf16(96, 0, (b, m, k)), synth.normal_bf16(96, 1, (b, k, n))
+    else:
+        A, Bm = synth.uniform_u8(96, 0, (b, m, k)), synth.uniform_i8(96, 1, (b, k, n))
+    C0 = np.full((b, m, n), 7, np.float32 if dts[2] == M.f32 else np.int32)   # overwritten, not added to
+    spec = M.Matmul([b, m, k, n], dts)
+    assert M.Matmul([1, 4096, k, 4096], dts).plan().kernels == ["k_gemm_wide"]       # 256 tiles: one round
+    assert M.Matmul([1, 8192, k, 8192], dts).plan().kernels == ["k_gemm_big"]        # four rounds
+    sched = spec.tile_out([1, 256, 256]).split(128 // es).staged(M.Staging.DirectBWide)
+    assert sched.plan().kernels == ["k_gemm_wide"]
+    want = orc.matmul([b, m, k, n], codes, A, Bm, np.zeros_like(C0), False)
+    bufs = [M.DeviceBuffer.from_numpy(x) for x in (A, Bm, C0)]
+    sched.run_device([x.ptr for x in bufs])
+    got = bufs[2].to_numpy(C0.dtype, (b, m, n))
+    for x in bufs:
+        x.free()
+    if dts[2] == M.i32:
+        assert np.array_equal(got, want)
+    else:
+        assert rel_err(got, want) < 1e-5
+    with pytest.raises(M.MorelloError) as e:
+        M.MatmulAccum([b, m, k, n], dts).tile_out([1, 256, 256]).split(128 // es).staged(M.Staging.DirectBWide).plan()
+    assert e.value.status == 1
