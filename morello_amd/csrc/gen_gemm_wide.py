@@ -66,8 +66,8 @@ TM, TN = 8, 8       # MFMA blocks per wave
 MF = TM * TN        # MFMAs per slab
 SLABS = 2
 GAPS = SLABS * MF   # MFMAs per k step
-BARRIER_AT = int(os.environ.get("WIDE_BARRIER_AT", 96))     # the step's barrier comes before this MFMA
-GAP_SLOTS = int(os.environ.get("WIDE_GAP_SLOTS", 2))       # instructions placed behind one MFMA before the next is due (2: 63.7 us at 4096^3 int8, 3: 64.5)
+BARRIER_AT = 96     # the step's barrier comes before this MFMA (88, 100, 104: the same; 80: 1-2 % slower)
+GAP_SLOTS = 2       # instructions placed behind one MFMA before the next is due (2: 63.7 us at 4096^3 int8, 3: 64.5, 4: 65)
 C_STEPS = 16        # k steps that carry the loads of C's old values (16 registers a step)
 C_BLOCKS = 4        # blocks of C a step loads
 
@@ -525,8 +525,7 @@ def main():
     parts = ["// Generated by gen_gemm_wide.py -- do not edit; the generator documents the schedule.\n",
              f"#define GEMM_WIDE_MIN_STEPS {MIN_STEPS}\n"]
     for name, kind, wm, accum in variants():
-        # WIDE_OPTS: experiment switches (timing builds with an ingredient left out; results are wrong)
-        lines = gen(kind, wm, accum, {k: True for k in os.environ.get("WIDE_OPTS", "").split(",") if k})
+        lines = gen(kind, wm, accum)
         body = " \\\n".join('  "' + l + '\\n"' for l in lines)
         parts.append(f"#define {name} \\\n{body}\n")
     with open(out_path, "w") as f:
