@@ -559,7 +559,12 @@ hipError_t launch(const GemmArgs &g, hipStream_t stream) {
                2.0 * BM * BN * k_steps,
                // prologue and epilogue, then one barrier-to-barrier trip per step of K, longer for a
                // larger tile (measured 0.4-0.55 us at 64 x 64, 0.6-1.0 at 128 x 128, 1.4-2.0 at 256 x 256)
-               500.0 + (100.0 + 3.0 * (BM + BN)) * double((g.k * T::ES + TL::BKB - 1) / TL::BKB));
+               // on int8 and bf16, whose steps hold the same MFMA time; an f32 step's MFMAs take
+               // longer by the difference of the datasheet rates, and a workgroup alone on its unit
+               // does not overlap them with the trip (f32 at 64 x 64: 0.9 us per step)
+               500.0 + (100.0 + 3.0 * (BM + BN) +
+                        2.0 * BM * BN * ((TL::BKB / T::ES) / plan::nominal_unit_rate(T::ES) - TL::BKB / plan::nominal_unit_rate(1))) *
+                           double((g.k * T::ES + TL::BKB - 1) / TL::BKB));
   }
   MRL_LAUNCH((k_gemm<T, A_UNSIGNED, TL, EDGE, B_KMAJOR, CONV>), dim3(tiles_m * tiles_n, g.batch), dim3(TL::NT),
              2 * STAGE, stream, g, tiles_m, tiles_n, group_rows(tiles_m, tiles_n));
