@@ -14,6 +14,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libmorello_amd.so")
 OBJ_DIR = os.path.join(HERE, "build")
+GEN_DIR = os.path.join(OBJ_DIR, "gen")   # generated assembly (the k loops of the two 256 x 256 tiles)
+# generator -> the file the kernel header of the same tile includes
+GENERATED = {"gen_gemm_wide.py": "gemm_wide_gfx950.inc", "gen_gemm_loop.py": "gemm_loop_gfx950.inc"}
 
 SOURCES = ["api.hip", "generic.hip", "gemm_mfma.hip", "gemm_sched.hip", "gemm_nt.hip", "gemv.hip", "conv_gemm.hip", "conv_i8.hip", "unfold.hip", "softmax.hip", "parts.hip", "mfma_rate.hip", "attention.hip", "plan.hip"]
 
@@ -40,7 +43,7 @@ def _hipcc() -> str:
 
 def _compile(src: str) -> str:
     obj = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
-    cmd = [_hipcc(), *FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [_hipcc(), *FLAGS, *EXTRA_FLAGS.get(src, []), "-I", GEN_DIR, "-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
@@ -51,10 +54,24 @@ def _compile(src: str) -> str:
     return obj
 
 
+def generate() -> None:
+    """Runs the assembly generators.  Their output (2 MB of text) goes beside the object files, not
+    into the source directory, and is never kept in the tree; a copy left in the source directory
+    by an older build would shadow it (a quoted #include looks there first), so it is removed."""
+    os.makedirs(GEN_DIR, exist_ok=True)
+    for script, inc in GENERATED.items():
+        stale = os.path.join(CSRC, inc)
+        if os.path.exists(stale):
+            os.remove(stale)
+        res = subprocess.run([sys.executable, os.path.join(CSRC, script), os.path.join(GEN_DIR, inc)],
+                             capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError(f"{script} failed:\n{res.stdout}\n{res.stderr}")
+
+
 def build(verbose: bool = True) -> str:
     os.makedirs(OBJ_DIR, exist_ok=True)
-    # The assembly of the four-wave Matmul tile is generated (1.5 MB of text): not kept in the tree.
-    subprocess.run([sys.executable, os.path.join(CSRC, "gen_gemm_wide.py")], check=True, capture_output=True)
+    generate()
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
         objs = list(pool.map(_compile, SOURCES))
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", OUT, *objs]

@@ -56,7 +56,8 @@ constexpr int WIDE_MIN_STEPS = GEMM_WIDE_MIN_STEPS;
       MRL_WIDE_FIRST_100("a"), MRL_WIDE_100("a", 1), MRL_WIDE_10("a", 20), MRL_WIDE_10("a", 21),            \
       MRL_WIDE_10("a", 22), MRL_WIDE_10("a", 23), MRL_WIDE_10("a", 24), "a250", "a251", "a252", "a253",     \
       "a254", "a255", "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71",   \
-      "s72", "s73", "s78", "s79", "scc", "memory"
+      "s72", "s73", "s78", "s79", "s80", "s81", "s82", "s83", "s84", "s85", "s86", "s87", "s88", "s89", "s90",     \
+      "s91", "s92", "s93", "s94", "s95", "scc", "memory"
 
 #define MRL_WIDE_RUN(TEXT)                                                                                         \
   asm volatile(TEXT                                                                                                \
@@ -67,10 +68,12 @@ constexpr int WIDE_MIN_STEPS = GEMM_WIDE_MIN_STEPS;
                  [b_off4] "v"(b_off[4]), [b_off5] "v"(b_off[5]), [b_off6] "v"(b_off[6]), [b_off7] "v"(b_off[7]),   \
                  [a_wr] "v"(a_wr), [a_rd0] "v"(a_rd[0]), [a_rd1] "v"(a_rd[1]), [b_rd0] "v"(b_rd[0]),               \
                  [b_rd1] "v"(b_rd[1]), [b_rd2] "v"(b_rd[2]), [b_rd3] "v"(b_rd[3]), [b_rd4] "v"(b_rd[4]),           \
-                 [b_rd5] "v"(b_rd[5]), [b_rd6] "v"(b_rd[6]), [b_rd7] "v"(b_rd[7]), [c_row0] "v"(c_row[0]),         \
-                 [c_row1] "v"(c_row[1]), [c_row2] "v"(c_row[2]), [c_row3] "v"(c_row[3]), [part_wr] "v"(part_wr),   \
-                 [part_rd] "v"(part_rd), [abase] "s"(A), [bbase] "s"(B), [bstep] "s"(b_step), [nk] "s"(nk),        \
-                 [dma_base] "s"(dma_base), [cbase] "s"(c_base), [ldc16] "s"(ldc16), [k16] "s"(k16)                 \
+                 [b_rd5] "v"(b_rd[5]), [b_rd6] "v"(b_rd[6]), [b_rd7] "v"(b_rd[7]), [c_lo0] "v"(c_lo[0]),           \
+                 [c_lo1] "v"(c_lo[1]), [c_lo2] "v"(c_lo[2]), [c_lo3] "v"(c_lo[3]), [c_hi0] "v"(c_hi[0]),           \
+                 [c_hi1] "v"(c_hi[1]), [c_hi2] "v"(c_hi[2]), [c_hi3] "v"(c_hi[3]), [part_wr] "v"(part_wr),         \
+                 [part_rd_lo] "v"(part_rd_lo), [part_rd_hi] "v"(part_rd_hi), [abase] "s"(A), [bbase] "s"(B),       \
+                 [bstep] "s"(b_step), [nk] "s"(nk), [dma_base] "s"(dma_base), [cbase] "s"(c_base),                 \
+                 [ldc16] "s"(ldc16), [k32] "s"(k32)                                                                \
                : MRL_WIDE_CLOBBERS)
 
 // M, N multiples of 256; K an even number of k steps: GEMM_WIDE_MIN_STEPS at least for an accumulating
@@ -88,6 +91,12 @@ __global__ __launch_bounds__(256) void k_gemm_wide(GemmArgs g, int tiles_m, int 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
+  // The four waves run one instruction stream (a second one costs instruction-cache misses all
+  // through the unrolled steps: 340 cycles a step measured).  What differs between the wave rows
+  // is in registers: for a u8 operand the lower wave row numbers its eight block columns from the
+  // fifth on (rot = 4), so that "add up the column sums of block columns 0 .. 3" covers columns
+  // 64 .. 127 of the wave's 128 there and columns 0 .. 63 in the upper wave row.
+  const int rot = (A_UNSIGNED && wm == 1) ? TN / 2 : 0;
 
   // Workgroups go to the 8 XCDs round-robin; each XCD gets a contiguous run of tiles which, taken
   // group_m tile rows at a time, covers a compact block of C (its A rows and B columns stay in
@@ -145,23 +154,31 @@ __global__ __launch_bounds__(256) void k_gemm_wide(GemmArgs g, int tiles_m, int 
     const int p = lane & 15;
     const int k = GROUP_K * (lane >> 4) + p / LANES_PER_ROW;
 #pragma unroll
-    for (int tn = 0; tn < TN; tn++) {
+    for (int t = 0; t < TN; t++) {
+      const int tn = (t + rot) % TN;
       const int byte = (wn * WN + tn * 16 + (8 / ES) * (p % LANES_PER_ROW)) * ES;
-      b_rd[tn] = lds0 + k * B_ROWB + wide_b_swizzle<T>(byte, k);
+      b_rd[t] = lds0 + k * B_ROWB + wide_b_swizzle<T>(byte, k);
     }
   }
-  // C: register i of a 16 x 16 block holds row 4 * (l / 16) + i, column l % 16.
-  uint32_t c_row[4];
+  // C: register i of a 16 x 16 block holds row 4 * (l / 16) + i, column l % 16.  The loop addresses
+  // block column t as c_lo (t < 4) or c_hi (t >= 4) plus t * 64 bytes: with the columns rotated by
+  // four blocks the base pointer sits four blocks to the left and c_lo makes up for eight.
+  uint32_t c_lo[4], c_hi[4];
 #pragma unroll
-  for (int i = 0; i < 4; i++) c_row[i] = uint32_t((lane >> 4) * 4 + i) * ldc_b + (lane & 15) * 4;
-  const uint8_t *c_base = (const uint8_t *)(C + int64_t(wm * WM) * g.ldc + wn * WN);
+  for (int i = 0; i < 4; i++) {
+    c_hi[i] = uint32_t((lane >> 4) * 4 + i) * ldc_b + (lane & 15) * 4;
+    c_lo[i] = c_hi[i] + (rot ? 512 : 0);
+  }
+  const uint8_t *c_base = (const uint8_t *)(C + int64_t(wm * WM) * g.ldc + wn * WN) - (rot ? 256 : 0);
   const uint32_t ldc16 = 16 * ldc_b;
-  // Column-sum partials [wave row x lane group][256 columns], in LDS from its start once the loop is over.
-  const uint32_t part_wr = lds0 + ((wm * 4 + (lane >> 4)) * BN + wn * WN + (lane & 15)) * 4;
-  const uint32_t part_rd = lds0 + (wn * WN + (lane & 15)) * 4;
+  // Column-sum partials [lane group][256 columns] of 4 bytes, 1 KiB into LDS once the loop is over:
+  // a wave writes those of its block columns 0 .. 3 and reads all eight (rotated like C's).
+  const uint32_t part = lds0 + 1024 + (wn * WN + (lane & 15)) * 4;
+  const uint32_t part_wr = part + (lane >> 4) * (BN * 4) + (rot ? 256 : 0);
+  const uint32_t part_rd_lo = part + (rot ? 256 : 0), part_rd_hi = part - (rot ? 256 : 0);
 
   const uint32_t b_step = uint32_t(BK) * ldb_b;
-  const uint32_t nk = g.k / BK, k16 = 16 * g.k;
+  const uint32_t nk = g.k / BK, k32 = 32 * g.k;
 
   if constexpr (std::is_same<T, BF16>::value) {
     if (g.accum) MRL_WIDE_RUN(GEMM_WIDE_BF16_ACC);
@@ -170,14 +187,8 @@ __global__ __launch_bounds__(256) void k_gemm_wide(GemmArgs g, int tiles_m, int 
     if (g.accum) MRL_WIDE_RUN(GEMM_WIDE_I8_ACC);
     else MRL_WIDE_RUN(GEMM_WIDE_I8);
   } else {
-    // The two wave rows share B's columns and each adds up the column sums of one slab of every step.
-    if (g.accum) {
-      if (wm == 0) MRL_WIDE_RUN(GEMM_WIDE_U8_0_ACC);
-      else MRL_WIDE_RUN(GEMM_WIDE_U8_1_ACC);
-    } else {
-      if (wm == 0) MRL_WIDE_RUN(GEMM_WIDE_U8_0);
-      else MRL_WIDE_RUN(GEMM_WIDE_U8_1);
-    }
+    if (g.accum) MRL_WIDE_RUN(GEMM_WIDE_U8_ACC);
+    else MRL_WIDE_RUN(GEMM_WIDE_U8);
   }
 }
 

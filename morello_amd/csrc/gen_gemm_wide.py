@@ -32,7 +32,9 @@ free as long as both operands agree, and here both hold bytes 16 g .. 16 g + 15 
     addresses, tell the pieces apart);
   * the column sums of B that the u8 correction needs are added up from the B operand registers
     (xor 0x80, sum of unsigned bytes: b + 128; the dot-product instructions hold up the MFMAs
-    behind them); the two wave rows share the columns and take one slab of a step each;
+    behind them); the two wave rows share the columns and take half of them each -- in the code
+    it is block columns 0 .. 3 for every wave, and the kernel numbers the lower wave row's block
+    columns from the fifth on, so that all four waves run the same instructions;
   * one barrier, three quarters through the step, preceded by the step's wait for memory:
     everything requested before this step began has landed; the next tile's first operands are
     read behind it;
@@ -162,8 +164,8 @@ class Item:
         self.gap = None
 
 
-def gen(kind, wm, accum, opts=None):
-    """kind: 'u8' (A unsigned bytes), 'i8', 'bf16'.  wm: the wave row (which slab's column sums it adds).
+def gen(kind, accum, opts=None):
+    """kind: 'u8' (A unsigned bytes), 'i8', 'bf16'.
     accum: the Spec accumulates into C (its old contents are read)."""
     opts = opts or {}     # experiment switches; the shipped loops are generated with none
     unsigned = kind == "u8" and not opts.get("no_valu")
@@ -172,6 +174,27 @@ def gen(kind, wm, accum, opts=None):
     tr = "ds_read_b64_tr_b16" if is_float else "ds_read_b64_tr_b8"
     e = Emitter()
     E = e.emit
+
+    trace = bool(opts.get("trace"))
+
+    def stamp(pair):
+        """Timing build only: the shader clock counter into s[pair:pair+1] (read after the next
+        wait for lgkmcnt(0))."""
+        if trace:
+            E(f"s_memtime s[{pair}:{pair + 1}]")
+
+    if trace:
+        # s80..s95: s[80:81] start, s82 loop start, s83 end of the unrolled steps, s[84:89] a step's
+        # three stamps, s90 scratch, s91 cycles waited for memory before barriers, s92 cycles in
+        # barriers, s93 end of loop, s94 last stamp before a barrier, s95 real-time clock at start
+        stamp(80)
+        E("s_memrealtime s[86:87]")
+        E("s_mov_b32 s91, 0")
+        E("s_mov_b32 s92, 0")
+        E("s_mov_b32 s88, 0")
+        E("s_mov_b32 s94, 0")
+        E("s_waitcnt lgkmcnt(0)")
+        E("s_mov_b32 s95, s86")
 
     def advance(ptr_lo, ptr_hi, idx, step, tmp):
         """Next tile: one k step on; past the last tile the pointer stays (that tile is fetched
@@ -332,14 +355,16 @@ def gen(kind, wm, accum, opts=None):
         add(advance_a, 5, 84, after=last_a)
         add(advance_b, 5, 88, after=last_b)
         if unsigned:
-            s = wm                       # this wave row sums slab wm of every step
-            for tn in range(TN):
-                for w in range(4):
-                    # after the first MFMA that waited for this operand, before the reads that overwrite it
-                    add(lambda s=s, tn=tn, w=w: (e.need(bf(s, tn, w // 2)),
-                                                  E(f"v_xor_b32 v{TMP0}, 0x80808080, {bf(s, tn, w=w)}"),
-                                                  E(f"v_sad_u8 v{COL_SUM + tn}, v{TMP0}, 0, v{COL_SUM + tn}")),
-                        2, MF * s + tn + 1, MF * s + MF - 1 if s == 0 else GAPS - 1)
+            # Block columns 0 .. 3 of both slabs: the other wave row, whose block columns are the
+            # same columns rotated by four, adds up the other half.
+            for s in range(SLABS):
+                for tn in range(TN // 2):
+                    for w in range(4):
+                        # after the first MFMA that waited for this operand, before the reads that overwrite it
+                        add(lambda s=s, tn=tn, w=w: (e.need(bf(s, tn, w // 2)),
+                                                      E(f"v_xor_b32 v{TMP0}, 0x80808080, {bf(s, tn, w=w)}"),
+                                                      E(f"v_sad_u8 v{COL_SUM + tn}, v{TMP0}, 0, v{COL_SUM + tn}")),
+                            2, MF * s + tn + 1, MF * s + MF - 1 if s == 0 else GAPS - 1)
         for it in extra:
             items.append(it)
         # Place the items in the order given, each into the first gap from its earliest on with room.
@@ -363,10 +388,19 @@ def gen(kind, wm, accum, opts=None):
         def sync():
             # everything requested before this step has landed (B of tile kt + 1, A of tile kt + 2);
             # this wave's LDS writes are done and the operands of the rest of the step are in
+            stamp(84)
             e.vm_wait_index(vm_before_step - 1)
+            stamp(86)
             E("s_waitcnt lgkmcnt(0)")
             e.all_lds_done()
+            if trace:
+                E("s_sub_u32 s90, s88, s94")      # the previous step's barrier
+                E("s_add_u32 s92, s92, s90")
+                E("s_sub_u32 s90, s86, s84")      # this step's wait for memory
+                E("s_add_u32 s91, s91, s90")
+                E("s_mov_b32 s94, s86")
             E("s_barrier")
+            stamp(88)
             set_b_read_base("s65")
 
         header()
@@ -386,7 +420,7 @@ def gen(kind, wm, accum, opts=None):
                     n += 1
 
     # ---- C: register q = 0..255: block q / 4 (tm = block / 8, tn = block % 8), register i = q % 4,
-    # which holds row 4 * (lane / 16) + i of the block (%[c_row i]) and column lane % 16.
+    # which holds row 4 * (lane / 16) + i of the block (%[c_lo i] / %[c_hi i]) and column lane % 16.
     ptr_tm = [None]
 
     def c_ptr(tm):
@@ -400,6 +434,12 @@ def gen(kind, wm, accum, opts=None):
             E(f"s_mul_hi_u32 s79, %[ldc16], {tm}")
             E("s_add_u32 s72, s72, s78")
             E("s_addc_u32 s73, s73, s79")
+
+    def c_addr(tn, i):
+        """The lane's byte offset of row i of a block in block column tn, less tn * 64: one set of
+        registers for block columns 0 .. 3 and one for 4 .. 7 (they differ for a wave row whose
+        block columns are rotated)."""
+        return f"%[c_lo{i}]" if tn < TN // 2 else f"%[c_hi{i}]"
 
     def where(q):
         block = q // 4
@@ -418,7 +458,7 @@ def gen(kind, wm, accum, opts=None):
 
             def ld(tm=tm, tn=tn, i=i, reg=reg):
                 c_ptr(tm)
-                e.vm(f"global_load_dword {reg}, %[c_row{i}], s[72:73] offset:{tn * 64}", dst=reg)
+                e.vm(f"global_load_dword {reg}, {c_addr(tn, i)}, s[72:73] offset:{tn * 64}", dst=reg)
             out.append(Item(ld, 1, 6 * r))
         return out
 
@@ -452,6 +492,10 @@ def gen(kind, wm, accum, opts=None):
         E("s_cbranch_scc1 1b")
 
     # ---- the k loop ---------------------------------------------------------------------------------
+    if trace:
+        stamp(82)
+        E("s_waitcnt lgkmcnt(0)")
+        e.all_lds_done()
     unrolled = C_STEPS + 2 if accum else 2
     for j in range(unrolled):
         extra = []
@@ -460,6 +504,11 @@ def gen(kind, wm, accum, opts=None):
         if accum and 1 <= j <= C_STEPS and not opts.get("no_cops"):
             extra += add_old_values(j - 1)
         step(j & 1, zero_first=(j == 0), extra=extra)
+    if trace:
+        stamp(84)
+        E("s_waitcnt lgkmcnt(0)")
+        e.all_lds_done()
+        E("s_mov_b32 s83, s84")
     E(f"s_sub_u32 s64, %[nk], {unrolled}")
     E("s_cmp_eq_u32 s64, 0")
     E("s_cbranch_scc1 2f")
@@ -468,42 +517,68 @@ def gen(kind, wm, accum, opts=None):
     # nothing may land in LDS once the epilogue reuses it; the last MFMAs must have written the
     # accumulators before they are read
     E("s_waitcnt vmcnt(0) lgkmcnt(0)")
+    if trace:
+        E("s_sub_u32 s90, s88, s94")
+        E("s_add_u32 s92, s92, s90")
+        stamp(84)
+        E("s_waitcnt lgkmcnt(0)")
+        E("s_mov_b32 s93, s84")
     E("s_barrier")
 
     # ---- epilogue -----------------------------------------------------------------------------------
     if unsigned:
-        # Column sums: the partials of the two wave rows and the four lane groups meet in LDS
-        # (each summed K / 8 values of b + 128).
-        for tn in range(TN):
-            E(f"v_subrev_u32 v{COL_SUM + tn}, %[k16], v{COL_SUM + tn}")
+        # Column sums: a wave holds, per lane group, the sums of b + 128 over a quarter of K for its
+        # block columns 0 .. 3; the four groups' partials of every column meet in LDS, where each
+        # wave finds those of all eight of its block columns (its own and the other wave row's).
+        for tn in range(TN // 2):
+            E(f"v_subrev_u32 v{COL_SUM + tn}, %[k32], v{COL_SUM + tn}")
             e.lds_write(f"ds_write_b32 %[part_wr], v{COL_SUM + tn} offset:{tn * 64}")
         E("s_waitcnt lgkmcnt(0)")
         e.all_lds_done()
         E("s_barrier")
         for tn in range(TN):
-            for w in range(8):
-                reg = f"v{64 + 8 * tn + w}"
-                e.lds_read(reg, f"ds_read_b32 {reg}, %[part_rd] offset:{w * 1024 + tn * 64}")
+            for w in range(4):
+                reg = f"v{64 + 4 * tn + w}"
+                addr = "%[part_rd_lo]" if tn < TN // 2 else "%[part_rd_hi]"
+                e.lds_read(reg, f"ds_read_b32 {reg}, {addr} offset:{w * 1024 + tn * 64}")
         for tn in range(TN):
-            regs = [f"v{64 + 8 * tn + w}" for w in range(8)]
+            regs = [f"v{64 + 4 * tn + w}" for w in range(4)]
             e.need(*regs)
             E(f"v_add3_u32 v{COL_SUM + tn}, {regs[0]}, {regs[1]}, {regs[2]}")
-            E(f"v_add3_u32 v{COL_SUM + tn}, v{COL_SUM + tn}, {regs[3]}, {regs[4]}")
-            E(f"v_add3_u32 v{COL_SUM + tn}, v{COL_SUM + tn}, {regs[5]}, {regs[6]}")
-            E(f"v_add_lshl_u32 v{COL_SUM + tn}, v{COL_SUM + tn}, {regs[7]}, 7")
+            E(f"v_add_lshl_u32 v{COL_SUM + tn}, v{COL_SUM + tn}, {regs[3]}, 7")
     else:
         E("s_nop 15")
         E("s_nop 15")
-    for q in range(0 if not opts.get("no_epilogue") else 256, 256):
-        tm, tn, i = where(q)
-        c_ptr(tm)
-        if not unsigned:
-            E(f"global_store_dword %[c_row{i}], a{q}, s[72:73] offset:{tn * 64}")
-        else:
-            t = f"v{16 + q % 32}"
-            E(f"v_accvgpr_read_b32 {t}, a{q}")
-            E(f"v_add_u32 {t}, {t}, v{COL_SUM + tn}")
-            E(f"global_store_dword %[c_row{i}], {t}, s[72:73] offset:{tn * 64}")
+    st_flags = opts.get("st_flags", "")
+    if opts.get("no_epilogue"):
+        pass
+    else:
+        for q in range(256):
+            tm, tn, i = where(q)
+            c_ptr(tm)
+            if not unsigned:
+                E(f"global_store_dword {c_addr(tn, i)}, a{q}, s[72:73] offset:{tn * 64}{st_flags}")
+            else:
+                t = f"v{16 + q % 32}"
+                E(f"v_accvgpr_read_b32 {t}, a{q}")
+                E(f"v_add_u32 {t}, {t}, v{COL_SUM + tn}")
+                E(f"global_store_dword {c_addr(tn, i)}, {t}, s[72:73] offset:{tn * 64}{st_flags}")
+    if trace:
+        # The stamps replace the first rows of the wave's block of C (a timing build: its results are
+        # not looked at): value j at row j % 4, columns 16 * (j / 4) .. + 15 of the block.
+        stamp(84)
+        E("s_waitcnt vmcnt(0) lgkmcnt(0)")
+        stamp(86)
+        E("s_memrealtime s[88:89]")
+        E("s_getreg_b32 s90, hwreg(HW_REG_HW_ID)")
+        E("s_waitcnt lgkmcnt(0)")
+        ptr_tm[0] = None
+        c_ptr(0)
+        for j, sreg in enumerate(["s80", "s82", "s83", "s93", "s84", "s86", "s95", "s88", "s91", "s92", "s90",
+                                   "s81"]):
+            E(f"v_mov_b32 v{TMP0}, {sreg}")
+            E(f"global_store_dword %[c_lo{j % 4}], v{TMP0}, s[72:73] offset:{(j // 4) * 64}")
+            E("s_nop 1")
     return e.lines
 
 
@@ -511,21 +586,25 @@ MIN_STEPS = C_STEPS + 4   # k steps a problem needs: the steps that carry C's ol
 
 
 def variants():
-    for kind, wms in (("u8", (0, 1)), ("i8", (0,)), ("bf16", (0,))):
-        for wm in wms:
-            for accum in (False, True):
-                name = f"GEMM_WIDE_{kind.upper()}" + (f"_{wm}" if kind == "u8" else "") + ("_ACC" if accum else "")
-                yield name, kind, wm, accum
+    for kind in ("u8", "i8", "bf16"):
+        for accum in (False, True):
+            yield f"GEMM_WIDE_{kind.upper()}" + ("_ACC" if accum else ""), kind, accum
 
 
 def main():
     out_path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "gemm_wide_gfx950.inc")
     if len(sys.argv) > 1:
         out_path = sys.argv[1]
+    # Experiment switches (timing builds with one ingredient left out, the cycle-stamp build): a
+    # comma-separated list in MRL_WIDE_OPTS.  The library is built with none.
+    opts = {o: True for o in os.environ.get("MRL_WIDE_OPTS", "").split(",") if o}
+    for o in list(opts):
+        if o.startswith("st_"):       # st_nt, st_sc1, st_sc0_sc1: cache policy bits on the stores of C
+            opts["st_flags"] = " " + " ".join(o.split("_")[1:])
     parts = ["// Generated by gen_gemm_wide.py -- do not edit; the generator documents the schedule.\n",
              f"#define GEMM_WIDE_MIN_STEPS {MIN_STEPS}\n"]
-    for name, kind, wm, accum in variants():
-        lines = gen(kind, wm, accum)
+    for name, kind, accum in variants():
+        lines = gen(kind, accum, opts)
         body = " \\\n".join('  "' + l + '\\n"' for l in lines)
         parts.append(f"#define {name} \\\n{body}\n")
     with open(out_path, "w") as f:
