@@ -266,6 +266,148 @@ def device_name():
 MIN_REPEATS = 10
 
 
+class Sensors:
+    """Socket power and shader clock of GPU 0 as the kernel driver reports them (hwmon
+    power1_input in microwatts; the starred line of pp_dpm_sclk), sampled from a host thread."""
+
+    def __init__(self, period_s=0.01):
+        import glob
+        import threading
+        dev = "/sys/class/drm/card0/device"
+        power = sorted(glob.glob(dev + "/hwmon/hwmon*/power1_input")) + sorted(glob.glob(dev + "/hwmon/hwmon*/power1_average"))
+        self.power_path = power[0] if power else None
+        self.sclk_path = dev + "/pp_dpm_sclk"
+        self.period_s, self.samples, self.phase, self.stop = period_s, [], None, False
+        self.thread = threading.Thread(target=self._run, daemon=True)
+        self.thread.start()
+
+    def _read(self):
+        watts = mhz = None
+        try:
+            with open(self.power_path) as f:
+                watts = int(f.read()) / 1e6
+        except (OSError, TypeError, ValueError):
+            pass
+        try:
+            with open(self.sclk_path) as f:
+                for line in f:
+                    if "*" in line:
+                        mhz = float(line.split(":")[1].lower().replace("mhz", "").replace("*", "").strip())
+        except (OSError, ValueError, IndexError):
+            pass
+        return watts, mhz
+
+    def _run(self):
+        while not self.stop:
+            if self.phase is not None:
+                self.samples.append((self.phase, time.perf_counter()) + self._read())
+            time.sleep(self.period_s)
+
+    def summary(self, phase, skip_s=0.3):
+        """Mean / min / max over the phase's samples, the first skip_s seconds left out."""
+        rows = [r for r in self.samples if r[0] == phase]
+        if not rows:
+            return None
+        rows = [r for r in rows if r[1] - rows[0][1] >= skip_s] or rows
+        out = {"samples": len(rows)}
+        for key, col in (("watts", 2), ("sclk_mhz", 3)):
+            vals = [r[col] for r in rows if r[col] is not None]
+            out[key] = {"mean": sum(vals) / len(vals), "min": min(vals), "max": max(vals)} if vals else None
+        return out
+
+
+def power_trace(seconds):
+    """Socket power and shader clock while idle, during a sustained run of the metric workload
+    (C2) and during the matrix-core rate probe on zero and on random operands: the record behind
+    the statement that the board's power limit, not its 2.4 GHz, bounds the matrix cores."""
+    desc, spec, arrs, *_ = workload("c2")
+    bufs = [M.DeviceBuffer.from_numpy(a) for a in arrs]
+    ptrs = [b.ptr for b in bufs]
+    sens = Sensors()
+    out = {"workload": desc, "seconds_per_phase": seconds, "sensor_period_s": sens.period_s,
+           "sensors": {"power": sens.power_path, "sclk": sens.sclk_path}}
+    M.synchronize()
+    sens.phase = "idle"
+    time.sleep(seconds)
+    sens.phase = None
+    out["idle"] = sens.summary("idle", 0.0)
+
+    t0, launches, gpu_ms, last = time.perf_counter(), 0, 0.0, 0.0
+    sens.phase = "c2"
+    while time.perf_counter() - t0 < seconds:
+        last = spec.run_timed(ptrs, 200)
+        gpu_ms, launches = gpu_ms + last, launches + 200
+    M.synchronize()
+    sens.phase = None
+    ops = spec.flops()
+    out["c2"] = sens.summary("c2")
+    out["c2"].update({"launches": launches, "us_per_launch_mean": gpu_ms / launches * 1e3,
+                      "us_per_launch_last_200": last / 200 * 1e3, "tops_last_200": ops / (last / 200 * 1e-3) / 1e12})
+    for phase, rand in (("mfma_zero_operands", False), ("mfma_random_operands", True)):
+        t0, rates = time.perf_counter(), []
+        sens.phase = phase
+        while time.perf_counter() - t0 < seconds:
+            rates.append(M.measure_mfma_rate("int8", rand, 200000) / 1e12)
+        sens.phase = None
+        out[phase] = sens.summary(phase)
+        out[phase].update({"tops_mean": sum(rates) / len(rates), "tops_last": rates[-1], "probe_runs": len(rates),
+                           "clock_mhz_implied": rates[-1] / PEAK["int8"] * 2400.0})
+    sens.stop = True
+    for b in bufs:
+        b.free()
+    return out
+
+
+def cycle_stamps(launches):
+    """Reads the stamps a timing build of the wide Matmul kernel (the library built with
+    MRL_WIDE_OPTS=trace in the environment) leaves in the first rows of every wave's block of C:
+    shader-clock cycles of the prologue, the k steps, the epilogue, the waits at barriers, and
+    the 100 MHz real-time clock at both ends, which together give the clock the kernel ran at."""
+    m = k = n = 4096
+    desc, spec, arrs, *_ = workload("c2")
+    bufs = [M.DeviceBuffer.from_numpy(a) for a in arrs]
+    ptrs = [b.ptr for b in bufs]
+    spec.run_timed(ptrs, launches)
+    M.synchronize()
+    us = spec.run_timed(ptrs, 20) / 20 * 1e3
+    M.synchronize()
+    c = bufs[2].to_numpy(np.int32, (m, n)).view(np.uint32)
+    names = ["T0", "T1", "T2", "T3", "T4", "T5", "R0", "R5", "Wvm", "Wbar", "HWID", "XCC"]
+    v = {}
+    # wave (wm, wn) of tile (tm, tn): value j at row j % 4, column 16 * (j / 4) of its block; the
+    # lower wave row's block columns are numbered from the fifth on
+    rows = (np.arange(16)[:, None] * 256 + np.arange(2)[None, :] * 128).reshape(-1)
+    cols = (np.arange(16)[:, None] * 256 + np.arange(2)[None, :] * 128).reshape(-1)
+    for j, nm in enumerate(names):
+        sub = c[np.ix_(rows + j % 4, cols + 16 * (j // 4))].astype(np.int64)
+        sub_rot = c[np.ix_(rows + j % 4, cols + 16 * (j // 4) + 64)].astype(np.int64)
+        lower = (np.arange(32) % 2 == 1)[:, None]
+        v[nm] = np.where(lower, sub_rot, sub).reshape(-1)
+    d = lambda a, b: (v[a] - v[b]) & 0xffffffff
+    stat = lambda x: {"median": float(np.median(x)), "min": float(x.min()), "max": float(x.max())}
+    tot, ticks = d("T5", "T0"), d("R5", "R0")
+    if int(np.median(tot)) == 0 or int(ticks.min()) == 0:
+        raise SystemExit("no stamps in C: build the library with MRL_WIDE_OPTS=trace for this mode")
+    unrolled = 10   # the accumulating kernel's unrolled steps (the first eight load C's old values)
+    out = {"workload": desc, "launches_before": launches, "us_per_launch_last_20": us,
+           "wave_cycles": stat(tot), "wave_100mhz_ticks": stat(ticks), "shader_clock_mhz": stat(tot / ticks * 100.0),
+           "prologue_cycles": stat(d("T1", "T0")),
+           "cycles_per_step_first_10": stat(d("T2", "T1") / unrolled),
+           "cycles_per_step_last_22": stat(d("T3", "T2") / (32 - unrolled)),
+           "epilogue_store_issue_cycles": stat(d("T4", "T3")), "epilogue_drain_cycles": stat(d("T5", "T4")),
+           "cycles_waiting_for_memory_at_barriers": stat(v["Wvm"]), "cycles_in_barriers": stat(v["Wbar"]),
+           "launch_span_us": float(v["R5"].max() - v["R0"].min()) / 100.0,
+           "mfma_cycles_per_step_at_full_rate": 128 * 16}
+    xcc = v["XCC"] & 0xf
+    out["per_xcd"] = {str(x): {"waves": int((xcc == x).sum()),
+                               "epilogue_store_issue_cycles_median": float(np.median(d("T4", "T3")[xcc == x])),
+                               "end_us_after_first_wave_end_median": float(np.median((v["R5"] - v["R5"].min())[xcc == x])) / 100.0}
+                      for x in sorted(set(xcc.tolist()))}
+    for b in bufs:
+        b.free()
+    return out
+
+
 def measure(name, steps, warmup, min_gpu_s):
     """W warm-up launches, then bursts of `steps` launches until there are MIN_REPEATS of them and
     min_gpu_s seconds of GPU time; -> the workload and the figures of the fastest and the last burst."""
@@ -330,6 +472,12 @@ def main():
     ap.add_argument("--vendor-ref", action="store_true",
                     help="also time the vendor library's nearest operation through PyTorch (c2, c3, c5)")
     ap.add_argument("--vendor-child", action="store_true", help=argparse.SUPPRESS)
+    ap.add_argument("--power-trace", type=float, default=0.0, metavar="SECONDS",
+                    help="instead of the benchmark: socket power and shader clock while idle, under C2 and under "
+                         "the matrix-core rate probe, SECONDS each")
+    ap.add_argument("--cycle-stamps", type=int, default=0, metavar="LAUNCHES",
+                    help="instead of the benchmark: read the cycle stamps of a timing build of the C2 kernel "
+                         "(MRL_WIDE_OPTS=trace python -m morello_amd.build) after LAUNCHES launches")
     args = ap.parse_args()
     if args.vendor_child:
         # PyTorch brings its own HIP runtime, which cannot share a process with the library's:
@@ -341,6 +489,12 @@ def main():
                          "(Matmul/Conv/Compose tiles shard without communication); run with --gpus 1")
 
     M.init(0)
+    if args.power_trace > 0:
+        print(json.dumps(power_trace(args.power_trace)))
+        return
+    if args.cycle_stamps > 0:
+        print(json.dumps(cycle_stamps(args.cycle_stamps)))
+        return
     head = measure(args.spec, args.steps, args.warmup, min_gpu_s=0.2)
     desc, spec, arrs, dtype, unit = head["desc"], head["spec"], head["arrs"], head["dtype"], head["unit"]
     value, ms_per_step, roofline = head["value"], head["ms_per_step"], head["roofline"]

@@ -56,7 +56,7 @@ constexpr int WIDE_MIN_STEPS = GEMM_WIDE_MIN_STEPS;
       MRL_WIDE_FIRST_100("a"), MRL_WIDE_100("a", 1), MRL_WIDE_10("a", 20), MRL_WIDE_10("a", 21),            \
       MRL_WIDE_10("a", 22), MRL_WIDE_10("a", 23), MRL_WIDE_10("a", 24), "a250", "a251", "a252", "a253",     \
       "a254", "a255", "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71",   \
-      "s72", "s73", "s78", "s79", "s80", "s81", "s82", "s83", "s84", "s85", "s86", "s87", "s88", "s89", "s90",     \
+      "s72", "s73", "s74", "s78", "s79", "s80", "s81", "s82", "s83", "s84", "s85", "s86", "s87", "s88", "s89", "s90",     \
       "s91", "s92", "s93", "s94", "s95", "scc", "memory"
 
 #define MRL_WIDE_RUN(TEXT)                                                                                         \
@@ -77,7 +77,7 @@ constexpr int WIDE_MIN_STEPS = GEMM_WIDE_MIN_STEPS;
                : MRL_WIDE_CLOBBERS)
 
 // M, N multiples of 256; K an even number of k steps: GEMM_WIDE_MIN_STEPS at least for an accumulating
-// Spec (whose first sixteen steps carry the loads of C's old values), four otherwise; see wide_applicable().
+// Spec (whose first eight steps carry the loads of C's old values), four otherwise; see wide_applicable().
 template <class T, bool A_UNSIGNED>
 __global__ __launch_bounds__(256) void k_gemm_wide(GemmArgs g, int tiles_m, int tiles_n, int group_m) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -103,7 +103,11 @@ __global__ __launch_bounds__(256) void k_gemm_wide(GemmArgs g, int tiles_m, int 
   // that XCD's L2).
   int pid = blockIdx.x;
   const int ntiles = tiles_m * tiles_n;
+#ifdef MRL_WIDE_XCD_SWAP  // experiment: neighbouring XCDs exchange their blocks of tiles
+  if (ntiles % 8 == 0) pid = ((pid % 8) ^ 1) * (ntiles / 8) + pid / 8;
+#else
   if (ntiles % 8 == 0) pid = (pid % 8) * (ntiles / 8) + pid / 8;
+#endif
   const int group = pid / (group_m * tiles_n);
   const int first_m = group * group_m;
   const int gsz = min(tiles_m - first_m, group_m);
@@ -157,7 +161,7 @@ __global__ __launch_bounds__(256) void k_gemm_wide(GemmArgs g, int tiles_m, int 
     for (int t = 0; t < TN; t++) {
       const int tn = (t + rot) % TN;
       const int byte = (wn * WN + tn * 16 + (8 / ES) * (p % LANES_PER_ROW)) * ES;
-      b_rd[t] = lds0 + k * B_ROWB + wide_b_swizzle<T>(byte, k);
+      b_rd[t] = lds0 + WIDE_B_BASE + k * B_ROWB + wide_b_swizzle<T>(byte, k);
     }
   }
   // C: register i of a 16 x 16 block holds row 4 * (l / 16) + i, column l % 16.  The loop addresses
@@ -193,17 +197,19 @@ __global__ __launch_bounds__(256) void k_gemm_wide(GemmArgs g, int tiles_m, int 
 }
 
 // Whole tiles, an even number of k steps, offsets the loop's 32-bit arithmetic can hold.  An
-// accumulating Spec needs the steps that carry C's old values; another one may be as short as four
-// steps, and is taken that short when its tiles run in one round (measured against the eight-wave
-// tile, non-accumulating: int8 4096 x 512 x 4096 19.5 against 21.3 us, 3072 x 2048 x 3072 27.3 / 31.0,
-// bf16 4096 x 1024 x 4096 34.6 / 38.4; but 8192 x 768 x 8192, four rounds of tiles bound by the
-// write of C, 99.0 / 94.3: this kernel's stores are 64-byte row segments).
+// accumulating Spec needs the steps that carry C's old values (GEMM_WIDE_MIN_STEPS); another one
+// may be as short as four steps.  Below twenty steps the kernel is taken when its tiles run in one
+// round (measured against the eight-wave tile, non-accumulating: int8 4096 x 512 x 4096 19.5 against
+// 21.3 us, 3072 x 2048 x 3072 27.3 / 31.0, bf16 4096 x 1024 x 4096 34.6 / 38.4; but 8192 x 768 x 8192,
+// four rounds of tiles bound by the write of C, 99.0 / 94.3: this kernel's stores are 64-byte row
+// segments).
+constexpr int WIDE_LONG_K_STEPS = 20;
 inline bool wide_applicable(const GemmArgs &g, int elem_size) {
   const int64_t bk = 128 / elem_size;
-  const bool long_k = g.k >= WIDE_MIN_STEPS * bk;
+  const bool long_k = g.k >= WIDE_LONG_K_STEPS * bk;
   const bool one_round = uint64_t(g.m / 256) * (g.n / 256) * g.batch <= g_compute_units;
   return !g.b_kmajor && g.m % 256 == 0 && g.n % 256 == 0 && g.k % (2 * bk) == 0 &&
-         (long_k || (!g.accum && g.k >= 4 * bk && one_round)) &&
+         (long_k || (one_round && g.k >= (g.accum ? WIDE_MIN_STEPS : 4) * bk)) &&
          g.lda * elem_size * 256 < (int64_t(1) << 32) && g.ldb * elem_size * (bk + 1) < (int64_t(1) << 31) &&
          g.ldc * 4 * 32 < (int64_t(1) << 31);
 }

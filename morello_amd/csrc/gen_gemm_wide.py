@@ -38,9 +38,12 @@ free as long as both operands agree, and here both hold bytes 16 g .. 16 g + 15 
   * one barrier, three quarters through the step, preceded by the step's wait for memory:
     everything requested before this step began has landed; the next tile's first operands are
     read behind it;
-  * an accumulating Spec loads C's old values during the first sixteen steps, four blocks a step,
-    and adds them to the blocks' accumulators a step later, between two of a block's MFMAs, so
-    that the epilogue only stores.
+  * an accumulating Spec loads C's old values during the first eight steps, a block row a step,
+    and adds them to the blocks' accumulators a step later, clear of the blocks' own MFMAs, so
+    that the epilogue only stores.  These steps are unrolled (the additions name their
+    accumulators); the rest is a loop of six steps.  All of it together must stay well inside the
+    64 KB instruction cache: a body that does not fit is fetched anew by every launch, which cost
+    100 to 350 cycles a step when the unrolled steps numbered eighteen.
 
 Register map (all named in the clobber list of the asm statement):
   a[0:255]    accumulators, block (tm, tn) at 4 * (8 * tm + tn); register i of lane l holds row
@@ -48,13 +51,13 @@ Register map (all named in the clobber list of the asm statement):
   v[0:63]     A staging, set p chunk i at 32 * p + 4 * i; after the loop: values on their way to C
   v[64:95]    A operands, block row tm at 64 + 4 * tm; after the loop: the column sums' partials
   v[96:159]   B operands, set b block column tn at 96 + 32 * b + 4 * tn; after the loop: partials
-  v[160:167]  LDS address of the lane's B operand, per tn, in the slot being read
+  v[160:167]  LDS address of the lane's B operand, per tn, in the third slot (the first two are
+              reached from the kernel's %[b_rd] with the instruction's offset)
   v[168:175]  column sums of B (u8 correction), one per tn; after the loop: 128 * column sum
   v[176:177]  scratch
-  v[180:211]  old values of two times four blocks of C
+  v[180:211]  old values of a block row of C
   s[60:61] A tile pointer   s[62:63] B tile pointer   s64 loop counter   s67 index of the next
-  A tile to fetch, s68 of the next B tile   s71 byte offset of tile kt's B slot   s[72:73] C block row pointer
-  s65, s66, s69, s70, s[78:79] scratch
+  A tile to fetch, s68 of the next B tile   s[72:73] C block row pointer   s74 0x80808080   s69, s[78:79] scratch
 """
 import os
 import sys
@@ -70,8 +73,7 @@ SLABS = 2
 GAPS = SLABS * MF   # MFMAs per k step
 BARRIER_AT = 96     # the step's barrier comes before this MFMA (88, 100, 104: the same; 80: 1-2 % slower)
 GAP_SLOTS = 2       # instructions placed behind one MFMA before the next is due (2: 63.7 us at 4096^3 int8, 3: 64.5, 4: 65)
-C_STEPS = 16        # k steps that carry the loads of C's old values (16 registers a step)
-C_BLOCKS = 4        # blocks of C a step loads
+C_STEPS = 8         # k steps that carry the loads of C's old values: a block row (32 registers) a step
 
 
 def acc(tm, tn):
@@ -101,7 +103,7 @@ def bf(buf, tn, half=None, w=None):
 B_ADDR = 160    # v[160:167]
 COL_SUM = 168   # v[168:175]
 TMP0, TMP1 = 176, 177
-OLD_C = 180     # v[180:211]
+OLD_C = 180     # v[180:211]: the old values of one block row of C
 
 
 class Emitter:
@@ -153,6 +155,17 @@ class Emitter:
 
     def vm_need(self, reg):
         self.vm_wait_index(self.vm_producer.get(reg, -1))
+
+
+# Harmless instructions of each class for issue-cost experiments (v178, s90 are otherwise unused).
+FILLERS = {
+    "valu": "v_mov_b32 v178, v179",
+    "salu": "s_mov_b32 s90, s69",
+    "nop": "s_nop 0",
+    "lds": "ds_read_b32 v178, %[a_rd0]",
+    "vmem": "global_load_dword v178, %[a_off0], s[60:61]",
+    "wait": "s_waitcnt lgkmcnt(15)",
+}
 
 
 class Item:
@@ -213,33 +226,35 @@ def gen(kind, accum, opts=None):
         advance("s62", "s63", "s68", "%[bstep]", "s69")
 
     def load_a(p, i):
-        if opts.get("no_stage"):
+        if opts.get("no_stage") or step_no[0] > int(opts.get("stage_until", 1 << 30)):
             return
         e.vm(f"global_load_dwordx4 {areg(p, i)}, %[a_off{i}], s[60:61]", dst=areg(p, i))
 
     def flip_a(p, i, words):
         """u8 -> i8 (a - 128) of two of the chunk's four registers."""
-        if opts.get("no_stage"):
+        if opts.get("no_stage") or step_no[0] > int(opts.get("stage_until", 1 << 30)):
             return
         e.vm_need(areg(p, i))
         for w in words:
-            E(f"v_xor_b32 {areg(p, i, w)}, 0x80808080, {areg(p, i, w)}")
+            E(f"v_xor_b32 {areg(p, i, w)}, s74, {areg(p, i, w)}")
 
     def store_a(p, i, stage, flip=True):
-        if opts.get("no_stage"):
+        if opts.get("no_stage") or step_no[0] > int(opts.get("stage_until", 1 << 30)):
             return
         e.vm_need(areg(p, i))
         if unsigned and flip:
             for w in range(4):
-                E(f"v_xor_b32 {areg(p, i, w)}, 0x80808080, {areg(p, i, w)}")
+                E(f"v_xor_b32 {areg(p, i, w)}, s74, {areg(p, i, w)}")
         e.lds_write(f"ds_write_b128 %[a_wr], {areg(p, i)} offset:{stage * A_STAGE + i * 4096}")
 
-    def set_m0(base_sgpr):
-        E(f"s_add_u32 m0, {base_sgpr}, 4096")   # the immediate offsets run from -4096 to 3072
-        E("s_nop 0")                              # one wait state before M0 is read
+    def set_m0(slot):
+        E(f"s_add_u32 m0, %[dma_base], {slot * B_SLOT + 4096}")   # the immediate offsets run from -4096 to 3072
+        E("s_nop 0")                                                # one wait state before M0 is read
+
+    step_no = [0]        # steps written so far (the rolled loop counts as late)
 
     def dma_b(j):
-        if opts.get("no_dma"):
+        if opts.get("no_dma") or step_no[0] > int(opts.get("dma_until", 1 << 30)):
             return
         e.vm(f"global_load_lds_dwordx4 %[b_off{j}], s[62:63] offset:{j * 1024 - 4096}")
 
@@ -248,30 +263,31 @@ def gen(kind, accum, opts=None):
             return lambda: None
         return lambda: e.lds_read(af(tm), f"ds_read_b128 {af(tm)}, %[a_rd{slab}] offset:{stage * A_STAGE + tm * 2048}")
 
-    def b_read(slab, buf, tn, half):
+    def b_read(slot, slab, buf, tn, half):
+        """The slot is known when the code is written (the loop body is six steps long: two A
+        stages x three B slots), so the whole address is a register plus an immediate: %[b_rd] is
+        the lane's address in slot 0 and reaches slot 1 with the 16-bit offset, v[160:167] the
+        same in slot 2."""
         reg = bf(buf, tn, half)
         if opts.get("no_reads"):
             return lambda: None
-        return lambda: e.lds_read(reg, f"{tr} {reg}, v{B_ADDR + tn} offset:{slab * SLAB_BYTES + half * HI_BYTES}")
-
-    def set_b_read_base(slot_off_sgpr):
-        for tn in range(TN):
-            E(f"v_add_u32 v{B_ADDR + tn}, {slot_off_sgpr}, %[b_rd{tn}]")
+        base = f"%[b_rd{tn}]" if slot < 2 else f"v{B_ADDR + tn}"
+        off = (slot % 2) * B_SLOT + slab * SLAB_BYTES + half * HI_BYTES
+        return lambda: e.lds_read(reg, f"{tr} {reg}, {base} offset:{off}")
 
     # ---- prologue -------------------------------------------------------------------------
+    E("s_mov_b32 s74, 0x80808080")      # in a register: a literal would double the size of every xor
     E("s_mov_b64 s[60:61], %[abase]")
     E("s_mov_b64 s[62:63], %[bbase]")
     E("s_mov_b32 s67, 0")
     E("s_mov_b32 s68, 0")
-    E("s_mov_b32 s71, 0")
     # A tiles 0 and 1 into the two register sets, B tiles 0 and 1 into slots 0 and 1
     for p in range(2):
         for i in range(8):
             load_a(p, i)
         advance_a()
     for slot in range(2):
-        E(f"s_add_u32 s66, %[dma_base], {slot * B_SLOT}")
-        set_m0("s66")
+        set_m0(slot)
         for j in range(8):
             dma_b(j)
         advance_b()
@@ -286,20 +302,23 @@ def gen(kind, accum, opts=None):
     E("s_waitcnt lgkmcnt(0)")
     e.all_lds_done()
     E("s_barrier")
-    E(f"s_mov_b32 s65, {B_BASE}")
-    set_b_read_base("s65")
+    for tn in range(TN):
+        E(f"v_add_u32 v{B_ADDR + tn}, {2 * B_SLOT}, %[b_rd{tn}]")
     # What a step expects to find: slab 0's B operands in set 0 and its A operands but the last,
     # which every step reads behind its first MFMA.
     for tn in range(TN):
-        b_read(0, 0, tn, 0)()
-        b_read(0, 0, tn, 1)()
+        b_read(0, 0, 0, tn, 0)()
+        b_read(0, 0, 0, tn, 1)()
     for tm in range(TM - 1):
         a_read(0, 0, tm)()
 
     # ---- one k step ----------------------------------------------------------------------
-    def step(cur, zero_first=False, extra=()):
-        """cur: LDS stage of tile kt.  zero_first: the accumulators start from zero in this step.
-        extra: Items to place in the gaps besides the step's own."""
+    def step(kt, zero_first=False, extra=()):
+        """kt: the step's position in the cycle of six (tile kt is in A stage kt % 2 and B slot
+        kt % 3).  zero_first: the accumulators start from zero in this step.  extra: Items to place
+        in the gaps besides the step's own."""
+        cur, slot = kt % 2, kt % 3
+        step_no[0] += 1
         p = cur ^ 1  # register set holding tile kt + 1 = LDS stage it goes to
         vm_before_step = e.vm_issued
         items = []
@@ -307,18 +326,6 @@ def gen(kind, accum, opts=None):
         def add(fn, cost, earliest, latest=GAPS - 1, after=None):
             items.append(Item(fn, cost, earliest, latest, after))
             return items[-1]
-
-        def header():
-            # s69: slot of tile kt + 1 (read after the barrier); s70: slot of tile kt + 2 (fetched now)
-            E(f"s_add_u32 s69, s71, {B_SLOT}")
-            E(f"s_cmp_eq_u32 s69, {3 * B_SLOT}")
-            E("s_cselect_b32 s69, 0, s69")
-            E(f"s_sub_u32 s70, s71, {B_SLOT}")
-            E("s_cmp_eq_u32 s71, 0")
-            E(f"s_cselect_b32 s70, {2 * B_SLOT}, s70")
-            E("s_add_u32 s66, %[dma_base], s70")
-            E(f"s_add_u32 s65, s69, {B_BASE}")
-            E("s_mov_b32 s71, s69")
 
         # Operand reads: fixed places.  A's block row tm for the next slab right behind the last of
         # the eight MFMAs that use the current one (the last block row's lands in the next slab /
@@ -333,11 +340,11 @@ def gen(kind, accum, opts=None):
         for tm in range(TM):
             at(8 * tm + 8, a_read(cur, 1, tm))              # slab 1 (tm = 7: behind slab 1's first MFMA)
         for tn in range(TN):                                 # slab 1's B operands into set 1
-            at(2 + 6 * tn, b_read(1, 1, tn, 0))
-            at(3 + 6 * tn, b_read(1, 1, tn, 1))
+            at(2 + 6 * tn, b_read(slot, 1, 1, tn, 0))
+            at(3 + 6 * tn, b_read(slot, 1, 1, tn, 1))
         for tn in range(TN):                                 # the next tile's slab 0 into set 0
-            at(BARRIER_AT + 3 * tn, b_read(0, 0, tn, 0))
-            at(BARRIER_AT + 1 + 3 * tn, b_read(0, 0, tn, 1))
+            at(BARRIER_AT + 3 * tn, b_read((slot + 1) % 3, 0, 0, tn, 0))
+            at(BARRIER_AT + 1 + 3 * tn, b_read((slot + 1) % 3, 0, 0, tn, 1))
         for tm in range(TM - 1):                             # and its A operands as theirs go dead
             at(max(MF + 8 * tm + 8, BARRIER_AT + 2 + 3 * tm), a_read(cur ^ 1, 0, tm))
 
@@ -348,7 +355,7 @@ def gen(kind, accum, opts=None):
                 last_a = add(lambda i=i: flip_a(p, i, (0, 1)), 2, g, BARRIER_AT - 4, after=last_a)
                 last_a = add(lambda i=i: flip_a(p, i, (2, 3)), 2, g, BARRIER_AT - 3, after=last_a)
             last_a = add(lambda i=i: (store_a(p, i, cur ^ 1, flip=False), load_a(p, i)), 2, g, BARRIER_AT - 2, after=last_a)
-        m0 = add(lambda: set_m0("s66"), 2, 0)
+        m0 = add(lambda: set_m0((slot + 2) % 3), 2, 0)   # tile kt + 2 goes where tile kt - 1 was
         last_b = m0
         for j, g in enumerate([6, 17, 28, 39, 50, 61, 72, 83]):
             last_b = add(lambda j=j: dma_b(j), 1, g, after=last_b)
@@ -362,7 +369,7 @@ def gen(kind, accum, opts=None):
                     for w in range(4):
                         # after the first MFMA that waited for this operand, before the reads that overwrite it
                         add(lambda s=s, tn=tn, w=w: (e.need(bf(s, tn, w // 2)),
-                                                      E(f"v_xor_b32 v{TMP0}, 0x80808080, {bf(s, tn, w=w)}"),
+                                                      E(f"v_xor_b32 v{TMP0}, s74, {bf(s, tn, w=w)}"),
                                                       E(f"v_sad_u8 v{COL_SUM + tn}, v{TMP0}, 0, v{COL_SUM + tn}")),
                             2, MF * s + tn + 1, MF * s + MF - 1 if s == 0 else GAPS - 1)
         for it in extra:
@@ -401,9 +408,7 @@ def gen(kind, accum, opts=None):
                 E("s_mov_b32 s94, s86")
             E("s_barrier")
             stamp(88)
-            set_b_read_base("s65")
 
-        header()
         n = 0
         for s in range(SLABS):
             for tm in range(TM):
@@ -417,6 +422,11 @@ def gen(kind, accum, opts=None):
                         r()
                     for it in placed[n]:
                         it.fn()
+                    for kind_, text in FILLERS.items():   # timing experiments: fill_<kind>=<per step>
+                        per_step = int(opts.get("fill_" + kind_, 0))
+                        if per_step and (n * per_step) // GAPS != ((n + 1) * per_step) // GAPS:
+                            for _ in range(max(1, per_step // GAPS)):
+                                E(text)
                     n += 1
 
     # ---- C: register q = 0..255: block q / 4 (tm = block / 8, tn = block % 8), register i = q % 4,
@@ -445,51 +455,57 @@ def gen(kind, accum, opts=None):
         block = q // 4
         return block // TN, block % TN, q % 4
 
-    def old_reg(j, r):
-        return f"v{OLD_C + 16 * (j & 1) + r}"
-
-    def old_values(j):
-        """C's old values of blocks 4 j .. 4 j + 3 into bank j % 2 of the temporaries: one step before
-        they are added."""
+    def c_ops(j):
+        """Step j of an accumulating Spec: the old values of block row j - 1 (loaded a step ago) join
+        their accumulators, and behind each addition the same register is loaded with block row
+        j's.  An addition is three instructions (the accumulator out, the sum, back in); it keeps
+        clear of the block's own MFMAs (8 (j - 1) + tn in either slab): an MFMA's result is read
+        four MFMAs after it at the earliest, and a register written for the block's next MFMA has
+        other instructions between the write and that MFMA.  Spread over the whole step, one
+        every four MFMAs."""
         out = []
-        for r in range(16):
-            tm, tn, i = where(16 * j + r)
-            reg = old_reg(j, r)
+        for r in range(32):
+            tn, i = r // 4, r % 4
+            reg = f"v{OLD_C + r}"
+            g = 4 * r + 1
+            add_item = None
+            if 1 <= j <= C_STEPS:
+                q = 4 * (TN * (j - 1) + tn) + i
+                n0 = TN * (j - 1) + tn
+                zones = [(n0 - 2, n0 + 3), (MF + n0 - 2, MF + n0 + 3)]
+                for lo, hi in zones:
+                    if lo <= g <= hi:
+                        g = hi + 1
+                if g > GAPS - 1:                      # the last block row's second zone reaches the step's end
+                    g = zones[1][0] - 4
+                latest = min([lo - 1 for lo, hi in zones if lo > g] + [GAPS - 1])
 
-            def ld(tm=tm, tn=tn, i=i, reg=reg):
-                c_ptr(tm)
-                e.vm(f"global_load_dword {reg}, {c_addr(tn, i)}, s[72:73] offset:{tn * 64}", dst=reg)
-            out.append(Item(ld, 1, 6 * r))
+                def rmw(q=q, reg=reg):
+                    e.vm_need(reg)
+                    E(f"v_accvgpr_read_b32 v{TMP1}, a{q}")
+                    E(f"v_add_f32 v{TMP1}, v{TMP1}, {reg}" if is_float else f"v_add_u32 v{TMP1}, v{TMP1}, {reg}")
+                    E(f"v_accvgpr_write_b32 a{q}, v{TMP1}")
+                add_item = Item(rmw, 3, g, latest)
+                out.append(add_item)
+            if j < C_STEPS:
+                def ld(tn=tn, i=i, reg=reg):
+                    c_ptr(j)
+                    e.vm(f"global_load_dword {reg}, {c_addr(tn, i)}, s[72:73] offset:{tn * 64}", dst=reg)
+                out.append(Item(ld, 1, g, GAPS - 1, after=add_item))
         return out
 
-    def add_old_values(j):
-        """The old values of blocks 4 j .. 4 j + 3 join their accumulators between a block's MFMA of
-        slab 0 and its MFMA of slab 1 (64 apart): an MFMA's result is read four MFMAs after it at
-        the earliest, and a register written for the block's next MFMA has other instructions
-        between the write and that MFMA."""
-        out = []
-        for r in range(16):
-            q = 16 * j + r
-            tm, tn, _ = where(q)
-            n0 = TN * tm + tn                    # the block's MFMA in slab 0
-            first, last = n0 + 4, n0 + MF - 4
-            reg = old_reg(j, r)
-
-            def rmw(q=q, reg=reg):
-                e.vm_need(reg)
-                E(f"v_accvgpr_read_b32 v{TMP1}, a{q}")
-                E(f"v_add_f32 v{TMP1}, v{TMP1}, {reg}" if is_float else f"v_add_u32 v{TMP1}, v{TMP1}, {reg}")
-                E(f"v_accvgpr_write_b32 a{q}, v{TMP1}")
-            out.append(Item(rmw, 3, min(last, first + 3 * (r % 4) + 12 * ((r // 4) % 2)), last))
-        return out
-
-    def loop():
-        E("1:")
-        step(0)
-        step(1)
-        E("s_sub_u32 s64, s64, 2")
-        E("s_cmp_lg_u32 s64, 0")
-        E("s_cbranch_scc1 1b")
+    def loop(first):
+        """Six steps, left after any two of them when the tiles run out; entered at position
+        `first` (the number of unrolled steps before it, modulo six)."""
+        if first % 6:
+            E(f"s_branch 1{first % 6}f")
+        for pos in (0, 2, 4):
+            E(f"1{pos}:")
+            step(pos)
+            step(pos + 1)
+            E("s_sub_u32 s64, s64, 2")
+            E("s_cmp_lg_u32 s64, 0")
+            E("s_cbranch_scc1 10b" if pos == 4 else "s_cbranch_scc0 2f")
 
     # ---- the k loop ---------------------------------------------------------------------------------
     if trace:
@@ -498,12 +514,8 @@ def gen(kind, accum, opts=None):
         e.all_lds_done()
     unrolled = C_STEPS + 2 if accum else 2
     for j in range(unrolled):
-        extra = []
-        if accum and j < C_STEPS and not opts.get("no_cops"):
-            extra += old_values(j)
-        if accum and 1 <= j <= C_STEPS and not opts.get("no_cops"):
-            extra += add_old_values(j - 1)
-        step(j & 1, zero_first=(j == 0), extra=extra)
+        extra = c_ops(j) if accum and not opts.get("no_cops") else []
+        step(j % 6, zero_first=(j == 0), extra=extra)
     if trace:
         stamp(84)
         E("s_waitcnt lgkmcnt(0)")
@@ -512,7 +524,7 @@ def gen(kind, accum, opts=None):
     E(f"s_sub_u32 s64, %[nk], {unrolled}")
     E("s_cmp_eq_u32 s64, 0")
     E("s_cbranch_scc1 2f")
-    loop()
+    loop(unrolled)
     E("2:")
     # nothing may land in LDS once the epilogue reuses it; the last MFMAs must have written the
     # accumulators before they are read
@@ -571,6 +583,7 @@ def gen(kind, accum, opts=None):
         stamp(86)
         E("s_memrealtime s[88:89]")
         E("s_getreg_b32 s90, hwreg(HW_REG_HW_ID)")
+        E("s_getreg_b32 s81, hwreg(HW_REG_XCC_ID)")
         E("s_waitcnt lgkmcnt(0)")
         ptr_tm[0] = None
         c_ptr(0)
@@ -599,7 +612,10 @@ def main():
     # comma-separated list in MRL_WIDE_OPTS.  The library is built with none.
     opts = {o: True for o in os.environ.get("MRL_WIDE_OPTS", "").split(",") if o}
     for o in list(opts):
-        if o.startswith("st_"):       # st_nt, st_sc1, st_sc0_sc1: cache policy bits on the stores of C
+        if "=" in o:                  # fill_valu=32 and the like
+            del opts[o]
+            opts[o.split("=")[0]] = o.split("=")[1]
+        elif o.startswith("st_"):       # st_nt, st_sc1, st_sc0_sc1: cache policy bits on the stores of C
             opts["st_flags"] = " " + " ".join(o.split("_")[1:])
     parts = ["// Generated by gen_gemm_wide.py -- do not edit; the generator documents the schedule.\n",
              f"#define GEMM_WIDE_MIN_STEPS {MIN_STEPS}\n"]

@@ -565,9 +565,9 @@ def test_the_four_wave_kernel_turns_down_other_shapes(gpu):
 
 
 @pytest.mark.parametrize("dts,codes", [((M.u8, M.i8, M.i32), [0, 1, 5]), ((M.bf16, M.bf16, M.f32), [7, 7, 6])])
-@pytest.mark.parametrize("steps", [4, 6, 14])
+@pytest.mark.parametrize("steps", [4, 6, 10])
 def test_the_four_wave_kernel_on_a_short_k(gpu, dts, codes, steps):
-    """A Spec that does not accumulate needs none of the sixteen k steps that carry C's old values:
+    """A Spec that does not accumulate needs none of the eight k steps that carry C's old values:
     the kernel takes it from four steps of 128 bytes on (the dispatch rules' own choice where the
     tiles run in one round); an accumulating Spec that short is turned down."""
     b, m, n = 1, 512, 768
@@ -596,3 +596,33 @@ def test_the_four_wave_kernel_on_a_short_k(gpu, dts, codes, steps):
     with pytest.raises(M.MorelloError) as e:
         M.MatmulAccum([b, m, k, n], dts).tile_out([1, 256, 256]).split(128 // es).staged(M.Staging.DirectBWide).plan()
     assert e.value.status == 1
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dts,codes", [((M.u8, M.i8, M.i32), [0, 1, 5]), ((M.bf16, M.bf16, M.f32), [7, 7, 6])])
+@pytest.mark.parametrize("steps", [12, 14, 16, 18, 20, 22, 24, 28])
+def test_the_four_wave_kernel_accumulating_over_every_loop_exit(gpu, dts, codes, steps):
+    """An accumulating Spec runs ten unrolled steps (the first eight load C's old values) and then a
+    loop of six that is entered at its fifth step and left after any two: every number of steps
+    modulo six, from the shortest K the kernel takes, against the oracle on a C that is not zero."""
+    b, m, n = 2, 256, 512
+    es = 2 if dts[0] == M.bf16 else 1
+    k = steps * 128 // es
+    if dts[0] == M.bf16:
+        A, Bm = synth.normal_bf16(97, 0, (b, m, k)), synth.normal_bf16(97, 1, (b, k, n))
+        C0 = synth.normal_f32(97, 2, (b, m, n), 30.0)
+    else:
+        A, Bm = synth.uniform_u8(97, 0, (b, m, k)), synth.uniform_i8(97, 1, (b, k, n))
+        C0 = (synth.uniform_i8(97, 2, (b, m, n)).astype(np.int32) * 1000003)
+    sched = M.MatmulAccum([b, m, k, n], dts).tile_out([1, 256, 256]).split(128 // es).staged(M.Staging.DirectBWide)
+    assert sched.plan().kernels == ["k_gemm_wide"]
+    want = orc.matmul([b, m, k, n], codes, A, Bm, C0.copy(), True)
+    bufs = [M.DeviceBuffer.from_numpy(x) for x in (A, Bm, C0)]
+    sched.run_device([x.ptr for x in bufs])
+    got = bufs[2].to_numpy(C0.dtype, (b, m, n))
+    for x in bufs:
+        x.free()
+    if dts[2] == M.i32:
+        assert np.array_equal(got, want)
+    else:
+        assert rel_err(got, want) < 1e-5
