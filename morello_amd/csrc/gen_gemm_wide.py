@@ -73,6 +73,7 @@ SLABS = 2
 GAPS = SLABS * MF   # MFMAs per k step
 BARRIER_AT = 96     # the step's barrier comes before this MFMA (88, 100, 104: the same; 80: 1-2 % slower)
 GAP_SLOTS = 2       # instructions placed behind one MFMA before the next is due (2: 63.7 us at 4096^3 int8, 3: 64.5, 4: 65)
+VALU_SLOTS = 2      # of which vector instructions
 C_STEPS = 8         # k steps that carry the loads of C's old values: a block row (32 registers) a step
 
 
@@ -103,6 +104,7 @@ def bf(buf, tn, half=None, w=None):
 B_ADDR = 160    # v[160:167]
 COL_SUM = 168   # v[168:175]
 TMP0, TMP1 = 176, 177
+C_TMP = (177, 178, 179)   # temporaries of the additions of C's old values
 OLD_C = 180     # v[180:211]: the old values of one block row of C
 
 
@@ -157,23 +159,26 @@ class Emitter:
         self.vm_wait_index(self.vm_producer.get(reg, -1))
 
 
-# Harmless instructions of each class for issue-cost experiments (v178, s90 are otherwise unused).
+# Instructions of each class for issue-cost experiments (timing only: v176 is the column sums' temporary).
 FILLERS = {
-    "valu": "v_mov_b32 v178, v179",
+    "valu": "v_mov_b32 v176, v176",
     "salu": "s_mov_b32 s90, s69",
     "nop": "s_nop 0",
-    "lds": "ds_read_b32 v178, %[a_rd0]",
-    "vmem": "global_load_dword v178, %[a_off0], s[60:61]",
+    "lds": "ds_read_b32 v176, %[a_rd0]",
+    "vmem": "global_load_dword v176, %[a_off0], s[60:61]",
     "wait": "s_waitcnt lgkmcnt(15)",
 }
 
 
 class Item:
     """A piece of work to place behind some MFMA of a step: fn emits it, cost is its instruction
-    count, earliest / latest the gaps (MFMA indices) it may go to, after an Item it follows."""
+    count, earliest / latest the gaps (MFMA indices) it may go to, after an Item it follows.
+    Measured on the bare loop (MFMAs and the barrier only): two vector instructions behind every
+    MFMA cost half a cycle each, a third one four cycles; two scalar instructions cost nothing."""
 
-    def __init__(self, fn, cost, earliest=0, latest=GAPS - 1, after=None):
+    def __init__(self, fn, cost, earliest=0, latest=GAPS - 1, after=None, valu=0):
         self.fn, self.cost, self.earliest, self.latest, self.after = fn, cost, earliest, latest, after
+        self.valu = valu     # how many of its instructions go to the vector unit (the matrix core's own port)
         self.gap = None
 
 
@@ -323,8 +328,8 @@ def gen(kind, accum, opts=None):
         vm_before_step = e.vm_issued
         items = []
 
-        def add(fn, cost, earliest, latest=GAPS - 1, after=None):
-            items.append(Item(fn, cost, earliest, latest, after))
+        def add(fn, cost, earliest, latest=GAPS - 1, after=None, valu=0):
+            items.append(Item(fn, cost, earliest, latest, after, valu))
             return items[-1]
 
         # Operand reads: fixed places.  A's block row tm for the next slab right behind the last of
@@ -352,15 +357,15 @@ def gen(kind, accum, opts=None):
         last_a = None
         for i, g in enumerate([1, 12, 23, 34, 45, 56, 67, 78]):
             if unsigned:   # in pieces that fit a gap
-                last_a = add(lambda i=i: flip_a(p, i, (0, 1)), 2, g, BARRIER_AT - 4, after=last_a)
-                last_a = add(lambda i=i: flip_a(p, i, (2, 3)), 2, g, BARRIER_AT - 3, after=last_a)
+                last_a = add(lambda i=i: flip_a(p, i, (0, 1)), 2, g, BARRIER_AT - 4, after=last_a, valu=2)
+                last_a = add(lambda i=i: flip_a(p, i, (2, 3)), 2, g, BARRIER_AT - 3, after=last_a, valu=2)
             last_a = add(lambda i=i: (store_a(p, i, cur ^ 1, flip=False), load_a(p, i)), 2, g, BARRIER_AT - 2, after=last_a)
-        m0 = add(lambda: set_m0((slot + 2) % 3), 2, 0)   # tile kt + 2 goes where tile kt - 1 was
+        m0 = add(lambda: set_m0((slot + 2) % 3), 1, 0)   # tile kt + 2 goes where tile kt - 1 was
         last_b = m0
         for j, g in enumerate([6, 17, 28, 39, 50, 61, 72, 83]):
             last_b = add(lambda j=j: dma_b(j), 1, g, after=last_b)
-        add(advance_a, 5, 84, after=last_a)
-        add(advance_b, 5, 88, after=last_b)
+        add(advance_a, 2, 84, after=last_a)          # scalar instructions: next to free
+        add(advance_b, 2, 88, after=last_b)
         if unsigned:
             # Block columns 0 .. 3 of both slabs: the other wave row, whose block columns are the
             # same columns rotated by four, adds up the other half.
@@ -371,26 +376,30 @@ def gen(kind, accum, opts=None):
                         add(lambda s=s, tn=tn, w=w: (e.need(bf(s, tn, w // 2)),
                                                       E(f"v_xor_b32 v{TMP0}, s74, {bf(s, tn, w=w)}"),
                                                       E(f"v_sad_u8 v{COL_SUM + tn}, v{TMP0}, 0, v{COL_SUM + tn}")),
-                            2, MF * s + tn + 1, MF * s + MF - 1 if s == 0 else GAPS - 1)
+                            2, MF * s + tn + 1, MF * s + MF - 1 if s == 0 else GAPS - 1, valu=2)
         for it in extra:
             items.append(it)
-        # Place the items in the order given, each into the first gap from its earliest on with room.
-        room = [GAP_SLOTS - len(read_at.get(g, [])) for g in range(GAPS)]
+        # Place the items in the order given, each into the first gap from its earliest on with room
+        # for it: GAP_SLOTS instructions behind an MFMA in all, VALU_SLOTS of them vector ones.
+        slots, vslots = int(opts.get("slots", GAP_SLOTS)), int(opts.get("valu", VALU_SLOTS))
+        room = [slots - len(read_at.get(g, [])) for g in range(GAPS)]
+        vroom = [vslots] * GAPS
         room[BARRIER_AT - 1] -= 3              # the waits and the barrier
         placed = [[] for _ in range(GAPS)]
         for it in items:
             first = max(it.earliest, it.after.gap if it.after is not None else 0)
             last_gap = max(first, it.latest)
             g = first
-            while g <= last_gap and room[g] < it.cost:
+            while g <= last_gap and (room[g] < it.cost or vroom[g] < it.valu):
                 g += 1
             if g > last_gap:               # no gap has room: the emptiest one allowed
-                g = max(range(first, last_gap + 1), key=lambda x: (room[x], -x))
+                g = max(range(first, last_gap + 1), key=lambda x: (min(room[x] - it.cost, vroom[x] - it.valu), -x))
             room[g] -= it.cost
+            vroom[g] -= it.valu
             it.gap = g
             placed[g].append(it)
         if os.environ.get("WIDE_SHOW_GAPS"):
-            sys.stderr.write("gaps " + " ".join(str(GAP_SLOTS - r) for r in room) + "\n")
+            sys.stderr.write("gaps " + " ".join(str(slots - r) for r in room) + "\n")
 
         def sync():
             # everything requested before this step has landed (B of tile kt + 1, A of tile kt + 2);
@@ -462,8 +471,8 @@ def gen(kind, accum, opts=None):
         clear of the block's own MFMAs (8 (j - 1) + tn in either slab): an MFMA's result is read
         four MFMAs after it at the earliest, and a register written for the block's next MFMA has
         other instructions between the write and that MFMA.  Spread over the whole step, one
-        every four MFMAs."""
-        out = []
+        every four MFMAs, its pieces behind three MFMAs in a row (three temporaries take turns)."""
+        out, chain = [], []
         for r in range(32):
             tn, i = r // 4, r % 4
             reg = f"v{OLD_C + r}"
@@ -473,20 +482,26 @@ def gen(kind, accum, opts=None):
                 q = 4 * (TN * (j - 1) + tn) + i
                 n0 = TN * (j - 1) + tn
                 zones = [(n0 - 2, n0 + 3), (MF + n0 - 2, MF + n0 + 3)]
-                for lo, hi in zones:
-                    if lo <= g <= hi:
+                for lo, hi in zones:               # three gaps in a row outside both zones
+                    if lo - 2 <= g <= hi:
                         g = hi + 1
-                if g > GAPS - 1:                      # the last block row's second zone reaches the step's end
-                    g = zones[1][0] - 4
+                if g + 2 > GAPS - 1:                  # the last block row's second zone reaches the step's end
+                    g = zones[1][0] - 6
                 latest = min([lo - 1 for lo, hi in zones if lo > g] + [GAPS - 1])
 
-                def rmw(q=q, reg=reg):
+                tmp = f"v{C_TMP[r % len(C_TMP)]}"
+                read = Item(lambda q=q, tmp=tmp: E(f"v_accvgpr_read_b32 {tmp}, a{q}"), 1, g, latest - 2,
+                            after=chain[-len(C_TMP)] if len(chain) >= len(C_TMP) else None, valu=1)
+
+                def add_old(tmp=tmp, reg=reg):
+                    # its own wait: the loads of a step are 32 KiB in flight per compute unit, which at
+                    # HBM's latency is all the chip can have of C, so the last of them arrive late
                     e.vm_need(reg)
-                    E(f"v_accvgpr_read_b32 v{TMP1}, a{q}")
-                    E(f"v_add_f32 v{TMP1}, v{TMP1}, {reg}" if is_float else f"v_add_u32 v{TMP1}, v{TMP1}, {reg}")
-                    E(f"v_accvgpr_write_b32 a{q}, v{TMP1}")
-                add_item = Item(rmw, 3, g, latest)
-                out.append(add_item)
+                    E(f"v_add_f32 {tmp}, {tmp}, {reg}" if is_float else f"v_add_u32 {tmp}, {tmp}, {reg}")
+                add_item = Item(add_old, 1, g + 1, latest - 1, after=read, valu=1)
+                write = Item(lambda q=q, tmp=tmp: E(f"v_accvgpr_write_b32 a{q}, {tmp}"), 1, g + 2, latest, after=add_item, valu=1)
+                chain.append(write)     # the temporary is free again behind this
+                out += [read, add_item, write]
             if j < C_STEPS:
                 def ld(tn=tn, i=i, reg=reg):
                     c_ptr(j)

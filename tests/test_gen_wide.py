@@ -53,6 +53,30 @@ def test_old_values_join_the_accumulators_clear_of_the_blocks_mfmas(kind):
 
 
 @pytest.mark.parametrize("kind", ["u8", "i8", "bf16"])
+def test_the_additions_temporaries_are_not_shared_by_two_additions_in_flight(kind):
+    """An addition is three instructions that may sit behind three different MFMAs; a temporary
+    holds one accumulator's value from the read to the write back, and nothing else writes it."""
+    holds = {}
+    for l in G.gen(kind, True):
+        m = re.match(r"v_accvgpr_read_b32 (v\d+), a(\d+)", l)
+        if m and int(m.group(1)[1:]) in G.C_TMP:
+            assert m.group(1) not in holds, l
+            holds[m.group(1)] = m.group(2)
+            continue
+        m = re.match(r"v_accvgpr_write_b32 a(\d+), (v\d+)", l)
+        if m and m.group(2) in holds:
+            assert holds.pop(m.group(2)) == m.group(1), l
+            continue
+        m = re.match(r"v_add_(u32|f32) (v\d+), (v\d+), v\d+", l)
+        if m and m.group(2) in holds:
+            assert m.group(3) == m.group(2), l
+            continue
+        for t in holds:      # no other instruction writes a temporary that is in use
+            assert not re.match(r"\S+ " + t + r"\b", l), l
+    assert not holds
+
+
+@pytest.mark.parametrize("kind", ["u8", "i8", "bf16"])
 @pytest.mark.parametrize("accum", [False, True])
 def test_every_step_issues_the_same_work(kind, accum):
     """Each of the steps moves one A tile and one B tile and reads 48 operands, wherever the
