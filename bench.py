@@ -316,7 +316,7 @@ class Sensors:
         return out
 
 
-def power_trace(seconds):
+def power_trace(seconds, phases=("idle", "c2", "mfma_zero_operands", "mfma_random_operands")):
     """Socket power and shader clock while idle, during a sustained run of the metric workload
     (C2) and during the matrix-core rate probe on zero and on random operands: the record behind
     the statement that the board's power limit, not its 2.4 GHz, bounds the matrix cores."""
@@ -327,23 +327,28 @@ def power_trace(seconds):
     out = {"workload": desc, "seconds_per_phase": seconds, "sensor_period_s": sens.period_s,
            "sensors": {"power": sens.power_path, "sclk": sens.sclk_path}}
     M.synchronize()
-    sens.phase = "idle"
-    time.sleep(seconds)
-    sens.phase = None
-    out["idle"] = sens.summary("idle", 0.0)
-
-    t0, launches, gpu_ms, last = time.perf_counter(), 0, 0.0, 0.0
-    sens.phase = "c2"
-    while time.perf_counter() - t0 < seconds:
-        last = spec.run_timed(ptrs, 200)
-        gpu_ms, launches = gpu_ms + last, launches + 200
-    M.synchronize()
-    sens.phase = None
-    ops = spec.flops()
-    out["c2"] = sens.summary("c2")
-    out["c2"].update({"launches": launches, "us_per_launch_mean": gpu_ms / launches * 1e3,
-                      "us_per_launch_last_200": last / 200 * 1e3, "tops_last_200": ops / (last / 200 * 1e-3) / 1e12})
+    if "idle" in phases:
+        sens.phase = "idle"
+        time.sleep(seconds)
+        sens.phase = None
+        out["idle"] = sens.summary("idle", 0.0)
+    if "c2" in phases:
+        t0, launches, gpu_ms, last = time.perf_counter(), 0, 0.0, 0.0
+        sens.phase = "c2"
+        while time.perf_counter() - t0 < seconds:
+            last = spec.run_timed(ptrs, 200)
+            gpu_ms, launches = gpu_ms + last, launches + 200
+        M.synchronize()
+        sens.phase = None
+        ops = spec.flops()
+        out["c2"] = sens.summary("c2")
+        us = gpu_ms / launches * 1e3
+        out["c2"].update({"launches": launches, "us_per_launch_mean": us, "us_per_launch_last_200": last / 200 * 1e3,
+                          "tops_last_200": ops / (last / 200 * 1e-3) / 1e12,
+                          "millijoule_per_launch": out["c2"]["watts"]["mean"] * us * 1e-3 if out["c2"]["watts"] else None})
     for phase, rand in (("mfma_zero_operands", False), ("mfma_random_operands", True)):
+        if phase not in phases:
+            continue
         t0, rates = time.perf_counter(), []
         sens.phase = phase
         while time.perf_counter() - t0 < seconds:
@@ -475,6 +480,8 @@ def main():
     ap.add_argument("--power-trace", type=float, default=0.0, metavar="SECONDS",
                     help="instead of the benchmark: socket power and shader clock while idle, under C2 and under "
                          "the matrix-core rate probe, SECONDS each")
+    ap.add_argument("--phases", default="idle,c2,mfma_zero_operands,mfma_random_operands",
+                    help="with --power-trace: which of idle, c2, mfma_zero_operands, mfma_random_operands to run")
     ap.add_argument("--cycle-stamps", type=int, default=0, metavar="LAUNCHES",
                     help="instead of the benchmark: read the cycle stamps of a timing build of the C2 kernel "
                          "(MRL_WIDE_OPTS=trace python -m morello_amd.build) after LAUNCHES launches")
@@ -490,7 +497,7 @@ def main():
 
     M.init(0)
     if args.power_trace > 0:
-        print(json.dumps(power_trace(args.power_trace)))
+        print(json.dumps(power_trace(args.power_trace, tuple(args.phases.split(",")))))
         return
     if args.cycle_stamps > 0:
         print(json.dumps(cycle_stamps(args.cycle_stamps)))

@@ -536,11 +536,26 @@ def gen(kind, accum, opts=None):
         E("s_waitcnt lgkmcnt(0)")
         e.all_lds_done()
         E("s_mov_b32 s83, s84")
-    E(f"s_sub_u32 s64, %[nk], {unrolled}")
+    early = int(opts.get("early_stores", 0))   # timing experiment (C2's 32 steps only): see below
+    E(f"s_sub_u32 s64, %[nk], {unrolled + (2 if early else 0)}")
     E("s_cmp_eq_u32 s64, 0")
     E("s_cbranch_scc1 2f")
     loop(unrolled)
     E("2:")
+    if early:
+        # An upper bound for what any reordering of the last step could hide of the epilogue: the
+        # first `early` stores of C go out spread over the last step's MFMAs, whether or not their
+        # accumulators are final (they are not: the results are wrong).
+        def early_store(q):
+            tm, tn, i = where(q)
+            c_ptr(tm)
+            t = f"v{OLD_C + q % 32}"
+            E(f"v_accvgpr_read_b32 {t}, a{q}")
+            if unsigned:
+                E(f"v_add_u32 {t}, {t}, v{COL_SUM + tn}")
+            E(f"global_store_dword {c_addr(tn, i)}, {t}, s[72:73] offset:{tn * 64}")
+        step(30 % 6)
+        step(31 % 6, extra=[Item(lambda q=q: early_store(q), 3, (q * GAPS) // early, GAPS - 1, valu=2) for q in range(early)])
     # nothing may land in LDS once the epilogue reuses it; the last MFMAs must have written the
     # accumulators before they are read
     E("s_waitcnt vmcnt(0) lgkmcnt(0)")
@@ -580,7 +595,7 @@ def gen(kind, accum, opts=None):
     if opts.get("no_epilogue"):
         pass
     else:
-        for q in range(256):
+        for q in range(early, 256):
             tm, tn, i = where(q)
             c_ptr(tm)
             if not unsigned:
