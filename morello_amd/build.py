@@ -43,7 +43,8 @@ def _hipcc() -> str:
 
 def _compile(src: str) -> str:
     obj = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
-    cmd = [_hipcc(), *FLAGS, *EXTRA_FLAGS.get(src, []), "-I", GEN_DIR, "-c", os.path.join(CSRC, src), "-o", obj]
+    # MRL_HIPCC_EXTRA: extra compiler arguments for one-off measurement builds (-D switches the kernels document)
+    cmd = [_hipcc(), *FLAGS, *EXTRA_FLAGS.get(src, []), *os.environ.get("MRL_HIPCC_EXTRA", "").split(), "-I", GEN_DIR, "-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)

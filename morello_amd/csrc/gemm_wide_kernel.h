@@ -115,8 +115,13 @@ __global__ __launch_bounds__(256) void k_gemm_wide(GemmArgs g, int tiles_m, int 
   const int tile_m = first_m + in_group % gsz, tile_n = in_group / gsz;
   const int64_t m0 = int64_t(tile_m) * BM, n0 = int64_t(tile_n) * BN;
 
+#ifdef MRL_WIDE_SAME_PANELS  // energy experiment: every workgroup fetches the first tile's operands (L2 hits)
+  const uint8_t *A = (const uint8_t *)g.a + (int64_t(blockIdx.y) * g.sa) * ES;
+  const uint8_t *B = (const uint8_t *)g.b + (int64_t(blockIdx.y) * g.sb) * ES;
+#else
   const uint8_t *A = (const uint8_t *)g.a + (int64_t(blockIdx.y) * g.sa + m0 * g.lda) * ES;
   const uint8_t *B = (const uint8_t *)g.b + (int64_t(blockIdx.y) * g.sb + n0) * ES;
+#endif
   Out *C = (Out *)g.c + int64_t(blockIdx.y) * g.sc + m0 * g.ldc + n0;
   const uint32_t lda_b = uint32_t(g.lda) * ES, ldb_b = uint32_t(g.ldb) * ES, ldc_b = uint32_t(g.ldc) * 4;
   const uint32_t lds0 = uint32_t(uintptr_t(lds));
