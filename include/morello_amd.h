@@ -491,7 +491,19 @@ int mrl_compose_plan(const mrl_compose *c, mrl_plan *plan, mrl_plan_step *steps,
  *                   tile_out([tile_m, tile_n]) on that Matmul
  *   UNFOLD          Conv: the windows materialised (a Move), then the Matmul
  *   BUFFERIZE       Compose: both intermediates materialised (bufferize.rs:24-116), a kernel per stage
- *   GENERIC         Conv on the any-dtype kernel */
+ *   GENERIC         Conv on the any-dtype kernel
+ *   TO_SOFTMAX_PARTS            Softmax (f32): SoftmaxDenominatorAndUnscaled into the output, then
+ *                               DivideVecScalar (scheduling/to_softmax_parts.rs:33-108)
+ *   TO_SOFTMAX_PARTS_RECOMPUTE  Softmax: SoftmaxDenominatorAndMax, then SoftmaxComplete
+ *                               (to_softmax_parts.rs:110-181)
+ *   PARALLEL_SOFTMAX            the same with the first stage split along the scan dim in `parts`
+ *                               equal tiles (row-major input), a (max, denominator) pair per tile,
+ *                               merged by SoftmaxDenominatorAndMaxFromParts
+ *                               (scheduling/parallel_softmax.rs:24-223)
+ * Each action is a terminal lowering: it runs the Spec to its result.  The reference's actions
+ * return a partial Impl whose nested sub-Specs a search expands further; the nested Specs of the
+ * three Softmax rewrites are the primitive Specs of this header, so a caller that wants to
+ * schedule a stage itself runs the stages one by one instead of the action. */
 typedef enum {
   MRL_ACTION_SELECT = 0,
   MRL_ACTION_TILE_OUT_SPLIT = 1,
@@ -499,13 +511,16 @@ typedef enum {
   MRL_ACTION_SPATIAL_SPLIT = 3,
   MRL_ACTION_UNFOLD = 4,
   MRL_ACTION_BUFFERIZE = 5,
-  MRL_ACTION_GENERIC = 6
+  MRL_ACTION_GENERIC = 6,
+  MRL_ACTION_TO_SOFTMAX_PARTS = 7,
+  MRL_ACTION_TO_SOFTMAX_PARTS_RECOMPUTE = 8,
+  MRL_ACTION_PARALLEL_SOFTMAX = 9
 } mrl_action_kind;
 typedef struct {
   int32_t kind;             /* mrl_action_kind */
   uint32_t tile_m, tile_n;  /* TILE_OUT_SPLIT, SPATIAL_SPLIT; FUSED on a Compose: tile_m = queries per workgroup */
   uint32_t split_k;         /* TILE_OUT_SPLIT: elements of K per step */
-  uint32_t parts;           /* FUSED on a Compose: shares of the keys */
+  uint32_t parts;           /* FUSED on a Compose: shares of the keys; PARALLEL_SOFTMAX: tiles along the scan dim */
   uint32_t staging;         /* TILE_OUT_SPLIT: mrl_staging */
   uint32_t n_steps;         /* filled by mrl_target_actions: launches, */
   uint64_t scratch_bytes;   /*   device scratch (Kernel::memory_allocated) */

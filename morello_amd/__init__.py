@@ -600,6 +600,9 @@ class ActionKind(enum.IntEnum):
     Unfold = 4
     Bufferize = 5
     Generic = 6
+    ToSoftmaxParts = 7
+    ToSoftmaxPartsRecompute = 8
+    ParallelSoftmax = 9
 
 
 class Action:
@@ -618,6 +621,7 @@ class Action:
         knobs = {ActionKind.TileOutSplit: f" tile {self.tile_m}x{self.tile_n} split {self.split_k}" + (f" {self.staging.name}" if self.staging else ""),
                  ActionKind.SpatialSplit: f" tile {self.tile_m}x{self.tile_n}",
                  ActionKind.Fused: (f" rows {self.tile_m}" if self.tile_m else "") + (f" parts {self.parts}" if self.parts else ""),
+                 ActionKind.ParallelSoftmax: f" parts {self.parts}",
                  }.get(self.kind, "")
         return f"Action({self.kind.name}{knobs}: {self.cost_ns:.0f} ns, {self.n_steps} launches, scratch {self.scratch_bytes} B)"
 

@@ -1752,11 +1752,98 @@ int mrl_matmul_search_schedule(const mrl_spec *spec, mrl_matmul_schedule *best, 
 // ---- actions: the lowerings a search may choose among (Target::actions, target/mod.rs:69) ----
 
 namespace {
+// A primitive of the Softmax decomposition as a stand-alone Spec over row-major tensors.
+int part_spec(int kind, const uint32_t *shape, uint32_t rank, uint32_t scan_dim, mrl_spec *s) {
+  std::memset(s, 0, sizeof *s);
+  s->kind = kind, s->scan_dim = scan_dim, s->rank = rank, s->n_params = expected_params(kind);
+  for (uint32_t d = 0; d < rank; d++) s->spec_shape[d] = shape[d];
+  for (uint32_t i = 0; i < s->n_params; i++) {
+    s->dtypes[i] = MRL_F32;
+    uint32_t pshape[MRL_MAX_RANK], prank;
+    if (parameter_shape(*s, i, pshape, &prank) != MRL_OK) return MRL_ERR_BAD_SPEC;
+    mrl_layout_row_major(pshape, prank, &s->layouts[i]);
+  }
+  return check_spec(s);
+}
+
+// A Softmax Spec through one of the reference's rewrites instead of the fused kernels, each stage
+// a primitive Spec of its own (parts.hip), the tensors between the stages in scratch memory:
+//   TO_SOFTMAX_PARTS            SoftmaxDenominatorAndUnscaled, then DivideVecScalar on the output
+//                               (scheduling/to_softmax_parts.rs:33-108)
+//   TO_SOFTMAX_PARTS_RECOMPUTE  SoftmaxDenominatorAndMax, then SoftmaxComplete, which forms the
+//                               exponentials a second time (to_softmax_parts.rs:110-181)
+//   PARALLEL_SOFTMAX            the same with the first stage split along the scan dim in `parts`
+//                               tiles (scheduling/parallel_softmax.rs:24-223): a (max, denominator)
+//                               pair per tile, merged by SoftmaxDenominatorAndMaxFromParts
+int run_softmax_rewrite(const mrl_spec &s, void *const *params, Workspace &ws, const mrl_action &a) {
+  if (s.kind != MRL_SPEC_SOFTMAX || s.dtypes[0] != MRL_F32 || s.dtypes[1] != MRL_F32) return MRL_ERR_UNSUPPORTED;
+  const uint32_t scan = s.spec_shape[s.scan_dim];
+  uint64_t lines = 1;
+  for (uint32_t d = 0; d < s.rank; d++)
+    if (d != s.scan_dim) lines *= s.spec_shape[d];
+  int rc;
+  mrl_spec st;
+  if (a.kind == MRL_ACTION_TO_SOFTMAX_PARTS) {
+    void *denom = nullptr;
+    HIP_TRY(ws.alloc(&denom, lines * sizeof(float)));
+    if ((rc = part_spec(MRL_SPEC_SOFTMAX_DENOMINATOR_AND_UNSCALED, s.spec_shape, s.rank, s.scan_dim, &st)) != MRL_OK) return rc;
+    st.layouts[0] = s.layouts[0], st.layouts[2] = s.layouts[1];
+    void *p1[3] = {params[0], denom, params[1]};
+    if ((rc = dispatch(st, p1, ws)) != MRL_OK) return rc;
+    if ((rc = part_spec(MRL_SPEC_DIVIDE_VEC_SCALAR, s.spec_shape, s.rank, s.scan_dim, &st)) != MRL_OK) return rc;
+    st.layouts[0] = s.layouts[1];
+    void *p2[2] = {params[1], denom};
+    return dispatch(st, p2, ws);
+  }
+  void *mx = nullptr, *denom = nullptr;
+  HIP_TRY(ws.alloc(&mx, lines * sizeof(float)));
+  HIP_TRY(ws.alloc(&denom, lines * sizeof(float)));
+  if (a.kind == MRL_ACTION_TO_SOFTMAX_PARTS_RECOMPUTE) {
+    if ((rc = part_spec(MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX, s.spec_shape, s.rank, s.scan_dim, &st)) != MRL_OK) return rc;
+    st.layouts[0] = s.layouts[0];
+    void *p1[3] = {params[0], mx, denom};
+    if ((rc = dispatch(st, p1, ws)) != MRL_OK) return rc;
+  } else {
+    // The tiles are a dim of their own: [.., scan, ..] read as [.., parts, scan / parts, ..], which
+    // is the same buffer when the input is row-major and the tiles are equal.
+    const uint32_t parts = a.parts;
+    int64_t strides[MRL_MAX_RANK], running = 1;
+    bool dense = mrl::layout_strides(s.layouts[0], s.spec_shape, s.rank, strides);
+    for (int d = int(s.rank) - 1; dense && d >= 0; d--) {
+      dense = s.spec_shape[d] == 1 || strides[d] == running;
+      running *= s.spec_shape[d];
+    }
+    if (parts < 2 || scan % parts != 0 || s.rank + 1 > MRL_MAX_RANK || !dense) return MRL_ERR_UNSUPPORTED;
+    uint32_t split[MRL_MAX_RANK], tiles[MRL_MAX_RANK];
+    for (uint32_t d = 0, o = 0; d < s.rank; d++) {
+      tiles[d] = d == s.scan_dim ? parts : s.spec_shape[d];
+      if (d == s.scan_dim) split[o++] = parts, split[o++] = scan / parts;
+      else split[o++] = s.spec_shape[d];
+    }
+    void *tile_max = nullptr, *tile_denom = nullptr;
+    HIP_TRY(ws.alloc(&tile_max, lines * parts * sizeof(float)));
+    HIP_TRY(ws.alloc(&tile_denom, lines * parts * sizeof(float)));
+    if ((rc = part_spec(MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX, split, s.rank + 1, s.scan_dim + 1, &st)) != MRL_OK) return rc;
+    void *p1[3] = {params[0], tile_max, tile_denom};
+    if ((rc = dispatch(st, p1, ws)) != MRL_OK) return rc;
+    if ((rc = part_spec(MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX_FROM_PARTS, tiles, s.rank, s.scan_dim, &st)) != MRL_OK) return rc;
+    void *p2[4] = {tile_max, tile_denom, mx, denom};
+    if ((rc = dispatch(st, p2, ws)) != MRL_OK) return rc;
+  }
+  if ((rc = part_spec(MRL_SPEC_SOFTMAX_COMPLETE, s.spec_shape, s.rank, s.scan_dim, &st)) != MRL_OK) return rc;
+  st.layouts[0] = s.layouts[0], st.layouts[3] = s.layouts[1];
+  void *p3[4] = {params[0], mx, denom, params[1]};
+  return dispatch(st, p3, ws);
+}
+
 // Runs `spec` under `action` through `ws` (a recording Workspace when planning).
 int dispatch_action(const mrl_spec &spec, void *const *params, Workspace &ws, const mrl_action &a) {
   Forced f;
   switch (a.kind) {
     case MRL_ACTION_SELECT: return dispatch(spec, params, ws);
+    case MRL_ACTION_TO_SOFTMAX_PARTS:
+    case MRL_ACTION_TO_SOFTMAX_PARTS_RECOMPUTE:
+    case MRL_ACTION_PARALLEL_SOFTMAX: return run_softmax_rewrite(spec, params, ws, a);
     case MRL_ACTION_TILE_OUT_SPLIT: {
       if (spec.kind != MRL_SPEC_MATMUL) return MRL_ERR_UNSUPPORTED;
       const mrl_matmul_schedule sched = {a.tile_m, a.tile_n, a.split_k, a.staging};
@@ -1771,6 +1858,10 @@ int dispatch_action(const mrl_spec &spec, void *const *params, Workspace &ws, co
     case MRL_ACTION_BUFFERIZE: f.msm_path = 2; break;
     default: return MRL_ERR_BAD_SPEC;
   }
+  // A Compose's key shares: what mrl_target_actions lists, one share or at least two blocks of 64 keys each.
+  if (a.kind == MRL_ACTION_FUSED && spec.kind == MRL_SPEC_COMPOSE_MSM && a.parts > 1 &&
+      (a.parts > 64 || 2 * uint64_t(a.parts) > (uint64_t(spec.spec_shape[3]) + 63) / 64))
+    return MRL_ERR_UNSUPPORTED;
   const bool conv_action = a.kind == MRL_ACTION_SPATIAL_SPLIT || a.kind == MRL_ACTION_UNFOLD || a.kind == MRL_ACTION_GENERIC;
   if ((conv_action && spec.kind != MRL_SPEC_CONV) || (a.kind == MRL_ACTION_BUFFERIZE && spec.kind != MRL_SPEC_COMPOSE_MSM) ||
       (a.kind == MRL_ACTION_FUSED && spec.kind != MRL_SPEC_CONV && spec.kind != MRL_SPEC_COMPOSE_MSM) ||
@@ -1830,6 +1921,13 @@ uint32_t mrl_target_actions(const mrl_spec *spec, mrl_action *out, uint32_t cap)
     for (uint32_t parts = 1; parts <= 64 && (parts == 1 || 2 * parts <= blocks); parts *= 2)
       for (uint32_t rows : {128u, 64u}) candidate(MRL_ACTION_FUSED, rows, 0, 0, parts);
     candidate(MRL_ACTION_BUFFERIZE);
+  } else if (spec->kind == MRL_SPEC_SOFTMAX) {
+    candidate(MRL_ACTION_TO_SOFTMAX_PARTS);
+    candidate(MRL_ACTION_TO_SOFTMAX_PARTS_RECOMPUTE);
+    // parallel_softmax.rs:60-66: a tile shorter than the scan dim; here equal tiles of 64 elements or more
+    const uint32_t scan = spec->spec_shape[spec->scan_dim];
+    for (uint32_t parts = 2; parts <= 64 && scan / parts >= 64; parts *= 2)
+      if (scan % parts == 0) candidate(MRL_ACTION_PARALLEL_SOFTMAX, 0, 0, 0, parts);
   }
   uint32_t n = 0;
   for (mrl_action &a : candidates) {

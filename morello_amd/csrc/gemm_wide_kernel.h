@@ -232,7 +232,7 @@ hipError_t launch_wide(const GemmArgs &g, hipStream_t stream) {
   plan::work(T::ES == 1 ? plan::UNIT_MFMA_I8 : plan::UNIT_MFMA_BF16, 2.0 * mn * g.k,
              (double(g.m) * g.k + double(g.k) * g.n) * g.batch * T::ES + mn * 4 * (g.accum ? 2 : 1),
              2.0 * 256 * 256 * double(g.k), 500.0 + 1200.0 * double(g.k * T::ES / 128),
-             T::ES == 1 ? 1.50 : 1.18);  // measured: 2150 TOPS int8 at 4096^3, 1360 TFLOPS bf16 at 8192^3
+             T::ES == 1 ? 1.62 : 1.18);  // measured: 2230-2330 TOPS int8 at 4096^3, 1360 TFLOPS bf16 at 8192^3
   MRL_LAUNCH((k_gemm_wide<T, A_UNSIGNED>), dim3(tiles_m * tiles_n, g.batch), dim3(256), WIDE_LDS_BYTES, stream, g,
              tiles_m, tiles_n, group_rows(tiles_m, tiles_n));
   return mrl::plan::last_error();

@@ -77,6 +77,44 @@ def test_compose_actions_against_the_oracle(gpu):
         assert rel_err(got, want) < 1e-2, act
 
 
+@pytest.mark.parametrize("shape,dim", [((64, 1024), 1), ((3, 50, 256), 2), ((7, 128, 33), 1), ((2, 4, 640, 5), 2), ((1000, 96), 1),
+                                       ((4096, 8), 0)])
+def test_softmax_actions_against_the_oracle(gpu, shape, dim):
+    """The reference's Softmax rewrites as actions (scheduling_sugar.rs:69-95: to_softmax_parts,
+    to_softmax_parts_recompute, and the latter with its first stage split along the scan dim,
+    parallel_softmax.rs:24): each runs its stages as primitive Specs and must give the Softmax."""
+    x = synth.normal_f32(35, 0, shape, 3.0)
+    want = orc.softmax(list(shape), dim, x)
+    spec = M.Softmax(list(shape), dim)
+    acts = spec.actions()
+    kinds = [a.kind for a in acts]
+    assert kinds[:3] == [M.ActionKind.Select, M.ActionKind.ToSoftmaxParts, M.ActionKind.ToSoftmaxPartsRecompute]
+    scan = shape[dim]
+    assert [a.parts for a in acts[3:]] == [p for p in (2, 4, 8, 16, 32, 64) if scan % p == 0 and scan // p >= 64]
+    assert all(a.kind == M.ActionKind.ParallelSoftmax for a in acts[3:])
+    for act in acts:
+        got = run_action(act, [x, np.full(shape, 9.0, np.float32)])
+        assert np.abs(got - want).max() < 1e-5, act
+        # one launch per stage: two stages, or three with the merge of the tiles' pairs
+        if act.kind != M.ActionKind.Select:
+            assert act.n_steps == (3 if act.kind == M.ActionKind.ParallelSoftmax else 2), act
+
+
+def test_softmax_actions_keep_the_parameters_layouts(gpu):
+    """Input and output in another layout than row-major: the whole-tensor rewrites take them as
+    they are, the tiled one (which reads the scan dim as two dims of the same buffer) declines."""
+    shape = (48, 320)
+    x = synth.normal_f32(36, 0, shape, 2.0)
+    want = orc.softmax(list(shape), 1, x)
+    cm = M.col_major(list(shape))
+    spec = M.Softmax(list(shape), 1, layouts=[cm, cm])
+    acts = spec.actions()
+    assert [a.kind for a in acts] == [M.ActionKind.Select, M.ActionKind.ToSoftmaxParts, M.ActionKind.ToSoftmaxPartsRecompute]
+    for act in acts:
+        got = run_action(act, [np.ascontiguousarray(x.T), np.zeros((shape[1], shape[0]), np.float32)])
+        assert np.abs(got.T - want).max() < 1e-5, act
+
+
 @pytest.mark.parametrize("dims", [(1, 136, 128, 1000, 128), (3, 200, 128, 70, 128), (2, 1, 128, 1, 128), (1, 257, 64, 65, 64),
                                   (2, 300, 32, 129, 32), (2, 70, 96, 333, 40)])
 def test_compose_query_blocks_on_ragged_shapes(gpu, dims):

@@ -345,6 +345,17 @@ def test_bf16_matmul_full_size_sample(gpu):
     spec_acc.run_device([dA.ptr, dB.ptr, dC.ptr])
     # the old value of an element enters its sum first or last depending on the kernel: one rounding apart
     assert rel_err(dC.to_numpy(np.float32, (m, n)), got * 2) < 1e-5
+    # The accumulating Spec on a C that is neither zero nor the product: bands against the oracle.
+    C0 = synth.normal_f32(61, 2, (1, m, n), 100.0)
+    dC.free()
+    dC = M.DeviceBuffer.from_numpy(C0)
+    spec_acc.run_device([dA.ptr, dB.ptr, dC.ptr])
+    got = dC.to_numpy(np.float32, (m, n))
+    for lo in (0, 2600, 8184):
+        want = C0.copy()
+        orc.matmul([1, m, k, n], [7, 7, 6], A, Bm, want, True, rows=(lo, lo + 8))
+        assert rel_err(got[lo:lo + 8], want[0, lo:lo + 8]) < 1e-4
+        assert elem_err(got[lo:lo + 8], want[0, lo:lo + 8]) < 1e-3
 
 
 def test_matmul_layouts(gpu):

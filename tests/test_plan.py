@@ -260,9 +260,10 @@ def _median_ms(run, ptrs, launches=20, repeats=5):
 @pytest.mark.gpu
 def test_cost_model_against_measured_launches(gpu):
     """Predicted against measured per-launch time on benchmark-like operands for the kernels the
-    benchmark configurations and their neighbours run.  The ratios are printed (the fit's own
-    spread is 0.6-1.5); what is asserted is a sanity bound a change of clock state cannot reach:
-    a model off by an order of magnitude."""
+    benchmark configurations and their neighbours run, each timing the median of five bursts on
+    settled clocks.  The ratios are printed (measured on these ten: 0.80-1.21); the model, which
+    ranks the lowerings that mrl_target_actions and mrl_matmul_search_schedule offer, is held to
+    a factor of two either way for every kernel family here."""
     rng = np.random.default_rng(7)
     specs = [c2(), c4(), c5(), M.Matmul([1, 2048, 2048, 2048], (M.bf16, M.bf16, M.f32)),
              M.Matmul([1, 1024, 1024, 1024], (M.f32, M.f32, M.f32)), M.Softmax([16, 2048, 2048], 2),
@@ -285,7 +286,7 @@ def test_cost_model_against_measured_launches(gpu):
             b.free()
         print(f"cost model: {spec.plan().kernels} predicted {predicted_ns / 1e3:.1f} us measured {measured_ns / 1e3:.1f} us "
               f"ratio {predicted_ns / measured_ns:.2f}")
-        assert 0.1 < predicted_ns / measured_ns < 10.0, (spec, predicted_ns, measured_ns)
+        assert 0.5 < predicted_ns / measured_ns < 2.0, (spec, predicted_ns, measured_ns)
 
 
 @pytest.mark.gpu
@@ -293,7 +294,7 @@ def test_cost_model_ranks_manual_schedules(gpu):
     """What a search over tile_out / split needs from the model is an order.  Only quantities
     measured in this run, one after the other on settled clocks, are compared: where the model
     puts two schedules a factor of two or more apart, the measured order must not be the reverse
-    by more than a quarter, and the schedule it calls cheapest runs within 3x of the fastest
+    by more than a quarter, and the schedule it calls cheapest runs within 2x of the fastest
     (measured: the fastest itself or within 1.15x; bf16 2048^3 1.4x)."""
     rng = np.random.default_rng(11)
     _settle_clocks()
@@ -315,11 +316,27 @@ def test_cost_model_ranks_manual_schedules(gpu):
             for b in bufs:
                 b.free()
             pick = min(predicted, key=predicted.get)
-            assert measured[pick] <= 3.0 * min(measured.values()), (dts[0], m, k, n, pick, measured)
+            assert measured[pick] <= 2.0 * min(measured.values()), (dts[0], m, k, n, pick, measured)
             for x in predicted:
                 for y in predicted:
                     if predicted[x] * 2.0 <= predicted[y]:
                         assert measured[x] <= 1.25 * measured[y], (dts[0], m, k, n, x, y, measured, predicted)
+
+
+def test_actions_of_a_softmax():
+    """Host only: the Softmax stage of C5 on its own lists the fused kernels' choice, the two
+    whole-row rewrites and the tiled one for every power-of-two tile count down to 64-element
+    tiles, each priced; the fused kernel (8 bytes an element) is the cheapest."""
+    K = M.ActionKind
+    acts = M.Softmax([16, 2048, 2048], 2).actions()
+    assert [a.kind for a in acts] == [K.Select, K.ToSoftmaxParts, K.ToSoftmaxPartsRecompute] + [K.ParallelSoftmax] * 5
+    assert [a.parts for a in acts[3:]] == [2, 4, 8, 16, 32]
+    assert acts[0].plan().kernels == ["k_softmax_regs"]
+    assert acts[1].plan().kernels == ["k_parts", "k_parts"] and acts[3].plan().kernels == ["k_parts"] * 3
+    assert all(a.cost_ns > acts[0].cost_ns for a in acts[1:])
+    assert acts[1].scratch_bytes >= 16 * 2048 * 4 and acts[3].scratch_bytes >= 16 * 2048 * 4 * (2 + 2 * 2)
+    # integers and other dtypes have no Softmax; a Matmul lists none of these
+    assert not {K.ToSoftmaxParts, K.ParallelSoftmax} & {a.kind for a in c2().actions()}
 
 
 def test_actions_of_the_benchmark_configurations():
@@ -363,7 +380,7 @@ def test_actions_of_the_benchmark_configurations():
     assert fused[2].scratch_bytes == 16 * 2048 * 2 * (128 + 4) * 4
     assert acts[0].cost_ns == fused[1].cost_ns == min(a.cost_ns for a in acts)
     # Specs with one lowering list it alone; what no kernel takes lists nothing it cannot run.
-    assert [a.kind for a in M.Softmax([16, 2048, 2048], 2).actions()] == [K.Select]
+    assert [a.kind for a in M.Move([64, 64], (M.f32, M.f32)).actions()] == [K.Select]
     odd = M.Conv([2, 3, 5, 6, 6, 2, 2], (M.i16, M.i16, M.i32)).actions()
     assert {a.kind for a in odd} == {K.Select, K.Generic}
     assert [a.kind for a in M.ComposeMSM(2, 64, 256, 128, 256, layouts=[None, None, KT, None]).actions()] == [K.Select, K.Bufferize]
