@@ -78,7 +78,12 @@ typedef enum {
   MRL_SPEC_CONV = 1,       /* spec_shape [b,f,c,oh,ow,fh,fw]; params image, filters, out.
                               Both: any dtype triple; inputs are cast to the output dtype
                               (verification.rs:547-569, 629-631), integer outputs wrap, f32
-                              outputs sum in f32, bf16 outputs sum in f32 and round once    */
+                              outputs sum in f32.  bf16 outputs: PARITY UNPINNED -- the
+                              products are summed in f32 and rounded once, and an accumulating
+                              Spec adds the old output before that single rounding; the
+                              reference's interpreter rounds to bf16 after every operation
+                              and again after `o += intermed` (verification.rs:629-642), and
+                              holds no comparison for bf16 (verification.rs:597 is todo!)    */
   MRL_SPEC_SOFTMAX = 2,    /* spec_shape = tensor shape; params in, out; uses scan_dim   */
   MRL_SPEC_COMPOSE_MSM = 3,/* Matmul->Softmax->Matmul; spec_shape [b,m,k,n2,n];
                               params V[b,n2,n] Q[b,m,k] KT[b,k,n2] out[b,m,n]
@@ -155,6 +160,13 @@ const char *mrl_status_string(int status);
 const char *mrl_last_error(void);
 /* "major.minor.patch" of this library. */
 const char *mrl_version(void);
+/* The layout of the structs of this header as the loaded library was built with them.  A binding
+ * compares it with the MRL_ABI_VERSION it was written against before it passes a struct: the
+ * number goes up whenever a struct gains or changes a field (2: mrl_matmul_schedule.staging,
+ * mrl_action; 3: the Softmax actions).  Every struct is zero-initialised by the caller before
+ * its fields are set: fields added later mean "default" when zero. */
+#define MRL_ABI_VERSION 3u
+uint32_t mrl_abi_version(void);
 
 /* --------------------------------------------------- Spec surface (host) */
 
@@ -221,9 +233,12 @@ int mrl_run_async(const mrl_spec *spec, void *const *params, void *stream);
  * programs allocate their buffers up front.  Calls no hipMalloc / hipFree / stream-ordered
  * allocator: scratch comes out of one fixed array of MRL_NOALLOC_SCRATCH_BYTES per GPU, which the
  * library's code object brings along (each GPU the library runs on holds it until the process
- * ends).  mrl_init must have been called for the device (it looks the array up).  A Spec whose
- * scratch need (mrl_spec_plan: scratch_bytes) exceeds the array is turned down with
- * MRL_ERR_TOO_LARGE before anything is launched.  All calls on one GPU share the array: two that
+ * ends).  mrl_init must have been called for the device (it looks the array up) and that device
+ * must be the calling thread's current one (MRL_ERR_NO_DEVICE otherwise).  Parameters are 256-byte
+ * aligned, as device allocations are (MRL_ERR_UNSUPPORTED otherwise: the scratch need of a
+ * misaligned call is not the plan's).  A Spec whose scratch need (mrl_spec_plan: scratch_bytes)
+ * exceeds the array is turned down with MRL_ERR_TOO_LARGE before anything is launched.  All calls
+ * on one GPU share the array: two that
  * overlap in time (different streams, or different host threads on one stream) race; the caller
  * serialises them. */
 #define MRL_NOALLOC_SCRATCH_BYTES (32u << 20)
@@ -272,6 +287,7 @@ typedef enum {
   MRL_STAGING_DIRECT_B = 2,       /* B: HBM -> LDS (3 slots); eight waves of 128 x 64 (k_gemm_big)  */
   MRL_STAGING_DIRECT_B_WIDE = 3   /* B: HBM -> LDS (3 slots); four waves of 128 x 128 (k_gemm_wide) */
 } mrl_staging;
+/* Zero-initialise before setting fields (staging was added after the first three). */
 typedef struct {
   uint32_t tile_m, tile_n; /* tile_out */
   uint32_t split_k;        /* split, in elements of K */

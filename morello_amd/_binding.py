@@ -12,6 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libmorello_amd.so")
 
 MAX_PHYS, MAX_RANK, MAX_SPEC_RANK, MAX_PARAMS = 10, 5, 7, 4
+ABI_VERSION = 3   # MRL_ABI_VERSION of include/morello_amd.h
 
 
 class PhysDimC(C.Structure):
@@ -139,6 +140,7 @@ SIGNATURES = {
     "mrl_stream_synchronize": (C.c_int, [C.c_void_p]),
     "mrl_stream_release": (C.c_int, [C.c_void_p]),
     "mrl_device_mem_free": (C.c_int, [C.POINTER(C.c_size_t)]),
+    "mrl_abi_version": (C.c_uint32, []),
     "mrl_stream_destroy": (C.c_int, [C.c_void_p]),
     "mrl_target_id": (C.c_char_p, []),
     "mrl_target_line_size": (C.c_uint32, []),
@@ -179,5 +181,8 @@ def load() -> C.CDLL:
         fn = getattr(lib, name)  # AttributeError if the ABI lost a symbol
         fn.restype = res
         fn.argtypes = args
+    if lib.mrl_abi_version() != ABI_VERSION:
+        raise ImportError(f"{LIB_PATH} has struct layout version {lib.mrl_abi_version()}, this binding is written "
+                          f"for {ABI_VERSION}: rebuild with `python -m morello_amd.build`")
     _lib = lib
     return lib

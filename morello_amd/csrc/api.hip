@@ -1247,9 +1247,11 @@ int mrl_init(int device) {
   }
   HIP_TRY(hipSetDevice(device));
   if (device < MAX_DEVICES && !g_scratch_ptr[device]) {
+    // This device's copy of the array.  A failure here only takes mrl_run_noalloc away (it finds
+    // no pointer and says so): every other entry point allocates what it needs.
     void *ptr = nullptr;
-    HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));  // this device's copy of the array
-    g_scratch_ptr[device] = ptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) == hipSuccess) g_scratch_ptr[device] = ptr;
+    else (void)hipGetLastError();
   }
   g_device = device;
   mrl::g_compute_units = prop.multiProcessorCount > 0 ? uint32_t(prop.multiProcessorCount) : 256u;
@@ -1272,6 +1274,8 @@ const char *mrl_status_string(int status) {
 
 const char *mrl_last_error(void) { return g_last_error.c_str(); }
 const char *mrl_version(void) { return "0.1.0"; }
+
+uint32_t mrl_abi_version(void) { return MRL_ABI_VERSION; }
 
 size_t mrl_dtype_size(int dtype) {
   switch (dtype) {
@@ -1545,11 +1549,27 @@ int mrl_run_noalloc(const mrl_spec *spec, void *const *params, void *stream) {
     g_last_error = "mrl_run_noalloc: call mrl_init first (it looks up the device's scratch array)";
     return MRL_ERR_NO_DEVICE;
   }
+  // The array belongs to the device mrl_init chose: a thread that has made another one current
+  // would hand its kernels a pointer of the wrong GPU.
+  int current = -1;
+  HIP_TRY(hipGetDevice(&current));
+  if (current != g_device) {
+    g_last_error = "mrl_run_noalloc: the calling thread's current device is " + std::to_string(current) +
+                   ", the library was initialised for device " + std::to_string(g_device);
+    return MRL_ERR_NO_DEVICE;
+  }
   int rc = check_spec(spec);
   if (rc != MRL_OK) return rc;
   if (!params) return MRL_ERR_NULL;
-  for (uint32_t i = 0; i < spec->n_params; i++)
+  for (uint32_t i = 0; i < spec->n_params; i++) {
     if (!params[i]) return MRL_ERR_NULL;
+    // The plan below assumes parameters aligned as device allocations are; others could take a
+    // path with a larger scratch need, found only after kernels have written to the outputs.
+    if (reinterpret_cast<uintptr_t>(params[i]) & 255) {
+      g_last_error = "mrl_run_noalloc: parameter " + std::to_string(i) + " is not 256-byte aligned";
+      return MRL_ERR_UNSUPPORTED;
+    }
+  }
   // What the call would take, from the plan (host arithmetic only), so that a Spec that does not
   // fit is turned down before anything is launched.
   mrl_plan plan;

@@ -28,6 +28,12 @@ def test_every_declared_symbol_is_exported_and_bound():
     assert set(B.SIGNATURES) <= set(names)
 
 
+def test_abi_version_of_library_header_and_binding_agree():
+    text = open(os.path.join(ROOT, "include", "morello_amd.h")).read()
+    declared = int(re.search(r"#define MRL_ABI_VERSION (\d+)u", text).group(1))
+    assert B.load().mrl_abi_version() == declared == B.ABI_VERSION
+
+
 def test_struct_sizes_match_the_header():
     # mrl_physdim {u8,u8,u32} = 8 bytes; mrl_layout = 4 + 10*8; mrl_spec as declared.
     assert C.sizeof(B.PhysDimC) == 8

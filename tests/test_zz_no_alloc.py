@@ -17,8 +17,11 @@ def both_ways(spec, arrays):
     """-> (output of mrl_run, output of mrl_run_noalloc) on fresh copies of `arrays`."""
     want = run_spec(spec, arrays)
     bufs = [M.DeviceBuffer.from_numpy(a) for a in arrays]
+    M.synchronize()
+    free_before = M.device_free_bytes()
     spec.run_noalloc([b.ptr for b in bufs])
     M.synchronize()
+    assert M.device_free_bytes() == free_before      # the call took no device memory
     got = bufs[-1].to_numpy(arrays[-1].dtype, arrays[-1].shape)
     for b in bufs:
         b.free()
@@ -42,6 +45,36 @@ def test_noalloc_matches_run_on_two_calls_in_a_row(gpu):
                   np.full((1, m, n), -1, np.int32)]
         want, got = both_ways(spec, arrays)
         assert np.array_equal(got, want)
+
+
+def test_noalloc_between_calls_that_use_the_arena(gpu):
+    """mrl_run_async (scratch from the stream's arena) between two mrl_run_noalloc calls (scratch
+    from the fixed array): neither disturbs the other."""
+    m, k, n = 384, 4096, 256
+    spec = M.MatmulAccum([1, m, k, n], (M.u8, M.i8, M.i32))
+    assert spec.plan().scratch_bytes > 0
+    a, b = synth.uniform_u8(930, 0, (1, m, k)), synth.uniform_i8(930, 1, (1, k, n))
+    once = run_spec(spec, [a, b, np.zeros((1, m, n), np.int32)])
+    bufs = [M.DeviceBuffer.from_numpy(x) for x in (a, b, np.zeros((1, m, n), np.int32))]
+    ptrs = [x.ptr for x in bufs]
+    spec.run_noalloc(ptrs)
+    spec.run_device(ptrs)       # mrl_run: accumulates a second time
+    spec.run_noalloc(ptrs)
+    M.synchronize()
+    got = bufs[2].to_numpy(np.int32, (1, m, n))
+    for x in bufs:
+        x.free()
+    assert np.array_equal(got, once * 3)
+
+
+def test_noalloc_wants_aligned_parameters(gpu):
+    spec = M.MatmulAccum([1, 256, 256, 256], (M.u8, M.i8, M.i32))
+    bufs = [M.DeviceBuffer(spec.bytes_used(i) + 256) for i in range(3)]
+    with pytest.raises(M.MorelloError) as err:
+        spec.run_noalloc([bufs[0].ptr + 16, bufs[1].ptr, bufs[2].ptr])
+    assert err.value.status == 1 and "aligned" in str(err.value)
+    for x in bufs:
+        x.free()
 
 
 def test_noalloc_turns_down_what_does_not_fit(gpu):
