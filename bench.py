@@ -364,6 +364,38 @@ def power_trace(seconds, phases=("idle", "c2", "mfma_zero_operands", "mfma_rando
     return out
 
 
+def cycle_stamps_attention(launches):
+    """The same for the fused attention kernel of C5 (the library built with
+    MRL_HIPCC_EXTRA=-DMRL_ATTN_TRACE): each wave of the key half that stores the output leaves the
+    cycles of its start-up, loop, merge and stores, the cycles it waited at barriers and the sums of
+    its matrix and vector slots in the first floats of its first output row."""
+    desc, spec, arrs, *_ = workload("c5")
+    bufs = [M.DeviceBuffer.from_numpy(a) for a in arrs]
+    ptrs = [b.ptr for b in bufs]
+    spec.run_timed(ptrs, launches)
+    M.synchronize()
+    us = spec.run_timed(ptrs, 20) / 20 * 1e3
+    M.synchronize()
+    out = bufs[3].to_numpy(np.float32, (16, 2048, 128)).view(np.uint32)
+    rows = (np.arange(16)[:, None] * 128 + np.arange(4)[None, :] * 32).reshape(-1)   # a wave's first query row
+    st = out[:, rows, :11].reshape(-1, 11).astype(np.int64)
+    stat = lambda x: {"median": float(np.median(x)), "min": float(x.min()), "max": float(x.max())}
+    if int(np.median(st[:, 7])) == 0 or int(np.median(st[:, 10])) > 10 ** 7:
+        raise SystemExit("no stamps in the output: build the library with MRL_HIPCC_EXTRA=-DMRL_ATTN_TRACE for this mode")
+    blocks = 16   # 2048 keys in two halves of 16 blocks of 64
+    res = {"workload": desc, "launches_before": launches, "us_per_launch_last_20": us, "waves": int(len(st)),
+           "wave_cycles": stat(st[:, 10]), "shader_clock_mhz": stat(st[:, 10] / st[:, 7] * 100.0),
+           "startup_cycles": stat(st[:, 0]), "loop_cycles": stat(st[:, 1]), "loop_cycles_per_key_block": stat(st[:, 1] / blocks),
+           "matrix_slot_cycles": stat(st[:, 5] / (blocks - 1)), "vector_slot_cycles": stat(st[:, 6] / (blocks - 1)),
+           "barrier_wait_cycles_per_key_block": stat(st[:, 4] / blocks),
+           "merge_and_store_issue_cycles": stat(st[:, 2]), "store_drain_cycles": stat(st[:, 3]),
+           "launch_span_us": float((st[:, 9].max() - st[:, 8].min()) & 0xffffffff) / 100.0,
+           "mfma_cycles_per_matrix_slot": 68 * 16}
+    for b in bufs:
+        b.free()
+    return res
+
+
 def cycle_stamps(launches):
     """Reads the stamps a timing build of the wide Matmul kernel (the library built with
     MRL_WIDE_OPTS=trace in the environment) leaves in the first rows of every wave's block of C:
@@ -488,7 +520,8 @@ def main():
                     help="with --power-trace: which of idle, c2, mfma_zero_operands, mfma_random_operands to run")
     ap.add_argument("--cycle-stamps", type=int, default=0, metavar="LAUNCHES",
                     help="instead of the benchmark: read the cycle stamps of a timing build of the C2 kernel "
-                         "(MRL_WIDE_OPTS=trace python -m morello_amd.build) after LAUNCHES launches")
+                         "(MRL_WIDE_OPTS=trace python -m morello_amd.build) or, with --spec c5, of the attention "
+                         "kernel (MRL_HIPCC_EXTRA=-DMRL_ATTN_TRACE python -m morello_amd.build) after LAUNCHES launches")
     args = ap.parse_args()
     if args.vendor_child:
         # PyTorch brings its own HIP runtime, which cannot share a process with the library's:
@@ -504,7 +537,7 @@ def main():
         print(json.dumps(power_trace(args.power_trace, tuple(args.phases.split(",")))))
         return
     if args.cycle_stamps > 0:
-        print(json.dumps(cycle_stamps(args.cycle_stamps)))
+        print(json.dumps(cycle_stamps_attention(args.cycle_stamps) if args.spec == "c5" else cycle_stamps(args.cycle_stamps)))
         return
     head = measure(args.spec, args.steps, args.warmup, min_gpu_s=0.2)
     desc, spec, arrs, dtype, unit = head["desc"], head["spec"], head["arrs"], head["dtype"], head["unit"]

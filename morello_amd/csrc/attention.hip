@@ -116,6 +116,15 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
     float *partials;
   } const p = {q, kt, v, out, b, m, n2, n_out, key_splits, partials};
   typedef Dims<D> DD;
+#ifdef MRL_ATTN_TRACE  // timing build: cycle stamps replace the first floats of a wave's first output row
+  const uint64_t t_start = __builtin_amdgcn_s_memtime(), r_start = __builtin_amdgcn_s_memrealtime();
+  uint64_t t_wait = 0, t_slot_a = 0, t_slot_b = 0;
+#define MRL_ATTN_SYNC() do { const uint64_t t_ = __builtin_amdgcn_s_memtime(); __syncthreads(); t_wait += __builtin_amdgcn_s_memtime() - t_; } while (0)
+#define MRL_ATTN_TIMED(acc, stmt) do { const uint64_t t_ = __builtin_amdgcn_s_memtime(); stmt; acc += __builtin_amdgcn_s_memtime() - t_; } while (0)
+#else
+#define MRL_ATTN_SYNC() __syncthreads()
+#define MRL_ATTN_TIMED(acc, stmt) stmt
+#endif
   constexpr int ROW = DD::ROW, TILE = DD::TILE, HALF = DD::HALF;
   constexpr int NC = D / 32;   // 32-wide chunks of d: k steps of S = K.Q
   constexpr int NDB = D / 16;  // 16-row blocks of O^T
@@ -497,19 +506,25 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
   };
 
   // Every wave passes steps + 1 pairs of barriers; a half with fewer blocks idles through the rest.
+#ifdef MRL_ATTN_TRACE
+  const uint64_t t_loop = __builtin_amdgcn_s_memtime();
+#endif
   if (nblocks > 0) slot_a_first();
-  __syncthreads();
+  MRL_ATTN_SYNC();
   if (nblocks > 0) slot_b(0);
-  __syncthreads();
+  MRL_ATTN_SYNC();
   int vstage = 0;  // V stage of block j - 1
   for (int j = 1; j < nblocks; j++) {
-    slot_a(j, my_lds + (2 + vstage) * TILE);
+    MRL_ATTN_TIMED(t_slot_a, slot_a(j, my_lds + (2 + vstage) * TILE));
     vstage = vstage == 2 ? 0 : vstage + 1;
-    __syncthreads();
-    slot_b(j);
-    __syncthreads();
+    MRL_ATTN_SYNC();
+    MRL_ATTN_TIMED(t_slot_b, slot_b(j));
+    MRL_ATTN_SYNC();
   }
   if (nblocks > 0) slot_a_last(my_lds + (2 + vstage) * TILE);
+#ifdef MRL_ATTN_TRACE
+  const uint64_t t_loop_end = __builtin_amdgcn_s_memtime();
+#endif
   for (int j = max(nblocks, 1); j <= steps; j++) {
     __syncthreads();
     __syncthreads();
@@ -573,6 +588,20 @@ __global__ __launch_bounds__(512) void k_attn(const void *q, const void *kt, con
         }
     }
   }
+#ifdef MRL_ATTN_TRACE
+  {
+    const uint64_t t_issued = __builtin_amdgcn_s_memtime();
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // the stores have drained
+    const uint64_t t_end = __builtin_amdgcn_s_memtime(), r_end = __builtin_amdgcn_s_memrealtime();
+    if (lane == 0) {
+      uint32_t *stamp = (uint32_t *)(p.out + (head * p.m + q0 + 16 * half) * int64_t(p.n_out));
+      stamp[0] = uint32_t(t_loop - t_start), stamp[1] = uint32_t(t_loop_end - t_loop), stamp[2] = uint32_t(t_issued - t_loop_end);
+      stamp[3] = uint32_t(t_end - t_issued), stamp[4] = uint32_t(t_wait), stamp[5] = uint32_t(t_slot_a), stamp[6] = uint32_t(t_slot_b);
+      stamp[7] = uint32_t(r_end - r_start), stamp[8] = uint32_t(r_start), stamp[9] = uint32_t(r_end);
+      stamp[10] = uint32_t(t_end - t_start);
+    }
+  }
+#endif
 }
 
 // out[row][0 .. n_out) = sum_s O_s * 2^((m_s - M) log2 e) / sum_s l_s * 2^((m_s - M) log2 e), M = max_s m_s:
