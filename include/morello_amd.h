@@ -499,7 +499,10 @@ int mrl_compose_plan(const mrl_compose *c, mrl_plan *plan, mrl_plan_step *steps,
  * an action names the scheduling steps it stands for (scheduling_sugar.rs:37-132):
  *   SELECT          the dispatch rules' own choice for the Spec as it stands (Action::Select)
  *   TILE_OUT_SPLIT  Matmul: tile_out([1, tile_m, tile_n]).split(split_k), then the matrix-core kernel
- *   FUSED           Conv: the fused NHWC/KRSC kernel; Compose Matmul->Softmax->Matmul: the fused kernel
+ *   FUSED           Conv: the fused NHWC/KRSC kernel, a wave per 16-pixel tile (`tile_m` = 0) or, with
+ *                   `tile_m` = the output width, tile_out over whole output rows: a workgroup's waves
+ *                   share the rows' pixels through LDS and take 16 filters each (64 channels);
+ *                   Compose Matmul->Softmax->Matmul: the fused kernel
  *                   with tile_out over the rows (`tile_m` = 128 or 64 queries per workgroup, 0 = the
  *                   dispatch rules' choice) and the keys in `parts` shares (parallel_softmax.rs:31-223;
  *                   1 = one workgroup per query block, more = partial results merged with the parts formula)
@@ -534,7 +537,8 @@ typedef enum {
 } mrl_action_kind;
 typedef struct {
   int32_t kind;             /* mrl_action_kind */
-  uint32_t tile_m, tile_n;  /* TILE_OUT_SPLIT, SPATIAL_SPLIT; FUSED on a Compose: tile_m = queries per workgroup */
+  uint32_t tile_m, tile_n;  /* TILE_OUT_SPLIT, SPATIAL_SPLIT; FUSED on a Compose: tile_m = queries per workgroup;
+                               FUSED on a Conv: tile_m = 0 or the output width (whole rows per workgroup) */
   uint32_t split_k;         /* TILE_OUT_SPLIT: elements of K per step */
   uint32_t parts;           /* FUSED on a Compose: shares of the keys; PARALLEL_SOFTMAX: tiles along the scan dim */
   uint32_t staging;         /* TILE_OUT_SPLIT: mrl_staging */

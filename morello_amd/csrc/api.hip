@@ -543,6 +543,7 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
 struct Forced {
   int conv_path = 0;        // 1 fused kernel, 2 implicit Matmul (tile side conv_tile), 3 unfold + Matmul, 4 generic
   uint32_t conv_tile = 0;
+  bool conv_rows = false;   // fused kernel: whole output rows per workgroup, pixels shared through LDS
   int msm_path = 0;         // 1 fused kernel (key_splits workgroups per query block), 2 staged
   uint32_t key_splits = 0;
   uint32_t query_block = 0; // fused kernel: queries per workgroup (64 or 128), 0 = the rule below
@@ -639,7 +640,9 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
                          (reinterpret_cast<uintptr_t>(filt.t.ptr) & 15) == 0 && (reinterpret_cast<uintptr_t>(out.t.ptr) & 3) == 0;
   if ((forced == 1 && !fused_ok) || (forced == 2 && !implicit_ok) || (forced == 3 && !unfold_ok)) return MRL_ERR_UNSUPPORTED;
   if (fused_ok && forced <= 1) {
-    HIP_TRY(mrl::launch_conv_i8(cv, di == MRL_U8, ws.stream));
+    const bool rows = forced == 1 && g_forced->conv_rows;
+    if (rows && !mrl::conv_rows_applicable(cv)) return MRL_ERR_UNSUPPORTED;
+    HIP_TRY(mrl::launch_conv_i8(cv, di == MRL_U8, ws.stream, rows));
   } else if (implicit_ok && (forced == 0 || forced == 2)) {
     // Channel vectors of whole 16-byte chunks: the windows are read where they lie.  (A 1x1 filter
     // needs no window arithmetic: its image is the left operand of a plain Matmul, below.)
@@ -1512,7 +1515,7 @@ uint32_t mrl_target_layouts_for_shape(const uint32_t *shape, uint32_t rank, int 
 
 uint32_t mrl_target_kernels(const char **names, uint32_t cap) {
   static const char *const families[] = {
-      "k_gemm", "k_gemm_big", "k_gemm_wide", "k_gemv", "k_matmul_generic", "k_sum_splits", "k_conv_i8", "k_conv_generic", "k_conv_generic_wave", "k_unfold",
+      "k_gemm", "k_gemm_big", "k_gemm_wide", "k_gemv", "k_matmul_generic", "k_sum_splits", "k_conv_i8", "k_conv_rows_i8", "k_conv_generic", "k_conv_generic_wave", "k_unfold",
       "k_unfold_gather", "k_attn", "k_attn_merge", "k_softmax_regs", "k_softmax_regs1", "k_softmax_short", "k_softmax_block", "k_softmax_chunk_stats", "k_softmax_chunk_write",
       "k_softmax_cols",
       "k_softmax_generic", "k_parts", "k_broadcast", "k_fill", "k_fill_zero", "k_move_rows", "k_move_rows16",
@@ -1874,6 +1877,7 @@ int dispatch_action(const mrl_spec &spec, void *const *params, Workspace &ws, co
     case MRL_ACTION_GENERIC: f.conv_path = 4; break;
     case MRL_ACTION_FUSED:
       f.conv_path = 1, f.msm_path = 1, f.key_splits = a.parts ? a.parts : 1, f.query_block = a.tile_m;
+      f.conv_rows = spec.kind == MRL_SPEC_CONV && a.tile_m != 0;   // tile_out over whole output rows
       break;
     case MRL_ACTION_BUFFERIZE: f.msm_path = 2; break;
     default: return MRL_ERR_BAD_SPEC;
@@ -1932,6 +1936,7 @@ uint32_t mrl_target_actions(const mrl_spec *spec, mrl_action *out, uint32_t cap)
     }
   } else if (spec->kind == MRL_SPEC_CONV) {
     candidate(MRL_ACTION_FUSED);
+    candidate(MRL_ACTION_FUSED, spec->spec_shape[4]);   // tile_out over whole output rows (tile_m = ow)
     for (uint32_t side : {64u, 128u, 256u}) candidate(MRL_ACTION_SPATIAL_SPLIT, side, side, 0);
     candidate(MRL_ACTION_UNFOLD);
     candidate(MRL_ACTION_GENERIC);

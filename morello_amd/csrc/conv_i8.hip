@@ -177,6 +177,203 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(const void *image, const
   }
 }
 
+
+// ---- 64 channels, whole output rows per workgroup ----------------------------------------------
+// The same Conv with the roles of a workgroup's four waves turned round: wave w holds 16 of the 64
+// filters (TAPS x 4 operand registers instead of TAPS x 16: a quarter of the start-up, and room
+// for four waves per SIMD), and all four multiply them with the SAME pixels, which therefore come
+// through LDS once per workgroup instead of once per wave: the input rows that a run of output
+// rows touches are one contiguous piece of the NHWC image (also across an image boundary), moved
+// by direct-to-LDS loads (no staging registers), and the fh x fw taps of a pixel tile are reads
+// of that piece at different offsets, so the taps' overlap is served by LDS instead of by the
+// vector cache (the image crosses it 1.5-2 times instead of fh * fw / 1.2 times).  A u8 image is
+// made signed (xor 0x80) once per byte in LDS instead of once per tap and wave in registers.
+//   move_param(image, L1) -> global_load_lds_dwordx4, rows padded to 16 pixels, a pixel's four
+//   16-byte chunks rotated by (pixel / 2) % 4, which is what lets the 16 lanes of an operand read
+//   (pixels 64 bytes apart) run at the full LDS rate (measured: 2.75 cycles a read for 16 waves of a
+//   compute unit, as for a contiguous read; 4.27 with no rotation or with (pixel / 4) % 4); applied
+//   on the source side of the loads.
+// Output: a lane holds 4 consecutive filters of one pixel (16 bytes); the four waves' pieces of a
+// tile meet in LDS and are written as whole pixel rows.
+typedef __attribute__((address_space(3))) void lds_void_t;
+
+__device__ inline void conv_dma16(const uint8_t *base, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
+}
+
+template <int TAPS, bool IMG_UNSIGNED>
+__global__ __launch_bounds__(256) void k_conv_rows_i8(const void *image, const void *filters_all, void *out_all, uint32_t f,
+                                                      uint32_t oh, uint32_t ow, uint32_t fh, uint32_t fw, int accum,
+                                                      uint32_t total_rows, uint32_t rows_per_wg) {
+  struct {
+    const void *image, *filters;
+    void *out;
+    uint32_t f, oh, ow, fh, fw;
+    int accum;
+    uint32_t total_rows, rows_per_wg;
+  } const p = {image, filters_all, out_all, f, oh, ow, fh, fw, accum, total_rows, rows_per_wg};
+  extern __shared__ __attribute__((aligned(1024))) uint8_t rows_lds[];
+  const int lane = threadIdx.x & 63, li = lane & 15, lg = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t H = p.oh + p.fh - 1, W = p.ow + p.fw - 1, W16 = (W + 15) & ~15u;
+  const uint32_t row_bytes = W16 * 64, kb_per_row = W16 / 16;
+  // Output rows [g0, g1) (row g = image g / oh, line g % oh) and the input rows they read: input
+  // row b * H + y is row-major memory, and the last rows of one image are followed by the first of
+  // the next, so the piece is contiguous whatever the run crosses.
+  const uint32_t g0 = blockIdx.x * p.rows_per_wg, g1 = min(g0 + p.rows_per_wg, p.total_rows);
+  const uint32_t in_first = (g0 / p.oh) * H + g0 % p.oh;
+  const uint32_t in_last = ((g1 - 1) / p.oh) * H + (g1 - 1) % p.oh + p.fh - 1;
+  const uint32_t nkb = (in_last - in_first + 1) * kb_per_row;
+  const uint32_t lds0 = uint32_t(reinterpret_cast<uintptr_t>((lds_void_t *)rows_lds));
+  {
+    // KiB k of the piece: 16 pixels of input row in_first + k / kb_per_row; lane L fills 16-byte
+    // position L % 4 of pixel L / 4 with the chunk that belongs there.  Pixels past the row's end
+    // (the padding) fetch the row's last pixel again.
+    const uint32_t pl = lane >> 2, cp = lane & 3;
+    for (uint32_t k = wave; k < nkb; k += 4) {
+      const uint32_t ku = __builtin_amdgcn_readfirstlane(k);
+      const uint32_t row = in_first + ku / kb_per_row, xp = 16 * (ku % kb_per_row) + pl;
+      const uint32_t chunk = (cp - (xp >> 1)) & 3;
+      conv_dma16((const uint8_t *)p.image, (row * W + min(xp, W - 1)) * 64 + chunk * 16, lds0 + ku * 1024);
+    }
+  }
+  // This wave's 16 filters as MFMA operands: lane (li, lg) holds channels 16 lg .. + 15 of filter li, per tap.
+  const uint8_t *filters = (const uint8_t *)p.filters + (int64_t(blockIdx.y) * 64 + wave * 16 + li) * (TAPS * 64) + lg * 16;
+  v4i filt[TAPS];
+#pragma unroll
+  for (int t = 0; t < TAPS; t++) filt[t] = *(const v4i *)(filters + t * 64);
+  // Per tap the lane's address within an output row's first tile: pixel li + s of input row r.
+  uint32_t tap_addr[TAPS];
+#pragma unroll
+  for (int t = 0; t < TAPS; t++) {
+    const uint32_t r = t / p.fw, s0 = t % p.fw, xp = li + s0;
+    tap_addr[t] = r * row_bytes + xp * 64 + (((lg + (xp >> 1)) & 3) << 4);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // the piece and the filters are in
+  if (IMG_UNSIGNED) {
+    // a - 128 for every byte this wave fetched (its own KiBs: no barrier needed before)
+    for (uint32_t k = wave; k < nkb; k += 4) {
+      unsigned long long *q = (unsigned long long *)(rows_lds + k * 1024) + lane;
+      __hip_atomic_fetch_xor(q, 0x8080808080808080ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      __hip_atomic_fetch_xor(q + 64, 0x8080808080808080ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+  }
+  // u8 correction 128 * sum filt[f]: the same MFMAs against an all-ones pixel leave the filter sums
+  // in the accumulator layout; the accumulators start from it.
+  v4i corr = v4i{0, 0, 0, 0};
+  if (IMG_UNSIGNED) {
+    const v4i ones = v4i{0x01010101, 0x01010101, 0x01010101, 0x01010101};
+#pragma unroll
+    for (int t = 0; t < TAPS; t++) corr = __builtin_amdgcn_mfma_i32_16x16x64_i8(filt[t], ones, corr, 0, 0, 0);
+    corr *= 128;
+  }
+  __syncthreads();
+  const uint32_t ntiles = (p.ow + 15) / 16, count = (g1 - g0) * ntiles;
+  int32_t *out = (int32_t *)p.out + blockIdx.y * 64 + li * 4;
+  // The run's tiles in order: 16 pixels each, tile j of output row g.  A cursor walks them (no
+  // division per tile): LDS offset of the row's first input row and of the tile in it, and the
+  // output offset of the row's first pixel.  Past the last tile it stays on it.
+  struct Cursor {
+    uint32_t j, y, lds_off, left;   // tile within the row, line within the image, LDS offset of tile 0's pixel 0, tiles left
+    int64_t out_off;                // elements from `out` to the row's pixel 0
+  };
+  Cursor cur = {0, g0 % p.oh, 0, count, int64_t(g0) * p.ow * p.f};
+  auto advance = [&](Cursor &c) {
+    if (c.left <= 1) return;
+    c.left--;
+    if (++c.j < ntiles) return;
+    c.j = 0;
+    c.out_off += int64_t(p.ow) * p.f;
+    // the next output row's first input row: the next LDS row, or fh rows on where a new image begins
+    const bool wrap = c.y + 1 == p.oh;
+    c.lds_off += (wrap ? p.fh : 1u) * row_bytes;
+    c.y = wrap ? 0 : c.y + 1;
+  };
+  // The operands of the next tile are read from LDS while the current one is multiplied: two
+  // register sets taken in turn, every read and every MFMA issued whatever the tile (a tile past
+  // the end repeats the last one and stores nothing), so that the loop body is one straight line
+  // and a wait can be for one set's reads alone.
+  auto read_tile = [&](const Cursor &c, v4i *px) {
+    const uint8_t *at = rows_lds + c.lds_off + c.j * 1024;
+#pragma unroll
+    for (int t = 0; t < TAPS; t++) px[t] = *(const v4i *)(at + tap_addr[t]);
+  };
+  // A tile's 16 x 64 results are the four waves' 16 x 16 blocks side by side (a lane holds 4
+  // consecutive filters of one pixel, 16 bytes of its 256-byte row).  They meet in LDS (rows 272
+  // bytes apart: 16 bytes of padding shift the banks) and leave as whole rows, wave w the four
+  // pixels 4 w .. 4 w + 3: 1 KiB contiguous per store instruction when F = 64, where four waves
+  // writing their 64-byte pieces cost 3 us of a 9.7 us launch.  Two exchange buffers in turn,
+  // one barrier per tile.
+  constexpr int XROW = 272;
+  uint8_t *xbuf = rows_lds + (in_last - in_first + 1) * row_bytes + 1024;
+  uint32_t turn = 0;
+  auto finish_tile = [&](const Cursor &c, bool live, const v4i *px) {
+    v4i acc = corr;
+#pragma unroll
+    for (int t = 0; t < TAPS; t++) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(filt[t], px[t], acc, 0, 0, 0);
+    uint8_t *xb = xbuf + turn * (16 * XROW);
+    turn ^= 1;
+    *(v4i *)(xb + li * XROW + wave * 64 + lg * 16) = acc;
+    __syncthreads();
+    const uint32_t pixel = 4 * wave + lg, x = 16 * c.j + pixel;
+    v4i v = *(const v4i *)(xb + pixel * XROW + li * 16);
+    if (live && x < p.ow) {
+      v4i *d = (v4i *)(out + c.out_off + int64_t(x) * p.f);
+      if (p.accum) v += *d;
+      __builtin_nontemporal_store(v, d);
+    }
+  };
+  v4i px_a[TAPS], px_b[TAPS];
+  read_tile(cur, px_a);
+  for (uint32_t i = 0; i < count; i += 2) {
+    Cursor nxt = cur;
+    advance(nxt);
+    read_tile(nxt, px_b);
+    finish_tile(cur, true, px_a);
+    cur = nxt;
+    advance(nxt);
+    read_tile(nxt, px_a);
+    finish_tile(cur, i + 1 < count, px_b);
+    cur = nxt;
+  }
+}
+
+// Output rows per workgroup and the LDS the piece of the image takes, or 0 when the kernel does
+// not apply (the piece of the smallest run does not fit).
+struct RowsPlan {
+  uint32_t rows_per_wg, lds_bytes;
+};
+RowsPlan conv_rows_plan(const ConvArgs &c) {
+  const uint32_t W = c.ow + c.fw - 1, W16 = (W + 15) & ~15u, row_bytes = W16 * 64;
+  const uint64_t total_rows = uint64_t(c.b) * c.oh;
+  // four workgroups of four waves per compute unit when there are rows enough
+  uint32_t rows = uint32_t(std::min<uint64_t>(8, std::max<uint64_t>(1, (total_rows + 4 * g_compute_units - 1) / (4 * g_compute_units))));
+  for (; rows >= 1; rows--) {
+    const uint32_t crossings = (rows + c.oh - 2) / c.oh;   // image boundaries a run of `rows` can cross
+    const uint64_t in_rows = rows + uint64_t(c.fh - 1) * (1 + crossings);
+    const uint64_t lds = in_rows * row_bytes + 1024 + 2 * 16 * 272;   // the piece, slack for reads past it, two exchange buffers
+    if (lds <= 40 * 1024) return RowsPlan{rows, uint32_t(lds)};
+  }
+  return RowsPlan{0, 0};
+}
+
+template <int TAPS>
+hipError_t launch_rows(const ConvArgs &c, bool img_unsigned, const RowsPlan &rp, hipStream_t stream) {
+  const uint32_t total_rows = c.b * c.oh;
+  const dim3 grid((total_rows + rp.rows_per_wg - 1) / rp.rows_per_wg, c.f / 64);
+  const double pixels = double(total_rows) * c.ow;
+  plan::work(plan::UNIT_MFMA_I8, 2.0 * pixels * c.f * c.fh * c.fw * c.c,
+             double(c.b) * (c.oh + c.fh - 1) * (c.ow + c.fw - 1) * c.c + double(c.f) * c.fh * c.fw * c.c +
+                 4.0 * pixels * c.f * (c.accum ? 2 : 1));
+  if (img_unsigned)
+    MRL_LAUNCH((k_conv_rows_i8<TAPS, true>), grid, dim3(256), rp.lds_bytes, stream, c.image, c.filters, c.out, c.f, c.oh, c.ow, c.fh,
+               c.fw, c.accum, total_rows, rp.rows_per_wg);
+  else
+    MRL_LAUNCH((k_conv_rows_i8<TAPS, false>), grid, dim3(256), rp.lds_bytes, stream, c.image, c.filters, c.out, c.f, c.oh, c.ow, c.fh,
+               c.fw, c.accum, total_rows, rp.rows_per_wg);
+  return mrl::plan::last_error();
+}
+
 template <int SLABS>
 hipError_t launch_slabs(const ConvArgs &c, bool img_unsigned, hipStream_t stream) {
   const uint64_t pixels = uint64_t(c.b) * c.oh * c.ow;
@@ -216,7 +413,26 @@ bool conv_i8_applicable(const ConvArgs &c) {
          al16(c.filters) && al16(c.out);
 }
 
-hipError_t launch_conv_i8(const ConvArgs &c, bool img_unsigned, hipStream_t stream) {
+bool conv_rows_applicable(const ConvArgs &c) {
+  return conv_i8_applicable(c) && c.c == 64 && uint64_t(c.b) * c.oh < (1u << 31) && conv_rows_plan(c).rows_per_wg > 0;
+}
+
+hipError_t launch_conv_i8(const ConvArgs &c, bool img_unsigned, hipStream_t stream, bool whole_rows) {
+  // The kernel that shares a workgroup's pixels through LDS (64 channels: a tap is one k step)
+  // is taken when asked for: on the benchmark's Conv the two kernels measure the same (8.8-8.9 us:
+  // both are a launch, a start-up of one trip to memory and the 24 MB of output at HBM's rate).
+  if (whole_rows) {
+    if (!conv_rows_applicable(c)) return hipErrorInvalidValue;
+    const RowsPlan rp = conv_rows_plan(c);
+    switch (slabs_of(c)) {
+      case 1: return launch_rows<1>(c, img_unsigned, rp, stream);
+      case 2: return launch_rows<2>(c, img_unsigned, rp, stream);
+      case 3: return launch_rows<3>(c, img_unsigned, rp, stream);
+      case 4: return launch_rows<4>(c, img_unsigned, rp, stream);
+      case 6: return launch_rows<6>(c, img_unsigned, rp, stream);
+      default: return launch_rows<9>(c, img_unsigned, rp, stream);
+    }
+  }
   switch (slabs_of(c)) {
     case 1: return launch_slabs<1>(c, img_unsigned, stream);
     case 2: return launch_slabs<2>(c, img_unsigned, stream);

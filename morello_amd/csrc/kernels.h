@@ -134,7 +134,10 @@ struct ConvArgs {
   int accum;
 };
 bool conv_i8_applicable(const ConvArgs &c);
-hipError_t launch_conv_i8(const ConvArgs &c, bool img_unsigned, hipStream_t stream);
+// whole_rows: the kernel whose workgroups take whole output rows and share their pixels through LDS
+// (conv_rows_applicable: 64 channels, a run's piece of the image fits LDS); else a wave per 16-pixel tile.
+bool conv_rows_applicable(const ConvArgs &c);
+hipError_t launch_conv_i8(const ConvArgs &c, bool img_unsigned, hipStream_t stream, bool whole_rows = false);
 
 // ---- unfold.hip: the windows of a channels-last image as rows, for Conv as a Matmul ---------
 // image: [batch][oh+fh-1][ow+fw-1][c]; rows: [batch*oh*ow][row_elems], each row the fh*fw*c

@@ -57,6 +57,8 @@ def test_conv_actions_against_the_oracle(gpu):
     acts = spec.actions()
     assert {a.kind for a in acts} == {M.ActionKind.Select, M.ActionKind.Fused, M.ActionKind.SpatialSplit,
                                       M.ActionKind.Unfold, M.ActionKind.Generic}
+    # the fused kernel both ways: a wave per pixel tile, and whole output rows per workgroup
+    assert [a.tile_m for a in acts if a.kind == M.ActionKind.Fused] == [0, ow]
     for act in acts:
         got = run_action(act, [img, filt, np.full((b, oh, ow, f), -7, np.int32)])
         assert np.array_equal(got, want), act
@@ -75,6 +77,26 @@ def test_compose_actions_against_the_oracle(gpu):
     for act in acts:
         got = run_action(act, [v, q, kmat, np.zeros((b, m, n), np.float32)])
         assert rel_err(got, want) < 1e-2, act
+
+
+@pytest.mark.parametrize("dims,accum", [((3, 64, 64, 5, 7, 3, 3), False), ((2, 128, 64, 54, 54, 3, 3), True), ((5, 64, 64, 1, 40, 1, 1), False),
+                                        ((1, 64, 64, 9, 100, 2, 3), False), ((40, 64, 64, 2, 3, 3, 2), True), ((2, 192, 64, 6, 17, 1, 3), False)])
+def test_conv_over_whole_output_rows(gpu, dims, accum):
+    """The fused Conv kernel whose workgroups take runs of whole output rows (tile_out over rows; the
+    rows' pixels shared through LDS, 16 filters per wave): runs that cross image boundaries, rows
+    that are not whole tiles of 16 pixels, several groups of 64 filters, every tap count, u8 and i8
+    images, accumulating or not, against the oracle."""
+    b, f, c, oh, ow, fh, fw = dims
+    for img_dt, img_code, gen in ((M.u8, orc.U8, synth.uniform_u8), (M.i8, orc.I8, synth.uniform_i8)):
+        spec = M.Conv(list(dims), (img_dt, M.i8, M.i32), accum=accum)
+        img = gen(37, 0, (b, oh + fh - 1, ow + fw - 1, c))
+        filt = synth.uniform_i8(37, 1, (f, fh, fw, c))
+        out0 = (synth.uniform_i8(37, 2, (b, oh, ow, f)).astype(np.int32) * 77) if accum else np.full((b, oh, ow, f), -3, np.int32)
+        nhwc = orc.make_layout([0, 2, 3, 1])
+        want = orc.conv(list(dims), [img_code, orc.I8, orc.I32], img, filt, out0.copy(), accum, layouts=[nhwc, nhwc, nhwc])
+        rows = [a for a in spec.actions() if a.kind == M.ActionKind.Fused and a.tile_m == ow]
+        assert len(rows) == 1 and rows[0].plan().kernels == ["k_conv_rows_i8"]
+        assert np.array_equal(run_action(rows[0], [img, filt, out0.copy()]), want)
 
 
 @pytest.mark.parametrize("shape,dim", [((64, 1024), 1), ((3, 50, 256), 2), ((7, 128, 33), 1), ((2, 4, 640, 5), 2), ((1000, 96), 1),

@@ -360,9 +360,12 @@ def test_actions_of_the_benchmark_configurations():
     acts = c3().actions()
     assert len(acts) == 12 and acts[0].cost_ns == min(a.cost_ns for a in acts)
     acts = {(a.kind, a.tile_m): a for a in c4().actions()}
-    assert set(acts) == {(K.Select, 0), (K.Fused, 0), (K.SpatialSplit, 64), (K.SpatialSplit, 128), (K.SpatialSplit, 256),
+    assert set(acts) == {(K.Select, 0), (K.Fused, 0), (K.Fused, 54), (K.SpatialSplit, 64), (K.SpatialSplit, 128), (K.SpatialSplit, 256),
                          (K.Unfold, 0), (K.Generic, 0)}
     assert acts[(K.Fused, 0)].plan().kernels == ["k_conv_i8"] and acts[(K.Select, 0)].cost_ns == acts[(K.Fused, 0)].cost_ns
+    # tile_out over whole output rows: two rows per workgroup, their four input rows (padded to 64 pixels) in LDS
+    rows = acts[(K.Fused, 54)].plan().steps[0]
+    assert rows.kernel.startswith("k_conv_rows_i8") and rows.grid == (864, 1, 1) and rows.block == (256, 1, 1)
     assert acts[(K.SpatialSplit, 128)].plan().kernels == ["k_gemm"] and "CONV = true" in acts[(K.SpatialSplit, 128)].plan().steps[0].kernel
     assert acts[(K.Unfold, 0)].plan().kernels == ["k_unfold", "k_gemm"] and acts[(K.Unfold, 0)].scratch_bytes > 50e6
     assert acts[(K.Generic, 0)].plan().kernels == ["k_conv_generic"]
