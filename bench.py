@@ -446,21 +446,27 @@ def cycle_stamps(launches):
     return out
 
 
-def measure(name, steps, warmup, min_gpu_s):
+def measure(name, steps, warmup, min_gpu_s, action=None):
     """W warm-up launches, then bursts of `steps` launches until there are MIN_REPEATS of them and
-    min_gpu_s seconds of GPU time; -> the workload and the figures of the fastest and the last burst."""
+    min_gpu_s seconds of GPU time; -> the workload and the figures of the fastest and the last burst.
+    action: index into the Spec's list of lowerings (mrl_target_actions) to time instead of the
+    dispatch rules' own choice."""
     desc, spec, arrs, dtype, unit, bound, peak = workload(name)
+    runner = spec
+    if action is not None:
+        runner = spec.actions()[action]
+        desc += f" [action {action}: {runner!r}]"
     bufs = [M.DeviceBuffer.from_numpy(a) for a in arrs]
     ptrs = [b.ptr for b in bufs]
     ops = spec.flops()
     alg_bytes = sum(spec.bytes_used(i) for i in range(len(arrs)))
     for _ in range(warmup):
-        spec.run_device(ptrs)
+        runner.run_device(ptrs)
     M.synchronize()
     bursts, gpu_ms = [], 0.0
     while len(bursts) < MIN_REPEATS or (gpu_ms < min_gpu_s * 1e3 and len(bursts) < 5000):
         t0 = time.perf_counter()
-        device_ms = spec.run_timed(ptrs, steps)  # enqueues K launches between two events, waits for the last
+        device_ms = runner.run_timed(ptrs, steps)  # enqueues K launches between two events, waits for the last
         M.synchronize()
         bursts.append((device_ms / steps, (time.perf_counter() - t0) * 1e3 / steps))
         gpu_ms += device_ms
@@ -509,6 +515,9 @@ def main():
     ap.add_argument("--spec", default="c2", choices=["c1", "c2", "c2o", "c3", "c4", "c5", "softmax", "move", "matvec", "conv128", "decode", "softmax_long",
                                                      "transpose"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--action", type=int, default=None, metavar="K",
+                    help="time the K-th lowering the library lists for the workload's Spec (mrl_target_actions) "
+                         "instead of the dispatch rules' own choice; implies --no-configs")
     ap.add_argument("--no-configs", action="store_true", help="headline workload only: skip the `configs` object")
     ap.add_argument("--vendor-ref", action="store_true",
                     help="also time the vendor library's nearest operation through PyTorch (c2, c3, c5)")
@@ -539,7 +548,7 @@ def main():
     if args.cycle_stamps > 0:
         print(json.dumps(cycle_stamps_attention(args.cycle_stamps) if args.spec == "c5" else cycle_stamps(args.cycle_stamps)))
         return
-    head = measure(args.spec, args.steps, args.warmup, min_gpu_s=0.2)
+    head = measure(args.spec, args.steps, args.warmup, min_gpu_s=0.2, action=args.action)
     desc, spec, arrs, dtype, unit = head["desc"], head["spec"], head["arrs"], head["dtype"], head["unit"]
     value, ms_per_step, roofline = head["value"], head["ms_per_step"], head["roofline"]
 
@@ -554,10 +563,10 @@ def main():
         "roofline": roofline,
     }
     # Which kernels the timed launches were, and what the library's cost model expected of them.
-    plan = spec.plan()
+    plan = spec.plan() if args.action is None else spec.actions()[args.action].plan()
     out["plan"] = {"kernels": [s.kernel for s in plan.steps], "predicted_ms": plan.cost_ns * 1e-6,
                    "scratch_bytes": plan.scratch_bytes}
-    if args.spec == "c2" and not args.no_configs:
+    if args.spec == "c2" and not args.no_configs and args.action is None:
         # The other benchmark configurations, each by the same protocol (a quarter of the GPU time).
         out["configs"] = {}
         for name in ("c1", "c3", "c4", "c5"):

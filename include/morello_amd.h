@@ -555,6 +555,10 @@ int mrl_action_plan(const mrl_spec *spec, const mrl_action *action, mrl_plan *pl
  * to these operands (alignment); the result is the Spec's whatever the action: integer Specs bit
  * for bit, floating-point ones within the Spec's tolerance. */
 int mrl_run_action(const mrl_spec *spec, void *const *params, const mrl_action *action, void *stream);
+/* mrl_run_timed for a chosen action: `steps` launches back to back on the default stream between
+ * two events (what BuiltArtifact::measure_time does for one schedule, codegen/mod.rs:330-340). */
+int mrl_run_action_timed(const mrl_spec *spec, void *const *params, const mrl_action *action, uint32_t steps,
+                         double *device_ms_total);
 
 #ifdef __cplusplus
 }

@@ -636,6 +636,20 @@ class Action:
         _check(B.load().mrl_run_action(C.byref(self.spec._c), arr, C.byref(self._c), None), "mrl_run_action")
         synchronize()
 
+    def run_timed(self, ptrs: Sequence[int], steps: int) -> float:
+        """`steps` back-to-back launches of this action between two HIP events; total device milliseconds."""
+        arr = (C.c_void_p * len(ptrs))(*ptrs)
+        ms = C.c_double()
+        _check(B.load().mrl_run_action_timed(C.byref(self.spec._c), arr, C.byref(self._c), steps, C.byref(ms)),
+               "mrl_run_action_timed")
+        return ms.value
+
+    def flops(self) -> float:
+        return self.spec.flops()
+
+    def bytes_used(self, i: int) -> int:
+        return self.spec.bytes_used(i)
+
 
 def _plan_of(fn, c_spec, where: str) -> Plan:
     head, cap = B.PlanC(), 64

@@ -141,6 +141,7 @@ SIGNATURES = {
     "mrl_stream_release": (C.c_int, [C.c_void_p]),
     "mrl_device_mem_free": (C.c_int, [C.POINTER(C.c_size_t)]),
     "mrl_abi_version": (C.c_uint32, []),
+    "mrl_run_action_timed": (C.c_int, [C.POINTER(SpecC), _VPP, C.POINTER(ActionC), C.c_uint32, C.POINTER(C.c_double)]),
     "mrl_stream_destroy": (C.c_int, [C.c_void_p]),
     "mrl_target_id": (C.c_char_p, []),
     "mrl_target_line_size": (C.c_uint32, []),

@@ -2017,6 +2017,28 @@ int mrl_run_timed(const mrl_spec *spec, void *const *params, uint32_t steps,
   return MRL_OK;
 }
 
+int mrl_run_action_timed(const mrl_spec *spec, void *const *params, const mrl_action *action, uint32_t steps,
+                         double *device_ms_total) {
+  if (!device_ms_total || !action) return MRL_ERR_NULL;
+  if (steps == 0) return MRL_ERR_BAD_SPEC;
+  hipEvent_t t0, t1;
+  HIP_TRY(hipEventCreate(&t0));
+  HIP_TRY(hipEventCreate(&t1));
+  (void)hipEventRecord(t0, nullptr);
+  int rc = MRL_OK;
+  for (uint32_t i = 0; i < steps && rc == MRL_OK; i++) rc = mrl_run_action(spec, params, action, nullptr);
+  (void)hipEventRecord(t1, nullptr);
+  hipError_t e = hipEventSynchronize(t1);
+  float ms = 0.0f;
+  if (e == hipSuccess) e = hipEventElapsedTime(&ms, t0, t1);
+  (void)hipEventDestroy(t0);
+  (void)hipEventDestroy(t1);
+  if (rc != MRL_OK) return rc;
+  if (e != hipSuccess) return hip_fail(e, "event timing");
+  *device_ms_total = double(ms);
+  return MRL_OK;
+}
+
 int mrl_compose_init(mrl_compose *c) {
   if (!c) return MRL_ERR_NULL;
   std::vector<ComposeParam> ext;
