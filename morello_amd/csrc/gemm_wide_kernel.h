@@ -56,7 +56,7 @@ constexpr int WIDE_MIN_STEPS = GEMM_WIDE_MIN_STEPS;
       MRL_WIDE_FIRST_100("a"), MRL_WIDE_100("a", 1), MRL_WIDE_10("a", 20), MRL_WIDE_10("a", 21),            \
       MRL_WIDE_10("a", 22), MRL_WIDE_10("a", 23), MRL_WIDE_10("a", 24), "a250", "a251", "a252", "a253",     \
       "a254", "a255", "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71",   \
-      "s72", "s73", "s74", "s78", "s79", "s80", "s81", "s82", "s83", "s84", "s85", "s86", "s87", "s88", "s89", "s90",     \
+      "s72", "s73", "s74", "s75", "s78", "s79", "s80", "s81", "s82", "s83", "s84", "s85", "s86", "s87", "s88", "s89", "s90",     \
       "s91", "s92", "s93", "s94", "s95", "scc", "memory"
 
 #define MRL_WIDE_RUN(TEXT)                                                                                         \
@@ -189,16 +189,24 @@ __global__ __launch_bounds__(256) void k_gemm_wide(GemmArgs g, int tiles_m, int 
   const uint32_t b_step = uint32_t(BK) * ldb_b;
   const uint32_t nk = g.k / BK, k32 = 32 * g.k;
 
-  if constexpr (std::is_same<T, BF16>::value) {
-    if (g.accum) MRL_WIDE_RUN(GEMM_WIDE_BF16_ACC);
-    else MRL_WIDE_RUN(GEMM_WIDE_BF16);
-  } else if constexpr (!A_UNSIGNED) {
-    if (g.accum) MRL_WIDE_RUN(GEMM_WIDE_I8_ACC);
-    else MRL_WIDE_RUN(GEMM_WIDE_I8);
-  } else {
-    if (g.accum) MRL_WIDE_RUN(GEMM_WIDE_U8_ACC);
-    else MRL_WIDE_RUN(GEMM_WIDE_U8);
-  }
+  // An accumulating Spec loads C's old values in nine of its first steps and adds them to the
+  // accumulators a step later: one step after the other when K is short, with two or eleven steps
+  // of the loop between them when K has room.  Those loads sit in the same in-order queue as the
+  // operands', which wait behind them for HBM's latency: a step that carries them takes 2200
+  // cycles longer (bf16 8192^3, cycle stamps), and close together they also ask HBM for all it
+  // delivers (int8 4096^3: 64 MiB of C in the first quarter of the launch).
+  const int spacing = !g.accum ? -1 : nk >= GEMM_WIDE_G11_MIN_STEPS ? 11 : nk >= GEMM_WIDE_G2_MIN_STEPS ? 2 : 0;
+#define MRL_WIDE_PICK(KIND)                                           \
+  do {                                                                \
+    if (spacing < 0) MRL_WIDE_RUN(GEMM_WIDE_##KIND);                  \
+    else if (spacing == 11) MRL_WIDE_RUN(GEMM_WIDE_##KIND##_ACC_G11); \
+    else if (spacing == 2) MRL_WIDE_RUN(GEMM_WIDE_##KIND##_ACC_G2);   \
+    else MRL_WIDE_RUN(GEMM_WIDE_##KIND##_ACC);                        \
+  } while (0)
+  if constexpr (std::is_same<T, BF16>::value) MRL_WIDE_PICK(BF16);
+  else if constexpr (!A_UNSIGNED) MRL_WIDE_PICK(I8);
+  else MRL_WIDE_PICK(U8);
+#undef MRL_WIDE_PICK
 }
 
 // Whole tiles, an even number of k steps, offsets the loop's 32-bit arithmetic can hold.  An

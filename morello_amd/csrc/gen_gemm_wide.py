@@ -182,9 +182,16 @@ class Item:
         self.gap = None
 
 
-def gen(kind, accum, opts=None):
+def gen(kind, accum, opts=None, gap=0):
     """kind: 'u8' (A unsigned bytes), 'i8', 'bf16'.
-    accum: the Spec accumulates into C (its old contents are read)."""
+    accum: the Spec accumulates into C (its old contents are read).
+    gap: k steps of the loop run between two steps that load C's old values (0: those steps follow
+    one another).
+
+    Tried instead of loading C at all: the epilogue's stores as atomic additions that return nothing
+    (global_atomic_add / _f32, one per element, so the sums are the same).  Bit-exact, and the loop
+    is the plain one, but the additions leave a wave at a twelfth of the stores' rate (95 K cycles
+    for a wave's 256 instead of 8 K; bf16 8192^3 accumulating 980 us against 790)."""
     opts = opts or {}     # experiment switches; the shipped loops are generated with none
     unsigned = kind == "u8" and not opts.get("no_valu")
     is_float = kind == "bf16"
@@ -464,8 +471,11 @@ def gen(kind, accum, opts=None):
         block = q // 4
         return block // TN, block % TN, q % 4
 
-    def c_ops(j):
-        """Step j of an accumulating Spec: the old values of block row j - 1 (loaded a step ago) join
+    def c_ops(j, spaced=False):
+        """The j-th of the steps that carry C's old values (spaced: with steps of the loop between
+        them, so that what one of them loaded has long landed when the next one adds it, and the
+        additions go first in the step, the loads behind them with the rest of it to land in).
+        Step j of an accumulating Spec: the old values of block row j - 1 (loaded a step ago) join
         their accumulators, and behind each addition the same register is loaded with block row
         j's.  An addition is three instructions (the accumulator out, the sum, back in); it keeps
         clear of the block's own MFMAs (8 (j - 1) + tn in either slab): an MFMA's result is read
@@ -476,7 +486,7 @@ def gen(kind, accum, opts=None):
         for r in range(32):
             tn, i = r // 4, r % 4
             reg = f"v{OLD_C + r}"
-            g = 4 * r + 1
+            g = 2 * r + 1 if spaced else 4 * r + 1
             add_item = None
             if 1 <= j <= C_STEPS:
                 q = 4 * (TN * (j - 1) + tn) + i
@@ -496,7 +506,8 @@ def gen(kind, accum, opts=None):
                 def add_old(tmp=tmp, reg=reg):
                     # its own wait: the loads of a step are 32 KiB in flight per compute unit, which at
                     # HBM's latency is all the chip can have of C, so the last of them arrive late
-                    e.vm_need(reg)
+                    if not spaced:
+                        e.vm_need(reg)
                     E(f"v_add_f32 {tmp}, {tmp}, {reg}" if is_float else f"v_add_u32 {tmp}, {tmp}, {reg}")
                 add_item = Item(add_old, 1, g + 1, latest - 1, after=read, valu=1)
                 write = Item(lambda q=q, tmp=tmp: E(f"v_accvgpr_write_b32 a{q}, {tmp}"), 1, g + 2, latest, after=add_item, valu=1)
@@ -522,25 +533,77 @@ def gen(kind, accum, opts=None):
             E("s_cmp_lg_u32 s64, 0")
             E("s_cbranch_scc1 10b" if pos == 4 else "s_cbranch_scc0 2f")
 
+    def steady_state(kt):
+        """The emitter's bookkeeping (which load or LDS read fills which register, what is known to
+        have completed) as two ordinary steps before step kt leave it: code that is jumped to is
+        written from this state, whatever precedes it in the text."""
+        n0, saved = len(e.lines), step_no[0]
+        step((kt - 2) % 6)
+        step((kt - 1) % 6)
+        del e.lines[n0:]
+        step_no[0] = saved
+
+    def loop_any(returns):
+        """The loop of six steps as a subroutine: entered at any step (label 1<position>) with the
+        number of steps to run in s64, left after any step; s75 says where to: one of the steps
+        that carry C's old values (label 4<j>), or, zero, the epilogue."""
+        steady_state(0)
+        for pos in range(6):
+            E(f"1{pos}:")
+            step(pos)
+            E("s_sub_u32 s64, s64, 1")
+            E("s_cmp_eq_u32 s64, 0")
+            E("s_cbranch_scc1 20f" if pos < 5 else "s_cbranch_scc0 10b")
+        E("20:")
+        for j in returns:
+            E(f"s_cmp_eq_u32 s75, {j}")
+            E(f"s_cbranch_scc1 4{j}b")
+
     # ---- the k loop ---------------------------------------------------------------------------------
     if trace:
         stamp(82)
         E("s_waitcnt lgkmcnt(0)")
         e.all_lds_done()
-    unrolled = C_STEPS + 2 if accum else 2
-    for j in range(unrolled):
-        extra = c_ops(j) if accum and not opts.get("no_cops") else []
-        step(j % 6, zero_first=(j == 0), extra=extra)
-    if trace:
-        stamp(84)
-        E("s_waitcnt lgkmcnt(0)")
-        e.all_lds_done()
-        E("s_mov_b32 s83, s84")
     early = int(opts.get("early_stores", 0))   # timing experiment (C2's 32 steps only): see below
-    E(f"s_sub_u32 s64, %[nk], {unrolled + (2 if early else 0)}")
-    E("s_cmp_eq_u32 s64, 0")
-    E("s_cbranch_scc1 2f")
-    loop(unrolled)
+    if accum and gap > 0:
+        # C's old values at steps 0, gap + 1, 2 (gap + 1), ...: between them the loop runs `gap` steps.
+        kt = 0
+        for j in range(C_STEPS + 1):
+            if j > 0:
+                E(f"4{j}:")
+                steady_state(kt)
+            step(kt % 6, zero_first=(j == 0), extra=[] if opts.get("no_cops") else c_ops(j, spaced=True))
+            kt += 1
+            if j < C_STEPS:
+                E(f"s_mov_b32 s64, {gap}")
+                E(f"s_mov_b32 s75, {j + 1}")
+                E(f"s_branch 1{kt % 6}f")
+                kt += gap
+        if trace:
+            stamp(84)
+            E("s_waitcnt lgkmcnt(0)")
+            e.all_lds_done()
+            E("s_mov_b32 s83, s84")
+        E("s_mov_b32 s75, 0")
+        E(f"s_sub_u32 s64, %[nk], {kt}")
+        E("s_cmp_eq_u32 s64, 0")
+        E("s_cbranch_scc1 2f")
+        E(f"s_branch 1{kt % 6}f")
+        loop_any(range(1, C_STEPS + 1))
+    else:
+        unrolled = C_STEPS + 2 if accum else 2
+        for j in range(unrolled):
+            extra = c_ops(j) if accum and not opts.get("no_cops") else []
+            step(j % 6, zero_first=(j == 0), extra=extra)
+        if trace:
+            stamp(84)
+            E("s_waitcnt lgkmcnt(0)")
+            e.all_lds_done()
+            E("s_mov_b32 s83, s84")
+        E(f"s_sub_u32 s64, %[nk], {unrolled + (2 if early else 0)}")
+        E("s_cmp_eq_u32 s64, 0")
+        E("s_cbranch_scc1 2f")
+        loop(unrolled)
     E("2:")
     if early:
         # An upper bound for what any reordering of the last step could hide of the epilogue: the
@@ -628,10 +691,20 @@ def gen(kind, accum, opts=None):
 MIN_STEPS = C_STEPS + 4   # k steps a problem needs: the steps that carry C's old values, then the loop
 
 
+SPACED_GAPS = (2, 11)    # loop steps between the steps that carry C's old values, for K long enough
+
+
+def spaced_min_steps(gap):
+    """k steps a problem needs for the variant with `gap` loop steps between C's steps."""
+    return C_STEPS * (gap + 1) + 2
+
+
 def variants():
     for kind in ("u8", "i8", "bf16"):
-        for accum in (False, True):
-            yield f"GEMM_WIDE_{kind.upper()}" + ("_ACC" if accum else ""), kind, accum
+        yield f"GEMM_WIDE_{kind.upper()}", kind, False, 0
+        yield f"GEMM_WIDE_{kind.upper()}_ACC", kind, True, 0
+        for gap in SPACED_GAPS:
+            yield f"GEMM_WIDE_{kind.upper()}_ACC_G{gap}", kind, True, gap
 
 
 def main():
@@ -649,8 +722,10 @@ def main():
             opts["st_flags"] = " " + " ".join(o.split("_")[1:])
     parts = ["// Generated by gen_gemm_wide.py -- do not edit; the generator documents the schedule.\n",
              f"#define GEMM_WIDE_MIN_STEPS {MIN_STEPS}\n"]
-    for name, kind, accum in variants():
-        lines = gen(kind, accum, opts)
+    for gap in SPACED_GAPS:
+        parts.append(f"#define GEMM_WIDE_G{gap}_MIN_STEPS {spaced_min_steps(gap)}\n")
+    for name, kind, accum, gap in variants():
+        lines = gen(kind, accum, opts, gap)
         body = " \\\n".join('  "' + l + '\\n"' for l in lines)
         parts.append(f"#define {name} \\\n{body}\n")
     with open(out_path, "w") as f:

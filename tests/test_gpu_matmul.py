@@ -610,12 +610,45 @@ def test_the_four_wave_kernel_on_a_short_k(gpu, dts, codes, steps):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dts,codes", [((M.u8, M.i8, M.i32), [0, 1, 5]), ((M.i8, M.i8, M.i32), [1, 1, 5]),
+                                       ((M.bf16, M.bf16, M.f32), [7, 7, 6])])
+@pytest.mark.parametrize("steps", [20, 26])
+def test_the_four_wave_kernel_accumulating_over_several_rounds_of_tiles(gpu, dts, codes, steps):
+    """More tiles than compute units (workgroups that start while others are in their loops or
+    storing), on a C that is not zero, with a K that takes the variant with two loop steps between
+    the steps that carry C's old values (26 steps) and the consecutive one (20)."""
+    b, m, n = 33, 512, 1024         # 264 tiles
+    es = 2 if dts[0] == M.bf16 else 1
+    k = steps * 128 // es
+    if dts[0] == M.bf16:
+        A, Bm = synth.normal_bf16(98, 0, (b, m, k)), synth.normal_bf16(98, 1, (b, k, n))
+        C0 = synth.normal_f32(98, 2, (b, m, n), 30.0)
+    else:
+        A = synth.uniform_u8(98, 0, (b, m, k)) if dts[0] == M.u8 else synth.uniform_i8(98, 0, (b, m, k))
+        Bm = synth.uniform_i8(98, 1, (b, k, n))
+        C0 = (synth.uniform_i8(98, 2, (b, m, n)).astype(np.int32) * 1000003)
+    spec = M.MatmulAccum([b, m, k, n], dts)
+    assert spec.plan().kernels == ["k_gemm_wide"]
+    want = orc.matmul([b, m, k, n], codes, A, Bm, C0.copy(), True)
+    bufs = [M.DeviceBuffer.from_numpy(x) for x in (A, Bm, C0)]
+    spec.run_device([x.ptr for x in bufs])
+    got = bufs[2].to_numpy(C0.dtype, (b, m, n))
+    for x in bufs:
+        x.free()
+    if dts[2] == M.i32:
+        assert np.array_equal(got, want)
+    else:
+        assert rel_err(got, want) < 1e-5
+
+
 @pytest.mark.parametrize("dts,codes", [((M.u8, M.i8, M.i32), [0, 1, 5]), ((M.bf16, M.bf16, M.f32), [7, 7, 6])])
-@pytest.mark.parametrize("steps", [12, 14, 16, 18, 20, 22, 24, 28])
+@pytest.mark.parametrize("steps", [12, 14, 16, 18, 20, 22, 24, 26, 28, 30, 32, 98, 100, 102])
 def test_the_four_wave_kernel_accumulating_over_every_loop_exit(gpu, dts, codes, steps):
     """An accumulating Spec runs ten unrolled steps (the first eight load C's old values) and then a
-    loop of six that is entered at its fifth step and left after any two: every number of steps
-    modulo six, from the shortest K the kernel takes, against the oracle on a C that is not zero."""
+    loop of six that is entered at its fifth step and left after any two; from 26 and from 98
+    steps on, the steps with C's old values have two / eleven steps of the loop between them and
+    the loop is left after any step: every number of steps modulo six for each of the three,
+    from the shortest K the kernel takes, against the oracle on a C that is not zero."""
     b, m, n = 2, 256, 512
     es = 2 if dts[0] == M.bf16 else 1
     k = steps * 128 // es
