@@ -712,18 +712,33 @@ int run_softmax(const mrl_spec &s, void *const *params, Workspace &ws) {
                                      cols, scratch, ws.stream));
   } else if (s.scan_dim < last && dense_row_major(in.t) && dense_row_major(out.t) && in.count < (1ull << 31) &&
              [&] {
-               // The tensor as [before][scan][after].  The kernel that scans an outer dim takes 64
-               // positions of `after` per workgroup and walks the scan dim in a loop: too few
-               // workgroups (or an `after` too short for it) make that loop the whole run time.
                uint64_t after = 1;
                for (uint32_t d = s.scan_dim + 1; d < s.rank; d++) after *= s.spec_shape[d];
-               const uint64_t groups = in.count / s.spec_shape[s.scan_dim] / after * ((after + 63) / 64);
-               // Small tensors: three or four launches, ~14 us, against the one kernel's measured
-               // 2.5 us + 10 ns per scan step (generic) or 5 us + 50 ns (24 ns from 512 steps on).
+               return after >= 16;
+             }()) {
+    // The tensor as [before][scan][after] with `after` contiguous: the column kernel, 64
+    // positions of `after` per workgroup; with few columns the scan dim is shared out as well.
+    const uint32_t scan = s.spec_shape[s.scan_dim];
+    uint64_t before = 1, after = 1;
+    for (uint32_t d = 0; d < s.scan_dim; d++) before *= s.spec_shape[d];
+    for (uint32_t d = s.scan_dim + 1; d < s.rank; d++) after *= s.spec_shape[d];
+    mrl::Strided vi, vo;
+    vi.dtype = vo.dtype = MRL_F32, vi.rank = vo.rank = 3;
+    for (uint32_t d = 0; d < MRL_MAX_RANK; d++) vi.shape[d] = vo.shape[d] = 1, vi.stride[d] = vo.stride[d] = 0;
+    vi.shape[0] = vo.shape[0] = uint32_t(before), vi.shape[1] = vo.shape[1] = scan, vi.shape[2] = vo.shape[2] = uint32_t(after);
+    vi.stride[0] = vo.stride[0] = int64_t(scan) * after, vi.stride[1] = vo.stride[1] = int64_t(after), vi.stride[2] = vo.stride[2] = 1;
+    vi.ptr = in.t.ptr, vo.ptr = out.t.ptr;
+    void *pairs = nullptr;
+    if (const size_t bytes = mrl::softmax_cols_scratch_bytes(before * ((after + 63) / 64), scan)) HIP_TRY(ws.alloc(&pairs, bytes));
+    HIP_TRY(mrl::launch_softmax_generic(vi, vo, 1, pairs, ws.stream));
+  } else if (s.scan_dim < last && dense_row_major(in.t) && dense_row_major(out.t) && in.count < (1ull << 31) &&
+             [&] {
+               // Fewer than 16 contiguous elements behind the scan dim: the generic kernel, a
+               // wavefront per line with strided accesses, measured 2.5 us + 10 ns per scan step on
+               // small tensors; against it three or four launches, ~14 us.
                const double scan = s.spec_shape[s.scan_dim];
-               if (in.count <= (1u << 20))
-                 return (after < 16 ? 2.5 + 0.010 * scan : 5.0 + (scan < 512 ? 0.050 : 0.024) * scan) > 15.0;
-               return after < 16 || groups < 256;
+               if (in.count <= (1u << 20)) return 2.5 + 0.010 * scan > 15.0;
+               return true;
              }()) {
     // Scan dim made innermost by a transposing Move, the row kernels, and a Move back: three
     // passes of tuned kernels ([2149, 172] over dim 0: 57 -> 9 us; [1818, 10]: 23 -> 8 us).
@@ -749,7 +764,7 @@ int run_softmax(const mrl_spec &s, void *const *params, Workspace &ws) {
     as_given.ptr = out.t.ptr;
     HIP_TRY(mrl::launch_move_strided(as_turned, as_given, ws.stream));
   } else {
-    HIP_TRY(mrl::launch_softmax_generic(in.t, out.t, s.scan_dim, ws.stream));
+    HIP_TRY(mrl::launch_softmax_generic(in.t, out.t, s.scan_dim, nullptr, ws.stream));
   }
   return finish_output(out, ws);
 }
@@ -879,7 +894,7 @@ int run_compose_msm(const mrl_spec &s, void *const *params, Workspace &ws) {
     sv.ptr = sbuf, sv.dtype = MRL_F32, sv.rank = 3;
     sv.shape[0] = b, sv.shape[1] = m, sv.shape[2] = n2, sv.shape[3] = sv.shape[4] = 1;
     sv.stride[0] = int64_t(m) * n2, sv.stride[1] = n2, sv.stride[2] = 1, sv.stride[3] = sv.stride[4] = 0;
-    HIP_TRY(mrl::launch_softmax_generic(sv, sv, 2, ws.stream));
+    HIP_TRY(mrl::launch_softmax_generic(sv, sv, 2, nullptr, ws.stream));
   }
   st.spec_shape[2] = n2, st.spec_shape[3] = n;
   st.dtypes[0] = p_bf16 ? MRL_BF16 : MRL_F32, st.dtypes[1] = s.dtypes[0], st.dtypes[2] = s.dtypes[3];

@@ -919,11 +919,23 @@ __global__ __launch_bounds__(256) void k_softmax_generic(SM p) {
 // and its WAVES waves (16 for long scan dims) split the scan dim; each lane keeps the online (max, denominator) pair of
 // morello/src/spec.rs:96-106 over its share, the shares are merged through LDS with the
 // parts formula (spec.rs:107-132), and a second sweep writes exp(x - max) / denominator.
+// With few columns (fewer workgroups than compute units) the scan dim is also cut into `chunks`
+// pieces of chunk_len steps, blockIdx.y naming the piece, and the work into two launches
+// (morello/src/scheduling/parallel_softmax.rs:24-223 on the GPU's grid): PHASE 1 leaves every
+// piece's pair in `pairs` ([column tile][piece][lane]), PHASE 2 merges a column's pairs and writes
+// its own piece.  PHASE 0 is the whole Softmax in one launch.
 struct SMC {
   SM s;
   uint32_t fast, fast_tiles;
+  uint32_t chunks, chunk_len;
+  float2 *pairs;
 };
-template <int WAVES>
+__device__ inline void merge_pair(float &m, float &d, float om, float od) {
+  const float nm = (om != om || m != m) ? __uint_as_float(0x7fc00000u) : fmaxf(m, om);
+  d = d * expf(m - nm) + od * expf(om - nm);
+  m = nm;
+}
+template <int WAVES, int PHASE>
 __global__ __launch_bounds__(64 * WAVES) void k_softmax_cols(SMC q) {
   const SM &p = q.s;
   __shared__ float sm_max[WAVES][64], sm_den[WAVES][64];
@@ -941,42 +953,65 @@ __global__ __launch_bounds__(64 * WAVES) void k_softmax_cols(SMC q) {
   }
   const bool live = f < p.shape[q.fast];
   ibase += f, obase += f;  // unit stride on both sides
-  const uint32_t n = p.shape[p.scan_dim];
+  const uint32_t first = PHASE == 0 ? 0 : blockIdx.y * q.chunk_len;
+  const uint32_t n = PHASE == 0 ? p.shape[p.scan_dim] : min(p.shape[p.scan_dim], first + q.chunk_len);
   const int64_t is = p.si[p.scan_dim], os = p.so[p.scan_dim];
-  float mx = -3.40282347e+38f, den = 0.0f;
-  bool nan = false;
-  // Eight loads in flight per lane, then one rescale of the running denominator for the eight.
   constexpr int UNROLL = 8;
-  if (live)
-    for (uint32_t i0 = w; i0 < n; i0 += WAVES * UNROLL) {
-      float x[UNROLL];
-      float nm = mx;
+  float m, d;
+  if (PHASE != 2) {
+    float mx = -3.40282347e+38f, den = 0.0f;
+    bool nan = false;
+    // Eight loads in flight per lane, then one rescale of the running denominator for the eight.
+    if (live)
+      for (uint32_t i0 = first + w; i0 < n; i0 += WAVES * UNROLL) {
+        float x[UNROLL];
+        float nm = mx;
+#pragma unroll
+        for (int j = 0; j < UNROLL; j++) {
+          const uint32_t i = i0 + j * WAVES;
+          x[j] = i < n ? p.in[ibase + i * is] : -3.40282347e+38f;
+          nan |= x[j] != x[j];
+          nm = fmaxf(nm, x[j]);
+        }
+        float add = 0.0f;
+#pragma unroll
+        for (int j = 0; j < UNROLL; j++) add += i0 + j * WAVES < n ? expf(x[j] - nm) : 0.0f;
+        den = den * expf(mx - nm) + add;
+        mx = nm;
+      }
+    if (nan) mx = __uint_as_float(0x7fc00000u);
+    sm_max[w][lane] = mx, sm_den[w][lane] = den;
+    __syncthreads();
+    m = sm_max[0][lane], d = sm_den[0][lane];
+#pragma unroll
+    for (int o = 1; o < WAVES; o++) merge_pair(m, d, sm_max[o][lane], sm_den[o][lane]);
+    if (PHASE == 1) {
+      if (w == 0) q.pairs[(uint64_t(blockIdx.x) * q.chunks + blockIdx.y) * 64 + lane] = make_float2(m, d);
+      return;
+    }
+  } else {
+    // The column's pairs: every wave merges its share of the pieces, eight loads in flight at a
+    // time, and the waves' results meet in LDS.
+    const float2 *mine = q.pairs + uint64_t(blockIdx.x) * q.chunks * 64 + lane;
+    m = -3.40282347e+38f, d = 0.0f;
+    for (uint32_t c0 = w; c0 < q.chunks; c0 += WAVES * UNROLL) {
+      float2 pc[UNROLL];
 #pragma unroll
       for (int j = 0; j < UNROLL; j++) {
-        const uint32_t i = i0 + j * WAVES;
-        x[j] = i < n ? p.in[ibase + i * is] : -3.40282347e+38f;
-        nan |= x[j] != x[j];
-        nm = fmaxf(nm, x[j]);
+        const uint32_t c = c0 + j * WAVES;
+        pc[j] = c < q.chunks ? mine[uint64_t(c) * 64] : make_float2(-3.40282347e+38f, 0.0f);
       }
-      float add = 0.0f;
 #pragma unroll
-      for (int j = 0; j < UNROLL; j++) add += i0 + j * WAVES < n ? expf(x[j] - nm) : 0.0f;
-      den = den * expf(mx - nm) + add;
-      mx = nm;
+      for (int j = 0; j < UNROLL; j++) merge_pair(m, d, pc[j].x, pc[j].y);
     }
-  if (nan) mx = __uint_as_float(0x7fc00000u);
-  sm_max[w][lane] = mx, sm_den[w][lane] = den;
-  __syncthreads();
-  float m = sm_max[0][lane], d = sm_den[0][lane];
+    sm_max[w][lane] = m, sm_den[w][lane] = d;
+    __syncthreads();
+    m = sm_max[0][lane], d = sm_den[0][lane];
 #pragma unroll
-  for (int o = 1; o < WAVES; o++) {
-    const float om = sm_max[o][lane], od = sm_den[o][lane];
-    const float nm = (om != om || m != m) ? __uint_as_float(0x7fc00000u) : fmaxf(m, om);
-    d = d * expf(m - nm) + od * expf(om - nm);
-    m = nm;
+    for (int o = 1; o < WAVES; o++) merge_pair(m, d, sm_max[o][lane], sm_den[o][lane]);
   }
   if (live)
-    for (uint32_t i0 = w; i0 < n; i0 += WAVES * UNROLL) {
+    for (uint32_t i0 = first + w; i0 < n; i0 += WAVES * UNROLL) {
       float x[UNROLL];
 #pragma unroll
       for (int j = 0; j < UNROLL; j++) {
@@ -1400,7 +1435,21 @@ hipError_t launch_conv_generic(const Strided &img, const Strided &filt, const St
   return mrl::plan::last_error();
 }
 
-hipError_t launch_softmax_generic(const Strided &in, const Strided &out, uint32_t scan_dim,
+// Pieces the scan dim is cut into when the column kernel would have `blocks` workgroups: none
+// (1) when those fill the chip or the scan dim is short; else enough for about 1024 workgroups,
+// each piece at least 32 steps (a 256-thread workgroup takes 32 steps in one unrolled pass).
+uint32_t softmax_cols_chunks(uint64_t blocks, uint32_t scan) {
+  if (blocks >= 256 || scan < 128) return 1;
+  const uint64_t want = (1024 + blocks - 1) / blocks;
+  return uint32_t(std::max<uint64_t>(1, std::min<uint64_t>({want, scan / 32, 256})));
+}
+
+size_t softmax_cols_scratch_bytes(uint64_t blocks, uint32_t scan) {
+  const uint32_t chunks = softmax_cols_chunks(blocks, scan);
+  return chunks > 1 ? size_t(blocks) * chunks * 64 * sizeof(float2) : 0;
+}
+
+hipError_t launch_softmax_generic(const Strided &in, const Strided &out, uint32_t scan_dim, void *scratch,
                                   hipStream_t stream) {
   SM p;
   p.in = (const float *)in.ptr, p.out = (float *)out.ptr;
@@ -1419,10 +1468,25 @@ hipError_t launch_softmax_generic(const Strided &in, const Strided &out, uint32_
     if (d != scan_dim && in.shape[d] >= 16 && in.stride[d] == 1 && out.stride[d] == 1) {
       SMC q;
       q.s = p, q.fast = d, q.fast_tiles = (in.shape[d] + 63) / 64;
+      q.chunks = 1, q.chunk_len = in.shape[scan_dim], q.pairs = nullptr;
       const uint64_t blocks = lines / in.shape[d] * q.fast_tiles;
       if (blocks > 0x7fffffffull) break;
-      if (in.shape[scan_dim] >= 512) MRL_LAUNCH(k_softmax_cols<16>, dim3(uint32_t(blocks)), dim3(1024), 0, stream, q);
-      else MRL_LAUNCH(k_softmax_cols<4>, dim3(uint32_t(blocks)), dim3(256), 0, stream, q);
+      const uint32_t chunks = scratch ? softmax_cols_chunks(blocks, in.shape[scan_dim]) : 1;
+      if (chunks > 1) {
+        // Few columns: the scan dim shared out over blockIdx.y as well, in two launches.
+        q.chunks = chunks, q.chunk_len = (in.shape[scan_dim] + chunks - 1) / chunks, q.pairs = (float2 *)scratch;
+        const double count = double(lines) * in.shape[scan_dim];
+        // Measured 2.5-4.4 TB/s over their 12 bytes an element; a workgroup's chain of passes over
+        // its piece (32 steps a pass) is what small problems take: 2149 x 172 11 us, 100000 x 64 45 us.
+        const double chain_ns = 2500.0 + 700.0 * ((q.chunk_len + 31) / 32);
+        plan::work(plan::UNIT_STREAM, 0, 5.2 * count, 0, chain_ns);
+        MRL_LAUNCH((k_softmax_cols<4, 1>), dim3(uint32_t(blocks), chunks), dim3(256), 0, stream, q);
+        plan::work(plan::UNIT_STREAM, 0, 10.4 * count, 0, chain_ns);
+        MRL_LAUNCH((k_softmax_cols<4, 2>), dim3(uint32_t(blocks), chunks), dim3(256), 0, stream, q);
+        return mrl::plan::last_error();
+      }
+      if (in.shape[scan_dim] >= 512) MRL_LAUNCH((k_softmax_cols<16, 0>), dim3(uint32_t(blocks)), dim3(1024), 0, stream, q);
+      else MRL_LAUNCH((k_softmax_cols<4, 0>), dim3(uint32_t(blocks)), dim3(256), 0, stream, q);
       return mrl::plan::last_error();
     }
   const uint32_t blocks = uint32_t((lines + 3) / 4);

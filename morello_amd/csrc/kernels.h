@@ -42,7 +42,12 @@ hipError_t launch_matmul_generic(const Strided &a, const Strided &b, const Strid
                                  hipStream_t stream);
 hipError_t launch_conv_generic(const Strided &img, const Strided &filt, const Strided &out,
                                int accum, hipStream_t stream);
-hipError_t launch_softmax_generic(const Strided &in, const Strided &out, uint32_t scan_dim,
+// `scratch`: softmax_cols_scratch_bytes(blocks, scan) bytes when the caller wants a scan over an
+// outer dim of few columns shared out over workgroups (blocks = lines / columns * ceil(columns / 64)
+// for the contiguous dim the column kernel would take); nullptr: one launch whatever the shape.
+uint32_t softmax_cols_chunks(uint64_t blocks, uint32_t scan);
+size_t softmax_cols_scratch_bytes(uint64_t blocks, uint32_t scan);
+hipError_t launch_softmax_generic(const Strided &in, const Strided &out, uint32_t scan_dim, void *scratch,
                                   hipStream_t stream);
 hipError_t launch_fill_zero(void *ptr, uint64_t bytes, hipStream_t stream);
 // Move Spec: element-wise copy with dtype conversion between two arbitrary layouts.

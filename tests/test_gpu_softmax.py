@@ -109,13 +109,47 @@ def test_softmax_over_an_outer_dim_in_one_kernel(gpu, shape, dim):
     _softmax_outer(shape, dim)
 
 
+@pytest.mark.parametrize("shape,dim,grid", [((2048, 4096), 0, (64, 16, 1)), ((2149, 172), 0, (3, 67, 1)),
+                                            ((100000, 64), 0, (1, 256, 1)), ((5, 1000, 130), 1, (15, 31, 1)),
+                                            ((3, 129, 8, 16), 1, (6, 4, 1))])
+def test_softmax_over_an_outer_dim_of_few_columns(gpu, shape, dim, grid):
+    """Fewer column tiles than compute units: the scan dim is cut into pieces as well (ragged last
+    pieces, ragged column tiles, dims before and behind the scan dim), one launch leaves the
+    pieces' (max, denominator) pairs and a second merges them (spec.rs:107-132) and writes.  A
+    column with a NaN is NaN throughout, one of -inf only too, one with a single +inf as the
+    reference's interpreter has it; the others are untouched by them."""
+    plan = M.Softmax(list(shape), dim).plan()
+    assert plan.kernels == ["k_softmax_cols", "k_softmax_cols"] and plan.steps[0].grid == grid
+    _softmax_outer(shape, dim)
+    x = synth.normal_f32(207, 0, shape, std=3.0)
+    xs = np.moveaxis(x, dim, -1).copy()
+    flat = xs.reshape(-1, shape[dim])
+    flat[0, shape[dim] // 2] = np.nan
+    flat[1, :] = -np.inf
+    flat[2, shape[dim] - 1] = np.inf
+    x = np.ascontiguousarray(np.moveaxis(xs, -1, dim))
+    got = run_spec(M.Softmax(list(shape), dim), [x, np.zeros(shape, np.float32)])
+    want = orc.softmax(list(shape), dim, x)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    tol = 1e-5 if shape[dim] <= 4096 else 2e-4      # the oracle's own f32 sum, as above
+    assert (np.abs(got[ok] - want[ok]) <= tol * np.abs(want[ok]) + 1e-12).all()
+
+
 def _softmax_outer(shape, dim):
     """The scan dim is not the contiguous one: 64 columns per workgroup, the scan dim split over
-    its 4 or 16 waves (short and long scan dims, ragged column tiles and scan lengths)."""
+    its 4 or 16 waves (short and long scan dims, ragged column tiles and scan lengths).  1e-5
+    against the value computed in f64, and against the oracle 1e-5 plus the oracle's own distance
+    from it (its one-by-one f32 sum over 1e5 terms is 1e-4 off by itself)."""
     x = synth.normal_f32(206, 0, shape, std=3.0)
     got = run_spec(M.Softmax(list(shape), dim), [x, np.zeros(shape, np.float32)])
     want = orc.softmax(list(shape), dim, x)
-    assert (np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-12).all()
+    x64 = x.astype(np.float64)
+    e = np.exp(x64 - x64.max(axis=dim, keepdims=True))
+    exact = e / e.sum(axis=dim, keepdims=True)
+    assert (np.abs(got - exact) <= 1e-5 * exact + 1e-12).all()
+    oracle_off = (np.abs(want - exact) / np.maximum(exact, 1e-30)).max()
+    assert (np.abs(got - want) <= (1e-5 + oracle_off) * np.abs(want) + 1e-12).all()
 
 
 def test_softmax_full_size(gpu):

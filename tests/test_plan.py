@@ -116,8 +116,14 @@ def test_plans_follow_shape_dtype_and_layout():
     assert M.Softmax([64, 100000], 1).plan().kernels == ["k_softmax_chunk_stats", "k_softmax_chunk_write"]
     assert M.Softmax([8192, 8192], 1).plan().kernels == ["k_softmax_block"]
     assert M.Softmax([16, 2048, 2048], 1).plan().kernels == ["k_softmax_cols"]
-    # ... unless that kernel would have too few workgroups: scan dim turned innermost and back.
-    assert M.Softmax([2048, 4096], 0).plan().kernels == ["k_move_tiled32", "k_softmax_regs", "k_move_tiled32"]
+    # ... with too few columns for that, the scan dim is shared out over workgroups as well: a
+    # launch for the pieces' (max, denominator) pairs, one that merges them and writes.
+    p = M.Softmax([2048, 4096], 0).plan()
+    assert p.kernels == ["k_softmax_cols", "k_softmax_cols"] and p.steps[0].grid == (64, 16, 1)
+    assert p.steps[1].grid == (64, 16, 1) and p.steps[0].bytes == pytest.approx(5.2 * 2048 * 4096)
+    assert p.scratch_bytes == 64 * 16 * 64 * 8
+    # Fewer than 16 contiguous elements behind the scan dim: scan dim turned innermost and back.
+    assert M.Softmax([45, 1963, 4], 1).plan().kernels[0].startswith("k_move") and len(M.Softmax([45, 1963, 4], 1).plan().kernels) == 4
     assert M.Softmax([100000, 67], 1).plan().kernels == ["k_softmax_short"]
     # Moves: transpose tiled through LDS, Packed destination gathered, plain copy.
     sq = [4096, 4096]
