@@ -646,7 +646,22 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
   } else if (implicit_ok && (forced == 0 || forced == 2)) {
     // Channel vectors of whole 16-byte chunks: the windows are read where they lie.  (A 1x1 filter
     // needs no window arithmetic: its image is the left operand of a plain Matmul, below.)
-    HIP_TRY(mrl::launch_conv_gemm(conv_args, kind, ws.stream, forced == 2 ? g_forced->conv_tile : 0));
+    // Few output tiles and long windows (deep layers on small images): slices of the window as
+    // batch entries with partial results, summed in slice order, as for a Matmul.
+    const uint32_t splits = forced == 2 ? 1 : mrl::gemm_k_splits(conv_args, kind);
+    if (splits > 1) {
+      void *partial = nullptr;
+      HIP_TRY(ws.alloc(&partial, size_t(splits) * conv_args.m * conv_args.n * 4));
+      mrl::GemmArgs slices = conv_args;
+      slices.batch = splits, slices.k = conv_args.k / splits;
+      slices.sb = int64_t(slices.k), slices.conv.slice_bytes = uint32_t(slices.k * img.elem);
+      slices.c = partial, slices.ldc = conv_args.n, slices.sc = int64_t(conv_args.m) * conv_args.n, slices.accum = 0;
+      HIP_TRY(mrl::launch_conv_gemm(slices, kind, ws.stream, 64));
+      HIP_TRY(mrl::launch_sum_splits(partial, conv_args.c, splits, conv_args.m, conv_args.n, conv_args.ldc,
+                                     s.accum != 0, kind <= 1, ws.stream));
+    } else {
+      HIP_TRY(mrl::launch_conv_gemm(conv_args, kind, ws.stream, forced == 2 ? g_forced->conv_tile : 0));
+    }
   } else if (unfold_ok && (forced == 0 || forced == 3)) {
     // Filters in KRSC order are the B operand stored k-fastest; their rows padded like U's.
     const void *weights = filt.t.ptr;

@@ -24,7 +24,7 @@ hipError_t launch_for(const GemmArgs &g, uint32_t tile, hipStream_t stream) {
 bool conv_gemm_applicable(const GemmArgs &g, int kind) {
   const int es = kind == 3 ? 4 : kind == 2 ? 2 : 1;
   auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-  return g.b_kmajor && g.batch == 1 && g.conv.c_bytes != 0 && g.conv.c_bytes % 16 == 0 &&
+  return g.b_kmajor && (g.batch == 1 || (g.conv.slice_bytes != 0 && g.conv.slice_bytes % 16 == 0)) && g.conv.c_bytes != 0 && g.conv.c_bytes % 16 == 0 &&
          g.conv.image_bytes < (1ull << 31) && g.m >= 1 && g.n >= 1 && g.k >= 1 && g.ldb % (16 / es) == 0 &&
          al16(g.a) && al16(g.b) && (reinterpret_cast<uintptr_t>(g.c) & 3) == 0 && edge_addressable(g, es) &&
          uint64_t((g.m + 63) / 64) * ((g.n + 63) / 64) < (1u << 30);

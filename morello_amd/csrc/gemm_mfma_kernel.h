@@ -396,7 +396,7 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
       const bool a_in = ld_kb + a_kb0 < k_bytes;
       if constexpr (CONV) {
         const auto a_buf = buffer_of(g.a, int64_t(g.conv.image_bytes));
-        const uint32_t kb = uint32_t(ld_kb + a_kb0), pos = kb / g.conv.c_bytes, r = pos / g.conv.fw;
+        const uint32_t kb = blockIdx.y * g.conv.slice_bytes + uint32_t(ld_kb + a_kb0), pos = kb / g.conv.c_bytes, r = pos / g.conv.fw;
         const uint32_t in_window = ((r * g.conv.w + (pos - r * g.conv.fw)) * g.conv.c_bytes) + (kb - pos * g.conv.c_bytes);
 #pragma unroll
         for (int i = 0; i < A_CH; i++)

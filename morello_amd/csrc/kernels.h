@@ -90,6 +90,9 @@ struct GemmArgs {
     uint32_t h, w, oh, ow, fw;
     uint32_t c_bytes;       // bytes of one pixel's channels (a whole number of 16-byte chunks)
     uint64_t image_bytes;   // all of `a`
+    // K shared out over batch entries (each a slice of the windows, a partial result of its own):
+    // bytes of a window a slice starts behind the previous one; 0 = one entry, the whole window.
+    uint32_t slice_bytes;
   } conv = {};
 };
 // kind: 0 = i8 x i8, 1 = u8 x i8, 2 = bf16 x bf16, 3 = f32 x f32; B stored k-fastest (gemm_nt.hip).

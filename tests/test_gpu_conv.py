@@ -109,6 +109,30 @@ def test_conv_as_matmul(gpu, dts, codes, shape, accum):
         assert err < 1e-5
 
 
+@pytest.mark.parametrize("dts,codes", [((M.u8, M.i8, M.i32), [0, 1, 5]), ((M.i8, M.i8, M.i32), [1, 1, 5]),
+                                        ((M.bf16, M.bf16, M.f32), [7, 7, 6]), ((M.f32, M.f32, M.f32), [6, 6, 6])])
+@pytest.mark.parametrize("shape,accum", [((8, 512, 512, 5, 5, 3, 3), False), ((8, 512, 512, 5, 5, 3, 3), True),
+                                         ((3, 200, 256, 6, 7, 4, 4), True)])
+def test_deep_conv_on_small_images_shares_its_windows_out(gpu, dts, codes, shape, accum):
+    """Few output tiles and windows of thousands of elements: the implicit Matmul runs over
+    slices of the window as batch entries whose partial results are then summed in slice order
+    (exact for integers), into an output that may hold old values."""
+    b, f, c, oh, ow, fh, fw = shape
+    plan = M.Conv(shape, dts, accum=accum).plan()
+    assert plan.kernels == ["k_gemm", "k_sum_splits"] and plan.steps[0].grid[1] > 1
+    img = CONV_GEN[dts[0]](133, 0, (b, oh + fh - 1, ow + fw - 1, c))
+    filt = CONV_GEN[dts[1]](133, 1, (f, fh, fw, c))
+    out_np = np.int32 if dts[2] == M.i32 else np.float32
+    out0 = synth.uniform_u8(133, 2, (b, oh, ow, f)).astype(out_np) if accum else np.zeros((b, oh, ow, f), out_np)
+    got = run_spec(M.Conv(shape, dts, accum=accum), [img, filt, out0.copy()])
+    want = orc.conv(list(shape), codes, img, filt, out0.copy(), accum, layouts=[NHWC] * 3)
+    if dts[2] == M.i32:
+        assert np.array_equal(got, want)
+    else:
+        err = float(np.abs(got.astype(np.float64) - want).max() / np.abs(want).max())
+        assert err < 1e-5
+
+
 def test_conv_as_matmul_from_nchw(gpu):
     """Row-major (NCHW / FCRS) tensors at a shape the unfolded path takes: moved to channels-last
     and back around it."""
