@@ -165,7 +165,7 @@ const char *mrl_version(void);
  * number goes up whenever a struct gains or changes a field (2: mrl_matmul_schedule.staging,
  * mrl_action; 3: the Softmax actions).  Every struct is zero-initialised by the caller before
  * its fields are set: fields added later mean "default" when zero. */
-#define MRL_ABI_VERSION 3u
+#define MRL_ABI_VERSION 4u
 uint32_t mrl_abi_version(void);
 
 /* --------------------------------------------------- Spec surface (host) */
@@ -519,10 +519,11 @@ int mrl_compose_plan(const mrl_compose *c, mrl_plan *plan, mrl_plan_step *steps,
  *                               equal tiles (row-major input), a (max, denominator) pair per tile,
  *                               merged by SoftmaxDenominatorAndMaxFromParts
  *                               (scheduling/parallel_softmax.rs:24-223)
- * Each action is a terminal lowering: it runs the Spec to its result.  The reference's actions
- * return a partial Impl whose nested sub-Specs a search expands further; the nested Specs of the
- * three Softmax rewrites are the primitive Specs of this header, so a caller that wants to
- * schedule a stage itself runs the stages one by one instead of the action. */
+ * Every action runs the Spec to its result (mrl_run_action).  The reference's actions return a
+ * partial Impl whose nested sub-Specs a search expands further: the three Softmax rewrites and
+ * BUFFERIZE are such rewrites here too, and mrl_action_apply (below) lists their sub-Specs; every
+ * other action is a leaf, a terminal lowering by the library with a price.  There is no action
+ * for move_relayout / cast or for a partly tiled Conv or Softmax as steps of their own. */
 typedef enum {
   MRL_ACTION_SELECT = 0,
   MRL_ACTION_TILE_OUT_SPLIT = 1,
@@ -555,6 +556,36 @@ int mrl_action_plan(const mrl_spec *spec, const mrl_action *action, mrl_plan *pl
  * to these operands (alignment); the result is the Spec's whatever the action: integer Specs bit
  * for bit, floating-point ones within the Spec's tolerance. */
 int mrl_run_action(const mrl_spec *spec, void *const *params, const mrl_action *action, void *stream);
+/* The children of an action in Morello's sense.  ActionT::apply (scheduling/mod.rs:40-63) turns a
+ * Spec into a partial Impl whose leaves are sub-Specs that the search schedules in turn; for the
+ * actions here that are such rewrites, mrl_action_apply lists those sub-Specs in execution order
+ * with where each of their parameters comes from, and the buffers between them:
+ *   TO_SOFTMAX_PARTS            SoftmaxDenominatorAndUnscaled, DivideVecScalar
+ *                               (scheduling/to_softmax_parts.rs:33-108)
+ *   TO_SOFTMAX_PARTS_RECOMPUTE  SoftmaxDenominatorAndMax, SoftmaxComplete (to_softmax_parts.rs:110-181)
+ *   PARALLEL_SOFTMAX            SoftmaxDenominatorAndMax over [.., parts, scan / parts, ..],
+ *                               SoftmaxDenominatorAndMaxFromParts, SoftmaxComplete
+ *                               (scheduling/parallel_softmax.rs:24-223)
+ *   BUFFERIZE (on the Compose)  Matmul, Softmax, Matmul with the two tensors between them in
+ *                               buffers of the components' output dtype (scheduling/bufferize.rs:24-116)
+ * Every other action is a leaf (n_subspecs = 0): the library runs it as one piece.  Running the
+ * sub-Specs one after the other with mrl_run, each on the buffers its sources name, computes the
+ * Spec; each sub-Spec has actions of its own (mrl_target_actions), which is how a search over this
+ * backend recurses.  Host code: needs no GPU. */
+#define MRL_MAX_SUBSPECS 4
+typedef struct {
+  mrl_spec spec;
+  /* Per parameter of `spec`: i >= 0 = parameter i of the Spec the action was applied to;
+   * -1 - j = intermediate buffer j of the rewrite. */
+  int32_t source[MRL_MAX_PARAMS];
+} mrl_subspec;
+typedef struct {
+  uint32_t n_subspecs;
+  mrl_subspec subspecs[MRL_MAX_SUBSPECS];
+  uint32_t n_intermediates;
+  uint64_t intermediate_bytes[MRL_MAX_SUBSPECS]; /* dense row-major f32 tensors */
+} mrl_rewrite;
+int mrl_action_apply(const mrl_spec *spec, const mrl_action *action, mrl_rewrite *out);
 /* mrl_run_timed for a chosen action: `steps` launches back to back on the default stream between
  * two events (what BuiltArtifact::measure_time does for one schedule, codegen/mod.rs:330-340). */
 int mrl_run_action_timed(const mrl_spec *spec, void *const *params, const mrl_action *action, uint32_t steps,

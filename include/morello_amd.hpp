@@ -233,6 +233,13 @@ class Spec {
     if (!out.empty()) out.resize(mrl_target_actions(&c_, out.data(), uint32_t(out.size())));
     return out;
   }
+  // ActionT::apply (scheduling/mod.rs:40-63): the sub-Specs a rewrite turns this Spec into, with
+  // their parameter sources and the buffers between them; n_subspecs == 0 for a leaf.
+  mrl_rewrite apply(const mrl_action &action) const {
+    mrl_rewrite out{};
+    check(mrl_action_apply(&c_, &action, &out), "action_apply");
+    return out;
+  }
   // Runs the Spec under one of its actions: `params` are device pointers in parameter order.
   void run(const mrl_action &action, void *const *params, void *stream = nullptr) const {
     check(mrl_run_action(&c_, params, &action, stream), "run_action");

@@ -644,11 +644,46 @@ class Action:
                "mrl_run_action_timed")
         return ms.value
 
+    def apply(self) -> "Rewrite":
+        """The action's children (ActionT::apply, scheduling/mod.rs:40-63): for a rewrite, the
+        sub-Specs it turns the Spec into, in execution order, with each parameter's source, and
+        the sizes of the buffers between them; for a leaf, none."""
+        c = B.RewriteC()
+        _check(B.load().mrl_action_apply(C.byref(self.spec._c), C.byref(self._c), C.byref(c)), "mrl_action_apply")
+        subs = []
+        for i in range(c.n_subspecs):
+            sc = c.subspecs[i].spec
+            sub = Spec(SpecKind(sc.kind), list(sc.spec_shape[:sc.rank]), [Dtype(sc.dtypes[j]) for j in range(sc.n_params)],
+                       layouts=[Layout.from_c(sc.layouts[j]) for j in range(sc.n_params)], accum=bool(sc.accum), scan_dim=sc.scan_dim)
+            subs.append((sub, [int(c.subspecs[i].source[j]) for j in range(sc.n_params)]))
+        return Rewrite(subs, [int(c.intermediate_bytes[j]) for j in range(c.n_intermediates)])
+
     def flops(self) -> float:
         return self.spec.flops()
 
     def bytes_used(self, i: int) -> int:
         return self.spec.bytes_used(i)
+
+
+class Rewrite:
+    """What Action.apply returns: `subspecs` = [(Spec, sources)], a source i >= 0 naming parameter i
+    of the Spec the action was applied to and -1 - j the j-th of `intermediate_bytes`."""
+
+    def __init__(self, subspecs, intermediate_bytes):
+        self.subspecs, self.intermediate_bytes = subspecs, intermediate_bytes
+
+    def is_leaf(self) -> bool:
+        return not self.subspecs
+
+    def run_device(self, ptrs: Sequence[int]):
+        """Runs the sub-Specs one after the other with mrl_run, each on the buffers its sources name."""
+        between = [DeviceBuffer(n) for n in self.intermediate_bytes]
+        try:
+            for sub, sources in self.subspecs:
+                sub.run_device([ptrs[i] if i >= 0 else between[-1 - i].ptr for i in sources])
+        finally:
+            for b in between:
+                b.free()
 
 
 def _plan_of(fn, c_spec, where: str) -> Plan:

@@ -12,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libmorello_amd.so")
 
 MAX_PHYS, MAX_RANK, MAX_SPEC_RANK, MAX_PARAMS = 10, 5, 7, 4
-ABI_VERSION = 3   # MRL_ABI_VERSION of include/morello_amd.h
+ABI_VERSION = 4   # MRL_ABI_VERSION of include/morello_amd.h
 
 
 class PhysDimC(C.Structure):
@@ -43,6 +43,18 @@ class SpecC(C.Structure):
         ("dtypes", C.c_int32 * MAX_PARAMS),
         ("layouts", LayoutC * MAX_PARAMS),
     ]
+
+
+MAX_SUBSPECS = 4
+
+
+class SubspecC(C.Structure):
+    _fields_ = [("spec", SpecC), ("source", C.c_int32 * MAX_PARAMS)]
+
+
+class RewriteC(C.Structure):
+    _fields_ = [("n_subspecs", C.c_uint32), ("subspecs", SubspecC * MAX_SUBSPECS), ("n_intermediates", C.c_uint32),
+                ("intermediate_bytes", C.c_uint64 * MAX_SUBSPECS)]
 
 
 MAX_COMPONENTS = 8
@@ -141,6 +153,7 @@ SIGNATURES = {
     "mrl_stream_release": (C.c_int, [C.c_void_p]),
     "mrl_device_mem_free": (C.c_int, [C.POINTER(C.c_size_t)]),
     "mrl_abi_version": (C.c_uint32, []),
+    "mrl_action_apply": (C.c_int, [C.POINTER(SpecC), C.POINTER(ActionC), C.POINTER(RewriteC)]),
     "mrl_run_action_timed": (C.c_int, [C.POINTER(SpecC), _VPP, C.POINTER(ActionC), C.c_uint32, C.POINTER(C.c_double)]),
     "mrl_stream_destroy": (C.c_int, [C.c_void_p]),
     "mrl_target_id": (C.c_char_p, []),

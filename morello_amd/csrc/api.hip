@@ -1820,7 +1820,7 @@ int part_spec(int kind, const uint32_t *shape, uint32_t rank, uint32_t scan_dim,
 }
 
 // A Softmax Spec through one of the reference's rewrites instead of the fused kernels, each stage
-// a primitive Spec of its own (parts.hip), the tensors between the stages in scratch memory:
+// a primitive Spec of its own (parts.hip), the tensors between the stages in intermediate buffers:
 //   TO_SOFTMAX_PARTS            SoftmaxDenominatorAndUnscaled, then DivideVecScalar on the output
 //                               (scheduling/to_softmax_parts.rs:33-108)
 //   TO_SOFTMAX_PARTS_RECOMPUTE  SoftmaxDenominatorAndMax, then SoftmaxComplete, which forms the
@@ -1828,35 +1828,40 @@ int part_spec(int kind, const uint32_t *shape, uint32_t rank, uint32_t scan_dim,
 //   PARALLEL_SOFTMAX            the same with the first stage split along the scan dim in `parts`
 //                               tiles (scheduling/parallel_softmax.rs:24-223): a (max, denominator)
 //                               pair per tile, merged by SoftmaxDenominatorAndMaxFromParts
-int run_softmax_rewrite(const mrl_spec &s, void *const *params, Workspace &ws, const mrl_action &a) {
+// Written once, as the list of sub-Specs with their parameter sources (mrl_rewrite): what
+// mrl_action_apply hands out is what run_rewrite runs.
+int softmax_rewrite(const mrl_spec &s, const mrl_action &a, mrl_rewrite *rw) {
   if (s.kind != MRL_SPEC_SOFTMAX || s.dtypes[0] != MRL_F32 || s.dtypes[1] != MRL_F32) return MRL_ERR_UNSUPPORTED;
+  std::memset(rw, 0, sizeof *rw);
   const uint32_t scan = s.spec_shape[s.scan_dim];
   uint64_t lines = 1;
   for (uint32_t d = 0; d < s.rank; d++)
     if (d != s.scan_dim) lines *= s.spec_shape[d];
   int rc;
-  mrl_spec st;
+  auto child = [&](int kind, const uint32_t *shape, uint32_t rank, uint32_t scan_dim, std::initializer_list<int32_t> sources) -> mrl_spec * {
+    mrl_subspec &c = rw->subspecs[rw->n_subspecs++];
+    rc = part_spec(kind, shape, rank, scan_dim, &c.spec);
+    uint32_t i = 0;
+    for (int32_t src : sources) c.source[i++] = src;
+    return &c.spec;
+  };
+  auto intermediate = [&](uint64_t bytes) { rw->intermediate_bytes[rw->n_intermediates] = bytes; return -1 - int32_t(rw->n_intermediates++); };
   if (a.kind == MRL_ACTION_TO_SOFTMAX_PARTS) {
-    void *denom = nullptr;
-    HIP_TRY(ws.alloc(&denom, lines * sizeof(float)));
-    if ((rc = part_spec(MRL_SPEC_SOFTMAX_DENOMINATOR_AND_UNSCALED, s.spec_shape, s.rank, s.scan_dim, &st)) != MRL_OK) return rc;
-    st.layouts[0] = s.layouts[0], st.layouts[2] = s.layouts[1];
-    void *p1[3] = {params[0], denom, params[1]};
-    if ((rc = dispatch(st, p1, ws)) != MRL_OK) return rc;
-    if ((rc = part_spec(MRL_SPEC_DIVIDE_VEC_SCALAR, s.spec_shape, s.rank, s.scan_dim, &st)) != MRL_OK) return rc;
-    st.layouts[0] = s.layouts[1];
-    void *p2[2] = {params[1], denom};
-    return dispatch(st, p2, ws);
+    const int32_t denom = intermediate(lines * sizeof(float));
+    mrl_spec *st = child(MRL_SPEC_SOFTMAX_DENOMINATOR_AND_UNSCALED, s.spec_shape, s.rank, s.scan_dim, {0, denom, 1});
+    if (rc != MRL_OK) return rc;
+    st->layouts[0] = s.layouts[0], st->layouts[2] = s.layouts[1];
+    st = child(MRL_SPEC_DIVIDE_VEC_SCALAR, s.spec_shape, s.rank, s.scan_dim, {1, denom});
+    if (rc != MRL_OK) return rc;
+    st->layouts[0] = s.layouts[1];
+    return MRL_OK;
   }
-  void *mx = nullptr, *denom = nullptr;
-  HIP_TRY(ws.alloc(&mx, lines * sizeof(float)));
-  HIP_TRY(ws.alloc(&denom, lines * sizeof(float)));
+  const int32_t mx = intermediate(lines * sizeof(float)), denom = intermediate(lines * sizeof(float));
   if (a.kind == MRL_ACTION_TO_SOFTMAX_PARTS_RECOMPUTE) {
-    if ((rc = part_spec(MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX, s.spec_shape, s.rank, s.scan_dim, &st)) != MRL_OK) return rc;
-    st.layouts[0] = s.layouts[0];
-    void *p1[3] = {params[0], mx, denom};
-    if ((rc = dispatch(st, p1, ws)) != MRL_OK) return rc;
-  } else {
+    mrl_spec *st = child(MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX, s.spec_shape, s.rank, s.scan_dim, {0, mx, denom});
+    if (rc != MRL_OK) return rc;
+    st->layouts[0] = s.layouts[0];
+  } else if (a.kind == MRL_ACTION_PARALLEL_SOFTMAX) {
     // The tiles are a dim of their own: [.., scan, ..] read as [.., parts, scan / parts, ..], which
     // is the same buffer when the input is row-major and the tiles are equal.
     const uint32_t parts = a.parts;
@@ -1873,20 +1878,68 @@ int run_softmax_rewrite(const mrl_spec &s, void *const *params, Workspace &ws, c
       if (d == s.scan_dim) split[o++] = parts, split[o++] = scan / parts;
       else split[o++] = s.spec_shape[d];
     }
-    void *tile_max = nullptr, *tile_denom = nullptr;
-    HIP_TRY(ws.alloc(&tile_max, lines * parts * sizeof(float)));
-    HIP_TRY(ws.alloc(&tile_denom, lines * parts * sizeof(float)));
-    if ((rc = part_spec(MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX, split, s.rank + 1, s.scan_dim + 1, &st)) != MRL_OK) return rc;
-    void *p1[3] = {params[0], tile_max, tile_denom};
-    if ((rc = dispatch(st, p1, ws)) != MRL_OK) return rc;
-    if ((rc = part_spec(MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX_FROM_PARTS, tiles, s.rank, s.scan_dim, &st)) != MRL_OK) return rc;
-    void *p2[4] = {tile_max, tile_denom, mx, denom};
-    if ((rc = dispatch(st, p2, ws)) != MRL_OK) return rc;
+    const int32_t tile_max = intermediate(lines * parts * sizeof(float)), tile_denom = intermediate(lines * parts * sizeof(float));
+    child(MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX, split, s.rank + 1, s.scan_dim + 1, {0, tile_max, tile_denom});
+    if (rc != MRL_OK) return rc;
+    child(MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX_FROM_PARTS, tiles, s.rank, s.scan_dim, {tile_max, tile_denom, mx, denom});
+    if (rc != MRL_OK) return rc;
+  } else {
+    return MRL_ERR_UNSUPPORTED;
   }
-  if ((rc = part_spec(MRL_SPEC_SOFTMAX_COMPLETE, s.spec_shape, s.rank, s.scan_dim, &st)) != MRL_OK) return rc;
-  st.layouts[0] = s.layouts[0], st.layouts[3] = s.layouts[1];
-  void *p3[4] = {params[0], mx, denom, params[1]};
-  return dispatch(st, p3, ws);
+  mrl_spec *st = child(MRL_SPEC_SOFTMAX_COMPLETE, s.spec_shape, s.rank, s.scan_dim, {0, mx, denom, 1});
+  if (rc != MRL_OK) return rc;
+  st->layouts[0] = s.layouts[0], st->layouts[3] = s.layouts[1];
+  return MRL_OK;
+}
+
+// The attention-shaped Compose with both tensors between its components in buffers
+// (scheduling/bufferize.rs:24-116): S = Q . KT and P = softmax(S) as f32 tensors, row-major.
+int compose_msm_rewrite(const mrl_spec &s, mrl_rewrite *rw) {
+  if (s.kind != MRL_SPEC_COMPOSE_MSM) return MRL_ERR_UNSUPPORTED;
+  std::memset(rw, 0, sizeof *rw);
+  const uint32_t b = s.spec_shape[0], m = s.spec_shape[1], k = s.spec_shape[2], n2 = s.spec_shape[3], n = s.spec_shape[4];
+  const uint64_t scores = uint64_t(b) * m * n2 * sizeof(float);
+  rw->n_intermediates = 2, rw->intermediate_bytes[0] = rw->intermediate_bytes[1] = scores;
+  rw->n_subspecs = 3;
+  auto fill = [&](mrl_subspec &c, int kind, std::initializer_list<uint32_t> shape, uint32_t scan_dim, std::initializer_list<int32_t> dtypes,
+                  std::initializer_list<int32_t> sources) {
+    std::memset(&c, 0, sizeof c);
+    c.spec.kind = kind, c.spec.scan_dim = scan_dim, c.spec.rank = uint32_t(shape.size()), c.spec.n_params = uint32_t(dtypes.size());
+    uint32_t i = 0;
+    for (uint32_t d : shape) c.spec.spec_shape[i++] = d;
+    i = 0;
+    for (int32_t dt : dtypes) c.spec.dtypes[i++] = dt;
+    i = 0;
+    for (int32_t src : sources) c.source[i++] = src;
+    for (i = 0; i < c.spec.n_params; i++) {
+      uint32_t pshape[MRL_MAX_RANK], prank;
+      if (c.source[i] >= 0) c.spec.layouts[i] = s.layouts[c.source[i]];
+      else if (parameter_shape(c.spec, i, pshape, &prank) == MRL_OK) mrl_layout_row_major(pshape, prank, &c.spec.layouts[i]);
+    }
+    return check_spec(&c.spec);
+  };
+  // Parameters of the Compose: V [b, n2, n], Q [b, m, k], KT [b, k, n2], out [b, m, n].
+  int rc;
+  if ((rc = fill(rw->subspecs[0], MRL_SPEC_MATMUL, {b, m, k, n2}, 0, {s.dtypes[1], s.dtypes[2], MRL_F32}, {1, 2, -1})) != MRL_OK) return rc;
+  if ((rc = fill(rw->subspecs[1], MRL_SPEC_SOFTMAX, {b, m, n2}, 2, {MRL_F32, MRL_F32}, {-1, -2})) != MRL_OK) return rc;
+  return fill(rw->subspecs[2], MRL_SPEC_MATMUL, {b, m, n2, n}, 0, {MRL_F32, s.dtypes[0], s.dtypes[3]}, {-2, 0, 3});
+}
+
+int run_softmax_rewrite(const mrl_spec &s, void *const *params, Workspace &ws, const mrl_action &a) {
+  mrl_rewrite rw;
+  int rc;
+  if ((rc = softmax_rewrite(s, a, &rw)) != MRL_OK) return rc;
+  void *between[MRL_MAX_SUBSPECS] = {};
+  for (uint32_t j = 0; j < rw.n_intermediates; j++) HIP_TRY(ws.alloc(&between[j], rw.intermediate_bytes[j]));
+  for (uint32_t c = 0; c < rw.n_subspecs; c++) {
+    void *p[MRL_MAX_PARAMS];
+    for (uint32_t i = 0; i < rw.subspecs[c].spec.n_params; i++) {
+      const int32_t src = rw.subspecs[c].source[i];
+      p[i] = src >= 0 ? params[src] : between[-1 - src];
+    }
+    if ((rc = dispatch(rw.subspecs[c].spec, p, ws)) != MRL_OK) return rc;
+  }
+  return MRL_OK;
 }
 
 // Runs `spec` under `action` through `ws` (a recording Workspace when planning).
@@ -1927,6 +1980,24 @@ int dispatch_action(const mrl_spec &spec, void *const *params, Workspace &ws, co
   return rc;
 }
 }  // namespace
+
+int mrl_action_apply(const mrl_spec *spec, const mrl_action *action, mrl_rewrite *out) {
+  if (!action || !out) return MRL_ERR_NULL;
+  int rc = check_spec(spec);
+  if (rc != MRL_OK) return rc;
+  switch (action->kind) {
+    case MRL_ACTION_TO_SOFTMAX_PARTS:
+    case MRL_ACTION_TO_SOFTMAX_PARTS_RECOMPUTE:
+    case MRL_ACTION_PARALLEL_SOFTMAX: return softmax_rewrite(*spec, *action, out);
+    case MRL_ACTION_BUFFERIZE: return compose_msm_rewrite(*spec, out);
+    default: break;
+  }
+  // A leaf: the action must at least apply to the Spec.
+  mrl_plan plan;
+  if ((rc = mrl_action_plan(spec, action, &plan, nullptr, 0)) != MRL_OK) return rc;
+  std::memset(out, 0, sizeof *out);
+  return MRL_OK;
+}
 
 int mrl_action_plan(const mrl_spec *spec, const mrl_action *action, mrl_plan *plan, mrl_plan_step *steps, uint32_t cap) {
   if (!action) return MRL_ERR_NULL;

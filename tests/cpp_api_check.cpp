@@ -77,6 +77,20 @@ int main() {
     const mrl_matmul_schedule best =
         Spec::matmul({1, 4096, 4096, 4096}, Dtype::Uint8, Dtype::Sint8, Dtype::Sint32).search_schedule();
     EXPECT(best.tile_m == 256 && best.tile_n == 256);
+    // A leaf has no children; the Softmax rewrite to_softmax_parts has two, with one buffer between them.
+    const Spec mm = Spec::matmul({1, 4096, 4096, 4096}, Dtype::Uint8, Dtype::Sint8, Dtype::Sint32);
+    EXPECT(mm.apply(acts[1]).n_subspecs == 0);
+    const uint32_t rows[3] = {16, 2048, 2048};
+    mrl_spec sm{};
+    sm.kind = MRL_SPEC_SOFTMAX, sm.scan_dim = 2, sm.rank = 3, sm.n_params = 2;
+    for (int d = 0; d < 3; d++) sm.spec_shape[d] = rows[d];
+    for (int i = 0; i < 2; i++) sm.dtypes[i] = MRL_F32, mrl_layout_row_major(rows, 3, &sm.layouts[i]);
+    mrl_action parts{};
+    parts.kind = MRL_ACTION_TO_SOFTMAX_PARTS;
+    mrl_rewrite rw{};
+    EXPECT(mrl_action_apply(&sm, &parts, &rw) == MRL_OK && rw.n_subspecs == 2 && rw.n_intermediates == 1);
+    EXPECT(rw.subspecs[0].spec.kind == MRL_SPEC_SOFTMAX_DENOMINATOR_AND_UNSCALED && rw.subspecs[0].source[1] == -1 &&
+           rw.subspecs[1].spec.kind == MRL_SPEC_DIVIDE_VEC_SCALAR && rw.intermediate_bytes[0] == 16 * 2048 * 4);
   }
   std::printf("cpp api ok\n");
   return 0;

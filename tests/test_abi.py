@@ -39,6 +39,9 @@ def test_struct_sizes_match_the_header():
     assert C.sizeof(B.PhysDimC) == 8
     assert C.sizeof(B.LayoutC) == 84
     assert C.sizeof(B.SpecC) == 4 * 4 + 7 * 4 + 4 + 4 * 4 + 4 * 84
+    # mrl_subspec = mrl_spec + 4 sources; mrl_rewrite = count, 4 of those, count, 4 sizes (8-byte aligned)
+    assert C.sizeof(B.SubspecC) == C.sizeof(B.SpecC) + 16
+    assert C.sizeof(B.RewriteC) == 4 + 4 * C.sizeof(B.SubspecC) + 4 + 4 * 8
 
 
 def test_parameter_shapes_and_directions():

@@ -122,6 +122,43 @@ def test_softmax_actions_against_the_oracle(gpu, shape, dim):
             assert act.n_steps == (3 if act.kind == M.ActionKind.ParallelSoftmax else 2), act
 
 
+@pytest.mark.parametrize("shape,dim", [((6, 640), 1), ((3, 256, 40), 1), ((128, 33), 0)])
+def test_children_of_the_rewrites_compute_the_spec(gpu, shape, dim):
+    """mrl_action_apply: a rewrite's sub-Specs, run one after the other with mrl_run on the buffers
+    their sources name (the intermediates allocated by the caller), give the Softmax."""
+    x = synth.normal_f32(37, 0, shape, 3.0)
+    want = orc.softmax(list(shape), dim, x)
+    rewrites = [a for a in M.Softmax(list(shape), dim).actions() if a.kind != M.ActionKind.Select]
+    assert len(rewrites) >= 2
+    for act in rewrites:
+        rw = act.apply()
+        assert not rw.is_leaf() and sum(rw.intermediate_bytes) <= act.scratch_bytes   # the arena rounds each to 256 bytes
+        bufs = [M.DeviceBuffer.from_numpy(x), M.DeviceBuffer.from_numpy(np.full(shape, 9.0, np.float32))]
+        rw.run_device([b.ptr for b in bufs])
+        got = bufs[1].to_numpy(np.float32, shape)
+        for b in bufs:
+            b.free()
+        assert np.abs(got - want).max() < 1e-5, act
+
+
+def test_children_of_the_bufferized_compose_compute_it(gpu):
+    """The Compose's bufferize as sub-Specs: Matmul, Softmax, Matmul with S and P in f32 buffers of
+    the caller's; with f32 intermediates the result matches the oracle's closed form to 1e-5."""
+    b, m, k, n2, n = 2, 200, 128, 330, 128
+    spec = M.ComposeMSM(b, m, k, n2, n, layouts=[None, None, KT, None])
+    v, q, kmat = (synth.normal_bf16(38, 2, (b, n2, n), 0.5), synth.normal_bf16(38, 0, (b, m, k), 0.5),
+                  synth.normal_bf16(38, 1, (b, n2, k), 0.5))
+    want = orc.compose_msm(b, m, k, n2, n, [7, 7, 7, 6], v, q, kmat, np.zeros((b, m, n), np.float32),
+                           layouts=[None, None, KT_ORC, None])
+    rw = [a for a in spec.actions() if a.kind == M.ActionKind.Bufferize][0].apply()
+    bufs = [M.DeviceBuffer.from_numpy(a) for a in (v, q, kmat, np.full((b, m, n), 7.5, np.float32))]
+    rw.run_device([x.ptr for x in bufs])
+    got = bufs[3].to_numpy(np.float32, (b, m, n))
+    for x in bufs:
+        x.free()
+    assert rel_err(got, want) < 1e-5
+
+
 def test_softmax_actions_keep_the_parameters_layouts(gpu):
     """Input and output in another layout than row-major: the whole-tensor rewrites take them as
     they are, the tiled one (which reads the scan dim as two dims of the same buffer) declines."""

@@ -436,3 +436,44 @@ def test_a_run_launches_what_its_plan_lists(gpu):
         for b in bufs:
             b.free()
         assert launched == steps, (spec.plan(), launched)
+
+
+def test_rewrite_actions_have_children_and_the_others_are_leaves():
+    """mrl_action_apply: the Softmax rewrites and the Compose's bufferize hand out their sub-Specs
+    (scheduling/to_softmax_parts.rs:33-181, parallel_softmax.rs:24-223, bufferize.rs:24-116) with
+    the source of every parameter; what the library runs as one piece has none.  Each child is a
+    Spec of its own with actions of its own: the recursion of a search."""
+    K = M.ActionKind
+    sm = M.Softmax([16, 2048, 2048], 2)
+    by_kind = {}
+    for a in sm.actions():
+        by_kind.setdefault(a.kind, a)
+    assert by_kind[K.Select].apply().is_leaf()
+    rw = by_kind[K.ToSoftmaxParts].apply()
+    assert [(s.kind, src) for s, src in rw.subspecs] == [(M.SpecKind.SoftmaxDenominatorAndUnscaled, [0, -1, 1]),
+                                                         (M.SpecKind.DivideVecScalar, [1, -1])]
+    assert rw.intermediate_bytes == [16 * 2048 * 4]
+    rw = by_kind[K.ToSoftmaxPartsRecompute].apply()
+    assert [(s.kind, src) for s, src in rw.subspecs] == [(M.SpecKind.SoftmaxDenominatorAndMax, [0, -1, -2]),
+                                                         (M.SpecKind.SoftmaxComplete, [0, -1, -2, 1])]
+    rw = by_kind[K.ParallelSoftmax].apply()      # parts = 2
+    assert [(s.kind, s.spec_shape, src) for s, src in rw.subspecs] == [
+        (M.SpecKind.SoftmaxDenominatorAndMax, [16, 2048, 2, 1024], [0, -3, -4]),
+        (M.SpecKind.SoftmaxDenominatorAndMaxFromParts, [16, 2048, 2], [-3, -4, -1, -2]),
+        (M.SpecKind.SoftmaxComplete, [16, 2048, 2048], [0, -1, -2, 1])]
+    assert rw.intermediate_bytes == [16 * 2048 * 4] * 2 + [16 * 2048 * 2 * 4] * 2
+    for sub, _ in rw.subspecs:
+        assert sub.check() == 0 and sub.actions()[0].kind == K.Select and len(sub.plan().kernels) >= 1
+    # The Compose: parameters V, Q, KT, out; S and P between the components as f32.
+    KT = M.layout(0, 2, 1)
+    c5 = M.ComposeMSM(16, 2048, 128, 2048, 128, layouts=[None, None, KT, None])
+    buf = [a for a in c5.actions() if a.kind == K.Bufferize][0].apply()
+    assert [(s.kind, s.spec_shape, list(s.dtypes), src) for s, src in buf.subspecs] == [
+        (M.SpecKind.Matmul, [16, 2048, 128, 2048], [M.bf16, M.bf16, M.f32], [1, 2, -1]),
+        (M.SpecKind.Softmax, [16, 2048, 2048], [M.f32, M.f32], [-1, -2]),
+        (M.SpecKind.Matmul, [16, 2048, 2048, 128], [M.f32, M.bf16, M.f32], [-2, 0, 3])]
+    assert buf.subspecs[0][0].layouts[1] == KT and buf.intermediate_bytes == [16 * 2048 * 2048 * 4] * 2
+    assert len(buf.subspecs[1][0].actions()) > 3          # the Softmax child has the rewrites again
+    assert all(a.apply().is_leaf() for a in c5.actions() if a.kind != K.Bufferize)
+    assert all(a.apply().is_leaf() for a in M.MatmulAccum([1, 512, 512, 512], (M.u8, M.i8, M.i32)).actions())
+    assert all(a.apply().is_leaf() for a in M.Conv([2, 64, 64, 10, 10, 3, 3], (M.u8, M.i8, M.i32)).actions())
