@@ -519,11 +519,22 @@ int mrl_compose_plan(const mrl_compose *c, mrl_plan *plan, mrl_plan_step *steps,
  *                               equal tiles (row-major input), a (max, denominator) pair per tile,
  *                               merged by SoftmaxDenominatorAndMaxFromParts
  *                               (scheduling/parallel_softmax.rs:24-223)
+ *   TO_ACCUM        Matmul / Conv that overwrites: Fill{Zero} on the output, then the accumulating
+ *                   Spec (scheduling/to_accum.rs:12-60)
+ *   MOVE_RELAYOUT   parameter `tile_m` (not row-major) through a row-major copy: a Move before the
+ *                   Spec when the parameter is read, the Spec on the copy, a Move back when it is
+ *                   written (scheduling/moves.rs:16-130 with the source's dtype;
+ *                   scheduling_sugar.rs move_relayout)
+ *   CAST            input `tile_m` of a Matmul / Conv converted to dtype `tile_n` = the output's
+ *                   (the conversion the Spec's own semantics apply to every input,
+ *                   verification.rs:629-631, so the result is the same), in its own layout: a Move
+ *                   with that dtype pair, then the Spec on the copy (moves.rs:16-130 with another
+ *                   dtype; scheduling_sugar.rs cast)
  * Every action runs the Spec to its result (mrl_run_action).  The reference's actions return a
- * partial Impl whose nested sub-Specs a search expands further: the three Softmax rewrites and
- * BUFFERIZE are such rewrites here too, and mrl_action_apply (below) lists their sub-Specs; every
- * other action is a leaf, a terminal lowering by the library with a price.  There is no action
- * for move_relayout / cast or for a partly tiled Conv or Softmax as steps of their own. */
+ * partial Impl whose nested sub-Specs a search expands further: the three Softmax rewrites,
+ * BUFFERIZE, TO_ACCUM, MOVE_RELAYOUT and CAST are such rewrites here too, and mrl_action_apply
+ * (below) lists their sub-Specs; every other action is a leaf, a terminal lowering by the library
+ * with a price.  There is no action for a partly tiled Conv or Softmax as steps of their own. */
 typedef enum {
   MRL_ACTION_SELECT = 0,
   MRL_ACTION_TILE_OUT_SPLIT = 1,
@@ -534,12 +545,16 @@ typedef enum {
   MRL_ACTION_GENERIC = 6,
   MRL_ACTION_TO_SOFTMAX_PARTS = 7,
   MRL_ACTION_TO_SOFTMAX_PARTS_RECOMPUTE = 8,
-  MRL_ACTION_PARALLEL_SOFTMAX = 9
+  MRL_ACTION_PARALLEL_SOFTMAX = 9,
+  MRL_ACTION_TO_ACCUM = 10,
+  MRL_ACTION_MOVE_RELAYOUT = 11,
+  MRL_ACTION_CAST = 12
 } mrl_action_kind;
 typedef struct {
   int32_t kind;             /* mrl_action_kind */
   uint32_t tile_m, tile_n;  /* TILE_OUT_SPLIT, SPATIAL_SPLIT; FUSED on a Compose: tile_m = queries per workgroup;
-                               FUSED on a Conv: tile_m = 0 or the output width (whole rows per workgroup) */
+                               FUSED on a Conv: tile_m = 0 or the output width (whole rows per workgroup);
+                               MOVE_RELAYOUT, CAST: tile_m = index of the parameter moved; CAST: tile_n = mrl_dtype */
   uint32_t split_k;         /* TILE_OUT_SPLIT: elements of K per step */
   uint32_t parts;           /* FUSED on a Compose: shares of the keys; PARALLEL_SOFTMAX: tiles along the scan dim */
   uint32_t staging;         /* TILE_OUT_SPLIT: mrl_staging */
@@ -568,6 +583,8 @@ int mrl_run_action(const mrl_spec *spec, void *const *params, const mrl_action *
  *                               (scheduling/parallel_softmax.rs:24-223)
  *   BUFFERIZE (on the Compose)  Matmul, Softmax, Matmul with the two tensors between them in
  *                               buffers of the components' output dtype (scheduling/bufferize.rs:24-116)
+ *   TO_ACCUM                    Fill{Zero} of the output, the accumulating Spec
+ *   MOVE_RELAYOUT, CAST         [Move into the copy,] the Spec on the copy [, Move back]
  * Every other action is a leaf (n_subspecs = 0): the library runs it as one piece.  Running the
  * sub-Specs one after the other with mrl_run, each on the buffers its sources name, computes the
  * Spec; each sub-Spec has actions of its own (mrl_target_actions), which is how a search over this
@@ -583,7 +600,7 @@ typedef struct {
   uint32_t n_subspecs;
   mrl_subspec subspecs[MRL_MAX_SUBSPECS];
   uint32_t n_intermediates;
-  uint64_t intermediate_bytes[MRL_MAX_SUBSPECS]; /* dense row-major f32 tensors */
+  uint64_t intermediate_bytes[MRL_MAX_SUBSPECS]; /* dense tensors in the layout their sub-Specs name */
 } mrl_rewrite;
 int mrl_action_apply(const mrl_spec *spec, const mrl_action *action, mrl_rewrite *out);
 /* mrl_run_timed for a chosen action: `steps` launches back to back on the default stream between

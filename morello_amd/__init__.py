@@ -603,6 +603,9 @@ class ActionKind(enum.IntEnum):
     ToSoftmaxParts = 7
     ToSoftmaxPartsRecompute = 8
     ParallelSoftmax = 9
+    ToAccum = 10
+    MoveRelayout = 11
+    Cast = 12
 
 
 class Action:
@@ -622,6 +625,8 @@ class Action:
                  ActionKind.SpatialSplit: f" tile {self.tile_m}x{self.tile_n}",
                  ActionKind.Fused: (f" rows {self.tile_m}" if self.tile_m else "") + (f" parts {self.parts}" if self.parts else ""),
                  ActionKind.ParallelSoftmax: f" parts {self.parts}",
+                 ActionKind.MoveRelayout: f" parameter {self.tile_m}",
+                 ActionKind.Cast: f" parameter {self.tile_m} to {Dtype(self.tile_n) if self.kind == ActionKind.Cast else ''}",
                  }.get(self.kind, "")
         return f"Action({self.kind.name}{knobs}: {self.cost_ns:.0f} ns, {self.n_steps} launches, scratch {self.scratch_bytes} B)"
 

@@ -1925,10 +1925,92 @@ int compose_msm_rewrite(const mrl_spec &s, mrl_rewrite *rw) {
   return fill(rw->subspecs[2], MRL_SPEC_MATMUL, {b, m, n2, n}, 0, {MRL_F32, s.dtypes[0], s.dtypes[3]}, {-2, 0, 3});
 }
 
-int run_softmax_rewrite(const mrl_spec &s, void *const *params, Workspace &ws, const mrl_action &a) {
+// The rewrites that apply to any Spec with an output parameter last:
+//   TO_ACCUM       Fill{Zero} on the output, then the accumulating Spec (scheduling/to_accum.rs:12-60)
+//   MOVE_RELAYOUT  a parameter through a row-major copy, CAST an input through a copy of the
+//                  output's dtype: prologue Move when the parameter is read, the Spec on the copy,
+//                  epilogue Move when it is written (scheduling/moves.rs:49-130)
+int general_rewrite(const mrl_spec &s, const mrl_action &a, mrl_rewrite *rw) {
+  std::memset(rw, 0, sizeof *rw);
+  if (s.kind == MRL_SPEC_COMPOSE_MSM || s.n_params < 2) return MRL_ERR_UNSUPPORTED;
+  const uint32_t out = s.n_params - 1;
+  auto move_spec = [&](mrl_subspec &c, uint32_t i, int dt_from, const mrl_layout &l_from, int dt_to, const mrl_layout &l_to,
+                       int32_t src_from, int32_t src_to) -> int {
+    std::memset(&c, 0, sizeof c);
+    c.spec.kind = MRL_SPEC_MOVE, c.spec.n_params = 2;
+    if (parameter_shape(s, i, c.spec.spec_shape, &c.spec.rank) != MRL_OK) return MRL_ERR_BAD_SPEC;
+    c.spec.dtypes[0] = dt_from, c.spec.dtypes[1] = dt_to;
+    c.spec.layouts[0] = l_from, c.spec.layouts[1] = l_to;
+    c.source[0] = src_from, c.source[1] = src_to;
+    return check_spec(&c.spec);
+  };
+  int rc;
+  if (a.kind == MRL_ACTION_TO_ACCUM) {
+    if ((s.kind != MRL_SPEC_MATMUL && s.kind != MRL_SPEC_CONV) || s.accum) return MRL_ERR_UNSUPPORTED;
+    mrl_subspec &zero = rw->subspecs[0];
+    zero.spec.kind = MRL_SPEC_FILL, zero.spec.scan_dim = MRL_FILL_ZERO, zero.spec.n_params = 1;
+    if (parameter_shape(s, out, zero.spec.spec_shape, &zero.spec.rank) != MRL_OK) return MRL_ERR_BAD_SPEC;
+    zero.spec.dtypes[0] = s.dtypes[out], zero.spec.layouts[0] = s.layouts[out], zero.source[0] = int32_t(out);
+    if ((rc = check_spec(&zero.spec)) != MRL_OK) return rc;
+    mrl_subspec &body = rw->subspecs[1];
+    body.spec = s, body.spec.accum = 1;
+    for (uint32_t i = 0; i < s.n_params; i++) body.source[i] = int32_t(i);
+    rw->n_subspecs = 2;
+    return check_spec(&body.spec);
+  }
+  const uint32_t i = a.tile_m;
+  if (i >= s.n_params) return MRL_ERR_UNSUPPORTED;
+  uint32_t pshape[MRL_MAX_RANK], prank;
+  if (parameter_shape(s, i, pshape, &prank) != MRL_OK) return MRL_ERR_BAD_SPEC;
+  mrl_layout to_layout = s.layouts[i];
+  int to_dtype = s.dtypes[i];
+  if (a.kind == MRL_ACTION_MOVE_RELAYOUT) {
+    mrl_layout_row_major(pshape, prank, &to_layout);
+    int64_t now[MRL_MAX_RANK], rm[MRL_MAX_RANK];
+    const bool strided = mrl::layout_strides(s.layouts[i], pshape, prank, now) && mrl::layout_strides(to_layout, pshape, prank, rm);
+    bool same = strided;
+    for (uint32_t d = 0; same && d < prank; d++) same = pshape[d] == 1 || now[d] == rm[d];
+    if (same) return MRL_ERR_UNSUPPORTED;   // row-major already: nothing to move
+  } else if (a.kind == MRL_ACTION_CAST) {
+    if ((s.kind != MRL_SPEC_MATMUL && s.kind != MRL_SPEC_CONV) || i >= out || int(a.tile_n) != s.dtypes[out] ||
+        s.dtypes[i] == s.dtypes[out])
+      return MRL_ERR_UNSUPPORTED;
+    to_dtype = s.dtypes[out];
+  } else {
+    return MRL_ERR_UNSUPPORTED;
+  }
+  uint64_t count = 1;
+  for (uint32_t d = 0; d < prank; d++) count *= pshape[d];
+  rw->n_intermediates = 1, rw->intermediate_bytes[0] = count * mrl_dtype_size(to_dtype);
+  const bool written = i == out, read = !written || s.accum;
+  if (read && (rc = move_spec(rw->subspecs[rw->n_subspecs++], i, s.dtypes[i], s.layouts[i], to_dtype, to_layout, int32_t(i), -1)) != MRL_OK)
+    return rc;
+  mrl_subspec &body = rw->subspecs[rw->n_subspecs++];
+  body.spec = s, body.spec.dtypes[i] = to_dtype, body.spec.layouts[i] = to_layout;
+  for (uint32_t j = 0; j < s.n_params; j++) body.source[j] = j == i ? -1 : int32_t(j);
+  if ((rc = check_spec(&body.spec)) != MRL_OK) return rc;
+  if (written && (rc = move_spec(rw->subspecs[rw->n_subspecs++], i, to_dtype, to_layout, s.dtypes[i], s.layouts[i], -1, int32_t(i))) != MRL_OK)
+    return rc;
+  return MRL_OK;
+}
+
+int rewrite_of(const mrl_spec &s, const mrl_action &a, mrl_rewrite *rw) {
+  switch (a.kind) {
+    case MRL_ACTION_TO_SOFTMAX_PARTS:
+    case MRL_ACTION_TO_SOFTMAX_PARTS_RECOMPUTE:
+    case MRL_ACTION_PARALLEL_SOFTMAX: return softmax_rewrite(s, a, rw);
+    case MRL_ACTION_TO_ACCUM:
+    case MRL_ACTION_MOVE_RELAYOUT:
+    case MRL_ACTION_CAST: return general_rewrite(s, a, rw);
+    default: return MRL_ERR_UNSUPPORTED;
+  }
+}
+
+// A rewrite run as what it is: its sub-Specs one after the other, the buffers between them in scratch.
+int run_rewrite(const mrl_spec &s, void *const *params, Workspace &ws, const mrl_action &a) {
   mrl_rewrite rw;
   int rc;
-  if ((rc = softmax_rewrite(s, a, &rw)) != MRL_OK) return rc;
+  if ((rc = rewrite_of(s, a, &rw)) != MRL_OK) return rc;
   void *between[MRL_MAX_SUBSPECS] = {};
   for (uint32_t j = 0; j < rw.n_intermediates; j++) HIP_TRY(ws.alloc(&between[j], rw.intermediate_bytes[j]));
   for (uint32_t c = 0; c < rw.n_subspecs; c++) {
@@ -1949,7 +2031,10 @@ int dispatch_action(const mrl_spec &spec, void *const *params, Workspace &ws, co
     case MRL_ACTION_SELECT: return dispatch(spec, params, ws);
     case MRL_ACTION_TO_SOFTMAX_PARTS:
     case MRL_ACTION_TO_SOFTMAX_PARTS_RECOMPUTE:
-    case MRL_ACTION_PARALLEL_SOFTMAX: return run_softmax_rewrite(spec, params, ws, a);
+    case MRL_ACTION_PARALLEL_SOFTMAX:
+    case MRL_ACTION_TO_ACCUM:
+    case MRL_ACTION_MOVE_RELAYOUT:
+    case MRL_ACTION_CAST: return run_rewrite(spec, params, ws, a);
     case MRL_ACTION_TILE_OUT_SPLIT: {
       if (spec.kind != MRL_SPEC_MATMUL) return MRL_ERR_UNSUPPORTED;
       const mrl_matmul_schedule sched = {a.tile_m, a.tile_n, a.split_k, a.staging};
@@ -1988,7 +2073,10 @@ int mrl_action_apply(const mrl_spec *spec, const mrl_action *action, mrl_rewrite
   switch (action->kind) {
     case MRL_ACTION_TO_SOFTMAX_PARTS:
     case MRL_ACTION_TO_SOFTMAX_PARTS_RECOMPUTE:
-    case MRL_ACTION_PARALLEL_SOFTMAX: return softmax_rewrite(*spec, *action, out);
+    case MRL_ACTION_PARALLEL_SOFTMAX:
+    case MRL_ACTION_TO_ACCUM:
+    case MRL_ACTION_MOVE_RELAYOUT:
+    case MRL_ACTION_CAST: return rewrite_of(*spec, *action, out);
     case MRL_ACTION_BUFFERIZE: return compose_msm_rewrite(*spec, out);
     default: break;
   }
@@ -2054,6 +2142,13 @@ uint32_t mrl_target_actions(const mrl_spec *spec, mrl_action *out, uint32_t cap)
     const uint32_t scan = spec->spec_shape[spec->scan_dim];
     for (uint32_t parts = 2; parts <= 64 && scan / parts >= 64; parts *= 2)
       if (scan % parts == 0) candidate(MRL_ACTION_PARALLEL_SOFTMAX, 0, 0, 0, parts);
+  }
+  // The rewrites any Spec may take, last in the list: to_accum, and per parameter a row-major
+  // copy (move_relayout) or a copy in the output's dtype (cast); those that do not apply drop out below.
+  if (spec->kind != MRL_SPEC_COMPOSE_MSM) {
+    candidate(MRL_ACTION_TO_ACCUM);
+    for (uint32_t i = 0; i < spec->n_params; i++) candidate(MRL_ACTION_MOVE_RELAYOUT, i);
+    for (uint32_t i = 0; i + 1 < spec->n_params; i++) candidate(MRL_ACTION_CAST, i, uint32_t(spec->dtypes[spec->n_params - 1]));
   }
   uint32_t n = 0;
   for (mrl_action &a : candidates) {

@@ -72,7 +72,7 @@ int main() {
     EXPECT(std::string(p.steps[0].kernel).find("k_gemm_wide [T = I8, A_UNSIGNED = true") == 0);
     EXPECT(std::string(mrl_target_id()) == "Gfx950" && mrl_target_memories(nullptr, 0) == 4);
     const std::vector<mrl_action> acts = Spec::matmul({1, 4096, 4096, 4096}, Dtype::Uint8, Dtype::Sint8, Dtype::Sint32).actions();
-    EXPECT(acts.size() == 12 && acts[11].staging == MRL_STAGING_DIRECT_B_WIDE && acts[0].kind == MRL_ACTION_SELECT && acts[1].kind == MRL_ACTION_TILE_OUT_SPLIT &&
+    EXPECT(acts.size() == 15 && acts[12].kind == MRL_ACTION_TO_ACCUM && acts[14].kind == MRL_ACTION_CAST && acts[11].staging == MRL_STAGING_DIRECT_B_WIDE && acts[0].kind == MRL_ACTION_SELECT && acts[1].kind == MRL_ACTION_TILE_OUT_SPLIT &&
            acts[1].tile_m == 256 && acts[0].cost_ns > 20e3);
     const mrl_matmul_schedule best =
         Spec::matmul({1, 4096, 4096, 4096}, Dtype::Uint8, Dtype::Sint8, Dtype::Sint32).search_schedule();

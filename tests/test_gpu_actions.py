@@ -37,7 +37,7 @@ def test_matmul_actions_against_the_oracle(gpu):
             c0 = synth.normal_f32(31, 2, (1, m, n))
         want = orc.matmul([1, m, k, n], odt, a, b, c0.copy(), True)
         acts = spec.actions()
-        assert len(acts) == 12 and {a.staging for a in acts} == set(M.Staging)
+        assert len([a for a in acts if a.kind < M.ActionKind.ToAccum]) == 12 and {a.staging for a in acts} == set(M.Staging)
         for act in acts:
             got = run_action(act, [a, b, c0.copy()])
             if np_out == np.int32:
@@ -55,8 +55,8 @@ def test_conv_actions_against_the_oracle(gpu):
     want = orc.conv([b, f, c, oh, ow, fh, fw], [orc.U8, orc.I8, orc.I32], img, filt, np.zeros((b, oh, ow, f), np.int32),
                     layouts=[nhwc, nhwc, nhwc])
     acts = spec.actions()
-    assert {a.kind for a in acts} == {M.ActionKind.Select, M.ActionKind.Fused, M.ActionKind.SpatialSplit,
-                                      M.ActionKind.Unfold, M.ActionKind.Generic}
+    assert {a.kind for a in acts if a.kind < M.ActionKind.ToAccum} == {
+        M.ActionKind.Select, M.ActionKind.Fused, M.ActionKind.SpatialSplit, M.ActionKind.Unfold, M.ActionKind.Generic}
     # the fused kernel both ways: a wave per pixel tile, and whole output rows per workgroup
     assert [a.tile_m for a in acts if a.kind == M.ActionKind.Fused] == [0, ow]
     for act in acts:
@@ -141,6 +141,73 @@ def test_children_of_the_rewrites_compute_the_spec(gpu, shape, dim):
         assert np.abs(got - want).max() < 1e-5, act
 
 
+@pytest.mark.parametrize("dts,codes", [((M.u8, M.i8, M.i32), [0, 1, 5]), ((M.bf16, M.bf16, M.f32), [7, 7, 6])])
+@pytest.mark.parametrize("accum", [False, True])
+def test_to_accum_move_relayout_and_cast(gpu, dts, codes, accum):
+    """The rewrites any Spec may take (to_accum.rs:12-60, moves.rs:49-130), on a Matmul whose A and
+    C are stored column-major: each as the library runs it (mrl_run_action) and as its children
+    run one by one on caller-held copies (mrl_action_apply), against the oracle on an output
+    that starts from a sentinel (overwritten) or from old values (accumulated)."""
+    b, m, k, n = 2, 192, 128, 136
+    gen = {M.u8: synth.uniform_u8, M.i8: synth.uniform_i8, M.bf16: synth.normal_bf16}
+    A, Bm = gen[dts[0]](73, 0, (b, m, k)), gen[dts[1]](73, 1, (b, k, n))
+    out_np = np.int32 if dts[2] == M.i32 else np.float32
+    C0 = synth.uniform_u8(73, 2, (b, m, n)).astype(out_np) if accum else np.full((b, m, n), 5, out_np)
+    want = orc.matmul([b, m, k, n], codes, A, Bm, C0.copy() if accum else np.zeros((b, m, n), out_np), accum)
+    layouts = [M.batched_col_major([b, m, k]), None, M.batched_col_major([b, m, n])]
+    spec = M.Matmul([b, m, k, n], dts, layouts=layouts, accum=accum)
+    At, C0t = np.ascontiguousarray(A.transpose(0, 2, 1)), np.ascontiguousarray(C0.transpose(0, 2, 1))
+    K = M.ActionKind
+    acts = [a for a in spec.actions() if a.kind in (K.ToAccum, K.MoveRelayout, K.Cast)]
+    assert [(a.kind, a.tile_m) for a in acts] == ([] if accum else [(K.ToAccum, 0)]) + [(K.MoveRelayout, 0), (K.MoveRelayout, 2),
+                                                                                        (K.Cast, 0), (K.Cast, 1)]
+    for act in acts:
+        for how in ("library", "children"):
+            bufs = [M.DeviceBuffer.from_numpy(x) for x in (At, Bm, C0t)]
+            if how == "library":
+                act.run_device([x.ptr for x in bufs])
+            else:
+                act.apply().run_device([x.ptr for x in bufs])
+            got = bufs[2].to_numpy(out_np, (b, n, m)).transpose(0, 2, 1)
+            for x in bufs:
+                x.free()
+            if dts[2] == M.i32:
+                assert np.array_equal(got, want), (act, how)
+            else:
+                assert rel_err(got, want) < 1e-5, (act, how)
+
+
+def test_rewrites_of_a_conv_and_a_softmax_in_other_layouts(gpu):
+    """move_relayout of every parameter of a channels-last Conv (to NCHW / FCRS copies), its casts
+    and to_accum; move_relayout of a column-major Softmax's input and output."""
+    K = M.ActionKind
+    b, f, c, oh, ow, fh, fw = 2, 64, 32, 9, 11, 3, 3
+    spec = M.Conv([b, f, c, oh, ow, fh, fw], (M.u8, M.i8, M.i32))
+    img, filt = synth.uniform_u8(74, 0, (b, oh + fh - 1, ow + fw - 1, c)), synth.uniform_i8(74, 1, (f, fh, fw, c))
+    nhwc = orc.make_layout([0, 2, 3, 1])
+    want = orc.conv([b, f, c, oh, ow, fh, fw], [orc.U8, orc.I8, orc.I32], img, filt, np.zeros((b, oh, ow, f), np.int32),
+                    layouts=[nhwc, nhwc, nhwc])
+    acts = [a for a in spec.actions() if a.kind in (K.ToAccum, K.MoveRelayout, K.Cast)]
+    assert len(acts) == 6
+    for act in acts:
+        assert np.array_equal(run_action(act, [img, filt, np.full((b, oh, ow, f), -7, np.int32)]), want), act
+        bufs = [M.DeviceBuffer.from_numpy(x) for x in (img, filt, np.full((b, oh, ow, f), -7, np.int32))]
+        act.apply().run_device([x.ptr for x in bufs])
+        got = bufs[2].to_numpy(np.int32, (b, oh, ow, f))
+        for x in bufs:
+            x.free()
+        assert np.array_equal(got, want), act
+    shape = (48, 320)
+    x = synth.normal_f32(75, 0, shape, 2.0)
+    cm = M.col_major(list(shape))
+    sm = M.Softmax(list(shape), 1, layouts=[cm, cm])
+    moves = [a for a in sm.actions() if a.kind == K.MoveRelayout]
+    assert [a.tile_m for a in moves] == [0, 1]
+    for act in moves:
+        got = run_action(act, [np.ascontiguousarray(x.T), np.zeros((shape[1], shape[0]), np.float32)])
+        assert np.abs(got.T - orc.softmax(list(shape), 1, x)).max() < 1e-5, act
+
+
 def test_children_of_the_bufferized_compose_compute_it(gpu):
     """The Compose's bufferize as sub-Specs: Matmul, Softmax, Matmul with S and P in f32 buffers of
     the caller's; with f32 intermediates the result matches the oracle's closed form to 1e-5."""
@@ -168,7 +235,8 @@ def test_softmax_actions_keep_the_parameters_layouts(gpu):
     cm = M.col_major(list(shape))
     spec = M.Softmax(list(shape), 1, layouts=[cm, cm])
     acts = spec.actions()
-    assert [a.kind for a in acts] == [M.ActionKind.Select, M.ActionKind.ToSoftmaxParts, M.ActionKind.ToSoftmaxPartsRecompute]
+    assert [a.kind for a in acts] == [M.ActionKind.Select, M.ActionKind.ToSoftmaxParts, M.ActionKind.ToSoftmaxPartsRecompute,
+                                      M.ActionKind.MoveRelayout, M.ActionKind.MoveRelayout]
     for act in acts:
         got = run_action(act, [np.ascontiguousarray(x.T), np.zeros((shape[1], shape[0]), np.float32)])
         assert np.abs(got.T - want).max() < 1e-5, act

@@ -349,7 +349,12 @@ def test_actions_of_the_benchmark_configurations():
     """Target::actions (target/mod.rs:69) for C2-C5, host only: every lowering the backend can run,
     priced; the dispatch rules' own choice (Select) is among the cheapest the model knows."""
     K = M.ActionKind
-    acts = c2().actions()
+    rewrites = (K.ToAccum, K.MoveRelayout, K.Cast)     # last in every list, with children (tested below)
+    every = c2().actions()
+    # C2 accumulates and is row-major: of the general rewrites only the casts of its inputs to i32 apply.
+    assert [(a.kind, a.tile_m, a.tile_n) for a in every if a.kind in rewrites] == [(K.Cast, 0, int(M.i32)), (K.Cast, 1, int(M.i32))]
+    acts = [a for a in every if a.kind not in rewrites]
+    assert every[:len(acts)] == acts
     tiles = {(a.tile_m, a.tile_n, a.split_k) for a in acts if a.kind == K.TileOutSplit}
     assert acts[0].kind == K.Select and tiles == set(c2().available_schedules()) and len(tiles) == 8
     assert all(a.n_steps == 1 and a.scratch_bytes == 0 and a.cost_ns > 20e3 for a in acts)
@@ -364,8 +369,11 @@ def test_actions_of_the_benchmark_configurations():
     short = M.MatmulAccum([1, 512, 1024, 512], (M.u8, M.i8, M.i32)).actions()
     assert {a.staging for a in short if a.kind == K.TileOutSplit} == {M.Staging.Default, M.Staging.Registers, M.Staging.DirectB}
     acts = c3().actions()
-    assert len(acts) == 12 and acts[0].cost_ns == min(a.cost_ns for a in acts)
-    acts = {(a.kind, a.tile_m): a for a in c4().actions()}
+    assert len([a for a in acts if a.kind not in rewrites]) == 12 and acts[0].cost_ns == min(a.cost_ns for a in acts)
+    # C4 overwrites its output and its tensors are channels-last: to_accum, a row-major copy of each parameter, two casts.
+    assert [(a.kind, a.tile_m) for a in c4().actions() if a.kind in rewrites] == [
+        (K.ToAccum, 0), (K.MoveRelayout, 0), (K.MoveRelayout, 1), (K.MoveRelayout, 2), (K.Cast, 0), (K.Cast, 1)]
+    acts = {(a.kind, a.tile_m): a for a in c4().actions() if a.kind not in rewrites}
     assert set(acts) == {(K.Select, 0), (K.Fused, 0), (K.Fused, 54), (K.SpatialSplit, 64), (K.SpatialSplit, 128), (K.SpatialSplit, 256),
                          (K.Unfold, 0), (K.Generic, 0)}
     assert acts[(K.Fused, 0)].plan().kernels == ["k_conv_i8"] and acts[(K.Select, 0)].cost_ns == acts[(K.Fused, 0)].cost_ns
@@ -391,7 +399,7 @@ def test_actions_of_the_benchmark_configurations():
     # Specs with one lowering list it alone; what no kernel takes lists nothing it cannot run.
     assert [a.kind for a in M.Move([64, 64], (M.f32, M.f32)).actions()] == [K.Select]
     odd = M.Conv([2, 3, 5, 6, 6, 2, 2], (M.i16, M.i16, M.i32)).actions()
-    assert {a.kind for a in odd} == {K.Select, K.Generic}
+    assert {a.kind for a in odd} - set(rewrites) == {K.Select, K.Generic}
     assert [a.kind for a in M.ComposeMSM(2, 64, 256, 128, 256, layouts=[None, None, KT, None]).actions()] == [K.Select, K.Bufferize]
 
 
@@ -475,5 +483,28 @@ def test_rewrite_actions_have_children_and_the_others_are_leaves():
     assert buf.subspecs[0][0].layouts[1] == KT and buf.intermediate_bytes == [16 * 2048 * 2048 * 4] * 2
     assert len(buf.subspecs[1][0].actions()) > 3          # the Softmax child has the rewrites again
     assert all(a.apply().is_leaf() for a in c5.actions() if a.kind != K.Bufferize)
-    assert all(a.apply().is_leaf() for a in M.MatmulAccum([1, 512, 512, 512], (M.u8, M.i8, M.i32)).actions())
-    assert all(a.apply().is_leaf() for a in M.Conv([2, 64, 64, 10, 10, 3, 3], (M.u8, M.i8, M.i32)).actions())
+    general = (K.ToAccum, K.MoveRelayout, K.Cast)
+    assert all(a.apply().is_leaf() for a in M.MatmulAccum([1, 512, 512, 512], (M.u8, M.i8, M.i32)).actions() if a.kind not in general)
+    assert all(a.apply().is_leaf() for a in M.Conv([2, 64, 64, 10, 10, 3, 3], (M.u8, M.i8, M.i32)).actions() if a.kind not in general)
+    # to_accum (to_accum.rs:12-60): Zero on the output, then the accumulating Spec.
+    mm = M.Matmul([2, 100, 96, 70], (M.bf16, M.bf16, M.f32), layouts=[M.batched_col_major([2, 100, 96]), None, M.batched_col_major([2, 100, 70])])
+    by = {(a.kind, a.tile_m): a.apply() for a in mm.actions() if a.kind in general}
+    assert set(by) == {(K.ToAccum, 0), (K.MoveRelayout, 0), (K.MoveRelayout, 2), (K.Cast, 0), (K.Cast, 1)}
+    zero, body = by[(K.ToAccum, 0)].subspecs
+    assert (zero[0].kind, zero[0].spec_shape, zero[1]) == (M.SpecKind.Fill, [2, 100, 70], [2]) and zero[0].layouts[0] == mm.layouts[2]
+    assert body[0].kind == M.SpecKind.Matmul and body[0].accum and body[1] == [0, 1, 2] and by[(K.ToAccum, 0)].intermediate_bytes == []
+    # move_relayout (moves.rs:49-130) of an input: prologue Move, body on the row-major copy.
+    pro, body = by[(K.MoveRelayout, 0)].subspecs
+    assert pro[0].kind == M.SpecKind.Move and pro[0].layouts == [mm.layouts[0], M.row_major([2, 100, 96])] and pro[1] == [0, -1]
+    assert body[0].layouts[0] == M.row_major([2, 100, 96]) and body[1] == [-1, 1, 2]
+    assert by[(K.MoveRelayout, 0)].intermediate_bytes == [2 * 100 * 96 * 2]
+    # ... of the output of a Spec that overwrites it: no prologue, an epilogue Move back.
+    body, epi = by[(K.MoveRelayout, 2)].subspecs
+    assert body[1] == [0, 1, -1] and epi[0].kind == M.SpecKind.Move and epi[1] == [-1, 2] and epi[0].layouts[1] == mm.layouts[2]
+    acc = M.MatmulAccum([2, 100, 96, 70], (M.bf16, M.bf16, M.f32), layouts=[None, None, M.batched_col_major([2, 100, 70])])
+    three = [a for a in acc.actions() if a.kind == K.MoveRelayout][0].apply().subspecs
+    assert [s.kind for s, _ in three] == [M.SpecKind.Move, M.SpecKind.Matmul, M.SpecKind.Move]     # read and written
+    # cast (moves.rs with another dtype): the input as the output's dtype, in its own layout.
+    pro, body = by[(K.Cast, 0)].subspecs
+    assert list(pro[0].dtypes) == [M.bf16, M.f32] and pro[0].layouts == [mm.layouts[0]] * 2 and list(body[0].dtypes) == [M.f32, M.bf16, M.f32]
+    assert by[(K.Cast, 0)].intermediate_bytes == [2 * 100 * 96 * 4]
