@@ -530,9 +530,16 @@ int mrl_compose_plan(const mrl_compose *c, mrl_plan *plan, mrl_plan_step *steps,
  *                   verification.rs:629-631, so the result is the same), in its own layout: a Move
  *                   with that dtype pair, then the Spec on the copy (moves.rs:16-130 with another
  *                   dtype; scheduling_sugar.rs cast)
+ *   TO_MAX_AND_DENOMINATOR  SoftmaxDenominatorAndMax that overwrites: Max, then SoftmaxDenominator,
+ *                   on the Spec's own parameters (scheduling/to_max_and_denom.rs:13-72)
+ *   TO_MAX_AND_UNSCALED     SoftmaxDenominatorAndUnscaled: Max into a buffer, then
+ *                   SoftmaxDenominatorAndUnscaledFromMax (scheduling/to_max_and_unscaled.rs:30-110)
+ *   BROADCAST_FIRST DivideVecScalar: Broadcast of the denominators to the full shape, then
+ *                   DivideVec (scheduling/broadcast_first.rs:24-130)
  * Every action runs the Spec to its result (mrl_run_action).  The reference's actions return a
  * partial Impl whose nested sub-Specs a search expands further: the three Softmax rewrites,
- * BUFFERIZE, TO_ACCUM, MOVE_RELAYOUT and CAST are such rewrites here too, and mrl_action_apply
+ * BUFFERIZE, TO_ACCUM, MOVE_RELAYOUT, CAST and the three of the Softmax primitives (TO_MAX_AND_*,
+ * BROADCAST_FIRST) are such rewrites here too, and mrl_action_apply
  * (below) lists their sub-Specs; every other action is a leaf, a terminal lowering by the library
  * with a price.  There is no action for a partly tiled Conv or Softmax as steps of their own. */
 typedef enum {
@@ -548,7 +555,10 @@ typedef enum {
   MRL_ACTION_PARALLEL_SOFTMAX = 9,
   MRL_ACTION_TO_ACCUM = 10,
   MRL_ACTION_MOVE_RELAYOUT = 11,
-  MRL_ACTION_CAST = 12
+  MRL_ACTION_CAST = 12,
+  MRL_ACTION_TO_MAX_AND_DENOMINATOR = 13,
+  MRL_ACTION_TO_MAX_AND_UNSCALED = 14,
+  MRL_ACTION_BROADCAST_FIRST = 15
 } mrl_action_kind;
 typedef struct {
   int32_t kind;             /* mrl_action_kind */
@@ -585,6 +595,9 @@ int mrl_run_action(const mrl_spec *spec, void *const *params, const mrl_action *
  *                               buffers of the components' output dtype (scheduling/bufferize.rs:24-116)
  *   TO_ACCUM                    Fill{Zero} of the output, the accumulating Spec
  *   MOVE_RELAYOUT, CAST         [Move into the copy,] the Spec on the copy [, Move back]
+ *   TO_MAX_AND_DENOMINATOR      Max, SoftmaxDenominator
+ *   TO_MAX_AND_UNSCALED         Max, SoftmaxDenominatorAndUnscaledFromMax
+ *   BROADCAST_FIRST             Broadcast, DivideVec
  * Every other action is a leaf (n_subspecs = 0): the library runs it as one piece.  Running the
  * sub-Specs one after the other with mrl_run, each on the buffers its sources name, computes the
  * Spec; each sub-Spec has actions of its own (mrl_target_actions), which is how a search over this

@@ -606,6 +606,9 @@ class ActionKind(enum.IntEnum):
     ToAccum = 10
     MoveRelayout = 11
     Cast = 12
+    ToMaxAndDenominator = 13
+    ToMaxAndUnscaled = 14
+    BroadcastFirst = 15
 
 
 class Action:

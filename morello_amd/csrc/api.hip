@@ -1994,6 +1994,48 @@ int general_rewrite(const mrl_spec &s, const mrl_action &a, mrl_rewrite *rw) {
   return MRL_OK;
 }
 
+// The rewrites of the Softmax primitives, each two stages on f32 tensors:
+//   TO_MAX_AND_DENOMINATOR  SoftmaxDenominatorAndMax -> Max, SoftmaxDenominator (to_max_and_denom.rs:13-72)
+//   TO_MAX_AND_UNSCALED     SoftmaxDenominatorAndUnscaled -> Max into a buffer,
+//                           SoftmaxDenominatorAndUnscaledFromMax (to_max_and_unscaled.rs:30-110)
+//   BROADCAST_FIRST         DivideVecScalar -> Broadcast of the denominators, DivideVec (broadcast_first.rs:24-130)
+int primitive_rewrite(const mrl_spec &s, const mrl_action &a, mrl_rewrite *rw) {
+  std::memset(rw, 0, sizeof *rw);
+  for (uint32_t i = 0; i < s.n_params; i++)
+    if (s.dtypes[i] != MRL_F32) return MRL_ERR_UNSUPPORTED;
+  int rc = MRL_OK;
+  auto child = [&](int kind, std::initializer_list<int32_t> sources) {
+    mrl_subspec &c = rw->subspecs[rw->n_subspecs++];
+    if ((rc = part_spec(kind, s.spec_shape, s.rank, s.scan_dim, &c.spec)) != MRL_OK) return;
+    uint32_t i = 0;
+    for (int32_t src : sources) {
+      if (src >= 0) c.spec.layouts[i] = s.layouts[src];
+      c.source[i++] = src;
+    }
+    rc = check_spec(&c.spec);
+  };
+  uint64_t count = 1, lines = 1;
+  for (uint32_t d = 0; d < s.rank; d++) count *= s.spec_shape[d], lines *= d == s.scan_dim ? 1 : s.spec_shape[d];
+  if (a.kind == MRL_ACTION_TO_MAX_AND_DENOMINATOR) {
+    if (s.kind != MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX || s.accum) return MRL_ERR_UNSUPPORTED;
+    child(MRL_SPEC_MAX, {0, 1});
+    if (rc == MRL_OK) child(MRL_SPEC_SOFTMAX_DENOMINATOR, {0, 1, 2});
+  } else if (a.kind == MRL_ACTION_TO_MAX_AND_UNSCALED) {
+    if (s.kind != MRL_SPEC_SOFTMAX_DENOMINATOR_AND_UNSCALED || s.accum) return MRL_ERR_UNSUPPORTED;
+    rw->n_intermediates = 1, rw->intermediate_bytes[0] = lines * sizeof(float);
+    child(MRL_SPEC_MAX, {0, -1});
+    if (rc == MRL_OK) child(MRL_SPEC_SOFTMAX_DENOMINATOR_AND_UNSCALED_FROM_MAX, {0, -1, 1, 2});
+  } else if (a.kind == MRL_ACTION_BROADCAST_FIRST) {
+    if (s.kind != MRL_SPEC_DIVIDE_VEC_SCALAR) return MRL_ERR_UNSUPPORTED;
+    rw->n_intermediates = 1, rw->intermediate_bytes[0] = count * sizeof(float);
+    child(MRL_SPEC_BROADCAST, {1, -1});
+    if (rc == MRL_OK) child(MRL_SPEC_DIVIDE_VEC, {0, -1});
+  } else {
+    return MRL_ERR_UNSUPPORTED;
+  }
+  return rc;
+}
+
 int rewrite_of(const mrl_spec &s, const mrl_action &a, mrl_rewrite *rw) {
   switch (a.kind) {
     case MRL_ACTION_TO_SOFTMAX_PARTS:
@@ -2002,6 +2044,9 @@ int rewrite_of(const mrl_spec &s, const mrl_action &a, mrl_rewrite *rw) {
     case MRL_ACTION_TO_ACCUM:
     case MRL_ACTION_MOVE_RELAYOUT:
     case MRL_ACTION_CAST: return general_rewrite(s, a, rw);
+    case MRL_ACTION_TO_MAX_AND_DENOMINATOR:
+    case MRL_ACTION_TO_MAX_AND_UNSCALED:
+    case MRL_ACTION_BROADCAST_FIRST: return primitive_rewrite(s, a, rw);
     default: return MRL_ERR_UNSUPPORTED;
   }
 }
@@ -2034,7 +2079,10 @@ int dispatch_action(const mrl_spec &spec, void *const *params, Workspace &ws, co
     case MRL_ACTION_PARALLEL_SOFTMAX:
     case MRL_ACTION_TO_ACCUM:
     case MRL_ACTION_MOVE_RELAYOUT:
-    case MRL_ACTION_CAST: return run_rewrite(spec, params, ws, a);
+    case MRL_ACTION_CAST:
+    case MRL_ACTION_TO_MAX_AND_DENOMINATOR:
+    case MRL_ACTION_TO_MAX_AND_UNSCALED:
+    case MRL_ACTION_BROADCAST_FIRST: return run_rewrite(spec, params, ws, a);
     case MRL_ACTION_TILE_OUT_SPLIT: {
       if (spec.kind != MRL_SPEC_MATMUL) return MRL_ERR_UNSUPPORTED;
       const mrl_matmul_schedule sched = {a.tile_m, a.tile_n, a.split_k, a.staging};
@@ -2076,7 +2124,10 @@ int mrl_action_apply(const mrl_spec *spec, const mrl_action *action, mrl_rewrite
     case MRL_ACTION_PARALLEL_SOFTMAX:
     case MRL_ACTION_TO_ACCUM:
     case MRL_ACTION_MOVE_RELAYOUT:
-    case MRL_ACTION_CAST: return rewrite_of(*spec, *action, out);
+    case MRL_ACTION_CAST:
+    case MRL_ACTION_TO_MAX_AND_DENOMINATOR:
+    case MRL_ACTION_TO_MAX_AND_UNSCALED:
+    case MRL_ACTION_BROADCAST_FIRST: return rewrite_of(*spec, *action, out);
     case MRL_ACTION_BUFFERIZE: return compose_msm_rewrite(*spec, out);
     default: break;
   }
@@ -2143,6 +2194,9 @@ uint32_t mrl_target_actions(const mrl_spec *spec, mrl_action *out, uint32_t cap)
     for (uint32_t parts = 2; parts <= 64 && scan / parts >= 64; parts *= 2)
       if (scan % parts == 0) candidate(MRL_ACTION_PARALLEL_SOFTMAX, 0, 0, 0, parts);
   }
+  if (spec->kind == MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX) candidate(MRL_ACTION_TO_MAX_AND_DENOMINATOR);
+  if (spec->kind == MRL_SPEC_SOFTMAX_DENOMINATOR_AND_UNSCALED) candidate(MRL_ACTION_TO_MAX_AND_UNSCALED);
+  if (spec->kind == MRL_SPEC_DIVIDE_VEC_SCALAR) candidate(MRL_ACTION_BROADCAST_FIRST);
   // The rewrites any Spec may take, last in the list: to_accum, and per parameter a row-major
   // copy (move_relayout) or a copy in the output's dtype (cast); those that do not apply drop out below.
   if (spec->kind != MRL_SPEC_COMPOSE_MSM) {

@@ -133,6 +133,54 @@ def test_divide_vec_and_scalar(gpu, shape, dim):
     assert np.array_equal(got[0], want)
 
 
+def _both_ways(action, arrays):
+    """Every parameter after the action ran as the library runs it, and after its children ran one
+    by one on caller-held intermediates (mrl_action_apply)."""
+    out = []
+    for how in ("library", "children"):
+        bufs = [M.DeviceBuffer.from_numpy(a) for a in arrays]
+        (action if how == "library" else action.apply()).run_device([b.ptr for b in bufs])
+        out.append([b.to_numpy(a.dtype, a.shape) for a, b in zip(arrays, bufs)])
+        for b in bufs:
+            b.free()
+    return out
+
+
+@pytest.mark.parametrize("shape,dim", SHAPES)
+def test_rewrites_of_the_softmax_primitives(gpu, shape, dim):
+    """to_max_and_denominator on SoftmaxDenominatorAndMax (to_max_and_denom.rs:13-72),
+    to_max_and_unscaled on SoftmaxDenominatorAndUnscaled (to_max_and_unscaled.rs:30-110),
+    broadcast_first on DivideVecScalar (broadcast_first.rs:24-130): each gives what the Spec
+    gives, as an action and as its children."""
+    K = M.ActionKind
+    x = rnd(shape)
+    red = reduced(shape, dim)
+    spec = M.SoftmaxDenominatorAndMax(shape, dim)
+    act = [a for a in spec.actions() if a.kind == K.ToMaxAndDenominator]
+    assert len(act) == 1 and [s.kind for s, _ in act[0].apply().subspecs] == [M.SpecKind.Max, M.SpecKind.SoftmaxDenominator]
+    want = orc.softmax_part(orc.PART_DENOM_MAX, shape, dim, [x, np.zeros(red, np.float32), np.zeros(red, np.float32)])
+    for got in _both_ways(act[0], [x, np.full(red, 7, np.float32), np.full(red, 7, np.float32)]):
+        assert np.array_equal(got[1], want[1])
+        np.testing.assert_allclose(got[2], want[2], **tol(shape, dim))
+    assert not [a for a in M.SoftmaxDenominatorAndMax(shape, dim, accum=True).actions() if a.kind == K.ToMaxAndDenominator]
+
+    spec = M.SoftmaxDenominatorAndUnscaled(shape, dim)
+    act = [a for a in spec.actions() if a.kind == K.ToMaxAndUnscaled]
+    assert len(act) == 1 and act[0].apply().intermediate_bytes == [4 * int(np.prod(red))]
+    want = orc.softmax_part(orc.PART_UNSCALED, shape, dim, [x, np.zeros(red, np.float32), np.zeros(shape, np.float32)])
+    for got in _both_ways(act[0], [x, np.full(red, 7, np.float32), np.full(shape, 7, np.float32)]):
+        np.testing.assert_allclose(got[1], want[1], **tol(shape, dim))
+        np.testing.assert_allclose(got[2], want[2], **tol(shape, dim))
+
+    a, bs = rnd(shape), np.abs(rnd(red)) + np.float32(0.5)
+    spec = M.DivideVecScalar(shape, dim)
+    act = [a_ for a_ in spec.actions() if a_.kind == K.BroadcastFirst]
+    assert len(act) == 1 and [s.kind for s, _ in act[0].apply().subspecs] == [M.SpecKind.Broadcast, M.SpecKind.DivideVec]
+    want = orc.softmax_part(orc.PART_DIVIDE_VEC_SCALAR, shape, dim, [a.copy(), bs])[0]
+    for got in _both_ways(act[0], [a, bs]):
+        assert np.array_equal(got[0], want) and np.array_equal(got[1], bs)
+
+
 def test_decomposed_softmax_matches_the_fused_spec(gpu):
     """Max -> DenominatorAndUnscaledFromMax -> DivideVecScalar, as Softmax is scheduled by
     hand in the reference, equals the Softmax Spec on the same input."""

@@ -508,3 +508,15 @@ def test_rewrite_actions_have_children_and_the_others_are_leaves():
     pro, body = by[(K.Cast, 0)].subspecs
     assert list(pro[0].dtypes) == [M.bf16, M.f32] and pro[0].layouts == [mm.layouts[0]] * 2 and list(body[0].dtypes) == [M.f32, M.bf16, M.f32]
     assert by[(K.Cast, 0)].intermediate_bytes == [2 * 100 * 96 * 4]
+    # The rewrites of the Softmax primitives (to_max_and_denom.rs, to_max_and_unscaled.rs, broadcast_first.rs).
+    dm = [a for a in M.SoftmaxDenominatorAndMax([6, 640], 1).actions() if a.kind == K.ToMaxAndDenominator][0].apply()
+    assert [(s.kind, src) for s, src in dm.subspecs] == [(M.SpecKind.Max, [0, 1]), (M.SpecKind.SoftmaxDenominator, [0, 1, 2])]
+    assert dm.intermediate_bytes == []
+    du = [a for a in M.SoftmaxDenominatorAndUnscaled([6, 640], 1).actions() if a.kind == K.ToMaxAndUnscaled][0].apply()
+    assert [(s.kind, src) for s, src in du.subspecs] == [(M.SpecKind.Max, [0, -1]),
+                                                         (M.SpecKind.SoftmaxDenominatorAndUnscaledFromMax, [0, -1, 1, 2])]
+    assert du.intermediate_bytes == [6 * 4]
+    bf = [a for a in M.DivideVecScalar([6, 640], 1).actions() if a.kind == K.BroadcastFirst][0].apply()
+    assert [(s.kind, s.parameter_shapes(), src) for s, src in bf.subspecs] == [
+        (M.SpecKind.Broadcast, [[6, 1], [6, 640]], [1, -1]), (M.SpecKind.DivideVec, [[6, 640], [6, 640]], [0, -1])]
+    assert bf.intermediate_bytes == [6 * 640 * 4]
