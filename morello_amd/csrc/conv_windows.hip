@@ -1,0 +1,270 @@
+// Conv NHWC u8|i8 x KRSC i8 -> i32 for pixels of few channels (a first layer: 3 channels, 7 x 7
+// filters), where a pixel's channels are not whole 16-byte chunks and the implicit Matmul of
+// conv_gemm.hip does not apply (morello/src/spec.rs:486-494: no stride, no padding).  The other
+// route for such shapes writes every window to memory first (unfold.hip) and multiplies the rows:
+// 64 MB of windows for 32 x 3 x 118 x 118 -> 64 x 112 x 112.  Here the windows are formed in LDS.
+//
+// A workgroup of four waves takes tiles of 8 x 16 output pixels of one image, one after the other:
+//   1. the tile's input patch ((8 + fh - 1) x (16 + fw - 1) pixels) goes into LDS (u8 as a - 128);
+//      its bytes are fetched into registers while the previous tile is multiplied;
+//   2. every output pixel's window is copied out of the patch into a row of its own: fh runs of
+//      fw * c contiguous bytes, each run padded to whole dwords (so that the copies are dwords: two
+//      aligned reads and a byte alignment per dword written), the row to whole MFMA k steps of 64 bytes;
+//   3. each wave multiplies two rows of the tile (16 pixels each: a B operand block) with the
+//      filters (A operands from LDS, staged once per workgroup in the same padded order, zeros in
+//      the padding, so that whatever the windows hold there counts for nothing):
+//      v_mfma_i32_16x16x64_i8, a lane ends up with 4 consecutive filters of one pixel, 16
+//      contiguous bytes of the channels-last output.
+// The u8 correction 128 * sum of a filter's weights comes from the same MFMAs against an operand
+// of ones, once per workgroup.  Rows of windows and filters lie 16 bytes more than their length
+// apart, which spreads the 16 lanes of an operand read over all banks.
+#include "kernels.h"
+#include "plan.h"
+
+namespace mrl {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+constexpr int TILE_H = 8, TILE_W = 16, TILE_PIXELS = TILE_H * TILE_W;
+constexpr int PATCH_REGS = 8;   // patch bytes a thread holds in flight: patches of up to 2 KiB
+
+struct WindowsArgs {
+  const uint8_t *image, *filters;
+  int32_t *out;
+  uint32_t b, f, c, oh, ow, fh, fw;
+  int accum;
+  uint32_t tiles_x, tiles_y, tiles;   // per image, per image, in all
+  uint32_t seg, seg_padded;           // fw * c: bytes of one run of a window; the same in whole dwords
+  uint32_t patch_stride;              // bytes between the patch's rows in LDS (whole dwords)
+};
+
+// KS: MFMA k steps per window (fh * seg_padded bytes, padded to 64 KS).
+template <int KS, bool IMG_UNSIGNED>
+__global__ __launch_bounds__(256) void k_conv_windows_i8(WindowsArgs p) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t win_lds[];
+  // Rows of windows and filters: 16 bytes more than their length apart (144 at least: two pixel
+  // blocks' rows also hold a block's 16 x 272 bytes of results on their way out).
+  constexpr int KPAD = 64 * KS, ROW = KS == 1 ? 144 : KPAD + 16;
+  const int tid = threadIdx.x, lane = tid & 63, li = lane & 15, lg = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  uint8_t *filt = win_lds;                    // [64][ROW]
+  uint8_t *rows = filt + 64 * ROW;            // [128][ROW]
+  uint8_t *patch = rows + TILE_PIXELS * ROW;  // [TILE_H + fh - 1][patch_stride] + 4
+  const uint32_t f0 = blockIdx.y * 64, nf = min(64u, p.f - f0);   // this workgroup's filters (a multiple of 16)
+  const int nfb = int(nf / 16);
+  const uint32_t k = p.fh * p.seg;
+
+  // The filters, once: run r of filter f at r * seg_padded of the filter's row, zeros everywhere
+  // else.  Their nf * k bytes are one contiguous piece of memory: fetched with every load in
+  // flight at once into the space the window rows will take, then copied from there run by run
+  // as dwords (as the windows are below), the bytes behind a run's end masked to zero.
+  {
+    const uint32_t raw_bytes = nf * k;
+    const uint8_t *from = p.filters + uint64_t(f0) * k;
+    const uint32_t head = uint32_t(-reinterpret_cast<uintptr_t>(from)) & 15;   // bytes up to the first 16-byte boundary
+    uint8_t *raw = rows + 16;                                                   // raw[i] for byte i; raw + head is 16-byte aligned
+    raw -= head;
+    const uint32_t chunks = raw_bytes > head ? (raw_bytes - head) / 16 : 0;
+    constexpr int FILTER_LOADS = 4;   // 16 KiB with all loads in flight; the rest in further rounds
+    for (uint32_t c0 = 0; c0 < chunks; c0 += FILTER_LOADS * 256) {
+      v4i got[FILTER_LOADS];
+#pragma unroll
+      for (int j = 0; j < FILTER_LOADS; j++) {
+        const uint32_t ch = c0 + j * 256 + tid;
+        if (ch < chunks) got[j] = *(const v4i *)(from + head + ch * 16);
+      }
+#pragma unroll
+      for (int j = 0; j < FILTER_LOADS; j++) {
+        const uint32_t ch = c0 + j * 256 + tid;
+        if (ch < chunks) *(v4i *)(raw + head + ch * 16) = got[j];
+      }
+    }
+    // the bytes before the first and behind the last whole chunk
+    if (uint32_t(tid) < 32) {
+      const uint32_t i = uint32_t(tid) < 16 ? uint32_t(tid) : head + chunks * 16 + (tid - 16);
+      if ((uint32_t(tid) < 16 ? i < min(head, raw_bytes) : i < raw_bytes)) raw[i] = from[i];
+    }
+    for (uint32_t i = tid; i < 64 * ROW / 16; i += 256) ((v4i *)filt)[i] = v4i{0, 0, 0, 0};
+    __syncthreads();
+    const uint32_t dwords = p.seg_padded / 4;
+    for (uint32_t run = tid; run < nf * p.fh; run += 256) {
+      const uint32_t fi = run / p.fh, r = run % p.fh;
+      const uint32_t at = uint32_t(raw - rows) + fi * k + r * p.seg, shift = at & 3;   // byte offset within `rows` (16-byte aligned)
+      const uint32_t *src = (const uint32_t *)rows + (at >> 2);
+      uint32_t *dst = (uint32_t *)(filt + fi * ROW + r * p.seg_padded);
+      for (uint32_t d = 0; d < dwords; d++) {
+        uint32_t v = __builtin_amdgcn_alignbyte(src[d + 1], src[d], shift);
+        const uint32_t valid = p.seg - 4 * d;   // bytes of this dword that belong to the run
+        if (valid < 4) v &= (1u << (8 * valid)) - 1;
+        dst[d] = v;
+      }
+    }
+    __syncthreads();   // the raw bytes are no longer needed: the rows are free for the windows
+  }
+  const uint32_t patch_h = TILE_H + p.fh - 1, patch_wb = (TILE_W + p.fw - 1) * p.c, patch_bytes = patch_h * patch_wb;
+  const uint32_t h = p.oh + p.fh - 1, w = p.ow + p.fw - 1;
+  // A tile's patch: rows y0 .. of the image from pixel x0 on; past the image's edge (a ragged
+  // tile) the last row / the row's last byte again, which only reaches pixels that are not stored.
+  uint8_t held[PATCH_REGS];
+  auto patch_source = [&](uint32_t t, uint32_t i) {
+    const uint32_t img = t / (p.tiles_x * p.tiles_y), in_img = t % (p.tiles_x * p.tiles_y);
+    const uint32_t y0 = (in_img / p.tiles_x) * TILE_H, x0 = (in_img % p.tiles_x) * TILE_W;
+    const uint32_t r = i / patch_wb, xb = i % patch_wb;
+    const uint32_t y = min(y0 + r, h - 1), x = min(x0 * p.c + xb, w * p.c - 1);
+    return p.image + (uint64_t(img) * h + y) * w * p.c + x;
+  };
+  auto fetch_patch = [&](uint32_t t) {
+#pragma unroll
+    for (int j = 0; j < PATCH_REGS; j++) {
+      const uint32_t i = tid + j * 256;
+      if (i < patch_bytes) held[j] = *patch_source(t, i);
+    }
+  };
+  auto put = [&](uint32_t i, uint8_t v) { patch[(i / patch_wb) * p.patch_stride + i % patch_wb] = IMG_UNSIGNED ? uint8_t(v ^ 0x80) : v; };
+  if (blockIdx.x < p.tiles) fetch_patch(blockIdx.x);
+  __syncthreads();
+  v4i corr[4] = {};
+  if (IMG_UNSIGNED) {
+    const v4i ones = v4i{0x01010101, 0x01010101, 0x01010101, 0x01010101};
+#pragma unroll
+    for (int fb = 0; fb < 4; fb++) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++)
+        corr[fb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(*(const v4i *)(filt + (fb * 16 + li) * ROW + ks * 64 + lg * 16), ones,
+                                                         corr[fb], 0, 0, 0);
+      corr[fb] *= 128;
+    }
+  }
+  for (uint32_t t = blockIdx.x; t < p.tiles; t += gridDim.x) {
+    const uint32_t img = t / (p.tiles_x * p.tiles_y), in_img = t % (p.tiles_x * p.tiles_y);
+    const uint32_t y0 = (in_img / p.tiles_x) * TILE_H, x0 = (in_img % p.tiles_x) * TILE_W;
+    // 1. the patch out of the registers (what they do not hold, straight from memory)
+#pragma unroll
+    for (int j = 0; j < PATCH_REGS; j++) {
+      const uint32_t i = tid + j * 256;
+      if (i < patch_bytes) put(i, held[j]);
+    }
+    for (uint32_t i = tid + PATCH_REGS * 256; i < patch_bytes; i += 256) put(i, *patch_source(t, i));
+    __syncthreads();   // also: every wave is done with the previous tile's windows
+    // 2. the windows: thread (pixel, half) copies every other run of the pixel's window, eight
+    //    dwords at a time (nine aligned dwords read, shifted by the run's byte offset)
+    {
+      const uint32_t px = tid & 127, ty = px >> 4, tx = px & 15;
+      const uint32_t *__restrict__ patch32 = (const uint32_t *)patch;
+      uint32_t *__restrict__ dst = (uint32_t *)(rows + px * ROW);
+      const uint32_t dwords = p.seg_padded / 4;
+      for (uint32_t r = tid >> 7; r < p.fh; r += 2) {
+        const uint32_t from = (ty + r) * p.patch_stride + tx * p.c, shift = from & 3;
+        const uint32_t *src = patch32 + (from >> 2);
+        for (uint32_t d0 = 0; d0 < dwords; d0 += 8) {
+          uint32_t v[9];
+#pragma unroll
+          for (int d = 0; d < 9; d++) v[d] = d0 + d <= dwords ? src[d0 + d] : 0;
+#pragma unroll
+          for (int d = 0; d < 8; d++)
+            if (d0 + d < dwords) dst[r * dwords + d0 + d] = __builtin_amdgcn_alignbyte(v[d + 1], v[d], shift);
+        }
+      }
+    }
+    __syncthreads();
+    const uint32_t next = t + gridDim.x;
+    if (next < p.tiles) fetch_patch(next);   // in flight under the MFMAs and the stores
+    // 3. two rows of the tile per wave against the group's filters
+    v4i acc[2][4];
+#pragma unroll
+    for (int pb = 0; pb < 2; pb++)
+#pragma unroll
+      for (int fb = 0; fb < 4; fb++) acc[pb][fb] = corr[fb];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      v4i a[4], bop[2];
+#pragma unroll
+      for (int fb = 0; fb < 4; fb++) a[fb] = *(const v4i *)(filt + (fb * 16 + li) * ROW + ks * 64 + lg * 16);
+#pragma unroll
+      for (int pb = 0; pb < 2; pb++) bop[pb] = *(const v4i *)(rows + ((2 * wave + pb) * 16 + li) * ROW + ks * 64 + lg * 16);
+#pragma unroll
+      for (int pb = 0; pb < 2; pb++)
+#pragma unroll
+        for (int fb = 0; fb < 4; fb++) acc[pb][fb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[fb], bop[pb], acc[pb][fb], 0, 0, 0);
+    }
+    // A lane holds filters 16 fb + 4 lg .. + 3 of pixel (y0 + 2 wave + pb, x0 + li): 16-byte pieces
+    // 64 bytes apart.  A pixel block's 16 x 64 results go through the wave's own window rows (no
+    // other wave reads them, and this wave is done with them) and leave as whole rows: four pixels
+    // per store instruction, 1 KiB contiguous when the Spec has 64 filters.
+    uint8_t *xb = rows + (2 * wave) * 16 * ROW;
+    constexpr int XROW = 272;
+#pragma unroll
+    for (int pb = 0; pb < 2; pb++) {
+#pragma unroll
+      for (int fb = 0; fb < 4; fb++) *(v4i *)(xb + li * XROW + fb * 64 + lg * 16) = acc[pb][fb];
+      const uint32_t y = y0 + 2 * wave + pb;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const uint32_t pixel = 4 * j + lg, x = x0 + pixel;
+        v4i v = *(const v4i *)(xb + pixel * XROW + li * 16);
+        if (y < p.oh && x < p.ow && li < 4 * nfb) {
+          v4i *d = (v4i *)(p.out + ((uint64_t(img) * p.oh + y) * p.ow + x) * p.f + f0 + 4 * li);
+          if (p.accum) v += *d;
+          __builtin_nontemporal_store(v, d);
+        }
+      }
+    }
+  }
+}
+
+template <int KS>
+hipError_t launch_ks(const WindowsArgs &p, bool img_unsigned, dim3 grid, size_t lds, hipStream_t stream) {
+  static std::atomic<uint64_t> limit_u{0}, limit_s{0};
+  if (!plan::recording()) {
+    hipError_t e = img_unsigned ? raise_lds_limit(limit_u, (const void *)k_conv_windows_i8<KS, true>, lds)
+                                : raise_lds_limit(limit_s, (const void *)k_conv_windows_i8<KS, false>, lds);
+    if (e != hipSuccess) return e;
+  }
+  if (img_unsigned) MRL_LAUNCH((k_conv_windows_i8<KS, true>), grid, dim3(256), lds, stream, p);
+  else MRL_LAUNCH((k_conv_windows_i8<KS, false>), grid, dim3(256), lds, stream, p);
+  return plan::last_error();
+}
+
+}  // namespace
+
+// Filters in 16s, windows of at most 256 bytes with their runs padded to dwords, and not a shape
+// conv_gemm.hip reads in place.
+bool conv_windows_applicable(const ConvArgs &c) {
+  const uint64_t seg_padded = (uint64_t(c.fw) * c.c + 3) & ~3ull;
+  return c.f % 16 == 0 && c.f / 64 < 65535 && c.c % 16 != 0 && uint64_t(c.fh) * seg_padded <= 256 &&
+         uint64_t(c.b) * ((c.oh + TILE_H - 1) / TILE_H) * ((c.ow + TILE_W - 1) / TILE_W) < (1ull << 31) &&
+         (reinterpret_cast<uintptr_t>(c.out) & 15) == 0;
+}
+
+hipError_t launch_conv_windows(const ConvArgs &c, bool img_unsigned, hipStream_t stream) {
+  if (!conv_windows_applicable(c)) return hipErrorInvalidValue;
+  WindowsArgs p;
+  p.image = (const uint8_t *)c.image, p.filters = (const uint8_t *)c.filters, p.out = (int32_t *)c.out;
+  p.b = c.b, p.f = c.f, p.c = c.c, p.oh = c.oh, p.ow = c.ow, p.fh = c.fh, p.fw = c.fw, p.accum = c.accum;
+  p.tiles_x = (c.ow + TILE_W - 1) / TILE_W, p.tiles_y = (c.oh + TILE_H - 1) / TILE_H, p.tiles = c.b * p.tiles_x * p.tiles_y;
+  p.seg = c.fw * c.c, p.seg_padded = (p.seg + 3) & ~3u;
+  p.patch_stride = ((TILE_W + c.fw - 1) * c.c + 3) & ~3u;
+  const int ks = int((c.fh * p.seg_padded + 63) / 64);
+  const size_t row = ks == 1 ? 144 : 64 * ks + 16;
+  // the copies read one dword past a run's last: four bytes behind the patch
+  const size_t lds = (64 + TILE_PIXELS) * row + size_t(TILE_H + c.fh - 1) * p.patch_stride + 16;
+  // Workgroups walk the tiles with the grid's stride: as many as fit the chip at once, so that
+  // the filters are staged once each.
+  const uint32_t per_cu = uint32_t(std::max<size_t>(1, std::min<size_t>(4, (160 * 1024) / lds)));
+  const uint32_t groups = (c.f + 63) / 64;
+  const uint32_t wgs = std::min<uint32_t>(p.tiles, std::max(1u, g_compute_units * per_cu / groups));
+  const double pixels = double(c.b) * c.oh * c.ow;
+  plan::work(plan::UNIT_STREAM, 0, 1.5 * (pixels * c.f * 4 * (c.accum ? 2 : 1) + double(c.b) * (c.oh + c.fh - 1) * (c.ow + c.fw - 1) * c.c),
+             0, 6000.0 + (1500.0 + 1000.0 * ks) * double((p.tiles + wgs - 1) / wgs));   // staging the filters; a tile
+  const dim3 grid(wgs, groups);
+  switch (ks) {
+    case 1: return launch_ks<1>(p, img_unsigned, grid, lds, stream);
+    case 2: return launch_ks<2>(p, img_unsigned, grid, lds, stream);
+    case 3: return launch_ks<3>(p, img_unsigned, grid, lds, stream);
+    case 4: return launch_ks<4>(p, img_unsigned, grid, lds, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace mrl
