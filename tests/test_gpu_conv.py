@@ -133,6 +133,41 @@ def test_deep_conv_on_small_images_shares_its_windows_out(gpu, dts, codes, shape
         assert err < 1e-5
 
 
+@pytest.mark.parametrize("shape,accum", [
+    ((2, 64, 3, 20, 37, 7, 7), False),    # a first layer: three k steps, ragged tiles both ways
+    ((4, 16, 1, 30, 30, 3, 3), True),     # one channel, one k step, sixteen filters
+    ((3, 48, 4, 8, 33, 3, 3), False),     # runs that are whole dwords
+    ((2, 80, 3, 17, 15, 5, 5), True),     # two groups of filters, the second of sixteen; two k steps
+    ((1, 128, 24, 5, 50, 3, 3), False),   # 24 channels: runs of 72 bytes, four k steps
+    ((64, 32, 2, 1, 3, 2, 9), True),      # three output pixels per image
+    ((1, 64, 5, 30, 30, 1, 1), False),    # 1 x 1 filters
+    ((2, 32, 3, 11, 40, 9, 3), False),    # tall filters
+])
+@pytest.mark.parametrize("img_dt,img_code,gen", [(M.u8, 0, synth.uniform_u8), (M.i8, 1, synth.uniform_i8)])
+def test_conv_with_few_channels_forms_its_windows_in_lds(gpu, shape, accum, img_dt, img_code, gen):
+    """Pixels that are not whole 16-byte chunks, windows of at most 256 bytes (runs padded to
+    dwords), filters in 16s: one kernel forms the windows in LDS and multiplies them.  Against
+    the oracle, bit for bit, with old values in the output when accumulating and a sentinel
+    otherwise; once more with the image and the filters at addresses that are not 16-byte aligned."""
+    b, f, c, oh, ow, fh, fw = shape
+    spec = M.Conv(list(shape), (img_dt, M.i8, M.i32), accum=accum)
+    assert spec.plan().kernels == ["k_conv_windows_i8"]
+    img = gen(134, 0, (b, oh + fh - 1, ow + fw - 1, c))
+    filt = synth.uniform_i8(134, 1, (f, fh, fw, c))
+    out0 = (synth.uniform_i8(134, 2, (b, oh, ow, f)).astype(np.int32) * 1001) if accum else np.full((b, oh, ow, f), -5, np.int32)
+    want = orc.conv(list(shape), [img_code, 1, 5], img, filt, out0.copy(), accum, layouts=[NHWC] * 3)
+    assert np.array_equal(run_spec(spec, [img, filt, out0.copy()]), want)
+    # the same from unaligned addresses: the operands 3 and 5 bytes into their buffers
+    pad_img, pad_filt = np.zeros(img.size + 16, img.dtype), np.zeros(filt.size + 16, np.int8)
+    pad_img[3:3 + img.size], pad_filt[5:5 + filt.size] = img.reshape(-1), filt.reshape(-1)
+    bufs = [M.DeviceBuffer.from_numpy(x) for x in (pad_img, pad_filt, out0)]
+    spec.run_device([bufs[0].ptr + 3, bufs[1].ptr + 5, bufs[2].ptr])
+    got = bufs[2].to_numpy(np.int32, (b, oh, ow, f))
+    for x in bufs:
+        x.free()
+    assert np.array_equal(got, want)
+
+
 def test_conv_as_matmul_from_nchw(gpu):
     """Row-major (NCHW / FCRS) tensors at a shape the unfolded path takes: moved to channels-last
     and back around it."""
