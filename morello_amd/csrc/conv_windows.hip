@@ -55,6 +55,27 @@ __global__ __launch_bounds__(256) void k_conv_windows_i8(WindowsArgs p) {
   const int nfb = int(nf / 16);
   const uint32_t k = p.fh * p.seg;
 
+  const uint32_t patch_h = TILE_H + p.fh - 1, patch_wb = (TILE_W + p.fw - 1) * p.c, patch_bytes = patch_h * patch_wb;
+  const uint32_t h = p.oh + p.fh - 1, w = p.ow + p.fw - 1;
+  // A tile's patch: rows y0 .. of the image from pixel x0 on; past the image's edge (a ragged
+  // tile) the last row / the row's last byte again, which only reaches pixels that are not stored.
+  uint8_t held[PATCH_REGS];
+  auto patch_source = [&](uint32_t t, uint32_t i) {
+    const uint32_t img = t / (p.tiles_x * p.tiles_y), in_img = t % (p.tiles_x * p.tiles_y);
+    const uint32_t y0 = (in_img / p.tiles_x) * TILE_H, x0 = (in_img % p.tiles_x) * TILE_W;
+    const uint32_t r = i / patch_wb, xb = i % patch_wb;
+    const uint32_t y = min(y0 + r, h - 1), x = min(x0 * p.c + xb, w * p.c - 1);
+    return p.image + (uint64_t(img) * h + y) * w * p.c + x;
+  };
+  auto fetch_patch = [&](uint32_t t) {
+#pragma unroll
+    for (int j = 0; j < PATCH_REGS; j++) {
+      const uint32_t i = tid + j * 256;
+      if (i < patch_bytes) held[j] = *patch_source(t, i);
+    }
+  };
+  auto put = [&](uint32_t i, uint8_t v) { patch[(i / patch_wb) * p.patch_stride + i % patch_wb] = IMG_UNSIGNED ? uint8_t(v ^ 0x80) : v; };
+  if (blockIdx.x < p.tiles) fetch_patch(blockIdx.x);   // the first tile's patch: in flight while the filters are staged
   // The filters, once: run r of filter f at r * seg_padded of the filter's row, zeros everywhere
   // else.  Their nf * k bytes are one contiguous piece of memory: fetched with every load in
   // flight at once into the space the window rows will take, then copied from there run by run
@@ -102,28 +123,6 @@ __global__ __launch_bounds__(256) void k_conv_windows_i8(WindowsArgs p) {
     }
     __syncthreads();   // the raw bytes are no longer needed: the rows are free for the windows
   }
-  const uint32_t patch_h = TILE_H + p.fh - 1, patch_wb = (TILE_W + p.fw - 1) * p.c, patch_bytes = patch_h * patch_wb;
-  const uint32_t h = p.oh + p.fh - 1, w = p.ow + p.fw - 1;
-  // A tile's patch: rows y0 .. of the image from pixel x0 on; past the image's edge (a ragged
-  // tile) the last row / the row's last byte again, which only reaches pixels that are not stored.
-  uint8_t held[PATCH_REGS];
-  auto patch_source = [&](uint32_t t, uint32_t i) {
-    const uint32_t img = t / (p.tiles_x * p.tiles_y), in_img = t % (p.tiles_x * p.tiles_y);
-    const uint32_t y0 = (in_img / p.tiles_x) * TILE_H, x0 = (in_img % p.tiles_x) * TILE_W;
-    const uint32_t r = i / patch_wb, xb = i % patch_wb;
-    const uint32_t y = min(y0 + r, h - 1), x = min(x0 * p.c + xb, w * p.c - 1);
-    return p.image + (uint64_t(img) * h + y) * w * p.c + x;
-  };
-  auto fetch_patch = [&](uint32_t t) {
-#pragma unroll
-    for (int j = 0; j < PATCH_REGS; j++) {
-      const uint32_t i = tid + j * 256;
-      if (i < patch_bytes) held[j] = *patch_source(t, i);
-    }
-  };
-  auto put = [&](uint32_t i, uint8_t v) { patch[(i / patch_wb) * p.patch_stride + i % patch_wb] = IMG_UNSIGNED ? uint8_t(v ^ 0x80) : v; };
-  if (blockIdx.x < p.tiles) fetch_patch(blockIdx.x);
-  __syncthreads();
   v4i corr[4] = {};
   if (IMG_UNSIGNED) {
     const v4i ones = v4i{0x01010101, 0x01010101, 0x01010101, 0x01010101};
