@@ -426,12 +426,14 @@ def cycle_stamps(launches):
     tot, ticks = d("T5", "T0"), d("R5", "R0")
     if int(np.median(tot)) == 0 or int(ticks.min()) == 0:
         raise SystemExit("no stamps in C: build the library with MRL_WIDE_OPTS=trace for this mode")
-    unrolled = 10   # the accumulating kernel's unrolled steps (the first eight load C's old values)
+    # k steps before the second stamp: the nine steps that carry C's old values with two steps of
+    # the loop behind each of the first eight (the variant 4096^3's 32 steps take)
+    unrolled = 25
     out = {"workload": desc, "launches_before": launches, "us_per_launch_last_20": us,
            "wave_cycles": stat(tot), "wave_100mhz_ticks": stat(ticks), "shader_clock_mhz": stat(tot / ticks * 100.0),
            "prologue_cycles": stat(d("T1", "T0")),
-           "cycles_per_step_first_10": stat(d("T2", "T1") / unrolled),
-           "cycles_per_step_last_22": stat(d("T3", "T2") / (32 - unrolled)),
+           "cycles_per_step_first_25": stat(d("T2", "T1") / unrolled),
+           "cycles_per_step_last_7": stat(d("T3", "T2") / (32 - unrolled)),
            "epilogue_store_issue_cycles": stat(d("T4", "T3")), "epilogue_drain_cycles": stat(d("T5", "T4")),
            "cycles_waiting_for_memory_at_barriers": stat(v["Wvm"]), "cycles_in_barriers": stat(v["Wbar"]),
            "launch_span_us": float(v["R5"].max() - v["R0"].min()) / 100.0,
