@@ -271,7 +271,7 @@ def _median_ms(run, ptrs, launches=20, repeats=5):
 def test_cost_model_against_measured_launches(gpu):
     """Predicted against measured per-launch time on benchmark-like operands for the kernels the
     benchmark configurations and their neighbours run, each timing the median of five bursts on
-    settled clocks.  The ratios are printed (measured on these ten: 0.80-1.21); the model, which
+    settled clocks.  The ratios are printed (measured on the first ten: 0.80-1.21); the model, which
     ranks the lowerings that mrl_target_actions and mrl_matmul_search_schedule offer, is held to
     a factor of two either way for every kernel family here."""
     rng = np.random.default_rng(7)
@@ -279,7 +279,11 @@ def test_cost_model_against_measured_launches(gpu):
              M.Matmul([1, 1024, 1024, 1024], (M.f32, M.f32, M.f32)), M.Softmax([16, 2048, 2048], 2),
              M.Softmax([64, 100000], 1), M.ComposeMSM(16, 1, 128, 32768, 128, layouts=[None, None, KT, None]),
              M.Matmul([1, 1, 2048, 16384], (M.bf16, M.bf16, M.f32), layouts=[None, KT, None]),
-             M.Move([4096, 4096], (M.f32, M.f32), layouts=[M.row_major([4096, 4096]), M.col_major([4096, 4096])])]
+             M.Move([4096, 4096], (M.f32, M.f32), layouts=[M.row_major([4096, 4096]), M.col_major([4096, 4096])]),
+             # a first-layer Conv (windows formed in LDS), a deep one on small images (windows shared out), a Softmax
+             # over an outer dim of few columns (scan dim shared out)
+             M.Conv([32, 64, 3, 112, 112, 7, 7], (M.u8, M.i8, M.i32)), M.Conv([32, 512, 512, 5, 5, 3, 3], (M.u8, M.i8, M.i32)),
+             M.Softmax([2048, 4096], 0)]
     _settle_clocks()
     for spec in specs:
         bufs = []
