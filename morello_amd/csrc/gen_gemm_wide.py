@@ -193,6 +193,11 @@ def gen(kind, accum, opts=None, gap=0):
     is the plain one, but the additions leave a wave at a twelfth of the stores' rate (95 K cycles
     for a wave's 256 instead of 8 K; bf16 8192^3 accumulating 980 us against 790)."""
     opts = opts or {}     # experiment switches; the shipped loops are generated with none
+    # Experiment (atomic_c): an accumulating variant as the plain loop with the epilogue's stores
+    # turned into atomic additions (see above); results are the same, the launch is slower.
+    add_in_memory = bool(accum and opts.get("atomic_c"))
+    if add_in_memory:
+        accum, gap = False, 0
     unsigned = kind == "u8" and not opts.get("no_valu")
     is_float = kind == "bf16"
     mfma = "v_mfma_f32_16x16x32_bf16" if is_float else "v_mfma_i32_16x16x64_i8"
@@ -565,6 +570,7 @@ def gen(kind, accum, opts=None, gap=0):
         E("s_waitcnt lgkmcnt(0)")
         e.all_lds_done()
     early = int(opts.get("early_stores", 0))   # timing experiment (C2's 32 steps only): see below
+    landing = min(int(opts.get("landing", 0)), max(gap - 1, 0))
     if accum and gap > 0:
         # C's old values at steps 0, gap + 1, 2 (gap + 1), ...: between them the loop runs `gap` steps.
         kt = 0
@@ -575,10 +581,16 @@ def gen(kind, accum, opts=None, gap=0):
             step(kt % 6, zero_first=(j == 0), extra=[] if opts.get("no_cops") else c_ops(j, spaced=True))
             kt += 1
             if j < C_STEPS:
-                E(f"s_mov_b32 s64, {gap}")
+                # Experiment (landing=N): N plain steps written here, behind the loads of C, so that
+                # their waits count those loads exactly; the loop's waits are written for a queue
+                # without them.  Measured the same as without: vector memory returns in order.
+                for _ in range(landing):
+                    step(kt % 6)
+                    kt += 1
+                E(f"s_mov_b32 s64, {gap - landing}")
                 E(f"s_mov_b32 s75, {j + 1}")
                 E(f"s_branch 1{kt % 6}f")
-                kt += gap
+                kt += gap - landing
         if trace:
             stamp(84)
             E("s_waitcnt lgkmcnt(0)")
@@ -661,13 +673,16 @@ def gen(kind, accum, opts=None, gap=0):
         for q in range(early, 256):
             tm, tn, i = where(q)
             c_ptr(tm)
+            out = "global_store_dword"
+            if add_in_memory:
+                out = "global_atomic_add_f32" if is_float else "global_atomic_add"
             if not unsigned:
-                E(f"global_store_dword {c_addr(tn, i)}, a{q}, s[72:73] offset:{tn * 64}{st_flags}")
+                E(f"{out} {c_addr(tn, i)}, a{q}, s[72:73] offset:{tn * 64}{st_flags}")
             else:
                 t = f"v{16 + q % 32}"
                 E(f"v_accvgpr_read_b32 {t}, a{q}")
                 E(f"v_add_u32 {t}, {t}, v{COL_SUM + tn}")
-                E(f"global_store_dword {c_addr(tn, i)}, {t}, s[72:73] offset:{tn * 64}{st_flags}")
+                E(f"{out} {c_addr(tn, i)}, {t}, s[72:73] offset:{tn * 64}{st_flags}")
     if trace:
         # The stamps replace the first rows of the wave's block of C (a timing build: its results are
         # not looked at): value j at row j % 4, columns 16 * (j / 4) .. + 15 of the block.
@@ -711,8 +726,9 @@ def main():
     out_path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "gemm_wide_gfx950.inc")
     if len(sys.argv) > 1:
         out_path = sys.argv[1]
-    # Experiment switches (timing builds with one ingredient left out, the cycle-stamp build): a
-    # comma-separated list in MRL_WIDE_OPTS.  The library is built with none.
+    # Experiment switches (timing builds with one ingredient left out, the cycle-stamp build, and the
+    # two alternatives landing=N and atomic_c, whose results stay right): a comma-separated list in
+    # MRL_WIDE_OPTS.  The library is built with none.
     opts = {o: True for o in os.environ.get("MRL_WIDE_OPTS", "").split(",") if o}
     for o in list(opts):
         if "=" in o:                  # fill_valu=32 and the like
