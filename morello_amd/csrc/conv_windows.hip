@@ -59,22 +59,33 @@ __global__ __launch_bounds__(256) void k_conv_windows_i8(WindowsArgs p) {
   const uint32_t h = p.oh + p.fh - 1, w = p.ow + p.fw - 1;
   // A tile's patch: rows y0 .. of the image from pixel x0 on; past the image's edge (a ragged
   // tile) the last row / the row's last byte again, which only reaches pixels that are not stored.
+  // Which row and byte of the patch a thread's j-th byte is does not depend on the tile: the
+  // divisions are done once.
   uint8_t held[PATCH_REGS];
-  auto patch_source = [&](uint32_t t, uint32_t i) {
-    const uint32_t img = t / (p.tiles_x * p.tiles_y), in_img = t % (p.tiles_x * p.tiles_y);
-    const uint32_t y0 = (in_img / p.tiles_x) * TILE_H, x0 = (in_img % p.tiles_x) * TILE_W;
-    const uint32_t r = i / patch_wb, xb = i % patch_wb;
-    const uint32_t y = min(y0 + r, h - 1), x = min(x0 * p.c + xb, w * p.c - 1);
-    return p.image + (uint64_t(img) * h + y) * w * p.c + x;
+  uint32_t held_row[PATCH_REGS], held_byte[PATCH_REGS];
+#pragma unroll
+  for (int j = 0; j < PATCH_REGS; j++) {
+    const uint32_t i = tid + j * 256;
+    held_row[j] = i / patch_wb, held_byte[j] = i % patch_wb;
+  }
+  struct Corner {
+    uint32_t img, y0, x0;
+  };
+  auto corner_of = [&](uint32_t t) {
+    const uint32_t per_image = p.tiles_x * p.tiles_y, img = t / per_image, in_img = t - img * per_image, ty = in_img / p.tiles_x;
+    return Corner{img, ty * TILE_H, (in_img - ty * p.tiles_x) * TILE_W};
+  };
+  auto patch_source = [&](const Corner &at, uint32_t r, uint32_t xb) {
+    const uint32_t y = min(at.y0 + r, h - 1), x = min(at.x0 * p.c + xb, w * p.c - 1);
+    return p.image + (uint64_t(at.img) * h + y) * w * p.c + x;
   };
   auto fetch_patch = [&](uint32_t t) {
+    const Corner at = corner_of(t);
 #pragma unroll
-    for (int j = 0; j < PATCH_REGS; j++) {
-      const uint32_t i = tid + j * 256;
-      if (i < patch_bytes) held[j] = *patch_source(t, i);
-    }
+    for (int j = 0; j < PATCH_REGS; j++)
+      if (tid + j * 256 < patch_bytes) held[j] = *patch_source(at, held_row[j], held_byte[j]);
   };
-  auto put = [&](uint32_t i, uint8_t v) { patch[(i / patch_wb) * p.patch_stride + i % patch_wb] = IMG_UNSIGNED ? uint8_t(v ^ 0x80) : v; };
+  auto put = [&](uint32_t r, uint32_t xb, uint8_t v) { patch[r * p.patch_stride + xb] = IMG_UNSIGNED ? uint8_t(v ^ 0x80) : v; };
   if (blockIdx.x < p.tiles) fetch_patch(blockIdx.x);   // the first tile's patch: in flight while the filters are staged
   // The filters, once: run r of filter f at r * seg_padded of the filter's row, zeros everywhere
   // else.  Their nf * k bytes are one contiguous piece of memory: fetched with every load in
@@ -136,15 +147,13 @@ __global__ __launch_bounds__(256) void k_conv_windows_i8(WindowsArgs p) {
     }
   }
   for (uint32_t t = blockIdx.x; t < p.tiles; t += gridDim.x) {
-    const uint32_t img = t / (p.tiles_x * p.tiles_y), in_img = t % (p.tiles_x * p.tiles_y);
-    const uint32_t y0 = (in_img / p.tiles_x) * TILE_H, x0 = (in_img % p.tiles_x) * TILE_W;
+    const Corner at = corner_of(t);
+    const uint32_t img = at.img, y0 = at.y0, x0 = at.x0;
     // 1. the patch out of the registers (what they do not hold, straight from memory)
 #pragma unroll
-    for (int j = 0; j < PATCH_REGS; j++) {
-      const uint32_t i = tid + j * 256;
-      if (i < patch_bytes) put(i, held[j]);
-    }
-    for (uint32_t i = tid + PATCH_REGS * 256; i < patch_bytes; i += 256) put(i, *patch_source(t, i));
+    for (int j = 0; j < PATCH_REGS; j++)
+      if (tid + j * 256 < patch_bytes) put(held_row[j], held_byte[j], held[j]);
+    for (uint32_t i = tid + PATCH_REGS * 256; i < patch_bytes; i += 256) put(i / patch_wb, i % patch_wb, *patch_source(at, i / patch_wb, i % patch_wb));
     __syncthreads();   // also: every wave is done with the previous tile's windows
     // 2. the windows: thread (pixel, half) copies every other run of the pixel's window, eight
     //    dwords at a time (nine aligned dwords read, shifted by the run's byte offset)
