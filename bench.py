@@ -53,6 +53,8 @@ MEASURED_TRAFFIC_BYTES = {
     "decode": 268960727,
     "softmax_long": 77155935,
     "transpose": 537003671,
+    "conv_first": 109303133,
+    "softmax_outer": 101886842,
 }
 KT_LAYOUT = M.layout(0, 2, 1)
 
@@ -130,6 +132,21 @@ def workload(name):
                 np.zeros((32, 28, 28, 128), np.int32)]
         return ("Conv NHWC u8[32x30x30x128] * KRSC i8[128x3x3x128] -> i32[32x28x28x128], valid (implicit Matmul)",
                 spec, arrs, "u8", "TOPS", "hbm", PEAK["hbm_gbs"])
+    if name == "conv_first":
+        # A first layer: three channels per pixel, 7 x 7 filters; the windows are formed in LDS.
+        shape = [32, 64, 3, 112, 112, 7, 7]
+        spec = M.Conv(shape, (M.u8, M.i8, M.i32))
+        arrs = [synth.uniform_u8(13, 0, (32, 118, 118, 3)), synth.uniform_i8(13, 1, (64, 7, 7, 3)),
+                np.zeros((32, 112, 112, 64), np.int32)]
+        return ("Conv NHWC u8[32x118x118x3] * KRSC i8[64x7x7x3] -> i32[32x112x112x64], valid (windows formed in LDS)",
+                spec, arrs, "u8", "TOPS", "hbm", PEAK["hbm_gbs"])
+    if name == "softmax_outer":
+        # A scan over the outer dim of few columns: the scan dim is shared out over workgroups too.
+        shape = [2048, 4096]
+        spec = M.Softmax(shape, 0)
+        arrs = [synth.normal_f32(14, 0, tuple(shape), 2.0), np.zeros(tuple(shape), np.float32)]
+        return ("Softmax{scan_dim 0} f32[2048x4096] (column tiles x pieces of the scan dim, two launches)", spec, arrs,
+                "f32", "GFLOPS", "hbm", PEAK["hbm_gbs"])
     if name == "decode":
         # One query row per entry against a long key sequence: the keys are shared out over
         # workgroups (a stream over K and V).
@@ -515,7 +532,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--spec", default="c2", choices=["c1", "c2", "c2o", "c3", "c4", "c5", "softmax", "move", "matvec", "conv128", "decode", "softmax_long",
-                                                     "transpose"])
+                                                     "transpose", "conv_first", "softmax_outer"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--action", type=int, default=None, metavar="K",
                     help="time the K-th lowering the library lists for the workload's Spec (mrl_target_actions) "
