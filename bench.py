@@ -53,7 +53,7 @@ MEASURED_TRAFFIC_BYTES = {
     "decode": 268960727,
     "softmax_long": 77155935,
     "transpose": 537003671,
-    "conv_first": 109303133,
+    "conv_first": 109310051,
     "softmax_outer": 101886842,
 }
 KT_LAYOUT = M.layout(0, 2, 1)

@@ -639,15 +639,15 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
   const bool unfold_ok = as_matmul && can_unfold && (reinterpret_cast<uintptr_t>(img.t.ptr) & 15) == 0 &&
                          (reinterpret_cast<uintptr_t>(filt.t.ptr) & 15) == 0 && (reinterpret_cast<uintptr_t>(out.t.ptr) & 3) == 0;
   // Few channels per pixel (a first layer): the fused kernel that forms the windows in LDS.
-  const bool windows_ok = fast_types && as_matmul && channels_last(img.t) && channels_last(filt.t) && channels_last(out.t) &&
-                          mrl::conv_windows_applicable(cv) && !(forced == 1 && g_forced->conv_rows);
+  const bool windows_ok = kind >= 0 && kind <= 2 && as_matmul && channels_last(img.t) && channels_last(filt.t) && channels_last(out.t) &&
+                          mrl::conv_windows_applicable(cv, kind) && !(forced == 1 && g_forced->conv_rows);
   if ((forced == 1 && !fused_ok && !windows_ok) || (forced == 2 && !implicit_ok) || (forced == 3 && !unfold_ok)) return MRL_ERR_UNSUPPORTED;
   if (fused_ok && forced <= 1) {
     const bool rows = forced == 1 && g_forced->conv_rows;
     if (rows && !mrl::conv_rows_applicable(cv)) return MRL_ERR_UNSUPPORTED;
     HIP_TRY(mrl::launch_conv_i8(cv, di == MRL_U8, ws.stream, rows));
   } else if (windows_ok && forced <= 1) {
-    HIP_TRY(mrl::launch_conv_windows(cv, di == MRL_U8, ws.stream));
+    HIP_TRY(mrl::launch_conv_windows(cv, kind, ws.stream));
   } else if (implicit_ok && (forced == 0 || forced == 2)) {
     // Channel vectors of whole 16-byte chunks: the windows are read where they lie.  (A 1x1 filter
     // needs no window arithmetic: its image is the left operand of a plain Matmul, below.)
@@ -1550,7 +1550,7 @@ uint32_t mrl_target_layouts_for_shape(const uint32_t *shape, uint32_t rank, int 
 
 uint32_t mrl_target_kernels(const char **names, uint32_t cap) {
   static const char *const families[] = {
-      "k_gemm", "k_gemm_big", "k_gemm_wide", "k_gemv", "k_matmul_generic", "k_sum_splits", "k_conv_i8", "k_conv_rows_i8", "k_conv_windows_i8", "k_conv_generic", "k_conv_generic_wave", "k_unfold",
+      "k_gemm", "k_gemm_big", "k_gemm_wide", "k_gemv", "k_matmul_generic", "k_sum_splits", "k_conv_i8", "k_conv_rows_i8", "k_conv_windows", "k_conv_generic", "k_conv_generic_wave", "k_unfold",
       "k_unfold_gather", "k_attn", "k_attn_merge", "k_softmax_regs", "k_softmax_regs1", "k_softmax_short", "k_softmax_block", "k_softmax_chunk_stats", "k_softmax_chunk_write",
       "k_softmax_cols",
       "k_softmax_generic", "k_parts", "k_broadcast", "k_fill", "k_fill_zero", "k_move_rows", "k_move_rows16",

@@ -1,4 +1,4 @@
-// Conv NHWC u8|i8 x KRSC i8 -> i32 for pixels of few channels (a first layer: 3 channels, 7 x 7
+// Conv NHWC u8|i8 x KRSC i8 -> i32 and bf16 x bf16 -> f32 for pixels of few channels (a first layer: 3 channels, 7 x 7
 // filters), where a pixel's channels are not whole 16-byte chunks and the implicit Matmul of
 // conv_gemm.hip does not apply (morello/src/spec.rs:486-494: no stride, no padding).  The other
 // route for such shapes writes every window to memory first (unfold.hip) and multiplies the rows:
@@ -13,8 +13,10 @@
 //   3. each wave multiplies two rows of the tile (16 pixels each: a B operand block) with the
 //      filters (A operands from LDS, staged once per workgroup in the same padded order, zeros in
 //      the padding, so that whatever the windows hold there counts for nothing):
-//      v_mfma_i32_16x16x64_i8, a lane ends up with 4 consecutive filters of one pixel, 16
-//      contiguous bytes of the channels-last output.
+//      v_mfma_i32_16x16x64_i8 / v_mfma_f32_16x16x32_bf16 (the same 64 bytes of window a step, the
+//      same 16 bytes a lane group), a lane ends up with 4 consecutive filters of one pixel, 16
+//      contiguous bytes of the channels-last output.  bf16: the padding of the windows is zeros
+//      as well (a NaN there times a zero weight would not be zero).
 // The u8 correction 128 * sum of a filter's weights comes from the same MFMAs against an operand
 // of ones, once per workgroup.  Rows of windows and filters lie 16 bytes more than their length
 // apart, which spreads the 16 lanes of an operand read over all banks.
@@ -25,6 +27,9 @@ namespace mrl {
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+enum { IMG_I8 = 0, IMG_U8 = 1, IMG_BF16 = 2 };
 
 constexpr int TILE_H = 8, TILE_W = 16, TILE_PIXELS = TILE_H * TILE_W;
 constexpr int PATCH_REGS = 8;   // patch bytes a thread holds in flight: patches of up to 2 KiB
@@ -32,7 +37,7 @@ constexpr int PATCH_REGS = 8;   // patch bytes a thread holds in flight: patches
 struct WindowsArgs {
   const uint8_t *image, *filters;
   int32_t *out;
-  uint32_t b, f, c, oh, ow, fh, fw;
+  uint32_t b, f, c, oh, ow, fh, fw;   // c: BYTES of one pixel's channels
   int accum;
   uint32_t tiles_x, tiles_y, tiles;   // per image, per image, in all
   uint32_t seg, seg_padded;           // fw * c: bytes of one run of a window; the same in whole dwords
@@ -40,8 +45,14 @@ struct WindowsArgs {
 };
 
 // KS: MFMA k steps per window (fh * seg_padded bytes, padded to 64 KS).
-template <int KS, bool IMG_UNSIGNED>
-__global__ __launch_bounds__(256) void k_conv_windows_i8(WindowsArgs p) {
+template <int KS, int KIND>
+__global__ __launch_bounds__(256) void k_conv_windows(WindowsArgs p) {
+  constexpr bool IMG_UNSIGNED = KIND == IMG_U8, FLOATS = KIND == IMG_BF16;
+  typedef typename std::conditional<FLOATS, v4f, v4i>::type Acc;
+  auto mfma = [](v4i a, v4i b, Acc c) {
+    if constexpr (FLOATS) return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+    else return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+  };
   extern __shared__ __attribute__((aligned(16))) uint8_t win_lds[];
   // Rows of windows and filters: 16 bytes more than their length apart (144 at least: two pixel
   // blocks' rows also hold a block's 16 x 272 bytes of results on their way out).
@@ -134,8 +145,8 @@ __global__ __launch_bounds__(256) void k_conv_windows_i8(WindowsArgs p) {
     }
     __syncthreads();   // the raw bytes are no longer needed: the rows are free for the windows
   }
-  v4i corr[4] = {};
-  if (IMG_UNSIGNED) {
+  Acc corr[4] = {};
+  if constexpr (IMG_UNSIGNED) {
     const v4i ones = v4i{0x01010101, 0x01010101, 0x01010101, 0x01010101};
 #pragma unroll
     for (int fb = 0; fb < 4; fb++) {
@@ -171,15 +182,22 @@ __global__ __launch_bounds__(256) void k_conv_windows_i8(WindowsArgs p) {
           for (int d = 0; d < 9; d++) v[d] = d0 + d <= dwords ? src[d0 + d] : 0;
 #pragma unroll
           for (int d = 0; d < 8; d++)
-            if (d0 + d < dwords) dst[r * dwords + d0 + d] = __builtin_amdgcn_alignbyte(v[d + 1], v[d], shift);
+            if (d0 + d < dwords) {
+              uint32_t out = __builtin_amdgcn_alignbyte(v[d + 1], v[d], shift);
+              if (FLOATS && p.seg - 4 * (d0 + d) < 4) out &= 0xffffu;   // the run ends with half a dword: its padding is zero
+              dst[r * dwords + d0 + d] = out;
+            }
         }
       }
+      // bf16: zeros behind the last run too (the results that left through these rows lie there)
+      if (FLOATS)
+        for (uint32_t d = p.fh * dwords + (tid >> 7); d < KPAD / 4; d += 2) dst[d] = 0;
     }
     __syncthreads();
     const uint32_t next = t + gridDim.x;
     if (next < p.tiles) fetch_patch(next);   // in flight under the MFMAs and the stores
     // 3. two rows of the tile per wave against the group's filters
-    v4i acc[2][4];
+    Acc acc[2][4];
 #pragma unroll
     for (int pb = 0; pb < 2; pb++)
 #pragma unroll
@@ -194,7 +212,7 @@ __global__ __launch_bounds__(256) void k_conv_windows_i8(WindowsArgs p) {
 #pragma unroll
       for (int pb = 0; pb < 2; pb++)
 #pragma unroll
-        for (int fb = 0; fb < 4; fb++) acc[pb][fb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[fb], bop[pb], acc[pb][fb], 0, 0, 0);
+        for (int fb = 0; fb < 4; fb++) acc[pb][fb] = mfma(a[fb], bop[pb], acc[pb][fb]);
     }
     // A lane holds filters 16 fb + 4 lg .. + 3 of pixel (y0 + 2 wave + pb, x0 + li): 16-byte pieces
     // 64 bytes apart.  A pixel block's 16 x 64 results go through the wave's own window rows (no
@@ -205,14 +223,14 @@ __global__ __launch_bounds__(256) void k_conv_windows_i8(WindowsArgs p) {
 #pragma unroll
     for (int pb = 0; pb < 2; pb++) {
 #pragma unroll
-      for (int fb = 0; fb < 4; fb++) *(v4i *)(xb + li * XROW + fb * 64 + lg * 16) = acc[pb][fb];
+      for (int fb = 0; fb < 4; fb++) *(Acc *)(xb + li * XROW + fb * 64 + lg * 16) = acc[pb][fb];
       const uint32_t y = y0 + 2 * wave + pb;
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         const uint32_t pixel = 4 * j + lg, x = x0 + pixel;
-        v4i v = *(const v4i *)(xb + pixel * XROW + li * 16);
+        Acc v = *(const Acc *)(xb + pixel * XROW + li * 16);
         if (y < p.oh && x < p.ow && li < 4 * nfb) {
-          v4i *d = (v4i *)(p.out + ((uint64_t(img) * p.oh + y) * p.ow + x) * p.f + f0 + 4 * li);
+          Acc *d = (Acc *)(p.out + ((uint64_t(img) * p.oh + y) * p.ow + x) * p.f + f0 + 4 * li);
           if (p.accum) v += *d;
           __builtin_nontemporal_store(v, d);
         }
@@ -221,38 +239,51 @@ __global__ __launch_bounds__(256) void k_conv_windows_i8(WindowsArgs p) {
   }
 }
 
-template <int KS>
-hipError_t launch_ks(const WindowsArgs &p, bool img_unsigned, dim3 grid, size_t lds, hipStream_t stream) {
-  static std::atomic<uint64_t> limit_u{0}, limit_s{0};
+template <int KS, int KIND>
+hipError_t launch_kind(const WindowsArgs &p, dim3 grid, size_t lds, hipStream_t stream) {
+  static std::atomic<uint64_t> limit{0};
   if (!plan::recording()) {
-    hipError_t e = img_unsigned ? raise_lds_limit(limit_u, (const void *)k_conv_windows_i8<KS, true>, lds)
-                                : raise_lds_limit(limit_s, (const void *)k_conv_windows_i8<KS, false>, lds);
+    hipError_t e = raise_lds_limit(limit, (const void *)k_conv_windows<KS, KIND>, int(lds));
     if (e != hipSuccess) return e;
   }
-  if (img_unsigned) MRL_LAUNCH((k_conv_windows_i8<KS, true>), grid, dim3(256), lds, stream, p);
-  else MRL_LAUNCH((k_conv_windows_i8<KS, false>), grid, dim3(256), lds, stream, p);
+  MRL_LAUNCH((k_conv_windows<KS, KIND>), grid, dim3(256), lds, stream, p);
   return plan::last_error();
 }
+template <int KS>
+hipError_t launch_ks(const WindowsArgs &p, int kind, dim3 grid, size_t lds, hipStream_t stream) {
+  switch (kind) {
+    case IMG_I8: return launch_kind<KS, IMG_I8>(p, grid, lds, stream);
+    case IMG_U8: return launch_kind<KS, IMG_U8>(p, grid, lds, stream);
+    case IMG_BF16: return launch_kind<KS, IMG_BF16>(p, grid, lds, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+constexpr uint32_t MAX_KS = 6;   // windows of up to 384 bytes: 75 KiB of rows, two workgroups to a compute unit
 
 }  // namespace
 
-// Filters in 16s, windows of at most 256 bytes with their runs padded to dwords, and not a shape
-// conv_gemm.hip reads in place.
-bool conv_windows_applicable(const ConvArgs &c) {
-  const uint64_t seg_padded = (uint64_t(c.fw) * c.c + 3) & ~3ull;
-  return c.f % 16 == 0 && c.f / 64 < 65535 && c.c % 16 != 0 && uint64_t(c.fh) * seg_padded <= 256 &&
+// kind: 0 i8 x i8 -> i32, 1 u8 x i8 -> i32, 2 bf16 x bf16 -> f32.  Filters in 16s, pixels that are
+// not whole 16-byte chunks (those conv_gemm.hip reads in place), windows of at most 64 MAX_KS
+// bytes with their runs padded to dwords.
+bool conv_windows_applicable(const ConvArgs &c, int kind) {
+  if (kind < 0 || kind > 2) return false;
+  const uint64_t es = kind == 2 ? 2 : 1, c_bytes = c.c * es, seg_padded = (uint64_t(c.fw) * c_bytes + 3) & ~3ull;
+  return c.f % 16 == 0 && c.f / 64 < 65535 && c_bytes % 16 != 0 && uint64_t(c.fh) * seg_padded <= 64 * MAX_KS &&
          uint64_t(c.b) * ((c.oh + TILE_H - 1) / TILE_H) * ((c.ow + TILE_W - 1) / TILE_W) < (1ull << 31) &&
-         (reinterpret_cast<uintptr_t>(c.out) & 15) == 0;
+         (reinterpret_cast<uintptr_t>(c.out) & 15) == 0 && (reinterpret_cast<uintptr_t>(c.image) & (es - 1)) == 0 &&
+         (reinterpret_cast<uintptr_t>(c.filters) & (es - 1)) == 0;
 }
 
-hipError_t launch_conv_windows(const ConvArgs &c, bool img_unsigned, hipStream_t stream) {
-  if (!conv_windows_applicable(c)) return hipErrorInvalidValue;
+hipError_t launch_conv_windows(const ConvArgs &c, int kind, hipStream_t stream) {
+  if (!conv_windows_applicable(c, kind)) return hipErrorInvalidValue;
+  const uint32_t es = kind == 2 ? 2 : 1;
   WindowsArgs p;
   p.image = (const uint8_t *)c.image, p.filters = (const uint8_t *)c.filters, p.out = (int32_t *)c.out;
-  p.b = c.b, p.f = c.f, p.c = c.c, p.oh = c.oh, p.ow = c.ow, p.fh = c.fh, p.fw = c.fw, p.accum = c.accum;
+  p.b = c.b, p.f = c.f, p.c = c.c * es, p.oh = c.oh, p.ow = c.ow, p.fh = c.fh, p.fw = c.fw, p.accum = c.accum;
   p.tiles_x = (c.ow + TILE_W - 1) / TILE_W, p.tiles_y = (c.oh + TILE_H - 1) / TILE_H, p.tiles = c.b * p.tiles_x * p.tiles_y;
-  p.seg = c.fw * c.c, p.seg_padded = (p.seg + 3) & ~3u;
-  p.patch_stride = ((TILE_W + c.fw - 1) * c.c + 3) & ~3u;
+  p.seg = c.fw * p.c, p.seg_padded = (p.seg + 3) & ~3u;
+  p.patch_stride = ((TILE_W + c.fw - 1) * p.c + 3) & ~3u;
   const int ks = int((c.fh * p.seg_padded + 63) / 64);
   const size_t row = ks == 1 ? 144 : 64 * ks + 16;
   // the copies read one dword past a run's last: four bytes behind the patch
@@ -263,14 +294,16 @@ hipError_t launch_conv_windows(const ConvArgs &c, bool img_unsigned, hipStream_t
   const uint32_t groups = (c.f + 63) / 64;
   const uint32_t wgs = std::min<uint32_t>(p.tiles, std::max(1u, g_compute_units * per_cu / groups));
   const double pixels = double(c.b) * c.oh * c.ow;
-  plan::work(plan::UNIT_STREAM, 0, 1.5 * (pixels * c.f * 4 * (c.accum ? 2 : 1) + double(c.b) * (c.oh + c.fh - 1) * (c.ow + c.fw - 1) * c.c),
+  plan::work(plan::UNIT_STREAM, 0, 1.5 * (pixels * c.f * 4 * (c.accum ? 2 : 1) + double(c.b) * (c.oh + c.fh - 1) * (c.ow + c.fw - 1) * p.c),
              0, 6000.0 + (1500.0 + 1000.0 * ks) * double((p.tiles + wgs - 1) / wgs));   // staging the filters; a tile
   const dim3 grid(wgs, groups);
   switch (ks) {
-    case 1: return launch_ks<1>(p, img_unsigned, grid, lds, stream);
-    case 2: return launch_ks<2>(p, img_unsigned, grid, lds, stream);
-    case 3: return launch_ks<3>(p, img_unsigned, grid, lds, stream);
-    case 4: return launch_ks<4>(p, img_unsigned, grid, lds, stream);
+    case 1: return launch_ks<1>(p, kind, grid, lds, stream);
+    case 2: return launch_ks<2>(p, kind, grid, lds, stream);
+    case 3: return launch_ks<3>(p, kind, grid, lds, stream);
+    case 4: return launch_ks<4>(p, kind, grid, lds, stream);
+    case 5: return launch_ks<5>(p, kind, grid, lds, stream);
+    case 6: return launch_ks<6>(p, kind, grid, lds, stream);
     default: return hipErrorInvalidValue;
   }
 }

@@ -147,10 +147,11 @@ bool conv_i8_applicable(const ConvArgs &c);
 bool conv_rows_applicable(const ConvArgs &c);
 hipError_t launch_conv_i8(const ConvArgs &c, bool img_unsigned, hipStream_t stream, bool whole_rows = false);
 
-// ---- conv_windows.hip: Conv u8|i8 x i8 -> i32, channels-last, pixels of few channels (not whole
-// 16-byte chunks), windows of at most 256 bytes, filters in 16s: the windows are formed in LDS.
-bool conv_windows_applicable(const ConvArgs &c);
-hipError_t launch_conv_windows(const ConvArgs &c, bool img_unsigned, hipStream_t stream);
+// ---- conv_windows.hip: Conv u8|i8 x i8 -> i32 and bf16 x bf16 -> f32 (kind 0, 1, 2 as for a Matmul),
+// channels-last, pixels of few channels (not whole 16-byte chunks), windows of at most 384
+// bytes, filters in 16s: the windows are formed in LDS.
+bool conv_windows_applicable(const ConvArgs &c, int kind);
+hipError_t launch_conv_windows(const ConvArgs &c, int kind, hipStream_t stream);
 
 // ---- unfold.hip: the windows of a channels-last image as rows, for Conv as a Matmul ---------
 // image: [batch][oh+fh-1][ow+fw-1][c]; rows: [batch*oh*ow][row_elems], each row the fh*fw*c

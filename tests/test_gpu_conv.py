@@ -151,7 +151,7 @@ def test_conv_with_few_channels_forms_its_windows_in_lds(gpu, shape, accum, img_
     otherwise; once more with the image and the filters at addresses that are not 16-byte aligned."""
     b, f, c, oh, ow, fh, fw = shape
     spec = M.Conv(list(shape), (img_dt, M.i8, M.i32), accum=accum)
-    assert spec.plan().kernels == ["k_conv_windows_i8"]
+    assert spec.plan().kernels == ["k_conv_windows"]
     img = gen(134, 0, (b, oh + fh - 1, ow + fw - 1, c))
     filt = synth.uniform_i8(134, 1, (f, fh, fw, c))
     out0 = (synth.uniform_i8(134, 2, (b, oh, ow, f)).astype(np.int32) * 1001) if accum else np.full((b, oh, ow, f), -5, np.int32)
@@ -166,6 +166,36 @@ def test_conv_with_few_channels_forms_its_windows_in_lds(gpu, shape, accum, img_
     for x in bufs:
         x.free()
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("shape,accum", [
+    ((2, 64, 3, 20, 37, 7, 7), False),    # a first layer in bf16: runs of 42 bytes padded to 44, five k steps
+    ((4, 16, 1, 30, 30, 3, 3), True),     # runs of 6 bytes
+    ((2, 80, 3, 17, 15, 5, 5), True),     # two groups of filters
+    ((1, 64, 5, 30, 30, 1, 1), False),    # 1 x 1 filters, runs of 10 bytes
+    ((2, 32, 12, 9, 21, 3, 3), False),    # 24 bytes a pixel
+])
+def test_bf16_conv_with_few_channels_forms_its_windows_in_lds(gpu, shape, accum):
+    """The same kernel on bf16 operands (f32 sums, as a bf16 Matmul's).  An image that holds a NaN
+    and an infinity: they reach exactly the outputs whose windows contain them, not their
+    neighbours through the padding of the windows' runs."""
+    b, f, c, oh, ow, fh, fw = shape
+    spec = M.Conv(list(shape), (M.bf16, M.bf16, M.f32), accum=accum)
+    assert spec.plan().kernels == ["k_conv_windows"] and "KIND = 2" in spec.plan().steps[0].kernel
+    img = synth.normal_bf16(135, 0, (b, oh + fh - 1, ow + fw - 1, c))
+    filt = synth.normal_bf16(135, 1, (f, fh, fw, c))
+    out0 = synth.uniform_u8(135, 2, (b, oh, ow, f)).astype(np.float32) if accum else np.full((b, oh, ow, f), 7, np.float32)
+    want = orc.conv(list(shape), [7, 7, 6], img, filt, out0.copy(), accum, layouts=[NHWC] * 3)
+    got = run_spec(spec, [img, filt, out0.copy()])
+    assert float(np.abs(got.astype(np.float64) - want).max() / np.abs(want).max()) < 1e-5
+    img = img.copy()
+    img[0, 0, 0, 0] = 0x7fc0                                   # NaN in the first pixel's first channel
+    img[b - 1, oh + fh - 2, ow + fw - 2, c - 1] = 0x7f80       # +inf in the last pixel's last channel
+    want = orc.conv(list(shape), [7, 7, 6], img, filt, out0.copy(), accum, layouts=[NHWC] * 3)
+    got = run_spec(spec, [img, filt, out0.copy()])
+    assert np.array_equal(np.isfinite(got), np.isfinite(want))
+    ok = np.isfinite(want)
+    assert float(np.abs(got[ok].astype(np.float64) - want[ok]).max() / np.abs(want[ok]).max()) < 1e-5
 
 
 def test_conv_as_matmul_from_nchw(gpu):
