@@ -998,6 +998,24 @@ int run_broadcast(const mrl_spec &s, void *const *params, Workspace &ws) {
   uint32_t ishape[MRL_MAX_RANK], oshape[MRL_MAX_RANK], rank;
   parameter_shape(s, 0, ishape, &rank);
   parameter_shape(s, 1, oshape, &rank);
+  // Both tensors row-major: whole 16-byte pieces, no index arithmetic per element.
+  int64_t si[MRL_MAX_RANK], so[MRL_MAX_RANK];
+  if (mrl::layout_strides(s.layouts[0], ishape, rank, si) && mrl::layout_strides(s.layouts[1], oshape, rank, so)) {
+    bool dense = true;
+    int64_t run_i = 1, run_o = 1;
+    for (int d = int(rank) - 1; d >= 0; d--) {
+      dense = dense && (ishape[d] == 1 || si[d] == run_i) && (oshape[d] == 1 || so[d] == run_o);
+      run_i *= ishape[d], run_o *= oshape[d];
+    }
+    uint64_t before = 1, after = 1;
+    for (uint32_t d = 0; d < rank; d++) (d < s.scan_dim ? before : after) *= d == s.scan_dim ? 1 : oshape[d];
+    hipError_t err = hipSuccess;
+    if (dense && mrl::launch_broadcast_rows(params[0], params[1], before, oshape[s.scan_dim], after,
+                                            uint32_t(mrl_dtype_size(s.dtypes[0])), ws.stream, &err)) {
+      HIP_TRY(err);
+      return MRL_OK;
+    }
+  }
   mrl::LayoutEval il, ol;
   if (!mrl::make_layout_eval(s.layouts[0], ishape, rank, &il) ||
       !mrl::make_layout_eval(s.layouts[1], oshape, rank, &ol))
@@ -1553,7 +1571,7 @@ uint32_t mrl_target_kernels(const char **names, uint32_t cap) {
       "k_gemm", "k_gemm_big", "k_gemm_wide", "k_gemv", "k_matmul_generic", "k_sum_splits", "k_conv_i8", "k_conv_rows_i8", "k_conv_windows", "k_conv_generic", "k_conv_generic_wave", "k_unfold",
       "k_unfold_gather", "k_attn", "k_attn_merge", "k_softmax_regs", "k_softmax_regs1", "k_softmax_short", "k_softmax_block", "k_softmax_chunk_stats", "k_softmax_chunk_write",
       "k_softmax_cols",
-      "k_softmax_generic", "k_parts", "k_broadcast", "k_fill", "k_fill_zero", "k_move_rows", "k_move_rows16",
+      "k_softmax_generic", "k_parts", "k_parts_rows", "k_parts_cols", "k_broadcast", "k_broadcast_rows", "k_broadcast_fill_rows", "k_fill", "k_fill_zero", "k_move_rows", "k_move_rows16",
       "k_move_tiled", "k_move_tiled_as", "k_move_tiled8v", "k_move_tiled16", "k_move_tiled16v", "k_move_tiled32", "k_move_gather", "k_move_generic", "k_relayout", "k_convert4", "k_copy1",
       "k_copy16", "k_pad_rows", "k_pad_rows16", "k_widen_bf16"};
   const uint32_t n = sizeof families / sizeof families[0];

@@ -185,6 +185,11 @@ struct PartsArgs {
 hipError_t launch_parts(const PartsArgs &p, hipStream_t stream);
 hipError_t launch_broadcast(const void *in, void *out, const LayoutEval &il, const LayoutEval &ol,
                             uint32_t dim, uint32_t elem_size, uint64_t count, hipStream_t stream);
+// Broadcast between row-major tensors as out[before][n][after] <- in[before][after], elements of es
+// bytes: true (and *err set) if one of the 16-byte forms took it, false if the shape or the
+// pointers' alignment leave it to launch_broadcast.
+bool launch_broadcast_rows(const void *in, void *out, uint64_t before, uint32_t n, uint64_t after, uint32_t es,
+                           hipStream_t stream, hipError_t *err);
 hipError_t launch_fill(void *out, int dtype, int fill_value, uint64_t count, hipStream_t stream);
 
 // ---- mfma_rate.hip: sustained matrix-core rate of this board (measurement, not a Spec) ----

@@ -13,7 +13,11 @@ pytestmark = pytest.mark.gpu
 
 RNG = np.random.default_rng(77)
 SHAPES = [((7, 33), 1), ((5, 9, 4), 1), ((3, 4, 130), 2), ((6, 5), 0), ((2, 3, 4, 5), 2),
-          ((64, 2048), 1), ((1, 1, 1), 1), ((4, 1, 300), 2)]
+          ((64, 2048), 1), ((1, 1, 1), 1), ((4, 1, 300), 2),
+          # contiguous lines of whole 16-byte vectors: register-resident (4, 8, 16 vectors a lane)
+          ((33, 1024), 1), ((5, 12), 1), ((7, 3, 2048), 2), ((9, 4096), 1), ((3, 4100), 1),
+          # the scan dim is not the innermost: lines side by side, 16, 32 or 64 to a workgroup
+          ((37, 70), 0), ((3, 50, 33), 1), ((2, 300, 64), 1), ((5, 20000), 0), ((8, 40000), 0), ((1, 18), 0)]
 TOL = dict(rtol=1e-5, atol=1e-7)
 
 
@@ -79,7 +83,44 @@ def test_softmax_denominator_and_max(gpu, shape, dim, accum):
     np.testing.assert_allclose(got[2], want[2], **tol(shape, dim))
 
 
-@pytest.mark.parametrize("shape,dim", [((6, 5), 1), ((3, 9, 4), 1), ((4, 70), 1), ((8, 3), 0)])
+@pytest.mark.parametrize("shape,dim", [((9, 130), 1), ((6, 1024), 1), ((300, 40), 0), ((5, 20000), 0)])
+def test_softmax_denominator_and_max_of_masked_lines(gpu, shape, dim):
+    """Lines with elements of -inf (masked positions), at their start too, and one line that is
+    -inf throughout: the pair is the closed form's -- max over the line, sum of exp(x - max), a
+    masked element adding exp(-inf) = 0 -- on every kernel that takes these Specs (a wavefront
+    per line, the register-resident form, lines side by side); the line of nothing but -inf has
+    max -inf and a denominator of NaN (every term is exp(-inf - -inf)), as the reference's
+    recurrence gives it (codegen/cpu.rs:1360-1389).  The reference's recurrence, fed -inf before
+    the first finite element, turns the whole line's denominator into NaN; that is not copied."""
+    x = rnd(shape)
+    mask = RNG.random(shape) < 0.3
+    lead = [slice(None)] * len(shape)
+    lead[dim] = slice(0, min(11, shape[dim] - 1))
+    mask[tuple(lead)] = True
+    x[mask] = -np.inf
+    whole = [0] * len(shape)
+    whole[dim] = slice(None)
+    x[tuple(whole)] = -np.inf
+    mx, dn = np.zeros(reduced(shape, dim), np.float32), np.zeros(reduced(shape, dim), np.float32)
+    got = run_all(M.SoftmaxDenominatorAndMax(shape, dim), [x, mx, dn])
+    x64 = x.astype(np.float64)
+    m = x64.max(axis=dim, keepdims=True)
+    with np.errstate(invalid="ignore"):
+        d = np.exp(x64 - m).sum(axis=dim, keepdims=True)
+    assert np.array_equal(got[1], m.astype(np.float32))
+    first = tuple(0 for _ in shape)
+    assert np.isnan(got[2][first]) and np.isnan(d[first])
+    keep = np.ones(d.shape, bool)
+    keep[first] = False
+    np.testing.assert_allclose(got[2][keep], d[keep], rtol=2e-5)
+    # the two-step forms agree: Max, then SoftmaxDenominator against it
+    got_m = run_all(M.Max(shape, dim), [x, mx])[1]
+    got_d = run_all(M.SoftmaxDenominator(shape, dim), [x, got_m, dn])[2]
+    assert np.array_equal(got_m, got[1])
+    np.testing.assert_allclose(got_d[keep], got[2][keep], rtol=2e-5)
+
+
+@pytest.mark.parametrize("shape,dim", [((6, 5), 1), ((3, 9, 4), 1), ((4, 70), 1), ((8, 3), 0), ((40, 33), 0), ((3, 20, 64), 1)])
 @pytest.mark.parametrize("accum", [False, True])
 def test_softmax_denominator_and_max_from_parts(gpu, shape, dim, accum):
     tmax, tden = rnd(shape, 4.0), np.abs(rnd(shape)) + np.float32(1.0)
@@ -231,7 +272,10 @@ def test_fill(gpu, dtype, np_dtype, code, value):
     assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
 
 
-@pytest.mark.parametrize("shape,dim", [((4, 9), 0), ((4, 9), 1), ((3, 5, 7), 1), ((2, 3, 4, 5), 3)])
+@pytest.mark.parametrize("shape,dim", [((4, 9), 0), ((4, 9), 1), ((3, 5, 7), 1), ((2, 3, 4, 5), 3),
+                                       # whole 16-byte pieces behind the dim, or of the innermost dim itself
+                                       ((4, 8, 64), 1), ((70, 16), 0), ((300, 3, 48), 1), ((16, 256), 1), ((1000, 32), 1),
+                                       ((5, 6, 16), 2), ((3, 40, 20), 1)])
 @pytest.mark.parametrize("dtype,np_dtype", [(M.f32, np.float32), (M.u8, np.uint8), (M.bf16, np.uint16)])
 def test_broadcast(gpu, shape, dim, dtype, np_dtype):
     x = RNG.integers(0, 250, size=reduced(shape, dim)).astype(np_dtype)

@@ -338,6 +338,31 @@ def test_cost_model_ranks_manual_schedules(gpu):
                         assert measured[x] <= 1.25 * measured[y], (dts[0], m, k, n, x, y, measured, predicted)
 
 
+def test_plans_of_the_softmax_primitives():
+    """Host only: which kernel a primitive of the decomposition takes.  Contiguous lines of up to
+    4096 elements in whole 16-byte vectors stay in a wavefront's registers; a scan dim that is
+    not the innermost puts 16, 32 or 64 lines side by side in a workgroup, as many as still
+    leave two workgroups per compute unit; anything else a wavefront per line.  Broadcast
+    between row-major tensors moves 16-byte pieces."""
+    kernel = lambda spec: (spec.plan().steps[0].family, spec.plan().steps[0].grid[:2])
+    assert kernel(M.Max([16, 2048, 2048], 2)) == ("k_parts_rows", (8192, 1))
+    assert kernel(M.SoftmaxComplete([7, 12], 1))[0] == "k_parts_rows"
+    assert kernel(M.Max([3, 4100], 1))[0] == "k_parts" and kernel(M.Max([7, 33], 1))[0] == "k_parts"
+    assert kernel(M.DivideVec([64, 64]))[0] == "k_parts"
+    assert kernel(M.SoftmaxDenominatorAndMax([2048, 4096], 0)) == ("k_parts_cols", (256, 1))     # 16 lines each
+    assert kernel(M.SoftmaxDenominatorAndMax([5, 20000], 0)) == ("k_parts_cols", (625, 1))       # 32
+    assert kernel(M.SoftmaxDenominatorAndMax([8, 40000], 0)) == ("k_parts_cols", (625, 1))       # 64
+    assert kernel(M.Max([5, 9, 4], 1))[0] == "k_parts"                                           # rows of 4 elements: not worth lining up
+    # col-major: the lines are contiguous, each starting on any 4 bytes
+    assert kernel(M.Max([33, 64], 0, layouts=[M.col_major([33, 64]), None]))[0] == "k_parts"
+    one_read, two_reads = M.SoftmaxDenominatorAndUnscaled([64, 1024], 1).plan(), M.SoftmaxDenominatorAndUnscaled([1024, 64], 0).plan()
+    assert one_read.steps[0].bytes == 2 * 4 * 65536 and two_reads.steps[0].bytes == 3 * 4 * 65536
+    assert kernel(M.Broadcast([16, 2048, 2048], 2))[0] == "k_broadcast_fill_rows"
+    assert kernel(M.Broadcast([2048, 4096], 0)) == ("k_broadcast_rows", (4, 512))
+    assert kernel(M.Broadcast([4, 9], 1))[0] == "k_broadcast" and kernel(M.Broadcast([6, 32], 1, M.u8))[0] == "k_broadcast_fill_rows"
+    assert kernel(M.Broadcast([4, 8, 64], 1, layouts=[None, M.layout(2, 1, 0)]))[0] == "k_broadcast"
+
+
 def test_actions_of_a_softmax():
     """Host only: the Softmax stage of C5 on its own lists the fused kernels' choice, the two
     whole-row rewrites and the tiled one for every power-of-two tile count down to 64-element
@@ -347,7 +372,8 @@ def test_actions_of_a_softmax():
     assert [a.kind for a in acts] == [K.Select, K.ToSoftmaxParts, K.ToSoftmaxPartsRecompute] + [K.ParallelSoftmax] * 5
     assert [a.parts for a in acts[3:]] == [2, 4, 8, 16, 32]
     assert acts[0].plan().kernels == ["k_softmax_regs"]
-    assert acts[1].plan().kernels == ["k_parts", "k_parts"] and acts[3].plan().kernels == ["k_parts"] * 3
+    # whole contiguous lines stay in a wavefront's registers; the merge of the tiles' pairs walks a handful of them
+    assert acts[1].plan().kernels == ["k_parts_rows"] * 2 and acts[3].plan().kernels == ["k_parts_rows", "k_parts", "k_parts_rows"]
     assert all(a.cost_ns > acts[0].cost_ns for a in acts[1:])
     assert acts[1].scratch_bytes >= 16 * 2048 * 4 and acts[3].scratch_bytes >= 16 * 2048 * 4 * (2 + 2 * 2)
     # integers and other dtypes have no Softmax; a Matmul lists none of these
