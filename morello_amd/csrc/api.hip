@@ -714,58 +714,92 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
   return finish_output(out, ws);
 }
 
+// A Softmax's two tensors and shape, possibly with the dims renumbered into storage order.
+struct Shaped {
+  uint32_t rank, scan_dim, shape[MRL_MAX_RANK];
+  mrl::Strided in, out;
+};
+
 int run_softmax(const mrl_spec &s, void *const *params, Workspace &ws) {
   Prepared in, out;
   int rc;
   if ((rc = prepare(s, 0, params[0], true, ws, &in)) != MRL_OK) return rc;
   if ((rc = prepare(s, 1, params[1], false, ws, &out)) != MRL_OK) return rc;
+  // The dims in the order the tensors are stored, when both are stored the same dense way: a
+  // column-major tensor scanned along dim 0 is a row-major one scanned along its rows.
+  Shaped v;
+  v.rank = s.rank, v.scan_dim = s.scan_dim, v.in = in.t, v.out = out.t;
+  for (uint32_t d = 0; d < MRL_MAX_RANK; d++) v.shape[d] = d < s.rank ? s.spec_shape[d] : 1;
+  if (!dense_row_major(in.t) && s.spec_shape[s.scan_dim] > 1) {
+    uint32_t order[MRL_MAX_RANK];
+    bool same = true;
+    for (uint32_t d = 0; d < s.rank; d++) {
+      order[d] = d;
+      same = same && (s.spec_shape[d] == 1 || in.t.stride[d] == out.t.stride[d]);
+    }
+    // size-one dims first (they address nothing), the others by falling stride
+    std::stable_sort(order, order + s.rank, [&](uint32_t x, uint32_t y) {
+      const bool ux = s.spec_shape[x] == 1, uy = s.spec_shape[y] == 1;
+      if (ux != uy) return ux;
+      return !ux && in.t.stride[x] > in.t.stride[y];
+    });
+    Shaped w = v;
+    for (uint32_t i = 0; i < s.rank; i++) {
+      const uint32_t d = order[i];
+      w.shape[i] = s.spec_shape[d];
+      w.in.shape[i] = w.out.shape[i] = s.spec_shape[d];
+      w.in.stride[i] = in.t.stride[d], w.out.stride[i] = out.t.stride[d];
+      if (d == s.scan_dim) w.scan_dim = i;
+    }
+    if (same && dense_row_major(w.in) && dense_row_major(w.out)) v = w;
+  }
   // Trailing size-one dims do not change which dim is innermost.
-  uint32_t last = s.rank - 1;
-  while (last > s.scan_dim && s.spec_shape[last] == 1) last--;
-  if (s.scan_dim == last && dense_row_major(in.t) && dense_row_major(out.t) &&
-      (reinterpret_cast<uintptr_t>(in.t.ptr) & 15) == 0 &&
-      (reinterpret_cast<uintptr_t>(out.t.ptr) & 15) == 0) {
-    const uint32_t cols = s.spec_shape[s.scan_dim];
+  uint32_t last = v.rank - 1;
+  while (last > v.scan_dim && v.shape[last] == 1) last--;
+  if (v.scan_dim == last && dense_row_major(v.in) && dense_row_major(v.out) &&
+      (reinterpret_cast<uintptr_t>(v.in.ptr) & 15) == 0 &&
+      (reinterpret_cast<uintptr_t>(v.out.ptr) & 15) == 0) {
+    const uint32_t cols = v.shape[v.scan_dim];
     void *scratch = nullptr;
     if (const size_t bytes = mrl::softmax_scratch_bytes(in.count / cols, cols)) HIP_TRY(ws.alloc(&scratch, bytes));
-    HIP_TRY(mrl::launch_softmax_rows((const float *)in.t.ptr, (float *)out.t.ptr, in.count / cols,
+    HIP_TRY(mrl::launch_softmax_rows((const float *)v.in.ptr, (float *)v.out.ptr, in.count / cols,
                                      cols, scratch, ws.stream));
-  } else if (s.scan_dim < last && dense_row_major(in.t) && dense_row_major(out.t) && in.count < (1ull << 31) &&
+  } else if (v.scan_dim < last && dense_row_major(v.in) && dense_row_major(v.out) && in.count < (1ull << 31) &&
              [&] {
                uint64_t after = 1;
-               for (uint32_t d = s.scan_dim + 1; d < s.rank; d++) after *= s.spec_shape[d];
+               for (uint32_t d = v.scan_dim + 1; d < v.rank; d++) after *= v.shape[d];
                return after >= 16;
              }()) {
     // The tensor as [before][scan][after] with `after` contiguous: the column kernel, 64
     // positions of `after` per workgroup; with few columns the scan dim is shared out as well.
-    const uint32_t scan = s.spec_shape[s.scan_dim];
+    const uint32_t scan = v.shape[v.scan_dim];
     uint64_t before = 1, after = 1;
-    for (uint32_t d = 0; d < s.scan_dim; d++) before *= s.spec_shape[d];
-    for (uint32_t d = s.scan_dim + 1; d < s.rank; d++) after *= s.spec_shape[d];
+    for (uint32_t d = 0; d < v.scan_dim; d++) before *= v.shape[d];
+    for (uint32_t d = v.scan_dim + 1; d < v.rank; d++) after *= v.shape[d];
     mrl::Strided vi, vo;
     vi.dtype = vo.dtype = MRL_F32, vi.rank = vo.rank = 3;
     for (uint32_t d = 0; d < MRL_MAX_RANK; d++) vi.shape[d] = vo.shape[d] = 1, vi.stride[d] = vo.stride[d] = 0;
     vi.shape[0] = vo.shape[0] = uint32_t(before), vi.shape[1] = vo.shape[1] = scan, vi.shape[2] = vo.shape[2] = uint32_t(after);
     vi.stride[0] = vo.stride[0] = int64_t(scan) * after, vi.stride[1] = vo.stride[1] = int64_t(after), vi.stride[2] = vo.stride[2] = 1;
-    vi.ptr = in.t.ptr, vo.ptr = out.t.ptr;
+    vi.ptr = v.in.ptr, vo.ptr = v.out.ptr;
     void *pairs = nullptr;
     if (const size_t bytes = mrl::softmax_cols_scratch_bytes(before * ((after + 63) / 64), scan)) HIP_TRY(ws.alloc(&pairs, bytes));
     HIP_TRY(mrl::launch_softmax_generic(vi, vo, 1, pairs, ws.stream));
-  } else if (s.scan_dim < last && dense_row_major(in.t) && dense_row_major(out.t) && in.count < (1ull << 31) &&
+  } else if (v.scan_dim < last && dense_row_major(v.in) && dense_row_major(v.out) && in.count < (1ull << 31) &&
              [&] {
                // Fewer than 16 contiguous elements behind the scan dim: the generic kernel, a
                // wavefront per line with strided accesses, measured 2.5 us + 10 ns per scan step on
                // small tensors; against it three or four launches, ~14 us.
-               const double scan = s.spec_shape[s.scan_dim];
+               const double scan = v.shape[v.scan_dim];
                if (in.count <= (1u << 20)) return 2.5 + 0.010 * scan > 15.0;
                return true;
              }()) {
     // Scan dim made innermost by a transposing Move, the row kernels, and a Move back: three
     // passes of tuned kernels ([2149, 172] over dim 0: 57 -> 9 us; [1818, 10]: 23 -> 8 us).
-    const uint32_t scan = s.spec_shape[s.scan_dim];
+    const uint32_t scan = v.shape[v.scan_dim];
     uint64_t before = 1, after = 1;
-    for (uint32_t d = 0; d < s.scan_dim; d++) before *= s.spec_shape[d];
-    for (uint32_t d = s.scan_dim + 1; d < s.rank; d++) after *= s.spec_shape[d];
+    for (uint32_t d = 0; d < v.scan_dim; d++) before *= v.shape[d];
+    for (uint32_t d = v.scan_dim + 1; d < v.rank; d++) after *= v.shape[d];
     void *turned = nullptr, *scratch = nullptr;
     HIP_TRY(ws.alloc(&turned, in.count * sizeof(float)));
     mrl::Strided as_given, as_turned;  // both over the index space (before, scan, after)
@@ -776,15 +810,15 @@ int run_softmax(const mrl_spec &s, void *const *params, Workspace &ws) {
     as_given.shape[2] = as_turned.shape[2] = uint32_t(after);
     as_given.stride[0] = int64_t(scan) * after, as_given.stride[1] = int64_t(after), as_given.stride[2] = 1;
     as_turned.stride[0] = int64_t(scan) * after, as_turned.stride[1] = 1, as_turned.stride[2] = scan;
-    as_given.ptr = in.t.ptr, as_turned.ptr = turned;
+    as_given.ptr = v.in.ptr, as_turned.ptr = turned;
     HIP_TRY(mrl::launch_move_strided(as_given, as_turned, ws.stream));
     const uint64_t rows = before * after;
     if (const size_t bytes = mrl::softmax_scratch_bytes(rows, scan)) HIP_TRY(ws.alloc(&scratch, bytes));
     HIP_TRY(mrl::launch_softmax_rows((const float *)turned, (float *)turned, rows, scan, scratch, ws.stream));
-    as_given.ptr = out.t.ptr;
+    as_given.ptr = v.out.ptr;
     HIP_TRY(mrl::launch_move_strided(as_turned, as_given, ws.stream));
   } else {
-    HIP_TRY(mrl::launch_softmax_generic(in.t, out.t, s.scan_dim, nullptr, ws.stream));
+    HIP_TRY(mrl::launch_softmax_generic(v.in, v.out, v.scan_dim, nullptr, ws.stream));
   }
   return finish_output(out, ws);
 }
@@ -1041,12 +1075,14 @@ int run_one_prefix(const mrl_spec &s, void *const *params, Workspace &ws) {
     pd.logical_dim--;
     lo.dims[lo.ndims++] = pd;
   }
-  mrl::LayoutEval sl, dl;
-  if (!mrl::make_layout_eval(s.layouts[0], shape, rank, &sl) || !mrl::make_layout_eval(lo, shape, rank, &dl))
-    return MRL_ERR_BAD_LAYOUT;
-  HIP_TRY(mrl::launch_move_generic(params[0], params[1], sl, dl, s.dtypes[0], s.dtypes[1],
-                                   volume(shape, rank), ws.stream));
-  return MRL_OK;
+  // What is left is a Move over the input's shape: the plain copy when the two orders agree,
+  // the strided kernels when they share a view.
+  mrl_spec mv;
+  std::memset(&mv, 0, sizeof mv);
+  mv.kind = MRL_SPEC_MOVE, mv.n_params = 2, mv.rank = rank;
+  for (uint32_t d = 0; d < rank; d++) mv.spec_shape[d] = shape[d];
+  mv.dtypes[0] = s.dtypes[0], mv.dtypes[1] = s.dtypes[1], mv.layouts[0] = s.layouts[0], mv.layouts[1] = lo;
+  return run_move(mv, params, ws);
 }
 
 // Matmul / Conv with a bf16 output (a legal dtype triple, spec.rs:3663-3698).  The reference's
@@ -1571,7 +1607,7 @@ uint32_t mrl_target_kernels(const char **names, uint32_t cap) {
       "k_gemm", "k_gemm_big", "k_gemm_wide", "k_gemv", "k_matmul_generic", "k_sum_splits", "k_conv_i8", "k_conv_rows_i8", "k_conv_windows", "k_conv_generic", "k_conv_generic_wave", "k_unfold",
       "k_unfold_gather", "k_attn", "k_attn_merge", "k_softmax_regs", "k_softmax_regs1", "k_softmax_short", "k_softmax_block", "k_softmax_chunk_stats", "k_softmax_chunk_write",
       "k_softmax_cols",
-      "k_softmax_generic", "k_parts", "k_parts_rows", "k_parts_cols", "k_broadcast", "k_broadcast_rows", "k_broadcast_fill_rows", "k_fill", "k_fill_zero", "k_move_rows", "k_move_rows16",
+      "k_softmax_generic", "k_parts", "k_parts_rows", "k_parts_cols", "k_broadcast", "k_broadcast_rows", "k_broadcast_fill_rows", "k_fill", "k_fill16", "k_fill_zero", "k_move_rows", "k_move_rows16",
       "k_move_tiled", "k_move_tiled_as", "k_move_tiled8v", "k_move_tiled16", "k_move_tiled16v", "k_move_tiled32", "k_move_gather", "k_move_generic", "k_relayout", "k_convert4", "k_copy1",
       "k_copy16", "k_pad_rows", "k_pad_rows16", "k_widen_bf16"};
   const uint32_t n = sizeof families / sizeof families[0];

@@ -428,8 +428,11 @@ hipError_t launch_parts(const PartsArgs &p, hipStream_t stream) {
   // Contiguous lines in whole, aligned 16-byte vectors: the register-resident form.
   bool rows = n % 4 == 0 && n > 1 && n <= 4096 && p.kind != MRL_SPEC_DIVIDE_VEC &&
               p.kind != MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX_FROM_PARTS && full_size(p, 0);
-  // Lines side by side: the innermost dim is another one, and contiguous in the full-size parameters.
-  const uint32_t last = p.rank - 1;
+  // Lines side by side: the dim along which consecutive lines differ (the last one that is not
+  // the scan dim) is contiguous in the full-size parameters, as the innermost dim of a row-major
+  // tensor scanned along another dim is, or dim 0 of a column-major matrix scanned along dim 1.
+  uint32_t last = p.rank - 1;
+  if (last == p.scan_dim && last > 0) last--;
   bool cols = p.rank >= 2 && p.scan_dim != last && p.shape[last] >= 16;
   for (uint32_t t = 0; t < p.n_params; t++) {
     if (!full_size(p, t)) continue;
@@ -484,6 +487,19 @@ hipError_t launch_broadcast(const void *in, void *out, const LayoutEval &il, con
 
 // FillValue (spec.rs:165-170): 0 Zero, 1 NegInf (floats), 2 Min (the dtype's minimum;
 // f32::MIN / bf16::MIN for floats, as verification.rs:534-545 fills).
+// Fill in 16-byte stores of the replicated pattern; the elements past the last whole 16 bytes are
+// written one each by the first threads.
+__global__ __launch_bounds__(256) void k_fill16(u4 *out, uint32_t word, uint64_t units, uint8_t *tail, uint32_t tail_elems,
+                                                uint32_t es) {
+  const uint64_t t = uint64_t(blockIdx.x) * 256 + threadIdx.x;
+  if (t < units) __builtin_nontemporal_store(u4{word, word, word, word}, out + t);
+  if (t < tail_elems) {
+    if (es == 1) tail[t] = uint8_t(word);
+    else if (es == 2) ((uint16_t *)tail)[t] = uint16_t(word);
+    else ((uint32_t *)tail)[t] = word;
+  }
+}
+
 bool launch_broadcast_rows(const void *in, void *out, uint64_t before, uint32_t n, uint64_t after, uint32_t es,
                            hipStream_t stream, hipError_t *err) {
   if (before == 0 || n == 0 || after == 0) return false;
@@ -534,6 +550,13 @@ hipError_t launch_fill(void *out, int dtype, int fill_value, uint64_t count, hip
   }
   const uint32_t es = dtype == MRL_U8 || dtype == MRL_I8 ? 1 : (dtype == MRL_U16 || dtype == MRL_I16 || dtype == MRL_BF16 ? 2 : 4);
   plan::work(plan::UNIT_STREAM, 0, double(count) * es);
+  const uint64_t units = count * es / 16;
+  if ((reinterpret_cast<uintptr_t>(out) & 15) == 0 && units > 0 && (units + 255) / 256 <= 0x7fffffffull) {
+    const uint32_t word = es == 1 ? pattern * 0x01010101u : es == 2 ? pattern * 0x00010001u : pattern;
+    MRL_LAUNCH(k_fill16, dim3(uint32_t((units + 255) / 256)), dim3(256), 0, stream, (u4 *)out, word, units,
+               (uint8_t *)out + units * 16, uint32_t((count * es - units * 16) / es), es);
+    return mrl::plan::last_error();
+  }
   MRL_LAUNCH(k_fill, dim3(uint32_t((count + 255) / 256)), dim3(256), 0, stream, (uint8_t *)out,
                      pattern, es, count);
   return mrl::plan::last_error();

@@ -256,6 +256,51 @@ def test_parts_through_non_row_major_layouts(gpu):
     np.testing.assert_allclose(got[2].reshape(shape), want[2], **TOL)
 
 
+@pytest.mark.parametrize("shape,dim", [((70, 48), 1), ((48, 70), 0), ((64, 1024), 0), ((130, 20), 1)])
+def test_parts_of_column_major_tensors(gpu, shape, dim):
+    """Column-major parameters are strided tensors to these kernels: scanned along dim 0 their
+    lines are contiguous (the register-resident form where they are whole vectors), scanned
+    along dim 1 consecutive lines are neighbours in memory (the side-by-side form)."""
+    x = rnd(shape)
+    cm, cm_red = M.col_major(list(shape)), M.col_major(list(reduced(shape, dim)))
+    stored = lambda a: np.ascontiguousarray(a.T)
+    mx, dn = np.zeros(reduced(shape, dim), np.float32), np.zeros(reduced(shape, dim), np.float32)
+    got = run_all(M.SoftmaxDenominatorAndMax(shape, dim, layouts=[cm, cm_red, cm_red]), [stored(x), stored(mx), stored(dn)])
+    want = orc.softmax_part(orc.PART_DENOM_MAX, shape, dim, [x, mx.copy(), dn.copy()])
+    assert np.array_equal(got[1], stored(want[1]))
+    np.testing.assert_allclose(got[2], stored(want[2]), **tol(shape, dim))
+    out = np.zeros(shape, np.float32)
+    got = run_all(M.SoftmaxComplete(shape, dim, layouts=[cm, cm_red, cm_red, cm]), [stored(x), stored(want[1]), stored(want[2]), stored(out)])
+    want_y = orc.softmax_part(orc.PART_COMPLETE, shape, dim, [x, want[1], want[2], out])[3]
+    np.testing.assert_allclose(got[3], stored(want_y), **tol(shape, dim))
+
+
+def test_one_prefix_of_a_large_tensor_is_a_copy(gpu):
+    shape = (1024, 1000)
+    x = rnd(shape)
+    spec = M.OnePrefix(shape)
+    assert spec.plan().kernels == ["k_copy16"]
+    assert np.array_equal(run_all(spec, [x, np.zeros((1,) + shape, np.float32)])[1][0], x)
+    spec = M.OnePrefix(shape, layouts=[None, M.layout(0, 2, 1)])
+    assert "k_move_generic" not in spec.plan().kernels
+    assert np.array_equal(run_all(spec, [x, np.zeros((1, 1000, 1024), np.float32)])[1][0], x.T)
+
+
+@pytest.mark.parametrize("dtype,np_dtype", [(M.u8, np.uint8), (M.bf16, np.uint16), (M.f32, np.float32)])
+@pytest.mark.parametrize("count", [1, 15, 16, 185, 4099])
+def test_fill_stays_inside_its_tensor(gpu, dtype, np_dtype, count):
+    """The 16-byte stores cover the whole units of the tensor and single elements the rest;
+    nothing behind the tensor changes."""
+    whole = np.full(count + 64, 0x55, np_dtype)
+    buf = M.DeviceBuffer.from_numpy(whole)
+    M.Fill([count], dtype, M.FillValue.Min).run_device([buf.ptr])
+    back = buf.to_numpy(np_dtype, whole.shape)
+    buf.free()
+    want = orc.fill({M.u8: orc.U8, M.bf16: orc.BF16, M.f32: orc.F32}[dtype], int(M.FillValue.Min), count)
+    assert np.array_equal(back[:count].view(np.uint8), want.view(np.uint8))
+    assert np.all(back[count:] == 0x55)
+
+
 @pytest.mark.parametrize("dtype,np_dtype,code", [(M.u8, np.uint8, orc.U8), (M.i8, np.int8, orc.I8),
                                                   (M.i16, np.int16, orc.I16), (M.u32, np.uint32, orc.U32),
                                                   (M.i32, np.int32, orc.I32), (M.f32, np.float32, orc.F32),

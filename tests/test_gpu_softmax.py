@@ -152,6 +152,29 @@ def _softmax_outer(shape, dim):
     assert (np.abs(got - want) <= (1e-5 + oracle_off) * np.abs(want) + 1e-12).all()
 
 
+@pytest.mark.parametrize("shape,perm,dim", [((300, 200), (1, 0), 0), ((300, 200), (1, 0), 1), ((70, 4096), (1, 0), 1),
+                                            ((8, 300, 64), (2, 1, 0), 0), ((8, 300, 64), (2, 1, 0), 1), ((8, 300, 64), (2, 1, 0), 2),
+                                            ((6, 40, 500), (1, 0, 2), 2), ((6, 40, 500), (0, 2, 1), 2), ((5, 1, 260), (2, 1, 0), 0)])
+def test_softmax_of_tensors_stored_in_another_order(gpu, shape, perm, dim):
+    """Both tensors in the same permuted order (column-major, say): the dispatch goes by the order
+    the dims are stored in, so a column-major matrix scanned along dim 0 takes the row kernels
+    and one scanned along dim 1 the column kernels.  With only one of the two permuted the
+    strided kernel runs."""
+    lay = M.layout(*perm)
+    x = (synth.normal_f32(31, 0, shape) * 3).astype(np.float32)
+    want = orc.softmax(list(shape), dim, x)
+    stored = lambda a: np.ascontiguousarray(a.transpose(perm))
+    spec = M.Softmax(list(shape), dim, layouts=[lay, lay])
+    # stored order [.., scan, after]: the column kernels want 16 contiguous elements behind the scan dim
+    behind = int(np.prod([shape[d] for d in perm[perm.index(dim) + 1:]]))
+    if behind == 1 or behind >= 16:
+        assert spec.plan().kernels[0] in ("k_softmax_regs", "k_softmax_short", "k_softmax_block", "k_softmax_cols"), spec.plan()
+    got = run_spec(spec, [stored(x), np.zeros(stored(x).shape, np.float32)])
+    np.testing.assert_allclose(got, stored(want), rtol=2e-5, atol=1e-8)
+    got = run_spec(M.Softmax(list(shape), dim, layouts=[lay, None]), [stored(x), np.zeros(shape, np.float32)])
+    np.testing.assert_allclose(got, want, rtol=2e-5, atol=1e-8)
+
+
 def test_softmax_full_size(gpu):
     """The Softmax stage of benchmark configuration 5 alone: 16x2048 rows of 2048."""
     shape = (16, 2048, 2048)
