@@ -519,17 +519,28 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
     return finish_output(c, ws);
   }
   if (kind >= 0 && rows && mrl::gemm_possible(g, kind) && mrl::gemm_pays(g, kind)) {
-    const uint32_t splits = mrl::gemm_k_splits(g, kind);
+    uint32_t left = 0;
+    const uint32_t splits = mrl::gemm_k_splits(g, kind, &left);
     if (splits > 1) {
-      // Slices of K as batch entries writing dense partial results, summed into C in slice order.
+      // Slices of K as batch entries writing dense partial results, summed into C in slice order;
+      // what K has behind the equal slices is one more, shorter slice in a launch of its own.
       void *partial = nullptr;
-      HIP_TRY(ws.alloc(&partial, size_t(splits) * g.m * g.n * 4));
+      HIP_TRY(ws.alloc(&partial, size_t(splits + (left ? 1 : 0)) * g.m * g.n * 4));
       mrl::GemmArgs slices = g;
-      slices.batch = splits, slices.k = g.k / splits;
+      slices.batch = splits, slices.k = (g.k - left) / splits;
       slices.sa = slices.k, slices.sb = g.b_kmajor ? int64_t(slices.k) : int64_t(slices.k) * g.ldb;
       slices.c = partial, slices.ldc = g.n, slices.sc = int64_t(g.m) * g.n, slices.accum = 0;
       HIP_TRY(mrl::launch_gemm(slices, kind, ws.stream));
-      HIP_TRY(mrl::launch_sum_splits(partial, g.c, splits, g.m, g.n, g.ldc, g.accum != 0, kind <= 1, ws.stream));
+      if (left) {
+        mrl::GemmArgs rest = slices;
+        const size_t elem = kind <= 1 ? 1 : kind == 2 ? 2 : 4;
+        rest.batch = 1, rest.k = left;
+        rest.a = (const char *)g.a + size_t(g.k - left) * elem;
+        rest.b = (const char *)g.b + (g.b_kmajor ? size_t(g.k - left) : size_t(g.k - left) * g.ldb) * elem;
+        rest.c = (char *)partial + size_t(splits) * g.m * g.n * 4;
+        HIP_TRY(mrl::launch_gemm(rest, kind, ws.stream));
+      }
+      HIP_TRY(mrl::launch_sum_splits(partial, g.c, splits + (left ? 1 : 0), g.m, g.n, g.ldc, g.accum != 0, kind <= 1, ws.stream));
     } else {
       HIP_TRY(mrl::launch_gemm(g, kind, ws.stream));
     }

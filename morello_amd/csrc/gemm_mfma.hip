@@ -69,14 +69,25 @@ uint32_t gemm_tile_side(const GemmArgs &g, int kind) { return tile_side(g, elem_
 // Fewer than three quarters of the compute units would get a 64 x 64 tile and every tile walks at
 // least sixteen k steps: share K out so that up to 512 workgroups run, eight steps each at least
 // (int8 512 x 8192 x 512: 64 tiles of 64 steps, 36 us; as 8 x 64 tiles of 8 steps plus the sum, 10 us).
-uint32_t gemm_k_splits(const GemmArgs &g, int kind) {
+uint32_t gemm_k_splits(const GemmArgs &g, int kind, uint32_t *remainder) {
+  // remainder: where the caller can run one more, shorter slice behind the equal ones (a K that
+  // is not a whole number of 128-byte steps, or whose steps have no divisor near the wanted
+  // count: 300 x 30000 x 300 int8 is 234 steps and 48 bytes); without it only equal slices.
+  if (remainder) *remainder = 0;
   const uint64_t es = elem_size_of(kind);
-  if (g.batch != 1 || gemv_applicable(g, kind) || (uint64_t(g.k) * es) % 128 != 0) return 1;
-  const uint64_t steps = uint64_t(g.k) * es / 128;
+  const uint64_t k_bytes = uint64_t(g.k) * es;
+  if (g.batch != 1 || gemv_applicable(g, kind) || (k_bytes % 128 != 0 && !remainder)) return 1;
+  const uint64_t steps = k_bytes / 128;
   const uint64_t tiles = uint64_t((g.m + 63) / 64) * ((g.n + 63) / 64);
   if (tiles >= 384 || steps < 16) return 1;
-  uint64_t want = std::min<uint64_t>({32, 768 / tiles, steps / 8});
-  while (want > 1 && steps % want != 0) want--;
+  const uint64_t wanted = std::min<uint64_t>({32, 768 / tiles, steps / 8});
+  uint64_t want = wanted;
+  while (want > 1 && (steps % want != 0 || k_bytes % 128 != 0)) want--;
+  uint64_t left = 0;   // elements of K behind the equal slices
+  if (remainder && wanted > 1 && want * 2 <= wanted) {
+    want = wanted;
+    left = g.k - want * (steps / want) * (128 / es);
+  }
   if (want <= 1) return 1;
   // What the slices save: a workgroup's chain of k steps (~0.48 us each on the 64 x 64 tile)
   // shortens by the factor by which they add workgroups the chip has room for (about 384
@@ -84,8 +95,9 @@ uint32_t gemm_k_splits(const GemmArgs &g, int kind) {
   // of 16 steps) ran 15 us in two slices against 8.8 us whole.
   const double spread = std::min<double>(double(want), 384.0 / double(tiles));
   const double saved_us = double(steps) * (1.0 - 1.0 / spread) * 0.48;
-  const double cost_us = 2.5 + (double(want) + 1.0) * double(g.m) * double(g.n) * 4.0 / 5.5e6;
+  const double cost_us = 2.5 + (left ? 3.0 : 0.0) + (double(want) + (left ? 2.0 : 1.0)) * double(g.m) * double(g.n) * 4.0 / 5.5e6;
   if (spread <= 1.0 || saved_us < 1.2 * cost_us) return 1;
+  if (remainder) *remainder = uint32_t(left);
   return uint32_t(want);
 }
 

@@ -113,7 +113,7 @@ hipError_t launch_gemm(const GemmArgs &g, int kind, hipStream_t stream);
 uint32_t gemm_tile_side(const GemmArgs &g, int kind);
 // A single Matmul with few output tiles and a long K runs as `splits` batch entries over slices
 // of K whose partial results are summed afterwards (1: as it is).  The slices are whole k steps.
-uint32_t gemm_k_splits(const GemmArgs &g, int kind);
+uint32_t gemm_k_splits(const GemmArgs &g, int kind, uint32_t *remainder = nullptr);
 // c[r][col] (+)= sum over s of partial[s][r][col]; partial is dense [splits][m][n], 32-bit
 // elements (int32 when `integers`, else f32), summed in order of s.
 hipError_t launch_sum_splits(const void *partial, void *c, uint32_t splits, uint32_t m, uint32_t n, int64_t ldc,

@@ -255,12 +255,15 @@ def test_matrix_vector_shapes(gpu, dts, codes, shape, accum, b_k_fastest):
                                        ((M.bf16, M.bf16, M.f32), [7, 7, 6]), ((M.f32, M.f32, M.f32), [6, 6, 6])])
 @pytest.mark.parametrize("shape,accum", [((1, 512, 8192, 512), False), ((1, 256, 16384, 192), True),
                                          ((1, 100, 4096, 300), True), ((1, 32, 4096, 1000), False),
-                                         ((1, 130, 2048, 70), False)])
+                                         ((1, 130, 2048, 70), False),
+                                         # K is no whole number of equal slices: a shorter one behind them
+                                         ((1, 300, 30000, 300), True), ((1, 64, 16256, 128), False), ((1, 96, 5008, 40), False)])
 @pytest.mark.parametrize("b_k_fastest", [True, False])
 def test_matmul_with_k_shared_out_over_workgroups(gpu, dts, codes, shape, accum, b_k_fastest):
     """Few output tiles and a long K: slices of K run as batch entries and their partial results
     are summed in slice order (exact for integers, the f32 sum in another association for floats).
-    Whole and ragged M and N, accumulation into C, both B orientations, every dtype kind."""
+    Whole and ragged M and N, accumulation into C, both B orientations, every dtype kind; a K of
+    127 steps (no divisor), of 234 steps and 48 bytes, of 39 steps and 16 bytes."""
     b, m, k, n = shape
     if dts[0] == M.f32:
         k //= 2  # the same number of 128-byte k steps at twice the element size would take twice as long on the oracle
