@@ -269,7 +269,17 @@ constexpr uint32_t MAX_KS = 6;   // windows of up to 384 bytes: 75 KiB of rows, 
 bool conv_windows_applicable(const ConvArgs &c, int kind) {
   if (kind < 0 || kind > 2) return false;
   const uint64_t es = kind == 2 ? 2 : 1, c_bytes = c.c * es, seg_padded = (uint64_t(c.fw) * c_bytes + 3) & ~3ull;
-  return c.f % 16 == 0 && c.f / 64 < 65535 && c_bytes % 16 != 0 && uint64_t(c.fh) * seg_padded <= 64 * MAX_KS &&
+  // Pixels that are not whole 16-byte chunks (the implicit Matmul cannot read those in place), and
+  // pixels of one chunk with windows of up to 192 bytes, where this kernel measured faster than
+  // the implicit Matmul's chunk-by-chunk addressing (32 x (16 -> 16) x 112^2 3 x 3 int8 27.5
+  // against 39 us, bf16 8 -> 32 28 against 34); with longer windows or wider pixels it is the slower
+  // one (int8 32 -> 32 3 x 3: 60 against 44 us; 48 -> 48 2 x 2 at 56^2: 17 against 13).
+#ifdef MRL_WINDOWS_ANY_C   // measurement builds: every pixel width
+  const bool c_ok = true;
+#else
+  const bool c_ok = c_bytes % 16 != 0 || (c_bytes == 16 && uint64_t(c.fh) * seg_padded <= 192);
+#endif
+  return c.f % 16 == 0 && c.f / 64 < 65535 && c_ok && uint64_t(c.fh) * seg_padded <= 64 * MAX_KS &&
          uint64_t(c.b) * ((c.oh + TILE_H - 1) / TILE_H) * ((c.ow + TILE_W - 1) / TILE_W) < (1ull << 31) &&
          (reinterpret_cast<uintptr_t>(c.out) & 15) == 0 && (reinterpret_cast<uintptr_t>(c.image) & (es - 1)) == 0 &&
          (reinterpret_cast<uintptr_t>(c.filters) & (es - 1)) == 0;

@@ -142,6 +142,8 @@ def test_deep_conv_on_small_images_shares_its_windows_out(gpu, dts, codes, shape
     ((64, 32, 2, 1, 3, 2, 9), True),      # three output pixels per image
     ((1, 64, 5, 30, 30, 1, 1), False),    # 1 x 1 filters
     ((2, 32, 3, 11, 40, 9, 3), False),    # tall filters
+    ((3, 32, 16, 20, 33, 3, 3), True),    # pixels of one whole chunk, windows of 144 bytes: taken from the implicit Matmul
+    ((2, 16, 16, 9, 40, 2, 5), False),    # two runs of 80 bytes
 ])
 @pytest.mark.parametrize("img_dt,img_code,gen", [(M.u8, 0, synth.uniform_u8), (M.i8, 1, synth.uniform_i8)])
 def test_conv_with_few_channels_forms_its_windows_in_lds(gpu, shape, accum, img_dt, img_code, gen):
@@ -174,6 +176,7 @@ def test_conv_with_few_channels_forms_its_windows_in_lds(gpu, shape, accum, img_
     ((2, 80, 3, 17, 15, 5, 5), True),     # two groups of filters
     ((1, 64, 5, 30, 30, 1, 1), False),    # 1 x 1 filters, runs of 10 bytes
     ((2, 32, 12, 9, 21, 3, 3), False),    # 24 bytes a pixel
+    ((2, 32, 8, 9, 21, 3, 3), True),      # one whole chunk a pixel, windows of 144 bytes
 ])
 def test_bf16_conv_with_few_channels_forms_its_windows_in_lds(gpu, shape, accum):
     """The same kernel on bf16 operands (f32 sums, as a bf16 Matmul's).  An image that holds a NaN

@@ -338,6 +338,15 @@ def test_cost_model_ranks_manual_schedules(gpu):
                         assert measured[x] <= 1.25 * measured[y], (dts[0], m, k, n, x, y, measured, predicted)
 
 
+def test_one_chunk_pixels_with_short_windows_take_the_windows_kernel():
+    """Host only: pixels of exactly 16 bytes with windows of up to 192 bytes go to the kernel that
+    forms windows in LDS; wider pixels and longer windows stay with the implicit Matmul."""
+    kernels = lambda c, fs, dts: M.Conv([32, 32, c, 112, 112, fs, fs], dts).plan().kernels
+    i8, bf = (M.u8, M.i8, M.i32), (M.bf16, M.bf16, M.f32)
+    assert kernels(16, 3, i8) == ["k_conv_windows"] and kernels(8, 3, bf) == ["k_conv_windows"]
+    assert kernels(32, 3, i8) == ["k_gemm"] and kernels(16, 3, bf) == ["k_gemm"] and kernels(16, 5, i8) == ["k_gemm"]
+
+
 def test_plans_of_the_softmax_primitives():
     """Host only: which kernel a primitive of the decomposition takes.  Contiguous lines of up to
     4096 elements in whole 16-byte vectors stay in a wavefront's registers; a scan dim that is
