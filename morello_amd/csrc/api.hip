@@ -650,7 +650,7 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
   const bool unfold_ok = as_matmul && can_unfold && (reinterpret_cast<uintptr_t>(img.t.ptr) & 15) == 0 &&
                          (reinterpret_cast<uintptr_t>(filt.t.ptr) & 15) == 0 && (reinterpret_cast<uintptr_t>(out.t.ptr) & 3) == 0;
   // Few channels per pixel (a first layer): the fused kernel that forms the windows in LDS.
-  const bool windows_ok = kind >= 0 && kind <= 2 && as_matmul && channels_last(img.t) && channels_last(filt.t) && channels_last(out.t) &&
+  const bool windows_ok = kind >= 0 && kind <= 3 && as_matmul && channels_last(img.t) && channels_last(filt.t) && channels_last(out.t) &&
                           mrl::conv_windows_applicable(cv, kind) && !(forced == 1 && g_forced->conv_rows);
   if ((forced == 1 && !fused_ok && !windows_ok) || (forced == 2 && !implicit_ok) || (forced == 3 && !unfold_ok)) return MRL_ERR_UNSUPPORTED;
   if (fused_ok && forced <= 1) {

@@ -1,4 +1,4 @@
-// Conv NHWC u8|i8 x KRSC i8 -> i32 and bf16 x bf16 -> f32 for pixels of few channels (a first layer: 3 channels, 7 x 7
+// Conv NHWC u8|i8 x KRSC i8 -> i32, bf16 x bf16 -> f32 and f32 x f32 -> f32 for pixels of few channels (a first layer: 3 channels, 7 x 7
 // filters), where a pixel's channels are not whole 16-byte chunks and the implicit Matmul of
 // conv_gemm.hip does not apply (morello/src/spec.rs:486-494: no stride, no padding).  The other
 // route for such shapes writes every window to memory first (unfold.hip) and multiplies the rows:
@@ -15,8 +15,10 @@
 //      the padding, so that whatever the windows hold there counts for nothing):
 //      v_mfma_i32_16x16x64_i8 / v_mfma_f32_16x16x32_bf16 (the same 64 bytes of window a step, the
 //      same 16 bytes a lane group), a lane ends up with 4 consecutive filters of one pixel, 16
-//      contiguous bytes of the channels-last output.  bf16: the padding of the windows is zeros
-//      as well (a NaN there times a zero weight would not be zero).
+//      contiguous bytes of the channels-last output.  f32: four v_mfma_f32_16x16x4_f32 per
+//      64 bytes, the j-th on the j-th of the 16 bytes' four values (a lane group's 16 bytes are
+//      four k indices; which ones is free as long as both operands agree).  Floats: the padding
+//      of the windows is zeros as well (a NaN there times a zero weight would not be zero).
 // The u8 correction 128 * sum of a filter's weights comes from the same MFMAs against an operand
 // of ones, once per workgroup.  Rows of windows and filters lie 16 bytes more than their length
 // apart, which spreads the 16 lanes of an operand read over all banks.
@@ -29,7 +31,7 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
-enum { IMG_I8 = 0, IMG_U8 = 1, IMG_BF16 = 2 };
+enum { IMG_I8 = 0, IMG_U8 = 1, IMG_BF16 = 2, IMG_F32 = 3 };
 
 constexpr int TILE_H = 8, TILE_W = 16, TILE_PIXELS = TILE_H * TILE_W;
 constexpr int PATCH_REGS = 8;   // patch bytes a thread holds in flight: patches of up to 2 KiB
@@ -47,11 +49,19 @@ struct WindowsArgs {
 // KS: MFMA k steps per window (fh * seg_padded bytes, padded to 64 KS).
 template <int KS, int KIND>
 __global__ __launch_bounds__(256) void k_conv_windows(WindowsArgs p) {
-  constexpr bool IMG_UNSIGNED = KIND == IMG_U8, FLOATS = KIND == IMG_BF16;
+  constexpr bool IMG_UNSIGNED = KIND == IMG_U8, FLOATS = KIND == IMG_BF16 || KIND == IMG_F32, HALVES = KIND == IMG_BF16;
   typedef typename std::conditional<FLOATS, v4f, v4i>::type Acc;
   auto mfma = [](v4i a, v4i b, Acc c) {
-    if constexpr (FLOATS) return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
-    else return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+    if constexpr (KIND == IMG_F32) {
+      const v4f fa = __builtin_bit_cast(v4f, a), fb = __builtin_bit_cast(v4f, b);
+#pragma unroll
+      for (int j = 0; j < 4; j++) c = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[j], fb[j], c, 0, 0, 0);
+      return c;
+    } else if constexpr (KIND == IMG_BF16) {
+      return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+    } else {
+      return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+    }
   };
   extern __shared__ __attribute__((aligned(16))) uint8_t win_lds[];
   // Rows of windows and filters: 16 bytes more than their length apart (144 at least: two pixel
@@ -184,12 +194,12 @@ __global__ __launch_bounds__(256) void k_conv_windows(WindowsArgs p) {
           for (int d = 0; d < 8; d++)
             if (d0 + d < dwords) {
               uint32_t out = __builtin_amdgcn_alignbyte(v[d + 1], v[d], shift);
-              if (FLOATS && p.seg - 4 * (d0 + d) < 4) out &= 0xffffu;   // the run ends with half a dword: its padding is zero
+              if (HALVES && p.seg - 4 * (d0 + d) < 4) out &= 0xffffu;   // the run ends with half a dword: its padding is zero
               dst[r * dwords + d0 + d] = out;
             }
         }
       }
-      // bf16: zeros behind the last run too (the results that left through these rows lie there)
+      // floats: zeros behind the last run too (the results that left through these rows lie there)
       if (FLOATS)
         for (uint32_t d = p.fh * dwords + (tid >> 7); d < KPAD / 4; d += 2) dst[d] = 0;
     }
@@ -255,20 +265,22 @@ hipError_t launch_ks(const WindowsArgs &p, int kind, dim3 grid, size_t lds, hipS
     case IMG_I8: return launch_kind<KS, IMG_I8>(p, grid, lds, stream);
     case IMG_U8: return launch_kind<KS, IMG_U8>(p, grid, lds, stream);
     case IMG_BF16: return launch_kind<KS, IMG_BF16>(p, grid, lds, stream);
+    case IMG_F32: return launch_kind<KS, IMG_F32>(p, grid, lds, stream);
     default: return hipErrorInvalidValue;
   }
 }
 
-constexpr uint32_t MAX_KS = 6;   // windows of up to 384 bytes: 75 KiB of rows, two workgroups to a compute unit
+constexpr uint32_t MAX_KS = 6;       // windows of up to 384 bytes: 75 KiB of rows, two workgroups to a compute unit
+constexpr uint32_t MAX_KS_F32 = 10;  // f32: up to 640 bytes (3 channels, 7 x 7: 588), 126 KiB of rows, one workgroup
 
 }  // namespace
 
-// kind: 0 i8 x i8 -> i32, 1 u8 x i8 -> i32, 2 bf16 x bf16 -> f32.  Filters in 16s, pixels that are
+// kind: 0 i8 x i8 -> i32, 1 u8 x i8 -> i32, 2 bf16 x bf16 -> f32, 3 f32 x f32 -> f32.  Filters in 16s, pixels that are
 // not whole 16-byte chunks (those conv_gemm.hip reads in place), windows of at most 64 MAX_KS
 // bytes with their runs padded to dwords.
 bool conv_windows_applicable(const ConvArgs &c, int kind) {
-  if (kind < 0 || kind > 2) return false;
-  const uint64_t es = kind == 2 ? 2 : 1, c_bytes = c.c * es, seg_padded = (uint64_t(c.fw) * c_bytes + 3) & ~3ull;
+  if (kind < 0 || kind > 3) return false;
+  const uint64_t es = kind == 3 ? 4 : kind == 2 ? 2 : 1, c_bytes = c.c * es, seg_padded = (uint64_t(c.fw) * c_bytes + 3) & ~3ull;
   // Pixels that are not whole 16-byte chunks (the implicit Matmul cannot read those in place), and
   // pixels of one chunk with windows of up to 192 bytes, where this kernel measured faster than
   // the implicit Matmul's chunk-by-chunk addressing (32 x (16 -> 16) x 112^2 3 x 3 int8 27.5
@@ -279,7 +291,7 @@ bool conv_windows_applicable(const ConvArgs &c, int kind) {
 #else
   const bool c_ok = c_bytes % 16 != 0 || (c_bytes == 16 && uint64_t(c.fh) * seg_padded <= 192);
 #endif
-  return c.f % 16 == 0 && c.f / 64 < 65535 && c_ok && uint64_t(c.fh) * seg_padded <= 64 * MAX_KS &&
+  return c.f % 16 == 0 && c.f / 64 < 65535 && c_ok && uint64_t(c.fh) * seg_padded <= 64 * (kind == 3 ? MAX_KS_F32 : MAX_KS) &&
          uint64_t(c.b) * ((c.oh + TILE_H - 1) / TILE_H) * ((c.ow + TILE_W - 1) / TILE_W) < (1ull << 31) &&
          (reinterpret_cast<uintptr_t>(c.out) & 15) == 0 && (reinterpret_cast<uintptr_t>(c.image) & (es - 1)) == 0 &&
          (reinterpret_cast<uintptr_t>(c.filters) & (es - 1)) == 0;
@@ -287,7 +299,7 @@ bool conv_windows_applicable(const ConvArgs &c, int kind) {
 
 hipError_t launch_conv_windows(const ConvArgs &c, int kind, hipStream_t stream) {
   if (!conv_windows_applicable(c, kind)) return hipErrorInvalidValue;
-  const uint32_t es = kind == 2 ? 2 : 1;
+  const uint32_t es = kind == 3 ? 4 : kind == 2 ? 2 : 1;
   WindowsArgs p;
   p.image = (const uint8_t *)c.image, p.filters = (const uint8_t *)c.filters, p.out = (int32_t *)c.out;
   p.b = c.b, p.f = c.f, p.c = c.c * es, p.oh = c.oh, p.ow = c.ow, p.fh = c.fh, p.fw = c.fw, p.accum = c.accum;
@@ -314,6 +326,10 @@ hipError_t launch_conv_windows(const ConvArgs &c, int kind, hipStream_t stream) 
     case 4: return launch_ks<4>(p, kind, grid, lds, stream);
     case 5: return launch_ks<5>(p, kind, grid, lds, stream);
     case 6: return launch_ks<6>(p, kind, grid, lds, stream);
+    case 7: return launch_kind<7, IMG_F32>(p, grid, lds, stream);
+    case 8: return launch_kind<8, IMG_F32>(p, grid, lds, stream);
+    case 9: return launch_kind<9, IMG_F32>(p, grid, lds, stream);
+    case 10: return launch_kind<10, IMG_F32>(p, grid, lds, stream);
     default: return hipErrorInvalidValue;
   }
 }

@@ -147,7 +147,7 @@ def test_deep_conv_on_small_images_shares_its_windows_out(gpu, dts, codes, shape
 ])
 @pytest.mark.parametrize("img_dt,img_code,gen", [(M.u8, 0, synth.uniform_u8), (M.i8, 1, synth.uniform_i8)])
 def test_conv_with_few_channels_forms_its_windows_in_lds(gpu, shape, accum, img_dt, img_code, gen):
-    """Pixels that are not whole 16-byte chunks, windows of at most 256 bytes (runs padded to
+    """Pixels that are not whole 16-byte chunks, windows of at most 384 bytes (runs padded to
     dwords), filters in 16s: one kernel forms the windows in LDS and multiplies them.  Against
     the oracle, bit for bit, with old values in the output when accumulating and a sentinel
     otherwise; once more with the image and the filters at addresses that are not 16-byte aligned."""
@@ -168,6 +168,49 @@ def test_conv_with_few_channels_forms_its_windows_in_lds(gpu, shape, accum, img_
     for x in bufs:
         x.free()
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("shape,accum", [
+    ((2, 64, 3, 20, 37, 5, 5), False),    # runs of 60 bytes, five k steps
+    ((4, 16, 1, 30, 30, 3, 3), True),     # runs of 12 bytes
+    ((2, 80, 3, 17, 15, 3, 3), True),     # two groups of filters
+    ((1, 64, 5, 30, 30, 1, 1), False),    # 1 x 1 filters, runs of 20 bytes
+    ((2, 32, 6, 9, 21, 3, 3), False),     # 24 bytes a pixel
+    ((3, 48, 2, 33, 5, 9, 2), True),      # tall filters, ragged tiles
+])
+def test_f32_conv_with_few_channels_forms_its_windows_in_lds(gpu, shape, accum):
+    """The same kernel on f32 operands: four MFMAs of k = 4 per 64 bytes of window, windows of up
+    to 640 bytes.  To 1e-5 of the oracle (f32 sums in another order), and NaN and infinity reach
+    exactly the outputs whose windows hold them."""
+    b, f, c, oh, ow, fh, fw = shape
+    spec = M.Conv(list(shape), (M.f32, M.f32, M.f32), accum=accum)
+    assert spec.plan().kernels == ["k_conv_windows"] and "KIND = 3" in spec.plan().steps[0].kernel
+    img = synth.normal_f32(136, 0, (b, oh + fh - 1, ow + fw - 1, c))
+    filt = synth.normal_f32(136, 1, (f, fh, fw, c))
+    out0 = synth.uniform_u8(136, 2, (b, oh, ow, f)).astype(np.float32) if accum else np.full((b, oh, ow, f), 7, np.float32)
+    want = orc.conv(list(shape), [6, 6, 6], img, filt, out0.copy(), accum, layouts=[NHWC] * 3)
+    got = run_spec(spec, [img, filt, out0.copy()])
+    assert float(np.abs(got.astype(np.float64) - want).max() / np.abs(want).max()) < 1e-5
+    img = img.copy()
+    img[0, 0, 0, 0] = np.nan
+    img[b - 1, oh + fh - 2, ow + fw - 2, c - 1] = np.inf
+    want = orc.conv(list(shape), [6, 6, 6], img, filt, out0.copy(), accum, layouts=[NHWC] * 3)
+    got = run_spec(spec, [img, filt, out0.copy()])
+    assert np.array_equal(np.isfinite(got), np.isfinite(want))
+    ok = np.isfinite(want)
+    assert float(np.abs(got[ok].astype(np.float64) - want[ok]).max() / np.abs(want[ok]).max()) < 1e-5
+
+
+def test_f32_first_layer_conv_at_its_longest_window(gpu):
+    """3 channels, 7 x 7 filters: runs of 84 bytes, 588 bytes a window, ten k steps of 64."""
+    shape = (2, 64, 3, 20, 37, 7, 7)
+    spec = M.Conv(list(shape), (M.f32, M.f32, M.f32))
+    assert spec.plan().kernels == ["k_conv_windows"] and "KS = 10" in spec.plan().steps[0].kernel
+    img, filt = synth.normal_f32(137, 0, (2, 26, 43, 3)), synth.normal_f32(137, 1, (64, 7, 7, 3))
+    out0 = np.full((2, 20, 37, 64), 7, np.float32)
+    want = orc.conv(list(shape), [6, 6, 6], img, filt, out0.copy(), False, layouts=[NHWC] * 3)
+    got = run_spec(spec, [img, filt, out0])
+    assert float(np.abs(got.astype(np.float64) - want).max() / np.abs(want).max()) < 1e-5
 
 
 @pytest.mark.parametrize("shape,accum", [

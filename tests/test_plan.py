@@ -111,7 +111,8 @@ def test_plans_follow_shape_dtype_and_layout():
     # Conv shapes beside the benchmark's: implicit Matmul; three channels: unfolded first.
     assert M.Conv([32, 128, 128, 26, 26, 3, 3], (M.bf16, M.bf16, M.f32)).plan().kernels == ["k_gemm"]
     assert "CONV = true" in M.Conv([32, 128, 128, 26, 26, 3, 3], (M.bf16, M.bf16, M.f32)).plan().steps[0].kernel
-    assert "k_unfold" in M.Conv([8, 32, 3, 110, 110, 5, 5], (M.f32, M.f32, M.f32)).plan().kernels
+    assert M.Conv([8, 32, 3, 110, 110, 5, 5], (M.f32, M.f32, M.f32)).plan().kernels == ["k_conv_windows"]
+    assert "k_unfold" in M.Conv([8, 32, 3, 110, 110, 11, 11], (M.f32, M.f32, M.f32)).plan().kernels   # windows of 1452 bytes
     # ... in int8 and bf16 with windows of up to 384 bytes: formed in LDS by the kernel that multiplies them.
     assert "KIND = 2" in M.Conv([8, 32, 3, 110, 110, 5, 5], (M.bf16, M.bf16, M.f32)).plan().steps[0].kernel
     first = M.Conv([32, 64, 3, 112, 112, 7, 7], (M.u8, M.i8, M.i32)).plan()
