@@ -245,3 +245,91 @@ def test_random_compose_msm(gpu, seed):
         assert np.isfinite(got).all(), (what, target)
         assert rel_err(got, want) < 1e-2, (what, target)
         assert elem_err(got, want, floor_frac=1.0) < 2e-2, (what, target)
+
+
+PART_SPECS = [  # (constructor, oracle kind, which parameters span the scan dim, takes accum)
+    (M.Max, orc.PART_MAX, (True, False), True),
+    (M.SoftmaxDenominator, orc.PART_DENOM, (True, False, False), True),
+    (M.SoftmaxDenominatorAndMax, orc.PART_DENOM_MAX, (True, False, False), True),
+    (M.SoftmaxDenominatorAndMaxFromParts, orc.PART_FROM_PARTS, (True, True, False, False), True),
+    (M.SoftmaxDenominatorAndUnscaled, orc.PART_UNSCALED, (True, False, True), False),
+    (M.SoftmaxDenominatorAndUnscaledFromMax, orc.PART_UNSCALED_FROM_MAX, (True, False, False, True), True),
+    (M.SoftmaxComplete, orc.PART_COMPLETE, (True, False, False, True), False),
+    (M.DivideVecScalar, orc.PART_DIVIDE_VEC_SCALAR, (True, False), False),
+]
+
+
+@pytest.mark.parametrize("seed", range(96))
+def test_random_softmax_primitives(gpu, seed):
+    """The primitives of the Softmax decomposition over random shapes (one dim sometimes long, so
+    that every way of sharing out the lines is met: a wavefront per line, register-resident lines,
+    lines side by side), scan dims, accumulation and a random order of the dims per parameter;
+    every parameter as it stands afterwards against the oracle's."""
+    rng = np.random.default_rng(9300 + seed)
+    ctor, kind, full, takes_accum = PART_SPECS[seed % len(PART_SPECS)]
+    rank = int(rng.integers(1, 5))
+    shape = [int(rng.choice(SIZES[:24])) for _ in range(rank)]
+    if rng.random() < 0.6:
+        shape[int(rng.integers(rank))] = int(rng.choice([256, 1000, 1024, 2048, 4096, 4100, 20000]))
+    while int(np.prod(shape)) > (1 << 21):   # drop the smallest dim that is not 1 yet
+        shape[min((d for d in range(rank) if shape[d] > 1), key=lambda d: shape[d])] = 1
+    dim = int(rng.integers(rank))
+    accum = takes_accum and bool(rng.integers(2))
+    red = list(shape)
+    red[dim] = 1
+    x = (synth.normal_f32(9300 + seed, 0, shape) * 3).astype(np.float32)
+    mx = x.max(axis=dim, keepdims=True) + np.float32(rng.integers(0, 2))
+    positive = lambda i, s: np.abs(synth.normal_f32(9300 + seed, i, s)) + np.float32(0.5)
+    if kind == orc.PART_MAX:
+        params = [x, synth.normal_f32(9300 + seed, 1, red)]
+    elif kind in (orc.PART_DENOM, orc.PART_DENOM_MAX):
+        params = [x, mx if kind == orc.PART_DENOM else synth.normal_f32(9300 + seed, 1, red), positive(2, red)]
+    elif kind == orc.PART_FROM_PARTS:
+        params = [x, positive(1, shape), synth.normal_f32(9300 + seed, 2, red), positive(3, red)]
+    elif kind == orc.PART_UNSCALED:
+        params = [x, positive(1, red), np.zeros(shape, np.float32)]
+    elif kind == orc.PART_UNSCALED_FROM_MAX:
+        params = [x, mx, positive(2, red), np.zeros(shape, np.float32)]
+    elif kind == orc.PART_COMPLETE:
+        params = [x, mx, positive(2, red), np.zeros(shape, np.float32)]
+    else:
+        params = [x, positive(1, red)]
+    perms = [tuple(int(d) for d in rng.permutation(rank)) for _ in params]
+    stored = [np.ascontiguousarray(p.transpose(perm)) for p, perm in zip(params, perms)]
+    kwargs = dict(accum=accum) if takes_accum else {}
+    spec = ctor(shape, dim, layouts=[M.layout(*perm) for perm in perms], **kwargs)
+    bufs = [M.DeviceBuffer.from_numpy(a) for a in stored]
+    spec.run_device([b.ptr for b in bufs])
+    got = [b.to_numpy(np.float32, a.shape) for a, b in zip(stored, bufs)]
+    for b in bufs:
+        b.free()
+    want = orc.softmax_part(kind, shape, dim, [p.copy() for p in params], accum)
+    what = (ctor.__name__, shape, dim, accum, perms, spec.plan().kernels)
+    for g, w, perm in zip(got, want, perms):
+        np.testing.assert_allclose(g, w.transpose(perm), rtol=1e-4 if shape[dim] > 512 else 2e-5, atol=1e-7, err_msg=str(what))
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_broadcast_and_fill(gpu, seed):
+    rng = np.random.default_rng(9400 + seed)
+    rank = int(rng.integers(1, 5))
+    shape = [int(rng.choice(SIZES)) for _ in range(rank)]
+    dim = int(rng.integers(rank))
+    dtype = [M.u8, M.bf16, M.f32, M.i16, M.u32][seed % 5]
+    red = list(shape)
+    red[dim] = 1
+    x = random_values(rng, dtype, red, 9400 + seed)
+    lay = random_layout(rng, shape)[0] if rng.random() < 0.3 else None
+    if lay is None:
+        got = run_spec(M.Broadcast(shape, dim, dtype), [x, np.zeros(shape, NP[dtype])])
+        assert np.array_equal(got, np.broadcast_to(x, shape)), (shape, dim, dtype)
+    count = int(np.prod(shape))
+    value = M.FillValue.NegInf if dtype in (M.bf16, M.f32) and seed % 2 else M.FillValue.Min
+    whole = np.full(count + 40, 0x55, NP[dtype])
+    buf = M.DeviceBuffer.from_numpy(whole)
+    M.Fill(shape, dtype, value, layout=lay).run_device([buf.ptr])
+    back = buf.to_numpy(NP[dtype], whole.shape)
+    buf.free()
+    codes = {M.u8: orc.U8, M.bf16: orc.BF16, M.f32: orc.F32, M.i16: orc.I16, M.u32: orc.U32}
+    assert np.array_equal(back[:count].view(np.uint8), orc.fill(codes[dtype], int(value), count).view(np.uint8))
+    assert np.all(back[count:] == 0x55)
