@@ -1350,9 +1350,22 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
 
 // Move between two strided layouts of the same logical shape.
 hipError_t launch_move_strided(const Strided &src, const Strided &dst, hipStream_t stream) {
+  // Dims of size one address nothing; neighbours that continue each other on both sides (h and w
+  // of an image between NCHW and NHWC) are one dim: the tiled kernels then see its whole length
+  // (56 x 56 pixels as 3136, whole 16-byte vectors, where a row of 56 is not).
   MoveDim dims[MRL_MAX_RANK];
-  for (uint32_t d = 0; d < src.rank; d++) dims[d] = {src.shape[d], src.stride[d], dst.stride[d]};
-  return launch_move_view(src.ptr, src.dtype, dst.ptr, dst.dtype, dims, src.rank, stream);
+  uint32_t n = 0;
+  for (uint32_t d = 0; d < src.rank; d++) {
+    if (src.shape[d] == 1) continue;
+    const MoveDim next = {src.shape[d], src.stride[d], dst.stride[d]};
+    if (n > 0 && dims[n - 1].ss == next.ss * int64_t(next.size) && dims[n - 1].ds == next.ds * int64_t(next.size) &&
+        uint64_t(dims[n - 1].size) * next.size <= 0xffffffffull)
+      dims[n - 1] = {dims[n - 1].size * next.size, next.ss, next.ds};
+    else
+      dims[n++] = next;
+  }
+  if (n == 0) dims[n++] = {1, 1, 1};
+  return launch_move_view(src.ptr, src.dtype, dst.ptr, dst.dtype, dims, n, stream);
 }
 
 hipError_t launch_pad_rows(const Strided &src, void *dst, uint32_t dst_ld, uint32_t elem_size,
