@@ -18,7 +18,7 @@ GEN_DIR = os.path.join(OBJ_DIR, "gen")   # generated assembly (the k loops of th
 # generator -> the file the kernel header of the same tile includes
 GENERATED = {"gen_gemm_wide.py": "gemm_wide_gfx950.inc", "gen_gemm_loop.py": "gemm_loop_gfx950.inc"}
 
-SOURCES = ["api.hip", "generic.hip", "gemm_mfma.hip", "gemm_sched.hip", "gemm_nt.hip", "gemv.hip", "conv_gemm.hip", "conv_i8.hip", "conv_windows.hip", "unfold.hip", "softmax.hip", "parts.hip", "mfma_rate.hip", "attention.hip", "plan.hip"]
+SOURCES = ["api.hip", "generic.hip", "gemm_mfma.hip", "gemm_sched.hip", "gemm_nt.hip", "gemv.hip", "conv_gemm.hip", "conv_i8.hip", "conv_windows.hip", "conv_small.hip", "unfold.hip", "softmax.hip", "parts.hip", "mfma_rate.hip", "attention.hip", "plan.hip"]
 
 # -packed-fp32-ops off: the compiler must not form v_pk_{add,mul,fma}_f32.
 FLAGS = [

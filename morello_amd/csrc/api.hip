@@ -561,6 +561,17 @@ struct Forced {
 };
 thread_local const Forced *g_forced = nullptr;
 
+// Where the kernel of conv_small.hip is taken (switches for measurement builds).
+#ifndef MRL_CONV_SMALL_MIN_PIXELS
+#define MRL_CONV_SMALL_MIN_PIXELS 16384ull
+#endif
+#ifndef MRL_CONV_SMALL_MAX_FILTERS
+#define MRL_CONV_SMALL_MAX_FILTERS 48u
+#endif
+#ifndef MRL_CONV_SMALL_MAX_WINDOW
+#define MRL_CONV_SMALL_MAX_WINDOW 320ull
+#endif
+
 int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
   const int forced = g_forced ? g_forced->conv_path : 0;
   Prepared img, filt, out;
@@ -652,6 +663,18 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
   // Few channels per pixel (a first layer): the fused kernel that forms the windows in LDS.
   const bool windows_ok = kind >= 0 && kind <= 3 && as_matmul && channels_last(img.t) && channels_last(filt.t) && channels_last(out.t) &&
                           mrl::conv_windows_applicable(cv, kind) && !(forced == 1 && g_forced->conv_rows);
+  // Short windows over pixels of whole chunks and few filters (early layers of 16 or 32 channels):
+  // the filters stay in registers and the pixels come straight from memory.  Measured against
+  // the implicit Matmul, whose 64-wide tiles are then mostly padding (us, this kernel / implicit):
+  // 32 x (32 -> 32) x 112^2 3 x 3 int8 35.6 / 44.3, bf16 16 -> 16 24.7 / 40.1, int8 48 -> 48 2 x 2 at
+  // 56^2 11.7 / 13.2; with 64 filters or more, or windows beyond five k steps, it is the slower one
+  // (a wave has one tile of 16 pixels in flight: int8 32 -> 64 at 56^2 17.6 / 13.9, 16 -> 32 5 x 5 62.7 /
+  // 47.3, bf16 32 -> 32 3 x 3 71.5 / 49.5), so those stay implicit.
+  const bool small_ok = kind >= 0 && kind <= 2 && as_matmul && !(cv.fh == 1 && cv.fw == 1) && channels_last(img.t) &&
+                        channels_last(filt.t) && channels_last(out.t) && mrl::conv_small_applicable(cv, kind) &&
+                        cv.f <= MRL_CONV_SMALL_MAX_FILTERS &&
+                        uint64_t(cv.fh) * cv.fw * cv.c * (kind == 2 ? 2 : 1) <= MRL_CONV_SMALL_MAX_WINDOW &&
+                        uint64_t(cv.b) * cv.oh * cv.ow >= MRL_CONV_SMALL_MIN_PIXELS;
   if ((forced == 1 && !fused_ok && !windows_ok) || (forced == 2 && !implicit_ok) || (forced == 3 && !unfold_ok)) return MRL_ERR_UNSUPPORTED;
   if (fused_ok && forced <= 1) {
     const bool rows = forced == 1 && g_forced->conv_rows;
@@ -659,6 +682,8 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
     HIP_TRY(mrl::launch_conv_i8(cv, di == MRL_U8, ws.stream, rows));
   } else if (windows_ok && forced <= 1) {
     HIP_TRY(mrl::launch_conv_windows(cv, kind, ws.stream));
+  } else if (small_ok && forced == 0) {
+    HIP_TRY(mrl::launch_conv_small(cv, kind, ws.stream));
   } else if (implicit_ok && (forced == 0 || forced == 2)) {
     // Channel vectors of whole 16-byte chunks: the windows are read where they lie.  (A 1x1 filter
     // needs no window arithmetic: its image is the left operand of a plain Matmul, below.)
@@ -1615,7 +1640,7 @@ uint32_t mrl_target_layouts_for_shape(const uint32_t *shape, uint32_t rank, int 
 
 uint32_t mrl_target_kernels(const char **names, uint32_t cap) {
   static const char *const families[] = {
-      "k_gemm", "k_gemm_big", "k_gemm_wide", "k_gemv", "k_matmul_generic", "k_sum_splits", "k_conv_i8", "k_conv_rows_i8", "k_conv_windows", "k_conv_generic", "k_conv_generic_wave", "k_unfold",
+      "k_gemm", "k_gemm_big", "k_gemm_wide", "k_gemv", "k_matmul_generic", "k_sum_splits", "k_conv_i8", "k_conv_rows_i8", "k_conv_windows", "k_conv_small", "k_conv_generic", "k_conv_generic_wave", "k_unfold",
       "k_unfold_gather", "k_attn", "k_attn_merge", "k_softmax_regs", "k_softmax_regs1", "k_softmax_short", "k_softmax_block", "k_softmax_chunk_stats", "k_softmax_chunk_write",
       "k_softmax_cols",
       "k_softmax_generic", "k_parts", "k_parts_rows", "k_parts_cols", "k_broadcast", "k_broadcast_rows", "k_broadcast_fill_rows", "k_fill", "k_fill16", "k_fill_zero", "k_move_rows", "k_move_rows16",

@@ -150,6 +150,10 @@ hipError_t launch_conv_i8(const ConvArgs &c, bool img_unsigned, hipStream_t stre
 // ---- conv_windows.hip: Conv u8|i8 x i8 -> i32 and bf16 x bf16 -> f32 (kind 0, 1, 2 as for a Matmul),
 // channels-last, pixels of few channels (not whole 16-byte chunks), windows of at most 384
 // bytes, filters in 16s: the windows are formed in LDS.
+// conv_small.hip: windows of at most 576 bytes over pixels of whole 16-byte chunks, the filters
+// resident in registers (kind: 0 i8, 1 u8, 2 bf16 operands).
+bool conv_small_applicable(const ConvArgs &c, int kind);
+hipError_t launch_conv_small(const ConvArgs &c, int kind, hipStream_t stream);
 bool conv_windows_applicable(const ConvArgs &c, int kind);
 hipError_t launch_conv_windows(const ConvArgs &c, int kind, hipStream_t stream);
 

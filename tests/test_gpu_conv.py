@@ -171,6 +171,42 @@ def test_conv_with_few_channels_forms_its_windows_in_lds(gpu, shape, accum, img_
 
 
 @pytest.mark.parametrize("shape,accum", [
+    ((16, 32, 32, 40, 41, 3, 3), False),  # 32 channels, 3 x 3: 288 bytes, the last k step half empty
+    ((9, 48, 16, 50, 45, 4, 4), True),    # 16 channels, 4 x 4: four whole k steps; three tiles of filters
+    ((20, 16, 48, 30, 31, 2, 2), False),  # 48 channels: runs of 96 bytes, k steps across runs
+    ((3, 32, 32, 90, 70, 2, 5), True),    # 320 bytes, five k steps
+    ((1, 16, 64, 130, 129, 2, 2), False), # 64 channels under 2 x 2 with 16 filters (the 64-channel kernel wants filters in 64s)
+])
+@pytest.mark.parametrize("dts,codes", [((M.u8, M.i8, M.i32), [0, 1, 5]), ((M.i8, M.i8, M.i32), [1, 1, 5]), ((M.bf16, M.bf16, M.f32), [7, 7, 6])])
+def test_early_layer_conv_with_the_filters_in_registers(gpu, shape, accum, dts, codes):
+    """Pixels of whole 16-byte chunks, windows of up to 320 bytes, up to 48 filters, 16384 pixels or
+    more: the kernel that keeps the filter bank in registers.  Integers bit for bit, bf16 to 1e-5
+    of the oracle; an infinity in a bf16 image reaches the outputs whose windows hold it as an
+    infinity (the chunks past the window's end are zero on both sides)."""
+    b, f, c, oh, ow, fh, fw = shape
+    if dts[0] == M.bf16:
+        c //= 2   # the same bytes per pixel
+    shape = (b, f, c, oh, ow, fh, fw)
+    spec = M.Conv(list(shape), dts, accum=accum)
+    assert spec.plan().kernels == ["k_conv_small"], spec.plan()
+    floats = dts[0] == M.bf16
+    gen = {M.u8: synth.uniform_u8, M.i8: synth.uniform_i8, M.bf16: synth.normal_bf16}
+    img, filt = gen[dts[0]](138, 0, (b, oh + fh - 1, ow + fw - 1, c)), gen[dts[1]](138, 1, (f, fh, fw, c))
+    out0 = synth.uniform_u8(138, 2, (b, oh, ow, f)).astype(np.float32 if floats else np.int32) - 100
+    want = orc.conv(list(shape), codes, img, filt, out0.copy(), accum, layouts=[NHWC] * 3)
+    got = run_spec(spec, [img, filt, out0.copy()])
+    if not floats:
+        assert np.array_equal(got, want)
+        return
+    assert float(np.abs(got.astype(np.float64) - want).max() / np.abs(want).max()) < 1e-5
+    img = img.copy()
+    img[b - 1, oh + fh - 2, ow + fw - 2, c - 1] = 0x7f80       # +inf in the last pixel's last channel
+    want = orc.conv(list(shape), codes, img, filt, out0.copy(), accum, layouts=[NHWC] * 3)
+    got = run_spec(spec, [img, filt, out0.copy()])
+    assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(np.isinf(got), np.isinf(want))
+
+
+@pytest.mark.parametrize("shape,accum", [
     ((2, 64, 3, 20, 37, 5, 5), False),    # runs of 60 bytes, five k steps
     ((4, 16, 1, 30, 30, 3, 3), True),     # runs of 12 bytes
     ((2, 80, 3, 17, 15, 3, 3), True),     # two groups of filters

@@ -339,13 +339,17 @@ def test_cost_model_ranks_manual_schedules(gpu):
                         assert measured[x] <= 1.25 * measured[y], (dts[0], m, k, n, x, y, measured, predicted)
 
 
-def test_one_chunk_pixels_with_short_windows_take_the_windows_kernel():
+def test_early_layer_convs_of_whole_chunk_pixels():
     """Host only: pixels of exactly 16 bytes with windows of up to 192 bytes go to the kernel that
-    forms windows in LDS; wider pixels and longer windows stay with the implicit Matmul."""
-    kernels = lambda c, fs, dts: M.Conv([32, 32, c, 112, 112, fs, fs], dts).plan().kernels
+    forms windows in LDS; wider pixels with windows of up to 320 bytes and at most 48 filters to
+    the kernel that keeps the filters in registers; more filters, longer windows and small
+    problems stay with the implicit Matmul."""
+    kernels = lambda c, f, fs, dts, b=32: M.Conv([b, f, c, 112, 112, fs, fs], dts).plan().kernels
     i8, bf = (M.u8, M.i8, M.i32), (M.bf16, M.bf16, M.f32)
-    assert kernels(16, 3, i8) == ["k_conv_windows"] and kernels(8, 3, bf) == ["k_conv_windows"]
-    assert kernels(32, 3, i8) == ["k_gemm"] and kernels(16, 3, bf) == ["k_gemm"] and kernels(16, 5, i8) == ["k_gemm"]
+    assert kernels(16, 32, 3, i8) == ["k_conv_windows"] and kernels(8, 32, 3, bf) == ["k_conv_windows"]
+    assert kernels(32, 32, 3, i8) == ["k_conv_small"] and kernels(16, 32, 3, bf) == ["k_conv_small"] and kernels(48, 48, 2, i8) == ["k_conv_small"]
+    assert kernels(32, 64, 3, i8) == ["k_gemm"] and kernels(16, 32, 5, i8) == ["k_gemm"] and kernels(32, 32, 3, bf) == ["k_gemm"]
+    assert kernels(32, 32, 3, i8, b=1) == ["k_gemm"]     # 12544 pixels: too few tiles for one per wave
 
 
 def test_plans_of_the_softmax_primitives():
