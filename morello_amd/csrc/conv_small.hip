@@ -13,9 +13,11 @@
 //
 // Taken for early layers of 16 or 32 channels with at most 48 filters and windows of at most 320
 // bytes, where the implicit Matmul (conv_gemm.hip) pads its 64-wide tiles: 32 x (32 -> 32) x 112^2,
-// 3 x 3, int8 44 -> 36 us, bf16 16 -> 16 40 -> 25 us.  A wave has one tile of 16 pixels in flight
-// beside the one it multiplies, which with more filters or longer windows hides less of the
-// memory's latency than the implicit kernel's workgroups do; the dispatch keeps those there.
+// 3 x 3, int8 44 -> 34 us, bf16 16 -> 16 40 -> 23 us.  A wave's loads of its next pixels are
+// counted complete only behind the stores it issued before them (a wave's vector memory
+// operations complete in order), so a round lasts about as long as a store's acknowledgement
+// whatever is in flight; with more filters or longer windows the implicit kernel's workgroups
+// hide more of that, and the dispatch keeps those there.
 #include <algorithm>
 
 #include "kernels.h"
@@ -33,6 +35,9 @@ constexpr int FT = 4;       // filter tiles of 16 per workgroup: groups of 64 fi
 constexpr int WAVES = 4;
 constexpr int TURN_ROW = 68;  // dwords between the pixel rows of a wave's patch of results
 
+// Tiles a wave has in flight per round: two while their pixel registers fit beside the filters'.
+constexpr int tiles_per_round(int slabs) { return slabs <= 5 ? 2 : 1; }
+
 struct SmallArgs {
   const uint8_t *image, *filters;
   void *out;
@@ -42,8 +47,10 @@ struct SmallArgs {
   uint32_t k_bytes;   // fh * fw * c_bytes, a multiple of 16
 };
 
-// SLABS: k steps of 64 bytes per window, ceil(k_bytes / 64).
-template <int SLABS, int KIND>
+// SLABS: k steps of 64 bytes per window, ceil(k_bytes / 64).  TILES: tiles of 16 pixels a wave takes
+// per round (their pixels are all requested before the first is used: with short windows a
+// tile's MFMAs are too few to cover the next tile's trip to memory).
+template <int SLABS, int KIND, int TILES>
 __global__ __launch_bounds__(64 * WAVES) void k_conv_small(SmallArgs p) {
   constexpr bool IMG_UNSIGNED = KIND == SMALL_U8, FLOATS = KIND == SMALL_BF16;
   typedef typename std::conditional<FLOATS, v4f, v4i>::type Acc;
@@ -90,16 +97,22 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_small(SmallArgs p) {
     const uint32_t qc = chunk_valid[s] ? q : 0, r = qc / run_chunks;
     slab_off[s] = int((r * W) * p.c_bytes + (qc - r * run_chunks) * 16);
   }
-  auto load_tile = [&](uint32_t t, v4i *img) {
-    const uint32_t pix = min(t * 16 + li, p.pixels - 1);   // past the end: the last pixel again, not stored
+  // The lane's pixel of tile t (past the end: the last pixel again, which is not stored).
+  auto pixel_of = [&](uint32_t t) {
+    const uint32_t pix = min(min(t, p.tiles - 1) * 16 + li, p.pixels - 1);
     const uint32_t x = pix % p.ow, y = (pix / p.ow) % p.oh, b = pix / (p.ow * p.oh);
-    const uint8_t *src = p.image + (int64_t(b) * H * W + int64_t(y) * W + x) * p.c_bytes;
-#pragma unroll
-    for (int s = 0; s < SLABS; s++) img[s] = *(const v4i *)(src + slab_off[s]);
+    return p.image + (int64_t(b) * H * W + int64_t(y) * W + x) * p.c_bytes;
   };
-  v4i img[SLABS];
-  uint32_t t = wave;
-  if (t < p.tiles) load_tile(t, img);
+  v4i img[TILES][SLABS];
+  uint32_t t = wave * TILES;   // a round's tiles follow one another
+  if (t < p.tiles) {
+#pragma unroll
+    for (int u = 0; u < TILES; u++) {
+      const uint8_t *src = pixel_of(t + u);
+#pragma unroll
+      for (int s = 0; s < SLABS; s++) img[u][s] = *(const v4i *)(src + slab_off[s]);
+    }
+  }
   __syncthreads();
   v4i filt[FT][SLABS];
 #pragma unroll
@@ -127,52 +140,54 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_small(SmallArgs p) {
   }
 
   while (t < p.tiles) {
-    const uint32_t tn = t + nwaves;
-    const uint32_t pix_n = min(min(tn, p.tiles - 1) * 16 + li, p.pixels - 1);
-    const uint32_t xn = pix_n % p.ow, yn = (pix_n / p.ow) % p.oh, bn = pix_n / (p.ow * p.oh);
-    const uint8_t *src_n = p.image + (int64_t(bn) * H * W + int64_t(yn) * W + xn) * p.c_bytes;
-    Acc acc[FT] = {};
+    const uint32_t tn = t + nwaves * TILES;
 #pragma unroll
-    for (int s = 0; s < SLABS; s++) {
-      v4i px = img[s];
-      if constexpr (IMG_UNSIGNED) px ^= v4i{int(0x80808080), int(0x80808080), int(0x80808080), int(0x80808080)};
-      if constexpr (FLOATS)
-        if (s == SLABS - 1 && !chunk_valid[s]) px = v4i{0, 0, 0, 0};
+    for (int u = 0; u < TILES; u++) {
+      const uint8_t *src_n = pixel_of(tn + u);
+      Acc acc[FT] = {};
 #pragma unroll
-      for (int ft = 0; ft < FT; ft++)
-        if (ft < nft) acc[ft] = mfma(filt[ft][s], px, acc[ft]);
-      img[s] = *(const v4i *)(src_n + slab_off[s]);
-    }
-    // A lane holds filters 16 ft + 4 lg .. + 3 of pixel li: through the wave's patch of LDS, then
-    // out as whole pixel rows (lane (li, lg): pixel 4 i + lg, filters 4 li .. + 3).
+      for (int s = 0; s < SLABS; s++) {
+        v4i px = img[u][s];
+        if constexpr (IMG_UNSIGNED) px ^= v4i{int(0x80808080), int(0x80808080), int(0x80808080), int(0x80808080)};
+        if constexpr (FLOATS)
+          if (s == SLABS - 1 && !chunk_valid[s]) px = v4i{0, 0, 0, 0};
 #pragma unroll
-    for (int ft = 0; ft < FT; ft++) {
-      Acc v = acc[ft];
-      if constexpr (IMG_UNSIGNED) v += *(const v4i *)(corr_lds + ft * 16 + lg * 4);
-      *(Acc *)(turn_lds + li * TURN_ROW + ft * 16 + lg * 4) = v;
-    }
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const uint32_t row = i * 4 + lg, pix = t * 16 + row;
-      Acc v = *(const Acc *)(turn_lds + row * TURN_ROW + li * 4);
-      if (pix < p.pixels && uint32_t(li * 4) < nf) {
-        Acc *d = (Acc *)((uint32_t *)p.out + int64_t(pix) * p.f + f0 + li * 4);
-        if (p.accum) v += *d;
-        __builtin_nontemporal_store(v, d);
+        for (int ft = 0; ft < FT; ft++)
+          if (ft < nft) acc[ft] = mfma(filt[ft][s], px, acc[ft]);
+        img[u][s] = *(const v4i *)(src_n + slab_off[s]);   // the next round's, as soon as this one's is used
       }
+      // A lane holds filters 16 ft + 4 lg .. + 3 of pixel li: through the wave's patch of LDS, then
+      // out as whole pixel rows (lane (li, lg): pixel 4 i + lg, filters 4 li .. + 3).
+#pragma unroll
+      for (int ft = 0; ft < FT; ft++) {
+        Acc v = acc[ft];
+        if constexpr (IMG_UNSIGNED) v += *(const v4i *)(corr_lds + ft * 16 + lg * 4);
+        *(Acc *)(turn_lds + li * TURN_ROW + ft * 16 + lg * 4) = v;
+      }
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const uint32_t row = i * 4 + lg, pix = (t + u) * 16 + row;
+        Acc v = *(const Acc *)(turn_lds + row * TURN_ROW + li * 4);
+        if (pix < p.pixels && uint32_t(li * 4) < nf) {
+          Acc *d = (Acc *)((uint32_t *)p.out + int64_t(pix) * p.f + f0 + li * 4);
+          if (p.accum) v += *d;
+          __builtin_nontemporal_store(v, d);
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
     }
-    __builtin_amdgcn_wave_barrier();
     t = tn;
   }
 }
 
 template <int SLABS>
 hipError_t launch_slabs(const SmallArgs &p, int kind, dim3 grid, size_t lds, hipStream_t stream) {
+  constexpr int TILES = tiles_per_round(SLABS);
   switch (kind) {
-    case SMALL_I8: MRL_LAUNCH((k_conv_small<SLABS, SMALL_I8>), grid, dim3(64 * WAVES), lds, stream, p); break;
-    case SMALL_U8: MRL_LAUNCH((k_conv_small<SLABS, SMALL_U8>), grid, dim3(64 * WAVES), lds, stream, p); break;
-    case SMALL_BF16: MRL_LAUNCH((k_conv_small<SLABS, SMALL_BF16>), grid, dim3(64 * WAVES), lds, stream, p); break;
+    case SMALL_I8: MRL_LAUNCH((k_conv_small<SLABS, SMALL_I8, TILES>), grid, dim3(64 * WAVES), lds, stream, p); break;
+    case SMALL_U8: MRL_LAUNCH((k_conv_small<SLABS, SMALL_U8, TILES>), grid, dim3(64 * WAVES), lds, stream, p); break;
+    case SMALL_BF16: MRL_LAUNCH((k_conv_small<SLABS, SMALL_BF16, TILES>), grid, dim3(64 * WAVES), lds, stream, p); break;
     default: return hipErrorInvalidValue;
   }
   return plan::last_error();
@@ -203,8 +218,9 @@ hipError_t launch_conv_small(const ConvArgs &c, int kind, hipStream_t stream) {
   const int slabs = int((p.k_bytes + 63) / 64);
   const uint32_t groups = (c.f + 63) / 64;
   // as many waves as the chip holds at this kernel's register count, never more than tiles
-  uint32_t blocks = std::max<uint32_t>(1, (slabs > 5 ? 2048u : 4096u) / WAVES / groups);
-  if (blocks * WAVES > p.tiles) blocks = (p.tiles + WAVES - 1) / WAVES;
+  uint32_t blocks = std::max<uint32_t>(1, 2048u / WAVES / groups);
+  const uint32_t rounds = (p.tiles + tiles_per_round(slabs) - 1) / tiles_per_round(slabs);
+  if (blocks * WAVES > rounds) blocks = (rounds + WAVES - 1) / WAVES;
   const size_t lds = size_t(FT) * 16 * p.k_bytes + FT * 16 * sizeof(int) + size_t(WAVES) * 16 * TURN_ROW * sizeof(int);
   plan::work(kind == 2 ? plan::UNIT_MFMA_BF16 : plan::UNIT_MFMA_I8, 2.0 * pixels * c.f * c.fh * c.fw * c.c,
              double(c.b) * (c.oh + c.fh - 1) * (c.ow + c.fw - 1) * p.c_bytes + double(c.f) * p.k_bytes +
