@@ -21,7 +21,8 @@
 //   k_parts_cols   the scan dim is not the innermost one: C adjacent lines side by side in a
 //                  workgroup (adjacent in memory when the innermost dim is contiguous, so a
 //                  wavefront's loads are whole cache lines), each shared by 256 / C threads that
-//                  walk the scan dim in steps of 256 / C and combine through LDS.
+//                  walk the scan dim in steps of 256 / C and combine through LDS; with C = 256, a
+//                  thread per line, also the form for lines of a handful of elements.
 // The arithmetic is written once (parts_line) over a Share: how the threads of a line divide
 // it and combine their partial results.
 #include "kernels.h"
@@ -456,7 +457,11 @@ hipError_t launch_parts(const PartsArgs &p, hipStream_t stream) {
     default: break;
   }
   plan::work(plan::UNIT_STREAM, 0, 4.0 * passes * p.lines * n);
-  if (rows) {
+  if (n <= 16 && p.lines >= 1024) {
+    // Lines of a handful of elements (the merge of a few tiles' pairs): a thread per line; a
+    // wavefront per line would leave all but a few lanes idle (65536 lines of 2: 25 us).
+    MRL_LAUNCH(k_parts_cols<256>, dim3(uint32_t((p.lines + 255) / 256)), dim3(256), 0, stream, p);
+  } else if (rows) {
     if (n <= 1024) MRL_LAUNCH(k_parts_rows<4>, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
     else if (n <= 2048) MRL_LAUNCH(k_parts_rows<8>, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
     else MRL_LAUNCH(k_parts_rows<16>, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);

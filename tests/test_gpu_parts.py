@@ -17,7 +17,9 @@ SHAPES = [((7, 33), 1), ((5, 9, 4), 1), ((3, 4, 130), 2), ((6, 5), 0), ((2, 3, 4
           # contiguous lines of whole 16-byte vectors: register-resident (4, 8, 16 vectors a lane)
           ((33, 1024), 1), ((5, 12), 1), ((7, 3, 2048), 2), ((9, 4096), 1), ((3, 4100), 1),
           # the scan dim is not the innermost: lines side by side, 16, 32 or 64 to a workgroup
-          ((37, 70), 0), ((3, 50, 33), 1), ((2, 300, 64), 1), ((5, 20000), 0), ((8, 40000), 0), ((1, 18), 0)]
+          ((37, 70), 0), ((3, 50, 33), 1), ((2, 300, 64), 1), ((40, 20000), 0), ((24, 40000), 0), ((1, 18), 0),
+          # lines of a handful of elements: a thread per line
+          ((5, 20000), 0), ((3000, 8), 1), ((40, 50, 2), 2)]
 TOL = dict(rtol=1e-5, atol=1e-7)
 
 
@@ -120,7 +122,8 @@ def test_softmax_denominator_and_max_of_masked_lines(gpu, shape, dim):
     np.testing.assert_allclose(got_d[keep], got[2][keep], rtol=2e-5)
 
 
-@pytest.mark.parametrize("shape,dim", [((6, 5), 1), ((3, 9, 4), 1), ((4, 70), 1), ((8, 3), 0), ((40, 33), 0), ((3, 20, 64), 1)])
+@pytest.mark.parametrize("shape,dim", [((6, 5), 1), ((3, 9, 4), 1), ((4, 70), 1), ((8, 3), 0), ((40, 33), 0), ((3, 20, 64), 1),
+                                       ((16, 300, 2), 2), ((2000, 7), 1)])
 @pytest.mark.parametrize("accum", [False, True])
 def test_softmax_denominator_and_max_from_parts(gpu, shape, dim, accum):
     tmax, tden = rnd(shape, 4.0), np.abs(rnd(shape)) + np.float32(1.0)

@@ -364,8 +364,11 @@ def test_plans_of_the_softmax_primitives():
     assert kernel(M.Max([3, 4100], 1))[0] == "k_parts" and kernel(M.Max([7, 33], 1))[0] == "k_parts"
     assert kernel(M.DivideVec([64, 64]))[0] == "k_parts"
     assert kernel(M.SoftmaxDenominatorAndMax([2048, 4096], 0)) == ("k_parts_cols", (256, 1))     # 16 lines each
-    assert kernel(M.SoftmaxDenominatorAndMax([5, 20000], 0)) == ("k_parts_cols", (625, 1))       # 32
-    assert kernel(M.SoftmaxDenominatorAndMax([8, 40000], 0)) == ("k_parts_cols", (625, 1))       # 64
+    assert kernel(M.SoftmaxDenominatorAndMax([40, 20000], 0)) == ("k_parts_cols", (625, 1))      # 32
+    assert kernel(M.SoftmaxDenominatorAndMax([40, 40000], 0)) == ("k_parts_cols", (625, 1))      # 64
+    # lines of a handful of elements (the merge of a few tiles' pairs): a thread per line
+    assert kernel(M.SoftmaxDenominatorAndMax([5, 20000], 0)) == ("k_parts_cols", (79, 1))
+    assert kernel(M.SoftmaxDenominatorAndMaxFromParts([16, 2048, 2], 2)) == ("k_parts_cols", (128, 1))
     assert kernel(M.Max([5, 9, 4], 1))[0] == "k_parts"                                           # rows of 4 elements: not worth lining up
     # col-major: the lines are contiguous, each starting on any 4 bytes
     assert kernel(M.Max([33, 64], 0, layouts=[M.col_major([33, 64]), None]))[0] == "k_parts"
@@ -386,8 +389,8 @@ def test_actions_of_a_softmax():
     assert [a.kind for a in acts] == [K.Select, K.ToSoftmaxParts, K.ToSoftmaxPartsRecompute] + [K.ParallelSoftmax] * 5
     assert [a.parts for a in acts[3:]] == [2, 4, 8, 16, 32]
     assert acts[0].plan().kernels == ["k_softmax_regs"]
-    # whole contiguous lines stay in a wavefront's registers; the merge of the tiles' pairs walks a handful of them
-    assert acts[1].plan().kernels == ["k_parts_rows"] * 2 and acts[3].plan().kernels == ["k_parts_rows", "k_parts", "k_parts_rows"]
+    # whole contiguous lines stay in a wavefront's registers; the merge of two tiles' pairs is a thread per line
+    assert acts[1].plan().kernels == ["k_parts_rows"] * 2 and acts[3].plan().kernels == ["k_parts_rows", "k_parts_cols", "k_parts_rows"]
     assert all(a.cost_ns > acts[0].cost_ns for a in acts[1:])
     assert acts[1].scratch_bytes >= 16 * 2048 * 4 and acts[3].scratch_bytes >= 16 * 2048 * 4 * (2 + 2 * 2)
     # integers and other dtypes have no Softmax; a Matmul lists none of these
