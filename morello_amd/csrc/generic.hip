@@ -401,7 +401,7 @@ __global__ __launch_bounds__(256) void k_move_tiled16v(MoveStrided p) {
     const uint32_t r = row + 16 * i;
     v[i] = quad_t{0, 0, 0, 0};
     if (d0 + r < nd && s0 + col < ns)
-      v[i] = __builtin_nontemporal_load((const quad_t *)(src + so + int64_t(d0 + r) * p.ss[p.dim_d] + (s0 + col)));
+      v[i] = MRL_LOAD_ONCE((const quad_t *)(src + so + int64_t(d0 + r) * p.ss[p.dim_d] + (s0 + col)));
   }
 #pragma unroll
   for (int i = 0; i < 8; i++) {
@@ -453,7 +453,7 @@ __global__ __launch_bounds__(256) void k_move_tiled8v(MoveStrided p) {
     const uint32_t r = row + 32 * i;
     v[i] = quad_t{0, 0, 0, 0};
     if (d0 + r < nd && s0 + col < ns)
-      v[i] = __builtin_nontemporal_load((const quad_t *)(src + so + int64_t(d0 + r) * p.ss[p.dim_d] + (s0 + col)));
+      v[i] = MRL_LOAD_ONCE((const quad_t *)(src + so + int64_t(d0 + r) * p.ss[p.dim_d] + (s0 + col)));
   }
 #pragma unroll
   for (int i = 0; i < 4; i++) {
@@ -522,7 +522,7 @@ __global__ __launch_bounds__(256) void k_move_tiled32(MoveStrided p) {
     const uint32_t r = row + 16 * i;
     v[i] = quad_t{0, 0, 0, 0};
     if (d0 + r < nd && s0 + col < ns)
-      v[i] = __builtin_nontemporal_load((const quad_t *)(src + so + int64_t(d0 + r) * p.ss[p.dim_d] + (s0 + col)));
+      v[i] = MRL_LOAD_ONCE((const quad_t *)(src + so + int64_t(d0 + r) * p.ss[p.dim_d] + (s0 + col)));
   }
 #pragma unroll
   for (int i = 0; i < 4; i++) {
@@ -667,7 +667,7 @@ __global__ __launch_bounds__(256) void k_copy16(const v4u *__restrict__ src, v4u
     v4u v[COPY_UNROLL];
 #pragma unroll
     for (int u = 0; u < COPY_UNROLL; u++)
-      if (i + u * 256 < vecs) v[u] = __builtin_nontemporal_load(src + i + u * 256);
+      if (i + u * 256 < vecs) v[u] = MRL_LOAD_ONCE(src + i + u * 256);
 #pragma unroll
     for (int u = 0; u < COPY_UNROLL; u++)
       if (i + u * 256 < vecs) __builtin_nontemporal_store(v[u], dst + i + u * 256);
@@ -715,7 +715,7 @@ __global__ __launch_bounds__(256) void k_pad_rows16(const v4u *__restrict__ src,
   const uint64_t line = i / dst_ld;
   const uint32_t col = uint32_t(i % dst_ld);
   v4u v{0, 0, 0, 0};
-  if (col < cols) v = __builtin_nontemporal_load(src + int64_t(line / rows) * src_batch + int64_t(line % rows) * src_ld + col);
+  if (col < cols) v = MRL_LOAD_ONCE(src + int64_t(line / rows) * src_batch + int64_t(line % rows) * src_ld + col);
   __builtin_nontemporal_store(v, dst + i);
 }
 

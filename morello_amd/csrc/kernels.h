@@ -26,6 +26,21 @@ inline hipError_t raise_lds_limit(std::atomic<uint64_t> &done, const void *kerne
 
 
 // A tensor whose layout is a pure permutation of its logical dims.
+// Accesses of kernels that touch their data once.  Loads are ordinary ones and stores non-temporal:
+// measured on the Softmax of 16 x 2048 rows of 2048 f32 (one read, one write of 268 MB each), that
+// pairing took 83 us, non-temporal loads and stores 89, ordinary loads and stores 104, non-temporal
+// loads with ordinary stores 85.  (The switches are for such measurements.)
+#ifdef MRL_NT_LOADS
+#define MRL_LOAD_ONCE(p) __builtin_nontemporal_load(p)
+#else
+#define MRL_LOAD_ONCE(p) (*(p))
+#endif
+#ifdef MRL_PLAIN_STORES
+#define MRL_STORE_ONCE(v, p) (*(p) = (v))
+#else
+#define MRL_STORE_ONCE(v, p) __builtin_nontemporal_store(v, p)
+#endif
+
 struct Strided {
   void *ptr;
   int dtype;

@@ -297,7 +297,7 @@ __global__ __launch_bounds__(256) void k_parts_rows(PartsArgs p) {
   };
   auto store = [&](f4 *dst) {
 #pragma unroll
-    EACH(i, idx) dst[idx] = v[i];
+    EACH(i, idx) MRL_STORE_ONCE(v[i], dst + idx);
   };
   switch (p.kind) {
     case MRL_SPEC_MAX: {

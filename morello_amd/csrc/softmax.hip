@@ -54,8 +54,7 @@ __global__ __launch_bounds__(256) void k_softmax_regs(const float *__restrict__ 
   for (int i = 0; i < NV; i++) {
     const uint32_t idx = i * 64 + lane;
     if (idx < nvec) {
-      // Streamed once: keep it out of the caches' way.
-      const f4 t = __builtin_nontemporal_load((const f4 *)src + idx);
+      const f4 t = MRL_LOAD_ONCE((const f4 *)src + idx);
       v[i] = float4{t[0], t[1], t[2], t[3]};
       nan |= (v[i].x != v[i].x) | (v[i].y != v[i].y) | (v[i].z != v[i].z) | (v[i].w != v[i].w);
       mx = fmaxf(fmaxf(mx, fmaxf(v[i].x, v[i].y)), fmaxf(v[i].z, v[i].w));
@@ -108,7 +107,7 @@ __global__ __launch_bounds__(256) void k_softmax_regs1(const float *__restrict__
 #pragma unroll
   for (int i = 0; i < NE; i++) {
     const uint32_t e = i * 64 + lane;
-    v[i] = e < cols ? __builtin_nontemporal_load(src + e) : F32_MIN;
+    v[i] = e < cols ? MRL_LOAD_ONCE(src + e) : F32_MIN;
     nan |= v[i] != v[i];
     mx = fmaxf(mx, v[i]);
   }
@@ -326,7 +325,7 @@ __global__ __launch_bounds__(256) void k_softmax_block(const float *__restrict__
   for (int i = 0; i < NV; i++) {
     const uint32_t idx = i * 256 + threadIdx.x;
     if (idx < nvec) {
-      v[i] = __builtin_nontemporal_load(src + idx);
+      v[i] = MRL_LOAD_ONCE(src + idx);
       nan |= (v[i][0] != v[i][0]) | (v[i][1] != v[i][1]) | (v[i][2] != v[i][2]) | (v[i][3] != v[i][3]);
       mx = fmaxf(fmaxf(mx, fmaxf(v[i][0], v[i][1])), fmaxf(v[i][2], v[i][3]));
     }
