@@ -46,15 +46,15 @@ MEASURED_TRAFFIC_BYTES = {
     "c3": 2299689530,
     "c4": 41176586,
     "c5": 42162440,
-    "softmax": 536985852,
+    "softmax": 537353602,
     "move": 536870912,
     "matvec": 67270103,
     "conv128": 19390667,
     "decode": 268960727,
     "softmax_long": 77155935,
-    "transpose": 537003671,
+    "transpose": 537368281,
     "conv_first": 109310051,
-    "softmax_outer": 101886842,
+    "softmax_outer": 101921724,
 }
 KT_LAYOUT = M.layout(0, 2, 1)
 

@@ -157,6 +157,8 @@ __device__ inline uint32_t convert_raw(uint32_t raw, int sdt, int ddt) {
 
 // Move of a contiguous run with a dtype conversion: four elements per thread, one vector load
 // and one vector store (SE, DE: element sizes in bytes).
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
+typedef unsigned v4u_t __attribute__((ext_vector_type(4)));
 template <int SE, int DE>
 __global__ __launch_bounds__(256) void k_convert4(const void *__restrict__ src, void *__restrict__ dst, int sdt,
                                                   int ddt, uint64_t count) {
@@ -175,7 +177,10 @@ __global__ __launch_bounds__(256) void k_convert4(const void *__restrict__ src, 
 #pragma unroll
       for (int k = 0; k < DE; k++) out.b[e * DE + k] = uint8_t(v >> (8 * k));
     }
-    static_cast<DstQuad *>(dst)[i] = out;
+    // the four converted elements as one store of 4, 8 or 16 bytes
+    if constexpr (DE == 1) MRL_STORE_ONCE(__builtin_bit_cast(uint32_t, out), static_cast<uint32_t *>(dst) + i);
+    else if constexpr (DE == 2) MRL_STORE_ONCE(__builtin_bit_cast(v2u, out), static_cast<v2u *>(dst) + i);
+    else MRL_STORE_ONCE(__builtin_bit_cast(v4u_t, out), static_cast<v4u_t *>(dst) + i);
   }
   // The up to three elements past the last quad.
   if (blockIdx.x == 0 && threadIdx.x < count % 4) {
@@ -240,7 +245,7 @@ __global__ __launch_bounds__(256) void k_move_rows16(MoveStrided p) {
     rem /= p.shape[d];
     so += int64_t(c) * p.ss[d], d_o += int64_t(c) * p.ds[d];
   }
-  static_cast<uint4 *>(p.dst)[d_o] = static_cast<const uint4 *>(p.src)[so];
+  MRL_STORE_ONCE(static_cast<const v4u_t *>(p.src)[so], static_cast<v4u_t *>(p.dst) + d_o);
 }
 
 // The two sides are contiguous along different dims: a 64 x 64 tile of (dim_d, dim_s) goes
@@ -417,8 +422,8 @@ __global__ __launch_bounds__(256) void k_move_tiled16v(MoveStrided p) {
   for (uint32_t sp = wave; sp < 64; sp += 4) {
     const uint32_t a = tile[2 * lane][sp], b = tile[2 * lane + 1][sp];
     const uint32_t sidx = s0 + 2 * sp;
-    if (sidx < ns) *(uint32_t *)(dst + d_o + int64_t(sidx) * p.ds[p.dim_s] + d) = (a & 0xffffu) | (b << 16);
-    if (sidx + 1 < ns) *(uint32_t *)(dst + d_o + int64_t(sidx + 1) * p.ds[p.dim_s] + d) = (a >> 16) | (b & 0xffff0000u);
+    if (sidx < ns) MRL_STORE_ONCE((a & 0xffffu) | (b << 16), (uint32_t *)(dst + d_o + int64_t(sidx) * p.ds[p.dim_s] + d));
+    if (sidx + 1 < ns) MRL_STORE_ONCE((a >> 16) | (b & 0xffff0000u), (uint32_t *)(dst + d_o + int64_t(sidx + 1) * p.ds[p.dim_s] + d));
   }
 }
 
@@ -487,7 +492,7 @@ __global__ __launch_bounds__(256) void k_move_tiled8v(MoveStrided p) {
 #pragma unroll
       for (uint32_t k = 0; k < 4; k++) {
         const uint32_t sidx = s0 + 4 * sq + k;
-        if (sidx < ns) *(uint32_t *)(dst + d_o + int64_t(sidx) * p.ds[p.dim_s] + d) = out[k];
+        if (sidx < ns) MRL_STORE_ONCE(out[k], (uint32_t *)(dst + d_o + int64_t(sidx) * p.ds[p.dim_s] + d));
       }
     }
   }
@@ -1032,7 +1037,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_softmax_cols(SMC q) {
 #pragma unroll
       for (int j = 0; j < UNROLL; j++) {
         const uint32_t i = i0 + j * WAVES;
-        if (i < n) p.out[obase + i * os] = exp_nonpositive(x[j] - m) * inv_d;
+        if (i < n) MRL_STORE_ONCE(exp_nonpositive(x[j] - m) * inv_d, p.out + obase + i * os);
       }
     }
 }

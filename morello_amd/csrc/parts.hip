@@ -119,7 +119,7 @@ __device__ inline void parts_line(const PartsArgs &p, const Line &l, const S &sh
 #define STORE8(t, i, x)                                       \
   _Pragma("unroll") for (uint32_t k = 0; k < 8; k++) {        \
     const uint32_t at = i + k * sh.stride;                    \
-    if (at < n) AT(t, at) = x[k];                             \
+    if (at < n) MRL_STORE_ONCE(x[k], &AT(t, at));             \
   }
   auto line_max = [&](uint32_t t) {
     float m = NEG_INF;

@@ -174,7 +174,7 @@ __global__ __launch_bounds__(256) void k_softmax_short(const float *__restrict__
     if (e >= cols) continue;
     const float y = x[i] / sum;
     if constexpr (OUT_BF16) (static_cast<uint16_t *>(out_any) + row * cols)[e] = uint16_t(bf16_bits(y));
-    else (static_cast<float *>(out_any) + row * cols)[e] = y;
+    else MRL_STORE_ONCE(y, static_cast<float *>(out_any) + row * cols + e);
   }
 }
 
