@@ -206,6 +206,8 @@ def gen(kind, accum, opts=None, gap=0):
     E = e.emit
 
     trace = bool(opts.get("trace"))
+    # Experiment (c_load_nt): C's old values, read once, loaded with the non-temporal hint.
+    c_load_hint = " nt" if opts.get("c_load_nt") else ""
 
     def stamp(pair):
         """Timing build only: the shader clock counter into s[pair:pair+1] (read after the next
@@ -521,7 +523,7 @@ def gen(kind, accum, opts=None, gap=0):
             if j < C_STEPS:
                 def ld(tn=tn, i=i, reg=reg):
                     c_ptr(j)
-                    e.vm(f"global_load_dword {reg}, {c_addr(tn, i)}, s[72:73] offset:{tn * 64}", dst=reg)
+                    e.vm(f"global_load_dword {reg}, {c_addr(tn, i)}, s[72:73] offset:{tn * 64}{c_load_hint}", dst=reg)
                 out.append(Item(ld, 1, g, GAPS - 1, after=add_item))
         return out
 
