@@ -89,6 +89,7 @@ struct GroupShare {
   uint32_t col;
   template <bool MAX>
   __device__ float combine(float v) const {
+    if constexpr (G == 1) return v;   // a thread per line: nothing to combine
     __syncthreads();  // the previous round's readers are done
     lds[first * C + col] = v;
     __syncthreads();
