@@ -634,9 +634,14 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
     };
     if ((rc = to_channels_last(img, true)) != MRL_OK) return rc;
     if ((rc = to_channels_last(filt, true)) != MRL_OK) return rc;
-    out_moved = !channels_last(out.t);
-    if ((rc = to_channels_last(out, s.accum != 0)) != MRL_OK) return rc;
-    cv.image = img.t.ptr, cv.filters = filt.t.ptr, cv.out = out.t.ptr;
+    // The fused kernel also writes planes of filters: a dense row-major (NCHW) output stays where
+    // it is (the Move back would be the largest of the three: 24 MB at the benchmark's shape).
+    cv.image = img.t.ptr, cv.filters = filt.t.ptr;
+    cv.out_planes = fused_shape && forced <= 1 && !(forced == 1 && g_forced->conv_rows) && !channels_last(out.t) &&
+                    dense_row_major(out.t) && mrl::conv_i8_applicable(cv);
+    out_moved = !channels_last(out.t) && !cv.out_planes;
+    if (!cv.out_planes && (rc = to_channels_last(out, s.accum != 0)) != MRL_OK) return rc;
+    cv.out = out.t.ptr;
   }
   // The Conv as an implicit Matmul: left operand = the image's windows, B = the KRSC filters.
   mrl::GemmArgs conv_args;
@@ -654,7 +659,7 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
     g->conv.image_bytes = uint64_t(cv.b) * h * w * c_bytes;
     return true;
   };
-  const bool fused_ok = fast_types && channels_last(img.t) && channels_last(filt.t) && channels_last(out.t) &&
+  const bool fused_ok = fast_types && channels_last(img.t) && channels_last(filt.t) && (channels_last(out.t) || cv.out_planes) &&
                         mrl::conv_i8_applicable(cv);
   const bool implicit_ok = as_matmul && !(cv.fh == 1 && cv.fw == 1) && implicit_args(&conv_args) &&
                            mrl::conv_gemm_applicable(conv_args, kind);

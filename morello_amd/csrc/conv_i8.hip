@@ -30,7 +30,7 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 constexpr int FT = 4;          // filter tiles of 16 -> F = 64
 constexpr int CONV_WAVES = 4;  // waves per workgroup: 4 measured fastest (8: 9.8 us against 9.4 at 32x64x56x56)
 
-template <int SLABS, bool IMG_UNSIGNED, int WAVES>
+template <int SLABS, bool IMG_UNSIGNED, int WAVES, bool OUT_PLANES>
 __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(const void *image, const void *filters_all, void *out_all, uint32_t c, uint32_t f,
                                                          uint32_t oh, uint32_t ow, uint32_t fh, uint32_t fw, int accum, uint32_t pixels,
                                                          uint32_t tiles) {
@@ -152,7 +152,34 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(const void *image, const
       img[s] = *(const v4i *)(src_n + slab_off[s]);
     }
     // D[row = filter 4*lg + r][col = pixel li]: lane owns 4 consecutive filters of its pixel in
-    // each filter tile, i.e. 16-byte pieces 64 bytes apart.  The tile's 16 x 64 results go through
+    // each filter tile.  An output stored as planes of filters takes them as they are: register r
+    // of the 16 lanes of a group is 16 consecutive pixels of one filter's plane, 64 contiguous
+    // bytes (a tile that crosses into the next image continues in that image's plane).
+    if constexpr (OUT_PLANES) {
+      const uint32_t pix = t * 16 + li;
+      if (pix < pixels) {
+        const uint32_t plane = p.oh * p.ow, b = pix / plane;
+        int32_t *first = (int32_t *)p.out + (int64_t(b) * p.f + blockIdx.y * (FT * 16) + lg * 4) * plane + (pix - b * plane);
+#pragma unroll
+        for (int ft = 0; ft < FT; ft++) {
+          v4i v = acc[ft];
+          if (p.accum) {   // a filter tile's four old values requested together (all sixteen: too many registers beside nine slabs of filters)
+            v4i old;
+#pragma unroll
+            for (int r = 0; r < 4; r++) old[r] = first[int64_t(ft * 16 + r) * plane];
+            v += old;
+          }
+          if (IMG_UNSIGNED) v += *(const v4i *)(corr_lds + ft * 16 + lg * 4);
+          // ordinary stores: half a cache line each, the other half comes from the neighbouring tile
+          // (non-temporal ones measured 16.1 against 11.7 us at 32 x 64 x 56 x 56)
+#pragma unroll
+          for (int r = 0; r < 4; r++) first[int64_t(ft * 16 + r) * plane] = v[r];
+        }
+      }
+      t = tn;
+      continue;
+    }
+    // Channels-last: 16-byte pieces 64 bytes apart.  The tile's 16 x 64 results go through
     // this wave's own patch of LDS so that the stores are whole 256-byte pixel rows, four
     // pixels per instruction (1 KiB contiguous when F = 64), instead of 64-byte segments.
 #pragma unroll
@@ -389,12 +416,14 @@ hipError_t launch_slabs(const ConvArgs &c, bool img_unsigned, hipStream_t stream
   plan::work(plan::UNIT_MFMA_I8, 2.0 * pixels * c.f * c.fh * c.fw * c.c,
              double(c.b) * (c.oh + c.fh - 1) * (c.ow + c.fw - 1) * c.c + double(c.f) * c.fh * c.fw * c.c +
                  4.0 * pixels * c.f * (c.accum ? 2 : 1));
-  if (img_unsigned)
-    MRL_LAUNCH((k_conv_i8<SLABS, true, WAVES>), dim3(blocks, groups), dim3(64 * WAVES), lds, stream, c.image, c.filters, c.out, c.c, c.f, c.oh, c.ow,
-               c.fh, c.fw, c.accum, uint32_t(pixels), tiles);
-  else
-    MRL_LAUNCH((k_conv_i8<SLABS, false, WAVES>), dim3(blocks, groups), dim3(64 * WAVES), lds, stream, c.image, c.filters, c.out, c.c, c.f, c.oh, c.ow,
-               c.fh, c.fw, c.accum, uint32_t(pixels), tiles);
+#define MRL_CONV_I8(U, PLANES)                                                                                                      \
+  MRL_LAUNCH((k_conv_i8<SLABS, U, WAVES, PLANES>), dim3(blocks, groups), dim3(64 * WAVES), lds, stream, c.image, c.filters, c.out, c.c, \
+             c.f, c.oh, c.ow, c.fh, c.fw, c.accum, uint32_t(pixels), tiles)
+  if (img_unsigned && c.out_planes) MRL_CONV_I8(true, true);
+  else if (img_unsigned) MRL_CONV_I8(true, false);
+  else if (c.out_planes) MRL_CONV_I8(false, true);
+  else MRL_CONV_I8(false, false);
+#undef MRL_CONV_I8
   return mrl::plan::last_error();
 }
 
@@ -414,7 +443,7 @@ bool conv_i8_applicable(const ConvArgs &c) {
 }
 
 bool conv_rows_applicable(const ConvArgs &c) {
-  return conv_i8_applicable(c) && c.c == 64 && uint64_t(c.b) * c.oh < (1u << 31) && conv_rows_plan(c).rows_per_wg > 0;
+  return conv_i8_applicable(c) && !c.out_planes && c.c == 64 && uint64_t(c.b) * c.oh < (1u << 31) && conv_rows_plan(c).rows_per_wg > 0;
 }
 
 hipError_t launch_conv_i8(const ConvArgs &c, bool img_unsigned, hipStream_t stream, bool whole_rows) {

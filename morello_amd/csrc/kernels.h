@@ -159,6 +159,10 @@ struct ConvArgs {
   void *out;
   uint32_t b, f, c, oh, ow, fh, fw;
   int accum;
+  // The output as planes of filters, [b][f][oh][ow] dense (row-major NCHW), instead of channels-last:
+  // written in place by the kernels that can (conv_i8.hip's tile-per-wave kernel), where the
+  // others write channels-last into scratch and a Move turns it.
+  bool out_planes = false;
 };
 bool conv_i8_applicable(const ConvArgs &c);
 // whole_rows: the kernel whose workgroups take whole output rows and share their pixels through LDS

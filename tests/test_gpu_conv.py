@@ -75,6 +75,24 @@ def test_conv_nchw_layout_on_the_matrix_cores(gpu, accum):
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("shape,accum", [((3, 64, 64, 9, 11, 3, 3), True), ((2, 128, 64, 13, 7, 2, 2), False),
+                                         ((5, 192, 128, 6, 6, 1, 2), True), ((1, 64, 64, 54, 54, 3, 3), False)])
+@pytest.mark.parametrize("img_dt,img_code,gen", [(M.u8, 0, synth.uniform_u8), (M.i8, 1, synth.uniform_i8)])
+def test_fused_conv_writes_a_row_major_output_in_place(gpu, shape, accum, img_dt, img_code, gen):
+    """A dense NCHW output of a shape the fused kernel takes: the kernel writes the planes of
+    filters itself (16 consecutive pixels of a plane per lane group, tiles that cross from one
+    image into the next included), no Move of the output remains in the plan; bit for bit, with
+    old values when accumulating and a sentinel otherwise."""
+    b, f, c, oh, ow, fh, fw = shape
+    img = gen(113, 0, (b, oh + fh - 1, ow + fw - 1, c))
+    filt = synth.uniform_i8(113, 1, (f, fh, fw, c))
+    out0 = (synth.uniform_i8(113, 2, (b, f, oh, ow)).astype(np.int32) * 999) if accum else np.full((b, f, oh, ow), -5, np.int32)
+    spec = M.Conv(list(shape), (img_dt, M.i8, M.i32), layouts=[None, None, M.row_major([b, f, oh, ow])], accum=accum)
+    assert spec.plan().kernels == ["k_conv_i8"]
+    want = orc.conv(list(shape), [img_code, 1, 5], img, filt, out0.copy(), accum, layouts=[NHWC, NHWC, None])
+    assert np.array_equal(run_spec(spec, [img, filt, out0.copy()]), want)
+
+
 CONV_GEN = {M.u8: synth.uniform_u8, M.i8: synth.uniform_i8, M.bf16: synth.normal_bf16, M.f32: synth.uniform_f32}
 
 
