@@ -632,13 +632,22 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
       p.t = dense;
       return MRL_OK;
     };
-    if ((rc = to_channels_last(img, true)) != MRL_OK) return rc;
     if ((rc = to_channels_last(filt, true)) != MRL_OK) return rc;
-    // The fused kernel also writes planes of filters: a dense row-major (NCHW) output stays where
-    // it is (the Move back would be the largest of the three: 24 MB at the benchmark's shape).
-    cv.image = img.t.ptr, cv.filters = filt.t.ptr;
-    cv.out_planes = fused_shape && forced <= 1 && !(forced == 1 && g_forced->conv_rows) && !channels_last(out.t) &&
-                    dense_row_major(out.t) && mrl::conv_i8_applicable(cv);
+    cv.filters = filt.t.ptr;
+    // Two kernels take dense row-major (NCHW) tensors as they are, and those stay where they are:
+    // the fused kernel writes planes of filters (the Move back would be the largest of the three:
+    // 24 MB at the benchmark's shape), the kernel that forms windows in LDS also reads planes of
+    // channels.
+    const bool plain_choice = forced <= 1 && !(forced == 1 && g_forced->conv_rows);
+    const bool img_planes = !channels_last(img.t) && dense_row_major(img.t), out_planes = !channels_last(out.t) && dense_row_major(out.t);
+    if (plain_choice && !fused_shape && kind >= 0 && kind <= 3 && as_matmul && channels_last(filt.t) && (img_planes || out_planes)) {
+      mrl::ConvArgs as_is = cv;
+      as_is.in_planes = img_planes, as_is.out_planes = out_planes;
+      if (mrl::conv_windows_applicable(as_is, kind)) cv = as_is;
+    }
+    if (!cv.in_planes && (rc = to_channels_last(img, true)) != MRL_OK) return rc;
+    cv.image = img.t.ptr;
+    if (fused_shape && plain_choice && out_planes && mrl::conv_i8_applicable(cv)) cv.out_planes = true;
     out_moved = !channels_last(out.t) && !cv.out_planes;
     if (!cv.out_planes && (rc = to_channels_last(out, s.accum != 0)) != MRL_OK) return rc;
     cv.out = out.t.ptr;
@@ -666,8 +675,9 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
   const bool unfold_ok = as_matmul && can_unfold && (reinterpret_cast<uintptr_t>(img.t.ptr) & 15) == 0 &&
                          (reinterpret_cast<uintptr_t>(filt.t.ptr) & 15) == 0 && (reinterpret_cast<uintptr_t>(out.t.ptr) & 3) == 0;
   // Few channels per pixel (a first layer): the fused kernel that forms the windows in LDS.
-  const bool windows_ok = kind >= 0 && kind <= 3 && as_matmul && channels_last(img.t) && channels_last(filt.t) && channels_last(out.t) &&
-                          mrl::conv_windows_applicable(cv, kind) && !(forced == 1 && g_forced->conv_rows);
+  const bool windows_ok = kind >= 0 && kind <= 3 && as_matmul && (channels_last(img.t) || cv.in_planes) && channels_last(filt.t) &&
+                          (channels_last(out.t) || cv.out_planes) && mrl::conv_windows_applicable(cv, kind) &&
+                          !(forced == 1 && g_forced->conv_rows);
   // Short windows over pixels of whole chunks and few filters (early layers of 16 or 32 channels):
   // the filters stay in registers and the pixels come straight from memory.  Measured against
   // the implicit Matmul, whose 64-wide tiles are then mostly padding (us, this kernel / implicit):

@@ -44,6 +44,11 @@ struct WindowsArgs {
   uint32_t tiles_x, tiles_y, tiles;   // per image, per image, in all
   uint32_t seg, seg_padded;           // fw * c: bytes of one run of a window; the same in whole dwords
   uint32_t patch_stride;              // bytes between the patch's rows in LDS (whole dwords)
+  // The image / the output as planes ([b][c][h][w], [b][f][oh][ow]: dense NCHW) instead of channels-last.
+  // A patch's bytes are fetched one by one either way, so planes only change where a byte comes
+  // from; the accumulators hold 16 consecutive pixels of a filter per register and lane group,
+  // 64 contiguous bytes of that filter's plane, and are stored as they are.
+  int in_planes, out_planes;
 };
 
 // KS: MFMA k steps per window (fh * seg_padded bytes, padded to 64 KS).
@@ -96,8 +101,13 @@ __global__ __launch_bounds__(256) void k_conv_windows(WindowsArgs p) {
     const uint32_t per_image = p.tiles_x * p.tiles_y, img = t / per_image, in_img = t - img * per_image, ty = in_img / p.tiles_x;
     return Corner{img, ty * TILE_H, (in_img - ty * p.tiles_x) * TILE_W};
   };
+  constexpr uint32_t ES = KIND == IMG_F32 ? 4 : KIND == IMG_BF16 ? 2 : 1;   // bytes of an element
   auto patch_source = [&](const Corner &at, uint32_t r, uint32_t xb) {
     const uint32_t y = min(at.y0 + r, h - 1), x = min(at.x0 * p.c + xb, w * p.c - 1);
+    if (p.in_planes) {
+      const uint32_t pixel = x / p.c, in_pixel = x - pixel * p.c, channel = in_pixel / ES;
+      return p.image + ((uint64_t(at.img) * (p.c / ES) + channel) * h + y) * w * ES + pixel * ES + (in_pixel - channel * ES);
+    }
     return p.image + (uint64_t(at.img) * h + y) * w * p.c + x;
   };
   auto fetch_patch = [&](uint32_t t) {
@@ -228,6 +238,31 @@ __global__ __launch_bounds__(256) void k_conv_windows(WindowsArgs p) {
     // 64 bytes apart.  A pixel block's 16 x 64 results go through the wave's own window rows (no
     // other wave reads them, and this wave is done with them) and leave as whole rows: four pixels
     // per store instruction, 1 KiB contiguous when the Spec has 64 filters.
+    if (p.out_planes) {
+#pragma unroll
+      for (int pb = 0; pb < 2; pb++) {
+        const uint32_t y = y0 + 2 * wave + pb, x = x0 + li;
+        if (y < p.oh && x < p.ow) {
+          const uint64_t plane = uint64_t(p.oh) * p.ow;
+          typedef typename std::conditional<FLOATS, float, int32_t>::type Out;
+          Out *first = (Out *)p.out + (uint64_t(img) * p.f + f0 + 4 * lg) * plane + uint64_t(y) * p.ow + x;
+#pragma unroll
+          for (int fb = 0; fb < 4; fb++)
+            if (fb < nfb) {
+              Acc v = acc[pb][fb];
+              if (p.accum) {
+                Acc old;
+#pragma unroll
+                for (int r = 0; r < 4; r++) old[r] = first[(16 * fb + r) * plane];
+                v += old;
+              }
+#pragma unroll
+              for (int r = 0; r < 4; r++) first[(16 * fb + r) * plane] = v[r];
+            }
+        }
+      }
+      continue;
+    }
     uint8_t *xb = rows + (2 * wave) * 16 * ROW;
     constexpr int XROW = 272;
 #pragma unroll
@@ -279,6 +314,8 @@ constexpr uint32_t MAX_KS_F32 = 10;  // f32: up to 640 bytes (3 channels, 7 x 7:
 // not whole 16-byte chunks (those conv_gemm.hip reads in place), windows of at most 64 MAX_KS
 // bytes with their runs padded to dwords.
 bool conv_windows_applicable(const ConvArgs &c, int kind) {
+  // (The same for an image or an output stored as planes: only the alignment of the output's 16-byte
+  // stores does not apply to planes, which are written a dword at a time.)
   if (kind < 0 || kind > 3) return false;
   const uint64_t es = kind == 3 ? 4 : kind == 2 ? 2 : 1, c_bytes = c.c * es, seg_padded = (uint64_t(c.fw) * c_bytes + 3) & ~3ull;
   // Pixels that are not whole 16-byte chunks (the implicit Matmul cannot read those in place), and
@@ -293,7 +330,7 @@ bool conv_windows_applicable(const ConvArgs &c, int kind) {
 #endif
   return c.f % 16 == 0 && c.f / 64 < 65535 && c_ok && uint64_t(c.fh) * seg_padded <= 64 * (kind == 3 ? MAX_KS_F32 : MAX_KS) &&
          uint64_t(c.b) * ((c.oh + TILE_H - 1) / TILE_H) * ((c.ow + TILE_W - 1) / TILE_W) < (1ull << 31) &&
-         (reinterpret_cast<uintptr_t>(c.out) & 15) == 0 && (reinterpret_cast<uintptr_t>(c.image) & (es - 1)) == 0 &&
+         (reinterpret_cast<uintptr_t>(c.out) & (c.out_planes ? 3 : 15)) == 0 && (reinterpret_cast<uintptr_t>(c.image) & (es - 1)) == 0 &&
          (reinterpret_cast<uintptr_t>(c.filters) & (es - 1)) == 0;
 }
 
@@ -306,6 +343,7 @@ hipError_t launch_conv_windows(const ConvArgs &c, int kind, hipStream_t stream) 
   p.tiles_x = (c.ow + TILE_W - 1) / TILE_W, p.tiles_y = (c.oh + TILE_H - 1) / TILE_H, p.tiles = c.b * p.tiles_x * p.tiles_y;
   p.seg = c.fw * p.c, p.seg_padded = (p.seg + 3) & ~3u;
   p.patch_stride = ((TILE_W + c.fw - 1) * p.c + 3) & ~3u;
+  p.in_planes = c.in_planes, p.out_planes = c.out_planes;
   const int ks = int((c.fh * p.seg_padded + 63) / 64);
   const size_t row = ks == 1 ? 144 : 64 * ks + 16;
   // the copies read one dword past a run's last: four bytes behind the patch

@@ -163,6 +163,8 @@ struct ConvArgs {
   // written in place by the kernels that can (conv_i8.hip's tile-per-wave kernel), where the
   // others write channels-last into scratch and a Move turns it.
   bool out_planes = false;
+  // The image as planes of channels, [b][c][h][w] dense (conv_windows.hip fetches its patches from either).
+  bool in_planes = false;
 };
 bool conv_i8_applicable(const ConvArgs &c);
 // whole_rows: the kernel whose workgroups take whole output rows and share their pixels through LDS

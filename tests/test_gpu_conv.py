@@ -93,6 +93,42 @@ def test_fused_conv_writes_a_row_major_output_in_place(gpu, shape, accum, img_dt
     assert np.array_equal(run_spec(spec, [img, filt, out0.copy()]), want)
 
 
+@pytest.mark.parametrize("dts,codes", [((M.u8, M.i8, M.i32), [0, 1, 5]), ((M.i8, M.i8, M.i32), [1, 1, 5]),
+                                        ((M.bf16, M.bf16, M.f32), [7, 7, 6]), ((M.f32, M.f32, M.f32), [6, 6, 6])])
+@pytest.mark.parametrize("shape,accum", [((2, 64, 3, 20, 37, 5, 5), False), ((3, 32, 3, 9, 50, 3, 3), True),
+                                         ((2, 80, 5, 17, 15, 2, 3), True), ((1, 16, 1, 33, 33, 3, 3), False)])
+@pytest.mark.parametrize("which", ["all", "image", "output"])
+def test_first_layer_conv_on_row_major_tensors(gpu, dts, codes, shape, accum, which):
+    """A first layer on NCHW tensors: the kernel that forms its windows in LDS fetches a patch's
+    bytes from planes of channels as well as from channels-last pixels, and writes planes of
+    filters from its accumulators; only the (small) filters are moved.  All three tensors
+    row-major, or the image alone, or the output alone."""
+    b, f, c, oh, ow, fh, fw = shape
+    gen = {M.u8: synth.uniform_u8, M.i8: synth.uniform_i8, M.bf16: synth.normal_bf16, M.f32: synth.normal_f32}
+    img = gen[dts[0]](114, 0, (b, c, oh + fh - 1, ow + fw - 1))
+    filt = gen[dts[1]](114, 1, (f, c, fh, fw))
+    floats = dts[2] == M.f32
+    out0 = synth.uniform_u8(114, 2, (b, f, oh, ow)).astype(np.float32 if floats else np.int32) - 90
+    want = orc.conv(list(shape), codes, img, filt, out0.copy(), accum)     # everything row-major
+    spec0 = M.Conv(list(shape), dts)
+    rm = [M.row_major(s) for s in spec0.parameter_shapes()]
+    cl = lambda a: np.ascontiguousarray(a.transpose(0, 2, 3, 1))
+    if which == "all":
+        layouts, bufs, back = rm, [img, filt, out0.copy()], lambda a: a
+    elif which == "image":
+        layouts, bufs, back = [rm[0], None, None], [img, cl(filt), cl(out0)], lambda a: a.transpose(0, 3, 1, 2)
+    else:
+        layouts, bufs, back = [None, None, rm[2]], [cl(img), cl(filt), out0.copy()], lambda a: a
+    spec = M.Conv(list(shape), dts, layouts=layouts, accum=accum)
+    # (filters of one channel are channels-last as they stand)
+    assert spec.plan().kernels == (["k_move_rows", "k_conv_windows"] if which == "all" and c > 1 else ["k_conv_windows"]), spec.plan()
+    got = back(run_spec(spec, bufs))
+    if floats:
+        assert float(np.abs(got.astype(np.float64) - want).max() / np.abs(want).max()) < 1e-5
+    else:
+        assert np.array_equal(got, want)
+
+
 CONV_GEN = {M.u8: synth.uniform_u8, M.i8: synth.uniform_i8, M.bf16: synth.normal_bf16, M.f32: synth.uniform_f32}
 
 
