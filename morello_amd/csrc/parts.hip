@@ -353,6 +353,13 @@ __global__ __launch_bounds__(256) void k_parts_rows(PartsArgs p) {
       store(VEC(0));
       break;
     }
+    case MRL_SPEC_DIVIDE_VEC: {   // the denominators' line vector by vector beside the numerators'
+      const f4 *den = VEC(1);
+#pragma unroll
+      EACH(i, idx) v[i] = v[i] / den[idx];
+      store(VEC(0));
+      break;
+    }
     default:
       break;
   }
@@ -428,8 +435,7 @@ hipError_t launch_parts(const PartsArgs &p, hipStream_t stream) {
   if (p.lines == 0) return hipSuccess;
   const uint32_t n = p.shape[p.scan_dim];
   // Contiguous lines in whole, aligned 16-byte vectors: the register-resident form.
-  bool rows = n % 4 == 0 && n > 1 && n <= 4096 && p.kind != MRL_SPEC_DIVIDE_VEC &&
-              p.kind != MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX_FROM_PARTS && full_size(p, 0);
+  bool rows = n % 4 == 0 && n > 1 && n <= 4096 && p.kind != MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX_FROM_PARTS && full_size(p, 0);
   // Lines side by side: the dim along which consecutive lines differ (the last one that is not
   // the scan dim) is contiguous in the full-size parameters, as the innermost dim of a row-major
   // tensor scanned along another dim is, or dim 0 of a column-major matrix scanned along dim 1.

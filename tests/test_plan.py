@@ -362,7 +362,7 @@ def test_plans_of_the_softmax_primitives():
     assert kernel(M.Max([16, 2048, 2048], 2)) == ("k_parts_rows", (8192, 1))
     assert kernel(M.SoftmaxComplete([7, 12], 1))[0] == "k_parts_rows"
     assert kernel(M.Max([3, 4100], 1))[0] == "k_parts" and kernel(M.Max([7, 33], 1))[0] == "k_parts"
-    assert kernel(M.DivideVec([64, 64]))[0] == "k_parts"
+    assert kernel(M.DivideVec([64, 64]))[0] == "k_parts_rows" and kernel(M.DivideVec([64, 66]))[0] == "k_parts"
     assert kernel(M.SoftmaxDenominatorAndMax([2048, 4096], 0)) == ("k_parts_cols", (256, 1))     # 16 lines each
     assert kernel(M.SoftmaxDenominatorAndMax([40, 20000], 0)) == ("k_parts_cols", (625, 1))      # 32
     assert kernel(M.SoftmaxDenominatorAndMax([40, 40000], 0)) == ("k_parts_cols", (625, 1))      # 64
