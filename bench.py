@@ -465,32 +465,48 @@ def cycle_stamps(launches):
     return out
 
 
-def measure(name, steps, warmup, min_gpu_s, action=None):
+def measure(name, steps, warmup, min_gpu_s, action=None, buffer_sets=1):
     """W warm-up launches, then bursts of `steps` launches until there are MIN_REPEATS of them and
     min_gpu_s seconds of GPU time; -> the workload and the figures of the fastest and the last burst.
     action: index into the Spec's list of lowerings (mrl_target_actions) to time instead of the
-    dispatch rules' own choice."""
+    dispatch rules' own choice.
+    buffer_sets: with N > 1 the operands exist N times and the launches of a burst take the sets in
+    turn, so that a launch finds none of its input in the 256 MB memory-side cache from the launch
+    before (choose N so that N - 1 sets exceed that cache); such bursts are timed on the host clock
+    only, between two synchronisations."""
     desc, spec, arrs, dtype, unit, bound, peak = workload(name)
     runner = spec
     if action is not None:
         runner = spec.actions()[action]
         desc += f" [action {action}: {runner!r}]"
-    bufs = [M.DeviceBuffer.from_numpy(a) for a in arrs]
-    ptrs = [b.ptr for b in bufs]
+    sets = [[M.DeviceBuffer.from_numpy(a) for a in arrs] for _ in range(buffer_sets)]
+    ptrs = [b.ptr for b in sets[0]]
     ops = spec.flops()
     alg_bytes = sum(spec.bytes_used(i) for i in range(len(arrs)))
-    for _ in range(warmup):
-        runner.run_device(ptrs)
+    for i in range(warmup):
+        runner.run_device([b.ptr for b in sets[i % buffer_sets]])
     M.synchronize()
     bursts, gpu_ms = [], 0.0
+    stream = M.Stream() if buffer_sets > 1 else None
     while len(bursts) < MIN_REPEATS or (gpu_ms < min_gpu_s * 1e3 and len(bursts) < 5000):
         t0 = time.perf_counter()
-        device_ms = runner.run_timed(ptrs, steps)  # enqueues K launches between two events, waits for the last
-        M.synchronize()
-        bursts.append((device_ms / steps, (time.perf_counter() - t0) * 1e3 / steps))
+        if stream is None:
+            device_ms = runner.run_timed(ptrs, steps)  # enqueues K launches between two events, waits for the last
+            M.synchronize()
+            host_ms = (time.perf_counter() - t0) * 1e3
+        else:
+            for i in range(steps):
+                spec.run_async([b.ptr for b in sets[i % buffer_sets]], stream)
+            stream.synchronize()
+            device_ms = host_ms = (time.perf_counter() - t0) * 1e3
+        bursts.append((device_ms / steps, host_ms / steps))
         gpu_ms += device_ms
-    for b in bufs:
-        b.free()
+    if stream is not None:
+        stream.destroy()
+        desc += f" [{buffer_sets} sets of operands in rotation, host clock]"
+    for bufs in sets:
+        for b in bufs:
+            b.free()
     kernel_ms_min = min(k for k, _ in bursts)
     kernel_ms, ms_per_step = bursts[-1]
     value = ops / (ms_per_step * 1e-3) / 1e12
@@ -538,6 +554,9 @@ def main():
                     help="time the K-th lowering the library lists for the workload's Spec (mrl_target_actions) "
                          "instead of the dispatch rules' own choice; implies --no-configs")
     ap.add_argument("--no-configs", action="store_true", help="headline workload only: skip the `configs` object")
+    ap.add_argument("--buffer-sets", type=int, default=1, metavar="N",
+                    help="keep N copies of the operands and launch on them in turn, so that no launch finds its input "
+                         "left in the memory-side cache by the one before (timed on the host clock; implies --no-configs)")
     ap.add_argument("--vendor-ref", action="store_true",
                     help="also time the vendor library's nearest operation through PyTorch (c2, c3, c5)")
     ap.add_argument("--vendor-child", action="store_true", help=argparse.SUPPRESS)
@@ -567,7 +586,9 @@ def main():
     if args.cycle_stamps > 0:
         print(json.dumps(cycle_stamps_attention(args.cycle_stamps) if args.spec == "c5" else cycle_stamps(args.cycle_stamps)))
         return
-    head = measure(args.spec, args.steps, args.warmup, min_gpu_s=0.2, action=args.action)
+    if args.buffer_sets < 1 or (args.buffer_sets > 1 and args.action is not None):
+        raise SystemExit("--buffer-sets takes N >= 1 and times the dispatch rules' own choice (no --action)")
+    head = measure(args.spec, args.steps, args.warmup, min_gpu_s=0.2, action=args.action, buffer_sets=args.buffer_sets)
     desc, spec, arrs, dtype, unit = head["desc"], head["spec"], head["arrs"], head["dtype"], head["unit"]
     value, ms_per_step, roofline = head["value"], head["ms_per_step"], head["roofline"]
 
@@ -585,7 +606,7 @@ def main():
     plan = spec.plan() if args.action is None else spec.actions()[args.action].plan()
     out["plan"] = {"kernels": [s.kernel for s in plan.steps], "predicted_ms": plan.cost_ns * 1e-6,
                    "scratch_bytes": plan.scratch_bytes}
-    if args.spec == "c2" and not args.no_configs and args.action is None:
+    if args.spec == "c2" and not args.no_configs and args.action is None and args.buffer_sets == 1:
         # The other benchmark configurations, each by the same protocol (a quarter of the GPU time).
         out["configs"] = {}
         for name in ("c1", "c3", "c4", "c5"):
