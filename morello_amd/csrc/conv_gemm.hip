@@ -30,9 +30,13 @@ bool conv_gemm_applicable(const GemmArgs &g, int kind) {
          uint64_t((g.m + 63) / 64) * ((g.n + 63) / 64) < (1u << 30);
 }
 
-hipError_t launch_conv_gemm(const GemmArgs &g, int kind, hipStream_t stream, uint32_t tile) {
-  if (!conv_gemm_applicable(g, kind) || (tile != 0 && tile != 64 && tile != 128 && tile != 256)) return hipErrorInvalidValue;
-  if (tile == 0) tile = gemm_tile_side(g, kind);
+hipError_t launch_conv_gemm(const GemmArgs &args, int kind, hipStream_t stream, uint32_t tile) {
+  if (!conv_gemm_applicable(args, kind) || (tile != 0 && tile != 64 && tile != 128 && tile != 256)) return hipErrorInvalidValue;
+  if (tile == 0) tile = gemm_tile_side(args, kind);
+  // Pixel numbers and window bytes stay below 2^31 (conv_gemm_applicable), as FastDiv asks.
+  GemmArgs g = args;
+  g.conv.by_ow = FastDiv(g.conv.ow), g.conv.by_oh = FastDiv(g.conv.oh);
+  g.conv.by_c_bytes = FastDiv(g.conv.c_bytes), g.conv.by_fw = FastDiv(g.conv.fw);
   switch (kind) {
     case 0: return launch_for<I8, false>(g, tile, stream);
     case 1: return launch_for<I8, true>(g, tile, stream);

@@ -381,7 +381,7 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
     for (int i = 0; i < A_CH; i++) {
       const int64_t p = m0 + tid / A_ROW_CH + i * A_ROWS_PER_I;
       const uint32_t q = uint32_t(min(p, int64_t(g.m) - 1));
-      const uint32_t x = q % g.conv.ow, y = (q / g.conv.ow) % g.conv.oh, img = q / (g.conv.ow * g.conv.oh);
+      const uint32_t row = g.conv.by_ow.div(q), x = q - row * g.conv.ow, img = g.conv.by_oh.div(row), y = row - img * g.conv.oh;
       a_corner[i] = p < int64_t(g.m) ? ((img * g.conv.h + y) * g.conv.w + x) * g.conv.c_bytes : OUT_OF_RANGE;
     }
   }
@@ -396,7 +396,7 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
       const bool a_in = ld_kb + a_kb0 < k_bytes;
       if constexpr (CONV) {
         const auto a_buf = buffer_of(g.a, int64_t(g.conv.image_bytes));
-        const uint32_t kb = blockIdx.y * g.conv.slice_bytes + uint32_t(ld_kb + a_kb0), pos = kb / g.conv.c_bytes, r = pos / g.conv.fw;
+        const uint32_t kb = blockIdx.y * g.conv.slice_bytes + uint32_t(ld_kb + a_kb0), pos = g.conv.by_c_bytes.div(kb), r = g.conv.by_fw.div(pos);
         const uint32_t in_window = ((r * g.conv.w + (pos - r * g.conv.fw)) * g.conv.c_bytes) + (kb - pos * g.conv.c_bytes);
 #pragma unroll
         for (int i = 0; i < A_CH; i++)

@@ -91,6 +91,23 @@ hipError_t launch_widen_bf16(const void *src, void *dst, uint64_t count, hipStre
 // Move Spec fast path: same bytes on both sides (16-byte aligned buffers).
 hipError_t launch_copy(const void *src, void *dst, uint64_t bytes, hipStream_t stream);
 
+// Division of a number below 2^31 by a divisor fixed at launch: with s = ceil(log2 d) and
+// mul = floor(2^(31+s) / d) + 1, n / d = (n * mul) >> (31 + s) exactly (the error term
+// n * (mul * d - 2^(31+s)) stays below 2^(31+s) because n < 2^31 and mul * d - 2^(31+s) <= d <= 2^s).
+// A multiply-high, a multiply-low and a shift where the hardware's division takes some thirty
+// instructions.
+struct FastDiv {
+  uint32_t mul = 0, shift = 0;
+  FastDiv() = default;
+  explicit FastDiv(uint32_t d) {
+    uint32_t s = 0;
+    while ((1ull << s) < d) s++;
+    mul = uint32_t((1ull << (31 + s)) / d + 1);
+    shift = 31 + s;
+  }
+  __host__ __device__ uint32_t div(uint32_t n) const { return uint32_t((uint64_t(n) * mul) >> shift); }
+};
+
 // ---- gemm_mfma.hip / gemm_nt.hip: Matmul on the matrix cores (kernel: gemm_mfma_kernel.h) ----
 // A and C row-major, B row-major or k-fastest; leading dimensions and batch strides in elements.
 struct GemmArgs {
@@ -114,6 +131,8 @@ struct GemmArgs {
     // K shared out over batch entries (each a slice of the windows, a partial result of its own):
     // bytes of a window a slice starts behind the previous one; 0 = one entry, the whole window.
     uint32_t slice_bytes;
+    // Filled in by launch_conv_gemm: the divisions of the window arithmetic.
+    FastDiv by_ow, by_oh, by_c_bytes, by_fw;
   } conv = {};
 };
 // kind: 0 = i8 x i8, 1 = u8 x i8, 2 = bf16 x bf16, 3 = f32 x f32; B stored k-fastest (gemm_nt.hip).
