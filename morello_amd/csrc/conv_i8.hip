@@ -32,16 +32,25 @@ constexpr int CONV_WAVES = 4;  // waves per workgroup: 4 measured fastest (8: 9.
 
 template <int SLABS, bool IMG_UNSIGNED, int WAVES, bool OUT_PLANES>
 __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(const void *image, const void *filters_all, void *out_all, uint32_t c, uint32_t f,
-                                                         uint32_t oh, uint32_t ow, uint32_t fh, uint32_t fw, int accum, uint32_t pixels,
-                                                         uint32_t tiles) {
+                                                         uint32_t oh, uint32_t ow, uint32_t fh_fw_accum, uint32_t pixels,
+                                                         uint32_t ow_mul, uint32_t oh_mul, uint32_t shifts) {
   // Scalar arguments, fifteen dwords: few enough to arrive preloaded in SGPRs with the wave
-  // instead of through a load the first instructions would wait for.
+  // instead of through a load the first instructions would wait for.  (fh, fw, accum share a
+  // dword, a byte each; the two divisions' shifts another.)
   struct {
     const void *image, *filters;
     void *out;
     uint32_t c, f, oh, ow, fh, fw;
     int accum;
-  } const p = {image, filters_all, out_all, c, f, oh, ow, fh, fw, accum};
+  } const p = {image, filters_all, out_all, c, f, oh, ow, fh_fw_accum & 255, (fh_fw_accum >> 8) & 255, int(fh_fw_accum >> 16)};
+  const uint32_t tiles = (pixels + 15) / 16;
+  // pixel number -> (image, row, column) by multiply-and-shift (FastDiv: exact below 2^31)
+  FastDiv by_ow, by_oh;
+  by_ow.mul = ow_mul, by_ow.shift = shifts & 255, by_oh.mul = oh_mul, by_oh.shift = shifts >> 8;
+  auto corner = [&](uint32_t pix) {
+    const uint32_t row = by_ow.div(pix), b = by_oh.div(row);
+    return (int64_t(b) * (p.oh + p.fh - 1) + (row - b * p.oh)) * (p.ow + p.fw - 1) + (pix - row * p.ow);
+  };
   // The filter bank, staged once per workgroup: rows of krow bytes, 16-byte chunks.
   extern __shared__ __attribute__((aligned(16))) uint8_t filt_lds[];
   const int lane = threadIdx.x & 63;
@@ -49,7 +58,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(const void *image, const
   const uint32_t wave = blockIdx.x * WAVES + (threadIdx.x >> 6);
   const uint32_t nwaves = gridDim.x * WAVES;
   const int li = lane & 15, lg = lane >> 4;
-  const int H = p.oh + p.fh - 1, W = p.ow + p.fw - 1;
+  const int W = p.ow + p.fw - 1;
   const int sub = p.c / 64;  // 64-channel slabs per filter position
   const int krow = p.fh * p.fw * p.c;  // bytes per filter
   // blockIdx.y: which group of 64 filters (= 64 output channels) this workgroup computes.
@@ -69,19 +78,25 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(const void *image, const
   }
 
   // Byte offset of each slab's source relative to the pixel's own (y, x) position.
+  // (Slab s is channels 64 * (s % sub) .. of filter position s / sub; counted up rather than divided.)
   int slab_off[SLABS];
+  {
+    int r = 0, q = 0, cs = 0;
 #pragma unroll
-  for (int s = 0; s < SLABS; s++) {
-    const int pos = s / sub, r = pos / p.fw, q = pos % p.fw;
-    slab_off[s] = (r * W + q) * p.c + (s % sub) * 64 + lg * 16;
+    for (int s = 0; s < SLABS; s++) {
+      slab_off[s] = (r * W + q) * p.c + cs * 64 + lg * 16;
+      if (++cs == sub) {
+        cs = 0;
+        if (++q == int(p.fw)) q = 0, r++;
+      }
+    }
   }
   // Pixel operand of one tile: lane (li, lg) holds pixel t*16+li, channels 16*lg .. +15 of
   // every slab.  Out-of-range pixels of the last tile are clamped for the loads and masked
   // for the store.
   auto load_tile = [&](uint32_t t, v4i *img) {
     uint32_t pix = min(t * 16 + li, pixels - 1);
-    const uint32_t x = pix % p.ow, y = (pix / p.ow) % p.oh, b = pix / (p.ow * p.oh);
-    const uint8_t *src = (const uint8_t *)p.image + (int64_t(b) * H * W + int64_t(y) * W + x) * p.c;
+    const uint8_t *src = (const uint8_t *)p.image + corner(pix) * p.c;
 #pragma unroll
     for (int s = 0; s < SLABS; s++) img[s] = *(const v4i *)(src + slab_off[s]);
   };
@@ -137,8 +152,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(const void *image, const
   while (t < tiles) {
     const uint32_t tn = t + nwaves;
     const uint32_t pix_n = min(min(tn, tiles - 1) * 16 + li, pixels - 1);  // clamped: always loadable
-    const uint32_t xn = pix_n % p.ow, yn = (pix_n / p.ow) % p.oh, bn = pix_n / (p.ow * p.oh);
-    const uint8_t *src_n = (const uint8_t *)p.image + (int64_t(bn) * H * W + int64_t(yn) * W + xn) * p.c;
+    const uint8_t *src_n = (const uint8_t *)p.image + corner(pix_n) * p.c;
     v4i acc[FT];
 #pragma unroll
     for (int ft = 0; ft < FT; ft++) acc[ft] = v4i{0, 0, 0, 0};
@@ -158,7 +172,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(const void *image, const
     if constexpr (OUT_PLANES) {
       const uint32_t pix = t * 16 + li;
       if (pix < pixels) {
-        const uint32_t plane = p.oh * p.ow, b = pix / plane;
+        const uint32_t plane = p.oh * p.ow, b = by_oh.div(by_ow.div(pix));
         int32_t *first = (int32_t *)p.out + (int64_t(b) * p.f + blockIdx.y * (FT * 16) + lg * 4) * plane + (pix - b * plane);
 #pragma unroll
         for (int ft = 0; ft < FT; ft++) {
@@ -416,9 +430,11 @@ hipError_t launch_slabs(const ConvArgs &c, bool img_unsigned, hipStream_t stream
   plan::work(plan::UNIT_MFMA_I8, 2.0 * pixels * c.f * c.fh * c.fw * c.c,
              double(c.b) * (c.oh + c.fh - 1) * (c.ow + c.fw - 1) * c.c + double(c.f) * c.fh * c.fw * c.c +
                  4.0 * pixels * c.f * (c.accum ? 2 : 1));
+  const FastDiv by_ow(c.ow), by_oh(c.oh);
 #define MRL_CONV_I8(U, PLANES)                                                                                                      \
   MRL_LAUNCH((k_conv_i8<SLABS, U, WAVES, PLANES>), dim3(blocks, groups), dim3(64 * WAVES), lds, stream, c.image, c.filters, c.out, c.c, \
-             c.f, c.oh, c.ow, c.fh, c.fw, c.accum, uint32_t(pixels), tiles)
+             c.f, c.oh, c.ow, c.fh | c.fw << 8 | uint32_t(c.accum != 0) << 16, uint32_t(pixels), by_ow.mul, by_oh.mul,                     \
+             by_ow.shift | by_oh.shift << 8)
   if (img_unsigned && c.out_planes) MRL_CONV_I8(true, true);
   else if (img_unsigned) MRL_CONV_I8(true, false);
   else if (c.out_planes) MRL_CONV_I8(false, true);
