@@ -31,32 +31,34 @@ constexpr int FT = 4;          // filter tiles of 16 -> F = 64
 constexpr int CONV_WAVES = 4;  // waves per workgroup: 4 measured fastest (8: 9.8 us against 9.4 at 32x64x56x56)
 
 template <int SLABS, bool IMG_UNSIGNED, int WAVES, bool OUT_PLANES>
-__global__ __launch_bounds__(64 * WAVES) void k_conv_i8(const void *image, const void *filters_all, void *out_all, uint32_t c, uint32_t f,
-                                                         uint32_t oh, uint32_t ow, uint32_t fh_fw_accum, uint32_t pixels,
-                                                         uint32_t ow_mul, uint32_t oh_mul, uint32_t shifts) {
-  // Scalar arguments, fifteen dwords: few enough to arrive preloaded in SGPRs with the wave
-  // instead of through a load the first instructions would wait for.  (fh, fw, accum share a
-  // dword, a byte each; the two divisions' shifts another.)
+__global__ __launch_bounds__(64 * WAVES) void k_conv_i8(const void *image, const void *filters_all, void *out_all, uint32_t f, uint32_t oh,
+                                                         uint32_t ow, uint32_t packed, uint32_t pixels, uint32_t ow_mul, uint32_t oh_mul,
+                                                         uint32_t nwaves) {
+  // Scalar arguments, fourteen dwords: what arrives preloaded in SGPRs with the wave instead of
+  // through a load the first instructions would wait for (the waves of the whole grid included,
+  // which the launch would otherwise leave behind the explicit arguments).  `packed`: fh, fw in
+  // four bits each, accum in bit 8, the 64-channel slabs of a pixel from bit 9, the two divisions'
+  // shifts in bits 16-21 and 24-29.
   struct {
     const void *image, *filters;
     void *out;
     uint32_t c, f, oh, ow, fh, fw;
     int accum;
-  } const p = {image, filters_all, out_all, c, f, oh, ow, fh_fw_accum & 255, (fh_fw_accum >> 8) & 255, int(fh_fw_accum >> 16)};
+  } const p = {image, filters_all, out_all, ((packed >> 9) & 15) * 64, f, oh, ow, packed & 15, (packed >> 4) & 15, int((packed >> 8) & 1)};
   const uint32_t tiles = (pixels + 15) / 16;
   // pixel number -> (image, row, column) by multiply-and-shift (FastDiv: exact below 2^31)
   FastDiv by_ow, by_oh;
-  by_ow.mul = ow_mul, by_ow.shift = shifts & 255, by_oh.mul = oh_mul, by_oh.shift = shifts >> 8;
+  by_ow.mul = ow_mul, by_ow.shift = (packed >> 16) & 63, by_oh.mul = oh_mul, by_oh.shift = (packed >> 24) & 63;
+  // (byte offset of the pixel's window corner in the image: below 2^31, conv_i8_applicable)
   auto corner = [&](uint32_t pix) {
     const uint32_t row = by_ow.div(pix), b = by_oh.div(row);
-    return (int64_t(b) * (p.oh + p.fh - 1) + (row - b * p.oh)) * (p.ow + p.fw - 1) + (pix - row * p.ow);
+    return ((b * (p.oh + p.fh - 1) + (row - b * p.oh)) * (p.ow + p.fw - 1) + (pix - row * p.ow)) * p.c;
   };
   // The filter bank, staged once per workgroup: rows of krow bytes, 16-byte chunks.
   extern __shared__ __attribute__((aligned(16))) uint8_t filt_lds[];
   const int lane = threadIdx.x & 63;
   constexpr int NT = 64 * WAVES;
   const uint32_t wave = blockIdx.x * WAVES + (threadIdx.x >> 6);
-  const uint32_t nwaves = gridDim.x * WAVES;
   const int li = lane & 15, lg = lane >> 4;
   const int W = p.ow + p.fw - 1;
   const int sub = p.c / 64;  // 64-channel slabs per filter position
@@ -70,25 +72,27 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(const void *image, const
   // nothing but the pointer and the thread index, so they go out first and are in flight
   // during the address arithmetic of the first pixel tile.
   constexpr int PER_THREAD = (SLABS * 256 + NT - 1) / NT;
+  constexpr bool EVEN_SHARES = SLABS * 256 % NT == 0;   // every thread moves PER_THREAD chunks: no bounds to test
   v4i stage[PER_THREAD];
 #pragma unroll
   for (int i = 0; i < PER_THREAD; i++) {
     const int c = i * NT + threadIdx.x;
-    if (c < SLABS * 256) stage[i] = *(const v4i *)(filters + c * 16);
+    if (EVEN_SHARES || c < SLABS * 256) stage[i] = *(const v4i *)(filters + c * 16);
   }
 
   // Byte offset of each slab's source relative to the pixel's own (y, x) position.
-  // (Slab s is channels 64 * (s % sub) .. of filter position s / sub; counted up rather than divided.)
-  int slab_off[SLABS];
+  // Slab s is channels 64 * (s % sub) .. of filter position s / sub.  The fw * sub slabs of a
+  // filter row are consecutive bytes of the image (channels fastest, then pixels), and the next
+  // row starts (W - fw) pixels further on: counted up, not divided.
+  uint32_t slab_off[SLABS];
   {
-    int r = 0, q = 0, cs = 0;
+    uint32_t off = 0, in_row = 0;
+    const uint32_t row_slabs = p.fw * sub, skip = (W - p.fw) * p.c;
 #pragma unroll
     for (int s = 0; s < SLABS; s++) {
-      slab_off[s] = (r * W + q) * p.c + cs * 64 + lg * 16;
-      if (++cs == sub) {
-        cs = 0;
-        if (++q == int(p.fw)) q = 0, r++;
-      }
+      slab_off[s] = off + lg * 16;
+      off += 64;
+      if (++in_row == row_slabs) in_row = 0, off += skip;
     }
   }
   // Pixel operand of one tile: lane (li, lg) holds pixel t*16+li, channels 16*lg .. +15 of
@@ -96,9 +100,9 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(const void *image, const
   // for the store.
   auto load_tile = [&](uint32_t t, v4i *img) {
     uint32_t pix = min(t * 16 + li, pixels - 1);
-    const uint8_t *src = (const uint8_t *)p.image + corner(pix) * p.c;
+    const uint32_t src = corner(pix);
 #pragma unroll
-    for (int s = 0; s < SLABS; s++) img[s] = *(const v4i *)(src + slab_off[s]);
+    for (int s = 0; s < SLABS; s++) img[s] = *(const v4i *)((const uint8_t *)p.image + (src + slab_off[s]));
   };
 
   // First tile's pixels are requested before anything else: their latency overlaps the
@@ -111,7 +115,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(const void *image, const
 #pragma unroll
   for (int i = 0; i < PER_THREAD; i++) {
     const int c = i * NT + threadIdx.x;
-    if (c < SLABS * 256) *(v4i *)(filt_lds + c * 16) = stage[i];
+    if (EVEN_SHARES || c < SLABS * 256) *(v4i *)(filt_lds + c * 16) = stage[i];
   }
   __syncthreads();
   v4i filt[FT][SLABS];
@@ -152,7 +156,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(const void *image, const
   while (t < tiles) {
     const uint32_t tn = t + nwaves;
     const uint32_t pix_n = min(min(tn, tiles - 1) * 16 + li, pixels - 1);  // clamped: always loadable
-    const uint8_t *src_n = (const uint8_t *)p.image + corner(pix_n) * p.c;
+    const uint32_t src_n = corner(pix_n);
     v4i acc[FT];
 #pragma unroll
     for (int ft = 0; ft < FT; ft++) acc[ft] = v4i{0, 0, 0, 0};
@@ -163,7 +167,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_i8(const void *image, const
 #pragma unroll
       for (int ft = 0; ft < FT; ft++)
         acc[ft] = __builtin_amdgcn_mfma_i32_16x16x64_i8(filt[ft][s], px, acc[ft], 0, 0, 0);
-      img[s] = *(const v4i *)(src_n + slab_off[s]);
+      img[s] = *(const v4i *)((const uint8_t *)p.image + (src_n + slab_off[s]));
     }
     // D[row = filter 4*lg + r][col = pixel li]: lane owns 4 consecutive filters of its pixel in
     // each filter tile.  An output stored as planes of filters takes them as they are: register r
@@ -431,10 +435,11 @@ hipError_t launch_slabs(const ConvArgs &c, bool img_unsigned, hipStream_t stream
              double(c.b) * (c.oh + c.fh - 1) * (c.ow + c.fw - 1) * c.c + double(c.f) * c.fh * c.fw * c.c +
                  4.0 * pixels * c.f * (c.accum ? 2 : 1));
   const FastDiv by_ow(c.ow), by_oh(c.oh);
+  // (a window of at most nine slabs: fh, fw and the slabs of a pixel are at most nine each)
+  const uint32_t packed = c.fh | c.fw << 4 | uint32_t(c.accum != 0) << 8 | (c.c / 64) << 9 | by_ow.shift << 16 | by_oh.shift << 24;
 #define MRL_CONV_I8(U, PLANES)                                                                                                      \
-  MRL_LAUNCH((k_conv_i8<SLABS, U, WAVES, PLANES>), dim3(blocks, groups), dim3(64 * WAVES), lds, stream, c.image, c.filters, c.out, c.c, \
-             c.f, c.oh, c.ow, c.fh | c.fw << 8 | uint32_t(c.accum != 0) << 16, uint32_t(pixels), by_ow.mul, by_oh.mul,                     \
-             by_ow.shift | by_oh.shift << 8)
+  MRL_LAUNCH((k_conv_i8<SLABS, U, WAVES, PLANES>), dim3(blocks, groups), dim3(64 * WAVES), lds, stream, c.image, c.filters, c.out, c.f, \
+             c.oh, c.ow, packed, uint32_t(pixels), by_ow.mul, by_oh.mul, blocks * WAVES)
   if (img_unsigned && c.out_planes) MRL_CONV_I8(true, true);
   else if (img_unsigned) MRL_CONV_I8(true, false);
   else if (c.out_planes) MRL_CONV_I8(false, true);
