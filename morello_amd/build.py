@@ -25,16 +25,16 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-command-line-argument",
+    # The first kernel arguments (up to 14 dwords) arrive preloaded in SGPRs with the wave instead of
+    # through a load the first instructions wait for: it takes a load's latency off the start of
+    # kernels that only run for a few microseconds (k_conv_i8 and k_attn keep all of theirs within
+    # the fourteen; a 3 us Softmax or conversion gains 0.2 us, the long kernels nothing).
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
 ]
 
 
-# Per-file additions.  Kernels whose arguments are few scalars get them preloaded into SGPRs with
-# the wave (up to 14 dwords) instead of loading them first thing: it takes a load's latency off the
-# start of kernels that only run for a few microseconds.
-EXTRA_FLAGS = {
-    "conv_i8.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
-    "attention.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
-}
+# Per-file additions.
+EXTRA_FLAGS = {}
 
 
 def _hipcc() -> str:
