@@ -44,7 +44,7 @@ ROUND_PEAK = {5033.0: 5000.0, 2516.0: 2500.0, 8000.0: 8000.0}  # the same peaks 
 MEASURED_TRAFFIC_BYTES = {
     "c2": 235721632,
     "c3": 2299689530,
-    "c4": 41165081,
+    "c4": 41134548,
     "c5": 42162440,
     "softmax": 537353602,
     "move": 536870912,
