@@ -58,6 +58,48 @@ inline int group_rows(int tiles_m, int tiles_n) {
   return best ? best : 4;
 }
 
+// Where a workgroup works, as scalars the launch works out and the kernel takes as its FIRST
+// arguments: those arrive in SGPRs with the wave (the GemmArgs structure behind them is loaded),
+// so the tile's coordinates are known, without a division, by the time the operands' addresses
+// are.  The divisions by a run-time value that this replaces are some thirty instructions each as
+// the compiler expands them, on the scalar unit one after the other, in front of the first load.
+struct TileWalk {
+  uint32_t tiles_m, tiles_n, group_m;
+  uint32_t per_xcd;     // tiles per XCD when the tiles divide evenly among the eight, else 0
+  uint32_t group_mul, full_mul, last_mul;   // FastDiv by group_m * tiles_n, by group_m, by the last group's rows
+  uint32_t shifts;      // their shift counts, a byte each
+};
+inline TileWalk tile_walk(int tiles_m, int tiles_n) {
+  TileWalk w;
+  w.tiles_m = uint32_t(tiles_m), w.tiles_n = uint32_t(tiles_n), w.group_m = uint32_t(group_rows(tiles_m, tiles_n));
+  const uint32_t ntiles = w.tiles_m * w.tiles_n;
+  w.per_xcd = ntiles % 8 == 0 ? ntiles / 8 : 0;
+  const FastDiv group(w.group_m * w.tiles_n), full(w.group_m), last(std::max(1u, w.tiles_m % w.group_m));
+  w.group_mul = group.mul, w.full_mul = full.mul, w.last_mul = last.mul;
+  w.shifts = group.shift | full.shift << 8 | last.shift << 16;
+  return w;
+}
+#define MRL_WALK_PARAMS                                                                                              \
+  uint32_t tiles_m, uint32_t tiles_n, uint32_t group_m, uint32_t per_xcd, uint32_t group_mul, uint32_t full_mul, \
+      uint32_t last_mul, uint32_t walk_shifts
+#define MRL_WALK_ARGS(w) (w).tiles_m, (w).tiles_n, (w).group_m, (w).per_xcd, (w).group_mul, (w).full_mul, (w).last_mul, (w).shifts
+// Workgroups are handed to the 8 XCDs round-robin; each XCD gets a contiguous run of tiles,
+// ordered so that a run, taken group_m tile rows at a time, covers a compact block of C (shared
+// A rows and B columns stay in that XCD's L2).
+#define MRL_WALK_TILE(tile_m, tile_n)                                                                     \
+  uint32_t tile_m, tile_n;                                                                                \
+  {                                                                                                       \
+    uint32_t pid = blockIdx.x;                                                                            \
+    if (per_xcd) pid = (pid & 7) * per_xcd + (pid >> 3);                                                  \
+    FastDiv by;                                                                                           \
+    by.mul = group_mul, by.shift = walk_shifts & 255;                                                     \
+    const uint32_t group = by.div(pid), first_m = group * group_m, gsz = min(tiles_m - first_m, group_m); \
+    const uint32_t in_group = pid - group * (group_m * tiles_n);                                          \
+    const bool full = gsz == group_m;                                                                     \
+    by.mul = full ? full_mul : last_mul, by.shift = (full ? walk_shifts >> 8 : walk_shifts >> 16) & 255;  \
+    tile_n = by.div(in_group), tile_m = first_m + (in_group - tile_n * gsz);                              \
+  }
+
 // Ragged tiles (EDGE) address memory through buffer resources: `records` bytes from `base` on
 // are in range, a load beyond them returns zeros and a store beyond them is dropped, both
 // without a branch.  Offsets are unsigned 32-bit, which is why the EDGE kernels want every
@@ -263,7 +305,7 @@ __device__ inline void sched_slots(bool staging) {
 // a channels-last image, g.conv; row p's 16-byte chunk at k byte kb lies at
 // corner(p) + ((r * w + s) * c_bytes + kb % c_bytes) with (r, s) = divmod(kb / c_bytes, fw).
 template <class T, bool A_UNSIGNED, class TL, bool EDGE, bool B_KMAJOR = false, bool CONV = false>
-__global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int tiles_n, int group_m) {
+__global__ __launch_bounds__(TL::NT) void k_gemm(MRL_WALK_PARAMS, GemmArgs g) {
   static_assert(!CONV || (EDGE && B_KMAJOR), "the implicit Conv operand is addressed through the buffer path");
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   constexpr int BM = TL::BM, BN = TL::BN, BKB = TL::BKB, WAVES_M = TL::WAVES_M, WAVES_N = TL::WAVES_N;
@@ -286,17 +328,7 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(GemmArgs g, int tiles_m, int ti
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lives in an SGPR
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
-  // Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous run of
-  // tiles, ordered so that a run covers a compact block of C (shared A rows and B columns
-  // stay in that XCD's L2).
-  int pid = blockIdx.x;
-  const int ntiles = tiles_m * tiles_n;
-  if (ntiles % 8 == 0) pid = (pid % 8) * (ntiles / 8) + pid / 8;
-  const int group = pid / (group_m * tiles_n);
-  const int first_m = group * group_m;
-  const int gsz = min(tiles_m - first_m, group_m);
-  const int in_group = pid % (group_m * tiles_n);
-  const int tile_m = first_m + in_group % gsz, tile_n = in_group / gsz;
+  MRL_WALK_TILE(tile_m, tile_n)
   const int64_t m0 = int64_t(tile_m) * BM, n0 = int64_t(tile_n) * BN;
 
   const uint8_t *A = (const uint8_t *)g.a + (int64_t(blockIdx.y) * g.sa + m0 * g.lda) * ES;
@@ -551,6 +583,7 @@ hipError_t launch(const GemmArgs &g, hipStream_t stream) {
     if (e != hipSuccess) return e;
   }
   const int tiles_m = int((g.m + BM - 1) / BM), tiles_n = int((g.n + BN - 1) / BN);
+  const TileWalk walk = tile_walk(tiles_m, tiles_n);
   {
     const double k_steps = double((g.k * T::ES + TL::BKB - 1) / TL::BKB) * (TL::BKB / T::ES);  // k, padded to steps
     const double mn = double(g.m) * g.n * g.batch;
@@ -567,7 +600,7 @@ hipError_t launch(const GemmArgs &g, hipStream_t stream) {
                            double((g.k * T::ES + TL::BKB - 1) / TL::BKB));
   }
   MRL_LAUNCH((k_gemm<T, A_UNSIGNED, TL, EDGE, B_KMAJOR, CONV>), dim3(tiles_m * tiles_n, g.batch), dim3(TL::NT),
-             2 * STAGE, stream, g, tiles_m, tiles_n, group_rows(tiles_m, tiles_n));
+             2 * STAGE, stream, MRL_WALK_ARGS(walk), g);
   return mrl::plan::last_error();
 }
 
