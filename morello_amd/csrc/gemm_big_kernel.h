@@ -50,7 +50,7 @@ constexpr int BIG_LDS_BYTES = 5 * 32768;  // two A stages and three B slots
 
 // M, N multiples of 256; K a multiple of two k steps (256 bytes); see big_applicable().
 template <class T, bool A_UNSIGNED>
-__global__ __launch_bounds__(512) void k_gemm_big(GemmArgs g, int tiles_m, int tiles_n, int group_m) {
+__global__ __launch_bounds__(512) void k_gemm_big(MRL_WALK_PARAMS, GemmArgs g) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   constexpr int BM = 256, BN = 256, BKB = 128, WAVES_M = 2, WAVES_N = 4, NT = 512;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
@@ -72,14 +72,7 @@ __global__ __launch_bounds__(512) void k_gemm_big(GemmArgs g, int tiles_m, int t
   // Workgroups go to the 8 XCDs round-robin; each XCD gets a contiguous run of tiles which, taken
   // group_m tile rows at a time, covers a compact block of C (its A rows and B columns stay in
   // that XCD's L2).
-  int pid = blockIdx.x;
-  const int ntiles = tiles_m * tiles_n;
-  if (ntiles % 8 == 0) pid = (pid % 8) * (ntiles / 8) + pid / 8;
-  const int group = pid / (group_m * tiles_n);
-  const int first_m = group * group_m;
-  const int gsz = min(tiles_m - first_m, group_m);
-  const int in_group = pid % (group_m * tiles_n);
-  const int tile_m = first_m + in_group % gsz, tile_n = in_group / gsz;
+  MRL_WALK_TILE(tile_m, tile_n)
   const int64_t m0 = int64_t(tile_m) * BM, n0 = int64_t(tile_n) * BN;
 
   const uint8_t *A = (const uint8_t *)g.a + (int64_t(blockIdx.y) * g.sa + m0 * g.lda) * ES;
@@ -175,8 +168,9 @@ hipError_t launch_big(const GemmArgs &g, hipStream_t stream) {
              (double(g.m) * g.k + double(g.k) * g.n) * g.batch * T::ES + mn * 4 * (g.accum ? 2 : 1),
              2.0 * 256 * 256 * double(g.k), 500.0 + 1200.0 * double(g.k * T::ES / 128),
              T::ES == 1 ? 1.25 : 1.08);  // measured: 1800 TOPS int8 at 4096^3
-  MRL_LAUNCH((k_gemm_big<T, A_UNSIGNED>), dim3(tiles_m * tiles_n, g.batch), dim3(512), BIG_LDS_BYTES, stream, g,
-             tiles_m, tiles_n, group_rows(tiles_m, tiles_n));
+  const TileWalk walk = tile_walk(tiles_m, tiles_n);
+  MRL_LAUNCH((k_gemm_big<T, A_UNSIGNED>), dim3(tiles_m * tiles_n, g.batch), dim3(512), BIG_LDS_BYTES, stream,
+             MRL_WALK_ARGS(walk), g);
   return mrl::plan::last_error();
 }
 

@@ -79,6 +79,11 @@ inline TileWalk tile_walk(int tiles_m, int tiles_n) {
   w.shifts = group.shift | full.shift << 8 | last.shift << 16;
   return w;
 }
+#ifdef MRL_WIDE_XCD_SWAP  // experiment: neighbouring XCDs exchange their blocks of tiles
+#define MRL_XCD_FLIP 1
+#else
+#define MRL_XCD_FLIP 0
+#endif
 #define MRL_WALK_PARAMS                                                                                              \
   uint32_t tiles_m, uint32_t tiles_n, uint32_t group_m, uint32_t per_xcd, uint32_t group_mul, uint32_t full_mul, \
       uint32_t last_mul, uint32_t walk_shifts
@@ -90,7 +95,7 @@ inline TileWalk tile_walk(int tiles_m, int tiles_n) {
   uint32_t tile_m, tile_n;                                                                                \
   {                                                                                                       \
     uint32_t pid = blockIdx.x;                                                                            \
-    if (per_xcd) pid = (pid & 7) * per_xcd + (pid >> 3);                                                  \
+    if (per_xcd) pid = ((pid & 7) ^ MRL_XCD_FLIP) * per_xcd + (pid >> 3);                                 \
     FastDiv by;                                                                                           \
     by.mul = group_mul, by.shift = walk_shifts & 255;                                                     \
     const uint32_t group = by.div(pid), first_m = group * group_m, gsz = min(tiles_m - first_m, group_m); \

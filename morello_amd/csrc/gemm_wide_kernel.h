@@ -79,7 +79,7 @@ constexpr int WIDE_MIN_STEPS = GEMM_WIDE_MIN_STEPS;
 // M, N multiples of 256; K an even number of k steps: GEMM_WIDE_MIN_STEPS at least for an accumulating
 // Spec (whose first eight steps carry the loads of C's old values), four otherwise; see wide_applicable().
 template <class T, bool A_UNSIGNED>
-__global__ __launch_bounds__(256) void k_gemm_wide(GemmArgs g, int tiles_m, int tiles_n, int group_m) {
+__global__ __launch_bounds__(256) void k_gemm_wide(MRL_WALK_PARAMS, GemmArgs g) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   constexpr int BM = 256, BN = 256, BKB = 128, WM = 128, WN = 128, TN = 8;
   constexpr int ES = T::ES, BK = BKB / ES;
@@ -101,18 +101,7 @@ __global__ __launch_bounds__(256) void k_gemm_wide(GemmArgs g, int tiles_m, int 
   // Workgroups go to the 8 XCDs round-robin; each XCD gets a contiguous run of tiles which, taken
   // group_m tile rows at a time, covers a compact block of C (its A rows and B columns stay in
   // that XCD's L2).
-  int pid = blockIdx.x;
-  const int ntiles = tiles_m * tiles_n;
-#ifdef MRL_WIDE_XCD_SWAP  // experiment: neighbouring XCDs exchange their blocks of tiles
-  if (ntiles % 8 == 0) pid = ((pid % 8) ^ 1) * (ntiles / 8) + pid / 8;
-#else
-  if (ntiles % 8 == 0) pid = (pid % 8) * (ntiles / 8) + pid / 8;
-#endif
-  const int group = pid / (group_m * tiles_n);
-  const int first_m = group * group_m;
-  const int gsz = min(tiles_m - first_m, group_m);
-  const int in_group = pid % (group_m * tiles_n);
-  const int tile_m = first_m + in_group % gsz, tile_n = in_group / gsz;
+  MRL_WALK_TILE(tile_m, tile_n)
   const int64_t m0 = int64_t(tile_m) * BM, n0 = int64_t(tile_n) * BN;
 
 #ifdef MRL_WIDE_SAME_PANELS  // energy experiment: every workgroup fetches the first tile's operands (L2 hits)
@@ -241,8 +230,9 @@ hipError_t launch_wide(const GemmArgs &g, hipStream_t stream) {
              (double(g.m) * g.k + double(g.k) * g.n) * g.batch * T::ES + mn * 4 * (g.accum ? 2 : 1),
              2.0 * 256 * 256 * double(g.k), 500.0 + 1200.0 * double(g.k * T::ES / 128),
              T::ES == 1 ? 1.62 : 1.18);  // measured: 2230-2330 TOPS int8 at 4096^3, 1360 TFLOPS bf16 at 8192^3
-  MRL_LAUNCH((k_gemm_wide<T, A_UNSIGNED>), dim3(tiles_m * tiles_n, g.batch), dim3(256), WIDE_LDS_BYTES, stream, g,
-             tiles_m, tiles_n, group_rows(tiles_m, tiles_n));
+  const TileWalk walk = tile_walk(tiles_m, tiles_n);
+  MRL_LAUNCH((k_gemm_wide<T, A_UNSIGNED>), dim3(tiles_m * tiles_n, g.batch), dim3(256), WIDE_LDS_BYTES, stream,
+             MRL_WALK_ARGS(walk), g);
   return mrl::plan::last_error();
 }
 

@@ -231,6 +231,7 @@ struct PartsArgs {
   float *ptr[4];
   int64_t stride[4][MRL_MAX_RANK];        // element strides per parameter (0 on reduced dims)
   uint64_t lines;                         // product of the dims other than scan_dim
+  FastDiv by_shape[MRL_MAX_RANK];         // filled in by launch_parts: a line number into coordinates without dividing
 };
 hipError_t launch_parts(const PartsArgs &p, hipStream_t stream);
 hipError_t launch_broadcast(const void *in, void *out, const LayoutEval &il, const LayoutEval &ol,

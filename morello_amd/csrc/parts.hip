@@ -53,14 +53,28 @@ __device__ inline Line line_of(const PartsArgs &p, uint64_t line) {
   Line l;
 #pragma unroll
   for (int t = 0; t < 4; t++) l.base[t] = 0;
-  uint64_t r = line;
+  if (p.lines < (1ull << 31)) {
+    // multiply-and-shift (FastDiv: exact below 2^31) where a 64-bit division by a run-time value is
+    // a hundred instructions and more, per dim, in front of the line's first load
+    uint32_t r = uint32_t(line);
 #pragma unroll
-  for (int d = MRL_MAX_RANK - 1; d >= 0; d--) {
-    if (uint32_t(d) >= p.rank || uint32_t(d) == p.scan_dim) continue;
-    const uint32_t c = uint32_t(r % p.shape[d]);
-    r /= p.shape[d];
+    for (int d = MRL_MAX_RANK - 1; d >= 0; d--) {
+      if (uint32_t(d) >= p.rank || uint32_t(d) == p.scan_dim) continue;
+      const uint32_t q = p.by_shape[d].div(r), c = r - q * p.shape[d];
+      r = q;
 #pragma unroll
-    for (int t = 0; t < 4; t++) l.base[t] += int64_t(c) * p.stride[t][d];   // 0 for a parameter the Spec does not have
+      for (int t = 0; t < 4; t++) l.base[t] += int64_t(c) * p.stride[t][d];   // 0 for a parameter the Spec does not have
+    }
+  } else {
+    uint64_t r = line;
+#pragma unroll
+    for (int d = MRL_MAX_RANK - 1; d >= 0; d--) {
+      if (uint32_t(d) >= p.rank || uint32_t(d) == p.scan_dim) continue;
+      const uint32_t c = uint32_t(r % p.shape[d]);
+      r /= p.shape[d];
+#pragma unroll
+      for (int t = 0; t < 4; t++) l.base[t] += int64_t(c) * p.stride[t][d];
+    }
   }
 #pragma unroll
   for (int t = 0; t < 4; t++) {
@@ -431,8 +445,10 @@ __global__ void k_fill(uint8_t *out, uint32_t pattern, uint32_t es, uint64_t cou
 // A parameter that has the scan dim in full (the others hold one value per line).
 inline bool full_size(const PartsArgs &p, uint32_t t) { return p.stride[t][p.scan_dim] != 0; }
 
-hipError_t launch_parts(const PartsArgs &p, hipStream_t stream) {
-  if (p.lines == 0) return hipSuccess;
+hipError_t launch_parts(const PartsArgs &args, hipStream_t stream) {
+  if (args.lines == 0) return hipSuccess;
+  PartsArgs p = args;
+  for (uint32_t d = 0; d < p.rank && d < MRL_MAX_RANK; d++) p.by_shape[d] = FastDiv(std::max(1u, p.shape[d]));
   const uint32_t n = p.shape[p.scan_dim];
   // Contiguous lines in whole, aligned 16-byte vectors: the register-resident form.
   bool rows = n % 4 == 0 && n > 1 && n <= 4096 && p.kind != MRL_SPEC_SOFTMAX_DENOMINATOR_AND_MAX_FROM_PARTS && full_size(p, 0);
