@@ -48,7 +48,7 @@ MEASURED_TRAFFIC_BYTES = {
     "c5": 42162440,
     "softmax": 537353602,
     "move": 536870912,
-    "matvec": 67270103,
+    "matvec": 67247424,
     "conv128": 19390667,
     "decode": 268960727,
     "softmax_long": 77155935,

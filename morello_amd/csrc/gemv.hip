@@ -12,6 +12,15 @@ namespace mrl {
 namespace {
 using gemm::v4i;
 
+// Rows of B per wavefront (up to four rows of A) and steps of K in flight: two and four measured
+// fastest (bf16 1 x 2048 x 16384: 10.5 us; four rows and two steps 12.4, eight rows 13.3, one row
+// 11.2); the switches are for such measurements.
+#ifndef MRL_GEMV_UNROLL
+#define MRL_GEMV_UNROLL 4
+#endif
+#ifndef MRL_GEMV_COLS
+#define MRL_GEMV_COLS 2
+#endif
 constexpr int WAVES = 4;         // wavefronts per workgroup
 constexpr int MAX_ROWS = 8;      // rows of A the kernel is built for
 
@@ -76,7 +85,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_gemv(GemmArgs g) {
 #pragma unroll
     for (int r = 0; r < ROWS; r++) acc[r][c] = 0;
   }
-#pragma unroll 2
+#pragma unroll MRL_GEMV_UNROLL
   for (int kb = lane * 16; kb < k_bytes; kb += 64 * 16) {
     v4i bv[COLS], av[ROWS];
 #pragma unroll
@@ -133,9 +142,9 @@ hipError_t launch_as(const GemmArgs &g, hipStream_t stream) {
 
 template <int KIND>
 hipError_t launch_rows(const GemmArgs &g, hipStream_t stream) {
-  if (g.m == 1) return launch_as<KIND, 1, 4>(g, stream);
-  if (g.m == 2) return launch_as<KIND, 2, 4>(g, stream);
-  if (g.m <= 4) return launch_as<KIND, 4, 4>(g, stream);
+  if (g.m == 1) return launch_as<KIND, 1, MRL_GEMV_COLS>(g, stream);
+  if (g.m == 2) return launch_as<KIND, 2, MRL_GEMV_COLS>(g, stream);
+  if (g.m <= 4) return launch_as<KIND, 4, MRL_GEMV_COLS>(g, stream);
   return launch_as<KIND, MAX_ROWS, 2>(g, stream);
 }
 
