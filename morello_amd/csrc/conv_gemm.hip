@@ -9,13 +9,12 @@ namespace mrl {
 namespace {
 using namespace gemm;
 
-typedef Tile<128, 128, 128, 2, 2> T128;
 typedef Tile<64, 64, 128, 2, 2> T64;
 
 template <class T, bool A_UNSIGNED>
 hipError_t launch_for(const GemmArgs &g, uint32_t tile, hipStream_t stream) {
   if (tile == 64) return launch<T, A_UNSIGNED, T64, true, true, true>(g, stream);
-  if (tile == 128) return launch<T, A_UNSIGNED, T128, true, true, true>(g, stream);
+  if (tile == 128) return launch<T, A_UNSIGNED, Tile128<T, true>, true, true, true>(g, stream);
   return launch<T, A_UNSIGNED, TileBig, true, true, true>(g, stream);
 }
 

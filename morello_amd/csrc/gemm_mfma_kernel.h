@@ -128,6 +128,15 @@ struct Tile {
   template <class T> static constexpr int stage() { return A_STAGE + (BKB / T::ES) * b_row<T>(); }
 };
 typedef Tile<256, 256, 128, 2, 4> TileBig;   // one workgroup per CU, 136 KiB of LDS
+// The 128 x 128 tile with a 128-byte step: eight waves of 32 x 64 outputs each for int8 (either
+// orientation of B) and for bf16 against a k-fastest B, four waves of 64 x 64 otherwise.  Twice the
+// waves hide more of a step's trip through LDS behind the other waves' MFMAs (one workgroup of this
+// tile is all a compute unit holds at mid sizes).  Measured, four / eight waves as 4 x 2 / as 2 x 4:
+// int8 1792^3 15.3 / 14.0 / 14.7 us, 2560 x 640 x 1280 9.05 / 8.28 / 8.31, 3072 x 3072 x 1024 22.6 /
+// 21.0 / 22.2, Conv 32 x (128 -> 128) x 28 x 28 3 x 3 13.2 / 11.1 / 11.6; bf16 row-major 2048^3 25.4 /
+// 27.2 / 25.9 (stays at four), the same Conv in bf16 17.4 / 15.8 / 15.6.
+template <class T, bool B_KMAJOR>
+using Tile128 = std::conditional_t<T::ES == 1 || (T::ES == 2 && B_KMAJOR), Tile<128, 128, 128, 4, 2>, Tile<128, 128, 128, 2, 2>>;
 
 typedef __attribute__((address_space(3))) v2i lds_v2i;
 typedef __attribute__((address_space(3))) v4s lds_v4s;

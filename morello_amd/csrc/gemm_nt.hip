@@ -7,13 +7,12 @@ namespace mrl {
 namespace {
 using namespace gemm;
 
-typedef Tile<128, 128, 128, 2, 2> T128;
 typedef Tile<64, 64, 128, 2, 2> T64;
 
 template <class T, bool A_UNSIGNED>
 hipError_t launch_for(const GemmArgs &g, uint32_t tile, hipStream_t stream) {
   if (tile == 64) return launch<T, A_UNSIGNED, T64, true, true>(g, stream);
-  if (tile == 128) return launch<T, A_UNSIGNED, T128, true, true>(g, stream);
+  if (tile == 128) return launch<T, A_UNSIGNED, Tile128<T, true>, true, true>(g, stream);
   const bool whole = g.m % TileBig::BM == 0 && g.n % TileBig::BN == 0 && g.k % (TileBig::BKB / T::ES) == 0;
   return whole ? launch<T, A_UNSIGNED, TileBig, false, true>(g, stream)
                : launch<T, A_UNSIGNED, TileBig, true, true>(g, stream);

@@ -18,7 +18,6 @@ typedef Tile<128, 256, 64, 2, 2> T128x256k64;
 typedef Tile<128, 128, 64, 2, 2> T128x128k64;
 typedef Tile<64, 64, 64, 2, 2> T64x64k64;
 typedef Tile<64, 64, 128, 2, 2> T64x64k128;
-typedef Tile<128, 128, 128, 2, 2> T128x128k128;
 
 struct Entry {
   uint32_t tile_m, tile_n, k_bytes, staging;
@@ -34,6 +33,16 @@ hipError_t launch_kind(const GemmArgs &g, int kind, hipStream_t stream) {
     case 1: return launch<I8, true, TL, true>(g, stream);
     case 2: return launch<BF16, false, TL, true>(g, stream);
     default: return launch<F32, false, TL, true>(g, stream);
+  }
+}
+
+// The 128 x 128 tile with a 128-byte step is laid out over its waves per element type (Tile128).
+hipError_t launch_128(const GemmArgs &g, int kind, hipStream_t stream) {
+  switch (kind) {
+    case 0: return launch<I8, false, Tile128<I8, false>, true>(g, stream);
+    case 1: return launch<I8, true, Tile128<I8, false>, true>(g, stream);
+    case 2: return launch<BF16, false, Tile128<BF16, false>, true>(g, stream);
+    default: return launch<F32, false, Tile128<F32, false>, true>(g, stream);
   }
 }
 
@@ -60,7 +69,7 @@ hipError_t launch_gemm_scheduled(const GemmArgs &g, int kind, uint32_t tile_m, u
   if (tile_m == 128 && tile_n == 256 && k_bytes == 64) return launch_kind<T128x256k64>(g, kind, stream);
   if (tile_m == 128 && tile_n == 128 && k_bytes == 64) return launch_kind<T128x128k64>(g, kind, stream);
   if (tile_m == 64 && tile_n == 64 && k_bytes == 64) return launch_kind<T64x64k64>(g, kind, stream);
-  if (tile_m == 128 && tile_n == 128 && k_bytes == 128) return launch_kind<T128x128k128>(g, kind, stream);
+  if (tile_m == 128 && tile_n == 128 && k_bytes == 128) return launch_128(g, kind, stream);
   if (tile_m == 64 && tile_n == 64 && k_bytes == 128) return launch_kind<T64x64k128>(g, kind, stream);
   return hipErrorInvalidValue;
 }
