@@ -15,6 +15,9 @@ using gemm::v4i;
 // Rows of B per wavefront (up to four rows of A) and steps of K in flight: two and four measured
 // fastest (bf16 1 x 2048 x 16384: 10.5 us; four rows and two steps 12.4, eight rows 13.3, one row
 // 11.2); the switches are for such measurements.
+#ifndef MRL_GEMV_MAX_M
+#define MRL_GEMV_MAX_M 8
+#endif
 #ifndef MRL_GEMV_UNROLL
 #define MRL_GEMV_UNROLL 4
 #endif
@@ -150,12 +153,25 @@ hipError_t launch_rows(const GemmArgs &g, hipStream_t stream) {
 
 }  // namespace
 
-// Few rows, long k-fastest rows of B: the problem is a stream over B.
+// Few rows, long k-fastest rows of B: the problem is a stream over B.  The dot products' VALU work
+// grows with the rows of A, while the matrix-core kernel with K shared out over workgroups takes the
+// same time for any row count up to its tile's 64, about what streaming B at 5.8 TB/s takes plus
+// the summing launch; so beyond two rows (f32, whose MFMA is slow: four) only the smaller problems
+// (8 MiB of B, 4 MiB from five rows on) stay here, and rows of B too long for their number (16 KiB and more, at most 2048 of them: too few
+// wavefronts with too long a walk each) go to the other kernel at any row count.  Measured, this
+// kernel / the other (us): bf16 4 x 4096 x 16384 28.2 / 22.8, 8 rows 42.0 / 23.0, u8 8 x 4096 x 16384
+// 29.8 / 15.2, bf16 4 x 2048 x 2048 4.6 / 7.2, 8 rows 6.5 / 7.2, bf16 2 x 8192 x 1024 11.1 / 8.1,
+// f32 4 x 4096 x 16384 52.6 / 72.8.
 bool gemv_applicable(const GemmArgs &g, int kind) {
   const int es = kind == 3 ? 4 : kind == 2 ? 2 : 1;
   const int64_t per16 = 16 / es;
   auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-  return g.b_kmajor && g.m >= 1 && g.m <= uint32_t(MAX_ROWS) && g.n >= 64 && int64_t(g.k) * es >= 1024 &&
+  // (all batch entries count: the slices of a K shared out are batch entries, and follow what was decided for the whole)
+  const uint64_t k_bytes = uint64_t(g.k) * es, b_bytes = k_bytes * g.n * g.batch;
+  const uint32_t few = kind == 3 ? 4 : 2;   // rows of A up to which the stream, not the arithmetic, sets the time
+  if (k_bytes >= 16384 && g.n <= 2048) return false;   // (its slices, once K is shared out, may come back here: 2 x 8192 x 1024 bf16 7.6 us that way)
+  if (g.m > few && b_bytes > (g.m <= 2 * few ? (8ull << 20) : (4ull << 20))) return false;
+  return g.b_kmajor && g.m >= 1 && g.m <= uint32_t(MRL_GEMV_MAX_M) && g.n >= 64 && int64_t(g.k) * es >= 1024 &&
          g.k % per16 == 0 && g.lda % per16 == 0 && g.ldb % per16 == 0 && g.sa % per16 == 0 && g.sb % per16 == 0 &&
          al16(g.a) && al16(g.b) && (reinterpret_cast<uintptr_t>(g.c) & 3) == 0 && g.batch <= 65535 &&
          uint64_t(g.n) < (1ull << 31);
