@@ -562,8 +562,15 @@ struct Forced {
 thread_local const Forced *g_forced = nullptr;
 
 // Where the kernel of conv_small.hip is taken (switches for measurement builds).
+// Measured against the implicit Matmul (us, this kernel / the other): int8 32 x (16 -> 16) x 110^2
+// 3 x 3 19.5 / 33.8, 16 -> 48 27.3 / 32, 32 -> 32 32.8 / 36, 32 -> 48 39.4 / 36.7; bf16 16 -> 48 38.9 /
+// 32.9; 8 x (16 -> 32) x 56^2 5.9 / 5.3, 8 x (32 -> 48) x 56^2 8.3 / 5.9: large images, and filters
+// times window bytes within what 32 filters of a 288-byte window make.
 #ifndef MRL_CONV_SMALL_MIN_PIXELS
-#define MRL_CONV_SMALL_MIN_PIXELS 16384ull
+#define MRL_CONV_SMALL_MIN_PIXELS 65536ull
+#endif
+#ifndef MRL_CONV_SMALL_MAX_BANK
+#define MRL_CONV_SMALL_MAX_BANK 9216ull
 #endif
 #ifndef MRL_CONV_SMALL_MAX_FILTERS
 #define MRL_CONV_SMALL_MAX_FILTERS 48u
@@ -689,6 +696,7 @@ int run_conv(const mrl_spec &s, void *const *params, Workspace &ws) {
                         channels_last(filt.t) && channels_last(out.t) && mrl::conv_small_applicable(cv, kind) &&
                         cv.f <= MRL_CONV_SMALL_MAX_FILTERS &&
                         uint64_t(cv.fh) * cv.fw * cv.c * (kind == 2 ? 2 : 1) <= MRL_CONV_SMALL_MAX_WINDOW &&
+                        uint64_t(cv.fh) * cv.fw * cv.c * (kind == 2 ? 2 : 1) * cv.f <= MRL_CONV_SMALL_MAX_BANK &&
                         uint64_t(cv.b) * cv.oh * cv.ow >= MRL_CONV_SMALL_MIN_PIXELS;
   if ((forced == 1 && !fused_ok && !windows_ok) || (forced == 2 && !implicit_ok) || (forced == 3 && !unfold_ok)) return MRL_ERR_UNSUPPORTED;
   if (fused_ok && forced <= 1) {

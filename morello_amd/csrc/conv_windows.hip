@@ -318,15 +318,14 @@ bool conv_windows_applicable(const ConvArgs &c, int kind) {
   // stores does not apply to planes, which are written a dword at a time.)
   if (kind < 0 || kind > 3) return false;
   const uint64_t es = kind == 3 ? 4 : kind == 2 ? 2 : 1, c_bytes = c.c * es, seg_padded = (uint64_t(c.fw) * c_bytes + 3) & ~3ull;
-  // Pixels that are not whole 16-byte chunks (the implicit Matmul cannot read those in place), and
-  // pixels of one chunk with windows of up to 192 bytes, where this kernel measured faster than
-  // the implicit Matmul's chunk-by-chunk addressing (32 x (16 -> 16) x 112^2 3 x 3 int8 27.5
-  // against 39 us, bf16 8 -> 32 28 against 34); with longer windows or wider pixels it is the slower
-  // one (int8 32 -> 32 3 x 3: 60 against 44 us; 48 -> 48 2 x 2 at 56^2: 17 against 13).
+  // Pixels that are not whole 16-byte chunks: the implicit Matmul cannot read those in place.  With
+  // whole chunks it is the faster one, pixels of a single chunk included (32 x (16 -> 16) x 110^2
+  // 3 x 3 int8: 33.8 us against 45.8 here, 16 -> 64 31.8 against 47.7, bf16 8 -> 32 29.1 against
+  // 31.0, 8 x (8 -> 32) x 56^2 4.9 against 8.9; int8 32 -> 32 3 x 3: 44 against 60).
 #ifdef MRL_WINDOWS_ANY_C   // measurement builds: every pixel width
   const bool c_ok = true;
 #else
-  const bool c_ok = c_bytes % 16 != 0 || (c_bytes == 16 && uint64_t(c.fh) * seg_padded <= 192);
+  const bool c_ok = c_bytes % 16 != 0;
 #endif
   return c.f % 16 == 0 && c.f / 64 < 65535 && c_ok && uint64_t(c.fh) * seg_padded <= 64 * (kind == 3 ? MAX_KS_F32 : MAX_KS) &&
          uint64_t(c.b) * ((c.oh + TILE_H - 1) / TILE_H) * ((c.ow + TILE_W - 1) / TILE_W) < (1ull << 31) &&

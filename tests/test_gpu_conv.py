@@ -196,8 +196,8 @@ def test_deep_conv_on_small_images_shares_its_windows_out(gpu, dts, codes, shape
     ((64, 32, 2, 1, 3, 2, 9), True),      # three output pixels per image
     ((1, 64, 5, 30, 30, 1, 1), False),    # 1 x 1 filters
     ((2, 32, 3, 11, 40, 9, 3), False),    # tall filters
-    ((3, 32, 16, 20, 33, 3, 3), True),    # pixels of one whole chunk, windows of 144 bytes: taken from the implicit Matmul
-    ((2, 16, 16, 9, 40, 2, 5), False),    # two runs of 80 bytes
+    ((3, 32, 20, 20, 33, 3, 3), True),    # pixels of a chunk and a quarter, windows of 180 bytes
+    ((2, 16, 10, 9, 40, 2, 5), False),    # two runs of 50 bytes
 ])
 @pytest.mark.parametrize("img_dt,img_code,gen", [(M.u8, 0, synth.uniform_u8), (M.i8, 1, synth.uniform_i8)])
 def test_conv_with_few_channels_forms_its_windows_in_lds(gpu, shape, accum, img_dt, img_code, gen):
@@ -225,16 +225,16 @@ def test_conv_with_few_channels_forms_its_windows_in_lds(gpu, shape, accum, img_
 
 
 @pytest.mark.parametrize("shape,accum", [
-    ((16, 32, 32, 40, 41, 3, 3), False),  # 32 channels, 3 x 3: 288 bytes, the last k step half empty
-    ((9, 48, 16, 50, 45, 4, 4), True),    # 16 channels, 4 x 4: four whole k steps; three tiles of filters
-    ((20, 16, 48, 30, 31, 2, 2), False),  # 48 channels: runs of 96 bytes, k steps across runs
-    ((3, 32, 32, 90, 70, 2, 5), True),    # 320 bytes, five k steps
-    ((1, 16, 64, 130, 129, 2, 2), False), # 64 channels under 2 x 2 with 16 filters (the 64-channel kernel wants filters in 64s)
+    ((41, 32, 32, 40, 41, 3, 3), False),  # 32 channels, 3 x 3: 288 bytes, the last k step half empty
+    ((30, 32, 16, 50, 45, 4, 4), True),   # 16 channels (pixels of one chunk), 4 x 4: four whole k steps
+    ((71, 48, 48, 30, 31, 2, 2), False),  # 48 channels: runs of 96 bytes, k steps across runs; three tiles of filters
+    ((11, 16, 32, 90, 70, 2, 5), True),   # 320 bytes, five k steps
+    ((4, 16, 64, 130, 129, 2, 2), False), # 64 channels under 2 x 2 with 16 filters (the 64-channel kernel wants filters in 64s)
 ])
 @pytest.mark.parametrize("dts,codes", [((M.u8, M.i8, M.i32), [0, 1, 5]), ((M.i8, M.i8, M.i32), [1, 1, 5]), ((M.bf16, M.bf16, M.f32), [7, 7, 6])])
 def test_early_layer_conv_with_the_filters_in_registers(gpu, shape, accum, dts, codes):
-    """Pixels of whole 16-byte chunks, windows of up to 320 bytes, up to 48 filters, 16384 pixels or
-    more: the kernel that keeps the filter bank in registers.  Integers bit for bit, bf16 to 1e-5
+    """Pixels of whole 16-byte chunks, windows of up to 320 bytes, up to 48 filters (and 9216 bytes of
+    filters times window), 65536 pixels or more: the kernel that keeps the filter bank in registers.  Integers bit for bit, bf16 to 1e-5
     of the oracle; an infinity in a bf16 image reaches the outputs whose windows hold it as an
     infinity (the chunks past the window's end are zero on both sides)."""
     b, f, c, oh, ow, fh, fw = shape
@@ -309,7 +309,7 @@ def test_f32_first_layer_conv_at_its_longest_window(gpu):
     ((2, 80, 3, 17, 15, 5, 5), True),     # two groups of filters
     ((1, 64, 5, 30, 30, 1, 1), False),    # 1 x 1 filters, runs of 10 bytes
     ((2, 32, 12, 9, 21, 3, 3), False),    # 24 bytes a pixel
-    ((2, 32, 8, 9, 21, 3, 3), True),      # one whole chunk a pixel, windows of 144 bytes
+    ((2, 32, 10, 9, 21, 3, 3), True),     # 20 bytes a pixel, windows of 180 bytes
 ])
 def test_bf16_conv_with_few_channels_forms_its_windows_in_lds(gpu, shape, accum):
     """The same kernel on bf16 operands (f32 sums, as a bf16 Matmul's).  An image that holds a NaN

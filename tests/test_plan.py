@@ -340,16 +340,19 @@ def test_cost_model_ranks_manual_schedules(gpu):
 
 
 def test_early_layer_convs_of_whole_chunk_pixels():
-    """Host only: pixels of exactly 16 bytes with windows of up to 192 bytes go to the kernel that
-    forms windows in LDS; wider pixels with windows of up to 320 bytes and at most 48 filters to
-    the kernel that keeps the filters in registers; more filters, longer windows and small
-    problems stay with the implicit Matmul."""
+    """Host only: pixels of whole 16-byte chunks with windows of up to 320 bytes, at most 48 filters
+    and filters x window bytes of at most 9216 go to the kernel that keeps the filters in
+    registers (pixels of a single chunk included: the kernel that forms windows in LDS is for
+    pixels that are not whole chunks); more filters, longer windows and small problems stay with
+    the implicit Matmul."""
     kernels = lambda c, f, fs, dts, b=32: M.Conv([b, f, c, 112, 112, fs, fs], dts).plan().kernels
     i8, bf = (M.u8, M.i8, M.i32), (M.bf16, M.bf16, M.f32)
-    assert kernels(16, 32, 3, i8) == ["k_conv_windows"] and kernels(8, 32, 3, bf) == ["k_conv_windows"]
+    assert kernels(16, 32, 3, i8) == ["k_conv_small"] and kernels(8, 32, 3, bf) == ["k_conv_small"]
     assert kernels(32, 32, 3, i8) == ["k_conv_small"] and kernels(16, 32, 3, bf) == ["k_conv_small"] and kernels(48, 48, 2, i8) == ["k_conv_small"]
     assert kernels(32, 64, 3, i8) == ["k_gemm"] and kernels(16, 32, 5, i8) == ["k_gemm"] and kernels(32, 32, 3, bf) == ["k_gemm"]
-    assert kernels(32, 32, 3, i8, b=1) == ["k_gemm"]     # 12544 pixels: too few tiles for one per wave
+    assert kernels(32, 48, 3, i8) == ["k_gemm"]          # 48 filters of 288 bytes: more than the bank the rule allows
+    assert kernels(32, 32, 3, i8, b=4) == ["k_gemm"]     # 50176 pixels: too few for a tile per wave to pay
+    assert kernels(12, 32, 3, i8) == ["k_conv_windows"]  # pixels of 12 bytes are not whole chunks
 
 
 def test_plans_of_the_softmax_primitives():
