@@ -35,11 +35,11 @@ bool applicable(const GemmArgs &g, int es) {
 // All three step through K 128 bytes at a time (a 64-byte step costs the small tiles 10-30 %).
 //   int8, bf16: 256 once a round is at least half full (3072^3, 144 tiles: int8 47 us against
 //     49 us for 128 and 62 us for 64); below that 64 while the 128 tile would leave well over a
-//     third of the compute units without one (1024^3: 6.5 us against 10.0 and 17.7; int8 up to 512
-//     tiles of 64: 6272 x 2304 x 256, 392 of them, 15.4 us against 16.2, 2048 x 2048 x 1024, 512,
-//     14.8 against 15.6, at 576 13.6 against 14.4 the other way; bf16 up to 500: 392 tiles 22.9
-//     against 23.5, even at 512), then 128 (2048^3: 17.3 us against 20.6 and 29.9; 1792^3, 784
-//     tiles: 16.5 against 19.4).
+//     third of the compute units without one (1024^3: 6.5 us against 10.0 and 17.7; up to 512
+//     tiles of 64: int8 6272 x 2304 x 256, 392 of them, 15.4 us against 16.2, 2048 x 2048 x 1024, 512,
+//     14.8 against 15.6, at 576 13.6 against 14.4 the other way; bf16 392 tiles 22.9 against 23.5,
+//     8 x 512^3, 512 tiles, 7.7 against 8.8, 1536^3, 576, 21.3 against 17.6 the other way), then 128
+//     (2048^3: 17.3 us against 20.6 and 29.9; 1792^3, 784 tiles: 16.5 against 19.4).
 //   f32: its MFMA has a sixteenth of the int8 rate, so operand traffic never limits a small
 //     tile: 64 (1024^3: 27 us against 70 and 239; 3072^3: 460 against 559 and 711) until the
 //     256 tile fills its rounds (4096^3: 948 us against 1066).
@@ -52,7 +52,12 @@ uint32_t tile_side(const GemmArgs &g, int es) {
   if (cap == 256 && round_fill >= (es == 4 ? 0.85 : 0.5)) return 256;
   if (es == 4 || cap == 64) return 64;
   const uint64_t small = uint64_t((g.m + 63) / 64) * ((g.n + 63) / 64) * g.batch;
-  return small <= (es == 1 ? 512 : 500) ? 64 : 128;
+  if (small <= 512) return 64;
+  // A side that the 128 tile pads by much more than the 64 tile does (192 rows: 256 against 192)
+  // costs it more than its larger tile gains (bf16 192 x 192 x 16384: 5.8 us against 6.3).
+  const double area64 = double((g.m + 63) / 64 * 64) * double((g.n + 63) / 64 * 64);
+  const double area128 = double((g.m + 127) / 128 * 128) * double((g.n + 127) / 128 * 128);
+  return area128 > 1.25 * area64 ? 64 : 128;
 }
 
 constexpr int elem_size_of(int kind) { return kind == 3 ? 4 : kind == 2 ? 2 : 1; }
