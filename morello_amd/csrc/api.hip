@@ -955,9 +955,19 @@ int run_compose_msm(const mrl_spec &s, void *const *params, Workspace &ws) {
       at.out = static_cast<float *>(result);
       // Queries per workgroup (tile_out over the Compose's rows): 64 where 128 would leave half of
       // the compute units or more without a workgroup, or pad a query dimension of 64 or less.
-      const uint64_t groups128 = uint64_t(b) * ((m + 127) / 128);
+      // Unless the keys are many enough to share out instead: 128 queries with the keys in as many
+      // parts as fill the chip measured faster once a part holds 4096 keys, or 1024 with at most a
+      // quarter of the units taken (2 x 8192 x 8192 keys: 68.8 us against 77.1, 1 x 8192 x 8192 39.9
+      // against 49.7, 2 x 4096 x 4096 30.6 against 34.1; 4 x 4096 x 4096 the other way, 47.2 against 42.8).
+      const uint64_t groups128 = uint64_t(b) * ((m + 127) / 128), units = mrl::g_compute_units;
+      bool few_groups = 2 * groups128 <= units;
+      if (few_groups && m > 64) {
+        const uint64_t parts = std::min<uint64_t>(units / groups128, ((n2 + 63) / 64) / 4);
+        const uint64_t keys = parts >= 2 ? n2 / parts : 0;
+        if (keys >= 4096 || (4 * groups128 <= units && keys >= 1024)) few_groups = false;
+      }
       at.query_block = forced == 1 && g_forced->query_block ? g_forced->query_block
-                       : (m <= 64 || 2 * groups128 <= mrl::g_compute_units) && m > 32 ? 64 : 128;
+                       : (m <= 64 || few_groups) && m > 32 ? 64 : 128;
       at.key_splits = forced == 1 && g_forced->key_splits ? g_forced->key_splits : mrl::attn_key_splits(at);
       if (at.key_splits > 1) {
         void *partials = nullptr;
