@@ -557,6 +557,7 @@ struct MoveTile {
   uint32_t tstride_s[MOVE_MAX_RANK], tstride_d[MOVE_MAX_RANK];
   uint32_t inv_s[MOVE_MAX_RANK], inv_d[MOVE_MAX_RANK], inv_ext[MOVE_MAX_RANK];  // ceil(2^32 / x)
   uint32_t tile;  // elements per tile
+  FastDiv by_chunks[MOVE_MAX_RANK];   // a block number into tile coordinates without dividing (blocks number below 2^31)
   // Runs of V > 1 elements per thread: the LDS distance between neighbours along the
   // destination's fastest digit, and whether whole runs may be loaded / stored as one vector.
   uint32_t lds_step;
@@ -584,15 +585,16 @@ __global__ __launch_bounds__(256) void k_move_gather(MoveTile p) {
   static_assert(V == 1 || !CONVERT, "runs are for elements that are not converted");
   typedef Cell Run __attribute__((ext_vector_type(V == 1 ? 2 : V)));  // used only when V > 1
   __shared__ Cell lds[MOVE_TILE_MAX + MOVE_TILE_MAX / 64];
-  uint64_t blk = blockIdx.x;
+  uint32_t blk = blockIdx.x;
   int64_t base_s = 0, base_d = 0;
   uint32_t room[MOVE_MAX_RANK];  // how much of each digit is left from this tile's origin on
 #pragma unroll
   for (uint32_t d = 0; d < MOVE_MAX_RANK; d++) {
     room[d] = 1;
     if (d < p.m.rank) {
-      const uint32_t origin = uint32_t(blk % p.chunks[d]) * p.ext[d];
-      blk /= p.chunks[d];
+      const uint32_t rest = p.by_chunks[d].div(blk);
+      const uint32_t origin = (blk - rest * p.chunks[d]) * p.ext[d];
+      blk = rest;
       room[d] = p.m.shape[d] - origin;
       base_s += int64_t(origin) * p.m.ss[d], base_d += int64_t(origin) * p.m.ds[d];
     }
@@ -1317,7 +1319,7 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
     for (uint32_t i = 0; i < MOVE_MAX_RANK; i++) {
       const uint32_t d = perm[i];
       t.m.shape[i] = o.m.shape[d], t.m.ss[i] = o.m.ss[d], t.m.ds[i] = o.m.ds[d];
-      t.ext[i] = o.ext[d], t.chunks[i] = o.chunks[d];
+      t.ext[i] = o.ext[d], t.chunks[i] = o.chunks[d], t.by_chunks[i] = FastDiv(o.chunks[d]);
       t.tstride_s[i] = o.tstride_s[d], t.tstride_d[i] = o.tstride_d[d];
       t.inv_s[i] = o.inv_s[d], t.inv_d[i] = o.inv_d[d], t.inv_ext[i] = o.inv_ext[d];
     }
