@@ -93,6 +93,23 @@ struct WaveShare {
   __device__ float max(float v) const { return wave_max(v); }
   __device__ float sum(float v) const { return wave_sum(v); }
 };
+// A workgroup of four wavefronts per line: a wavefront's partial result first, then the four meet in LDS.
+struct BlockShare {
+  uint32_t first, stride;
+  bool lead;
+  float *lds;  // [4]
+  template <bool MAX>
+  __device__ float combine(float v) const {
+    v = MAX ? wave_max(v) : wave_sum(v);
+    __syncthreads();  // the previous round's readers are done
+    if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+    __syncthreads();
+    const float a = lds[0], b = lds[1], c = lds[2], d = lds[3];
+    return MAX ? fmaxf(fmaxf(a, b), fmaxf(c, d)) : (a + b) + (c + d);
+  }
+  __device__ float max(float v) const { return combine<true>(v); }
+  __device__ float sum(float v) const { return combine<false>(v); }
+};
 // 256 / C threads of a workgroup per line, C lines side by side: partial results meet in LDS.
 template <int C>
 struct GroupShare {
@@ -261,6 +278,14 @@ __global__ __launch_bounds__(256) void k_parts(PartsArgs p) {
   const uint32_t lane = threadIdx.x & 63;
   const WaveShare sh{lane, 64, lane == 0};
   parts_line(p, line_of(p, line), sh, p.shape[p.scan_dim], true);
+}
+
+// Few long lines: a workgroup per line (a wavefront per line would leave most of the chip's load
+// queues empty: 1000 lines of 65536, denominator and max 138 -> 62 us).
+__global__ __launch_bounds__(256) void k_parts_block(PartsArgs p) {
+  __shared__ float lds[4];
+  const BlockShare sh{threadIdx.x, 256, threadIdx.x == 0, lds};
+  parts_line(p, line_of(p, blockIdx.x), sh, p.shape[p.scan_dim], true);
 }
 
 template <int C>
@@ -498,6 +523,8 @@ hipError_t launch_parts(const PartsArgs &args, hipStream_t stream) {
       MRL_LAUNCH(k_parts_cols<32>, dim3(uint32_t((p.lines + 31) / 32)), dim3(256), 0, stream, p);
     else
       MRL_LAUNCH(k_parts_cols<16>, dim3(uint32_t((p.lines + 15) / 16)), dim3(256), 0, stream, p);
+  } else if (n >= 4096 && p.lines <= 8ull * g_compute_units) {
+    MRL_LAUNCH(k_parts_block, dim3(uint32_t(p.lines)), dim3(256), 0, stream, p);
   } else {
     MRL_LAUNCH(k_parts, dim3(uint32_t(blocks)), dim3(256), 0, stream, p);
   }

@@ -16,6 +16,8 @@ SHAPES = [((7, 33), 1), ((5, 9, 4), 1), ((3, 4, 130), 2), ((6, 5), 0), ((2, 3, 4
           ((64, 2048), 1), ((1, 1, 1), 1), ((4, 1, 300), 2),
           # contiguous lines of whole 16-byte vectors: register-resident (4, 8, 16 vectors a lane)
           ((33, 1024), 1), ((5, 12), 1), ((7, 3, 2048), 2), ((9, 4096), 1), ((3, 4100), 1),
+          # few long lines that are not whole vectors: a workgroup per line
+          ((5, 9001), 1), ((2, 2, 4099), 2),
           # the scan dim is not the innermost: lines side by side, 16, 32 or 64 to a workgroup
           ((37, 70), 0), ((3, 50, 33), 1), ((2, 300, 64), 1), ((40, 20000), 0), ((24, 40000), 0), ((1, 18), 0),
           # lines of a handful of elements: a thread per line

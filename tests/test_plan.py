@@ -364,7 +364,8 @@ def test_plans_of_the_softmax_primitives():
     kernel = lambda spec: (spec.plan().steps[0].family, spec.plan().steps[0].grid[:2])
     assert kernel(M.Max([16, 2048, 2048], 2)) == ("k_parts_rows", (8192, 1))
     assert kernel(M.SoftmaxComplete([7, 12], 1))[0] == "k_parts_rows"
-    assert kernel(M.Max([3, 4100], 1))[0] == "k_parts" and kernel(M.Max([7, 33], 1))[0] == "k_parts"
+    assert kernel(M.Max([4096, 4100], 1))[0] == "k_parts" and kernel(M.Max([7, 33], 1))[0] == "k_parts"
+    assert kernel(M.Max([3, 4100], 1)) == ("k_parts_block", (3, 1))   # few long lines: a workgroup per line
     assert kernel(M.DivideVec([64, 64]))[0] == "k_parts_rows" and kernel(M.DivideVec([64, 66]))[0] == "k_parts"
     assert kernel(M.SoftmaxDenominatorAndMax([2048, 4096], 0)) == ("k_parts_cols", (256, 1))     # 16 lines each
     assert kernel(M.SoftmaxDenominatorAndMax([40, 20000], 0)) == ("k_parts_cols", (625, 1))      # 32
