@@ -1676,7 +1676,7 @@ uint32_t mrl_target_kernels(const char **names, uint32_t cap) {
       "k_gemm", "k_gemm_big", "k_gemm_wide", "k_gemv", "k_matmul_generic", "k_sum_splits", "k_conv_i8", "k_conv_rows_i8", "k_conv_windows", "k_conv_small", "k_conv_generic", "k_conv_generic_wave", "k_unfold",
       "k_unfold_gather", "k_attn", "k_attn_merge", "k_softmax_regs", "k_softmax_regs1", "k_softmax_short", "k_softmax_block", "k_softmax_chunk_stats", "k_softmax_chunk_write",
       "k_softmax_cols",
-      "k_softmax_generic", "k_parts", "k_parts_block", "k_parts_rows", "k_parts_cols", "k_broadcast", "k_broadcast_rows", "k_broadcast_fill_rows", "k_fill", "k_fill16", "k_fill_zero", "k_move_rows", "k_move_rows16",
+      "k_softmax_generic", "k_softmax_cols_short", "k_parts", "k_parts_block", "k_parts_rows", "k_parts_cols", "k_broadcast", "k_broadcast_rows", "k_broadcast_fill_rows", "k_fill", "k_fill16", "k_fill_zero", "k_move_rows", "k_move_rows16",
       "k_move_tiled", "k_move_tiled_as", "k_move_tiled8v", "k_move_tiled16", "k_move_tiled16v", "k_move_tiled32", "k_move_gather", "k_move_generic", "k_relayout", "k_convert4", "k_copy1",
       "k_copy16", "k_pad_rows", "k_pad_rows16", "k_widen_bf16"};
   const uint32_t n = sizeof families / sizeof families[0];

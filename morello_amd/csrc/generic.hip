@@ -954,6 +954,49 @@ __device__ inline void merge_pair(float &m, float &d, float om, float od) {
   d = d * expf(m - nm) + od * expf(om - nm);
   m = nm;
 }
+// A scan dim of at most 16 elements beside a contiguous dim: a thread per column, the column in
+// registers, 256 consecutive columns per workgroup (q.fast_tiles counts tiles of 256 here).  The
+// kernel below would give each handful of rows a workgroup of its own, with its start-up and its
+// exchange through LDS: 8 x 8 x 1024 x 1024 over dim 1 took 295 us that way.
+__global__ __launch_bounds__(256) void k_softmax_cols_short(SMC q) {
+  const SM &p = q.s;
+  uint64_t r = blockIdx.x;
+  const uint32_t f = uint32_t(r % q.fast_tiles) * 256 + threadIdx.x;
+  r /= q.fast_tiles;
+  int64_t ibase = 0, obase = 0;
+  for (int d = int(p.rank) - 1; d >= 0; d--) {
+    if (uint32_t(d) == p.scan_dim || uint32_t(d) == q.fast) continue;
+    const uint32_t c = uint32_t(r % p.shape[d]);
+    r /= p.shape[d];
+    ibase += c * p.si[d];
+    obase += c * p.so[d];
+  }
+  if (f >= p.shape[q.fast]) return;
+  ibase += f, obase += f;  // unit stride on both sides
+  const uint32_t n = p.shape[p.scan_dim];
+  const int64_t is = p.si[p.scan_dim], os = p.so[p.scan_dim];
+  float x[16];
+  float m = -3.40282347e+38f;
+  bool nan = false;
+#pragma unroll
+  for (int j = 0; j < 16; j++) {
+    x[j] = uint32_t(j) < n ? p.in[ibase + j * is] : -3.40282347e+38f;
+    nan |= x[j] != x[j];
+    m = fmaxf(m, x[j]);
+  }
+  if (nan) m = __uint_as_float(0x7fc00000u);
+  float den = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 16; j++) {
+    x[j] = exp_nonpositive(x[j] - m);
+    den += uint32_t(j) < n ? x[j] : 0.0f;
+  }
+  const float inv = 1.0f / den;
+#pragma unroll
+  for (int j = 0; j < 16; j++)
+    if (uint32_t(j) < n) MRL_STORE_ONCE(x[j] * inv, p.out + obase + j * os);
+}
+
 template <int WAVES, int PHASE>
 __global__ __launch_bounds__(64 * WAVES) void k_softmax_cols(SMC q) {
   const SM &p = q.s;
@@ -1509,6 +1552,13 @@ hipError_t launch_softmax_generic(const Strided &in, const Strided &out, uint32_
       SMC q;
       q.s = p, q.fast = d, q.fast_tiles = (in.shape[d] + 63) / 64;
       q.chunks = 1, q.chunk_len = in.shape[scan_dim], q.pairs = nullptr;
+      if (in.shape[scan_dim] <= 16 && lines >= 65536) {
+        q.fast_tiles = (in.shape[d] + 255) / 256;
+        const uint64_t wgs = lines / in.shape[d] * q.fast_tiles;
+        if (wgs > 0x7fffffffull) break;
+        MRL_LAUNCH(k_softmax_cols_short, dim3(uint32_t(wgs)), dim3(256), 0, stream, q);
+        return mrl::plan::last_error();
+      }
       const uint64_t blocks = lines / in.shape[d] * q.fast_tiles;
       if (blocks > 0x7fffffffull) break;
       const uint32_t chunks = scratch ? softmax_cols_chunks(blocks, in.shape[scan_dim]) : 1;

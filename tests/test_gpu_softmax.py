@@ -101,6 +101,13 @@ def test_softmax_over_an_outer_dim(gpu, shape, dim):
     _softmax_outer(shape, dim)
 
 
+@pytest.mark.parametrize("shape,dim", [((8, 70000), 0), ((3, 5, 300, 100), 1), ((2, 16, 40000), 1), ((1, 70001), 0)])
+def test_softmax_over_a_short_outer_dim(gpu, shape, dim):
+    """A scan dim of at most 16 elements beside 65536 columns or more: a thread per column."""
+    assert M.Softmax(list(shape), dim).plan().kernels == ["k_softmax_cols_short"]
+    _softmax_outer(shape, dim)
+
+
 @pytest.mark.parametrize("shape,dim", [((600, 64, 300), 0), ((100, 64, 300), 0), ((3, 520, 20000), 1)])
 def test_softmax_over_an_outer_dim_in_one_kernel(gpu, shape, dim):
     """Enough columns for 256 workgroups of 64: the kernel that walks the scan dim itself, on 16
@@ -419,10 +426,11 @@ def test_softmax_tensor_beyond_4_gib(gpu):
 
 
 @pytest.mark.parametrize("shape,dim", [((6, 256), 1), ((6, 2048), 1), ((6, 4100), 1), ((6, 9000), 1), ((6, 40000), 1),
-                                       ((6, 33), 1), ((6, 5), 1), ((300, 6, 12), 2), ((6, 700, 8), 1), ((3, 2, 1100), 2)])
+                                       ((6, 33), 1), ((6, 5), 1), ((300, 6, 12), 2), ((6, 700, 8), 1), ((3, 2, 1100), 2),
+                                       ((6, 70000), 0)])
 def test_softmax_infinities_follow_the_reference(gpu, shape, dim):
     """Rows with infinities and NaNs on every Softmax kernel (rows in registers, short rows, a
-    workgroup per row, rows in chunks, a scan dim that is not the innermost), as the reference's
+    workgroup per row, rows in chunks, a scan dim that is not the innermost, a thread per column), as the reference's
     interpreter treats them (verification.rs:166-184 with the NaN-propagating max that starts
     from f32::MIN, :842-861): -inf among finite scores gives exact zeros; a row that is all
     -inf, or holds +inf or a NaN, is NaN throughout; the other rows are untouched by it."""
