@@ -486,7 +486,6 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
       p.t = dense;
       return MRL_OK;
     };
-    if (!walkable(a.t) && (rc = densify(a, true, true)) != MRL_OK) return rc;
     bool b_walkable = walkable(b.t);
     if (!b_walkable) {
       mrl::Strided bt = b.t;  // [b, n, k] view: B with k fastest needs whole chunks along K
@@ -494,9 +493,28 @@ int run_matmul(const mrl_spec &s, void *const *params, Workspace &ws,
       std::swap(bt.stride[1], bt.stride[2]);
       b_walkable = walkable(bt);
     }
-    if (!b_walkable) {
-      if ((rc = densify(b, true, true)) != MRL_OK) return rc;
+    int64_t any_ld, any_bs;
+    if (!walkable(a.t) && !b_walkable && a.elem == b.elem && as_rows(a.t, &any_ld, &any_bs) && as_rows(b.t, &any_ld, &any_bs)) {
+      // Both operands keep their rows and only need them padded: the two copies in one launch.
+      Prepared *both[2] = {&a, &b};
+      mrl::Strided dense[2];
+      for (int i = 0; i < 2; i++) {
+        const Prepared &p = *both[i];
+        dense[i] = p.t;
+        const int64_t cols = p.t.shape[2], ld = (cols + per16 - 1) / per16 * per16;
+        dense[i].stride[2] = 1, dense[i].stride[1] = ld, dense[i].stride[0] = int64_t(p.t.shape[1]) * ld;
+        HIP_TRY(ws.alloc(&dense[i].ptr, size_t(p.t.shape[0]) * dense[i].stride[0] * p.elem));
+      }
+      HIP_TRY(mrl::launch_pad_rows_pair(a.t, dense[0].ptr, uint32_t(dense[0].stride[1]), b.t, dense[1].ptr,
+                                        uint32_t(dense[1].stride[1]), a.elem, ws.stream));
+      a.t = dense[0], b.t = dense[1];
       g.b_kmajor = false;
+    } else {
+      if (!walkable(a.t) && (rc = densify(a, true, true)) != MRL_OK) return rc;
+      if (!b_walkable) {
+        if ((rc = densify(b, true, true)) != MRL_OK) return rc;
+        g.b_kmajor = false;
+      }
     }
     int64_t ld, bs;
     c_densified = !as_rows(c.t, &ld, &bs);
@@ -1678,7 +1696,7 @@ uint32_t mrl_target_kernels(const char **names, uint32_t cap) {
       "k_softmax_cols",
       "k_softmax_generic", "k_softmax_cols_short", "k_parts", "k_parts_block", "k_parts_rows", "k_parts_cols", "k_broadcast", "k_broadcast_rows", "k_broadcast_fill_rows", "k_fill", "k_fill16", "k_fill_zero", "k_move_rows", "k_move_rows16",
       "k_move_tiled", "k_move_tiled_as", "k_move_tiled8v", "k_move_tiled16", "k_move_tiled16v", "k_move_tiled32", "k_move_gather", "k_move_generic", "k_relayout", "k_convert4", "k_copy1",
-      "k_copy16", "k_pad_rows", "k_pad_rows16", "k_widen_bf16"};
+      "k_copy16", "k_pad_rows", "k_pad_rows_pair", "k_pad_rows16", "k_widen_bf16"};
   const uint32_t n = sizeof families / sizeof families[0];
   for (uint32_t i = 0; i < n && i < cap && names; i++) names[i] = families[i];
   return n;

@@ -86,6 +86,9 @@ hipError_t launch_move_view(const void *src, int src_dtype, void *dst, int dst_d
 // (a whole number of dwords), zeros from each row's end to `dst_ld`.
 hipError_t launch_pad_rows(const Strided &src, void *dst, uint32_t dst_ld, uint32_t elem_size,
                            hipStream_t stream);
+// Two such copies (elements of the same size) in one launch.
+hipError_t launch_pad_rows_pair(const Strided &src0, void *dst0, uint32_t dst_ld0, const Strided &src1, void *dst1,
+                                uint32_t dst_ld1, uint32_t elem_size, hipStream_t stream);
 // bf16 -> f32 of a whole buffer, position by position.
 hipError_t launch_widen_bf16(const void *src, void *dst, uint64_t count, hipStream_t stream);
 // Move Spec fast path: same bytes on both sides (16-byte aligned buffers).
