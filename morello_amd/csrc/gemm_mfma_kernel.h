@@ -552,6 +552,32 @@ __global__ __launch_bounds__(TL::NT) void k_gemm(MRL_WALK_PARAMS, GemmArgs g) {
   __syncthreads();
   read_frags(0, 0, 0);
 
+  // One or two k steps on the smallest tile (a 64^3 problem is one workgroup and two steps): no
+  // loop.  The loop below stays free of branches by loading and staging the last tile again past
+  // the end of K, and with so few steps those extra trips to L2 are most of what the launch waits for.
+  if constexpr (BM == 64 && BN == 64) {
+    if (kt_count <= 2) {
+#pragma unroll
+      for (int s = 0; s < SLABS; s++) {
+        if (s + 1 < SLABS) read_frags(0, s + 1, (s + 1) & 1);
+        mfma_slab(s, s & 1);
+      }
+      if (kt_count == 2) {
+        store_lds(1);  // the second tile has been in registers since the prologue
+        __syncthreads();
+        read_frags(1, 0, 0);
+#pragma unroll
+        for (int s = 0; s < SLABS; s++) {
+          if (s + 1 < SLABS) read_frags(1, s + 1, (s + 1) & 1);
+          mfma_slab(s, s & 1);
+        }
+      }
+      epilogue<T, A_UNSIGNED, EDGE, BN, WAVES_M, TM, TN>(g, C, lds, acc, colsum, lane, wm, wm * WM, wn * WN,
+                                                         int(g.m - m0), int(g.n - n0));
+      return;
+    }
+  }
+
   for (int kt = 0; kt < kt_count; kt++) {
     const int cur = kt & 1;
     // Tile kt+2 is loaded next (or the last tile again when there is none).
