@@ -49,7 +49,7 @@ MEASURED_TRAFFIC_BYTES = {
     "softmax": 537353602,
     "move": 536870912,
     "matvec": 67247424,
-    "conv128": 19298257,
+    "conv128": 19317177,
     "decode": 268960727,
     "softmax_long": 77155935,
     "transpose": 537368281,
