@@ -251,6 +251,28 @@ def test_matrix_vector_shapes(gpu, dts, codes, shape, accum, b_k_fastest):
         assert rel_err(got, want) < 1e-5
 
 
+@pytest.mark.parametrize("dts,codes,shape,accum", [((M.bf16, M.bf16, M.f32), [7, 7, 6], (1, 1, 4096, 32768), True),
+                                                    ((M.u8, M.i8, M.i32), [0, 1, 5], (1, 1, 8192, 32770), False)])
+def test_matrix_vector_against_a_very_large_b(gpu, dts, codes, shape, accum):
+    """One row of A against a k-fastest B of 200 MB and more: a row of B per wavefront (the
+    smaller ones take two).  Same results as any other Matmul; the second shape's last
+    workgroup holds two columns of its four."""
+    b, m, k, n = shape
+    gen = {M.u8: synth.uniform_u8, M.i8: synth.uniform_i8, M.bf16: synth.normal_bf16}
+    A, Bm = gen[dts[0]](76, 0, (b, m, k)), gen[dts[1]](76, 1, (b, k, n))
+    Bt = np.ascontiguousarray(Bm.transpose(0, 2, 1))   # B as stored: [n][k]
+    out_np = np.int32 if dts[2] == M.i32 else np.float32
+    C0 = synth.uniform_u8(76, 2, (b, m, n)).astype(out_np) if accum else np.zeros((b, m, n), out_np)
+    spec = M.Matmul(shape, dts, layouts=[None, M.layout(0, 2, 1), None], accum=accum)
+    assert spec.plan().kernels == ["k_gemv"] and "COLS = 1" in spec.plan().steps[0].kernel
+    got = run_spec(spec, [A, Bt, C0])
+    want = orc.matmul(list(shape), codes, A, Bm, C0.copy(), accum)
+    if dts[2] == M.i32:
+        assert np.array_equal(got, want)
+    else:
+        assert rel_err(got, want) < 1e-5
+
+
 @pytest.mark.parametrize("dts,codes", [((M.u8, M.i8, M.i32), [0, 1, 5]), ((M.i8, M.i8, M.i32), [1, 1, 5]),
                                        ((M.bf16, M.bf16, M.f32), [7, 7, 6]), ((M.f32, M.f32, M.f32), [6, 6, 6])])
 @pytest.mark.parametrize("shape,accum", [((1, 512, 8192, 512), False), ((1, 256, 16384, 192), True),
